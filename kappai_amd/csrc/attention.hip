@@ -1,0 +1,205 @@
+// Attention over the paged cache.
+//
+//   qk_norm_rope_store  per-head RMSNorm of q and k (src/backend/cpu/scalar/quants.c:1521-1531),
+//                       rotation at the row's absolute position
+//                       (src/backend/cpu/quants.h:395-438: rotate-half or interleaved pairs),
+//                       q rewritten in place, k and v stored into their pages
+//                       (src/backend/cpu/common.c:1603-1622).
+//   paged_attention_rows  one wave per (row, head): causal softmax(q.k/sqrt(d)) v over the keys
+//                       lo..pos of the row's request, read through its block table
+//                       (src/backend/cpu/scalar/core.c:383-433, 623-666), online softmax in float.
+//
+// Pools are [page][kv_head][page_size][head_dim]; token p of a request lives in page
+// block_table[p / page_size] at offset p % page_size.
+#include "common.h"
+
+#define MAX_HEAD_DIM 512
+
+// rot_mode: 0 none, 1 rotate-half pairs (j, j+rot/2), 2 interleaved pairs (2j, 2j+1)
+template <typename T>
+__global__ __launch_bounds__(64) void qk_norm_rope_store_kernel(
+    T* __restrict__ qkv, int row_stride, const float* __restrict__ q_norm_w,
+    const float* __restrict__ k_norm_w, float eps, const float* __restrict__ cos_tab,
+    const float* __restrict__ sin_tab, int rot_dim, int rot_mode, T* __restrict__ k_pool,
+    T* __restrict__ v_pool, const int* __restrict__ row_pos, const int* __restrict__ row_seg,
+    const int* __restrict__ block_tables, int max_blocks, int H, int G, int d, int ps,
+    int store_kv) {
+  __shared__ float buf[MAX_HEAD_DIM];
+  const int t = blockIdx.x, slot = blockIdx.y, lane = threadIdx.x;
+  const int pos = row_pos[t];
+  T* src = qkv + (size_t)t * row_stride + (size_t)slot * d;
+  T* dst = src;
+  if (slot >= H) {
+    const int g = (slot - H) % G;
+    const int* bt = block_tables + (size_t)row_seg[t] * max_blocks;
+    const size_t row = ((size_t)bt[pos / ps] * G + g) * ps + pos % ps;
+    dst = (slot < H + G ? k_pool : v_pool) + row * d;
+  }
+  if (slot >= H + G) {  // v: plain copy into its page
+    for (int e = lane; e < d; e += WAVE) dst[e] = src[e];
+    return;
+  }
+  const float* nw = slot < H ? q_norm_w : k_norm_w;
+  float ss = 0.f;
+  for (int e = lane; e < d; e += WAVE) {
+    const float v = to_f32(src[e]);
+    buf[e] = v;
+    ss += v * v;
+  }
+  if (nw) {
+    ss = wave_sum(ss);
+    const float sc = 1.0f / sqrtf(ss / (float)d + eps);
+    for (int e = lane; e < d; e += WAVE) buf[e] = buf[e] * sc * nw[e];
+  }
+  __syncthreads();
+  if (rot_mode == 0) rot_dim = 0;
+  const int half = rot_dim / 2;
+  const float* ct = cos_tab + (size_t)pos * half;
+  const float* st = sin_tab + (size_t)pos * half;
+  for (int j = lane; j < half; j += WAVE) {
+    const int i0 = rot_mode == 1 ? j : 2 * j;
+    const int i1 = rot_mode == 1 ? j + half : 2 * j + 1;
+    const float c = ct[j], s = st[j];
+    const float v0 = buf[i0], v1 = buf[i1];
+    from_f32(dst + i0, v0 * c - v1 * s);
+    from_f32(dst + i1, v0 * s + v1 * c);
+  }
+  for (int e = rot_dim + lane; e < d; e += WAVE) from_f32(dst + e, buf[e]);
+}
+
+extern "C" int kappai_qk_norm_rope_store(void* qkv, int row_stride, const float* q_norm_w,
+                                         const float* k_norm_w, float eps, const float* cos_tab,
+                                         const float* sin_tab, int rot_dim, int rot_mode,
+                                         void* k_pool, void* v_pool, const int* row_pos,
+                                         const int* row_seg, const int* block_tables,
+                                         int max_blocks, int T, int H, int G, int d, int ps,
+                                         int store_kv, int is_bf16, hipStream_t stream) {
+  if (T <= 0) return 0;
+  if (d > MAX_HEAD_DIM || d < 1 || rot_dim > d || (rot_dim & 1)) return (int)hipErrorInvalidValue;
+  dim3 grid(T, store_kv ? H + 2 * G : H);
+  if (is_bf16)
+    hipLaunchKernelGGL(qk_norm_rope_store_kernel<bf16_t>, grid, dim3(WAVE), 0, stream,
+                       (bf16_t*)qkv, row_stride, q_norm_w, k_norm_w, eps, cos_tab, sin_tab,
+                       rot_dim, rot_mode, (bf16_t*)k_pool, (bf16_t*)v_pool, row_pos, row_seg,
+                       block_tables, max_blocks, H, G, d, ps, store_kv);
+  else
+    hipLaunchKernelGGL(qk_norm_rope_store_kernel<float>, grid, dim3(WAVE), 0, stream, (float*)qkv,
+                       row_stride, q_norm_w, k_norm_w, eps, cos_tab, sin_tab, rot_dim, rot_mode,
+                       (float*)k_pool, (float*)v_pool, row_pos, row_seg, block_tables, max_blocks,
+                       H, G, d, ps, store_kv);
+  KAPPAI_RETURN_LAUNCH_STATUS();
+}
+
+// ---------------------------------------------------------------------------------------
+__device__ __forceinline__ float dot_row(const float* __restrict__ qs, const float* __restrict__ k,
+                                         int d) {
+  float s = 0.f;
+  for (int e = 0; e < d; e += 4) {
+    const float4 kv = *reinterpret_cast<const float4*>(k + e);
+    s = fmaf(qs[e], kv.x, s);
+    s = fmaf(qs[e + 1], kv.y, s);
+    s = fmaf(qs[e + 2], kv.z, s);
+    s = fmaf(qs[e + 3], kv.w, s);
+  }
+  return s;
+}
+
+__device__ __forceinline__ float dot_row(const float* __restrict__ qs,
+                                         const bf16_t* __restrict__ k, int d) {
+  float s = 0.f;
+  for (int e = 0; e < d; e += 8) {
+    const uint4 kv = *reinterpret_cast<const uint4*>(k + e);
+    const uint32_t w[4] = {kv.x, kv.y, kv.z, kv.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      s = fmaf(qs[e + 2 * i], __uint_as_float(w[i] << 16), s);
+      s = fmaf(qs[e + 2 * i + 1], __uint_as_float(w[i] & 0xffff0000u), s);
+    }
+  }
+  return s;
+}
+
+#define ATT_NPL (MAX_HEAD_DIM / WAVE)
+
+template <typename T>
+__global__ __launch_bounds__(64) void paged_attention_rows_kernel(
+    const T* __restrict__ q, int q_stride, const T* __restrict__ k_pool,
+    const T* __restrict__ v_pool, T* __restrict__ out, int out_stride,
+    const int* __restrict__ row_pos, const int* __restrict__ row_seg,
+    const int* __restrict__ block_tables, int max_blocks, int H, int G, int d, int ps, int window,
+    float scale) {
+  __shared__ float qs[MAX_HEAD_DIM];
+  const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const int g = h / (H / G);
+  const int pos = row_pos[t];
+  const int* bt = block_tables + (size_t)row_seg[t] * max_blocks;
+  const int lo = (window > 0 && pos + 1 > window) ? pos + 1 - window : 0;
+  const T* qr = q + (size_t)t * q_stride + (size_t)h * d;
+  for (int e = lane; e < d; e += WAVE) qs[e] = to_f32(qr[e]);
+  __syncthreads();
+
+  float m = -INFINITY, l = 0.f;
+  float acc[ATT_NPL];
+#pragma unroll
+  for (int i = 0; i < ATT_NPL; ++i) acc[i] = 0.f;
+
+  for (int base = lo; base <= pos; base += WAVE) {
+    const int tk = base + lane;
+    const bool valid = tk <= pos;
+    float s = -INFINITY;
+    unsigned long long voff = 0;
+    if (valid) {
+      const size_t row = ((size_t)bt[tk / ps] * G + g) * ps + tk % ps;
+      s = dot_row(qs, k_pool + row * d, d) * scale;
+      voff = (unsigned long long)row * d;
+    }
+    const float m_new = fmaxf(m, wave_max(s));
+    const float p = valid ? expf(s - m_new) : 0.f;
+    const float corr = expf(m - m_new);
+    l = l * corr + wave_sum(p);
+#pragma unroll
+    for (int i = 0; i < ATT_NPL; ++i) acc[i] *= corr;
+    const int nk = min(WAVE, pos - base + 1);
+    for (int kk = 0; kk < nk; ++kk) {
+      const float pk = __shfl(p, kk, WAVE);
+      const unsigned lo32 = __shfl((unsigned)(voff & 0xffffffffull), kk, WAVE);
+      const unsigned hi32 = __shfl((unsigned)(voff >> 32), kk, WAVE);
+      const T* vr = v_pool + (((unsigned long long)hi32 << 32) | lo32);
+#pragma unroll
+      for (int i = 0; i < ATT_NPL; ++i) {
+        const int e = lane + i * WAVE;
+        if (e < d) acc[i] = fmaf(pk, to_f32(vr[e]), acc[i]);
+      }
+    }
+    m = m_new;
+  }
+  const float inv = 1.0f / l;
+  T* o = out + (size_t)t * out_stride + (size_t)h * d;
+#pragma unroll
+  for (int i = 0; i < ATT_NPL; ++i) {
+    const int e = lane + i * WAVE;
+    if (e < d) from_f32(o + e, acc[i] * inv);
+  }
+}
+
+extern "C" int kappai_paged_attention_rows(const void* q, int q_stride, const void* k_pool,
+                                           const void* v_pool, void* out, int out_stride,
+                                           const int* row_pos, const int* row_seg,
+                                           const int* block_tables, int max_blocks, int T, int H,
+                                           int G, int d, int ps, int window, float scale,
+                                           int is_bf16, hipStream_t stream) {
+  if (T <= 0) return 0;
+  if (d > MAX_HEAD_DIM || d % 8 || G < 1 || H % G || H > 65535) return (int)hipErrorInvalidValue;
+  dim3 grid(T, H);
+  if (is_bf16)
+    hipLaunchKernelGGL(paged_attention_rows_kernel<bf16_t>, grid, dim3(WAVE), 0, stream,
+                       (const bf16_t*)q, q_stride, (const bf16_t*)k_pool, (const bf16_t*)v_pool,
+                       (bf16_t*)out, out_stride, row_pos, row_seg, block_tables, max_blocks, H, G,
+                       d, ps, window, scale);
+  else
+    hipLaunchKernelGGL(paged_attention_rows_kernel<float>, grid, dim3(WAVE), 0, stream,
+                       (const float*)q, q_stride, (const float*)k_pool, (const float*)v_pool,
+                       (float*)out, out_stride, row_pos, row_seg, block_tables, max_blocks, H, G, d,
+                       ps, window, scale);
+  KAPPAI_RETURN_LAUNCH_STATUS();
+}

@@ -1,0 +1,67 @@
+// Shared device helpers for the gfx950 kernels: raw bfloat16 storage, wave (64 lanes)
+// and block reductions, and the error convention of the host launchers.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+typedef uint16_t bf16_t;  // storage of a bfloat16; arithmetic is always done in float
+
+#define WAVE 64
+
+// every launcher returns 0 or the hipError_t of its launch
+#define KAPPAI_RETURN_LAUNCH_STATUS() return (int)hipGetLastError()
+
+__device__ __forceinline__ float bf16_to_f32(bf16_t v) {
+  return __uint_as_float(((uint32_t)v) << 16);
+}
+
+// round to nearest, ties to even; NaN stays NaN
+__device__ __forceinline__ bf16_t f32_to_bf16(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (bf16_t)((u >> 16) | 0x40u);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (bf16_t)(u >> 16);
+}
+
+__device__ __forceinline__ float to_f32(float v) { return v; }
+__device__ __forceinline__ float to_f32(bf16_t v) { return bf16_to_f32(v); }
+__device__ __forceinline__ void from_f32(float* p, float v) { *p = v; }
+__device__ __forceinline__ void from_f32(bf16_t* p, float v) { *p = f32_to_bf16(v); }
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int m = WAVE / 2; m > 0; m >>= 1) v += __shfl_xor(v, m, WAVE);
+  return v;
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int m = WAVE / 2; m > 0; m >>= 1) v = fmaxf(v, __shfl_xor(v, m, WAVE));
+  return v;
+}
+
+// Sum over a block of up to 1024 threads; `red` is LDS for 16 floats.  All threads get
+// the result.  Ends with a barrier so that `red` may be used again at once.
+__device__ __forceinline__ float block_sum(float v, float* red) {
+  v = wave_sum(v);
+  const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+  const int nw = (blockDim.x + WAVE - 1) / WAVE;
+  if (lane == 0) red[wave] = v;
+  __syncthreads();
+  float t = 0.f;
+  for (int i = 0; i < nw; ++i) t += red[i];
+  __syncthreads();
+  return t;
+}
+
+__device__ __forceinline__ float block_max(float v, float* red) {
+  v = wave_max(v);
+  const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+  const int nw = (blockDim.x + WAVE - 1) / WAVE;
+  if (lane == 0) red[wave] = v;
+  __syncthreads();
+  float t = red[0];
+  for (int i = 1; i < nw; ++i) t = fmaxf(t, red[i]);
+  __syncthreads();
+  return t;
+}

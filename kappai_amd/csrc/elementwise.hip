@@ -1,0 +1,157 @@
+// Embedding rows, (residual add +) RMSNorm, SwiGLU gate, casts and row gathers.
+//
+// The residual stream is float in every run; `T` is the run's compute type (float or
+// bf16_t) in which normalised activations and GEMM outputs are stored.
+#include "common.h"
+
+// ---------------------------------------------------------------------------------------
+// out[t, :] = table[ids[t], :]  widened to float        (kappai: src/recipe/scratch.c:195-235)
+// ---------------------------------------------------------------------------------------
+template <typename TW>
+__global__ void embed_rows_kernel(const int* __restrict__ ids, const TW* __restrict__ table,
+                                  float* __restrict__ out, int D) {
+  const int t = blockIdx.x;
+  const TW* src = table + (size_t)ids[t] * D;
+  float* dst = out + (size_t)t * D;
+  for (int i = threadIdx.x; i < D; i += blockDim.x) dst[i] = to_f32(src[i]);
+}
+
+extern "C" int kappai_embed_rows(const int* ids, const void* table, int table_is_bf16, float* out,
+                                 int T, int D, hipStream_t stream) {
+  if (T <= 0) return 0;
+  const int threads = D >= 1024 ? 256 : (D >= 256 ? 128 : 64);
+  if (table_is_bf16)
+    hipLaunchKernelGGL(embed_rows_kernel<bf16_t>, dim3(T), dim3(threads), 0, stream, ids,
+                       (const bf16_t*)table, out, D);
+  else
+    hipLaunchKernelGGL(embed_rows_kernel<float>, dim3(T), dim3(threads), 0, stream, ids,
+                       (const float*)table, out, D);
+  KAPPAI_RETURN_LAUNCH_STATUS();
+}
+
+// ---------------------------------------------------------------------------------------
+// RMSNorm with the residual sum folded in:
+//   x = resid[r] (+ delta[r]);  if write_resid: resid[r] = x;
+//   out[i] = x * rsqrt(mean(x^2) + eps) * w           (src/backend/cpu/scalar/quants.c:1507-1512)
+// r = rows ? rows[i] : i.  Sum of squares and scaling in float.
+// ---------------------------------------------------------------------------------------
+template <typename T>
+__global__ void add_rmsnorm_kernel(float* __restrict__ resid, const T* __restrict__ delta,
+                                   const float* __restrict__ w, T* __restrict__ out,
+                                   const int* __restrict__ rows, int D, float eps,
+                                   int write_resid) {
+  __shared__ float red[16];
+  const int i = blockIdx.x;
+  const int r = rows ? rows[i] : i;
+  float* x = resid + (size_t)r * D;
+  const T* dl = delta ? delta + (size_t)r * D : nullptr;
+  T* o = out + (size_t)i * D;
+  float ss = 0.f;
+  for (int j = threadIdx.x; j < D; j += blockDim.x) {
+    float v = x[j];
+    if (dl) {
+      v += to_f32(dl[j]);
+      if (write_resid) x[j] = v;
+    }
+    ss += v * v;
+  }
+  ss = block_sum(ss, red);
+  const float scale = 1.0f / sqrtf(ss / (float)D + eps);
+  for (int j = threadIdx.x; j < D; j += blockDim.x) {
+    float v = x[j];
+    if (dl && !write_resid) v += to_f32(dl[j]);
+    from_f32(o + j, v * scale * w[j]);
+  }
+}
+
+extern "C" int kappai_add_rmsnorm(float* resid, const void* delta, const float* w, void* out,
+                                  const int* rows, int n_rows, int D, float eps, int write_resid,
+                                  int is_bf16, hipStream_t stream) {
+  if (n_rows <= 0) return 0;
+  const int threads = D >= 2048 ? 512 : (D >= 512 ? 256 : (D >= 128 ? 128 : 64));
+  if (is_bf16)
+    hipLaunchKernelGGL(add_rmsnorm_kernel<bf16_t>, dim3(n_rows), dim3(threads), 0, stream, resid,
+                       (const bf16_t*)delta, w, (bf16_t*)out, rows, D, eps, write_resid);
+  else
+    hipLaunchKernelGGL(add_rmsnorm_kernel<float>, dim3(n_rows), dim3(threads), 0, stream, resid,
+                       (const float*)delta, w, (float*)out, rows, D, eps, write_resid);
+  KAPPAI_RETURN_LAUNCH_STATUS();
+}
+
+// resid[r] += delta[r] without a norm (the last residual sum of a model whose output is
+// the hidden state itself)
+template <typename T>
+__global__ void add_residual_kernel(float* __restrict__ resid, const T* __restrict__ delta,
+                                    size_t n) {
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) resid[i] += to_f32(delta[i]);
+}
+
+extern "C" int kappai_add_residual(float* resid, const void* delta, long n, int is_bf16,
+                                   hipStream_t stream) {
+  if (n <= 0) return 0;
+  const int threads = 256;
+  const unsigned blocks = (unsigned)((n + threads - 1) / threads);
+  if (is_bf16)
+    hipLaunchKernelGGL(add_residual_kernel<bf16_t>, dim3(blocks), dim3(threads), 0, stream, resid,
+                       (const bf16_t*)delta, (size_t)n);
+  else
+    hipLaunchKernelGGL(add_residual_kernel<float>, dim3(blocks), dim3(threads), 0, stream, resid,
+                       (const float*)delta, (size_t)n);
+  KAPPAI_RETURN_LAUNCH_STATUS();
+}
+
+// ---------------------------------------------------------------------------------------
+// act[t, f] = silu(gu[t, f]) * gu[t, F + f],  silu(z) = z / (1 + exp(-z))
+//                                                      (src/backend/cpu/quants.h:369-371)
+// ---------------------------------------------------------------------------------------
+template <typename T>
+__global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ act, int F, size_t n) {
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const size_t t = i / F;
+  const int f = (int)(i - t * F);
+  const float g = to_f32(gu[t * 2 * F + f]);
+  const float u = to_f32(gu[t * 2 * F + F + f]);
+  from_f32(act + i, g / (1.0f + expf(-g)) * u);
+}
+
+extern "C" int kappai_swiglu(const void* gu, void* act, int T, int F, int is_bf16,
+                             hipStream_t stream) {
+  const size_t n = (size_t)T * F;
+  if (n == 0) return 0;
+  const int threads = 256;
+  const unsigned blocks = (unsigned)((n + threads - 1) / threads);
+  if (is_bf16)
+    hipLaunchKernelGGL(swiglu_kernel<bf16_t>, dim3(blocks), dim3(threads), 0, stream,
+                       (const bf16_t*)gu, (bf16_t*)act, F, n);
+  else
+    hipLaunchKernelGGL(swiglu_kernel<float>, dim3(blocks), dim3(threads), 0, stream,
+                       (const float*)gu, (float*)act, F, n);
+  KAPPAI_RETURN_LAUNCH_STATUS();
+}
+
+// ---------------------------------------------------------------------------------------
+// casts between float and bf16 (activations that meet a matrix stored in 32 bits)
+// ---------------------------------------------------------------------------------------
+template <typename TI, typename TO>
+__global__ void cast_kernel(const TI* __restrict__ in, TO* __restrict__ out, size_t n) {
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) from_f32(out + i, to_f32(in[i]));
+}
+
+extern "C" int kappai_cast(const void* in, void* out, long n, int in_is_bf16, int out_is_bf16,
+                           hipStream_t stream) {
+  if (n <= 0) return 0;
+  const int threads = 256;
+  const unsigned blocks = (unsigned)((n + threads - 1) / threads);
+  if (in_is_bf16 && !out_is_bf16)
+    hipLaunchKernelGGL((cast_kernel<bf16_t, float>), dim3(blocks), dim3(threads), 0, stream,
+                       (const bf16_t*)in, (float*)out, (size_t)n);
+  else if (!in_is_bf16 && out_is_bf16)
+    hipLaunchKernelGGL((cast_kernel<float, bf16_t>), dim3(blocks), dim3(threads), 0, stream,
+                       (const float*)in, (bf16_t*)out, (size_t)n);
+  else
+    return (int)hipErrorInvalidValue;
+  KAPPAI_RETURN_LAUNCH_STATUS();
+}

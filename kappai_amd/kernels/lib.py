@@ -1,0 +1,163 @@
+"""Building and loading the HIP libraries.
+
+Every ``csrc/<name>.hip`` becomes one shared library ``csrc/_build/<name>.so`` for gfx950,
+compiled with hipcc the first time one of its kernels is called and loaded through
+ctypes.  There is no other implementation behind these kernels: if hipcc or a library is
+missing, the call fails with an error that says so.
+"""
+from __future__ import annotations
+
+import ctypes
+import hashlib
+import os
+import shutil
+import subprocess
+import sys
+import tempfile
+import threading
+import time
+from pathlib import Path
+from typing import Dict, List
+
+CSRC = Path(__file__).resolve().parent.parent / "csrc"
+GPU_ARCH = "gfx950"
+# packed fp32 instructions are switched off for all device code of this package
+HIPCC_FLAGS = ["-O3", "-std=c++17", f"--offload-arch={GPU_ARCH}", "-shared", "-fPIC",
+               "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+               "-Wno-unused-command-line-argument", "-Wno-pass-failed"]
+LIBRARIES = ["elementwise", "gemm", "shortconv", "attention", "sampling"]
+
+
+class KernelBuildError(RuntimeError):
+    pass
+
+
+class KernelLaunchError(RuntimeError):
+    pass
+
+
+_loaded: Dict[str, ctypes.CDLL] = {}
+_lock = threading.Lock()
+
+
+def _hipcc() -> str:
+    for cand in (os.environ.get("HIPCC"), shutil.which("hipcc"), "/opt/rocm/bin/hipcc"):
+        if cand and Path(cand).exists():
+            return cand
+    raise KernelBuildError("hipcc was not found (looked at $HIPCC, PATH and /opt/rocm/bin): the "
+                           "HIP kernels of kappai_amd cannot be built, and there is no other path")
+
+
+def _source_hash(name: str) -> str:
+    h = hashlib.sha256()
+    for p in [CSRC / f"{name}.hip"] + sorted(CSRC.glob("*.h")):
+        h.update(p.name.encode())
+        h.update(p.read_bytes())
+    h.update(" ".join(HIPCC_FLAGS).encode())
+    return h.hexdigest()
+
+
+def _build_dirs() -> List[Path]:
+    dirs = [CSRC / "_build"]
+    uid = os.getuid() if hasattr(os, "getuid") else 0
+    dirs.append(Path(tempfile.gettempdir()) / f"kappai_amd_build_{uid}")
+    return dirs
+
+
+def _writable_build_dir() -> Path:
+    for d in _build_dirs():
+        try:
+            d.mkdir(parents=True, exist_ok=True)
+            probe = d / f".probe_{os.getpid()}"
+            probe.write_text("")
+            probe.unlink()
+            return d
+        except OSError:
+            continue
+    raise KernelBuildError("no writable folder for the built kernels: tried "
+                           + ", ".join(str(d) for d in _build_dirs()))
+
+
+def _find_built(name: str, want_hash: str):
+    for d in _build_dirs():
+        so, tag = d / f"{name}.so", d / f"{name}.hash"
+        if so.is_file() and tag.is_file() and tag.read_text().strip() == want_hash:
+            return so
+    return None
+
+
+def compile_library(name: str, verbose: bool = True) -> Path:
+    """Compile ``csrc/<name>.hip`` now, whether or not a built library is there."""
+    src = CSRC / f"{name}.hip"
+    if not src.is_file():
+        raise KernelBuildError(f"{src}: no such kernel source")
+    out_dir = _writable_build_dir()
+    so, tag = out_dir / f"{name}.so", out_dir / f"{name}.hash"
+    tmp = out_dir / f".{name}.{os.getpid()}.so"
+    cmd = [_hipcc(), *HIPCC_FLAGS, f"-I{CSRC}", str(src), "-o", str(tmp)]
+    if verbose:
+        print(f"[kappai_amd] compiling {src.name} for {GPU_ARCH} ...", file=sys.stderr, flush=True)
+    t0 = time.time()
+    proc = subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    while True:
+        try:
+            out, _ = proc.communicate(timeout=20)
+            break
+        except subprocess.TimeoutExpired:
+            if verbose:
+                print(f"[kappai_amd] ... still compiling {src.name} ({time.time() - t0:.0f} s)",
+                      file=sys.stderr, flush=True)
+    if proc.returncode != 0:
+        tmp.unlink(missing_ok=True)
+        raise KernelBuildError(f"hipcc failed on {src.name}:\n{out}")
+    os.replace(tmp, so)
+    tag.write_text(_source_hash(name))
+    if verbose:
+        print(f"[kappai_amd] built {so.name} in {time.time() - t0:.1f} s", file=sys.stderr,
+              flush=True)
+    return so
+
+
+def build_all(verbose: bool = True, force: bool = True) -> None:
+    """Compile every library (used by the build check); in parallel threads."""
+    errors = []
+
+    def work(n):
+        try:
+            if force or _find_built(n, _source_hash(n)) is None:
+                compile_library(n, verbose)
+        except Exception as exc:  # noqa: BLE001 - collected and raised below
+            errors.append(exc)
+
+    threads = [threading.Thread(target=work, args=(n,)) for n in LIBRARIES]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    if errors:
+        raise errors[0]
+
+
+def library(name: str) -> ctypes.CDLL:
+    """The loaded library ``name``; compiled first if no up-to-date build exists."""
+    lib = _loaded.get(name)
+    if lib is not None:
+        return lib
+    with _lock:
+        lib = _loaded.get(name)
+        if lib is not None:
+            return lib
+        so = _find_built(name, _source_hash(name))
+        if so is None:
+            so = compile_library(name)
+        try:
+            lib = ctypes.CDLL(str(so))
+        except OSError as exc:
+            raise KernelBuildError(f"cannot load {so}: {exc}") from exc
+        _loaded[name] = lib
+        return lib
+
+
+def check(status: int, what: str) -> None:
+    if status != 0:
+        raise KernelLaunchError(f"{what}: HIP error {status}")

@@ -1,0 +1,310 @@
+"""Python faces of the HIP kernels.
+
+Each function checks on the host that shapes, dtypes, strides and devices are what the
+kernel and its grid assume, then launches on torch's current HIP stream.  Tensors must
+live on the GPU; nothing here computes on the CPU.
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import Optional
+
+import torch
+
+from .lib import check, library
+
+F32, BF16, I32 = torch.float32, torch.bfloat16, torch.int32
+MAX_HEAD_DIM = 512
+MAX_GRID_Y = 65535
+
+_c_int, _c_float, _c_long, _vp = ctypes.c_int, ctypes.c_float, ctypes.c_long, ctypes.c_void_p
+
+
+def _stream() -> _vp:
+    return _vp(torch.cuda.current_stream().cuda_stream)
+
+
+def _ptr(t: Optional[torch.Tensor]) -> _vp:
+    return _vp(0 if t is None else t.data_ptr())
+
+
+def _need(cond: bool, msg: str) -> None:
+    if not cond:
+        raise ValueError(msg)
+
+
+def _gpu(name: str, t: torch.Tensor, dtype=None, contiguous=True) -> None:
+    _need(isinstance(t, torch.Tensor), f"{name}: a tensor is needed")
+    _need(t.is_cuda, f"{name}: must live on the GPU (kappai_amd has no CPU path), got {t.device}")
+    if dtype is not None:
+        dts = dtype if isinstance(dtype, (tuple, list)) else (dtype,)
+        _need(t.dtype in dts, f"{name}: dtype {t.dtype}, expected {' or '.join(map(str, dts))}")
+    if contiguous:
+        _need(t.is_contiguous(), f"{name}: must be contiguous")
+
+
+def _is_bf16(dtype) -> int:
+    _need(dtype in (F32, BF16), f"compute dtype must be float32 or bfloat16, got {dtype}")
+    return 1 if dtype == BF16 else 0
+
+
+# ---------------------------------------------------------------------------------------
+def embed_rows(ids: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
+    """float32 [T, D] rows of ``table`` ([V, D], float32 or bfloat16) at ``ids`` (int32)."""
+    _gpu("ids", ids, I32)
+    _gpu("table", table, (F32, BF16))
+    _need(ids.dim() == 1 and table.dim() == 2, "embed_rows: ids [T], table [V, D]")
+    T, D = ids.shape[0], table.shape[1]
+    out = torch.empty((T, D), dtype=F32, device=table.device)
+    check(library("elementwise").kappai_embed_rows(
+        _ptr(ids), _ptr(table), _c_int(_is_bf16(table.dtype)), _ptr(out), _c_int(T), _c_int(D),
+        _stream()), "embed_rows")
+    return out
+
+
+def add_rmsnorm(resid: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Tensor,
+                eps: float, out_dtype, rows: Optional[torch.Tensor] = None,
+                write_resid: bool = True) -> torch.Tensor:
+    """RMSNorm of ``resid (+ delta)``; with ``write_resid`` the sum replaces ``resid``.
+    ``rows`` (int32) picks the rows to normalise; the result then has one row per entry."""
+    _gpu("resid", resid, F32)
+    _gpu("weight", weight, F32)
+    _need(resid.dim() == 2 and weight.shape == (resid.shape[1],),
+          f"add_rmsnorm: resid {tuple(resid.shape)} and weight {tuple(weight.shape)} disagree")
+    isb = _is_bf16(out_dtype)
+    if delta is not None:
+        _gpu("delta", delta, out_dtype)
+        _need(delta.shape == resid.shape, "add_rmsnorm: delta must have resid's shape")
+    n = resid.shape[0]
+    if rows is not None:
+        _gpu("rows", rows, I32)
+        _need(not (write_resid and delta is not None),
+              "add_rmsnorm: a row selection cannot update the residual")
+        n = rows.shape[0]
+    D = resid.shape[1]
+    out = torch.empty((n, D), dtype=out_dtype, device=resid.device)
+    check(library("elementwise").kappai_add_rmsnorm(
+        _ptr(resid), _ptr(delta), _ptr(weight), _ptr(out), _ptr(rows), _c_int(n), _c_int(D),
+        _c_float(eps), _c_int(1 if write_resid else 0), _c_int(isb), _stream()), "add_rmsnorm")
+    return out
+
+
+def add_residual(resid: torch.Tensor, delta: torch.Tensor) -> None:
+    _gpu("resid", resid, F32)
+    _gpu("delta", delta, (F32, BF16))
+    _need(delta.shape == resid.shape, "add_residual: shapes differ")
+    check(library("elementwise").kappai_add_residual(
+        _ptr(resid), _ptr(delta), _c_long(resid.numel()), _c_int(_is_bf16(delta.dtype)),
+        _stream()), "add_residual")
+
+
+def swiglu(gate_up: torch.Tensor) -> torch.Tensor:
+    """``silu(gate_up[:, :F]) * gate_up[:, F:]`` for a fused [T, 2F] projection."""
+    _gpu("gate_up", gate_up, (F32, BF16))
+    _need(gate_up.dim() == 2 and gate_up.shape[1] % 2 == 0, "swiglu: [T, 2F] is needed")
+    T, F = gate_up.shape[0], gate_up.shape[1] // 2
+    out = torch.empty((T, F), dtype=gate_up.dtype, device=gate_up.device)
+    check(library("elementwise").kappai_swiglu(
+        _ptr(gate_up), _ptr(out), _c_int(T), _c_int(F), _c_int(_is_bf16(gate_up.dtype)),
+        _stream()), "swiglu")
+    return out
+
+
+def cast(x: torch.Tensor, dtype) -> torch.Tensor:
+    _gpu("x", x, (F32, BF16))
+    if x.dtype == dtype:
+        return x
+    out = torch.empty(x.shape, dtype=dtype, device=x.device)
+    check(library("elementwise").kappai_cast(
+        _ptr(x), _ptr(out), _c_long(x.numel()), _c_int(_is_bf16(x.dtype)),
+        _c_int(_is_bf16(dtype)), _stream()), "cast")
+    return out
+
+
+# ---------------------------------------------------------------------------------------
+def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
+           out_dtype=None, force_kernel: int = 0) -> torch.Tensor:
+    """``x [M, K] @ weight[N, K]^T (+ bias)``.  A bfloat16 matrix runs on the matrix cores
+    with float accumulation; a float32 matrix runs in true 32-bit arithmetic, whatever the
+    activations' dtype.  ``x`` may be a view with a row stride."""
+    _gpu("x", x, (F32, BF16), contiguous=False)
+    _gpu("weight", weight, (F32, BF16))
+    _need(x.dim() == 2 and weight.dim() == 2 and x.shape[1] == weight.shape[1],
+          f"linear: x {tuple(x.shape)} does not meet weight {tuple(weight.shape)}")
+    _need(x.stride(1) == 1 or x.shape[1] == 1, "linear: x must have unit stride along K")
+    M, K = x.shape
+    N = weight.shape[0]
+    out_dtype = out_dtype or x.dtype
+    if bias is not None:
+        _gpu("bias", bias, F32)
+        _need(bias.shape == (N,), f"linear: bias {tuple(bias.shape)} for N={N}")
+    if weight.dtype == F32:
+        xf = x if x.dtype == F32 else cast(x.contiguous(), F32)
+        out = torch.empty((M, N), dtype=F32, device=x.device)
+        check(library("gemm").kappai_gemm_f32(
+            _ptr(xf), _ptr(weight), _ptr(bias), _ptr(out), _c_int(M), _c_int(N), _c_int(K),
+            _c_int(xf.stride(0) if M > 1 else K), _c_int(N), _stream()), "gemm_f32")
+        return out if out_dtype == F32 else cast(out, out_dtype)
+    xb = x if x.dtype == BF16 else cast(x.contiguous(), BF16)
+    lda = xb.stride(0) if M > 1 else K
+    _need(K % 8 == 0 and lda % 8 == 0 and xb.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0,
+          f"linear: the bfloat16 kernels read 16 bytes at a time: K ({K}) and the row stride "
+          f"({lda}) must be multiples of 8 and the tensors 16-byte aligned")
+    out = torch.empty((M, N), dtype=out_dtype, device=x.device)
+    check(library("gemm").kappai_gemm_bf16(
+        _ptr(xb), _ptr(weight), _ptr(bias), _ptr(out), _c_int(M), _c_int(N), _c_int(K),
+        _c_int(lda), _c_int(N), _c_int(0 if out_dtype == BF16 else 1), _c_int(force_kernel),
+        _stream()), "gemm_bf16")
+    return out
+
+
+# ---------------------------------------------------------------------------------------
+def shortconv(proj: torch.Tensor, taps: torch.Tensor, bias: Optional[torch.Tensor],
+              state: torch.Tensor, row_seg: torch.Tensor, seg_start: torch.Tensor,
+              seg_pos0: torch.Tensor, seg_slot: torch.Tensor) -> torch.Tensor:
+    """Gated causal depthwise convolution of ``proj`` [T, 3D] = (B | C | x) per segment with
+    taps [D, L]; reads and then updates ``state`` [slots, D, L-1] (float32) of every
+    segment's slot.  Returns C * conv(B * x) as [T, D]."""
+    _gpu("proj", proj, (F32, BF16))
+    _gpu("taps", taps, F32)
+    _gpu("state", state, F32)
+    for n, t in (("row_seg", row_seg), ("seg_start", seg_start), ("seg_pos0", seg_pos0),
+                 ("seg_slot", seg_slot)):
+        _gpu(n, t, I32)
+    T = proj.shape[0]
+    D, L = taps.shape
+    S = seg_pos0.shape[0]
+    _need(proj.shape == (T, 3 * D), f"shortconv: proj {tuple(proj.shape)} for D={D}")
+    _need(L >= 2 and state.dim() == 3 and state.shape[1:] == (D, L - 1),
+          f"shortconv: state {tuple(state.shape)} for D={D}, L={L}")
+    _need(row_seg.shape[0] == T and seg_start.shape[0] == S + 1 and seg_slot.shape[0] == S,
+          "shortconv: segment tables do not fit the batch")
+    _need(T <= 2 ** 31 - 1 and S >= 1, "shortconv: batch too large or empty")
+    if bias is not None:
+        _gpu("bias", bias, F32)
+        _need(bias.shape == (D,), "shortconv: bias must be [D]")
+    out = torch.empty((T, D), dtype=proj.dtype, device=proj.device)
+    check(library("shortconv").kappai_shortconv(
+        _ptr(proj), _ptr(taps), _ptr(bias), _ptr(state), _ptr(out), _ptr(row_seg), _ptr(seg_start),
+        _ptr(seg_pos0), _ptr(seg_slot), _c_int(T), _c_int(S), _c_int(D), _c_int(L),
+        _c_int(_is_bf16(proj.dtype)), _stream()), "shortconv")
+    return out
+
+
+ROT_NONE, ROT_HALF, ROT_INTERLEAVED = 0, 1, 2
+
+
+def qk_norm_rope_store(qkv: torch.Tensor, n_heads: int, n_kv_heads: int, head_dim: int,
+                       q_norm_w: Optional[torch.Tensor], k_norm_w: Optional[torch.Tensor],
+                       eps: float, cos: Optional[torch.Tensor], sin: Optional[torch.Tensor],
+                       rot_dim: int, rot_mode: int, k_pool: Optional[torch.Tensor],
+                       v_pool: Optional[torch.Tensor], row_pos: torch.Tensor,
+                       row_seg: torch.Tensor, block_tables: torch.Tensor, page_size: int,
+                       store_kv: bool = True) -> None:
+    """In ``qkv`` [T, (H + 2G) d]: normalise every q and k head, rotate them at the row's
+    position (tables [positions, rot_dim/2]), rewrite q in place and store k and v into the
+    pools [pages, G, page_size, d] through the block tables [S, max_blocks]."""
+    H, G, d = n_heads, n_kv_heads, head_dim
+    _gpu("qkv", qkv, (F32, BF16))
+    T = qkv.shape[0]
+    width = (H + 2 * G) * d if store_kv else H * d
+    _need(qkv.dim() == 2 and qkv.shape[1] >= width, f"qk_norm_rope_store: qkv {tuple(qkv.shape)}")
+    _need(1 <= d <= MAX_HEAD_DIM, f"head_dim {d} is beyond the kernels' limit {MAX_HEAD_DIM}")
+    _need(H + 2 * G <= MAX_GRID_Y, "too many heads for one launch")
+    for n, t in (("q_norm_w", q_norm_w), ("k_norm_w", k_norm_w)):
+        if t is not None:
+            _gpu(n, t, F32)
+            _need(t.shape == (d,), f"{n} must be [head_dim]")
+    if rot_mode != ROT_NONE:
+        _gpu("cos", cos, F32)
+        _gpu("sin", sin, F32)
+        _need(rot_dim % 2 == 0 and 0 < rot_dim <= d, f"rot_dim {rot_dim} for head_dim {d}")
+        _need(cos.shape == sin.shape and cos.dim() == 2 and cos.shape[1] == rot_dim // 2,
+              "rotation tables must be [positions, rot_dim/2]")
+    _gpu("row_pos", row_pos, I32)
+    _gpu("row_seg", row_seg, I32)
+    _need(row_pos.shape[0] == T and row_seg.shape[0] == T, "row tables do not fit the batch")
+    max_blocks = 0
+    if store_kv:
+        _gpu("k_pool", k_pool, qkv.dtype)
+        _gpu("v_pool", v_pool, qkv.dtype)
+        _gpu("block_tables", block_tables, I32)
+        _need(k_pool.shape == v_pool.shape and k_pool.dim() == 4
+              and k_pool.shape[1:] == (G, page_size, d),
+              f"pools {tuple(k_pool.shape)} are not [pages, {G}, {page_size}, {d}]")
+        _need(block_tables.dim() == 2, "block_tables must be [segments, max_blocks]")
+        max_blocks = block_tables.shape[1]
+    check(library("attention").kappai_qk_norm_rope_store(
+        _ptr(qkv), _c_int(qkv.stride(0)), _ptr(q_norm_w), _ptr(k_norm_w), _c_float(eps), _ptr(cos),
+        _ptr(sin), _c_int(rot_dim if rot_mode else 0), _c_int(rot_mode), _ptr(k_pool),
+        _ptr(v_pool), _ptr(row_pos), _ptr(row_seg), _ptr(block_tables if store_kv else None),
+        _c_int(max_blocks), _c_int(T), _c_int(H), _c_int(G), _c_int(d), _c_int(page_size),
+        _c_int(1 if store_kv else 0), _c_int(_is_bf16(qkv.dtype)), _stream()),
+        "qk_norm_rope_store")
+
+
+def paged_attention(q: torch.Tensor, n_heads: int, n_kv_heads: int, head_dim: int,
+                    k_pool: torch.Tensor, v_pool: torch.Tensor, row_pos: torch.Tensor,
+                    row_seg: torch.Tensor, block_tables: torch.Tensor, page_size: int,
+                    scale: float, window: int = 0) -> torch.Tensor:
+    """Causal attention of every row over the keys of its request that are in the cache
+    (its own included; the last ``window`` of them when a window is set).  ``q`` is
+    [T, >= H d] with a row stride (the q columns of the fused projection).  Returns [T, H d]."""
+    H, G, d = n_heads, n_kv_heads, head_dim
+    _gpu("q", q, (F32, BF16), contiguous=False)
+    T = q.shape[0]
+    _need(q.dim() == 2 and q.shape[1] >= H * d and (q.stride(1) == 1),
+          f"paged_attention: q {tuple(q.shape)}")
+    _need(d % 8 == 0 and d <= MAX_HEAD_DIM,
+          f"head_dim {d}: the attention kernels take multiples of 8 up to {MAX_HEAD_DIM}")
+    _need(G >= 1 and H % G == 0 and H <= MAX_GRID_Y, f"{H} heads over {G} kv heads")
+    _gpu("k_pool", k_pool, q.dtype)
+    _gpu("v_pool", v_pool, q.dtype)
+    _need(k_pool.shape == v_pool.shape and k_pool.dim() == 4
+          and k_pool.shape[1:] == (G, page_size, d),
+          f"pools {tuple(k_pool.shape)} are not [pages, {G}, {page_size}, {d}]")
+    _gpu("row_pos", row_pos, I32)
+    _gpu("row_seg", row_seg, I32)
+    _gpu("block_tables", block_tables, I32)
+    _need(row_pos.shape[0] == T and row_seg.shape[0] == T and block_tables.dim() == 2,
+          "row tables do not fit the batch")
+    out = torch.empty((T, H * d), dtype=q.dtype, device=q.device)
+    check(library("attention").kappai_paged_attention_rows(
+        _ptr(q), _c_int(q.stride(0)), _ptr(k_pool), _ptr(v_pool), _ptr(out), _c_int(H * d),
+        _ptr(row_pos), _ptr(row_seg), _ptr(block_tables), _c_int(block_tables.shape[1]), _c_int(T),
+        _c_int(H), _c_int(G), _c_int(d), _c_int(page_size), _c_int(window or 0), _c_float(scale),
+        _c_int(_is_bf16(q.dtype)), _stream()), "paged_attention")
+    return out
+
+
+# ---------------------------------------------------------------------------------------
+def sample_rows(logits: torch.Tensor, temperature: torch.Tensor,
+                uniform: torch.Tensor) -> torch.Tensor:
+    """One token per row of ``logits`` [n, V] (float32): argmax (lowest id on ties) where the
+    row's temperature is <= 0, else an inverse-CDF draw of softmax(logits / T) at the row's
+    uniform number."""
+    _gpu("logits", logits, F32)
+    _gpu("temperature", temperature, F32)
+    _gpu("uniform", uniform, F32)
+    n, V = logits.shape
+    _need(temperature.shape == (n,) and uniform.shape == (n,), "one temperature and uniform a row")
+    out = torch.empty((n,), dtype=I32, device=logits.device)
+    check(library("sampling").kappai_sample_rows(
+        _ptr(logits), _ptr(temperature), _ptr(uniform), _ptr(out), _c_int(n), _c_int(V),
+        _stream()), "sample_rows")
+    return out
+
+
+def repeat_penalty(logits: torch.Tensor, row_start: torch.Tensor, tokens: torch.Tensor,
+                   penalty: torch.Tensor) -> None:
+    """In place: for row r and each token in ``tokens[row_start[r]:row_start[r+1]]`` divide a
+    positive logit by ``penalty[r]`` and multiply any other by it."""
+    _gpu("logits", logits, F32)
+    _gpu("row_start", row_start, I32)
+    _gpu("tokens", tokens, I32)
+    _gpu("penalty", penalty, F32)
+    n, V = logits.shape
+    _need(row_start.shape == (n + 1,) and penalty.shape == (n,), "repeat_penalty: tables per row")
+    check(library("sampling").kappai_repeat_penalty(
+        _ptr(logits), _ptr(row_start), _ptr(tokens), _ptr(penalty), _c_int(n), _c_int(V),
+        _stream()), "repeat_penalty")

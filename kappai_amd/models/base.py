@@ -1,0 +1,121 @@
+"""A model as data: blocks, and the order in which they run.
+
+``schedule`` is a list of ``LayerCall``: which block runs, and which cache it uses.  A
+block may be named more than once (then every call has a cache of its own), and a call
+may read the cache that an earlier call wrote instead of owning one (``reads_cache_of``).
+The caches are numbered by the calls that own them; the cache manager groups them by
+what they need.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Dict, List, Optional, Sequence
+
+import torch
+
+from ..config.base import ModelConfig
+from ..parts.base import Block, Hidden, Norm, PositionEncoding
+from ..parts.embedding import OutputHead, TokenEmbedding
+from ..weights.spec import TensorSpec
+
+
+@dataclass(frozen=True)
+class LayerCall:
+    layer: int                            # index into Model.layers
+    reads_cache_of: Optional[int] = None  # index into the schedule of the call whose cache is read
+
+
+class Model:
+    def __init__(self, config: ModelConfig, dtype: torch.dtype, embedding: TokenEmbedding,
+                 layers: Sequence[Block], final_norm: Norm, head: OutputHead,
+                 schedule: Optional[Sequence[LayerCall]] = None,
+                 embedding_position: Optional[PositionEncoding] = None):
+        self.config, self.dtype = config, dtype
+        self.embedding, self.layers = embedding, list(layers)
+        self.final_norm, self.head = final_norm, head
+        self.embedding_position = embedding_position
+        self.schedule: List[LayerCall] = list(schedule) if schedule is not None else [
+            LayerCall(i) for i in range(len(self.layers))]
+        self._check_schedule()
+        self.bound = False
+
+    def _check_schedule(self) -> None:
+        for ci, call in enumerate(self.schedule):
+            if not 0 <= call.layer < len(self.layers):
+                raise ValueError(f"schedule[{ci}] names layer {call.layer}; there are "
+                                 f"{len(self.layers)}")
+            src = call.reads_cache_of
+            if src is not None:
+                if not 0 <= src < ci:
+                    raise ValueError(f"schedule[{ci}] reads the cache of call {src}, which does "
+                                     f"not run before it")
+                if self.schedule[src].reads_cache_of is not None:
+                    raise ValueError(f"schedule[{ci}] reads the cache of call {src}, which owns none")
+                a = self.layers[call.layer].cache_spec()
+                b = self.layers[self.schedule[src].layer].cache_spec()
+                if a != b:
+                    raise ValueError(f"schedule[{ci}] needs {a} but call {src} keeps {b}")
+
+    # -- caches ----------------------------------------------------------------------------
+    def cache_specs(self) -> list:
+        """One entry per call of the schedule: what its own cache needs, or None when the
+        call owns none."""
+        return [None if c.reads_cache_of is not None else self.layers[c.layer].cache_spec()
+                for c in self.schedule]
+
+    def cache_id(self, call_index: int) -> int:
+        c = self.schedule[call_index]
+        return call_index if c.reads_cache_of is None else c.reads_cache_of
+
+    # -- weights ---------------------------------------------------------------------------
+    def _parts(self):
+        parts = [self.embedding, *self.layers, self.final_norm, self.head]
+        if self.embedding_position is not None:
+            parts.append(self.embedding_position)
+        return parts
+
+    def tensor_specs(self) -> List[TensorSpec]:
+        seen: Dict[str, TensorSpec] = {}
+        for p in self._parts():
+            for s in p.tensor_specs():
+                if s.name in seen and seen[s.name] != s:
+                    raise ValueError(f"tensor {s.name} is declared twice with different shapes")
+                seen[s.name] = s
+        return list(seen.values())
+
+    def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
+        for p in self._parts():
+            p.bind(tensors)
+        self.bound = True
+
+    def weight_bytes_per_step(self) -> int:
+        """Bytes of weights a step reads once: every block as often as the schedule runs it,
+        the final norm and the head."""
+        n = sum(self.layers[c.layer].weight_bytes() for c in self.schedule)
+        return n + self.final_norm.weight_bytes() + self.head.weight_bytes()
+
+    @property
+    def vocab_size(self) -> int:
+        return self.config.vocab_size
+
+    # -- the forward pass of one step ------------------------------------------------------
+    def forward(self, batch, cache) -> torch.Tensor:
+        """Run the rows of ``batch`` through every call of the schedule and return float32
+        logits [len(batch.logit_rows), vocab] (kappai: compute_forward_rows,
+        src/recipe/exec.c:704-758)."""
+        if not self.bound:
+            raise RuntimeError("the model has no weights yet: call bind() or load_model()")
+        x = self.embedding.forward(batch.tokens)
+        if self.embedding_position is not None:
+            self.embedding_position.on_embedding(x, batch)
+        h = Hidden(x, None)
+        for ci, call in enumerate(self.schedule):
+            block = self.layers[call.layer]
+            view = None
+            if block.cache_spec() is not None:
+                view = cache.view(self.cache_id(ci))
+            h = block.forward(h, batch, view, shared_cache=call.reads_cache_of is not None)
+        if batch.n_logit_rows == 0:
+            return torch.empty((0, self.vocab_size), dtype=torch.float32, device=x.device)
+        xb = self.final_norm.add_norm(h.resid, h.delta, rows=batch.logit_rows)
+        return self.head.forward(xb)

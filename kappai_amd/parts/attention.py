@@ -1,0 +1,89 @@
+"""Grouped-query attention over the paged cache.
+
+Order as kappai's attention block (src/models/lfm.c:32-51): q, k, v projections (one
+product over the stacked matrices); optional per-head RMSNorm of q and k with one shared
+weight per head size (src/backend/cpu/scalar/quants.c:1521-1531); rotation at the row's
+absolute position; k and v stored before attention so that a portion's own keys are
+visible (src/recipe/ops_basic.c:567-632); softmax(q k / sqrt(d)) v over keys 0..p, head h
+reading kv head h // (H/G) (src/backend/cpu/scalar/core.c:383-433, 623-666); output
+projection.
+"""
+from __future__ import annotations
+
+import math
+from typing import Dict, List, Optional
+
+import torch
+
+from ..cache.specs import PagedKV
+from ..kernels import ops
+from ..weights.spec import INIT_ONES, VECTOR, TensorSpec
+from .base import Mixer, PositionEncoding, register_part
+from .linear import Linear
+
+
+class GroupedQueryAttention(Mixer):
+    def __init__(self, prefix: str, width: int, num_heads: int, num_kv_heads: int, head_dim: int,
+                 dtype: torch.dtype, position: Optional[PositionEncoding] = None,
+                 qk_norm_eps: Optional[float] = None, window: Optional[int] = None,
+                 bias: bool = False, scale: Optional[float] = None, names=None):
+        n = {"q": "q_proj", "k": "k_proj", "v": "v_proj", "o": "out_proj",
+             "q_norm": "q_layernorm", "k_norm": "k_layernorm"}
+        n.update(names or {})
+        if num_heads % num_kv_heads:
+            raise ValueError(f"{num_heads} heads cannot be shared out over {num_kv_heads} kv heads")
+        self.prefix, self.width, self.dtype = prefix, width, dtype
+        self.H, self.G, self.d = num_heads, num_kv_heads, head_dim
+        self.window = window
+        self.position = position
+        self.qk_norm_eps = qk_norm_eps
+        self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(head_dim)
+        self.qkv = Linear([prefix + n["q"], prefix + n["k"], prefix + n["v"]], width,
+                          [num_heads * head_dim, num_kv_heads * head_dim, num_kv_heads * head_dim],
+                          bias=bias)
+        self.q_only = Linear([prefix + n["q"]], width, [num_heads * head_dim], bias=bias)
+        self.out = Linear([prefix + n["o"]], num_heads * head_dim, [width], bias=bias)
+        self._qn, self._kn = prefix + n["q_norm"], prefix + n["k_norm"]
+        self.q_norm_w: Optional[torch.Tensor] = None
+        self.k_norm_w: Optional[torch.Tensor] = None
+
+    def cache_spec(self):
+        return PagedKV(self.G, self.d, self.window)
+
+    def tensor_specs(self) -> List[TensorSpec]:
+        specs = self.qkv.tensor_specs() + self.out.tensor_specs()
+        if self.qk_norm_eps is not None:
+            specs.append(TensorSpec(self._qn + ".weight", (self.d,), VECTOR, INIT_ONES))
+            specs.append(TensorSpec(self._kn + ".weight", (self.d,), VECTOR, INIT_ONES))
+        return specs
+
+    def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
+        self.qkv.bind(tensors)
+        self.out.bind(tensors)
+        # the q rows of the stacked matrix, for a layer that reads another layer's keys
+        self.q_only.weight = self.qkv.weight[: self.H * self.d]
+        self.q_only.bias = None if self.qkv.bias is None else self.qkv.bias[: self.H * self.d]
+        if self.qk_norm_eps is not None:
+            self.q_norm_w = tensors[self._qn + ".weight"].to(torch.float32).contiguous()
+            self.k_norm_w = tensors[self._kn + ".weight"].to(torch.float32).contiguous()
+
+    def forward(self, x, batch, cache, shared_cache: bool = False):
+        H, G, d = self.H, self.G, self.d
+        proj = (self.q_only if shared_cache else self.qkv).forward(x)
+        rot = self.position.rotation(x.device, batch.max_position) if self.position else None
+        tables = batch.block_tables[cache.group]
+        ops.qk_norm_rope_store(
+            proj, H, G, d, self.q_norm_w, self.k_norm_w, self.qk_norm_eps or 0.0,
+            rot.cos if rot else None, rot.sin if rot else None, rot.rot_dim if rot else 0,
+            rot.mode if rot else ops.ROT_NONE, cache.k_pool, cache.v_pool, batch.row_pos,
+            batch.row_seg, tables, cache.page_size, store_kv=not shared_cache)
+        ctx = ops.paged_attention(proj, H, G, d, cache.k_pool, cache.v_pool, batch.row_pos,
+                                  batch.row_seg, tables, cache.page_size, self.scale,
+                                  window=self.window or 0)
+        return self.out.forward(ctx)
+
+    def weight_bytes(self) -> int:
+        return self.qkv.weight_bytes() + self.out.weight_bytes() + 2 * self.d * 4
+
+
+register_part("mixer", "attention", GroupedQueryAttention)

@@ -1,0 +1,124 @@
+"""The interfaces that layers are put together from, and the registries that a
+configuration chooses parts by.
+
+A model is a list of blocks and a list that says in which order they run.  A block
+arranges a norm, a token mixer, a second norm and a feed-forward; each of those is a
+part with its sizes and constants as constructor arguments.  No part knows which model
+it is in: it sees its own tensors, the rows of the step (``RowBatch``) and, if it asked
+for one, its view of the cache.
+
+Adding a part means writing a class with the interface below and registering it under a
+name; an architecture's builder then picks it layer by layer.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Callable, Dict, List, Optional
+
+import torch
+
+from ..weights.spec import TensorSpec
+
+
+class Part:
+    """Anything that owns tensors of the checkpoint."""
+
+    def tensor_specs(self) -> List[TensorSpec]:
+        """Full names, shapes and roles of the tensors this part reads from the file."""
+        return []
+
+    def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
+        """Take the loaded tensors (by full name) and lay them out for the kernels."""
+
+    def weight_bytes(self) -> int:
+        """Bytes of weights that one step reads from this part."""
+        return 0
+
+
+class Norm(Part):
+    """``add_norm`` adds ``delta`` (may be None) into the float32 residual in place and
+    returns the normalised rows in the compute dtype.  With ``rows`` only those rows are
+    normalised and the residual is left as it is."""
+
+    def add_norm(self, resid: torch.Tensor, delta: Optional[torch.Tensor],
+                 rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class PositionEncoding(Part):
+    """How positions enter the model.  ``rotation(max_position)`` gives what the attention
+    kernels rotate queries and keys with (or None); ``on_embedding`` may change the
+    embedded rows in place (absolute encodings)."""
+
+    def rotation(self, device, max_position: int):
+        return None
+
+    def on_embedding(self, x: torch.Tensor, batch) -> None:
+        return None
+
+
+class Mixer(Part):
+    """A token mixer.  ``cache_spec`` says what it needs from the cache manager (PagedKV,
+    FixedState or None); ``forward`` gets the normalised rows [T, width] in the compute
+    dtype, the step's ``RowBatch`` and its cache view, and returns [T, width]."""
+
+    def cache_spec(self):
+        return None
+
+    def forward(self, x: torch.Tensor, batch, cache, shared_cache: bool = False) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    def forward(self, x: torch.Tensor, batch) -> torch.Tensor:
+        raise NotImplementedError
+
+
+@dataclass
+class Hidden:
+    """The residual stream between blocks: ``resid`` (float32, [T, width]) and the last
+    part's output ``delta`` that has not been added yet.  The next norm adds it while it
+    normalises, so the sum is made in float32 and costs no pass of its own."""
+    resid: torch.Tensor
+    delta: Optional[torch.Tensor] = None
+
+
+class Block(Part):
+    """An arrangement of parts around the residual stream."""
+
+    mixer: Mixer
+
+    def cache_spec(self):
+        return self.mixer.cache_spec()
+
+    def forward(self, h: Hidden, batch, cache, shared_cache: bool = False) -> Hidden:
+        raise NotImplementedError
+
+
+# --------------------------------------------------------------------------------------
+# registries: name -> constructor
+# --------------------------------------------------------------------------------------
+MIXERS: Dict[str, Callable[..., Mixer]] = {}
+FEED_FORWARDS: Dict[str, Callable[..., FeedForward]] = {}
+NORMS: Dict[str, Callable[..., Norm]] = {}
+POSITION_ENCODINGS: Dict[str, Callable[..., PositionEncoding]] = {}
+BLOCKS: Dict[str, Callable[..., Block]] = {}
+
+_REGISTRIES = {"mixer": MIXERS, "feed_forward": FEED_FORWARDS, "norm": NORMS,
+               "position_encoding": POSITION_ENCODINGS, "block": BLOCKS}
+
+
+def register_part(kind: str, part_name: str, ctor: Callable) -> None:
+    if kind not in _REGISTRIES:
+        raise KeyError(f"unknown kind of part {kind!r}; known: {', '.join(_REGISTRIES)}")
+    _REGISTRIES[kind][part_name] = ctor
+
+
+def make_part(kind: str, part_name: str, /, **kwargs):
+    """Construct the part registered as ``part_name``; ``kwargs`` go to its constructor."""
+    if kind not in _REGISTRIES:
+        raise KeyError(f"unknown kind of part {kind!r}; known: {', '.join(_REGISTRIES)}")
+    reg = _REGISTRIES[kind]
+    if part_name not in reg:
+        raise KeyError(f"no {kind} named {part_name!r}; known: {', '.join(sorted(reg)) or 'none'}")
+    return reg[part_name](**kwargs)

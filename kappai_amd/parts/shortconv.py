@@ -1,0 +1,69 @@
+"""Gated short convolution (the LFM2 conv layer's mixer).
+
+kappai: src/models/lfm.c:13-19 and src/backend/cpu/common.c:2393-2431.  p = W_in x is cut
+into B, C, x in this order; bx = B*x; a causal depthwise FIR of ``kernel_size`` taps runs
+over bx, its history before the portion coming from the request's state slot
+([width, kernel_size-1] float32, oldest first); y = C * s; out = W_out y.  With ``bias`` the
+three linear maps (in_proj, the FIR, out_proj) have one each.
+"""
+from __future__ import annotations
+
+from typing import Dict, List, Optional
+
+import torch
+
+from ..cache.specs import FixedState
+from ..kernels import ops
+from ..weights.spec import INIT_NORMAL, INIT_SMALL, VECTOR, TensorSpec
+from .base import Mixer, register_part
+from .linear import Linear
+
+
+class GatedShortConv(Mixer):
+    def __init__(self, prefix: str, width: int, kernel_size: int, dtype: torch.dtype,
+                 bias: bool = False, names=None):
+        n = {"in": "in_proj", "conv": "conv", "out": "out_proj"}
+        n.update(names or {})
+        if kernel_size < 2:
+            raise ValueError(f"a short convolution needs at least 2 taps, got {kernel_size}")
+        self.prefix, self.width, self.L, self.dtype, self.has_bias = (
+            prefix, width, kernel_size, dtype, bias)
+        self.in_proj = Linear([prefix + n["in"]], width, [3 * width], bias=bias)
+        self.out_proj = Linear([prefix + n["out"]], width, [width], bias=bias)
+        self._conv = prefix + n["conv"]
+        self.taps: Optional[torch.Tensor] = None
+        self.conv_bias: Optional[torch.Tensor] = None
+
+    def cache_spec(self):
+        return FixedState((self.width, self.L - 1), "float32")
+
+    def tensor_specs(self) -> List[TensorSpec]:
+        specs = self.in_proj.tensor_specs() + self.out_proj.tensor_specs()
+        # depthwise taps in the checkpoint's layout [channels, 1, taps]
+        specs.append(TensorSpec(self._conv + ".weight", (self.width, 1, self.L), VECTOR,
+                                INIT_NORMAL))
+        if self.has_bias:
+            specs.append(TensorSpec(self._conv + ".bias", (self.width,), VECTOR, INIT_SMALL))
+        return specs
+
+    def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
+        self.in_proj.bind(tensors)
+        self.out_proj.bind(tensors)
+        self.taps = tensors[self._conv + ".weight"].to(torch.float32).reshape(
+            self.width, self.L).contiguous()
+        if self.has_bias:
+            self.conv_bias = tensors[self._conv + ".bias"].to(torch.float32).contiguous()
+
+    def forward(self, x, batch, cache, shared_cache: bool = False):
+        if shared_cache:
+            raise ValueError("a short convolution's state cannot be read by another layer")
+        proj = self.in_proj.forward(x)
+        y = ops.shortconv(proj, self.taps, self.conv_bias, cache.state, batch.row_seg,
+                          batch.seg_start, batch.seg_pos0, batch.seg_slot)
+        return self.out_proj.forward(y)
+
+    def weight_bytes(self) -> int:
+        return self.in_proj.weight_bytes() + self.out_proj.weight_bytes() + self.width * self.L * 4
+
+
+register_part("mixer", "conv", GatedShortConv)

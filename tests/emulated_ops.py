@@ -1,0 +1,191 @@
+"""A stand-in for ``kappai_amd.kernels.ops`` made of torch CPU operations, so that the
+engine's own logic (row tables, cache manager, step function, scheduler, replay) can be
+tested where there is no GPU.  It belongs to the tests; the package never imports it.
+Every function has the contract of the kernel it stands for, including the dtype in which
+results are stored."""
+from __future__ import annotations
+
+import math
+
+import numpy as np
+import torch
+
+F32, BF16 = torch.float32, torch.bfloat16
+ROT_NONE, ROT_HALF, ROT_INTERLEAVED = 0, 1, 2
+
+
+def embed_rows(ids, table):
+    return table[ids.long()].to(F32)
+
+
+def add_rmsnorm(resid, delta, weight, eps, out_dtype, rows=None, write_resid=True):
+    x = resid if delta is None else resid + delta.to(F32)
+    if delta is not None and write_resid and rows is None:
+        resid.copy_(x)
+    if rows is not None:
+        x = x[rows.long()]
+    y = x * (1.0 / torch.sqrt((x * x).mean(dim=-1, keepdim=True) + eps)) * weight
+    return y.to(out_dtype)
+
+
+def add_residual(resid, delta):
+    resid.add_(delta.to(F32))
+
+
+def swiglu(gate_up):
+    F = gate_up.shape[1] // 2
+    g, u = gate_up[:, :F].to(F32), gate_up[:, F:].to(F32)
+    return (g / (1.0 + torch.exp(-g)) * u).to(gate_up.dtype)
+
+
+def cast(x, dtype):
+    return x.to(dtype)
+
+
+def linear(x, weight, bias=None, out_dtype=None, force_kernel=0):
+    out_dtype = out_dtype or x.dtype
+    y = x.to(F32) @ weight.to(F32).T
+    if bias is not None:
+        y = y + bias
+    return y.to(out_dtype)
+
+
+def shortconv(proj, taps, bias, state, row_seg, seg_start, seg_pos0, seg_slot):
+    T = proj.shape[0]
+    D, L = taps.shape
+    H = L - 1
+    p = proj.to(F32)
+    B, C, X = p[:, :D], p[:, D:2 * D], p[:, 2 * D:]
+    bx = B * X
+    out = torch.empty((T, D), dtype=F32)
+    for s in range(seg_pos0.shape[0]):
+        t0, t1 = int(seg_start[s]), int(seg_start[s + 1])
+        slot = int(seg_slot[s])
+        hist = torch.zeros((H, D)) if int(seg_pos0[s]) == 0 else state[slot].T.clone()
+        seq = torch.cat([hist, bx[t0:t1]], dim=0)            # [H + n, D]
+        for r in range(t1 - t0):
+            acc = torch.zeros(D) if bias is None else bias.clone()
+            for k in range(L):
+                acc = acc + taps[:, k] * seq[r + k]
+            out[t0 + r] = C[t0 + r] * acc
+        state[slot] = seq[-H:].T
+    return out.to(proj.dtype)
+
+
+def qk_norm_rope_store(qkv, n_heads, n_kv_heads, head_dim, q_norm_w, k_norm_w, eps, cos, sin,
+                       rot_dim, rot_mode, k_pool, v_pool, row_pos, row_seg, block_tables,
+                       page_size, store_kv=True):
+    H, G, d = n_heads, n_kv_heads, head_dim
+    T = qkv.shape[0]
+    pos = row_pos.long()
+
+    def norm_rot(x, w):                                      # x: [T, heads, d] float32
+        if w is not None:
+            x = x * (1.0 / torch.sqrt((x * x).mean(dim=-1, keepdim=True) + eps)) * w
+        if rot_mode == ROT_NONE:
+            return x
+        half = rot_dim // 2
+        c, s = cos[pos][:, None, :], sin[pos][:, None, :]
+        y = x.clone()
+        if rot_mode == ROT_HALF:
+            a, b = x[..., :half], x[..., half:rot_dim]
+            y[..., :half] = a * c - b * s
+            y[..., half:rot_dim] = a * s + b * c
+        else:
+            a, b = x[..., 0:rot_dim:2], x[..., 1:rot_dim:2]
+            y[..., 0:rot_dim:2] = a * c - b * s
+            y[..., 1:rot_dim:2] = a * s + b * c
+        return y
+
+    q = norm_rot(qkv[:, :H * d].to(F32).reshape(T, H, d), q_norm_w)
+    qkv[:, :H * d] = q.reshape(T, H * d).to(qkv.dtype)
+    if not store_kv:
+        return
+    k = norm_rot(qkv[:, H * d:(H + G) * d].to(F32).reshape(T, G, d), k_norm_w)
+    v = qkv[:, (H + G) * d:(H + 2 * G) * d].reshape(T, G, d)
+    for t in range(T):
+        p = int(row_pos[t])
+        page = int(block_tables[int(row_seg[t]), p // page_size])
+        assert page >= 0, "a row is stored into a page that was given back"
+        k_pool[page, :, p % page_size, :] = k[t].to(k_pool.dtype)
+        v_pool[page, :, p % page_size, :] = v[t].to(v_pool.dtype)
+
+
+def paged_attention(q, n_heads, n_kv_heads, head_dim, k_pool, v_pool, row_pos, row_seg,
+                    block_tables, page_size, scale, window=0):
+    H, G, d = n_heads, n_kv_heads, head_dim
+    T = q.shape[0]
+    out = torch.empty((T, H * d), dtype=F32)
+    for t in range(T):
+        p = int(row_pos[t])
+        lo = p + 1 - window if window and p + 1 > window else 0
+        bt = block_tables[int(row_seg[t])]
+        idx = torch.arange(lo, p + 1)
+        pages = bt[(idx // page_size).long()].long()
+        assert bool((pages >= 0).all()), "attention reads a page that was given back"
+        keys = k_pool[pages, :, (idx % page_size).long(), :].to(F32)     # [n, G, d]
+        vals = v_pool[pages, :, (idx % page_size).long(), :].to(F32)
+        qt = q[t, :H * d].to(F32).reshape(H, d)
+        for h in range(H):
+            g = h // (H // G)
+            sc = (keys[:, g, :] @ qt[h]) * scale
+            a = torch.softmax(sc, dim=0)
+            out[t, h * d:(h + 1) * d] = a @ vals[:, g, :]
+    return out.to(q.dtype)
+
+
+def sample_rows(logits, temperature, uniform):
+    out = torch.empty(logits.shape[0], dtype=torch.int32)
+    for r in range(logits.shape[0]):
+        lg = logits[r].double()
+        t = float(temperature[r])
+        if not t > 0:
+            m = lg.max()
+            out[r] = int(torch.nonzero(lg == m)[0])
+            continue
+        z = (logits[r] * (1.0 / t))
+        e = torch.exp(z - z.max()).double()
+        acc = torch.cumsum(e, 0)
+        target = float(uniform[r]) * float(acc[-1])
+        i = int(torch.searchsorted(acc, torch.tensor(target, dtype=torch.float64), right=True))
+        out[r] = min(i, logits.shape[1] - 1)
+    return out
+
+
+def repeat_penalty(logits, row_start, tokens, penalty):
+    for r in range(logits.shape[0]):
+        pen = float(penalty[r])
+        if pen == 1.0:
+            continue
+        for i in range(int(row_start[r]), int(row_start[r + 1])):
+            tok = int(tokens[i])
+            if 0 <= tok < logits.shape[1]:
+                logits[r, tok] = logits[r, tok] / pen if logits[r, tok] > 0 else logits[r, tok] * pen
+
+
+ALL = ["embed_rows", "add_rmsnorm", "add_residual", "swiglu", "cast", "linear", "shortconv",
+       "qk_norm_rope_store", "paged_attention", "sample_rows", "repeat_penalty"]
+
+
+def install(monkeypatch):
+    """Replace the kernels' Python faces by these functions for one test."""
+    import sys
+
+    from kappai_amd.kernels import ops
+    me = sys.modules[__name__]
+    for name in ALL:
+        monkeypatch.setattr(ops, name, getattr(me, name))
+
+
+def make_cpu_runner(model, cache):
+    """A StepRunner whose tables stay on the host (the emulated kernels read them there)."""
+    from kappai_amd.engine.step import StepRunner
+
+    class HostTableRunner(StepRunner):
+        def __init__(self, model, cache):
+            super().__init__(model, cache, device="cpu")
+
+        def _upload(self, arrays):
+            return {k: torch.from_numpy(np.ascontiguousarray(v).copy()) for k, v in arrays.items()}
+
+    return HostTableRunner(model, cache)

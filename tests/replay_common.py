@@ -1,0 +1,76 @@
+"""Shared by the replay tests: random requests, the plain implementation's logits for
+them, and the comparison of a replay's output with those."""
+from __future__ import annotations
+
+import functools
+import json
+from pathlib import Path
+
+import numpy as np
+
+from plain import lfm2 as plain
+
+
+def make_requests(vocab: int, lengths, seed: int):
+    rng = np.random.default_rng(seed)
+    return {f"r{i}": [int(t) for t in rng.integers(0, vocab, size=n)]
+            for i, n in enumerate(lengths)}
+
+
+_plain_cache = {}
+
+
+def plain_logits(model_dir, requests, rnd=None):
+    """{id: float64 [len, vocab]} from the plain implementation (cached per folder)."""
+    key = (str(model_dir), json.dumps(requests, sort_keys=True), rnd is not None)
+    if key not in _plain_cache:
+        cfg, w = plain.read_model_dir(model_dir)
+        kw = {} if rnd is None else {"rnd": rnd}
+        _plain_cache[key] = {rid: plain.forward(cfg, w, toks, **kw)
+                             for rid, toks in requests.items()}
+    return _plain_cache[key]
+
+
+def collect(index, outputs, vocab):
+    """outputs: {step: float32 [wanted, vocab]} -> {(id, pos): logits row}."""
+    got = {}
+    for step, idx in enumerate(index):
+        if not idx:
+            continue
+        arr = outputs[step]
+        assert arr.shape == (len(idx), vocab), (step, arr.shape, len(idx))
+        for row, key in zip(arr, idx):
+            assert key not in got, f"{key} was asked for twice"
+            got[key] = row
+    return got
+
+
+def worst_error(got, ref):
+    """Largest |difference| over all wanted rows, relative to the largest |logit| of the
+    reference, and where it is: (error, (id, pos))."""
+    scale = max(float(np.abs(v).max()) for v in ref.values())
+    worst, where = 0.0, None
+    for (rid, pos), row in got.items():
+        assert np.isfinite(row).all(), f"non-finite logits at {rid} position {pos}"
+        err = float(np.abs(row.astype(np.float64) - ref[rid][pos]).max()) / scale
+        if err > worst:
+            worst, where = err, (rid, pos)
+    return worst, where
+
+
+def first_bad(got, ref, tol):
+    """The first (id, position) whose error exceeds ``tol`` (for the failure message)."""
+    scale = max(float(np.abs(v).max()) for v in ref.values())
+    for (rid, pos) in sorted(got):
+        err = float(np.abs(got[(rid, pos)].astype(np.float64) - ref[rid][pos]).max()) / scale
+        if err > tol:
+            return rid, pos, err
+    return None
+
+
+def read_outputs(out_dir, index, vocab):
+    out = {}
+    for step, idx in enumerate(index):
+        if idx:
+            out[step] = np.fromfile(Path(out_dir) / f"{step}.f32", dtype="<f4").reshape(-1, vocab)
+    return out

@@ -1,0 +1,62 @@
+"""Tiny configurations of the architecture that differ in every size and option, and
+helpers that write them as model folders with random weights."""
+from __future__ import annotations
+
+import copy
+
+from kappai_amd.config import config_from_dict
+from kappai_amd.weights import write_random_model
+
+# 4 layers conv/attention alternating, GQA 2:1, direct feed-forward width, tied head
+TINY_A = {
+    "architectures": ["Lfm2ForCausalLM"], "model_type": "lfm2",
+    "hidden_size": 64, "num_hidden_layers": 4,
+    "layer_types": ["conv", "full_attention", "conv", "full_attention"],
+    "num_attention_heads": 4, "num_key_value_heads": 2, "head_dim": 16,
+    "intermediate_size": 192, "block_auto_adjust_ff_dim": False,
+    "vocab_size": 256, "norm_eps": 1e-5, "rope_theta": 10000.0,
+    "conv_L_cache": 3, "conv_bias": False, "tie_embedding": True,
+    "max_position_embeddings": 4096,
+}
+INIT_A = dict(seed=0, std=0.02, norm_jitter=0.0)
+
+# 6 layers, attention at 0, 3, 4, one kv head for three heads, width that is no power of two,
+# auto-adjusted feed-forward width (480 -> 320), 4 taps with biases, untied head
+TINY_B = {
+    "architectures": ["Lfm2ForCausalLM"], "model_type": "lfm2",
+    "hidden_size": 96, "num_hidden_layers": 6,
+    "layer_types": ["full_attention", "conv", "conv", "full_attention", "full_attention", "conv"],
+    "num_attention_heads": 3, "num_key_value_heads": 1, "head_dim": 32,
+    "intermediate_size": 480, "block_auto_adjust_ff_dim": True, "block_multiple_of": 64,
+    "block_ffn_dim_multiplier": 1.0,
+    "vocab_size": 512, "norm_eps": 1e-6, "rope_theta": 1000000.0,
+    "conv_L_cache": 4, "conv_bias": True, "tie_embedding": False,
+    "max_position_embeddings": 8192,
+}
+INIT_B = dict(seed=1, std=0.05, norm_jitter=0.1)
+
+# 3 layers, as many kv heads as heads over two, head size 48 with heads * head size != width,
+# a vocabulary and widths that are no powers of two, 2 taps
+TINY_C = {
+    "architectures": ["Lfm2ForCausalLM"], "model_type": "lfm2",
+    "hidden_size": 120, "num_hidden_layers": 3,
+    "layer_types": ["full_attention", "conv", "full_attention"],
+    "num_attention_heads": 6, "num_key_value_heads": 3, "head_dim": 48,
+    "intermediate_size": 200, "block_auto_adjust_ff_dim": False,
+    "vocab_size": 333, "norm_eps": 1e-4, "rope_theta": 50000.0,
+    "conv_L_cache": 2, "conv_bias": False, "tie_embedding": False,
+    "max_position_embeddings": 2048,
+}
+INIT_C = dict(seed=2, std=0.04, norm_jitter=0.05)
+
+TINY = {"A": (TINY_A, INIT_A), "B": (TINY_B, INIT_B), "C": (TINY_C, INIT_C)}
+
+
+def tiny_config(name: str) -> dict:
+    return copy.deepcopy(TINY[name][0])
+
+
+def write_tiny(name: str, folder, **overrides):
+    cfg, init = TINY[name]
+    init = {**init, **overrides}
+    return write_random_model(folder, config_from_dict(copy.deepcopy(cfg)), **init)
