@@ -68,9 +68,9 @@ def _writable_build_dir() -> Path:
     for d in _build_dirs():
         try:
             d.mkdir(parents=True, exist_ok=True)
-            probe = d / f".probe_{os.getpid()}"
-            probe.write_text("")
-            probe.unlink()
+            fd, probe = tempfile.mkstemp(prefix=".probe_", dir=d)
+            os.close(fd)
+            os.unlink(probe)
             return d
         except OSError:
             continue
@@ -93,7 +93,7 @@ def compile_library(name: str, verbose: bool = True) -> Path:
         raise KernelBuildError(f"{src}: no such kernel source")
     out_dir = _writable_build_dir()
     so, tag = out_dir / f"{name}.so", out_dir / f"{name}.hash"
-    tmp = out_dir / f".{name}.{os.getpid()}.so"
+    tmp = out_dir / f".{name}.{os.getpid()}.{threading.get_ident()}.so"
     cmd = [_hipcc(), *HIPCC_FLAGS, f"-I{CSRC}", str(src), "-o", str(tmp)]
     if verbose:
         print(f"[kappai_amd] compiling {src.name} for {GPU_ARCH} ...", file=sys.stderr, flush=True)

@@ -1,0 +1,323 @@
+"""Each HIP kernel alone against a plain torch reference of the same operation (the CPU
+stand-ins of emulated_ops.py, or float64 torch), at sizes other than the engine's."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import emulated_ops as ref
+
+pytestmark = pytest.mark.gpu
+
+F32, BF16 = torch.float32, torch.bfloat16
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from kappai_amd.kernels import ops as real
+    return real
+
+
+def rand(shape, dtype, seed, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(shape, generator=g) * scale).to(dtype)
+
+
+def close(got, want, rel, what=""):
+    got, want = got.detach().cpu().double(), want.detach().cpu().double()
+    assert got.shape == want.shape, (what, got.shape, want.shape)
+    assert torch.isfinite(got).all(), what
+    scale = max(float(want.abs().max()), 1e-30)
+    err = float((got - want).abs().max()) / scale
+    assert err <= rel, f"{what}: error {err:.3g} of the largest value, allowed {rel:.3g}"
+
+
+BF16_ULP = 2.0 ** -8      # half a unit in the last place of a bfloat16 is 2^-9 of its value
+
+
+# ---------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [F32, BF16])
+def test_embed_rows(ops, dtype):
+    table = rand((1000, 200), dtype, 1)
+    ids = torch.tensor([0, 999, 5, 5, 17, 123, 998], dtype=torch.int32)
+    got = ops.embed_rows(ids.to(DEV), table.to(DEV))
+    assert got.dtype == F32
+    assert torch.equal(got.cpu(), table[ids.long()].float())
+
+
+@pytest.mark.parametrize("dtype", [F32, BF16])
+@pytest.mark.parametrize("D", [64, 96, 1000, 2048, 5000])
+def test_add_rmsnorm(ops, dtype, D):
+    T = 13
+    resid = rand((T, D), F32, 2, 3.0)
+    delta = rand((T, D), dtype, 3)
+    w = 1 + rand((D,), F32, 4, 0.2)
+    for eps in (1e-5, 1e-2):
+        r_dev = resid.to(DEV).clone()
+        got = ops.add_rmsnorm(r_dev, delta.to(DEV), w.to(DEV), eps, dtype)
+        r_ref = resid.clone()
+        want = ref.add_rmsnorm(r_ref, delta, w, eps, F32)
+        close(got.float(), want, BF16_ULP if dtype == BF16 else 2e-6, "normed")
+        close(r_dev, r_ref, 1e-7, "residual")
+    # no delta; row selection leaves the residual alone
+    rows = torch.tensor([12, 0, 5], dtype=torch.int32)
+    r_dev = resid.to(DEV).clone()
+    got = ops.add_rmsnorm(r_dev, delta.to(DEV), w.to(DEV), 1e-6, dtype, rows=rows.to(DEV),
+                          write_resid=False)
+    want = ref.add_rmsnorm(resid.clone(), delta, w, 1e-6, F32, rows=rows, write_resid=False)
+    close(got.float(), want, BF16_ULP if dtype == BF16 else 2e-6, "selected rows")
+    assert torch.equal(r_dev.cpu(), resid)
+    got = ops.add_rmsnorm(r_dev, None, w.to(DEV), 1e-6, dtype)
+    close(got.float(), ref.add_rmsnorm(resid.clone(), None, w, 1e-6, F32),
+          BF16_ULP if dtype == BF16 else 2e-6, "no delta")
+
+
+@pytest.mark.parametrize("dtype", [F32, BF16])
+def test_swiglu(ops, dtype):
+    gu = rand((9, 2 * 333), dtype, 5, 2.0)
+    got = ops.swiglu(gu.to(DEV))
+    want = ref.swiglu(gu.float())
+    close(got.float(), want, BF16_ULP if dtype == BF16 else 2e-6, "swiglu")
+    z = torch.zeros((2, 8), dtype=dtype)
+    assert float(ops.swiglu(z.to(DEV)).abs().max()) == 0.0
+
+
+# ---------------------------------------------------------------------------------------
+GEMM_SHAPES = [(1, 64, 64), (7, 100, 72), (16, 33, 136), (17, 257, 320), (64, 2048, 96),
+               (65, 96, 320), (130, 257, 136), (200, 1000, 2048), (3, 16, 8)]
+
+
+@pytest.mark.parametrize("M,N,K", GEMM_SHAPES)
+def test_linear_float32(ops, M, N, K):
+    x, w, b = rand((M, K), F32, 6), rand((N, K), F32, 7), rand((N,), F32, 8)
+    want = x.double() @ w.double().T
+    close(ops.linear(x.to(DEV), w.to(DEV)), want, 3e-6, "no bias")
+    close(ops.linear(x.to(DEV), w.to(DEV), b.to(DEV)), want + b.double(), 3e-6, "bias")
+    # a row's result does not depend on what else is in the batch
+    if M > 1:
+        one = ops.linear(x[:1].to(DEV).contiguous(), w.to(DEV))
+        assert torch.equal(one, ops.linear(x.to(DEV), w.to(DEV))[:1])
+
+
+def test_linear_float32_is_not_reduced_precision(ops):
+    """Inputs that differ only below bfloat16/tf32 precision must give different results."""
+    K = 8
+    x = torch.full((1, K), 1.0 + 2.0 ** -12, dtype=F32)
+    w = torch.full((1, K), 1.0 + 2.0 ** -12, dtype=F32)
+    got = float(ops.linear(x.to(DEV), w.to(DEV))[0, 0])
+    assert abs(got - K * (1.0 + 2.0 ** -12) ** 2) < 4e-6 and got != float(K)
+
+
+@pytest.mark.parametrize("M,N,K", GEMM_SHAPES + [(33, 130, 72), (48, 6144, 2048), (128, 128, 32)])
+@pytest.mark.parametrize("out_dtype", [F32, BF16])
+def test_linear_bfloat16(ops, M, N, K, out_dtype):
+    x, w, b = rand((M, K), BF16, 9), rand((N, K), BF16, 10), rand((N,), F32, 11)
+    want = x.double() @ w.double().T
+    tol = 2e-5 if out_dtype == F32 else BF16_ULP
+    for force in ([0, 1, 2] if M <= 64 else [0]):
+        got = ops.linear(x.to(DEV), w.to(DEV), out_dtype=out_dtype, force_kernel=force)
+        assert got.dtype == out_dtype
+        close(got.float(), want, tol, f"kernel {force}")
+        got = ops.linear(x.to(DEV), w.to(DEV), b.to(DEV), out_dtype=out_dtype, force_kernel=force)
+        close(got.float(), want + b.double(), tol, f"kernel {force} with bias")
+
+
+def test_linear_views_and_mixed_storage(ops):
+    # x as the leading columns of a wider buffer (a row stride), as attention hands q over
+    wide = rand((20, 96 + 40), BF16, 12).to(DEV)
+    w = rand((50, 96), BF16, 13)
+    got = ops.linear(wide[:, :96], w.to(DEV))
+    close(got.float(), wide[:, :96].cpu().double() @ w.double().T, BF16_ULP, "strided x")
+    # a matrix stored in 32 bits is multiplied in 32 bits, whatever the activations are
+    w32 = rand((50, 96), F32, 14)
+    xb = rand((5, 96), BF16, 15)
+    got = ops.linear(xb.to(DEV), w32.to(DEV), out_dtype=F32)
+    close(got, xb.double() @ w32.double().T, 3e-6, "float32 matrix, bfloat16 activations")
+
+
+def test_linear_refuses_what_it_cannot_do(ops):
+    with pytest.raises(ValueError, match="multiples of 8"):
+        ops.linear(rand((4, 20), BF16, 1).to(DEV), rand((8, 20), BF16, 2).to(DEV))
+    with pytest.raises(ValueError, match="GPU"):
+        ops.linear(rand((4, 16), BF16, 1), rand((8, 16), BF16, 2))
+
+
+# ---------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [F32, BF16])
+@pytest.mark.parametrize("D", [1, 3, 7, 33, 300])
+@pytest.mark.parametrize("L", [2, 3, 4])
+def test_shortconv(ops, dtype, D, L):
+    """Segments of 1, 2, 9 and 40 rows, fresh and continued, in two steps so that the state
+    written by the first is read by the second (kappai: src/test/test_hybrid.c:78-151)."""
+    slots = 6
+    taps = rand((D, L), F32, 20, 0.5)
+    bias = rand((D,), F32, 21, 0.3)
+    state0 = rand((slots, D, L - 1), F32, 22)
+    for use_bias in (False, True):
+        st_dev, st_ref = state0.to(DEV).clone(), state0.clone()
+        for step, (lens, pos0, slot) in enumerate([
+                ([1, 2, 9, 40], [0, 5, 0, 17], [3, 0, 5, 1]),
+                ([2, 1, 1, 3], [1, 7, 9, 57], [3, 0, 5, 1])]):
+            T = sum(lens)
+            proj = rand((T, 3 * D), dtype, 23 + step)
+            seg_start = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+            row_seg = np.repeat(np.arange(len(lens)), lens).astype(np.int32)
+            meta = [torch.from_numpy(a) for a in (row_seg, seg_start, np.asarray(pos0, np.int32),
+                                                  np.asarray(slot, np.int32))]
+            b = bias if use_bias else None
+            got = ops.shortconv(proj.to(DEV), taps.to(DEV), b.to(DEV) if use_bias else None,
+                                st_dev, *[m.to(DEV) for m in meta])
+            want = ref.shortconv(proj.float(), taps, b, st_ref, *meta)
+            close(got.float(), want, BF16_ULP if dtype == BF16 else 2e-6, f"step {step}")
+            used = sorted(set(slot))
+            close(st_dev[used], st_ref[used], 1e-6, f"state after step {step}")
+            untouched = [s for s in range(slots) if s not in used]
+            assert torch.equal(st_dev[untouched].cpu(), state0[untouched])
+
+
+# ---------------------------------------------------------------------------------------
+def paged_case(seed, dtype, H, G, d, ps, lens_before, lens_new, n_pages=None, shuffle=True):
+    """Requests that already hold ``lens_before`` tokens get ``lens_new`` more.  Returns
+    everything both implementations need; pools start as NaN."""
+    rng = np.random.default_rng(seed)
+    S = len(lens_new)
+    total = [a + b for a, b in zip(lens_before, lens_new)]
+    blocks = [(t + ps - 1) // ps for t in total]
+    n_pages = n_pages or sum(blocks) + 3
+    perm = rng.permutation(n_pages) if shuffle else np.arange(n_pages)
+    bt = np.full((S, max(blocks)), -1, dtype=np.int32)
+    k = 0
+    for s in range(S):
+        for b in range(blocks[s]):
+            bt[s, b] = perm[k]
+            k += 1
+    T = sum(lens_new)
+    row_seg = np.repeat(np.arange(S), lens_new).astype(np.int32)
+    row_pos = np.concatenate([np.arange(a, a + b) for a, b in zip(lens_before, lens_new)]).astype(
+        np.int32)
+    k_pool = torch.full((n_pages, G, ps, d), float("nan"), dtype=dtype)
+    v_pool = torch.full((n_pages, G, ps, d), float("nan"), dtype=dtype)
+    # history: what earlier steps would have stored
+    for s in range(S):
+        for p in range(lens_before[s]):
+            k_pool[bt[s, p // ps], :, p % ps, :] = rand((G, d), dtype, seed * 1000 + s * 100 + p)
+            v_pool[bt[s, p // ps], :, p % ps, :] = rand((G, d), dtype, seed * 2000 + s * 100 + p)
+    qkv = rand((T, (H + 2 * G) * d), dtype, seed + 5)
+    return dict(qkv=qkv, k_pool=k_pool, v_pool=v_pool, row_pos=torch.from_numpy(row_pos),
+                row_seg=torch.from_numpy(row_seg), bt=torch.from_numpy(bt), T=T)
+
+
+def rope_tables(n, rot_dim, theta=10000.0):
+    half = rot_dim // 2
+    freq = np.power(theta, -2.0 * np.arange(half) / rot_dim)
+    ang = np.arange(n)[:, None] * freq[None, :]
+    return (torch.from_numpy(np.cos(ang).astype(np.float32)),
+            torch.from_numpy(np.sin(ang).astype(np.float32)))
+
+
+ATT_CASES = [
+    # H, G, d, page, tokens held, new tokens, rot_dim, mode, norm, window
+    (4, 2, 16, 4, [0, 5, 9], [7, 1, 3], 16, 1, True, 0),
+    (3, 1, 32, 16, [0, 31, 16], [33, 1, 2], 32, 1, True, 0),
+    (6, 3, 48, 16, [100, 0], [1, 70], 48, 1, True, 0),
+    (8, 8, 64, 64, [63, 64, 200], [2, 1, 1], 64, 1, False, 0),
+    (5, 5, 128, 8, [17], [20], 64, 2, True, 0),          # partial, interleaved rotation
+    (2, 1, 256, 16, [3, 40], [5, 1], 0, 0, True, 0),      # no rotation
+    (4, 2, 64, 16, [90, 0, 45], [1, 50, 6], 64, 1, True, 24),   # window
+    (32, 8, 64, 16, [300], [1], 64, 1, True, 0),
+]
+
+
+@pytest.mark.parametrize("dtype", [F32, BF16])
+@pytest.mark.parametrize("case", ATT_CASES)
+def test_store_and_attention(ops, dtype, case):
+    H, G, d, ps, before, new, rot_dim, mode, norm, window = case
+    c = paged_case(7, dtype, H, G, d, ps, before, new)
+    qn = (1 + rand((d,), F32, 30, 0.2)) if norm else None
+    kn = (1 + rand((d,), F32, 31, 0.2)) if norm else None
+    cos, sin = rope_tables(max(a + b for a, b in zip(before, new)) + 1, rot_dim or 2)
+    dev = {k: (v.to(DEV) if torch.is_tensor(v) else v) for k, v in c.items()}
+    tol = BF16_ULP if dtype == BF16 else 3e-6
+
+    ops.qk_norm_rope_store(dev["qkv"], H, G, d, None if qn is None else qn.to(DEV),
+                           None if kn is None else kn.to(DEV), 1e-5, cos.to(DEV), sin.to(DEV),
+                           rot_dim, mode, dev["k_pool"], dev["v_pool"], dev["row_pos"],
+                           dev["row_seg"], dev["bt"], ps)
+    qkv_ref, k_ref, v_ref = c["qkv"].float(), c["k_pool"].float(), c["v_pool"].float()
+    ref.qk_norm_rope_store(qkv_ref, H, G, d, qn, kn, 1e-5, cos, sin, rot_dim, mode, k_ref, v_ref,
+                           c["row_pos"], c["row_seg"], c["bt"], ps)
+    close(dev["qkv"][:, :H * d].float(), qkv_ref[:, :H * d], tol, "q")
+    written = ~torch.isnan(k_ref)
+    assert torch.equal(written, ~torch.isnan(dev["k_pool"].cpu().float())), "other slots touched"
+    close(torch.nan_to_num(dev["k_pool"].float()), torch.nan_to_num(k_ref), tol, "k pages")
+    close(torch.nan_to_num(dev["v_pool"].float()), torch.nan_to_num(v_ref), 0.0, "v pages")
+
+    scale = 1.0 / math.sqrt(d)
+    got = ops.paged_attention(dev["qkv"], H, G, d, dev["k_pool"], dev["v_pool"], dev["row_pos"],
+                              dev["row_seg"], dev["bt"], ps, scale, window=window)
+    # reference attention over the pools the kernel itself wrote (rounded as the run stores them)
+    want = ref.paged_attention(dev["qkv"].cpu().float(), H, G, d, dev["k_pool"].cpu().float(),
+                               dev["v_pool"].cpu().float(), c["row_pos"], c["row_seg"], c["bt"],
+                               ps, scale, window=window)
+    close(got.float(), want, tol * 2, "attention")
+
+
+@pytest.mark.parametrize("dtype", [F32, BF16])
+def test_attention_finds_one_far_key(ops, dtype):
+    """Among 700 keys one is made to match the query: the output must be its value.  A kernel
+    that skips a key, a page or a tile's edge fails here, wherever the key lies."""
+    H, G, d, ps = 4, 2, 64, 16
+    n = 700
+    for far in (0, 15, 16, 63, 64, 65, 319, 640, 698, 699):
+        c = paged_case(11, dtype, H, G, d, ps, [n], [1])
+        q = torch.zeros(d)
+        q[3] = 40.0
+        c["qkv"][0, :H * d] = q.repeat(H).to(dtype)
+        c["k_pool"].zero_()
+        c["v_pool"].copy_(rand(c["v_pool"].shape, dtype, 12))
+        bt = c["bt"]
+        c["k_pool"][bt[0, far // ps], :, far % ps, 3] = 8.0
+        marker = rand((G, d), dtype, 13) + 3.0
+        c["v_pool"][bt[0, far // ps], :, far % ps, :] = marker
+        dev = {k: (v.to(DEV) if torch.is_tensor(v) else v) for k, v in c.items()}
+        # the query's own key (position n) must exist too: store zeros for it
+        dev["k_pool"][bt[0, n // ps], :, n % ps, :] = 0
+        got = ops.paged_attention(dev["qkv"], H, G, d, dev["k_pool"], dev["v_pool"], dev["row_pos"],
+                                  dev["row_seg"], dev["bt"], ps, 1.0 / math.sqrt(d))
+        want = marker.float().repeat_interleave(H // G, dim=0).reshape(1, H * d)
+        close(got.float(), want, 2 * BF16_ULP if dtype == BF16 else 1e-5, f"far key at {far}")
+
+
+# ---------------------------------------------------------------------------------------
+def test_sample_rows(ops):
+    V = 1003
+    logits = rand((6, V), F32, 40, 3.0)
+    logits[0, 17] = logits[0, 900] = 50.0          # a tie: the lowest id wins
+    logits[1, V - 1] = 60.0
+    temp = torch.tensor([0.0, 0.0, 0.8, 0.8, 2.0, 0.3])
+    u = torch.tensor([0.5, 0.5, 0.0, 0.999999, 0.37, 0.62])
+    got = ops.sample_rows(logits.to(DEV), temp.to(DEV), u.to(DEV)).cpu()
+    want = ref.sample_rows(logits, temp, u)
+    assert got.tolist() == want.tolist()
+    assert got[0] == 17 and got[1] == V - 1
+    # many draws follow the distribution
+    lg = torch.log(torch.tensor([0.5, 0.2, 0.15, 0.1, 0.03, 0.01, 0.007, 0.003])).repeat(4000, 1)
+    uu = torch.rand(4000, generator=torch.Generator().manual_seed(1))
+    draws = ops.sample_rows(lg.to(DEV).contiguous(), torch.ones(4000).to(DEV), uu.to(DEV)).cpu()
+    freq = torch.bincount(draws.long(), minlength=8).double() / 4000
+    assert abs(freq[0] - 0.5) < 0.03 and abs(freq[1] - 0.2) < 0.03
+
+
+def test_repeat_penalty(ops):
+    logits = torch.tensor([[1.0, 0.9, 0.0, -1.0], [2.0, -2.0, 0.5, 0.0]])
+    row_start = torch.tensor([0, 3, 4], dtype=torch.int32)
+    toks = torch.tensor([0, 3, 0, 1], dtype=torch.int32)
+    pen = torch.tensor([2.0, 1.5])
+    dev = logits.to(DEV).clone()
+    ops.repeat_penalty(dev, row_start.to(DEV), toks.to(DEV), pen.to(DEV))
+    want = logits.clone()
+    ref.repeat_penalty(want, row_start, toks, pen)
+    assert torch.allclose(dev.cpu(), want)
+    assert want[0].tolist() == pytest.approx([0.25, 0.9, 0.0, -2.0])

@@ -1,0 +1,144 @@
+"""Trace replay on the GPU against the plain implementation: each request alone and whole;
+most of it in one step and the last 32 tokens one by one; in portions of changing size;
+and mixed, up to four live requests with so few pages that they are used again; in true
+32-bit and in bfloat16."""
+import json
+import os
+import subprocess
+import sys
+from pathlib import Path
+
+import numpy as np
+import pytest
+import torch
+
+import schedules
+from plain import lfm2 as plain
+from replay_common import (collect, first_bad, make_requests, plain_logits, read_outputs,
+                           worst_error)
+from tiny import TINY, write_tiny
+
+pytestmark = pytest.mark.gpu
+
+ROOT = Path(__file__).resolve().parent.parent
+FP32_TOL = 2e-5     # of the largest |logit|
+# bfloat16: the engine may be off by 2.5 times what rounding the same intermediate values to
+# bfloat16 costs the plain implementation itself on the same requests
+BF16_FACTOR = 2.5
+
+LENGTHS = {"A": [70, 45, 100, 37, 83, 64], "B": [33, 97, 40, 71, 52], "C": [66, 35, 90, 41]}
+MIXED_LENGTHS = {"A": [70, 45, 100, 37, 83, 64, 29, 58, 91, 40],
+                 "B": [33, 97, 40, 71, 52, 64, 18, 85, 47],
+                 "C": [66, 35, 90, 41, 23, 77, 50, 62]}
+
+
+@pytest.fixture(scope="module")
+def model_dirs(tmp_path_factory):
+    base = tmp_path_factory.mktemp("models")
+    return {name: write_tiny(name, base / name) for name in TINY}
+
+
+_models = {}
+
+
+def gpu_model(model_dir, dtype):
+    from kappai_amd.models import load_model
+    key = (str(model_dir), dtype)
+    if key not in _models:
+        _models[key] = load_model(model_dir, dtype, "cuda:0")
+    return _models[key]
+
+
+def replay_in_process(model_dir, dtype, steps, index, max_tokens, out_dir, page_size=16):
+    from kappai_amd.engine.replay import TraceReplayer, make_replay_cache
+    from kappai_amd.engine.step import StepRunner
+    model = gpu_model(model_dir, dtype)
+    cache = make_replay_cache(model, max_tokens, page_size)
+    cache.allocate_storage(model.dtype, "cuda:0", poison=True)
+    rep = TraceReplayer(StepRunner(model, cache, "cuda:0"), out_dir)
+    outputs = {}
+    for obj in steps:
+        res = rep.run_step(obj)
+        if res is not None:
+            outputs[obj["step"]] = res
+    cache.check()
+    assert not cache.live_requests()
+    return collect(index, outputs, model.vocab_size)
+
+
+def tolerance(model_dir, requests, dtype):
+    if dtype == "float32":
+        return FP32_TOL
+    ref = plain_logits(model_dir, requests)
+    rounded = plain_logits(model_dir, requests, rnd=plain.round_bf16)
+    scale = max(float(np.abs(v).max()) for v in ref.values())
+    inherent = max(float(np.abs(rounded[r] - ref[r]).max()) for r in ref) / scale
+    return BF16_FACTOR * inherent
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("family", ["whole", "prefill_then_decode", "changing_portions", "mixed"])
+def test_schedules(tmp_path, model_dirs, name, family, dtype):
+    cfg = TINY[name][0]
+    lengths = MIXED_LENGTHS[name] if family == "mixed" else LENGTHS[name]
+    requests = make_requests(cfg["vocab_size"], lengths, seed=10)
+    steps, index, peak = getattr(schedules, family)(requests)
+    got = replay_in_process(model_dirs[name], dtype, steps, index, peak, tmp_path / "out")
+    ref = plain_logits(model_dirs[name], requests)
+    tol = tolerance(model_dirs[name], requests, dtype)
+    assert len(got) == sum(len(t) for t in requests.values())
+    err, where = worst_error(got, ref)
+    assert err < tol, (err, tol, where, first_bad(got, ref, tol))
+
+
+@pytest.mark.parametrize("page_size", [4, 64])
+def test_other_page_sizes(tmp_path, model_dirs, page_size):
+    cfg = TINY["B"][0]
+    requests = make_requests(cfg["vocab_size"], MIXED_LENGTHS["B"], seed=11)
+    steps, index, peak = schedules.mixed(requests)
+    got = replay_in_process(model_dirs["B"], "float32", steps, index, peak, tmp_path / "out",
+                            page_size=page_size)
+    ref = plain_logits(model_dirs["B"], requests)
+    err, where = worst_error(got, ref)
+    assert err < FP32_TOL, (err, where, first_bad(got, ref, FP32_TOL))
+
+
+def test_long_decoding_and_first_tokens(tmp_path, model_dirs):
+    """Two tokens of prompt, then 300 tokens one by one (the first tokens of a sequence, page
+    edges, conv history shorter than the taps), two requests side by side."""
+    cfg = TINY["B"][0]
+    requests = make_requests(cfg["vocab_size"], [302, 301], seed=12)
+    plans = {"r0": (0, [2] + [1] * 300), "r1": (0, [1] * 301)}
+    steps, index, peak = schedules.build(requests, plans)
+    for dtype in ("float32", "bfloat16"):
+        got = replay_in_process(model_dirs["B"], dtype, steps, index, peak, tmp_path / dtype)
+        ref = plain_logits(model_dirs["B"], requests)
+        tol = tolerance(model_dirs["B"], requests, dtype)
+        err, where = worst_error(got, ref)
+        assert err < tol, (dtype, err, tol, where, first_bad(got, ref, tol))
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_run_program(tmp_path, model_dirs, dtype):
+    """The program itself, as a user runs it: steps on standard input, 'done <step>' after
+    each, <step>.f32 files, exit code 0."""
+    cfg = TINY["A"][0]
+    requests = make_requests(cfg["vocab_size"], MIXED_LENGTHS["A"][:6], seed=13)
+    steps, index, peak = schedules.mixed(requests)
+    out = tmp_path / "out"
+    proc = subprocess.Popen(
+        [sys.executable, str(ROOT / "bin" / "trace_run"), "--model", str(model_dirs["A"]),
+         "--dtype", dtype, "--out", str(out), "--max-tokens", str(peak)],
+        stdin=subprocess.PIPE, stdout=subprocess.PIPE, text=True, cwd=str(tmp_path))
+    for obj in steps:
+        proc.stdin.write(json.dumps(obj) + "\n")
+        proc.stdin.flush()
+        assert proc.stdout.readline().strip() == f"done {obj['step']}"
+    proc.stdin.close()
+    assert proc.wait(timeout=120) == 0
+    got = collect(index, read_outputs(out, index, cfg["vocab_size"]), cfg["vocab_size"])
+    ref = plain_logits(model_dirs["A"], requests)
+    tol = tolerance(model_dirs["A"], requests, dtype)
+    err, where = worst_error(got, ref)
+    assert err < tol, (err, tol, where, first_bad(got, ref, tol))
