@@ -106,13 +106,21 @@ def register_architecture(name: str, config_cls: type, build_model: Callable[...
     _ARCHITECTURES[name] = Architecture(name, config_cls, build_model)
 
 
+def _load_builtin_architectures() -> None:
+    """The package's own architectures register themselves when ``kappai_amd.models`` is
+    imported; make sure that has happened before a name is looked up."""
+    from .. import models  # noqa: F401
+
+
 def known_architectures():
+    _load_builtin_architectures()
     return sorted(_ARCHITECTURES)
 
 
 def lookup_architecture(name: str) -> Architecture:
     """Unknown names are an error that lists what is known (kappai: "unrecognized
     architecture", src/arch.c:126-139)."""
+    _load_builtin_architectures()
     if name not in _ARCHITECTURES:
         raise ConfigError(
             f"unrecognized architecture '{name}'; known: {', '.join(known_architectures()) or 'none'}")

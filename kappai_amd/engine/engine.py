@@ -1,0 +1,223 @@
+"""The engine: model, cache, step function, scheduler and sampler behind one object.
+
+kappai's C API is ``engine_init / engine_run / engine_shutdown`` (src/engine.h:12-17) over a
+session that prefills in portions and then decodes token by token
+(src/context.c:995-1110, 1312-1457), measuring prefill and generation speed with a device
+synchronisation before each timestamp (:1507-1512, 1607-1615).  ``Engine`` is the same for
+token ids and many requests at once.
+"""
+from __future__ import annotations
+
+import time
+from dataclasses import dataclass, field
+from typing import Dict, List, Optional, Sequence, Union
+
+import torch
+
+from ..cache.manager import CacheManager
+from ..models import Model, load_model
+from ..sampling import RequestSampler, Sampler, SamplingParams
+from .batch import StepEntry
+from .scheduler import FAILED, FINISHED, Request, Scheduler, SchedulerConfig
+from .step import StepRunner
+
+
+@dataclass
+class EngineConfig:
+    """Engine options with kappai's names where it has them (``config``, src/config.h:15-92):
+    ``ctx_size`` is -c/--ctx-size (0: from the model)."""
+    model: Optional[str] = None          # folder with config.json and model.safetensors
+    dtype: str = "bfloat16"
+    device: str = "cuda:0"
+    ctx_size: int = 0                    # longest sequence; 0: the model's max_position_embeddings
+    page_size: int = 16
+    num_pages: int = 0                   # 0: from free memory
+    memory_fraction: float = 0.8         # share of free GPU memory for pages when num_pages = 0
+    max_batch: int = 64                  # requests live at the same time (state slots)
+    token_budget: int = 512
+    chunk: int = 512
+
+
+@dataclass
+class Metrics:
+    prefill_tokens: int = 0
+    prefill_seconds: float = 0.0
+    decode_tokens: int = 0
+    decode_seconds: float = 0.0
+    first_token_ms: float = -1.0
+    steps: int = 0
+
+    @property
+    def pp(self) -> float:
+        return self.prefill_tokens / self.prefill_seconds if self.prefill_seconds > 0 else 0.0
+
+    @property
+    def tg(self) -> float:
+        return self.decode_tokens / self.decode_seconds if self.decode_seconds > 0 else 0.0
+
+    def line(self, spec: str = "pp,tg") -> str:
+        """kappai's metrics line (src/context.c:1519-1568)."""
+        parts = []
+        for name in spec.replace(" ", ",").split(","):
+            n = name.lower()
+            if n == "pp":
+                parts.append(f"PP: {self.pp:.2f} t/s")
+            elif n == "tg":
+                parts.append(f"TG: {self.tg:.2f} t/s")
+            elif n == "ttft":
+                parts.append(f"TTFT: {self.first_token_ms:.2f} ms" if self.first_token_ms >= 0
+                             else "TTFT: --")
+        return "[ " + " | ".join(parts) + " ]" if parts else ""
+
+
+@dataclass
+class StepOutput:
+    request_id: object
+    token: Optional[int]
+    finished: bool
+    finish_reason: Optional[str] = None
+
+
+class Engine:
+    def __init__(self, config: Union[EngineConfig, str, None] = None, model: Optional[Model] = None,
+                 **overrides):
+        if isinstance(config, str):
+            config = EngineConfig(model=config)
+        config = config or EngineConfig()
+        for k, v in overrides.items():
+            if not hasattr(config, k):
+                raise TypeError(f"unknown engine option {k!r}")
+            setattr(config, k, v)
+        self.config = config
+        if not torch.cuda.is_available():
+            raise RuntimeError("kappai_amd runs on the GPU only and no GPU is visible")
+        self.device = torch.device(config.device)
+        if model is None:
+            if not config.model:
+                raise ValueError("an engine needs a model folder (-m/--model)")
+            model = load_model(config.model, config.dtype, self.device)
+        self.model = model
+        mc = model.config
+        model_ctx = getattr(mc, "max_position_embeddings", 0) or 0
+        self.ctx_size = min(config.ctx_size, model_ctx) if config.ctx_size and model_ctx else (
+            config.ctx_size or model_ctx)
+        specs = model.cache_specs()
+        probe = CacheManager(specs, config.page_size, 1, 1)
+        elem = 2 if model.dtype == torch.bfloat16 else 4
+        page_bytes = max(probe.bytes_per_token(elem) * config.page_size, 1)
+        num_pages = config.num_pages
+        if not num_pages:
+            free, _ = torch.cuda.mem_get_info(self.device)
+            num_pages = int(free * config.memory_fraction) // page_bytes
+            if self.ctx_size:      # no more than every live request at full context
+                cap = config.max_batch * ((self.ctx_size + config.page_size - 1) // config.page_size)
+                num_pages = min(num_pages, cap)
+        if num_pages < 1:
+            raise RuntimeError("not enough free GPU memory for a single cache page")
+        self.cache = CacheManager(specs, config.page_size, num_pages, config.max_batch)
+        self.cache.allocate_storage(model.dtype, self.device)
+        self.runner = StepRunner(model, self.cache, self.device)
+        eos = getattr(mc, "eos_token_id", None)
+        self.scheduler = Scheduler(
+            self.cache,
+            SchedulerConfig(config.token_budget, config.chunk, config.max_batch, self.ctx_size),
+            eos_token_ids=[] if eos is None else ([eos] if isinstance(eos, int) else eos))
+        self.sampler = Sampler()
+        self.metrics = Metrics()
+        self.requests: Dict[object, Request] = {}
+        self._next_id = 0
+        self._t_first_add: Optional[float] = None
+        self.last_logits: Optional[torch.Tensor] = None
+
+    # -- requests ----------------------------------------------------------------------------
+    def add_request(self, prompt: Sequence[int], params: Optional[SamplingParams] = None,
+                    request_id=None) -> object:
+        params = params or SamplingParams()
+        rid = self._next_id if request_id is None else request_id
+        if rid in self.requests:
+            raise ValueError(f"request id {rid!r} is in use")
+        vocab = self.model.vocab_size
+        prompt = [int(t) for t in prompt]
+        for t in prompt:
+            if not 0 <= t < vocab:
+                raise ValueError(f"token id {t} is outside the vocabulary of {vocab}")
+        req = Request(rid, prompt, params)
+        req.sampler = RequestSampler(params, seed_offset=self._next_id)
+        req.sampler.observe(prompt)
+        self._next_id += 1
+        self.requests[rid] = req
+        self.scheduler.add(req)
+        if self._t_first_add is None:
+            self._t_first_add = time.perf_counter()
+        return rid
+
+    def has_unfinished(self) -> bool:
+        return self.scheduler.has_unfinished()
+
+    # -- one engine step -----------------------------------------------------------------------
+    def step(self) -> List[StepOutput]:
+        """Schedule, run one step of the model, sample, and report every request that got a
+        token or ended."""
+        outputs: List[StepOutput] = []
+        entries, failed = self.scheduler.schedule()
+        for req in failed:
+            outputs.append(StepOutput(req.request_id, None, True, req.finish_reason))
+        if not entries:
+            return outputs
+        torch.cuda.synchronize(self.device)
+        t0 = time.perf_counter()
+        step_entries = []
+        for e in entries:
+            toks = e.request.tokens[e.request.computed:e.request.computed + e.n_tokens]
+            step_entries.append(StepEntry(e.request.cache, toks,
+                                          [e.n_tokens - 1] if e.samples else []))
+        logits = self.runner.step(step_entries)
+        self.scheduler.advance(entries)
+        sampling = [e.request for e in entries if e.samples]
+        self.last_logits = logits
+        tokens = self.sampler.sample(logits, [r.sampler for r in sampling]) if sampling else []
+        torch.cuda.synchronize(self.device)
+        dt = time.perf_counter() - t0
+        n_prefill = sum(e.n_tokens for e in entries if e.n_tokens > 1 or not e.request.output)
+        n_decode = sum(e.n_tokens for e in entries) - n_prefill
+        m = self.metrics
+        m.steps += 1
+        total = n_prefill + n_decode
+        m.prefill_tokens += n_prefill
+        m.decode_tokens += n_decode
+        m.prefill_seconds += dt * n_prefill / total
+        m.decode_seconds += dt * n_decode / total
+        if tokens and m.first_token_ms < 0 and self._t_first_add is not None:
+            m.first_token_ms = (time.perf_counter() - self._t_first_add) * 1e3
+        for req, tok in zip(sampling, tokens):
+            req.sampler.observe([tok])
+            done = self.scheduler.append_token(req, tok)
+            outputs.append(StepOutput(req.request_id, tok, done, req.finish_reason))
+        return outputs
+
+    # -- convenience ---------------------------------------------------------------------------
+    def generate(self, prompts: Sequence[Sequence[int]],
+                 params: Union[SamplingParams, Sequence[SamplingParams], None] = None,
+                 on_token=None) -> List[List[int]]:
+        """Run the prompts to completion and return the generated token ids of each.  A
+        request that fails (it cannot fit the cache) raises."""
+        if params is None or isinstance(params, SamplingParams):
+            params = [params or SamplingParams()] * len(prompts)
+        ids = [self.add_request(p, sp) for p, sp in zip(prompts, params)]
+        while self.has_unfinished():
+            for out in self.step():
+                if on_token is not None and out.token is not None:
+                    on_token(out.request_id, out.token)
+        result = []
+        for rid in ids:
+            req = self.requests.pop(rid)
+            if req.state == FAILED:
+                raise RuntimeError(f"request {rid!r} failed: {req.finish_reason}")
+            result.append(list(req.output))
+        return result
+
+    def shutdown(self) -> None:
+        for req in list(self.scheduler.running):
+            self.scheduler.finish(req, "shutdown")
+        self.scheduler.waiting.clear()
+        self.requests.clear()

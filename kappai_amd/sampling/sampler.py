@@ -1,0 +1,126 @@
+"""Choosing the next token of every row of a step's logits.
+
+kappai samples on the host for hybrid models (src/context.c:1318-1319).  Here greedy
+choice, the whole-vocabulary temperature draw and the repeat penalty run in HIP kernels
+on the logits where they lie; the draw's uniform number comes from the request's own
+random stream on the host, so that a request's tokens do not depend on what else is in
+the batch.  Rows that narrow their candidates (top-k, top-p, min-p) are copied to the
+host and drawn there in kappai's order of operations (src/sampler.c:218-332).
+"""
+from __future__ import annotations
+
+from typing import List, Optional, Sequence
+
+import numpy as np
+import torch
+
+from ..kernels import ops
+from .params import SamplingParams
+from .rng import RandomStream
+
+FILTER_CAP = 1024     # candidates kept when only top-p/min-p narrow (src/sampler.c:7, :225-231)
+
+
+class RequestSampler:
+    """Per-request sampling state: options, random stream, and the recent tokens that the
+    repeat penalty looks at (prompt included, src/context.c:1513-1514)."""
+
+    def __init__(self, params: SamplingParams, seed_offset: int = 0):
+        params.validate()
+        self.params = params
+        seed = params.seed if params.seed == 0 else params.seed + seed_offset
+        self.rng = RandomStream(seed)
+        self.recent: List[int] = []
+
+    def observe(self, tokens: Sequence[int]) -> None:
+        self.recent.extend(int(t) for t in tokens)
+        keep = max(self.params.repeat_last_n, 1)
+        if len(self.recent) > 4 * keep:
+            del self.recent[:len(self.recent) - keep]
+
+    def penalty_window(self) -> List[int]:
+        n = min(self.params.repeat_last_n, len(self.recent))
+        return self.recent[len(self.recent) - n:] if n else []
+
+
+def filtered_draw(logits: np.ndarray, p: SamplingParams, u: float) -> int:
+    """Host draw with top-k / top-p / min-p (src/sampler.c:218-332): candidates by
+    descending logit, softmax of logit/T in float32, top-p keeps the token that crosses the
+    mass, min-p is relative to the best, then an inverse-CDF draw over what is left."""
+    lg = np.asarray(logits, dtype=np.float32)
+    vocab = lg.shape[0]
+    if 0 < p.top_k < vocab:
+        keep = p.top_k
+    elif p.top_p < 1.0 or p.min_p > 0.0:
+        keep = min(vocab, FILTER_CAP)
+    else:
+        keep = vocab
+    if keep < vocab:
+        part = np.argpartition(-lg, keep - 1)[:keep]
+        order = part[np.argsort(-lg[part], kind="stable")]
+    else:
+        order = np.argsort(-lg, kind="stable")
+    vals = lg[order]
+    inv = np.float32(1.0) / np.float32(p.temperature)
+    e = np.exp(vals * inv - vals[0] * inv, dtype=np.float32)
+    cum = np.cumsum(e, dtype=np.float32)
+    total = cum[-1]
+    kept = len(e)
+    if p.top_p < 1.0:
+        over = np.nonzero(cum / total > np.float32(p.top_p))[0]
+        if over.size:
+            kept = int(over[0]) + 1
+    if p.min_p > 0.0:
+        floor = np.float32(p.min_p) * (e[0] / total)
+        ok = (e[:kept] / total) >= floor
+        n = int(np.argmin(ok)) if not ok.all() else kept
+        kept = n if n > 0 else 1
+    cum = np.cumsum(e[:kept], dtype=np.float32)
+    target = np.float32(u) * cum[-1]
+    i = int(np.searchsorted(cum, target, side="right"))
+    return int(order[min(i, kept - 1)])
+
+
+class Sampler:
+    """Samples one token for each row of ``logits`` [n, vocab] (float32, on the GPU; changed
+    in place where a repeat penalty applies)."""
+
+    def sample(self, logits: torch.Tensor, samplers: Sequence[RequestSampler]) -> List[int]:
+        n, vocab = logits.shape
+        if n != len(samplers):
+            raise ValueError(f"{n} rows of logits for {len(samplers)} requests")
+        if n == 0:
+            return []
+        dev = logits.device
+        # repeat penalty: one scatter over all rows that ask for it
+        if any(s.params.repeat_penalty != 1.0 and s.recent for s in samplers):
+            starts, toks, pens = [0], [], []
+            for s in samplers:
+                if s.params.repeat_penalty != 1.0:
+                    toks.extend(s.penalty_window())
+                starts.append(len(toks))
+                pens.append(float(s.params.repeat_penalty))
+            ops.repeat_penalty(
+                logits, torch.tensor(starts, dtype=torch.int32, device=dev),
+                torch.tensor(toks or [0], dtype=torch.int32, device=dev),
+                torch.tensor(pens, dtype=torch.float32, device=dev))
+        temps, unis, host_rows = [], [], []
+        for i, s in enumerate(samplers):
+            p = s.params
+            if p.is_greedy():
+                temps.append(0.0)
+                unis.append(0.0)
+            elif p.is_filtered(vocab):
+                temps.append(0.0)            # the kernel's choice for this row is not used
+                unis.append(0.0)
+                host_rows.append(i)
+            else:
+                temps.append(float(p.temperature))
+                unis.append(s.rng.uniform())
+        out = ops.sample_rows(logits, torch.tensor(temps, dtype=torch.float32, device=dev),
+                              torch.tensor(unis, dtype=torch.float32, device=dev)).tolist()
+        if host_rows:
+            rows = logits[torch.tensor(host_rows, device=dev)].cpu().numpy()
+            for row, i in zip(rows, host_rows):
+                out[i] = filtered_draw(row, samplers[i].params, samplers[i].rng.uniform())
+        return [int(t) for t in out]

@@ -1,0 +1,108 @@
+"""Configuration: typed reading of config.json keys, the registry, and validation."""
+import copy
+import json
+
+import pytest
+
+from kappai_amd.config import (ConfigError, Lfm2Config, adjusted_ff_dim, config_from_dict,
+                               known_architectures, load_config, lookup_architecture)
+from plain import lfm2 as plain
+from tiny import TINY_A, TINY_B, TINY_C
+
+LFM2_1_2B = {
+    "architectures": ["Lfm2ForCausalLM"], "hidden_size": 2048, "num_hidden_layers": 16,
+    "layer_types": ["conv", "conv", "full_attention", "conv", "conv", "full_attention", "conv",
+                    "conv", "full_attention", "conv", "full_attention", "conv", "full_attention",
+                    "conv", "full_attention", "conv"],
+    "num_attention_heads": 32, "num_key_value_heads": 8, "intermediate_size": 12288,
+    "block_auto_adjust_ff_dim": True, "block_multiple_of": 256, "block_ffn_dim_multiplier": 1.0,
+    "vocab_size": 65536, "norm_eps": 1e-5, "rope_theta": 1000000.0, "conv_L_cache": 3,
+    "conv_bias": False, "tie_embedding": True, "max_position_embeddings": 128000,
+}
+
+
+def test_feed_forward_width_examples():
+    # the worked examples of the architecture's published sizes
+    assert adjusted_ff_dim(12288, True, 256, 1.0) == 8192
+    assert adjusted_ff_dim(6656, True, 256, 1.0) == 4608
+    assert adjusted_ff_dim(10752, True, 256, 1.0) == 7168
+    assert adjusted_ff_dim(480, True, 64, 1.0) == 320
+    assert adjusted_ff_dim(192, False, 256, None) == 192
+    assert adjusted_ff_dim(480, True, 64, None) == 320
+    for cfg in (TINY_A, TINY_B, TINY_C, LFM2_1_2B):
+        assert config_from_dict(copy.deepcopy(cfg)).ff_dim == plain.feed_forward_width(cfg)
+
+
+def test_lfm2_1_2b_shape():
+    c = config_from_dict(copy.deepcopy(LFM2_1_2B))
+    assert isinstance(c, Lfm2Config)
+    assert c.head_dim == 64 and c.ff_dim == 8192
+    assert c.attention_layers == [2, 5, 8, 10, 12, 14] and len(c.conv_layers) == 10
+    again = config_from_dict(c.to_dict())
+    assert again == c
+
+
+def test_full_attn_idxs_form():
+    raw = copy.deepcopy(LFM2_1_2B)
+    del raw["layer_types"]
+    raw["full_attn_idxs"] = [2, 5, 8, 10, 12, 14]
+    assert config_from_dict(raw).attention_layers == [2, 5, 8, 10, 12, 14]
+
+
+def test_registry():
+    assert "Lfm2ForCausalLM" in known_architectures()
+    assert lookup_architecture("Lfm2ForCausalLM").config_cls is Lfm2Config
+    with pytest.raises(ConfigError, match="unrecognized architecture 'LlamaForCausalLM'.*Lfm2"):
+        config_from_dict({"architectures": ["LlamaForCausalLM"]})
+    with pytest.raises(ConfigError, match="architectures"):
+        config_from_dict({"hidden_size": 8})
+
+
+@pytest.mark.parametrize("key", ["hidden_size", "num_hidden_layers", "num_attention_heads",
+                                 "num_key_value_heads", "intermediate_size", "vocab_size",
+                                 "norm_eps", "rope_theta", "conv_L_cache",
+                                 "max_position_embeddings"])
+def test_required_keys(key):
+    raw = copy.deepcopy(TINY_A)
+    del raw[key]
+    with pytest.raises(ConfigError, match=key):
+        config_from_dict(raw)
+
+
+@pytest.mark.parametrize("change,match", [
+    ({"num_key_value_heads": 3}, "multiple of num_key_value_heads"),
+    ({"num_key_value_heads": 0}, "at least 1"),
+    ({"conv_L_cache": 1}, "conv_L_cache"),
+    ({"head_dim": 15}, "even"),
+    ({"head_dim": 1024}, "exceeds"),
+    ({"layer_types": ["conv"]}, "layer_types has 1 entries for 4 layers"),
+    ({"layer_types": ["conv", "mamba", "conv", "full_attention"]}, "layer_types\\[1\\]"),
+    ({"hidden_size": "64"}, "integer"),
+    ({"conv_bias": 1}, "true or false"),
+    ({"norm_eps": 0.0}, "norm_eps"),
+])
+def test_rejected(change, match):
+    raw = copy.deepcopy(TINY_A)
+    raw.update(change)
+    with pytest.raises(ConfigError, match=match):
+        config_from_dict(raw)
+
+
+def test_head_dim_defaults_to_width_over_heads():
+    raw = copy.deepcopy(TINY_A)
+    del raw["head_dim"]
+    assert config_from_dict(raw).head_dim == 16
+    raw["num_attention_heads"] = 5
+    raw["num_key_value_heads"] = 5
+    with pytest.raises(ConfigError, match="head_dim"):
+        config_from_dict(raw)
+
+
+def test_load_config_errors(tmp_path):
+    with pytest.raises(ConfigError, match="no config.json"):
+        load_config(tmp_path)
+    (tmp_path / "config.json").write_text("{not json")
+    with pytest.raises(ConfigError, match="not valid JSON"):
+        load_config(tmp_path)
+    (tmp_path / "config.json").write_text(json.dumps(TINY_B))
+    assert load_config(tmp_path).hidden_size == 96

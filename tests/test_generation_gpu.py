@@ -1,0 +1,158 @@
+"""Generation through the Python entry point and the command line, against the plain
+implementation: greedy chains, sampled chains from a fixed seed, prompts cut into portions
+and mixed with decoding, and preemption when pages run out."""
+import json
+import subprocess
+import sys
+from pathlib import Path
+
+import numpy as np
+import pytest
+
+from plain import lfm2 as P
+from plain import sampler as S
+from tiny import TINY, write_tiny
+
+pytestmark = pytest.mark.gpu
+ROOT = Path(__file__).resolve().parent.parent
+
+
+@pytest.fixture(scope="module")
+def model_dirs(tmp_path_factory):
+    base = tmp_path_factory.mktemp("models")
+    return {name: write_tiny(name, base / name) for name in TINY}
+
+
+def prompts_for(name, lengths, seed):
+    rng = np.random.default_rng(seed)
+    return [[int(t) for t in rng.integers(0, TINY[name][0]["vocab_size"], size=n)] for n in lengths]
+
+
+def plain_generate(model_dir, prompt, n, make_sampler):
+    """Token by token with the plain implementation: the whole sequence again for every
+    token, no cache."""
+    cfg, w = P.read_model_dir(model_dir)
+    sampler = make_sampler()
+    for t in prompt:
+        sampler.observe(t)
+    toks, out, rows = list(prompt), [], []
+    for _ in range(n):
+        logits = P.forward(cfg, w, toks)[-1]
+        tok = sampler.sample(logits.astype(np.float32))
+        sampler.observe(tok)
+        rows.append(logits)
+        toks.append(tok)
+        out.append(tok)
+    return out, rows
+
+
+def test_greedy_float32_tiny_a(model_dirs):
+    """Two prompts of 7 and 12 ids, then 8 greedy tokens each."""
+    from kappai_amd.engine import Engine
+    from kappai_amd.sampling import SamplingParams
+    prompts = prompts_for("A", [7, 12], seed=0)
+    eng = Engine(str(model_dirs["A"]), dtype="float32", num_pages=64, max_batch=4)
+    got = eng.generate(prompts, SamplingParams.greedy(n_predict=8))
+    for p, g in zip(prompts, got):
+        want, _ = plain_generate(model_dirs["A"], p, 8, lambda: S.PlainSampler(1, temperature=0.0))
+        assert g == want
+    assert eng.cache.num_free_pages() == 64 and eng.cache.num_free_slots == 4
+    assert eng.metrics.decode_tokens == 14 and eng.metrics.prefill_tokens == 19
+    assert eng.metrics.line("pp,tg,ttft").startswith("[ PP: ")
+
+
+def test_sampled_float32_tiny_b_in_portions(model_dirs):
+    """Three prompts of 5, 17 and 33 ids, prefilled in portions of 4 beside decoding, then 10
+    tokens each at temperature 0.8 from a fixed seed (whole-vocabulary draw)."""
+    from kappai_amd.engine import Engine
+    from kappai_amd.sampling import SamplingParams
+    prompts = prompts_for("B", [5, 17, 33], seed=1)
+    params = SamplingParams(temperature=0.8, top_k=0, top_p=1.0, min_p=0.0, seed=1234, n_predict=10)
+    eng = Engine(str(model_dirs["B"]), dtype="float32", num_pages=64, max_batch=4, chunk=4,
+                 token_budget=9)
+    got = eng.generate(prompts, params)
+    assert eng.metrics.steps > 10
+    for i, (p, g) in enumerate(zip(prompts, got)):
+        want, _ = plain_generate(model_dirs["B"], p, 10, lambda: S.PlainSampler(
+            1234 + i, temperature=0.8, top_k=0, top_p=1.0, min_p=0.0))
+        assert g == want, (i, g, want)
+
+
+def test_default_options_and_repeat_penalty(model_dirs):
+    """kappai's default options (top-k 40, top-p 0.9, min-p 0.1) and a repeat penalty."""
+    from kappai_amd.engine import Engine
+    from kappai_amd.sampling import SamplingParams
+    prompts = prompts_for("C", [9, 21], seed=2)
+    params = SamplingParams(seed=77, n_predict=12, repeat_penalty=1.3, repeat_last_n=8)
+    eng = Engine(str(model_dirs["C"]), dtype="float32", num_pages=32, max_batch=2)
+    got = eng.generate(prompts, params)
+    for i, (p, g) in enumerate(zip(prompts, got)):
+        want, _ = plain_generate(model_dirs["C"], p, 12, lambda: S.PlainSampler(
+            77 + i, repeat_penalty=1.3, repeat_last_n=8))
+        assert g == want, (i, g, want)
+
+
+def test_greedy_bfloat16_follows_the_plain_logits(model_dirs):
+    """In bfloat16 the chain may leave the plain one at a near tie; every token the engine
+    picks must be (nearly) the best under the plain logits for the engine's own prefix."""
+    from kappai_amd.engine import Engine
+    from kappai_amd.sampling import SamplingParams
+    prompts = prompts_for("B", [11, 30], seed=3)
+    eng = Engine(str(model_dirs["B"]), dtype="bfloat16", num_pages=64, max_batch=4, chunk=7)
+    got = eng.generate(prompts, SamplingParams.greedy(n_predict=12))
+    cfg, w = P.read_model_dir(model_dirs["B"])
+    for p, g in zip(prompts, got):
+        assert len(g) == 12
+        logits = P.forward(cfg, w, p + g)
+        for j, tok in enumerate(g):
+            row = logits[len(p) - 1 + j]
+            assert row[tok] >= row.max() - 0.03 * np.abs(row).max(), (j, tok, int(row.argmax()))
+
+
+def test_preemption_gives_the_same_tokens(model_dirs):
+    """With so few pages that requests are preempted and computed again, greedy output is what
+    it is with plenty of pages."""
+    from kappai_amd.engine import Engine
+    from kappai_amd.sampling import SamplingParams
+    prompts = prompts_for("A", [30, 25, 28, 9], seed=4)
+    params = SamplingParams.greedy(n_predict=20)
+    roomy = Engine(str(model_dirs["A"]), dtype="float32", num_pages=64, max_batch=4)
+    want = roomy.generate(prompts, params)
+    tight = Engine(str(model_dirs["A"]), dtype="float32", num_pages=8, page_size=16, max_batch=4,
+                   token_budget=40)
+    got = tight.generate(prompts, params)
+    assert tight.scheduler.preempted_total > 0
+    assert got == want
+    assert tight.cache.num_free_pages() == 8
+    too_long = Engine(str(model_dirs["A"]), dtype="float32", num_pages=2, max_batch=2)
+    with pytest.raises(RuntimeError, match="context exceeds cache"):
+        too_long.generate([list(range(40))], params)
+
+
+def test_command_line(model_dirs, tmp_path):
+    prompt = prompts_for("A", [7], seed=5)[0]
+    want, _ = plain_generate(model_dirs["A"], prompt, 6, lambda: S.PlainSampler(1, temperature=0.0))
+    out = subprocess.run(
+        [sys.executable, "-m", "kappai_amd", "-m", str(model_dirs["A"]), "--dtype", "float32",
+         "-p", ",".join(map(str, prompt)), "-n", "6", "-t", "0", "--metrics", "pp,tg,ttft",
+         "--num-pages", "16", "--dump-logits", str(tmp_path / "lg.f32")],
+        cwd=str(ROOT), capture_output=True, text=True, timeout=300)
+    assert out.returncode == 0, out.stderr
+    assert [int(t) for t in out.stdout.split()] == want
+    assert "[ PP: " in out.stderr and "TG: " in out.stderr and "TTFT: " in out.stderr
+    assert (tmp_path / "lg.f32").stat().st_size == 6 * 256 * 4
+    # random-weights mode from a config.json
+    cfgp = tmp_path / "cfg.json"
+    cfgp.write_text(json.dumps(TINY["C"][0]))
+    out = subprocess.run(
+        [sys.executable, str(ROOT / "bin" / "kappai-cli"), "--random-weights", str(cfgp),
+         "--weight-seed", "3", "-n", "4", "-s", "5", "--num-pages", "16", "1 2 3"],
+        cwd=str(tmp_path), capture_output=True, text=True, timeout=300)
+    assert out.returncode == 0, out.stderr
+    assert len(out.stdout.split()) == 4
+
+
+def test_smoke_entry():
+    sys.path.insert(0, str(ROOT))
+    import __graft_entry__
+    __graft_entry__.smoke()

@@ -1,0 +1,283 @@
+"""Each part alone, built with sizes of its own and bound to random tensors, against the
+plain implementation's function for it; and a toy mixer with state of its own, defined
+here, registered, built into a toy architecture and stepped without a change to the
+framework's files."""
+import copy
+import math
+from dataclasses import dataclass
+from typing import Dict, List
+
+import numpy as np
+import pytest
+import torch
+
+from plain import lfm2 as P
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+F32, BF16 = torch.float32, torch.bfloat16
+
+
+def bind_random(part, seed, dtype, std=0.1, jitter=0.1):
+    from kappai_amd.weights import random_tensors, stored_to_runtime
+    t = random_tensors(part.tensor_specs(), seed, std=std, norm_jitter=jitter)
+    part.bind({k: stored_to_runtime(v, dtype).to(DEV) for k, v in t.items()})
+    return {k: v.double().numpy() for k, v in t.items()}
+
+
+def one_segment_batch(cm, n, rid="r", first=True, rc=None):
+    """A RowBatch for ``n`` more tokens of one request."""
+    from kappai_amd.engine import StepEntry, StepRunner
+    rc = rc or cm.open(rid)
+    cm.extend(rc, n)
+    runner = StepRunner.__new__(StepRunner)
+    runner.model = type("M", (), {"vocab_size": 10 ** 9})()
+    runner.cache, runner.device, runner._staging, runner._staged = cm, torch.device(DEV), None, None
+    batch = runner.make_batch([StepEntry(rc, [0] * n, [])])
+    return rc, batch
+
+
+def rel_err(got, want):
+    got = got.detach().float().cpu().double().numpy()
+    return float(np.abs(got - want).max() / max(np.abs(want).max(), 1e-30))
+
+
+@pytest.mark.parametrize("dtype,tol", [(F32, 1e-5), (BF16, 2e-2)])
+def test_attention_part(dtype, tol):
+    from kappai_amd.cache import CacheManager
+    from kappai_amd.parts import GroupedQueryAttention, RotaryEncoding
+    W, H, G, d, T = 80, 5, 1, 48, 37
+    part = GroupedQueryAttention("a.", W, H, G, d, dtype, position=RotaryEncoding(d, 12345.0),
+                                 qk_norm_eps=1e-4)
+    w = bind_random(part, 1, dtype)
+    cm = CacheManager([part.cache_spec()], 8, 16, 1)
+    cm.allocate_storage(dtype, DEV, poison=True)
+    x = torch.randn(T, W, generator=torch.Generator().manual_seed(2)).to(dtype)
+    # in two portions, so that the second reads the first's keys from the cache
+    rc, b1 = one_segment_batch(cm, 20)
+    y1 = part.forward(x[:20].to(DEV), b1, cm.view(0))
+    cm.commit(rc, 20)
+    _, b2 = one_segment_batch(cm, T - 20, rc=rc)
+    y2 = part.forward(x[20:].to(DEV), b2, cm.view(0))
+    lw = {n: w[f"a.{n}.weight"] for n in ("q_proj", "k_proj", "v_proj", "out_proj", "q_layernorm",
+                                          "k_layernorm")}
+    cfg = {"num_attention_heads": H, "num_key_value_heads": G, "head_dim": d, "hidden_size": W,
+           "norm_eps": 1e-4, "rope_theta": 12345.0}
+    want = P.gqa_attention_mixer(x.double().numpy(), lw, cfg, np.arange(T))
+    assert rel_err(torch.cat([y1, y2]), want) < tol
+
+
+@pytest.mark.parametrize("dtype,tol", [(F32, 1e-5), (BF16, 2e-2)])
+@pytest.mark.parametrize("bias", [False, True])
+def test_short_conv_part(dtype, tol, bias):
+    from kappai_amd.cache import CacheManager
+    from kappai_amd.parts import GatedShortConv
+    W, L, T = 40, 5, 23
+    part = GatedShortConv("c.", W, L, dtype, bias=bias)
+    w = bind_random(part, 3, dtype, std=0.3)
+    cm = CacheManager([part.cache_spec()], 8, 1, 2)
+    cm.allocate_storage(dtype, DEV, poison=True)
+    x = torch.randn(T, W, generator=torch.Generator().manual_seed(4)).to(dtype)
+    rc, outs, done = None, [], 0
+    for n in (2, 1, 3, 1, 9, 7):                   # portions shorter than the taps' history too
+        rc, b = one_segment_batch(cm, n, rc=rc)
+        outs.append(part.forward(x[done:done + n].to(DEV), b, cm.view(0)))
+        cm.commit(rc, n)
+        done += n
+    lw = {"in_proj": w["c.in_proj.weight"], "out_proj": w["c.out_proj.weight"],
+          "conv": w["c.conv.weight"].reshape(W, L)}
+    if bias:
+        lw.update(in_proj_bias=w["c.in_proj.bias"], conv_bias=w["c.conv.bias"],
+                  out_proj_bias=w["c.out_proj.bias"])
+    want = P.short_conv_mixer(x.double().numpy(), lw, {"hidden_size": W})
+    assert rel_err(torch.cat(outs), want) < tol
+
+
+@pytest.mark.parametrize("dtype,tol", [(F32, 1e-5), (BF16, 2e-2)])
+def test_feed_forward_norm_and_block(dtype, tol):
+    from kappai_amd.cache import CacheManager
+    from kappai_amd.parts import GatedShortConv, Hidden, PreNormBlock, RMSNorm, SwiGLU
+    W, Fh, T = 56, 104, 9
+    ffn = SwiGLU("f.", W, Fh, dtype)
+    w = bind_random(ffn, 5, dtype, std=0.2)
+    x = torch.randn(T, W, generator=torch.Generator().manual_seed(6)).to(dtype)
+    lw = {n: w[f"f.{n}.weight"] for n in ("w1", "w2", "w3")}
+    assert rel_err(ffn.forward(x.to(DEV), None), P.swiglu_feed_forward(x.double().numpy(), lw)) < tol
+
+    norm = RMSNorm("n", W, 1e-3, dtype)
+    wn = bind_random(norm, 7, dtype)
+    resid = torch.randn(T, W, generator=torch.Generator().manual_seed(8)) * 2
+    r = resid.to(DEV).clone()
+    got = norm.add_norm(r, x.to(DEV))
+    total = resid.double().numpy() + x.double().numpy()
+    assert rel_err(got, P.rmsnorm(total, wn["n.weight"], 1e-3)) < max(tol, 1e-6) / 2
+    assert rel_err(r, total) < 1e-6                       # the sum is kept in float32
+
+    block = PreNormBlock(RMSNorm("b.n1", W, 1e-5, dtype), GatedShortConv("b.c.", W, 3, dtype),
+                         RMSNorm("b.n2", W, 1e-5, dtype), SwiGLU("b.f.", W, Fh, dtype))
+    wb = bind_random(block, 9, dtype, std=0.2)
+    cm = CacheManager([block.cache_spec()], 8, 1, 1)
+    cm.allocate_storage(dtype, DEV)
+    rc, b = one_segment_batch(cm, T)
+    h = block.forward(Hidden(resid.to(DEV).clone(), None), b, cm.view(0))
+    xr = resid.double().numpy()
+    lwc = {"in_proj": wb["b.c.in_proj.weight"], "out_proj": wb["b.c.out_proj.weight"],
+           "conv": wb["b.c.conv.weight"].reshape(W, 3)}
+    xr = xr + P.short_conv_mixer(P.rmsnorm(xr, wb["b.n1.weight"], 1e-5), lwc, {"hidden_size": W})
+    assert rel_err(h.resid, xr) < tol                      # the first sum is in; the second pending
+    lwf = {n: wb[f"b.f.{n}.weight"] for n in ("w1", "w2", "w3")}
+    assert rel_err(h.delta, P.swiglu_feed_forward(P.rmsnorm(xr, wb["b.n2.weight"], 1e-5), lwf)) < tol
+
+
+def test_rotary_tables():
+    from kappai_amd.parts import RotaryEncoding
+    r = RotaryEncoding(64, 1e6).rotation(DEV, 5000)
+    assert r.cos.shape[0] > 5000 and r.cos.shape[1] == 32
+    ang = P.rope_angles(np.arange(r.cos.shape[0]), 64, 1e6)
+    assert np.abs(r.cos.cpu().double().numpy() - np.cos(ang)).max() < 1e-7
+    assert np.abs(r.sin.cpu().double().numpy() - np.sin(ang)).max() < 1e-7
+
+
+# ---------------------------------------------------------------------------------------------
+# a toy architecture made in the test
+# ---------------------------------------------------------------------------------------------
+def test_toy_mixer_with_its_own_state_and_a_shared_cache():
+    """A mixer whose state is the running sum of its inputs (and a count), registered under a
+    name; a toy architecture that uses it beside attention, runs one block twice and lets a
+    later attention call read the keys of an earlier one.  Everything goes through the
+    framework's registries, builder, weights mode, cache manager and step function."""
+    import tempfile
+
+    from kappai_amd.cache import FixedState
+    from kappai_amd.config import ModelConfig, config_from_dict, register_architecture
+    from kappai_amd.engine import StepEntry, StepRunner
+    from kappai_amd.engine.replay import make_replay_cache
+    from kappai_amd.models import LayerCall, Model, load_model
+    from kappai_amd.parts import (Linear, Mixer, OutputHead, TokenEmbedding, make_part,
+                                  register_part)
+    from kappai_amd.weights import write_random_model
+
+    class RunningMean(Mixer):
+        """out_t = W * mean(x_0..x_t): state [width + 1] = (sum, count), float32."""
+
+        def __init__(self, prefix, width, dtype):
+            self.width, self.dtype = width, dtype
+            self.proj = Linear([prefix + "proj"], width, [width])
+
+        def cache_spec(self):
+            return FixedState((self.width + 1,), "float32")
+
+        def tensor_specs(self):
+            return self.proj.tensor_specs()
+
+        def bind(self, tensors):
+            self.proj.bind(tensors)
+
+        def forward(self, x, batch, cache, shared_cache=False):
+            out = torch.empty_like(x)
+            starts = batch.host["seg_start"]
+            for s in range(batch.n_segments):
+                t0, t1 = int(starts[s]), int(starts[s + 1])
+                slot = int(batch.host["seg_slot"][s])
+                st = cache.state[slot]
+                if int(batch.host["seg_pos0"][s]) == 0:      # a fresh request has no history
+                    st.zero_()
+                sums = st[:-1] + torch.cumsum(x[t0:t1].float(), dim=0)
+                counts = st[-1] + torch.arange(1, t1 - t0 + 1, device=x.device)
+                out[t0:t1] = (sums / counts[:, None]).to(x.dtype)
+                st[:-1] = sums[-1]
+                st[-1] = counts[-1]
+            return self.proj.forward(out)
+
+    register_part("mixer", "running_mean", RunningMean)
+
+    @dataclass
+    class ToyConfig(ModelConfig):
+        width: int = 0
+        vocab_size: int = 0
+        heads: int = 0
+        head_dim: int = 0
+        ff: int = 0
+        eps: float = 1e-5
+        max_position_embeddings: int = 512
+
+        @classmethod
+        def from_dict(cls, raw):
+            return cls(architecture="ToyForCausalLM", **{k: raw[k] for k in
+                       ("width", "vocab_size", "heads", "head_dim", "ff", "eps")})
+
+        def to_dict(self):
+            return {"architectures": ["ToyForCausalLM"], "width": self.width,
+                    "vocab_size": self.vocab_size, "heads": self.heads, "head_dim": self.head_dim,
+                    "ff": self.ff, "eps": self.eps}
+
+    def build_toy(cfg, dtype):
+        def block(i, mixer):
+            p = f"blocks.{i}."
+            return make_part("block", "pre_norm",
+                             mixer_norm=make_part("norm", "rmsnorm", name=p + "n1", width=cfg.width,
+                                                  eps=cfg.eps, dtype=dtype),
+                             mixer=mixer,
+                             ffn_norm=make_part("norm", "rmsnorm", name=p + "n2", width=cfg.width,
+                                                eps=cfg.eps, dtype=dtype),
+                             feed_forward=make_part("feed_forward", "swiglu", prefix=p + "ff.",
+                                                    width=cfg.width, hidden=cfg.ff, dtype=dtype))
+        rot = make_part("position_encoding", "rotary", head_dim=cfg.head_dim, theta=100.0,
+                        rot_dim=cfg.head_dim // 2, pairing="interleaved")
+
+        def attn(i):
+            return make_part("mixer", "attention", prefix=f"blocks.{i}.att.", width=cfg.width,
+                             num_heads=cfg.heads, num_kv_heads=cfg.heads, head_dim=cfg.head_dim,
+                             dtype=dtype, position=rot, qk_norm_eps=None)
+        layers = [block(0, make_part("mixer", "running_mean", prefix="blocks.0.mix.",
+                                     width=cfg.width, dtype=dtype)),
+                  block(1, attn(1)), block(2, attn(2))]
+        emb = TokenEmbedding("emb", cfg.vocab_size, cfg.width)
+        # block 0 runs twice (two states), block 2 reads the keys that block 1 stored
+        schedule = [LayerCall(0), LayerCall(1), LayerCall(0), LayerCall(2, reads_cache_of=1)]
+        return Model(cfg, dtype, emb, layers,
+                     make_part("norm", "rmsnorm", name="final", width=cfg.width, eps=cfg.eps,
+                               dtype=dtype),
+                     OutputHead("head", cfg.vocab_size, cfg.width, tied_to=None), schedule=schedule)
+
+    register_architecture("ToyForCausalLM", ToyConfig, build_toy)
+    cfg = config_from_dict({"architectures": ["ToyForCausalLM"], "width": 40, "vocab_size": 99,
+                            "heads": 2, "head_dim": 32, "ff": 72, "eps": 1e-5})
+    with tempfile.TemporaryDirectory() as tmp:
+        write_random_model(tmp, cfg, seed=3, std=0.2)
+        model = load_model(tmp, "float32", DEV)
+    specs = model.cache_specs()
+    assert specs[3] is None and specs[0] == specs[2] and specs[1].num_kv_heads == 2
+    toks = [int(t) for t in np.random.default_rng(0).integers(0, 99, size=45)]
+
+    def run(portions):
+        cache = make_replay_cache(model, 128)
+        cache.allocate_storage(model.dtype, DEV, poison=True)
+        runner = StepRunner(model, cache, DEV)
+        rc, done, rows = cache.open("t"), 0, []
+        other = cache.open("other")                       # a second request beside it
+        for n in portions:
+            entries = [StepEntry(rc, toks[done:done + n], list(range(n)))]
+            if done % 2 == 0:
+                entries.insert(0, StepEntry(other, [5, 6], [1]))
+            lg = runner.step(entries)
+            rows.append(lg[-n:].cpu())
+            done += n
+        return torch.cat(rows)
+
+    whole = run([45])
+    assert torch.isfinite(whole).all() and float(whole.abs().max()) > 0.1
+    cut = run([7, 1, 2, 16, 3, 2, 14])
+    assert float((cut - whole).abs().max()) < 2e-5 * float(whole.abs().max())
+    # the toy mixer does what it says: with the other parts' outputs zeroed the first block's
+    # residual gets W * running mean
+    mix = model.layers[0].mixer
+    from kappai_amd.cache import CacheManager
+    cm = CacheManager([mix.cache_spec()], 8, 1, 1)
+    cm.allocate_storage(F32, DEV)
+    x = torch.randn(9, 40, generator=torch.Generator().manual_seed(1))
+    rc, b = one_segment_batch(cm, 9)
+    got = mix.forward(x.to(DEV), b, cm.view(0))
+    means = torch.cumsum(x, 0) / torch.arange(1, 10)[:, None]
+    want = means.double() @ mix.proj.weight.cpu().double().T
+    assert float((got.cpu().double() - want).abs().max()) < 1e-5
