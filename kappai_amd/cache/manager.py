@@ -183,14 +183,16 @@ class CacheManager:
 
     # -- device storage -------------------------------------------------------------------
     def allocate_storage(self, dtype: torch.dtype, device, poison: bool = False) -> None:
-        """Create the pools [pages, kv_heads, page_size, head_dim] and the slot arrays.
-        ``poison`` fills the pools with NaN so that a read of a key nobody wrote shows."""
+        """Create the key pools [pages, kv_heads, page_size, head_dim], the value pools (stored
+        transposed: [pages, kv_heads, head_dim, page_size]) and the slot arrays.  ``poison``
+        fills the pools with NaN so that a read of a key nobody wrote shows."""
         self.device, self.dtype = device, dtype
         for g in self.paged_groups:
-            shape = (max(g.allocator.num_pages, 1), g.spec.num_kv_heads, self.page_size,
-                     g.spec.head_dim)
+            n = max(g.allocator.num_pages, 1)
+            kshape = (n, g.spec.num_kv_heads, self.page_size, g.spec.head_dim)
+            vshape = (n, g.spec.num_kv_heads, g.spec.head_dim, self.page_size)
             for cid in g.cache_ids:
-                for pools in (g.k_pools, g.v_pools):
+                for pools, shape in ((g.k_pools, kshape), (g.v_pools, vshape)):
                     t = torch.empty(shape, dtype=dtype, device=device)
                     t.fill_(float("nan")) if poison else t.zero_()
                     pools[cid] = t

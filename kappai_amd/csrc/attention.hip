@@ -9,8 +9,9 @@
 //                       lo..pos of the row's request, read through its block table
 //                       (src/backend/cpu/scalar/core.c:383-433, 623-666), online softmax in float.
 //
-// Pools are [page][kv_head][page_size][head_dim]; token p of a request lives in page
-// block_table[p / page_size] at offset p % page_size.
+// The key pool is [page][kv_head][page_size][head_dim]; the value pool is stored transposed,
+// [page][kv_head][head_dim][page_size], which is what the matrix-core kernels want.  Token p of
+// a request lives in page block_table[p / page_size] at offset p % page_size.
 #include "common.h"
 
 #define MAX_HEAD_DIM 512
@@ -32,12 +33,13 @@ __global__ __launch_bounds__(64) void qk_norm_rope_store_kernel(
   if (slot >= H) {
     const int g = (slot - H) % G;
     const int* bt = block_tables + (size_t)row_seg[t] * max_blocks;
-    const size_t row = ((size_t)bt[pos / ps] * G + g) * ps + pos % ps;
-    dst = (slot < H + G ? k_pool : v_pool) + row * d;
-  }
-  if (slot >= H + G) {  // v: plain copy into its page
-    for (int e = lane; e < d; e += WAVE) dst[e] = src[e];
-    return;
+    const size_t pg = (size_t)bt[pos / ps] * G + g;
+    if (slot >= H + G) {  // v: copied into its page, transposed
+      T* vdst = v_pool + pg * d * ps + pos % ps;
+      for (int e = lane; e < d; e += WAVE) vdst[(size_t)e * ps] = src[e];
+      return;
+    }
+    dst = k_pool + (pg * ps + pos % ps) * d;
   }
   const float* nw = slot < H ? q_norm_w : k_norm_w;
   float ss = 0.f;
@@ -149,9 +151,9 @@ __global__ __launch_bounds__(64) void paged_attention_rows_kernel(
     float s = -INFINITY;
     unsigned long long voff = 0;
     if (valid) {
-      const size_t row = ((size_t)bt[tk / ps] * G + g) * ps + tk % ps;
-      s = dot_row(qs, k_pool + row * d, d) * scale;
-      voff = (unsigned long long)row * d;
+      const size_t pg = (size_t)bt[tk / ps] * G + g;
+      s = dot_row(qs, k_pool + (pg * ps + tk % ps) * d, d) * scale;
+      voff = (unsigned long long)(pg * d * ps + tk % ps);
     }
     const float m_new = fmaxf(m, wave_max(s));
     const float p = valid ? expf(s - m_new) : 0.f;
@@ -168,7 +170,7 @@ __global__ __launch_bounds__(64) void paged_attention_rows_kernel(
 #pragma unroll
       for (int i = 0; i < ATT_NPL; ++i) {
         const int e = lane + i * WAVE;
-        if (e < d) acc[i] = fmaf(pk, to_f32(vr[e]), acc[i]);
+        if (e < d) acc[i] = fmaf(pk, to_f32(vr[(size_t)e * ps]), acc[i]);
       }
     }
     m = m_new;

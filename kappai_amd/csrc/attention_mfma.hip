@@ -1,0 +1,364 @@
+// bfloat16 attention over the paged cache on the matrix cores, for one head size
+// (HEAD_DIM, a multiple of 16, set when the file is compiled).
+//
+// Both kernels keep "one query per lane column".  For a tile of keys they compute
+//     S^T = K Q^T        A = K rows (a key per lane row, 8 consecutive d per lane)
+//                        B = Q     (a query per lane column)
+//     O^T += V^T P^T     A = V^T   (a d index per lane row, 8 key slots per lane)
+//                        B = P^T   (the lane's own values of S^T, no data movement)
+// so that a lane holds, for ITS query, scores of several keys and later outputs of several d
+// indices: the running maximum, the running sum and the rescaling are per lane, in float.
+// The value pool is stored transposed, [page][kv_head][head_dim][page_size], which makes the
+// 8 key slots of the A operand two 8-byte loads.  page_size must be a multiple of 16.
+//
+//   attn_prefill   v_mfma_f32_32x32x16_bf16; one wave per (tile of 32 rows of a segment, head)
+//   attn_decode    v_mfma_f32_16x16x32_bf16; one wave per (row, kv head, split of the keys): the
+//                  query heads that share the kv head are the columns; partial results are
+//                  merged by attn_merge.
+// Formulas: softmax(q.k/sqrt(d)) v over keys lo..pos (kappai: src/backend/cpu/scalar/core.c:383-433,
+// 623-666), online softmax as in its flash form (:386-413).
+#include "common.h"
+
+#ifndef HEAD_DIM
+#error "compile with -DHEAD_DIM=<multiple of 16>"
+#endif
+static_assert(HEAD_DIM % 16 == 0 && HEAD_DIM >= 16 && HEAD_DIM <= 256, "unsupported head size");
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+typedef __attribute__((ext_vector_type(4))) float f32x4_t;
+typedef __attribute__((ext_vector_type(16))) float f32x16_t;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4_t;
+typedef __attribute__((ext_vector_type(2))) uint32_t u32x2_t;
+
+__device__ __forceinline__ bf16x8_t as_frag(u32x4_t v) { return __builtin_bit_cast(bf16x8_t, v); }
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
+  return (uint32_t)f32_to_bf16(lo) | ((uint32_t)f32_to_bf16(hi) << 16);
+}
+// keep the j-th of four bf16 values only if keep bit j is set
+__device__ __forceinline__ u32x2_t mask4(u32x2_t v, int keep) {
+  const uint32_t m0 = ((keep & 1) ? 0x0000ffffu : 0u) | ((keep & 2) ? 0xffff0000u : 0u);
+  const uint32_t m1 = ((keep & 4) ? 0x0000ffffu : 0u) | ((keep & 8) ? 0xffff0000u : 0u);
+  return (u32x2_t){v.x & m0, v.y & m1};
+}
+
+#define LOG2E 1.4426950408889634f
+
+// four key slots of V^T for d index `dd`, keys key0..key0+3 (one 16-key group: one page);
+// keys outside [lo, hi] read as zero
+__device__ __forceinline__ u32x2_t load_vt4(const bf16_t* __restrict__ vt_pool,
+                                            const int* __restrict__ bt, int G, int g, int ps,
+                                            int dd, int key0, int lo, int hi) {
+  u32x2_t z = {0u, 0u};
+  if (dd >= HEAD_DIM || key0 > hi || key0 + 3 < lo) return z;
+  const int page = bt[key0 / ps];
+  if (page < 0) return z;
+  const bf16_t* p = vt_pool + (((size_t)page * G + g) * HEAD_DIM + dd) * ps + key0 % ps;
+  u32x2_t v = *reinterpret_cast<const u32x2_t*>(p);
+  int keep = 0;
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+    if (key0 + i >= lo && key0 + i <= hi) keep |= 1 << i;
+  return keep == 15 ? v : mask4(v, keep);
+}
+
+// eight consecutive d of key `key` starting at d0; zero outside [lo, hi] or beyond the head
+__device__ __forceinline__ u32x4_t load_k8(const bf16_t* __restrict__ k_pool,
+                                           const int* __restrict__ bt, int G, int g, int ps,
+                                           int key, int d0, int lo, int hi) {
+  u32x4_t z = {0u, 0u, 0u, 0u};
+  if (d0 >= HEAD_DIM || key < lo || key > hi) return z;
+  const int page = bt[key / ps];
+  if (page < 0) return z;
+  return *reinterpret_cast<const u32x4_t*>(
+      k_pool + (((size_t)page * G + g) * ps + key % ps) * HEAD_DIM + d0);
+}
+
+// ---------------------------------------------------------------------------------------
+// prefill: q_tiles[tile] = (segment, first row, rows <= 32, unused)
+// ---------------------------------------------------------------------------------------
+#define P_KS (HEAD_DIM / 16)            // k-steps of S^T over d
+#define P_MT ((HEAD_DIM + 31) / 32)     // row tiles of O^T over d
+
+__global__ __launch_bounds__(64) void attn_prefill_kernel(
+    const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ k_pool,
+    const bf16_t* __restrict__ vt_pool, bf16_t* __restrict__ out, int out_stride,
+    const int* __restrict__ q_tiles, const int* __restrict__ row_pos,
+    const int* __restrict__ block_tables, int max_blocks, int H, int G, int ps, int window,
+    float scale) {
+  const int tile = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const int seg = q_tiles[4 * tile], r0 = q_tiles[4 * tile + 1], nr = q_tiles[4 * tile + 2];
+  const int g = h / (H / G);
+  const int col = lane % 32, hh = lane / 32;
+  const int* bt = block_tables + (size_t)seg * max_blocks;
+  const int pos_first = row_pos[r0], pos_last = pos_first + nr - 1;
+  const bool row_ok = col < nr;
+  const int my_pos = row_ok ? pos_first + col : -1;
+  const int my_lo = (window > 0 && my_pos + 1 > window) ? my_pos + 1 - window : 0;
+  const int lo_tile = (window > 0 && pos_first + 1 > window) ? pos_first + 1 - window : 0;
+
+  bf16x8_t qf[P_KS];
+  {
+    const bf16_t* qr = q + (size_t)(r0 + (row_ok ? col : 0)) * q_stride + (size_t)h * HEAD_DIM;
+#pragma unroll
+    for (int ks = 0; ks < P_KS; ++ks) {
+      u32x4_t v = {0u, 0u, 0u, 0u};
+      if (row_ok) v = *reinterpret_cast<const u32x4_t*>(qr + 16 * ks + 8 * hh);
+      qf[ks] = as_frag(v);
+    }
+  }
+  f32x16_t o[P_MT];
+#pragma unroll
+  for (int mt = 0; mt < P_MT; ++mt)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) o[mt][v] = 0.f;
+  float m_run = -INFINITY, l_run = 0.f;
+  const float sc = scale * LOG2E;
+
+  for (int kb = (lo_tile / 32) * 32; kb <= pos_last; kb += 32) {
+    // ---- S^T tile: 32 keys x 32 queries -------------------------------------------------
+    f32x16_t s;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) s[v] = 0.f;
+    const int my_key = kb + col;
+#pragma unroll
+    for (int ks = 0; ks < P_KS; ++ks) {
+      const bf16x8_t kf =
+          as_frag(load_k8(k_pool, bt, G, g, ps, my_key, 16 * ks + 8 * hh, lo_tile, pos_last));
+      s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[ks], s, 0, 0, 0);
+    }
+    // lane holds, for query `col`, keys kb + 8*(v/4) + 4*hh + v%4
+    float mloc = -INFINITY;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const int key = kb + 8 * (v / 4) + 4 * hh + v % 4;
+      const bool ok = key <= my_pos && key >= my_lo;
+      s[v] = ok ? s[v] * sc : -INFINITY;
+      mloc = fmaxf(mloc, s[v]);
+    }
+    mloc = fmaxf(mloc, __shfl_xor(mloc, 32, WAVE));
+    const float m_new = fmaxf(m_run, mloc);
+    const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+    const float corr = exp2f(m_run - m_safe);
+    float lsum = 0.f;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      s[v] = exp2f(s[v] - m_safe);
+      lsum += s[v];
+    }
+    lsum += __shfl_xor(lsum, 32, WAVE);
+    l_run = l_run * corr + lsum;
+    m_run = m_new;
+#pragma unroll
+    for (int mt = 0; mt < P_MT; ++mt)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) o[mt][v] *= corr;
+    // ---- O^T += V^T P^T, two k-steps of 16 keys ---------------------------------------
+#pragma unroll
+    for (int st = 0; st < 2; ++st) {
+      const u32x4_t pw = {pack_bf16(s[8 * st + 0], s[8 * st + 1]),
+                          pack_bf16(s[8 * st + 2], s[8 * st + 3]),
+                          pack_bf16(s[8 * st + 4], s[8 * st + 5]),
+                          pack_bf16(s[8 * st + 6], s[8 * st + 7])};
+      const bf16x8_t pf = as_frag(pw);
+      const int key0 = kb + 16 * st + 4 * hh;
+#pragma unroll
+      for (int mt = 0; mt < P_MT; ++mt) {
+        const int dd = 32 * mt + col;
+        const u32x2_t a = load_vt4(vt_pool, bt, G, g, ps, dd, key0, lo_tile, pos_last);
+        const u32x2_t b = load_vt4(vt_pool, bt, G, g, ps, dd, key0 + 8, lo_tile, pos_last);
+        const u32x4_t vw = {a.x, a.y, b.x, b.y};
+        o[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_frag(vw), pf, o[mt], 0, 0, 0);
+      }
+    }
+  }
+  if (!row_ok) return;
+  const float inv = l_run > 0.f ? 1.0f / l_run : 0.f;
+  bf16_t* orow = out + (size_t)(r0 + col) * out_stride + (size_t)h * HEAD_DIM;
+#pragma unroll
+  for (int mt = 0; mt < P_MT; ++mt)
+#pragma unroll
+    for (int v4 = 0; v4 < 4; ++v4) {
+      const int dd = 32 * mt + 8 * v4 + 4 * hh;     // four consecutive d: v = 4*v4 .. 4*v4+3
+      if (dd < HEAD_DIM) {
+        u32x2_t w = {pack_bf16(o[mt][4 * v4] * inv, o[mt][4 * v4 + 1] * inv),
+                     pack_bf16(o[mt][4 * v4 + 2] * inv, o[mt][4 * v4 + 3] * inv)};
+        *reinterpret_cast<u32x2_t*>(orow + dd) = w;
+      }
+    }
+}
+
+// ---------------------------------------------------------------------------------------
+// decode: one row a request; columns are the query heads of one kv head (at most 16)
+// ---------------------------------------------------------------------------------------
+#define D_KS ((HEAD_DIM + 31) / 32)     // k-steps of S^T over d (32 each)
+#define D_MT (HEAD_DIM / 16)            // row tiles of O^T over d
+
+__global__ __launch_bounds__(64) void attn_decode_kernel(
+    const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ k_pool,
+    const bf16_t* __restrict__ vt_pool, float* __restrict__ part_o, float* __restrict__ part_ml,
+    const int* __restrict__ row_pos, const int* __restrict__ row_seg,
+    const int* __restrict__ block_tables, int max_blocks, int H, int G, int ps, int window,
+    float scale, int keys_per_split, int n_splits) {
+  const int t = blockIdx.x, g = blockIdx.y, split = blockIdx.z, lane = threadIdx.x;
+  const int rep = H / G;
+  const int col = lane % 16, kg = lane / 16;
+  const int pos = row_pos[t];
+  const int* bt = block_tables + (size_t)row_seg[t] * max_blocks;
+  const int lo = (window > 0 && pos + 1 > window) ? pos + 1 - window : 0;
+  const int k_begin = (lo / 32) * 32 + split * keys_per_split;
+  const int k_end = min(k_begin + keys_per_split, pos + 1);     // exclusive
+  const int hi = k_end - 1;
+  const bool head_ok = col < rep;
+  const int h = g * rep + (head_ok ? col : 0);
+  const size_t pbase = ((size_t)t * H + h) * n_splits + split;
+
+  bf16x8_t qf[D_KS];
+  {
+    const bf16_t* qr = q + (size_t)t * q_stride + (size_t)h * HEAD_DIM;
+#pragma unroll
+    for (int ks = 0; ks < D_KS; ++ks) {
+      u32x4_t v = {0u, 0u, 0u, 0u};
+      const int d0 = 32 * ks + 8 * kg;
+      if (head_ok && d0 < HEAD_DIM) v = *reinterpret_cast<const u32x4_t*>(qr + d0);
+      qf[ks] = as_frag(v);
+    }
+  }
+  f32x4_t o[D_MT];
+#pragma unroll
+  for (int mt = 0; mt < D_MT; ++mt) o[mt] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+  float m_run = -INFINITY, l_run = 0.f;
+  const float sc = scale * LOG2E;
+
+  for (int kb = k_begin; kb < k_end; kb += 32) {
+    f32x4_t s[2];
+#pragma unroll
+    for (int tt = 0; tt < 2; ++tt) {
+      s[tt] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+      const int my_key = kb + 16 * tt + col;
+#pragma unroll
+      for (int ks = 0; ks < D_KS; ++ks) {
+        const bf16x8_t kf =
+            as_frag(load_k8(k_pool, bt, G, g, ps, my_key, 32 * ks + 8 * kg, lo, hi));
+        s[tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[ks], s[tt], 0, 0, 0);
+      }
+    }
+    // lane holds, for head `col`, keys kb + 16*tt + 4*kg + v
+    float mloc = -INFINITY;
+#pragma unroll
+    for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        const int key = kb + 16 * tt + 4 * kg + v;
+        const bool ok = key >= lo && key <= hi;
+        s[tt][v] = ok ? s[tt][v] * sc : -INFINITY;
+        mloc = fmaxf(mloc, s[tt][v]);
+      }
+    mloc = fmaxf(mloc, __shfl_xor(mloc, 16, WAVE));
+    mloc = fmaxf(mloc, __shfl_xor(mloc, 32, WAVE));
+    const float m_new = fmaxf(m_run, mloc);
+    const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+    const float corr = exp2f(m_run - m_safe);
+    float lsum = 0.f;
+#pragma unroll
+    for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        s[tt][v] = exp2f(s[tt][v] - m_safe);
+        lsum += s[tt][v];
+      }
+    lsum += __shfl_xor(lsum, 16, WAVE);
+    lsum += __shfl_xor(lsum, 32, WAVE);
+    l_run = l_run * corr + lsum;
+    m_run = m_new;
+    const u32x4_t pw = {pack_bf16(s[0][0], s[0][1]), pack_bf16(s[0][2], s[0][3]),
+                        pack_bf16(s[1][0], s[1][1]), pack_bf16(s[1][2], s[1][3])};
+    const bf16x8_t pf = as_frag(pw);
+#pragma unroll
+    for (int mt = 0; mt < D_MT; ++mt) {
+      const int dd = 16 * mt + col;
+      const u32x2_t a = load_vt4(vt_pool, bt, G, g, ps, dd, kb + 4 * kg, lo, hi);
+      const u32x2_t b = load_vt4(vt_pool, bt, G, g, ps, dd, kb + 16 + 4 * kg, lo, hi);
+      const u32x4_t vw = {a.x, a.y, b.x, b.y};
+      o[mt] = o[mt] * corr;
+      o[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_frag(vw), pf, o[mt], 0, 0, 0);
+    }
+  }
+  if (!head_ok) return;
+  if (kg == 0) {
+    part_ml[2 * pbase] = m_run;
+    part_ml[2 * pbase + 1] = l_run;
+  }
+  float* po = part_o + pbase * HEAD_DIM;
+#pragma unroll
+  for (int mt = 0; mt < D_MT; ++mt)
+    *reinterpret_cast<f32x4_t*>(po + 16 * mt + 4 * kg) = o[mt];
+}
+
+// out[t, h, :] = sum_s o_s 2^(m_s - M) / sum_s l_s 2^(m_s - M)
+__global__ __launch_bounds__(64) void attn_merge_kernel(const float* __restrict__ part_o,
+                                                        const float* __restrict__ part_ml,
+                                                        bf16_t* __restrict__ out, int out_stride,
+                                                        int H, int n_splits) {
+  const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const size_t base = ((size_t)t * H + h) * n_splits;
+  float M = -INFINITY;
+  for (int s = 0; s < n_splits; ++s) M = fmaxf(M, part_ml[2 * (base + s)]);
+  float L = 0.f;
+  float acc[(HEAD_DIM + WAVE - 1) / WAVE];
+#pragma unroll
+  for (int i = 0; i < (HEAD_DIM + WAVE - 1) / WAVE; ++i) acc[i] = 0.f;
+  for (int s = 0; s < n_splits; ++s) {
+    const float m = part_ml[2 * (base + s)];
+    if (m == -INFINITY) continue;
+    const float w = exp2f(m - M);
+    L += part_ml[2 * (base + s) + 1] * w;
+#pragma unroll
+    for (int i = 0; i < (HEAD_DIM + WAVE - 1) / WAVE; ++i) {
+      const int e = lane + i * WAVE;
+      if (e < HEAD_DIM) acc[i] += part_o[(base + s) * HEAD_DIM + e] * w;
+    }
+  }
+  const float inv = L > 0.f ? 1.0f / L : 0.f;
+  bf16_t* o = out + (size_t)t * out_stride + (size_t)h * HEAD_DIM;
+#pragma unroll
+  for (int i = 0; i < (HEAD_DIM + WAVE - 1) / WAVE; ++i) {
+    const int e = lane + i * WAVE;
+    if (e < HEAD_DIM) o[e] = f32_to_bf16(acc[i] * inv);
+  }
+}
+
+extern "C" int kappai_attn_head_dim(void) { return HEAD_DIM; }
+
+extern "C" int kappai_attn_prefill(const void* q, int q_stride, const void* k_pool,
+                                   const void* vt_pool, void* out, int out_stride,
+                                   const int* q_tiles, int n_tiles, const int* row_pos,
+                                   const int* block_tables, int max_blocks, int H, int G, int ps,
+                                   int window, float scale, hipStream_t stream) {
+  if (n_tiles <= 0) return 0;
+  if (ps % 16 || G < 1 || H % G || H > 65535 || (q_stride % 8) || (out_stride % 4))
+    return (int)hipErrorInvalidValue;
+  hipLaunchKernelGGL(attn_prefill_kernel, dim3(n_tiles, H), dim3(WAVE), 0, stream,
+                     (const bf16_t*)q, q_stride, (const bf16_t*)k_pool, (const bf16_t*)vt_pool,
+                     (bf16_t*)out, out_stride, q_tiles, row_pos, block_tables, max_blocks, H, G,
+                     ps, window, scale);
+  KAPPAI_RETURN_LAUNCH_STATUS();
+}
+
+extern "C" int kappai_attn_decode(const void* q, int q_stride, const void* k_pool,
+                                  const void* vt_pool, void* out, int out_stride, float* part_o,
+                                  float* part_ml, const int* row_pos, const int* row_seg,
+                                  const int* block_tables, int max_blocks, int T, int H, int G,
+                                  int ps, int window, float scale, int keys_per_split,
+                                  int n_splits, hipStream_t stream) {
+  if (T <= 0) return 0;
+  if (ps % 16 || G < 1 || H % G || H / G > 16 || G > 65535 || n_splits < 1 || n_splits > 65535 ||
+      keys_per_split < 32 || keys_per_split % 32 || (q_stride % 8))
+    return (int)hipErrorInvalidValue;
+  hipLaunchKernelGGL(attn_decode_kernel, dim3(T, G, n_splits), dim3(WAVE), 0, stream,
+                     (const bf16_t*)q, q_stride, (const bf16_t*)k_pool, (const bf16_t*)vt_pool,
+                     part_o, part_ml, row_pos, row_seg, block_tables, max_blocks, H, G, ps, window,
+                     scale, keys_per_split, n_splits);
+  hipLaunchKernelGGL(attn_merge_kernel, dim3(T, H), dim3(WAVE), 0, stream, (const float*)part_o,
+                     (const float*)part_ml, (bf16_t*)out, out_stride, H, n_splits);
+  KAPPAI_RETURN_LAUNCH_STATUS();
+}

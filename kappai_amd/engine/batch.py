@@ -8,7 +8,7 @@ request; a decoded token is a segment of length one.
 from __future__ import annotations
 
 from dataclasses import dataclass, field
-from typing import Dict, List, Sequence
+from typing import Dict, List, Optional, Sequence
 
 import numpy as np
 import torch
@@ -32,7 +32,8 @@ class RowBatch:
     tokens[T], row_pos[T] (absolute position), row_seg[T] (segment of the row),
     seg_start[S+1] (first row of each segment), seg_pos0[S] (position of that row),
     seg_slot[S] (the request's state slot), block_tables[g] [S, max_blocks] for every paged
-    group g, logit_rows[n] (rows whose logits are wanted, in the order asked)."""
+    group g, logit_rows[n] (rows whose logits are wanted, in the order asked), q_tiles: the
+    segments cut into runs of at most ATTENTION_TILE_ROWS rows for the attention kernel."""
     n_rows: int
     n_segments: int
     n_logit_rows: int
@@ -45,8 +46,12 @@ class RowBatch:
     seg_pos0: torch.Tensor
     seg_slot: torch.Tensor
     logit_rows: torch.Tensor
+    q_tiles: Optional[torch.Tensor] = None      # [tiles, 4]: (segment, first row, rows, 0)
     block_tables: List[torch.Tensor] = field(default_factory=list)
     host: Dict[str, np.ndarray] = field(default_factory=dict)
+
+
+ATTENTION_TILE_ROWS = 32
 
 
 def layout_rows(entries: Sequence[StepEntry], cache: CacheManager, vocab_size: int):
@@ -56,6 +61,7 @@ def layout_rows(entries: Sequence[StepEntry], cache: CacheManager, vocab_size: i
         raise ValueError("a step needs at least one entry")
     seen = set()
     tokens, row_pos, row_seg, seg_start, seg_pos0, seg_slot, logit_rows = [], [], [], [0], [], [], []
+    q_tiles = []
     for si, e in enumerate(entries):
         n = len(e.tokens)
         if n < 1:
@@ -77,6 +83,8 @@ def layout_rows(entries: Sequence[StepEntry], cache: CacheManager, vocab_size: i
         row_pos.extend(range(p0, p0 + n))
         row_seg.extend([si] * n)
         seg_start.append(base + n)
+        for r in range(0, n, ATTENTION_TILE_ROWS):
+            q_tiles.append((si, base + r, min(ATTENTION_TILE_ROWS, n - r), 0))
         seg_pos0.append(p0)
         seg_slot.append(e.cache.slot)
         logit_rows.extend(base + int(w) for w in e.want)
@@ -97,6 +105,7 @@ def layout_rows(entries: Sequence[StepEntry], cache: CacheManager, vocab_size: i
         "seg_pos0": np.asarray(seg_pos0, dtype=np.int32),
         "seg_slot": np.asarray(seg_slot, dtype=np.int32),
         "logit_rows": np.asarray(logit_rows, dtype=np.int32),
+        "q_tiles": np.asarray(q_tiles, dtype=np.int32).reshape(-1, 4),
     }
     for gi, bt in enumerate(tables):
         arrays[f"block_table_{gi}"] = bt

@@ -64,7 +64,7 @@ class StepRunner:
             max_segment_rows=sizes["max_segment_rows"],
             tokens=dev["tokens"], row_pos=dev["row_pos"], row_seg=dev["row_seg"],
             seg_start=dev["seg_start"], seg_pos0=dev["seg_pos0"], seg_slot=dev["seg_slot"],
-            logit_rows=dev["logit_rows"],
+            logit_rows=dev["logit_rows"], q_tiles=dev["q_tiles"],
             block_tables=[dev[f"block_table_{g}"] for g in range(sizes["n_groups"])],
             host=arrays)
 

@@ -26,6 +26,8 @@ HIPCC_FLAGS = ["-O3", "-std=c++17", f"--offload-arch={GPU_ARCH}", "-shared", "-f
                "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
                "-Wno-unused-command-line-argument", "-Wno-pass-failed"]
 LIBRARIES = ["elementwise", "gemm", "shortconv", "attention", "sampling"]
+# libraries compiled once per value of a constant: name -> (constant, values built ahead)
+VARIANT_LIBRARIES = {"attention_mfma": ("HEAD_DIM", [16, 32, 48, 64, 128, 256])}
 
 
 class KernelBuildError(RuntimeError):
@@ -48,12 +50,20 @@ def _hipcc() -> str:
                            "HIP kernels of kappai_amd cannot be built, and there is no other path")
 
 
-def _source_hash(name: str) -> str:
+def _defines_flags(defines) -> List[str]:
+    return [f"-D{k}={v}" for k, v in sorted((defines or {}).items())]
+
+
+def _built_name(name: str, defines) -> str:
+    return name + "".join(f"__{k}{v}" for k, v in sorted((defines or {}).items()))
+
+
+def _source_hash(name: str, defines=None) -> str:
     h = hashlib.sha256()
     for p in [CSRC / f"{name}.hip"] + sorted(CSRC.glob("*.h")):
         h.update(p.name.encode())
         h.update(p.read_bytes())
-    h.update(" ".join(HIPCC_FLAGS).encode())
+    h.update(" ".join(HIPCC_FLAGS + _defines_flags(defines)).encode())
     return h.hexdigest()
 
 
@@ -78,25 +88,28 @@ def _writable_build_dir() -> Path:
                            + ", ".join(str(d) for d in _build_dirs()))
 
 
-def _find_built(name: str, want_hash: str):
+def _find_built(built: str, want_hash: str):
     for d in _build_dirs():
-        so, tag = d / f"{name}.so", d / f"{name}.hash"
+        so, tag = d / f"{built}.so", d / f"{built}.hash"
         if so.is_file() and tag.is_file() and tag.read_text().strip() == want_hash:
             return so
     return None
 
 
-def compile_library(name: str, verbose: bool = True) -> Path:
+def compile_library(name: str, verbose: bool = True, defines=None) -> Path:
     """Compile ``csrc/<name>.hip`` now, whether or not a built library is there."""
     src = CSRC / f"{name}.hip"
     if not src.is_file():
         raise KernelBuildError(f"{src}: no such kernel source")
     out_dir = _writable_build_dir()
-    so, tag = out_dir / f"{name}.so", out_dir / f"{name}.hash"
-    tmp = out_dir / f".{name}.{os.getpid()}.{threading.get_ident()}.so"
-    cmd = [_hipcc(), *HIPCC_FLAGS, f"-I{CSRC}", str(src), "-o", str(tmp)]
+    built = _built_name(name, defines)
+    so, tag = out_dir / f"{built}.so", out_dir / f"{built}.hash"
+    tmp = out_dir / f".{built}.{os.getpid()}.{threading.get_ident()}.so"
+    cmd = [_hipcc(), *HIPCC_FLAGS, *_defines_flags(defines), f"-I{CSRC}", str(src), "-o", str(tmp)]
+    what = src.name + (" (" + ", ".join(f"{k}={v}" for k, v in sorted(defines.items())) + ")"
+                       if defines else "")
     if verbose:
-        print(f"[kappai_amd] compiling {src.name} for {GPU_ARCH} ...", file=sys.stderr, flush=True)
+        print(f"[kappai_amd] compiling {what} for {GPU_ARCH} ...", file=sys.stderr, flush=True)
     t0 = time.time()
     proc = subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     while True:
@@ -105,13 +118,13 @@ def compile_library(name: str, verbose: bool = True) -> Path:
             break
         except subprocess.TimeoutExpired:
             if verbose:
-                print(f"[kappai_amd] ... still compiling {src.name} ({time.time() - t0:.0f} s)",
+                print(f"[kappai_amd] ... still compiling {what} ({time.time() - t0:.0f} s)",
                       file=sys.stderr, flush=True)
     if proc.returncode != 0:
         tmp.unlink(missing_ok=True)
-        raise KernelBuildError(f"hipcc failed on {src.name}:\n{out}")
+        raise KernelBuildError(f"hipcc failed on {what}:\n{out}")
     os.replace(tmp, so)
-    tag.write_text(_source_hash(name))
+    tag.write_text(_source_hash(name, defines))
     if verbose:
         print(f"[kappai_amd] built {so.name} in {time.time() - t0:.1f} s", file=sys.stderr,
               flush=True)
@@ -122,14 +135,17 @@ def build_all(verbose: bool = True, force: bool = True) -> None:
     """Compile every library (used by the build check); in parallel threads."""
     errors = []
 
-    def work(n):
+    def work(n, defines):
         try:
-            if force or _find_built(n, _source_hash(n)) is None:
-                compile_library(n, verbose)
+            if force or _find_built(_built_name(n, defines), _source_hash(n, defines)) is None:
+                compile_library(n, verbose, defines)
         except Exception as exc:  # noqa: BLE001 - collected and raised below
             errors.append(exc)
 
-    threads = [threading.Thread(target=work, args=(n,)) for n in LIBRARIES]
+    jobs = [(n, None) for n in LIBRARIES]
+    for n, (const, values) in VARIANT_LIBRARIES.items():
+        jobs += [(n, {const: v}) for v in values]
+    threads = [threading.Thread(target=work, args=job) for job in jobs]
     for t in threads:
         t.start()
     for t in threads:
@@ -138,23 +154,25 @@ def build_all(verbose: bool = True, force: bool = True) -> None:
         raise errors[0]
 
 
-def library(name: str) -> ctypes.CDLL:
-    """The loaded library ``name``; compiled first if no up-to-date build exists."""
-    lib = _loaded.get(name)
+def library(name: str, **defines) -> ctypes.CDLL:
+    """The loaded library ``name`` (compiled with ``defines`` as -D constants); compiled
+    first if no up-to-date build exists."""
+    built = _built_name(name, defines)
+    lib = _loaded.get(built)
     if lib is not None:
         return lib
     with _lock:
-        lib = _loaded.get(name)
+        lib = _loaded.get(built)
         if lib is not None:
             return lib
-        so = _find_built(name, _source_hash(name))
+        so = _find_built(built, _source_hash(name, defines))
         if so is None:
-            so = compile_library(name)
+            so = compile_library(name, defines=defines)
         try:
             lib = ctypes.CDLL(str(so))
         except OSError as exc:
             raise KernelBuildError(f"cannot load {so}: {exc}") from exc
-        _loaded[name] = lib
+        _loaded[built] = lib
         return lib
 
 

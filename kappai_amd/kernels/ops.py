@@ -192,6 +192,15 @@ def shortconv(proj: torch.Tensor, taps: torch.Tensor, bias: Optional[torch.Tenso
 
 
 ROT_NONE, ROT_HALF, ROT_INTERLEAVED = 0, 1, 2
+ATTENTION_TILE_ROWS = 32      # rows of a segment that one wave of the prefill kernel takes
+
+
+def _check_pools(k_pool, v_pool, G, page_size, d) -> None:
+    _need(k_pool.dim() == 4 and v_pool.dim() == 4 and k_pool.shape[0] == v_pool.shape[0]
+          and tuple(k_pool.shape[1:]) == (G, page_size, d)
+          and tuple(v_pool.shape[1:]) == (G, d, page_size),
+          f"pools {tuple(k_pool.shape)} / {tuple(v_pool.shape)} are not keys [pages, {G}, "
+          f"{page_size}, {d}] and transposed values [pages, {G}, {d}, {page_size}]")
 
 
 def qk_norm_rope_store(qkv: torch.Tensor, n_heads: int, n_kv_heads: int, head_dim: int,
@@ -229,9 +238,7 @@ def qk_norm_rope_store(qkv: torch.Tensor, n_heads: int, n_kv_heads: int, head_di
         _gpu("k_pool", k_pool, qkv.dtype)
         _gpu("v_pool", v_pool, qkv.dtype)
         _gpu("block_tables", block_tables, I32)
-        _need(k_pool.shape == v_pool.shape and k_pool.dim() == 4
-              and k_pool.shape[1:] == (G, page_size, d),
-              f"pools {tuple(k_pool.shape)} are not [pages, {G}, {page_size}, {d}]")
+        _check_pools(k_pool, v_pool, G, page_size, d)
         _need(block_tables.dim() == 2, "block_tables must be [segments, max_blocks]")
         max_blocks = block_tables.shape[1]
     check(library("attention").kappai_qk_norm_rope_store(
@@ -246,10 +253,18 @@ def qk_norm_rope_store(qkv: torch.Tensor, n_heads: int, n_kv_heads: int, head_di
 def paged_attention(q: torch.Tensor, n_heads: int, n_kv_heads: int, head_dim: int,
                     k_pool: torch.Tensor, v_pool: torch.Tensor, row_pos: torch.Tensor,
                     row_seg: torch.Tensor, block_tables: torch.Tensor, page_size: int,
-                    scale: float, window: int = 0) -> torch.Tensor:
+                    scale: float, window: int = 0, q_tiles: Optional[torch.Tensor] = None,
+                    single_rows: bool = False, max_position: Optional[int] = None,
+                    kernel: str = "auto") -> torch.Tensor:
     """Causal attention of every row over the keys of its request that are in the cache
     (its own included; the last ``window`` of them when a window is set).  ``q`` is
-    [T, >= H d] with a row stride (the q columns of the fused projection).  Returns [T, H d]."""
+    [T, >= H d] with a row stride (the q columns of the fused projection).  Returns [T, H d].
+
+    bfloat16 with a page size and head size that are multiples of 16 runs on the matrix
+    cores: the split-key decode kernel when every segment is a single row (``single_rows``;
+    ``max_position`` sizes the splits), else the tiled kernel over ``q_tiles`` [tiles, 4] =
+    (segment, first row, rows <= 32, 0).  Everything else, float32 included, runs the plain
+    kernel.  ``kernel`` = "rows" | "prefill" | "decode" forces one (for tests)."""
     H, G, d = n_heads, n_kv_heads, head_dim
     _gpu("q", q, (F32, BF16), contiguous=False)
     T = q.shape[0]
@@ -260,20 +275,61 @@ def paged_attention(q: torch.Tensor, n_heads: int, n_kv_heads: int, head_dim: in
     _need(G >= 1 and H % G == 0 and H <= MAX_GRID_Y, f"{H} heads over {G} kv heads")
     _gpu("k_pool", k_pool, q.dtype)
     _gpu("v_pool", v_pool, q.dtype)
-    _need(k_pool.shape == v_pool.shape and k_pool.dim() == 4
-          and k_pool.shape[1:] == (G, page_size, d),
-          f"pools {tuple(k_pool.shape)} are not [pages, {G}, {page_size}, {d}]")
+    _check_pools(k_pool, v_pool, G, page_size, d)
     _gpu("row_pos", row_pos, I32)
     _gpu("row_seg", row_seg, I32)
     _gpu("block_tables", block_tables, I32)
     _need(row_pos.shape[0] == T and row_seg.shape[0] == T and block_tables.dim() == 2,
           "row tables do not fit the batch")
     out = torch.empty((T, H * d), dtype=q.dtype, device=q.device)
-    check(library("attention").kappai_paged_attention_rows(
+    mfma_ok = (q.dtype == BF16 and page_size % 16 == 0 and d % 16 == 0 and d <= 256
+               and q.stride(0) % 8 == 0 and q.data_ptr() % 16 == 0)
+    if kernel == "auto":
+        if not mfma_ok:
+            kernel = "rows"
+        elif single_rows and H // G <= 16 and max_position is not None:
+            kernel = "decode"
+        elif q_tiles is not None:
+            kernel = "prefill"
+        else:
+            kernel = "rows"
+    if kernel == "rows":
+        check(library("attention").kappai_paged_attention_rows(
+            _ptr(q), _c_int(q.stride(0)), _ptr(k_pool), _ptr(v_pool), _ptr(out), _c_int(H * d),
+            _ptr(row_pos), _ptr(row_seg), _ptr(block_tables), _c_int(block_tables.shape[1]),
+            _c_int(T), _c_int(H), _c_int(G), _c_int(d), _c_int(page_size), _c_int(window or 0),
+            _c_float(scale), _c_int(_is_bf16(q.dtype)), _stream()), "paged_attention_rows")
+        return out
+    _need(mfma_ok, "the matrix-core attention kernels need bfloat16, a page size and a head size "
+          f"that are multiples of 16 (head size at most 256) and 16-byte aligned rows; got "
+          f"{q.dtype}, page {page_size}, head {d}")
+    lib = library("attention_mfma", HEAD_DIM=d)
+    if kernel == "prefill":
+        _gpu("q_tiles", q_tiles, I32)
+        _need(q_tiles.dim() == 2 and q_tiles.shape[1] == 4, "q_tiles must be [tiles, 4]")
+        check(lib.kappai_attn_prefill(
+            _ptr(q), _c_int(q.stride(0)), _ptr(k_pool), _ptr(v_pool), _ptr(out), _c_int(H * d),
+            _ptr(q_tiles), _c_int(q_tiles.shape[0]), _ptr(row_pos), _ptr(block_tables),
+            _c_int(block_tables.shape[1]), _c_int(H), _c_int(G), _c_int(page_size),
+            _c_int(window or 0), _c_float(scale), _stream()), "attn_prefill")
+        return out
+    _need(kernel == "decode", f"unknown attention kernel {kernel!r}")
+    _need(H // G <= 16, "the decode kernel takes at most 16 query heads per kv head")
+    _need(max_position is not None, "the decode kernel needs the batch's largest position")
+    n_keys = min(max_position + 1, window) + 32 if window else max_position + 1
+    # enough waves to fill the chip, but at least 64 keys a split
+    want = max(1, 2048 // max(T * G, 1))
+    n_splits = max(1, min(want, (n_keys + 63) // 64))
+    keys_per_split = ((n_keys + n_splits - 1) // n_splits + 31) // 32 * 32
+    n_splits = (n_keys + keys_per_split - 1) // keys_per_split
+    part_o = torch.empty((T, H, n_splits, d), dtype=F32, device=q.device)
+    part_ml = torch.empty((T, H, n_splits, 2), dtype=F32, device=q.device)
+    check(lib.kappai_attn_decode(
         _ptr(q), _c_int(q.stride(0)), _ptr(k_pool), _ptr(v_pool), _ptr(out), _c_int(H * d),
-        _ptr(row_pos), _ptr(row_seg), _ptr(block_tables), _c_int(block_tables.shape[1]), _c_int(T),
-        _c_int(H), _c_int(G), _c_int(d), _c_int(page_size), _c_int(window or 0), _c_float(scale),
-        _c_int(_is_bf16(q.dtype)), _stream()), "paged_attention")
+        _ptr(part_o), _ptr(part_ml), _ptr(row_pos), _ptr(row_seg), _ptr(block_tables),
+        _c_int(block_tables.shape[1]), _c_int(T), _c_int(H), _c_int(G), _c_int(page_size),
+        _c_int(window or 0), _c_float(scale), _c_int(keys_per_split), _c_int(n_splits),
+        _stream()), "attn_decode")
     return out
 
 

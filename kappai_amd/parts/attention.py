@@ -79,7 +79,9 @@ class GroupedQueryAttention(Mixer):
             batch.row_seg, tables, cache.page_size, store_kv=not shared_cache)
         ctx = ops.paged_attention(proj, H, G, d, cache.k_pool, cache.v_pool, batch.row_pos,
                                   batch.row_seg, tables, cache.page_size, self.scale,
-                                  window=self.window or 0)
+                                  window=self.window or 0, q_tiles=batch.q_tiles,
+                                  single_rows=batch.max_segment_rows == 1,
+                                  max_position=batch.max_position)
         return self.out.forward(ctx)
 
     def weight_bytes(self) -> int:

@@ -108,11 +108,11 @@ def qk_norm_rope_store(qkv, n_heads, n_kv_heads, head_dim, q_norm_w, k_norm_w, e
         page = int(block_tables[int(row_seg[t]), p // page_size])
         assert page >= 0, "a row is stored into a page that was given back"
         k_pool[page, :, p % page_size, :] = k[t].to(k_pool.dtype)
-        v_pool[page, :, p % page_size, :] = v[t].to(v_pool.dtype)
+        v_pool[page, :, :, p % page_size] = v[t].to(v_pool.dtype)
 
 
 def paged_attention(q, n_heads, n_kv_heads, head_dim, k_pool, v_pool, row_pos, row_seg,
-                    block_tables, page_size, scale, window=0):
+                    block_tables, page_size, scale, window=0, **_unused):
     H, G, d = n_heads, n_kv_heads, head_dim
     T = q.shape[0]
     out = torch.empty((T, H * d), dtype=F32)
@@ -124,7 +124,7 @@ def paged_attention(q, n_heads, n_kv_heads, head_dim, k_pool, v_pool, row_pos, r
         pages = bt[(idx // page_size).long()].long()
         assert bool((pages >= 0).all()), "attention reads a page that was given back"
         keys = k_pool[pages, :, (idx % page_size).long(), :].to(F32)     # [n, G, d]
-        vals = v_pool[pages, :, (idx % page_size).long(), :].to(F32)
+        vals = v_pool[pages, :, :, (idx % page_size).long()].to(F32)             # [n, G, d]
         qt = q[t, :H * d].to(F32).reshape(H, d)
         for h in range(H):
             g = h // (H // G)

@@ -198,15 +198,21 @@ def paged_case(seed, dtype, H, G, d, ps, lens_before, lens_new, n_pages=None, sh
     row_pos = np.concatenate([np.arange(a, a + b) for a, b in zip(lens_before, lens_new)]).astype(
         np.int32)
     k_pool = torch.full((n_pages, G, ps, d), float("nan"), dtype=dtype)
-    v_pool = torch.full((n_pages, G, ps, d), float("nan"), dtype=dtype)
+    v_pool = torch.full((n_pages, G, d, ps), float("nan"), dtype=dtype)     # values transposed
     # history: what earlier steps would have stored
     for s in range(S):
         for p in range(lens_before[s]):
             k_pool[bt[s, p // ps], :, p % ps, :] = rand((G, d), dtype, seed * 1000 + s * 100 + p)
-            v_pool[bt[s, p // ps], :, p % ps, :] = rand((G, d), dtype, seed * 2000 + s * 100 + p)
+            v_pool[bt[s, p // ps], :, :, p % ps] = rand((G, d), dtype, seed * 2000 + s * 100 + p)
     qkv = rand((T, (H + 2 * G) * d), dtype, seed + 5)
+    tiles, base = [], 0
+    for s, n in enumerate(lens_new):
+        tiles += [(s, base + r, min(32, n - r), 0) for r in range(0, n, 32)]
+        base += n
     return dict(qkv=qkv, k_pool=k_pool, v_pool=v_pool, row_pos=torch.from_numpy(row_pos),
-                row_seg=torch.from_numpy(row_seg), bt=torch.from_numpy(bt), T=T)
+                row_seg=torch.from_numpy(row_seg), bt=torch.from_numpy(bt), T=T,
+                q_tiles=torch.tensor(tiles, dtype=torch.int32), max_pos=int(row_pos.max()),
+                single=all(n == 1 for n in lens_new))
 
 
 def rope_tables(n, rot_dim, theta=10000.0):
@@ -227,6 +233,10 @@ ATT_CASES = [
     (2, 1, 256, 16, [3, 40], [5, 1], 0, 0, True, 0),      # no rotation
     (4, 2, 64, 16, [90, 0, 45], [1, 50, 6], 64, 1, True, 24),   # window
     (32, 8, 64, 16, [300], [1], 64, 1, True, 0),
+    (8, 2, 64, 16, [0, 1, 31, 32, 33, 500, 63, 64], [1] * 8, 64, 1, True, 0),     # decode rows
+    (6, 3, 48, 32, [200, 7, 95], [1, 1, 1], 48, 1, True, 40),                   # decode, window
+    (16, 1, 32, 16, [130, 2], [1, 1], 32, 1, False, 0),                         # 16 heads a kv head
+    (4, 4, 128, 16, [77, 140], [40, 1], 128, 1, True, 0),
 ]
 
 
@@ -255,13 +265,19 @@ def test_store_and_attention(ops, dtype, case):
     close(torch.nan_to_num(dev["v_pool"].float()), torch.nan_to_num(v_ref), 0.0, "v pages")
 
     scale = 1.0 / math.sqrt(d)
-    got = ops.paged_attention(dev["qkv"], H, G, d, dev["k_pool"], dev["v_pool"], dev["row_pos"],
-                              dev["row_seg"], dev["bt"], ps, scale, window=window)
     # reference attention over the pools the kernel itself wrote (rounded as the run stores them)
     want = ref.paged_attention(dev["qkv"].cpu().float(), H, G, d, dev["k_pool"].cpu().float(),
                                dev["v_pool"].cpu().float(), c["row_pos"], c["row_seg"], c["bt"],
                                ps, scale, window=window)
-    close(got.float(), want, tol * 2, "attention")
+    kernels = ["rows"]
+    if dtype == BF16 and ps % 16 == 0 and d % 16 == 0 and d <= 256:
+        kernels += ["prefill"] + (["decode"] if c["single"] and H // G <= 16 else [])
+    for kernel in kernels:
+        got = ops.paged_attention(dev["qkv"], H, G, d, dev["k_pool"], dev["v_pool"],
+                                  dev["row_pos"], dev["row_seg"], dev["bt"], ps, scale,
+                                  window=window, q_tiles=dev["q_tiles"], single_rows=c["single"],
+                                  max_position=c["max_pos"], kernel=kernel)
+        close(got.float(), want, tol * 2, f"attention kernel {kernel}")
 
 
 @pytest.mark.parametrize("dtype", [F32, BF16])
@@ -280,14 +296,18 @@ def test_attention_finds_one_far_key(ops, dtype):
         bt = c["bt"]
         c["k_pool"][bt[0, far // ps], :, far % ps, 3] = 8.0
         marker = rand((G, d), dtype, 13) + 3.0
-        c["v_pool"][bt[0, far // ps], :, far % ps, :] = marker
+        c["v_pool"][bt[0, far // ps], :, :, far % ps] = marker
         dev = {k: (v.to(DEV) if torch.is_tensor(v) else v) for k, v in c.items()}
         # the query's own key (position n) must exist too: store zeros for it
         dev["k_pool"][bt[0, n // ps], :, n % ps, :] = 0
-        got = ops.paged_attention(dev["qkv"], H, G, d, dev["k_pool"], dev["v_pool"], dev["row_pos"],
-                                  dev["row_seg"], dev["bt"], ps, 1.0 / math.sqrt(d))
         want = marker.float().repeat_interleave(H // G, dim=0).reshape(1, H * d)
-        close(got.float(), want, 2 * BF16_ULP if dtype == BF16 else 1e-5, f"far key at {far}")
+        for kernel in (["rows", "prefill", "decode"] if dtype == BF16 else ["rows"]):
+            got = ops.paged_attention(dev["qkv"], H, G, d, dev["k_pool"], dev["v_pool"],
+                                      dev["row_pos"], dev["row_seg"], dev["bt"], ps,
+                                      1.0 / math.sqrt(d), q_tiles=dev["q_tiles"], single_rows=True,
+                                      max_position=c["max_pos"], kernel=kernel)
+            close(got.float(), want, 2 * BF16_ULP if dtype == BF16 else 1e-5,
+                  f"far key at {far}, kernel {kernel}")
 
 
 # ---------------------------------------------------------------------------------------
