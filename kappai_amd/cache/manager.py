@@ -188,7 +188,7 @@ class CacheManager:
         fills the pools with NaN so that a read of a key nobody wrote shows."""
         self.device, self.dtype = device, dtype
         for g in self.paged_groups:
-            n = max(g.allocator.num_pages, 1)
+            n = g.allocator.num_pages + 1          # the last page is scratch (see scratch_page)
             kshape = (n, g.spec.num_kv_heads, self.page_size, g.spec.head_dim)
             vshape = (n, g.spec.num_kv_heads, g.spec.head_dim, self.page_size)
             for cid in g.cache_ids:
@@ -199,10 +199,20 @@ class CacheManager:
         for g in self.state_groups:
             sdt = getattr(torch, g.spec.dtype)
             for cid in g.cache_ids:
-                t = torch.zeros((self.num_slots, *g.spec.shape), dtype=sdt, device=device)
+                t = torch.zeros((self.num_slots + 1, *g.spec.shape), dtype=sdt, device=device)
                 if poison:
                     t.fill_(float("nan"))
                 g.states[cid] = t
+
+    def scratch_page(self, group: int) -> int:
+        """A page beyond the allocator's reach that no request ever reads: rows of a warm-up
+        run are stored there."""
+        return self.paged_groups[group].allocator.num_pages
+
+    @property
+    def scratch_slot(self) -> int:
+        """A state slot beyond the allocator's reach, for warm-up runs."""
+        return self.num_slots
 
     def bytes_per_token(self, dtype_bytes: int) -> int:
         """Bytes of keys and values that one token takes over all paged layers (kappai:

@@ -229,18 +229,33 @@ __global__ __launch_bounds__(64) void attn_decode_kernel(
   float m_run = -INFINITY, l_run = 0.f;
   const float sc = scale * LOG2E;
 
-  for (int kb = k_begin; kb < k_end; kb += 32) {
+  // The loads of the next 32 keys are issued before the current 32 are worked on, so that
+  // their latency hides behind the matrix products and the softmax (head sizes up to 128;
+  // beyond that the registers do not suffice and the loop runs without the look-ahead).
+  constexpr bool AHEAD = HEAD_DIM <= 128;
+  u32x4_t kf[2][2][D_KS];
+  u32x2_t va[2][D_MT], vb[2][D_MT];
+  auto fetch = [&](int buf, int kb) {
+#pragma unroll
+    for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+      for (int ks = 0; ks < D_KS; ++ks)
+        kf[buf][tt][ks] = load_k8(k_pool, bt, G, g, ps, kb + 16 * tt + col, 32 * ks + 8 * kg, lo, hi);
+#pragma unroll
+    for (int mt = 0; mt < D_MT; ++mt) {
+      va[buf][mt] = load_vt4(vt_pool, bt, G, g, ps, 16 * mt + col, kb + 4 * kg, lo, hi);
+      vb[buf][mt] = load_vt4(vt_pool, bt, G, g, ps, 16 * mt + col, kb + 16 + 4 * kg, lo, hi);
+    }
+  };
+  auto work = [&](int buf, int kb) {
     f32x4_t s[2];
 #pragma unroll
     for (int tt = 0; tt < 2; ++tt) {
       s[tt] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
-      const int my_key = kb + 16 * tt + col;
 #pragma unroll
-      for (int ks = 0; ks < D_KS; ++ks) {
-        const bf16x8_t kf =
-            as_frag(load_k8(k_pool, bt, G, g, ps, my_key, 32 * ks + 8 * kg, lo, hi));
-        s[tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[ks], s[tt], 0, 0, 0);
-      }
+      for (int ks = 0; ks < D_KS; ++ks)
+        s[tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_frag(kf[buf][tt][ks]), qf[ks], s[tt], 0,
+                                                        0, 0);
     }
     // lane holds, for head `col`, keys kb + 16*tt + 4*kg + v
     float mloc = -INFINITY;
@@ -275,12 +290,25 @@ __global__ __launch_bounds__(64) void attn_decode_kernel(
     const bf16x8_t pf = as_frag(pw);
 #pragma unroll
     for (int mt = 0; mt < D_MT; ++mt) {
-      const int dd = 16 * mt + col;
-      const u32x2_t a = load_vt4(vt_pool, bt, G, g, ps, dd, kb + 4 * kg, lo, hi);
-      const u32x2_t b = load_vt4(vt_pool, bt, G, g, ps, dd, kb + 16 + 4 * kg, lo, hi);
-      const u32x4_t vw = {a.x, a.y, b.x, b.y};
+      const u32x4_t vw = {va[buf][mt].x, va[buf][mt].y, vb[buf][mt].x, vb[buf][mt].y};
       o[mt] = o[mt] * corr;
       o[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_frag(vw), pf, o[mt], 0, 0, 0);
+    }
+  };
+  if (AHEAD) {
+    if (k_begin < k_end) fetch(0, k_begin);
+    for (int kb = k_begin; kb < k_end; kb += 64) {
+      if (kb + 32 < k_end) fetch(1, kb + 32);
+      work(0, kb);
+      if (kb + 32 < k_end) {
+        if (kb + 64 < k_end) fetch(0, kb + 64);
+        work(1, kb + 32);
+      }
+    }
+  } else {
+    for (int kb = k_begin; kb < k_end; kb += 32) {
+      fetch(0, kb);
+      work(0, kb);
     }
   }
   if (!head_ok) return;
@@ -294,34 +322,46 @@ __global__ __launch_bounds__(64) void attn_decode_kernel(
     *reinterpret_cast<f32x4_t*>(po + 16 * mt + 4 * kg) = o[mt];
 }
 
-// out[t, h, :] = sum_s o_s 2^(m_s - M) / sum_s l_s 2^(m_s - M)
+// out[t, h, :] = sum_s o_s 2^(m_s - M) / sum_s l_s 2^(m_s - M).  The weights of up to 64
+// splits at a time are computed one per lane; the sums over d then read independent rows.
 __global__ __launch_bounds__(64) void attn_merge_kernel(const float* __restrict__ part_o,
                                                         const float* __restrict__ part_ml,
                                                         bf16_t* __restrict__ out, int out_stride,
                                                         int H, int n_splits) {
   const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const size_t base = ((size_t)t * H + h) * n_splits;
+  constexpr int NPL = (HEAD_DIM + WAVE - 1) / WAVE;
   float M = -INFINITY;
-  for (int s = 0; s < n_splits; ++s) M = fmaxf(M, part_ml[2 * (base + s)]);
+  for (int s = lane; s < n_splits; s += WAVE) M = fmaxf(M, part_ml[2 * (base + s)]);
+  M = wave_max(M);
   float L = 0.f;
-  float acc[(HEAD_DIM + WAVE - 1) / WAVE];
+  float acc[NPL];
 #pragma unroll
-  for (int i = 0; i < (HEAD_DIM + WAVE - 1) / WAVE; ++i) acc[i] = 0.f;
-  for (int s = 0; s < n_splits; ++s) {
-    const float m = part_ml[2 * (base + s)];
-    if (m == -INFINITY) continue;
-    const float w = exp2f(m - M);
-    L += part_ml[2 * (base + s) + 1] * w;
+  for (int i = 0; i < NPL; ++i) acc[i] = 0.f;
+  for (int s0 = 0; s0 < n_splits; s0 += WAVE) {
+    const int s = s0 + lane;
+    float wgt = 0.f, l = 0.f;
+    if (s < n_splits) {
+      const float m = part_ml[2 * (base + s)];
+      wgt = m == -INFINITY ? 0.f : exp2f(m - M);
+      l = part_ml[2 * (base + s) + 1] * wgt;
+    }
+    L += wave_sum(l);
+    const int n = min(WAVE, n_splits - s0);
+#pragma unroll 4
+    for (int k = 0; k < n; ++k) {
+      const float wk = __shfl(wgt, k, WAVE);
 #pragma unroll
-    for (int i = 0; i < (HEAD_DIM + WAVE - 1) / WAVE; ++i) {
-      const int e = lane + i * WAVE;
-      if (e < HEAD_DIM) acc[i] += part_o[(base + s) * HEAD_DIM + e] * w;
+      for (int i = 0; i < NPL; ++i) {
+        const int e = lane + i * WAVE;
+        if (e < HEAD_DIM) acc[i] = fmaf(part_o[(base + s0 + k) * HEAD_DIM + e], wk, acc[i]);
+      }
     }
   }
   const float inv = L > 0.f ? 1.0f / L : 0.f;
   bf16_t* o = out + (size_t)t * out_stride + (size_t)h * HEAD_DIM;
 #pragma unroll
-  for (int i = 0; i < (HEAD_DIM + WAVE - 1) / WAVE; ++i) {
+  for (int i = 0; i < NPL; ++i) {
     const int e = lane + i * WAVE;
     if (e < HEAD_DIM) o[e] = f32_to_bf16(acc[i] * inv);
   }

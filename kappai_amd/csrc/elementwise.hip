@@ -64,10 +64,97 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const T* __restric
   }
 }
 
+// The same for widths that are multiples of 8 up to 8 * 64 * RN_MAX_VEC: one wave per row, the
+// row kept in registers between the sum of squares and the scaling, 16/32-byte loads and stores,
+// no LDS and no barrier.  This is what decode steps (few rows) run.
+#define RN_MAX_VEC 4   // 8-element groups per lane: D <= 2048 with 64 lanes
+
+__device__ __forceinline__ void load8(const float* p, float* v) {
+  const float4 a = *reinterpret_cast<const float4*>(p);
+  const float4 b = *reinterpret_cast<const float4*>(p + 4);
+  v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+}
+__device__ __forceinline__ void load8(const bf16_t* p, float* v) {
+  const uint4 a = *reinterpret_cast<const uint4*>(p);
+  const uint32_t w[4] = {a.x, a.y, a.z, a.w};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    v[2 * i] = __uint_as_float(w[i] << 16);
+    v[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+  }
+}
+__device__ __forceinline__ void store8(float* p, const float* v) {
+  *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+  *reinterpret_cast<float4*>(p + 4) = make_float4(v[4], v[5], v[6], v[7]);
+}
+__device__ __forceinline__ void store8(bf16_t* p, const float* v) {
+  uint4 o;
+  o.x = (uint32_t)f32_to_bf16(v[0]) | ((uint32_t)f32_to_bf16(v[1]) << 16);
+  o.y = (uint32_t)f32_to_bf16(v[2]) | ((uint32_t)f32_to_bf16(v[3]) << 16);
+  o.z = (uint32_t)f32_to_bf16(v[4]) | ((uint32_t)f32_to_bf16(v[5]) << 16);
+  o.w = (uint32_t)f32_to_bf16(v[6]) | ((uint32_t)f32_to_bf16(v[7]) << 16);
+  *reinterpret_cast<uint4*>(p) = o;
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void add_rmsnorm_wave_kernel(
+    float* __restrict__ resid, const T* __restrict__ delta, const float* __restrict__ w,
+    T* __restrict__ out, const int* __restrict__ rows, int n_rows, int D, float eps,
+    int write_resid) {
+  const int i = blockIdx.x * (blockDim.x / WAVE) + threadIdx.x / WAVE;
+  if (i >= n_rows) return;
+  const int lane = threadIdx.x % WAVE;
+  const int r = rows ? rows[i] : i;
+  float* x = resid + (size_t)r * D;
+  const T* dl = delta ? delta + (size_t)r * D : nullptr;
+  float v[RN_MAX_VEC][8];
+  float ss = 0.f;
+#pragma unroll
+  for (int g = 0; g < RN_MAX_VEC; ++g) {
+    const int j = (g * WAVE + lane) * 8;
+    if (j < D) {
+      load8(x + j, v[g]);
+      if (dl) {
+        float d8[8];
+        load8(dl + j, d8);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[g][e] += d8[e];
+        if (write_resid) store8(x + j, v[g]);
+      }
+#pragma unroll
+      for (int e = 0; e < 8; ++e) ss += v[g][e] * v[g][e];
+    }
+  }
+  ss = wave_sum(ss);
+  const float scale = 1.0f / sqrtf(ss / (float)D + eps);
+#pragma unroll
+  for (int g = 0; g < RN_MAX_VEC; ++g) {
+    const int j = (g * WAVE + lane) * 8;
+    if (j < D) {
+      float w8[8];
+      load8(w + j, w8);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) w8[e] = v[g][e] * scale * w8[e];
+      store8(out + (size_t)i * D + j, w8);
+    }
+  }
+}
+
 extern "C" int kappai_add_rmsnorm(float* resid, const void* delta, const float* w, void* out,
                                   const int* rows, int n_rows, int D, float eps, int write_resid,
                                   int is_bf16, hipStream_t stream) {
   if (n_rows <= 0) return 0;
+  if (D % 8 == 0 && D <= 8 * WAVE * RN_MAX_VEC) {
+    const int wpb = 4;   // waves (rows) a block
+    dim3 grid((n_rows + wpb - 1) / wpb), block(wpb * WAVE);
+    if (is_bf16)
+      hipLaunchKernelGGL(add_rmsnorm_wave_kernel<bf16_t>, grid, block, 0, stream, resid,
+                         (const bf16_t*)delta, w, (bf16_t*)out, rows, n_rows, D, eps, write_resid);
+    else
+      hipLaunchKernelGGL(add_rmsnorm_wave_kernel<float>, grid, block, 0, stream, resid,
+                         (const float*)delta, w, (float*)out, rows, n_rows, D, eps, write_resid);
+    KAPPAI_RETURN_LAUNCH_STATUS();
+  }
   const int threads = D >= 2048 ? 512 : (D >= 512 ? 256 : (D >= 128 ? 128 : 64));
   if (is_bf16)
     hipLaunchKernelGGL(add_rmsnorm_kernel<bf16_t>, dim3(n_rows), dim3(threads), 0, stream, resid,

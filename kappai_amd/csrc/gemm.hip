@@ -6,7 +6,7 @@
 //                    the order k = 0..K-1, so a row's result does not depend on M.
 //   gemm_bf16_tile   bf16 inputs, fp32 accumulation on the matrix cores
 //                    (v_mfma_f32_32x32x16_bf16), 128x128x32 block tiles staged through LDS.
-//   gemm_bf16_skinny M <= 64 (decode): every block streams 16 rows of W once, its four
+//   gemm_bf16_skinny M <= 64 (decode): every block streams 16 rows of W once, its 4 to 16
 //                    waves split K and meet in LDS (v_mfma_f32_16x16x32_bf16).
 #include "common.h"
 
@@ -100,7 +100,12 @@ __device__ __forceinline__ void store_out(bf16_t* p, float v) { *p = f32_to_bf16
 #define T_BK 32
 #define T_LDS (T_BK + 8)  // row stride in bf16: 80 bytes keeps 16-byte alignment, spreads banks
 
-template <typename TO>
+__device__ __forceinline__ float silu_f(float g) { return g / (1.0f + expf(-g)); }
+
+// EPI 1 (SwiGLU): W holds gate and up rows interleaved in groups of 16 (16 gate rows, the 16 up
+// rows of the same columns, ...); the kernel writes silu(gate) * up, N/2 columns wide
+// (kappai: src/backend/cpu/quants.h:369-371, src/recipe/builders.c:344-370).
+template <typename TO, int EPI>
 __global__ __launch_bounds__(256) void gemm_bf16_tile_kernel(const bf16_t* __restrict__ A,
                                                              const bf16_t* __restrict__ W,
                                                              const float* __restrict__ bias,
@@ -166,6 +171,26 @@ __global__ __launch_bounds__(256) void gemm_bf16_tile_kernel(const bf16_t* __res
     __syncthreads();
   }
   // D[m][n] of a 32x32 tile: lane holds column lane%32, rows 8*(v/4) + 4*(lane/32) + v%4
+  if (EPI == 1) {
+    // a 32-column tile is 16 gate columns and their 16 up columns: lane c < 16 holds gate,
+    // lane c + 16 the matching up
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const int c = lane % 32;
+        const int gcol = n0 + wn * 64 + j * 32;          // first interleaved column of the tile
+        const int on = gcol / 2 + c;                     // output column for c < 16
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          const float other = __shfl_xor(acc[i][j][v], 16, WAVE);
+          const int gm = m0 + wm * 64 + i * 32 + 8 * (v / 4) + 4 * (lane / 32) + v % 4;
+          if (c < 16 && gm < M && gcol + c < N)
+            store_out(C + (size_t)gm * ldc + on, silu_f(acc[i][j][v]) * other);
+        }
+      }
+    return;
+  }
 #pragma unroll
   for (int i = 0; i < 2; ++i)
 #pragma unroll
@@ -181,91 +206,134 @@ __global__ __launch_bounds__(256) void gemm_bf16_tile_kernel(const bf16_t* __res
     }
 }
 
-// M <= 16*MT.  Block = 4 waves = 16 columns of the result; wave w takes the k-chunks
-// c = w, w+4, ... of 32 elements.  A fragment: lane holds row lane%16, k-group lane/16;
-// W fragment: lane holds column lane%16, k-group lane/16; result: lane holds column
-// lane%16, rows 4*(lane/16) + v.
-template <typename TO, int MT>
-__global__ __launch_bounds__(256) void gemm_bf16_skinny_kernel(const bf16_t* __restrict__ A,
-                                                               const bf16_t* __restrict__ W,
-                                                               const float* __restrict__ bias,
-                                                               TO* __restrict__ C, int M, int N,
-                                                               int K, int lda, int ldc) {
-  __shared__ float red[4][MT][WAVE][4];
+// M <= 16*MT (decode).  Bound by reading W once: a block owns 16 columns of the result and
+// streams their 16 rows of W; its NW waves split K into contiguous ranges and meet in LDS.
+// Every wave issues SK_UNROLL independent 16-byte loads of W per lane before it consumes
+// them, so that enough bytes are in flight to keep HBM busy.  A fragment: lane holds row
+// lane%16, k-group lane/16; W fragment: lane holds column lane%16, k-group lane/16; result:
+// lane holds column lane%16, rows 4*(lane/16) + v.
+#define SK_UNROLL 8
+
+// EPI 1 (SwiGLU, see the tile kernel): a block owns 16 output columns = 16 gate rows and
+// their 16 up rows of the interleaved W; N is the number of output columns.
+template <typename TO, int MT, int NW, int EPI>
+__global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny_kernel(
+    const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, const float* __restrict__ bias,
+    TO* __restrict__ C, int M, int N, int K, int lda, int ldc) {
+  constexpr int NG = EPI == 1 ? 2 : 1;      // row groups of W a block streams
+  __shared__ float red[NW][NG * MT][WAVE][4];
   const int tid = threadIdx.x;
   const int lane = tid % WAVE, wave = tid / WAVE;
   const int n0 = blockIdx.x * 16;
   const int col = lane % 16, kg = (lane / 16) * 8;
   const int gn = n0 + col;
   const u32x4_t zero = {0u, 0u, 0u, 0u};
-  f32x4_t acc[MT];
+  f32x4_t acc[NG * MT];
 #pragma unroll
-  for (int t = 0; t < MT; ++t) acc[t] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
-  const bf16_t* wrow = W + (size_t)(gn < N ? gn : 0) * K;
-  for (int k0 = wave * 32; k0 < K; k0 += 128) {
-    const int gk = k0 + kg;
-    const bool kin = gk < K;
-    const u32x4_t wv = (kin && gn < N) ? load16(wrow + gk) : zero;
-    u32x4_t av[MT];
+  for (int t = 0; t < NG * MT; ++t) acc[t] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+  // plain: row gn.  SwiGLU: gate row 32*block + col, up row 16 further
+  const size_t wr0 = EPI == 1 ? (size_t)blockIdx.x * 32 + col : (size_t)gn;
+  const bf16_t* wrow = W + (gn < N ? wr0 : 0) * K + kg;
+  const bf16_t* arow[MT];
 #pragma unroll
-    for (int t = 0; t < MT; ++t) {
-      const int gm = t * 16 + col;
-      av[t] = (kin && gm < M) ? load16(A + (size_t)gm * lda + gk) : zero;
+  for (int t = 0; t < MT; ++t) {
+    const int gm = t * 16 + col;
+    arow[t] = A + (size_t)(gm < M ? gm : 0) * lda + kg;
+  }
+  const int kper = ((K + 32 * NW - 1) / (32 * NW)) * 32;
+  const int k0 = wave * kper;
+  const int k1 = min(K, k0 + kper);
+  // loads in flight a lane: U * (NG + MT)
+  constexpr int U = (NG + MT) <= 2 ? SK_UNROLL : ((NG + MT) <= 4 ? 4 : 2);
+  for (int k = k0; k < k1; k += 32 * U) {
+    u32x4_t wv[U][NG], av[U][MT];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int gk = k + 32 * u;
+      const bool kin = gk + kg < k1;
+#pragma unroll
+      for (int r = 0; r < NG; ++r)
+        wv[u][r] = (kin && gn < N) ? load16(wrow + (size_t)r * 16 * K + gk) : zero;
+#pragma unroll
+      for (int t = 0; t < MT; ++t)
+        av[u][t] = (kin && t * 16 + col < M) ? load16(arow[t] + gk) : zero;
     }
 #pragma unroll
-    for (int t = 0; t < MT; ++t)
-      acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(av[t]), as_bf16x8(wv), acc[t], 0,
-                                                       0, 0);
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int r = 0; r < NG; ++r)
+#pragma unroll
+        for (int t = 0; t < MT; ++t)
+          acc[r * MT + t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+              as_bf16x8(av[u][t]), as_bf16x8(wv[u][r]), acc[r * MT + t], 0, 0, 0);
   }
 #pragma unroll
-  for (int t = 0; t < MT; ++t)
+  for (int t = 0; t < NG * MT; ++t)
 #pragma unroll
     for (int v = 0; v < 4; ++v) red[wave][t][lane][v] = acc[t][v];
   __syncthreads();
-  if (wave == 0 && gn < N) {
+  // the first MT waves each sum one row tile over the NW partial results, in a fixed order
+  if (wave < MT && gn < N) {
+    const int t = wave;
     const float bv = bias ? bias[gn] : 0.f;
 #pragma unroll
-    for (int t = 0; t < MT; ++t)
+    for (int v = 0; v < 4; ++v) {
+      const int gm = t * 16 + 4 * (lane / 16) + v;
+      if (gm < M) {
+        float sum = red[0][t][lane][v];
 #pragma unroll
-      for (int v = 0; v < 4; ++v) {
-        const int gm = t * 16 + 4 * (lane / 16) + v;
-        if (gm < M) {
-          const float s = ((red[0][t][lane][v] + red[1][t][lane][v]) + red[2][t][lane][v]) +
-                          red[3][t][lane][v];
-          store_out(C + (size_t)gm * ldc + gn, s + bv);
+        for (int w = 1; w < NW; ++w) sum += red[w][t][lane][v];
+        if (EPI == 1) {
+          float up = red[0][MT + t][lane][v];
+#pragma unroll
+          for (int w = 1; w < NW; ++w) up += red[w][MT + t][lane][v];
+          store_out(C + (size_t)gm * ldc + gn, silu_f(sum) * up);
+        } else {
+          store_out(C + (size_t)gm * ldc + gn, sum + bv);
         }
       }
+    }
   }
 }
 
-template <typename TO>
+template <typename TO, int MT, int NW, int EPI>
+static void launch_skinny(const bf16_t* A, const bf16_t* W, const float* bias, TO* C, int M, int N,
+                          int K, int lda, int ldc, hipStream_t stream) {
+  hipLaunchKernelGGL((gemm_bf16_skinny_kernel<TO, MT, NW, EPI>), dim3((N + 15) / 16),
+                     dim3(NW * WAVE), 0, stream, A, W, bias, C, M, N, K, lda, ldc);
+}
+
+// more waves a block when there are few blocks, so that about 2048 waves or more stream W
+template <typename TO, int MT, int EPI>
+static void launch_skinny_mt(const bf16_t* A, const bf16_t* W, const float* bias, TO* C, int M,
+                             int N, int K, int lda, int ldc, hipStream_t stream) {
+  const int blocks = (N + 15) / 16;
+  constexpr int MAXW = 16 / (MT * (EPI == 1 ? 2 : 1));   // LDS for the partial results
+  if (blocks * 4 >= 2048 || K <= 512 || MAXW <= 4)
+    launch_skinny<TO, MT, 4, EPI>(A, W, bias, C, M, N, K, lda, ldc, stream);
+  else if (blocks * 8 >= 2048 || K <= 1024 || MAXW <= 8)
+    launch_skinny<TO, MT, (MAXW >= 8 ? 8 : 4), EPI>(A, W, bias, C, M, N, K, lda, ldc, stream);
+  else
+    launch_skinny<TO, MT, (MAXW >= 16 ? 16 : 4), EPI>(A, W, bias, C, M, N, K, lda, ldc, stream);
+}
+
+template <typename TO, int EPI>
 static int launch_bf16(const bf16_t* A, const bf16_t* W, const float* bias, TO* C, int M, int N,
-                       int K, int lda, int ldc, hipStream_t stream) {
-  if (M <= 64) {
-    dim3 grid((N + 15) / 16), block(256);
+                       int K, int lda, int ldc, int force_kernel, hipStream_t stream) {
+  // N counts output columns; with the SwiGLU epilogue W has 2N rows
+  if (M <= 64 && force_kernel != 1) {
     const int mt = (M + 15) / 16;
     switch (mt) {
-      case 1:
-        hipLaunchKernelGGL((gemm_bf16_skinny_kernel<TO, 1>), grid, block, 0, stream, A, W, bias, C,
-                           M, N, K, lda, ldc);
-        break;
-      case 2:
-        hipLaunchKernelGGL((gemm_bf16_skinny_kernel<TO, 2>), grid, block, 0, stream, A, W, bias, C,
-                           M, N, K, lda, ldc);
-        break;
-      case 3:
-        hipLaunchKernelGGL((gemm_bf16_skinny_kernel<TO, 3>), grid, block, 0, stream, A, W, bias, C,
-                           M, N, K, lda, ldc);
-        break;
-      default:
-        hipLaunchKernelGGL((gemm_bf16_skinny_kernel<TO, 4>), grid, block, 0, stream, A, W, bias, C,
-                           M, N, K, lda, ldc);
-        break;
+      case 1: launch_skinny_mt<TO, 1, EPI>(A, W, bias, C, M, N, K, lda, ldc, stream); break;
+      case 2: launch_skinny_mt<TO, 2, EPI>(A, W, bias, C, M, N, K, lda, ldc, stream); break;
+      case 3: launch_skinny_mt<TO, 3, EPI>(A, W, bias, C, M, N, K, lda, ldc, stream); break;
+      default: launch_skinny_mt<TO, 4, EPI>(A, W, bias, C, M, N, K, lda, ldc, stream); break;
     }
   } else {
-    dim3 grid((N + T_BN - 1) / T_BN, (M + T_BM - 1) / T_BM);
-    hipLaunchKernelGGL(gemm_bf16_tile_kernel<TO>, grid, dim3(256), 0, stream, A, W, bias, C, M, N,
-                       K, lda, ldc);
+    const int NW_ = EPI == 1 ? 2 * N : N;           // rows of W = columns the tiles run over
+    dim3 grid((NW_ + T_BN - 1) / T_BN, (M + T_BM - 1) / T_BM);
+    hipLaunchKernelGGL((gemm_bf16_tile_kernel<TO, EPI>), grid, dim3(256), 0, stream, A, W, bias, C,
+                       M, NW_, K, lda, ldc);
   }
   KAPPAI_RETURN_LAUNCH_STATUS();
 }
@@ -278,19 +346,20 @@ extern "C" int kappai_gemm_bf16(const void* A, const void* W, const float* bias,
   if (M <= 0 || N <= 0) return 0;
   if ((K % 8) || (lda % 8)) return (int)hipErrorInvalidValue;
   if (force_kernel == 2 && M > 64) return (int)hipErrorInvalidValue;
-  if (force_kernel == 1) {
-    dim3 grid((N + T_BN - 1) / T_BN, (M + T_BM - 1) / T_BM);
-    if (out_is_f32)
-      hipLaunchKernelGGL(gemm_bf16_tile_kernel<float>, grid, dim3(256), 0, stream,
-                         (const bf16_t*)A, (const bf16_t*)W, bias, (float*)C, M, N, K, lda, ldc);
-    else
-      hipLaunchKernelGGL(gemm_bf16_tile_kernel<bf16_t>, grid, dim3(256), 0, stream,
-                         (const bf16_t*)A, (const bf16_t*)W, bias, (bf16_t*)C, M, N, K, lda, ldc);
-    KAPPAI_RETURN_LAUNCH_STATUS();
-  }
   if (out_is_f32)
-    return launch_bf16<float>((const bf16_t*)A, (const bf16_t*)W, bias, (float*)C, M, N, K, lda,
-                              ldc, stream);
-  return launch_bf16<bf16_t>((const bf16_t*)A, (const bf16_t*)W, bias, (bf16_t*)C, M, N, K, lda,
-                             ldc, stream);
+    return launch_bf16<float, 0>((const bf16_t*)A, (const bf16_t*)W, bias, (float*)C, M, N, K, lda,
+                                 ldc, force_kernel, stream);
+  return launch_bf16<bf16_t, 0>((const bf16_t*)A, (const bf16_t*)W, bias, (bf16_t*)C, M, N, K, lda,
+                                ldc, force_kernel, stream);
+}
+
+// C[M, F] = silu(A Wg^T) * (A Wu^T) with W = gate and up rows interleaved in groups of 16,
+// [2F, K]; F must be a multiple of 16.
+extern "C" int kappai_gemm_bf16_swiglu(const void* A, const void* W, void* C, int M, int F, int K,
+                                       int lda, int ldc, int force_kernel, hipStream_t stream) {
+  if (M <= 0 || F <= 0) return 0;
+  if ((K % 8) || (lda % 8) || (F % 16)) return (int)hipErrorInvalidValue;
+  if (force_kernel == 2 && M > 64) return (int)hipErrorInvalidValue;
+  return launch_bf16<bf16_t, 1>((const bf16_t*)A, (const bf16_t*)W, nullptr, (bf16_t*)C, M, F, K,
+                                lda, ldc, force_kernel, stream);
 }

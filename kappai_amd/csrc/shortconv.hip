@@ -69,6 +69,34 @@ __global__ void shortconv_state_kernel(const T* __restrict__ proj, float* __rest
   }
 }
 
+// Every segment is a single row (decode): one thread per (segment, channel) computes the output
+// and shifts the state, which nobody else reads.
+template <typename T>
+__global__ void shortconv_step_kernel(const T* __restrict__ proj, const float* __restrict__ w,
+                                      const float* __restrict__ bias, float* __restrict__ state,
+                                      T* __restrict__ out, const int* __restrict__ seg_pos0,
+                                      const int* __restrict__ seg_slot, int D, int L) {
+  const int c = blockIdx.y * blockDim.x + threadIdx.x;
+  const int t = blockIdx.x;
+  if (c >= D) return;
+  const bool fresh = seg_pos0[t] == 0;
+  const int H = L - 1;
+  float* st = state + ((size_t)seg_slot[t] * D + c) * H;
+  const float* wc = w + (size_t)c * L;
+  const T* p = proj + (size_t)t * 3 * D;
+  const float bx = to_f32(p[c]) * to_f32(p[2 * D + c]);
+  float sum = (bias ? bias[c] : 0.f);
+  float prev = fresh ? 0.f : st[0];
+  for (int k = 0; k < H; ++k) {
+    sum += wc[k] * prev;                       // tap k meets history entry k
+    const float next = (k + 1 < H) ? (fresh ? 0.f : st[k + 1]) : bx;
+    st[k] = next;                              // shift: entry k becomes entry k+1, the last bx
+    prev = next;
+  }
+  sum += wc[H] * bx;
+  from_f32(out + (size_t)t * D + c, to_f32(p[D + c]) * sum);
+}
+
 extern "C" int kappai_shortconv(const void* proj, const float* w, const float* bias, float* state,
                                 void* out, const int* row_seg, const int* seg_start,
                                 const int* seg_pos0, const int* seg_slot, int T, int S, int D,
@@ -77,6 +105,16 @@ extern "C" int kappai_shortconv(const void* proj, const float* w, const float* b
   if (L < 2) return (int)hipErrorInvalidValue;
   const int threads = D >= 256 ? 256 : 64;
   dim3 g1(T, (D + threads - 1) / threads), g2(S, (D + threads - 1) / threads);
+  if (T == S) {   // one row a segment: row t is segment t
+    if (is_bf16)
+      hipLaunchKernelGGL(shortconv_step_kernel<bf16_t>, g1, dim3(threads), 0, stream,
+                         (const bf16_t*)proj, w, bias, state, (bf16_t*)out, seg_pos0, seg_slot, D,
+                         L);
+    else
+      hipLaunchKernelGGL(shortconv_step_kernel<float>, g1, dim3(threads), 0, stream,
+                         (const float*)proj, w, bias, state, (float*)out, seg_pos0, seg_slot, D, L);
+    KAPPAI_RETURN_LAUNCH_STATUS();
+  }
   if (is_bf16) {
     hipLaunchKernelGGL(shortconv_out_kernel<bf16_t>, g1, dim3(threads), 0, stream,
                        (const bf16_t*)proj, w, bias, (const float*)state, (bf16_t*)out, row_seg,

@@ -158,6 +158,43 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] =
     return out
 
 
+SWIGLU_GROUP = 16     # gate and up rows alternate in groups of this many rows
+
+
+def interleave_gate_up(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
+    """The layout ``linear_swiglu`` reads: 16 gate rows, the 16 up rows of the same columns, the
+    next 16 gate rows, ...  [2F, K] from two [F, K] matrices; F must be a multiple of 16."""
+    F, K = gate.shape
+    _need(up.shape == gate.shape and F % SWIGLU_GROUP == 0,
+          f"interleave_gate_up: {tuple(gate.shape)} and {tuple(up.shape)}; F must be a multiple "
+          f"of {SWIGLU_GROUP}")
+    g = gate.reshape(F // SWIGLU_GROUP, 1, SWIGLU_GROUP, K)
+    u = up.reshape(F // SWIGLU_GROUP, 1, SWIGLU_GROUP, K)
+    return torch.cat([g, u], dim=1).reshape(2 * F, K).contiguous()
+
+
+def linear_swiglu(x: torch.Tensor, weight: torch.Tensor, force_kernel: int = 0) -> torch.Tensor:
+    """``silu(x Wg^T) * (x Wu^T)`` in one kernel: ``weight`` [2F, K] holds the gate and up
+    matrices interleaved by ``interleave_gate_up``; bfloat16 only.  Returns [M, F]."""
+    _gpu("x", x, BF16, contiguous=False)
+    _gpu("weight", weight, BF16)
+    _need(x.dim() == 2 and weight.dim() == 2 and x.shape[1] == weight.shape[1]
+          and weight.shape[0] % (2 * SWIGLU_GROUP) == 0,
+          f"linear_swiglu: x {tuple(x.shape)}, weight {tuple(weight.shape)}")
+    _need(x.stride(1) == 1 or x.shape[1] == 1, "linear_swiglu: x must have unit stride along K")
+    M, K = x.shape
+    F = weight.shape[0] // 2
+    lda = x.stride(0) if M > 1 else K
+    _need(K % 8 == 0 and lda % 8 == 0 and x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0,
+          f"linear_swiglu: K ({K}) and the row stride ({lda}) must be multiples of 8 and the "
+          f"tensors 16-byte aligned")
+    out = torch.empty((M, F), dtype=BF16, device=x.device)
+    check(library("gemm").kappai_gemm_bf16_swiglu(
+        _ptr(x), _ptr(weight), _ptr(out), _c_int(M), _c_int(F), _c_int(K), _c_int(lda), _c_int(F),
+        _c_int(force_kernel), _stream()), "gemm_bf16_swiglu")
+    return out
+
+
 # ---------------------------------------------------------------------------------------
 def shortconv(proj: torch.Tensor, taps: torch.Tensor, bias: Optional[torch.Tensor],
               state: torch.Tensor, row_seg: torch.Tensor, seg_start: torch.Tensor,

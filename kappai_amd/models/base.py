@@ -95,6 +95,11 @@ class Model:
         return n + self.final_norm.weight_bytes() + self.head.weight_bytes()
 
     @property
+    def capturable(self) -> bool:
+        """True if every part allows decode steps to be captured in HIP graphs."""
+        return all(getattr(p, "capturable", True) for p in self._parts())
+
+    @property
     def vocab_size(self) -> int:
         return self.config.vocab_size
 

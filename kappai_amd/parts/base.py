@@ -23,6 +23,11 @@ from ..weights.spec import TensorSpec
 class Part:
     """Anything that owns tensors of the checkpoint."""
 
+    # True if ``forward`` only launches GPU work whose shapes depend on the batch's sizes, not
+    # on its contents, so that a decode step may be captured in a HIP graph and replayed.  A
+    # part that reads the batch's tables on the host sets this to False.
+    capturable = True
+
     def tensor_specs(self) -> List[TensorSpec]:
         """Full names, shapes and roles of the tensors this part reads from the file."""
         return []

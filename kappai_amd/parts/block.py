@@ -21,6 +21,10 @@ class PreNormBlock(Block):
     def _parts(self):
         return (self.mixer_norm, self.mixer, self.ffn_norm, self.feed_forward)
 
+    @property
+    def capturable(self) -> bool:
+        return all(p.capturable for p in self._parts())
+
     def tensor_specs(self) -> List[TensorSpec]:
         return [s for p in self._parts() for s in p.tensor_specs()]
 

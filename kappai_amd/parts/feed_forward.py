@@ -1,6 +1,7 @@
 """SwiGLU feed-forward: ``W2 (silu(W1 x) * W3 x)`` (kappai: src/recipe/builders.c:344-370,
 383-386; silu at src/backend/cpu/quants.h:369-371).  W1 and W3 are stacked into one
-product."""
+product; in bfloat16 their rows are interleaved so that the product's epilogue applies the
+gate and the [T, 2F] intermediate never reaches memory."""
 from __future__ import annotations
 
 from typing import Dict, List
@@ -18,6 +19,7 @@ class SwiGLU(FeedForward):
         n = {"gate": "w1", "up": "w3", "down": "w2"}
         n.update(names or {})
         self.width, self.hidden, self.dtype = width, hidden, dtype
+        self.fused = False
         self.gate_up = Linear([prefix + n["gate"], prefix + n["up"]], width, [hidden, hidden])
         self.down = Linear([prefix + n["down"]], hidden, [width])
 
@@ -27,8 +29,15 @@ class SwiGLU(FeedForward):
     def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
         self.gate_up.bind(tensors)
         self.down.bind(tensors)
+        w = self.gate_up.weight
+        self.fused = (w.dtype == torch.bfloat16 and self.hidden % ops.SWIGLU_GROUP == 0
+                      and self.width % 8 == 0)
+        if self.fused:
+            self.gate_up.weight = ops.interleave_gate_up(w[:self.hidden], w[self.hidden:])
 
     def forward(self, x, batch):
+        if self.fused and x.dtype == torch.bfloat16:
+            return self.down.forward(ops.linear_swiglu(x, self.gate_up.weight))
         return self.down.forward(ops.swiglu(self.gate_up.forward(x)))
 
     def weight_bytes(self) -> int:

@@ -38,6 +38,7 @@ class RotaryEncoding(PositionEncoding):
             raise ValueError(f"rot_dim {self.rot_dim} must be even and at most head_dim {head_dim}")
         self.mode = ops.ROT_HALF if pairing == "half" else ops.ROT_INTERLEAVED
         self._rotation: Optional[Rotation] = None
+        self._retired = []      # earlier, shorter tables: captured graphs may still read them
 
     def tables(self, n_positions: int):
         half = self.rot_dim // 2
@@ -53,6 +54,8 @@ class RotaryEncoding(PositionEncoding):
             while n <= max_position:
                 n *= 2
             c, s = self.tables(n)
+            if r is not None:
+                self._retired.append(r)
             self._rotation = Rotation(torch.from_numpy(c).to(device), torch.from_numpy(s).to(device),
                                       self.rot_dim, self.mode)
         return self._rotation

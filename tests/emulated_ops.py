@@ -50,6 +50,23 @@ def linear(x, weight, bias=None, out_dtype=None, force_kernel=0):
     return y.to(out_dtype)
 
 
+SWIGLU_GROUP = 16
+
+
+def interleave_gate_up(gate, up):
+    F, K = gate.shape
+    g = gate.reshape(F // SWIGLU_GROUP, 1, SWIGLU_GROUP, K)
+    u = up.reshape(F // SWIGLU_GROUP, 1, SWIGLU_GROUP, K)
+    return torch.cat([g, u], dim=1).reshape(2 * F, K).contiguous()
+
+
+def linear_swiglu(x, weight, force_kernel=0):
+    F = weight.shape[0] // 2
+    y = (x.to(F32) @ weight.to(F32).T).reshape(x.shape[0], F // SWIGLU_GROUP, 2, SWIGLU_GROUP)
+    g, u = y[:, :, 0, :].reshape(-1, F), y[:, :, 1, :].reshape(-1, F)
+    return (g / (1.0 + torch.exp(-g)) * u).to(x.dtype)
+
+
 def shortconv(proj, taps, bias, state, row_seg, seg_start, seg_pos0, seg_slot):
     T = proj.shape[0]
     D, L = taps.shape
@@ -163,7 +180,8 @@ def repeat_penalty(logits, row_start, tokens, penalty):
                 logits[r, tok] = logits[r, tok] / pen if logits[r, tok] > 0 else logits[r, tok] * pen
 
 
-ALL = ["embed_rows", "add_rmsnorm", "add_residual", "swiglu", "cast", "linear", "shortconv",
+ALL = ["embed_rows", "add_rmsnorm", "add_residual", "swiglu", "cast", "linear", "linear_swiglu",
+       "interleave_gate_up", "shortconv",
        "qk_norm_rope_store", "paged_attention", "sample_rows", "repeat_penalty"]
 
 

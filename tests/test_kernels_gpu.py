@@ -124,6 +124,19 @@ def test_linear_bfloat16(ops, M, N, K, out_dtype):
         close(got.float(), want + b.double(), tol, f"kernel {force} with bias")
 
 
+@pytest.mark.parametrize("M,F,K", [(1, 16, 64), (8, 192, 64), (16, 320, 96), (33, 208, 120),
+                                   (64, 8192, 2048), (65, 320, 96), (200, 1008, 256)])
+def test_linear_swiglu(ops, M, F, K):
+    x, wg, wu = rand((M, K), BF16, 16), rand((F, K), BF16, 17, 0.2), rand((F, K), BF16, 18, 0.2)
+    w = ops.interleave_gate_up(wg.to(DEV), wu.to(DEV))
+    assert torch.equal(w.cpu(), ref.interleave_gate_up(wg, wu))
+    g, u = x.double() @ wg.double().T, x.double() @ wu.double().T
+    want = g / (1 + torch.exp(-g)) * u
+    for force in ([0, 1, 2] if M <= 64 else [0]):
+        got = ops.linear_swiglu(x.to(DEV), w, force_kernel=force)
+        close(got.float(), want, BF16_ULP, f"kernel {force}")
+
+
 def test_linear_views_and_mixed_storage(ops):
     # x as the leading columns of a wider buffer (a row stride), as attention hands q over
     wide = rand((20, 96 + 40), BF16, 12).to(DEV)

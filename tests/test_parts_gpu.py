@@ -160,6 +160,8 @@ def test_toy_mixer_with_its_own_state_and_a_shared_cache():
     class RunningMean(Mixer):
         """out_t = W * mean(x_0..x_t): state [width + 1] = (sum, count), float32."""
 
+        capturable = False      # it walks the segments on the host
+
         def __init__(self, prefix, width, dtype):
             self.width, self.dtype = width, dtype
             self.proj = Linear([prefix + "proj"], width, [width])

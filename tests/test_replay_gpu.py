@@ -142,3 +142,30 @@ def test_trace_run_program(tmp_path, model_dirs, dtype):
     tol = tolerance(model_dirs["A"], requests, dtype)
     err, where = worst_error(got, ref)
     assert err < tol, (err, tol, where, first_bad(got, ref, tol))
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_decode_graphs_replay_what_eager_steps_compute(tmp_path, model_dirs, dtype):
+    """Steps of single decoded tokens are replayed from captured HIP graphs.  Every replay, with
+    eager prompt portions of other requests between them, must give bit for bit what the same
+    step gives without graphs."""
+    from kappai_amd.engine.replay import TraceReplayer, make_replay_cache
+    from kappai_amd.engine.step import StepRunner
+    cfg = TINY["B"][0]
+    requests = make_requests(cfg["vocab_size"], [40, 44, 91], seed=14)
+    plans = {"r0": (0, [10] + [1] * 30), "r1": (0, [14] + [1] * 30),
+             "r2": (12, [20, 1, 1, 1, 30, 1, 1, 1, 1, 1, 33])}
+    steps, index, peak = schedules.build(requests, plans)
+    results = {}
+    for graphs in (False, True):
+        model = gpu_model(model_dirs["B"], dtype)
+        cache = make_replay_cache(model, peak)
+        cache.allocate_storage(model.dtype, "cuda:0", poison=True)
+        runner = StepRunner(model, cache, "cuda:0", decode_graphs=graphs)
+        rep = TraceReplayer(runner, tmp_path / f"g{graphs}")
+        results[graphs] = [rep.run_step(obj) for obj in steps]
+        assert (runner.graph_replays > 15) == graphs
+    for a, b in zip(results[False], results[True]):
+        assert (a is None) == (b is None)
+        if a is not None:
+            assert np.array_equal(a, b)
