@@ -61,6 +61,28 @@ __device__ __forceinline__ u32x2_t load_vt4(const bf16_t* __restrict__ vt_pool,
   return keep == 15 ? v : mask4(v, keep);
 }
 
+// the same with the page already looked up
+__device__ __forceinline__ u32x2_t load_vt4_pg(const bf16_t* __restrict__ vt_pool, int page, int G,
+                                               int g, int ps, int dd, int key0, int lo, int hi) {
+  u32x2_t z = {0u, 0u};
+  if (dd >= HEAD_DIM || key0 > hi || key0 + 3 < lo || page < 0) return z;
+  const bf16_t* p = vt_pool + (((size_t)page * G + g) * HEAD_DIM + dd) * ps + key0 % ps;
+  u32x2_t v = *reinterpret_cast<const u32x2_t*>(p);
+  int keep = 0;
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+    if (key0 + i >= lo && key0 + i <= hi) keep |= 1 << i;
+  return keep == 15 ? v : mask4(v, keep);
+}
+
+__device__ __forceinline__ u32x4_t load_k8_pg(const bf16_t* __restrict__ k_pool, int page, int G,
+                                              int g, int ps, int key, int d0, int lo, int hi) {
+  u32x4_t z = {0u, 0u, 0u, 0u};
+  if (d0 >= HEAD_DIM || key < lo || key > hi || page < 0) return z;
+  return *reinterpret_cast<const u32x4_t*>(
+      k_pool + (((size_t)page * G + g) * ps + key % ps) * HEAD_DIM + d0);
+}
+
 // eight consecutive d of key `key` starting at d0; zero outside [lo, hi] or beyond the head
 __device__ __forceinline__ u32x4_t load_k8(const bf16_t* __restrict__ k_pool,
                                            const int* __restrict__ bt, int G, int g, int ps,
@@ -192,6 +214,8 @@ __global__ __launch_bounds__(64) void attn_prefill_kernel(
 // ---------------------------------------------------------------------------------------
 #define D_KS ((HEAD_DIM + 31) / 32)     // k-steps of S^T over d (32 each)
 #define D_MT (HEAD_DIM / 16)            // row tiles of O^T over d
+// keys whose loads a wave has in flight at once (their registers: keys * HEAD_DIM / 64)
+#define D_KPW (HEAD_DIM <= 64 ? 128 : (HEAD_DIM <= 128 ? 64 : 32))
 
 __global__ __launch_bounds__(64) void attn_decode_kernel(
     const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ k_pool,
@@ -229,86 +253,86 @@ __global__ __launch_bounds__(64) void attn_decode_kernel(
   float m_run = -INFINITY, l_run = 0.f;
   const float sc = scale * LOG2E;
 
-  // The loads of the next 32 keys are issued before the current 32 are worked on, so that
-  // their latency hides behind the matrix products and the softmax (head sizes up to 128;
-  // beyond that the registers do not suffice and the loop runs without the look-ahead).
-  constexpr bool AHEAD = HEAD_DIM <= 128;
-  u32x4_t kf[2][2][D_KS];
-  u32x2_t va[2][D_MT], vb[2][D_MT];
-  auto fetch = [&](int buf, int kb) {
+  // A wave takes its keys in chunks of D_KPW: first the chunk's page ids (one load, handed
+  // round by shuffles), then every key and value load of the chunk at once, then the matrix
+  // products and the softmax: two memory round trips a chunk, whatever its length.
+  constexpr int NCH = D_KPW / 32;
+  for (int c0 = k_begin; c0 < k_end; c0 += D_KPW) {
+    const int first_page = c0 / ps;
+    int my_page = -1;
+    if (first_page + lane < max_blocks && (first_page + lane) * ps <= hi)
+      my_page = bt[first_page + lane];
+    u32x4_t kf[NCH][2][D_KS];
+    u32x2_t va[NCH][D_MT], vb[NCH][D_MT];
 #pragma unroll
-    for (int tt = 0; tt < 2; ++tt)
+    for (int c = 0; c < NCH; ++c) {
+      const int kb = c0 + 32 * c;
 #pragma unroll
-      for (int ks = 0; ks < D_KS; ++ks)
-        kf[buf][tt][ks] = load_k8(k_pool, bt, G, g, ps, kb + 16 * tt + col, 32 * ks + 8 * kg, lo, hi);
+      for (int tt = 0; tt < 2; ++tt) {
+        const int key = kb + 16 * tt + col;
+        const int page = __shfl(my_page, min(key / ps - first_page, WAVE - 1), WAVE);
 #pragma unroll
-    for (int mt = 0; mt < D_MT; ++mt) {
-      va[buf][mt] = load_vt4(vt_pool, bt, G, g, ps, 16 * mt + col, kb + 4 * kg, lo, hi);
-      vb[buf][mt] = load_vt4(vt_pool, bt, G, g, ps, 16 * mt + col, kb + 16 + 4 * kg, lo, hi);
-    }
-  };
-  auto work = [&](int buf, int kb) {
-    f32x4_t s[2];
-#pragma unroll
-    for (int tt = 0; tt < 2; ++tt) {
-      s[tt] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int ks = 0; ks < D_KS; ++ks)
-        s[tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_frag(kf[buf][tt][ks]), qf[ks], s[tt], 0,
-                                                        0, 0);
-    }
-    // lane holds, for head `col`, keys kb + 16*tt + 4*kg + v
-    float mloc = -INFINITY;
-#pragma unroll
-    for (int tt = 0; tt < 2; ++tt)
-#pragma unroll
-      for (int v = 0; v < 4; ++v) {
-        const int key = kb + 16 * tt + 4 * kg + v;
-        const bool ok = key >= lo && key <= hi;
-        s[tt][v] = ok ? s[tt][v] * sc : -INFINITY;
-        mloc = fmaxf(mloc, s[tt][v]);
+        for (int ks = 0; ks < D_KS; ++ks)
+          kf[c][tt][ks] = load_k8_pg(k_pool, page, G, g, ps, key, 32 * ks + 8 * kg, lo, hi);
       }
-    mloc = fmaxf(mloc, __shfl_xor(mloc, 16, WAVE));
-    mloc = fmaxf(mloc, __shfl_xor(mloc, 32, WAVE));
-    const float m_new = fmaxf(m_run, mloc);
-    const float m_safe = m_new == -INFINITY ? 0.f : m_new;
-    const float corr = exp2f(m_run - m_safe);
-    float lsum = 0.f;
+      const int pa = __shfl(my_page, min((kb + 4 * kg) / ps - first_page, WAVE - 1), WAVE);
+      const int pb = __shfl(my_page, min((kb + 16 + 4 * kg) / ps - first_page, WAVE - 1), WAVE);
 #pragma unroll
-    for (int tt = 0; tt < 2; ++tt)
-#pragma unroll
-      for (int v = 0; v < 4; ++v) {
-        s[tt][v] = exp2f(s[tt][v] - m_safe);
-        lsum += s[tt][v];
-      }
-    lsum += __shfl_xor(lsum, 16, WAVE);
-    lsum += __shfl_xor(lsum, 32, WAVE);
-    l_run = l_run * corr + lsum;
-    m_run = m_new;
-    const u32x4_t pw = {pack_bf16(s[0][0], s[0][1]), pack_bf16(s[0][2], s[0][3]),
-                        pack_bf16(s[1][0], s[1][1]), pack_bf16(s[1][2], s[1][3])};
-    const bf16x8_t pf = as_frag(pw);
-#pragma unroll
-    for (int mt = 0; mt < D_MT; ++mt) {
-      const u32x4_t vw = {va[buf][mt].x, va[buf][mt].y, vb[buf][mt].x, vb[buf][mt].y};
-      o[mt] = o[mt] * corr;
-      o[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_frag(vw), pf, o[mt], 0, 0, 0);
-    }
-  };
-  if (AHEAD) {
-    if (k_begin < k_end) fetch(0, k_begin);
-    for (int kb = k_begin; kb < k_end; kb += 64) {
-      if (kb + 32 < k_end) fetch(1, kb + 32);
-      work(0, kb);
-      if (kb + 32 < k_end) {
-        if (kb + 64 < k_end) fetch(0, kb + 64);
-        work(1, kb + 32);
+      for (int mt = 0; mt < D_MT; ++mt) {
+        va[c][mt] = load_vt4_pg(vt_pool, pa, G, g, ps, 16 * mt + col, kb + 4 * kg, lo, hi);
+        vb[c][mt] = load_vt4_pg(vt_pool, pb, G, g, ps, 16 * mt + col, kb + 16 + 4 * kg, lo, hi);
       }
     }
-  } else {
-    for (int kb = k_begin; kb < k_end; kb += 32) {
-      fetch(0, kb);
-      work(0, kb);
+#pragma unroll
+    for (int c = 0; c < NCH; ++c) {
+      const int kb = c0 + 32 * c;
+      if (kb >= k_end) break;
+      f32x4_t s[2];
+#pragma unroll
+      for (int tt = 0; tt < 2; ++tt) {
+        s[tt] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int ks = 0; ks < D_KS; ++ks)
+          s[tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_frag(kf[c][tt][ks]), qf[ks], s[tt], 0,
+                                                          0, 0);
+      }
+      // lane holds, for head `col`, keys kb + 16*tt + 4*kg + v
+      float mloc = -INFINITY;
+#pragma unroll
+      for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+          const int key = kb + 16 * tt + 4 * kg + v;
+          const bool ok = key >= lo && key <= hi;
+          s[tt][v] = ok ? s[tt][v] * sc : -INFINITY;
+          mloc = fmaxf(mloc, s[tt][v]);
+        }
+      mloc = fmaxf(mloc, __shfl_xor(mloc, 16, WAVE));
+      mloc = fmaxf(mloc, __shfl_xor(mloc, 32, WAVE));
+      const float m_new = fmaxf(m_run, mloc);
+      const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+      const float corr = exp2f(m_run - m_safe);
+      float lsum = 0.f;
+#pragma unroll
+      for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+          s[tt][v] = exp2f(s[tt][v] - m_safe);
+          lsum += s[tt][v];
+        }
+      lsum += __shfl_xor(lsum, 16, WAVE);
+      lsum += __shfl_xor(lsum, 32, WAVE);
+      l_run = l_run * corr + lsum;
+      m_run = m_new;
+      const u32x4_t pw = {pack_bf16(s[0][0], s[0][1]), pack_bf16(s[0][2], s[0][3]),
+                          pack_bf16(s[1][0], s[1][1]), pack_bf16(s[1][2], s[1][3])};
+      const bf16x8_t pf = as_frag(pw);
+#pragma unroll
+      for (int mt = 0; mt < D_MT; ++mt) {
+        const u32x4_t vw = {va[c][mt].x, va[c][mt].y, vb[c][mt].x, vb[c][mt].y};
+        o[mt] = o[mt] * corr;
+        o[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_frag(vw), pf, o[mt], 0, 0, 0);
+      }
     }
   }
   if (!head_ok) return;
@@ -322,15 +346,18 @@ __global__ __launch_bounds__(64) void attn_decode_kernel(
     *reinterpret_cast<f32x4_t*>(po + 16 * mt + 4 * kg) = o[mt];
 }
 
-// out[t, h, :] = sum_s o_s 2^(m_s - M) / sum_s l_s 2^(m_s - M).  The weights of up to 64
-// splits at a time are computed one per lane; the sums over d then read independent rows.
-__global__ __launch_bounds__(64) void attn_merge_kernel(const float* __restrict__ part_o,
-                                                        const float* __restrict__ part_ml,
-                                                        bf16_t* __restrict__ out, int out_stride,
-                                                        int H, int n_splits) {
-  const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
-  const size_t base = ((size_t)t * H + h) * n_splits;
+// out[t, h, :] = sum_s o_s 2^(m_s - M) / sum_s l_s 2^(m_s - M).  Four waves share the splits
+// (wave w takes s = w, w+4, ...); each computes its splits' weights one per lane.
+#define MERGE_WAVES 4
+__global__ __launch_bounds__(MERGE_WAVES * WAVE) void attn_merge_kernel(
+    const float* __restrict__ part_o, const float* __restrict__ part_ml,
+    bf16_t* __restrict__ out, int out_stride, int H, int n_splits) {
   constexpr int NPL = (HEAD_DIM + WAVE - 1) / WAVE;
+  __shared__ float sh_acc[MERGE_WAVES][NPL * WAVE];
+  __shared__ float sh_l[MERGE_WAVES];
+  const int t = blockIdx.x, h = blockIdx.y;
+  const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE;
+  const size_t base = ((size_t)t * H + h) * n_splits;
   float M = -INFINITY;
   for (int s = lane; s < n_splits; s += WAVE) M = fmaxf(M, part_ml[2 * (base + s)]);
   M = wave_max(M);
@@ -338,8 +365,9 @@ __global__ __launch_bounds__(64) void attn_merge_kernel(const float* __restrict_
   float acc[NPL];
 #pragma unroll
   for (int i = 0; i < NPL; ++i) acc[i] = 0.f;
-  for (int s0 = 0; s0 < n_splits; s0 += WAVE) {
-    const int s = s0 + lane;
+  // this wave's splits, 64 at a time: split index s = wave + MERGE_WAVES * j
+  for (int j0 = 0; wave + MERGE_WAVES * j0 < n_splits; j0 += WAVE) {
+    const int s = wave + MERGE_WAVES * (j0 + lane);
     float wgt = 0.f, l = 0.f;
     if (s < n_splits) {
       const float m = part_ml[2 * (base + s)];
@@ -347,25 +375,35 @@ __global__ __launch_bounds__(64) void attn_merge_kernel(const float* __restrict_
       l = part_ml[2 * (base + s) + 1] * wgt;
     }
     L += wave_sum(l);
-    const int n = min(WAVE, n_splits - s0);
-#pragma unroll 4
-    for (int k = 0; k < n; ++k) {
+    for (int k = 0; k < WAVE; ++k) {
+      const int sk = wave + MERGE_WAVES * (j0 + k);
+      if (sk >= n_splits) break;
       const float wk = __shfl(wgt, k, WAVE);
 #pragma unroll
       for (int i = 0; i < NPL; ++i) {
         const int e = lane + i * WAVE;
-        if (e < HEAD_DIM) acc[i] = fmaf(part_o[(base + s0 + k) * HEAD_DIM + e], wk, acc[i]);
+        if (e < HEAD_DIM) acc[i] = fmaf(part_o[(base + sk) * HEAD_DIM + e], wk, acc[i]);
       }
     }
   }
+#pragma unroll
+  for (int i = 0; i < NPL; ++i) sh_acc[wave][i * WAVE + lane] = acc[i];
+  if (lane == 0) sh_l[wave] = L;
+  __syncthreads();
+  if (wave != 0) return;
+  L = (sh_l[0] + sh_l[1]) + (sh_l[2] + sh_l[3]);
   const float inv = L > 0.f ? 1.0f / L : 0.f;
   bf16_t* o = out + (size_t)t * out_stride + (size_t)h * HEAD_DIM;
 #pragma unroll
   for (int i = 0; i < NPL; ++i) {
     const int e = lane + i * WAVE;
-    if (e < HEAD_DIM) o[e] = f32_to_bf16(acc[i] * inv);
+    const float v = (sh_acc[0][i * WAVE + lane] + sh_acc[1][i * WAVE + lane]) +
+                    (sh_acc[2][i * WAVE + lane] + sh_acc[3][i * WAVE + lane]);
+    if (e < HEAD_DIM) o[e] = f32_to_bf16(v * inv);
   }
 }
+
+extern "C" int kappai_attn_keys_per_wave(void) { return D_KPW; }
 
 extern "C" int kappai_attn_head_dim(void) { return HEAD_DIM; }
 
@@ -392,13 +430,14 @@ extern "C" int kappai_attn_decode(const void* q, int q_stride, const void* k_poo
                                   int n_splits, hipStream_t stream) {
   if (T <= 0) return 0;
   if (ps % 16 || G < 1 || H % G || H / G > 16 || G > 65535 || n_splits < 1 || n_splits > 65535 ||
-      keys_per_split < 32 || keys_per_split % 32 || (q_stride % 8))
+      keys_per_split < D_KPW || keys_per_split % D_KPW || (q_stride % 8))
     return (int)hipErrorInvalidValue;
   hipLaunchKernelGGL(attn_decode_kernel, dim3(T, G, n_splits), dim3(WAVE), 0, stream,
                      (const bf16_t*)q, q_stride, (const bf16_t*)k_pool, (const bf16_t*)vt_pool,
                      part_o, part_ml, row_pos, row_seg, block_tables, max_blocks, H, G, ps, window,
                      scale, keys_per_split, n_splits);
-  hipLaunchKernelGGL(attn_merge_kernel, dim3(T, H), dim3(WAVE), 0, stream, (const float*)part_o,
-                     (const float*)part_ml, (bf16_t*)out, out_stride, H, n_splits);
+  hipLaunchKernelGGL(attn_merge_kernel, dim3(T, H), dim3(MERGE_WAVES * WAVE), 0, stream,
+                     (const float*)part_o, (const float*)part_ml, (bf16_t*)out, out_stride, H,
+                     n_splits);
   KAPPAI_RETURN_LAUNCH_STATUS();
 }

@@ -33,24 +33,25 @@ extern "C" int kappai_embed_rows(const int* ids, const void* table, int table_is
 // RMSNorm with the residual sum folded in:
 //   x = resid[r] (+ delta[r]);  if write_resid: resid[r] = x;
 //   out[i] = x * rsqrt(mean(x^2) + eps) * w           (src/backend/cpu/scalar/quants.c:1507-1512)
-// r = rows ? rows[i] : i.  Sum of squares and scaling in float.
+// r = rows ? rows[i] : i.  Sum of squares and scaling in float.  delta may be n_part partial
+// sums (a product split over K), `pstride` elements apart; they are added in order.
 // ---------------------------------------------------------------------------------------
-template <typename T>
-__global__ void add_rmsnorm_kernel(float* __restrict__ resid, const T* __restrict__ delta,
-                                   const float* __restrict__ w, T* __restrict__ out,
-                                   const int* __restrict__ rows, int D, float eps,
-                                   int write_resid) {
+template <typename T, typename TD>
+__global__ void add_rmsnorm_kernel(float* __restrict__ resid, const TD* __restrict__ delta,
+                                   int n_part, size_t pstride, const float* __restrict__ w,
+                                   T* __restrict__ out, const int* __restrict__ rows, int D,
+                                   float eps, int write_resid) {
   __shared__ float red[16];
   const int i = blockIdx.x;
   const int r = rows ? rows[i] : i;
   float* x = resid + (size_t)r * D;
-  const T* dl = delta ? delta + (size_t)r * D : nullptr;
+  const TD* dl = delta ? delta + (size_t)r * D : nullptr;
   T* o = out + (size_t)i * D;
   float ss = 0.f;
   for (int j = threadIdx.x; j < D; j += blockDim.x) {
     float v = x[j];
     if (dl) {
-      v += to_f32(dl[j]);
+      for (int p = 0; p < n_part; ++p) v += to_f32(dl[p * pstride + j]);
       if (write_resid) x[j] = v;
     }
     ss += v * v;
@@ -59,16 +60,15 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const T* __restric
   const float scale = 1.0f / sqrtf(ss / (float)D + eps);
   for (int j = threadIdx.x; j < D; j += blockDim.x) {
     float v = x[j];
-    if (dl && !write_resid) v += to_f32(dl[j]);
+    if (dl && !write_resid)
+      for (int p = 0; p < n_part; ++p) v += to_f32(dl[p * pstride + j]);
     from_f32(o + j, v * scale * w[j]);
   }
 }
 
-// The same for widths that are multiples of 8 up to 8 * 64 * RN_MAX_VEC: one wave per row, the
-// row kept in registers between the sum of squares and the scaling, 16/32-byte loads and stores,
-// no LDS and no barrier.  This is what decode steps (few rows) run.
-#define RN_MAX_VEC 4   // 8-element groups per lane: D <= 2048 with 64 lanes
-
+// The same for widths that are multiples of 8 up to 8192: one block per row, eight elements per
+// thread kept in registers between the sum of squares and the scaling, 16/32-byte loads and
+// stores, all loads (the row, every partial sum, the weights) issued before anything waits.
 __device__ __forceinline__ void load8(const float* p, float* v) {
   const float4 a = *reinterpret_cast<const float4*>(p);
   const float4 b = *reinterpret_cast<const float4*>(p + 4);
@@ -96,72 +96,81 @@ __device__ __forceinline__ void store8(bf16_t* p, const float* v) {
   *reinterpret_cast<uint4*>(p) = o;
 }
 
-template <typename T>
-__global__ __launch_bounds__(256) void add_rmsnorm_wave_kernel(
-    float* __restrict__ resid, const T* __restrict__ delta, const float* __restrict__ w,
-    T* __restrict__ out, const int* __restrict__ rows, int n_rows, int D, float eps,
-    int write_resid) {
-  const int i = blockIdx.x * (blockDim.x / WAVE) + threadIdx.x / WAVE;
-  if (i >= n_rows) return;
-  const int lane = threadIdx.x % WAVE;
+#define RN_MAX_PART 8
+
+template <typename T, typename TD>
+__global__ __launch_bounds__(1024) void add_rmsnorm_row_kernel(
+    float* __restrict__ resid, const TD* __restrict__ delta, int n_part, size_t pstride,
+    const float* __restrict__ w, T* __restrict__ out, const int* __restrict__ rows, int D,
+    float eps, int write_resid) {
+  __shared__ float red[16];
+  const int i = blockIdx.x;
   const int r = rows ? rows[i] : i;
+  const int j = threadIdx.x * 8;
+  const bool in = j < D;
   float* x = resid + (size_t)r * D;
-  const T* dl = delta ? delta + (size_t)r * D : nullptr;
-  float v[RN_MAX_VEC][8];
+  const TD* dl = delta ? delta + (size_t)r * D : nullptr;
+  float v[8], w8[8], d8[RN_MAX_PART][8];
   float ss = 0.f;
+  if (in) {
+    load8(w + j, w8);
+    load8(x + j, v);
+    if (dl) {
 #pragma unroll
-  for (int g = 0; g < RN_MAX_VEC; ++g) {
-    const int j = (g * WAVE + lane) * 8;
-    if (j < D) {
-      load8(x + j, v[g]);
-      if (dl) {
-        float d8[8];
-        load8(dl + j, d8);
+      for (int p = 0; p < RN_MAX_PART; ++p)
+        if (p < n_part) load8(dl + p * pstride + j, d8[p]);
 #pragma unroll
-        for (int e = 0; e < 8; ++e) v[g][e] += d8[e];
-        if (write_resid) store8(x + j, v[g]);
-      }
+      for (int p = 0; p < RN_MAX_PART; ++p)
+        if (p < n_part)
 #pragma unroll
-      for (int e = 0; e < 8; ++e) ss += v[g][e] * v[g][e];
+          for (int e = 0; e < 8; ++e) v[e] += d8[p][e];
+      if (write_resid) store8(x + j, v);
     }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) ss += v[e] * v[e];
   }
-  ss = wave_sum(ss);
+  ss = block_sum(ss, red);
   const float scale = 1.0f / sqrtf(ss / (float)D + eps);
+  if (in) {
 #pragma unroll
-  for (int g = 0; g < RN_MAX_VEC; ++g) {
-    const int j = (g * WAVE + lane) * 8;
-    if (j < D) {
-      float w8[8];
-      load8(w + j, w8);
-#pragma unroll
-      for (int e = 0; e < 8; ++e) w8[e] = v[g][e] * scale * w8[e];
-      store8(out + (size_t)i * D + j, w8);
-    }
+    for (int e = 0; e < 8; ++e) w8[e] = v[e] * scale * w8[e];
+    store8(out + (size_t)i * D + j, w8);
   }
 }
 
-extern "C" int kappai_add_rmsnorm(float* resid, const void* delta, const float* w, void* out,
-                                  const int* rows, int n_rows, int D, float eps, int write_resid,
-                                  int is_bf16, hipStream_t stream) {
-  if (n_rows <= 0) return 0;
-  if (D % 8 == 0 && D <= 8 * WAVE * RN_MAX_VEC) {
-    const int wpb = 4;   // waves (rows) a block
-    dim3 grid((n_rows + wpb - 1) / wpb), block(wpb * WAVE);
-    if (is_bf16)
-      hipLaunchKernelGGL(add_rmsnorm_wave_kernel<bf16_t>, grid, block, 0, stream, resid,
-                         (const bf16_t*)delta, w, (bf16_t*)out, rows, n_rows, D, eps, write_resid);
-    else
-      hipLaunchKernelGGL(add_rmsnorm_wave_kernel<float>, grid, block, 0, stream, resid,
-                         (const float*)delta, w, (float*)out, rows, n_rows, D, eps, write_resid);
-    KAPPAI_RETURN_LAUNCH_STATUS();
+template <typename T, typename TD>
+static void launch_add_rmsnorm(float* resid, const void* delta, int n_part, size_t pstride,
+                               const float* w, void* out, const int* rows, int n_rows, int D,
+                               float eps, int write_resid, hipStream_t stream) {
+  if (D % 8 == 0 && D <= 8192 && n_part <= RN_MAX_PART) {
+    const int threads = ((D / 8 + WAVE - 1) / WAVE) * WAVE;
+    hipLaunchKernelGGL((add_rmsnorm_row_kernel<T, TD>), dim3(n_rows), dim3(threads), 0, stream,
+                       resid, (const TD*)delta, n_part, pstride, w, (T*)out, rows, D, eps,
+                       write_resid);
+    return;
   }
   const int threads = D >= 2048 ? 512 : (D >= 512 ? 256 : (D >= 128 ? 128 : 64));
-  if (is_bf16)
-    hipLaunchKernelGGL(add_rmsnorm_kernel<bf16_t>, dim3(n_rows), dim3(threads), 0, stream, resid,
-                       (const bf16_t*)delta, w, (bf16_t*)out, rows, D, eps, write_resid);
+  hipLaunchKernelGGL((add_rmsnorm_kernel<T, TD>), dim3(n_rows), dim3(threads), 0, stream, resid,
+                     (const TD*)delta, n_part, pstride, w, (T*)out, rows, D, eps, write_resid);
+}
+
+// out is bf16 or float (is_bf16); delta is of out's type, or float when delta_is_f32 (then it
+// may consist of n_part partial sums, pstride elements apart).
+extern "C" int kappai_add_rmsnorm(float* resid, const void* delta, int delta_is_f32, int n_part,
+                                  long pstride, const float* w, void* out, const int* rows,
+                                  int n_rows, int D, float eps, int write_resid, int is_bf16,
+                                  hipStream_t stream) {
+  if (n_rows <= 0) return 0;
+  if (n_part < 1 || (n_part > 1 && !delta_is_f32)) return (int)hipErrorInvalidValue;
+  if (!is_bf16)
+    launch_add_rmsnorm<float, float>(resid, delta, n_part, (size_t)pstride, w, out, rows, n_rows,
+                                     D, eps, write_resid, stream);
+  else if (delta_is_f32)
+    launch_add_rmsnorm<bf16_t, float>(resid, delta, n_part, (size_t)pstride, w, out, rows, n_rows,
+                                      D, eps, write_resid, stream);
   else
-    hipLaunchKernelGGL(add_rmsnorm_kernel<float>, dim3(n_rows), dim3(threads), 0, stream, resid,
-                       (const float*)delta, w, (float*)out, rows, D, eps, write_resid);
+    launch_add_rmsnorm<bf16_t, bf16_t>(resid, delta, n_part, (size_t)pstride, w, out, rows, n_rows,
+                                       D, eps, write_resid, stream);
   KAPPAI_RETURN_LAUNCH_STATUS();
 }
 

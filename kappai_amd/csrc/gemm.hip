@@ -216,6 +216,8 @@ __global__ __launch_bounds__(256) void gemm_bf16_tile_kernel(const bf16_t* __res
 
 // EPI 1 (SwiGLU, see the tile kernel): a block owns 16 output columns = 16 gate rows and
 // their 16 up rows of the interleaved W; N is the number of output columns.
+// gridDim.y > 1 splits K over blocks as well: block (x, y) writes its partial sums to
+// C + y * M * ldc (float), which the consumer adds up in a fixed order.
 template <typename TO, int MT, int NW, int EPI>
 __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny_kernel(
     const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, const float* __restrict__ bias,
@@ -240,9 +242,12 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny_kernel(
     const int gm = t * 16 + col;
     arow[t] = A + (size_t)(gm < M ? gm : 0) * lda + kg;
   }
-  const int kper = ((K + 32 * NW - 1) / (32 * NW)) * 32;
-  const int k0 = wave * kper;
-  const int k1 = min(K, k0 + kper);
+  const int kblk = ((K + 32 * (int)gridDim.y - 1) / (32 * (int)gridDim.y)) * 32;   // K a block
+  const int kb0 = blockIdx.y * kblk, kb1 = min(K, kb0 + kblk);
+  const int kper = ((kb1 - kb0 + 32 * NW - 1) / (32 * NW)) * 32;
+  const int k0 = kb0 + wave * kper;
+  const int k1 = min(kb1, k0 + kper);
+  C += (size_t)blockIdx.y * M * ldc;
   // loads in flight a lane: U * (NG + MT)
   constexpr int U = (NG + MT) <= 2 ? SK_UNROLL : ((NG + MT) <= 4 ? 4 : 2);
   for (int k = k0; k < k1; k += 32 * U) {
@@ -275,7 +280,7 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny_kernel(
   // the first MT waves each sum one row tile over the NW partial results, in a fixed order
   if (wave < MT && gn < N) {
     const int t = wave;
-    const float bv = bias ? bias[gn] : 0.f;
+    const float bv = (bias && blockIdx.y == 0) ? bias[gn] : 0.f;
 #pragma unroll
     for (int v = 0; v < 4; ++v) {
       const int gm = t * 16 + 4 * (lane / 16) + v;
@@ -298,36 +303,39 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny_kernel(
 
 template <typename TO, int MT, int NW, int EPI>
 static void launch_skinny(const bf16_t* A, const bf16_t* W, const float* bias, TO* C, int M, int N,
-                          int K, int lda, int ldc, hipStream_t stream) {
-  hipLaunchKernelGGL((gemm_bf16_skinny_kernel<TO, MT, NW, EPI>), dim3((N + 15) / 16),
+                          int K, int lda, int ldc, int ksplit, hipStream_t stream) {
+  hipLaunchKernelGGL((gemm_bf16_skinny_kernel<TO, MT, NW, EPI>), dim3((N + 15) / 16, ksplit),
                      dim3(NW * WAVE), 0, stream, A, W, bias, C, M, N, K, lda, ldc);
 }
 
 // more waves a block when there are few blocks, so that about 2048 waves or more stream W
 template <typename TO, int MT, int EPI>
 static void launch_skinny_mt(const bf16_t* A, const bf16_t* W, const float* bias, TO* C, int M,
-                             int N, int K, int lda, int ldc, hipStream_t stream) {
-  const int blocks = (N + 15) / 16;
+                             int N, int K, int lda, int ldc, int ksplit, hipStream_t stream) {
+  const int blocks = ((N + 15) / 16) * ksplit;
+  const int kb = K / ksplit;                              // K a block
   constexpr int MAXW = 16 / (MT * (EPI == 1 ? 2 : 1));   // LDS for the partial results
-  if (blocks * 4 >= 2048 || K <= 512 || MAXW <= 4)
-    launch_skinny<TO, MT, 4, EPI>(A, W, bias, C, M, N, K, lda, ldc, stream);
-  else if (blocks * 8 >= 2048 || K <= 1024 || MAXW <= 8)
-    launch_skinny<TO, MT, (MAXW >= 8 ? 8 : 4), EPI>(A, W, bias, C, M, N, K, lda, ldc, stream);
+  if (blocks * 4 >= 2048 || kb <= 512 || MAXW <= 4)
+    launch_skinny<TO, MT, 4, EPI>(A, W, bias, C, M, N, K, lda, ldc, ksplit, stream);
+  else if (blocks * 8 >= 2048 || kb <= 1024 || MAXW <= 8)
+    launch_skinny<TO, MT, (MAXW >= 8 ? 8 : 4), EPI>(A, W, bias, C, M, N, K, lda, ldc, ksplit,
+                                                    stream);
   else
-    launch_skinny<TO, MT, (MAXW >= 16 ? 16 : 4), EPI>(A, W, bias, C, M, N, K, lda, ldc, stream);
+    launch_skinny<TO, MT, (MAXW >= 16 ? 16 : 4), EPI>(A, W, bias, C, M, N, K, lda, ldc, ksplit,
+                                                      stream);
 }
 
 template <typename TO, int EPI>
 static int launch_bf16(const bf16_t* A, const bf16_t* W, const float* bias, TO* C, int M, int N,
-                       int K, int lda, int ldc, int force_kernel, hipStream_t stream) {
+                       int K, int lda, int ldc, int force_kernel, int ksplit, hipStream_t stream) {
   // N counts output columns; with the SwiGLU epilogue W has 2N rows
   if (M <= 64 && force_kernel != 1) {
     const int mt = (M + 15) / 16;
     switch (mt) {
-      case 1: launch_skinny_mt<TO, 1, EPI>(A, W, bias, C, M, N, K, lda, ldc, stream); break;
-      case 2: launch_skinny_mt<TO, 2, EPI>(A, W, bias, C, M, N, K, lda, ldc, stream); break;
-      case 3: launch_skinny_mt<TO, 3, EPI>(A, W, bias, C, M, N, K, lda, ldc, stream); break;
-      default: launch_skinny_mt<TO, 4, EPI>(A, W, bias, C, M, N, K, lda, ldc, stream); break;
+      case 1: launch_skinny_mt<TO, 1, EPI>(A, W, bias, C, M, N, K, lda, ldc, ksplit, stream); break;
+      case 2: launch_skinny_mt<TO, 2, EPI>(A, W, bias, C, M, N, K, lda, ldc, ksplit, stream); break;
+      case 3: launch_skinny_mt<TO, 3, EPI>(A, W, bias, C, M, N, K, lda, ldc, ksplit, stream); break;
+      default: launch_skinny_mt<TO, 4, EPI>(A, W, bias, C, M, N, K, lda, ldc, ksplit, stream); break;
     }
   } else {
     const int NW_ = EPI == 1 ? 2 * N : N;           // rows of W = columns the tiles run over
@@ -340,17 +348,19 @@ static int launch_bf16(const bf16_t* A, const bf16_t* W, const float* bias, TO* 
 
 // K, lda must be multiples of 8 and A, W 16-byte aligned (checked by the caller).
 // force_kernel: 0 = by M, 1 = tile kernel, 2 = skinny kernel (M <= 64 only); for tests.
+// ksplit > 1 (M <= 64, float output only): C is [ksplit][M][ldc] partial sums over K ranges.
 extern "C" int kappai_gemm_bf16(const void* A, const void* W, const float* bias, void* C, int M,
                                 int N, int K, int lda, int ldc, int out_is_f32, int force_kernel,
-                                hipStream_t stream) {
+                                int ksplit, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
-  if ((K % 8) || (lda % 8)) return (int)hipErrorInvalidValue;
+  if ((K % 8) || (lda % 8) || ksplit < 1 || ksplit > 64) return (int)hipErrorInvalidValue;
   if (force_kernel == 2 && M > 64) return (int)hipErrorInvalidValue;
+  if (ksplit > 1 && (M > 64 || force_kernel == 1 || !out_is_f32)) return (int)hipErrorInvalidValue;
   if (out_is_f32)
     return launch_bf16<float, 0>((const bf16_t*)A, (const bf16_t*)W, bias, (float*)C, M, N, K, lda,
-                                 ldc, force_kernel, stream);
+                                 ldc, force_kernel, ksplit, stream);
   return launch_bf16<bf16_t, 0>((const bf16_t*)A, (const bf16_t*)W, bias, (bf16_t*)C, M, N, K, lda,
-                                ldc, force_kernel, stream);
+                                ldc, force_kernel, 1, stream);
 }
 
 // C[M, F] = silu(A Wg^T) * (A Wu^T) with W = gate and up rows interleaved in groups of 16,
@@ -361,5 +371,5 @@ extern "C" int kappai_gemm_bf16_swiglu(const void* A, const void* W, void* C, in
   if ((K % 8) || (lda % 8) || (F % 16)) return (int)hipErrorInvalidValue;
   if (force_kernel == 2 && M > 64) return (int)hipErrorInvalidValue;
   return launch_bf16<bf16_t, 1>((const bf16_t*)A, (const bf16_t*)W, nullptr, (bf16_t*)C, M, F, K,
-                                lda, ldc, force_kernel, stream);
+                                lda, ldc, force_kernel, 1, stream);
 }

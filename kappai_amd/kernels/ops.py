@@ -66,15 +66,24 @@ def add_rmsnorm(resid: torch.Tensor, delta: Optional[torch.Tensor], weight: torc
                 eps: float, out_dtype, rows: Optional[torch.Tensor] = None,
                 write_resid: bool = True) -> torch.Tensor:
     """RMSNorm of ``resid (+ delta)``; with ``write_resid`` the sum replaces ``resid``.
-    ``rows`` (int32) picks the rows to normalise; the result then has one row per entry."""
+    ``delta`` is [T, D] in the compute dtype, or float32 partial sums [S, T, D] (a product
+    split over K) that are added in order.  ``rows`` (int32) picks the rows to normalise; the
+    result then has one row per entry."""
     _gpu("resid", resid, F32)
     _gpu("weight", weight, F32)
     _need(resid.dim() == 2 and weight.shape == (resid.shape[1],),
           f"add_rmsnorm: resid {tuple(resid.shape)} and weight {tuple(weight.shape)} disagree")
     isb = _is_bf16(out_dtype)
+    n_part, pstride, delta_f32 = 1, 0, 0
     if delta is not None:
-        _gpu("delta", delta, out_dtype)
-        _need(delta.shape == resid.shape, "add_rmsnorm: delta must have resid's shape")
+        if delta.dim() == 3:
+            _gpu("delta", delta, F32)
+            _need(delta.shape[1:] == resid.shape, "add_rmsnorm: partial sums must be [S, T, D]")
+            n_part, pstride, delta_f32 = delta.shape[0], resid.numel(), 1
+        else:
+            _gpu("delta", delta, (out_dtype, F32))
+            _need(delta.shape == resid.shape, "add_rmsnorm: delta must have resid's shape")
+            delta_f32 = 1 if delta.dtype == F32 else 0
     n = resid.shape[0]
     if rows is not None:
         _gpu("rows", rows, I32)
@@ -84,8 +93,9 @@ def add_rmsnorm(resid: torch.Tensor, delta: Optional[torch.Tensor], weight: torc
     D = resid.shape[1]
     out = torch.empty((n, D), dtype=out_dtype, device=resid.device)
     check(library("elementwise").kappai_add_rmsnorm(
-        _ptr(resid), _ptr(delta), _ptr(weight), _ptr(out), _ptr(rows), _c_int(n), _c_int(D),
-        _c_float(eps), _c_int(1 if write_resid else 0), _c_int(isb), _stream()), "add_rmsnorm")
+        _ptr(resid), _ptr(delta), _c_int(delta_f32), _c_int(n_part), _c_long(pstride), _ptr(weight),
+        _ptr(out), _ptr(rows), _c_int(n), _c_int(D), _c_float(eps),
+        _c_int(1 if write_resid else 0), _c_int(isb), _stream()), "add_rmsnorm")
     return out
 
 
@@ -122,11 +132,22 @@ def cast(x: torch.Tensor, dtype) -> torch.Tensor:
 
 
 # ---------------------------------------------------------------------------------------
+def split_k_for(M: int, N: int, K: int) -> int:
+    """How many K ranges a decode product is cut into so that about 512 blocks stream the
+    matrix (1: not split)."""
+    if M > 64:
+        return 1
+    col_groups = (N + 15) // 16
+    return max(1, min(8, 512 // col_groups, K // 512))
+
+
 def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
-           out_dtype=None, force_kernel: int = 0) -> torch.Tensor:
+           out_dtype=None, force_kernel: int = 0, partial_sums: bool = False) -> torch.Tensor:
     """``x [M, K] @ weight[N, K]^T (+ bias)``.  A bfloat16 matrix runs on the matrix cores
     with float accumulation; a float32 matrix runs in true 32-bit arithmetic, whatever the
-    activations' dtype.  ``x`` may be a view with a row stride."""
+    activations' dtype.  ``x`` may be a view with a row stride.  With ``partial_sums`` the
+    result may come back as float32 [S, M, N], the sums over S ranges of K, for a consumer
+    that adds them (a matrix with few columns is then streamed by enough blocks)."""
     _gpu("x", x, (F32, BF16), contiguous=False)
     _gpu("weight", weight, (F32, BF16))
     _need(x.dim() == 2 and weight.dim() == 2 and x.shape[1] == weight.shape[1],
@@ -150,10 +171,16 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] =
     _need(K % 8 == 0 and lda % 8 == 0 and xb.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0,
           f"linear: the bfloat16 kernels read 16 bytes at a time: K ({K}) and the row stride "
           f"({lda}) must be multiples of 8 and the tensors 16-byte aligned")
-    out = torch.empty((M, N), dtype=out_dtype, device=x.device)
+    ksplit = split_k_for(M, N, K) if (partial_sums and force_kernel != 1) else 1
+    if ksplit > 1:
+        out = torch.empty((ksplit, M, N), dtype=F32, device=x.device)
+        out_is_f32 = 1
+    else:
+        out = torch.empty((M, N), dtype=out_dtype, device=x.device)
+        out_is_f32 = 0 if out_dtype == BF16 else 1
     check(library("gemm").kappai_gemm_bf16(
         _ptr(xb), _ptr(weight), _ptr(bias), _ptr(out), _c_int(M), _c_int(N), _c_int(K),
-        _c_int(lda), _c_int(N), _c_int(0 if out_dtype == BF16 else 1), _c_int(force_kernel),
+        _c_int(lda), _c_int(N), _c_int(out_is_f32), _c_int(force_kernel), _c_int(ksplit),
         _stream()), "gemm_bf16")
     return out
 
@@ -354,10 +381,11 @@ def paged_attention(q: torch.Tensor, n_heads: int, n_kv_heads: int, head_dim: in
     _need(H // G <= 16, "the decode kernel takes at most 16 query heads per kv head")
     _need(max_position is not None, "the decode kernel needs the batch's largest position")
     n_keys = min(max_position + 1, window) + 32 if window else max_position + 1
-    # enough waves to fill the chip, but at least 64 keys a split
-    want = max(1, 2048 // max(T * G, 1))
-    n_splits = max(1, min(want, (n_keys + 63) // 64))
-    keys_per_split = ((n_keys + n_splits - 1) // n_splits + 31) // 32 * 32
+    # one wave keeps the loads of `kpw` keys in flight; splits are whole numbers of that, and
+    # at most 64 of them are merged
+    kpw = lib.kappai_attn_keys_per_wave()
+    n_splits = max(1, min(64, (n_keys + kpw - 1) // kpw))
+    keys_per_split = ((n_keys + n_splits - 1) // n_splits + kpw - 1) // kpw * kpw
     n_splits = (n_keys + keys_per_split - 1) // keys_per_split
     part_o = torch.empty((T, H, n_splits, d), dtype=F32, device=q.device)
     part_ml = torch.empty((T, H, n_splits, 2), dtype=F32, device=q.device)

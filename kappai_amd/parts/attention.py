@@ -82,7 +82,7 @@ class GroupedQueryAttention(Mixer):
                                   window=self.window or 0, q_tiles=batch.q_tiles,
                                   single_rows=batch.max_segment_rows == 1,
                                   max_position=batch.max_position)
-        return self.out.forward(ctx)
+        return self.out.forward(ctx, partial_sums=True)
 
     def weight_bytes(self) -> int:
         return self.qkv.weight_bytes() + self.out.weight_bytes() + 2 * self.d * 4

@@ -65,7 +65,8 @@ class PositionEncoding(Part):
 class Mixer(Part):
     """A token mixer.  ``cache_spec`` says what it needs from the cache manager (PagedKV,
     FixedState or None); ``forward`` gets the normalised rows [T, width] in the compute
-    dtype, the step's ``RowBatch`` and its cache view, and returns [T, width]."""
+    dtype, the step's ``RowBatch`` and its cache view, and returns [T, width] in the compute
+    dtype, or float32 partial sums [S, T, width] that the next norm adds up."""
 
     def cache_spec(self):
         return None
@@ -82,8 +83,9 @@ class FeedForward(Part):
 @dataclass
 class Hidden:
     """The residual stream between blocks: ``resid`` (float32, [T, width]) and the last
-    part's output ``delta`` that has not been added yet.  The next norm adds it while it
-    normalises, so the sum is made in float32 and costs no pass of its own."""
+    part's output ``delta`` that has not been added yet ([T, width], or float32 partial sums
+    [S, T, width]).  The next norm adds it while it normalises, so the sum is made in float32
+    and costs no pass of its own."""
     resid: torch.Tensor
     delta: Optional[torch.Tensor] = None
 

@@ -37,8 +37,9 @@ class SwiGLU(FeedForward):
 
     def forward(self, x, batch):
         if self.fused and x.dtype == torch.bfloat16:
-            return self.down.forward(ops.linear_swiglu(x, self.gate_up.weight))
-        return self.down.forward(ops.swiglu(self.gate_up.forward(x)))
+            return self.down.forward(ops.linear_swiglu(x, self.gate_up.weight),
+                                     partial_sums=True)
+        return self.down.forward(ops.swiglu(self.gate_up.forward(x)), partial_sums=True)
 
     def weight_bytes(self) -> int:
         return self.gate_up.weight_bytes() + self.down.weight_bytes()

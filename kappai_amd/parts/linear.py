@@ -50,8 +50,11 @@ class Linear(Part):
         """Use a tensor that another part owns (a tied output head)."""
         self.weight = weight
 
-    def forward(self, x: torch.Tensor, out_dtype=None) -> torch.Tensor:
-        return ops.linear(x, self.weight, self.bias, out_dtype=out_dtype)
+    def forward(self, x: torch.Tensor, out_dtype=None, partial_sums: bool = False) -> torch.Tensor:
+        """``partial_sums``: the caller hands the result to a norm as the pending residual
+        update, which may then arrive as float32 sums over ranges of the input dimension."""
+        return ops.linear(x, self.weight, self.bias, out_dtype=out_dtype,
+                          partial_sums=partial_sums)
 
     def weight_bytes(self) -> int:
         n = self.weight.numel() * self.weight.element_size()

@@ -60,7 +60,7 @@ class GatedShortConv(Mixer):
         proj = self.in_proj.forward(x)
         y = ops.shortconv(proj, self.taps, self.conv_bias, cache.state, batch.row_seg,
                           batch.seg_start, batch.seg_pos0, batch.seg_slot)
-        return self.out_proj.forward(y)
+        return self.out_proj.forward(y, partial_sums=True)
 
     def weight_bytes(self) -> int:
         return self.in_proj.weight_bytes() + self.out_proj.weight_bytes() + self.width * self.L * 4

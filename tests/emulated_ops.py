@@ -19,7 +19,11 @@ def embed_rows(ids, table):
 
 
 def add_rmsnorm(resid, delta, weight, eps, out_dtype, rows=None, write_resid=True):
-    x = resid if delta is None else resid + delta.to(F32)
+    x = resid
+    if delta is not None:
+        parts = delta if delta.dim() == 3 else delta[None]
+        for p in parts:                       # partial sums are added in order
+            x = x + p.to(F32)
     if delta is not None and write_resid and rows is None:
         resid.copy_(x)
     if rows is not None:
@@ -42,7 +46,7 @@ def cast(x, dtype):
     return x.to(dtype)
 
 
-def linear(x, weight, bias=None, out_dtype=None, force_kernel=0):
+def linear(x, weight, bias=None, out_dtype=None, force_kernel=0, partial_sums=False):
     out_dtype = out_dtype or x.dtype
     y = x.to(F32) @ weight.to(F32).T
     if bias is not None:

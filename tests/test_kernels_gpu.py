@@ -137,6 +137,36 @@ def test_linear_swiglu(ops, M, F, K):
         close(got.float(), want, BF16_ULP, f"kernel {force}")
 
 
+@pytest.mark.parametrize("M,N,K", [(1, 2048, 2048), (8, 2048, 8192), (16, 96, 1024), (40, 1000, 4096),
+                                   (64, 64, 512), (5, 6144, 2048)])
+def test_linear_partial_sums(ops, M, N, K):
+    """A decode product split over K: float32 partial sums that add up to the product, and an
+    RMSNorm that consumes them like an ordinary residual update."""
+    x, w, b = rand((M, K), BF16, 19), rand((N, K), BF16, 20, 0.05), rand((N,), F32, 21)
+    want = x.double() @ w.double().T + b.double()
+    parts = ops.linear(x.to(DEV), w.to(DEV), b.to(DEV), partial_sums=True)
+    S = ops.split_k_for(M, N, K)
+    if S == 1:
+        assert parts.shape == (M, N) and parts.dtype == BF16
+        close(parts.float(), want, BF16_ULP, "unsplit")
+        return
+    assert parts.shape == (S, M, N) and parts.dtype == F32
+    close(parts.sum(0), want, 2e-5, "sum of the partial sums")
+    resid = rand((M, N), F32, 22, 2.0)
+    wn = 1 + rand((N,), F32, 23, 0.1)
+    r_dev = resid.to(DEV).clone()
+    got = ops.add_rmsnorm(r_dev, parts, wn.to(DEV), 1e-5, BF16)
+    r_ref = resid.clone()
+    want_n = ref.add_rmsnorm(r_ref, parts.cpu(), wn, 1e-5, F32)
+    close(got.float(), want_n, BF16_ULP, "norm over partial sums")
+    close(r_dev, r_ref, 1e-6, "residual")
+    rows = torch.tensor([M - 1, 0], dtype=torch.int32)
+    got = ops.add_rmsnorm(resid.to(DEV), parts, wn.to(DEV), 1e-5, BF16, rows=rows.to(DEV),
+                          write_resid=False)
+    close(got.float(), ref.add_rmsnorm(resid.clone(), parts.cpu(), wn, 1e-5, F32, rows=rows,
+                                       write_resid=False), BF16_ULP, "selected rows")
+
+
 def test_linear_views_and_mixed_storage(ops):
     # x as the leading columns of a wider buffer (a row stride), as attention hands q over
     wide = rand((20, 96 + 40), BF16, 12).to(DEV)
