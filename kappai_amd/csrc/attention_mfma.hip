@@ -136,18 +136,43 @@ __global__ __launch_bounds__(64) void attn_prefill_kernel(
   float m_run = -INFINITY, l_run = 0.f;
   const float sc = scale * LOG2E;
 
-  for (int kb = (lo_tile / 32) * 32; kb <= pos_last; kb += 32) {
+  // The loads of the next 32 keys (their two page ids, key fragments, value fragments) are
+  // issued before the current 32 are worked on.  Page ids are the same for all lanes of a
+  // 16-key group, so they are looked up once per group.
+  constexpr bool P_AHEAD = HEAD_DIM <= 128;      // beyond that the registers do not suffice
+  constexpr int P_NB = P_AHEAD ? 2 : 1;
+  u32x4_t kfr[P_NB][P_KS];
+  u32x2_t vfa[P_NB][2][P_MT], vfb[P_NB][2][P_MT];
+  auto fetch = [&](int buf, int kb) {
+    const int g0 = min(kb / ps, max_blocks - 1), g1 = min((kb + 16) / ps, max_blocks - 1);
+    const int pg0 = kb <= pos_last ? bt[g0] : -1;
+    const int pg1 = kb + 16 <= pos_last ? bt[g1] : -1;
+    const int my_key = kb + col;
+    const int my_pg = col < 16 ? pg0 : pg1;
+#pragma unroll
+    for (int ks = 0; ks < P_KS; ++ks)
+      kfr[buf][ks] =
+          load_k8_pg(k_pool, my_pg, G, g, ps, my_key, 16 * ks + 8 * hh, lo_tile, pos_last);
+#pragma unroll
+    for (int st = 0; st < 2; ++st) {
+      const int key0 = kb + 16 * st + 4 * hh;
+      const int pg = st == 0 ? pg0 : pg1;
+#pragma unroll
+      for (int mt = 0; mt < P_MT; ++mt) {
+        const int dd = 32 * mt + col;
+        vfa[buf][st][mt] = load_vt4_pg(vt_pool, pg, G, g, ps, dd, key0, lo_tile, pos_last);
+        vfb[buf][st][mt] = load_vt4_pg(vt_pool, pg, G, g, ps, dd, key0 + 8, lo_tile, pos_last);
+      }
+    }
+  };
+  auto work = [&](int buf, int kb) {
     // ---- S^T tile: 32 keys x 32 queries -------------------------------------------------
     f32x16_t s;
 #pragma unroll
     for (int v = 0; v < 16; ++v) s[v] = 0.f;
-    const int my_key = kb + col;
 #pragma unroll
-    for (int ks = 0; ks < P_KS; ++ks) {
-      const bf16x8_t kf =
-          as_frag(load_k8(k_pool, bt, G, g, ps, my_key, 16 * ks + 8 * hh, lo_tile, pos_last));
-      s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[ks], s, 0, 0, 0);
-    }
+    for (int ks = 0; ks < P_KS; ++ks)
+      s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_frag(kfr[buf][ks]), qf[ks], s, 0, 0, 0);
     // lane holds, for query `col`, keys kb + 8*(v/4) + 4*hh + v%4
     float mloc = -INFINITY;
 #pragma unroll
@@ -182,15 +207,29 @@ __global__ __launch_bounds__(64) void attn_prefill_kernel(
                           pack_bf16(s[8 * st + 4], s[8 * st + 5]),
                           pack_bf16(s[8 * st + 6], s[8 * st + 7])};
       const bf16x8_t pf = as_frag(pw);
-      const int key0 = kb + 16 * st + 4 * hh;
 #pragma unroll
       for (int mt = 0; mt < P_MT; ++mt) {
-        const int dd = 32 * mt + col;
-        const u32x2_t a = load_vt4(vt_pool, bt, G, g, ps, dd, key0, lo_tile, pos_last);
-        const u32x2_t b = load_vt4(vt_pool, bt, G, g, ps, dd, key0 + 8, lo_tile, pos_last);
-        const u32x4_t vw = {a.x, a.y, b.x, b.y};
+        const u32x4_t vw = {vfa[buf][st][mt].x, vfa[buf][st][mt].y, vfb[buf][st][mt].x,
+                            vfb[buf][st][mt].y};
         o[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_frag(vw), pf, o[mt], 0, 0, 0);
       }
+    }
+  };
+  const int kb0 = (lo_tile / 32) * 32;
+  if (P_AHEAD) {
+    fetch(0, kb0);
+    for (int kb = kb0; kb <= pos_last; kb += 64) {
+      if (kb + 32 <= pos_last) fetch(P_NB - 1, kb + 32);
+      work(0, kb);
+      if (kb + 32 <= pos_last) {
+        if (kb + 64 <= pos_last) fetch(0, kb + 64);
+        work(P_NB - 1, kb + 32);
+      }
+    }
+  } else {
+    for (int kb = kb0; kb <= pos_last; kb += 32) {
+      fetch(0, kb);
+      work(0, kb);
     }
   }
   if (!row_ok) return;

@@ -95,78 +95,132 @@ __device__ __forceinline__ bf16x8_t as_bf16x8(u32x4_t v) {
 __device__ __forceinline__ void store_out(float* p, float v) { *p = v; }
 __device__ __forceinline__ void store_out(bf16_t* p, float v) { *p = f32_to_bf16(v); }
 
-#define T_BM 128
-#define T_BN 128
-#define T_BK 32
-#define T_LDS (T_BK + 8)  // row stride in bf16: 80 bytes keeps 16-byte alignment, spreads banks
-
 __device__ __forceinline__ float silu_f(float g) { return g / (1.0f + expf(-g)); }
 
+// Block = WAVES_M x WAVES_N waves, each owning (WM*32) x (WN*32) of the result as WM*WN
+// accumulator tiles of 32x32: per 16 of K a wave reads WM+WN fragments from LDS for WM*WN
+// matrix instructions, so large wave tiles keep LDS traffic below what the matrix cores
+// consume.  Tiles of A (BM x BK) and W (BN x BK) go global -> registers -> LDS,
+// double-buffered: the loads of tile k+1 are in flight while tile k is multiplied, one
+// barrier a tile.
+// Blocks are renumbered so that the blocks that run on one XCD (every eighth) work on
+// neighbouring tiles and share their L2.
+//
 // EPI 1 (SwiGLU): W holds gate and up rows interleaved in groups of 16 (16 gate rows, the 16 up
 // rows of the same columns, ...); the kernel writes silu(gate) * up, N/2 columns wide
 // (kappai: src/backend/cpu/quants.h:369-371, src/recipe/builders.c:344-370).
-template <typename TO, int EPI>
-__global__ __launch_bounds__(256) void gemm_bf16_tile_kernel(const bf16_t* __restrict__ A,
-                                                             const bf16_t* __restrict__ W,
-                                                             const float* __restrict__ bias,
-                                                             TO* __restrict__ C, int M, int N,
-                                                             int K, int lda, int ldc) {
-  __shared__ __attribute__((aligned(16))) bf16_t As[T_BM * T_LDS];
-  __shared__ __attribute__((aligned(16))) bf16_t Ws[T_BN * T_LDS];
+template <typename TO, int EPI, int WAVES_M, int WAVES_N, int WM, int WN, int BK, int NBUF,
+          int OCC>
+__global__ __launch_bounds__(WAVES_M * WAVES_N * WAVE)
+    __attribute__((amdgpu_waves_per_eu(OCC, OCC))) void gemm_bf16_tile_kernel(
+        const bf16_t* __restrict__ A, const bf16_t* __restrict__ W,
+        const float* __restrict__ bias, TO* __restrict__ C, int M, int N, int K, int lda, int ldc,
+        int tiles_n) {
+  constexpr int BM = WAVES_M * WM * 32, BN = WAVES_N * WN * 32;
+  constexpr int LDS_STRIDE = BK + 8;   // in bf16: rows stay 16-byte aligned, banks are spread
+  constexpr int THREADS = WAVES_M * WAVES_N * WAVE;
+  constexpr int CPR = BK / 8;                              // 16-byte chunks a row
+  constexpr int A_CHUNKS = BM * CPR / THREADS;             // chunks a thread stages
+  constexpr int W_CHUNKS = BN * CPR / THREADS;
+  extern __shared__ __attribute__((aligned(16))) bf16_t lds[];
+  // LDS: the A tiles of the NBUF buffers, then their W tiles
+  constexpr int A_TILE = BM * LDS_STRIDE, W_TILE = BN * LDS_STRIDE;
   const int tid = threadIdx.x;
   const int lane = tid % WAVE, wave = tid / WAVE;
-  const int wm = wave / 2, wn = wave % 2;
-  const int m0 = blockIdx.y * T_BM, n0 = blockIdx.x * T_BN;
+  const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+  // block -> tile, XCD-aware
+  int b = blockIdx.x;
+  const int nb = gridDim.x;
+  if (nb % 8 == 0) b = (b % 8) * (nb / 8) + b / 8;
+  const int m0 = (b / tiles_n) * BM, n0 = (b % tiles_n) * BN;
+  // gridDim.y > 1 splits K over blocks: block y writes its partial sums to C + y * M * ldc
+  const int kblk = ((K + BK * (int)gridDim.y - 1) / (BK * (int)gridDim.y)) * BK;
+  const int kbeg = blockIdx.y * kblk, kend = min(K, kbeg + kblk);
+  C += (size_t)blockIdx.y * M * ldc;
 
-  // global -> register staging: thread loads 16 bytes of rows lr and lr+64 of each tile
-  const int lr = tid / 4, lc = (tid % 4) * 8;
-  f32x16_t acc[2][2];
+  f32x16_t acc[WM][WN];
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < WM; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int j = 0; j < WN; ++j)
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
+  // Staging: a thread copies 16-byte chunks; consecutive lanes take consecutive chunks of a
+  // row, so that a row's bytes are asked for by neighbouring lanes and coalesce.
   const u32x4_t zero = {0u, 0u, 0u, 0u};
-  u32x4_t ra[2], rw[2];
+  u32x4_t ra[A_CHUNKS], rw[W_CHUNKS];
+  auto chunk_row = [&](int idx) { return idx / CPR; };
+  auto chunk_col = [&](int idx) { return (idx % CPR) * 8; };
   auto fetch = [&](int k0) {
 #pragma unroll
-    for (int h = 0; h < 2; ++h) {
-      const int r = lr + h * 64;
-      const int gk = k0 + lc;
-      const int gm = m0 + r, gn = n0 + r;
-      ra[h] = (gm < M && gk < K) ? load16(A + (size_t)gm * lda + gk) : zero;
-      rw[h] = (gn < N && gk < K) ? load16(W + (size_t)gn * K + gk) : zero;
+    for (int c = 0; c < A_CHUNKS; ++c) {
+      const int idx = tid + c * THREADS;
+      const int r = chunk_row(idx), gk = k0 + chunk_col(idx);
+      ra[c] = (m0 + r < M && gk < kend) ? load16(A + (size_t)(m0 + r) * lda + gk) : zero;
+    }
+#pragma unroll
+    for (int c = 0; c < W_CHUNKS; ++c) {
+      const int idx = tid + c * THREADS;
+      const int r = chunk_row(idx), gk = k0 + chunk_col(idx);
+      rw[c] = (n0 + r < N && gk < kend) ? load16(W + (size_t)(n0 + r) * K + gk) : zero;
     }
   };
-  fetch(0);
-  for (int k0 = 0; k0 < K; k0 += T_BK) {
+  auto stage = [&](int buf) {
 #pragma unroll
-    for (int h = 0; h < 2; ++h) {
-      const int r = lr + h * 64;
-      *reinterpret_cast<u32x4_t*>(&As[r * T_LDS + lc]) = ra[h];
-      *reinterpret_cast<u32x4_t*>(&Ws[r * T_LDS + lc]) = rw[h];
+    for (int c = 0; c < A_CHUNKS; ++c) {
+      const int idx = tid + c * THREADS;
+      *reinterpret_cast<u32x4_t*>(lds + buf * A_TILE + chunk_row(idx) * LDS_STRIDE +
+                                  chunk_col(idx)) = ra[c];
     }
-    __syncthreads();
-    if (k0 + T_BK < K) fetch(k0 + T_BK);
 #pragma unroll
-    for (int ks = 0; ks < T_BK; ks += 16) {
-      bf16x8_t a[2], b[2];
-      const int kc = ks + (lane / 32) * 8;
+    for (int c = 0; c < W_CHUNKS; ++c) {
+      const int idx = tid + c * THREADS;
+      *reinterpret_cast<u32x4_t*>(lds + NBUF * A_TILE + buf * W_TILE +
+                                  chunk_row(idx) * LDS_STRIDE + chunk_col(idx)) = rw[c];
+    }
+  };
+  // While tile k is multiplied out of LDS, the loads of tile k+1 are in flight into registers;
+  // after the products they are written to LDS: into the other buffer (NBUF 2, one barrier a
+  // tile) or, after a barrier, into the same one (NBUF 1: half the LDS, so that two blocks fit
+  // a CU even with long tiles, whose products give the loads more time to arrive).
+  fetch(kbeg);
+  stage(0);
+  __syncthreads();
+  int buf = 0;
+  for (int k0 = kbeg; k0 < kend; k0 += BK) {
+    const bool more = k0 + BK < kend;
+    if (more) fetch(k0 + BK);
+    const bf16_t* as =
+        lds + buf * A_TILE + (wm * WM * 32 + lane % 32) * LDS_STRIDE + (lane / 32) * 8;
+    const bf16_t* ws = lds + NBUF * A_TILE + buf * W_TILE +
+                       (wn * WN * 32 + lane % 32) * LDS_STRIDE + (lane / 32) * 8;
+    bf16x8_t a[2][WM], w[2][WN];
+    auto frags = [&](int fb, int ks) {
 #pragma unroll
-      for (int i = 0; i < 2; ++i)
-        a[i] = as_bf16x8(*reinterpret_cast<const u32x4_t*>(
-            &As[(wm * 64 + i * 32 + lane % 32) * T_LDS + kc]));
+      for (int i = 0; i < WM; ++i)
+        a[fb][i] = as_bf16x8(*reinterpret_cast<const u32x4_t*>(as + i * 32 * LDS_STRIDE + ks));
 #pragma unroll
-      for (int j = 0; j < 2; ++j)
-        b[j] = as_bf16x8(*reinterpret_cast<const u32x4_t*>(
-            &Ws[(wn * 64 + j * 32 + lane % 32) * T_LDS + kc]));
+      for (int j = 0; j < WN; ++j)
+        w[fb][j] = as_bf16x8(*reinterpret_cast<const u32x4_t*>(ws + j * 32 * LDS_STRIDE + ks));
+    };
+    frags(0, 0);
 #pragma unroll
-      for (int i = 0; i < 2; ++i)
+    for (int s2 = 0; s2 < BK / 16; ++s2) {
+      if (s2 + 1 < BK / 16) frags((s2 + 1) & 1, (s2 + 1) * 16);
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
+      for (int i = 0; i < WM; ++i)
+#pragma unroll
+        for (int j = 0; j < WN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[s2 & 1][i], w[s2 & 1][j],
+                                                              acc[i][j], 0, 0, 0);
+    }
+    if (NBUF == 1) {
+      __syncthreads();
+      if (more) stage(0);
+    } else {
+      if (more) stage(buf ^ 1);
+      buf ^= 1;
     }
     __syncthreads();
   }
@@ -175,16 +229,16 @@ __global__ __launch_bounds__(256) void gemm_bf16_tile_kernel(const bf16_t* __res
     // a 32-column tile is 16 gate columns and their 16 up columns: lane c < 16 holds gate,
     // lane c + 16 the matching up
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < WM; ++i)
 #pragma unroll
-      for (int j = 0; j < 2; ++j) {
+      for (int j = 0; j < WN; ++j) {
         const int c = lane % 32;
-        const int gcol = n0 + wn * 64 + j * 32;          // first interleaved column of the tile
+        const int gcol = n0 + (wn * WN + j) * 32;        // first interleaved column of the tile
         const int on = gcol / 2 + c;                     // output column for c < 16
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
           const float other = __shfl_xor(acc[i][j][v], 16, WAVE);
-          const int gm = m0 + wm * 64 + i * 32 + 8 * (v / 4) + 4 * (lane / 32) + v % 4;
+          const int gm = m0 + (wm * WM + i) * 32 + 8 * (v / 4) + 4 * (lane / 32) + v % 4;
           if (c < 16 && gm < M && gcol + c < N)
             store_out(C + (size_t)gm * ldc + on, silu_f(acc[i][j][v]) * other);
         }
@@ -192,18 +246,68 @@ __global__ __launch_bounds__(256) void gemm_bf16_tile_kernel(const bf16_t* __res
     return;
   }
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < WM; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const int gn = n0 + wn * 64 + j * 32 + lane % 32;
+    for (int j = 0; j < WN; ++j) {
+      const int gn = n0 + (wn * WN + j) * 32 + lane % 32;
       if (gn >= N) continue;
-      const float bv = bias ? bias[gn] : 0.f;
+      const float bv = (bias && blockIdx.y == 0) ? bias[gn] : 0.f;
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
-        const int gm = m0 + wm * 64 + i * 32 + 8 * (v / 4) + 4 * (lane / 32) + v % 4;
+        const int gm = m0 + (wm * WM + i) * 32 + 8 * (v / 4) + 4 * (lane / 32) + v % 4;
         if (gm < M) store_out(C + (size_t)gm * ldc + gn, acc[i][j][v] + bv);
       }
     }
+}
+
+template <typename TO, int EPI, int WAVES_M, int WAVES_N, int WM, int WN, int BK, int NBUF,
+          int OCC>
+static void launch_tile_cfg(const bf16_t* A, const bf16_t* W, const float* bias, TO* C, int M,
+                            int n_rows_w, int K, int lda, int ldc, int ksplit,
+                            hipStream_t stream) {
+  constexpr int BM = WAVES_M * WM * 32, BN = WAVES_N * WN * 32;
+  constexpr size_t lds_bytes = (size_t)NBUF * (BM + BN) * (BK + 8) * sizeof(bf16_t);
+  auto kern = gemm_bf16_tile_kernel<TO, EPI, WAVES_M, WAVES_N, WM, WN, BK, NBUF, OCC>;
+  static bool attr_set = false;       // more than 64 KB of LDS has to be asked for once
+  if (!attr_set) {
+    hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
+                        (int)lds_bytes);
+    attr_set = true;
+  }
+  const int tn = (n_rows_w + BN - 1) / BN, tm = (M + BM - 1) / BM;
+  hipLaunchKernelGGL(kern, dim3(tm * tn, ksplit), dim3(WAVES_M * WAVES_N * WAVE), lds_bytes,
+                     stream, A, W, bias, C, M, n_rows_w, K, lda, ldc, tn);
+}
+
+// shape: 0 = chosen by size, 1 = 128x128 blocks of two waves, 2 = 256x128 blocks (tiles of 32
+// of K, two LDS buffers), 3 = 256x128 blocks (tiles of 64 of K, one LDS buffer), 4 = 256x256
+// blocks (tiles of 64 of K)
+template <typename TO, int EPI>
+static void launch_tile(const bf16_t* A, const bf16_t* W, const float* bias, TO* C, int M,
+                        int n_rows_w, int K, int lda, int ldc, int ksplit, int shape,
+                        hipStream_t stream) {
+  if (shape == 0) {
+    const int big = ((M + 255) / 256) * ((n_rows_w + 127) / 128) * ksplit;
+    shape = big >= 128 ? 3 : 1;
+  }
+  switch (shape) {
+    case 1:
+      launch_tile_cfg<TO, EPI, 1, 2, 4, 2, 32, 2, 2>(A, W, bias, C, M, n_rows_w, K, lda, ldc, ksplit,
+                                                  stream);
+      break;
+    case 2:
+      launch_tile_cfg<TO, EPI, 2, 2, 4, 2, 32, 2, 2>(A, W, bias, C, M, n_rows_w, K, lda, ldc, ksplit,
+                                                  stream);
+      break;
+    case 3:
+      launch_tile_cfg<TO, EPI, 2, 2, 4, 2, 64, 1, 2>(A, W, bias, C, M, n_rows_w, K, lda, ldc, ksplit,
+                                                  stream);
+      break;
+    default:
+      launch_tile_cfg<TO, EPI, 2, 2, 4, 4, 64, 2, 1>(A, W, bias, C, M, n_rows_w, K, lda, ldc, ksplit,
+                                                  stream);
+      break;
+  }
 }
 
 // M <= 16*MT (decode).  Bound by reading W once: a block owns 16 columns of the result and
@@ -329,7 +433,7 @@ template <typename TO, int EPI>
 static int launch_bf16(const bf16_t* A, const bf16_t* W, const float* bias, TO* C, int M, int N,
                        int K, int lda, int ldc, int force_kernel, int ksplit, hipStream_t stream) {
   // N counts output columns; with the SwiGLU epilogue W has 2N rows
-  if (M <= 64 && force_kernel != 1) {
+  if (M <= 64 && force_kernel != 1 && force_kernel < 3) {
     const int mt = (M + 15) / 16;
     switch (mt) {
       case 1: launch_skinny_mt<TO, 1, EPI>(A, W, bias, C, M, N, K, lda, ldc, ksplit, stream); break;
@@ -338,24 +442,24 @@ static int launch_bf16(const bf16_t* A, const bf16_t* W, const float* bias, TO* 
       default: launch_skinny_mt<TO, 4, EPI>(A, W, bias, C, M, N, K, lda, ldc, ksplit, stream); break;
     }
   } else {
-    const int NW_ = EPI == 1 ? 2 * N : N;           // rows of W = columns the tiles run over
-    dim3 grid((NW_ + T_BN - 1) / T_BN, (M + T_BM - 1) / T_BM);
-    hipLaunchKernelGGL((gemm_bf16_tile_kernel<TO, EPI>), grid, dim3(256), 0, stream, A, W, bias, C,
-                       M, NW_, K, lda, ldc);
+    // rows of W = columns the tiles run over
+    launch_tile<TO, EPI>(A, W, bias, C, M, EPI == 1 ? 2 * N : N, K, lda, ldc, ksplit,
+                         force_kernel >= 3 ? force_kernel - 2 : 0, stream);
   }
   KAPPAI_RETURN_LAUNCH_STATUS();
 }
 
 // K, lda must be multiples of 8 and A, W 16-byte aligned (checked by the caller).
-// force_kernel: 0 = by M, 1 = tile kernel, 2 = skinny kernel (M <= 64 only); for tests.
-// ksplit > 1 (M <= 64, float output only): C is [ksplit][M][ldc] partial sums over K ranges.
+// force_kernel: 0 = by M, 1 = tile kernel, 2 = skinny kernel (M <= 64 only), 3..6 = tile kernel
+// with block shape 1..4 (see launch_tile); for tests and tuning.
+// ksplit > 1 (float output only): C is [ksplit][M][ldc] partial sums over K ranges.
 extern "C" int kappai_gemm_bf16(const void* A, const void* W, const float* bias, void* C, int M,
                                 int N, int K, int lda, int ldc, int out_is_f32, int force_kernel,
                                 int ksplit, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
   if ((K % 8) || (lda % 8) || ksplit < 1 || ksplit > 64) return (int)hipErrorInvalidValue;
   if (force_kernel == 2 && M > 64) return (int)hipErrorInvalidValue;
-  if (ksplit > 1 && (M > 64 || force_kernel == 1 || !out_is_f32)) return (int)hipErrorInvalidValue;
+  if (ksplit > 1 && !out_is_f32) return (int)hipErrorInvalidValue;
   if (out_is_f32)
     return launch_bf16<float, 0>((const bf16_t*)A, (const bf16_t*)W, bias, (float*)C, M, N, K, lda,
                                  ldc, force_kernel, ksplit, stream);

@@ -110,7 +110,9 @@ def test_linear_float32_is_not_reduced_precision(ops):
     assert abs(got - K * (1.0 + 2.0 ** -12) ** 2) < 4e-6 and got != float(K)
 
 
-@pytest.mark.parametrize("M,N,K", GEMM_SHAPES + [(33, 130, 72), (48, 6144, 2048), (128, 128, 32)])
+@pytest.mark.parametrize("M,N,K", GEMM_SHAPES + [(33, 130, 72), (48, 6144, 2048), (128, 128, 32),
+                                                 (513, 640, 264), (2048, 3200, 96),
+                                                 (1999, 3330, 40)])
 @pytest.mark.parametrize("out_dtype", [F32, BF16])
 def test_linear_bfloat16(ops, M, N, K, out_dtype):
     x, w, b = rand((M, K), BF16, 9), rand((N, K), BF16, 10), rand((N,), F32, 11)
@@ -125,7 +127,8 @@ def test_linear_bfloat16(ops, M, N, K, out_dtype):
 
 
 @pytest.mark.parametrize("M,F,K", [(1, 16, 64), (8, 192, 64), (16, 320, 96), (33, 208, 120),
-                                   (64, 8192, 2048), (65, 320, 96), (200, 1008, 256)])
+                                   (64, 8192, 2048), (65, 320, 96), (200, 1008, 256),
+                                   (2048, 1616, 72)])
 def test_linear_swiglu(ops, M, F, K):
     x, wg, wu = rand((M, K), BF16, 16), rand((F, K), BF16, 17, 0.2), rand((F, K), BF16, 18, 0.2)
     w = ops.interleave_gate_up(wg.to(DEV), wu.to(DEV))
