@@ -31,9 +31,10 @@ typedef __attribute__((ext_vector_type(4))) uint32_t u32x4_t;
 typedef __attribute__((ext_vector_type(2))) uint32_t u32x2_t;
 
 __device__ __forceinline__ bf16x8_t as_frag(u32x4_t v) { return __builtin_bit_cast(bf16x8_t, v); }
-__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
-  return (uint32_t)f32_to_bf16(lo) | ((uint32_t)f32_to_bf16(hi) << 16);
-}
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) { return pack_bf16x2(lo, hi); }
+// 2^x for x <= 0 straight from the hardware (v_exp_f32); results below the normal range flush
+// to zero, which is what a softmax weight that small is worth
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 // keep the j-th of four bf16 values only if keep bit j is set
 __device__ __forceinline__ u32x2_t mask4(u32x2_t v, int keep) {
   const uint32_t m0 = ((keep & 1) ? 0x0000ffffu : 0u) | ((keep & 2) ? 0xffff0000u : 0u);
@@ -61,26 +62,29 @@ __device__ __forceinline__ u32x2_t load_vt4(const bf16_t* __restrict__ vt_pool,
   return keep == 15 ? v : mask4(v, keep);
 }
 
-// the same with the page already looked up
+// the same with the page already looked up.  The load itself is unconditional (from the pool's
+// first page when the keys are not wanted) and its result is masked, so that the compiler
+// keeps it in straight-line code and can leave it in flight across other work.
 __device__ __forceinline__ u32x2_t load_vt4_pg(const bf16_t* __restrict__ vt_pool, int page, int G,
                                                int g, int ps, int dd, int key0, int lo, int hi) {
-  u32x2_t z = {0u, 0u};
-  if (dd >= HEAD_DIM || key0 > hi || key0 + 3 < lo || page < 0) return z;
-  const bf16_t* p = vt_pool + (((size_t)page * G + g) * HEAD_DIM + dd) * ps + key0 % ps;
-  u32x2_t v = *reinterpret_cast<const u32x2_t*>(p);
+  const bool want = dd < HEAD_DIM && key0 <= hi && key0 + 3 >= lo && page >= 0;
+  const size_t off =
+      want ? (((size_t)page * G + g) * HEAD_DIM + dd) * ps + key0 % ps : (size_t)0;
+  u32x2_t v = *reinterpret_cast<const u32x2_t*>(vt_pool + off);
   int keep = 0;
 #pragma unroll
   for (int i = 0; i < 4; ++i)
-    if (key0 + i >= lo && key0 + i <= hi) keep |= 1 << i;
-  return keep == 15 ? v : mask4(v, keep);
+    if (want && key0 + i >= lo && key0 + i <= hi) keep |= 1 << i;
+  return mask4(v, keep);
 }
 
 __device__ __forceinline__ u32x4_t load_k8_pg(const bf16_t* __restrict__ k_pool, int page, int G,
                                               int g, int ps, int key, int d0, int lo, int hi) {
-  u32x4_t z = {0u, 0u, 0u, 0u};
-  if (d0 >= HEAD_DIM || key < lo || key > hi || page < 0) return z;
-  return *reinterpret_cast<const u32x4_t*>(
-      k_pool + (((size_t)page * G + g) * ps + key % ps) * HEAD_DIM + d0);
+  const bool want = d0 < HEAD_DIM && key >= lo && key <= hi && page >= 0;
+  const size_t off = want ? (((size_t)page * G + g) * ps + key % ps) * HEAD_DIM + d0 : (size_t)0;
+  u32x4_t v = *reinterpret_cast<const u32x4_t*>(k_pool + off);
+  const uint32_t m = want ? 0xffffffffu : 0u;
+  return (u32x4_t){v.x & m, v.y & m, v.z & m, v.w & m};
 }
 
 // eight consecutive d of key `key` starting at d0; zero outside [lo, hi] or beyond the head
@@ -136,9 +140,15 @@ __global__ __launch_bounds__(64) void attn_prefill_kernel(
   float m_run = -INFINITY, l_run = 0.f;
   const float sc = scale * LOG2E;
 
-  // The loads of the next 32 keys (their two page ids, key fragments, value fragments) are
-  // issued before the current 32 are worked on.  Page ids are the same for all lanes of a
-  // 16-key group, so they are looked up once per group.
+  // A tile of 32 keys is "whole" when every row of the q tile sees all of its keys: then nothing
+  // is masked, and addresses are a base that is the same for all lanes of a 16-key group (its
+  // page) plus an offset that a lane computes once.  The tiles at the window's lower edge and at
+  // the diagonal take the general path.  Either way the loads of the next tile are issued
+  // before the current one is worked on.
+  const int lo_last = (window > 0 && pos_last + 1 > window) ? pos_last + 1 - window : 0;
+  auto whole = [&](int kb) { return kb >= lo_last && kb + 31 <= pos_first; };
+  const int k_lane = (col % 16) * HEAD_DIM + 8 * hh;       // + 16*ks
+  const int v_lane = col * ps + 4 * hh;                    // + 32*mt*ps (+ 8)
   constexpr bool P_AHEAD = HEAD_DIM <= 128;      // beyond that the registers do not suffice
   constexpr int P_NB = P_AHEAD ? 2 : 1;
   u32x4_t kfr[P_NB][P_KS];
@@ -147,6 +157,30 @@ __global__ __launch_bounds__(64) void attn_prefill_kernel(
     const int g0 = min(kb / ps, max_blocks - 1), g1 = min((kb + 16) / ps, max_blocks - 1);
     const int pg0 = kb <= pos_last ? bt[g0] : -1;
     const int pg1 = kb + 16 <= pos_last ? bt[g1] : -1;
+    if (whole(kb)) {
+      const bf16_t* kb0p = k_pool + (((size_t)pg0 * G + g) * ps + kb % ps) * HEAD_DIM;
+      const bf16_t* kb1p = k_pool + (((size_t)pg1 * G + g) * ps + (kb + 16) % ps) * HEAD_DIM;
+      const bf16_t* kp = (col < 16 ? kb0p : kb1p) + k_lane;
+#pragma unroll
+      for (int ks = 0; ks < P_KS; ++ks)
+        kfr[buf][ks] = *reinterpret_cast<const u32x4_t*>(kp + 16 * ks);
+#pragma unroll
+      for (int st = 0; st < 2; ++st) {
+        const bf16_t* vp = vt_pool + ((size_t)(st == 0 ? pg0 : pg1) * G + g) * HEAD_DIM * ps +
+                           (kb + 16 * st) % ps + v_lane;
+#pragma unroll
+        for (int mt = 0; mt < P_MT; ++mt) {
+          const bool dok = HEAD_DIM % 32 == 0 || 32 * mt + col < HEAD_DIM;
+          const bf16_t* vq = vp + (dok ? 32 * mt * ps : -v_lane);
+          u32x2_t a = *reinterpret_cast<const u32x2_t*>(vq);
+          u32x2_t b = *reinterpret_cast<const u32x2_t*>(vq + 8);
+          if (!dok) a = b = (u32x2_t){0u, 0u};
+          vfa[buf][st][mt] = a;
+          vfb[buf][st][mt] = b;
+        }
+      }
+      return;
+    }
     const int my_key = kb + col;
     const int my_pg = col < 16 ? pg0 : pg1;
 #pragma unroll
@@ -175,21 +209,27 @@ __global__ __launch_bounds__(64) void attn_prefill_kernel(
       s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_frag(kfr[buf][ks]), qf[ks], s, 0, 0, 0);
     // lane holds, for query `col`, keys kb + 8*(v/4) + 4*hh + v%4
     float mloc = -INFINITY;
+    if (whole(kb)) {
 #pragma unroll
-    for (int v = 0; v < 16; ++v) {
-      const int key = kb + 8 * (v / 4) + 4 * hh + v % 4;
-      const bool ok = key <= my_pos && key >= my_lo;
-      s[v] = ok ? s[v] * sc : -INFINITY;
-      mloc = fmaxf(mloc, s[v]);
+      for (int v = 0; v < 16; ++v) mloc = fmaxf(mloc, s[v]);
+      mloc *= sc;           // sc > 0: scaling commutes with the maximum
+    } else {
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int key = kb + 8 * (v / 4) + 4 * hh + v % 4;
+        const bool ok = key <= my_pos && key >= my_lo;
+        s[v] = ok ? s[v] : -INFINITY;
+        mloc = fmaxf(mloc, s[v] * sc);
+      }
     }
     mloc = fmaxf(mloc, __shfl_xor(mloc, 32, WAVE));
     const float m_new = fmaxf(m_run, mloc);
     const float m_safe = m_new == -INFINITY ? 0.f : m_new;
-    const float corr = exp2f(m_run - m_safe);
+    const float corr = fast_exp2(m_run - m_safe);
     float lsum = 0.f;
 #pragma unroll
     for (int v = 0; v < 16; ++v) {
-      s[v] = exp2f(s[v] - m_safe);
+      s[v] = fast_exp2(fmaf(s[v], sc, -m_safe));
       lsum += s[v];
     }
     lsum += __shfl_xor(lsum, 32, WAVE);
@@ -350,13 +390,13 @@ __global__ __launch_bounds__(64) void attn_decode_kernel(
       mloc = fmaxf(mloc, __shfl_xor(mloc, 32, WAVE));
       const float m_new = fmaxf(m_run, mloc);
       const float m_safe = m_new == -INFINITY ? 0.f : m_new;
-      const float corr = exp2f(m_run - m_safe);
+      const float corr = fast_exp2(m_run - m_safe);
       float lsum = 0.f;
 #pragma unroll
       for (int tt = 0; tt < 2; ++tt)
 #pragma unroll
         for (int v = 0; v < 4; ++v) {
-          s[tt][v] = exp2f(s[tt][v] - m_safe);
+          s[tt][v] = fast_exp2(s[tt][v] - m_safe);
           lsum += s[tt][v];
         }
       lsum += __shfl_xor(lsum, 16, WAVE);
@@ -410,7 +450,7 @@ __global__ __launch_bounds__(MERGE_WAVES * WAVE) void attn_merge_kernel(
     float wgt = 0.f, l = 0.f;
     if (s < n_splits) {
       const float m = part_ml[2 * (base + s)];
-      wgt = m == -INFINITY ? 0.f : exp2f(m - M);
+      wgt = m == -INFINITY ? 0.f : fast_exp2(m - M);
       l = part_ml[2 * (base + s) + 1] * wgt;
     }
     L += wave_sum(l);
