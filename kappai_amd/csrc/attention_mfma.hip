@@ -11,7 +11,8 @@
 // The value pool is stored transposed, [page][kv_head][head_dim][page_size], which makes the
 // 8 key slots of the A operand two 8-byte loads.  page_size must be a multiple of 16.
 //
-//   attn_prefill   v_mfma_f32_32x32x16_bf16; one wave per (tile of 32 rows of a segment, head)
+//   attn_prefill   v_mfma_f32_32x32x16_bf16; one block per (tile of 32 rows of a segment, head),
+//                  its waves sharing out the key tiles
 //   attn_decode    v_mfma_f32_16x16x32_bf16; one wave per (row, kv head, split of the keys): the
 //                  query heads that share the kv head are the columns; partial results are
 //                  merged by attn_merge.
@@ -105,13 +106,19 @@ __device__ __forceinline__ u32x4_t load_k8(const bf16_t* __restrict__ k_pool,
 #define P_KS (HEAD_DIM / 16)            // k-steps of S^T over d
 #define P_MT ((HEAD_DIM + 31) / 32)     // row tiles of O^T over d
 
-__global__ __launch_bounds__(64) void attn_prefill_kernel(
+// waves of a block: they share one q tile and take its key tiles in turn, which shortens the
+// longest chain of dependent work fourfold; their partial results meet in LDS
+#define P_NW (HEAD_DIM <= 128 ? 4 : 1)
+
+__global__ __launch_bounds__(P_NW * WAVE) void attn_prefill_kernel(
     const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ k_pool,
     const bf16_t* __restrict__ vt_pool, bf16_t* __restrict__ out, int out_stride,
     const int* __restrict__ q_tiles, const int* __restrict__ row_pos,
     const int* __restrict__ block_tables, int max_blocks, int H, int G, int ps, int window,
     float scale) {
-  const int tile = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  // later tiles of a segment have more keys: they are started first
+  const int tile = gridDim.x - 1 - blockIdx.x, h = blockIdx.y;
+  const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE;
   const int seg = q_tiles[4 * tile], r0 = q_tiles[4 * tile + 1], nr = q_tiles[4 * tile + 2];
   const int g = h / (H / G);
   const int col = lane % 32, hh = lane / 32;
@@ -255,22 +262,57 @@ __global__ __launch_bounds__(64) void attn_prefill_kernel(
       }
     }
   };
-  const int kb0 = (lo_tile / 32) * 32;
+  // wave w takes the key tiles kb0 + 32 * (w + P_NW * i)
+  const int kb0 = (lo_tile / 32) * 32 + 32 * wave;
+  constexpr int KSTEP = 32 * P_NW;
   if (P_AHEAD) {
-    fetch(0, kb0);
-    for (int kb = kb0; kb <= pos_last; kb += 64) {
-      if (kb + 32 <= pos_last) fetch(P_NB - 1, kb + 32);
+    if (kb0 <= pos_last) fetch(0, kb0);
+    for (int kb = kb0; kb <= pos_last; kb += 2 * KSTEP) {
+      if (kb + KSTEP <= pos_last) fetch(P_NB - 1, kb + KSTEP);
       work(0, kb);
-      if (kb + 32 <= pos_last) {
-        if (kb + 64 <= pos_last) fetch(0, kb + 64);
-        work(P_NB - 1, kb + 32);
+      if (kb + KSTEP <= pos_last) {
+        if (kb + 2 * KSTEP <= pos_last) fetch(0, kb + 2 * KSTEP);
+        work(P_NB - 1, kb + KSTEP);
       }
     }
   } else {
-    for (int kb = kb0; kb <= pos_last; kb += 32) {
+    for (int kb = kb0; kb <= pos_last; kb += KSTEP) {
       fetch(0, kb);
       work(0, kb);
     }
+  }
+  if (P_NW > 1) {
+    // merge: every wave rescales to the common maximum; waves 1.. hand their sums to wave 0
+    __shared__ float sh_m[P_NW][32], sh_l[P_NW][32];
+    __shared__ float sh_o[P_NW > 1 ? P_NW - 1 : 1][P_MT * 16][WAVE];
+    if (hh == 0) sh_m[wave][col] = m_run;
+    __syncthreads();
+    float M = sh_m[0][col];
+#pragma unroll
+    for (int w = 1; w < P_NW; ++w) M = fmaxf(M, sh_m[w][col]);
+    const float f = m_run == -INFINITY ? 0.f : fast_exp2(m_run - M);
+    l_run *= f;
+    if (hh == 0) sh_l[wave][col] = l_run;
+    if (wave > 0) {
+#pragma unroll
+      for (int mt = 0; mt < P_MT; ++mt)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) sh_o[wave - 1][mt * 16 + v][lane] = o[mt][v] * f;
+    }
+    __syncthreads();
+    if (wave > 0) return;
+    l_run = sh_l[0][col];
+#pragma unroll
+    for (int w = 1; w < P_NW; ++w) l_run += sh_l[w][col];
+#pragma unroll
+    for (int mt = 0; mt < P_MT; ++mt)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        float acc = o[mt][v] * f;
+#pragma unroll
+        for (int w = 1; w < P_NW; ++w) acc += sh_o[w - 1][mt * 16 + v][lane];
+        o[mt][v] = acc;
+      }
   }
   if (!row_ok) return;
   const float inv = l_run > 0.f ? 1.0f / l_run : 0.f;
@@ -494,7 +536,7 @@ extern "C" int kappai_attn_prefill(const void* q, int q_stride, const void* k_po
   if (n_tiles <= 0) return 0;
   if (ps % 16 || G < 1 || H % G || H > 65535 || (q_stride % 8) || (out_stride % 4))
     return (int)hipErrorInvalidValue;
-  hipLaunchKernelGGL(attn_prefill_kernel, dim3(n_tiles, H), dim3(WAVE), 0, stream,
+  hipLaunchKernelGGL(attn_prefill_kernel, dim3(n_tiles, H), dim3(P_NW * WAVE), 0, stream,
                      (const bf16_t*)q, q_stride, (const bf16_t*)k_pool, (const bf16_t*)vt_pool,
                      (bf16_t*)out, out_stride, q_tiles, row_pos, block_tables, max_blocks, H, G,
                      ps, window, scale);
