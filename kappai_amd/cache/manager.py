@@ -131,6 +131,7 @@ class RequestCache:
         self.length = 0
         self.blocks: List[List[int]] = [[] for _ in range(n_paged_groups)]  # -1 = given back
         self.closed = False
+        self.version = 0        # counts changes of `blocks`, for callers that mirror them
 
     def __repr__(self):
         return f"RequestCache({self.request_id!r}, slot={self.slot}, length={self.length})"
@@ -178,6 +179,7 @@ class CacheManager:
                 self._where[cid] = (kind, gi)
         self._free_slots: List[int] = list(range(num_slots - 1, -1, -1))
         self._live: Dict[Hashable, RequestCache] = {}
+        self._has_windows = any(g.spec.window for g in self.paged_groups)
         self.device = None
         self.dtype = None
 
@@ -284,6 +286,24 @@ class CacheManager:
         for gi, g in enumerate(self.paged_groups):
             for _ in range(need[gi]):
                 rc.blocks[gi].append(g.allocator.take(rc.request_id))
+        if any(need):
+            rc.version += 1
+
+    def extend_one(self, rc: RequestCache) -> None:
+        """``extend(rc, 1)`` for the common case of a decoded token: nothing to do unless the
+        token opens a new page."""
+        if rc.length % self.page_size == 0 or any(
+                len(b) * self.page_size <= rc.length for b in rc.blocks):
+            self.extend(rc, 1)
+        elif rc.closed:
+            raise CacheError(f"{rc} is not an open request of this cache")
+
+    def commit_one(self, rc: RequestCache) -> None:
+        """``commit(rc, 1)``; without window groups only the length changes."""
+        if self._has_windows:
+            self.commit(rc, 1)
+        else:
+            rc.length += 1
 
     def commit(self, rc: RequestCache, n_new: int) -> None:
         """The step has stored ``n_new`` tokens.  Pages that no later position can see
@@ -302,6 +322,7 @@ class CacheManager:
                 if rc.blocks[gi][b] >= 0:
                     g.allocator.give_back(rc.blocks[gi][b], rc.request_id)
                     rc.blocks[gi][b] = -1
+                    rc.version += 1
                 b += 1
 
     def trim_uncommitted(self, rc: RequestCache) -> None:
@@ -310,6 +331,7 @@ class CacheManager:
         for gi, g in enumerate(self.paged_groups):
             while len(rc.blocks[gi]) > keep:
                 page = rc.blocks[gi].pop()
+                rc.version += 1
                 if page >= 0:
                     g.allocator.give_back(page, rc.request_id)
 

@@ -34,57 +34,79 @@ def _context_bucket(n_positions: int) -> int:
 class _DecodeGraph:
     """One captured HIP graph of the model's forward pass for B single-token segments whose
     positions lie below ``ctx_cap``: static row tables that every step overwrites, a static
-    logits tensor that every replay fills."""
+    logits tensor that every replay fills.  The host keeps a mirror of the tables and rewrites
+    only what changes from step to step (a block-table row only when its request's pages
+    changed)."""
 
-    def __init__(self, runner: "StepRunner", arrays, sizes, ctx_cap: int):
-        self.order = list(arrays)
-        self.shapes = {k: arrays[k].shape for k in self.order}
+    def __init__(self, runner: "StepRunner", B: int, n_logit: int, ctx_cap: int):
+        cache = runner.cache
+        n_groups = len(cache.paged_groups)
+        self.B, self.n_logit, self.width = B, n_logit, ctx_cap // cache.page_size + 1
+        shapes = [("tokens", (B,)), ("row_pos", (B,)), ("row_seg", (B,)), ("seg_start", (B + 1,)),
+                  ("seg_pos0", (B,)), ("seg_slot", (B,)), ("logit_rows", (n_logit,)),
+                  ("q_tiles", (B, 4))]
+        shapes += [(f"block_table_{g}", (B, self.width)) for g in range(n_groups)]
         self.offsets, total = {}, 0
-        for k in self.order:
+        for k, shp in shapes:
             self.offsets[k] = total
-            total += (arrays[k].size + 3) // 4 * 4
+            total += (int(np.prod(shp)) + 3) // 4 * 4
         self.total = max(total, 4)
+        self.mirror = np.zeros(self.total, dtype=np.int32)
+        self.h = {k: self.mirror[self.offsets[k]:self.offsets[k] + int(np.prod(shp))].reshape(shp)
+                  for k, shp in shapes}
         dev = runner.device
         self.static = torch.zeros(self.total, dtype=torch.int32, device=dev)
-        views = {k: self.static[self.offsets[k]:self.offsets[k] + arrays[k].size].view(
-            arrays[k].shape) for k in self.order}
-        B = sizes["n_rows"]
+        views = {k: self.static[self.offsets[k]:self.offsets[k] + int(np.prod(shp))].view(shp)
+                 for k, shp in shapes}
         self.batch = RowBatch(
-            n_rows=B, n_segments=B, n_logit_rows=sizes["n_logit_rows"], max_position=ctx_cap - 1,
+            n_rows=B, n_segments=B, n_logit_rows=n_logit, max_position=ctx_cap - 1,
             max_segment_rows=1, tokens=views["tokens"], row_pos=views["row_pos"],
             row_seg=views["row_seg"], seg_start=views["seg_start"], seg_pos0=views["seg_pos0"],
             seg_slot=views["seg_slot"], logit_rows=views["logit_rows"], q_tiles=views["q_tiles"],
-            block_tables=[views[f"block_table_{g}"] for g in range(sizes["n_groups"])], host={})
+            block_tables=[views[f"block_table_{g}"] for g in range(n_groups)], host={})
+        # what never changes
+        self.h["row_seg"][:] = np.arange(B)
+        self.h["seg_start"][:] = np.arange(B + 1)
+        self.h["q_tiles"][:, 0] = np.arange(B)
+        self.h["q_tiles"][:, 1] = np.arange(B)
+        self.h["q_tiles"][:, 2] = 1
         # a warm-up run on the scratch page and the scratch slot: every kernel of this shape is
         # loaded and has run once before the capture, and no request's cache is touched
-        cache = runner.cache
-        warm = {k: np.zeros(arrays[k].shape, dtype=np.int32) for k in self.order}
-        warm["row_seg"][:] = np.arange(B)
-        warm["seg_start"][:] = np.arange(B + 1)
-        warm["seg_slot"][:] = cache.scratch_slot
-        warm["logit_rows"][:] = np.arange(sizes["n_logit_rows"]) % B
-        warm["q_tiles"][:, 0] = np.arange(B)
-        warm["q_tiles"][:, 1] = np.arange(B)
-        warm["q_tiles"][:, 2] = 1
-        for g in range(sizes["n_groups"]):
-            warm[f"block_table_{g}"][:] = cache.scratch_page(g)
-        self.load(runner, warm)
+        self.h["seg_slot"][:] = cache.scratch_slot
+        self.h["logit_rows"][:] = np.arange(n_logit) % B
+        for g in range(n_groups):
+            self.h[f"block_table_{g}"][:] = cache.scratch_page(g)
+        self.rows_of = [None] * B        # (request cache, version) whose pages row si mirrors
+        self._upload(runner)
         runner.model.forward(self.batch, cache)
         torch.cuda.synchronize(dev)
         self.graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(self.graph):
             self.logits = runner.model.forward(self.batch, cache)
 
-    def load(self, runner: "StepRunner", arrays) -> None:
+    def _upload(self, runner: "StepRunner") -> None:
         host = runner._stage(self.total)
-        for k in self.order:
-            a = arrays[k].reshape(-1)
-            host[self.offsets[k]:self.offsets[k] + a.size] = a
+        host[:self.total] = self.mirror
         self.static.copy_(runner._staging[:self.total], non_blocking=True)
         runner._mark_staged()
 
-    def run(self, runner: "StepRunner", arrays) -> torch.Tensor:
-        self.load(runner, arrays)
+    def run(self, runner: "StepRunner", caches, tokens, pos, slots, logit_rows) -> torch.Tensor:
+        h = self.h
+        h["tokens"][:] = tokens
+        h["row_pos"][:] = pos
+        h["seg_pos0"][:] = pos
+        h["seg_slot"][:] = slots
+        h["logit_rows"][:] = logit_rows
+        for si, rc in enumerate(caches):
+            seen = self.rows_of[si]
+            if seen is None or seen[0] is not rc or seen[1] != rc.version:
+                for g in range(len(rc.blocks)):
+                    row = h[f"block_table_{g}"][si]
+                    b = rc.blocks[g]
+                    row[:len(b)] = b
+                    row[len(b):] = -1
+                self.rows_of[si] = (rc, rc.version)
+        self._upload(runner)
         self.graph.replay()
         return self.logits
 
@@ -159,17 +181,26 @@ class StepRunner:
         """Replay the graph for this many single-token segments, capturing it the second time
         its shape is seen.  Returns None when the step should run eagerly.  The logits live in
         the graph's own buffer and are overwritten by its next replay."""
-        arrays, sizes = layout_rows(entries, self.cache, self.model.vocab_size)
-        ctx_cap = _context_bucket(sizes["max_position"] + 1)
-        width = ctx_cap // self.cache.page_size + 1
-        for g in range(sizes["n_groups"]):
-            bt = arrays[f"block_table_{g}"]
-            if bt.shape[1] > width:
+        B = len(entries)
+        caches = [e.cache for e in entries]
+        if len({id(c) for c in caches}) != B:
+            return None                     # the eager path reports the duplicate
+        tokens = np.fromiter((e.tokens[0] for e in entries), dtype=np.int64, count=B)
+        if tokens.min() < 0 or tokens.max() >= self.model.vocab_size:
+            return None                     # the eager path reports the bad id
+        logit_rows = []
+        for si, e in enumerate(entries):
+            if len(e.want) == 1 and int(e.want[0]) == 0:
+                logit_rows.append(si)
+            elif len(e.want) != 0:
                 return None
-            padded = np.full((bt.shape[0], width), -1, dtype=np.int32)
-            padded[:, :bt.shape[1]] = bt
-            arrays[f"block_table_{g}"] = padded
-        key = (sizes["n_rows"], sizes["n_logit_rows"], ctx_cap)
+        # positions before this step's tokens were made room for: length is not yet committed
+        pos = np.fromiter((c.length for c in caches), dtype=np.int32, count=B)
+        ctx_cap = _context_bucket(int(pos.max()) + 1)
+        width = ctx_cap // self.cache.page_size + 1
+        if any(len(b) > width for c in caches for b in c.blocks):
+            return None
+        key = (B, len(logit_rows), ctx_cap)
         graph = self._graphs.get(key)
         if graph is None:
             self._graph_seen[key] = self._graph_seen.get(key, 0) + 1
@@ -177,9 +208,10 @@ class StepRunner:
                 return None
             if len(self._graphs) >= MAX_DECODE_GRAPHS:
                 self._graphs.pop(next(iter(self._graphs)))
-            graph = self._graphs[key] = _DecodeGraph(self, arrays, sizes, ctx_cap)
+            graph = self._graphs[key] = _DecodeGraph(self, B, len(logit_rows), ctx_cap)
+        slots = np.fromiter((c.slot for c in caches), dtype=np.int32, count=B)
         self.graph_replays += 1
-        return graph.run(self, arrays)
+        return graph.run(self, caches, tokens, pos, slots, logit_rows)
 
     # -- one step ----------------------------------------------------------------------------
     def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
@@ -188,10 +220,14 @@ class StepRunner:
         their ``want``.  If the pages do not suffice, ``OutOfPages`` is raised and neither
         the cache nor any request has changed."""
         entries = list(entries)
+        single = all(len(e.tokens) == 1 for e in entries)
         extended: List[StepEntry] = []
         try:
             for e in entries:
-                self.cache.extend(e.cache, len(e.tokens))
+                if single:
+                    self.cache.extend_one(e.cache)
+                else:
+                    self.cache.extend(e.cache, len(e.tokens))
                 extended.append(e)
         except OutOfPages:
             for e in extended:
@@ -199,7 +235,7 @@ class StepRunner:
             raise
         try:
             logits = None
-            if self.decode_graphs and all(len(e.tokens) == 1 for e in entries):
+            if self.decode_graphs and single:
                 logits = self._decode_step(entries)
             if logits is None:
                 batch = self.make_batch(entries)
@@ -209,6 +245,9 @@ class StepRunner:
                 self.cache.trim_uncommitted(e.cache)
             raise
         for e in entries:
-            self.cache.commit(e.cache, len(e.tokens))
+            if single:
+                self.cache.commit_one(e.cache)
+            else:
+                self.cache.commit(e.cache, len(e.tokens))
         self.steps_run += 1
         return logits

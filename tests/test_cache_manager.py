@@ -168,3 +168,21 @@ def test_random_orders(seed):
     assert all(g.allocator.num_free == g.allocator.num_pages for g in cm.paged_groups)
     assert cm.num_free_slots == cm.num_slots
     assert ended > 20
+
+
+def test_one_token_shortcuts_equal_the_general_calls():
+    for window in (None, 6):
+        a = CacheManager([PagedKV(1, 8, window=window), FixedState((4,))], 4, 12, 1)
+        b = CacheManager([PagedKV(1, 8, window=window), FixedState((4,))], 4, 12, 1)
+        ra, rb = a.open("x"), b.open("x")
+        a.extend(ra, 3); a.commit(ra, 3)
+        b.extend(rb, 3); b.commit(rb, 3)
+        versions = []
+        for _ in range(30):
+            a.extend(ra, 1); a.commit(ra, 1)
+            b.extend_one(rb); b.commit_one(rb)
+            assert ra.blocks == rb.blocks and ra.length == rb.length
+            a.check(); b.check()
+            versions.append(rb.version)
+        assert versions[-1] > versions[0]           # page changes are counted
+        assert len(set(versions)) < len(versions)   # and only they
