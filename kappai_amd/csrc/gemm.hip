@@ -270,8 +270,8 @@ static void launch_tile_cfg(const bf16_t* A, const bf16_t* W, const float* bias,
   auto kern = gemm_bf16_tile_kernel<TO, EPI, WAVES_M, WAVES_N, WM, WN, BK, NBUF, OCC>;
   static bool attr_set = false;       // more than 64 KB of LDS has to be asked for once
   if (!attr_set) {
-    hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
-                        (int)lds_bytes);
+    (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
+                              (int)lds_bytes);
     attr_set = true;
   }
   const int tn = (n_rows_w + BN - 1) / BN, tm = (M + BM - 1) / BM;
@@ -322,11 +322,24 @@ static void launch_tile(const bf16_t* A, const bf16_t* W, const float* bias, TO*
 // their 16 up rows of the interleaved W; N is the number of output columns.
 // gridDim.y > 1 splits K over blocks as well: block (x, y) writes its partial sums to
 // C + y * M * ldc (float), which the consumer adds up in a fixed order.
+// EPI 2 (gated short convolution, one decoded row a request; kappai:
+// src/backend/cpu/common.c:2393-2431): W is the conv layer's in_proj [3N, K]; a block owns 16
+// channels and streams their B, C and x rows (N rows apart), then bx = B*x meets the request's
+// state, the taps give s, the kernel writes C*s and shifts the state.
+struct ConvStep {
+  const float* taps;       // [N, L]
+  const float* conv_bias;  // [N] or null
+  float* state;            // [slots, N, L-1]
+  const int* seg_pos0;     // [M]: position of the row (0: no history)
+  const int* seg_slot;     // [M]
+  int L;
+};
+
 template <typename TO, int MT, int NW, int EPI>
 __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny_kernel(
     const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, const float* __restrict__ bias,
-    TO* __restrict__ C, int M, int N, int K, int lda, int ldc) {
-  constexpr int NG = EPI == 1 ? 2 : 1;      // row groups of W a block streams
+    TO* __restrict__ C, int M, int N, int K, int lda, int ldc, ConvStep cs) {
+  constexpr int NG = EPI == 1 ? 2 : (EPI == 2 ? 3 : 1);      // row groups of W a block streams
   __shared__ float red[NW][NG * MT][WAVE][4];
   const int tid = threadIdx.x;
   const int lane = tid % WAVE, wave = tid / WAVE;
@@ -337,8 +350,10 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny_kernel(
   f32x4_t acc[NG * MT];
 #pragma unroll
   for (int t = 0; t < NG * MT; ++t) acc[t] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
-  // plain: row gn.  SwiGLU: gate row 32*block + col, up row 16 further
+  // plain: row gn.  SwiGLU: gate row 32*block + col, up row 16 further.  Conv: rows gn, N + gn,
+  // 2N + gn.
   const size_t wr0 = EPI == 1 ? (size_t)blockIdx.x * 32 + col : (size_t)gn;
+  const size_t group_rows = EPI == 2 ? (size_t)N : 16;
   const bf16_t* wrow = W + (gn < N ? wr0 : 0) * K + kg;
   const bf16_t* arow[MT];
 #pragma unroll
@@ -353,7 +368,7 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny_kernel(
   const int k1 = min(kb1, k0 + kper);
   C += (size_t)blockIdx.y * M * ldc;
   // loads in flight a lane: U * (NG + MT)
-  constexpr int U = (NG + MT) <= 2 ? SK_UNROLL : ((NG + MT) <= 4 ? 4 : 2);
+  constexpr int U = (NG + MT) <= 3 ? SK_UNROLL : ((NG + MT) <= 4 ? 4 : 2);
   for (int k = k0; k < k1; k += 32 * U) {
     u32x4_t wv[U][NG], av[U][MT];
 #pragma unroll
@@ -362,7 +377,7 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny_kernel(
       const bool kin = gk + kg < k1;
 #pragma unroll
       for (int r = 0; r < NG; ++r)
-        wv[u][r] = (kin && gn < N) ? load16(wrow + (size_t)r * 16 * K + gk) : zero;
+        wv[u][r] = (kin && gn < N) ? load16(wrow + r * group_rows * K + gk) : zero;
 #pragma unroll
       for (int t = 0; t < MT; ++t)
         av[u][t] = (kin && t * 16 + col < M) ? load16(arow[t] + gk) : zero;
@@ -397,6 +412,35 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny_kernel(
 #pragma unroll
           for (int w = 1; w < NW; ++w) up += red[w][MT + t][lane][v];
           store_out(C + (size_t)gm * ldc + gn, silu_f(sum) * up);
+        } else if (EPI == 2) {
+          float cg = red[0][MT + t][lane][v], xg = red[0][2 * MT + t][lane][v];
+#pragma unroll
+          for (int w = 1; w < NW; ++w) {
+            cg += red[w][MT + t][lane][v];
+            xg += red[w][2 * MT + t][lane][v];
+          }
+          float bg = sum;
+          if (bias) {
+            bg += bias[gn];
+            cg += bias[N + gn];
+            xg += bias[2 * N + gn];
+          }
+          // the three gates are rounded as the unfused path stores them
+          const float bx = to_f32(f32_to_bf16(bg)) * to_f32(f32_to_bf16(xg));
+          const int H = cs.L - 1;
+          const bool fresh = cs.seg_pos0[gm] == 0;
+          float* st = cs.state + ((size_t)cs.seg_slot[gm] * N + gn) * H;
+          const float* wc = cs.taps + (size_t)gn * cs.L;
+          float s = cs.conv_bias ? cs.conv_bias[gn] : 0.f;
+          float prev = fresh ? 0.f : st[0];
+          for (int k = 0; k < H; ++k) {
+            s += wc[k] * prev;
+            const float next = (k + 1 < H) ? (fresh ? 0.f : st[k + 1]) : bx;
+            st[k] = next;
+            prev = next;
+          }
+          s += wc[H] * bx;
+          store_out(C + (size_t)gm * ldc + gn, to_f32(f32_to_bf16(cg)) * s);
         } else {
           store_out(C + (size_t)gm * ldc + gn, sum + bv);
         }
@@ -407,39 +451,50 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny_kernel(
 
 template <typename TO, int MT, int NW, int EPI>
 static void launch_skinny(const bf16_t* A, const bf16_t* W, const float* bias, TO* C, int M, int N,
-                          int K, int lda, int ldc, int ksplit, hipStream_t stream) {
+                          int K, int lda, int ldc, int ksplit, ConvStep cs, hipStream_t stream) {
   hipLaunchKernelGGL((gemm_bf16_skinny_kernel<TO, MT, NW, EPI>), dim3((N + 15) / 16, ksplit),
-                     dim3(NW * WAVE), 0, stream, A, W, bias, C, M, N, K, lda, ldc);
+                     dim3(NW * WAVE), 0, stream, A, W, bias, C, M, N, K, lda, ldc, cs);
 }
 
 // more waves a block when there are few blocks, so that about 2048 waves or more stream W
 template <typename TO, int MT, int EPI>
 static void launch_skinny_mt(const bf16_t* A, const bf16_t* W, const float* bias, TO* C, int M,
-                             int N, int K, int lda, int ldc, int ksplit, hipStream_t stream) {
+                             int N, int K, int lda, int ldc, int ksplit, ConvStep cs,
+                             hipStream_t stream) {
   const int blocks = ((N + 15) / 16) * ksplit;
   const int kb = K / ksplit;                              // K a block
-  constexpr int MAXW = 16 / (MT * (EPI == 1 ? 2 : 1));   // LDS for the partial results
-  if (blocks * 4 >= 2048 || kb <= 512 || MAXW <= 4)
-    launch_skinny<TO, MT, 4, EPI>(A, W, bias, C, M, N, K, lda, ldc, ksplit, stream);
-  else if (blocks * 8 >= 2048 || kb <= 1024 || MAXW <= 8)
-    launch_skinny<TO, MT, (MAXW >= 8 ? 8 : 4), EPI>(A, W, bias, C, M, N, K, lda, ldc, ksplit,
+  constexpr int NG = EPI == 1 ? 2 : (EPI == 2 ? 3 : 1);
+  constexpr int MAXW = 48 / (MT * NG);                    // 1 KB of LDS a wave, group and row tile
+  if (blocks * 4 >= 2048 || kb <= 512 || MAXW < 8)
+    launch_skinny<TO, MT, 4, EPI>(A, W, bias, C, M, N, K, lda, ldc, ksplit, cs, stream);
+  else if (blocks * 8 >= 2048 || kb <= 1024 || MAXW < 16)
+    launch_skinny<TO, MT, (MAXW >= 8 ? 8 : 4), EPI>(A, W, bias, C, M, N, K, lda, ldc, ksplit, cs,
                                                     stream);
   else
-    launch_skinny<TO, MT, (MAXW >= 16 ? 16 : 4), EPI>(A, W, bias, C, M, N, K, lda, ldc, ksplit,
+    launch_skinny<TO, MT, (MAXW >= 16 ? 16 : 4), EPI>(A, W, bias, C, M, N, K, lda, ldc, ksplit, cs,
                                                       stream);
 }
 
 template <typename TO, int EPI>
 static int launch_bf16(const bf16_t* A, const bf16_t* W, const float* bias, TO* C, int M, int N,
-                       int K, int lda, int ldc, int force_kernel, int ksplit, hipStream_t stream) {
+                       int K, int lda, int ldc, int force_kernel, int ksplit, hipStream_t stream,
+                       ConvStep cs = ConvStep{}) {
   // N counts output columns; with the SwiGLU epilogue W has 2N rows
   if (M <= 64 && force_kernel != 1 && force_kernel < 3) {
     const int mt = (M + 15) / 16;
     switch (mt) {
-      case 1: launch_skinny_mt<TO, 1, EPI>(A, W, bias, C, M, N, K, lda, ldc, ksplit, stream); break;
-      case 2: launch_skinny_mt<TO, 2, EPI>(A, W, bias, C, M, N, K, lda, ldc, ksplit, stream); break;
-      case 3: launch_skinny_mt<TO, 3, EPI>(A, W, bias, C, M, N, K, lda, ldc, ksplit, stream); break;
-      default: launch_skinny_mt<TO, 4, EPI>(A, W, bias, C, M, N, K, lda, ldc, ksplit, stream); break;
+      case 1:
+        launch_skinny_mt<TO, 1, EPI>(A, W, bias, C, M, N, K, lda, ldc, ksplit, cs, stream);
+        break;
+      case 2:
+        launch_skinny_mt<TO, 2, EPI>(A, W, bias, C, M, N, K, lda, ldc, ksplit, cs, stream);
+        break;
+      case 3:
+        launch_skinny_mt<TO, 3, EPI>(A, W, bias, C, M, N, K, lda, ldc, ksplit, cs, stream);
+        break;
+      default:
+        launch_skinny_mt<TO, 4, EPI>(A, W, bias, C, M, N, K, lda, ldc, ksplit, cs, stream);
+        break;
     }
   } else {
     // rows of W = columns the tiles run over
@@ -476,4 +531,18 @@ extern "C" int kappai_gemm_bf16_swiglu(const void* A, const void* W, void* C, in
   if (force_kernel == 2 && M > 64) return (int)hipErrorInvalidValue;
   return launch_bf16<bf16_t, 1>((const bf16_t*)A, (const bf16_t*)W, nullptr, (bf16_t*)C, M, F, K,
                                 lda, ldc, force_kernel, 1, stream);
+}
+
+// Conv layer decode step in one kernel: C[M, D] = Cgate * conv(Bgate * x | state) from A [M, K]
+// and the in_proj matrix W [3D, K]; M <= 64, one row a request; D a multiple of 16.
+extern "C" int kappai_gemm_bf16_shortconv_step(const void* A, const void* W, const float* bias,
+                                               void* C, int M, int D, int K, int lda,
+                                               const float* taps, const float* conv_bias,
+                                               float* state, const int* seg_pos0,
+                                               const int* seg_slot, int L, hipStream_t stream) {
+  if (M <= 0 || D <= 0) return 0;
+  if ((K % 8) || (lda % 8) || (D % 16) || M > 64 || L < 2) return (int)hipErrorInvalidValue;
+  ConvStep cs{taps, conv_bias, state, seg_pos0, seg_slot, L};
+  return launch_bf16<bf16_t, 2>((const bf16_t*)A, (const bf16_t*)W, bias, (bf16_t*)C, M, D, K, lda,
+                                D, 2, 1, stream, cs);
 }

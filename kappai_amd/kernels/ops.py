@@ -226,6 +226,43 @@ def linear_swiglu(x: torch.Tensor, weight: torch.Tensor, force_kernel: int = 0) 
     return out
 
 
+def linear_shortconv_step(x: torch.Tensor, in_proj: torch.Tensor, in_bias: Optional[torch.Tensor],
+                          taps: torch.Tensor, conv_bias: Optional[torch.Tensor],
+                          state: torch.Tensor, seg_pos0: torch.Tensor,
+                          seg_slot: torch.Tensor) -> torch.Tensor:
+    """A conv layer's decode step in one kernel, for a batch in which every row is its own
+    segment: ``proj = x in_proj^T (+ bias)`` cut into (B | C | x), ``C * conv(B * x)`` with the
+    rows' state slots read and shifted.  bfloat16, at most 64 rows, width a multiple of 16.
+    Equals ``shortconv(linear(x, in_proj, in_bias), ...)``."""
+    _gpu("x", x, BF16, contiguous=False)
+    _gpu("in_proj", in_proj, BF16)
+    _gpu("taps", taps, F32)
+    _gpu("state", state, F32)
+    _gpu("seg_pos0", seg_pos0, I32)
+    _gpu("seg_slot", seg_slot, I32)
+    M, K = x.shape
+    D, L = taps.shape
+    _need(in_proj.shape == (3 * D, K), f"in_proj {tuple(in_proj.shape)} for D={D}, K={K}")
+    _need(M <= 64 and D % 16 == 0, "linear_shortconv_step: at most 64 rows, width a multiple of 16")
+    _need(seg_pos0.shape == (M,) and seg_slot.shape == (M,), "one segment a row")
+    _need(L >= 2 and state.dim() == 3 and state.shape[1:] == (D, L - 1),
+          f"state {tuple(state.shape)} for D={D}, L={L}")
+    lda = x.stride(0) if M > 1 else K
+    _need((x.stride(1) == 1 or K == 1) and K % 8 == 0 and lda % 8 == 0
+          and x.data_ptr() % 16 == 0 and in_proj.data_ptr() % 16 == 0,
+          "linear_shortconv_step: K and the row stride must be multiples of 8, tensors aligned")
+    for n, t, shp in (("in_bias", in_bias, (3 * D,)), ("conv_bias", conv_bias, (D,))):
+        if t is not None:
+            _gpu(n, t, F32)
+            _need(t.shape == shp, f"{n} must be {shp}")
+    out = torch.empty((M, D), dtype=BF16, device=x.device)
+    check(library("gemm").kappai_gemm_bf16_shortconv_step(
+        _ptr(x), _ptr(in_proj), _ptr(in_bias), _ptr(out), _c_int(M), _c_int(D), _c_int(K),
+        _c_int(lda), _ptr(taps), _ptr(conv_bias), _ptr(state), _ptr(seg_pos0), _ptr(seg_slot),
+        _c_int(L), _stream()), "gemm_bf16_shortconv_step")
+    return out
+
+
 # ---------------------------------------------------------------------------------------
 def shortconv(proj: torch.Tensor, taps: torch.Tensor, bias: Optional[torch.Tensor],
               state: torch.Tensor, row_seg: torch.Tensor, seg_start: torch.Tensor,

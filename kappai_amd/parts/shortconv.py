@@ -19,6 +19,11 @@ from .base import Mixer, register_part
 from .linear import Linear
 
 
+# The fused decode kernel gives one block 16 channels; below this width it has too few blocks to
+# fill the chip and the separate product (which may split K) plus the small step kernel win.
+FUSED_STEP_MIN_WIDTH = 4096
+
+
 class GatedShortConv(Mixer):
     def __init__(self, prefix: str, width: int, kernel_size: int, dtype: torch.dtype,
                  bias: bool = False, names=None):
@@ -57,6 +62,14 @@ class GatedShortConv(Mixer):
     def forward(self, x, batch, cache, shared_cache: bool = False):
         if shared_cache:
             raise ValueError("a short convolution's state cannot be read by another layer")
+        w = self.in_proj.weight
+        if (batch.max_segment_rows == 1 and x.shape[0] <= 64 and x.dtype == torch.bfloat16
+                and w.dtype == torch.bfloat16 and self.width % 16 == 0
+                and self.width >= FUSED_STEP_MIN_WIDTH):
+            # decode: projection, convolution and state shift in one kernel
+            y = ops.linear_shortconv_step(x, w, self.in_proj.bias, self.taps, self.conv_bias,
+                                          cache.state, batch.seg_pos0, batch.seg_slot)
+            return self.out_proj.forward(y, partial_sums=True)
         proj = self.in_proj.forward(x)
         y = ops.shortconv(proj, self.taps, self.conv_bias, cache.state, batch.row_seg,
                           batch.seg_start, batch.seg_pos0, batch.seg_slot)

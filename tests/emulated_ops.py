@@ -93,6 +93,14 @@ def shortconv(proj, taps, bias, state, row_seg, seg_start, seg_pos0, seg_slot):
     return out.to(proj.dtype)
 
 
+def linear_shortconv_step(x, in_proj, in_bias, taps, conv_bias, state, seg_pos0, seg_slot):
+    M = x.shape[0]
+    proj = linear(x, in_proj, in_bias)
+    row_seg = torch.arange(M, dtype=torch.int32)
+    seg_start = torch.arange(M + 1, dtype=torch.int32)
+    return shortconv(proj, taps, conv_bias, state, row_seg, seg_start, seg_pos0, seg_slot)
+
+
 def qk_norm_rope_store(qkv, n_heads, n_kv_heads, head_dim, q_norm_w, k_norm_w, eps, cos, sin,
                        rot_dim, rot_mode, k_pool, v_pool, row_pos, row_seg, block_tables,
                        page_size, store_kv=True):
@@ -185,7 +193,7 @@ def repeat_penalty(logits, row_start, tokens, penalty):
 
 
 ALL = ["embed_rows", "add_rmsnorm", "add_residual", "swiglu", "cast", "linear", "linear_swiglu",
-       "interleave_gate_up", "shortconv",
+       "interleave_gate_up", "shortconv", "linear_shortconv_step",
        "qk_norm_rope_store", "paged_attention", "sample_rows", "repeat_penalty"]
 
 

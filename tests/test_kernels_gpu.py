@@ -223,6 +223,39 @@ def test_shortconv(ops, dtype, D, L):
             assert torch.equal(st_dev[untouched].cpu(), state0[untouched])
 
 
+@pytest.mark.parametrize("M,D,K,L,bias", [(1, 64, 64, 3, False), (8, 2048, 2048, 3, False),
+                                          (5, 96, 96, 4, True), (33, 48, 120, 2, True),
+                                          (64, 320, 72, 5, False)])
+def test_linear_shortconv_step(ops, M, D, K, L, bias):
+    """The fused decode step of a conv layer against the unfused kernels and the CPU stand-in,
+    over two steps so that the state written by the first is read by the second."""
+    slots = M + 3
+    x = [rand((M, K), BF16, 50 + i) for i in range(2)]
+    w = rand((3 * D, K), BF16, 52, 0.2)
+    b_in = rand((3 * D,), F32, 53, 0.2) if bias else None
+    b_cv = rand((D,), F32, 54, 0.2) if bias else None
+    taps = rand((D, L), F32, 55, 0.5)
+    state0 = rand((slots, D, L - 1), F32, 56)
+    slot = torch.randperm(slots, generator=torch.Generator().manual_seed(3))[:M].to(torch.int32)
+    st_f, st_u, st_r = state0.to(DEV).clone(), state0.to(DEV).clone(), state0.clone()
+    dev = lambda t: None if t is None else t.to(DEV)
+    for step in range(2):
+        pos0 = (torch.arange(M, dtype=torch.int32) % 3 if step == 0
+                else torch.arange(M, dtype=torch.int32) % 3 + 1)      # some rows start fresh
+        fused = ops.linear_shortconv_step(x[step].to(DEV), w.to(DEV), dev(b_in), taps.to(DEV),
+                                          dev(b_cv), st_f, pos0.to(DEV), slot.to(DEV))
+        proj = ops.linear(x[step].to(DEV), w.to(DEV), dev(b_in))
+        seg = torch.arange(M, dtype=torch.int32)
+        unfused = ops.shortconv(proj, taps.to(DEV), dev(b_cv), st_u, seg.to(DEV),
+                                torch.arange(M + 1, dtype=torch.int32).to(DEV), pos0.to(DEV),
+                                slot.to(DEV))
+        want = ref.linear_shortconv_step(x[step], w, b_in, taps, b_cv, st_r, pos0, slot)
+        close(fused.float(), unfused.float(), BF16_ULP, f"fused against unfused, step {step}")
+        close(fused.float(), want.float(), BF16_ULP * 2, f"fused against the stand-in, step {step}")
+        close(st_f, st_u, 2 * BF16_ULP, f"state, step {step}")
+        close(st_f, st_r, 2e-2, f"state against the stand-in, step {step}")
+
+
 # ---------------------------------------------------------------------------------------
 def paged_case(seed, dtype, H, G, d, ps, lens_before, lens_new, n_pages=None, shuffle=True):
     """Requests that already hold ``lens_before`` tokens get ``lens_new`` more.  Returns
