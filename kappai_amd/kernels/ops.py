@@ -457,6 +457,30 @@ def sample_rows(logits: torch.Tensor, temperature: torch.Tensor,
     return out
 
 
+FILTER_MAX_KEEP = 1024     # candidates the filtered-sampling kernel can hold
+
+
+def sample_filtered(logits: torch.Tensor, rows: torch.Tensor, keep: torch.Tensor,
+                    temperature: torch.Tensor, top_p: torch.Tensor, min_p: torch.Tensor,
+                    uniform: torch.Tensor, out: torch.Tensor) -> None:
+    """For every entry i: draw a token for row ``rows[i]`` of ``logits`` from its ``keep[i]``
+    (at most 1024) largest logits after temperature, top-p and min-p, at ``uniform[i]``, and
+    write it to ``out[rows[i]]`` (int32)."""
+    _gpu("logits", logits, F32)
+    _gpu("rows", rows, I32)
+    _gpu("keep", keep, I32)
+    _gpu("out", out, I32)
+    n = rows.shape[0]
+    for name, t in (("temperature", temperature), ("top_p", top_p), ("min_p", min_p),
+                    ("uniform", uniform)):
+        _gpu(name, t, F32)
+        _need(t.shape == (n,), f"{name}: one value per entry")
+    _need(keep.shape == (n,) and out.shape == (logits.shape[0],), "sample_filtered: table sizes")
+    check(library("sampling").kappai_sample_filtered(
+        _ptr(logits), _ptr(rows), _ptr(keep), _ptr(temperature), _ptr(top_p), _ptr(min_p),
+        _ptr(uniform), _ptr(out), _c_int(n), _c_int(logits.shape[1]), _stream()), "sample_filtered")
+
+
 def repeat_penalty(logits: torch.Tensor, row_start: torch.Tensor, tokens: torch.Tensor,
                    penalty: torch.Tensor) -> None:
     """In place: for row r and each token in ``tokens[row_start[r]:row_start[r+1]]`` divide a

@@ -1,11 +1,11 @@
 """Choosing the next token of every row of a step's logits.
 
 kappai samples on the host for hybrid models (src/context.c:1318-1319).  Here greedy
-choice, the whole-vocabulary temperature draw and the repeat penalty run in HIP kernels
-on the logits where they lie; the draw's uniform number comes from the request's own
-random stream on the host, so that a request's tokens do not depend on what else is in
-the batch.  Rows that narrow their candidates (top-k, top-p, min-p) are copied to the
-host and drawn there in kappai's order of operations (src/sampler.c:218-332).
+choice, the whole-vocabulary temperature draw, the repeat penalty and the draw from
+narrowed candidates (top-k, top-p, min-p; kappai's order of operations,
+src/sampler.c:218-332) run in HIP kernels on the logits where they lie; the draw's uniform
+number comes from the request's own random stream on the host, so that a request's tokens
+do not depend on what else is in the batch.  Only a top-k above 1024 is drawn on the host.
 """
 from __future__ import annotations
 
@@ -104,21 +104,33 @@ class Sampler:
                 logits, torch.tensor(starts, dtype=torch.int32, device=dev),
                 torch.tensor(toks or [0], dtype=torch.int32, device=dev),
                 torch.tensor(pens, dtype=torch.float32, device=dev))
-        temps, unis, host_rows = [], [], []
+        temps, unis, host_rows, filt = [], [], [], []
         for i, s in enumerate(samplers):
             p = s.params
             if p.is_greedy():
                 temps.append(0.0)
                 unis.append(0.0)
             elif p.is_filtered(vocab):
-                temps.append(0.0)            # the kernel's choice for this row is not used
+                temps.append(0.0)            # the kernel's choice for this row is replaced
                 unis.append(0.0)
-                host_rows.append(i)
+                keep = p.top_k if 0 < p.top_k < vocab else min(vocab, FILTER_CAP)
+                if keep <= ops.FILTER_MAX_KEEP:
+                    filt.append((i, keep, float(p.temperature), float(p.top_p), float(p.min_p),
+                                 s.rng.uniform()))
+                else:
+                    host_rows.append(i)
             else:
                 temps.append(float(p.temperature))
                 unis.append(s.rng.uniform())
-        out = ops.sample_rows(logits, torch.tensor(temps, dtype=torch.float32, device=dev),
-                              torch.tensor(unis, dtype=torch.float32, device=dev)).tolist()
+        out_dev = ops.sample_rows(logits, torch.tensor(temps, dtype=torch.float32, device=dev),
+                                  torch.tensor(unis, dtype=torch.float32, device=dev))
+        if filt:
+            cols = list(zip(*filt))
+            f32 = lambda v: torch.tensor(v, dtype=torch.float32, device=dev)
+            ops.sample_filtered(logits, torch.tensor(cols[0], dtype=torch.int32, device=dev),
+                                torch.tensor(cols[1], dtype=torch.int32, device=dev), f32(cols[2]),
+                                f32(cols[3]), f32(cols[4]), f32(cols[5]), out_dev)
+        out = out_dev.tolist()
         if host_rows:
             rows = logits[torch.tensor(host_rows, device=dev)].cpu().numpy()
             for row, i in zip(rows, host_rows):

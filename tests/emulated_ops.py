@@ -181,6 +181,19 @@ def sample_rows(logits, temperature, uniform):
     return out
 
 
+FILTER_MAX_KEEP = 1024
+
+
+def sample_filtered(logits, rows, keep, temperature, top_p, min_p, uniform, out):
+    from plain import sampler as plain_sampler
+    for i in range(rows.shape[0]):
+        r = int(rows[i])
+        k = int(keep[i])
+        out[r] = plain_sampler.sample_filtered(
+            logits[r].numpy(), float(temperature[i]), k if k < logits.shape[1] else 0,
+            float(top_p[i]), float(min_p[i]), float(uniform[i]), cap=k)
+
+
 def repeat_penalty(logits, row_start, tokens, penalty):
     for r in range(logits.shape[0]):
         pen = float(penalty[r])
@@ -194,7 +207,8 @@ def repeat_penalty(logits, row_start, tokens, penalty):
 
 ALL = ["embed_rows", "add_rmsnorm", "add_residual", "swiglu", "cast", "linear", "linear_swiglu",
        "interleave_gate_up", "shortconv", "linear_shortconv_step",
-       "qk_norm_rope_store", "paged_attention", "sample_rows", "repeat_penalty"]
+       "qk_norm_rope_store", "paged_attention", "sample_rows", "sample_filtered",
+       "repeat_penalty"]
 
 
 def install(monkeypatch):

@@ -409,6 +409,37 @@ def test_sample_rows(ops):
     assert abs(freq[0] - 0.5) < 0.03 and abs(freq[1] - 0.2) < 0.03
 
 
+def test_sample_filtered(ops):
+    """The candidate-narrowing draw against the plain sampler, row by row: default options,
+    top-k only, top-p only, min-p only, ties in the logits, a vocabulary below the cap."""
+    from plain import sampler as plain_sampler
+    rng = np.random.default_rng(5)
+    for V in (65536, 1003, 300):
+        n = 12
+        logits = (rng.normal(size=(n, V)) * 3).astype(np.float32)
+        logits[1, :50] = logits[1, 0]                      # many equal values at the top-k edge
+        logits[2] = np.round(logits[2])                    # ties everywhere
+        opts = [(0.8, 40, 0.9, 0.1), (1.3, 5, 1.0, 0.0), (0.5, 0, 0.6, 0.0), (1.0, 0, 1.0, 0.3),
+                (2.0, 1000, 0.95, 0.01), (0.7, 2, 0.5, 0.5)]
+        rows, keep, temp, tp, mp, uni, want = [], [], [], [], [], [], {}
+        for r in range(n):
+            t, k, p, m = opts[r % len(opts)]
+            u = float(np.float32(rng.random()))
+            kk = k if 0 < k < V else min(V, 1024)
+            rows.append(r); keep.append(kk); temp.append(t); tp.append(p); mp.append(m); uni.append(u)
+            want[r] = plain_sampler.sample_filtered(logits[r], t, k, p, m, u)
+        out = torch.full((n,), -1, dtype=torch.int32, device=DEV)
+        f32 = lambda v: torch.tensor(v, dtype=torch.float32, device=DEV)
+        i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=DEV)
+        ops.sample_filtered(torch.from_numpy(logits).to(DEV), i32(rows), i32(keep), f32(temp),
+                            f32(tp), f32(mp), f32(uni), out)
+        got = out.cpu().tolist()
+        for r in range(n):
+            if got[r] != want[r]:
+                # equal logits may be ordered differently: the pick must then have the same value
+                assert logits[r, got[r]] == logits[r, want[r]], (V, r, got[r], want[r])
+
+
 def test_repeat_penalty(ops):
     logits = torch.tensor([[1.0, 0.9, 0.0, -1.0], [2.0, -2.0, 0.5, 0.0]])
     row_start = torch.tensor([0, 3, 4], dtype=torch.int32)
