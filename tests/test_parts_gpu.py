@@ -64,7 +64,39 @@ def test_attention_part(dtype, tol):
     cfg = {"num_attention_heads": H, "num_key_value_heads": G, "head_dim": d, "hidden_size": W,
            "norm_eps": 1e-4, "rope_theta": 12345.0}
     want = P.gqa_attention_mixer(x.double().numpy(), lw, cfg, np.arange(T))
-    assert rel_err(torch.cat([y1, y2]), want) < tol
+    assert rel_err(torch.cat([y if y.dim() == 2 else y.sum(0) for y in (y1, y2)]), want) < tol
+
+
+@pytest.mark.parametrize("dtype,tol", [(F32, 1e-5), (BF16, 2e-2)])
+def test_attention_part_with_a_window(dtype, tol):
+    """A window of 20 keys over 150 tokens with pages of 16: a prompt portion, then tokens one
+    by one (twice, so that the second time the decode graph's kernels run), while the cache
+    manager gives the pages back that the window has passed; a pool of 5 pages suffices."""
+    from kappai_amd.cache import CacheManager
+    from kappai_amd.parts import GroupedQueryAttention, RotaryEncoding
+    W, H, G, d, T, win = 64, 4, 2, 32, 150, 20
+    part = GroupedQueryAttention("a.", W, H, G, d, dtype, position=RotaryEncoding(d, 1e4),
+                                 qk_norm_eps=1e-5, window=win)
+    w = bind_random(part, 11, dtype)
+    cm = CacheManager([part.cache_spec()], 16, 5, 1)
+    cm.allocate_storage(dtype, DEV, poison=True)
+    x = torch.randn(T, W, generator=torch.Generator().manual_seed(12)).to(dtype)
+    rc, outs, done = None, [], 0
+    for n in [37, 3] + [1] * 60 + [25] + [1] * 25:
+        rc, b = one_segment_batch(cm, n, rc=rc)
+        outs.append(part.forward(x[done:done + n].to(DEV), b, cm.view(0)))
+        cm.commit(rc, n)
+        cm.check()
+        done += n
+    assert done == T
+    assert sum(p >= 0 for p in rc.blocks[0]) <= 3 and rc.blocks[0][0] == -1
+    lw = {n: w[f"a.{n}.weight"] for n in ("q_proj", "k_proj", "v_proj", "out_proj", "q_layernorm",
+                                          "k_layernorm")}
+    cfg = {"num_attention_heads": H, "num_key_value_heads": G, "head_dim": d, "hidden_size": W,
+           "norm_eps": 1e-5, "rope_theta": 1e4}
+    want = P.gqa_attention_mixer(x.double().numpy(), lw, cfg, np.arange(T), window=win)
+    got = torch.cat([o if o.dim() == 2 else o.sum(0) for o in outs])
+    assert rel_err(got, want) < tol
 
 
 @pytest.mark.parametrize("dtype,tol", [(F32, 1e-5), (BF16, 2e-2)])
@@ -90,7 +122,7 @@ def test_short_conv_part(dtype, tol, bias):
         lw.update(in_proj_bias=w["c.in_proj.bias"], conv_bias=w["c.conv.bias"],
                   out_proj_bias=w["c.out_proj.bias"])
     want = P.short_conv_mixer(x.double().numpy(), lw, {"hidden_size": W})
-    assert rel_err(torch.cat(outs), want) < tol
+    assert rel_err(torch.cat([o if o.dim() == 2 else o.sum(0) for o in outs]), want) < tol
 
 
 @pytest.mark.parametrize("dtype,tol", [(F32, 1e-5), (BF16, 2e-2)])
@@ -283,3 +315,132 @@ def test_toy_mixer_with_its_own_state_and_a_shared_cache():
     means = torch.cumsum(x, 0) / torch.arange(1, 10)[:, None]
     want = means.double() @ mix.proj.weight.cpu().double().T
     assert float((got.cpu().double() - want).abs().max()) < 1e-5
+
+
+def test_toy_feed_forward_with_routing_and_an_absolute_position_encoding():
+    """Two more parts made in the test: a feed-forward that routes every row to one of two
+    experts, and a learned absolute position encoding added to the embedded rows; and a
+    sliding-window attention beside a full one, so that the cache manager runs two paged groups.
+    Built through the registries, run cut into portions and whole."""
+    import tempfile
+
+    from kappai_amd.config import ModelConfig, config_from_dict, register_architecture
+    from kappai_amd.engine import StepEntry, StepRunner
+    from kappai_amd.engine.replay import make_replay_cache
+    from kappai_amd.kernels import ops
+    from kappai_amd.models import Model, load_model
+    from kappai_amd.parts import (FeedForward, Linear, OutputHead, PositionEncoding,
+                                  TokenEmbedding, make_part, register_part)
+    from kappai_amd.weights import write_random_model
+    from kappai_amd.weights.spec import INIT_NORMAL, TABLE, TensorSpec
+
+    class RoutedFeedForward(FeedForward):
+        """Row t goes to expert argmax(router x_t); each expert is a SwiGLU of its own."""
+
+        def __init__(self, prefix, width, hidden, n_experts, dtype):
+            self.router = Linear([prefix + "router"], width, [n_experts])
+            self.experts = [make_part("feed_forward", "swiglu", prefix=f"{prefix}experts.{e}.",
+                                      width=width, hidden=hidden, dtype=dtype)
+                            for e in range(n_experts)]
+
+        def tensor_specs(self):
+            return self.router.tensor_specs() + [s for e in self.experts for s in e.tensor_specs()]
+
+        def bind(self, tensors):
+            self.router.bind(tensors)
+            for e in self.experts:
+                e.bind(tensors)
+
+        def forward(self, x, batch):
+            choice = self.router.forward(x, out_dtype=torch.float32).argmax(dim=1)
+            out = torch.zeros_like(x)
+            for e, expert in enumerate(self.experts):
+                rows = torch.nonzero(choice == e).flatten()
+                if rows.numel():
+                    y = expert.forward(x[rows].contiguous(), batch)
+                    out[rows] = (y if y.dim() == 2 else y.sum(0)).to(x.dtype)
+            return out
+
+        capturable = False        # the rows of an expert are counted on the host
+
+    class LearnedPositions(PositionEncoding):
+        def __init__(self, name, n_positions, width):
+            self.name, self.n, self.width = name, n_positions, width
+
+        def tensor_specs(self):
+            return [TensorSpec(self.name + ".weight", (self.n, self.width), TABLE, INIT_NORMAL)]
+
+        def bind(self, tensors):
+            self.table = tensors[self.name + ".weight"]
+
+        def on_embedding(self, x, batch):
+            x += ops.embed_rows(batch.row_pos, self.table)
+
+    register_part("feed_forward", "toy_routed", RoutedFeedForward)
+    register_part("position_encoding", "toy_learned", LearnedPositions)
+
+    @dataclass
+    class Toy2Config(ModelConfig):
+        width: int = 0
+        vocab_size: int = 0
+        max_position_embeddings: int = 256
+
+        @classmethod
+        def from_dict(cls, raw):
+            return cls(architecture="Toy2ForCausalLM", width=raw["width"],
+                       vocab_size=raw["vocab_size"])
+
+        def to_dict(self):
+            return {"architectures": ["Toy2ForCausalLM"], "width": self.width,
+                    "vocab_size": self.vocab_size}
+
+    def build(cfg, dtype):
+        def block(i, window):
+            p = f"l.{i}."
+            return make_part(
+                "block", "pre_norm",
+                mixer_norm=make_part("norm", "rmsnorm", name=p + "n1", width=cfg.width, eps=1e-5,
+                                     dtype=dtype),
+                mixer=make_part("mixer", "attention", prefix=p + "att.", width=cfg.width,
+                                num_heads=4, num_kv_heads=2, head_dim=16, dtype=dtype,
+                                position=None, qk_norm_eps=None, window=window),
+                ffn_norm=make_part("norm", "rmsnorm", name=p + "n2", width=cfg.width, eps=1e-5,
+                                   dtype=dtype),
+                feed_forward=make_part("feed_forward", "toy_routed", prefix=p + "ff.",
+                                       width=cfg.width, hidden=48, n_experts=2, dtype=dtype))
+        emb = TokenEmbedding("emb", cfg.vocab_size, cfg.width)
+        return Model(cfg, dtype, emb, [block(0, 12), block(1, None)],
+                     make_part("norm", "rmsnorm", name="final", width=cfg.width, eps=1e-5,
+                               dtype=dtype),
+                     OutputHead("head", cfg.vocab_size, cfg.width, tied_to=emb),
+                     embedding_position=make_part("position_encoding", "toy_learned", name="pos",
+                                                  n_positions=256, width=cfg.width))
+
+    register_architecture("Toy2ForCausalLM", Toy2Config, build)
+    cfg = config_from_dict({"architectures": ["Toy2ForCausalLM"], "width": 64, "vocab_size": 77})
+    for dtype, tol in (("float32", 2e-5), ("bfloat16", 6e-2)):
+        with tempfile.TemporaryDirectory() as tmp:
+            write_random_model(tmp, cfg, seed=4, std=0.25)
+            model = load_model(tmp, dtype, DEV)
+        assert len({type(s).__name__ + str(getattr(s, "window", "")) for s in model.cache_specs()}) == 2
+        toks = [int(t) for t in np.random.default_rng(1).integers(0, 77, size=70)]
+
+        def run(portions):
+            cache = make_replay_cache(model, 128)
+            assert len(cache.paged_groups) == 2
+            cache.allocate_storage(model.dtype, DEV, poison=True)
+            runner = StepRunner(model, cache, DEV)
+            rc, done, rows = cache.open("t"), 0, []
+            for n in portions:
+                rows.append(runner.step([StepEntry(rc, toks[done:done + n], list(range(n)))]).cpu())
+                done += n
+            assert rc.blocks[0][0] == -1 and rc.blocks[1][0] >= 0     # only the window let go
+            return torch.cat(rows)
+
+        whole = run([70])
+        cut = run([9, 1, 2, 30, 1, 1, 1, 25])
+        assert torch.isfinite(whole).all() and float(whole.abs().max()) > 0.1
+        # routing is an argmax: in bfloat16 a near tie may send a row to the other expert
+        diff = (cut - whole).abs().amax(dim=1) / float(whole.abs().max())
+        assert float(diff.median()) < tol and float((diff > tol).float().mean()) < (
+            0.0 if dtype == "float32" else 0.1) + 1e-9
