@@ -164,8 +164,7 @@ class Engine:
             outputs.append(StepOutput(req.request_id, None, True, req.finish_reason))
         if not entries:
             return outputs
-        torch.cuda.synchronize(self.device)
-        t0 = time.perf_counter()
+        t0 = time.perf_counter()          # the last step ended with a synchronisation
         step_entries = []
         for e in entries:
             toks = e.request.tokens[e.request.computed:e.request.computed + e.n_tokens]
@@ -175,8 +174,11 @@ class Engine:
         self.scheduler.advance(entries)
         sampling = [e.request for e in entries if e.samples]
         self.last_logits = logits
-        tokens = self.sampler.sample(logits, [r.sampler for r in sampling]) if sampling else []
-        torch.cuda.synchronize(self.device)
+        if sampling:                      # reading the tokens back waits for the step
+            tokens = self.sampler.sample(logits, [r.sampler for r in sampling])
+        else:
+            tokens = []
+            torch.cuda.synchronize(self.device)
         dt = time.perf_counter() - t0
         n_prefill = sum(e.n_tokens for e in entries if e.n_tokens > 1 or not e.request.output)
         n_decode = sum(e.n_tokens for e in entries) - n_prefill

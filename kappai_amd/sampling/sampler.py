@@ -85,6 +85,9 @@ class Sampler:
     """Samples one token for each row of ``logits`` [n, vocab] (float32, on the GPU; changed
     in place where a repeat penalty applies)."""
 
+    def __init__(self):
+        self._zeros = {}      # (rows, device) -> zero temperature / uniform tensors (all greedy)
+
     def sample(self, logits: torch.Tensor, samplers: Sequence[RequestSampler]) -> List[int]:
         n, vocab = logits.shape
         if n != len(samplers):
@@ -122,14 +125,31 @@ class Sampler:
             else:
                 temps.append(float(p.temperature))
                 unis.append(s.rng.uniform())
-        out_dev = ops.sample_rows(logits, torch.tensor(temps, dtype=torch.float32, device=dev),
-                                  torch.tensor(unis, dtype=torch.float32, device=dev))
-        if filt:
-            cols = list(zip(*filt))
-            f32 = lambda v: torch.tensor(v, dtype=torch.float32, device=dev)
-            ops.sample_filtered(logits, torch.tensor(cols[0], dtype=torch.int32, device=dev),
-                                torch.tensor(cols[1], dtype=torch.int32, device=dev), f32(cols[2]),
-                                f32(cols[3]), f32(cols[4]), f32(cols[5]), out_dev)
+        # every per-row number goes to the GPU in ONE copy: [temperature | uniform] for all
+        # rows, then [row | keep | temperature | top_p | min_p | uniform] for the narrowed ones
+        m = len(filt)
+        if not any(temps) and not m and (n, str(dev)) in self._zeros:
+            out_dev = ops.sample_rows(logits, *self._zeros[(n, str(dev))])
+        else:
+            packed = np.zeros(2 * n + 6 * m, dtype=np.float32)
+            packed[:n] = temps
+            packed[n:2 * n] = unis
+            if m:
+                cols = list(zip(*filt))
+                ints = packed[2 * n:2 * n + 2 * m].view(np.int32)
+                ints[:m] = cols[0]
+                ints[m:] = cols[1]
+                for j in range(4):
+                    packed[2 * n + (2 + j) * m:2 * n + (3 + j) * m] = cols[2 + j]
+            d = torch.from_numpy(packed).to(dev)
+            if not any(temps) and not m:
+                self._zeros[(n, str(dev))] = (d[:n], d[n:2 * n])
+            out_dev = ops.sample_rows(logits, d[:n], d[n:2 * n])
+            if m:
+                di = d[2 * n:2 * n + 2 * m].view(torch.int32)
+                f = d[2 * n + 2 * m:]
+                ops.sample_filtered(logits, di[:m], di[m:], f[:m], f[m:2 * m], f[2 * m:3 * m],
+                                    f[3 * m:4 * m], out_dev)
         out = out_dev.tolist()
         if host_rows:
             rows = logits[torch.tensor(host_rows, device=dev)].cpu().numpy()
