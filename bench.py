@@ -73,7 +73,7 @@ class DecodeBench:
     """``batch`` requests whose caches hold ``start`` tokens of random keys and values, then
     decoded greedily one token a step."""
 
-    def __init__(self, model, batch, start, total, page_size, device, seed=1):
+    def __init__(self, model, batch, start, total, page_size, device, seed=1, graphs=True):
         import torch
 
         from kappai_amd.cache import CacheManager
@@ -88,7 +88,7 @@ class DecodeBench:
                 for cid in pools:
                     pools[cid].copy_(torch.randn(pools[cid].shape, generator=gen, device=device,
                                                  dtype=torch.float32) * 0.5)
-        self.runner = StepRunner(model, self.cache, device)
+        self.runner = StepRunner(model, self.cache, device, decode_graphs=graphs)
         self.requests = [self.cache.open(i) for i in range(batch)]
         for rc in self.requests:
             self.cache.extend(rc, start)
@@ -148,6 +148,8 @@ def main() -> int:
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--page-size", type=int, default=16)
     ap.add_argument("--skip-points", action="store_true", help="only the headline batch")
+    ap.add_argument("--no-graphs", action="store_true",
+                    help="launch decode steps kernel by kernel (for counter collection)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this engine runs on one GPU; --gpus must be 1 (nothing was measured)")
@@ -174,7 +176,8 @@ def main() -> int:
         return 2
 
     def decode(batch):
-        b = DecodeBench(model, batch, start, args.context, args.page_size, device)
+        b = DecodeBench(model, batch, start, args.context, args.page_size, device,
+                        graphs=not args.no_graphs)
         dt = b.run(W, K)
         kv_bytes = b.cache.bytes_per_token(elem)
         b.close()

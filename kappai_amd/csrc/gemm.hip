@@ -109,6 +109,25 @@ __device__ __forceinline__ float silu_f(float g) { return g / (1.0f + expf(-g));
 // EPI 1 (SwiGLU): W holds gate and up rows interleaved in groups of 16 (16 gate rows, the 16 up
 // rows of the same columns, ...); the kernel writes silu(gate) * up, N/2 columns wide
 // (kappai: src/backend/cpu/quants.h:369-371, src/recipe/builders.c:344-370).
+// Block number -> (row tile, column tile).  Consecutive block numbers go to the 8 XCDs in
+// turn, each with an L2 of its own.  An XCD is given a band of column tiles (an eighth of W, so
+// that W is fetched from memory once) and walks it in groups of up to 8 x 8 tiles, row tiles
+// fastest: the blocks that run on it at one time then share both their rows of A and their
+// rows of W in its L2.
+__device__ __forceinline__ int2 xcd_tile(int b, int tiles_m, int tiles_n) {
+  constexpr int XCDS = 8, GROUP = 8;
+  if (tiles_n % XCDS != 0) return make_int2(b / tiles_n, b % tiles_n);
+  const int band = tiles_n / XCDS;             // column tiles of one XCD
+  const int xcd = b % XCDS;
+  int j = b / XCDS;                            // position in the XCD's own order
+  const int per_group = GROUP * band;
+  const int groups = (tiles_m + GROUP - 1) / GROUP;
+  const int g = min(j / per_group, groups - 1);
+  j -= g * per_group;
+  const int gm = min(GROUP, tiles_m - g * GROUP);
+  return make_int2(g * GROUP + j % gm, xcd * band + j / gm);
+}
+
 template <typename TO, int EPI, int WAVES_M, int WAVES_N, int WM, int WN, int BK, int NBUF,
           int OCC>
 __global__ __launch_bounds__(WAVES_M * WAVES_N * WAVE)
@@ -129,10 +148,8 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * WAVE)
   const int lane = tid % WAVE, wave = tid / WAVE;
   const int wm = wave / WAVES_N, wn = wave % WAVES_N;
   // block -> tile, XCD-aware
-  int b = blockIdx.x;
-  const int nb = gridDim.x;
-  if (nb % 8 == 0) b = (b % 8) * (nb / 8) + b / 8;
-  const int m0 = (b / tiles_n) * BM, n0 = (b % tiles_n) * BN;
+  const int2 tile = xcd_tile(blockIdx.x, gridDim.x / tiles_n, tiles_n);
+  const int m0 = tile.x * BM, n0 = tile.y * BN;
   // gridDim.y > 1 splits K over blocks: block y writes its partial sums to C + y * M * ldc
   const int kblk = ((K + BK * (int)gridDim.y - 1) / (BK * (int)gridDim.y)) * BK;
   const int kbeg = blockIdx.y * kblk, kend = min(K, kbeg + kblk);
@@ -279,18 +296,266 @@ static void launch_tile_cfg(const bf16_t* A, const bf16_t* W, const float* bias,
                      stream, A, W, bias, C, M, n_rows_w, K, lda, ldc, tn);
 }
 
+// ---------------------------------------------------------------------------------------
+// 256 x 256 blocks for large products (prefill)
+// ---------------------------------------------------------------------------------------
+// Four waves, one on each SIMD, each owning 128 x 128 of the result as 4 x 4 accumulator tiles
+// (256 accumulator registers): per 16 of K a wave reads 8 fragments from LDS for 16 matrix
+// instructions.  Tiles of 64 of K (128-byte rows, whole cache lines) go from global memory
+// straight into LDS (global_load_lds), two buffers; the 16-byte chunks of a row are permuted
+// by (chunk ^ row % 8) on the way in, so that fragment reads meet no bank conflict without
+// padding.  The order of LDS reads, loads and matrix instructions is written out slot by slot
+// and fenced, one wave has to hide every latency by itself: while the products of one 16 of K
+// run, the fragments of the next are read; the loads of tile k+2 are issued as soon as the
+// barrier of tile k has shown that everybody is done with its buffer.
+//
+// The matrix instruction takes the W fragment as its first operand: a lane then holds one row
+// of C and 4 consecutive columns per register group, which the epilogue packs, transposes
+// through LDS and stores as whole 16-byte chunks of rows (the SwiGLU pairs gate and up in one
+// lane: registers v and v + 8).
+//
+// Host side guarantees: K / gridDim.y is a multiple of 128, rows of W a multiple of 8 (32 with
+// SwiGLU), C and its row stride 16-byte aligned, M * lda and N * K below 2^31 elements.
+#define KAPPAI_GPTR(p) ((const __attribute__((address_space(1))) void*)(p))
+#define KAPPAI_LPTR(p) ((__attribute__((address_space(3))) void*)(p))
+#define SCHED_FENCE() __builtin_amdgcn_sched_barrier(0)
+
+template <int N> struct IntC { static constexpr int value = N; };
+
+template <typename TO, int EPI>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
+void gemm_bf16_block256_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W,
+                               const float* __restrict__ bias, TO* __restrict__ C, int M, int N,
+                               int K, int lda, int ldc, int tiles_n) {
+  constexpr int BM = 256, BN = 256, BK = 64;
+  constexpr int A_TILE = BM * BK, BUF = (BM + BN) * BK;        // in bf16
+  extern __shared__ __attribute__((aligned(1024))) bf16_t lds[];
+  const int tid = threadIdx.x, lane = tid % WAVE;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / WAVE);
+  const int wm = wave / 2, wn = wave % 2;
+  const int2 tile = xcd_tile(blockIdx.x, gridDim.x / tiles_n, tiles_n);
+  const int m0 = tile.x * BM, n0 = tile.y * BN;
+  const int kblk = K / (int)gridDim.y;
+  const int nk = kblk / BK;
+  C += (size_t)blockIdx.y * M * ldc;
+
+  f32x16_t acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+
+  // One load instruction = 8 rows x 128 bytes: lane -> (row lane/8, LDS chunk lane%8), which
+  // receives the row's chunk (lane%8) ^ (row%8).  Waves 0, 1 bring the A tile, waves 2, 3 the W
+  // tile, 16 instructions each; rows past the end of the matrix repeat its last row (their
+  // products are never stored).
+  const bool brings_a = wave < 2;
+  const char* gk = reinterpret_cast<const char*>(brings_a ? A : W) +
+                   (size_t)blockIdx.y * kblk * sizeof(bf16_t);
+  const int ld = brings_a ? lda : K;
+  const int last_row = (brings_a ? M : N) - 1;
+  const int row0 = brings_a ? m0 + wave * 128 : n0 + (wave - 2) * 128;
+  const int lrow = lane / 8, lchunk = (lane % 8) ^ lrow;
+  uint32_t roff[16];
+#pragma unroll
+  for (int i = 0; i < 16; ++i)
+    roff[i] = (uint32_t)(min(row0 + i * 8 + lrow, last_row) * ld + lchunk * 8) *
+              (uint32_t)sizeof(bf16_t);
+  // the address of a load is a wave-uniform 64-bit base (the tile's first column) plus the
+  // lane's 32-bit row offset; pinning the base into scalar registers keeps the compiler from
+  // folding the two into sixteen 64-bit per-lane pointers
+  auto tile_base = [&](int kt) {
+    const uint64_t p = reinterpret_cast<uint64_t>(gk) + (uint64_t)kt * (BK * sizeof(bf16_t));
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)p);
+    const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(p >> 32));
+    return reinterpret_cast<const char*>(((uint64_t)hi << 32) | lo);
+  };
+  auto load_one = [&](int buf, const char* base, int i) {
+    __builtin_amdgcn_global_load_lds(KAPPAI_GPTR(base + roff[i]),
+                                     KAPPAI_LPTR(lds + buf * BUF + (wave * 16 + i) * 8 * BK), 16,
+                                     0, 0);
+  };
+  // fragments of the 16 of K number s: chunks 2s and 2s+1; lane -> (row lane%32, chunk 2s+lane/32)
+  const int r_in = lane % 32, hh = lane / 32;
+  int aoff[4], woff[4];
+#pragma unroll
+  for (int s = 0; s < 4; ++s) {
+    aoff[s] = (wm * 128 + r_in) * BK + (((s * 2 + hh) ^ (r_in & 7)) * 8);
+    woff[s] = A_TILE + (wn * 128 + r_in) * BK + (((s * 2 + hh) ^ (r_in & 7)) * 8);
+  }
+  bf16x8_t fa[2][4], fw[2][4];
+  // in the order the products ask for them: w0 a0 w1 w2 w3 a1 a2 a3
+  auto read_one = [&](int fb, int buf, int s, int idx) {
+    const bool is_w = idx == 0 || (idx >= 2 && idx <= 4);
+    const int n = idx <= 1 ? 0 : idx <= 4 ? idx - 1 : idx - 4;
+    if (is_w)
+      fw[fb][n] = as_bf16x8(
+          *reinterpret_cast<const u32x4_t*>(lds + buf * BUF + woff[s] + n * 32 * BK));
+    else
+      fa[fb][n] = as_bf16x8(
+          *reinterpret_cast<const u32x4_t*>(lds + buf * BUF + aoff[s] + n * 32 * BK));
+  };
+  auto product = [&](int fb, int t) {
+    const int i = t / 4, j = t % 4;
+    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fw[fb][j], fa[fb][i], acc[i][j], 0, 0, 0);
+  };
+  // One tile of K out of buffer U.  next: there is a tile kt+1 (its second half is loaded
+  // here, its first fragments are read at the end); next2: there is a tile kt+2 (its first
+  // half is loaded into this tile's buffer once the barrier has passed).  Both are uniform.
+  auto tile_step = [&](auto u_c, int kt, bool next, bool next2) {
+    constexpr int U = decltype(u_c)::value;
+    const char* base1 = tile_base(kt + 1);
+    const char* base2 = tile_base(kt + 2);
+#pragma unroll
+    for (int s = 0; s < 3; ++s) {
+#pragma unroll
+      for (int t = 0; t < 16; ++t) {
+        if (t < 8) read_one((s + 1) & 1, U, s + 1, t);
+        if (s == 0 && t >= 8 && next) load_one(U ^ 1, base1, t);
+        product(s & 1, t);
+        SCHED_FENCE();
+      }
+    }
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      product(1, t);
+      SCHED_FENCE();
+    }
+    if (next) {
+      __builtin_amdgcn_s_waitcnt(0x0F70);       // vmcnt(0): tile kt+1 has landed
+      __builtin_amdgcn_s_barrier();
+    }
+    SCHED_FENCE();
+#pragma unroll
+    for (int t = 4; t < 16; ++t) {
+      if (t < 12 && next) read_one(0, U ^ 1, 0, t - 4);
+      if (t < 12 && next2) load_one(U, base2, t - 4);
+      product(1, t);
+      SCHED_FENCE();
+    }
+  };
+
+#pragma unroll
+  for (int i = 0; i < 16; ++i) load_one(0, tile_base(0), i);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) load_one(1, tile_base(1), i);
+  __builtin_amdgcn_s_waitcnt(0x0F70 | 8);       // vmcnt(8): tile 0 has landed
+  __builtin_amdgcn_s_barrier();
+  SCHED_FENCE();
+#pragma unroll
+  for (int t = 0; t < 8; ++t) read_one(0, 0, 0, t);
+
+  // nk is even: the loop body is straight-line code for the accumulators (a conditional
+  // second tile would merge two versions of all 256 of them)
+  for (int kt = 0; kt < nk; kt += 2) {
+    const bool more = kt + 2 < nk;
+    tile_step(IntC<0>{}, kt, true, more);
+    tile_step(IntC<1>{}, kt + 1, more, more);
+  }
+
+  // Epilogue: a wave turns 32 rows of its tile at a time through its own piece of LDS.
+  // acc[i][j][4g + e] is C[row (wm*4+i)*32 + lane%32][column (wn*4+j)*32 + 8g + 4*(lane/32) + e].
+  __syncthreads();                               // everybody is done with the last tile
+  constexpr int OUT_COLS = EPI == 1 ? 64 : 128;  // columns a wave writes
+  constexpr int ROW_BYTES = OUT_COLS * (int)sizeof(TO) + 16;
+  char* mine = reinterpret_cast<char*>(lds) + wave * 32 * ROW_BYTES;
+  const int out_n = EPI == 1 ? N / 2 : N;
+  const int col0 = EPI == 1 ? (n0 + wn * 128) / 2 : n0 + wn * 128;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    char* wrow = mine + r_in * ROW_BYTES;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+#pragma unroll
+      for (int g = 0; g < (EPI == 1 ? 2 : 4); ++g) {
+        float v4[4];
+        int c;                                   // first of the 4 columns, within the wave's
+        if (EPI == 1) {
+          c = j * 16 + 8 * g + 4 * hh;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) v4[e] = silu_f(acc[i][j][4 * g + e]) * acc[i][j][4 * g + 8 + e];
+        } else {
+          c = j * 32 + 8 * g + 4 * hh;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) v4[e] = acc[i][j][4 * g + e];
+          if (bias && blockIdx.y == 0) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              if (col0 + c + e < out_n) v4[e] += bias[col0 + c + e];
+          }
+        }
+        if (sizeof(TO) == 2) {
+          uint2 pk;
+          pk.x = pack_bf16x2(v4[0], v4[1]);
+          pk.y = pack_bf16x2(v4[2], v4[3]);
+          *reinterpret_cast<uint2*>(wrow + c * 2) = pk;
+        } else {
+          *reinterpret_cast<float4*>(wrow + c * 4) = make_float4(v4[0], v4[1], v4[2], v4[3]);
+        }
+      }
+    }
+    // rows back out, 16 bytes a lane
+    constexpr int CHUNKS = OUT_COLS * (int)sizeof(TO) / 16;   // per row
+    constexpr int ROWS_PER = WAVE / CHUNKS;
+    constexpr int PER = 16 / (int)sizeof(TO);                 // columns a chunk
+#pragma unroll
+    for (int it = 0; it < 32 / ROWS_PER; ++it) {
+      const int rr = it * ROWS_PER + lane / CHUNKS, ch = lane % CHUNKS;
+      const u32x4_t v = *reinterpret_cast<const u32x4_t*>(mine + rr * ROW_BYTES + ch * 16);
+      const int gm = m0 + (wm * 4 + i) * 32 + rr, gn = col0 + ch * PER;
+      if (gm < M && gn < out_n) *reinterpret_cast<u32x4_t*>(C + (size_t)gm * ldc + gn) = v;
+    }
+  }
+}
+
+template <typename TO, int EPI>
+static bool block256_fits(const bf16_t* A, const bf16_t* W, TO* C, int M, int n_rows_w, int K,
+                          int lda, int ldc, int ksplit) {
+  const long long limit = 1ll << 31;
+  return K % (128 * ksplit) == 0 && n_rows_w % (EPI == 1 ? 32 : 8) == 0 &&
+         ((uintptr_t)C % 16) == 0 && ((size_t)ldc * sizeof(TO)) % 16 == 0 &&
+         (long long)M * lda < limit && (long long)n_rows_w * K < limit;
+}
+
+template <typename TO, int EPI>
+static void launch_block256(const bf16_t* A, const bf16_t* W, const float* bias, TO* C, int M,
+                            int n_rows_w, int K, int lda, int ldc, int ksplit,
+                            hipStream_t stream) {
+  constexpr size_t lds_bytes = 2 * (256 + 256) * 64 * sizeof(bf16_t);
+  auto kern = gemm_bf16_block256_kernel<TO, EPI>;
+  static bool attr_set = false;
+  if (!attr_set) {
+    (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
+                              (int)lds_bytes);
+    attr_set = true;
+  }
+  const int tn = (n_rows_w + 255) / 256, tm = (M + 255) / 256;
+  hipLaunchKernelGGL(kern, dim3(tm * tn, ksplit), dim3(256), lds_bytes, stream, A, W, bias, C, M,
+                     n_rows_w, K, lda, ldc, tn);
+}
+
 // shape: 0 = chosen by size, 1 = 128x128 blocks of two waves, 2 = 256x128 blocks (tiles of 32
 // of K, two LDS buffers), 3 = 256x128 blocks (tiles of 64 of K, one LDS buffer), 4 = 256x256
-// blocks (tiles of 64 of K)
+// blocks of the same kernel (tiles of 64 of K), 5 = the 256x256 kernel with one wave a SIMD
+// (when the sizes fit it, else 3)
 template <typename TO, int EPI>
 static void launch_tile(const bf16_t* A, const bf16_t* W, const float* bias, TO* C, int M,
                         int n_rows_w, int K, int lda, int ldc, int ksplit, int shape,
                         hipStream_t stream) {
+  const bool fits = EPI != 2 && block256_fits<TO, EPI>(A, W, C, M, n_rows_w, K, lda, ldc, ksplit);
   if (shape == 0) {
     const int big = ((M + 255) / 256) * ((n_rows_w + 127) / 128) * ksplit;
-    shape = big >= 128 ? 3 : 1;
+    const int blocks256 = ((M + 255) / 256) * ((n_rows_w + 255) / 256) * ksplit;
+    shape = (fits && M > 128 && blocks256 >= 48) ? 5 : big >= 128 ? 3 : 1;
   }
+  if (shape == 5 && !fits) shape = 3;
   switch (shape) {
+    case 5:
+      if constexpr (EPI != 2)
+        launch_block256<TO, EPI>(A, W, bias, C, M, n_rows_w, K, lda, ldc, ksplit, stream);
+      break;
     case 1:
       launch_tile_cfg<TO, EPI, 1, 2, 4, 2, 32, 2, 2>(A, W, bias, C, M, n_rows_w, K, lda, ldc, ksplit,
                                                   stream);
@@ -505,8 +770,8 @@ static int launch_bf16(const bf16_t* A, const bf16_t* W, const float* bias, TO* 
 }
 
 // K, lda must be multiples of 8 and A, W 16-byte aligned (checked by the caller).
-// force_kernel: 0 = by M, 1 = tile kernel, 2 = skinny kernel (M <= 64 only), 3..6 = tile kernel
-// with block shape 1..4 (see launch_tile); for tests and tuning.
+// force_kernel: 0 = by M, 1 = tile kernel, 2 = skinny kernel (M <= 64 only), 3..7 = tile kernel
+// with block shape 1..5 (see launch_tile); for tests and tuning.
 // ksplit > 1 (float output only): C is [ksplit][M][ldc] partial sums over K ranges.
 extern "C" int kappai_gemm_bf16(const void* A, const void* W, const float* bias, void* C, int M,
                                 int N, int K, int lda, int ldc, int out_is_f32, int force_kernel,

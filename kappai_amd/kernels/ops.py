@@ -135,18 +135,23 @@ def cast(x: torch.Tensor, dtype) -> torch.Tensor:
 def split_k_for(M: int, N: int, K: int) -> int:
     """How many K ranges a product is cut into when its consumer takes partial sums (1: not
     split).  Decode (M <= 64): so that about 512 blocks stream the matrix.  Larger M: so that
-    the 256 x 128 blocks of the tiled kernel fill the chip when N is small."""
+    the 256 x 256 blocks of the large-product kernel fill the chip when N is small; every range
+    is a multiple of 128 long, as that kernel asks."""
     if M > 64:
-        blocks = ((M + 255) // 256) * ((N + 127) // 128)
-        if blocks >= 192 or blocks < 16:
+        blocks = ((M + 255) // 256) * ((N + 255) // 256)
+        if blocks >= 128 or blocks < 8:
             return 1
-        return max(1, min(4, 256 // blocks, K // 1024))
+        split = max(1, min(8, 256 // blocks, K // 1024))
+        while split > 1 and K % (128 * split):
+            split -= 1
+        return split
     col_groups = (N + 15) // 16
     return max(1, min(8, 512 // col_groups, K // 512))
 
 
 def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
-           out_dtype=None, force_kernel: int = 0, partial_sums: bool = False) -> torch.Tensor:
+           out_dtype=None, force_kernel: int = 0, partial_sums: bool = False,
+           split_k: Optional[int] = None) -> torch.Tensor:
     """``x [M, K] @ weight[N, K]^T (+ bias)``.  A bfloat16 matrix runs on the matrix cores
     with float accumulation; a float32 matrix runs in true 32-bit arithmetic, whatever the
     activations' dtype.  ``x`` may be a view with a row stride.  With ``partial_sums`` the
@@ -175,7 +180,7 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] =
     _need(K % 8 == 0 and lda % 8 == 0 and xb.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0,
           f"linear: the bfloat16 kernels read 16 bytes at a time: K ({K}) and the row stride "
           f"({lda}) must be multiples of 8 and the tensors 16-byte aligned")
-    ksplit = split_k_for(M, N, K) if partial_sums else 1
+    ksplit = (split_k or split_k_for(M, N, K)) if partial_sums else 1
     if ksplit > 1:
         out = torch.empty((ksplit, M, N), dtype=F32, device=x.device)
         out_is_f32 = 1

@@ -140,6 +140,49 @@ def test_linear_swiglu(ops, M, F, K):
         close(got.float(), want, BF16_ULP, f"kernel {force}")
 
 
+BLOCK256 = 7          # force_kernel: 256 x 256 blocks, one wave a SIMD
+
+
+@pytest.mark.parametrize("M,N,K", [(256, 256, 128), (300, 520, 256), (129, 8, 128), (1000, 1096, 384),
+                                   (2048, 2048, 2048), (513, 264, 1280)])
+@pytest.mark.parametrize("out_dtype", [F32, BF16])
+def test_linear_block256(ops, M, N, K, out_dtype):
+    """The large-product kernel at sizes that end inside its 256 x 256 blocks, with a row stride
+    on the input, with bias, and against the other tiled kernel on the same data."""
+    wide = rand((M, K + 24), BF16, 41)
+    x, w, b = wide[:, :K], rand((N, K), BF16, 42), rand((N,), F32, 43)
+    want = x.double() @ w.double().T
+    tol = 2e-5 if out_dtype == F32 else BF16_ULP
+    xd = wide.to(DEV)[:, :K]
+    got = ops.linear(xd, w.to(DEV), out_dtype=out_dtype, force_kernel=BLOCK256)
+    close(got.float(), want, tol, "block256")
+    got = ops.linear(xd, w.to(DEV), b.to(DEV), out_dtype=out_dtype, force_kernel=BLOCK256)
+    close(got.float(), want + b.double(), tol, "block256 with bias")
+    other = ops.linear(xd, w.to(DEV), b.to(DEV), out_dtype=out_dtype, force_kernel=5)
+    close(got.float(), other.float(), tol, "against 256 x 128 blocks")
+
+
+@pytest.mark.parametrize("M,F,K", [(256, 128, 128), (300, 1008, 256), (2048, 1616, 384)])
+def test_linear_swiglu_block256(ops, M, F, K):
+    x, wg, wu = rand((M, K), BF16, 44), rand((F, K), BF16, 45, 0.2), rand((F, K), BF16, 46, 0.2)
+    w = ops.interleave_gate_up(wg.to(DEV), wu.to(DEV))
+    g, u = x.double() @ wg.double().T, x.double() @ wu.double().T
+    want = g / (1 + torch.exp(-g)) * u
+    got = ops.linear_swiglu(x.to(DEV), w, force_kernel=BLOCK256)
+    close(got.float(), want, BF16_ULP, "block256")
+
+
+def test_linear_block256_split_k(ops):
+    """Partial sums over K ranges from the large-product kernel add up to the product."""
+    M, N, K = 2048, 2048, 8192
+    x, w = rand((M, K), BF16, 47), rand((N, K), BF16, 48, 0.05)
+    S = ops.split_k_for(M, N, K)
+    assert S > 1
+    parts = ops.linear(x.to(DEV), w.to(DEV), partial_sums=True)
+    assert parts.shape == (S, M, N) and parts.dtype == F32
+    close(parts.sum(0), x.double() @ w.double().T, 2e-5, "sum of the partial sums")
+
+
 @pytest.mark.parametrize("M,N,K", [(1, 2048, 2048), (8, 2048, 8192), (16, 96, 1024), (40, 1000, 4096),
                                    (64, 64, 512), (5, 6144, 2048)])
 def test_linear_partial_sums(ops, M, N, K):
