@@ -600,23 +600,25 @@ struct ConvStep {
   int L;
 };
 
-template <typename TO, int MT, int NW, int EPI>
+template <typename TO, int MT, int NW, int EPI, int NT>
 __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny_kernel(
     const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, const float* __restrict__ bias,
     TO* __restrict__ C, int M, int N, int K, int lda, int ldc, ConvStep cs) {
-  constexpr int NG = EPI == 1 ? 2 : (EPI == 2 ? 3 : 1);      // row groups of W a block streams
+  static_assert(NT == 1 || EPI == 0, "several column tiles a wave: plain products only");
+  // row groups of W a block streams: gate/up, the three conv gates, or NT column tiles
+  constexpr int NG = EPI == 1 ? 2 : (EPI == 2 ? 3 : NT);
   __shared__ float red[NW][NG * MT][WAVE][4];
   const int tid = threadIdx.x;
   const int lane = tid % WAVE, wave = tid / WAVE;
-  const int n0 = blockIdx.x * 16;
+  const int n0 = blockIdx.x * 16 * NT;
   const int col = lane % 16, kg = (lane / 16) * 8;
   const int gn = n0 + col;
   const u32x4_t zero = {0u, 0u, 0u, 0u};
   f32x4_t acc[NG * MT];
 #pragma unroll
   for (int t = 0; t < NG * MT; ++t) acc[t] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
-  // plain: row gn.  SwiGLU: gate row 32*block + col, up row 16 further.  Conv: rows gn, N + gn,
-  // 2N + gn.
+  // plain: row gn (and 16 further for the next column tile).  SwiGLU: gate row 32*block + col, up
+  // row 16 further.  Conv: rows gn, N + gn, 2N + gn.
   const size_t wr0 = EPI == 1 ? (size_t)blockIdx.x * 32 + col : (size_t)gn;
   const size_t group_rows = EPI == 2 ? (size_t)N : 16;
   const bf16_t* wrow = W + (gn < N ? wr0 : 0) * K + kg;
@@ -633,7 +635,7 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny_kernel(
   const int k1 = min(kb1, k0 + kper);
   C += (size_t)blockIdx.y * M * ldc;
   // loads in flight a lane: U * (NG + MT)
-  constexpr int U = (NG + MT) <= 3 ? SK_UNROLL : ((NG + MT) <= 4 ? 4 : 2);
+  constexpr int U = (NG + MT) <= 3 ? SK_UNROLL : ((NG + MT) <= 6 ? 4 : 2);
   for (int k = k0; k < k1; k += 32 * U) {
     u32x4_t wv[U][NG], av[U][MT];
 #pragma unroll
@@ -642,7 +644,8 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny_kernel(
       const bool kin = gk + kg < k1;
 #pragma unroll
       for (int r = 0; r < NG; ++r)
-        wv[u][r] = (kin && gn < N) ? load16(wrow + r * group_rows * K + gk) : zero;
+        wv[u][r] = (kin && gn + (EPI == 0 ? r * 16 : 0) < N) ? load16(wrow + r * group_rows * K + gk)
+                                                               : zero;
 #pragma unroll
       for (int t = 0; t < MT; ++t)
         av[u][t] = (kin && t * 16 + col < M) ? load16(arow[t] + gk) : zero;
@@ -662,7 +665,24 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny_kernel(
     for (int v = 0; v < 4; ++v) red[wave][t][lane][v] = acc[t][v];
   __syncthreads();
   // the first MT waves each sum one row tile over the NW partial results, in a fixed order
-  if (wave < MT && gn < N) {
+  if (EPI == 0 && NT > 1) {
+    // waves take the NT * MT tiles in turn
+    for (int tile = wave; tile < NT * MT; tile += NW) {
+      const int r = tile / MT, t = tile % MT;
+      const int gnr = gn + r * 16;
+      if (gnr >= N) continue;
+      const float bv = (bias && blockIdx.y == 0) ? bias[gnr] : 0.f;
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        const int gm = t * 16 + 4 * (lane / 16) + v;
+        if (gm >= M) continue;
+        float sum = red[0][tile][lane][v];
+#pragma unroll
+        for (int w = 1; w < NW; ++w) sum += red[w][tile][lane][v];
+        store_out(C + (size_t)gm * ldc + gnr, sum + bv);
+      }
+    }
+  } else if (wave < MT && gn < N) {
     const int t = wave;
     const float bv = (bias && blockIdx.y == 0) ? bias[gn] : 0.f;
 #pragma unroll
@@ -714,11 +734,12 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny_kernel(
   }
 }
 
-template <typename TO, int MT, int NW, int EPI>
+template <typename TO, int MT, int NW, int EPI, int NT = 1>
 static void launch_skinny(const bf16_t* A, const bf16_t* W, const float* bias, TO* C, int M, int N,
                           int K, int lda, int ldc, int ksplit, ConvStep cs, hipStream_t stream) {
-  hipLaunchKernelGGL((gemm_bf16_skinny_kernel<TO, MT, NW, EPI>), dim3((N + 15) / 16, ksplit),
-                     dim3(NW * WAVE), 0, stream, A, W, bias, C, M, N, K, lda, ldc, cs);
+  hipLaunchKernelGGL((gemm_bf16_skinny_kernel<TO, MT, NW, EPI, NT>),
+                     dim3((N + 16 * NT - 1) / (16 * NT), ksplit), dim3(NW * WAVE), 0, stream, A, W,
+                     bias, C, M, N, K, lda, ldc, cs);
 }
 
 // more waves a block when there are few blocks, so that about 2048 waves or more stream W
@@ -726,6 +747,14 @@ template <typename TO, int MT, int EPI>
 static void launch_skinny_mt(const bf16_t* A, const bf16_t* W, const float* bias, TO* C, int M,
                              int N, int K, int lda, int ldc, int ksplit, ConvStep cs,
                              hipStream_t stream) {
+  // several row tiles and a plain product: a wave takes two column tiles for every fragment
+  // of A it loads, which halves the reads of A (every block reads all of it)
+  if constexpr (EPI == 0 && MT >= 2) {
+    if (N >= 64) {
+      launch_skinny<TO, MT, 4, EPI, 2>(A, W, bias, C, M, N, K, lda, ldc, ksplit, cs, stream);
+      return;
+    }
+  }
   const int blocks = ((N + 15) / 16) * ksplit;
   const int kb = K / ksplit;                              // K a block
   constexpr int NG = EPI == 1 ? 2 : (EPI == 2 ? 3 : 1);
