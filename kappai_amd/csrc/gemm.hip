@@ -303,8 +303,8 @@ static void launch_tile_cfg(const bf16_t* A, const bf16_t* W, const float* bias,
 // (256 accumulator registers): per 16 of K a wave reads 8 fragments from LDS for 16 matrix
 // instructions.  Tiles of 64 of K (128-byte rows, whole cache lines) go from global memory
 // straight into LDS (global_load_lds), two buffers; the 16-byte chunks of a row are permuted
-// by (chunk ^ row % 8) on the way in, so that fragment reads meet no bank conflict without
-// padding.  The order of LDS reads, loads and matrix instructions is written out slot by slot
+// by (chunk ^ (row / 2) % 8) on the way in, so that the 16 lanes of a fragment read (16 rows,
+// one chunk each) fall on 16 different 16-byte bank groups without padding.  The order of LDS reads, loads and matrix instructions is written out slot by slot
 // and fenced, one wave has to hide every latency by itself: while the products of one 16 of K
 // run, the fragments of the next are read; the loads of tile k+2 are issued as soon as the
 // barrier of tile k has shown that everybody is done with its buffer.
@@ -348,7 +348,7 @@ void gemm_bf16_block256_kernel(const bf16_t* __restrict__ A, const bf16_t* __res
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
   // One load instruction = 8 rows x 128 bytes: lane -> (row lane/8, LDS chunk lane%8), which
-  // receives the row's chunk (lane%8) ^ (row%8).  Waves 0, 1 bring the A tile, waves 2, 3 the W
+  // receives the row's chunk (lane%8) ^ ((row/2)%8).  Waves 0, 1 bring the A tile, waves 2, 3 the W
   // tile, 16 instructions each; rows past the end of the matrix repeat its last row (their
   // products are never stored).
   const bool brings_a = wave < 2;
@@ -357,12 +357,14 @@ void gemm_bf16_block256_kernel(const bf16_t* __restrict__ A, const bf16_t* __res
   const int ld = brings_a ? lda : K;
   const int last_row = (brings_a ? M : N) - 1;
   const int row0 = brings_a ? m0 + wave * 128 : n0 + (wave - 2) * 128;
-  const int lrow = lane / 8, lchunk = (lane % 8) ^ lrow;
+  const int lrow = lane / 8;
   uint32_t roff[16];
 #pragma unroll
-  for (int i = 0; i < 16; ++i)
+  for (int i = 0; i < 16; ++i) {
+    const int lchunk = (lane % 8) ^ (((i * 8 + lrow) >> 1) & 7);
     roff[i] = (uint32_t)(min(row0 + i * 8 + lrow, last_row) * ld + lchunk * 8) *
               (uint32_t)sizeof(bf16_t);
+  }
   // the address of a load is a wave-uniform 64-bit base (the tile's first column) plus the
   // lane's 32-bit row offset; pinning the base into scalar registers keeps the compiler from
   // folding the two into sixteen 64-bit per-lane pointers
@@ -382,8 +384,8 @@ void gemm_bf16_block256_kernel(const bf16_t* __restrict__ A, const bf16_t* __res
   int aoff[4], woff[4];
 #pragma unroll
   for (int s = 0; s < 4; ++s) {
-    aoff[s] = (wm * 128 + r_in) * BK + (((s * 2 + hh) ^ (r_in & 7)) * 8);
-    woff[s] = A_TILE + (wn * 128 + r_in) * BK + (((s * 2 + hh) ^ (r_in & 7)) * 8);
+    aoff[s] = (wm * 128 + r_in) * BK + (((s * 2 + hh) ^ ((r_in >> 1) & 7)) * 8);
+    woff[s] = A_TILE + (wn * 128 + r_in) * BK + (((s * 2 + hh) ^ ((r_in >> 1) & 7)) * 8);
   }
   bf16x8_t fa[2][4], fw[2][4];
   // in the order the products ask for them: w0 a0 w1 w2 w3 a1 a2 a3
