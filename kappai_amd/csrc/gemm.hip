@@ -322,12 +322,16 @@ static void launch_tile_cfg(const bf16_t* A, const bf16_t* W, const float* bias,
 
 template <int N> struct IntC { static constexpr int value = N; };
 
-template <typename TO, int EPI>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
+template <typename TO, int EPI, int WT>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4 / WT, 4 / WT)))
 void gemm_bf16_block256_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W,
                                const float* __restrict__ bias, TO* __restrict__ C, int M, int N,
                                int K, int lda, int ldc, int tiles_n) {
-  constexpr int BM = 256, BN = 256, BK = 64;
+  // WT x WT accumulator tiles of 32 x 32 a wave: 4 -> 256 x 256 blocks, 2 -> 128 x 128
+  constexpr int BM = WT * 64, BN = WT * 64, BK = 64;
+  constexpr int WROWS = WT * 32;                               // rows (columns) of a wave's tile
+  constexpr int NPROD = WT * WT, NREAD = 2 * WT;               // per 16 of K
+  constexpr int NLOAD = 4 * WT, HALF = NLOAD / 2;              // load instructions a wave and tile
   constexpr int A_TILE = BM * BK, BUF = (BM + BN) * BK;        // in bf16
   extern __shared__ __attribute__((aligned(1024))) bf16_t lds[];
   const int tid = threadIdx.x, lane = tid % WAVE;
@@ -339,28 +343,28 @@ void gemm_bf16_block256_kernel(const bf16_t* __restrict__ A, const bf16_t* __res
   const int nk = kblk / BK;
   C += (size_t)blockIdx.y * M * ldc;
 
-  f32x16_t acc[4][4];
+  f32x16_t acc[WT][WT];
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int i = 0; i < WT; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
+    for (int j = 0; j < WT; ++j)
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
   // One load instruction = 8 rows x 128 bytes: lane -> (row lane/8, LDS chunk lane%8), which
   // receives the row's chunk (lane%8) ^ ((row/2)%8).  Waves 0, 1 bring the A tile, waves 2, 3 the W
-  // tile, 16 instructions each; rows past the end of the matrix repeat its last row (their
+  // tile, NLOAD instructions each; rows past the end of the matrix repeat its last row (their
   // products are never stored).
   const bool brings_a = wave < 2;
   const char* gk = reinterpret_cast<const char*>(brings_a ? A : W) +
                    (size_t)blockIdx.y * kblk * sizeof(bf16_t);
   const int ld = brings_a ? lda : K;
   const int last_row = (brings_a ? M : N) - 1;
-  const int row0 = brings_a ? m0 + wave * 128 : n0 + (wave - 2) * 128;
+  const int row0 = brings_a ? m0 + wave * WROWS : n0 + (wave - 2) * WROWS;
   const int lrow = lane / 8;
-  uint32_t roff[16];
+  uint32_t roff[NLOAD];
 #pragma unroll
-  for (int i = 0; i < 16; ++i) {
+  for (int i = 0; i < NLOAD; ++i) {
     const int lchunk = (lane % 8) ^ (((i * 8 + lrow) >> 1) & 7);
     roff[i] = (uint32_t)(min(row0 + i * 8 + lrow, last_row) * ld + lchunk * 8) *
               (uint32_t)sizeof(bf16_t);
@@ -376,7 +380,7 @@ void gemm_bf16_block256_kernel(const bf16_t* __restrict__ A, const bf16_t* __res
   };
   auto load_one = [&](int buf, const char* base, int i) {
     __builtin_amdgcn_global_load_lds(KAPPAI_GPTR(base + roff[i]),
-                                     KAPPAI_LPTR(lds + buf * BUF + (wave * 16 + i) * 8 * BK), 16,
+                                     KAPPAI_LPTR(lds + buf * BUF + (wave * NLOAD + i) * 8 * BK), 16,
                                      0, 0);
   };
   // fragments of the 16 of K number s: chunks 2s and 2s+1; lane -> (row lane%32, chunk 2s+lane/32)
@@ -384,14 +388,14 @@ void gemm_bf16_block256_kernel(const bf16_t* __restrict__ A, const bf16_t* __res
   int aoff[4], woff[4];
 #pragma unroll
   for (int s = 0; s < 4; ++s) {
-    aoff[s] = (wm * 128 + r_in) * BK + (((s * 2 + hh) ^ ((r_in >> 1) & 7)) * 8);
-    woff[s] = A_TILE + (wn * 128 + r_in) * BK + (((s * 2 + hh) ^ ((r_in >> 1) & 7)) * 8);
+    aoff[s] = (wm * WROWS + r_in) * BK + (((s * 2 + hh) ^ ((r_in >> 1) & 7)) * 8);
+    woff[s] = A_TILE + (wn * WROWS + r_in) * BK + (((s * 2 + hh) ^ ((r_in >> 1) & 7)) * 8);
   }
-  bf16x8_t fa[2][4], fw[2][4];
-  // in the order the products ask for them: w0 a0 w1 w2 w3 a1 a2 a3
+  bf16x8_t fa[2][WT], fw[2][WT];
+  // in the order the products ask for them: w0 a0, the other w, the other a
   auto read_one = [&](int fb, int buf, int s, int idx) {
-    const bool is_w = idx == 0 || (idx >= 2 && idx <= 4);
-    const int n = idx <= 1 ? 0 : idx <= 4 ? idx - 1 : idx - 4;
+    const bool is_w = idx == 0 || (idx >= 2 && idx <= WT);
+    const int n = idx <= 1 ? 0 : idx <= WT ? idx - 1 : idx - WT;
     if (is_w)
       fw[fb][n] = as_bf16x8(
           *reinterpret_cast<const u32x4_t*>(lds + buf * BUF + woff[s] + n * 32 * BK));
@@ -400,7 +404,7 @@ void gemm_bf16_block256_kernel(const bf16_t* __restrict__ A, const bf16_t* __res
           *reinterpret_cast<const u32x4_t*>(lds + buf * BUF + aoff[s] + n * 32 * BK));
   };
   auto product = [&](int fb, int t) {
-    const int i = t / 4, j = t % 4;
+    const int i = t / WT, j = t % WT;
     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fw[fb][j], fa[fb][i], acc[i][j], 0, 0, 0);
   };
   // One tile of K out of buffer U.  next: there is a tile kt+1 (its second half is loaded
@@ -413,15 +417,22 @@ void gemm_bf16_block256_kernel(const bf16_t* __restrict__ A, const bf16_t* __res
 #pragma unroll
     for (int s = 0; s < 3; ++s) {
 #pragma unroll
-      for (int t = 0; t < 16; ++t) {
-        if (t < 8) read_one((s + 1) & 1, U, s + 1, t);
-        if (s == 0 && t >= 8 && next) load_one(U ^ 1, base1, t);
+      for (int t = 0; t < NPROD; ++t) {
+        if (t < NREAD) read_one((s + 1) & 1, U, s + 1, t);
+        if (s == 0 && t >= NPROD - HALF && next) load_one(U ^ 1, base1, HALF + t - (NPROD - HALF));
         product(s & 1, t);
         SCHED_FENCE();
       }
     }
+    // the last 16 of K: a few products first, so that the matrix cores have work while the
+    // wave waits at the barrier
+    constexpr int PRE = WT == 4 ? 4 : 1;
+    constexpr int REST = NPROD - PRE;
+    constexpr int SPREAD = REST < 8 ? REST : 8;         // slots that also read and load
+    constexpr int READS_PER = (NREAD + SPREAD - 1) / SPREAD;
+    constexpr int LOADS_PER = (HALF + SPREAD - 1) / SPREAD;
 #pragma unroll
-    for (int t = 0; t < 4; ++t) {
+    for (int t = 0; t < PRE; ++t) {
       product(1, t);
       SCHED_FENCE();
     }
@@ -431,23 +442,28 @@ void gemm_bf16_block256_kernel(const bf16_t* __restrict__ A, const bf16_t* __res
     }
     SCHED_FENCE();
 #pragma unroll
-    for (int t = 4; t < 16; ++t) {
-      if (t < 12 && next) read_one(0, U ^ 1, 0, t - 4);
-      if (t < 12 && next2) load_one(U, base2, t - 4);
+    for (int t = PRE; t < NPROD; ++t) {
+      const int k = t - PRE;
+#pragma unroll
+      for (int q = 0; q < READS_PER; ++q)
+        if (k * READS_PER + q < NREAD && next) read_one(0, U ^ 1, 0, k * READS_PER + q);
+#pragma unroll
+      for (int q = 0; q < LOADS_PER; ++q)
+        if (k * LOADS_PER + q < HALF && next2) load_one(U, base2, k * LOADS_PER + q);
       product(1, t);
       SCHED_FENCE();
     }
   };
 
 #pragma unroll
-  for (int i = 0; i < 16; ++i) load_one(0, tile_base(0), i);
+  for (int i = 0; i < NLOAD; ++i) load_one(0, tile_base(0), i);
 #pragma unroll
-  for (int i = 0; i < 8; ++i) load_one(1, tile_base(1), i);
-  __builtin_amdgcn_s_waitcnt(0x0F70 | 8);       // vmcnt(8): tile 0 has landed
+  for (int i = 0; i < HALF; ++i) load_one(1, tile_base(1), i);
+  __builtin_amdgcn_s_waitcnt(0x0F70 | HALF);    // vmcnt(HALF): tile 0 has landed
   __builtin_amdgcn_s_barrier();
   SCHED_FENCE();
 #pragma unroll
-  for (int t = 0; t < 8; ++t) read_one(0, 0, 0, t);
+  for (int t = 0; t < NREAD; ++t) read_one(0, 0, 0, t);
 
   // nk is even: the loop body is straight-line code for the accumulators (a conditional
   // second tile would merge two versions of all 256 of them)
@@ -458,18 +474,18 @@ void gemm_bf16_block256_kernel(const bf16_t* __restrict__ A, const bf16_t* __res
   }
 
   // Epilogue: a wave turns 32 rows of its tile at a time through its own piece of LDS.
-  // acc[i][j][4g + e] is C[row (wm*4+i)*32 + lane%32][column (wn*4+j)*32 + 8g + 4*(lane/32) + e].
+  // acc[i][j][4g + e] is C[row (wm*WT+i)*32 + lane%32][column (wn*WT+j)*32 + 8g + 4*(lane/32) + e].
   __syncthreads();                               // everybody is done with the last tile
-  constexpr int OUT_COLS = EPI == 1 ? 64 : 128;  // columns a wave writes
+  constexpr int OUT_COLS = EPI == 1 ? WROWS / 2 : WROWS;   // columns a wave writes
   constexpr int ROW_BYTES = OUT_COLS * (int)sizeof(TO) + 16;
   char* mine = reinterpret_cast<char*>(lds) + wave * 32 * ROW_BYTES;
   const int out_n = EPI == 1 ? N / 2 : N;
-  const int col0 = EPI == 1 ? (n0 + wn * 128) / 2 : n0 + wn * 128;
+  const int col0 = EPI == 1 ? (n0 + wn * WROWS) / 2 : n0 + wn * WROWS;
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
+  for (int i = 0; i < WT; ++i) {
     char* wrow = mine + r_in * ROW_BYTES;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < WT; ++j) {
 #pragma unroll
       for (int g = 0; g < (EPI == 1 ? 2 : 4); ++g) {
         float v4[4];
@@ -506,7 +522,7 @@ void gemm_bf16_block256_kernel(const bf16_t* __restrict__ A, const bf16_t* __res
     for (int it = 0; it < 32 / ROWS_PER; ++it) {
       const int rr = it * ROWS_PER + lane / CHUNKS, ch = lane % CHUNKS;
       const u32x4_t v = *reinterpret_cast<const u32x4_t*>(mine + rr * ROW_BYTES + ch * 16);
-      const int gm = m0 + (wm * 4 + i) * 32 + rr, gn = col0 + ch * PER;
+      const int gm = m0 + (wm * WT + i) * 32 + rr, gn = col0 + ch * PER;
       if (gm < M && gn < out_n) *reinterpret_cast<u32x4_t*>(C + (size_t)gm * ldc + gn) = v;
     }
   }
@@ -521,27 +537,28 @@ static bool block256_fits(const bf16_t* A, const bf16_t* W, TO* C, int M, int n_
          (long long)M * lda < limit && (long long)n_rows_w * K < limit;
 }
 
-template <typename TO, int EPI>
+template <typename TO, int EPI, int WT>
 static void launch_block256(const bf16_t* A, const bf16_t* W, const float* bias, TO* C, int M,
                             int n_rows_w, int K, int lda, int ldc, int ksplit,
                             hipStream_t stream) {
-  constexpr size_t lds_bytes = 2 * (256 + 256) * 64 * sizeof(bf16_t);
-  auto kern = gemm_bf16_block256_kernel<TO, EPI>;
+  constexpr int B = WT * 64;                     // block edge
+  constexpr size_t lds_bytes = 2 * (B + B) * 64 * sizeof(bf16_t);
+  auto kern = gemm_bf16_block256_kernel<TO, EPI, WT>;
   static bool attr_set = false;
   if (!attr_set) {
     (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
                               (int)lds_bytes);
     attr_set = true;
   }
-  const int tn = (n_rows_w + 255) / 256, tm = (M + 255) / 256;
+  const int tn = (n_rows_w + B - 1) / B, tm = (M + B - 1) / B;
   hipLaunchKernelGGL(kern, dim3(tm * tn, ksplit), dim3(256), lds_bytes, stream, A, W, bias, C, M,
                      n_rows_w, K, lda, ldc, tn);
 }
 
 // shape: 0 = chosen by size, 1 = 128x128 blocks of two waves, 2 = 256x128 blocks (tiles of 32
 // of K, two LDS buffers), 3 = 256x128 blocks (tiles of 64 of K, one LDS buffer), 4 = 256x256
-// blocks of the same kernel (tiles of 64 of K), 5 = the 256x256 kernel with one wave a SIMD
-// (when the sizes fit it, else 3)
+// blocks of the same kernel (tiles of 64 of K), 5 = the 256x256 kernel with one wave a SIMD, 6 = its
+// 128x128 form (when the sizes fit them, else 3)
 template <typename TO, int EPI>
 static void launch_tile(const bf16_t* A, const bf16_t* W, const float* bias, TO* C, int M,
                         int n_rows_w, int K, int lda, int ldc, int ksplit, int shape,
@@ -550,13 +567,19 @@ static void launch_tile(const bf16_t* A, const bf16_t* W, const float* bias, TO*
   if (shape == 0) {
     const int big = ((M + 255) / 256) * ((n_rows_w + 127) / 128) * ksplit;
     const int blocks256 = ((M + 255) / 256) * ((n_rows_w + 255) / 256) * ksplit;
-    shape = (fits && M > 128 && blocks256 >= 48) ? 5 : big >= 128 ? 3 : 1;
+    // the one-wave-a-SIMD kernel when its 256 x 256 blocks fill most of the chip, its
+    // 128 x 128 form (two blocks a CU) below that
+    shape = !fits ? (big >= 128 ? 3 : 1) : blocks256 >= 192 ? 5 : 6;
   }
-  if (shape == 5 && !fits) shape = 3;
+  if ((shape == 5 || shape == 6) && !fits) shape = 3;
   switch (shape) {
     case 5:
       if constexpr (EPI != 2)
-        launch_block256<TO, EPI>(A, W, bias, C, M, n_rows_w, K, lda, ldc, ksplit, stream);
+        launch_block256<TO, EPI, 4>(A, W, bias, C, M, n_rows_w, K, lda, ldc, ksplit, stream);
+      break;
+    case 6:
+      if constexpr (EPI != 2)
+        launch_block256<TO, EPI, 2>(A, W, bias, C, M, n_rows_w, K, lda, ldc, ksplit, stream);
       break;
     case 1:
       launch_tile_cfg<TO, EPI, 1, 2, 4, 2, 32, 2, 2>(A, W, bias, C, M, n_rows_w, K, lda, ldc, ksplit,
@@ -801,8 +824,8 @@ static int launch_bf16(const bf16_t* A, const bf16_t* W, const float* bias, TO* 
 }
 
 // K, lda must be multiples of 8 and A, W 16-byte aligned (checked by the caller).
-// force_kernel: 0 = by M, 1 = tile kernel, 2 = skinny kernel (M <= 64 only), 3..7 = tile kernel
-// with block shape 1..5 (see launch_tile); for tests and tuning.
+// force_kernel: 0 = by M, 1 = tile kernel, 2 = skinny kernel (M <= 64 only), 3..8 = tile kernel
+// with block shape 1..6 (see launch_tile); for tests and tuning.
 // ksplit > 1 (float output only): C is [ksplit][M][ldc] partial sums over K ranges.
 extern "C" int kappai_gemm_bf16(const void* A, const void* W, const float* bias, void* C, int M,
                                 int N, int K, int lda, int ldc, int out_is_f32, int force_kernel,

@@ -134,14 +134,12 @@ def cast(x: torch.Tensor, dtype) -> torch.Tensor:
 # ---------------------------------------------------------------------------------------
 def split_k_for(M: int, N: int, K: int) -> int:
     """How many K ranges a product is cut into when its consumer takes partial sums (1: not
-    split).  Decode (M <= 64): so that about 512 blocks stream the matrix.  Larger M: so that
-    the 256 x 256 blocks of the large-product kernel fill the chip when N is small; every range
-    is a multiple of 128 long, as that kernel asks."""
+    split).  Decode (M <= 64): so that about 512 blocks stream the matrix.  Larger M: only long
+    K (ranges of 2048 or more) and few 128 x 128 blocks; every range is a multiple of 128 long,
+    as the large-product kernel asks."""
     if M > 64:
-        blocks = ((M + 255) // 256) * ((N + 255) // 256)
-        if blocks >= 128 or blocks < 8:
-            return 1
-        split = max(1, min(8, 256 // blocks, K // 1024))
+        blocks = ((M + 127) // 128) * ((N + 127) // 128)
+        split = max(1, min(8, 512 // blocks, K // 2048))
         while split > 1 and K % (128 * split):
             split -= 1
         return split

@@ -141,12 +141,14 @@ def test_linear_swiglu(ops, M, F, K):
 
 
 BLOCK256 = 7          # force_kernel: 256 x 256 blocks, one wave a SIMD
+BLOCK128 = 8          # the same kernel with 128 x 128 blocks
 
 
 @pytest.mark.parametrize("M,N,K", [(256, 256, 128), (300, 520, 256), (129, 8, 128), (1000, 1096, 384),
                                    (2048, 2048, 2048), (513, 264, 1280)])
 @pytest.mark.parametrize("out_dtype", [F32, BF16])
-def test_linear_block256(ops, M, N, K, out_dtype):
+@pytest.mark.parametrize("block", [BLOCK256, BLOCK128])
+def test_linear_block256(ops, M, N, K, out_dtype, block):
     """The large-product kernel at sizes that end inside its 256 x 256 blocks, with a row stride
     on the input, with bias, and against the other tiled kernel on the same data."""
     wide = rand((M, K + 24), BF16, 41)
@@ -154,21 +156,22 @@ def test_linear_block256(ops, M, N, K, out_dtype):
     want = x.double() @ w.double().T
     tol = 2e-5 if out_dtype == F32 else BF16_ULP
     xd = wide.to(DEV)[:, :K]
-    got = ops.linear(xd, w.to(DEV), out_dtype=out_dtype, force_kernel=BLOCK256)
+    got = ops.linear(xd, w.to(DEV), out_dtype=out_dtype, force_kernel=block)
     close(got.float(), want, tol, "block256")
-    got = ops.linear(xd, w.to(DEV), b.to(DEV), out_dtype=out_dtype, force_kernel=BLOCK256)
+    got = ops.linear(xd, w.to(DEV), b.to(DEV), out_dtype=out_dtype, force_kernel=block)
     close(got.float(), want + b.double(), tol, "block256 with bias")
     other = ops.linear(xd, w.to(DEV), b.to(DEV), out_dtype=out_dtype, force_kernel=5)
     close(got.float(), other.float(), tol, "against 256 x 128 blocks")
 
 
 @pytest.mark.parametrize("M,F,K", [(256, 128, 128), (300, 1008, 256), (2048, 1616, 384)])
-def test_linear_swiglu_block256(ops, M, F, K):
+@pytest.mark.parametrize("block", [BLOCK256, BLOCK128])
+def test_linear_swiglu_block256(ops, M, F, K, block):
     x, wg, wu = rand((M, K), BF16, 44), rand((F, K), BF16, 45, 0.2), rand((F, K), BF16, 46, 0.2)
     w = ops.interleave_gate_up(wg.to(DEV), wu.to(DEV))
     g, u = x.double() @ wg.double().T, x.double() @ wu.double().T
     want = g / (1 + torch.exp(-g)) * u
-    got = ops.linear_swiglu(x.to(DEV), w, force_kernel=BLOCK256)
+    got = ops.linear_swiglu(x.to(DEV), w, force_kernel=block)
     close(got.float(), want, BF16_ULP, "block256")
 
 
