@@ -118,7 +118,10 @@ __global__ __launch_bounds__(P_NW * WAVE) void attn_prefill_kernel(
     float scale) {
   // later tiles of a segment have more keys: they are started first
   const int tile = gridDim.x - 1 - blockIdx.x, h = blockIdx.y;
-  const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE;
+  const int lane = threadIdx.x % WAVE;
+  // the wave's number in scalar registers: everything that depends only on the key tile (its
+  // pages, its base addresses, whether it is masked) is then scalar work
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);
   const int seg = q_tiles[4 * tile], r0 = q_tiles[4 * tile + 1], nr = q_tiles[4 * tile + 2];
   const int g = h / (H / G);
   const int col = lane % 32, hh = lane / 32;
@@ -331,6 +334,236 @@ __global__ __launch_bounds__(P_NW * WAVE) void attn_prefill_kernel(
 }
 
 // ---------------------------------------------------------------------------------------
+// prefill, key tiles shared by the query heads of a kv head
+// ---------------------------------------------------------------------------------------
+// One block = one q tile (32 rows) x four query heads of one kv head, a wave each.  The four
+// waves walk the same key tiles, so a tile of K (32 keys x d) and of V^T (d x 32 keys) is brought
+// from global memory once, straight into LDS (global_load_lds, three buffers, two tiles ahead),
+// and every wave reads its matrix operands from there: a quarter of the cache traffic of one
+// wave per (tile, head).  K rows keep their 16-byte chunks permuted (chunk ^ f(key)) so that the
+// 16 keys of a fragment read fall on different banks; V^T lies as [16-key group][d][16 keys].
+// The running maximum is only moved when a tile's maximum exceeds it by more than 2^8: most
+// tiles then leave the output accumulators alone (no rescaling), and the weights stay <= 256.
+#if HEAD_DIM == 64 || HEAD_DIM == 128
+#define PG_OK 1
+#define PG_NBUF 3
+#define PG_GPTR(p) ((const __attribute__((address_space(1))) void*)(p))
+#define PG_LPTR(p) ((__attribute__((address_space(3))) void*)(p))
+
+__global__ __launch_bounds__(4 * WAVE) void attn_prefill_shared_kernel(
+    const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ k_pool,
+    const bf16_t* __restrict__ vt_pool, bf16_t* __restrict__ out, int out_stride,
+    const int* __restrict__ q_tiles, const int* __restrict__ row_pos,
+    const int* __restrict__ block_tables, int max_blocks, int H, int G, int ps, int window,
+    float scale) {
+  constexpr int ROWB = HEAD_DIM * 2;                // bytes of a key's row
+  constexpr int KTILE = 32 * ROWB, VGROUP = HEAD_DIM * 32, BUF = KTILE + 2 * VGROUP;   // bytes
+  constexpr int CPR = ROWB / 16;                    // 16-byte chunks a K row
+  constexpr int K_ROWS_PER = 1024 / ROWB;           // K rows one load instruction brings
+  constexpr int K_LOADS = 8 / K_ROWS_PER;           // a wave brings 8 keys
+  constexpr int V_LOADS = (HEAD_DIM / 2) / 32;      // and half of a 16-key group of V^T
+  __shared__ __attribute__((aligned(1024))) char lds[PG_NBUF * BUF];
+  const int tile = gridDim.x - 1 - blockIdx.x;      // later tiles have more keys: start them first
+  const int rep = H / G, quads = rep / 4;
+  const int g = blockIdx.y / quads;
+  const int lane = threadIdx.x % WAVE;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);
+  const int h = g * rep + (blockIdx.y % quads) * 4 + wave;
+  const int seg = q_tiles[4 * tile], r0 = q_tiles[4 * tile + 1], nr = q_tiles[4 * tile + 2];
+  const int col = lane % 32, hh = lane / 32;
+  const int* bt = block_tables + (size_t)seg * max_blocks;
+  const int pos_first = row_pos[r0], pos_last = pos_first + nr - 1;
+  const bool row_ok = col < nr;
+  const int my_pos = row_ok ? pos_first + col : -1;
+  const int my_lo = (window > 0 && my_pos + 1 > window) ? my_pos + 1 - window : 0;
+  const int lo_tile = (window > 0 && pos_first + 1 > window) ? pos_first + 1 - window : 0;
+  const int lo_last = (window > 0 && pos_last + 1 > window) ? pos_last + 1 - window : 0;
+
+  bf16x8_t qf[P_KS];
+  {
+    const bf16_t* qr = q + (size_t)(r0 + (row_ok ? col : 0)) * q_stride + (size_t)h * HEAD_DIM;
+#pragma unroll
+    for (int ks = 0; ks < P_KS; ++ks) {
+      u32x4_t v = {0u, 0u, 0u, 0u};
+      if (row_ok) v = *reinterpret_cast<const u32x4_t*>(qr + 16 * ks + 8 * hh);
+      qf[ks] = as_frag(v);
+    }
+  }
+  f32x16_t o[P_MT];
+#pragma unroll
+  for (int mt = 0; mt < P_MT; ++mt)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) o[mt][v] = 0.f;
+  float m_ref = -INFINITY, l_run = 0.f;
+  const float sc = scale * LOG2E;
+
+  const int kbase = (lo_tile / 32) * 32;
+  const int n_tiles = (pos_last - kbase) / 32 + 1;
+  auto swz = [](int key) { return HEAD_DIM == 64 ? (key >> 1) & 7 : key & 15; };
+  // what this lane brings: K row 8*wave + ..., V^T rows of group wave/2
+  const int k_row_in = lane / CPR, k_slot = lane % CPR;
+  const int v_st = wave / 2, v_d0 = (wave % 2) * (HEAD_DIM / 2) + lane / 2, v_half = lane % 2;
+  auto issue = [&](int it) {
+    const int kb = kbase + 32 * it;
+    char* buf = lds + (it % PG_NBUF) * BUF;
+    {
+      // the wave's 8 keys lie in one 16-key group, hence in one page; a group past the last
+      // key is read from the pool's first page instead and masked when it is used
+      const int key0 = kb + 8 * wave;
+      const int pidx = min(key0 / ps, max_blocks - 1);
+      int page = key0 <= pos_last ? bt[pidx] : 0;
+      page = max(page, 0);
+      const bf16_t* base = k_pool + (((size_t)page * G + g) * ps + key0 % ps) * HEAD_DIM;
+#pragma unroll
+      for (int i = 0; i < K_LOADS; ++i) {
+        const int row = i * K_ROWS_PER + k_row_in;               // 0..7 within the wave's keys
+        const int chunk = k_slot ^ swz(8 * wave + row);
+        __builtin_amdgcn_global_load_lds(PG_GPTR(base + row * HEAD_DIM + chunk * 8),
+                                         PG_LPTR(buf + (8 * wave + i * K_ROWS_PER) * ROWB), 16, 0,
+                                         0);
+      }
+    }
+    {
+      const int key0 = kb + 16 * v_st;
+      const int pidx = min(key0 / ps, max_blocks - 1);
+      int page = key0 <= pos_last ? bt[pidx] : 0;
+      page = max(page, 0);
+      const bf16_t* base = vt_pool + ((size_t)page * G + g) * HEAD_DIM * ps + key0 % ps;
+#pragma unroll
+      for (int i = 0; i < V_LOADS; ++i) {
+        const int dd = v_d0 + 32 * i;
+        __builtin_amdgcn_global_load_lds(
+            PG_GPTR(base + (size_t)dd * ps + 8 * v_half),
+            PG_LPTR(buf + KTILE + v_st * VGROUP + ((wave % 2) * (HEAD_DIM / 2) + 32 * i) * 32), 16,
+            0, 0);
+      }
+    }
+  };
+  auto whole = [&](int kb) { return kb >= lo_last && kb + 31 <= pos_first; };
+  auto work = [&](int it) {
+    const int kb = kbase + 32 * it;
+    const char* buf = lds + (it % PG_NBUF) * BUF;
+    const bool full = whole(kb);
+    // ---- S^T tile: 32 keys x 32 queries -------------------------------------------------
+    f32x16_t s;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) s[v] = 0.f;
+#pragma unroll
+    for (int ks = 0; ks < P_KS; ++ks) {
+      const u32x4_t kf = *reinterpret_cast<const u32x4_t*>(
+          buf + col * ROWB + (((2 * ks + hh) ^ swz(col)) * 16));
+      s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_frag(kf), qf[ks], s, 0, 0, 0);
+    }
+    // V^T operands: d index 32*mt + col, keys 16*st + 4*hh .. +3 and 8 more
+    u32x2_t va[2][P_MT], vb[2][P_MT];
+#pragma unroll
+    for (int st = 0; st < 2; ++st)
+#pragma unroll
+      for (int mt = 0; mt < P_MT; ++mt) {
+        const char* vp = buf + KTILE + st * VGROUP + (32 * mt + col) * 32 + 8 * hh;
+        va[st][mt] = *reinterpret_cast<const u32x2_t*>(vp);
+        vb[st][mt] = *reinterpret_cast<const u32x2_t*>(vp + 16);
+      }
+    // lane holds, for query `col`, keys kb + 8*(v/4) + 4*hh + v%4
+    float mloc = -INFINITY;
+    if (full) {
+#pragma unroll
+      for (int v = 0; v < 16; ++v) mloc = fmaxf(mloc, s[v]);
+      mloc *= sc;           // sc > 0: scaling commutes with the maximum
+    } else {
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int key = kb + 8 * (v / 4) + 4 * hh + v % 4;
+        const bool ok = key <= my_pos && key >= my_lo;
+        s[v] = ok ? s[v] : -INFINITY;
+        mloc = fmaxf(mloc, s[v] * sc);
+      }
+      // what lies in LDS for keys outside the tile's range is not cache content: zero it
+#pragma unroll
+      for (int st = 0; st < 2; ++st) {
+        int keep_a = 0, keep_b = 0;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int ka = kb + 16 * st + 4 * hh + i, kbb = ka + 8;
+          if (ka >= lo_tile && ka <= pos_last) keep_a |= 1 << i;
+          if (kbb >= lo_tile && kbb <= pos_last) keep_b |= 1 << i;
+        }
+#pragma unroll
+        for (int mt = 0; mt < P_MT; ++mt) {
+          va[st][mt] = mask4(va[st][mt], keep_a);
+          vb[st][mt] = mask4(vb[st][mt], keep_b);
+        }
+      }
+    }
+    mloc = fmaxf(mloc, __shfl_xor(mloc, 32, WAVE));
+    // move the reference only when it is far off (or unset): uniform for the wave's branch
+    const bool move = mloc > m_ref + 8.0f || (m_ref == -INFINITY && mloc > -INFINITY);
+    if (__builtin_amdgcn_ballot_w64(move) != 0) {
+      const float m_new = move ? mloc : m_ref;
+      const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+      const float corr = move ? fast_exp2(m_ref - m_safe) : 1.0f;
+      l_run *= corr;
+#pragma unroll
+      for (int mt = 0; mt < P_MT; ++mt)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) o[mt][v] *= corr;
+      m_ref = m_new;
+    }
+    const float m_safe = m_ref == -INFINITY ? 0.f : m_ref;
+    float lsum = 0.f;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      s[v] = fast_exp2(fmaf(s[v], sc, -m_safe));
+      lsum += s[v];
+    }
+    lsum += __shfl_xor(lsum, 32, WAVE);
+    l_run += lsum;
+    // ---- O^T += V^T P^T, two k-steps of 16 keys ---------------------------------------
+#pragma unroll
+    for (int st = 0; st < 2; ++st) {
+      const u32x4_t pw = {pack_bf16(s[8 * st + 0], s[8 * st + 1]),
+                          pack_bf16(s[8 * st + 2], s[8 * st + 3]),
+                          pack_bf16(s[8 * st + 4], s[8 * st + 5]),
+                          pack_bf16(s[8 * st + 6], s[8 * st + 7])};
+      const bf16x8_t pf = as_frag(pw);
+#pragma unroll
+      for (int mt = 0; mt < P_MT; ++mt) {
+        const u32x4_t vw = {va[st][mt].x, va[st][mt].y, vb[st][mt].x, vb[st][mt].y};
+        o[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_frag(vw), pf, o[mt], 0, 0, 0);
+      }
+    }
+  };
+
+  constexpr int NL = K_LOADS + V_LOADS;              // loads a wave issues per tile
+  issue(0);
+  if (n_tiles > 1) issue(1);
+  for (int it = 0; it < n_tiles; ++it) {
+    // tile `it` has landed (this wave's part; the barrier makes it everybody's), tile it+1 may
+    // still be on its way
+    if (it + 1 < n_tiles) __builtin_amdgcn_s_waitcnt(0x0F70 | NL);
+    else __builtin_amdgcn_s_waitcnt(0x0F70);
+    __builtin_amdgcn_s_barrier();     // no fence: a fence would wait for the loads in flight
+    if (it + 2 < n_tiles) issue(it + 2);             // into the buffer of tile it-1: all done with it
+    work(it);
+  }
+  if (!row_ok) return;
+  const float inv = l_run > 0.f ? 1.0f / l_run : 0.f;
+  bf16_t* orow = out + (size_t)(r0 + col) * out_stride + (size_t)h * HEAD_DIM;
+#pragma unroll
+  for (int mt = 0; mt < P_MT; ++mt)
+#pragma unroll
+    for (int v4 = 0; v4 < 4; ++v4) {
+      const int dd = 32 * mt + 8 * v4 + 4 * hh;     // four consecutive d: v = 4*v4 .. 4*v4+3
+      u32x2_t w = {pack_bf16(o[mt][4 * v4] * inv, o[mt][4 * v4 + 1] * inv),
+                   pack_bf16(o[mt][4 * v4 + 2] * inv, o[mt][4 * v4 + 3] * inv)};
+      *reinterpret_cast<u32x2_t*>(orow + dd) = w;
+    }
+}
+#else
+#define PG_OK 0
+#endif
+
+// ---------------------------------------------------------------------------------------
 // decode: one row a request; columns are the query heads of one kv head (at most 16)
 // ---------------------------------------------------------------------------------------
 #define D_KS ((HEAD_DIM + 31) / 32)     // k-steps of S^T over d (32 each)
@@ -528,14 +761,31 @@ extern "C" int kappai_attn_keys_per_wave(void) { return D_KPW; }
 
 extern "C" int kappai_attn_head_dim(void) { return HEAD_DIM; }
 
+// variant: 0 = chosen by shape, 1 = one block per (tile, head), 2 = key tiles shared by four
+// query heads of a kv head (head sizes 64 and 128, a multiple of four heads per kv head).
 extern "C" int kappai_attn_prefill(const void* q, int q_stride, const void* k_pool,
                                    const void* vt_pool, void* out, int out_stride,
                                    const int* q_tiles, int n_tiles, const int* row_pos,
                                    const int* block_tables, int max_blocks, int H, int G, int ps,
-                                   int window, float scale, hipStream_t stream) {
+                                   int window, float scale, int variant, hipStream_t stream) {
   if (n_tiles <= 0) return 0;
   if (ps % 16 || G < 1 || H % G || H > 65535 || (q_stride % 8) || (out_stride % 4))
     return (int)hipErrorInvalidValue;
+  const int rep = H / G;
+  const bool shared_ok = PG_OK && rep % 4 == 0;
+  if (variant == 2 && !shared_ok) return (int)hipErrorInvalidValue;
+  // sharing pays when there are blocks enough to fill the chip without splitting the keys of
+  // a q tile over waves
+  const bool shared = variant == 2 || (variant == 0 && shared_ok && n_tiles * (H / 4) >= 256);
+#if PG_OK
+  if (shared) {
+    hipLaunchKernelGGL(attn_prefill_shared_kernel, dim3(n_tiles, H / 4), dim3(4 * WAVE), 0, stream,
+                       (const bf16_t*)q, q_stride, (const bf16_t*)k_pool, (const bf16_t*)vt_pool,
+                       (bf16_t*)out, out_stride, q_tiles, row_pos, block_tables, max_blocks, H, G,
+                       ps, window, scale);
+    KAPPAI_RETURN_LAUNCH_STATUS();
+  }
+#endif
   hipLaunchKernelGGL(attn_prefill_kernel, dim3(n_tiles, H), dim3(P_NW * WAVE), 0, stream,
                      (const bf16_t*)q, q_stride, (const bf16_t*)k_pool, (const bf16_t*)vt_pool,
                      (bf16_t*)out, out_stride, q_tiles, row_pos, block_tables, max_blocks, H, G,

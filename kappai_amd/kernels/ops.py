@@ -363,7 +363,7 @@ def paged_attention(q: torch.Tensor, n_heads: int, n_kv_heads: int, head_dim: in
                     row_seg: torch.Tensor, block_tables: torch.Tensor, page_size: int,
                     scale: float, window: int = 0, q_tiles: Optional[torch.Tensor] = None,
                     single_rows: bool = False, max_position: Optional[int] = None,
-                    kernel: str = "auto") -> torch.Tensor:
+                    kernel: str = "auto", prefill_variant: int = 0) -> torch.Tensor:
     """Causal attention of every row over the keys of its request that are in the cache
     (its own included; the last ``window`` of them when a window is set).  ``q`` is
     [T, >= H d] with a row stride (the q columns of the fused projection).  Returns [T, H d].
@@ -372,7 +372,9 @@ def paged_attention(q: torch.Tensor, n_heads: int, n_kv_heads: int, head_dim: in
     cores: the split-key decode kernel when every segment is a single row (``single_rows``;
     ``max_position`` sizes the splits), else the tiled kernel over ``q_tiles`` [tiles, 4] =
     (segment, first row, rows <= 32, 0).  Everything else, float32 included, runs the plain
-    kernel.  ``kernel`` = "rows" | "prefill" | "decode" forces one (for tests)."""
+    kernel.  ``kernel`` = "rows" | "prefill" | "decode" forces one (for tests);
+    ``prefill_variant`` 1 / 2 forces the tiled kernel's form (2: key tiles shared by four query
+    heads of a kv head through LDS; head sizes 64 and 128 only)."""
     H, G, d = n_heads, n_kv_heads, head_dim
     _gpu("q", q, (F32, BF16), contiguous=False)
     T = q.shape[0]
@@ -419,7 +421,8 @@ def paged_attention(q: torch.Tensor, n_heads: int, n_kv_heads: int, head_dim: in
             _ptr(q), _c_int(q.stride(0)), _ptr(k_pool), _ptr(v_pool), _ptr(out), _c_int(H * d),
             _ptr(q_tiles), _c_int(q_tiles.shape[0]), _ptr(row_pos), _ptr(block_tables),
             _c_int(block_tables.shape[1]), _c_int(H), _c_int(G), _c_int(page_size),
-            _c_int(window or 0), _c_float(scale), _stream()), "attn_prefill")
+            _c_int(window or 0), _c_float(scale), _c_int(prefill_variant), _stream()),
+            "attn_prefill")
         return out
     _need(kernel == "decode", f"unknown attention kernel {kernel!r}")
     _need(H // G <= 16, "the decode kernel takes at most 16 query heads per kv head")

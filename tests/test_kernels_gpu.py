@@ -362,6 +362,9 @@ ATT_CASES = [
     (6, 3, 48, 32, [200, 7, 95], [1, 1, 1], 48, 1, True, 40),                   # decode, window
     (16, 1, 32, 16, [130, 2], [1, 1], 32, 1, False, 0),                         # 16 heads a kv head
     (4, 4, 128, 16, [77, 140], [40, 1], 128, 1, True, 0),
+    (8, 2, 64, 16, [0, 300, 31], [130, 70, 1], 64, 1, True, 0),                 # 4 heads a kv head
+    (8, 1, 128, 32, [250, 0], [45, 97], 128, 1, True, 0),                       # 8 heads a kv head
+    (4, 1, 64, 48, [120, 0, 66], [80, 33, 2], 64, 1, True, 50),                 # window, page 48
 ]
 
 
@@ -397,11 +400,14 @@ def test_store_and_attention(ops, dtype, case):
     kernels = ["rows"]
     if dtype == BF16 and ps % 16 == 0 and d % 16 == 0 and d <= 256:
         kernels += ["prefill"] + (["decode"] if c["single"] and H // G <= 16 else [])
+        if d in (64, 128) and (H // G) % 4 == 0:
+            kernels += ["prefill-shared"]
     for kernel in kernels:
         got = ops.paged_attention(dev["qkv"], H, G, d, dev["k_pool"], dev["v_pool"],
                                   dev["row_pos"], dev["row_seg"], dev["bt"], ps, scale,
                                   window=window, q_tiles=dev["q_tiles"], single_rows=c["single"],
-                                  max_position=c["max_pos"], kernel=kernel)
+                                  max_position=c["max_pos"], kernel=kernel.split("-")[0],
+                                  prefill_variant=2 if kernel == "prefill-shared" else 1)
         close(got.float(), want, tol * 2, f"attention kernel {kernel}")
 
 
@@ -430,9 +436,41 @@ def test_attention_finds_one_far_key(ops, dtype):
             got = ops.paged_attention(dev["qkv"], H, G, d, dev["k_pool"], dev["v_pool"],
                                       dev["row_pos"], dev["row_seg"], dev["bt"], ps,
                                       1.0 / math.sqrt(d), q_tiles=dev["q_tiles"], single_rows=True,
-                                      max_position=c["max_pos"], kernel=kernel)
+                                      max_position=c["max_pos"], kernel=kernel, prefill_variant=1)
             close(got.float(), want, 2 * BF16_ULP if dtype == BF16 else 1e-5,
                   f"far key at {far}, kernel {kernel}")
+
+
+def test_attention_shared_tiles_find_one_far_key(ops):
+    """The same for the kernel that shares key tiles between four heads of a kv head: a prompt
+    portion of 40 rows after 700 cached keys; every row's query matches one far key only."""
+    H, G, d, ps = 8, 2, 64, 16
+    n, new = 700, 40
+    for far in (0, 15, 16, 31, 32, 63, 64, 65, 319, 640, 698, 699, 700, 731):
+        c = paged_case(11, BF16, H, G, d, ps, [n], [new])
+        q = torch.zeros(d)
+        q[3] = 40.0
+        c["qkv"][:, :H * d] = q.repeat(H).to(BF16)
+        c["k_pool"].zero_()
+        c["v_pool"].copy_(rand(c["v_pool"].shape, BF16, 12))
+        bt = c["bt"]
+        c["k_pool"][bt[0, far // ps], :, far % ps, 3] = 8.0
+        marker = rand((G, d), BF16, 13) + 3.0
+        c["v_pool"][bt[0, far // ps], :, :, far % ps] = marker
+        # positions past the cached keys are the rows' own: zero keys, random values
+        for p in range(n, n + new):
+            if p != far:
+                c["k_pool"][bt[0, p // ps], :, p % ps, :] = 0
+        dev = {k: (v.to(DEV) if torch.is_tensor(v) else v) for k, v in c.items()}
+        got = ops.paged_attention(dev["qkv"], H, G, d, dev["k_pool"], dev["v_pool"],
+                                  dev["row_pos"], dev["row_seg"], dev["bt"], ps,
+                                  1.0 / math.sqrt(d), q_tiles=dev["q_tiles"], kernel="prefill",
+                                  prefill_variant=2)
+        want = marker.float().repeat_interleave(H // G, dim=0).reshape(1, H * d)
+        # rows that can see the far key return its value
+        first = max(0, far - n)
+        close(got[first:].float(), want.expand(new - first, -1), 2 * BF16_ULP,
+              f"far key at {far}")
 
 
 # ---------------------------------------------------------------------------------------
