@@ -45,6 +45,14 @@ __device__ __forceinline__ u32x2_t mask4(u32x2_t v, int keep) {
 
 #define LOG2E 1.4426950408889634f
 
+// the value that lane ^ 32 holds, by one swap of the wave's halves (no trip through LDS)
+__device__ __forceinline__ float other_half(float x) {
+  const uint32_t u = __float_as_uint(x);
+  const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  // r[0] = the lower half's values in both halves, r[1] = the upper half's
+  return __uint_as_float((threadIdx.x & 32) ? r[0] : r[1]);
+}
+
 // four key slots of V^T for d index `dd`, keys key0..key0+3 (one 16-key group: one page);
 // keys outside [lo, hi] read as zero
 __device__ __forceinline__ u32x2_t load_vt4(const bf16_t* __restrict__ vt_pool,
@@ -232,7 +240,7 @@ __global__ __launch_bounds__(P_NW * WAVE) void attn_prefill_kernel(
         mloc = fmaxf(mloc, s[v] * sc);
       }
     }
-    mloc = fmaxf(mloc, __shfl_xor(mloc, 32, WAVE));
+    mloc = fmaxf(mloc, other_half(mloc));
     const float m_new = fmaxf(m_run, mloc);
     const float m_safe = m_new == -INFINITY ? 0.f : m_new;
     const float corr = fast_exp2(m_run - m_safe);
@@ -242,7 +250,7 @@ __global__ __launch_bounds__(P_NW * WAVE) void attn_prefill_kernel(
       s[v] = fast_exp2(fmaf(s[v], sc, -m_safe));
       lsum += s[v];
     }
-    lsum += __shfl_xor(lsum, 32, WAVE);
+    lsum += other_half(lsum);
     l_run = l_run * corr + lsum;
     m_run = m_new;
 #pragma unroll
@@ -336,21 +344,23 @@ __global__ __launch_bounds__(P_NW * WAVE) void attn_prefill_kernel(
 // ---------------------------------------------------------------------------------------
 // prefill, key tiles shared by the query heads of a kv head
 // ---------------------------------------------------------------------------------------
-// One block = one q tile (32 rows) x four query heads of one kv head, a wave each.  The four
-// waves walk the same key tiles, so a tile of K (32 keys x d) and of V^T (d x 32 keys) is brought
-// from global memory once, straight into LDS (global_load_lds, three buffers, two tiles ahead),
-// and every wave reads its matrix operands from there: a quarter of the cache traffic of one
-// wave per (tile, head).  K rows keep their 16-byte chunks permuted (chunk ^ f(key)) so that the
+// One block = two q tiles (32 rows each) of one segment x four query heads of one kv head, a
+// wave each.  The eight waves walk the same key tiles, so a tile of K (32 keys x d) and of V^T
+// (d x 32 keys) is brought from global memory once, straight into LDS (global_load_lds, three
+// buffers, two tiles ahead), and every wave reads its matrix operands from there.  Pairing an
+// early q tile with a late one gives every block the same number of keys to walk.  K rows keep their 16-byte chunks permuted (chunk ^ f(key)) so that the
 // 16 keys of a fragment read fall on different banks; V^T lies as [16-key group][d][16 keys].
 // The running maximum is only moved when a tile's maximum exceeds it by more than 2^8: most
 // tiles then leave the output accumulators alone (no rescaling), and the weights stay <= 256.
 #if HEAD_DIM == 64 || HEAD_DIM == 128
 #define PG_OK 1
 #define PG_NBUF 3
+#define PG_SUB 2
+template <int N> struct PgBuf { static constexpr int value = N; };
 #define PG_GPTR(p) ((const __attribute__((address_space(1))) void*)(p))
 #define PG_LPTR(p) ((__attribute__((address_space(3))) void*)(p))
 
-__global__ __launch_bounds__(4 * WAVE) void attn_prefill_shared_kernel(
+__global__ __launch_bounds__(8 * WAVE) void attn_prefill_shared_kernel(
     const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ k_pool,
     const bf16_t* __restrict__ vt_pool, bf16_t* __restrict__ out, int out_stride,
     const int* __restrict__ q_tiles, const int* __restrict__ row_pos,
@@ -360,16 +370,40 @@ __global__ __launch_bounds__(4 * WAVE) void attn_prefill_shared_kernel(
   constexpr int KTILE = 32 * ROWB, VGROUP = HEAD_DIM * 32, BUF = KTILE + 2 * VGROUP;   // bytes
   constexpr int CPR = ROWB / 16;                    // 16-byte chunks a K row
   constexpr int K_ROWS_PER = 1024 / ROWB;           // K rows one load instruction brings
-  constexpr int K_LOADS = 8 / K_ROWS_PER;           // a wave brings 8 keys
-  constexpr int V_LOADS = (HEAD_DIM / 2) / 32;      // and half of a 16-key group of V^T
-  __shared__ __attribute__((aligned(1024))) char lds[PG_NBUF * BUF];
-  const int tile = gridDim.x - 1 - blockIdx.x;      // later tiles have more keys: start them first
+  constexpr int NL = 8 / K_ROWS_PER;                // loads a wave issues per tile: a K wave
+                                                    // brings 8 keys, a V wave half a 16-key group
+  static_assert(NL == (HEAD_DIM / 2) / 32, "K and V waves issue the same number of loads");
+  // a buffer holds PG_SUB key tiles: one barrier for that many tiles
+  __shared__ __attribute__((aligned(1024))) char lds[PG_NBUF * PG_SUB * BUF];
+  const int t_a = gridDim.x - 1 - blockIdx.x;
+  // The block's second q tile.  q_tiles[t][3] = (index of the tile within its segment) |
+  // (tiles of the segment << 16), 0 if unknown.  Without a window tile j is paired with tile
+  // n-1-j, so that every block walks about the same number of keys; with a window, with its
+  // neighbour, whose keys are nearly the same.  The later tile of a pair has no block of its own.
+  int t_b = -1;
+  {
+    const int info = q_tiles[4 * t_a + 3];
+    const int j = info & 0xffff, n = info >> 16;
+    if (n > 0) {
+      if (window == 0) {
+        if (2 * j > n - 1) return;
+        if (2 * j < n - 1) t_b = t_a + (n - 1 - 2 * j);
+      } else {
+        if (j & 1) return;
+        if (j + 1 < n) t_b = t_a + 1;
+      }
+    }
+  }
   const int rep = H / G, quads = rep / 4;
   const int g = blockIdx.y / quads;
   const int lane = threadIdx.x % WAVE;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);
-  const int h = g * rep + (blockIdx.y % quads) * 4 + wave;
-  const int seg = q_tiles[4 * tile], r0 = q_tiles[4 * tile + 1], nr = q_tiles[4 * tile + 2];
+  const int grp = wave / 4;                         // 0: tile a, 1: tile b
+  const int h = g * rep + (blockIdx.y % quads) * 4 + wave % 4;
+  const int tile = grp == 0 ? t_a : t_b;
+  const bool has_tile = tile >= 0;
+  const int seg = q_tiles[4 * t_a];                 // both tiles are of one segment
+  const int r0 = has_tile ? q_tiles[4 * tile + 1] : 0, nr = has_tile ? q_tiles[4 * tile + 2] : 0;
   const int col = lane % 32, hh = lane / 32;
   const int* bt = block_tables + (size_t)seg * max_blocks;
   const int pos_first = row_pos[r0], pos_last = pos_first + nr - 1;
@@ -378,6 +412,18 @@ __global__ __launch_bounds__(4 * WAVE) void attn_prefill_shared_kernel(
   const int my_lo = (window > 0 && my_pos + 1 > window) ? my_pos + 1 - window : 0;
   const int lo_tile = (window > 0 && pos_first + 1 > window) ? pos_first + 1 - window : 0;
   const int lo_last = (window > 0 && pos_last + 1 > window) ? pos_last + 1 - window : 0;
+  // the keys the block walks: from the first key of either tile to the last key of either
+  int blk_first, blk_last;
+  {
+    const int ra = q_tiles[4 * t_a + 1], pa0 = row_pos[ra], pa1 = pa0 + q_tiles[4 * t_a + 2] - 1;
+    blk_first = (window > 0 && pa0 + 1 > window) ? pa0 + 1 - window : 0;
+    blk_last = pa1;
+    if (t_b >= 0) {
+      const int rb = q_tiles[4 * t_b + 1], pb0 = row_pos[rb], pb1 = pb0 + q_tiles[4 * t_b + 2] - 1;
+      blk_first = min(blk_first, (window > 0 && pb0 + 1 > window) ? pb0 + 1 - window : 0);
+      blk_last = max(blk_last, pb1);
+    }
+  }
 
   bf16x8_t qf[P_KS];
   {
@@ -397,52 +443,66 @@ __global__ __launch_bounds__(4 * WAVE) void attn_prefill_shared_kernel(
   float m_ref = -INFINITY, l_run = 0.f;
   const float sc = scale * LOG2E;
 
-  const int kbase = (lo_tile / 32) * 32;
-  const int n_tiles = (pos_last - kbase) / 32 + 1;
+  const int kbase = (blk_first / 32) * 32;
+  const int n_tiles = (blk_last - kbase) / 32 + 1;
   auto swz = [](int key) { return HEAD_DIM == 64 ? (key >> 1) & 7 : key & 15; };
-  // what this lane brings: K row 8*wave + ..., V^T rows of group wave/2
+  // what this lane brings: waves 0-3 eight rows of K each, waves 4-7 half a 16-key group of V^T
   const int k_row_in = lane / CPR, k_slot = lane % CPR;
-  const int v_st = wave / 2, v_d0 = (wave % 2) * (HEAD_DIM / 2) + lane / 2, v_half = lane % 2;
-  auto issue = [&](int it) {
-    const int kb = kbase + 32 * it;
-    char* buf = lds + (it % PG_NBUF) * BUF;
-    {
-      // the wave's 8 keys lie in one 16-key group, hence in one page; a group past the last
-      // key is read from the pool's first page instead and masked when it is used
-      const int key0 = kb + 8 * wave;
-      const int pidx = min(key0 / ps, max_blocks - 1);
-      int page = key0 <= pos_last ? bt[pidx] : 0;
-      page = max(page, 0);
-      const bf16_t* base = k_pool + (((size_t)page * G + g) * ps + key0 % ps) * HEAD_DIM;
+  const int vw = wave - 4, v_st = vw / 2, v_d0 = (vw % 2) * (HEAD_DIM / 2) + lane / 2;
+  const int v_half = lane % 2;
+  // The buffer of a tile is a compile-time constant (the tile loop is unrolled three times):
+  // only then can the compiler tell that the loads it issues into one buffer do not touch
+  // the buffer it reads from, and leave them in flight across the reads.
+  // Tiles are issued in order, so the wave keeps the place of its next keys (block table
+  // index, offset in the page) and looks the next page up one tile ahead; a group past the
+  // last key (or given back by the window) is read from the pool's first page instead and
+  // masked when it is used.  A wave's keys (8 of K, 16 of V^T) lie in one page.
+  int nx_key = kbase + (wave < 4 ? 8 * wave : 16 * v_st);
+  int nx_pidx = nx_key / ps, nx_off = nx_key % ps;
+  auto lookup = [&]() {
+    const int page = nx_key <= blk_last ? bt[min(nx_pidx, max_blocks - 1)] : 0;
+    return max(page, 0);
+  };
+  int nx_page = lookup();
+  auto issue_one = [&](char* buf) {
+    if (wave < 4) {
+      const bf16_t* base = k_pool + (((size_t)nx_page * G + g) * ps + nx_off) * HEAD_DIM;
 #pragma unroll
-      for (int i = 0; i < K_LOADS; ++i) {
+      for (int i = 0; i < NL; ++i) {
         const int row = i * K_ROWS_PER + k_row_in;               // 0..7 within the wave's keys
         const int chunk = k_slot ^ swz(8 * wave + row);
         __builtin_amdgcn_global_load_lds(PG_GPTR(base + row * HEAD_DIM + chunk * 8),
                                          PG_LPTR(buf + (8 * wave + i * K_ROWS_PER) * ROWB), 16, 0,
                                          0);
       }
-    }
-    {
-      const int key0 = kb + 16 * v_st;
-      const int pidx = min(key0 / ps, max_blocks - 1);
-      int page = key0 <= pos_last ? bt[pidx] : 0;
-      page = max(page, 0);
-      const bf16_t* base = vt_pool + ((size_t)page * G + g) * HEAD_DIM * ps + key0 % ps;
+    } else {
+      const bf16_t* base = vt_pool + ((size_t)nx_page * G + g) * HEAD_DIM * ps + nx_off;
 #pragma unroll
-      for (int i = 0; i < V_LOADS; ++i) {
+      for (int i = 0; i < NL; ++i) {
         const int dd = v_d0 + 32 * i;
         __builtin_amdgcn_global_load_lds(
             PG_GPTR(base + (size_t)dd * ps + 8 * v_half),
-            PG_LPTR(buf + KTILE + v_st * VGROUP + ((wave % 2) * (HEAD_DIM / 2) + 32 * i) * 32), 16,
-            0, 0);
+            PG_LPTR(buf + KTILE + v_st * VGROUP + ((vw % 2) * (HEAD_DIM / 2) + 32 * i) * 32), 16, 0,
+            0);
       }
     }
+    nx_key += 32;
+    nx_off += 32;
+    while (nx_off >= ps) {
+      nx_off -= ps;
+      ++nx_pidx;
+    }
+    nx_page = lookup();
+  };
+  auto issue = [&](auto buf_c) {
+#pragma unroll
+    for (int sub = 0; sub < PG_SUB; ++sub)
+      issue_one(lds + (decltype(buf_c)::value * PG_SUB + sub) * BUF);
   };
   auto whole = [&](int kb) { return kb >= lo_last && kb + 31 <= pos_first; };
-  auto work = [&](int it) {
+  auto work = [&](auto buf_c, auto sub_c, int it) {
     const int kb = kbase + 32 * it;
-    const char* buf = lds + (it % PG_NBUF) * BUF;
+    const char* buf = lds + (decltype(buf_c)::value * PG_SUB + decltype(sub_c)::value) * BUF;
     const bool full = whole(kb);
     // ---- S^T tile: 32 keys x 32 queries -------------------------------------------------
     f32x16_t s;
@@ -495,9 +555,9 @@ __global__ __launch_bounds__(4 * WAVE) void attn_prefill_shared_kernel(
         }
       }
     }
-    mloc = fmaxf(mloc, __shfl_xor(mloc, 32, WAVE));
+    mloc = fmaxf(mloc, other_half(mloc));
     // move the reference only when it is far off (or unset): uniform for the wave's branch
-    const bool move = mloc > m_ref + 8.0f || (m_ref == -INFINITY && mloc > -INFINITY);
+    const bool move = mloc > m_ref + 8.0f;
     if (__builtin_amdgcn_ballot_w64(move) != 0) {
       const float m_new = move ? mloc : m_ref;
       const float m_safe = m_new == -INFINITY ? 0.f : m_new;
@@ -516,7 +576,7 @@ __global__ __launch_bounds__(4 * WAVE) void attn_prefill_shared_kernel(
       s[v] = fast_exp2(fmaf(s[v], sc, -m_safe));
       lsum += s[v];
     }
-    lsum += __shfl_xor(lsum, 32, WAVE);
+    lsum += other_half(lsum);
     l_run += lsum;
     // ---- O^T += V^T P^T, two k-steps of 16 keys ---------------------------------------
 #pragma unroll
@@ -528,23 +588,35 @@ __global__ __launch_bounds__(4 * WAVE) void attn_prefill_shared_kernel(
       const bf16x8_t pf = as_frag(pw);
 #pragma unroll
       for (int mt = 0; mt < P_MT; ++mt) {
-        const u32x4_t vw = {va[st][mt].x, va[st][mt].y, vb[st][mt].x, vb[st][mt].y};
-        o[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_frag(vw), pf, o[mt], 0, 0, 0);
+        const u32x4_t vw4 = {va[st][mt].x, va[st][mt].y, vb[st][mt].x, vb[st][mt].y};
+        o[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_frag(vw4), pf, o[mt], 0, 0, 0);
       }
     }
   };
 
-  constexpr int NL = K_LOADS + V_LOADS;              // loads a wave issues per tile
-  issue(0);
-  if (n_tiles > 1) issue(1);
-  for (int it = 0; it < n_tiles; ++it) {
-    // tile `it` has landed (this wave's part; the barrier makes it everybody's), tile it+1 may
-    // still be on its way
-    if (it + 1 < n_tiles) __builtin_amdgcn_s_waitcnt(0x0F70 | NL);
+  // `it` counts buffers' worth of tiles (PG_SUB each)
+  const int n_steps = (n_tiles + PG_SUB - 1) / PG_SUB;
+  auto step = [&](auto buf_c, int it) {
+    constexpr int B = decltype(buf_c)::value;
+    // the tiles of this step have landed (this wave's part; the barrier makes it everybody's),
+    // those of the next step may still be on their way
+    if (it + 1 < n_steps) __builtin_amdgcn_s_waitcnt(0x0F70 | (PG_SUB * NL));
     else __builtin_amdgcn_s_waitcnt(0x0F70);
     __builtin_amdgcn_s_barrier();     // no fence: a fence would wait for the loads in flight
-    if (it + 2 < n_tiles) issue(it + 2);             // into the buffer of tile it-1: all done with it
-    work(it);
+    // step it+2 goes into the buffer of step it-1: everybody is done with it
+    if (it + 2 < n_steps) issue(PgBuf<(B + 2) % PG_NBUF>{});
+    const int kb = kbase + 32 * PG_SUB * it;
+    if (has_tile && kb + 31 >= lo_tile && kb <= pos_last) work(buf_c, PgBuf<0>{}, PG_SUB * it);
+    if (has_tile && kb + 63 >= lo_tile && kb + 32 <= pos_last)
+      work(buf_c, PgBuf<1>{}, PG_SUB * it + 1);
+  };
+  static_assert(PG_SUB == 2, "the step works on two tiles");
+  issue(PgBuf<0>{});
+  if (n_steps > 1) issue(PgBuf<1>{});
+  for (int it = 0; it < n_steps; it += PG_NBUF) {
+    step(PgBuf<0>{}, it);
+    if (it + 1 < n_steps) step(PgBuf<1>{}, it + 1);
+    if (it + 2 < n_steps) step(PgBuf<2>{}, it + 2);
   }
   if (!row_ok) return;
   const float inv = l_run > 0.f ? 1.0f / l_run : 0.f;
@@ -662,7 +734,7 @@ __global__ __launch_bounds__(64) void attn_decode_kernel(
           mloc = fmaxf(mloc, s[tt][v]);
         }
       mloc = fmaxf(mloc, __shfl_xor(mloc, 16, WAVE));
-      mloc = fmaxf(mloc, __shfl_xor(mloc, 32, WAVE));
+      mloc = fmaxf(mloc, other_half(mloc));
       const float m_new = fmaxf(m_run, mloc);
       const float m_safe = m_new == -INFINITY ? 0.f : m_new;
       const float corr = fast_exp2(m_run - m_safe);
@@ -675,7 +747,7 @@ __global__ __launch_bounds__(64) void attn_decode_kernel(
           lsum += s[tt][v];
         }
       lsum += __shfl_xor(lsum, 16, WAVE);
-      lsum += __shfl_xor(lsum, 32, WAVE);
+      lsum += other_half(lsum);
       l_run = l_run * corr + lsum;
       m_run = m_new;
       const u32x4_t pw = {pack_bf16(s[0][0], s[0][1]), pack_bf16(s[0][2], s[0][3]),
@@ -779,7 +851,7 @@ extern "C" int kappai_attn_prefill(const void* q, int q_stride, const void* k_po
   const bool shared = variant == 2 || (variant == 0 && shared_ok && n_tiles * (H / 4) >= 256);
 #if PG_OK
   if (shared) {
-    hipLaunchKernelGGL(attn_prefill_shared_kernel, dim3(n_tiles, H / 4), dim3(4 * WAVE), 0, stream,
+    hipLaunchKernelGGL(attn_prefill_shared_kernel, dim3(n_tiles, H / 4), dim3(8 * WAVE), 0, stream,
                        (const bf16_t*)q, q_stride, (const bf16_t*)k_pool, (const bf16_t*)vt_pool,
                        (bf16_t*)out, out_stride, q_tiles, row_pos, block_tables, max_blocks, H, G,
                        ps, window, scale);

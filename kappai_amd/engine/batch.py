@@ -46,12 +46,20 @@ class RowBatch:
     seg_pos0: torch.Tensor
     seg_slot: torch.Tensor
     logit_rows: torch.Tensor
-    q_tiles: Optional[torch.Tensor] = None      # [tiles, 4]: (segment, first row, rows, 0)
+    q_tiles: Optional[torch.Tensor] = None      # [tiles, 4]: (segment, first row, rows, place)
     block_tables: List[torch.Tensor] = field(default_factory=list)
     host: Dict[str, np.ndarray] = field(default_factory=dict)
 
 
 ATTENTION_TILE_ROWS = 32
+
+
+def tile_place(index: int, tiles_in_segment: int) -> int:
+    """The fourth number of a q tile; 0 (place unknown) when the segment has more tiles than
+    the 16 bits of either half hold."""
+    if tiles_in_segment > 0x7fff:
+        return 0
+    return index | (tiles_in_segment << 16)
 
 
 def layout_rows(entries: Sequence[StepEntry], cache: CacheManager, vocab_size: int):
@@ -83,8 +91,12 @@ def layout_rows(entries: Sequence[StepEntry], cache: CacheManager, vocab_size: i
         row_pos.extend(range(p0, p0 + n))
         row_seg.extend([si] * n)
         seg_start.append(base + n)
-        for r in range(0, n, ATTENTION_TILE_ROWS):
-            q_tiles.append((si, base + r, min(ATTENTION_TILE_ROWS, n - r), 0))
+        n_seg_tiles = (n + ATTENTION_TILE_ROWS - 1) // ATTENTION_TILE_ROWS
+        for j, r in enumerate(range(0, n, ATTENTION_TILE_ROWS)):
+            # the fourth number tells a kernel where the tile stands in its segment
+            # (index | tiles of the segment << 16), so that it can pair tiles of one segment
+            q_tiles.append((si, base + r, min(ATTENTION_TILE_ROWS, n - r),
+                            tile_place(j, n_seg_tiles)))
         seg_pos0.append(p0)
         seg_slot.append(e.cache.slot)
         logit_rows.extend(base + int(w) for w in e.want)

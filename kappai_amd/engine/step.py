@@ -70,6 +70,7 @@ class _DecodeGraph:
         self.h["q_tiles"][:, 0] = np.arange(B)
         self.h["q_tiles"][:, 1] = np.arange(B)
         self.h["q_tiles"][:, 2] = 1
+        self.h["q_tiles"][:, 3] = 1 << 16         # tile 0 of 1 in its segment
         # a warm-up run on the scratch page and the scratch slot: every kernel of this shape is
         # loaded and has run once before the capture, and no request's cache is touched
         self.h["seg_slot"][:] = cache.scratch_slot

@@ -371,7 +371,8 @@ def paged_attention(q: torch.Tensor, n_heads: int, n_kv_heads: int, head_dim: in
     bfloat16 with a page size and head size that are multiples of 16 runs on the matrix
     cores: the split-key decode kernel when every segment is a single row (``single_rows``;
     ``max_position`` sizes the splits), else the tiled kernel over ``q_tiles`` [tiles, 4] =
-    (segment, first row, rows <= 32, 0).  Everything else, float32 included, runs the plain
+    (segment, first row, rows <= 32, place of the tile in its segment: index | tiles << 16, or 0).
+    Everything else, float32 included, runs the plain
     kernel.  ``kernel`` = "rows" | "prefill" | "decode" forces one (for tests);
     ``prefill_variant`` 1 / 2 forces the tiled kernel's form (2: key tiles shared by four query
     heads of a kv head through LDS; head sizes 64 and 128 only)."""

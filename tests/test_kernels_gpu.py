@@ -332,7 +332,8 @@ def paged_case(seed, dtype, H, G, d, ps, lens_before, lens_new, n_pages=None, sh
     qkv = rand((T, (H + 2 * G) * d), dtype, seed + 5)
     tiles, base = [], 0
     for s, n in enumerate(lens_new):
-        tiles += [(s, base + r, min(32, n - r), 0) for r in range(0, n, 32)]
+        nt = (n + 31) // 32
+        tiles += [(s, base + r, min(32, n - r), j | (nt << 16)) for j, r in enumerate(range(0, n, 32))]
         base += n
     return dict(qkv=qkv, k_pool=k_pool, v_pool=v_pool, row_pos=torch.from_numpy(row_pos),
                 row_seg=torch.from_numpy(row_seg), bt=torch.from_numpy(bt), T=T,
