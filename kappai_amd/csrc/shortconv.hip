@@ -41,6 +41,104 @@ __global__ void shortconv_out_kernel(const T* __restrict__ proj, const float* __
   from_f32(out + (size_t)t * D + c, cg * sum);
 }
 
+// bfloat16, D a multiple of 8, L <= 4: a thread takes 8 channels and a run of SC_RUN rows, 16
+// bytes a load, every load of the run in flight at once.  It carries the last L-1 values of bx
+// from row to row; at the run's first row (and where a new segment begins inside the run) they
+// come from the rows before, or from the state when those lie before the segment.
+#define SC_RUN 4
+#define SC_HMAX 3
+typedef __attribute__((ext_vector_type(4))) uint32_t sc_u32x4_t;
+
+__device__ __forceinline__ void sc_unpack8(sc_u32x4_t v, float* f) {
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    f[2 * i] = __uint_as_float(v[i] << 16);
+    f[2 * i + 1] = __uint_as_float(v[i] & 0xffff0000u);
+  }
+}
+
+template <int L>
+__global__ __launch_bounds__(256) void shortconv_out_vec_kernel(
+    const bf16_t* __restrict__ proj, const float* __restrict__ w, const float* __restrict__ bias,
+    const float* __restrict__ state, bf16_t* __restrict__ out, const int* __restrict__ row_seg,
+    const int* __restrict__ seg_start, const int* __restrict__ seg_pos0,
+    const int* __restrict__ seg_slot, int T, int D) {
+  constexpr int H = L - 1;
+  const int c0 = (blockIdx.y * blockDim.x + threadIdx.x) * 8;
+  const int t0 = blockIdx.x * SC_RUN;
+  if (c0 >= D) return;
+  const size_t ld = (size_t)3 * D;
+  // rows t0-H .. t0+SC_RUN-1: the gates of the run and of the rows just before it
+  sc_u32x4_t vb[SC_RUN + H], vx[SC_RUN + H], vc[SC_RUN];
+  const sc_u32x4_t zero = {0u, 0u, 0u, 0u};
+#pragma unroll
+  for (int i = 0; i < SC_RUN + H; ++i) {
+    const int t = t0 - H + i;
+    const bool in = t >= 0 && t < T;
+    const bf16_t* p = proj + (size_t)(in ? t : 0) * ld + c0;
+    vb[i] = in ? *reinterpret_cast<const sc_u32x4_t*>(p) : zero;
+    vx[i] = in ? *reinterpret_cast<const sc_u32x4_t*>(p + 2 * D) : zero;
+    if (i >= H) vc[i - H] = in ? *reinterpret_cast<const sc_u32x4_t*>(p + D) : zero;
+  }
+  // the 8 channels' taps lie together: 8 L floats from a 16-byte aligned address
+  float wt[8 * L], bs[8];
+  {
+    const float4* wp = reinterpret_cast<const float4*>(w + (size_t)c0 * L);
+#pragma unroll
+    for (int i = 0; i < 2 * L; ++i) {
+      const float4 v = wp[i];
+      wt[4 * i] = v.x, wt[4 * i + 1] = v.y, wt[4 * i + 2] = v.z, wt[4 * i + 3] = v.w;
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) bs[j] = 0.f;
+    if (bias) {
+      const float4 b0 = *reinterpret_cast<const float4*>(bias + c0);
+      const float4 b1 = *reinterpret_cast<const float4*>(bias + c0 + 4);
+      bs[0] = b0.x, bs[1] = b0.y, bs[2] = b0.z, bs[3] = b0.w;
+      bs[4] = b1.x, bs[5] = b1.y, bs[6] = b1.z, bs[7] = b1.w;
+    }
+  }
+  float bx[SC_RUN + H][8];
+#pragma unroll
+  for (int i = 0; i < SC_RUN + H; ++i) {
+    float b[8], x[8];
+    sc_unpack8(vb[i], b);
+    sc_unpack8(vx[i], x);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) bx[i][j] = b[j] * x[j];
+  }
+#pragma unroll
+  for (int r = 0; r < SC_RUN; ++r) {
+    const int t = t0 + r;
+    if (t >= T) break;
+    const int seg = row_seg[t];
+    const int first = seg_start[seg];
+    const bool fresh = seg_pos0[seg] == 0;
+    const float* st = state + ((size_t)seg_slot[seg] * D + c0) * H;
+    float cg[8], res[8];
+    sc_unpack8(vc[r], cg);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) res[j] = bs[j];
+    // tap k meets the row t - H + k, which is loaded row r + k
+#pragma unroll
+    for (int k = 0; k < L; ++k) {
+      const int src = t - H + k;
+      if (src >= first) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) res[j] = fmaf(wt[j * L + k], bx[r + k][j], res[j]);
+      } else if (!fresh) {
+        const int e = H + (src - first);            // entry of the state: H-1 is the newest
+#pragma unroll
+        for (int j = 0; j < 8; ++j) res[j] = fmaf(wt[j * L + k], st[(size_t)j * H + e], res[j]);
+      }
+    }
+    sc_u32x4_t o;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) o[i] = pack_bf16x2(cg[2 * i] * res[2 * i], cg[2 * i + 1] * res[2 * i + 1]);
+    *reinterpret_cast<sc_u32x4_t*>(out + (size_t)t * D + c0) = o;
+  }
+}
+
 template <typename T>
 __global__ void shortconv_state_kernel(const T* __restrict__ proj, float* __restrict__ state,
                                        const int* __restrict__ seg_start,
@@ -115,7 +213,22 @@ extern "C" int kappai_shortconv(const void* proj, const float* w, const float* b
                          (const float*)proj, w, bias, state, (float*)out, seg_pos0, seg_slot, D, L);
     KAPPAI_RETURN_LAUNCH_STATUS();
   }
-  if (is_bf16) {
+  if (is_bf16 && D % 8 == 0 && L <= SC_HMAX + 1 && ((uintptr_t)proj % 16) == 0 &&
+      ((uintptr_t)out % 16) == 0 && ((uintptr_t)w % 16) == 0 && (!bias || ((uintptr_t)bias % 16) == 0)) {
+    const int groups = D / 8;
+    const int th = groups >= 256 ? 256 : 64;
+    const dim3 gv((T + SC_RUN - 1) / SC_RUN, (groups + th - 1) / th);
+#define SC_LAUNCH(LL)                                                                           \
+  hipLaunchKernelGGL(shortconv_out_vec_kernel<LL>, gv, dim3(th), 0, stream, (const bf16_t*)proj, \
+                     w, bias, (const float*)state, (bf16_t*)out, row_seg, seg_start, seg_pos0,  \
+                     seg_slot, T, D)
+    if (L == 2) SC_LAUNCH(2);
+    else if (L == 3) SC_LAUNCH(3);
+    else SC_LAUNCH(4);
+#undef SC_LAUNCH
+    hipLaunchKernelGGL(shortconv_state_kernel<bf16_t>, g2, dim3(threads), 0, stream,
+                       (const bf16_t*)proj, state, seg_start, seg_pos0, seg_slot, D, L);
+  } else if (is_bf16) {
     hipLaunchKernelGGL(shortconv_out_kernel<bf16_t>, g1, dim3(threads), 0, stream,
                        (const bf16_t*)proj, w, bias, (const float*)state, (bf16_t*)out, row_seg,
                        seg_start, seg_pos0, seg_slot, D, L);

@@ -238,8 +238,8 @@ def test_linear_refuses_what_it_cannot_do(ops):
 
 # ---------------------------------------------------------------------------------------
 @pytest.mark.parametrize("dtype", [F32, BF16])
-@pytest.mark.parametrize("D", [1, 3, 7, 33, 300])
-@pytest.mark.parametrize("L", [2, 3, 4])
+@pytest.mark.parametrize("D", [1, 3, 7, 33, 300, 8, 64, 304, 2048])
+@pytest.mark.parametrize("L", [2, 3, 4, 5])
 def test_shortconv(ops, dtype, D, L):
     """Segments of 1, 2, 9 and 40 rows, fresh and continued, in two steps so that the state
     written by the first is read by the second (kappai: src/test/test_hybrid.c:78-151)."""
