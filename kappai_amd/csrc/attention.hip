@@ -17,56 +17,163 @@
 #define MAX_HEAD_DIM 512
 
 // rot_mode: 0 none, 1 rotate-half pairs (j, j+rot/2), 2 interleaved pairs (2j, 2j+1)
+// A block of QKS_WAVES waves takes QKS_SLOTS heads (q, k or v) of one row, a wave a head at a
+// time, each wave with its own piece of LDS.
+#define QKS_WAVES 4
+#define QKS_SLOTS 16
 template <typename T>
-__global__ __launch_bounds__(64) void qk_norm_rope_store_kernel(
+__global__ __launch_bounds__(QKS_WAVES * WAVE) void qk_norm_rope_store_kernel(
     T* __restrict__ qkv, int row_stride, const float* __restrict__ q_norm_w,
     const float* __restrict__ k_norm_w, float eps, const float* __restrict__ cos_tab,
     const float* __restrict__ sin_tab, int rot_dim, int rot_mode, T* __restrict__ k_pool,
     T* __restrict__ v_pool, const int* __restrict__ row_pos, const int* __restrict__ row_seg,
     const int* __restrict__ block_tables, int max_blocks, int H, int G, int d, int ps,
-    int store_kv) {
-  __shared__ float buf[MAX_HEAD_DIM];
-  const int t = blockIdx.x, slot = blockIdx.y, lane = threadIdx.x;
+    int n_slots) {
+  __shared__ float bufs[QKS_WAVES][MAX_HEAD_DIM];
+  const int t = blockIdx.x, lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE;
+  float* buf = bufs[wave];
   const int pos = row_pos[t];
-  T* src = qkv + (size_t)t * row_stride + (size_t)slot * d;
-  T* dst = src;
-  if (slot >= H) {
-    const int g = (slot - H) % G;
-    const int* bt = block_tables + (size_t)row_seg[t] * max_blocks;
-    const size_t pg = (size_t)bt[pos / ps] * G + g;
-    if (slot >= H + G) {  // v: copied into its page, transposed
-      T* vdst = v_pool + pg * d * ps + pos % ps;
-      for (int e = lane; e < d; e += WAVE) vdst[(size_t)e * ps] = src[e];
-      return;
-    }
-    dst = k_pool + (pg * ps + pos % ps) * d;
-  }
-  const float* nw = slot < H ? q_norm_w : k_norm_w;
-  float ss = 0.f;
-  for (int e = lane; e < d; e += WAVE) {
-    const float v = to_f32(src[e]);
-    buf[e] = v;
-    ss += v * v;
-  }
-  if (nw) {
-    ss = wave_sum(ss);
-    const float sc = 1.0f / sqrtf(ss / (float)d + eps);
-    for (int e = lane; e < d; e += WAVE) buf[e] = buf[e] * sc * nw[e];
-  }
-  __syncthreads();
   if (rot_mode == 0) rot_dim = 0;
   const int half = rot_dim / 2;
   const float* ct = cos_tab + (size_t)pos * half;
   const float* st = sin_tab + (size_t)pos * half;
-  for (int j = lane; j < half; j += WAVE) {
-    const int i0 = rot_mode == 1 ? j : 2 * j;
-    const int i1 = rot_mode == 1 ? j + half : 2 * j + 1;
-    const float c = ct[j], s = st[j];
-    const float v0 = buf[i0], v1 = buf[i1];
-    from_f32(dst + i0, v0 * c - v1 * s);
-    from_f32(dst + i1, v0 * s + v1 * c);
+  const int* bt = block_tables + (size_t)row_seg[t] * max_blocks;
+  const int slot_end = min(n_slots, (int)(blockIdx.y + 1) * QKS_SLOTS);
+  for (int slot = blockIdx.y * QKS_SLOTS + wave; slot < slot_end; slot += QKS_WAVES) {
+    T* src = qkv + (size_t)t * row_stride + (size_t)slot * d;
+    T* dst = src;
+    if (slot >= H) {
+      const int g = (slot - H) % G;
+      const size_t pg = (size_t)bt[pos / ps] * G + g;
+      if (slot >= H + G) {  // v: copied into its page, transposed
+        T* vdst = v_pool + pg * d * ps + pos % ps;
+        for (int e = lane; e < d; e += WAVE) vdst[(size_t)e * ps] = src[e];
+        continue;
+      }
+      dst = k_pool + (pg * ps + pos % ps) * d;
+    }
+    const float* nw = slot < H ? q_norm_w : k_norm_w;
+    float ss = 0.f;
+    for (int e = lane; e < d; e += WAVE) {
+      const float v = to_f32(src[e]);
+      buf[e] = v;
+      ss += v * v;
+    }
+    if (nw) {
+      ss = wave_sum(ss);
+      const float sc = 1.0f / sqrtf(ss / (float)d + eps);
+      for (int e = lane; e < d; e += WAVE) buf[e] = buf[e] * sc * nw[e];
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    for (int j = lane; j < half; j += WAVE) {
+      const int i0 = rot_mode == 1 ? j : 2 * j;
+      const int i1 = rot_mode == 1 ? j + half : 2 * j + 1;
+      const float c = ct[j], s = st[j];
+      const float v0 = buf[i0], v1 = buf[i1];
+      from_f32(dst + i0, v0 * c - v1 * s);
+      from_f32(dst + i1, v0 * s + v1 * c);
+    }
+    for (int e = rot_dim + lane; e < d; e += WAVE) from_f32(dst + e, buf[e]);
+    // the next head overwrites the wave's piece of LDS
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
   }
-  for (int e = rot_dim + lane; e < d; e += WAVE) from_f32(dst + e, buf[e]);
+}
+
+// bfloat16, the whole head rotated in halves (or not at all), d / 8 a power of two up to 64:
+// a lane takes 8 consecutive elements of a head, so that a wave works on 512 / d heads at once
+// without LDS; the sum of squares and the rotation's partner (the lane d / 16 away) come by
+// shuffles.
+typedef __attribute__((ext_vector_type(4))) uint32_t qks_u32x4_t;
+template <int LPH>
+__global__ __launch_bounds__(256) void qk_norm_rope_store_vec_kernel(
+    bf16_t* __restrict__ qkv, int row_stride, const float* __restrict__ q_norm_w,
+    const float* __restrict__ k_norm_w, float eps, const float* __restrict__ cos_tab,
+    const float* __restrict__ sin_tab, int rotate, bf16_t* __restrict__ k_pool,
+    bf16_t* __restrict__ v_pool, const int* __restrict__ row_pos,
+    const int* __restrict__ row_seg, const int* __restrict__ block_tables, int max_blocks, int T,
+    int H, int G, int ps, int n_slots) {
+  constexpr int d = LPH * 8, half = d / 2;
+  const long long total = (long long)T * n_slots * LPH;
+  const long long gid = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  const bool active = gid < total;
+  const long long idx = active ? gid : total - 1;
+  const int part = (int)(idx % LPH);
+  const long long head = idx / LPH;
+  const int t = (int)(head / n_slots), slot = (int)(head % n_slots);
+  const int pos = row_pos[t];
+  const int e0 = 8 * part;
+  bf16_t* src = qkv + (size_t)t * row_stride + (size_t)slot * d + e0;
+  const qks_u32x4_t raw = *reinterpret_cast<const qks_u32x4_t*>(src);
+  float v[8];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    v[2 * i] = __uint_as_float(raw[i] << 16);
+    v[2 * i + 1] = __uint_as_float(raw[i] & 0xffff0000u);
+  }
+  const bool is_v = slot >= H + G;
+  const float* nw = slot < H ? q_norm_w : k_norm_w;
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) ss = fmaf(v[i], v[i], ss);
+#pragma unroll
+  for (int m = LPH / 2; m >= 1; m /= 2) ss += __shfl_xor(ss, m, WAVE);
+  if (nw && !is_v) {
+    const float sc = 1.0f / sqrtf(ss / (float)d + eps);
+    const float4 w0 = *reinterpret_cast<const float4*>(nw + e0);
+    const float4 w1 = *reinterpret_cast<const float4*>(nw + e0 + 4);
+    const float wv[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = v[i] * sc * wv[i];
+  }
+  float r[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) r[i] = v[i];
+  if (LPH >= 2) {
+    // partner element e +- d/2 lives in the lane LPH/2 away, same place
+    float other[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) other[i] = __shfl_xor(v[i], LPH / 2 > 0 ? LPH / 2 : 1, WAVE);
+    if (rotate && !is_v) {
+      const bool low = e0 < half;
+      const int j0 = low ? e0 : e0 - half;
+      const float* ct = cos_tab + (size_t)pos * half + j0;
+      const float* st = sin_tab + (size_t)pos * half + j0;
+      const float4 c0 = *reinterpret_cast<const float4*>(ct), c1 = *reinterpret_cast<const float4*>(ct + 4);
+      const float4 s0 = *reinterpret_cast<const float4*>(st), s1 = *reinterpret_cast<const float4*>(st + 4);
+      const float cv[8] = {c0.x, c0.y, c0.z, c0.w, c1.x, c1.y, c1.z, c1.w};
+      const float sv[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+        r[i] = low ? v[i] * cv[i] - other[i] * sv[i] : other[i] * sv[i] + v[i] * cv[i];
+    }
+  }
+  if (!active) return;
+  if (slot < H) {
+    qks_u32x4_t o;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) o[i] = pack_bf16x2(r[2 * i], r[2 * i + 1]);
+    *reinterpret_cast<qks_u32x4_t*>(src) = o;
+    return;
+  }
+  const int g = (slot - H) % G;
+  const int* bt = block_tables + (size_t)row_seg[t] * max_blocks;
+  const size_t pg = (size_t)bt[pos / ps] * G + g;
+  if (is_v) {
+    bf16_t* vdst = v_pool + (pg * d + e0) * ps + pos % ps;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      vdst[(size_t)(2 * i) * ps] = (bf16_t)(raw[i] & 0xffffu);
+      vdst[(size_t)(2 * i + 1) * ps] = (bf16_t)(raw[i] >> 16);
+    }
+    return;
+  }
+  qks_u32x4_t o;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) o[i] = pack_bf16x2(r[2 * i], r[2 * i + 1]);
+  *reinterpret_cast<qks_u32x4_t*>(k_pool + (pg * ps + pos % ps) * d + e0) = o;
 }
 
 extern "C" int kappai_qk_norm_rope_store(void* qkv, int row_stride, const float* q_norm_w,
@@ -78,17 +185,44 @@ extern "C" int kappai_qk_norm_rope_store(void* qkv, int row_stride, const float*
                                          int store_kv, int is_bf16, hipStream_t stream) {
   if (T <= 0) return 0;
   if (d > MAX_HEAD_DIM || d < 1 || rot_dim > d || (rot_dim & 1)) return (int)hipErrorInvalidValue;
-  dim3 grid(T, store_kv ? H + 2 * G : H);
+  const int n_slots = store_kv ? H + 2 * G : H;
+  const bool whole_rot = rot_mode == 0 || rot_dim == 0 || (rot_mode == 1 && rot_dim == d);
+  const int lph = d / 8;
+  if (is_bf16 && whole_rot && d % 8 == 0 && lph >= 2 && lph <= 64 && (lph & (lph - 1)) == 0 &&
+      row_stride % 8 == 0 && ((uintptr_t)qkv % 16) == 0 && ((uintptr_t)k_pool % 16) == 0 &&
+      ((uintptr_t)cos_tab % 16) == 0 && ((uintptr_t)sin_tab % 16) == 0 &&
+      (!q_norm_w || ((uintptr_t)q_norm_w % 16) == 0) &&
+      (!k_norm_w || ((uintptr_t)k_norm_w % 16) == 0)) {
+    const int rotate = rot_mode == 1 && rot_dim == d;
+    const long long total = (long long)T * n_slots * lph;
+    const dim3 gv((unsigned)((total + 255) / 256));
+#define QKS_LAUNCH(N)                                                                            \
+  hipLaunchKernelGGL(qk_norm_rope_store_vec_kernel<N>, gv, dim3(256), 0, stream, (bf16_t*)qkv,   \
+                     row_stride, q_norm_w, k_norm_w, eps, cos_tab, sin_tab, rotate,              \
+                     (bf16_t*)k_pool, (bf16_t*)v_pool, row_pos, row_seg, block_tables,           \
+                     max_blocks, T, H, G, ps, n_slots)
+    switch (lph) {
+      case 2: QKS_LAUNCH(2); break;
+      case 4: QKS_LAUNCH(4); break;
+      case 8: QKS_LAUNCH(8); break;
+      case 16: QKS_LAUNCH(16); break;
+      case 32: QKS_LAUNCH(32); break;
+      default: QKS_LAUNCH(64); break;
+    }
+#undef QKS_LAUNCH
+    KAPPAI_RETURN_LAUNCH_STATUS();
+  }
+  dim3 grid(T, (n_slots + QKS_SLOTS - 1) / QKS_SLOTS);
   if (is_bf16)
-    hipLaunchKernelGGL(qk_norm_rope_store_kernel<bf16_t>, grid, dim3(WAVE), 0, stream,
+    hipLaunchKernelGGL(qk_norm_rope_store_kernel<bf16_t>, grid, dim3(QKS_WAVES * WAVE), 0, stream,
                        (bf16_t*)qkv, row_stride, q_norm_w, k_norm_w, eps, cos_tab, sin_tab,
                        rot_dim, rot_mode, (bf16_t*)k_pool, (bf16_t*)v_pool, row_pos, row_seg,
-                       block_tables, max_blocks, H, G, d, ps, store_kv);
+                       block_tables, max_blocks, H, G, d, ps, n_slots);
   else
-    hipLaunchKernelGGL(qk_norm_rope_store_kernel<float>, grid, dim3(WAVE), 0, stream, (float*)qkv,
+    hipLaunchKernelGGL(qk_norm_rope_store_kernel<float>, grid, dim3(QKS_WAVES * WAVE), 0, stream, (float*)qkv,
                        row_stride, q_norm_w, k_norm_w, eps, cos_tab, sin_tab, rot_dim, rot_mode,
                        (float*)k_pool, (float*)v_pool, row_pos, row_seg, block_tables, max_blocks,
-                       H, G, d, ps, store_kv);
+                       H, G, d, ps, n_slots);
   KAPPAI_RETURN_LAUNCH_STATUS();
 }
 
