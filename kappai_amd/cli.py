@@ -52,8 +52,8 @@ def build_parser() -> argparse.ArgumentParser:
     e.add_argument("--page-size", type=int, default=16, help="tokens per cache page")
     e.add_argument("--num-pages", type=int, default=0, help="cache pages (0 = from free memory)")
     e.add_argument("--max-batch", type=int, default=64, help="requests live at the same time")
-    e.add_argument("--token-budget", type=int, default=512, help="tokens per step at most")
-    e.add_argument("--chunk", type=int, default=512, help="longest prompt portion in a step")
+    e.add_argument("--token-budget", type=int, default=2048, help="tokens per step at most")
+    e.add_argument("--chunk", type=int, default=2048, help="longest prompt portion in a step")
     e.add_argument("--random-weights", metavar="CONFIG.json", help="make a model folder with "
                    "random weights from this config.json and run it")
     e.add_argument("--weight-seed", type=int, default=0, help="seed of --random-weights")

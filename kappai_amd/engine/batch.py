@@ -70,6 +70,7 @@ def layout_rows(entries: Sequence[StepEntry], cache: CacheManager, vocab_size: i
     seen = set()
     tokens, row_pos, row_seg, seg_start, seg_pos0, seg_slot, logit_rows = [], [], [], [0], [], [], []
     q_tiles = []
+    max_position = 0
     for si, e in enumerate(entries):
         n = len(e.tokens)
         if n < 1:
@@ -77,19 +78,21 @@ def layout_rows(entries: Sequence[StepEntry], cache: CacheManager, vocab_size: i
         if id(e.cache) in seen:
             raise ValueError(f"request {e.cache.request_id!r} appears twice in one step")
         seen.add(id(e.cache))
-        for t in e.tokens:
-            if not 0 <= int(t) < vocab_size:
-                raise ValueError(f"entry {si} ({e.cache.request_id!r}): token id {t} is outside "
-                                 f"the vocabulary of {vocab_size}")
+        toks = np.asarray(e.tokens, dtype=np.int64)
+        if toks.ndim != 1 or int(toks.min()) < 0 or int(toks.max()) >= vocab_size:
+            bad = next(int(t) for t in toks.reshape(-1) if not 0 <= int(t) < vocab_size)
+            raise ValueError(f"entry {si} ({e.cache.request_id!r}): token id {bad} is outside "
+                             f"the vocabulary of {vocab_size}")
         for w in e.want:
             if not 0 <= int(w) < n:
                 raise ValueError(f"entry {si} ({e.cache.request_id!r}): wanted place {w} is "
                                  f"outside its {n} tokens")
         base = seg_start[-1]
         p0 = e.cache.length
-        tokens.extend(int(t) for t in e.tokens)
-        row_pos.extend(range(p0, p0 + n))
-        row_seg.extend([si] * n)
+        tokens.append(toks.astype(np.int32))
+        row_pos.append(np.arange(p0, p0 + n, dtype=np.int32))
+        row_seg.append(np.full(n, si, dtype=np.int32))
+        max_position = max(max_position, p0 + n - 1)
         seg_start.append(base + n)
         n_seg_tiles = (n + ATTENTION_TILE_ROWS - 1) // ATTENTION_TILE_ROWS
         for j, r in enumerate(range(0, n, ATTENTION_TILE_ROWS)):
@@ -110,9 +113,9 @@ def layout_rows(entries: Sequence[StepEntry], cache: CacheManager, vocab_size: i
             bt[si, :len(b)] = b
         tables.append(bt)
     arrays = {
-        "tokens": np.asarray(tokens, dtype=np.int32),
-        "row_pos": np.asarray(row_pos, dtype=np.int32),
-        "row_seg": np.asarray(row_seg, dtype=np.int32),
+        "tokens": np.concatenate(tokens),
+        "row_pos": np.concatenate(row_pos),
+        "row_seg": np.concatenate(row_seg),
         "seg_start": np.asarray(seg_start, dtype=np.int32),
         "seg_pos0": np.asarray(seg_pos0, dtype=np.int32),
         "seg_slot": np.asarray(seg_slot, dtype=np.int32),
@@ -122,8 +125,8 @@ def layout_rows(entries: Sequence[StepEntry], cache: CacheManager, vocab_size: i
     for gi, bt in enumerate(tables):
         arrays[f"block_table_{gi}"] = bt
     sizes = {
-        "n_rows": len(tokens), "n_segments": S, "n_logit_rows": len(logit_rows),
-        "max_position": max(row_pos),
+        "n_rows": seg_start[-1], "n_segments": S, "n_logit_rows": len(logit_rows),
+        "max_position": max_position,
         "max_segment_rows": max(len(e.tokens) for e in entries),
         "n_groups": len(tables),
     }

@@ -34,8 +34,8 @@ class EngineConfig:
     num_pages: int = 0                   # 0: from free memory
     memory_fraction: float = 0.8         # share of free GPU memory for pages when num_pages = 0
     max_batch: int = 64                  # requests live at the same time (state slots)
-    token_budget: int = 512
-    chunk: int = 512
+    token_budget: int = 2048
+    chunk: int = 2048
 
 
 @dataclass
