@@ -169,3 +169,38 @@ def test_decode_graphs_replay_what_eager_steps_compute(tmp_path, model_dirs, dty
         assert (a is None) == (b is None)
         if a is not None:
             assert np.array_equal(a, b)
+
+
+# A wider configuration with a long prompt, so that the kernels for large steps run inside the
+# engine: the 128 x 128 / 256 x 256 block products (K a multiple of 128, more than 64 rows) and
+# the prefill attention that shares key tiles between four heads of a kv head (head size 64,
+# 66 q tiles x 4 head quads).
+WIDE = {
+    "architectures": ["Lfm2ForCausalLM"], "model_type": "lfm2",
+    "hidden_size": 1024, "num_hidden_layers": 4,
+    "layer_types": ["conv", "full_attention", "conv", "full_attention"],
+    "num_attention_heads": 16, "num_key_value_heads": 4, "head_dim": 64,
+    "intermediate_size": 2688, "block_auto_adjust_ff_dim": False,
+    "vocab_size": 2048, "norm_eps": 1e-5, "rope_theta": 1000000.0,
+    "conv_L_cache": 3, "conv_bias": False, "tie_embedding": True,
+    "max_position_embeddings": 8192,
+}
+
+
+@pytest.mark.parametrize("dtype", ["bfloat16", "float32"])
+def test_long_prompt_on_a_wide_model(tmp_path, dtype):
+    import copy
+    from kappai_amd.config import config_from_dict
+    from kappai_amd.weights import write_random_model
+    folder = write_random_model(tmp_path / "wide", config_from_dict(copy.deepcopy(WIDE)), seed=5,
+                                std=0.02, norm_jitter=0.05)
+    requests = make_requests(WIDE["vocab_size"], [2200, 300], seed=15)
+    # r0: 66 q tiles in one step, a short portion, then token by token; r1 beside it, cut in two
+    plans = {"r0": (0, [2112, 56] + [1] * 32), "r1": (1, [200, 100])}
+    steps, index, peak = schedules.build(requests, plans)
+    got = replay_in_process(folder, dtype, steps, index, peak, tmp_path / "out")
+    ref = plain_logits(folder, requests)
+    tol = tolerance(folder, requests, dtype)
+    assert len(got) == 2500
+    err, where = worst_error(got, ref)
+    assert err < tol, (err, tol, where, first_bad(got, ref, tol))
