@@ -349,7 +349,8 @@ __global__ __launch_bounds__(P_NW * WAVE) void attn_prefill_kernel(
 // (d x 32 keys) is brought from global memory once, straight into LDS (global_load_lds, three
 // buffers, two tiles ahead), and every wave reads its matrix operands from there.  Pairing an
 // early q tile with a late one gives every block the same number of keys to walk.  K rows keep their 16-byte chunks permuted (chunk ^ f(key)) so that the
-// 16 keys of a fragment read fall on different banks; V^T lies as [16-key group][d][16 keys].
+// 16 keys of a fragment read fall on different banks; V^T lies as [16-key group][d][16 keys],
+// every other 8 rows with their two halves of 8 keys swapped, for the same reason.
 // The running maximum is only moved when a tile's maximum exceeds it by more than 2^8: most
 // tiles then leave the output accumulators alone (no rescaling), and the weights stay <= 256.
 #if HEAD_DIM == 64 || HEAD_DIM == 128
@@ -480,8 +481,10 @@ __global__ __launch_bounds__(8 * WAVE) void attn_prefill_shared_kernel(
 #pragma unroll
       for (int i = 0; i < NL; ++i) {
         const int dd = v_d0 + 32 * i;
+        // rows 8 apart would meet on the same banks: every other group of 8 rows keeps its two
+        // 16-byte halves swapped
         __builtin_amdgcn_global_load_lds(
-            PG_GPTR(base + (size_t)dd * ps + 8 * v_half),
+            PG_GPTR(base + (size_t)dd * ps + 8 * (v_half ^ ((dd >> 3) & 1))),
             PG_LPTR(buf + KTILE + v_st * VGROUP + ((vw % 2) * (HEAD_DIM / 2) + 32 * i) * 32), 16, 0,
             0);
       }
@@ -520,9 +523,10 @@ __global__ __launch_bounds__(8 * WAVE) void attn_prefill_shared_kernel(
     for (int st = 0; st < 2; ++st)
 #pragma unroll
       for (int mt = 0; mt < P_MT; ++mt) {
+        const int sw = ((col >> 3) & 1) * 16;      // this row's halves are swapped
         const char* vp = buf + KTILE + st * VGROUP + (32 * mt + col) * 32 + 8 * hh;
-        va[st][mt] = *reinterpret_cast<const u32x2_t*>(vp);
-        vb[st][mt] = *reinterpret_cast<const u32x2_t*>(vp + 16);
+        va[st][mt] = *reinterpret_cast<const u32x2_t*>(vp + sw);
+        vb[st][mt] = *reinterpret_cast<const u32x2_t*>(vp + (16 - sw));
       }
     // lane holds, for query `col`, keys kb + 8*(v/4) + 4*hh + v%4
     float mloc = -INFINITY;
