@@ -4,9 +4,12 @@
 //
 //   gemm_f32         true 32-bit on the vector ALUs: every product and sum is an fp32 FMA in
 //                    the order k = 0..K-1, so a row's result does not depend on M.
-//   gemm_bf16_tile   bf16 inputs, fp32 accumulation on the matrix cores
-//                    (v_mfma_f32_32x32x16_bf16), 128x128x32 block tiles staged through LDS.
-//   gemm_bf16_skinny M <= 64 (decode): every block streams 16 rows of W once, its 4 to 16
+//   gemm_bf16_block256  large products (K a multiple of 128 per K range): bf16 inputs, fp32
+//                    accumulation on the matrix cores (v_mfma_f32_32x32x16_bf16), 256x256 or
+//                    128x128 blocks, tiles of 64 of K loaded straight into LDS.
+//   gemm_bf16_tile   any K that is a multiple of 8: 256x128 or 128x128 blocks staged through
+//                    registers into LDS.
+//   gemm_bf16_skinny M <= 64 (decode): every block streams 16 or 32 rows of W once, its 4 to 16
 //                    waves split K and meet in LDS (v_mfma_f32_16x16x32_bf16).
 #include "common.h"
 
