@@ -167,7 +167,7 @@ class Engine:
         t0 = time.perf_counter()          # the last step ended with a synchronisation
         step_entries = []
         for e in entries:
-            toks = e.request.tokens[e.request.computed:e.request.computed + e.n_tokens]
+            toks = e.request.tokens_from(e.request.computed, e.n_tokens)
             step_entries.append(StepEntry(e.request.cache, toks,
                                           [e.n_tokens - 1] if e.samples else []))
         logits = self.runner.step(step_entries)

@@ -47,6 +47,15 @@ class Request:
     def tokens(self) -> List[int]:
         return self.prompt + self.output
 
+    def tokens_from(self, start: int, n: int) -> List[int]:
+        """``tokens[start:start + n]`` without putting prompt and output together first."""
+        p = len(self.prompt)
+        if start >= p:
+            return self.output[start - p:start - p + n]
+        if start + n <= p:
+            return self.prompt[start:start + n]
+        return self.prompt[start:] + self.output[:start + n - p]
+
     @property
     def pending(self) -> int:
         return len(self.prompt) + len(self.output) - self.computed
