@@ -20,7 +20,13 @@ MAX_GRID_Y = 65535
 _c_int, _c_float, _c_long, _vp = ctypes.c_int, ctypes.c_float, ctypes.c_long, ctypes.c_void_p
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream() -> _vp:
+    """The current stream of the current device, as the handle the kernels' launchers take."""
+    if _raw_stream is not None:         # the same value without building a Stream object
+        return _vp(_raw_stream(torch.cuda.current_device()))
     return _vp(torch.cuda.current_stream().cuda_stream)
 
 
