@@ -802,7 +802,11 @@ static int launch_bf16(const bf16_t* A, const bf16_t* W, const float* bias, TO* 
                        int K, int lda, int ldc, int force_kernel, int ksplit, hipStream_t stream,
                        ConvStep cs = ConvStep{}) {
   // N counts output columns; with the SwiGLU epilogue W has 2N rows
-  if (M <= 64 && force_kernel != 1 && force_kernel < 3) {
+  // a very wide plain product (the output head) with more than 32 rows streams faster through
+  // the 128 x 128 blocks than through the decode kernel, which reads the rows once per 32 columns
+  const bool wide_head = EPI == 0 && M > 32 && N >= 16384 && force_kernel == 0 && ksplit == 1 &&
+                         block256_fits<TO, EPI>(A, W, C, M, N, K, lda, ldc, ksplit);
+  if (M <= 64 && force_kernel != 1 && force_kernel < 3 && !wide_head) {
     const int mt = (M + 15) / 16;
     switch (mt) {
       case 1:
@@ -821,7 +825,8 @@ static int launch_bf16(const bf16_t* A, const bf16_t* W, const float* bias, TO* 
   } else {
     // rows of W = columns the tiles run over
     launch_tile<TO, EPI>(A, W, bias, C, M, EPI == 1 ? 2 * N : N, K, lda, ldc, ksplit,
-                         force_kernel >= 3 ? force_kernel - 2 : 0, stream);
+                         force_kernel >= 3 ? force_kernel - 2 : (wide_head && M <= 64 ? 6 : 0),
+                         stream);
   }
   KAPPAI_RETURN_LAUNCH_STATUS();
 }

@@ -111,6 +111,7 @@ def test_linear_float32_is_not_reduced_precision(ops):
 
 
 @pytest.mark.parametrize("M,N,K", GEMM_SHAPES + [(33, 130, 72), (48, 6144, 2048), (128, 128, 32),
+                                                 (40, 16392, 256), (64, 16384, 128), (32, 16384, 128),
                                                  (513, 640, 264), (2048, 3200, 96),
                                                  (1999, 3330, 40)])
 @pytest.mark.parametrize("out_dtype", [F32, BF16])
