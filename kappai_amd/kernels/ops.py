@@ -16,6 +16,7 @@ from .lib import check, library
 F32, BF16, I32 = torch.float32, torch.bfloat16, torch.int32
 MAX_HEAD_DIM = 512
 MAX_GRID_Y = 65535
+DECODE_WAVES = 2048       # waves the split-key decode attention aims to have at work
 
 _c_int, _c_float, _c_long, _vp = ctypes.c_int, ctypes.c_float, ctypes.c_long, ctypes.c_void_p
 
@@ -438,7 +439,9 @@ def paged_attention(q: torch.Tensor, n_heads: int, n_kv_heads: int, head_dim: in
     # one wave keeps the loads of `kpw` keys in flight; splits are whole numbers of that, and
     # at most 64 of them are merged
     kpw = lib.kappai_attn_keys_per_wave()
-    n_splits = max(1, min(64, (n_keys + kpw - 1) // kpw))
+    # and no more splits than it takes to have DECODE_WAVES waves at work: with many rows a
+    # wave rather takes several chunks in turn than writes a partial result for each
+    n_splits = max(1, min(64, (n_keys + kpw - 1) // kpw, max(1, DECODE_WAVES // (T * G))))
     keys_per_split = ((n_keys + n_splits - 1) // n_splits + kpw - 1) // kpw * kpw
     n_splits = (n_keys + keys_per_split - 1) // keys_per_split
     part_o = torch.empty((T, H, n_splits, d), dtype=F32, device=q.device)
