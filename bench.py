@@ -104,13 +104,30 @@ class DecodeBench:
         logits = self.runner.step(entries)
         self.tokens = ops.sample_rows(logits, self.temp, self.uni).tolist()
 
-    def run(self, warmup, steps):
+    def _choose(self, logits, step, out_row):
+        from kappai_amd.kernels import ops
+        ops.sample_rows(logits, self.temp, self.uni, out=out_row)
+
+    def run(self, warmup, steps, run_len=8):
+        """``steps`` decode steps, taken the way the engine takes them when nothing but decoding
+        is going on: up to ``run_len`` steps queued back to back, each step's token handed to the
+        next on the GPU, the host reading the tokens at the end of the run."""
         for _ in range(warmup):
             self.step()
         sync()
         t0 = time.perf_counter()
-        for _ in range(steps):
-            self.step()
+        left = steps
+        while left > 0:
+            n = min(run_len, left)
+            out = None
+            if n > 1:
+                out = self.runner.decode_run(self.requests, self.tokens, n, self._choose)
+            if out is None:
+                self.step()
+                left -= 1
+            else:
+                self.tokens = out[-1].tolist()
+                left -= n
         sync()
         return time.perf_counter() - t0
 

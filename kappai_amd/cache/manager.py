@@ -270,6 +270,15 @@ class CacheManager:
                 return False
         return True
 
+    def can_extend_all(self, caches: Sequence[RequestCache], n_new: int) -> bool:
+        """True if every one of ``caches`` can grow by ``n_new`` tokens at the same time (pages
+        that a window would give back meanwhile are not counted on)."""
+        total = [0] * len(self.paged_groups)
+        for rc in caches:
+            for gi, need in enumerate(self.pages_needed(rc, n_new)):
+                total[gi] += need
+        return all(total[gi] <= g.allocator.num_free for gi, g in enumerate(self.paged_groups))
+
     def extend(self, rc: RequestCache, n_new: int) -> None:
         """Make room for tokens ``length .. length + n_new - 1`` in every paged group.
         Either every group gets its pages or nothing changes."""

@@ -121,7 +121,9 @@ def main(argv=None) -> int:
     engine = Engine(EngineConfig(
         model=model_dir, dtype=args.dtype, ctx_size=args.ctx_size, page_size=args.page_size,
         num_pages=args.num_pages, max_batch=args.max_batch, token_budget=args.token_budget,
-        chunk=args.chunk))
+        chunk=args.chunk,
+        # per-step output (logits, timing) needs every step waited for
+        decode_run=1 if (args.debug_forward or args.dump_logits or args.time) else 8))
     params = SamplingParams(
         temperature=args.temperature, top_k=args.top_k, top_p=args.top_p, min_p=args.min_p,
         repeat_penalty=args.repeat_penalty, repeat_last_n=args.repeat_last_n, seed=args.seed,

@@ -18,7 +18,7 @@ from ..cache.manager import CacheManager
 from ..models import Model, load_model
 from ..sampling import RequestSampler, Sampler, SamplingParams
 from .batch import StepEntry
-from .scheduler import FAILED, FINISHED, Request, Scheduler, SchedulerConfig
+from .scheduler import FAILED, FINISHED, RUNNING, Request, Scheduler, SchedulerConfig
 from .step import StepRunner
 
 
@@ -36,6 +36,8 @@ class EngineConfig:
     max_batch: int = 64                  # requests live at the same time (state slots)
     token_budget: int = 2048
     chunk: int = 2048
+    decode_run: int = 8                  # decode steps queued back to back when nothing but
+                                         # decoding is going on (1: every step is waited for)
 
 
 @dataclass
@@ -164,6 +166,9 @@ class Engine:
             outputs.append(StepOutput(req.request_id, None, True, req.finish_reason))
         if not entries:
             return outputs
+        run = self._decode_run(entries)
+        if run is not None:
+            return outputs + run
         t0 = time.perf_counter()          # the last step ended with a synchronisation
         step_entries = []
         for e in entries:
@@ -195,6 +200,49 @@ class Engine:
             req.sampler.observe([tok])
             done = self.scheduler.append_token(req, tok)
             outputs.append(StepOutput(req.request_id, tok, done, req.finish_reason))
+        return outputs
+
+    def _decode_run(self, entries) -> Optional[List[StepOutput]]:
+        """When every entry is one decoded token, run several steps back to back: each step's
+        token goes to the next on the GPU and the host reads them all at the end.  A request
+        that meets its end-of-sequence token inside the run has run a few steps too many; they
+        are dropped with its cache.  Returns None when the steps have to be taken one by one."""
+        n = self.config.decode_run
+        if n < 2 or any(e.n_tokens != 1 or not e.samples for e in entries):
+            return None
+        reqs = [e.request for e in entries]
+        for r in reqs:       # nobody may pass its own limits inside the run
+            if r.params.n_predict >= 0:
+                n = min(n, r.params.n_predict - len(r.output))
+            n = min(n, self.scheduler.max_context - (len(r.prompt) + len(r.output)))
+        samplers = [r.sampler for r in reqs]
+        if n < 2 or not Sampler.runs_on_device(samplers, self.model.vocab_size):
+            return None
+        first = [r.tokens_from(r.computed, 1)[0] for r in reqs]
+
+        def choose(logits, step, out_row):
+            self.sampler.launch(logits, samplers, out=out_row)
+
+        t0 = time.perf_counter()
+        tokens = self.runner.decode_run([r.cache for r in reqs], first, n, choose)
+        if tokens is None:
+            return None
+        self.last_logits = None
+        rows = tokens.tolist()            # waits for the run
+        dt = time.perf_counter() - t0
+        m = self.metrics
+        m.steps += n
+        m.decode_tokens += n * len(reqs)
+        m.decode_seconds += dt
+        outputs: List[StepOutput] = []
+        for row in rows:
+            for req, tok in zip(reqs, row):
+                if req.state != RUNNING:
+                    continue              # ended earlier in the run
+                req.computed += 1
+                req.sampler.observe([tok])
+                done = self.scheduler.append_token(req, tok)
+                outputs.append(StepOutput(req.request_id, tok, done, req.finish_reason))
         return outputs
 
     # -- convenience ---------------------------------------------------------------------------

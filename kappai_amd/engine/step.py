@@ -15,12 +15,13 @@ from typing import List, Optional, Sequence
 import numpy as np
 import torch
 
-from ..cache.manager import CacheManager, OutOfPages
+from ..cache.manager import CacheManager, OutOfPages, RequestCache
 from ..models.base import Model
 from .batch import RowBatch, StepEntry, layout_rows
 
 
 CONTEXT_BUCKET_MIN = 1024     # decode graphs are captured for contexts up to a power of two
+DECODE_RING = 8            # decode steps whose tables can be queued ahead of the GPU
 MAX_DECODE_GRAPHS = 48
 
 
@@ -78,6 +79,9 @@ class _DecodeGraph:
         for g in range(n_groups):
             self.h[f"block_table_{g}"][:] = cache.scratch_page(g)
         self.rows_of = [None] * B        # (request cache, version) whose pages row si mirrors
+        self._ring: List[Optional[torch.Tensor]] = [None] * DECODE_RING
+        self._ring_done: List[Optional[torch.cuda.Event]] = [None] * DECODE_RING
+        self._ring_at = 0
         self._upload(runner)
         runner.model.forward(self.batch, cache)
         torch.cuda.synchronize(dev)
@@ -86,14 +90,26 @@ class _DecodeGraph:
             self.logits = runner.model.forward(self.batch, cache)
 
     def _upload(self, runner: "StepRunner") -> None:
-        host = runner._stage(self.total)
-        host[:self.total] = self.mirror
-        self.static.copy_(runner._staging[:self.total], non_blocking=True)
-        runner._mark_staged()
+        """The mirror to the device through the next pinned buffer of the graph's ring, so that
+        several steps can be queued before the first of them has run."""
+        i = self._ring_at
+        self._ring_at = (i + 1) % len(self._ring)
+        if self._ring_done[i] is not None:
+            self._ring_done[i].synchronize()
+        if self._ring[i] is None:
+            self._ring[i] = torch.empty(self.total, dtype=torch.int32, pin_memory=True)
+        self._ring[i].numpy()[:] = self.mirror
+        self.static.copy_(self._ring[i], non_blocking=True)
+        ev = self._ring_done[i] = torch.cuda.Event()
+        ev.record()
 
-    def run(self, runner: "StepRunner", caches, tokens, pos, slots, logit_rows) -> torch.Tensor:
+    def run(self, runner: "StepRunner", caches, tokens, pos, slots, logit_rows,
+            device_tokens: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """``tokens`` from the host, or ``device_tokens`` (int32 [B] on the GPU, e.g. what the last
+        step's sampling kernel wrote) copied into place on the GPU."""
         h = self.h
-        h["tokens"][:] = tokens
+        if device_tokens is None:
+            h["tokens"][:] = tokens
         h["row_pos"][:] = pos
         h["seg_pos0"][:] = pos
         h["seg_slot"][:] = slots
@@ -108,6 +124,8 @@ class _DecodeGraph:
                     row[len(b):] = -1
                 self.rows_of[si] = (rc, rc.version)
         self._upload(runner)
+        if device_tokens is not None:
+            self.batch.tokens.copy_(device_tokens)
         self.graph.replay()
         return self.logits
 
@@ -213,6 +231,44 @@ class StepRunner:
         slots = np.fromiter((c.slot for c in caches), dtype=np.int32, count=B)
         self.graph_replays += 1
         return graph.run(self, caches, tokens, pos, slots, logit_rows)
+
+    def decode_run(self, caches: Sequence[RequestCache], first_tokens: Sequence[int], n_steps: int,
+                   choose, out: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+        """``n_steps`` decode steps of the same requests, queued back to back: the token a step
+        chooses goes to the next step on the GPU, and the host does not wait in between.
+        ``choose(logits, step, out_row)`` queues the kernels that write one token per request
+        (int32) into ``out_row``.  Returns the tokens [n_steps, B] on the GPU (not yet waited
+        for), or None when the run cannot be made this way (no captured graph for the shape
+        yet, not enough pages for all the steps): then nothing has changed.  After the run
+        every cache holds ``n_steps`` more tokens."""
+        B = len(caches)
+        if not self.decode_graphs or B == 0 or n_steps < 1 or n_steps > DECODE_RING:
+            return None
+        if len({id(c) for c in caches}) != B:
+            return None
+        ctx_cap = _context_bucket(max(c.length for c in caches) + n_steps)
+        graph = self._graphs.get((B, B, ctx_cap))
+        if graph is None or not self.cache.can_extend_all(caches, n_steps):
+            return None
+        tokens = np.asarray(first_tokens, dtype=np.int64)
+        if tokens.shape != (B,) or tokens.min() < 0 or tokens.max() >= self.model.vocab_size:
+            return None
+        if out is None:
+            out = torch.empty((n_steps, B), dtype=torch.int32, device=self.device)
+        slots = np.fromiter((c.slot for c in caches), dtype=np.int32, count=B)
+        rows = list(range(B))
+        for s in range(n_steps):
+            for c in caches:
+                self.cache.extend_one(c)
+            pos = np.fromiter((c.length for c in caches), dtype=np.int32, count=B)
+            logits = graph.run(self, caches, tokens, pos, slots, rows,
+                               device_tokens=None if s == 0 else out[s - 1])
+            for c in caches:
+                self.cache.commit_one(c)
+            choose(logits, s, out[s])
+            self.graph_replays += 1
+            self.steps_run += 1
+        return out
 
     # -- one step ----------------------------------------------------------------------------
     def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:

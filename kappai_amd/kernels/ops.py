@@ -456,17 +456,21 @@ def paged_attention(q: torch.Tensor, n_heads: int, n_kv_heads: int, head_dim: in
 
 
 # ---------------------------------------------------------------------------------------
-def sample_rows(logits: torch.Tensor, temperature: torch.Tensor,
-                uniform: torch.Tensor) -> torch.Tensor:
+def sample_rows(logits: torch.Tensor, temperature: torch.Tensor, uniform: torch.Tensor,
+                out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """One token per row of ``logits`` [n, V] (float32): argmax (lowest id on ties) where the
     row's temperature is <= 0, else an inverse-CDF draw of softmax(logits / T) at the row's
-    uniform number."""
+    uniform number.  ``out`` (int32 [n]) receives the tokens when given."""
     _gpu("logits", logits, F32)
     _gpu("temperature", temperature, F32)
     _gpu("uniform", uniform, F32)
     n, V = logits.shape
     _need(temperature.shape == (n,) and uniform.shape == (n,), "one temperature and uniform a row")
-    out = torch.empty((n,), dtype=I32, device=logits.device)
+    if out is None:
+        out = torch.empty((n,), dtype=I32, device=logits.device)
+    else:
+        _gpu("out", out, I32)
+        _need(out.shape == (n,), "sample_rows: out must hold one token a row")
     check(library("sampling").kappai_sample_rows(
         _ptr(logits), _ptr(temperature), _ptr(uniform), _ptr(out), _c_int(n), _c_int(V),
         _stream()), "sample_rows")

@@ -85,28 +85,51 @@ class Sampler:
     """Samples one token for each row of ``logits`` [n, vocab] (float32, on the GPU; changed
     in place where a repeat penalty applies)."""
 
+    RING = 8      # pinned buffers for the per-row numbers of steps that are queued ahead
+
     def __init__(self):
         self._zeros = {}      # (rows, device) -> zero temperature / uniform tensors (all greedy)
+        self._pinned: List[Optional[torch.Tensor]] = [None] * self.RING
+        self._pinned_done: List[Optional[torch.cuda.Event]] = [None] * self.RING
+        self._ring_at = 0
 
-    def sample(self, logits: torch.Tensor, samplers: Sequence[RequestSampler]) -> List[int]:
+    def _to_device(self, packed: np.ndarray, dev) -> torch.Tensor:
+        """``packed`` (float32) on the GPU through a pinned buffer, without waiting for the GPU."""
+        i = self._ring_at
+        self._ring_at = (i + 1) % self.RING
+        if self._pinned_done[i] is not None:
+            self._pinned_done[i].synchronize()
+        buf = self._pinned[i]
+        if buf is None or buf.numel() < packed.size:
+            buf = self._pinned[i] = torch.empty(max(2 * packed.size, 1024), dtype=torch.float32,
+                                                pin_memory=True)
+        buf.numpy()[:packed.size] = packed
+        d = torch.empty(packed.size, dtype=torch.float32, device=dev)
+        d.copy_(buf[:packed.size], non_blocking=True)
+        ev = self._pinned_done[i] = torch.cuda.Event()
+        ev.record()
+        return d
+
+    @staticmethod
+    def runs_on_device(samplers: Sequence[RequestSampler], vocab: int) -> bool:
+        """True when every row's token can be chosen without the host seeing the logits or the
+        row's earlier tokens: no repeat penalty, no narrowing beyond what the kernel holds."""
+        for s in samplers:
+            p = s.params
+            if p.repeat_penalty != 1.0:
+                return False
+            if not p.is_greedy() and p.is_filtered(vocab):
+                keep = p.top_k if 0 < p.top_k < vocab else min(vocab, FILTER_CAP)
+                if keep > ops.FILTER_MAX_KEEP:
+                    return False
+        return True
+
+    def launch(self, logits: torch.Tensor, samplers: Sequence[RequestSampler],
+               out: Optional[torch.Tensor] = None):
+        """Queue the kernels that choose a token for every row; returns (int32 tokens on the GPU,
+        rows that the host still has to draw).  Nothing here waits for the GPU."""
         n, vocab = logits.shape
-        if n != len(samplers):
-            raise ValueError(f"{n} rows of logits for {len(samplers)} requests")
-        if n == 0:
-            return []
         dev = logits.device
-        # repeat penalty: one scatter over all rows that ask for it
-        if any(s.params.repeat_penalty != 1.0 and s.recent for s in samplers):
-            starts, toks, pens = [0], [], []
-            for s in samplers:
-                if s.params.repeat_penalty != 1.0:
-                    toks.extend(s.penalty_window())
-                starts.append(len(toks))
-                pens.append(float(s.params.repeat_penalty))
-            ops.repeat_penalty(
-                logits, torch.tensor(starts, dtype=torch.int32, device=dev),
-                torch.tensor(toks or [0], dtype=torch.int32, device=dev),
-                torch.tensor(pens, dtype=torch.float32, device=dev))
         temps, unis, host_rows, filt = [], [], [], []
         for i, s in enumerate(samplers):
             p = s.params
@@ -129,7 +152,7 @@ class Sampler:
         # rows, then [row | keep | temperature | top_p | min_p | uniform] for the narrowed ones
         m = len(filt)
         if not any(temps) and not m and (n, str(dev)) in self._zeros:
-            out_dev = ops.sample_rows(logits, *self._zeros[(n, str(dev))])
+            out_dev = ops.sample_rows(logits, *self._zeros[(n, str(dev))], out=out)
         else:
             packed = np.zeros(2 * n + 6 * m, dtype=np.float32)
             packed[:n] = temps
@@ -141,15 +164,37 @@ class Sampler:
                 ints[m:] = cols[1]
                 for j in range(4):
                     packed[2 * n + (2 + j) * m:2 * n + (3 + j) * m] = cols[2 + j]
-            d = torch.from_numpy(packed).to(dev)
+            d = self._to_device(packed, dev)
             if not any(temps) and not m:
                 self._zeros[(n, str(dev))] = (d[:n], d[n:2 * n])
-            out_dev = ops.sample_rows(logits, d[:n], d[n:2 * n])
+            out_dev = ops.sample_rows(logits, d[:n], d[n:2 * n], out=out)
             if m:
                 di = d[2 * n:2 * n + 2 * m].view(torch.int32)
                 f = d[2 * n + 2 * m:]
                 ops.sample_filtered(logits, di[:m], di[m:], f[:m], f[m:2 * m], f[2 * m:3 * m],
                                     f[3 * m:4 * m], out_dev)
+        return out_dev, host_rows
+
+    def sample(self, logits: torch.Tensor, samplers: Sequence[RequestSampler]) -> List[int]:
+        n, vocab = logits.shape
+        if n != len(samplers):
+            raise ValueError(f"{n} rows of logits for {len(samplers)} requests")
+        if n == 0:
+            return []
+        dev = logits.device
+        # repeat penalty: one scatter over all rows that ask for it
+        if any(s.params.repeat_penalty != 1.0 and s.recent for s in samplers):
+            starts, toks, pens = [0], [], []
+            for s in samplers:
+                if s.params.repeat_penalty != 1.0:
+                    toks.extend(s.penalty_window())
+                starts.append(len(toks))
+                pens.append(float(s.params.repeat_penalty))
+            ops.repeat_penalty(
+                logits, torch.tensor(starts, dtype=torch.int32, device=dev),
+                torch.tensor(toks or [0], dtype=torch.int32, device=dev),
+                torch.tensor(pens, dtype=torch.float32, device=dev))
+        out_dev, host_rows = self.launch(logits, samplers)
         out = out_dev.tolist()
         if host_rows:
             rows = logits[torch.tensor(host_rows, device=dev)].cpu().numpy()

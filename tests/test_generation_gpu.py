@@ -156,3 +156,66 @@ def test_smoke_entry():
     sys.path.insert(0, str(ROOT))
     import __graft_entry__
     __graft_entry__.smoke()
+
+
+def _engine(model_dir, dtype, **kw):
+    from kappai_amd.engine import Engine, EngineConfig
+    return Engine(EngineConfig(model=str(model_dir), dtype=dtype, num_pages=256, max_batch=8, **kw))
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_decode_runs_give_the_same_tokens(model_dirs, dtype):
+    """Several decode steps queued back to back (each step's token handed to the next on the
+    GPU) must give exactly the tokens of steps that are waited for one by one: greedy and
+    sampled requests side by side, ending at different lengths, inside and at the end of runs."""
+    from kappai_amd.sampling import SamplingParams
+    prompts = prompts_for("B", [9, 30, 4, 17, 11], seed=21)
+    params = [SamplingParams.greedy(n_predict=41), SamplingParams.greedy(n_predict=23),
+              SamplingParams(temperature=0.9, top_k=0, top_p=1.0, min_p=0.0, seed=5, n_predict=36),
+              SamplingParams(temperature=0.7, top_k=12, top_p=0.9, min_p=0.05, seed=6, n_predict=29),
+              SamplingParams.greedy(n_predict=2)]
+    results = {}
+    for run_len in (1, 8, 3):
+        eng = _engine(model_dirs["B"], dtype, decode_run=run_len)
+        results[run_len] = eng.generate(prompts, params)
+        eng.cache.check()
+        assert eng.cache.num_free_pages() == 256 and eng.cache.num_free_slots == 8
+        if run_len > 1:
+            assert eng.runner.graph_replays > 20
+        assert [len(o) for o in results[run_len]] == [41, 23, 36, 29, 2]
+    assert results[8] == results[1]
+    assert results[3] == results[1]
+
+
+def test_end_of_sequence_inside_a_decode_run(model_dirs, tmp_path):
+    """A request that draws its end-of-sequence token in the middle of a run ends there: the
+    tokens of the steps that were queued behind it are dropped, its pages and its slot come
+    back, and the other requests are not disturbed."""
+    from kappai_amd.sampling import SamplingParams
+    prompts = prompts_for("B", [6, 13, 8], seed=22)
+    params = [SamplingParams(temperature=1.0, top_k=0, top_p=1.0, min_p=0.0, seed=40 + i,
+                             n_predict=40) for i in range(3)]
+    eng = _engine(model_dirs["B"], "float32", decode_run=1)
+    free = eng.generate(prompts, params)
+    # a token that request 0 draws late enough to fall inside a run, and that nobody drew before
+    pick = None
+    for k in range(12, 40):
+        t = free[0][k]
+        if t not in free[0][:k] and all(t not in o for o in free[1:]):
+            pick = (k, t)
+            break
+    assert pick is not None, "the chains share all their tokens"
+    k, eos = pick
+    cfg = json.loads((model_dirs["B"] / "config.json").read_text())
+    cfg["eos_token_id"] = eos
+    folder = tmp_path / "with_eos"
+    folder.mkdir()
+    (folder / "config.json").write_text(json.dumps(cfg))
+    (folder / "model.safetensors").write_bytes((model_dirs["B"] / "model.safetensors").read_bytes())
+    for run_len in (1, 8):
+        eng = _engine(folder, "float32", decode_run=run_len)
+        got = eng.generate(prompts, params)
+        assert got[0] == free[0][:k + 1] and got[0][-1] == eos
+        assert got[1] == free[1] and got[2] == free[2]
+        eng.cache.check()
+        assert eng.cache.num_free_pages() == 256 and eng.cache.num_free_slots == 8
