@@ -11,6 +11,8 @@
 //                    registers into LDS.
 //   gemm_bf16_skinny M <= 64 (decode): every block streams 16 or 32 rows of W once, its 4 to 16
 //                    waves split K and meet in LDS (v_mfma_f32_16x16x32_bf16).
+//   gemm_bf16_shared_rows  17 <= M <= 64 and a W with many rows: as above, but two waves that
+//                    stream different rows of W share the rows of A through LDS.
 #include "common.h"
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
@@ -797,6 +799,227 @@ static void launch_skinny_mt(const bf16_t* A, const bf16_t* W, const float* bias
                                                       stream);
 }
 
+// ---------------------------------------------------------------------------------------
+// 17 to 64 rows (decode at larger batches): the activations go through LDS
+// ---------------------------------------------------------------------------------------
+// With several row tiles every wave of the kernel above reads all rows of A for its K range
+// from L2 again, which at 64 rows is twice the bytes of W it streams.  Here a block is
+// NWN x NWK waves: wave (wn, wk) owns 32 rows of W (two column tiles, or the gate and up rows
+// of 16 SwiGLU columns) and the wk-th part of the block's K range, and the NWN waves with the
+// same wk share the rows of A: chunk by chunk of KC of K they are loaded once, straight into
+// LDS (global_load_lds, two buffers, 16-byte chunks permuted so that a fragment read is free of
+// bank conflicts), while W goes from global memory into registers, one chunk ahead.  The waves
+// meet in LDS at the end to add their K parts in a fixed order.
+//
+// Host side guarantees: K / gridDim.y is a multiple of NWK * KC, M * lda < 2^31.  Rows of A
+// past M and rows of W past the end repeat the last row (their products are not stored).
+template <int MT, int NWN, int NWK, int KC>
+struct SharedRows {
+  static constexpr int NW = NWN * NWK, ROWS = 16 * MT, CH = KC / 8, UK = KC / 32;
+  static constexpr int RPI = 64 / CH;                        // rows a load instruction brings
+  static constexpr int INSTR = NWK * ROWS / RPI;             // load instructions a chunk
+  static constexpr int PER_WAVE = (INSTR + NW - 1) / NW;
+  static constexpr int BUF = NWK * ROWS * KC;                // bf16 elements a buffer
+  static constexpr size_t stage_bytes = 2 * (size_t)BUF * sizeof(bf16_t);
+  static constexpr size_t red_bytes = (size_t)NW * 2 * MT * WAVE * sizeof(f32x4_t);
+  static constexpr size_t lds_bytes = stage_bytes > red_bytes ? stage_bytes : red_bytes;
+  __device__ static int swz(int row) { return CH == 16 ? (row & 15) : ((row >> 1) & 7); }
+};
+
+template <typename TO, int MT, int EPI, int NWN, int NWK, int KC, int NSETS>
+__global__ __launch_bounds__(NWN * NWK * WAVE) void gemm_bf16_shared_rows_kernel(
+    const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, const float* __restrict__ bias,
+    TO* __restrict__ C, int M, int n_rows_w, int K, int lda, int ldc) {
+  static_assert(NSETS % 2 == 0 && 2 * (KC / 32) * (NSETS - 1) < 64, "register sets");
+  using S = SharedRows<MT, NWN, NWK, KC>;
+  constexpr int NW = S::NW, UK = S::UK, CH = S::CH;
+  extern __shared__ __attribute__((aligned(1024))) bf16_t lds[];
+  const int tid = threadIdx.x, lane = tid % WAVE;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / WAVE);
+  const int wn = wave / NWK, wk = wave % NWK;
+  const int col = lane % 16, kgi = lane / 16;
+  const int kblk = K / (int)gridDim.y;               // K of the block
+  const int kper = kblk / NWK;                       // K of a wave
+  const int nchunks = kper / KC;
+  const int kb0 = blockIdx.y * kblk;
+  C += (size_t)blockIdx.y * M * ldc;
+
+  // rows of W of this wave: group r = rows wrow0 + 16 r + (0..15)
+  const int wrow0 = (blockIdx.x * NWN + wn) * 32;
+  const bf16_t* wptr[2];
+#pragma unroll
+  for (int r = 0; r < 2; ++r)
+    wptr[r] = W + (size_t)min(wrow0 + 16 * r + col, n_rows_w - 1) * K + kb0 + wk * kper + kgi * 8;
+
+  // the block's load instructions for a chunk of A, dealt round the waves: instruction j
+  // brings rows (j % (ROWS / RPI)) * RPI + lane / CH of K part j / (ROWS / RPI)
+  uint32_t aoff[S::PER_WAVE];
+#pragma unroll
+  for (int i = 0; i < S::PER_WAVE; ++i) {
+    const int j = i * NW + wave;
+    const int part = j / (S::ROWS / S::RPI), row = (j % (S::ROWS / S::RPI)) * S::RPI + lane / CH;
+    const int chunk = (lane % CH) ^ S::swz(row);
+    aoff[i] = (uint32_t)(min(row, M - 1) * lda + kb0 + part * kper + chunk * 8) *
+              (uint32_t)sizeof(bf16_t);
+  }
+  auto stage = [&](int buf, int c) {
+    const uint64_t p = reinterpret_cast<uint64_t>(A) + (uint64_t)c * (KC * sizeof(bf16_t));
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)p);
+    const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(p >> 32));
+    const char* base = reinterpret_cast<const char*>(((uint64_t)hi << 32) | lo);
+#pragma unroll
+    for (int i = 0; i < S::PER_WAVE; ++i) {
+      const int j = i * NW + wave;
+      if (S::INSTR % NW == 0 || j < S::INSTR)
+        __builtin_amdgcn_global_load_lds(KAPPAI_GPTR(base + aoff[i]),
+                                         KAPPAI_LPTR(lds + buf * S::BUF + j * 512), 16, 0, 0);
+    }
+  };
+  auto load_w = [&](u32x4_t (&wv)[UK][2], int c) {
+#pragma unroll
+    for (int u = 0; u < UK; ++u)
+#pragma unroll
+      for (int r = 0; r < 2; ++r) wv[u][r] = load16(wptr[r] + c * KC + 32 * u);
+  };
+  f32x4_t acc[2 * MT];
+#pragma unroll
+  for (int t = 0; t < 2 * MT; ++t) acc[t] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+  // fragment of A: lane holds row 16 t + col, the 8 of K number 4 u + kgi of the chunk
+  int roff[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) roff[t] = (wk * S::ROWS + 16 * t + col) * KC;
+  auto products = [&](const u32x4_t (&wv)[UK][2], int buf) {
+#pragma unroll
+    for (int u = 0; u < UK; ++u) {
+      u32x4_t av[MT];
+#pragma unroll
+      for (int t = 0; t < MT; ++t)
+        av[t] = *reinterpret_cast<const u32x4_t*>(
+            lds + buf * S::BUF + roff[t] + (((4 * u + kgi) ^ S::swz(16 * t + col)) * 8));
+#pragma unroll
+      for (int r = 0; r < 2; ++r)
+#pragma unroll
+        for (int t = 0; t < MT; ++t)
+          acc[r * MT + t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+              as_bf16x8(av[t]), as_bf16x8(wv[u][r]), acc[r * MT + t], 0, 0, 0);
+    }
+  };
+
+  // W is loaded NSETS - 1 chunks ahead into register sets used in turn; A one chunk ahead.  In
+  // every round the loads of A are issued before those of W, and loads come back in the order
+  // they were issued: waiting until only the last round's loads of W are out means that the
+  // chunk of A issued before them has landed.  NSETS is even, so that the LDS buffer of a round
+  // is known at compile time (else the compiler waits for every load before it reads LDS).
+  u32x4_t wv[NSETS][UK][2];
+  stage(0, 0);
+#pragma unroll
+  for (int s = 0; s < NSETS - 1; ++s)
+    if (s < nchunks) load_w(wv[s], s);
+  constexpr int VM_ROUND = 0x0F70 | ((2 * UK) & 15) | (((2 * UK) >> 4) << 14);
+  constexpr int VM_FIRST = 0x0F70 | ((2 * UK * (NSETS - 1)) & 15) | (((2 * UK * (NSETS - 1)) >> 4) << 14);
+  for (int c = 0; c < nchunks; c += NSETS) {
+#pragma unroll
+    for (int s = 0; s < NSETS; ++s) {
+      const int cc = c + s;
+      if (cc >= nchunks) break;
+      // chunk cc of A was issued in round cc - 1 and after it that round's chunk of W, if there
+      // was one left to load (before the loop: chunk 0 of A, then NSETS - 1 chunks of W)
+      if (cc == 0 && nchunks >= NSETS - 1)
+        __builtin_amdgcn_s_waitcnt(VM_FIRST);
+      else if (cc > 0 && cc + NSETS - 2 < nchunks)
+        __builtin_amdgcn_s_waitcnt(VM_ROUND);
+      else
+        __builtin_amdgcn_s_waitcnt(0x0F70);
+      // everybody's part of chunk cc is there and nobody reads the other buffer any more (a
+      // bare barrier: a fence would wait for the loads of W that are meant to stay in flight)
+      __builtin_amdgcn_s_barrier();
+      SCHED_FENCE();
+      if (cc + 1 < nchunks) stage((s + 1) & 1, cc + 1);
+      if (cc + NSETS - 1 < nchunks) load_w(wv[(s + NSETS - 1) % NSETS], cc + NSETS - 1);
+      products(wv[s], s & 1);
+    }
+  }
+  __syncthreads();
+  // the K parts meet: wave (wn, wk) adds up and stores row tiles wk, wk + NWK, ...
+  f32x4_t* red = reinterpret_cast<f32x4_t*>(lds);
+#pragma unroll
+  for (int t = 0; t < 2 * MT; ++t) red[(wave * 2 * MT + t) * WAVE + lane] = acc[t];
+  __syncthreads();
+  for (int t = wk; t < MT; t += NWK) {
+    f32x4_t sum[2];
+#pragma unroll
+    for (int r = 0; r < 2; ++r) {
+      sum[r] = red[((wn * NWK) * 2 * MT + r * MT + t) * WAVE + lane];
+#pragma unroll
+      for (int w = 1; w < NWK; ++w) sum[r] += red[((wn * NWK + w) * 2 * MT + r * MT + t) * WAVE + lane];
+    }
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+      const int gm = 16 * t + 4 * kgi + v;
+      if (gm >= M) continue;
+      if (EPI == 1) {
+        const int on = wrow0 / 2 + col;                 // 16 output columns a wave
+        if (wrow0 + 16 + col < n_rows_w)
+          store_out(C + (size_t)gm * ldc + on, silu_f(sum[0][v]) * sum[1][v]);
+      } else {
+#pragma unroll
+        for (int r = 0; r < 2; ++r) {
+          const int gn = wrow0 + 16 * r + col;
+          if (gn < n_rows_w)
+            store_out(C + (size_t)gm * ldc + gn,
+                      sum[r][v] + ((bias && blockIdx.y == 0) ? bias[gn] : 0.f));
+        }
+      }
+    }
+  }
+}
+
+template <int NWK, int KC>
+static bool shared_rows_fits(int M, int K, int lda, int ksplit) {
+  return M > 16 && M <= 64 && ksplit >= 1 && K % (ksplit * NWK * KC) == 0 &&
+         (long)M * lda < (1L << 31) - 8 * (long)KC;
+}
+
+template <typename TO, int MT, int EPI, int NWN, int NWK, int KC, int NSETS>
+static void launch_shared_rows_cfg(const bf16_t* A, const bf16_t* W, const float* bias, TO* C,
+                                   int M, int n_rows_w, int K, int lda, int ldc, int ksplit,
+                                   hipStream_t stream) {
+  using S = SharedRows<MT, NWN, NWK, KC>;
+  auto kern = gemm_bf16_shared_rows_kernel<TO, MT, EPI, NWN, NWK, KC, NSETS>;
+  static bool attr_set = false;       // more than 64 KB of LDS has to be asked for once
+  if (!attr_set) {
+    (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
+                              (int)S::lds_bytes);
+    attr_set = true;
+  }
+  hipLaunchKernelGGL(kern, dim3((n_rows_w + 32 * NWN - 1) / (32 * NWN), ksplit),
+                     dim3(S::NW * WAVE), S::lds_bytes, stream, A, W, bias, C, M, n_rows_w, K, lda,
+                     ldc);
+}
+
+// 2 x 4 waves, chunks of 128 of K, two register sets of W.  (4 x 4 waves leave half the CUs
+// without a block on the layer shapes; more register sets or 16 waves with chunks of 64 gain
+// nothing.)  Returns false when the shape does not fit.
+#define SR_NWN 2
+#define SR_NWK 4
+#define SR_KC 128
+template <typename TO, int EPI>
+static bool launch_shared_rows(const bf16_t* A, const bf16_t* W, const float* bias, TO* C, int M,
+                               int n_rows_w, int K, int lda, int ldc, int ksplit,
+                               hipStream_t stream) {
+  if (!shared_rows_fits<SR_NWK, SR_KC>(M, K, lda, ksplit)) return false;
+  if (M <= 32)
+    launch_shared_rows_cfg<TO, 2, EPI, SR_NWN, SR_NWK, SR_KC, 2>(A, W, bias, C, M, n_rows_w, K, lda,
+                                                                 ldc, ksplit, stream);
+  else if (M <= 48)
+    launch_shared_rows_cfg<TO, 3, EPI, SR_NWN, SR_NWK, SR_KC, 2>(A, W, bias, C, M, n_rows_w, K, lda,
+                                                                 ldc, ksplit, stream);
+  else
+    launch_shared_rows_cfg<TO, 4, EPI, SR_NWN, SR_NWK, SR_KC, 2>(A, W, bias, C, M, n_rows_w, K, lda,
+                                                                 ldc, ksplit, stream);
+  return true;
+}
+
 template <typename TO, int EPI>
 static int launch_bf16(const bf16_t* A, const bf16_t* W, const float* bias, TO* C, int M, int N,
                        int K, int lda, int ldc, int force_kernel, int ksplit, hipStream_t stream,
@@ -806,6 +1029,18 @@ static int launch_bf16(const bf16_t* A, const bf16_t* W, const float* bias, TO* 
   // the 128 x 128 blocks than through the decode kernel, which reads the rows once per 32 columns
   const bool wide_head = EPI == 0 && M > 32 && N >= 16384 && force_kernel == 0 && ksplit == 1 &&
                          block256_fits<TO, EPI>(A, W, C, M, N, K, lda, ldc, ksplit);
+  // 17 to 64 rows and blocks enough to fill half the chip: the rows go through LDS
+  if constexpr (EPI != 2) {
+    const int n_rows_w = EPI == 1 ? 2 * N : N;
+    const long sr_blocks = (long)((n_rows_w + 32 * SR_NWN - 1) / (32 * SR_NWN)) * ksplit;
+    if (force_kernel == 9 || (force_kernel == 0 && M > 16 && M <= 64 && sr_blocks >= 128)) {
+      if (launch_shared_rows<TO, EPI>(A, W, bias, C, M, n_rows_w, K, lda, ldc, ksplit, stream))
+        KAPPAI_RETURN_LAUNCH_STATUS();
+      if (force_kernel == 9) return (int)hipErrorInvalidValue;
+    }
+  } else if (force_kernel == 9) {
+    return (int)hipErrorInvalidValue;
+  }
   if (M <= 64 && force_kernel != 1 && force_kernel < 3 && !wide_head) {
     const int mt = (M + 15) / 16;
     switch (mt) {
@@ -833,7 +1068,8 @@ static int launch_bf16(const bf16_t* A, const bf16_t* W, const float* bias, TO* 
 
 // K, lda must be multiples of 8 and A, W 16-byte aligned (checked by the caller).
 // force_kernel: 0 = by M, 1 = tile kernel, 2 = skinny kernel (M <= 64 only), 3..8 = tile kernel
-// with block shape 1..6 (see launch_tile); for tests and tuning.
+// with block shape 1..6 (see launch_tile), 9 = shared-rows kernel (17 to 64 rows, K / ksplit a
+// multiple of 512); for tests and tuning.
 // ksplit > 1 (float output only): C is [ksplit][M][ldc] partial sums over K ranges.
 extern "C" int kappai_gemm_bf16(const void* A, const void* W, const float* bias, void* C, int M,
                                 int N, int K, int lda, int ldc, int out_is_f32, int force_kernel,

@@ -17,6 +17,7 @@ F32, BF16, I32 = torch.float32, torch.bfloat16, torch.int32
 MAX_HEAD_DIM = 512
 MAX_GRID_Y = 65535
 DECODE_WAVES = 2048       # waves the split-key decode attention aims to have at work
+DECODE_MAX_SPLITS = 128   # partial results of a row's head that the merge kernel adds up at most
 
 _c_int, _c_float, _c_long, _vp = ctypes.c_int, ctypes.c_float, ctypes.c_long, ctypes.c_void_p
 
@@ -141,7 +142,8 @@ def cast(x: torch.Tensor, dtype) -> torch.Tensor:
 # ---------------------------------------------------------------------------------------
 def split_k_for(M: int, N: int, K: int) -> int:
     """How many K ranges a product is cut into when its consumer takes partial sums (1: not
-    split).  Decode (M <= 64): so that about 512 blocks stream the matrix.  Larger M: only long
+    split).  Decode (M <= 64): so that about 512 blocks stream the matrix (17 rows and more: what
+    suits the kernel that takes them).  Larger M: only long
     K (ranges of 2048 or more) and few 128 x 128 blocks; every range is a multiple of 128 long,
     as the large-product kernel asks."""
     if M > 64:
@@ -150,6 +152,14 @@ def split_k_for(M: int, N: int, K: int) -> int:
         while split > 1 and K % (128 * split):
             split -= 1
         return split
+    if M > 16:
+        # the kernel that shares the rows through LDS: blocks of 64 columns, K ranges that are
+        # multiples of 512 and at least 1024 long, 128 blocks or more
+        split = min(8, K // 1024)
+        while split > 1 and K % (512 * split):
+            split -= 1
+        if split >= 1 and K % (512 * split) == 0 and ((N + 63) // 64) * split >= 128:
+            return split
     col_groups = (N + 15) // 16
     return max(1, min(8, 512 // col_groups, K // 512))
 
@@ -437,11 +447,12 @@ def paged_attention(q: torch.Tensor, n_heads: int, n_kv_heads: int, head_dim: in
     _need(max_position is not None, "the decode kernel needs the batch's largest position")
     n_keys = min(max_position + 1, window) + 32 if window else max_position + 1
     # one wave keeps the loads of `kpw` keys in flight; splits are whole numbers of that, and
-    # at most 64 of them are merged
+    # at most DECODE_MAX_SPLITS of them are merged
     kpw = lib.kappai_attn_keys_per_wave()
     # and no more splits than it takes to have DECODE_WAVES waves at work: with many rows a
     # wave rather takes several chunks in turn than writes a partial result for each
-    n_splits = max(1, min(64, (n_keys + kpw - 1) // kpw, max(1, DECODE_WAVES // (T * G))))
+    n_splits = max(1, min(DECODE_MAX_SPLITS, (n_keys + kpw - 1) // kpw,
+                          max(1, DECODE_WAVES // (T * G))))
     keys_per_split = ((n_keys + n_splits - 1) // n_splits + kpw - 1) // kpw * kpw
     n_splits = (n_keys + keys_per_split - 1) // keys_per_split
     part_o = torch.empty((T, H, n_splits, d), dtype=F32, device=q.device)

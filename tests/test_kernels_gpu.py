@@ -176,6 +176,53 @@ def test_linear_swiglu_block256(ops, M, F, K, block):
     close(got.float(), want, BF16_ULP, "block256")
 
 
+SHARED_ROWS = 9       # force_kernel: 17 to 64 rows, the rows shared through LDS
+
+
+@pytest.mark.parametrize("M", [17, 32, 33, 47, 64])
+@pytest.mark.parametrize("N,K", [(64, 512), (200, 1024), (2048, 2048), (8200, 1536)])
+@pytest.mark.parametrize("out_dtype", [F32, BF16])
+def test_linear_shared_rows(ops, M, N, K, out_dtype):
+    """The kernel for 17 to 64 rows: every row-tile count, matrices that end inside a block's 64
+    columns or inside a wave's 32, one and several chunks of K per wave, a row stride, bias."""
+    wide = rand((M, K + 8), BF16, 51)
+    x, w, b = wide[:, :K], rand((N, K), BF16, 52), rand((N,), F32, 53)
+    want = x.double() @ w.double().T
+    tol = 2e-5 if out_dtype == F32 else BF16_ULP
+    xd = wide.to(DEV)[:, :K]
+    got = ops.linear(xd, w.to(DEV), out_dtype=out_dtype, force_kernel=SHARED_ROWS)
+    close(got.float(), want, tol, "shared rows")
+    got = ops.linear(xd, w.to(DEV), b.to(DEV), out_dtype=out_dtype, force_kernel=SHARED_ROWS)
+    close(got.float(), want + b.double(), tol, "shared rows with bias")
+
+
+@pytest.mark.parametrize("M,F,K", [(17, 48, 512), (40, 1008, 1024), (64, 8192, 2048)])
+def test_linear_swiglu_shared_rows(ops, M, F, K):
+    x, wg, wu = rand((M, K), BF16, 54), rand((F, K), BF16, 55, 0.2), rand((F, K), BF16, 56, 0.2)
+    w = ops.interleave_gate_up(wg.to(DEV), wu.to(DEV))
+    g, u = x.double() @ wg.double().T, x.double() @ wu.double().T
+    want = g / (1 + torch.exp(-g)) * u
+    got = ops.linear_swiglu(x.to(DEV), w, force_kernel=SHARED_ROWS)
+    close(got.float(), want, BF16_ULP, "shared rows")
+
+
+@pytest.mark.parametrize("M,N,K,S", [(24, 2048, 8192, 8), (64, 100, 3072, 3), (33, 2048, 2048, 2)])
+def test_linear_shared_rows_split_k(ops, M, N, K, S):
+    x, w, b = rand((M, K), BF16, 57), rand((N, K), BF16, 58, 0.05), rand((N,), F32, 59)
+    parts = ops.linear(x.to(DEV), w.to(DEV), b.to(DEV), partial_sums=True, split_k=S,
+                       force_kernel=SHARED_ROWS)
+    assert parts.shape == (S, M, N) and parts.dtype == F32
+    close(parts.sum(0), x.double() @ w.double().T + b.double(), 2e-5, "sum of the partial sums")
+
+
+def test_linear_shared_rows_refuses_what_does_not_fit(ops):
+    x, w = rand((32, 520), BF16, 60).to(DEV), rand((64, 520), BF16, 61).to(DEV)
+    with pytest.raises(RuntimeError):
+        ops.linear(x, w, force_kernel=SHARED_ROWS)          # K is no multiple of 512
+    with pytest.raises(RuntimeError):
+        ops.linear(x[:8, :512].contiguous(), w[:, :512].contiguous(), force_kernel=SHARED_ROWS)
+
+
 def test_linear_block256_split_k(ops):
     """Partial sums over K ranges from the large-product kernel add up to the product."""
     M, N, K = 2048, 2048, 8192
@@ -188,7 +235,7 @@ def test_linear_block256_split_k(ops):
 
 
 @pytest.mark.parametrize("M,N,K", [(1, 2048, 2048), (8, 2048, 8192), (16, 96, 1024), (40, 1000, 4096),
-                                   (64, 64, 512), (5, 6144, 2048)])
+                                   (64, 64, 512), (5, 6144, 2048), (64, 2048, 8192), (20, 2048, 2048)])
 def test_linear_partial_sums(ops, M, N, K):
     """A decode product split over K: float32 partial sums that add up to the product, and an
     RMSNorm that consumes them like an ordinary residual update."""
