@@ -204,3 +204,65 @@ def test_long_prompt_on_a_wide_model(tmp_path, dtype):
     assert len(got) == 2500
     err, where = worst_error(got, ref)
     assert err < tol, (err, tol, where, first_bad(got, ref, tol))
+
+
+# Products with 17 to 64 rows and many rows of W run in a kernel of their own (activation rows
+# shared through LDS): hidden size and feed-forward width are multiples of 512 here, and gate/up
+# and the output head have 8192 rows, so a decode step of 40 requests takes it where a step of 8
+# takes the kernel for few rows.
+MANY = {
+    "architectures": ["Lfm2ForCausalLM"], "model_type": "lfm2",
+    "hidden_size": 512, "num_hidden_layers": 2, "layer_types": ["conv", "full_attention"],
+    "num_attention_heads": 8, "num_key_value_heads": 2, "head_dim": 64,
+    "intermediate_size": 4096, "block_auto_adjust_ff_dim": False,
+    "vocab_size": 8192, "norm_eps": 1e-5, "rope_theta": 10000.0,
+    "conv_L_cache": 3, "conv_bias": False, "tie_embedding": True,
+    "max_position_embeddings": 512,
+}
+
+
+@pytest.mark.parametrize("dtype", ["bfloat16", "float32"])
+def test_decode_steps_of_forty_requests(tmp_path, dtype):
+    """Forty requests decoded side by side (and the same requests eight at a time) give the
+    logits of each request alone in the plain implementation: the result does not depend on
+    which product kernel the number of rows selects."""
+    import copy
+    from kappai_amd.cache import CacheManager
+    from kappai_amd.config import config_from_dict
+    from kappai_amd.engine import StepEntry, StepRunner
+    from kappai_amd.weights import write_random_model
+    folder = write_random_model(tmp_path / "many", config_from_dict(copy.deepcopy(MANY)), seed=6,
+                                std=0.03, norm_jitter=0.05)
+    n_req, n_decode = 40, 5
+    lengths = [3 + (7 * i) % 23 + n_decode for i in range(n_req)]
+    requests = make_requests(MANY["vocab_size"], lengths, seed=16)
+    ref = plain_logits(folder, requests)
+    tol = tolerance(folder, requests, dtype)
+    model = gpu_model(folder, dtype)
+    ids = list(requests)
+    for group in (40, 8):
+        cache = CacheManager(model.cache_specs(), 16, n_req * 4, n_req)
+        cache.allocate_storage(model.dtype, "cuda:0", poison=True)
+        runner = StepRunner(model, cache, "cuda:0")
+        got = {}
+        for g0 in range(0, n_req, group):
+            part = ids[g0:g0 + group]
+            caches = {rid: cache.open(rid) for rid in part}
+            # the prompts of the group in one step, then its decode steps
+            entries = [StepEntry(caches[rid], requests[rid][:-n_decode],
+                                 [len(requests[rid]) - n_decode - 1]) for rid in part]
+            rows = runner.step(entries).cpu().numpy()
+            for rid, row in zip(part, rows):
+                got[(rid, len(requests[rid]) - n_decode - 1)] = row
+            for s in range(n_decode):
+                entries = [StepEntry(caches[rid], [requests[rid][s - n_decode]], [0])
+                           for rid in part]
+                rows = runner.step(entries).cpu().numpy()
+                for rid, row in zip(part, rows):
+                    got[(rid, len(requests[rid]) - n_decode + s)] = row
+            for rid in part:
+                cache.close(caches[rid])
+        cache.check()
+        assert len(got) == n_req * (n_decode + 1)
+        err, where = worst_error(got, ref)
+        assert err < tol, (group, err, tol, where, first_bad(got, ref, tol))
