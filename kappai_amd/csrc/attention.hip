@@ -4,7 +4,8 @@
 //                       rotation at the row's absolute position
 //                       (src/backend/cpu/quants.h:395-438: rotate-half or interleaved pairs),
 //                       q rewritten in place, k and v stored into their pages
-//                       (src/backend/cpu/common.c:1603-1622).
+//                       (src/backend/cpu/common.c:1603-1622).  The projection may also arrive
+//                       as float partial sums of a product split over its input dimension.
 //   paged_attention_rows  one wave per (row, head): causal softmax(q.k/sqrt(d)) v over the keys
 //                       lo..pos of the row's request, read through its block table
 //                       (src/backend/cpu/scalar/core.c:383-433, 623-666), online softmax in float.
@@ -28,7 +29,8 @@ __global__ __launch_bounds__(QKS_WAVES * WAVE) void qk_norm_rope_store_kernel(
     const float* __restrict__ sin_tab, int rot_dim, int rot_mode, T* __restrict__ k_pool,
     T* __restrict__ v_pool, const int* __restrict__ row_pos, const int* __restrict__ row_seg,
     const int* __restrict__ block_tables, int max_blocks, int H, int G, int d, int ps,
-    int n_slots) {
+    int n_slots, const float* __restrict__ parts, int n_parts, T* __restrict__ q_out,
+    int q_stride) {
   __shared__ float bufs[QKS_WAVES][MAX_HEAD_DIM];
   const int t = blockIdx.x, lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE;
   float* buf = bufs[wave];
@@ -40,14 +42,26 @@ __global__ __launch_bounds__(QKS_WAVES * WAVE) void qk_norm_rope_store_kernel(
   const int* bt = block_tables + (size_t)row_seg[t] * max_blocks;
   const int slot_end = min(n_slots, (int)(blockIdx.y + 1) * QKS_SLOTS);
   for (int slot = blockIdx.y * QKS_SLOTS + wave; slot < slot_end; slot += QKS_WAVES) {
-    T* src = qkv + (size_t)t * row_stride + (size_t)slot * d;
-    T* dst = src;
+    const size_t at = (size_t)t * row_stride + (size_t)slot * d;
+    // with `parts` the row arrives as float sums over n_parts ranges of the projection's input
+    // dimension, [n_parts][rows][row_stride]; added in order and rounded to T they are what the
+    // unsplit projection would have stored, and q goes to a buffer of its own
+    const size_t plane = (size_t)gridDim.x * row_stride;
+    auto value = [&](int e) -> float {
+      if (!parts) return to_f32(qkv[at + e]);
+      float sum = parts[at + e];
+      for (int k = 1; k < n_parts; ++k) sum += parts[k * plane + at + e];
+      T rounded;
+      from_f32(&rounded, sum);
+      return to_f32(rounded);
+    };
+    T* dst = parts ? q_out + (size_t)t * q_stride + (size_t)slot * d : qkv + at;
     if (slot >= H) {
       const int g = (slot - H) % G;
       const size_t pg = (size_t)bt[pos / ps] * G + g;
       if (slot >= H + G) {  // v: copied into its page, transposed
         T* vdst = v_pool + pg * d * ps + pos % ps;
-        for (int e = lane; e < d; e += WAVE) vdst[(size_t)e * ps] = src[e];
+        for (int e = lane; e < d; e += WAVE) from_f32(vdst + (size_t)e * ps, value(e));
         continue;
       }
       dst = k_pool + (pg * ps + pos % ps) * d;
@@ -55,7 +69,7 @@ __global__ __launch_bounds__(QKS_WAVES * WAVE) void qk_norm_rope_store_kernel(
     const float* nw = slot < H ? q_norm_w : k_norm_w;
     float ss = 0.f;
     for (int e = lane; e < d; e += WAVE) {
-      const float v = to_f32(src[e]);
+      const float v = value(e);
       buf[e] = v;
       ss += v * v;
     }
@@ -87,14 +101,15 @@ __global__ __launch_bounds__(QKS_WAVES * WAVE) void qk_norm_rope_store_kernel(
 // without LDS; the sum of squares and the rotation's partner (the lane d / 16 away) come by
 // shuffles.
 typedef __attribute__((ext_vector_type(4))) uint32_t qks_u32x4_t;
-template <int LPH>
+template <int LPH, bool PARTS>
 __global__ __launch_bounds__(256) void qk_norm_rope_store_vec_kernel(
     bf16_t* __restrict__ qkv, int row_stride, const float* __restrict__ q_norm_w,
     const float* __restrict__ k_norm_w, float eps, const float* __restrict__ cos_tab,
     const float* __restrict__ sin_tab, int rotate, bf16_t* __restrict__ k_pool,
     bf16_t* __restrict__ v_pool, const int* __restrict__ row_pos,
     const int* __restrict__ row_seg, const int* __restrict__ block_tables, int max_blocks, int T,
-    int H, int G, int ps, int n_slots) {
+    int H, int G, int ps, int n_slots, const float* __restrict__ parts, int n_parts,
+    bf16_t* __restrict__ q_out, int q_stride) {
   constexpr int d = LPH * 8, half = d / 2;
   const long long total = (long long)T * n_slots * LPH;
   const long long gid = (long long)blockIdx.x * blockDim.x + threadIdx.x;
@@ -105,8 +120,27 @@ __global__ __launch_bounds__(256) void qk_norm_rope_store_vec_kernel(
   const int t = (int)(head / n_slots), slot = (int)(head % n_slots);
   const int pos = row_pos[t];
   const int e0 = 8 * part;
-  bf16_t* src = qkv + (size_t)t * row_stride + (size_t)slot * d + e0;
-  const qks_u32x4_t raw = *reinterpret_cast<const qks_u32x4_t*>(src);
+  const size_t at = (size_t)t * row_stride + (size_t)slot * d + e0;
+  qks_u32x4_t raw;
+  if (PARTS) {
+    // float sums over n_parts ranges of the projection's input dimension, added in order and
+    // rounded to bfloat16: what the unsplit projection would have stored
+    const size_t plane = (size_t)T * row_stride;
+    float4 lo = *reinterpret_cast<const float4*>(parts + at);
+    float4 hi = *reinterpret_cast<const float4*>(parts + at + 4);
+    for (int k = 1; k < n_parts; ++k) {
+      const float4 a = *reinterpret_cast<const float4*>(parts + k * plane + at);
+      const float4 b = *reinterpret_cast<const float4*>(parts + k * plane + at + 4);
+      lo.x += a.x; lo.y += a.y; lo.z += a.z; lo.w += a.w;
+      hi.x += b.x; hi.y += b.y; hi.z += b.z; hi.w += b.w;
+    }
+    raw[0] = pack_bf16x2(lo.x, lo.y);
+    raw[1] = pack_bf16x2(lo.z, lo.w);
+    raw[2] = pack_bf16x2(hi.x, hi.y);
+    raw[3] = pack_bf16x2(hi.z, hi.w);
+  } else {
+    raw = *reinterpret_cast<const qks_u32x4_t*>(qkv + at);
+  }
   float v[8];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
@@ -155,7 +189,8 @@ __global__ __launch_bounds__(256) void qk_norm_rope_store_vec_kernel(
     qks_u32x4_t o;
 #pragma unroll
     for (int i = 0; i < 4; ++i) o[i] = pack_bf16x2(r[2 * i], r[2 * i + 1]);
-    *reinterpret_cast<qks_u32x4_t*>(src) = o;
+    bf16_t* qdst = PARTS ? q_out + (size_t)t * q_stride + (size_t)slot * d + e0 : qkv + at;
+    *reinterpret_cast<qks_u32x4_t*>(qdst) = o;
     return;
   }
   const int g = (slot - H) % G;
@@ -182,25 +217,34 @@ extern "C" int kappai_qk_norm_rope_store(void* qkv, int row_stride, const float*
                                          void* k_pool, void* v_pool, const int* row_pos,
                                          const int* row_seg, const int* block_tables,
                                          int max_blocks, int T, int H, int G, int d, int ps,
-                                         int store_kv, int is_bf16, hipStream_t stream) {
+                                         int store_kv, int is_bf16, const float* parts,
+                                         int n_parts, void* q_out, int q_stride,
+                                         hipStream_t stream) {
+  // parts != null: the projection as [n_parts][T][row_stride] float partial sums instead of
+  // qkv; q is then written to q_out [T][q_stride] (bfloat16 only)
   if (T <= 0) return 0;
   if (d > MAX_HEAD_DIM || d < 1 || rot_dim > d || (rot_dim & 1)) return (int)hipErrorInvalidValue;
+  if (parts && (!is_bf16 || n_parts < 1 || !q_out)) return (int)hipErrorInvalidValue;
   const int n_slots = store_kv ? H + 2 * G : H;
   const bool whole_rot = rot_mode == 0 || rot_dim == 0 || (rot_mode == 1 && rot_dim == d);
   const int lph = d / 8;
   if (is_bf16 && whole_rot && d % 8 == 0 && lph >= 2 && lph <= 64 && (lph & (lph - 1)) == 0 &&
       row_stride % 8 == 0 && ((uintptr_t)qkv % 16) == 0 && ((uintptr_t)k_pool % 16) == 0 &&
+      ((uintptr_t)parts % 16) == 0 && ((uintptr_t)q_out % 16) == 0 && q_stride % 8 == 0 &&
       ((uintptr_t)cos_tab % 16) == 0 && ((uintptr_t)sin_tab % 16) == 0 &&
       (!q_norm_w || ((uintptr_t)q_norm_w % 16) == 0) &&
       (!k_norm_w || ((uintptr_t)k_norm_w % 16) == 0)) {
     const int rotate = rot_mode == 1 && rot_dim == d;
     const long long total = (long long)T * n_slots * lph;
     const dim3 gv((unsigned)((total + 255) / 256));
+#define QKS_LAUNCH_AS(N, P)                                                                      \
+  hipLaunchKernelGGL((qk_norm_rope_store_vec_kernel<N, P>), gv, dim3(256), 0, stream,            \
+                     (bf16_t*)qkv, row_stride, q_norm_w, k_norm_w, eps, cos_tab, sin_tab,        \
+                     rotate, (bf16_t*)k_pool, (bf16_t*)v_pool, row_pos, row_seg, block_tables,   \
+                     max_blocks, T, H, G, ps, n_slots, parts, n_parts, (bf16_t*)q_out, q_stride)
 #define QKS_LAUNCH(N)                                                                            \
-  hipLaunchKernelGGL(qk_norm_rope_store_vec_kernel<N>, gv, dim3(256), 0, stream, (bf16_t*)qkv,   \
-                     row_stride, q_norm_w, k_norm_w, eps, cos_tab, sin_tab, rotate,              \
-                     (bf16_t*)k_pool, (bf16_t*)v_pool, row_pos, row_seg, block_tables,           \
-                     max_blocks, T, H, G, ps, n_slots)
+  if (parts) QKS_LAUNCH_AS(N, true);                                                             \
+  else QKS_LAUNCH_AS(N, false)
     switch (lph) {
       case 2: QKS_LAUNCH(2); break;
       case 4: QKS_LAUNCH(4); break;
@@ -210,6 +254,7 @@ extern "C" int kappai_qk_norm_rope_store(void* qkv, int row_stride, const float*
       default: QKS_LAUNCH(64); break;
     }
 #undef QKS_LAUNCH
+#undef QKS_LAUNCH_AS
     KAPPAI_RETURN_LAUNCH_STATUS();
   }
   dim3 grid(T, (n_slots + QKS_SLOTS - 1) / QKS_SLOTS);
@@ -217,12 +262,13 @@ extern "C" int kappai_qk_norm_rope_store(void* qkv, int row_stride, const float*
     hipLaunchKernelGGL(qk_norm_rope_store_kernel<bf16_t>, grid, dim3(QKS_WAVES * WAVE), 0, stream,
                        (bf16_t*)qkv, row_stride, q_norm_w, k_norm_w, eps, cos_tab, sin_tab,
                        rot_dim, rot_mode, (bf16_t*)k_pool, (bf16_t*)v_pool, row_pos, row_seg,
-                       block_tables, max_blocks, H, G, d, ps, n_slots);
+                       block_tables, max_blocks, H, G, d, ps, n_slots, parts, n_parts,
+                       (bf16_t*)q_out, q_stride);
   else
     hipLaunchKernelGGL(qk_norm_rope_store_kernel<float>, grid, dim3(QKS_WAVES * WAVE), 0, stream, (float*)qkv,
                        row_stride, q_norm_w, k_norm_w, eps, cos_tab, sin_tab, rot_dim, rot_mode,
                        (float*)k_pool, (float*)v_pool, row_pos, row_seg, block_tables, max_blocks,
-                       H, G, d, ps, n_slots);
+                       H, G, d, ps, n_slots, nullptr, 0, nullptr, 0);
   KAPPAI_RETURN_LAUNCH_STATUS();
 }
 

@@ -169,21 +169,12 @@ __global__ void shortconv_state_kernel(const T* __restrict__ proj, float* __rest
 
 // Every segment is a single row (decode): one thread per (segment, channel) computes the output
 // and shifts the state, which nobody else reads.
-template <typename T>
-__global__ void shortconv_step_kernel(const T* __restrict__ proj, const float* __restrict__ w,
-                                      const float* __restrict__ bias, float* __restrict__ state,
-                                      T* __restrict__ out, const int* __restrict__ seg_pos0,
-                                      const int* __restrict__ seg_slot, int D, int L) {
-  const int c = blockIdx.y * blockDim.x + threadIdx.x;
-  const int t = blockIdx.x;
-  if (c >= D) return;
-  const bool fresh = seg_pos0[t] == 0;
+__device__ __forceinline__ float shortconv_step_one(float bg, float cg, float xg,
+                                                    const float* __restrict__ wc, float cbias,
+                                                    float* __restrict__ st, bool fresh, int L) {
   const int H = L - 1;
-  float* st = state + ((size_t)seg_slot[t] * D + c) * H;
-  const float* wc = w + (size_t)c * L;
-  const T* p = proj + (size_t)t * 3 * D;
-  const float bx = to_f32(p[c]) * to_f32(p[2 * D + c]);
-  float sum = (bias ? bias[c] : 0.f);
+  const float bx = bg * xg;
+  float sum = cbias;
   float prev = fresh ? 0.f : st[0];
   for (int k = 0; k < H; ++k) {
     sum += wc[k] * prev;                       // tap k meets history entry k
@@ -192,7 +183,62 @@ __global__ void shortconv_step_kernel(const T* __restrict__ proj, const float* _
     prev = next;
   }
   sum += wc[H] * bx;
-  from_f32(out + (size_t)t * D + c, to_f32(p[D + c]) * sum);
+  return cg * sum;
+}
+
+template <typename T>
+__global__ void shortconv_step_kernel(const T* __restrict__ proj, const float* __restrict__ w,
+                                      const float* __restrict__ bias, float* __restrict__ state,
+                                      T* __restrict__ out, const int* __restrict__ seg_pos0,
+                                      const int* __restrict__ seg_slot, int D, int L) {
+  const int c = blockIdx.y * blockDim.x + threadIdx.x;
+  const int t = blockIdx.x;
+  if (c >= D) return;
+  const T* p = proj + (size_t)t * 3 * D;
+  float* st = state + ((size_t)seg_slot[t] * D + c) * (L - 1);
+  from_f32(out + (size_t)t * D + c,
+           shortconv_step_one(to_f32(p[c]), to_f32(p[D + c]), to_f32(p[2 * D + c]),
+                              w + (size_t)c * L, bias ? bias[c] : 0.f, st, seg_pos0[t] == 0, L));
+}
+
+// The same step when the projection arrives as float sums over n_parts ranges of its input
+// dimension, [n_parts][T][3D] (a product split over K): they are added in order and rounded to
+// bfloat16, which is what the unsplit product would have stored.
+__global__ void shortconv_step_parts_kernel(const float* __restrict__ parts, int n_parts,
+                                            const float* __restrict__ w,
+                                            const float* __restrict__ bias,
+                                            float* __restrict__ state, bf16_t* __restrict__ out,
+                                            const int* __restrict__ seg_pos0,
+                                            const int* __restrict__ seg_slot, int T, int D, int L) {
+  const int c = blockIdx.y * blockDim.x + threadIdx.x;
+  const int t = blockIdx.x;
+  if (c >= D) return;
+  const size_t plane = (size_t)T * 3 * D;
+  const float* p = parts + (size_t)t * 3 * D + c;
+  float g[3];
+#pragma unroll
+  for (int i = 0; i < 3; ++i) {
+    float sum = p[(size_t)i * D];
+    for (int s = 1; s < n_parts; ++s) sum += p[s * plane + (size_t)i * D];
+    g[i] = to_f32(f32_to_bf16(sum));
+  }
+  float* st = state + ((size_t)seg_slot[t] * D + c) * (L - 1);
+  from_f32(out + (size_t)t * D + c,
+           shortconv_step_one(g[0], g[1], g[2], w + (size_t)c * L, bias ? bias[c] : 0.f, st,
+                              seg_pos0[t] == 0, L));
+}
+
+extern "C" int kappai_shortconv_step_parts(const float* parts, int n_parts, const float* w,
+                                           const float* bias, float* state, void* out,
+                                           const int* seg_pos0, const int* seg_slot, int T, int D,
+                                           int L, hipStream_t stream) {
+  if (T <= 0) return 0;
+  if (L < 2 || n_parts < 1 || D < 1) return (int)hipErrorInvalidValue;
+  const int threads = D >= 256 ? 256 : 64;
+  hipLaunchKernelGGL(shortconv_step_parts_kernel, dim3(T, (D + threads - 1) / threads),
+                     dim3(threads), 0, stream, parts, n_parts, w, bias, state, (bf16_t*)out,
+                     seg_pos0, seg_slot, T, D, L);
+  KAPPAI_RETURN_LAUNCH_STATUS();
 }
 
 extern "C" int kappai_shortconv(const void* proj, const float* w, const float* bias, float* state,

@@ -161,7 +161,10 @@ def split_k_for(M: int, N: int, K: int) -> int:
         if split >= 1 and K % (512 * split) == 0 and ((N + 63) // 64) * split >= 128:
             return split
     col_groups = (N + 15) // 16
-    return max(1, min(8, 512 // col_groups, K // 512))
+    want = 512 // col_groups
+    if want < 2 and col_groups <= 448:
+        want = 2        # measured: 6144 x 2048 in 8.3 us in two ranges, 9.7 us in one
+    return max(1, min(8, want, K // 512))
 
 
 def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
@@ -289,8 +292,13 @@ def shortconv(proj: torch.Tensor, taps: torch.Tensor, bias: Optional[torch.Tenso
               seg_pos0: torch.Tensor, seg_slot: torch.Tensor) -> torch.Tensor:
     """Gated causal depthwise convolution of ``proj`` [T, 3D] = (B | C | x) per segment with
     taps [D, L]; reads and then updates ``state`` [slots, D, L-1] (float32) of every
-    segment's slot.  Returns C * conv(B * x) as [T, D]."""
+    segment's slot.  Returns C * conv(B * x) as [T, D].  When every segment is a single row,
+    ``proj`` may be the float32 partial sums [S, T, 3D] of a projection split over its input
+    dimension: they are added in order and rounded to bfloat16 first, and the result is
+    bfloat16."""
     _gpu("proj", proj, (F32, BF16))
+    if proj.dim() == 3:
+        return _shortconv_step_parts(proj, taps, bias, state, seg_pos0, seg_slot)
     _gpu("taps", taps, F32)
     _gpu("state", state, F32)
     for n, t in (("row_seg", row_seg), ("seg_start", seg_start), ("seg_pos0", seg_pos0),
@@ -316,6 +324,29 @@ def shortconv(proj: torch.Tensor, taps: torch.Tensor, bias: Optional[torch.Tenso
     return out
 
 
+def _shortconv_step_parts(parts, taps, bias, state, seg_pos0, seg_slot) -> torch.Tensor:
+    _gpu("taps", taps, F32)
+    _gpu("state", state, F32)
+    _gpu("seg_pos0", seg_pos0, I32)
+    _gpu("seg_slot", seg_slot, I32)
+    S, T, W = parts.shape
+    D, L = taps.shape
+    _need(parts.dtype == F32 and W == 3 * D and parts.is_contiguous(),
+          f"shortconv: partial sums {tuple(parts.shape)} for D={D}")
+    _need(seg_pos0.shape[0] == T and seg_slot.shape[0] == T,
+          "shortconv: partial sums are taken only when every segment is a single row")
+    _need(L >= 2 and state.dim() == 3 and state.shape[1:] == (D, L - 1),
+          f"shortconv: state {tuple(state.shape)} for D={D}, L={L}")
+    if bias is not None:
+        _gpu("bias", bias, F32)
+        _need(bias.shape == (D,), "shortconv: bias must be [D]")
+    out = torch.empty((T, D), dtype=BF16, device=parts.device)
+    check(library("shortconv").kappai_shortconv_step_parts(
+        _ptr(parts), _c_int(S), _ptr(taps), _ptr(bias), _ptr(state), _ptr(out), _ptr(seg_pos0),
+        _ptr(seg_slot), _c_int(T), _c_int(D), _c_int(L), _stream()), "shortconv_step_parts")
+    return out
+
+
 ROT_NONE, ROT_HALF, ROT_INTERLEAVED = 0, 1, 2
 ATTENTION_TILE_ROWS = 32      # rows of a segment that one wave of the prefill kernel takes
 
@@ -334,15 +365,28 @@ def qk_norm_rope_store(qkv: torch.Tensor, n_heads: int, n_kv_heads: int, head_di
                        rot_dim: int, rot_mode: int, k_pool: Optional[torch.Tensor],
                        v_pool: Optional[torch.Tensor], row_pos: torch.Tensor,
                        row_seg: torch.Tensor, block_tables: torch.Tensor, page_size: int,
-                       store_kv: bool = True) -> None:
+                       store_kv: bool = True) -> torch.Tensor:
     """In ``qkv`` [T, (H + 2G) d]: normalise every q and k head, rotate them at the row's
     position (tables [positions, rot_dim/2]), rewrite q in place and store k and v into the
-    pools [pages, G, page_size, d] through the block tables [S, max_blocks]."""
+    pools [pages, G, page_size, d] through the block tables [S, max_blocks].  Returns the
+    tensor whose leading H d columns hold q: ``qkv`` itself, or, when ``qkv`` is the float32
+    partial sums [S, T, width] of a projection split over its input dimension (they are added
+    in order and rounded to bfloat16 first), a new bfloat16 [T, H d]."""
     H, G, d = n_heads, n_kv_heads, head_dim
     _gpu("qkv", qkv, (F32, BF16))
-    T = qkv.shape[0]
     width = (H + 2 * G) * d if store_kv else H * d
-    _need(qkv.dim() == 2 and qkv.shape[1] >= width, f"qk_norm_rope_store: qkv {tuple(qkv.shape)}")
+    parts = qkv if qkv.dim() == 3 else None
+    if parts is not None:
+        _need(parts.dtype == F32 and parts.shape[2] >= width and parts.is_contiguous(),
+              f"qk_norm_rope_store: partial sums {tuple(parts.shape)}")
+        T = parts.shape[1]
+        q_out = torch.empty((T, H * d), dtype=BF16, device=parts.device)
+        row_stride, data_dtype = parts.shape[2], BF16
+    else:
+        T = qkv.shape[0]
+        _need(qkv.dim() == 2 and qkv.shape[1] >= width,
+              f"qk_norm_rope_store: qkv {tuple(qkv.shape)}")
+        q_out, row_stride, data_dtype = None, qkv.stride(0), qkv.dtype
     _need(1 <= d <= MAX_HEAD_DIM, f"head_dim {d} is beyond the kernels' limit {MAX_HEAD_DIM}")
     _need(H + 2 * G <= MAX_GRID_Y, "too many heads for one launch")
     for n, t in (("q_norm_w", q_norm_w), ("k_norm_w", k_norm_w)):
@@ -360,19 +404,22 @@ def qk_norm_rope_store(qkv: torch.Tensor, n_heads: int, n_kv_heads: int, head_di
     _need(row_pos.shape[0] == T and row_seg.shape[0] == T, "row tables do not fit the batch")
     max_blocks = 0
     if store_kv:
-        _gpu("k_pool", k_pool, qkv.dtype)
-        _gpu("v_pool", v_pool, qkv.dtype)
+        _gpu("k_pool", k_pool, data_dtype)
+        _gpu("v_pool", v_pool, data_dtype)
         _gpu("block_tables", block_tables, I32)
         _check_pools(k_pool, v_pool, G, page_size, d)
         _need(block_tables.dim() == 2, "block_tables must be [segments, max_blocks]")
         max_blocks = block_tables.shape[1]
     check(library("attention").kappai_qk_norm_rope_store(
-        _ptr(qkv), _c_int(qkv.stride(0)), _ptr(q_norm_w), _ptr(k_norm_w), _c_float(eps), _ptr(cos),
+        _ptr(None if parts is not None else qkv), _c_int(row_stride), _ptr(q_norm_w),
+        _ptr(k_norm_w), _c_float(eps), _ptr(cos),
         _ptr(sin), _c_int(rot_dim if rot_mode else 0), _c_int(rot_mode), _ptr(k_pool),
         _ptr(v_pool), _ptr(row_pos), _ptr(row_seg), _ptr(block_tables if store_kv else None),
         _c_int(max_blocks), _c_int(T), _c_int(H), _c_int(G), _c_int(d), _c_int(page_size),
-        _c_int(1 if store_kv else 0), _c_int(_is_bf16(qkv.dtype)), _stream()),
-        "qk_norm_rope_store")
+        _c_int(1 if store_kv else 0), _c_int(_is_bf16(data_dtype)), _ptr(parts),
+        _c_int(parts.shape[0] if parts is not None else 0), _ptr(q_out),
+        _c_int(H * d), _stream()), "qk_norm_rope_store")
+    return qkv if parts is None else q_out
 
 
 def paged_attention(q: torch.Tensor, n_heads: int, n_kv_heads: int, head_dim: int,

@@ -69,15 +69,18 @@ class GroupedQueryAttention(Mixer):
 
     def forward(self, x, batch, cache, shared_cache: bool = False):
         H, G, d = self.H, self.G, self.d
-        proj = (self.q_only if shared_cache else self.qkv).forward(x)
+        # decode: the projection may come as sums over ranges of its input dimension (more
+        # blocks stream the matrix), which the next kernel adds up
+        proj = (self.q_only if shared_cache else self.qkv).forward(
+            x, partial_sums=batch.max_segment_rows == 1)
         rot = self.position.rotation(x.device, batch.max_position) if self.position else None
         tables = batch.block_tables[cache.group]
-        ops.qk_norm_rope_store(
+        q = ops.qk_norm_rope_store(
             proj, H, G, d, self.q_norm_w, self.k_norm_w, self.qk_norm_eps or 0.0,
             rot.cos if rot else None, rot.sin if rot else None, rot.rot_dim if rot else 0,
             rot.mode if rot else ops.ROT_NONE, cache.k_pool, cache.v_pool, batch.row_pos,
             batch.row_seg, tables, cache.page_size, store_kv=not shared_cache)
-        ctx = ops.paged_attention(proj, H, G, d, cache.k_pool, cache.v_pool, batch.row_pos,
+        ctx = ops.paged_attention(q, H, G, d, cache.k_pool, cache.v_pool, batch.row_pos,
                                   batch.row_seg, tables, cache.page_size, self.scale,
                                   window=self.window or 0, q_tiles=batch.q_tiles,
                                   single_rows=batch.max_segment_rows == 1,

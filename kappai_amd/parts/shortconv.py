@@ -70,7 +70,9 @@ class GatedShortConv(Mixer):
             y = ops.linear_shortconv_step(x, w, self.in_proj.bias, self.taps, self.conv_bias,
                                           cache.state, batch.seg_pos0, batch.seg_slot)
             return self.out_proj.forward(y, partial_sums=True)
-        proj = self.in_proj.forward(x)
+        # decode: the projection may come as sums over ranges of its input dimension (more
+        # blocks stream the matrix), which the step kernel adds up
+        proj = self.in_proj.forward(x, partial_sums=batch.max_segment_rows == 1)
         y = ops.shortconv(proj, self.taps, self.conv_bias, cache.state, batch.row_seg,
                           batch.seg_start, batch.seg_pos0, batch.seg_slot)
         return self.out_proj.forward(y, partial_sums=True)

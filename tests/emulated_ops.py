@@ -129,7 +129,7 @@ def qk_norm_rope_store(qkv, n_heads, n_kv_heads, head_dim, q_norm_w, k_norm_w, e
     q = norm_rot(qkv[:, :H * d].to(F32).reshape(T, H, d), q_norm_w)
     qkv[:, :H * d] = q.reshape(T, H * d).to(qkv.dtype)
     if not store_kv:
-        return
+        return qkv
     k = norm_rot(qkv[:, H * d:(H + G) * d].to(F32).reshape(T, G, d), k_norm_w)
     v = qkv[:, (H + G) * d:(H + 2 * G) * d].reshape(T, G, d)
     for t in range(T):
@@ -138,6 +138,7 @@ def qk_norm_rope_store(qkv, n_heads, n_kv_heads, head_dim, q_norm_w, k_norm_w, e
         assert page >= 0, "a row is stored into a page that was given back"
         k_pool[page, :, p % page_size, :] = k[t].to(k_pool.dtype)
         v_pool[page, :, :, p % page_size] = v[t].to(v_pool.dtype)
+    return qkv
 
 
 def paged_attention(q, n_heads, n_kv_heads, head_dim, k_pool, v_pool, row_pos, row_seg,

@@ -460,6 +460,71 @@ def test_store_and_attention(ops, dtype, case):
         close(got.float(), want, tol * 2, f"attention kernel {kernel}")
 
 
+@pytest.mark.parametrize("case", ATT_CASES)
+@pytest.mark.parametrize("n_parts", [1, 3])
+def test_store_from_partial_sums(ops, case, n_parts):
+    """The projection handed over as float partial sums (a product split over its input
+    dimension): the same q, keys and values as from their bfloat16 sum."""
+    H, G, d, ps, before, new, rot_dim, mode, norm, window = case
+    c = paged_case(7, BF16, H, G, d, ps, before, new)
+    qn = (1 + rand((d,), F32, 30, 0.2)) if norm else None
+    kn = (1 + rand((d,), F32, 31, 0.2)) if norm else None
+    cos, sin = rope_tables(max(a + b for a, b in zip(before, new)) + 1, rot_dim or 2)
+    T, W = c["qkv"].shape
+    parts = rand((n_parts, T, W), F32, 32)
+    total = parts[0].clone()
+    for i in range(1, n_parts):
+        total += parts[i]
+    qkv = total.to(BF16)
+    dev = {k: (v.to(DEV) if torch.is_tensor(v) else v) for k, v in c.items()}
+    args = (H, G, d, None if qn is None else qn.to(DEV), None if kn is None else kn.to(DEV), 1e-5,
+            cos.to(DEV), sin.to(DEV), rot_dim, mode)
+    k2, v2 = dev["k_pool"].clone(), dev["v_pool"].clone()
+    q_parts = ops.qk_norm_rope_store(parts.to(DEV), *args, dev["k_pool"], dev["v_pool"],
+                                     dev["row_pos"], dev["row_seg"], dev["bt"], ps)
+    q_whole = ops.qk_norm_rope_store(qkv.to(DEV), *args, k2, v2, dev["row_pos"], dev["row_seg"],
+                                     dev["bt"], ps)
+    assert q_parts.shape == (T, H * d) and q_parts.dtype == BF16
+    assert torch.equal(q_parts.cpu(), q_whole[:, :H * d].cpu()), "q"
+    nan = lambda t: torch.nan_to_num(t.float().cpu(), nan=-7.0)
+    assert torch.equal(nan(dev["k_pool"]), nan(k2)), "k pages"
+    assert torch.equal(nan(dev["v_pool"]), nan(v2)), "v pages"
+    # and q alone, for a layer that reads another layer's keys
+    q_only = ops.qk_norm_rope_store(parts[:, :, :H * d].contiguous().to(DEV), *args, None, None,
+                                    dev["row_pos"], dev["row_seg"], dev["bt"], ps, store_kv=False)
+    assert torch.equal(q_only.cpu(), q_parts.cpu())
+
+
+@pytest.mark.parametrize("D,L,bias", [(8, 2, False), (304, 3, True), (2048, 3, False), (33, 5, True)])
+@pytest.mark.parametrize("n_parts", [1, 2, 4])
+def test_shortconv_step_from_partial_sums(ops, D, L, bias, n_parts):
+    """The decode step of the short convolution from float partial sums of the projection: the
+    same output and state as from their bfloat16 sum, over two steps."""
+    M, slots = 9, 12
+    taps, cb = rand((D, L), F32, 70, 0.5), (rand((D,), F32, 71, 0.3) if bias else None)
+    state0 = rand((slots, D, L - 1), F32, 72)
+    slot = torch.randperm(slots, generator=torch.Generator().manual_seed(4))[:M].to(torch.int32)
+    st_p, st_w = state0.to(DEV).clone(), state0.to(DEV).clone()
+    seg = torch.arange(M, dtype=torch.int32).to(DEV)
+    seg_start = torch.arange(M + 1, dtype=torch.int32).to(DEV)
+    dev = lambda t: None if t is None else t.to(DEV)
+    for step in range(2):
+        pos0 = ((torch.arange(M, dtype=torch.int32) % 3) + step).to(DEV)      # some rows start fresh
+        parts = rand((n_parts, M, 3 * D), F32, 73 + step)
+        total = parts[0].clone()
+        for i in range(1, n_parts):
+            total += parts[i]
+        got = ops.shortconv(parts.to(DEV), taps.to(DEV), dev(cb), st_p, seg, seg_start, pos0,
+                            slot.to(DEV))
+        want = ops.shortconv(total.to(BF16).to(DEV), taps.to(DEV), dev(cb), st_w, seg, seg_start,
+                             pos0, slot.to(DEV))
+        assert got.dtype == BF16 and torch.equal(got.cpu(), want.cpu()), f"step {step}"
+        assert torch.equal(st_p.cpu(), st_w.cpu()), f"state after step {step}"
+    with pytest.raises(ValueError, match="single row"):
+        ops.shortconv(parts.to(DEV), taps.to(DEV), dev(cb), st_p, seg, seg_start[:5], pos0[:4],
+                      slot[:4].to(DEV))
+
+
 @pytest.mark.parametrize("dtype", [F32, BF16])
 def test_attention_finds_one_far_key(ops, dtype):
     """Among 700 keys one is made to match the query: the output must be its value.  A kernel
