@@ -130,53 +130,181 @@ extern "C" int kappai_repeat_penalty(float* logits, const int* row_start, const 
 // (top-k, or the best 1024 when only top-p / min-p narrow), sorted by descending logit;
 // softmax of logit/T in float; top-p keeps the token that crosses the mass; min-p is relative
 // to the best; inverse-CDF draw at the row's uniform over what is left.  One block per row:
-// radix select of the keep-th largest value, gather, bitonic sort in LDS, then one thread walks
-// the (at most 1024) candidates in the reference's order of operations.
+// radix select of the keep-th largest value, gather, bitonic sort in LDS, then the (at most
+// 1024) candidates in the reference's order of operations: the exponentials and quotients are
+// computed by all threads, the running sums by one.
+//
+// Every wave owns a contiguous part of the row and reads it 256 values a step (16 bytes a
+// lane).  Logits share their high bits, so in the first radix pass all lanes add to a handful
+// of counters: the digits are 11 bits wide (sign, exponent and two bits of the mantissa in the
+// first) and every counter exists 4 times (lane % 4, in different LDS banks).
 // ---------------------------------------------------------------------------------------
 #define FILT_THREADS 1024
+#define FILT_WAVES (FILT_THREADS / WAVE)
 #define FILT_MAX_KEEP 1024
+#define FILT_BINS 2048
+#define FILT_SUBS 4
 
 __device__ __forceinline__ uint32_t order_key(float f) {   // larger float -> larger key
   const uint32_t u = __float_as_uint(f);
   return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
 }
+__device__ __forceinline__ float key_value(uint32_t k) {   // the float a key came from
+  return __uint_as_float((k & 0x80000000u) ? (k ^ 0x80000000u) : ~k);
+}
 
+// p(e) = exp(l_e/T - max/T) and q(e) = p(e) / sum of the candidates in descending order: top-p
+// keeps the token that crosses the mass, min-p is relative to the best, then the inverse-CDF
+// draw at u over what is left (src/sampler.c:271-332).  Returns the place of the chosen one.
+template <typename P, typename Q>
+__device__ __forceinline__ int narrow_and_draw(P&& p, Q&& q, int keep, float tp, float mp,
+                                               float u) {
+  int kept = keep;
+  if (tp < 1.0f) {
+    float cum = 0.f;
+    for (int e = 0; e < keep; ++e) {
+      cum += q(e);
+      if (cum > tp) { kept = e + 1; break; }
+    }
+  }
+  if (mp > 0.f) {
+    const float floor_p = mp * q(0);
+    int n = 0;
+    while (n < kept && q(n) >= floor_p) ++n;
+    kept = n > 0 ? n : 1;
+  }
+  float psum = 0.f;
+  for (int e = 0; e < kept; ++e) psum += p(e);
+  const float target = u * psum;
+  float acc = 0.f;
+  for (int e = 0; e < kept; ++e) {
+    acc += p(e);
+    if (target < acc) return e;
+  }
+  return kept - 1;
+}
+
+// CACHED: the row has at most FILT_THREADS * 4 * FILT_STEPS values, and every lane keeps its
+// share of the row (4 values of each of the wave's steps) in registers from the first read on.
+#define FILT_STEPS 16
+template <bool CACHED>
 __global__ __launch_bounds__(FILT_THREADS) void sample_filtered_kernel(
     const float* __restrict__ logits, const int* __restrict__ rows, const int* __restrict__ keep_n,
     const float* __restrict__ temperature, const float* __restrict__ top_p,
     const float* __restrict__ min_p, const float* __restrict__ uniform, int* __restrict__ out,
     int V) {
-  __shared__ uint32_t hist[256];
+  __shared__ uint32_t hist_p[FILT_BINS][FILT_SUBS];
+  __shared__ uint32_t hist[FILT_BINS];
   __shared__ uint32_t sh_prefix, sh_remaining, sh_count;
-  __shared__ uint32_t scan[FILT_THREADS];
+  __shared__ uint32_t wave_ties[FILT_WAVES];
   __shared__ float cval[FILT_MAX_KEEP];
+  __shared__ float cq[FILT_MAX_KEEP];
   __shared__ int cidx[FILT_MAX_KEEP];
+  __shared__ float sh_sum;
   const int i = blockIdx.x, tid = threadIdx.x;
+  const int lane = tid % WAVE, wave = tid / WAVE;
   const float* lg = logits + (size_t)rows[i] * V;
   const int keep = min(min(keep_n[i], V), FILT_MAX_KEEP);
 
-  // ---- the keep-th largest key, byte by byte from the top --------------------------------
+  // the wave's part of the row, a whole number of 256-value steps
+  const int region = (((V + FILT_WAVES - 1) / FILT_WAVES) + 255) / 256 * 256;
+  const int w0 = min(wave * region, V), w1 = min(w0 + region, V);
+  const bool vec = V % 4 == 0 && (reinterpret_cast<uintptr_t>(lg) % 16) == 0;
+  // keys of the values base + 4 lane + (0..3) of a step; 0 (below every number's key) past the
+  // end of the part
+  auto load4 = [&](int base, uint32_t (&k)[4]) {
+    const int idx = base + 4 * lane;
+    if (vec) {
+      const bool in = idx < w1;          // V and the parts are multiples of 4
+      float4 q = {0.f, 0.f, 0.f, 0.f};
+      if (in) q = *reinterpret_cast<const float4*>(lg + idx);
+      k[0] = in ? order_key(q.x) : 0u;
+      k[1] = in ? order_key(q.y) : 0u;
+      k[2] = in ? order_key(q.z) : 0u;
+      k[3] = in ? order_key(q.w) : 0u;
+    } else {
+#pragma unroll
+      for (int c = 0; c < 4; ++c) k[c] = idx + c < w1 ? order_key(lg[idx + c]) : 0u;
+    }
+  };
+  // every step of the wave's part in turn: f(first index of the step, this lane's four keys)
+  uint32_t held[CACHED ? FILT_STEPS : 1][4];
+  if (CACHED) {
+#pragma unroll
+    for (int st = 0; st < FILT_STEPS; ++st) load4(w0 + 256 * st, held[st]);
+  }
+  auto each_step = [&](auto&& f) {
+    if (CACHED) {
+#pragma unroll
+      for (int st = 0; st < FILT_STEPS; ++st) f(w0 + 256 * st, held[st]);
+    } else {
+      for (int base = w0; base < w1; base += 256) {
+        uint32_t k[4];
+        load4(base, k);
+        f(base, k);
+      }
+    }
+  };
+
+  // ---- the keep-th largest key, 11, 11 and 10 bits at a time from the top ------------------
   if (tid == 0) { sh_prefix = 0; sh_remaining = keep; }
-  __syncthreads();
-  for (int shift = 24; shift >= 0; shift -= 8) {
-    if (tid < 256) hist[tid] = 0;
+#pragma unroll 1
+  for (int pass = 0; pass < 3; ++pass) {
+    const int shift = pass == 0 ? 21 : (pass == 1 ? 10 : 0);
+    const uint32_t digit = pass == 2 ? 0x3ffu : 0x7ffu;
+    for (int e = tid; e < FILT_BINS * FILT_SUBS; e += FILT_THREADS) (&hist_p[0][0])[e] = 0;
     __syncthreads();
     const uint32_t prefix = sh_prefix;
-    const uint32_t mask = shift == 24 ? 0u : (0xffffffffu << (shift + 8));
-    for (int e = tid; e < V; e += FILT_THREADS) {
-      const uint32_t k = order_key(lg[e]);
-      if ((k & mask) == prefix) atomicAdd(&hist[(k >> shift) & 0xff], 1u);
+    const uint32_t mask = pass == 0 ? 0u : (0xffffffffu << (pass == 1 ? 21 : 10));
+    uint32_t* mine = &hist_p[0][lane % FILT_SUBS];
+    each_step([&](int base, const uint32_t (&k)[4]) {
+      // after the first pass few values still match the prefix: one test for the lane's four
+      bool hit[4];
+#pragma unroll
+      for (int c = 0; c < 4; ++c) hit[c] = k[c] != 0u && (k[c] & mask) == prefix;
+      if (!(hit[0] || hit[1] || hit[2] || hit[3])) return;
+#pragma unroll
+      for (int c = 0; c < 4; ++c)
+        if (hit[c]) atomicAdd(mine + ((k[c] >> shift) & digit) * FILT_SUBS, 1u);
+    });
+    __syncthreads();
+    for (int bin = tid; bin < FILT_BINS; bin += FILT_THREADS) {
+      uint32_t sum = 0;
+#pragma unroll
+      for (int sub = 0; sub < FILT_SUBS; ++sub) sum += hist_p[bin][sub];
+      hist[bin] = sum;
     }
     __syncthreads();
-    if (tid == 0) {
-      uint32_t rem = sh_remaining, above = 0;
-      int b = 255;
-      for (; b > 0; --b) {
-        if (above + hist[b] >= rem) break;
-        above += hist[b];
+    if (wave == 0) {
+      // the largest bin b whose count together with all bins above it reaches what is still
+      // wanted: lane holds bins PER lane .. PER lane + PER - 1; sums from the top by a suffix
+      // scan over the lanes
+      constexpr int PER = FILT_BINS / WAVE;
+      uint32_t mine_sum = 0;
+      for (int j = 0; j < PER; ++j) mine_sum += hist[PER * lane + j];
+      uint32_t suf = mine_sum;
+#pragma unroll
+      for (int off = 1; off < WAVE; off <<= 1) {
+        const uint32_t o = __shfl_down(suf, off, WAVE);
+        if (lane + off < WAVE) suf += o;
       }
-      sh_prefix = prefix | ((uint32_t)b << shift);
-      sh_remaining = rem - above;
+      const uint32_t rem = sh_remaining;
+      // count of the bins >= b falls with b: the bins that reach `rem` are 0..cnt-1
+      int cnt = 0;
+      uint32_t from = suf;                 // count of bins >= PER lane + j
+      for (int j = 0; j < PER; ++j) {
+        cnt += from >= rem ? 1 : 0;
+        from -= hist[PER * lane + j];
+      }
+#pragma unroll
+      for (int m = WAVE / 2; m > 0; m >>= 1) cnt += __shfl_xor(cnt, m, WAVE);
+      const int b = max(cnt - 1, 0);
+      if (lane == b / PER) {
+        uint32_t above = suf;              // count of bins > b
+        for (int j = 0; j <= b % PER; ++j) above -= hist[PER * lane + j];
+        sh_prefix = prefix | ((uint32_t)b << shift);
+        sh_remaining = rem - above;
+      }
     }
     __syncthreads();
   }
@@ -185,44 +313,87 @@ __global__ __launch_bounds__(FILT_THREADS) void sample_filtered_kernel(
   // ---- gather: everything above the threshold, then the first ties in index order ---------
   if (tid == 0) sh_count = 0;
   __syncthreads();
-  const int chunk = (V + FILT_THREADS - 1) / FILT_THREADS;
-  const int e0 = min(tid * chunk, V), e1 = min(e0 + chunk, V);
   uint32_t my_ties = 0;
-  for (int e = e0; e < e1; ++e) {
-    const float v = lg[e];
-    const uint32_t k = order_key(v);
-    if (k > thr) {
-      const uint32_t slot = atomicAdd(&sh_count, 1u);
-      cval[slot] = v;
-      cidx[slot] = e;
-    } else if (k == thr) {
-      ++my_ties;
-    }
-  }
-  scan[tid] = my_ties;
-  __syncthreads();
-  for (int off = 1; off < FILT_THREADS; off <<= 1) {
-    const uint32_t add = tid >= off ? scan[tid - off] : 0u;
-    __syncthreads();
-    scan[tid] += add;
-    __syncthreads();
-  }
-  {
-    const uint32_t n_above = sh_count;
-    uint32_t rank = scan[tid] - my_ties;      // ties before this thread's range
-    for (int e = e0; e < e1 && rank < n_ties; ++e) {
-      const float v = lg[e];
-      if (order_key(v) == thr) {
-        cval[n_above + rank] = v;
-        cidx[n_above + rank] = e;
-        ++rank;
+  each_step([&](int base, const uint32_t (&k)[4]) {
+    if (max(max(k[0], k[1]), max(k[2], k[3])) < thr) return;      // the usual case
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      if (k[c] > thr) {                     // thr is a number's key: above the 0 of the padding
+        const uint32_t slot = atomicAdd(&sh_count, 1u);
+        cval[slot] = key_value(k[c]);
+        cidx[slot] = base + 4 * lane + c;
+      } else if (k[c] == thr) {
+        ++my_ties;
       }
+    }
+  });
+#pragma unroll
+  for (int m = WAVE / 2; m > 0; m >>= 1) my_ties += __shfl_xor(my_ties, m, WAVE);
+  if (lane == 0) wave_ties[wave] = my_ties;
+  __syncthreads();
+  {
+    const uint32_t n_above = sh_count;      // = keep - n_ties
+    uint32_t running = 0;                   // ties in the parts before this wave's
+    for (int w = 0; w < wave; ++w) running += wave_ties[w];
+    if (my_ties > 0 && running < n_ties) {
+      // index order inside a step: lane, then the lane's four values
+      const uint64_t below = lane == 0 ? 0ull : (~0ull >> (WAVE - lane));
+      each_step([&](int base, const uint32_t (&k)[4]) {
+        if (running >= n_ties) return;
+        uint32_t before = 0, in_step = 0;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+          const uint64_t m = __ballot(k[c] == thr);
+          before += (uint32_t)__popcll(m & below);
+          in_step += (uint32_t)__popcll(m);
+        }
+        uint32_t r = running + before;
+#pragma unroll
+        for (int c = 0; c < 4; ++c)
+          if (k[c] == thr) {
+            if (r < n_ties) {
+              cval[n_above + r] = key_value(thr);
+              cidx[n_above + r] = base + 4 * lane + c;
+            }
+            ++r;
+          }
+        running += in_step;
+      });
     }
   }
   __syncthreads();
   // pad to a power of two for the sort
   int n2 = 1;
   while (n2 < keep) n2 <<= 1;
+  if (n2 <= WAVE) {
+    // few candidates (the usual top-k): the first wave sorts them in registers, one a lane, and
+    // finishes alone, without block barriers
+    if (wave != 0) return;
+    float v = lane < keep ? cval[lane] : -INFINITY;
+    int id = lane < keep ? cidx[lane] : 0x7fffffff;
+    for (int k = 2; k <= n2; k <<= 1)
+      for (int j = k >> 1; j > 0; j >>= 1) {
+        const float ov = __shfl_xor(v, j, WAVE);
+        const int oi = __shfl_xor(id, j, WAVE);
+        const bool lower = (lane & j) == 0, desc = (lane & k) == 0;
+        const bool mine_first = v > ov || (v == ov && id < oi);
+        const bool keep_mine = lower ? (mine_first == desc) : (mine_first != desc);
+        if (!keep_mine) { v = ov; id = oi; }
+      }
+    // lane e holds candidate e; the running sums go through the lanes in order, every lane
+    // computing the same
+    const float inv_t = 1.0f / temperature[i];
+    const float mx = __shfl(v, 0, WAVE) * inv_t;
+    const float p = expf(v * inv_t - mx);
+    auto p_of = [&](int e) { return __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(p), e)); };
+    float sum = 0.f;
+    for (int e = 0; e < keep; ++e) sum += p_of(e);
+    const float q = p / sum;
+    auto q_of = [&](int e) { return __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(q), e)); };
+    const int pick = narrow_and_draw(p_of, q_of, keep, top_p[i], min_p[i], uniform[i]);
+    if (lane == 0) out[rows[i]] = __builtin_amdgcn_readlane(id, pick);
+    return;
+  }
   for (int e = keep + tid; e < n2; e += FILT_THREADS) { cval[e] = -INFINITY; cidx[e] = 0x7fffffff; }
   __syncthreads();
   // ---- bitonic sort: descending value, ascending index on ties ----------------------------
@@ -238,43 +409,23 @@ __global__ __launch_bounds__(FILT_THREADS) void sample_filtered_kernel(
       }
       __syncthreads();
     }
-  // ---- one thread: temperature, top-p, min-p, draw (float, in the reference's order) -------
+  // ---- temperature, top-p, min-p, draw (float, in the reference's order) -------------------
+  const float inv_t = 1.0f / temperature[i];
+  const float mx = cval[0] * inv_t;
+  __syncthreads();
+  if (tid < keep) cval[tid] = expf(cval[tid] * inv_t - mx);
+  __syncthreads();
   if (tid == 0) {
-    const float inv_t = 1.0f / temperature[i];
-    const float mx = cval[0] * inv_t;
     float sum = 0.f;
-    for (int e = 0; e < keep; ++e) {
-      const float p = expf(cval[e] * inv_t - mx);
-      cval[e] = p;
-      sum += p;
-    }
-    int kept = keep;
-    const float tp = top_p[i];
-    if (tp < 1.0f) {
-      float cum = 0.f;
-      for (int e = 0; e < keep; ++e) {
-        cum += cval[e] / sum;
-        if (cum > tp) { kept = e + 1; break; }
-      }
-    }
-    const float mp = min_p[i];
-    if (mp > 0.f) {
-      const float floor_p = mp * (cval[0] / sum);
-      int n = 0;
-      while (n < kept && (cval[n] / sum) >= floor_p) ++n;
-      kept = n > 0 ? n : 1;
-    }
-    float psum = 0.f;
-    for (int e = 0; e < kept; ++e) psum += cval[e];
-    const float target = uniform[i] * psum;
-    float acc = 0.f;
-    int pick = kept - 1;
-    for (int e = 0; e < kept; ++e) {
-      acc += cval[e];
-      if (target < acc) { pick = e; break; }
-    }
-    out[rows[i]] = cidx[pick];
+    for (int e = 0; e < keep; ++e) sum += cval[e];
+    sh_sum = sum;
   }
+  __syncthreads();
+  if (tid < keep) cq[tid] = cval[tid] / sh_sum;
+  __syncthreads();
+  if (tid == 0)
+    out[rows[i]] = cidx[narrow_and_draw([&](int e) { return cval[e]; }, [&](int e) { return cq[e]; },
+                                        keep, top_p[i], min_p[i], uniform[i])];
 }
 
 // rows[i] names the row of `logits` (and of `out`) that entry i samples for; keep_n[i] <= 1024.
@@ -284,7 +435,11 @@ extern "C" int kappai_sample_filtered(const float* logits, const int* rows, cons
                                       int n_entries, int V, hipStream_t stream) {
   if (n_entries <= 0) return 0;
   if (V < 1) return (int)hipErrorInvalidValue;
-  hipLaunchKernelGGL(sample_filtered_kernel, dim3(n_entries), dim3(FILT_THREADS), 0, stream,
-                     logits, rows, keep_n, temperature, top_p, min_p, uniform, out, V);
+  if (V <= FILT_THREADS * 4 * FILT_STEPS)
+    hipLaunchKernelGGL(sample_filtered_kernel<true>, dim3(n_entries), dim3(FILT_THREADS), 0, stream,
+                       logits, rows, keep_n, temperature, top_p, min_p, uniform, out, V);
+  else
+    hipLaunchKernelGGL(sample_filtered_kernel<false>, dim3(n_entries), dim3(FILT_THREADS), 0,
+                       stream, logits, rows, keep_n, temperature, top_p, min_p, uniform, out, V);
   KAPPAI_RETURN_LAUNCH_STATUS();
 }
