@@ -609,10 +609,11 @@ def test_sample_rows(ops):
 
 def test_sample_filtered(ops):
     """The candidate-narrowing draw against the plain sampler, row by row: default options,
-    top-k only, top-p only, min-p only, ties in the logits, a vocabulary below the cap."""
+    top-k only, top-p only, min-p only, ties in the logits, a vocabulary below the cap, and
+    vocabularies above the 65,536 values that the kernel keeps in registers."""
     from plain import sampler as plain_sampler
     rng = np.random.default_rng(5)
-    for V in (65536, 1003, 300):
+    for V in (65536, 1003, 300, 70001, 131072):
         n = 12
         logits = (rng.normal(size=(n, V)) * 3).astype(np.float32)
         logits[1, :50] = logits[1, 0]                      # many equal values at the top-k edge
