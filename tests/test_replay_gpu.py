@@ -266,3 +266,48 @@ def test_decode_steps_of_forty_requests(tmp_path, dtype):
         assert len(got) == n_req * (n_decode + 1)
         err, where = worst_error(got, ref)
         assert err < tol, (group, err, tol, where, first_bad(got, ref, tol))
+
+
+# The layer sizes of LFM2-1.2B (width 2048, 32 query heads over 8 kv heads of size 64, feed-forward
+# 8192 from intermediate_size 12288, 65,536 tokens) with three of its sixteen layers, so that the
+# plain implementation in float64 stays a matter of seconds: the kernels run at the shapes that
+# the benchmark measures.
+SIZES_1_2B = {
+    "architectures": ["Lfm2ForCausalLM"], "model_type": "lfm2", "hidden_size": 2048,
+    "num_hidden_layers": 3, "layer_types": ["conv", "full_attention", "conv"],
+    "num_attention_heads": 32, "num_key_value_heads": 8, "head_dim": 64,
+    "intermediate_size": 12288, "block_auto_adjust_ff_dim": True, "block_multiple_of": 256,
+    "block_ffn_dim_multiplier": 1.0, "vocab_size": 65536, "norm_eps": 1e-5,
+    "rope_theta": 1000000.0, "conv_L_cache": 3, "conv_bias": False, "tie_embedding": True,
+    "max_position_embeddings": 128000,
+}
+
+
+@pytest.fixture(scope="module")
+def sizes_1_2b_dir(tmp_path_factory):
+    import copy
+    from kappai_amd.config import config_from_dict
+    from kappai_amd.weights import write_random_model
+    cfg = config_from_dict(copy.deepcopy(SIZES_1_2B))
+    assert cfg.ff_dim == 8192
+    return write_random_model(tmp_path_factory.mktemp("sizes") / "m", cfg, seed=8, std=0.02,
+                              norm_jitter=0.05)
+
+
+@pytest.mark.parametrize("dtype", ["bfloat16", "float32"])
+def test_layer_sizes_of_the_1_2b_model(tmp_path, sizes_1_2b_dir, dtype):
+    """A prompt of 150 tokens in one step and cut in three, a second request beside it, then
+    decoded tokens of both side by side, at the layer sizes of LFM2-1.2B."""
+    folder = sizes_1_2b_dir
+    requests = make_requests(SIZES_1_2B["vocab_size"], [158, 97, 158], seed=17)
+    requests["r2"] = list(requests["r0"])          # the same tokens, cut differently
+    plans = {"r0": (0, [150] + [1] * 8), "r1": (1, [70, 19] + [1] * 8),
+             "r2": (2, [64, 2, 84] + [1] * 8)}
+    steps, index, peak = schedules.build(requests, plans, want="last")
+    got = replay_in_process(folder, dtype, steps, index, peak, tmp_path / "out")
+    ref = plain_logits(folder, requests)
+    tol = tolerance(folder, requests, dtype)
+    assert len(got) == sum(len(p) for _, p in plans.values())
+    err, where = worst_error(got, ref)
+    assert err < tol, (err, tol, where, first_bad(got, ref, tol))
+    _models.pop((str(folder), dtype), None)        # 0.7 to 1.3 GB on the GPU
