@@ -161,10 +161,7 @@ def split_k_for(M: int, N: int, K: int) -> int:
         if split >= 1 and K % (512 * split) == 0 and ((N + 63) // 64) * split >= 128:
             return split
     col_groups = (N + 15) // 16
-    want = 512 // col_groups
-    if want < 2 and col_groups <= 448:
-        want = 2        # measured: 6144 x 2048 in 8.3 us in two ranges, 9.7 us in one
-    return max(1, min(8, want, K // 512))
+    return max(1, min(8, 512 // col_groups, K // 512))
 
 
 def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,

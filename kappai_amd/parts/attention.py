@@ -19,7 +19,7 @@ from ..cache.specs import PagedKV
 from ..kernels import ops
 from ..weights.spec import INIT_ONES, VECTOR, TensorSpec
 from .base import Mixer, PositionEncoding, register_part
-from .linear import Linear
+from .linear import PARTIAL_SUMS_MIN_ROWS, Linear
 
 
 class GroupedQueryAttention(Mixer):
@@ -69,10 +69,10 @@ class GroupedQueryAttention(Mixer):
 
     def forward(self, x, batch, cache, shared_cache: bool = False):
         H, G, d = self.H, self.G, self.d
-        # decode: the projection may come as sums over ranges of its input dimension (more
-        # blocks stream the matrix), which the next kernel adds up
+        # decode with more than 16 rows: the projection may come as sums over ranges of its input
+        # dimension (more blocks stream the matrix), which the next kernel adds up
         proj = (self.q_only if shared_cache else self.qkv).forward(
-            x, partial_sums=batch.max_segment_rows == 1)
+            x, partial_sums=batch.max_segment_rows == 1 and x.shape[0] > PARTIAL_SUMS_MIN_ROWS)
         rot = self.position.rotation(x.device, batch.max_position) if self.position else None
         tables = batch.block_tables[cache.group]
         q = ops.qk_norm_rope_store(

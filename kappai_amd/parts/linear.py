@@ -11,6 +11,12 @@ from ..weights.spec import INIT_NORMAL, INIT_SMALL, MATRIX, VECTOR, TensorSpec
 from .base import Part
 
 
+# A projection whose consumer can add partial sums asks for them only above this many rows:
+# measured on the 1.2B shape, 6144 x 2048 plus the conv step takes 13.0 us unsplit and 13.3 us
+# in two K ranges at 8 rows, 18 us and 12 us at 64 rows.
+PARTIAL_SUMS_MIN_ROWS = 16
+
+
 class Linear(Part):
     """One or several matrices of the checkpoint that share their input, run as ONE
     product: the matrices are stacked along their output dimension when they are bound

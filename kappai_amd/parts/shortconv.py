@@ -16,7 +16,7 @@ from ..cache.specs import FixedState
 from ..kernels import ops
 from ..weights.spec import INIT_NORMAL, INIT_SMALL, VECTOR, TensorSpec
 from .base import Mixer, register_part
-from .linear import Linear
+from .linear import PARTIAL_SUMS_MIN_ROWS, Linear
 
 
 # The fused decode kernel gives one block 16 channels; below this width it has too few blocks to
@@ -70,9 +70,11 @@ class GatedShortConv(Mixer):
             y = ops.linear_shortconv_step(x, w, self.in_proj.bias, self.taps, self.conv_bias,
                                           cache.state, batch.seg_pos0, batch.seg_slot)
             return self.out_proj.forward(y, partial_sums=True)
-        # decode: the projection may come as sums over ranges of its input dimension (more
-        # blocks stream the matrix), which the step kernel adds up
-        proj = self.in_proj.forward(x, partial_sums=batch.max_segment_rows == 1)
+        # decode with more than 16 rows: the projection may come as sums over ranges of its input
+        # dimension (more blocks stream the matrix), which the step kernel adds up; with fewer
+        # rows the unsplit product and the plain step are as fast or faster
+        proj = self.in_proj.forward(
+            x, partial_sums=batch.max_segment_rows == 1 and x.shape[0] > PARTIAL_SUMS_MIN_ROWS)
         y = ops.shortconv(proj, self.taps, self.conv_bias, cache.state, batch.row_seg,
                           batch.seg_start, batch.seg_pos0, batch.seg_slot)
         return self.out_proj.forward(y, partial_sums=True)

@@ -209,11 +209,13 @@ def test_long_prompt_on_a_wide_model(tmp_path, dtype):
 # Products with 17 to 64 rows and many rows of W run in a kernel of their own (activation rows
 # shared through LDS): hidden size and feed-forward width are multiples of 512 here, and gate/up
 # and the output head have 8192 rows, so a decode step of 40 requests takes it where a step of 8
-# takes the kernel for few rows.
+# takes the kernel for few rows.  With more than 16 rows in_proj and qkv are also split over
+# their input dimension (1024: two ranges) and the conv step and the qk-norm kernel add the
+# partial sums.
 MANY = {
     "architectures": ["Lfm2ForCausalLM"], "model_type": "lfm2",
-    "hidden_size": 512, "num_hidden_layers": 2, "layer_types": ["conv", "full_attention"],
-    "num_attention_heads": 8, "num_key_value_heads": 2, "head_dim": 64,
+    "hidden_size": 1024, "num_hidden_layers": 2, "layer_types": ["conv", "full_attention"],
+    "num_attention_heads": 16, "num_key_value_heads": 4, "head_dim": 64,
     "intermediate_size": 4096, "block_auto_adjust_ff_dim": False,
     "vocab_size": 8192, "norm_eps": 1e-5, "rope_theta": 10000.0,
     "conv_L_cache": 3, "conv_bias": False, "tie_embedding": True,
@@ -263,6 +265,8 @@ def test_decode_steps_of_forty_requests(tmp_path, dtype):
             for rid in part:
                 cache.close(caches[rid])
         cache.check()
+        from kappai_amd.kernels import ops
+        assert ops.split_k_for(40, 3 * MANY["hidden_size"], MANY["hidden_size"]) > 1
         assert len(got) == n_req * (n_decode + 1)
         err, where = worst_error(got, ref)
         assert err < tol, (group, err, tol, where, first_bad(got, ref, tol))
