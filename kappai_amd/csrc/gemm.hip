@@ -630,11 +630,30 @@ struct ConvStep {
   int L;
 };
 
-template <typename TO, int MT, int NW, int EPI, int NT>
+// PRO (at most NORM_ROWS rows, K <= NORM_MAX_K): the rows are not read from A but made here, by
+// every block for itself, as the RMSNorm of resid + delta (kappai: src/backend/cpu/scalar/
+// quants.c:1507-1512; delta absent, bfloat16, or n_parts float partial sums), with the thread
+// layout and the order of sums of add_rmsnorm_row_kernel, so that the kernel between two
+// products of a decode step is saved.  The first block also writes the updated residual to
+// resid_out, which must not be resid itself (the other blocks still read it).
+#define NORM_ROWS 4
+#define NORM_MAX_K 4096
+struct NormIn {
+  const float* resid;      // [M, K]
+  const void* delta;       // null, bf16 [M, K] or float [n_parts][M][K]
+  int n_parts;
+  int delta_f32;
+  const float* w;          // [K]
+  float eps;
+  float* resid_out;        // [M, K], or null when there is no delta
+};
+
+template <typename TO, int MT, int NW, int EPI, int NT, bool PRO = false>
 __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny_kernel(
     const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, const float* __restrict__ bias,
-    TO* __restrict__ C, int M, int N, int K, int lda, int ldc, ConvStep cs) {
+    TO* __restrict__ C, int M, int N, int K, int lda, int ldc, ConvStep cs, NormIn nin) {
   static_assert(NT == 1 || EPI == 0, "several column tiles a wave: plain products only");
+  static_assert(!PRO || (MT == 1 && NT == 1), "normalised rows: one row tile");
   // row groups of W a block streams: gate/up, the three conv gates, or NT column tiles
   constexpr int NG = EPI == 1 ? 2 : (EPI == 2 ? 3 : NT);
   __shared__ float red[NW][NG * MT][WAVE][4];
@@ -658,6 +677,52 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny_kernel(
     const int gm = t * 16 + col;
     arow[t] = A + (size_t)(gm < M ? gm : 0) * lda + kg;
   }
+  __shared__ __attribute__((aligned(16))) bf16_t xs[PRO ? NORM_ROWS : 1][PRO ? NORM_MAX_K : 8];
+  __shared__ float red16[PRO ? 16 : 1];
+  auto make_rows = [&]() {
+    const bool writer = blockIdx.x == 0 && blockIdx.y == 0 && nin.resid_out != nullptr;
+    for (int m = 0; m < M; ++m) {
+      const float* x = nin.resid + (size_t)m * K;
+      // one pass when the block has a thread for every 8 values (the usual case), else the
+      // values are made again after the sum of squares is known
+      float v[8], w8[8];
+      auto make = [&](int j) {
+        load8(x + j, v);
+        if (nin.delta && nin.delta_f32) {
+          const float* d = reinterpret_cast<const float*>(nin.delta) + (size_t)m * K + j;
+          for (int p = 0; p < nin.n_parts; ++p) {
+            float d8[8];
+            load8(d + (size_t)p * M * K, d8);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) v[e] += d8[e];
+          }
+        } else if (nin.delta) {
+          float d8[8];
+          load8(reinterpret_cast<const bf16_t*>(nin.delta) + (size_t)m * K + j, d8);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) v[e] += d8[e];
+        }
+      };
+      float ss = 0.f;
+      const int first = tid * 8;
+      for (int j = first; j < K; j += NW * WAVE * 8) {
+        make(j);
+        if (writer) store8(nin.resid_out + (size_t)m * K + j, v);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) ss += v[e] * v[e];
+      }
+      ss = block_sum(ss, red16);
+      const float scale = 1.0f / sqrtf(ss / (float)K + nin.eps);
+      for (int j = first; j < K; j += NW * WAVE * 8) {
+        if (K > NW * WAVE * 8) make(j);          // else v still holds the thread's only 8
+        load8(nin.w + j, w8);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) w8[e] = v[e] * scale * w8[e];
+        store8(&xs[m][j], w8);
+      }
+    }
+    __syncthreads();
+  };
   const int kblk = ((K + 32 * (int)gridDim.y - 1) / (32 * (int)gridDim.y)) * 32;   // K a block
   const int kb0 = blockIdx.y * kblk, kb1 = min(K, kb0 + kblk);
   const int kper = ((kb1 - kb0 + 32 * NW - 1) / (32 * NW)) * 32;
@@ -666,8 +731,7 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny_kernel(
   C += (size_t)blockIdx.y * M * ldc;
   // loads in flight a lane: U * (NG + MT)
   constexpr int U = (NG + MT) <= 3 ? SK_UNROLL : ((NG + MT) <= 6 ? 4 : 2);
-  for (int k = k0; k < k1; k += 32 * U) {
-    u32x4_t wv[U][NG], av[U][MT];
+  auto load_w = [&](int k, u32x4_t (&wv)[U][NG]) {
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int gk = k + 32 * u;
@@ -676,10 +740,24 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny_kernel(
       for (int r = 0; r < NG; ++r)
         wv[u][r] = (kin && gn + (EPI == 0 ? r * 16 : 0) < N) ? load16(wrow + r * group_rows * K + gk)
                                                                : zero;
-#pragma unroll
-      for (int t = 0; t < MT; ++t)
-        av[u][t] = (kin && t * 16 + col < M) ? load16(arow[t] + gk) : zero;
     }
+  };
+  auto load_a = [&](int k, u32x4_t (&av)[U][MT]) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int gk = k + 32 * u;
+      const bool kin = gk + kg < k1;
+#pragma unroll
+      for (int t = 0; t < MT; ++t) {
+        if constexpr (PRO)
+          av[u][t] = (kin && col < M) ? *reinterpret_cast<const u32x4_t*>(&xs[col % NORM_ROWS][gk + kg])
+                                      : zero;
+        else
+          av[u][t] = (kin && t * 16 + col < M) ? load16(arow[t] + gk) : zero;
+      }
+    }
+  };
+  auto products = [&](const u32x4_t (&wv)[U][NG], const u32x4_t (&av)[U][MT]) {
 #pragma unroll
     for (int u = 0; u < U; ++u)
 #pragma unroll
@@ -688,6 +766,36 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny_kernel(
         for (int t = 0; t < MT; ++t)
           acc[r * MT + t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
               as_bf16x8(av[u][t]), as_bf16x8(wv[u][r]), acc[r * MT + t], 0, 0, 0);
+  };
+  if constexpr (PRO) {
+    // the first loads of W are under way while the rows are made
+    u32x4_t wv[U][NG], av[U][MT];
+    load_w(k0, wv);
+    make_rows();
+    for (int k = k0; k < k1; k += 32 * U) {
+      if (k != k0) load_w(k, wv);
+      load_a(k, av);
+      products(wv, av);
+    }
+  } else {
+    for (int k = k0; k < k1; k += 32 * U) {
+      // the loads of W and of A alternate, in the order of K
+      u32x4_t wv[U][NG], av[U][MT];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int gk = k + 32 * u;
+        const bool kin = gk + kg < k1;
+#pragma unroll
+        for (int r = 0; r < NG; ++r)
+          wv[u][r] = (kin && gn + (EPI == 0 ? r * 16 : 0) < N)
+                         ? load16(wrow + r * group_rows * K + gk)
+                         : zero;
+#pragma unroll
+        for (int t = 0; t < MT; ++t)
+          av[u][t] = (kin && t * 16 + col < M) ? load16(arow[t] + gk) : zero;
+      }
+      products(wv, av);
+    }
   }
 #pragma unroll
   for (int t = 0; t < NG * MT; ++t)
@@ -766,17 +874,25 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny_kernel(
 
 template <typename TO, int MT, int NW, int EPI, int NT = 1>
 static void launch_skinny(const bf16_t* A, const bf16_t* W, const float* bias, TO* C, int M, int N,
-                          int K, int lda, int ldc, int ksplit, ConvStep cs, hipStream_t stream) {
-  hipLaunchKernelGGL((gemm_bf16_skinny_kernel<TO, MT, NW, EPI, NT>),
-                     dim3((N + 16 * NT - 1) / (16 * NT), ksplit), dim3(NW * WAVE), 0, stream, A, W,
-                     bias, C, M, N, K, lda, ldc, cs);
+                          int K, int lda, int ldc, int ksplit, ConvStep cs, hipStream_t stream,
+                          const NormIn* nin = nullptr) {
+  const dim3 grid((N + 16 * NT - 1) / (16 * NT), ksplit);
+  if constexpr (MT == 1 && NT == 1 && EPI != 2) {
+    if (nin) {
+      hipLaunchKernelGGL((gemm_bf16_skinny_kernel<TO, MT, NW, EPI, NT, true>), grid,
+                         dim3(NW * WAVE), 0, stream, A, W, bias, C, M, N, K, lda, ldc, cs, *nin);
+      return;
+    }
+  }
+  hipLaunchKernelGGL((gemm_bf16_skinny_kernel<TO, MT, NW, EPI, NT>), grid, dim3(NW * WAVE), 0,
+                     stream, A, W, bias, C, M, N, K, lda, ldc, cs, NormIn{});
 }
 
 // more waves a block when there are few blocks, so that about 2048 waves or more stream W
 template <typename TO, int MT, int EPI>
 static void launch_skinny_mt(const bf16_t* A, const bf16_t* W, const float* bias, TO* C, int M,
                              int N, int K, int lda, int ldc, int ksplit, ConvStep cs,
-                             hipStream_t stream) {
+                             hipStream_t stream, const NormIn* nin = nullptr) {
   // several row tiles and a plain product: a wave takes two column tiles for every fragment
   // of A it loads, which halves the reads of A (every block reads all of it)
   if constexpr (EPI == 0 && MT >= 2) {
@@ -790,13 +906,13 @@ static void launch_skinny_mt(const bf16_t* A, const bf16_t* W, const float* bias
   constexpr int NG = EPI == 1 ? 2 : (EPI == 2 ? 3 : 1);
   constexpr int MAXW = 48 / (MT * NG);                    // 1 KB of LDS a wave, group and row tile
   if (blocks * 4 >= 2048 || kb <= 512 || MAXW < 8)
-    launch_skinny<TO, MT, 4, EPI>(A, W, bias, C, M, N, K, lda, ldc, ksplit, cs, stream);
+    launch_skinny<TO, MT, 4, EPI>(A, W, bias, C, M, N, K, lda, ldc, ksplit, cs, stream, nin);
   else if (blocks * 8 >= 2048 || kb <= 1024 || MAXW < 16)
     launch_skinny<TO, MT, (MAXW >= 8 ? 8 : 4), EPI>(A, W, bias, C, M, N, K, lda, ldc, ksplit, cs,
-                                                    stream);
+                                                    stream, nin);
   else
     launch_skinny<TO, MT, (MAXW >= 16 ? 16 : 4), EPI>(A, W, bias, C, M, N, K, lda, ldc, ksplit, cs,
-                                                      stream);
+                                                      stream, nin);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -1108,4 +1224,46 @@ extern "C" int kappai_gemm_bf16_shortconv_step(const void* A, const void* W, con
   ConvStep cs{taps, conv_bias, state, seg_pos0, seg_slot, L};
   return launch_bf16<bf16_t, 2>((const bf16_t*)A, (const bf16_t*)W, bias, (bf16_t*)C, M, D, K, lda,
                                 D, 2, 1, stream, cs);
+}
+
+// The same products for at most NORM_ROWS rows that are still to be made: A = RMSNorm(resid +
+// delta) * norm_w, computed inside the product kernel (see NormIn).  delta: null, bfloat16 [M, K]
+// (delta_f32 = 0, n_parts = 1) or float [n_parts][M][K]; resid_out [M, K] receives resid + delta
+// when there is a delta (it must not be resid).  K a multiple of 8, at most NORM_MAX_K.
+static bool norm_in_ok(int M, int K, const NormIn& n) {
+  if (M < 1 || M > NORM_ROWS || (K % 8) || K > NORM_MAX_K || !n.resid || !n.w) return false;
+  if (n.delta && (n.n_parts < 1 || (!n.delta_f32 && n.n_parts != 1) || !n.resid_out ||
+                  n.resid_out == n.resid))
+    return false;
+  return true;
+}
+
+extern "C" int kappai_gemm_bf16_normed(const float* resid, const void* delta, int delta_f32,
+                                       int n_parts, const float* norm_w, float eps,
+                                       float* resid_out, const void* W, const float* bias, void* C,
+                                       int M, int N, int K, int ldc, int out_is_f32, int ksplit,
+                                       hipStream_t stream) {
+  if (N <= 0) return 0;
+  NormIn nin{resid, delta, delta ? n_parts : 0, delta_f32, norm_w, eps, delta ? resid_out : nullptr};
+  if (!norm_in_ok(M, K, nin) || ksplit < 1 || ksplit > 64 || (ksplit > 1 && !out_is_f32))
+    return (int)hipErrorInvalidValue;
+  if (out_is_f32)
+    launch_skinny_mt<float, 1, 0>(nullptr, (const bf16_t*)W, bias, (float*)C, M, N, K, K, ldc,
+                                  ksplit, ConvStep{}, stream, &nin);
+  else
+    launch_skinny_mt<bf16_t, 1, 0>(nullptr, (const bf16_t*)W, bias, (bf16_t*)C, M, N, K, K, ldc, 1,
+                                   ConvStep{}, stream, &nin);
+  KAPPAI_RETURN_LAUNCH_STATUS();
+}
+
+extern "C" int kappai_gemm_bf16_swiglu_normed(const float* resid, const void* delta, int delta_f32,
+                                              int n_parts, const float* norm_w, float eps,
+                                              float* resid_out, const void* W, void* C, int M,
+                                              int F, int K, int ldc, hipStream_t stream) {
+  if (F <= 0) return 0;
+  NormIn nin{resid, delta, delta ? n_parts : 0, delta_f32, norm_w, eps, delta ? resid_out : nullptr};
+  if (!norm_in_ok(M, K, nin) || (F % 16)) return (int)hipErrorInvalidValue;
+  launch_skinny_mt<bf16_t, 1, 1>(nullptr, (const bf16_t*)W, nullptr, (bf16_t*)C, M, F, K, K, ldc, 1,
+                                 ConvStep{}, stream, &nin);
+  KAPPAI_RETURN_LAUNCH_STATUS();
 }

@@ -107,6 +107,56 @@ def add_rmsnorm(resid: torch.Tensor, delta: Optional[torch.Tensor], weight: torc
     return out
 
 
+NORM_FUSE_MAX_ROWS = 1        # rows a product kernel normalises by itself
+NORM_FUSE_MAX_WIDTH = 4096
+
+
+class PendingNorm:
+    """Rows that are still to be made: ``RMSNorm(resid + delta) * weight``.  ``linear`` and
+    ``linear_swiglu`` take it in place of their input and make the rows inside the product
+    kernel (every block for itself), which saves the kernel between two products of a decode
+    step with very few rows.  ``resid`` is not changed; after the product ``resid_after`` holds
+    resid + delta (a new tensor, or ``resid`` itself without a delta).  ``materialize`` runs the
+    ordinary kernel instead."""
+
+    def __init__(self, resid: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Tensor,
+                 eps: float, out_dtype):
+        self.resid, self.delta, self.weight, self.eps, self.dtype = resid, delta, weight, eps, out_dtype
+        self.shape, self.device = resid.shape, resid.device
+        self.resid_after: Optional[torch.Tensor] = None
+
+    @staticmethod
+    def fits(resid: torch.Tensor, delta: Optional[torch.Tensor], out_dtype) -> bool:
+        if not (resid.is_cuda and out_dtype == BF16 and resid.dtype == F32 and resid.dim() == 2
+                and resid.is_contiguous()):
+            return False
+        M, D = resid.shape
+        if not (1 <= M <= NORM_FUSE_MAX_ROWS and D % 8 == 0 and D <= NORM_FUSE_MAX_WIDTH):
+            return False
+        if delta is None:
+            return True
+        if not delta.is_contiguous():
+            return False
+        if delta.dim() == 3:
+            return delta.dtype == F32 and delta.shape[1:] == resid.shape and delta.shape[0] <= 8
+        return delta.shape == resid.shape and delta.dtype in (F32, BF16)
+
+    def materialize(self) -> torch.Tensor:
+        x = add_rmsnorm(self.resid, self.delta, self.weight, self.eps, self.dtype)
+        self.resid_after = self.resid
+        return x
+
+    def _kernel_args(self):
+        """(resid, delta, delta_f32, n_parts, weight, eps, resid_out) for the product kernels."""
+        if self.resid_after is None:
+            self.resid_after = self.resid if self.delta is None else torch.empty_like(self.resid)
+        d = self.delta
+        n_parts = d.shape[0] if d is not None and d.dim() == 3 else 1
+        return (_ptr(self.resid), _ptr(d), _c_int(1 if d is not None and d.dtype == F32 else 0),
+                _c_int(n_parts), _ptr(self.weight), _c_float(self.eps),
+                _ptr(self.resid_after if d is not None else None))
+
+
 def add_residual(resid: torch.Tensor, delta: torch.Tensor) -> None:
     _gpu("resid", resid, F32)
     _gpu("delta", delta, (F32, BF16))
@@ -171,7 +221,14 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] =
     with float accumulation; a float32 matrix runs in true 32-bit arithmetic, whatever the
     activations' dtype.  ``x`` may be a view with a row stride.  With ``partial_sums`` the
     result may come back as float32 [S, M, N], the sums over S ranges of K, for a consumer
-    that adds them (a matrix with few columns is then streamed by enough blocks)."""
+    that adds them (a matrix with few columns is then streamed by enough blocks).  ``x`` may
+    be a ``PendingNorm``: the rows are then made inside the product kernel."""
+    if isinstance(x, PendingNorm):
+        if (weight.dtype != BF16 or force_kernel or weight.dim() != 2
+                or weight.shape[1] != x.shape[1] or weight.data_ptr() % 16):
+            x = x.materialize()
+        else:
+            return _linear_normed(x, weight, bias, out_dtype, partial_sums, split_k)
     _gpu("x", x, (F32, BF16), contiguous=False)
     _gpu("weight", weight, (F32, BF16))
     _need(x.dim() == 2 and weight.dim() == 2 and x.shape[1] == weight.shape[1],
@@ -209,6 +266,27 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] =
     return out
 
 
+def _linear_normed(x: PendingNorm, weight, bias, out_dtype, partial_sums, split_k) -> torch.Tensor:
+    _gpu("weight", weight, BF16)
+    M, K = x.shape
+    N = weight.shape[0]
+    out_dtype = out_dtype or x.dtype
+    if bias is not None:
+        _gpu("bias", bias, F32)
+        _need(bias.shape == (N,), f"linear: bias {tuple(bias.shape)} for N={N}")
+    ksplit = (split_k or split_k_for(M, N, K)) if partial_sums else 1
+    if ksplit > 1:
+        out = torch.empty((ksplit, M, N), dtype=F32, device=x.device)
+        out_is_f32 = 1
+    else:
+        out = torch.empty((M, N), dtype=out_dtype, device=x.device)
+        out_is_f32 = 0 if out_dtype == BF16 else 1
+    check(library("gemm").kappai_gemm_bf16_normed(
+        *x._kernel_args(), _ptr(weight), _ptr(bias), _ptr(out), _c_int(M), _c_int(N), _c_int(K),
+        _c_int(N), _c_int(out_is_f32), _c_int(ksplit), _stream()), "gemm_bf16_normed")
+    return out
+
+
 SWIGLU_GROUP = 16     # gate and up rows alternate in groups of this many rows
 
 
@@ -226,7 +304,22 @@ def interleave_gate_up(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
 
 def linear_swiglu(x: torch.Tensor, weight: torch.Tensor, force_kernel: int = 0) -> torch.Tensor:
     """``silu(x Wg^T) * (x Wu^T)`` in one kernel: ``weight`` [2F, K] holds the gate and up
-    matrices interleaved by ``interleave_gate_up``; bfloat16 only.  Returns [M, F]."""
+    matrices interleaved by ``interleave_gate_up``; bfloat16 only.  Returns [M, F].  ``x`` may
+    be a ``PendingNorm``."""
+    if isinstance(x, PendingNorm):
+        if (force_kernel or weight.dtype != BF16 or weight.dim() != 2
+                or weight.shape[1] != x.shape[1] or weight.shape[0] % (2 * SWIGLU_GROUP)
+                or weight.data_ptr() % 16):
+            x = x.materialize()
+        else:
+            _gpu("weight", weight, BF16)
+            M, K = x.shape
+            F = weight.shape[0] // 2
+            out = torch.empty((M, F), dtype=BF16, device=x.device)
+            check(library("gemm").kappai_gemm_bf16_swiglu_normed(
+                *x._kernel_args(), _ptr(weight), _ptr(out), _c_int(M), _c_int(F), _c_int(K),
+                _c_int(F), _stream()), "gemm_bf16_swiglu_normed")
+            return out
     _gpu("x", x, BF16, contiguous=False)
     _gpu("weight", weight, BF16)
     _need(x.dim() == 2 and weight.dim() == 2 and x.shape[1] == weight.shape[1]

@@ -23,6 +23,8 @@ from .linear import PARTIAL_SUMS_MIN_ROWS, Linear
 
 
 class GroupedQueryAttention(Mixer):
+    takes_pending_norm = True      # its first product may make the normalised rows itself
+
     def __init__(self, prefix: str, width: int, num_heads: int, num_kv_heads: int, head_dim: int,
                  dtype: torch.dtype, position: Optional[PositionEncoding] = None,
                  qk_norm_eps: Optional[float] = None, window: Optional[int] = None,

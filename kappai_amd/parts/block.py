@@ -9,6 +9,10 @@ from ..weights.spec import TensorSpec
 from .base import Block, FeedForward, Hidden, Mixer, Norm, register_part
 
 
+def _takes_defer(norm) -> bool:
+    return getattr(norm, "can_defer", False)
+
+
 class PreNormBlock(Block):
     """``x += mixer(norm(x)); x += feed_forward(norm(x))`` (kappai: src/models/lfm.c:7-53 with
     the tail src/recipe/builders.c:378-388).  Each residual sum is made inside the norm
@@ -33,10 +37,27 @@ class PreNormBlock(Block):
             p.bind(tensors)
 
     def forward(self, h: Hidden, batch, cache, shared_cache: bool = False) -> Hidden:
-        x = self.mixer_norm.add_norm(h.resid, h.delta)
+        # a part that says so may get its rows as a pending norm, which its first product makes
+        resid = h.resid
+        x = self._normed(self.mixer_norm, resid, h.delta, self.mixer)
         mixed = self.mixer.forward(x, batch, cache, shared_cache=shared_cache)
-        x = self.ffn_norm.add_norm(h.resid, mixed)
-        return Hidden(h.resid, self.feed_forward.forward(x, batch))
+        resid = self._resid_after(x, resid)
+        x = self._normed(self.ffn_norm, resid, mixed, self.feed_forward)
+        out = self.feed_forward.forward(x, batch)
+        return Hidden(self._resid_after(x, resid), out)
+
+    @staticmethod
+    def _normed(norm, resid, delta, consumer):
+        if getattr(consumer, "takes_pending_norm", False) and _takes_defer(norm):
+            return norm.add_norm(resid, delta, defer=True)
+        return norm.add_norm(resid, delta)
+
+    @staticmethod
+    def _resid_after(x, resid):
+        after = getattr(x, "resid_after", resid) if not isinstance(x, torch.Tensor) else resid
+        if after is None:
+            raise RuntimeError("a part that takes a pending norm did not use it")
+        return after
 
     def weight_bytes(self) -> int:
         return sum(p.weight_bytes() for p in self._parts())

@@ -15,6 +15,8 @@ from .linear import Linear
 
 
 class SwiGLU(FeedForward):
+    takes_pending_norm = True      # its first product may make the normalised rows itself
+
     def __init__(self, prefix: str, width: int, hidden: int, dtype: torch.dtype, names=None):
         n = {"gate": "w1", "up": "w3", "down": "w2"}
         n.update(names or {})

@@ -13,6 +13,8 @@ from .base import Norm, register_part
 
 
 class RMSNorm(Norm):
+    can_defer = True      # add_norm(..., defer=True) may hand out an ops.PendingNorm
+
     def __init__(self, name: str, width: int, eps: float, dtype: torch.dtype):
         self.name, self.width, self.eps, self.dtype = name, width, float(eps), dtype
         self.weight: Optional[torch.Tensor] = None
@@ -23,7 +25,11 @@ class RMSNorm(Norm):
     def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
         self.weight = tensors[self.name + ".weight"].to(torch.float32).contiguous()
 
-    def add_norm(self, resid, delta, rows=None):
+    def add_norm(self, resid, delta, rows=None, defer: bool = False):
+        """``defer``: the caller's next part takes an ``ops.PendingNorm`` in place of the rows
+        (a step with very few rows: the product kernel then makes them itself)."""
+        if defer and rows is None and ops.PendingNorm.fits(resid, delta, self.dtype):
+            return ops.PendingNorm(resid, delta, self.weight, self.eps, self.dtype)
         return ops.add_rmsnorm(resid, delta, self.weight, self.eps, self.dtype, rows=rows,
                                write_resid=rows is None)
 

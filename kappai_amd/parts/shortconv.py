@@ -25,6 +25,8 @@ FUSED_STEP_MIN_WIDTH = 4096
 
 
 class GatedShortConv(Mixer):
+    takes_pending_norm = True      # its first product may make the normalised rows itself
+
     def __init__(self, prefix: str, width: int, kernel_size: int, dtype: torch.dtype,
                  bias: bool = False, names=None):
         n = {"in": "in_proj", "conv": "conv", "out": "out_proj"}
@@ -63,6 +65,8 @@ class GatedShortConv(Mixer):
         if shared_cache:
             raise ValueError("a short convolution's state cannot be read by another layer")
         w = self.in_proj.weight
+        if isinstance(x, ops.PendingNorm) and self.width >= FUSED_STEP_MIN_WIDTH:
+            x = x.materialize()            # the fused step kernel below reads rows
         if (batch.max_segment_rows == 1 and x.shape[0] <= 64 and x.dtype == torch.bfloat16
                 and w.dtype == torch.bfloat16 and self.width % 16 == 0
                 and self.width >= FUSED_STEP_MIN_WIDTH):

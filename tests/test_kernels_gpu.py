@@ -264,6 +264,73 @@ def test_linear_partial_sums(ops, M, N, K):
                                        write_resid=False), BF16_ULP, "selected rows")
 
 
+@pytest.mark.parametrize("M", [1, 2, 4])
+@pytest.mark.parametrize("N,K", [(48, 64), (6144, 2048), (200, 520), (1000, 4096)])
+@pytest.mark.parametrize("delta_kind", ["none", "bf16", "f32", "parts"])
+def test_linear_makes_the_normalised_rows_itself(ops, M, N, K, delta_kind):
+    """A product whose input is a pending RMSNorm: the same result as the norm kernel followed by
+    the product, the residual untouched and resid + delta in a tensor of its own."""
+    resid = rand((M, K), F32, 80, 2.0)
+    wn = 1 + rand((K,), F32, 81, 0.1)
+    w, b = rand((N, K), BF16, 82, 0.1), rand((N,), F32, 83)
+    delta = {"none": None, "bf16": rand((M, K), BF16, 84), "f32": rand((M, K), F32, 84),
+             "parts": rand((3, M, K), F32, 84)}[delta_kind]
+    d_dev = None if delta is None else delta.to(DEV)
+    r_dev = resid.to(DEV)
+    x = ops.add_rmsnorm(r_dev.clone(), d_dev, wn.to(DEV), 1e-5, BF16)
+    for bias in (None, b.to(DEV)):
+        pend = ops.PendingNorm(r_dev, d_dev, wn.to(DEV), 1e-5, BF16)
+        got = ops.linear(pend, w.to(DEV), bias, out_dtype=F32)
+        want = ops.linear(x, w.to(DEV), bias, out_dtype=F32)
+        close(got, want.cpu().double(), 2 * BF16_ULP, "product of the pending norm")
+        assert torch.equal(r_dev.cpu(), resid), "the residual was changed"
+        total = resid.clone()
+        if delta is not None:
+            for part in (delta if delta.dim() == 3 else [delta]):
+                total += part.float()
+            assert pend.resid_after.data_ptr() != r_dev.data_ptr()
+        else:
+            assert pend.resid_after is r_dev
+        close(pend.resid_after, total.double(), 1e-6, "resid + delta")
+    # partial sums out of it, as the consumers of a split product take them
+    pend = ops.PendingNorm(r_dev, d_dev, wn.to(DEV), 1e-5, BF16)
+    parts = ops.linear(pend, w.to(DEV), partial_sums=True, split_k=2)
+    assert parts.shape == (2, M, N) and parts.dtype == F32
+    close(parts.sum(0), ops.linear(x, w.to(DEV), out_dtype=F32).cpu().double(), 2 * BF16_ULP,
+          "partial sums")
+
+
+@pytest.mark.parametrize("M,F,K", [(1, 8192, 2048), (3, 48, 136), (4, 320, 1024)])
+def test_linear_swiglu_makes_the_normalised_rows_itself(ops, M, F, K):
+    resid, wn = rand((M, K), F32, 85, 2.0), 1 + rand((K,), F32, 86, 0.1)
+    delta = rand((4, M, K), F32, 87)
+    wg, wu = rand((F, K), BF16, 88, 0.1), rand((F, K), BF16, 89, 0.1)
+    w = ops.interleave_gate_up(wg.to(DEV), wu.to(DEV))
+    x = ops.add_rmsnorm(resid.to(DEV), delta.to(DEV), wn.to(DEV), 1e-5, BF16)
+    pend = ops.PendingNorm(resid.to(DEV), delta.to(DEV), wn.to(DEV), 1e-5, BF16)
+    got = ops.linear_swiglu(pend, w)
+    close(got.float(), ops.linear_swiglu(x, w).float().cpu().double(), 2 * BF16_ULP, "swiglu")
+    close(pend.resid_after, (resid + delta.sum(0)).double(), 1e-5, "resid + delta")
+
+
+def test_pending_norm_falls_back_to_the_norm_kernel(ops):
+    """A float32 matrix (or anything else the fused kernel does not take) makes the rows with
+    the ordinary kernel, which updates the residual in place."""
+    resid, wn = rand((1, 64), F32, 90, 2.0), 1 + rand((64,), F32, 91, 0.1)
+    delta, w = rand((1, 64), BF16, 92), rand((24, 64), F32, 93)
+    r_dev = resid.to(DEV)
+    pend = ops.PendingNorm(r_dev, delta.to(DEV), wn.to(DEV), 1e-5, BF16)
+    got = ops.linear(pend, w.to(DEV))
+    assert pend.resid_after is r_dev
+    close(r_dev, (resid + delta.float()).double(), 1e-6, "residual updated in place")
+    x = ref.add_rmsnorm(resid.clone(), delta, wn, 1e-5, BF16)
+    close(got.float(), x.double() @ w.double().T, BF16_ULP, "product")
+    assert not ops.PendingNorm.fits(rand((9, 64), F32, 1).to(DEV), None, BF16)
+    assert not ops.PendingNorm.fits(rand((1, 64), F32, 1).to(DEV), None, F32)
+    assert not ops.PendingNorm.fits(rand((1, 8192), F32, 1).to(DEV), None, BF16)
+    assert ops.PendingNorm.fits(rand((1, 64), F32, 1).to(DEV), rand((2, 1, 64), F32, 2).to(DEV), BF16)
+
+
 def test_linear_views_and_mixed_storage(ops):
     # x as the leading columns of a wider buffer (a row stride), as attention hands q over
     wide = rand((20, 96 + 40), BF16, 12).to(DEV)
