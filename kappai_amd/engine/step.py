@@ -25,6 +25,19 @@ DECODE_RING = 8            # decode steps whose tables can be queued ahead of th
 MAX_DECODE_GRAPHS = 48
 
 
+# A decode step of B requests that all want logits is replayed from the graph of the next
+# batch size in this list, the rows beyond B being dummies on the scratch page and slot: a few
+# shapes serve every batch size, and a batch that shrinks as requests end needs no new capture.
+DECODE_BATCH_BUCKETS = (1, 2, 4, 8, 12, 16, 24, 32, 48, 64, 96, 128, 192, 256)
+
+
+def _batch_bucket(n_rows: int) -> int:
+    for b in DECODE_BATCH_BUCKETS:
+        if b >= n_rows:
+            return b
+    return n_rows
+
+
 def _context_bucket(n_positions: int) -> int:
     cap = CONTEXT_BUCKET_MIN
     while cap < n_positions:
@@ -79,6 +92,7 @@ class _DecodeGraph:
         for g in range(n_groups):
             self.h[f"block_table_{g}"][:] = cache.scratch_page(g)
         self.rows_of = [None] * B        # (request cache, version) whose pages row si mirrors
+        self.scratch = (cache.scratch_slot, [cache.scratch_page(g) for g in range(n_groups)])
         self._ring: List[Optional[torch.Tensor]] = [None] * DECODE_RING
         self._ring_done: List[Optional[torch.cuda.Event]] = [None] * DECODE_RING
         self._ring_at = 0
@@ -108,12 +122,20 @@ class _DecodeGraph:
         """``tokens`` from the host, or ``device_tokens`` (int32 [B] on the GPU, e.g. what the last
         step's sampling kernel wrote) copied into place on the GPU."""
         h = self.h
-        if device_tokens is None:
-            h["tokens"][:] = tokens
-        h["row_pos"][:] = pos
-        h["seg_pos0"][:] = pos
-        h["seg_slot"][:] = slots
-        h["logit_rows"][:] = logit_rows
+        n = len(caches)                  # rows n .. B-1 are dummies: token 0 at position 0 of
+        if device_tokens is None:        # the scratch slot and page, logits nobody reads
+            h["tokens"][:n] = tokens
+        h["tokens"][n:] = 0
+        h["row_pos"][:n] = pos
+        h["row_pos"][n:] = 0
+        h["seg_pos0"][:n] = pos
+        h["seg_pos0"][n:] = 0
+        h["seg_slot"][:n] = slots
+        h["seg_slot"][n:] = self.scratch[0]
+        if n < self.B:
+            h["logit_rows"][:] = np.arange(self.n_logit) % self.B
+        else:
+            h["logit_rows"][:] = logit_rows
         for si, rc in enumerate(caches):
             seen = self.rows_of[si]
             if seen is None or seen[0] is not rc or seen[1] != rc.version:
@@ -123,11 +145,16 @@ class _DecodeGraph:
                     row[:len(b)] = b
                     row[len(b):] = -1
                 self.rows_of[si] = (rc, rc.version)
+        for si in range(n, self.B):
+            if self.rows_of[si] is not None:
+                for g, page in enumerate(self.scratch[1]):
+                    h[f"block_table_{g}"][si] = page
+                self.rows_of[si] = None
         self._upload(runner)
         if device_tokens is not None:
-            self.batch.tokens.copy_(device_tokens)
+            self.batch.tokens[:n].copy_(device_tokens)
         self.graph.replay()
-        return self.logits
+        return self.logits if n == self.B else self.logits[:n]
 
 
 class StepRunner:
@@ -219,7 +246,10 @@ class StepRunner:
         width = ctx_cap // self.cache.page_size + 1
         if any(len(b) > width for c in caches for b in c.blocks):
             return None
-        key = (B, len(logit_rows), ctx_cap)
+        # every row wants its logits (the usual decode step): the graph of the next batch size
+        rows_b = _batch_bucket(B) if len(logit_rows) == B else B
+        n_logit = rows_b if len(logit_rows) == B else len(logit_rows)
+        key = (rows_b, n_logit, ctx_cap)
         graph = self._graphs.get(key)
         if graph is None:
             self._graph_seen[key] = self._graph_seen.get(key, 0) + 1
@@ -227,7 +257,7 @@ class StepRunner:
                 return None
             if len(self._graphs) >= MAX_DECODE_GRAPHS:
                 self._graphs.pop(next(iter(self._graphs)))
-            graph = self._graphs[key] = _DecodeGraph(self, B, len(logit_rows), ctx_cap)
+            graph = self._graphs[key] = _DecodeGraph(self, rows_b, n_logit, ctx_cap)
         slots = np.fromiter((c.slot for c in caches), dtype=np.int32, count=B)
         self.graph_replays += 1
         return graph.run(self, caches, tokens, pos, slots, logit_rows)
@@ -247,7 +277,8 @@ class StepRunner:
         if len({id(c) for c in caches}) != B:
             return None
         ctx_cap = _context_bucket(max(c.length for c in caches) + n_steps)
-        graph = self._graphs.get((B, B, ctx_cap))
+        rows_b = _batch_bucket(B)
+        graph = self._graphs.get((rows_b, rows_b, ctx_cap))
         if graph is None or not self.cache.can_extend_all(caches, n_steps):
             return None
         tokens = np.asarray(first_tokens, dtype=np.int64)

@@ -175,14 +175,20 @@ def test_decode_runs_give_the_same_tokens(model_dirs, dtype):
               SamplingParams(temperature=0.7, top_k=12, top_p=0.9, min_p=0.05, seed=6, n_predict=29),
               SamplingParams.greedy(n_predict=2)]
     results = {}
-    for run_len in (1, 8, 3):
-        eng = _engine(model_dirs["B"], dtype, decode_run=run_len)
+    for run_len in (0, 1, 8, 3):         # 0: no captured graphs at all, every step eager
+        eng = _engine(model_dirs["B"], dtype, decode_run=max(run_len, 1))
+        if run_len == 0:
+            eng.runner.decode_graphs = False
         results[run_len] = eng.generate(prompts, params)
         eng.cache.check()
         assert eng.cache.num_free_pages() == 256 and eng.cache.num_free_slots == 8
         if run_len > 1:
             assert eng.runner.graph_replays > 20
+        assert (eng.runner.graph_replays == 0) == (run_len == 0)
         assert [len(o) for o in results[run_len]] == [41, 23, 36, 29, 2]
+    # the batch shrinks from 5 to 1 as requests end: steps of 5 and 3 rows are replayed from the
+    # graphs of 8 and 4 rows with dummy rows
+    assert results[1] == results[0]
     assert results[8] == results[1]
     assert results[3] == results[1]
 
