@@ -13,6 +13,8 @@
 //                    waves split K and meet in LDS (v_mfma_f32_16x16x32_bf16).
 //   gemm_bf16_shared_rows  17 <= M <= 64 and a W with many rows: as above, but two waves that
 //                    stream different rows of W share the rows of A through LDS.
+//   gemm_bf16_any    K or a row stride that is no multiple of 8: a plain kernel, so that no
+//                    width is refused.
 #include "common.h"
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
@@ -1265,5 +1267,46 @@ extern "C" int kappai_gemm_bf16_swiglu_normed(const float* resid, const void* de
   if (!norm_in_ok(M, K, nin) || (F % 16)) return (int)hipErrorInvalidValue;
   launch_skinny_mt<bf16_t, 1, 1>(nullptr, (const bf16_t*)W, nullptr, (bf16_t*)C, M, F, K, K, ldc, 1,
                                  ConvStep{}, stream, &nin);
+  KAPPAI_RETURN_LAUNCH_STATUS();
+}
+
+// ---------------------------------------------------------------------------------------
+// bf16 at any size and alignment (K or a row stride that is no multiple of 8): one wave per
+// row and four output columns, lanes stride over K with 2-byte loads, float sums added up
+// across the wave.  Slow, and only there so that no width is refused.
+// ---------------------------------------------------------------------------------------
+template <typename TO>
+__global__ __launch_bounds__(WAVE) void gemm_bf16_any_kernel(
+    const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, const float* __restrict__ bias,
+    TO* __restrict__ C, int M, int N, int K, int lda, int ldc) {
+  const int m = blockIdx.y, n0 = blockIdx.x * 4, lane = threadIdx.x;
+  const bf16_t* a = A + (size_t)m * lda;
+  float acc[4] = {0.f, 0.f, 0.f, 0.f};
+  for (int k = lane; k < K; k += WAVE) {
+    const float x = bf16_to_f32(a[k]);
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      if (n0 + j < N) acc[j] = fmaf(x, bf16_to_f32(W[(size_t)(n0 + j) * K + k]), acc[j]);
+  }
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const float sum = wave_sum(acc[j]);
+    if (lane == 0 && n0 + j < N)
+      store_out(C + (size_t)m * ldc + n0 + j, sum + (bias ? bias[n0 + j] : 0.f));
+  }
+}
+
+extern "C" int kappai_gemm_bf16_any(const void* A, const void* W, const float* bias, void* C,
+                                    int M, int N, int K, int lda, int ldc, int out_is_f32,
+                                    hipStream_t stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (K < 1 || M > 65535) return (int)hipErrorInvalidValue;
+  const dim3 grid((N + 3) / 4, M);
+  if (out_is_f32)
+    hipLaunchKernelGGL(gemm_bf16_any_kernel<float>, grid, dim3(WAVE), 0, stream, (const bf16_t*)A,
+                       (const bf16_t*)W, bias, (float*)C, M, N, K, lda, ldc);
+  else
+    hipLaunchKernelGGL(gemm_bf16_any_kernel<bf16_t>, grid, dim3(WAVE), 0, stream,
+                       (const bf16_t*)A, (const bf16_t*)W, bias, (bf16_t*)C, M, N, K, lda, ldc);
   KAPPAI_RETURN_LAUNCH_STATUS();
 }

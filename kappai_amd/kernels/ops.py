@@ -249,9 +249,18 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] =
         return out if out_dtype == F32 else cast(out, out_dtype)
     xb = x if x.dtype == BF16 else cast(x.contiguous(), BF16)
     lda = xb.stride(0) if M > 1 else K
-    _need(K % 8 == 0 and lda % 8 == 0 and xb.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0,
-          f"linear: the bfloat16 kernels read 16 bytes at a time: K ({K}) and the row stride "
-          f"({lda}) must be multiples of 8 and the tensors 16-byte aligned")
+    if not (K % 8 == 0 and lda % 8 == 0 and xb.data_ptr() % 16 == 0
+            and weight.data_ptr() % 16 == 0):
+        # the matrix-core kernels read 16 bytes at a time; anything else goes the plain way
+        _need(not force_kernel, f"linear: K ({K}) and the row stride ({lda}) must be multiples of "
+              "8 and the tensors 16-byte aligned for the kernel that was asked for")
+        _need(M <= MAX_GRID_Y, f"linear: {M} rows with a width that is no multiple of 8")
+        out = torch.empty((M, N), dtype=out_dtype, device=x.device)
+        check(library("gemm").kappai_gemm_bf16_any(
+            _ptr(xb), _ptr(weight), _ptr(bias), _ptr(out), _c_int(M), _c_int(N), _c_int(K),
+            _c_int(lda), _c_int(N), _c_int(0 if out_dtype == BF16 else 1), _stream()),
+            "gemm_bf16_any")
+        return out
     ksplit = (split_k or split_k_for(M, N, K)) if partial_sums else 1
     if ksplit > 1:
         out = torch.empty((ksplit, M, N), dtype=F32, device=x.device)

@@ -331,6 +331,24 @@ def test_pending_norm_falls_back_to_the_norm_kernel(ops):
     assert ops.PendingNorm.fits(rand((1, 64), F32, 1).to(DEV), rand((2, 1, 64), F32, 2).to(DEV), BF16)
 
 
+@pytest.mark.parametrize("M,N,K", [(1, 7, 20), (5, 301, 100), (70, 33, 84), (3, 64, 1001)])
+@pytest.mark.parametrize("out_dtype", [F32, BF16])
+def test_linear_bfloat16_at_widths_that_are_no_multiple_of_8(ops, M, N, K, out_dtype):
+    x, w, b = rand((M, K), BF16, 94), rand((N, K), BF16, 95), rand((N,), F32, 96)
+    want = x.double() @ w.double().T
+    tol = 2e-5 if out_dtype == F32 else BF16_ULP
+    got = ops.linear(x.to(DEV), w.to(DEV), out_dtype=out_dtype)
+    assert got.dtype == out_dtype
+    close(got.float(), want, tol, "plain kernel")
+    got = ops.linear(x.to(DEV), w.to(DEV), b.to(DEV), out_dtype=out_dtype, partial_sums=True)
+    close(got.float(), want + b.double(), tol, "plain kernel with bias")
+    # a row stride that is no multiple of 8 although K is one
+    wide = rand((M, 43), BF16, 97).to(DEV)
+    w40 = rand((N, 40), BF16, 98)
+    got = ops.linear(wide[:, :40], w40.to(DEV), out_dtype=out_dtype)
+    close(got.float(), wide[:, :40].cpu().double() @ w40.double().T, tol, "odd row stride")
+
+
 def test_linear_views_and_mixed_storage(ops):
     # x as the leading columns of a wider buffer (a row stride), as attention hands q over
     wide = rand((20, 96 + 40), BF16, 12).to(DEV)
@@ -346,7 +364,7 @@ def test_linear_views_and_mixed_storage(ops):
 
 def test_linear_refuses_what_it_cannot_do(ops):
     with pytest.raises(ValueError, match="multiples of 8"):
-        ops.linear(rand((4, 20), BF16, 1).to(DEV), rand((8, 20), BF16, 2).to(DEV))
+        ops.linear(rand((4, 20), BF16, 1).to(DEV), rand((8, 20), BF16, 2).to(DEV), force_kernel=2)
     with pytest.raises(ValueError, match="GPU"):
         ops.linear(rand((4, 16), BF16, 1), rand((8, 16), BF16, 2))
 

@@ -26,10 +26,12 @@ FP32_TOL = 2e-5     # of the largest |logit|
 # bfloat16 costs the plain implementation itself on the same requests
 BF16_FACTOR = 2.5
 
-LENGTHS = {"A": [70, 45, 100, 37, 83, 64], "B": [33, 97, 40, 71, 52], "C": [66, 35, 90, 41]}
+LENGTHS = {"A": [70, 45, 100, 37, 83, 64], "B": [33, 97, 40, 71, 52], "C": [66, 35, 90, 41],
+           "D": [50, 81, 36]}
 MIXED_LENGTHS = {"A": [70, 45, 100, 37, 83, 64, 29, 58, 91, 40],
                  "B": [33, 97, 40, 71, 52, 64, 18, 85, 47],
-                 "C": [66, 35, 90, 41, 23, 77, 50, 62]}
+                 "C": [66, 35, 90, 41, 23, 77, 50, 62],
+                 "D": [50, 81, 36, 67, 44, 72]}
 
 
 @pytest.fixture(scope="module")
@@ -77,7 +79,7 @@ def tolerance(model_dir, requests, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
 @pytest.mark.parametrize("family", ["whole", "prefill_then_decode", "changing_portions", "mixed"])
 def test_schedules(tmp_path, model_dirs, name, family, dtype):
     cfg = TINY[name][0]

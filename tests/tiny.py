@@ -49,7 +49,21 @@ TINY_C = {
 }
 INIT_C = dict(seed=2, std=0.04, norm_jitter=0.05)
 
-TINY = {"A": (TINY_A, INIT_A), "B": (TINY_B, INIT_B), "C": (TINY_C, INIT_C)}
+# 2 layers, a width, a feed-forward width and a vocabulary that are no multiples of 8 (the
+# bfloat16 products then take their plain kernel), as many kv heads as heads, biases
+TINY_D = {
+    "architectures": ["Lfm2ForCausalLM"], "model_type": "lfm2",
+    "hidden_size": 100, "num_hidden_layers": 2, "layer_types": ["conv", "full_attention"],
+    "num_attention_heads": 5, "num_key_value_heads": 5, "head_dim": 16,
+    "intermediate_size": 84, "block_auto_adjust_ff_dim": False,
+    "vocab_size": 301, "norm_eps": 1e-5, "rope_theta": 10000.0,
+    "conv_L_cache": 3, "conv_bias": True, "tie_embedding": True,
+    "max_position_embeddings": 1024,
+}
+INIT_D = dict(seed=3, std=0.05, norm_jitter=0.1)
+
+TINY = {"A": (TINY_A, INIT_A), "B": (TINY_B, INIT_B), "C": (TINY_C, INIT_C),
+        "D": (TINY_D, INIT_D)}
 
 
 def tiny_config(name: str) -> dict:
