@@ -27,7 +27,7 @@ HIPCC_FLAGS = ["-O3", "-std=c++17", f"--offload-arch={GPU_ARCH}", "-shared", "-f
                "-Wno-unused-command-line-argument", "-Wno-pass-failed"]
 LIBRARIES = ["elementwise", "gemm", "shortconv", "attention", "sampling"]
 # libraries compiled once per value of a constant: name -> (constant, values built ahead)
-VARIANT_LIBRARIES = {"attention_mfma": ("HEAD_DIM", [16, 32, 48, 64, 128, 256])}
+VARIANT_LIBRARIES = {"attention_mfma": ("HEAD_DIM", [16, 32, 48, 64, 80, 128, 256])}
 
 
 class KernelBuildError(RuntimeError):

@@ -27,11 +27,13 @@ FP32_TOL = 2e-5     # of the largest |logit|
 BF16_FACTOR = 2.5
 
 LENGTHS = {"A": [70, 45, 100, 37, 83, 64], "B": [33, 97, 40, 71, 52], "C": [66, 35, 90, 41],
-           "D": [50, 81, 36]}
+           "D": [50, 81, 36], "E": [45, 70, 33], "F": [66, 40, 85]}
 MIXED_LENGTHS = {"A": [70, 45, 100, 37, 83, 64, 29, 58, 91, 40],
                  "B": [33, 97, 40, 71, 52, 64, 18, 85, 47],
                  "C": [66, 35, 90, 41, 23, 77, 50, 62],
-                 "D": [50, 81, 36, 67, 44, 72]}
+                 "D": [50, 81, 36, 67, 44, 72, 90, 33, 58, 41],
+                 "E": [45, 70, 33, 52, 61, 38, 88, 27, 95, 40],
+                 "F": [66, 40, 85, 37, 58, 49, 92, 31, 74, 43]}
 
 
 @pytest.fixture(scope="module")
@@ -79,7 +81,7 @@ def tolerance(model_dir, requests, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D", "E", "F"])
 @pytest.mark.parametrize("family", ["whole", "prefill_then_decode", "changing_portions", "mixed"])
 def test_schedules(tmp_path, model_dirs, name, family, dtype):
     cfg = TINY[name][0]

@@ -62,8 +62,33 @@ TINY_D = {
 }
 INIT_D = dict(seed=3, std=0.05, norm_jitter=0.1)
 
+# conv layers only: no paged cache at all, five taps
+TINY_E = {
+    "architectures": ["Lfm2ForCausalLM"], "model_type": "lfm2",
+    "hidden_size": 48, "num_hidden_layers": 3, "layer_types": ["conv", "conv", "conv"],
+    "num_attention_heads": 2, "num_key_value_heads": 1, "head_dim": 32,
+    "intermediate_size": 112, "block_auto_adjust_ff_dim": False,
+    "vocab_size": 200, "norm_eps": 1e-5, "rope_theta": 10000.0,
+    "conv_L_cache": 5, "conv_bias": False, "tie_embedding": True,
+    "max_position_embeddings": 1024,
+}
+INIT_E = dict(seed=4, std=0.05, norm_jitter=0.1)
+
+# attention layers only, a single head of size 80 (wider than the model), no fixed state
+TINY_F = {
+    "architectures": ["Lfm2ForCausalLM"], "model_type": "lfm2",
+    "hidden_size": 56, "num_hidden_layers": 2,
+    "layer_types": ["full_attention", "full_attention"],
+    "num_attention_heads": 1, "num_key_value_heads": 1, "head_dim": 80,
+    "intermediate_size": 144, "block_auto_adjust_ff_dim": False,
+    "vocab_size": 150, "norm_eps": 1e-5, "rope_theta": 500000.0,
+    "conv_L_cache": 3, "conv_bias": False, "tie_embedding": False,
+    "max_position_embeddings": 1024,
+}
+INIT_F = dict(seed=5, std=0.05, norm_jitter=0.1)
+
 TINY = {"A": (TINY_A, INIT_A), "B": (TINY_B, INIT_B), "C": (TINY_C, INIT_C),
-        "D": (TINY_D, INIT_D)}
+        "D": (TINY_D, INIT_D), "E": (TINY_E, INIT_E), "F": (TINY_F, INIT_F)}
 
 
 def tiny_config(name: str) -> dict:
