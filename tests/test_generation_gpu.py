@@ -225,3 +225,40 @@ def test_end_of_sequence_inside_a_decode_run(model_dirs, tmp_path):
         assert got[1] == free[1] and got[2] == free[2]
         eng.cache.check()
         assert eng.cache.num_free_pages() == 256 and eng.cache.num_free_slots == 8
+
+
+def test_random_workload_with_and_without_graphs(model_dirs):
+    """Forty requests of random lengths and options through the scheduler, prompts in portions
+    beside decoded tokens: captured graphs, runs of queued decode steps, batches filled up with
+    dummy rows and a pool so tight that requests are preempted and computed again must all give
+    the tokens of eager steps in a roomy pool (float32, so the arithmetic is the same)."""
+    import random
+    from kappai_amd.engine import Engine, EngineConfig
+    from kappai_amd.sampling import SamplingParams
+    rng = random.Random(1)
+    vocab = TINY["B"][0]["vocab_size"]
+    n = 40
+    prompts = [[rng.randrange(vocab) for _ in range(rng.randint(1, 200))] for _ in range(n)]
+    params = []
+    for i in range(n):
+        if rng.random() < 0.5:
+            params.append(SamplingParams.greedy(n_predict=rng.randint(1, 60)))
+        else:
+            params.append(SamplingParams(
+                temperature=rng.choice([0.7, 1.0]), top_k=rng.choice([0, 12, 40]),
+                top_p=rng.choice([1.0, 0.9]), min_p=rng.choice([0.0, 0.05]), seed=100 + i,
+                n_predict=rng.randint(1, 60)))
+    results = {}
+    for graphs, pages in ((False, 2000), (True, 2000), (True, 90)):
+        eng = Engine(EngineConfig(model=str(model_dirs["B"]), dtype="float32", num_pages=pages,
+                                  max_batch=16, token_budget=128, chunk=96,
+                                  decode_run=8 if graphs else 1))
+        eng.runner.decode_graphs = graphs
+        results[(graphs, pages)] = eng.generate(prompts, params)
+        eng.cache.check()
+        assert eng.cache.num_free_pages() == pages and eng.cache.num_free_slots == 16
+        assert (eng.scheduler.preempted_total > 0) == (pages == 90)
+        assert (eng.runner.graph_replays > 30) == graphs
+    assert [len(o) for o in results[(False, 2000)]] == [p.n_predict for p in params]
+    assert results[(True, 2000)] == results[(False, 2000)]
+    assert results[(True, 90)] == results[(False, 2000)]
