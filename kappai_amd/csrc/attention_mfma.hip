@@ -87,6 +87,24 @@ __device__ __forceinline__ u32x2_t load_vt4_pg(const bf16_t* __restrict__ vt_poo
   return mask4(v, keep);
 }
 
+// eight key slots of V^T for d index `dd`, keys key0..key0+7 (half a 16-key group: one page),
+// the page already looked up; keys outside [lo, hi] read as zero
+__device__ __forceinline__ u32x4_t load_vt8_pg(const bf16_t* __restrict__ vt_pool, int page, int G,
+                                               int g, int ps, int dd, int key0, int lo, int hi) {
+  const bool want = dd < HEAD_DIM && key0 <= hi && key0 + 7 >= lo && page >= 0;
+  const size_t off =
+      want ? (((size_t)page * G + g) * HEAD_DIM + dd) * ps + key0 % ps : (size_t)0;
+  const u32x4_t v = *reinterpret_cast<const u32x4_t*>(vt_pool + off);
+  uint32_t m[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const bool k0 = want && key0 + 2 * i >= lo && key0 + 2 * i <= hi;
+    const bool k1 = want && key0 + 2 * i + 1 >= lo && key0 + 2 * i + 1 <= hi;
+    m[i] = (k0 ? 0x0000ffffu : 0u) | (k1 ? 0xffff0000u : 0u);
+  }
+  return (u32x4_t){v.x & m[0], v.y & m[1], v.z & m[2], v.w & m[3]};
+}
+
 __device__ __forceinline__ u32x4_t load_k8_pg(const bf16_t* __restrict__ k_pool, int page, int G,
                                               int g, int ps, int key, int d0, int lo, int hi) {
   const bool want = d0 < HEAD_DIM && key >= lo && key <= hi && page >= 0;
@@ -684,34 +702,35 @@ __global__ __launch_bounds__(64) void attn_decode_kernel(
   const float sc = scale * LOG2E;
 
   // A wave takes its keys in chunks of D_KPW: first the chunk's page ids (one load, handed
-  // round by shuffles), then every key and value load of the chunk at once, then the matrix
-  // products and the softmax: two memory round trips a chunk, whatever its length.
+  // round by shuffles), then every key and value load of the chunk at once (16 bytes a lane
+  // each), then the matrix products and the softmax: two memory round trips a chunk, whatever
+  // its length.
   constexpr int NCH = D_KPW / 32;
   for (int c0 = k_begin; c0 < k_end; c0 += D_KPW) {
     const int first_page = c0 / ps;
     int my_page = -1;
     if (first_page + lane < max_blocks && (first_page + lane) * ps <= hi)
       my_page = bt[first_page + lane];
+    // Row r of the key tile tt (of the 32 keys from kb) is key kb + 8 (r / 4) + 4 tt + r % 4:
+    // the lane that holds rows 4 kg .. 4 kg + 3 of both tiles' scores then holds the keys
+    // kb + 8 kg .. + 7 in order, and their values are ONE 16-byte piece of a V^T row.
     u32x4_t kf[NCH][2][D_KS];
-    u32x2_t va[NCH][D_MT], vb[NCH][D_MT];
+    u32x4_t vv[NCH][D_MT];
 #pragma unroll
     for (int c = 0; c < NCH; ++c) {
       const int kb = c0 + 32 * c;
 #pragma unroll
       for (int tt = 0; tt < 2; ++tt) {
-        const int key = kb + 16 * tt + col;
+        const int key = kb + 8 * (col / 4) + 4 * tt + col % 4;
         const int page = __shfl(my_page, min(key / ps - first_page, WAVE - 1), WAVE);
 #pragma unroll
         for (int ks = 0; ks < D_KS; ++ks)
           kf[c][tt][ks] = load_k8_pg(k_pool, page, G, g, ps, key, 32 * ks + 8 * kg, lo, hi);
       }
-      const int pa = __shfl(my_page, min((kb + 4 * kg) / ps - first_page, WAVE - 1), WAVE);
-      const int pb = __shfl(my_page, min((kb + 16 + 4 * kg) / ps - first_page, WAVE - 1), WAVE);
+      const int pv = __shfl(my_page, min((kb + 8 * kg) / ps - first_page, WAVE - 1), WAVE);
 #pragma unroll
-      for (int mt = 0; mt < D_MT; ++mt) {
-        va[c][mt] = load_vt4_pg(vt_pool, pa, G, g, ps, 16 * mt + col, kb + 4 * kg, lo, hi);
-        vb[c][mt] = load_vt4_pg(vt_pool, pb, G, g, ps, 16 * mt + col, kb + 16 + 4 * kg, lo, hi);
-      }
+      for (int mt = 0; mt < D_MT; ++mt)
+        vv[c][mt] = load_vt8_pg(vt_pool, pv, G, g, ps, 16 * mt + col, kb + 8 * kg, lo, hi);
     }
 #pragma unroll
     for (int c = 0; c < NCH; ++c) {
@@ -726,13 +745,13 @@ __global__ __launch_bounds__(64) void attn_decode_kernel(
           s[tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_frag(kf[c][tt][ks]), qf[ks], s[tt], 0,
                                                           0, 0);
       }
-      // lane holds, for head `col`, keys kb + 16*tt + 4*kg + v
+      // lane holds, for head `col`, keys kb + 8*kg + 4*tt + v
       float mloc = -INFINITY;
 #pragma unroll
       for (int tt = 0; tt < 2; ++tt)
 #pragma unroll
         for (int v = 0; v < 4; ++v) {
-          const int key = kb + 16 * tt + 4 * kg + v;
+          const int key = kb + 8 * kg + 4 * tt + v;
           const bool ok = key >= lo && key <= hi;
           s[tt][v] = ok ? s[tt][v] * sc : -INFINITY;
           mloc = fmaxf(mloc, s[tt][v]);
@@ -759,9 +778,8 @@ __global__ __launch_bounds__(64) void attn_decode_kernel(
       const bf16x8_t pf = as_frag(pw);
 #pragma unroll
       for (int mt = 0; mt < D_MT; ++mt) {
-        const u32x4_t vw = {va[c][mt].x, va[c][mt].y, vb[c][mt].x, vb[c][mt].y};
         o[mt] = o[mt] * corr;
-        o[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_frag(vw), pf, o[mt], 0, 0, 0);
+        o[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_frag(vv[c][mt]), pf, o[mt], 0, 0, 0);
       }
     }
   }
