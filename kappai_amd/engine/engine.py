@@ -38,6 +38,8 @@ class EngineConfig:
     chunk: int = 2048
     decode_run: int = 8                  # decode steps queued back to back when nothing but
                                          # decoding is going on (1: every step is waited for)
+    warm_kernels: bool = True            # run one prompt portion of zeros at start-up, so that
+                                         # the first request does not pay for loading the kernels
 
 
 @dataclass
@@ -130,6 +132,28 @@ class Engine:
         self._next_id = 0
         self._t_first_add: Optional[float] = None
         self.last_logits: Optional[torch.Tensor] = None
+        if config.warm_kernels:
+            self._warm_kernels()
+
+    def _warm_kernels(self) -> None:
+        """One prompt portion of the longest size the scheduler will cut, then a single token,
+        for a request that is closed again: every kernel a step of that shape needs is loaded and
+        has run before the first request arrives (its time to the first token would otherwise
+        include that).  Nothing of it is counted in the metrics."""
+        pool = min((g.allocator.num_pages for g in self.cache.paged_groups), default=1 << 20)
+        n = min(self.config.chunk, self.config.token_budget, pool * self.config.page_size - 1,
+                (self.ctx_size or 1 << 30) - 1)
+        if n < 1 or self.cache.num_free_slots < 1:
+            return
+        rc = self.cache.open("warm-up")
+        try:
+            logits = self.runner.step([StepEntry(rc, [0] * n, [n - 1])])
+            warm = RequestSampler(SamplingParams.greedy())
+            self.sampler.sample(logits, [warm])
+            self.sampler.sample(self.runner.step([StepEntry(rc, [0], [0])]), [warm])
+        finally:
+            self.cache.close(rc)
+        self.runner.steps_run = 0
 
     # -- requests ----------------------------------------------------------------------------
     def add_request(self, prompt: Sequence[int], params: Optional[SamplingParams] = None,
