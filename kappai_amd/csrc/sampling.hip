@@ -87,13 +87,183 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_rows_kernel(
   if (tid == 0) out[r] = found;
 }
 
+// The same for rows of at most SAMPLE_THREADS * 4 * SR_STEPS values, which a block keeps in
+// registers: every wave owns a contiguous part of the row and reads it 256 values a step (16
+// bytes a lane), so that the order of the values is (wave, step, lane, place in the lane).  The
+// exponentials are summed in double per (wave, step), one wave finds the part that holds the
+// drawn point of the distribution, and its owner finds the lane and the value.
+#define SR_STEPS 16
+#define SR_WAVES (SAMPLE_THREADS / WAVE)
+
+__device__ __forceinline__ double wave_sum_f64(double v) {
+#pragma unroll
+  for (int m = WAVE / 2; m > 0; m >>= 1) v += __shfl_xor(v, m, WAVE);
+  return v;
+}
+
+__global__ __launch_bounds__(SAMPLE_THREADS) void sample_rows_held_kernel(
+    const float* __restrict__ logits, const float* __restrict__ temperature,
+    const float* __restrict__ uniform, int* __restrict__ out, int V) {
+  __shared__ float redf[SR_WAVES];
+  __shared__ int redi[SR_WAVES];
+  __shared__ double part[SR_WAVES * SR_STEPS];
+  __shared__ double sh_before, sh_target;
+  __shared__ int sh_part, found;
+  const int r = blockIdx.x, tid = threadIdx.x;
+  const int lane = tid % WAVE, wave = tid / WAVE;
+  const float* lg = logits + (size_t)r * V;
+  const float temp = temperature[r];
+  const int region = (((V + SR_WAVES - 1) / SR_WAVES) + 255) / 256 * 256;
+  const int w0 = min(wave * region, V), w1 = min(w0 + region, V);
+  const bool vec = V % 4 == 0 && (reinterpret_cast<uintptr_t>(lg) % 16) == 0;
+  float x[SR_STEPS][4];
+#pragma unroll
+  for (int st = 0; st < SR_STEPS; ++st) {
+    const int idx = w0 + 256 * st + 4 * lane;
+    if (vec) {
+      float4 q = {-INFINITY, -INFINITY, -INFINITY, -INFINITY};
+      if (idx < w1) q = *reinterpret_cast<const float4*>(lg + idx);
+      x[st][0] = q.x; x[st][1] = q.y; x[st][2] = q.z; x[st][3] = q.w;
+    } else {
+#pragma unroll
+      for (int c = 0; c < 4; ++c) x[st][c] = idx + c < w1 ? lg[idx + c] : -INFINITY;
+    }
+  }
+  // ---- max and its lowest index (a lane's indices grow with step and place) ---------------
+  float bv = -INFINITY;
+  int bi = 0x7fffffff;
+#pragma unroll
+  for (int st = 0; st < SR_STEPS; ++st)
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      const int idx = w0 + 256 * st + 4 * lane + c;
+      if (idx < w1 && x[st][c] > bv) { bv = x[st][c]; bi = idx; }
+    }
+#pragma unroll
+  for (int m = WAVE / 2; m > 0; m >>= 1) {
+    const float ov = __shfl_xor(bv, m, WAVE);
+    const int oi = __shfl_xor(bi, m, WAVE);
+    if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+  }
+  if (lane == 0) { redf[wave] = bv; redi[wave] = bi; }
+  __syncthreads();
+  bv = redf[0];
+  bi = redi[0];
+  for (int w = 1; w < SR_WAVES; ++w)
+    if (redf[w] > bv || (redf[w] == bv && redi[w] < bi)) { bv = redf[w]; bi = redi[w]; }
+  if (!(temp > 0.f)) {
+    if (tid == 0) out[r] = bi == 0x7fffffff ? 0 : bi;
+    return;
+  }
+  // ---- e = exp(l/T - max/T); sums per (wave, step) in double ---------------------------------
+  const float inv_t = 1.0f / temp;
+  const float mx = bv * inv_t;
+  double lane_sum[SR_STEPS];
+#pragma unroll
+  for (int st = 0; st < SR_STEPS; ++st) {
+    double sum = 0.0;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      const int idx = w0 + 256 * st + 4 * lane + c;
+      x[st][c] = idx < w1 ? expf(x[st][c] * inv_t - mx) : 0.f;
+      sum += (double)x[st][c];
+    }
+    lane_sum[st] = sum;
+    const double all = wave_sum_f64(sum);
+    if (lane == 0) part[wave * SR_STEPS + st] = all;
+  }
+  if (tid == 0) { found = V - 1; sh_part = -1; }
+  __syncthreads();
+  // ---- the part that holds the drawn point: one wave scans the 256 sums in order -----------
+  if (wave == 0) {
+    constexpr int PER = SR_WAVES * SR_STEPS / WAVE;       // 4 parts a lane
+    double mine[PER], incl = 0.0;
+#pragma unroll
+    for (int j = 0; j < PER; ++j) { mine[j] = part[PER * lane + j]; incl += mine[j]; }
+    // inclusive sums over the lanes
+#pragma unroll
+    for (int off = 1; off < WAVE; off <<= 1) {
+      const double o = __shfl_up(incl, off, WAVE);
+      if (lane >= off) incl += o;
+    }
+    const double total = __shfl(incl, WAVE - 1, WAVE);
+    const double target = (double)uniform[r] * total;
+    // sum of the parts before this lane's: the lane below's inclusive sum itself, so that the
+    // intervals of neighbouring lanes meet exactly (0 for the first)
+    double before = __shfl_up(incl, 1, WAVE);
+    if (lane == 0) before = 0.0;
+    // the lane's last part ends where the next lane begins (the last lane's at the total), so
+    // that the parts cover [0, total) without a gap whatever the rounding of the sums
+    double next = __shfl_down(before, 1, WAVE);
+    if (lane == WAVE - 1) next = total;
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+      const double end = j + 1 < PER ? before + mine[j] : next;
+      if (before <= target && target < end) {               // one part, unless target >= total
+        sh_part = PER * lane + j;
+        sh_before = before;
+        sh_target = target;
+      }
+      before = end;
+    }
+  }
+  __syncthreads();
+  const int p = sh_part;
+  if (p < 0 || wave != p / SR_STEPS) {
+    if (p < 0 && tid == 0) out[r] = found;                // the draw fell on the very end
+    return;
+  }
+  // ---- the wave that owns the part finds the lane, the lane its value --------------------------
+  const int st_p = p % SR_STEPS;
+  double mine = 0.0;
+  float e[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int st = 0; st < SR_STEPS; ++st)
+    if (st == st_p) {
+      mine = lane_sum[st];
+#pragma unroll
+      for (int c = 0; c < 4; ++c) e[c] = x[st][c];
+    }
+  double incl = mine;
+#pragma unroll
+  for (int off = 1; off < WAVE; off <<= 1) {
+    const double o = __shfl_up(incl, off, WAVE);
+    if (lane >= off) incl += o;
+  }
+  double below = __shfl_up(incl, 1, WAVE);
+  if (lane == 0) below = 0.0;
+  const double before = sh_before + below, target = sh_target;
+  const bool here = before <= target && target < sh_before + incl;   // ends where the next begins
+  // rounding may leave the point just past the last lane's sum: the last lane with values takes it
+  const unsigned long long any = __ballot(here);
+  if (any == 0ull) {
+    if (lane == 0) out[r] = min(w0 + 256 * st_p + 255, w1 - 1);
+    return;
+  }
+  if (here) {
+    // the lane's sum was made in this order, so the last step reaches it exactly; values past
+    // the end of the row are zero and cannot be the one at which the sum passes the point
+    double acc = before;
+    int pick = 3;
+    for (int c = 0; c < 4; ++c) {
+      acc += (double)e[c];
+      if (target < acc) { pick = c; break; }
+    }
+    out[r] = min(w0 + 256 * st_p + 4 * lane + pick, w1 - 1);
+  }
+}
+
 extern "C" int kappai_sample_rows(const float* logits, const float* temperature,
                                   const float* uniform, int* out, int n_rows, int V,
                                   hipStream_t stream) {
   if (n_rows <= 0) return 0;
   if (V < 1) return (int)hipErrorInvalidValue;
-  hipLaunchKernelGGL(sample_rows_kernel, dim3(n_rows), dim3(SAMPLE_THREADS), 0, stream, logits,
-                     temperature, uniform, out, V);
+  if (V <= SAMPLE_THREADS * 4 * SR_STEPS)
+    hipLaunchKernelGGL(sample_rows_held_kernel, dim3(n_rows), dim3(SAMPLE_THREADS), 0, stream,
+                       logits, temperature, uniform, out, V);
+  else
+    hipLaunchKernelGGL(sample_rows_kernel, dim3(n_rows), dim3(SAMPLE_THREADS), 0, stream, logits,
+                       temperature, uniform, out, V);
   KAPPAI_RETURN_LAUNCH_STATUS();
 }
 

@@ -674,16 +674,25 @@ def test_attention_shared_tiles_find_one_far_key(ops):
 
 # ---------------------------------------------------------------------------------------
 def test_sample_rows(ops):
-    V = 1003
-    logits = rand((6, V), F32, 40, 3.0)
-    logits[0, 17] = logits[0, 900] = 50.0          # a tie: the lowest id wins
-    logits[1, V - 1] = 60.0
-    temp = torch.tensor([0.0, 0.0, 0.8, 0.8, 2.0, 0.3])
-    u = torch.tensor([0.5, 0.5, 0.0, 0.999999, 0.37, 0.62])
-    got = ops.sample_rows(logits.to(DEV), temp.to(DEV), u.to(DEV)).cpu()
-    want = ref.sample_rows(logits, temp, u)
-    assert got.tolist() == want.tolist()
-    assert got[0] == 17 and got[1] == V - 1
+    # a vocabulary that is no multiple of 4, one that fills the registers of the block exactly,
+    # and one beyond them (the kernel that reads the row again)
+    for V in (1003, 65536, 70001):
+        logits = rand((6, V), F32, 40, 3.0)
+        logits[0, 17] = logits[0, 900] = 50.0          # a tie: the lowest id wins
+        logits[1, V - 1] = 60.0
+        temp = torch.tensor([0.0, 0.0, 0.8, 0.8, 2.0, 0.3])
+        u = torch.tensor([0.5, 0.5, 0.0, 0.999999, 0.37, 0.62])
+        got = ops.sample_rows(logits.to(DEV), temp.to(DEV), u.to(DEV)).cpu()
+        want = ref.sample_rows(logits, temp, u)
+        assert got.tolist() == want.tolist(), V
+        assert got[0] == 17 and got[1] == V - 1
+    # every place of a small row can be drawn, the last one too
+    flat = torch.zeros((1, 7))
+    for k in range(7):
+        uk = torch.tensor([(k + 0.5) / 7])
+        assert int(ops.sample_rows(flat.to(DEV), torch.ones(1).to(DEV), uk.to(DEV))[0]) == k
+    assert int(ops.sample_rows(flat.to(DEV), torch.ones(1).to(DEV),
+                               torch.tensor([0.99999994]).to(DEV))[0]) == 6
     # many draws follow the distribution
     lg = torch.log(torch.tensor([0.5, 0.2, 0.15, 0.1, 0.03, 0.01, 0.007, 0.003])).repeat(4000, 1)
     uu = torch.rand(4000, generator=torch.Generator().manual_seed(1))
