@@ -265,7 +265,7 @@ def test_linear_partial_sums(ops, M, N, K):
 
 
 @pytest.mark.parametrize("M", [1, 2, 4])
-@pytest.mark.parametrize("N,K", [(48, 64), (6144, 2048), (200, 520), (1000, 4096)])
+@pytest.mark.parametrize("N,K", [(48, 64), (6144, 2048), (200, 520), (1000, 4096), (64, 2048)])
 @pytest.mark.parametrize("delta_kind", ["none", "bf16", "f32", "parts"])
 def test_linear_makes_the_normalised_rows_itself(ops, M, N, K, delta_kind):
     """A product whose input is a pending RMSNorm: the same result as the norm kernel followed by
@@ -300,7 +300,8 @@ def test_linear_makes_the_normalised_rows_itself(ops, M, N, K, delta_kind):
           "partial sums")
 
 
-@pytest.mark.parametrize("M,F,K", [(1, 8192, 2048), (3, 48, 136), (4, 320, 1024)])
+@pytest.mark.parametrize("M,F,K", [(1, 8192, 2048), (3, 48, 136), (4, 320, 1024), (1, 64, 2048),
+                                   (2, 32, 4096)])
 def test_linear_swiglu_makes_the_normalised_rows_itself(ops, M, F, K):
     resid, wn = rand((M, K), F32, 85, 2.0), 1 + rand((K,), F32, 86, 0.1)
     delta = rand((4, M, K), F32, 87)
