@@ -500,6 +500,8 @@ ATT_CASES = [
     (8, 2, 64, 16, [0, 300, 31], [130, 70, 1], 64, 1, True, 0),                 # 4 heads a kv head
     (8, 1, 128, 32, [250, 0], [45, 97], 128, 1, True, 0),                       # 8 heads a kv head
     (4, 1, 64, 48, [120, 0, 66], [80, 33, 2], 64, 1, True, 50),                 # window, page 48
+    (4, 2, 64, 16, [20000, 9000], [1, 1], 64, 1, True, 0),       # decode over more than 64 key splits
+    (8, 2, 64, 16, [12000], [70], 64, 1, True, 0),               # a portion after a long history
 ]
 
 
