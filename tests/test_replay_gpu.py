@@ -319,3 +319,47 @@ def test_layer_sizes_of_the_1_2b_model(tmp_path, sizes_1_2b_dir, dtype):
     err, where = worst_error(got, ref)
     assert err < tol, (err, tol, where, first_bad(got, ref, tol))
     _models.pop((str(folder), dtype), None)        # 0.7 to 1.3 GB on the GPU
+
+
+def test_trace_semantics(tmp_path, model_dirs):
+    """What a trace may do beside the regular schedules: places asked for out of order and
+    twice, a request that is left out of steps and goes on later, a step that wants nothing
+    (no file), a request ended by a step that brings no tokens for it, an empty step."""
+    from kappai_amd.engine.replay import TraceReplayer, make_replay_cache
+    from kappai_amd.engine.step import StepRunner
+    cfg = TINY["C"][0]
+    vocab = cfg["vocab_size"]
+    requests = make_requests(vocab, [40, 23, 9], seed=18)
+    a, b, c = requests["r0"], requests["r1"], requests["r2"]
+    steps = [
+        {"step": 0, "entries": [{"id": "a", "tokens": a[:10], "want": [9, 0, 9, 3]}], "end": []},
+        {"step": 1, "entries": [{"id": "b", "tokens": b[:20], "want": []}], "end": []},
+        {"step": 2, "entries": [{"id": "a", "tokens": a[10:12], "want": [1]},
+                                {"id": "c", "tokens": c, "want": [8]}], "end": ["c"]},
+        {"step": 3, "entries": [], "end": []},
+        {"step": 4, "entries": [{"id": "b", "tokens": b[20:], "want": [2, 1, 0]}], "end": []},
+        {"step": 5, "entries": [{"id": "a", "tokens": a[12:], "want": [27]}], "end": ["b"]},
+        {"step": 6, "entries": [], "end": ["a"]},
+    ]
+    wanted = {0: [("r0", 9), ("r0", 0), ("r0", 9), ("r0", 3)], 2: [("r0", 11), ("r2", 8)],
+              4: [("r1", 22), ("r1", 21), ("r1", 20)], 5: [("r0", 39)]}
+    ref = plain_logits(model_dirs["C"], requests)
+    scale = max(float(np.abs(v).max()) for v in ref.values())
+    for dtype in ("float32", "bfloat16"):
+        model = gpu_model(model_dirs["C"], dtype)
+        cache = make_replay_cache(model, 64 + 64 + 64)
+        cache.allocate_storage(model.dtype, "cuda:0", poison=True)
+        out_dir = tmp_path / dtype
+        rep = TraceReplayer(StepRunner(model, cache, "cuda:0"), out_dir)
+        tol = tolerance(model_dirs["C"], requests, dtype)
+        for obj in steps:
+            res = rep.run_step(obj)
+            if obj["step"] in wanted:
+                rows = np.fromfile(out_dir / f"{obj['step']}.f32", dtype="<f4").reshape(-1, vocab)
+                assert rows.shape[0] == len(wanted[obj["step"]]) and np.array_equal(rows, res)
+                for row, (rid, pos) in zip(rows, wanted[obj["step"]]):
+                    assert float(np.abs(row - ref[rid][pos]).max()) / scale < tol, (dtype, obj["step"], rid, pos)
+            else:
+                assert res is None and not (out_dir / f"{obj['step']}.f32").exists()
+        cache.check()
+        assert not cache.live_requests()
