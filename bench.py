@@ -41,6 +41,72 @@ LFM2_1_2B = {
 }
 
 
+def lfm2_shape(hidden, layers, attention_at, heads, kv_heads, intermediate):
+    raw = dict(LFM2_1_2B)
+    raw.update(hidden_size=hidden, num_hidden_layers=layers, num_attention_heads=heads,
+               num_key_value_heads=kv_heads, intermediate_size=intermediate,
+               layer_types=["full_attention" if i in attention_at else "conv"
+                            for i in range(layers)])
+    return raw
+
+
+LFM2_350M = lfm2_shape(1024, 16, (2, 5, 8, 10, 12, 14), 16, 8, 6656)
+LFM2_2_6B = lfm2_shape(2048, 30, (2, 6, 10, 14, 18, 21, 24, 27), 32, 8, 10752)
+
+# Serving workloads (through Engine: scheduler, prompt portions beside decoded tokens, sampling)
+WORKLOADS = {
+    # 64 requests at once, prompts of 128..2048 tokens cut into portions of 512, 256 tokens each
+    "serve-350m": dict(raw=LFM2_350M, name="LFM2-350M shape", requests=64, prompt=(128, 2048),
+                       n_predict=256, chunk=512, token_budget=576, ctx=4096),
+    # 16 requests with 32,768-token contexts, 512 tokens each
+    "long-2.6b": dict(raw=LFM2_2_6B, name="LFM2-2.6B shape", requests=16, prompt=(32768 - 512, 32768 - 512),
+                      n_predict=512, chunk=2048, token_budget=2048, ctx=32768),
+}
+
+
+def run_workload(key, dtype, device):
+    """One serving workload from start to end through ``Engine.generate`` with greedy sampling:
+    all requests arrive together.  Prints one JSON line: generated tokens a second over the
+    whole run (prompts included in the time), and the engine's own prefill / decode rates."""
+    import torch
+
+    from kappai_amd.engine import Engine, EngineConfig
+    from kappai_amd.sampling import SamplingParams
+    w = WORKLOADS[key]
+    model = random_model(dict(w["raw"]), dtype, device)
+    n = w["requests"]
+    page = 16
+    eng = Engine(EngineConfig(dtype=dtype, ctx_size=w["ctx"], max_batch=n, page_size=page,
+                              num_pages=n * (w["ctx"] // page), token_budget=w["token_budget"],
+                              chunk=w["chunk"]), model=model)
+    g = torch.Generator().manual_seed(3)
+    lo, hi = w["prompt"]
+    lengths = [int(t) for t in torch.randint(lo, hi + 1, (n,), generator=g)]
+    prompts = [[int(t) for t in torch.randint(0, model.vocab_size, (L,), generator=g)]
+               for L in lengths]
+    sync()
+    t0 = time.perf_counter()
+    out = eng.generate(prompts, SamplingParams.greedy(n_predict=w["n_predict"]))
+    sync()
+    dt = time.perf_counter() - t0
+    m = eng.metrics
+    generated = sum(len(o) for o in out)
+    cfg = model.config
+    print(json.dumps({
+        "metric": f"generated tok/s, {key} workload ({w['name']})", "value": round(generated / dt, 1),
+        "unit": "tok/s", "n_gpus": 1, "seconds": round(dt, 3), "dtype": dtype, "data": "synthetic",
+        "config": {"model": w["name"] + ", random weights", "hidden_size": cfg.hidden_size,
+                   "num_layers": cfg.num_hidden_layers, "attention_layers": len(cfg.attention_layers),
+                   "ff_dim": cfg.ff_dim, "requests": n, "prompt_tokens": sum(lengths),
+                   "generated_tokens": generated, "chunk": w["chunk"],
+                   "token_budget": w["token_budget"], "ctx_size": w["ctx"]},
+        "engine": {"steps": m.steps, "prefill_tok_s": round(m.pp, 1), "decode_tok_s": round(m.tg, 1),
+                   "ttft_ms": round(m.first_token_ms, 2), "graph_replays": eng.runner.graph_replays,
+                   "preemptions": eng.scheduler.preempted_total},
+    }))
+    return 0
+
+
 def random_model(raw, dtype, device, seed=0, std=0.02):
     """The model of ``raw`` with N(0, std) weights made on the GPU (norm weights 1)."""
     import torch
@@ -167,10 +233,15 @@ def main() -> int:
     ap.add_argument("--skip-points", action="store_true", help="only the headline batch")
     ap.add_argument("--no-graphs", action="store_true",
                     help="launch decode steps kernel by kernel (for counter collection)")
+    ap.add_argument("--workload", default="decode", choices=["decode"] + sorted(WORKLOADS),
+                    help="decode: the headline run; the others are serving workloads through "
+                         "the engine's scheduler")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this engine runs on one GPU; --gpus must be 1 (nothing was measured)")
         return 2
+    if args.workload != "decode":
+        return run_workload(args.workload, args.dtype, "cuda:0")
 
     import torch
 
