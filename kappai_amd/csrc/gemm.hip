@@ -903,6 +903,14 @@ static void launch_skinny_mt(const bf16_t* A, const bf16_t* W, const float* bias
       return;
     }
   }
+  // 8 to 16 rows and columns enough (the output head): four column tiles for every fragment of
+  // A (58 against 62 us for 65,536 columns at 8 rows, 62 against 74 at 16; slower below 8 rows)
+  if constexpr (EPI == 0 && MT == 1) {
+    if (!nin && M >= 8 && (long)(N / 64) * ksplit >= 512) {
+      launch_skinny<TO, MT, 4, EPI, 4>(A, W, bias, C, M, N, K, lda, ldc, ksplit, cs, stream);
+      return;
+    }
+  }
   const int blocks = ((N + 15) / 16) * ksplit;
   const int kb = K / ksplit;                              // K a block
   constexpr int NG = EPI == 1 ? 2 : (EPI == 2 ? 3 : 1);

@@ -157,6 +157,10 @@ def build_all(verbose: bool = True, force: bool = True) -> None:
 def library(name: str, **defines) -> ctypes.CDLL:
     """The loaded library ``name`` (compiled with ``defines`` as -D constants); compiled
     first if no up-to-date build exists."""
+    if not defines:
+        lib = _loaded.get(name)          # every kernel launch comes through here
+        if lib is not None:
+            return lib
     built = _built_name(name, defines)
     lib = _loaded.get(built)
     if lib is not None:

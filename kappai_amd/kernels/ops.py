@@ -36,23 +36,29 @@ def _ptr(t: Optional[torch.Tensor]) -> _vp:
     return _vp(0 if t is None else t.data_ptr())
 
 
-def _need(cond: bool, msg: str) -> None:
+def _need(cond: bool, msg) -> None:
+    """``msg`` is the text or a function that makes it (the text is then only put together
+    when the check fails: these checks run for every kernel of every step)."""
     if not cond:
-        raise ValueError(msg)
+        raise ValueError(msg() if callable(msg) else msg)
 
 
 def _gpu(name: str, t: torch.Tensor, dtype=None, contiguous=True) -> None:
-    _need(isinstance(t, torch.Tensor), f"{name}: a tensor is needed")
-    _need(t.is_cuda, f"{name}: must live on the GPU (kappai_amd has no CPU path), got {t.device}")
-    if dtype is not None:
+    if not isinstance(t, torch.Tensor):
+        raise ValueError(f"{name}: a tensor is needed")
+    if not t.is_cuda:
+        raise ValueError(f"{name}: must live on the GPU (kappai_amd has no CPU path), "
+                         f"got {t.device}")
+    if dtype is not None and t.dtype is not dtype:
         dts = dtype if isinstance(dtype, (tuple, list)) else (dtype,)
-        _need(t.dtype in dts, f"{name}: dtype {t.dtype}, expected {' or '.join(map(str, dts))}")
-    if contiguous:
-        _need(t.is_contiguous(), f"{name}: must be contiguous")
+        if t.dtype not in dts:
+            raise ValueError(f"{name}: dtype {t.dtype}, expected {' or '.join(map(str, dts))}")
+    if contiguous and not t.is_contiguous():
+        raise ValueError(f"{name}: must be contiguous")
 
 
 def _is_bf16(dtype) -> int:
-    _need(dtype in (F32, BF16), f"compute dtype must be float32 or bfloat16, got {dtype}")
+    _need(dtype in (F32, BF16), lambda: f"compute dtype must be float32 or bfloat16, got {dtype}")
     return 1 if dtype == BF16 else 0
 
 
@@ -80,7 +86,8 @@ def add_rmsnorm(resid: torch.Tensor, delta: Optional[torch.Tensor], weight: torc
     _gpu("resid", resid, F32)
     _gpu("weight", weight, F32)
     _need(resid.dim() == 2 and weight.shape == (resid.shape[1],),
-          f"add_rmsnorm: resid {tuple(resid.shape)} and weight {tuple(weight.shape)} disagree")
+          lambda: f"add_rmsnorm: resid {tuple(resid.shape)} and weight {tuple(weight.shape)} "
+                  "disagree")
     isb = _is_bf16(out_dtype)
     n_part, pstride, delta_f32 = 1, 0, 0
     if delta is not None:
@@ -190,18 +197,39 @@ def cast(x: torch.Tensor, dtype) -> torch.Tensor:
 
 
 # ---------------------------------------------------------------------------------------
+def _split_k_large(M: int, N: int, K: int) -> int:
+    """K ranges for a product with more than 64 rows whose consumer adds partial sums: the
+    number that a model of the block kernel's time likes best (within 12 % of the best of a
+    sweep over 40 shapes, 1 % on average).  A 128 x 128 block that has a CU to itself takes
+    about 0.62 us per 64 of K whatever else goes on, so a product with few blocks is bound by
+    the length of K and gains almost linearly from being cut, until the chip is full (two
+    blocks a CU, each then a quarter slower; with 192 blocks of 256 x 256 or more the kernel
+    takes its 256 x 256 form, about 1 us per 64 of K) or the float partial sums ([S, M, N],
+    written here and read again by the consumer) cost more than the cut saves.  Every range is
+    a multiple of 128 long, as the kernel asks."""
+    best, best_t = 1, None
+    for split in range(1, 9):
+        if K % (128 * split) or (split > 1 and K // split < 256):
+            continue
+        steps = K / split / 64
+        blocks256 = ((M + 255) // 256) * ((N + 255) // 256) * split
+        if blocks256 >= 192:
+            t = -(-blocks256 // 256) * (steps * 1.0 + 4.5)
+        else:
+            blocks = ((M + 127) // 128) * ((N + 127) // 128) * split
+            t = -(-blocks // 512) * (steps * 0.62 * (1.25 if blocks > 256 else 1.0) + 2.5)
+        t += (split * M * N * 8 if split > 1 else M * N * 4) / 5e6     # written and read again
+        if best_t is None or t < best_t - 1e-9:
+            best, best_t = split, t
+    return best
+
+
 def split_k_for(M: int, N: int, K: int) -> int:
     """How many K ranges a product is cut into when its consumer takes partial sums (1: not
     split).  Decode (M <= 64): so that about 512 blocks stream the matrix (17 rows and more: what
-    suits the kernel that takes them).  Larger M: only long
-    K (ranges of 2048 or more) and few 128 x 128 blocks; every range is a multiple of 128 long,
-    as the large-product kernel asks."""
+    suits the kernel that takes them).  Larger M: see ``_split_k_large``."""
     if M > 64:
-        blocks = ((M + 127) // 128) * ((N + 127) // 128)
-        split = max(1, min(8, 512 // blocks, K // 2048))
-        while split > 1 and K % (128 * split):
-            split -= 1
-        return split
+        return _split_k_large(M, N, K)
     if M > 16:
         # the kernel that shares the rows through LDS: blocks of 64 columns, K ranges that are
         # multiples of 512 and at least 1024 long, 128 blocks or more
@@ -232,14 +260,14 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] =
     _gpu("x", x, (F32, BF16), contiguous=False)
     _gpu("weight", weight, (F32, BF16))
     _need(x.dim() == 2 and weight.dim() == 2 and x.shape[1] == weight.shape[1],
-          f"linear: x {tuple(x.shape)} does not meet weight {tuple(weight.shape)}")
+          lambda: f"linear: x {tuple(x.shape)} does not meet weight {tuple(weight.shape)}")
     _need(x.stride(1) == 1 or x.shape[1] == 1, "linear: x must have unit stride along K")
     M, K = x.shape
     N = weight.shape[0]
     out_dtype = out_dtype or x.dtype
     if bias is not None:
         _gpu("bias", bias, F32)
-        _need(bias.shape == (N,), f"linear: bias {tuple(bias.shape)} for N={N}")
+        _need(bias.shape == (N,), lambda: f"linear: bias {tuple(bias.shape)} for N={N}")
     if weight.dtype == F32:
         xf = x if x.dtype == F32 else cast(x.contiguous(), F32)
         out = torch.empty((M, N), dtype=F32, device=x.device)
@@ -252,9 +280,10 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] =
     if not (K % 8 == 0 and lda % 8 == 0 and xb.data_ptr() % 16 == 0
             and weight.data_ptr() % 16 == 0):
         # the matrix-core kernels read 16 bytes at a time; anything else goes the plain way
-        _need(not force_kernel, f"linear: K ({K}) and the row stride ({lda}) must be multiples of "
-              "8 and the tensors 16-byte aligned for the kernel that was asked for")
-        _need(M <= MAX_GRID_Y, f"linear: {M} rows with a width that is no multiple of 8")
+        _need(not force_kernel,
+              lambda: f"linear: K ({K}) and the row stride ({lda}) must be multiples of 8 and "
+                      "the tensors 16-byte aligned for the kernel that was asked for")
+        _need(M <= MAX_GRID_Y, lambda: f"linear: {M} rows with a width that is no multiple of 8")
         out = torch.empty((M, N), dtype=out_dtype, device=x.device)
         check(library("gemm").kappai_gemm_bf16_any(
             _ptr(xb), _ptr(weight), _ptr(bias), _ptr(out), _c_int(M), _c_int(N), _c_int(K),
@@ -282,7 +311,7 @@ def _linear_normed(x: PendingNorm, weight, bias, out_dtype, partial_sums, split_
     out_dtype = out_dtype or x.dtype
     if bias is not None:
         _gpu("bias", bias, F32)
-        _need(bias.shape == (N,), f"linear: bias {tuple(bias.shape)} for N={N}")
+        _need(bias.shape == (N,), lambda: f"linear: bias {tuple(bias.shape)} for N={N}")
     ksplit = (split_k or split_k_for(M, N, K)) if partial_sums else 1
     if ksplit > 1:
         out = torch.empty((ksplit, M, N), dtype=F32, device=x.device)
@@ -304,8 +333,8 @@ def interleave_gate_up(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
     next 16 gate rows, ...  [2F, K] from two [F, K] matrices; F must be a multiple of 16."""
     F, K = gate.shape
     _need(up.shape == gate.shape and F % SWIGLU_GROUP == 0,
-          f"interleave_gate_up: {tuple(gate.shape)} and {tuple(up.shape)}; F must be a multiple "
-          f"of {SWIGLU_GROUP}")
+          lambda: f"interleave_gate_up: {tuple(gate.shape)} and {tuple(up.shape)}; F must be a "
+                  f"multiple of {SWIGLU_GROUP}")
     g = gate.reshape(F // SWIGLU_GROUP, 1, SWIGLU_GROUP, K)
     u = up.reshape(F // SWIGLU_GROUP, 1, SWIGLU_GROUP, K)
     return torch.cat([g, u], dim=1).reshape(2 * F, K).contiguous()
@@ -333,14 +362,14 @@ def linear_swiglu(x: torch.Tensor, weight: torch.Tensor, force_kernel: int = 0) 
     _gpu("weight", weight, BF16)
     _need(x.dim() == 2 and weight.dim() == 2 and x.shape[1] == weight.shape[1]
           and weight.shape[0] % (2 * SWIGLU_GROUP) == 0,
-          f"linear_swiglu: x {tuple(x.shape)}, weight {tuple(weight.shape)}")
+          lambda: f"linear_swiglu: x {tuple(x.shape)}, weight {tuple(weight.shape)}")
     _need(x.stride(1) == 1 or x.shape[1] == 1, "linear_swiglu: x must have unit stride along K")
     M, K = x.shape
     F = weight.shape[0] // 2
     lda = x.stride(0) if M > 1 else K
     _need(K % 8 == 0 and lda % 8 == 0 and x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0,
-          f"linear_swiglu: K ({K}) and the row stride ({lda}) must be multiples of 8 and the "
-          f"tensors 16-byte aligned")
+          lambda: f"linear_swiglu: K ({K}) and the row stride ({lda}) must be multiples of 8 "
+                  "and the tensors 16-byte aligned")
     out = torch.empty((M, F), dtype=BF16, device=x.device)
     check(library("gemm").kappai_gemm_bf16_swiglu(
         _ptr(x), _ptr(weight), _ptr(out), _c_int(M), _c_int(F), _c_int(K), _c_int(lda), _c_int(F),
@@ -364,11 +393,11 @@ def linear_shortconv_step(x: torch.Tensor, in_proj: torch.Tensor, in_bias: Optio
     _gpu("seg_slot", seg_slot, I32)
     M, K = x.shape
     D, L = taps.shape
-    _need(in_proj.shape == (3 * D, K), f"in_proj {tuple(in_proj.shape)} for D={D}, K={K}")
+    _need(in_proj.shape == (3 * D, K), lambda: f"in_proj {tuple(in_proj.shape)} for D={D}, K={K}")
     _need(M <= 64 and D % 16 == 0, "linear_shortconv_step: at most 64 rows, width a multiple of 16")
     _need(seg_pos0.shape == (M,) and seg_slot.shape == (M,), "one segment a row")
     _need(L >= 2 and state.dim() == 3 and state.shape[1:] == (D, L - 1),
-          f"state {tuple(state.shape)} for D={D}, L={L}")
+          lambda: f"state {tuple(state.shape)} for D={D}, L={L}")
     lda = x.stride(0) if M > 1 else K
     _need((x.stride(1) == 1 or K == 1) and K % 8 == 0 and lda % 8 == 0
           and x.data_ptr() % 16 == 0 and in_proj.data_ptr() % 16 == 0,
@@ -376,7 +405,7 @@ def linear_shortconv_step(x: torch.Tensor, in_proj: torch.Tensor, in_bias: Optio
     for n, t, shp in (("in_bias", in_bias, (3 * D,)), ("conv_bias", conv_bias, (D,))):
         if t is not None:
             _gpu(n, t, F32)
-            _need(t.shape == shp, f"{n} must be {shp}")
+            _need(t.shape == shp, lambda: f"{n} must be {shp}")
     out = torch.empty((M, D), dtype=BF16, device=x.device)
     check(library("gemm").kappai_gemm_bf16_shortconv_step(
         _ptr(x), _ptr(in_proj), _ptr(in_bias), _ptr(out), _c_int(M), _c_int(D), _c_int(K),
@@ -406,9 +435,9 @@ def shortconv(proj: torch.Tensor, taps: torch.Tensor, bias: Optional[torch.Tenso
     T = proj.shape[0]
     D, L = taps.shape
     S = seg_pos0.shape[0]
-    _need(proj.shape == (T, 3 * D), f"shortconv: proj {tuple(proj.shape)} for D={D}")
+    _need(proj.shape == (T, 3 * D), lambda: f"shortconv: proj {tuple(proj.shape)} for D={D}")
     _need(L >= 2 and state.dim() == 3 and state.shape[1:] == (D, L - 1),
-          f"shortconv: state {tuple(state.shape)} for D={D}, L={L}")
+          lambda: f"shortconv: state {tuple(state.shape)} for D={D}, L={L}")
     _need(row_seg.shape[0] == T and seg_start.shape[0] == S + 1 and seg_slot.shape[0] == S,
           "shortconv: segment tables do not fit the batch")
     _need(T <= 2 ** 31 - 1 and S >= 1, "shortconv: batch too large or empty")
@@ -431,11 +460,11 @@ def _shortconv_step_parts(parts, taps, bias, state, seg_pos0, seg_slot) -> torch
     S, T, W = parts.shape
     D, L = taps.shape
     _need(parts.dtype == F32 and W == 3 * D and parts.is_contiguous(),
-          f"shortconv: partial sums {tuple(parts.shape)} for D={D}")
+          lambda: f"shortconv: partial sums {tuple(parts.shape)} for D={D}")
     _need(seg_pos0.shape[0] == T and seg_slot.shape[0] == T,
           "shortconv: partial sums are taken only when every segment is a single row")
     _need(L >= 2 and state.dim() == 3 and state.shape[1:] == (D, L - 1),
-          f"shortconv: state {tuple(state.shape)} for D={D}, L={L}")
+          lambda: f"shortconv: state {tuple(state.shape)} for D={D}, L={L}")
     if bias is not None:
         _gpu("bias", bias, F32)
         _need(bias.shape == (D,), "shortconv: bias must be [D]")
@@ -454,7 +483,7 @@ def _check_pools(k_pool, v_pool, G, page_size, d) -> None:
     _need(k_pool.dim() == 4 and v_pool.dim() == 4 and k_pool.shape[0] == v_pool.shape[0]
           and tuple(k_pool.shape[1:]) == (G, page_size, d)
           and tuple(v_pool.shape[1:]) == (G, d, page_size),
-          f"pools {tuple(k_pool.shape)} / {tuple(v_pool.shape)} are not keys [pages, {G}, "
+          lambda: f"pools {tuple(k_pool.shape)} / {tuple(v_pool.shape)} are not keys [pages, {G}, "
           f"{page_size}, {d}] and transposed values [pages, {G}, {d}, {page_size}]")
 
 
@@ -477,25 +506,26 @@ def qk_norm_rope_store(qkv: torch.Tensor, n_heads: int, n_kv_heads: int, head_di
     parts = qkv if qkv.dim() == 3 else None
     if parts is not None:
         _need(parts.dtype == F32 and parts.shape[2] >= width and parts.is_contiguous(),
-              f"qk_norm_rope_store: partial sums {tuple(parts.shape)}")
+              lambda: f"qk_norm_rope_store: partial sums {tuple(parts.shape)}")
         T = parts.shape[1]
         q_out = torch.empty((T, H * d), dtype=BF16, device=parts.device)
         row_stride, data_dtype = parts.shape[2], BF16
     else:
         T = qkv.shape[0]
         _need(qkv.dim() == 2 and qkv.shape[1] >= width,
-              f"qk_norm_rope_store: qkv {tuple(qkv.shape)}")
+              lambda: f"qk_norm_rope_store: qkv {tuple(qkv.shape)}")
         q_out, row_stride, data_dtype = None, qkv.stride(0), qkv.dtype
-    _need(1 <= d <= MAX_HEAD_DIM, f"head_dim {d} is beyond the kernels' limit {MAX_HEAD_DIM}")
+    _need(1 <= d <= MAX_HEAD_DIM,
+          lambda: f"head_dim {d} is beyond the kernels' limit {MAX_HEAD_DIM}")
     _need(H + 2 * G <= MAX_GRID_Y, "too many heads for one launch")
     for n, t in (("q_norm_w", q_norm_w), ("k_norm_w", k_norm_w)):
         if t is not None:
             _gpu(n, t, F32)
-            _need(t.shape == (d,), f"{n} must be [head_dim]")
+            _need(t.shape == (d,), lambda: f"{n} must be [head_dim]")
     if rot_mode != ROT_NONE:
         _gpu("cos", cos, F32)
         _gpu("sin", sin, F32)
-        _need(rot_dim % 2 == 0 and 0 < rot_dim <= d, f"rot_dim {rot_dim} for head_dim {d}")
+        _need(rot_dim % 2 == 0 and 0 < rot_dim <= d, lambda: f"rot_dim {rot_dim} for head_dim {d}")
         _need(cos.shape == sin.shape and cos.dim() == 2 and cos.shape[1] == rot_dim // 2,
               "rotation tables must be [positions, rot_dim/2]")
     _gpu("row_pos", row_pos, I32)
@@ -543,10 +573,10 @@ def paged_attention(q: torch.Tensor, n_heads: int, n_kv_heads: int, head_dim: in
     _gpu("q", q, (F32, BF16), contiguous=False)
     T = q.shape[0]
     _need(q.dim() == 2 and q.shape[1] >= H * d and (q.stride(1) == 1),
-          f"paged_attention: q {tuple(q.shape)}")
+          lambda: f"paged_attention: q {tuple(q.shape)}")
     _need(d % 8 == 0 and d <= MAX_HEAD_DIM,
-          f"head_dim {d}: the attention kernels take multiples of 8 up to {MAX_HEAD_DIM}")
-    _need(G >= 1 and H % G == 0 and H <= MAX_GRID_Y, f"{H} heads over {G} kv heads")
+          lambda: f"head_dim {d}: the attention kernels take multiples of 8 up to {MAX_HEAD_DIM}")
+    _need(G >= 1 and H % G == 0 and H <= MAX_GRID_Y, lambda: f"{H} heads over {G} kv heads")
     _gpu("k_pool", k_pool, q.dtype)
     _gpu("v_pool", v_pool, q.dtype)
     _check_pools(k_pool, v_pool, G, page_size, d)
@@ -588,7 +618,7 @@ def paged_attention(q: torch.Tensor, n_heads: int, n_kv_heads: int, head_dim: in
             _c_int(window or 0), _c_float(scale), _c_int(prefill_variant), _stream()),
             "attn_prefill")
         return out
-    _need(kernel == "decode", f"unknown attention kernel {kernel!r}")
+    _need(kernel == "decode", lambda: f"unknown attention kernel {kernel!r}")
     _need(H // G <= 16, "the decode kernel takes at most 16 query heads per kv head")
     _need(max_position is not None, "the decode kernel needs the batch's largest position")
     n_keys = min(max_position + 1, window) + 32 if window else max_position + 1
@@ -651,7 +681,7 @@ def sample_filtered(logits: torch.Tensor, rows: torch.Tensor, keep: torch.Tensor
     for name, t in (("temperature", temperature), ("top_p", top_p), ("min_p", min_p),
                     ("uniform", uniform)):
         _gpu(name, t, F32)
-        _need(t.shape == (n,), f"{name}: one value per entry")
+        _need(t.shape == (n,), lambda: f"{name}: one value per entry")
     _need(keep.shape == (n,) and out.shape == (logits.shape[0],), "sample_filtered: table sizes")
     check(library("sampling").kappai_sample_filtered(
         _ptr(logits), _ptr(rows), _ptr(keep), _ptr(temperature), _ptr(top_p), _ptr(min_p),
