@@ -329,12 +329,13 @@ static void launch_tile_cfg(const bf16_t* A, const bf16_t* W, const float* bias,
 
 template <int N> struct IntC { static constexpr int value = N; };
 
-template <typename TO, int EPI, int WT>
+template <typename TO, int EPI, int WT, bool DEEP = false>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4 / WT, 4 / WT)))
 void gemm_bf16_block256_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W,
                                const float* __restrict__ bias, TO* __restrict__ C, int M, int N,
                                int K, int lda, int ldc, int tiles_n) {
   // WT x WT accumulator tiles of 32 x 32 a wave: 4 -> 256 x 256 blocks, 2 -> 128 x 128
+  static_assert(!DEEP || WT == 2, "four LDS buffers: the 128 x 128 form only");
   constexpr int BM = WT * 64, BN = WT * 64, BK = 64;
   constexpr int WROWS = WT * 32;                               // rows (columns) of a wave's tile
   constexpr int NPROD = WT * WT, NREAD = 2 * WT;               // per 16 of K
@@ -462,6 +463,88 @@ void gemm_bf16_block256_kernel(const bf16_t* __restrict__ A, const bf16_t* __res
     }
   };
 
+  if constexpr (DEEP) {
+    // Four LDS buffers, the block alone on its CU (128 KB): a 128 x 128 block's products of one
+    // tile take about 0.2 us, far less than a tile's way from memory, so with two buffers a
+    // block that has no neighbour on its CU waits for every tile (0.62 us each).  Here the loads
+    // of tile kt+3 are issued while tile kt is multiplied: three tiles are under way.
+    // Buffer of tile kt: kt % 4.  After the barrier of step kt-1 nobody reads tile kt-1's
+    // buffer any more, which is where tile kt+3 goes.
+    auto load_deep = [&](int kt, const char* base, int i) {
+      __builtin_amdgcn_global_load_lds(
+          KAPPAI_GPTR(base + roff[i]),
+          KAPPAI_LPTR(lds + (kt & 3) * BUF + (wave * NLOAD + i) * 8 * BK), 16, 0, 0);
+    };
+    auto read_deep = [&](int fb, const bf16_t* buf, int s, int idx) {
+      const bool is_w = idx == 0 || (idx >= 2 && idx <= WT);
+      const int n = idx <= 1 ? 0 : idx <= WT ? idx - 1 : idx - WT;
+      if (is_w)
+        fw[fb][n] = as_bf16x8(*reinterpret_cast<const u32x4_t*>(buf + woff[s] + n * 32 * BK));
+      else
+        fa[fb][n] = as_bf16x8(*reinterpret_cast<const u32x4_t*>(buf + aoff[s] + n * 32 * BK));
+    };
+    const int pre = min(nk, 3);
+    for (int p = 0; p < pre; ++p) {
+      const char* base = tile_base(p);
+#pragma unroll
+      for (int i = 0; i < NLOAD; ++i) load_deep(p, base, i);
+    }
+    // tile 0 has landed when only the loads of the tiles after it are outstanding
+    if (pre == 3)
+      __builtin_amdgcn_s_waitcnt(0x4F70);         // vmcnt(16)
+    else if (pre == 2)
+      __builtin_amdgcn_s_waitcnt(0x0F78);         // vmcnt(8)
+    else
+      __builtin_amdgcn_s_waitcnt(0x0F70);         // vmcnt(0)
+    __builtin_amdgcn_s_barrier();
+    SCHED_FENCE();
+#pragma unroll
+    for (int t = 0; t < NREAD; ++t) read_deep(0, lds, 0, t);
+    static_assert(NLOAD == 2 * NPROD, "one load a slot over the first two 16s of K");
+    for (int kt = 0; kt < nk; ++kt) {
+      const bf16_t* cur = lds + (kt & 3) * BUF;
+      const bf16_t* nxt = lds + ((kt + 1) & 3) * BUF;
+      const bool has1 = kt + 1 < nk, has2 = kt + 2 < nk, has3 = kt + 3 < nk;
+      const char* base3 = tile_base(kt + 3);
+#pragma unroll
+      for (int s = 0; s < 3; ++s) {
+#pragma unroll
+        for (int t = 0; t < NPROD; ++t) {
+          if (t < NREAD) read_deep((s + 1) & 1, cur, s + 1, t);
+          if (s < 2 && has3) load_deep(kt + 3, base3, s * NPROD + t);
+          product(s & 1, t);
+          SCHED_FENCE();
+        }
+      }
+      product(1, 0);
+      SCHED_FENCE();
+      if (has1) {
+        // tile kt+1 has landed when only the loads of tiles kt+2 and kt+3 are outstanding
+        if (has3)
+          __builtin_amdgcn_s_waitcnt(0x4F70);     // vmcnt(16)
+        else if (has2)
+          __builtin_amdgcn_s_waitcnt(0x0F78);     // vmcnt(8)
+        else
+          __builtin_amdgcn_s_waitcnt(0x0F70);     // vmcnt(0)
+        __builtin_amdgcn_s_barrier();
+      }
+      SCHED_FENCE();
+#pragma unroll
+      for (int t = 1; t < NPROD; ++t) {
+        if (has1) {
+          if (t == 1) {
+            read_deep(0, nxt, 0, 0);
+            read_deep(0, nxt, 0, 1);
+          } else if (t == 2) {
+            read_deep(0, nxt, 0, 2);
+            read_deep(0, nxt, 0, 3);
+          }
+        }
+        product(1, t);
+        SCHED_FENCE();
+      }
+    }
+  } else {
 #pragma unroll
   for (int i = 0; i < NLOAD; ++i) load_one(0, tile_base(0), i);
 #pragma unroll
@@ -478,6 +561,7 @@ void gemm_bf16_block256_kernel(const bf16_t* __restrict__ A, const bf16_t* __res
     const bool more = kt + 2 < nk;
     tile_step(IntC<0>{}, kt, true, more);
     tile_step(IntC<1>{}, kt + 1, more, more);
+  }
   }
 
   // Epilogue: a wave turns 32 rows of its tile at a time through its own piece of LDS.
@@ -544,13 +628,13 @@ static bool block256_fits(const bf16_t* A, const bf16_t* W, TO* C, int M, int n_
          (long long)M * lda < limit && (long long)n_rows_w * K < limit;
 }
 
-template <typename TO, int EPI, int WT>
+template <typename TO, int EPI, int WT, bool DEEP = false>
 static void launch_block256(const bf16_t* A, const bf16_t* W, const float* bias, TO* C, int M,
                             int n_rows_w, int K, int lda, int ldc, int ksplit,
                             hipStream_t stream) {
   constexpr int B = WT * 64;                     // block edge
-  constexpr size_t lds_bytes = 2 * (B + B) * 64 * sizeof(bf16_t);
-  auto kern = gemm_bf16_block256_kernel<TO, EPI, WT>;
+  constexpr size_t lds_bytes = (DEEP ? 4 : 2) * (B + B) * 64 * sizeof(bf16_t);
+  auto kern = gemm_bf16_block256_kernel<TO, EPI, WT, DEEP>;
   static bool attr_set = false;
   if (!attr_set) {
     (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -565,7 +649,8 @@ static void launch_block256(const bf16_t* A, const bf16_t* W, const float* bias,
 // shape: 0 = chosen by size, 1 = 128x128 blocks of two waves, 2 = 256x128 blocks (tiles of 32
 // of K, two LDS buffers), 3 = 256x128 blocks (tiles of 64 of K, one LDS buffer), 4 = 256x256
 // blocks of the same kernel (tiles of 64 of K), 5 = the 256x256 kernel with one wave a SIMD, 6 = its
-// 128x128 form (when the sizes fit them, else 3)
+// 128x128 form (when the sizes fit them, else 3), 8 = the 128x128 form with four LDS buffers, one
+// block a CU
 template <typename TO, int EPI>
 static void launch_tile(const bf16_t* A, const bf16_t* W, const float* bias, TO* C, int M,
                         int n_rows_w, int K, int lda, int ldc, int ksplit, int shape,
@@ -576,9 +661,13 @@ static void launch_tile(const bf16_t* A, const bf16_t* W, const float* bias, TO*
     const int blocks256 = ((M + 255) / 256) * ((n_rows_w + 255) / 256) * ksplit;
     // the one-wave-a-SIMD kernel when its 256 x 256 blocks fill most of the chip, its
     // 128 x 128 form (two blocks a CU) below that
-    shape = !fits ? (big >= 128 ? 3 : 1) : blocks256 >= 192 ? 5 : 6;
+    // 128 x 128 blocks that would each have a CU to themselves anyway, and a long K: the form
+    // with four LDS buffers (0.46 against 0.62-0.87 us per 64 of K; its start costs 2 us more)
+    const long blocks128 = (long)((M + 127) / 128) * ((n_rows_w + 127) / 128) * ksplit;
+    const bool deep = blocks128 <= 256 && K / ksplit >= 2048;
+    shape = !fits ? (big >= 128 ? 3 : 1) : blocks256 >= 192 ? 5 : deep ? 8 : 6;
   }
-  if ((shape == 5 || shape == 6) && !fits) shape = 3;
+  if ((shape == 5 || shape == 6 || shape == 8) && !fits) shape = 3;
   switch (shape) {
     case 5:
       if constexpr (EPI != 2)
@@ -587,6 +676,10 @@ static void launch_tile(const bf16_t* A, const bf16_t* W, const float* bias, TO*
     case 6:
       if constexpr (EPI != 2)
         launch_block256<TO, EPI, 2>(A, W, bias, C, M, n_rows_w, K, lda, ldc, ksplit, stream);
+      break;
+    case 8:
+      if constexpr (EPI != 2)
+        launch_block256<TO, EPI, 2, true>(A, W, bias, C, M, n_rows_w, K, lda, ldc, ksplit, stream);
       break;
     case 1:
       launch_tile_cfg<TO, EPI, 1, 2, 4, 2, 32, 2, 2>(A, W, bias, C, M, n_rows_w, K, lda, ldc, ksplit,
@@ -1195,7 +1288,7 @@ static int launch_bf16(const bf16_t* A, const bf16_t* W, const float* bias, TO* 
 // K, lda must be multiples of 8 and A, W 16-byte aligned (checked by the caller).
 // force_kernel: 0 = by M, 1 = tile kernel, 2 = skinny kernel (M <= 64 only), 3..8 = tile kernel
 // with block shape 1..6 (see launch_tile), 9 = shared-rows kernel (17 to 64 rows, K / ksplit a
-// multiple of 512); for tests and tuning.
+// multiple of 512), 10 = block shape 8; for tests and tuning.
 // ksplit > 1 (float output only): C is [ksplit][M][ldc] partial sums over K ranges.
 extern "C" int kappai_gemm_bf16(const void* A, const void* W, const float* bias, void* C, int M,
                                 int N, int K, int lda, int ldc, int out_is_f32, int force_kernel,

@@ -143,12 +143,13 @@ def test_linear_swiglu(ops, M, F, K):
 
 BLOCK256 = 7          # force_kernel: 256 x 256 blocks, one wave a SIMD
 BLOCK128 = 8          # the same kernel with 128 x 128 blocks
+BLOCK128_DEEP = 10    # 128 x 128 blocks with four LDS buffers (tiles 0-2 loaded ahead)
 
 
 @pytest.mark.parametrize("M,N,K", [(256, 256, 128), (300, 520, 256), (129, 8, 128), (1000, 1096, 384),
                                    (2048, 2048, 2048), (513, 264, 1280)])
 @pytest.mark.parametrize("out_dtype", [F32, BF16])
-@pytest.mark.parametrize("block", [BLOCK256, BLOCK128])
+@pytest.mark.parametrize("block", [BLOCK256, BLOCK128, BLOCK128_DEEP])
 def test_linear_block256(ops, M, N, K, out_dtype, block):
     """The large-product kernel at sizes that end inside its 256 x 256 blocks, with a row stride
     on the input, with bias, and against the other tiled kernel on the same data."""
@@ -166,7 +167,7 @@ def test_linear_block256(ops, M, N, K, out_dtype, block):
 
 
 @pytest.mark.parametrize("M,F,K", [(256, 128, 128), (300, 1008, 256), (2048, 1616, 384)])
-@pytest.mark.parametrize("block", [BLOCK256, BLOCK128])
+@pytest.mark.parametrize("block", [BLOCK256, BLOCK128, BLOCK128_DEEP])
 def test_linear_swiglu_block256(ops, M, F, K, block):
     x, wg, wu = rand((M, K), BF16, 44), rand((F, K), BF16, 45, 0.2), rand((F, K), BF16, 46, 0.2)
     w = ops.interleave_gate_up(wg.to(DEV), wu.to(DEV))
@@ -232,6 +233,20 @@ def test_linear_block256_split_k(ops):
     parts = ops.linear(x.to(DEV), w.to(DEV), partial_sums=True)
     assert parts.shape == (S, M, N) and parts.dtype == F32
     close(parts.sum(0), x.double() @ w.double().T, 2e-5, "sum of the partial sums")
+
+
+@pytest.mark.parametrize("M,N,K,S,block", [(575, 1024, 4608, 6, 0), (300, 520, 4096, 2, BLOCK128_DEEP),
+                                           (130, 264, 1280, 5, BLOCK128_DEEP),
+                                           (1100, 2048, 7168, 7, 0)])
+def test_linear_block_split_k_at_prompt_portion_sizes(ops, M, N, K, S, block):
+    """Products of a few hundred rows in K ranges of any length that is a multiple of 128 (2 to 16
+    tiles a range, odd counts of ranges), in both 128 x 128 forms."""
+    x, w, b = rand((M, K), BF16, 49), rand((N, K), BF16, 50, 0.05), rand((N,), F32, 51)
+    parts = ops.linear(x.to(DEV), w.to(DEV), b.to(DEV), partial_sums=True, split_k=S,
+                       force_kernel=block)
+    assert parts.shape == (S, M, N) and parts.dtype == F32
+    close(parts.sum(0), x.double() @ w.double().T + b.double(), 2e-5, "sum of the partial sums")
+    assert 1 <= ops.split_k_for(M, N, K) <= 8 and K % (128 * ops.split_k_for(M, N, K)) == 0
 
 
 @pytest.mark.parametrize("M,N,K", [(1, 2048, 2048), (8, 2048, 8192), (16, 96, 1024), (40, 1000, 4096),
