@@ -177,6 +177,13 @@ class Engine:
             self._t_first_add = time.perf_counter()
         return rid
 
+    def abort(self, request_id) -> bool:
+        """Stop a request between two steps: its pages and state slot go back to the pool and
+        its output so far stays readable in ``requests[request_id]``.  Returns False when the
+        id is unknown or the request had ended already."""
+        req = self.requests.get(request_id)
+        return req is not None and self.scheduler.abort(req)
+
     def has_unfinished(self) -> bool:
         return self.scheduler.has_unfinished()
 

@@ -242,3 +242,14 @@ class Scheduler:
         if request in self.running:
             self.running.remove(request)
         request.state, request.finish_reason = FINISHED, reason
+
+    def abort(self, request: Request, reason: str = "aborted") -> bool:
+        """Take a request out, whether it waits or runs (kappai's interrupt: src/context.c:
+        1438-1441; a session with fixed-size state cannot be taken up again afterwards, so
+        what it holds is simply given back).  Returns False if it had ended before."""
+        if request.state in (FINISHED, FAILED):
+            return False
+        if request in self.waiting:
+            self.waiting.remove(request)
+        self.finish(request, reason)
+        return True

@@ -129,6 +129,32 @@ def test_preemption_gives_the_same_tokens(model_dirs):
         too_long.generate([list(range(40))], params)
 
 
+def test_abort_leaves_the_others_alone(model_dirs):
+    """One of three requests is aborted after a few steps (inside its decoding, while decode
+    graphs and queued decode runs are in use): the others end with the tokens they have without
+    it, its pages and slot are back, and a request added afterwards runs in what it freed."""
+    from kappai_amd.engine import Engine
+    from kappai_amd.sampling import SamplingParams
+    prompts = prompts_for("B", [9, 21, 14], seed=6)
+    params = SamplingParams.greedy(n_predict=24)
+    alone = Engine(str(model_dirs["B"]), dtype="float32", num_pages=32, max_batch=3)
+    want = alone.generate([prompts[0], prompts[2]], params)
+    eng = Engine(str(model_dirs["B"]), dtype="float32", num_pages=32, max_batch=3)
+    ids = [eng.add_request(p, params) for p in prompts]
+    for _ in range(3):
+        eng.step()
+    victim = eng.requests[ids[1]]
+    assert 0 < len(victim.output) < 24
+    assert eng.abort(ids[1]) and not eng.abort(ids[1]) and not eng.abort("no such request")
+    assert victim.finish_reason == "aborted" and eng.cache.num_free_slots == 1
+    late = eng.add_request(prompts[1], params)
+    while eng.has_unfinished():
+        eng.step()
+    assert [eng.requests[ids[0]].output, eng.requests[ids[2]].output] == want
+    assert len(eng.requests[late].output) == 24
+    assert eng.cache.num_free_pages() == 32 and eng.cache.num_free_slots == 3
+
+
 def test_command_line(model_dirs, tmp_path):
     prompt = prompts_for("A", [7], seed=5)[0]
     want, _ = plain_generate(model_dirs["A"], prompt, 6, lambda: S.PlainSampler(1, temperature=0.0))

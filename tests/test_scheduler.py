@@ -135,6 +135,28 @@ def test_preemption_when_pages_run_out():
     assert cm.num_free_pages() == 3 and cm.num_free_slots == 8
 
 
+def test_abort_gives_everything_back_and_lets_the_next_in():
+    """A request is taken out while it runs, another while it waits: pages and slot of the
+    first go back at once, the one behind them is admitted in the next step, and a second
+    abort of the same request changes nothing."""
+    cm, sch = make(pages=8, slots=1, page_size=4, token_budget=8, chunk=8)
+    a, b, c = req("a", 6), req("b", 5), req("c", 4)
+    for r in (a, b, c):
+        sch.add(r)
+    run_step(cm, sch)
+    assert a.state == RUNNING and b.state == WAITING
+    free_before = cm.paged_groups[0].allocator.num_free
+    assert sch.abort(a) and a.state == FINISHED and a.finish_reason == "aborted"
+    assert a.cache is None and cm.num_free_slots == 1
+    assert cm.paged_groups[0].allocator.num_free > free_before
+    assert sch.abort(b) and b not in sch.waiting
+    assert not sch.abort(a) and not sch.abort(b)
+    cm.check()
+    entries, failed, _ = run_step(cm, sch)
+    assert [e.request.request_id for e in entries] == ["c"] and not failed
+    assert sch.has_unfinished()
+
+
 def test_a_request_that_cannot_fit_alone_fails():
     cm, sch = make(pages=2, token_budget=64)
     sch.add(req("big", 9))              # 3 pages needed, the pool has 2: over max_context
