@@ -202,6 +202,25 @@ class DecodeBench:
             self.cache.close(rc)
 
 
+def measured_read_bandwidth(device, mb=256, buffers=5, reps=20):
+    """GB/s of a kernel that only reads: buffers of ``mb`` MB taken in turn (more than the
+    memory-side cache holds), ``reps`` reads between two synchronisations."""
+    import torch
+
+    from kappai_amd.kernels import ops
+    bufs = [torch.empty(mb * 1000 * 1000 // 4, dtype=torch.int32, device=device).random_()
+            for _ in range(buffers)]
+    for b in bufs:
+        ops.stream_read(b)
+    sync()
+    t0 = time.perf_counter()
+    total = 0
+    for i in range(reps):
+        total += ops.stream_read(bufs[i % buffers])
+    sync()
+    return total / (time.perf_counter() - t0) / 1e9
+
+
 def prefill_flops(cfg, n_tokens, n_layers_run):
     """Multiply-adds x 2 of a whole prompt of ``n_tokens``: every projection, attention over
     the causal half, and the head for the last row."""
@@ -290,6 +309,8 @@ def main() -> int:
             dtb, _ = decode(b)
             points[f"decode_b{b}"] = round(b * K / dtb, 1)
 
+    read_gbs = measured_read_bandwidth(device)
+
     # prefill of one prompt, whole, logits at its last token
     T = args.prefill_tokens
     cm = CacheManager(model.cache_specs(), args.page_size, (T + args.page_size - 1) // args.page_size + 1, 1)
@@ -328,7 +349,10 @@ def main() -> int:
         "prefill": {"value": round(T / pre_s, 1), "tokens": T, "ms": round(pre_s * 1e3, 3),
                     "frac": round(flops / pre_s / peak, 5)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 5)},
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 5),
+                     # what a kernel that only reads gets on this box, and the step against that
+                     "measured_read": round(read_gbs, 1),
+                     "frac_of_measured_read": round(achieved / read_gbs, 5)},
         "points": points,
     }
     print(json.dumps(out))

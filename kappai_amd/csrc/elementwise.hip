@@ -224,3 +224,39 @@ extern "C" int kappai_cast(const void* in, void* out, long n, int in_is_bf16, in
     return (int)hipErrorInvalidValue;
   KAPPAI_RETURN_LAUNCH_STATUS();
 }
+
+// ---------------------------------------------------------------------------------------
+// a plain read of a buffer: what the memory delivers to a kernel that does nothing else
+// (the yardstick beside the published peak for the kernels that stream weights and cache)
+// ---------------------------------------------------------------------------------------
+typedef uint32_t stream_u32x4_t __attribute__((ext_vector_type(4)));
+__global__ __launch_bounds__(256) void stream_read_kernel(const stream_u32x4_t* __restrict__ p,
+                                                          size_t n_per_block,
+                                                          uint32_t* __restrict__ sink) {
+  // every block reads its own contiguous range, 8 loads of 16 bytes a lane in flight
+  const stream_u32x4_t* b = p + n_per_block * blockIdx.x;
+  stream_u32x4_t acc = {0u, 0u, 0u, 0u};
+  for (size_t i = threadIdx.x; i + 7 * 256 < n_per_block; i += 8 * 256) {
+    stream_u32x4_t v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) v[u] = b[i + u * 256];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) acc ^= v[u];
+  }
+  // never true for data the host made, but the compiler cannot know: the loads stay
+  if ((acc.x ^ acc.y ^ acc.z ^ acc.w) == 0x9e3779b9u && sink != nullptr) sink[0] = acc.x;
+}
+
+// Reads the first `bytes` of `p` (rounded down to what 512 blocks share evenly in pieces of
+// 32 KB) once.  Returns the bytes read through *bytes_read.
+extern "C" int kappai_stream_read(const void* p, long bytes, uint32_t* sink, long* bytes_read,
+                                  hipStream_t stream) {
+  const int blocks = 512;
+  const size_t piece = 8 * 256;                                  // 16-byte elements a block and turn
+  const size_t n_per_block = ((size_t)bytes / 16 / blocks / piece) * piece;
+  if (bytes_read) *bytes_read = (long)(n_per_block * blocks * 16);
+  if (n_per_block == 0 || ((uintptr_t)p % 16)) return (int)hipErrorInvalidValue;
+  hipLaunchKernelGGL(stream_read_kernel, dim3(blocks), dim3(256), 0, stream,
+                     (const stream_u32x4_t*)p, n_per_block, sink);
+  KAPPAI_RETURN_LAUNCH_STATUS();
+}

@@ -173,6 +173,17 @@ def add_residual(resid: torch.Tensor, delta: torch.Tensor) -> None:
         _stream()), "add_residual")
 
 
+def stream_read(buf: torch.Tensor) -> int:
+    """Launches one plain read of ``buf`` (a kernel that only loads) and returns the bytes it
+    reads: the yardstick for the kernels that stream weights and cache."""
+    _gpu("buf", buf)
+    n = ctypes.c_long(0)
+    check(library("elementwise").kappai_stream_read(
+        _ptr(buf), _c_long(buf.numel() * buf.element_size()), _vp(0), ctypes.byref(n),
+        _stream()), "stream_read")
+    return n.value
+
+
 def swiglu(gate_up: torch.Tensor) -> torch.Tensor:
     """``silu(gate_up[:, :F]) * gate_up[:, F:]`` for a fused [T, 2F] projection."""
     _gpu("gate_up", gate_up, (F32, BF16))

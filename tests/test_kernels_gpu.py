@@ -47,6 +47,18 @@ def test_embed_rows(ops, dtype):
     assert torch.equal(got.cpu(), table[ids.long()].float())
 
 
+def test_stream_read_stays_inside_the_buffer(ops):
+    """The read-only yardstick kernel reads whole pieces of 32 KB for each of its 512 blocks and
+    never more than the buffer holds; a buffer too small for one piece a block is refused."""
+    for n_bytes in (16 << 20, (16 << 20) + 12345 * 16, 100 * 1000 * 1000):
+        buf = torch.zeros(n_bytes // 4, dtype=torch.int32, device=DEV)
+        got = ops.stream_read(buf)
+        assert 0 < got <= n_bytes and got % (512 * 32768) == 0 and n_bytes - got < 512 * 32768
+    torch.cuda.synchronize()
+    with pytest.raises(RuntimeError):
+        ops.stream_read(torch.zeros(1000, dtype=torch.int32, device=DEV))
+
+
 @pytest.mark.parametrize("dtype", [F32, BF16])
 @pytest.mark.parametrize("D", [64, 96, 1000, 2048, 5000])
 def test_add_rmsnorm(ops, dtype, D):
