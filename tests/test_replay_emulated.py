@@ -16,13 +16,16 @@ from kappai_amd.models import load_model
 FP32_TOL = 2e-5       # of the largest |logit|; float32 arithmetic against float64
 
 LENGTHS = {"A": [70, 45, 100, 37, 83, 64], "B": [33, 97, 40, 71, 52], "C": [66, 35, 90, 41],
-           "D": [50, 81, 36], "E": [45, 70, 33], "F": [66, 40, 85]}
+           "D": [50, 81, 36], "E": [45, 70, 33], "F": [66, 40, 85], "G": [70, 38, 51],
+           "H": [40, 77, 35]}
 MIXED_LENGTHS = {"A": [70, 45, 100, 37, 83, 64, 29, 58, 91, 40],
                  "B": [33, 97, 40, 71, 52, 64, 18, 85, 47],
                  "C": [66, 35, 90, 41, 23, 77, 50, 62],
                  "D": [50, 81, 36, 67, 44, 72, 90, 33, 58, 41],
                  "E": [45, 70, 33, 52, 61, 38, 88, 27, 95, 40],
-                 "F": [66, 40, 85, 37, 58, 49, 92, 31, 74, 43]}
+                 "F": [66, 40, 85, 37, 58, 49, 92, 31, 74, 43],
+                 "G": [70, 38, 51, 64, 33, 88, 45, 59, 36, 72],
+                 "H": [40, 77, 35, 66, 52, 90, 31, 48, 83, 44]}
 
 
 @pytest.fixture(scope="module")
@@ -50,7 +53,7 @@ def run_emulated(monkeypatch, model_dir, dtype, steps, index, max_tokens, tmp_pa
 
 @pytest.mark.parametrize("name,family", [(n, f) for n in "ABC" for f in
                                          ("whole", "prefill_then_decode", "changing_portions", "mixed")]
-                         + [(n, "mixed") for n in "DEF"])
+                         + [(n, "mixed") for n in "DEFGH"])
 def test_schedules_float32(monkeypatch, tmp_path, model_dirs, name, family):
     cfg = TINY[name][0]
     lengths = MIXED_LENGTHS[name] if family == "mixed" else LENGTHS[name]

@@ -27,13 +27,16 @@ FP32_TOL = 2e-5     # of the largest |logit|
 BF16_FACTOR = 2.5
 
 LENGTHS = {"A": [70, 45, 100, 37, 83, 64], "B": [33, 97, 40, 71, 52], "C": [66, 35, 90, 41],
-           "D": [50, 81, 36], "E": [45, 70, 33], "F": [66, 40, 85]}
+           "D": [50, 81, 36], "E": [45, 70, 33], "F": [66, 40, 85], "G": [70, 38, 51],
+           "H": [40, 77, 35]}
 MIXED_LENGTHS = {"A": [70, 45, 100, 37, 83, 64, 29, 58, 91, 40],
                  "B": [33, 97, 40, 71, 52, 64, 18, 85, 47],
                  "C": [66, 35, 90, 41, 23, 77, 50, 62],
                  "D": [50, 81, 36, 67, 44, 72, 90, 33, 58, 41],
                  "E": [45, 70, 33, 52, 61, 38, 88, 27, 95, 40],
-                 "F": [66, 40, 85, 37, 58, 49, 92, 31, 74, 43]}
+                 "F": [66, 40, 85, 37, 58, 49, 92, 31, 74, 43],
+                 "G": [70, 38, 51, 64, 33, 88, 45, 59, 36, 72],
+                 "H": [40, 77, 35, 66, 52, 90, 31, 48, 83, 44]}
 
 
 @pytest.fixture(scope="module")
@@ -81,7 +84,7 @@ def tolerance(model_dir, requests, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C", "D", "E", "F"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D", "E", "F", "G", "H"])
 @pytest.mark.parametrize("family", ["whole", "prefill_then_decode", "changing_portions", "mixed"])
 def test_schedules(tmp_path, model_dirs, name, family, dtype):
     cfg = TINY[name][0]
@@ -191,11 +194,22 @@ WIDE = {
 }
 
 
+# The same with heads of 128 and eight query heads for every kv head (two groups of four in the
+# kernel that shares key tiles; 64 keys a wave and turn in the decode kernel), a head width
+# (2048) that is not the model's, and a vocabulary that is no power of two.
+WIDE_HEADS = dict(WIDE, hidden_size=512, num_hidden_layers=2,
+                  layer_types=["conv", "full_attention"], num_attention_heads=16,
+                  num_key_value_heads=2, head_dim=128, intermediate_size=1024, vocab_size=1000,
+                  rope_theta=10000.0)
+
+
+@pytest.mark.parametrize("shape", ["wide", "wide_heads"])
 @pytest.mark.parametrize("dtype", ["bfloat16", "float32"])
-def test_long_prompt_on_a_wide_model(tmp_path, dtype):
+def test_long_prompt_on_a_wide_model(tmp_path, dtype, shape):
     import copy
     from kappai_amd.config import config_from_dict
     from kappai_amd.weights import write_random_model
+    WIDE = globals()["WIDE" if shape == "wide" else "WIDE_HEADS"]
     folder = write_random_model(tmp_path / "wide", config_from_dict(copy.deepcopy(WIDE)), seed=5,
                                 std=0.02, norm_jitter=0.05)
     requests = make_requests(WIDE["vocab_size"], [2200, 300], seed=15)

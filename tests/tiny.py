@@ -87,8 +87,34 @@ TINY_F = {
 }
 INIT_F = dict(seed=5, std=0.05, norm_jitter=0.1)
 
+# eighteen query heads on one kv head (more than the 16 columns of the matrix-core decode
+# kernel: the other attention kernels run), attention first, a vocabulary that is a prime
+TINY_G = {
+    "architectures": ["Lfm2ForCausalLM"], "model_type": "lfm2",
+    "hidden_size": 72, "num_hidden_layers": 2, "layer_types": ["full_attention", "conv"],
+    "num_attention_heads": 18, "num_key_value_heads": 1, "head_dim": 16,
+    "intermediate_size": 96, "block_auto_adjust_ff_dim": False,
+    "vocab_size": 257, "norm_eps": 1e-6, "rope_theta": 50000.0,
+    "conv_L_cache": 2, "conv_bias": False, "tie_embedding": True,
+    "max_position_embeddings": 1024,
+}
+INIT_G = dict(seed=6, std=0.05, norm_jitter=0.1)
+
+# heads of 256, the largest size of the matrix-core attention kernels
+TINY_H = {
+    "architectures": ["Lfm2ForCausalLM"], "model_type": "lfm2",
+    "hidden_size": 64, "num_hidden_layers": 2, "layer_types": ["conv", "full_attention"],
+    "num_attention_heads": 2, "num_key_value_heads": 2, "head_dim": 256,
+    "intermediate_size": 128, "block_auto_adjust_ff_dim": False,
+    "vocab_size": 128, "norm_eps": 1e-5, "rope_theta": 10000.0,
+    "conv_L_cache": 3, "conv_bias": False, "tie_embedding": False,
+    "max_position_embeddings": 1024,
+}
+INIT_H = dict(seed=7, std=0.05, norm_jitter=0.1)
+
 TINY = {"A": (TINY_A, INIT_A), "B": (TINY_B, INIT_B), "C": (TINY_C, INIT_C),
-        "D": (TINY_D, INIT_D), "E": (TINY_E, INIT_E), "F": (TINY_F, INIT_F)}
+        "D": (TINY_D, INIT_D), "E": (TINY_E, INIT_E), "F": (TINY_F, INIT_F),
+        "G": (TINY_G, INIT_G), "H": (TINY_H, INIT_H)}
 
 
 def tiny_config(name: str) -> dict:
