@@ -155,6 +155,43 @@ def test_abort_leaves_the_others_alone(model_dirs):
     assert eng.cache.num_free_pages() == 32 and eng.cache.num_free_slots == 3
 
 
+def test_random_engine_options_give_the_same_tokens(model_dirs):
+    """Thirty random combinations of page size, pool size (down to what the longest request
+    needs plus a page), live requests, token budget, longest portion and queued decode steps,
+    with greedy and seeded sampled requests: in float32 the tokens are those of a roomy engine
+    that takes every step by itself, and every page and slot comes back."""
+    import random
+    from kappai_amd.engine import Engine
+    from kappai_amd.sampling import SamplingParams
+    rng = random.Random(7)
+    for trial in range(30):
+        name = rng.choice(["A", "B", "G", "H"])
+        vocab = TINY[name][0]["vocab_size"]
+        n_req = rng.randint(1, 7)
+        prompts = [[rng.randrange(vocab) for _ in range(rng.randint(1, 60))] for _ in range(n_req)]
+        params = [SamplingParams.greedy(n_predict=rng.randint(1, 30)) if rng.random() < 0.6 else
+                  SamplingParams(temperature=0.8, top_k=rng.choice([0, 5, 40]),
+                                 top_p=rng.choice([1.0, 0.9]), min_p=rng.choice([0.0, 0.1]),
+                                 seed=rng.randint(1, 99), n_predict=rng.randint(1, 30))
+                  for _ in range(n_req)]
+        page = rng.choice([4, 16, 16, 32, 48, 64])
+        longest = max(len(p) + sp.n_predict for p, sp in zip(prompts, params))
+        least = (longest + page - 1) // page + 1
+        options = dict(page_size=page, num_pages=rng.choice([least, least + 2, 4 * least, 64]),
+                       max_batch=rng.choice([1, 2, 3, 8]),
+                       token_budget=rng.choice([1, 3, 17, 64, 2048]),
+                       chunk=rng.choice([1, 2, 5, 33, 2048]), decode_run=rng.choice([1, 2, 8]),
+                       warm_kernels=rng.random() < 0.5)
+        roomy = Engine(str(model_dirs[name]), dtype="float32", num_pages=256, page_size=16,
+                       max_batch=8, decode_run=1, warm_kernels=False)
+        want = roomy.generate(prompts, params)
+        eng = Engine(str(model_dirs[name]), dtype="float32", **options)
+        got = eng.generate(prompts, params)
+        assert got == want, (trial, name, options, [len(p) for p in prompts])
+        assert eng.cache.num_free_slots == options["max_batch"]
+        assert eng.cache.num_free_pages() == options["num_pages"]
+
+
 def test_command_line(model_dirs, tmp_path):
     prompt = prompts_for("A", [7], seed=5)[0]
     want, _ = plain_generate(model_dirs["A"], prompt, 6, lambda: S.PlainSampler(1, temperature=0.0))
