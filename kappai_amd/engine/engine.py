@@ -9,7 +9,7 @@ token ids and many requests at once.
 from __future__ import annotations
 
 import time
-from dataclasses import dataclass, field
+from dataclasses import dataclass
 from typing import Dict, List, Optional, Sequence, Union
 
 import torch
@@ -18,7 +18,7 @@ from ..cache.manager import CacheManager
 from ..models import Model, load_model
 from ..sampling import RequestSampler, Sampler, SamplingParams
 from .batch import StepEntry
-from .scheduler import FAILED, FINISHED, RUNNING, Request, Scheduler, SchedulerConfig
+from .scheduler import FAILED, RUNNING, Request, Scheduler, SchedulerConfig
 from .step import StepRunner
 
 

@@ -5,8 +5,6 @@ Every function has the contract of the kernel it stands for, including the dtype
 results are stored."""
 from __future__ import annotations
 
-import math
-
 import numpy as np
 import torch
 

@@ -1,8 +1,6 @@
 """Plain host sampler after src/sampler.c of System64fumo/kappai, one token at a time."""
 from __future__ import annotations
 
-import math
-
 import numpy as np
 
 MASK = (1 << 64) - 1

@@ -2,7 +2,6 @@
 them, and the comparison of a replay's output with those."""
 from __future__ import annotations
 
-import functools
 import json
 from pathlib import Path
 

@@ -2,10 +2,7 @@
 plain implementation's function for it; and a toy mixer with state of its own, defined
 here, registered, built into a toy architecture and stepped without a change to the
 framework's files."""
-import copy
-import math
 from dataclasses import dataclass
-from typing import Dict, List
 
 import numpy as np
 import pytest

@@ -2,17 +2,15 @@
 vectors, special cases that reduce to a library routine, and invariants, each chosen so
 that a plausible mistake (a wrong sign or pairing, a norm in the wrong place, a tap order)
 fails it."""
-import copy
 import math
 
 import numpy as np
-import pytest
 import scipy.signal
 import scipy.special
 
 from plain import lfm2 as P
 from plain import sampler as S
-from tiny import TINY_A, TINY_B, write_tiny
+from tiny import write_tiny
 
 RNG = np.random.default_rng(0)
 

@@ -1,9 +1,7 @@
 """The engine's own logic (row tables, cache manager, step function, replay) against the
 plain implementation, with the kernels replaced by torch CPU stand-ins.  No GPU needed.
 The same schedules run on the GPU in test_replay_gpu.py."""
-import numpy as np
 import pytest
-import torch
 
 import emulated_ops
 import schedules

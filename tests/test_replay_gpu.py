@@ -3,14 +3,12 @@ most of it in one step and the last 32 tokens one by one; in portions of changin
 and mixed, up to four live requests with so few pages that they are used again; in true
 32-bit and in bfloat16."""
 import json
-import os
 import subprocess
 import sys
 from pathlib import Path
 
 import numpy as np
 import pytest
-import torch
 
 import schedules
 from plain import lfm2 as plain

@@ -1,6 +1,5 @@
 """Weights: the container, loading by name, the one error that lists everything wrong, and
 the random-weights mode."""
-import copy
 import json
 import struct
 
@@ -8,12 +7,10 @@ import numpy as np
 import pytest
 import torch
 
-from kappai_amd.config import config_from_dict
-from kappai_amd.models import build_model, load_model
-from kappai_amd.weights import (SafetensorsError, SafetensorsFile, WeightsError, check_and_load,
-                                write_random_model, write_safetensors)
+from kappai_amd.models import load_model
+from kappai_amd.weights import SafetensorsError, SafetensorsFile, WeightsError, write_safetensors
 from plain import lfm2 as plain
-from tiny import TINY_A, TINY_B, write_tiny
+from tiny import write_tiny
 
 
 def test_container_round_trip(tmp_path):
