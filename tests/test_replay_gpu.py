@@ -333,6 +333,60 @@ def test_layer_sizes_of_the_1_2b_model(tmp_path, sizes_1_2b_dir, dtype):
     _models.pop((str(folder), dtype), None)        # 0.7 to 1.3 GB on the GPU
 
 
+# A pool of more than 2^31 elements (8.7 GB of bfloat16 keys and as much of values in the one
+# attention layer): the request's pages are the last of the pool, so every address of the
+# store, prefill and decode kernels that does not fit 32 bits is used.
+BIG_POOL = {
+    "architectures": ["Lfm2ForCausalLM"], "model_type": "lfm2",
+    "hidden_size": 128, "num_hidden_layers": 2, "layer_types": ["full_attention", "conv"],
+    "num_attention_heads": 8, "num_key_value_heads": 8, "head_dim": 64,
+    "intermediate_size": 256, "block_auto_adjust_ff_dim": False,
+    "vocab_size": 300, "norm_eps": 1e-5, "rope_theta": 10000.0,
+    "conv_L_cache": 3, "conv_bias": False, "tie_embedding": True,
+    "max_position_embeddings": 1024,
+}
+
+
+@pytest.mark.parametrize("dtype", ["bfloat16"])
+def test_pages_beyond_two_giga_elements(tmp_path, dtype):
+    import copy
+    from kappai_amd.cache import CacheManager
+    from kappai_amd.config import config_from_dict
+    from kappai_amd.engine.replay import TraceReplayer
+    from kappai_amd.engine.step import StepRunner
+    from kappai_amd.models import load_model
+    from kappai_amd.weights import write_random_model
+    folder = write_random_model(tmp_path / "m", config_from_dict(copy.deepcopy(BIG_POOL)), seed=9,
+                                std=0.05, norm_jitter=0.05)
+    model = load_model(folder, dtype, "cuda:0")
+    page = 16
+    per_page = 8 * page * 64
+    pages = 2 * (2 ** 31 // per_page) + 40               # 4.3 G elements a pool
+    cache = CacheManager(model.cache_specs(), page, pages, 4)
+    cache.allocate_storage(model.dtype, "cuda:0")
+    filler = cache.open("filler")                        # holds all pages but the last 24
+    cache.extend(filler, (pages - 24) * page)
+    requests = make_requests(BIG_POOL["vocab_size"], [150, 60], seed=19)
+    plans = {"r0": (0, [100, 18] + [1] * 32), "r1": (1, [33, 27])}
+    steps, index, peak = schedules.build(requests, plans)
+    rep = TraceReplayer(StepRunner(model, cache, "cuda:0"), tmp_path / "out")
+    outputs = {}
+    for obj in steps:
+        live = list(rep.live.values())
+        res = rep.run_step(obj)
+        assert all(min(b) >= pages - 24 for rc in live for b in rc.blocks if b)
+        if res is not None:
+            outputs[obj["step"]] = res
+    cache.close(filler)
+    cache.check()
+    got = collect(index, outputs, model.vocab_size)
+    ref = plain_logits(folder, requests)
+    tol = tolerance(folder, requests, dtype)
+    err, where = worst_error(got, ref)
+    assert err < tol, (err, tol, where, first_bad(got, ref, tol))
+    del rep, cache, model
+
+
 def test_trace_semantics(tmp_path, model_dirs):
     """What a trace may do beside the regular schedules: places asked for out of order and
     twice, a request that is left out of steps and goes on later, a step that wants nothing
