@@ -331,7 +331,7 @@ def main() -> int:
     peak = MFMA_PEAK_TFLOPS[args.dtype] * 1e12
 
     out = {
-        "metric": "decode tok/s at batch 8 (LFM2-1.2B shape, context 4096)",
+        "metric": f"decode tok/s at batch {args.batch} (LFM2-1.2B shape, context {args.context})",
         "value": round(value, 1), "unit": "tok/s", "n_gpus": 1, "steps": K, "warmup": W,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",

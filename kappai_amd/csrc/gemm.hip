@@ -750,22 +750,28 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny_kernel(
   static_assert(NT == 1 || EPI == 0, "several column tiles a wave: plain products only");
   static_assert(!PRO || (MT == 1 && NT == 1), "normalised rows: one row tile");
   // row groups of W a block streams: gate/up, the three conv gates, or NT column tiles
-  constexpr int NG = EPI == 1 ? 2 : (EPI == 2 ? 3 : NT);
+  constexpr int NG = EPI == 1 ? 2 : (EPI == 2 ? 3 : (EPI == 3 ? 2 : NT));
   __shared__ float red[NW][NG * MT][WAVE][4];
   const int tid = threadIdx.x;
   const int lane = tid % WAVE, wave = tid / WAVE;
-  const int n0 = blockIdx.x * 16 * NT;
+  const int n0 = blockIdx.x * (EPI == 3 ? 8 : 16 * NT);
   const int col = lane % 16, kg = (lane / 16) * 8;
-  const int gn = n0 + col;
+  // EPI 3: columns 0-7 and 8-15 are the same 8 channels (of two different gates)
+  const int gn = n0 + (EPI == 3 ? col % 8 : col);
   const u32x4_t zero = {0u, 0u, 0u, 0u};
   f32x4_t acc[NG * MT];
 #pragma unroll
   for (int t = 0; t < NG * MT; ++t) acc[t] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
   // plain: row gn (and 16 further for the next column tile).  SwiGLU: gate row 32*block + col, up
   // row 16 further.  Conv: rows gn, N + gn, 2N + gn.
-  const size_t wr0 = EPI == 1 ? (size_t)blockIdx.x * 32 + col : (size_t)gn;
-  const size_t group_rows = EPI == 2 ? (size_t)N : 16;
+  // EPI 3 (the conv step with 8 channels a block, twice as many blocks for narrow models): row
+  // group 0 is the B gate's rows in columns 0-7 and the C gate's in columns 8-15, row group 1 the
+  // x gate's rows in columns 0-7 (columns 8-15 stay zero).
+  const size_t wr0 = EPI == 1 ? (size_t)blockIdx.x * 32 + col
+                              : (EPI == 3 && col >= 8 ? (size_t)N + gn : (size_t)gn);
+  const size_t group_rows = EPI == 2 ? (size_t)N : (EPI == 3 ? 2 * (size_t)N : 16);
   const bf16_t* wrow = W + (gn < N ? wr0 : 0) * K + kg;
+  auto group_ok = [&](int r) { return EPI == 3 ? (r == 0 || col < 8) : true; };
   const bf16_t* arow[MT];
 #pragma unroll
   for (int t = 0; t < MT; ++t) {
@@ -833,8 +839,9 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny_kernel(
       const bool kin = gk + kg < k1;
 #pragma unroll
       for (int r = 0; r < NG; ++r)
-        wv[u][r] = (kin && gn + (EPI == 0 ? r * 16 : 0) < N) ? load16(wrow + r * group_rows * K + gk)
-                                                               : zero;
+        wv[u][r] = (kin && gn + (EPI == 0 ? r * 16 : 0) < N && group_ok(r))
+                       ? load16(wrow + r * group_rows * K + gk)
+                       : zero;
     }
   };
   auto load_a = [&](int k, u32x4_t (&av)[U][MT]) {
@@ -882,7 +889,7 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny_kernel(
         const bool kin = gk + kg < k1;
 #pragma unroll
         for (int r = 0; r < NG; ++r)
-          wv[u][r] = (kin && gn + (EPI == 0 ? r * 16 : 0) < N)
+          wv[u][r] = (kin && gn + (EPI == 0 ? r * 16 : 0) < N && group_ok(r))
                          ? load16(wrow + r * group_rows * K + gk)
                          : zero;
 #pragma unroll
@@ -915,7 +922,7 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny_kernel(
         store_out(C + (size_t)gm * ldc + gnr, sum + bv);
       }
     }
-  } else if (wave < MT && gn < N) {
+  } else if (wave < MT && gn < N && (EPI != 3 || col < 8)) {
     const int t = wave;
     const float bv = (bias && blockIdx.y == 0) ? bias[gn] : 0.f;
 #pragma unroll
@@ -930,12 +937,16 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny_kernel(
 #pragma unroll
           for (int w = 1; w < NW; ++w) up += red[w][MT + t][lane][v];
           store_out(C + (size_t)gm * ldc + gn, silu_f(sum) * up);
-        } else if (EPI == 2) {
-          float cg = red[0][MT + t][lane][v], xg = red[0][2 * MT + t][lane][v];
+        } else if (EPI == 2 || EPI == 3) {
+          // where the other two gates of this channel lie: EPI 2 in row groups 1 and 2 of this
+          // lane, EPI 3 the C gate 8 columns further in group 0 and the x gate in group 1
+          const int cg_t = EPI == 2 ? MT + t : t, cg_lane = EPI == 2 ? lane : lane + 8;
+          const int xg_t = EPI == 2 ? 2 * MT + t : MT + t;
+          float cg = red[0][cg_t][cg_lane][v], xg = red[0][xg_t][lane][v];
 #pragma unroll
           for (int w = 1; w < NW; ++w) {
-            cg += red[w][MT + t][lane][v];
-            xg += red[w][2 * MT + t][lane][v];
+            cg += red[w][cg_t][cg_lane][v];
+            xg += red[w][xg_t][lane][v];
           }
           float bg = sum;
           if (bias) {
@@ -971,8 +982,8 @@ template <typename TO, int MT, int NW, int EPI, int NT = 1>
 static void launch_skinny(const bf16_t* A, const bf16_t* W, const float* bias, TO* C, int M, int N,
                           int K, int lda, int ldc, int ksplit, ConvStep cs, hipStream_t stream,
                           const NormIn* nin = nullptr) {
-  const dim3 grid((N + 16 * NT - 1) / (16 * NT), ksplit);
-  if constexpr (MT == 1 && NT == 1 && EPI != 2) {
+  const dim3 grid(EPI == 3 ? (N + 7) / 8 : (N + 16 * NT - 1) / (16 * NT), ksplit);
+  if constexpr (MT == 1 && NT == 1 && EPI != 2 && EPI != 3) {
     if (nin) {
       hipLaunchKernelGGL((gemm_bf16_skinny_kernel<TO, MT, NW, EPI, NT, true>), grid,
                          dim3(NW * WAVE), 0, stream, A, W, bias, C, M, N, K, lda, ldc, cs, *nin);
@@ -1004,9 +1015,9 @@ static void launch_skinny_mt(const bf16_t* A, const bf16_t* W, const float* bias
       return;
     }
   }
-  const int blocks = ((N + 15) / 16) * ksplit;
+  const int blocks = (EPI == 3 ? (N + 7) / 8 : (N + 15) / 16) * ksplit;
   const int kb = K / ksplit;                              // K a block
-  constexpr int NG = EPI == 1 ? 2 : (EPI == 2 ? 3 : 1);
+  constexpr int NG = EPI == 1 ? 2 : (EPI == 2 ? 3 : (EPI == 3 ? 2 : 1));
   constexpr int MAXW = 48 / (MT * NG);                    // 1 KB of LDS a wave, group and row tile
   if (blocks * 4 >= 2048 || kb <= 512 || MAXW < 8)
     launch_skinny<TO, MT, 4, EPI>(A, W, bias, C, M, N, K, lda, ldc, ksplit, cs, stream, nin);
@@ -1325,6 +1336,19 @@ extern "C" int kappai_gemm_bf16_shortconv_step(const void* A, const void* W, con
   if (M <= 0 || D <= 0) return 0;
   if ((K % 8) || (lda % 8) || (D % 16) || M > 64 || L < 2) return (int)hipErrorInvalidValue;
   ConvStep cs{taps, conv_bias, state, seg_pos0, seg_slot, L};
+  if (D / 16 < 256) {
+    // too few blocks of 16 channels for the chip: 8 channels a block
+    const bf16_t* a = (const bf16_t*)A;
+    const bf16_t* w = (const bf16_t*)W;
+    bf16_t* c = (bf16_t*)C;
+    switch ((M + 15) / 16) {
+      case 1: launch_skinny_mt<bf16_t, 1, 3>(a, w, bias, c, M, D, K, lda, D, 1, cs, stream); break;
+      case 2: launch_skinny_mt<bf16_t, 2, 3>(a, w, bias, c, M, D, K, lda, D, 1, cs, stream); break;
+      case 3: launch_skinny_mt<bf16_t, 3, 3>(a, w, bias, c, M, D, K, lda, D, 1, cs, stream); break;
+      default: launch_skinny_mt<bf16_t, 4, 3>(a, w, bias, c, M, D, K, lda, D, 1, cs, stream); break;
+    }
+    KAPPAI_RETURN_LAUNCH_STATUS();
+  }
   return launch_bf16<bf16_t, 2>((const bf16_t*)A, (const bf16_t*)W, bias, (bf16_t*)C, M, D, K, lda,
                                 D, 2, 1, stream, cs);
 }

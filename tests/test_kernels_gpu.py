@@ -432,7 +432,8 @@ def test_shortconv(ops, dtype, D, L):
 
 @pytest.mark.parametrize("M,D,K,L,bias", [(1, 64, 64, 3, False), (8, 2048, 2048, 3, False),
                                           (5, 96, 96, 4, True), (33, 48, 120, 2, True),
-                                          (64, 320, 72, 5, False)])
+                                          (64, 320, 72, 5, False), (20, 128, 256, 3, True),
+                                          (8, 4096, 512, 3, False), (40, 4112, 64, 3, True)])
 def test_linear_shortconv_step(ops, M, D, K, L, bias):
     """The fused decode step of a conv layer against the unfused kernels and the CPU stand-in,
     over two steps so that the state written by the first is read by the second."""
