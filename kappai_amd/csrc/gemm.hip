@@ -28,6 +28,7 @@ typedef __attribute__((ext_vector_type(4))) uint32_t u32x4_t;
 #define F32_BM 64
 #define F32_BN 64
 #define F32_BK 16
+#define F32_SUM_TILES 8
 
 __global__ __launch_bounds__(256) void gemm_f32_kernel(const float* __restrict__ A,
                                                        const float* __restrict__ W,
@@ -39,13 +40,28 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const float* __restrict__
   const int tid = threadIdx.x;
   const int tx = tid % 16, ty = tid / 16;
   const int m0 = blockIdx.y * F32_BM, n0 = blockIdx.x * F32_BN;
-  float acc[4][4];
+  // Sums in two levels: `acc` runs over F32_SUM_TILES tiles of K (128 values), then goes into
+  // `tot`.  A single running sum over K = 8192 loses about sqrt(K) roundings; this way it is
+  // sqrt(128) + sqrt(K / 128), a quarter of that, for one more addition per 128 products.
+  float acc[4][4], tot[4][4];
 #pragma unroll
   for (int i = 0; i < 4; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j) acc[i][j] = 0.f;
+    for (int j = 0; j < 4; ++j) acc[i][j] = tot[i][j] = 0.f;
 
+  int tiles_in_acc = 0;
   for (int k0 = 0; k0 < K; k0 += F32_BK) {
+    if (tiles_in_acc == F32_SUM_TILES) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          tot[i][j] += acc[i][j];
+          acc[i][j] = 0.f;
+        }
+      tiles_in_acc = 0;
+    }
+    ++tiles_in_acc;
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       const int idx = tid + e * 256;         // 0..1023
@@ -76,7 +92,7 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const float* __restrict__
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int gn = n0 + tx * 4 + j;
-      if (gn < N) C[(size_t)gm * ldc + gn] = acc[i][j] + (bias ? bias[gn] : 0.f);
+      if (gn < N) C[(size_t)gm * ldc + gn] = (tot[i][j] + acc[i][j]) + (bias ? bias[gn] : 0.f);
     }
   }
 }
