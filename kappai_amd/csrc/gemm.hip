@@ -662,6 +662,16 @@ static void launch_block256(const bf16_t* A, const bf16_t* W, const float* bias,
                      n_rows_w, K, lda, ldc, tn);
 }
 
+// The 256 x 256 form (one block a CU, 40-55 us per round of up to 256 blocks at K = 2048) against
+// the 128 x 128 form (two blocks a CU): from 140 blocks on when one round does it, and with more
+// rounds when the last one is not mostly idle (idle CU-rounds under 30 % of the blocks); from a
+// sweep of the layer shapes at 1024 to 8192 rows.
+static bool use_256_form(long blocks256) {
+  if (blocks256 <= 256) return blocks256 >= 140;
+  const long rem = blocks256 % 256;
+  return rem == 0 || (256 - rem) * 10 < 3 * blocks256;
+}
+
 // shape: 0 = chosen by size, 1 = 128x128 blocks of two waves, 2 = 256x128 blocks (tiles of 32
 // of K, two LDS buffers), 3 = 256x128 blocks (tiles of 64 of K, one LDS buffer), 4 = 256x256
 // blocks of the same kernel (tiles of 64 of K), 5 = the 256x256 kernel with one wave a SIMD, 6 = its
@@ -681,7 +691,7 @@ static void launch_tile(const bf16_t* A, const bf16_t* W, const float* bias, TO*
     // with four LDS buffers (0.46 against 0.62-0.87 us per 64 of K; its start costs 2 us more)
     const long blocks128 = (long)((M + 127) / 128) * ((n_rows_w + 127) / 128) * ksplit;
     const bool deep = blocks128 <= 256 && K / ksplit >= 2048;
-    shape = !fits ? (big >= 128 ? 3 : 1) : blocks256 >= 192 ? 5 : deep ? 8 : 6;
+    shape = !fits ? (big >= 128 ? 3 : 1) : use_256_form(blocks256) ? 5 : deep ? 8 : 6;
   }
   if ((shape == 5 || shape == 6 || shape == 8) && !fits) shape = 3;
   switch (shape) {

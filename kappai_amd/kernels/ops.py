@@ -214,7 +214,7 @@ def _split_k_large(M: int, N: int, K: int) -> int:
     sweep over 40 shapes, 1 % on average).  A 128 x 128 block that has a CU to itself takes
     about 0.62 us per 64 of K whatever else goes on, so a product with few blocks is bound by
     the length of K and gains almost linearly from being cut, until the chip is full (two
-    blocks a CU, each then a quarter slower; with 192 blocks of 256 x 256 or more the kernel
+    blocks a CU, each then a quarter slower; with 140 blocks of 256 x 256 or more the kernel
     takes its 256 x 256 form, about 1 us per 64 of K) or the float partial sums ([S, M, N],
     written here and read again by the consumer) cost more than the cut saves.  Every range is
     a multiple of 128 long, as the kernel asks."""
@@ -224,7 +224,9 @@ def _split_k_large(M: int, N: int, K: int) -> int:
             continue
         steps = K / split / 64
         blocks256 = ((M + 255) // 256) * ((N + 255) // 256) * split
-        if blocks256 >= 192:
+        rem = blocks256 % 256       # the kernel's own rule for its 256 x 256 form (gemm.hip)
+        if (140 <= blocks256 <= 256) or (blocks256 > 256 and (
+                rem == 0 or (256 - rem) * 10 < 3 * blocks256)):
             t = -(-blocks256 // 256) * (steps * 1.0 + 4.5)
         else:
             blocks = ((M + 127) // 128) * ((N + 127) // 128) * split
