@@ -459,7 +459,17 @@ __global__ __launch_bounds__(8 * WAVE) void attn_prefill_shared_kernel(
   for (int mt = 0; mt < P_MT; ++mt)
 #pragma unroll
     for (int v = 0; v < 16; ++v) o[mt][v] = 0.f;
-  float m_ref = -INFINITY, l_run = 0.f;
+  // The sums of the weights come from the matrix cores too: a V^T fragment of ones gives a
+  // tile whose every row is the sum over the keys, of the same rounded weights the output is made
+  // of.  (The kernel is bound by the issue of vector instructions: 16 additions and an exchange
+  // between half waves less per tile.)  Only at head size 64: at 128 the 16 registers more spill.
+  constexpr bool MFMA_SUM = HEAD_DIM == 64;
+  float l_add = 0.f;
+  f32x16_t o_sum;
+#pragma unroll
+  for (int v = 0; v < 16; ++v) o_sum[v] = 0.f;
+  const bf16x8_t ones = as_frag((u32x4_t){0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u});
+  float m_ref = -INFINITY;
   const float sc = scale * LOG2E;
 
   const int kbase = (blk_first / 32) * 32;
@@ -584,7 +594,12 @@ __global__ __launch_bounds__(8 * WAVE) void attn_prefill_shared_kernel(
       const float m_new = move ? mloc : m_ref;
       const float m_safe = m_new == -INFINITY ? 0.f : m_new;
       const float corr = move ? fast_exp2(m_ref - m_safe) : 1.0f;
-      l_run *= corr;
+      if (MFMA_SUM) {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) o_sum[v] *= corr;
+      } else {
+        l_add *= corr;
+      }
 #pragma unroll
       for (int mt = 0; mt < P_MT; ++mt)
 #pragma unroll
@@ -596,10 +611,12 @@ __global__ __launch_bounds__(8 * WAVE) void attn_prefill_shared_kernel(
 #pragma unroll
     for (int v = 0; v < 16; ++v) {
       s[v] = fast_exp2(fmaf(s[v], sc, -m_safe));
-      lsum += s[v];
+      if (!MFMA_SUM) lsum += s[v];
     }
-    lsum += other_half(lsum);
-    l_run += lsum;
+    if (!MFMA_SUM) {
+      lsum += other_half(lsum);
+      l_add += lsum;
+    }
     // ---- O^T += V^T P^T, two k-steps of 16 keys ---------------------------------------
 #pragma unroll
     for (int st = 0; st < 2; ++st) {
@@ -608,6 +625,7 @@ __global__ __launch_bounds__(8 * WAVE) void attn_prefill_shared_kernel(
                           pack_bf16(s[8 * st + 4], s[8 * st + 5]),
                           pack_bf16(s[8 * st + 6], s[8 * st + 7])};
       const bf16x8_t pf = as_frag(pw);
+      if (MFMA_SUM) o_sum = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ones, pf, o_sum, 0, 0, 0);
 #pragma unroll
       for (int mt = 0; mt < P_MT; ++mt) {
         const u32x4_t vw4 = {va[st][mt].x, va[st][mt].y, vb[st][mt].x, vb[st][mt].y};
@@ -641,6 +659,7 @@ __global__ __launch_bounds__(8 * WAVE) void attn_prefill_shared_kernel(
     if (it + 2 < n_steps) step(PgBuf<2>{}, it + 2);
   }
   if (!row_ok) return;
+  const float l_run = MFMA_SUM ? o_sum[0] : l_add;
   const float inv = l_run > 0.f ? 1.0f / l_run : 0.f;
   bf16_t* orow = out + (size_t)(r0 + col) * out_stride + (size_t)h * HEAD_DIM;
 #pragma unroll
