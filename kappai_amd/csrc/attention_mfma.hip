@@ -634,6 +634,96 @@ __global__ __launch_bounds__(8 * WAVE) void attn_prefill_shared_kernel(
     }
   };
 
+  // Both tiles of a buffer when neither needs a mask (most steps of a long history): the
+  // products of the second tile's scores are issued before the first tile's exponentials, so
+  // that the matrix cores work while the vector unit does the softmax of the tile before.
+  auto work2 = [&](auto buf_c) {
+    const char* buf0 = lds + (decltype(buf_c)::value * PG_SUB) * BUF;
+    const char* buf1 = buf0 + BUF;
+    auto scores = [&](const char* buf) {
+      f32x16_t s;
+#pragma unroll
+      for (int v = 0; v < 16; ++v) s[v] = 0.f;
+#pragma unroll
+      for (int ks = 0; ks < P_KS; ++ks) {
+        const u32x4_t kf = *reinterpret_cast<const u32x4_t*>(
+            buf + col * ROWB + (((2 * ks + hh) ^ swz(col)) * 16));
+        s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_frag(kf), qf[ks], s, 0, 0, 0);
+      }
+      return s;
+    };
+    // the running reference moves only when a tile's maximum is far above it (rare: a branch)
+    auto update_reference = [&](const f32x16_t& s) {
+      float mloc = -INFINITY;
+#pragma unroll
+      for (int v = 0; v < 16; ++v) mloc = fmaxf(mloc, s[v]);
+      mloc *= sc;
+      mloc = fmaxf(mloc, other_half(mloc));
+      const bool move = mloc > m_ref + 8.0f;
+      if (__builtin_amdgcn_ballot_w64(move) != 0) {
+        const float m_new = move ? mloc : m_ref;
+        const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+        const float corr = move ? fast_exp2(m_ref - m_safe) : 1.0f;
+        if (MFMA_SUM) {
+#pragma unroll
+          for (int v = 0; v < 16; ++v) o_sum[v] *= corr;
+        } else {
+          l_add *= corr;
+        }
+#pragma unroll
+        for (int mt = 0; mt < P_MT; ++mt)
+#pragma unroll
+          for (int v = 0; v < 16; ++v) o[mt][v] *= corr;
+        m_ref = m_new;
+      }
+    };
+    auto weights_and_output = [&](const char* buf, f32x16_t s) {
+      u32x2_t va[2][P_MT], vb[2][P_MT];
+#pragma unroll
+      for (int st = 0; st < 2; ++st)
+#pragma unroll
+        for (int mt = 0; mt < P_MT; ++mt) {
+          const int sw = ((col >> 3) & 1) * 16;
+          const char* vp = buf + KTILE + st * VGROUP + (32 * mt + col) * 32 + 8 * hh;
+          va[st][mt] = *reinterpret_cast<const u32x2_t*>(vp + sw);
+          vb[st][mt] = *reinterpret_cast<const u32x2_t*>(vp + (16 - sw));
+        }
+      const float m_safe = m_ref == -INFINITY ? 0.f : m_ref;
+      float lsum = 0.f;
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        s[v] = fast_exp2(fmaf(s[v], sc, -m_safe));
+        if (!MFMA_SUM) lsum += s[v];
+      }
+      if (!MFMA_SUM) {
+        lsum += other_half(lsum);
+        l_add += lsum;
+      }
+#pragma unroll
+      for (int st = 0; st < 2; ++st) {
+        const u32x4_t pw = {pack_bf16(s[8 * st + 0], s[8 * st + 1]),
+                            pack_bf16(s[8 * st + 2], s[8 * st + 3]),
+                            pack_bf16(s[8 * st + 4], s[8 * st + 5]),
+                            pack_bf16(s[8 * st + 6], s[8 * st + 7])};
+        const bf16x8_t pf = as_frag(pw);
+        if (MFMA_SUM) o_sum = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ones, pf, o_sum, 0, 0, 0);
+#pragma unroll
+        for (int mt = 0; mt < P_MT; ++mt) {
+          const u32x4_t vw4 = {va[st][mt].x, va[st][mt].y, vb[st][mt].x, vb[st][mt].y};
+          o[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_frag(vw4), pf, o[mt], 0, 0, 0);
+        }
+      }
+    };
+    // the second tile's score products stand between the first tile's maximum and its
+    // exponentials: nothing in them depends on the other
+    const f32x16_t s0 = scores(buf0);
+    update_reference(s0);
+    const f32x16_t s1 = scores(buf1);
+    weights_and_output(buf0, s0);
+    update_reference(s1);
+    weights_and_output(buf1, s1);
+  };
+
   // `it` counts buffers' worth of tiles (PG_SUB each)
   const int n_steps = (n_tiles + PG_SUB - 1) / PG_SUB;
   auto step = [&](auto buf_c, int it) {
@@ -646,6 +736,10 @@ __global__ __launch_bounds__(8 * WAVE) void attn_prefill_shared_kernel(
     // step it+2 goes into the buffer of step it-1: everybody is done with it
     if (it + 2 < n_steps) issue(PgBuf<(B + 2) % PG_NBUF>{});
     const int kb = kbase + 32 * PG_SUB * it;
+    if (HEAD_DIM == 64 && has_tile && whole(kb) && whole(kb + 32)) {   // (128: registers spill)
+      work2(buf_c);
+      return;
+    }
     if (has_tile && kb + 31 >= lo_tile && kb <= pos_last) work(buf_c, PgBuf<0>{}, PG_SUB * it);
     if (has_tile && kb + 63 >= lo_tile && kb + 32 <= pos_last)
       work(buf_c, PgBuf<1>{}, PG_SUB * it + 1);
