@@ -772,7 +772,8 @@ struct NormIn {
 template <typename TO, int MT, int NW, int EPI, int NT, bool PRO = false>
 __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny_kernel(
     const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, const float* __restrict__ bias,
-    TO* __restrict__ C, int M, int N, int K, int lda, int ldc, ConvStep cs, NormIn nin) {
+    TO* __restrict__ C, int M, int N, int K, int lda, int ldc, ConvStep cs, NormIn nin,
+    int w_frag) {
   static_assert(NT == 1 || EPI == 0, "several column tiles a wave: plain products only");
   static_assert(!PRO || (MT == 1 && NT == 1), "normalised rows: one row tile");
   // row groups of W a block streams: gate/up, the three conv gates, or NT column tiles
@@ -796,7 +797,16 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny_kernel(
   const size_t wr0 = EPI == 1 ? (size_t)blockIdx.x * 32 + col
                               : (EPI == 3 && col >= 8 ? (size_t)N + gn : (size_t)gn);
   const size_t group_rows = EPI == 2 ? (size_t)N : (EPI == 3 ? 2 * (size_t)N : 16);
-  const bf16_t* wrow = W + (gn < N ? wr0 : 0) * K + kg;
+  // W as it is stored ([rows, K]), or its copy in fragment order (w_frag): [rows / 16][K / 32]
+  // pieces of 1 KB, each what one load instruction of a wave wants, lane by lane (lane =
+  // (k % 32) / 8 * 16 + row % 16, 8 values a lane).  A wave's loads then touch every cache line
+  // once instead of twice, and neighbouring lines: the products with 1-16 rows are bound by the
+  // number of lines asked for as much as by bytes (gate/up at 8 rows: 14.7 against 18.2 us).
+  // One step of 32 along K is 32 elements here and 512 there.
+  const size_t wr1 = gn < N ? wr0 : 0;
+  const int kmul = w_frag ? 16 : 1;
+  const bf16_t* wrow = w_frag ? W + (wr1 / 16) * 16 * K + ((size_t)(kg / 8) * 16 + wr1 % 16) * 8
+                              : W + wr1 * K + kg;
   auto group_ok = [&](int r) { return EPI == 3 ? (r == 0 || col < 8) : true; };
   const bf16_t* arow[MT];
 #pragma unroll
@@ -866,7 +876,7 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny_kernel(
 #pragma unroll
       for (int r = 0; r < NG; ++r)
         wv[u][r] = (kin && gn + (EPI == 0 ? r * 16 : 0) < N && group_ok(r))
-                       ? load16(wrow + r * group_rows * K + gk)
+                       ? load16(wrow + r * group_rows * K + (size_t)gk * kmul)
                        : zero;
     }
   };
@@ -916,7 +926,7 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny_kernel(
 #pragma unroll
         for (int r = 0; r < NG; ++r)
           wv[u][r] = (kin && gn + (EPI == 0 ? r * 16 : 0) < N && group_ok(r))
-                         ? load16(wrow + r * group_rows * K + gk)
+                         ? load16(wrow + r * group_rows * K + (size_t)gk * kmul)
                          : zero;
 #pragma unroll
         for (int t = 0; t < MT; ++t)
@@ -1007,29 +1017,35 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny_kernel(
 template <typename TO, int MT, int NW, int EPI, int NT = 1>
 static void launch_skinny(const bf16_t* A, const bf16_t* W, const float* bias, TO* C, int M, int N,
                           int K, int lda, int ldc, int ksplit, ConvStep cs, hipStream_t stream,
-                          const NormIn* nin = nullptr) {
+                          const NormIn* nin = nullptr, const bf16_t* Wf = nullptr) {
+  // Wf: the copy of W in fragment order (see the kernel), or null
+  const int w_frag = Wf != nullptr;
+  if (Wf) W = Wf;
   const dim3 grid(EPI == 3 ? (N + 7) / 8 : (N + 16 * NT - 1) / (16 * NT), ksplit);
   if constexpr (MT == 1 && NT == 1 && EPI != 2 && EPI != 3) {
     if (nin) {
       hipLaunchKernelGGL((gemm_bf16_skinny_kernel<TO, MT, NW, EPI, NT, true>), grid,
-                         dim3(NW * WAVE), 0, stream, A, W, bias, C, M, N, K, lda, ldc, cs, *nin);
+                         dim3(NW * WAVE), 0, stream, A, W, bias, C, M, N, K, lda, ldc, cs, *nin,
+                         w_frag);
       return;
     }
   }
   hipLaunchKernelGGL((gemm_bf16_skinny_kernel<TO, MT, NW, EPI, NT>), grid, dim3(NW * WAVE), 0,
-                     stream, A, W, bias, C, M, N, K, lda, ldc, cs, NormIn{});
+                     stream, A, W, bias, C, M, N, K, lda, ldc, cs, NormIn{}, w_frag);
 }
 
 // more waves a block when there are few blocks, so that about 2048 waves or more stream W
 template <typename TO, int MT, int EPI>
 static void launch_skinny_mt(const bf16_t* A, const bf16_t* W, const float* bias, TO* C, int M,
                              int N, int K, int lda, int ldc, int ksplit, ConvStep cs,
-                             hipStream_t stream, const NormIn* nin = nullptr) {
+                             hipStream_t stream, const NormIn* nin = nullptr,
+                             const bf16_t* Wf = nullptr) {
   // several row tiles and a plain product: a wave takes two column tiles for every fragment
   // of A it loads, which halves the reads of A (every block reads all of it)
   if constexpr (EPI == 0 && MT >= 2) {
     if (N >= 64) {
-      launch_skinny<TO, MT, 4, EPI, 2>(A, W, bias, C, M, N, K, lda, ldc, ksplit, cs, stream);
+      launch_skinny<TO, MT, 4, EPI, 2>(A, W, bias, C, M, N, K, lda, ldc, ksplit, cs, stream,
+                                       nullptr, Wf);
       return;
     }
   }
@@ -1037,7 +1053,8 @@ static void launch_skinny_mt(const bf16_t* A, const bf16_t* W, const float* bias
   // A (58 against 62 us for 65,536 columns at 8 rows, 62 against 74 at 16; slower below 8 rows)
   if constexpr (EPI == 0 && MT == 1) {
     if (!nin && M >= 8 && (long)(N / 64) * ksplit >= 512) {
-      launch_skinny<TO, MT, 4, EPI, 4>(A, W, bias, C, M, N, K, lda, ldc, ksplit, cs, stream);
+      launch_skinny<TO, MT, 4, EPI, 4>(A, W, bias, C, M, N, K, lda, ldc, ksplit, cs, stream,
+                                       nullptr, Wf);
       return;
     }
   }
@@ -1046,13 +1063,13 @@ static void launch_skinny_mt(const bf16_t* A, const bf16_t* W, const float* bias
   constexpr int NG = EPI == 1 ? 2 : (EPI == 2 ? 3 : (EPI == 3 ? 2 : 1));
   constexpr int MAXW = 48 / (MT * NG);                    // 1 KB of LDS a wave, group and row tile
   if (blocks * 4 >= 2048 || kb <= 512 || MAXW < 8)
-    launch_skinny<TO, MT, 4, EPI>(A, W, bias, C, M, N, K, lda, ldc, ksplit, cs, stream, nin);
+    launch_skinny<TO, MT, 4, EPI>(A, W, bias, C, M, N, K, lda, ldc, ksplit, cs, stream, nin, Wf);
   else if (blocks * 8 >= 2048 || kb <= 1024 || MAXW < 16)
     launch_skinny<TO, MT, (MAXW >= 8 ? 8 : 4), EPI>(A, W, bias, C, M, N, K, lda, ldc, ksplit, cs,
-                                                    stream, nin);
+                                                    stream, nin, Wf);
   else
     launch_skinny<TO, MT, (MAXW >= 16 ? 16 : 4), EPI>(A, W, bias, C, M, N, K, lda, ldc, ksplit, cs,
-                                                      stream, nin);
+                                                      stream, nin, Wf);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -1279,7 +1296,9 @@ static bool launch_shared_rows(const bf16_t* A, const bf16_t* W, const float* bi
 template <typename TO, int EPI>
 static int launch_bf16(const bf16_t* A, const bf16_t* W, const float* bias, TO* C, int M, int N,
                        int K, int lda, int ldc, int force_kernel, int ksplit, hipStream_t stream,
-                       ConvStep cs = ConvStep{}) {
+                       ConvStep cs = ConvStep{}, const bf16_t* Wf = nullptr) {
+  // Wf: W once more in fragment order, for the kernel of 1 to 16 rows (see there); the others
+  // read W
   // N counts output columns; with the SwiGLU epilogue W has 2N rows
   // a very wide plain product (the output head) with more than 32 rows streams faster through
   // the 128 x 128 blocks than through the decode kernel, which reads the rows once per 32 columns
@@ -1301,16 +1320,20 @@ static int launch_bf16(const bf16_t* A, const bf16_t* W, const float* bias, TO* 
     const int mt = (M + 15) / 16;
     switch (mt) {
       case 1:
-        launch_skinny_mt<TO, 1, EPI>(A, W, bias, C, M, N, K, lda, ldc, ksplit, cs, stream);
+        launch_skinny_mt<TO, 1, EPI>(A, W, bias, C, M, N, K, lda, ldc, ksplit, cs, stream, nullptr,
+                                     Wf);
         break;
       case 2:
-        launch_skinny_mt<TO, 2, EPI>(A, W, bias, C, M, N, K, lda, ldc, ksplit, cs, stream);
+        launch_skinny_mt<TO, 2, EPI>(A, W, bias, C, M, N, K, lda, ldc, ksplit, cs, stream, nullptr,
+                                     Wf);
         break;
       case 3:
-        launch_skinny_mt<TO, 3, EPI>(A, W, bias, C, M, N, K, lda, ldc, ksplit, cs, stream);
+        launch_skinny_mt<TO, 3, EPI>(A, W, bias, C, M, N, K, lda, ldc, ksplit, cs, stream, nullptr,
+                                     Wf);
         break;
       default:
-        launch_skinny_mt<TO, 4, EPI>(A, W, bias, C, M, N, K, lda, ldc, ksplit, cs, stream);
+        launch_skinny_mt<TO, 4, EPI>(A, W, bias, C, M, N, K, lda, ldc, ksplit, cs, stream, nullptr,
+                                     Wf);
         break;
     }
   } else {
@@ -1327,40 +1350,53 @@ static int launch_bf16(const bf16_t* A, const bf16_t* W, const float* bias, TO* 
 // with block shape 1..6 (see launch_tile), 9 = shared-rows kernel (17 to 64 rows, K / ksplit a
 // multiple of 512), 10 = block shape 8; for tests and tuning.
 // ksplit > 1 (float output only): C is [ksplit][M][ldc] partial sums over K ranges.
-extern "C" int kappai_gemm_bf16(const void* A, const void* W, const float* bias, void* C, int M,
-                                int N, int K, int lda, int ldc, int out_is_f32, int force_kernel,
-                                int ksplit, hipStream_t stream) {
+// W_frag: null, or W again in fragment order (K a multiple of 32, rows a multiple of 16).
+static bool frag_ok(const void* W_frag, int rows, int K) {
+  return W_frag == nullptr || (K % 32 == 0 && rows % 16 == 0 && ((uintptr_t)W_frag % 16) == 0);
+}
+
+extern "C" int kappai_gemm_bf16(const void* A, const void* W, const void* W_frag, const float* bias,
+                                void* C, int M, int N, int K, int lda, int ldc, int out_is_f32,
+                                int force_kernel, int ksplit, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
   if ((K % 8) || (lda % 8) || ksplit < 1 || ksplit > 64) return (int)hipErrorInvalidValue;
+  if (!frag_ok(W_frag, N, K)) return (int)hipErrorInvalidValue;
   if (force_kernel == 2 && M > 64) return (int)hipErrorInvalidValue;
   if (ksplit > 1 && !out_is_f32) return (int)hipErrorInvalidValue;
   if (out_is_f32)
     return launch_bf16<float, 0>((const bf16_t*)A, (const bf16_t*)W, bias, (float*)C, M, N, K, lda,
-                                 ldc, force_kernel, ksplit, stream);
+                                 ldc, force_kernel, ksplit, stream, ConvStep{},
+                                 (const bf16_t*)W_frag);
   return launch_bf16<bf16_t, 0>((const bf16_t*)A, (const bf16_t*)W, bias, (bf16_t*)C, M, N, K, lda,
-                                ldc, force_kernel, 1, stream);
+                                ldc, force_kernel, 1, stream, ConvStep{}, (const bf16_t*)W_frag);
 }
 
 // C[M, F] = silu(A Wg^T) * (A Wu^T) with W = gate and up rows interleaved in groups of 16,
 // [2F, K]; F must be a multiple of 16.
-extern "C" int kappai_gemm_bf16_swiglu(const void* A, const void* W, void* C, int M, int F, int K,
-                                       int lda, int ldc, int force_kernel, hipStream_t stream) {
+extern "C" int kappai_gemm_bf16_swiglu(const void* A, const void* W, const void* W_frag, void* C,
+                                       int M, int F, int K, int lda, int ldc, int force_kernel,
+                                       hipStream_t stream) {
   if (M <= 0 || F <= 0) return 0;
   if ((K % 8) || (lda % 8) || (F % 16)) return (int)hipErrorInvalidValue;
   if (force_kernel == 2 && M > 64) return (int)hipErrorInvalidValue;
+  if (!frag_ok(W_frag, 2 * F, K)) return (int)hipErrorInvalidValue;
   return launch_bf16<bf16_t, 1>((const bf16_t*)A, (const bf16_t*)W, nullptr, (bf16_t*)C, M, F, K,
-                                lda, ldc, force_kernel, 1, stream);
+                                lda, ldc, force_kernel, 1, stream, ConvStep{},
+                                (const bf16_t*)W_frag);
 }
 
 // Conv layer decode step in one kernel: C[M, D] = Cgate * conv(Bgate * x | state) from A [M, K]
 // and the in_proj matrix W [3D, K]; M <= 64, one row a request; D a multiple of 16.
-extern "C" int kappai_gemm_bf16_shortconv_step(const void* A, const void* W, const float* bias,
+extern "C" int kappai_gemm_bf16_shortconv_step(const void* A, const void* W, const void* W_frag,
+                                               const float* bias,
                                                void* C, int M, int D, int K, int lda,
                                                const float* taps, const float* conv_bias,
                                                float* state, const int* seg_pos0,
                                                const int* seg_slot, int L, hipStream_t stream) {
   if (M <= 0 || D <= 0) return 0;
   if ((K % 8) || (lda % 8) || (D % 16) || M > 64 || L < 2) return (int)hipErrorInvalidValue;
+  if (!frag_ok(W_frag, 3 * D, K)) return (int)hipErrorInvalidValue;
+  const bf16_t* wf = (const bf16_t*)W_frag;
   ConvStep cs{taps, conv_bias, state, seg_pos0, seg_slot, L};
   if (D / 16 < 256) {
     // too few blocks of 16 channels for the chip: 8 channels a block
@@ -1368,15 +1404,23 @@ extern "C" int kappai_gemm_bf16_shortconv_step(const void* A, const void* W, con
     const bf16_t* w = (const bf16_t*)W;
     bf16_t* c = (bf16_t*)C;
     switch ((M + 15) / 16) {
-      case 1: launch_skinny_mt<bf16_t, 1, 3>(a, w, bias, c, M, D, K, lda, D, 1, cs, stream); break;
-      case 2: launch_skinny_mt<bf16_t, 2, 3>(a, w, bias, c, M, D, K, lda, D, 1, cs, stream); break;
-      case 3: launch_skinny_mt<bf16_t, 3, 3>(a, w, bias, c, M, D, K, lda, D, 1, cs, stream); break;
-      default: launch_skinny_mt<bf16_t, 4, 3>(a, w, bias, c, M, D, K, lda, D, 1, cs, stream); break;
+      case 1:
+        launch_skinny_mt<bf16_t, 1, 3>(a, w, bias, c, M, D, K, lda, D, 1, cs, stream, nullptr, wf);
+        break;
+      case 2:
+        launch_skinny_mt<bf16_t, 2, 3>(a, w, bias, c, M, D, K, lda, D, 1, cs, stream, nullptr, wf);
+        break;
+      case 3:
+        launch_skinny_mt<bf16_t, 3, 3>(a, w, bias, c, M, D, K, lda, D, 1, cs, stream, nullptr, wf);
+        break;
+      default:
+        launch_skinny_mt<bf16_t, 4, 3>(a, w, bias, c, M, D, K, lda, D, 1, cs, stream, nullptr, wf);
+        break;
     }
     KAPPAI_RETURN_LAUNCH_STATUS();
   }
   return launch_bf16<bf16_t, 2>((const bf16_t*)A, (const bf16_t*)W, bias, (bf16_t*)C, M, D, K, lda,
-                                D, 2, 1, stream, cs);
+                                D, 2, 1, stream, cs, wf);
 }
 
 // The same products for at most NORM_ROWS rows that are still to be made: A = RMSNorm(resid +
@@ -1393,31 +1437,34 @@ static bool norm_in_ok(int M, int K, const NormIn& n) {
 
 extern "C" int kappai_gemm_bf16_normed(const float* resid, const void* delta, int delta_f32,
                                        int n_parts, const float* norm_w, float eps,
-                                       float* resid_out, const void* W, const float* bias, void* C,
-                                       int M, int N, int K, int ldc, int out_is_f32, int ksplit,
-                                       hipStream_t stream) {
+                                       float* resid_out, const void* W, const void* W_frag,
+                                       const float* bias, void* C, int M, int N, int K, int ldc,
+                                       int out_is_f32, int ksplit, hipStream_t stream) {
   if (N <= 0) return 0;
+  if (!frag_ok(W_frag, N, K)) return (int)hipErrorInvalidValue;
   NormIn nin{resid, delta, delta ? n_parts : 0, delta_f32, norm_w, eps, delta ? resid_out : nullptr};
   if (!norm_in_ok(M, K, nin) || ksplit < 1 || ksplit > 64 || (ksplit > 1 && !out_is_f32))
     return (int)hipErrorInvalidValue;
   if (out_is_f32)
     launch_skinny_mt<float, 1, 0>(nullptr, (const bf16_t*)W, bias, (float*)C, M, N, K, K, ldc,
-                                  ksplit, ConvStep{}, stream, &nin);
+                                  ksplit, ConvStep{}, stream, &nin, (const bf16_t*)W_frag);
   else
     launch_skinny_mt<bf16_t, 1, 0>(nullptr, (const bf16_t*)W, bias, (bf16_t*)C, M, N, K, K, ldc, 1,
-                                   ConvStep{}, stream, &nin);
+                                   ConvStep{}, stream, &nin, (const bf16_t*)W_frag);
   KAPPAI_RETURN_LAUNCH_STATUS();
 }
 
 extern "C" int kappai_gemm_bf16_swiglu_normed(const float* resid, const void* delta, int delta_f32,
                                               int n_parts, const float* norm_w, float eps,
-                                              float* resid_out, const void* W, void* C, int M,
-                                              int F, int K, int ldc, hipStream_t stream) {
+                                              float* resid_out, const void* W,
+                                              const void* W_frag, void* C, int M, int F, int K,
+                                              int ldc, hipStream_t stream) {
   if (F <= 0) return 0;
+  if (!frag_ok(W_frag, 2 * F, K)) return (int)hipErrorInvalidValue;
   NormIn nin{resid, delta, delta ? n_parts : 0, delta_f32, norm_w, eps, delta ? resid_out : nullptr};
   if (!norm_in_ok(M, K, nin) || (F % 16)) return (int)hipErrorInvalidValue;
   launch_skinny_mt<bf16_t, 1, 1>(nullptr, (const bf16_t*)W, nullptr, (bf16_t*)C, M, F, K, K, ldc, 1,
-                                 ConvStep{}, stream, &nin);
+                                 ConvStep{}, stream, &nin, (const bf16_t*)W_frag);
   KAPPAI_RETURN_LAUNCH_STATUS();
 }
 

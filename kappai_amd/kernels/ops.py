@@ -237,6 +237,33 @@ def _split_k_large(M: int, N: int, K: int) -> int:
     return best
 
 
+def fragment_order(weight: torch.Tensor) -> Optional[torch.Tensor]:
+    """A copy of a bfloat16 matrix [N, K] in the order in which the product kernel for 1 to 16
+    rows loads it: pieces of 16 rows x 32 of K, each laid out lane by lane ([N / 16][K / 32]
+    [(k % 32) / 8][row % 16][8 values]), so that one load instruction of a wave reads 1 KB in
+    one piece.  None when the shape does not allow it (N a multiple of 16, K of 32).  The
+    products take it beside the matrix itself (``weight_frag``); the kernels for more rows read
+    the matrix as it is."""
+    if weight.dtype != BF16 or weight.dim() != 2:
+        return None
+    N, K = weight.shape
+    if N % 16 or K % 32 or N == 0:
+        return None
+    return (weight.contiguous().view(N // 16, 16, K // 32, 4, 8).permute(0, 2, 3, 1, 4)
+            .contiguous().view(N, K))
+
+
+def _frag(weight: torch.Tensor, weight_frag: Optional[torch.Tensor]) -> _vp:
+    if weight_frag is None:
+        return _vp(0)
+    _gpu("weight_frag", weight_frag, BF16)
+    _need(weight_frag.shape == weight.shape and weight.shape[0] % 16 == 0
+          and weight.shape[1] % 32 == 0 and weight_frag.data_ptr() % 16 == 0,
+          "weight_frag: the fragment-order copy must have the matrix's shape [N, K] with N a "
+          "multiple of 16 and K of 32")
+    return _vp(weight_frag.data_ptr())
+
+
 def split_k_for(M: int, N: int, K: int) -> int:
     """How many K ranges a product is cut into when its consumer takes partial sums (1: not
     split).  Decode (M <= 64): so that about 512 blocks stream the matrix (17 rows and more: what
@@ -257,19 +284,21 @@ def split_k_for(M: int, N: int, K: int) -> int:
 
 def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
            out_dtype=None, force_kernel: int = 0, partial_sums: bool = False,
-           split_k: Optional[int] = None) -> torch.Tensor:
+           split_k: Optional[int] = None,
+           weight_frag: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``x [M, K] @ weight[N, K]^T (+ bias)``.  A bfloat16 matrix runs on the matrix cores
     with float accumulation; a float32 matrix runs in true 32-bit arithmetic, whatever the
     activations' dtype.  ``x`` may be a view with a row stride.  With ``partial_sums`` the
     result may come back as float32 [S, M, N], the sums over S ranges of K, for a consumer
     that adds them (a matrix with few columns is then streamed by enough blocks).  ``x`` may
-    be a ``PendingNorm``: the rows are then made inside the product kernel."""
+    be a ``PendingNorm``: the rows are then made inside the product kernel.  ``weight_frag``
+    (``fragment_order(weight)``) is read in place of ``weight`` by the kernel for 1 to 16 rows."""
     if isinstance(x, PendingNorm):
         if (weight.dtype != BF16 or force_kernel or weight.dim() != 2
                 or weight.shape[1] != x.shape[1] or weight.data_ptr() % 16):
             x = x.materialize()
         else:
-            return _linear_normed(x, weight, bias, out_dtype, partial_sums, split_k)
+            return _linear_normed(x, weight, bias, out_dtype, partial_sums, split_k, weight_frag)
     _gpu("x", x, (F32, BF16), contiguous=False)
     _gpu("weight", weight, (F32, BF16))
     _need(x.dim() == 2 and weight.dim() == 2 and x.shape[1] == weight.shape[1],
@@ -311,13 +340,15 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] =
         out = torch.empty((M, N), dtype=out_dtype, device=x.device)
         out_is_f32 = 0 if out_dtype == BF16 else 1
     check(library("gemm").kappai_gemm_bf16(
-        _ptr(xb), _ptr(weight), _ptr(bias), _ptr(out), _c_int(M), _c_int(N), _c_int(K),
+        _ptr(xb), _ptr(weight), _frag(weight, weight_frag), _ptr(bias), _ptr(out), _c_int(M),
+        _c_int(N), _c_int(K),
         _c_int(lda), _c_int(N), _c_int(out_is_f32), _c_int(force_kernel), _c_int(ksplit),
         _stream()), "gemm_bf16")
     return out
 
 
-def _linear_normed(x: PendingNorm, weight, bias, out_dtype, partial_sums, split_k) -> torch.Tensor:
+def _linear_normed(x: PendingNorm, weight, bias, out_dtype, partial_sums, split_k,
+                   weight_frag=None) -> torch.Tensor:
     _gpu("weight", weight, BF16)
     M, K = x.shape
     N = weight.shape[0]
@@ -333,7 +364,8 @@ def _linear_normed(x: PendingNorm, weight, bias, out_dtype, partial_sums, split_
         out = torch.empty((M, N), dtype=out_dtype, device=x.device)
         out_is_f32 = 0 if out_dtype == BF16 else 1
     check(library("gemm").kappai_gemm_bf16_normed(
-        *x._kernel_args(), _ptr(weight), _ptr(bias), _ptr(out), _c_int(M), _c_int(N), _c_int(K),
+        *x._kernel_args(), _ptr(weight), _frag(weight, weight_frag), _ptr(bias), _ptr(out),
+        _c_int(M), _c_int(N), _c_int(K),
         _c_int(N), _c_int(out_is_f32), _c_int(ksplit), _stream()), "gemm_bf16_normed")
     return out
 
@@ -353,7 +385,8 @@ def interleave_gate_up(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
     return torch.cat([g, u], dim=1).reshape(2 * F, K).contiguous()
 
 
-def linear_swiglu(x: torch.Tensor, weight: torch.Tensor, force_kernel: int = 0) -> torch.Tensor:
+def linear_swiglu(x: torch.Tensor, weight: torch.Tensor, force_kernel: int = 0,
+                  weight_frag: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``silu(x Wg^T) * (x Wu^T)`` in one kernel: ``weight`` [2F, K] holds the gate and up
     matrices interleaved by ``interleave_gate_up``; bfloat16 only.  Returns [M, F].  ``x`` may
     be a ``PendingNorm``."""
@@ -368,7 +401,8 @@ def linear_swiglu(x: torch.Tensor, weight: torch.Tensor, force_kernel: int = 0) 
             F = weight.shape[0] // 2
             out = torch.empty((M, F), dtype=BF16, device=x.device)
             check(library("gemm").kappai_gemm_bf16_swiglu_normed(
-                *x._kernel_args(), _ptr(weight), _ptr(out), _c_int(M), _c_int(F), _c_int(K),
+                *x._kernel_args(), _ptr(weight), _frag(weight, weight_frag), _ptr(out), _c_int(M),
+                _c_int(F), _c_int(K),
                 _c_int(F), _stream()), "gemm_bf16_swiglu_normed")
             return out
     _gpu("x", x, BF16, contiguous=False)
@@ -385,7 +419,8 @@ def linear_swiglu(x: torch.Tensor, weight: torch.Tensor, force_kernel: int = 0) 
                   "and the tensors 16-byte aligned")
     out = torch.empty((M, F), dtype=BF16, device=x.device)
     check(library("gemm").kappai_gemm_bf16_swiglu(
-        _ptr(x), _ptr(weight), _ptr(out), _c_int(M), _c_int(F), _c_int(K), _c_int(lda), _c_int(F),
+        _ptr(x), _ptr(weight), _frag(weight, weight_frag), _ptr(out), _c_int(M), _c_int(F), _c_int(K),
+        _c_int(lda), _c_int(F),
         _c_int(force_kernel), _stream()), "gemm_bf16_swiglu")
     return out
 
@@ -393,7 +428,8 @@ def linear_swiglu(x: torch.Tensor, weight: torch.Tensor, force_kernel: int = 0) 
 def linear_shortconv_step(x: torch.Tensor, in_proj: torch.Tensor, in_bias: Optional[torch.Tensor],
                           taps: torch.Tensor, conv_bias: Optional[torch.Tensor],
                           state: torch.Tensor, seg_pos0: torch.Tensor,
-                          seg_slot: torch.Tensor) -> torch.Tensor:
+                          seg_slot: torch.Tensor,
+                          weight_frag: Optional[torch.Tensor] = None) -> torch.Tensor:
     """A conv layer's decode step in one kernel, for a batch in which every row is its own
     segment: ``proj = x in_proj^T (+ bias)`` cut into (B | C | x), ``C * conv(B * x)`` with the
     rows' state slots read and shifted.  bfloat16, at most 64 rows, width a multiple of 16.
@@ -421,7 +457,8 @@ def linear_shortconv_step(x: torch.Tensor, in_proj: torch.Tensor, in_bias: Optio
             _need(t.shape == shp, lambda: f"{n} must be {shp}")
     out = torch.empty((M, D), dtype=BF16, device=x.device)
     check(library("gemm").kappai_gemm_bf16_shortconv_step(
-        _ptr(x), _ptr(in_proj), _ptr(in_bias), _ptr(out), _c_int(M), _c_int(D), _c_int(K),
+        _ptr(x), _ptr(in_proj), _frag(in_proj, weight_frag), _ptr(in_bias), _ptr(out), _c_int(M),
+        _c_int(D), _c_int(K),
         _c_int(lda), _ptr(taps), _ptr(conv_bias), _ptr(state), _ptr(seg_pos0), _ptr(seg_slot),
         _c_int(L), _stream()), "gemm_bf16_shortconv_step")
     return out

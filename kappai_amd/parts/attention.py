@@ -64,6 +64,9 @@ class GroupedQueryAttention(Mixer):
         self.out.bind(tensors)
         # the q rows of the stacked matrix, for a layer that reads another layer's keys
         self.q_only.weight = self.qkv.weight[: self.H * self.d]
+        frag = self.qkv.weight_frag          # whole pieces of 16 rows: the q rows come first
+        self.q_only.weight_frag = (None if frag is None or (self.H * self.d) % 16
+                                   else frag[: self.H * self.d])
         self.q_only.bias = None if self.qkv.bias is None else self.qkv.bias[: self.H * self.d]
         if self.qk_norm_eps is not None:
             self.q_norm_w = tensors[self._qn + ".weight"].to(torch.float32).contiguous()

@@ -35,12 +35,13 @@ class SwiGLU(FeedForward):
         self.fused = (w.dtype == torch.bfloat16 and self.hidden % ops.SWIGLU_GROUP == 0
                       and self.width % 8 == 0)
         if self.fused:
-            self.gate_up.weight = ops.interleave_gate_up(w[:self.hidden], w[self.hidden:])
+            self.gate_up.set_weight(ops.interleave_gate_up(w[:self.hidden], w[self.hidden:]))
 
     def forward(self, x, batch):
         if self.fused and x.dtype == torch.bfloat16:
-            return self.down.forward(ops.linear_swiglu(x, self.gate_up.weight),
-                                     partial_sums=True)
+            return self.down.forward(
+                ops.linear_swiglu(x, self.gate_up.weight, weight_frag=self.gate_up.weight_frag),
+                partial_sums=True)
         return self.down.forward(ops.swiglu(self.gate_up.forward(x)), partial_sums=True)
 
     def weight_bytes(self) -> int:

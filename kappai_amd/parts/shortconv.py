@@ -82,7 +82,8 @@ class GatedShortConv(Mixer):
                 and self.width % 16 == 0 and wide_enough):
             # decode: projection, convolution and state shift in one kernel
             y = ops.linear_shortconv_step(x, w, self.in_proj.bias, self.taps, self.conv_bias,
-                                          cache.state, batch.seg_pos0, batch.seg_slot)
+                                          cache.state, batch.seg_pos0, batch.seg_slot,
+                                          weight_frag=self.in_proj.weight_frag)
             return self.out_proj.forward(y, partial_sums=True)
         # decode with more than 16 rows: the projection may come as sums over ranges of its input
         # dimension (more blocks stream the matrix), which the step kernel adds up; with fewer

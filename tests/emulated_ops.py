@@ -44,7 +44,8 @@ def cast(x, dtype):
     return x.to(dtype)
 
 
-def linear(x, weight, bias=None, out_dtype=None, force_kernel=0, partial_sums=False):
+def linear(x, weight, bias=None, out_dtype=None, force_kernel=0, partial_sums=False,
+           split_k=None, weight_frag=None):
     out_dtype = out_dtype or x.dtype
     y = x.to(F32) @ weight.to(F32).T
     if bias is not None:
@@ -62,7 +63,7 @@ def interleave_gate_up(gate, up):
     return torch.cat([g, u], dim=1).reshape(2 * F, K).contiguous()
 
 
-def linear_swiglu(x, weight, force_kernel=0):
+def linear_swiglu(x, weight, force_kernel=0, weight_frag=None):
     F = weight.shape[0] // 2
     y = (x.to(F32) @ weight.to(F32).T).reshape(x.shape[0], F // SWIGLU_GROUP, 2, SWIGLU_GROUP)
     g, u = y[:, :, 0, :].reshape(-1, F), y[:, :, 1, :].reshape(-1, F)
@@ -91,7 +92,8 @@ def shortconv(proj, taps, bias, state, row_seg, seg_start, seg_pos0, seg_slot):
     return out.to(proj.dtype)
 
 
-def linear_shortconv_step(x, in_proj, in_bias, taps, conv_bias, state, seg_pos0, seg_slot):
+def linear_shortconv_step(x, in_proj, in_bias, taps, conv_bias, state, seg_pos0, seg_slot,
+                          weight_frag=None):
     M = x.shape[0]
     proj = linear(x, in_proj, in_bias)
     row_seg = torch.arange(M, dtype=torch.int32)

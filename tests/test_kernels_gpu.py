@@ -247,6 +247,63 @@ def test_linear_block256_split_k(ops):
     close(parts.sum(0), x.double() @ w.double().T, 2e-5, "sum of the partial sums")
 
 
+@pytest.mark.parametrize("M", [1, 3, 8, 16, 40, 200])
+@pytest.mark.parametrize("N,K", [(16, 32), (48, 96), (2048, 2048), (1008, 4128), (6144, 1024)])
+def test_products_read_the_fragment_order_copy(ops, M, N, K):
+    """With the copy of the matrix in fragment order beside it every product gives bit for bit
+    what it gives without: plain, with bias, as partial sums over K ranges, with the SwiGLU
+    epilogue, with a pending RMSNorm as its input, and as the fused conv step (the kernel for 1 to
+    16 rows reads the copy; with more rows it is passed and not read)."""
+    x = rand((M, K), BF16, 60).to(DEV)
+    w, b = rand((N, K), BF16, 61, 0.1).to(DEV), rand((N,), F32, 62).to(DEV)
+    wf = ops.fragment_order(w)
+    assert wf is not None and wf.shape == w.shape and not torch.equal(wf, w)
+    # the copy holds element (n, k) at its place in the piece of 16 rows x 32 of K
+    n, k = N - 3, K - 5
+    at = ((n // 16) * (K // 32) + k // 32) * 512 + ((k % 32) // 8 * 16 + n % 16) * 8 + k % 8
+    assert wf.reshape(-1)[at] == w[n, k]
+    for bias in (None, b):
+        for out_dtype in (BF16, F32):
+            assert torch.equal(ops.linear(x, w, bias, out_dtype=out_dtype, weight_frag=wf),
+                               ops.linear(x, w, bias, out_dtype=out_dtype))
+    if K % 64 == 0:
+        assert torch.equal(ops.linear(x, w, partial_sums=True, split_k=2, weight_frag=wf),
+                           ops.linear(x, w, partial_sums=True, split_k=2))
+    if N % 32 == 0:
+        assert torch.equal(ops.linear_swiglu(x, w, weight_frag=wf), ops.linear_swiglu(x, w))
+    if M <= ops.NORM_FUSE_MAX_ROWS and K <= ops.NORM_FUSE_MAX_WIDTH:
+        resid, wn = rand((M, K), F32, 63, 2.0).to(DEV), (1 + rand((K,), F32, 64, 0.1)).to(DEV)
+        delta = rand((M, K), BF16, 65).to(DEV)
+        outs = []
+        for frag in (wf, None):
+            pend = ops.PendingNorm(resid, delta, wn, 1e-5, BF16)
+            outs.append(ops.linear(pend, w, b, out_dtype=F32, weight_frag=frag))
+        assert torch.equal(outs[0], outs[1])
+    if N % 48 == 0 and M <= 64:
+        D, L = N // 3, 3
+        taps = rand((D, L), F32, 66, 0.5).to(DEV)
+        state = rand((M + 1, D, L - 1), F32, 67).to(DEV)
+        pos0 = torch.ones(M, dtype=torch.int32, device=DEV)
+        slot = torch.arange(M, dtype=torch.int32, device=DEV)
+        outs, states = [], []
+        for frag in (wf, None):
+            st = state.clone()
+            outs.append(ops.linear_shortconv_step(x, w, b, taps, None, st, pos0, slot,
+                                                  weight_frag=frag))
+            states.append(st)
+        assert torch.equal(outs[0], outs[1]) and torch.equal(states[0], states[1])
+
+
+def test_fragment_order_needs_whole_pieces(ops):
+    assert ops.fragment_order(rand((40, 64), BF16, 68)) is None          # rows
+    assert ops.fragment_order(rand((48, 72), BF16, 68)) is None          # K
+    assert ops.fragment_order(rand((48, 64), F32, 68)) is None
+    w = rand((48, 64), BF16, 68).to(DEV)
+    x = rand((4, 64), BF16, 69).to(DEV)
+    with pytest.raises(ValueError):
+        ops.linear(x, w, weight_frag=w[:32])
+
+
 @pytest.mark.parametrize("M,N,K,S,block", [(575, 1024, 4608, 6, 0), (300, 520, 4096, 2, BLOCK128_DEEP),
                                            (130, 264, 1280, 5, BLOCK128_DEEP),
                                            (1100, 2048, 7168, 7, 0)])
