@@ -1102,7 +1102,7 @@ struct SharedRows {
 template <typename TO, int MT, int EPI, int NWN, int NWK, int KC, int NSETS>
 __global__ __launch_bounds__(NWN * NWK * WAVE) void gemm_bf16_shared_rows_kernel(
     const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, const float* __restrict__ bias,
-    TO* __restrict__ C, int M, int n_rows_w, int K, int lda, int ldc) {
+    TO* __restrict__ C, int M, int n_rows_w, int K, int lda, int ldc, int w_frag) {
   static_assert(NSETS % 2 == 0 && 2 * (KC / 32) * (NSETS - 1) < 64, "register sets");
   using S = SharedRows<MT, NWN, NWK, KC>;
   constexpr int NW = S::NW, UK = S::UK, CH = S::CH;
@@ -1121,8 +1121,15 @@ __global__ __launch_bounds__(NWN * NWK * WAVE) void gemm_bf16_shared_rows_kernel
   const int wrow0 = (blockIdx.x * NWN + wn) * 32;
   const bf16_t* wptr[2];
 #pragma unroll
-  for (int r = 0; r < 2; ++r)
-    wptr[r] = W + (size_t)min(wrow0 + 16 * r + col, n_rows_w - 1) * K + kb0 + wk * kper + kgi * 8;
+  for (int r = 0; r < 2; ++r) {
+    // W as stored, or its copy in fragment order (see gemm_bf16_skinny_kernel): a step of 32
+    // along K is 32 elements here and 512 there
+    const size_t row = (size_t)min(wrow0 + 16 * r + col, n_rows_w - 1);
+    const size_t kbase = (size_t)kb0 + (size_t)wk * kper;
+    wptr[r] = w_frag ? W + (row / 16) * 16 * K + kbase * 16 + ((size_t)kgi * 16 + row % 16) * 8
+                     : W + row * K + kbase + kgi * 8;
+  }
+  const int kmul = w_frag ? 16 : 1;
 
   // the block's load instructions for a chunk of A, dealt round the waves: instruction j
   // brings rows (j % (ROWS / RPI)) * RPI + lane / CH of K part j / (ROWS / RPI)
@@ -1152,7 +1159,7 @@ __global__ __launch_bounds__(NWN * NWK * WAVE) void gemm_bf16_shared_rows_kernel
 #pragma unroll
     for (int u = 0; u < UK; ++u)
 #pragma unroll
-      for (int r = 0; r < 2; ++r) wv[u][r] = load16(wptr[r] + c * KC + 32 * u);
+      for (int r = 0; r < 2; ++r) wv[u][r] = load16(wptr[r] + (size_t)(c * KC + 32 * u) * kmul);
   };
   f32x4_t acc[2 * MT];
 #pragma unroll
@@ -1256,7 +1263,7 @@ static bool shared_rows_fits(int M, int K, int lda, int ksplit) {
 template <typename TO, int MT, int EPI, int NWN, int NWK, int KC, int NSETS>
 static void launch_shared_rows_cfg(const bf16_t* A, const bf16_t* W, const float* bias, TO* C,
                                    int M, int n_rows_w, int K, int lda, int ldc, int ksplit,
-                                   hipStream_t stream) {
+                                   hipStream_t stream, const bf16_t* Wf) {
   using S = SharedRows<MT, NWN, NWK, KC>;
   auto kern = gemm_bf16_shared_rows_kernel<TO, MT, EPI, NWN, NWK, KC, NSETS>;
   static bool attr_set = false;       // more than 64 KB of LDS has to be asked for once
@@ -1266,8 +1273,8 @@ static void launch_shared_rows_cfg(const bf16_t* A, const bf16_t* W, const float
     attr_set = true;
   }
   hipLaunchKernelGGL(kern, dim3((n_rows_w + 32 * NWN - 1) / (32 * NWN), ksplit),
-                     dim3(S::NW * WAVE), S::lds_bytes, stream, A, W, bias, C, M, n_rows_w, K, lda,
-                     ldc);
+                     dim3(S::NW * WAVE), S::lds_bytes, stream, A, Wf ? Wf : W, bias, C, M, n_rows_w, K,
+                     lda, ldc, Wf ? 1 : 0);
 }
 
 // 2 x 4 waves, chunks of 128 of K, two register sets of W.  (4 x 4 waves leave half the CUs
@@ -1279,17 +1286,17 @@ static void launch_shared_rows_cfg(const bf16_t* A, const bf16_t* W, const float
 template <typename TO, int EPI>
 static bool launch_shared_rows(const bf16_t* A, const bf16_t* W, const float* bias, TO* C, int M,
                                int n_rows_w, int K, int lda, int ldc, int ksplit,
-                               hipStream_t stream) {
+                               hipStream_t stream, const bf16_t* Wf) {
   if (!shared_rows_fits<SR_NWK, SR_KC>(M, K, lda, ksplit)) return false;
   if (M <= 32)
     launch_shared_rows_cfg<TO, 2, EPI, SR_NWN, SR_NWK, SR_KC, 2>(A, W, bias, C, M, n_rows_w, K, lda,
-                                                                 ldc, ksplit, stream);
+                                                                 ldc, ksplit, stream, Wf);
   else if (M <= 48)
     launch_shared_rows_cfg<TO, 3, EPI, SR_NWN, SR_NWK, SR_KC, 2>(A, W, bias, C, M, n_rows_w, K, lda,
-                                                                 ldc, ksplit, stream);
+                                                                 ldc, ksplit, stream, Wf);
   else
     launch_shared_rows_cfg<TO, 4, EPI, SR_NWN, SR_NWK, SR_KC, 2>(A, W, bias, C, M, n_rows_w, K, lda,
-                                                                 ldc, ksplit, stream);
+                                                                 ldc, ksplit, stream, Wf);
   return true;
 }
 
@@ -1297,8 +1304,8 @@ template <typename TO, int EPI>
 static int launch_bf16(const bf16_t* A, const bf16_t* W, const float* bias, TO* C, int M, int N,
                        int K, int lda, int ldc, int force_kernel, int ksplit, hipStream_t stream,
                        ConvStep cs = ConvStep{}, const bf16_t* Wf = nullptr) {
-  // Wf: W once more in fragment order, for the kernel of 1 to 16 rows (see there); the others
-  // read W
+  // Wf: W once more in fragment order, for the kernels of 1 to 64 rows (see the first of them);
+  // the others read W
   // N counts output columns; with the SwiGLU epilogue W has 2N rows
   // a very wide plain product (the output head) with more than 32 rows streams faster through
   // the 128 x 128 blocks than through the decode kernel, which reads the rows once per 32 columns
@@ -1309,7 +1316,7 @@ static int launch_bf16(const bf16_t* A, const bf16_t* W, const float* bias, TO* 
     const int n_rows_w = EPI == 1 ? 2 * N : N;
     const long sr_blocks = (long)((n_rows_w + 32 * SR_NWN - 1) / (32 * SR_NWN)) * ksplit;
     if (force_kernel == 9 || (force_kernel == 0 && M > 16 && M <= 64 && sr_blocks >= 128)) {
-      if (launch_shared_rows<TO, EPI>(A, W, bias, C, M, n_rows_w, K, lda, ldc, ksplit, stream))
+      if (launch_shared_rows<TO, EPI>(A, W, bias, C, M, n_rows_w, K, lda, ldc, ksplit, stream, Wf))
         KAPPAI_RETURN_LAUNCH_STATUS();
       if (force_kernel == 9) return (int)hipErrorInvalidValue;
     }

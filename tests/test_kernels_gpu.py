@@ -271,6 +271,15 @@ def test_products_read_the_fragment_order_copy(ops, M, N, K):
                            ops.linear(x, w, partial_sums=True, split_k=2))
     if N % 32 == 0:
         assert torch.equal(ops.linear_swiglu(x, w, weight_frag=wf), ops.linear_swiglu(x, w))
+    if 16 < M <= 64 and K % 512 == 0:       # the kernel for 17 to 64 rows reads the copy too
+        assert torch.equal(ops.linear(x, w, b, force_kernel=SHARED_ROWS, weight_frag=wf),
+                           ops.linear(x, w, b, force_kernel=SHARED_ROWS))
+        assert torch.equal(
+            ops.linear(x, w, partial_sums=True, split_k=2, force_kernel=SHARED_ROWS, weight_frag=wf),
+            ops.linear(x, w, partial_sums=True, split_k=2, force_kernel=SHARED_ROWS))
+        if N % 32 == 0:
+            assert torch.equal(ops.linear_swiglu(x, w, force_kernel=SHARED_ROWS, weight_frag=wf),
+                               ops.linear_swiglu(x, w, force_kernel=SHARED_ROWS))
     if M <= ops.NORM_FUSE_MAX_ROWS and K <= ops.NORM_FUSE_MAX_WIDTH:
         resid, wn = rand((M, K), F32, 63, 2.0).to(DEV), (1 + rand((K,), F32, 64, 0.1)).to(DEV)
         delta = rand((M, K), BF16, 65).to(DEV)
