@@ -1022,7 +1022,7 @@ static void launch_skinny(const bf16_t* A, const bf16_t* W, const float* bias, T
   const int w_frag = Wf != nullptr;
   if (Wf) W = Wf;
   const dim3 grid(EPI == 3 ? (N + 7) / 8 : (N + 16 * NT - 1) / (16 * NT), ksplit);
-  if constexpr (MT == 1 && NT == 1 && EPI != 2 && EPI != 3) {
+  if constexpr (MT == 1 && NT == 1 && EPI != 2) {
     if (nin) {
       hipLaunchKernelGGL((gemm_bf16_skinny_kernel<TO, MT, NW, EPI, NT, true>), grid,
                          dim3(NW * WAVE), 0, stream, A, W, bias, C, M, N, K, lda, ldc, cs, *nin,
@@ -1050,9 +1050,11 @@ static void launch_skinny_mt(const bf16_t* A, const bf16_t* W, const float* bias
     }
   }
   // 8 to 16 rows and columns enough (the output head): four column tiles for every fragment of
-  // A (58 against 62 us for 65,536 columns at 8 rows, 62 against 74 at 16; slower below 8 rows)
+  // A (58 against 62 us for 65,536 columns at 8 rows, 62 against 74 at 16; slower below 8 rows).
+  // With W in fragment order one tile a wave is the faster up to 11 rows (50 against 56 us at 8
+  // rows, 56 either way at 12, 62 against 56 at 16).
   if constexpr (EPI == 0 && MT == 1) {
-    if (!nin && M >= 8 && (long)(N / 64) * ksplit >= 512) {
+    if (!nin && M >= (Wf ? 12 : 8) && (long)(N / 64) * ksplit >= 512) {
       launch_skinny<TO, MT, 4, EPI, 4>(A, W, bias, C, M, N, K, lda, ldc, ksplit, cs, stream,
                                        nullptr, Wf);
       return;
@@ -1458,6 +1460,24 @@ extern "C" int kappai_gemm_bf16_normed(const float* resid, const void* delta, in
   else
     launch_skinny_mt<bf16_t, 1, 0>(nullptr, (const bf16_t*)W, bias, (bf16_t*)C, M, N, K, K, ldc, 1,
                                    ConvStep{}, stream, &nin, (const bf16_t*)W_frag);
+  KAPPAI_RETURN_LAUNCH_STATUS();
+}
+
+// The conv layer's decode step (8 channels a block) on rows that are still to be made (see
+// NormIn): RMSNorm, in_proj, gates, FIR and state shift of a single decoded row in one kernel.
+// D below 4096 (the 16-channel form takes no pending norm), K at most NORM_MAX_K.
+extern "C" int kappai_gemm_bf16_shortconv_step_normed(
+    const float* resid, const void* delta, int delta_f32, int n_parts, const float* norm_w, float eps,
+    float* resid_out, const void* W, const void* W_frag, const float* bias, void* C, int M, int D,
+    int K, const float* taps, const float* conv_bias, float* state, const int* seg_pos0,
+    const int* seg_slot, int L, hipStream_t stream) {
+  if (D <= 0) return 0;
+  NormIn nin{resid, delta, delta ? n_parts : 0, delta_f32, norm_w, eps, delta ? resid_out : nullptr};
+  if (!norm_in_ok(M, K, nin) || (D % 16) || D / 16 >= 256 || L < 2 || !frag_ok(W_frag, 3 * D, K))
+    return (int)hipErrorInvalidValue;
+  ConvStep cs{taps, conv_bias, state, seg_pos0, seg_slot, L};
+  launch_skinny_mt<bf16_t, 1, 3>(nullptr, (const bf16_t*)W, bias, (bf16_t*)C, M, D, K, K, D, 1, cs,
+                                 stream, &nin, (const bf16_t*)W_frag);
   KAPPAI_RETURN_LAUNCH_STATUS();
 }
 

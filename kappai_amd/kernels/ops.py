@@ -433,8 +433,16 @@ def linear_shortconv_step(x: torch.Tensor, in_proj: torch.Tensor, in_bias: Optio
     """A conv layer's decode step in one kernel, for a batch in which every row is its own
     segment: ``proj = x in_proj^T (+ bias)`` cut into (B | C | x), ``C * conv(B * x)`` with the
     rows' state slots read and shifted.  bfloat16, at most 64 rows, width a multiple of 16.
-    Equals ``shortconv(linear(x, in_proj, in_bias), ...)``."""
-    _gpu("x", x, BF16, contiguous=False)
+    Equals ``shortconv(linear(x, in_proj, in_bias), ...)``.  ``x`` may be a ``PendingNorm``
+    (widths below 4096): the kernel then makes the normalised row itself as well."""
+    pending = x if isinstance(x, PendingNorm) else None
+    if pending is not None and not (in_proj.dtype == BF16 and in_proj.dim() == 2
+                                    and taps.dim() == 2 and taps.shape[0] // 16 < 256
+                                    and in_proj.shape[1] == x.shape[1]
+                                    and in_proj.data_ptr() % 16 == 0):
+        x, pending = x.materialize(), None
+    if pending is None:
+        _gpu("x", x, BF16, contiguous=False)
     _gpu("in_proj", in_proj, BF16)
     _gpu("taps", taps, F32)
     _gpu("state", state, F32)
@@ -447,15 +455,23 @@ def linear_shortconv_step(x: torch.Tensor, in_proj: torch.Tensor, in_bias: Optio
     _need(seg_pos0.shape == (M,) and seg_slot.shape == (M,), "one segment a row")
     _need(L >= 2 and state.dim() == 3 and state.shape[1:] == (D, L - 1),
           lambda: f"state {tuple(state.shape)} for D={D}, L={L}")
-    lda = x.stride(0) if M > 1 else K
-    _need((x.stride(1) == 1 or K == 1) and K % 8 == 0 and lda % 8 == 0
-          and x.data_ptr() % 16 == 0 and in_proj.data_ptr() % 16 == 0,
-          "linear_shortconv_step: K and the row stride must be multiples of 8, tensors aligned")
+    if pending is None:
+        lda = x.stride(0) if M > 1 else K
+        _need((x.stride(1) == 1 or K == 1) and K % 8 == 0 and lda % 8 == 0
+              and x.data_ptr() % 16 == 0 and in_proj.data_ptr() % 16 == 0,
+              "linear_shortconv_step: K and the row stride must be multiples of 8, tensors aligned")
     for n, t, shp in (("in_bias", in_bias, (3 * D,)), ("conv_bias", conv_bias, (D,))):
         if t is not None:
             _gpu(n, t, F32)
             _need(t.shape == shp, lambda: f"{n} must be {shp}")
     out = torch.empty((M, D), dtype=BF16, device=x.device)
+    if pending is not None:
+        check(library("gemm").kappai_gemm_bf16_shortconv_step_normed(
+            *pending._kernel_args(), _ptr(in_proj), _frag(in_proj, weight_frag), _ptr(in_bias),
+            _ptr(out), _c_int(M), _c_int(D), _c_int(K), _ptr(taps), _ptr(conv_bias), _ptr(state),
+            _ptr(seg_pos0), _ptr(seg_slot), _c_int(L), _stream()),
+            "gemm_bf16_shortconv_step_normed")
+        return out
     check(library("gemm").kappai_gemm_bf16_shortconv_step(
         _ptr(x), _ptr(in_proj), _frag(in_proj, weight_frag), _ptr(in_bias), _ptr(out), _c_int(M),
         _c_int(D), _c_int(K),

@@ -22,12 +22,12 @@ from .linear import PARTIAL_SUMS_MIN_ROWS, Linear
 # The fused decode kernel gives one block 16 channels (8 below a width of 4096, where 16 would
 # leave CUs without a block).  From this width on it beats the separate product (which may split
 # K) plus the small step kernel for any number of rows up to 64; between FUSED_STEP_NARROW_WIDTH
-# and it only for 2 to 16 rows (12.6 against 13.2 us at a width of 2048 and 8 rows, 13.6 against
-# 14.9 at 16 rows; a single row rather lets the product make its RMSNorm input itself, and at a
-# width of 1024 the separate kernels win).
+# and it only up to 16 rows (at a width of 2048, W in fragment order: 8.3 against 9.9 us for one
+# row, which it also normalises itself when the norm before it is pending; 11.0 against 11.1 at
+# 8 rows, 11.5 against 12.8 at 16; at a width of 1024 the separate kernels win).
 FUSED_STEP_MIN_WIDTH = 4096
 FUSED_STEP_NARROW_WIDTH = 2048
-FUSED_STEP_NARROW_ROWS = (2, 16)
+FUSED_STEP_NARROW_ROWS = 16
 
 
 class GatedShortConv(Mixer):
@@ -72,14 +72,13 @@ class GatedShortConv(Mixer):
             raise ValueError("a short convolution's state cannot be read by another layer")
         w = self.in_proj.weight
         if isinstance(x, ops.PendingNorm) and self.width >= FUSED_STEP_MIN_WIDTH:
-            x = x.materialize()            # the fused step kernel below reads rows
+            x = x.materialize()            # the 16-channel form of the fused step reads rows
         rows = x.shape[0]
         wide_enough = self.width >= FUSED_STEP_MIN_WIDTH or (
-            self.width >= FUSED_STEP_NARROW_WIDTH
-            and FUSED_STEP_NARROW_ROWS[0] <= rows <= FUSED_STEP_NARROW_ROWS[1])
-        if (batch.max_segment_rows == 1 and rows <= 64 and not isinstance(x, ops.PendingNorm)
-                and x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16
-                and self.width % 16 == 0 and wide_enough):
+            self.width >= FUSED_STEP_NARROW_WIDTH and rows <= FUSED_STEP_NARROW_ROWS)
+        if (batch.max_segment_rows == 1 and rows <= 64
+                and (isinstance(x, ops.PendingNorm) or x.dtype == torch.bfloat16)
+                and w.dtype == torch.bfloat16 and self.width % 16 == 0 and wide_enough):
             # decode: projection, convolution and state shift in one kernel
             y = ops.linear_shortconv_step(x, w, self.in_proj.bias, self.taps, self.conv_bias,
                                           cache.state, batch.seg_pos0, batch.seg_slot,

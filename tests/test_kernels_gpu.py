@@ -530,6 +530,40 @@ def test_linear_shortconv_step(ops, M, D, K, L, bias):
         close(st_f, st_r, 2e-2, f"state against the stand-in, step {step}")
 
 
+@pytest.mark.parametrize("D,K,L,bias,frag", [(2048, 2048, 3, False, True), (96, 96, 4, True, True),
+                                             (48, 120, 2, True, False), (3072, 1024, 3, False, True)])
+@pytest.mark.parametrize("delta_kind", ["none", "bf16", "parts"])
+def test_linear_shortconv_step_on_a_pending_norm(ops, D, K, L, bias, frag, delta_kind):
+    """A single decoded row whose RMSNorm is still pending: norm, in_proj, gates, FIR and state
+    shift in one kernel give what the norm kernel followed by the fused step gives, and the
+    residual comes back in a tensor of its own."""
+    M = 1
+    resid = rand((M, K), F32, 90, 2.0).to(DEV)
+    wn = (1 + rand((K,), F32, 91, 0.1)).to(DEV)
+    delta = {"none": None, "bf16": rand((M, K), BF16, 92), "parts": rand((3, M, K), F32, 92)}[delta_kind]
+    d_dev = None if delta is None else delta.to(DEV)
+    w = rand((3 * D, K), BF16, 93, 0.2).to(DEV)
+    wf = ops.fragment_order(w) if frag else None
+    assert (wf is not None) == (frag and K % 32 == 0)
+    b_in = rand((3 * D,), F32, 94, 0.2).to(DEV) if bias else None
+    b_cv = rand((D,), F32, 95, 0.2).to(DEV) if bias else None
+    taps = rand((D, L), F32, 96, 0.5).to(DEV)
+    state0 = rand((3, D, L - 1), F32, 97).to(DEV)
+    pos0 = torch.tensor([5], dtype=torch.int32, device=DEV)
+    slot = torch.tensor([1], dtype=torch.int32, device=DEV)
+    st_a, st_b = state0.clone(), state0.clone()
+    pend = ops.PendingNorm(resid, d_dev, wn, 1e-5, BF16)
+    got = ops.linear_shortconv_step(pend, w, b_in, taps, b_cv, st_a, pos0, slot, weight_frag=wf)
+    r2 = resid.clone()
+    x = ops.add_rmsnorm(r2, d_dev, wn, 1e-5, BF16)
+    want = ops.linear_shortconv_step(x, w, b_in, taps, b_cv, st_b, pos0, slot, weight_frag=wf)
+    close(got.float(), want.float().cpu().double(), 2 * BF16_ULP, "fused step of the pending norm")
+    close(st_a, st_b.cpu().double(), 2 * BF16_ULP, "state")
+    close(pend.resid_after, r2.cpu().double(), 1e-6, "resid + delta")
+    if delta is not None:
+        assert pend.resid_after.data_ptr() != resid.data_ptr()
+
+
 # ---------------------------------------------------------------------------------------
 def paged_case(seed, dtype, H, G, d, ps, lens_before, lens_new, n_pages=None, shuffle=True):
     """Requests that already hold ``lens_before`` tokens get ``lens_new`` more.  Returns
