@@ -1317,7 +1317,10 @@ static int launch_bf16(const bf16_t* A, const bf16_t* W, const float* bias, TO* 
   if constexpr (EPI != 2) {
     const int n_rows_w = EPI == 1 ? 2 * N : N;
     const long sr_blocks = (long)((n_rows_w + 32 * SR_NWN - 1) / (32 * SR_NWN)) * ksplit;
-    if (force_kernel == 9 || (force_kernel == 0 && M > 16 && M <= 64 && sr_blocks >= 128)) {
+    // (with W in fragment order the kernel for few rows keeps up to 24 rows: gate/up 16.6
+    // against 17.5 us at 24 rows, 15.7 against 17.6 at 17)
+    if (force_kernel == 9 ||
+        (force_kernel == 0 && M > (Wf ? 24 : 16) && M <= 64 && sr_blocks >= 128)) {
       if (launch_shared_rows<TO, EPI>(A, W, bias, C, M, n_rows_w, K, lda, ldc, ksplit, stream, Wf))
         KAPPAI_RETURN_LAUNCH_STATUS();
       if (force_kernel == 9) return (int)hipErrorInvalidValue;
