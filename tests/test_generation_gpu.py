@@ -192,6 +192,45 @@ def test_random_engine_options_give_the_same_tokens(model_dirs):
         assert eng.cache.num_free_pages() == options["num_pages"]
 
 
+def test_fragment_copies_change_no_token(tmp_path):
+    """The copies of the matrices in fragment order are a layout only: a model loaded with and
+    without them generates the same tokens in bfloat16, greedy and sampled, through prompt
+    portions, decode graphs and queued decode steps (sizes at which every matrix has a copy)."""
+    import copy
+    from kappai_amd.config import config_from_dict
+    from kappai_amd.engine import Engine
+    from kappai_amd.parts import linear
+    from kappai_amd.sampling import SamplingParams
+    from kappai_amd.weights import write_random_model
+    raw = {"architectures": ["Lfm2ForCausalLM"], "model_type": "lfm2", "hidden_size": 256,
+           "num_hidden_layers": 4,
+           "layer_types": ["conv", "full_attention", "conv", "full_attention"],
+           "num_attention_heads": 4, "num_key_value_heads": 2, "head_dim": 64,
+           "intermediate_size": 512, "block_auto_adjust_ff_dim": False, "vocab_size": 1024,
+           "norm_eps": 1e-5, "rope_theta": 10000.0, "conv_L_cache": 3, "conv_bias": False,
+           "tie_embedding": True, "max_position_embeddings": 1024}
+    folder = write_random_model(tmp_path / "m", config_from_dict(copy.deepcopy(raw)), seed=11,
+                                std=0.05, norm_jitter=0.05)
+    rng = np.random.default_rng(12)
+    prompts = [[int(t) for t in rng.integers(0, 1024, size=n)] for n in (40, 3, 75, 18, 9)]
+    params = [SamplingParams.greedy(n_predict=24), SamplingParams(seed=3, n_predict=24),
+              SamplingParams.greedy(n_predict=10), SamplingParams(seed=4, top_k=0, n_predict=24),
+              SamplingParams.greedy(n_predict=24)]
+    outs = []
+    assert linear.FRAGMENT_COPIES
+    try:
+        for copies in (True, False):
+            linear.FRAGMENT_COPIES = copies
+            eng = Engine(str(folder), dtype="bfloat16", num_pages=64, max_batch=5, chunk=32,
+                         token_budget=48)
+            frag = [blk.feed_forward.down.weight_frag for blk in eng.model.layers]
+            assert all((f is not None) == copies for f in frag)
+            outs.append(eng.generate(prompts, params))
+    finally:
+        linear.FRAGMENT_COPIES = True
+    assert outs[0] == outs[1]
+
+
 def test_command_line(model_dirs, tmp_path):
     prompt = prompts_for("A", [7], seed=5)[0]
     want, _ = plain_generate(model_dirs["A"], prompt, 6, lambda: S.PlainSampler(1, temperature=0.0))
