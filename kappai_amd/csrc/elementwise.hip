@@ -75,7 +75,7 @@ template <typename T, typename TD>
 __global__ __launch_bounds__(1024) void add_rmsnorm_row_kernel(
     float* __restrict__ resid, const TD* __restrict__ delta, int n_part, size_t pstride,
     const float* __restrict__ w, T* __restrict__ out, const int* __restrict__ rows, int D,
-    float eps, int write_resid) {
+    float eps, int write_resid, int out_frag) {
   __shared__ float red[16];
   const int i = blockIdx.x;
   const int r = rows ? rows[i] : i;
@@ -107,19 +107,24 @@ __global__ __launch_bounds__(1024) void add_rmsnorm_row_kernel(
   if (in) {
 #pragma unroll
     for (int e = 0; e < 8; ++e) w8[e] = v[e] * scale * w8[e];
-    store8(out + (size_t)i * D + j, w8);
+    // out_frag (at most 16 rows, D a multiple of 32): the rows in the order in which the product
+    // kernel for 1 to 16 rows loads its activations, [D / 32][(k % 32) / 8][16 rows][8 values]:
+    // its load instructions then touch whole cache lines of neighbouring rows
+    const size_t at = out_frag ? (size_t)(j / 32) * 512 + ((size_t)((j % 32) / 8) * 16 + i) * 8
+                               : (size_t)i * D + j;
+    store8(out + at, w8);
   }
 }
 
 template <typename T, typename TD>
 static void launch_add_rmsnorm(float* resid, const void* delta, int n_part, size_t pstride,
                                const float* w, void* out, const int* rows, int n_rows, int D,
-                               float eps, int write_resid, hipStream_t stream) {
+                               float eps, int write_resid, int out_frag, hipStream_t stream) {
   if (D % 8 == 0 && D <= 8192 && n_part <= RN_MAX_PART) {
     const int threads = ((D / 8 + WAVE - 1) / WAVE) * WAVE;
     hipLaunchKernelGGL((add_rmsnorm_row_kernel<T, TD>), dim3(n_rows), dim3(threads), 0, stream,
                        resid, (const TD*)delta, n_part, pstride, w, (T*)out, rows, D, eps,
-                       write_resid);
+                       write_resid, out_frag);
     return;
   }
   const int threads = D >= 2048 ? 512 : (D >= 512 ? 256 : (D >= 128 ? 128 : 64));
@@ -132,18 +137,22 @@ static void launch_add_rmsnorm(float* resid, const void* delta, int n_part, size
 extern "C" int kappai_add_rmsnorm(float* resid, const void* delta, int delta_is_f32, int n_part,
                                   long pstride, const float* w, void* out, const int* rows,
                                   int n_rows, int D, float eps, int write_resid, int is_bf16,
-                                  hipStream_t stream) {
+                                  int out_frag, hipStream_t stream) {
   if (n_rows <= 0) return 0;
   if (n_part < 1 || (n_part > 1 && !delta_is_f32)) return (int)hipErrorInvalidValue;
+  // rows in fragment order: bfloat16, at most 16 of them, in the kernel that keeps a row in
+  // registers; out holds 16 x D values
+  if (out_frag && (!is_bf16 || n_rows > 16 || (D % 32) || D > 8192 || n_part > RN_MAX_PART))
+    return (int)hipErrorInvalidValue;
   if (!is_bf16)
     launch_add_rmsnorm<float, float>(resid, delta, n_part, (size_t)pstride, w, out, rows, n_rows,
-                                     D, eps, write_resid, stream);
+                                     D, eps, write_resid, out_frag, stream);
   else if (delta_is_f32)
     launch_add_rmsnorm<bf16_t, float>(resid, delta, n_part, (size_t)pstride, w, out, rows, n_rows,
-                                      D, eps, write_resid, stream);
+                                      D, eps, write_resid, out_frag, stream);
   else
     launch_add_rmsnorm<bf16_t, bf16_t>(resid, delta, n_part, (size_t)pstride, w, out, rows, n_rows,
-                                       D, eps, write_resid, stream);
+                                       D, eps, write_resid, out_frag, stream);
   KAPPAI_RETURN_LAUNCH_STATUS();
 }
 

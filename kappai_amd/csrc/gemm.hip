@@ -773,7 +773,7 @@ template <typename TO, int MT, int NW, int EPI, int NT, bool PRO = false>
 __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny_kernel(
     const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, const float* __restrict__ bias,
     TO* __restrict__ C, int M, int N, int K, int lda, int ldc, ConvStep cs, NormIn nin,
-    int w_frag) {
+    int w_frag, int a_frag) {
   static_assert(NT == 1 || EPI == 0, "several column tiles a wave: plain products only");
   static_assert(!PRO || (MT == 1 && NT == 1), "normalised rows: one row tile");
   // row groups of W a block streams: gate/up, the three conv gates, or NT column tiles
@@ -812,7 +812,10 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny_kernel(
 #pragma unroll
   for (int t = 0; t < MT; ++t) {
     const int gm = t * 16 + col;
-    arow[t] = A + (size_t)(gm < M ? gm : 0) * lda + kg;
+    // a_frag (at most 16 rows): the rows lie in fragment order too, [K / 32][(k % 32) / 8][16 rows]
+    // [8 values] (add_rmsnorm writes them so): a load then takes whole lines of neighbouring rows
+    arow[t] = a_frag ? A + ((size_t)(kg / 8) * 16 + (gm < M ? gm : 0)) * 8
+                     : A + (size_t)(gm < M ? gm : 0) * lda + kg;
   }
   __shared__ __attribute__((aligned(16))) bf16_t xs[PRO ? NORM_ROWS : 1][PRO ? NORM_MAX_K : 8];
   __shared__ float red16[PRO ? 16 : 1];
@@ -891,7 +894,7 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny_kernel(
           av[u][t] = (kin && col < M) ? *reinterpret_cast<const u32x4_t*>(&xs[col % NORM_ROWS][gk + kg])
                                       : zero;
         else
-          av[u][t] = (kin && t * 16 + col < M) ? load16(arow[t] + gk) : zero;
+          av[u][t] = (kin && t * 16 + col < M) ? load16(arow[t] + (size_t)gk * (a_frag ? 16 : 1)) : zero;
       }
     }
   };
@@ -930,7 +933,7 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny_kernel(
                          : zero;
 #pragma unroll
         for (int t = 0; t < MT; ++t)
-          av[u][t] = (kin && t * 16 + col < M) ? load16(arow[t] + gk) : zero;
+          av[u][t] = (kin && t * 16 + col < M) ? load16(arow[t] + (size_t)gk * (a_frag ? 16 : 1)) : zero;
       }
       products(wv, av);
     }
@@ -1017,7 +1020,8 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny_kernel(
 template <typename TO, int MT, int NW, int EPI, int NT = 1>
 static void launch_skinny(const bf16_t* A, const bf16_t* W, const float* bias, TO* C, int M, int N,
                           int K, int lda, int ldc, int ksplit, ConvStep cs, hipStream_t stream,
-                          const NormIn* nin = nullptr, const bf16_t* Wf = nullptr) {
+                          const NormIn* nin = nullptr, const bf16_t* Wf = nullptr,
+                          int a_frag = 0) {
   // Wf: the copy of W in fragment order (see the kernel), or null
   const int w_frag = Wf != nullptr;
   if (Wf) W = Wf;
@@ -1026,12 +1030,12 @@ static void launch_skinny(const bf16_t* A, const bf16_t* W, const float* bias, T
     if (nin) {
       hipLaunchKernelGGL((gemm_bf16_skinny_kernel<TO, MT, NW, EPI, NT, true>), grid,
                          dim3(NW * WAVE), 0, stream, A, W, bias, C, M, N, K, lda, ldc, cs, *nin,
-                         w_frag);
+                         w_frag, 0);
       return;
     }
   }
   hipLaunchKernelGGL((gemm_bf16_skinny_kernel<TO, MT, NW, EPI, NT>), grid, dim3(NW * WAVE), 0,
-                     stream, A, W, bias, C, M, N, K, lda, ldc, cs, NormIn{}, w_frag);
+                     stream, A, W, bias, C, M, N, K, lda, ldc, cs, NormIn{}, w_frag, a_frag);
 }
 
 // more waves a block when there are few blocks, so that about 2048 waves or more stream W
@@ -1039,13 +1043,13 @@ template <typename TO, int MT, int EPI>
 static void launch_skinny_mt(const bf16_t* A, const bf16_t* W, const float* bias, TO* C, int M,
                              int N, int K, int lda, int ldc, int ksplit, ConvStep cs,
                              hipStream_t stream, const NormIn* nin = nullptr,
-                             const bf16_t* Wf = nullptr) {
+                             const bf16_t* Wf = nullptr, int a_frag = 0) {
   // several row tiles and a plain product: a wave takes two column tiles for every fragment
   // of A it loads, which halves the reads of A (every block reads all of it)
   if constexpr (EPI == 0 && MT >= 2) {
     if (N >= 64) {
       launch_skinny<TO, MT, 4, EPI, 2>(A, W, bias, C, M, N, K, lda, ldc, ksplit, cs, stream,
-                                       nullptr, Wf);
+                                       nullptr, Wf, a_frag);
       return;
     }
   }
@@ -1056,7 +1060,7 @@ static void launch_skinny_mt(const bf16_t* A, const bf16_t* W, const float* bias
   if constexpr (EPI == 0 && MT == 1) {
     if (!nin && M >= (Wf ? 12 : 8) && (long)(N / 64) * ksplit >= 512) {
       launch_skinny<TO, MT, 4, EPI, 4>(A, W, bias, C, M, N, K, lda, ldc, ksplit, cs, stream,
-                                       nullptr, Wf);
+                                       nullptr, Wf, a_frag);
       return;
     }
   }
@@ -1065,13 +1069,13 @@ static void launch_skinny_mt(const bf16_t* A, const bf16_t* W, const float* bias
   constexpr int NG = EPI == 1 ? 2 : (EPI == 2 ? 3 : (EPI == 3 ? 2 : 1));
   constexpr int MAXW = 48 / (MT * NG);                    // 1 KB of LDS a wave, group and row tile
   if (blocks * 4 >= 2048 || kb <= 512 || MAXW < 8)
-    launch_skinny<TO, MT, 4, EPI>(A, W, bias, C, M, N, K, lda, ldc, ksplit, cs, stream, nin, Wf);
+    launch_skinny<TO, MT, 4, EPI>(A, W, bias, C, M, N, K, lda, ldc, ksplit, cs, stream, nin, Wf, a_frag);
   else if (blocks * 8 >= 2048 || kb <= 1024 || MAXW < 16)
     launch_skinny<TO, MT, (MAXW >= 8 ? 8 : 4), EPI>(A, W, bias, C, M, N, K, lda, ldc, ksplit, cs,
-                                                    stream, nin, Wf);
+                                                    stream, nin, Wf, a_frag);
   else
     launch_skinny<TO, MT, (MAXW >= 16 ? 16 : 4), EPI>(A, W, bias, C, M, N, K, lda, ldc, ksplit, cs,
-                                                      stream, nin, Wf);
+                                                      stream, nin, Wf, a_frag);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -1305,7 +1309,9 @@ static bool launch_shared_rows(const bf16_t* A, const bf16_t* W, const float* bi
 template <typename TO, int EPI>
 static int launch_bf16(const bf16_t* A, const bf16_t* W, const float* bias, TO* C, int M, int N,
                        int K, int lda, int ldc, int force_kernel, int ksplit, hipStream_t stream,
-                       ConvStep cs = ConvStep{}, const bf16_t* Wf = nullptr) {
+                       ConvStep cs = ConvStep{}, const bf16_t* Wf = nullptr, int a_frag = 0) {
+  // a_frag: the rows of A lie in fragment order, which only the kernel for 1 to 16 rows reads
+  if (a_frag && (M > 16 || force_kernel == 1 || force_kernel >= 3)) return (int)hipErrorInvalidValue;
   // Wf: W once more in fragment order, for the kernels of 1 to 64 rows (see the first of them);
   // the others read W
   // N counts output columns; with the SwiGLU epilogue W has 2N rows
@@ -1333,7 +1339,7 @@ static int launch_bf16(const bf16_t* A, const bf16_t* W, const float* bias, TO* 
     switch (mt) {
       case 1:
         launch_skinny_mt<TO, 1, EPI>(A, W, bias, C, M, N, K, lda, ldc, ksplit, cs, stream, nullptr,
-                                     Wf);
+                                     Wf, a_frag);
         break;
       case 2:
         launch_skinny_mt<TO, 2, EPI>(A, W, bias, C, M, N, K, lda, ldc, ksplit, cs, stream, nullptr,
@@ -1369,32 +1375,33 @@ static bool frag_ok(const void* W_frag, int rows, int K) {
 
 extern "C" int kappai_gemm_bf16(const void* A, const void* W, const void* W_frag, const float* bias,
                                 void* C, int M, int N, int K, int lda, int ldc, int out_is_f32,
-                                int force_kernel, int ksplit, hipStream_t stream) {
+                                int force_kernel, int ksplit, int a_frag, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
   if ((K % 8) || (lda % 8) || ksplit < 1 || ksplit > 64) return (int)hipErrorInvalidValue;
-  if (!frag_ok(W_frag, N, K)) return (int)hipErrorInvalidValue;
+  if (!frag_ok(W_frag, N, K) || (a_frag && (K % 32))) return (int)hipErrorInvalidValue;
   if (force_kernel == 2 && M > 64) return (int)hipErrorInvalidValue;
   if (ksplit > 1 && !out_is_f32) return (int)hipErrorInvalidValue;
   if (out_is_f32)
     return launch_bf16<float, 0>((const bf16_t*)A, (const bf16_t*)W, bias, (float*)C, M, N, K, lda,
                                  ldc, force_kernel, ksplit, stream, ConvStep{},
-                                 (const bf16_t*)W_frag);
+                                 (const bf16_t*)W_frag, a_frag);
   return launch_bf16<bf16_t, 0>((const bf16_t*)A, (const bf16_t*)W, bias, (bf16_t*)C, M, N, K, lda,
-                                ldc, force_kernel, 1, stream, ConvStep{}, (const bf16_t*)W_frag);
+                                ldc, force_kernel, 1, stream, ConvStep{}, (const bf16_t*)W_frag,
+                                a_frag);
 }
 
 // C[M, F] = silu(A Wg^T) * (A Wu^T) with W = gate and up rows interleaved in groups of 16,
 // [2F, K]; F must be a multiple of 16.
 extern "C" int kappai_gemm_bf16_swiglu(const void* A, const void* W, const void* W_frag, void* C,
                                        int M, int F, int K, int lda, int ldc, int force_kernel,
-                                       hipStream_t stream) {
+                                       int a_frag, hipStream_t stream) {
   if (M <= 0 || F <= 0) return 0;
   if ((K % 8) || (lda % 8) || (F % 16)) return (int)hipErrorInvalidValue;
   if (force_kernel == 2 && M > 64) return (int)hipErrorInvalidValue;
-  if (!frag_ok(W_frag, 2 * F, K)) return (int)hipErrorInvalidValue;
+  if (!frag_ok(W_frag, 2 * F, K) || (a_frag && (K % 32))) return (int)hipErrorInvalidValue;
   return launch_bf16<bf16_t, 1>((const bf16_t*)A, (const bf16_t*)W, nullptr, (bf16_t*)C, M, F, K,
                                 lda, ldc, force_kernel, 1, stream, ConvStep{},
-                                (const bf16_t*)W_frag);
+                                (const bf16_t*)W_frag, a_frag);
 }
 
 // Conv layer decode step in one kernel: C[M, D] = Cgate * conv(Bgate * x | state) from A [M, K]
@@ -1404,10 +1411,12 @@ extern "C" int kappai_gemm_bf16_shortconv_step(const void* A, const void* W, con
                                                void* C, int M, int D, int K, int lda,
                                                const float* taps, const float* conv_bias,
                                                float* state, const int* seg_pos0,
-                                               const int* seg_slot, int L, hipStream_t stream) {
+                                               const int* seg_slot, int L, int a_frag,
+                                               hipStream_t stream) {
   if (M <= 0 || D <= 0) return 0;
   if ((K % 8) || (lda % 8) || (D % 16) || M > 64 || L < 2) return (int)hipErrorInvalidValue;
-  if (!frag_ok(W_frag, 3 * D, K)) return (int)hipErrorInvalidValue;
+  if (!frag_ok(W_frag, 3 * D, K) || (a_frag && ((K % 32) || M > 16)))
+    return (int)hipErrorInvalidValue;
   const bf16_t* wf = (const bf16_t*)W_frag;
   ConvStep cs{taps, conv_bias, state, seg_pos0, seg_slot, L};
   if (D / 16 < 256) {
@@ -1417,7 +1426,8 @@ extern "C" int kappai_gemm_bf16_shortconv_step(const void* A, const void* W, con
     bf16_t* c = (bf16_t*)C;
     switch ((M + 15) / 16) {
       case 1:
-        launch_skinny_mt<bf16_t, 1, 3>(a, w, bias, c, M, D, K, lda, D, 1, cs, stream, nullptr, wf);
+        launch_skinny_mt<bf16_t, 1, 3>(a, w, bias, c, M, D, K, lda, D, 1, cs, stream, nullptr, wf,
+                                       a_frag);
         break;
       case 2:
         launch_skinny_mt<bf16_t, 2, 3>(a, w, bias, c, M, D, K, lda, D, 1, cs, stream, nullptr, wf);
@@ -1432,7 +1442,7 @@ extern "C" int kappai_gemm_bf16_shortconv_step(const void* A, const void* W, con
     KAPPAI_RETURN_LAUNCH_STATUS();
   }
   return launch_bf16<bf16_t, 2>((const bf16_t*)A, (const bf16_t*)W, bias, (bf16_t*)C, M, D, K, lda,
-                                D, 2, 1, stream, cs, wf);
+                                D, 2, 1, stream, cs, wf, a_frag);
 }
 
 // The same products for at most NORM_ROWS rows that are still to be made: A = RMSNorm(resid +

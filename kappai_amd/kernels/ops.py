@@ -78,11 +78,13 @@ def embed_rows(ids: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
 
 def add_rmsnorm(resid: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Tensor,
                 eps: float, out_dtype, rows: Optional[torch.Tensor] = None,
-                write_resid: bool = True) -> torch.Tensor:
+                write_resid: bool = True, fragment: bool = False):
     """RMSNorm of ``resid (+ delta)``; with ``write_resid`` the sum replaces ``resid``.
     ``delta`` is [T, D] in the compute dtype, or float32 partial sums [S, T, D] (a product
     split over K) that are added in order.  ``rows`` (int32) picks the rows to normalise; the
-    result then has one row per entry."""
+    result then has one row per entry.  ``fragment`` (at most 16 rows of bfloat16, a width that is
+    a multiple of 32): the rows come back as ``FragmentRows``, in the order in which the product
+    kernel for 1 to 16 rows loads them."""
     _gpu("resid", resid, F32)
     _gpu("weight", weight, F32)
     _need(resid.dim() == 2 and weight.shape == (resid.shape[1],),
@@ -106,12 +108,41 @@ def add_rmsnorm(resid: torch.Tensor, delta: Optional[torch.Tensor], weight: torc
               "add_rmsnorm: a row selection cannot update the residual")
         n = rows.shape[0]
     D = resid.shape[1]
-    out = torch.empty((n, D), dtype=out_dtype, device=resid.device)
+    if fragment:
+        _need(FragmentRows.fits(n, D, out_dtype) and n_part <= 8,
+              "add_rmsnorm: rows in fragment order need bfloat16, at most 16 rows and a width "
+              "that is a multiple of 32 (up to 8192)")
+    out = torch.empty((16 if fragment else n, D), dtype=out_dtype, device=resid.device)
     check(library("elementwise").kappai_add_rmsnorm(
         _ptr(resid), _ptr(delta), _c_int(delta_f32), _c_int(n_part), _c_long(pstride), _ptr(weight),
         _ptr(out), _ptr(rows), _c_int(n), _c_int(D), _c_float(eps),
-        _c_int(1 if write_resid else 0), _c_int(isb), _stream()), "add_rmsnorm")
-    return out
+        _c_int(1 if write_resid else 0), _c_int(isb), _c_int(1 if fragment else 0), _stream()),
+        "add_rmsnorm")
+    return FragmentRows(out, n, resid) if fragment else out
+
+
+class FragmentRows:
+    """At most 16 normalised rows [n, D] of a decode step, stored in the order in which the
+    product kernel for 1 to 16 rows loads its activations ([D / 32][(k % 32) / 8][16 rows][8
+    values], see ``fragment_order`` for the matrices): a load instruction of that kernel then
+    touches whole cache lines of neighbouring rows instead of half a line of every row.
+    ``linear``, ``linear_swiglu`` and ``linear_shortconv_step`` take it in place of the rows;
+    ``materialize`` gives the rows as an ordinary tensor.  ``resid_after`` is the residual the
+    norm has updated (the interface of ``PendingNorm``, so that a part takes either)."""
+
+    def __init__(self, data: torch.Tensor, n_rows: int, resid: torch.Tensor):
+        self.data, self.resid_after = data, resid
+        self.shape = torch.Size((n_rows, data.shape[1]))
+        self.device, self.dtype = data.device, data.dtype
+
+    @staticmethod
+    def fits(n_rows: int, width: int, out_dtype) -> bool:
+        return out_dtype == BF16 and 1 <= n_rows <= 16 and width % 32 == 0 and width <= 8192
+
+    def materialize(self) -> torch.Tensor:
+        n, D = self.shape
+        return (self.data.view(D // 32, 4, 16, 8).permute(2, 0, 1, 3).reshape(16, D)[:n]
+                .contiguous())
 
 
 NORM_FUSE_MAX_ROWS = 1        # rows a product kernel normalises by itself
@@ -299,12 +330,21 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] =
             x = x.materialize()
         else:
             return _linear_normed(x, weight, bias, out_dtype, partial_sums, split_k, weight_frag)
+    a_frag = 0
+    if isinstance(x, FragmentRows):
+        if (weight.dtype != BF16 or force_kernel not in (0, 2) or weight.dim() != 2
+                or weight.shape[1] != x.shape[1] or weight.data_ptr() % 16):
+            x = x.materialize()
+        else:
+            a_frag, n_frag, x = 1, x.shape[0], x.data     # 16 row slots, n_frag of them filled
     _gpu("x", x, (F32, BF16), contiguous=False)
     _gpu("weight", weight, (F32, BF16))
     _need(x.dim() == 2 and weight.dim() == 2 and x.shape[1] == weight.shape[1],
           lambda: f"linear: x {tuple(x.shape)} does not meet weight {tuple(weight.shape)}")
     _need(x.stride(1) == 1 or x.shape[1] == 1, "linear: x must have unit stride along K")
     M, K = x.shape
+    if a_frag:
+        M = n_frag
     N = weight.shape[0]
     out_dtype = out_dtype or x.dtype
     if bias is not None:
@@ -343,7 +383,7 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] =
         _ptr(xb), _ptr(weight), _frag(weight, weight_frag), _ptr(bias), _ptr(out), _c_int(M),
         _c_int(N), _c_int(K),
         _c_int(lda), _c_int(N), _c_int(out_is_f32), _c_int(force_kernel), _c_int(ksplit),
-        _stream()), "gemm_bf16")
+        _c_int(a_frag), _stream()), "gemm_bf16")
     return out
 
 
@@ -405,6 +445,12 @@ def linear_swiglu(x: torch.Tensor, weight: torch.Tensor, force_kernel: int = 0,
                 _c_int(F), _c_int(K),
                 _c_int(F), _stream()), "gemm_bf16_swiglu_normed")
             return out
+    a_frag, n_frag = 0, 0
+    if isinstance(x, FragmentRows):
+        if force_kernel not in (0, 2) or weight.dim() != 2 or weight.shape[1] != x.shape[1]:
+            x = x.materialize()
+        else:
+            a_frag, n_frag, x = 1, x.shape[0], x.data
     _gpu("x", x, BF16, contiguous=False)
     _gpu("weight", weight, BF16)
     _need(x.dim() == 2 and weight.dim() == 2 and x.shape[1] == weight.shape[1]
@@ -412,6 +458,8 @@ def linear_swiglu(x: torch.Tensor, weight: torch.Tensor, force_kernel: int = 0,
           lambda: f"linear_swiglu: x {tuple(x.shape)}, weight {tuple(weight.shape)}")
     _need(x.stride(1) == 1 or x.shape[1] == 1, "linear_swiglu: x must have unit stride along K")
     M, K = x.shape
+    if a_frag:
+        M = n_frag
     F = weight.shape[0] // 2
     lda = x.stride(0) if M > 1 else K
     _need(K % 8 == 0 and lda % 8 == 0 and x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0,
@@ -421,7 +469,7 @@ def linear_swiglu(x: torch.Tensor, weight: torch.Tensor, force_kernel: int = 0,
     check(library("gemm").kappai_gemm_bf16_swiglu(
         _ptr(x), _ptr(weight), _frag(weight, weight_frag), _ptr(out), _c_int(M), _c_int(F), _c_int(K),
         _c_int(lda), _c_int(F),
-        _c_int(force_kernel), _stream()), "gemm_bf16_swiglu")
+        _c_int(force_kernel), _c_int(a_frag), _stream()), "gemm_bf16_swiglu")
     return out
 
 
@@ -434,13 +482,20 @@ def linear_shortconv_step(x: torch.Tensor, in_proj: torch.Tensor, in_bias: Optio
     segment: ``proj = x in_proj^T (+ bias)`` cut into (B | C | x), ``C * conv(B * x)`` with the
     rows' state slots read and shifted.  bfloat16, at most 64 rows, width a multiple of 16.
     Equals ``shortconv(linear(x, in_proj, in_bias), ...)``.  ``x`` may be a ``PendingNorm``
-    (widths below 4096): the kernel then makes the normalised row itself as well."""
+    (widths below 4096): the kernel then makes the normalised row itself as well; or
+    ``FragmentRows``."""
     pending = x if isinstance(x, PendingNorm) else None
     if pending is not None and not (in_proj.dtype == BF16 and in_proj.dim() == 2
                                     and taps.dim() == 2 and taps.shape[0] // 16 < 256
                                     and in_proj.shape[1] == x.shape[1]
                                     and in_proj.data_ptr() % 16 == 0):
         x, pending = x.materialize(), None
+    a_frag, n_frag = 0, 0
+    if isinstance(x, FragmentRows):
+        if in_proj.dim() != 2 or in_proj.shape[1] != x.shape[1]:
+            x = x.materialize()
+        else:
+            a_frag, n_frag, x = 1, x.shape[0], x.data
     if pending is None:
         _gpu("x", x, BF16, contiguous=False)
     _gpu("in_proj", in_proj, BF16)
@@ -449,6 +504,8 @@ def linear_shortconv_step(x: torch.Tensor, in_proj: torch.Tensor, in_bias: Optio
     _gpu("seg_pos0", seg_pos0, I32)
     _gpu("seg_slot", seg_slot, I32)
     M, K = x.shape
+    if a_frag:
+        M = n_frag
     D, L = taps.shape
     _need(in_proj.shape == (3 * D, K), lambda: f"in_proj {tuple(in_proj.shape)} for D={D}, K={K}")
     _need(M <= 64 and D % 16 == 0, "linear_shortconv_step: at most 64 rows, width a multiple of 16")
@@ -476,7 +533,7 @@ def linear_shortconv_step(x: torch.Tensor, in_proj: torch.Tensor, in_bias: Optio
         _ptr(x), _ptr(in_proj), _frag(in_proj, weight_frag), _ptr(in_bias), _ptr(out), _c_int(M),
         _c_int(D), _c_int(K),
         _c_int(lda), _ptr(taps), _ptr(conv_bias), _ptr(state), _ptr(seg_pos0), _ptr(seg_slot),
-        _c_int(L), _stream()), "gemm_bf16_shortconv_step")
+        _c_int(L), _c_int(a_frag), _stream()), "gemm_bf16_shortconv_step")
     return out
 
 

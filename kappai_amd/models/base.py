@@ -122,5 +122,9 @@ class Model:
             h = block.forward(h, batch, view, shared_cache=call.reads_cache_of is not None)
         if batch.n_logit_rows == 0:
             return torch.empty((0, self.vocab_size), dtype=torch.float32, device=x.device)
-        xb = self.final_norm.add_norm(h.resid, h.delta, rows=batch.logit_rows)
+        if (getattr(self.final_norm, "can_defer", False)
+                and getattr(self.head, "takes_pending_norm", False)):
+            xb = self.final_norm.add_norm(h.resid, h.delta, rows=batch.logit_rows, defer=True)
+        else:
+            xb = self.final_norm.add_norm(h.resid, h.delta, rows=batch.logit_rows)
         return self.head.forward(xb)

@@ -49,7 +49,9 @@ class OutputHead(Part):
         else:
             self.linear.bind(tensors)
 
-    def forward(self, x: torch.Tensor) -> torch.Tensor:
+    takes_pending_norm = True      # a plain product: it takes what ops.linear takes
+
+    def forward(self, x) -> torch.Tensor:
         return self.linear.forward(x, out_dtype=torch.float32)
 
     def weight_bytes(self) -> int:

@@ -12,8 +12,16 @@ from ..weights.spec import INIT_ONES, VECTOR, TensorSpec
 from .base import Norm, register_part
 
 
+# Decode steps of 8 to 16 rows hand their normalised rows on in fragment order (a step of the
+# 1.2B shape: 1.06 against 1.08 ms at 16 rows, 0.994 against 1.000 at 12, even at 8; with
+# fewer rows the ordinary order is as fast or faster).
+FRAGMENT_ROWS = True
+FRAGMENT_ROWS_MIN = 8
+
+
 class RMSNorm(Norm):
-    can_defer = True      # add_norm(..., defer=True) may hand out an ops.PendingNorm
+    can_defer = True      # add_norm(..., defer=True) may hand out an ops.PendingNorm or
+                          # ops.FragmentRows in place of a tensor
 
     def __init__(self, name: str, width: int, eps: float, dtype: torch.dtype):
         self.name, self.width, self.eps, self.dtype = name, width, float(eps), dtype
@@ -26,12 +34,17 @@ class RMSNorm(Norm):
         self.weight = tensors[self.name + ".weight"].to(torch.float32).contiguous()
 
     def add_norm(self, resid, delta, rows=None, defer: bool = False):
-        """``defer``: the caller's next part takes an ``ops.PendingNorm`` in place of the rows
-        (a step with very few rows: the product kernel then makes them itself)."""
+        """``defer``: the caller's next part takes what the product kernels take in place of
+        the rows: an ``ops.PendingNorm`` (one row: the product kernel makes it itself) or
+        ``ops.FragmentRows`` (8 to 16 rows, made here in the order the product loads them)."""
         if defer and rows is None and ops.PendingNorm.fits(resid, delta, self.dtype):
             return ops.PendingNorm(resid, delta, self.weight, self.eps, self.dtype)
+        n = resid.shape[0] if rows is None else rows.shape[0]
+        fragment = (defer and FRAGMENT_ROWS and resid.is_cuda and n >= FRAGMENT_ROWS_MIN
+                    and ops.FragmentRows.fits(n, self.width, self.dtype)
+                    and (delta is None or delta.dim() == 2 or delta.shape[0] <= 8))
         return ops.add_rmsnorm(resid, delta, self.weight, self.eps, self.dtype, rows=rows,
-                               write_resid=rows is None)
+                               write_resid=rows is None, fragment=fragment)
 
     def weight_bytes(self) -> int:
         return self.width * 4

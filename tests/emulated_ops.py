@@ -16,7 +16,9 @@ def embed_rows(ids, table):
     return table[ids.long()].to(F32)
 
 
-def add_rmsnorm(resid, delta, weight, eps, out_dtype, rows=None, write_resid=True):
+def add_rmsnorm(resid, delta, weight, eps, out_dtype, rows=None, write_resid=True,
+                fragment=False):
+    assert not fragment, "rows in fragment order are made on the GPU only"
     x = resid
     if delta is not None:
         parts = delta if delta.dim() == 3 else delta[None]

@@ -193,13 +193,14 @@ def test_random_engine_options_give_the_same_tokens(model_dirs):
 
 
 def test_fragment_copies_change_no_token(tmp_path):
-    """The copies of the matrices in fragment order are a layout only: a model loaded with and
-    without them generates the same tokens in bfloat16, greedy and sampled, through prompt
-    portions, decode graphs and queued decode steps (sizes at which every matrix has a copy)."""
+    """The copies of the matrices in fragment order, and the normalised rows of a decode step in
+    that order, are layouts only: a model with and without them generates the same tokens in
+    bfloat16, greedy and sampled, through prompt portions, decode graphs and queued decode steps
+    (sizes at which every matrix has a copy)."""
     import copy
     from kappai_amd.config import config_from_dict
     from kappai_amd.engine import Engine
-    from kappai_amd.parts import linear
+    from kappai_amd.parts import linear, norm
     from kappai_amd.sampling import SamplingParams
     from kappai_amd.weights import write_random_model
     raw = {"architectures": ["Lfm2ForCausalLM"], "model_type": "lfm2", "hidden_size": 256,
@@ -212,23 +213,25 @@ def test_fragment_copies_change_no_token(tmp_path):
     folder = write_random_model(tmp_path / "m", config_from_dict(copy.deepcopy(raw)), seed=11,
                                 std=0.05, norm_jitter=0.05)
     rng = np.random.default_rng(12)
-    prompts = [[int(t) for t in rng.integers(0, 1024, size=n)] for n in (40, 3, 75, 18, 9)]
+    prompts = [[int(t) for t in rng.integers(0, 1024, size=n)]
+               for n in (40, 3, 75, 18, 9, 5, 31, 12, 22, 7)]
     params = [SamplingParams.greedy(n_predict=24), SamplingParams(seed=3, n_predict=24),
               SamplingParams.greedy(n_predict=10), SamplingParams(seed=4, top_k=0, n_predict=24),
-              SamplingParams.greedy(n_predict=24)]
+              SamplingParams.greedy(n_predict=24)] * 2
+    assert len(prompts) >= norm.FRAGMENT_ROWS_MIN      # decode steps with rows enough for the order
     outs = []
-    assert linear.FRAGMENT_COPIES
+    assert linear.FRAGMENT_COPIES and norm.FRAGMENT_ROWS
     try:
-        for copies in (True, False):
-            linear.FRAGMENT_COPIES = copies
-            eng = Engine(str(folder), dtype="bfloat16", num_pages=64, max_batch=5, chunk=32,
+        for copies, rows in ((True, True), (False, True), (True, False), (False, False)):
+            linear.FRAGMENT_COPIES, norm.FRAGMENT_ROWS = copies, rows
+            eng = Engine(str(folder), dtype="bfloat16", num_pages=128, max_batch=10, chunk=32,
                          token_budget=48)
             frag = [blk.feed_forward.down.weight_frag for blk in eng.model.layers]
             assert all((f is not None) == copies for f in frag)
             outs.append(eng.generate(prompts, params))
     finally:
-        linear.FRAGMENT_COPIES = True
-    assert outs[0] == outs[1]
+        linear.FRAGMENT_COPIES, norm.FRAGMENT_ROWS = True, True
+    assert outs[0] == outs[1] == outs[2] == outs[3]
 
 
 def test_command_line(model_dirs, tmp_path):

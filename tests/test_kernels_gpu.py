@@ -303,6 +303,76 @@ def test_products_read_the_fragment_order_copy(ops, M, N, K):
         assert torch.equal(outs[0], outs[1]) and torch.equal(states[0], states[1])
 
 
+@pytest.mark.parametrize("M", [1, 2, 5, 8, 13, 16])
+@pytest.mark.parametrize("N,K", [(16, 32), (48, 96), (2048, 2048), (1008, 4128), (6144, 1024),
+                                 (12288, 4096)])
+def test_products_read_rows_in_fragment_order(ops, M, N, K):
+    """The norm can write up to 16 rows in the order in which the kernel for 1 to 16 rows loads
+    them: the same values at other places, and every product that takes them (plain, with bias,
+    partial sums, SwiGLU, the fused conv step, with and without the matrix's fragment-order copy)
+    gives bit for bit what it gives from ordinary rows."""
+    resid0 = rand((M + 3, K), F32, 70, 2.0).to(DEV)
+    wn = (1 + rand((K,), F32, 71, 0.1)).to(DEV)
+    w, b = rand((N, K), BF16, 72, 0.1).to(DEV), rand((N,), F32, 73).to(DEV)
+    wf = ops.fragment_order(w)
+    sel = torch.tensor([(3 * i + 1) % (M + 3) for i in range(M)], dtype=torch.int32, device=DEV)
+    for delta, rows in ((None, sel), (rand((M + 3, K), BF16, 74).to(DEV), None),
+                        (rand((3, M + 3, K), F32, 75).to(DEV), None)):
+        r1, r2 = resid0.clone(), resid0.clone()
+        n = M if rows is not None else M + 3
+        if n > 16:
+            continue
+        x = ops.add_rmsnorm(r1, delta, wn, 1e-5, BF16, rows=rows, write_resid=rows is None)
+        fr = ops.add_rmsnorm(r2, delta, wn, 1e-5, BF16, rows=rows, write_resid=rows is None,
+                             fragment=True)
+        assert isinstance(fr, ops.FragmentRows) and fr.shape == x.shape and fr.dtype == BF16
+        assert fr.resid_after is r2 and torch.equal(r1, r2)
+        assert torch.equal(fr.materialize(), x)
+        # element (i, k) lies at its place in the piece of 16 rows x 32 of K
+        i, k = n - 1, K - 5
+        assert fr.data.reshape(-1)[(k // 32) * 512 + ((k % 32) // 8 * 16 + i) * 8 + k % 8] == x[i, k]
+        for frag in (wf, None):
+            for bias in (None, b):
+                for out_dtype in (BF16, F32):
+                    assert torch.equal(
+                        ops.linear(fr, w, bias, out_dtype=out_dtype, weight_frag=frag),
+                        ops.linear(x, w, bias, out_dtype=out_dtype, weight_frag=frag))
+            if K % 64 == 0:
+                for S in (2, 4) if K % 128 == 0 else (2,):
+                    assert torch.equal(
+                        ops.linear(fr, w, partial_sums=True, split_k=S, weight_frag=frag),
+                        ops.linear(x, w, partial_sums=True, split_k=S, weight_frag=frag))
+            if N % 32 == 0:
+                assert torch.equal(ops.linear_swiglu(fr, w, weight_frag=frag),
+                                   ops.linear_swiglu(x, w, weight_frag=frag))
+            if N % 48 == 0:
+                D, L = N // 3, 3
+                taps = rand((D, L), F32, 76, 0.5).to(DEV)
+                state = rand((n + 1, D, L - 1), F32, 77).to(DEV)
+                pos0 = torch.ones(n, dtype=torch.int32, device=DEV)
+                slot = torch.arange(n, dtype=torch.int32, device=DEV)
+                outs, states = [], []
+                for rows_in in (fr, x):
+                    st = state.clone()
+                    outs.append(ops.linear_shortconv_step(rows_in, w, b, taps, None, st, pos0, slot,
+                                                          weight_frag=frag))
+                    states.append(st)
+                assert torch.equal(outs[0], outs[1]) and torch.equal(states[0], states[1])
+        # a product that another kernel is asked for takes the rows as a tensor
+        assert torch.equal(ops.linear(fr, w, b, force_kernel=1), ops.linear(x, w, b, force_kernel=1))
+
+
+def test_rows_in_fragment_order_need_their_sizes(ops):
+    wn = torch.ones(64, device=DEV)
+    with pytest.raises(ValueError):                                       # 17 rows
+        ops.add_rmsnorm(rand((17, 64), F32, 78).to(DEV), None, wn, 1e-5, BF16, fragment=True)
+    with pytest.raises(ValueError):                                       # float32 rows
+        ops.add_rmsnorm(rand((4, 64), F32, 78).to(DEV), None, wn, 1e-5, F32, fragment=True)
+    with pytest.raises(ValueError):                                       # width 40
+        ops.add_rmsnorm(rand((4, 40), F32, 78).to(DEV), None, torch.ones(40, device=DEV), 1e-5,
+                        BF16, fragment=True)
+
+
 def test_fragment_order_needs_whole_pieces(ops):
     assert ops.fragment_order(rand((40, 64), BF16, 68)) is None          # rows
     assert ops.fragment_order(rand((48, 72), BF16, 68)) is None          # K
