@@ -30,18 +30,28 @@ class KeyReader:
         self.where = where
 
     def _get(self, key, default):
-        if key in self.raw and self.raw[key] is not None:
-            return self.raw[key]
+        """``key``: a name, or several names for the same thing of which the first present one
+        counts (checkpoints of one architecture written by different versions of its tools)."""
+        names = (key,) if isinstance(key, str) else tuple(key)
+        for name in names:
+            if name in self.raw and self.raw[name] is not None:
+                return self.raw[name]
         if default is _MISSING:
-            raise ConfigError(f"{self.where}: required key '{key}' is missing")
+            also = "" if len(names) == 1 else " (also read as " + ", ".join(
+                f"'{n}'" for n in names[1:]) + ")"
+            raise ConfigError(f"{self.where}: required key '{names[0]}' is missing{also}")
         return default
+
+    @staticmethod
+    def _name(key) -> str:
+        return key if isinstance(key, str) else key[0]
 
     def int(self, key, default=_MISSING) -> Optional[int]:
         v = self._get(key, default)
         if v is None:
             return None
         if isinstance(v, bool) or not isinstance(v, (int, float)) or int(v) != v:
-            raise ConfigError(f"{self.where}: key '{key}' must be an integer, got {v!r}")
+            raise ConfigError(f"{self.where}: key '{self._name(key)}' must be an integer, got {v!r}")
         return int(v)
 
     def float(self, key, default=_MISSING) -> Optional[float]:
@@ -49,13 +59,13 @@ class KeyReader:
         if v is None:
             return None
         if isinstance(v, bool) or not isinstance(v, (int, float)):
-            raise ConfigError(f"{self.where}: key '{key}' must be a number, got {v!r}")
+            raise ConfigError(f"{self.where}: key '{self._name(key)}' must be a number, got {v!r}")
         return float(v)
 
     def bool(self, key, default=_MISSING) -> bool:
         v = self._get(key, default)
         if not isinstance(v, bool):
-            raise ConfigError(f"{self.where}: key '{key}' must be true or false, got {v!r}")
+            raise ConfigError(f"{self.where}: key '{self._name(key)}' must be true or false, got {v!r}")
         return v
 
     def list(self, key, default=_MISSING):
@@ -63,7 +73,7 @@ class KeyReader:
         if v is None:
             return None
         if not isinstance(v, (list, tuple)):
-            raise ConfigError(f"{self.where}: key '{key}' must be a list, got {v!r}")
+            raise ConfigError(f"{self.where}: key '{self._name(key)}' must be a list, got {v!r}")
         return list(v)
 
 

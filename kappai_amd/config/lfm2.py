@@ -34,6 +34,16 @@ def adjusted_ff_dim(intermediate_size: int, auto_adjust: bool, multiple_of: int,
     return multiple_of * ((f + multiple_of - 1) // multiple_of)
 
 
+def _rope_theta(r: KeyReader) -> float:
+    """``rope_theta``, at the top level or inside ``rope_parameters`` (where newer exports of the
+    architecture's tools put it)."""
+    nested = r.raw.get("rope_parameters")
+    if r.raw.get("rope_theta") is None and isinstance(nested, dict) \
+            and nested.get("rope_theta") is not None:
+        return KeyReader(nested, r.where + ": rope_parameters").float("rope_theta")
+    return r.float("rope_theta")
+
+
 @dataclass
 class Lfm2Config(ModelConfig):
     hidden_size: int = 0
@@ -52,7 +62,7 @@ class Lfm2Config(ModelConfig):
     conv_L_cache: int = 0
     conv_bias: bool = False
     tie_embedding: bool = True
-    max_position_embeddings: int = 0
+    max_position_embeddings: int = 0         # 0: config.json names no longest sequence
     eos_token_id: Optional[int] = None
     bos_token_id: Optional[int] = None
     pad_token_id: Optional[int] = None
@@ -88,7 +98,7 @@ class Lfm2Config(ModelConfig):
                                   f"{', '.join(sorted(_LAYER_TYPE_NAMES))}")
             kinds.append(_LAYER_TYPE_NAMES[t])
         hidden = r.int("hidden_size")
-        heads = r.int("num_attention_heads")
+        heads = r.int(("num_attention_heads", "num_heads"))
         head_dim = r.int("head_dim", None)
         if head_dim is None:
             if heads <= 0 or hidden % heads:
@@ -103,17 +113,17 @@ class Lfm2Config(ModelConfig):
             num_attention_heads=heads,
             num_key_value_heads=r.int("num_key_value_heads"),
             head_dim=head_dim,
-            intermediate_size=r.int("intermediate_size"),
+            intermediate_size=r.int(("intermediate_size", "block_ff_dim")),
             block_auto_adjust_ff_dim=r.bool("block_auto_adjust_ff_dim", False),
             block_multiple_of=r.int("block_multiple_of", 256),
             block_ffn_dim_multiplier=r.float("block_ffn_dim_multiplier", None),
             vocab_size=r.int("vocab_size"),
-            norm_eps=r.float("norm_eps"),
-            rope_theta=r.float("rope_theta"),
+            norm_eps=r.float(("norm_eps", "block_norm_eps")),
+            rope_theta=_rope_theta(r),
             conv_L_cache=r.int("conv_L_cache"),
             conv_bias=r.bool("conv_bias", False),
-            tie_embedding=r.bool("tie_embedding", True),
-            max_position_embeddings=r.int("max_position_embeddings"),
+            tie_embedding=r.bool(("tie_embedding", "tie_word_embeddings"), True),
+            max_position_embeddings=r.int("max_position_embeddings", 0),
             eos_token_id=r.int("eos_token_id", None),
             bos_token_id=r.int("bos_token_id", None),
             pad_token_id=r.int("pad_token_id", None),
@@ -149,7 +159,7 @@ class Lfm2Config(ModelConfig):
         need(self.ff_dim >= 1, "the feed-forward width works out to zero")
         need(self.norm_eps > 0.0, "norm_eps must be positive")
         need(self.rope_theta > 0.0, "rope_theta must be positive")
-        need(self.max_position_embeddings >= 1, "max_position_embeddings must be positive")
+        need(self.max_position_embeddings >= 0, "max_position_embeddings must not be negative")
 
     def to_dict(self) -> Dict[str, Any]:
         d = {

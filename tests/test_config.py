@@ -60,13 +60,33 @@ def test_registry():
 
 @pytest.mark.parametrize("key", ["hidden_size", "num_hidden_layers", "num_attention_heads",
                                  "num_key_value_heads", "intermediate_size", "vocab_size",
-                                 "norm_eps", "rope_theta", "conv_L_cache",
-                                 "max_position_embeddings"])
+                                 "norm_eps", "rope_theta", "conv_L_cache"])
 def test_required_keys(key):
     raw = copy.deepcopy(TINY_A)
     del raw[key]
     with pytest.raises(ConfigError, match=key):
         config_from_dict(raw)
+
+
+def test_other_spellings_of_the_same_keys():
+    """Exports of the architecture's own tools have named some keys differently over time
+    (block_ff_dim, block_norm_eps, num_heads, tie_word_embeddings, rope_parameters.rope_theta);
+    the key of today wins where both are there.  A config without max_position_embeddings
+    names no longest sequence."""
+    raw = copy.deepcopy(TINY_A)
+    want = config_from_dict(copy.deepcopy(raw))
+    for old_key, new_key in (("intermediate_size", "block_ff_dim"), ("norm_eps", "block_norm_eps"),
+                             ("num_attention_heads", "num_heads"),
+                             ("tie_embedding", "tie_word_embeddings")):
+        raw[new_key] = raw.pop(old_key)
+    raw["rope_parameters"] = {"rope_theta": raw.pop("rope_theta"), "rope_type": "default"}
+    del raw["max_position_embeddings"]
+    got = config_from_dict(copy.deepcopy(raw))
+    assert got.max_position_embeddings == 0
+    got.max_position_embeddings = want.max_position_embeddings
+    assert got == want
+    raw["norm_eps"], raw["block_norm_eps"] = 1e-3, 1e-7
+    assert config_from_dict(raw).norm_eps == 1e-3
 
 
 @pytest.mark.parametrize("change,match", [
