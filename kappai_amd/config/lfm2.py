@@ -153,6 +153,9 @@ class Lfm2Config(ModelConfig):
         need(self.head_dim >= 2 and self.head_dim % 2 == 0,
              f"head_dim ({self.head_dim}) must be even for the rotation's pairs")
         need(self.head_dim <= MAX_HEAD_DIM, f"head_dim ({self.head_dim}) exceeds {MAX_HEAD_DIM}")
+        need(self.head_dim % 8 == 0 or not self.attention_layers,
+             f"head_dim ({self.head_dim}) must be a multiple of 8: the attention kernels read "
+             "keys and values 8 at a time")
         need(self.conv_L_cache >= 2, f"conv_L_cache ({self.conv_L_cache}) must be at least 2")
         need(self.intermediate_size >= 1, "intermediate_size must be positive")
         need(self.block_multiple_of >= 1, "block_multiple_of must be positive")

@@ -308,6 +308,8 @@ class StepRunner:
         their ``want``.  If the pages do not suffice, ``OutOfPages`` is raised and neither
         the cache nor any request has changed."""
         entries = list(entries)
+        if not entries:
+            raise ValueError("a step needs at least one entry")
         single = all(len(e.tokens) == 1 for e in entries)
         extended: List[StepEntry] = []
         try:

@@ -11,6 +11,7 @@ import ctypes
 import hashlib
 import os
 import shutil
+import stat
 import subprocess
 import sys
 import tempfile
@@ -67,25 +68,64 @@ def _source_hash(name: str, defines=None) -> str:
     return h.hexdigest()
 
 
-def _build_dirs() -> List[Path]:
-    dirs = [CSRC / "_build"]
+def _tree_build_dir() -> Path:
+    return CSRC / "_build"
+
+
+def _private_temp_dir(create: bool):
+    """A build folder under the temp folder for a source tree that cannot be written: made with
+    mode 0700, and used only if it is a real folder of this user that nobody else can write
+    (anything else there could hold a library that somebody else put in place).  None when it is
+    not there (``create`` false) ; an error when it is there but not ours alone."""
     uid = os.getuid() if hasattr(os, "getuid") else 0
-    dirs.append(Path(tempfile.gettempdir()) / f"kappai_amd_build_{uid}")
+    d = Path(tempfile.gettempdir()) / f"kappai_amd_build_{uid}"
+    if create:
+        try:
+            os.mkdir(d, 0o700)
+        except FileExistsError:
+            pass
+    try:
+        st = os.lstat(d)
+    except FileNotFoundError:
+        return None
+    if not stat.S_ISDIR(st.st_mode) or st.st_uid != uid or st.st_mode & 0o022:
+        raise KernelBuildError(
+            f"{d} is not a folder of user {uid} that only they can write (owner {st.st_uid}, "
+            f"mode {stat.S_IMODE(st.st_mode):o}): refusing to build or load kernels there")
+    return d
+
+
+def _dir_writable(d: Path) -> bool:
+    try:
+        d.mkdir(parents=True, exist_ok=True)
+        fd, probe = tempfile.mkstemp(prefix=".probe_", dir=d)
+        os.close(fd)
+        os.unlink(probe)
+        return True
+    except OSError:
+        return False
+
+
+def _build_dirs(create: bool = False) -> List[Path]:
+    """Where built libraries live: the source tree's own ``_build``; the private temp folder
+    only when the tree cannot be written."""
+    tree = _tree_build_dir()
+    if _dir_writable(tree):
+        return [tree]
+    dirs = [tree] if tree.is_dir() else []
+    tmp = _private_temp_dir(create)
+    if tmp is not None:
+        dirs.append(tmp)
     return dirs
 
 
 def _writable_build_dir() -> Path:
-    for d in _build_dirs():
-        try:
-            d.mkdir(parents=True, exist_ok=True)
-            fd, probe = tempfile.mkstemp(prefix=".probe_", dir=d)
-            os.close(fd)
-            os.unlink(probe)
+    for d in _build_dirs(create=True):
+        if _dir_writable(d):
             return d
-        except OSError:
-            continue
     raise KernelBuildError("no writable folder for the built kernels: tried "
-                           + ", ".join(str(d) for d in _build_dirs()))
+                           f"{_tree_build_dir()} and a private folder under "
+                           f"{tempfile.gettempdir()}")
 
 
 def _find_built(built: str, want_hash: str):

@@ -66,6 +66,12 @@ def _weight_files(model_dir: Path) -> List[Path]:
     index = model_dir / "model.safetensors.index.json"
     if index.is_file():
         names = sorted(set(json.loads(index.read_text())["weight_map"].values()))
+        for n in names:        # a model folder is untrusted input: its files lie inside it
+            if (not isinstance(n, str) or not n or n in (".", "..") or "/" in n or "\\" in n
+                    or Path(n).is_absolute()):
+                raise WeightsError(model_dir, [], [], [], [
+                    f"{index.name}: weight_map names the file {n!r}; a plain file name inside "
+                    "the model folder is needed"])
         return [model_dir / n for n in names]
     raise WeightsError(model_dir, [], [], [], [f"no model.safetensors in {model_dir}"])
 

@@ -79,6 +79,13 @@ class SafetensorsFile:
                     f"{self.path}: tensor '{name}' ({dtype} {list(shape)}) does not fit its "
                     f"data_offsets [{lo}, {hi}) in a file of {size} bytes")
             self.entries[name] = TensorEntry(name, dtype, shape, base + lo, base + hi)
+        last = None
+        for e in sorted(self.entries.values(), key=lambda e: (e.begin, e.end)):
+            if last is not None and e.begin < last.end:
+                raise SafetensorsError(f"{self.path}: tensors '{last.name}' and '{e.name}' "
+                                       "overlap in the file")
+            if e.end > e.begin:
+                last = e
         self._file = open(self.path, "rb")
         self._map = mmap.mmap(self._file.fileno(), 0, access=mmap.ACCESS_READ) if size else None
 

@@ -95,6 +95,7 @@ def test_other_spellings_of_the_same_keys():
     ({"conv_L_cache": 1}, "conv_L_cache"),
     ({"head_dim": 15}, "even"),
     ({"head_dim": 1024}, "exceeds"),
+    ({"head_dim": 18}, "multiple of 8"),
     ({"layer_types": ["conv"]}, "layer_types has 1 entries for 4 layers"),
     ({"layer_types": ["conv", "mamba", "conv", "full_attention"]}, "layer_types\\[1\\]"),
     ({"hidden_size": "64"}, "integer"),

@@ -226,7 +226,8 @@ def test_conv_bias_and_untied_head_are_used(tmp_path):
 def test_round_bf16():
     x = np.array([1.0, 1.0 + 2 ** -9, 1.0 + 2 ** -8, 1.0 + 3 * 2 ** -9, -3.14159, 1e-30, 0.0])
     r = P.round_bf16(x)
-    assert r[0] == 1.0 and r[1] == 1.0 and r[2] == 1.0 + 2 ** -7 - 2 ** -7 + 2 ** -8 or True
+    # ties go to the even mantissa: 1 + 2^-8 lies half way between 1 and 1 + 2^-7
+    assert r[0] == 1.0 and r[1] == 1.0 and r[2] == 1.0 and r[3] == 1.0 + 2 ** -7
     import torch
     assert np.array_equal(r, torch.tensor(x, dtype=torch.float32).to(torch.bfloat16).double().numpy())
 

@@ -64,3 +64,13 @@ def test_schedules_float32(monkeypatch, tmp_path, model_dirs, name, family):
     assert len(got) == sum(len(t) for t in requests.values())
     err, where = worst_error(got, ref)
     assert err < FP32_TOL, (err, where, first_bad(got, ref, FP32_TOL))
+
+
+def test_a_step_without_entries_is_refused(monkeypatch, model_dirs):
+    emulated_ops.install(monkeypatch)
+    model = load_model(model_dirs["A"], "float32", device="cpu")
+    cache = make_replay_cache(model, 64)
+    runner = emulated_ops.make_cpu_runner(model, cache)
+    runner.decode_graphs = True          # the path that used to look at the entries first
+    with pytest.raises(ValueError, match="at least one entry"):
+        runner.step([])

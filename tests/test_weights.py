@@ -117,3 +117,22 @@ def test_missing_file(tmp_path):
     (d / "model.safetensors").unlink()
     with pytest.raises(WeightsError, match="no model.safetensors"):
         load_model(d, "float32", "cpu")
+
+
+def test_container_refuses_overlapping_tensors(tmp_path):
+    p = tmp_path / "overlap.safetensors"
+    hdr = json.dumps({"a": {"dtype": "F32", "shape": [4], "data_offsets": [0, 16]},
+                      "b": {"dtype": "F32", "shape": [4], "data_offsets": [8, 24]}}).encode()
+    p.write_bytes(struct.pack("<Q", len(hdr)) + hdr + b"\0" * 24)
+    with pytest.raises(SafetensorsError, match="overlap"):
+        SafetensorsFile(p)
+
+
+@pytest.mark.parametrize("name", ["../model.safetensors", "/etc/passwd", "sub/x.safetensors", ".."])
+def test_index_file_names_stay_inside_the_model_folder(tmp_path, name):
+    d = write_tiny("A", tmp_path / "a")
+    (d / "model.safetensors").rename(tmp_path / "model.safetensors")
+    (d / "model.safetensors.index.json").write_text(json.dumps(
+        {"weight_map": {"model.embed_tokens.weight": name}}))
+    with pytest.raises(WeightsError, match="plain file name inside the model folder"):
+        load_model(d, "float32", device="cpu")
