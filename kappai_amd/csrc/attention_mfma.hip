@@ -19,6 +19,8 @@
 // Formulas: softmax(q.k/sqrt(d)) v over keys lo..pos (kappai: src/backend/cpu/scalar/core.c:383-433,
 // 623-666), online softmax as in its flash form (:386-413).
 #include "common.h"
+#include "no_alloc.h"
+#include <stdio.h>
 
 #ifndef HEAD_DIM
 #error "compile with -DHEAD_DIM=<multiple of 16>"
@@ -1018,4 +1020,93 @@ extern "C" int kappai_attn_decode(const void* q, int q_stride, const void* k_poo
                      (const float*)part_o, (const float*)part_ml, (bf16_t*)out, out_stride, H,
                      n_splits);
   KAPPAI_RETURN_LAUNCH_STATUS();
+}
+
+// ---------------------------------------------------------------------------------------
+// the decode attention for callers that cannot allocate: partial results in a device array
+// of the library's own
+// ---------------------------------------------------------------------------------------
+static __device__ __align__(256) float scratch[KAPPAI_ATTN_STATIC_SCRATCH_FLOATS];
+
+#define KAPPAI_MAX_DEVICES 64
+// the address of each device's copy of `scratch`; in host code the array's name is only a
+// stand-in for the symbol, never an address that a kernel could use
+static float* g_scratch_ptr[KAPPAI_MAX_DEVICES];
+static thread_local char g_static_error[256];
+
+extern "C" int kappai_attn_decode_static_capacity(void) { return KAPPAI_ATTN_STATIC_SCRATCH_FLOATS; }
+
+extern "C" const char* kappai_attn_decode_static_error(void) { return g_static_error; }
+
+static int static_scratch_of_current_device(float** ptr) {
+  int dev = -1;
+  hipError_t err = hipGetDevice(&dev);
+  if (err != hipSuccess) return (int)err;
+  if (dev < 0 || dev >= KAPPAI_MAX_DEVICES) {
+    snprintf(g_static_error, sizeof g_static_error,
+             "kappai_attn_decode_static: device %d is beyond the %d this library keeps track of",
+             dev, KAPPAI_MAX_DEVICES);
+    return (int)hipErrorInvalidDevice;
+  }
+  float* p = __atomic_load_n(&g_scratch_ptr[dev], __ATOMIC_ACQUIRE);
+  if (p == nullptr) {
+    void* sym = nullptr;
+    err = hipGetSymbolAddress(&sym, HIP_SYMBOL(scratch));
+    if (err != hipSuccess || sym == nullptr) {
+      snprintf(g_static_error, sizeof g_static_error,
+               "kappai_attn_decode_static: hipGetSymbolAddress failed on device %d: %s", dev,
+               hipGetErrorString(err));
+      return (int)(err != hipSuccess ? err : hipErrorInvalidSymbol);
+    }
+    p = static_cast<float*>(sym);
+    __atomic_store_n(&g_scratch_ptr[dev], p, __ATOMIC_RELEASE);   // the same value from any thread
+  }
+  *ptr = p;
+  return 0;
+}
+
+extern "C" int kappai_attn_decode_static_init(void) {
+  float* p = nullptr;
+  return static_scratch_of_current_device(&p);
+}
+
+extern "C" int kappai_attn_decode_static(const void* q, int q_stride, const void* k_pool,
+                                         const void* vt_pool, void* out, int out_stride,
+                                         const int* row_pos, const int* row_seg,
+                                         const int* block_tables, int max_blocks, int T, int H,
+                                         int G, int ps, int window, float scale,
+                                         int keys_per_split, int n_splits, hipStream_t stream) {
+  g_static_error[0] = 0;
+  if (T <= 0) return 0;
+  if (H < 1 || n_splits < 1) {
+    snprintf(g_static_error, sizeof g_static_error,
+             "kappai_attn_decode_static: H = %d heads and n_splits = %d must be positive", H,
+             n_splits);
+    return (int)hipErrorInvalidValue;
+  }
+  const long long entries = (long long)T * H * n_splits;
+  const long long need = entries * (HEAD_DIM + 2);
+  if (need > KAPPAI_ATTN_STATIC_SCRATCH_FLOATS) {
+    snprintf(g_static_error, sizeof g_static_error,
+             "kappai_attn_decode_static: %d rows x %d heads x %d splits need %lld floats of partial "
+             "results (head size %d); the library's array holds %d: use fewer splits or rows, or "
+             "kappai_attn_decode with a workspace of the caller's",
+             T, H, n_splits, need, HEAD_DIM, KAPPAI_ATTN_STATIC_SCRATCH_FLOATS);
+    return (int)hipErrorInvalidValue;
+  }
+  float* base = nullptr;
+  const int rc = static_scratch_of_current_device(&base);
+  if (rc != 0) return rc;
+  // part_o first (a multiple of 16 floats, so part_ml stays 16-byte aligned as well)
+  float* part_o = base;
+  float* part_ml = base + entries * HEAD_DIM;
+  const int status = kappai_attn_decode(q, q_stride, k_pool, vt_pool, out, out_stride, part_o,
+                                        part_ml, row_pos, row_seg, block_tables, max_blocks, T, H,
+                                        G, ps, window, scale, keys_per_split, n_splits, stream);
+  if (status == (int)hipErrorInvalidValue)
+    snprintf(g_static_error, sizeof g_static_error,
+             "kappai_attn_decode_static: an argument that kappai_attn_decode refuses (page size "
+             "%d, %d heads over %d kv heads, %d keys a split, q stride %d)",
+             ps, H, G, keys_per_split, q_stride);
+  return status;
 }
