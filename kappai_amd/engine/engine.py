@@ -132,6 +132,7 @@ class Engine:
         self._next_id = 0
         self._t_first_add: Optional[float] = None
         self.last_logits: Optional[torch.Tensor] = None
+        self.decode_runs = 0              # runs of queued decode steps taken so far
         if config.warm_kernels:
             self._warm_kernels()
 
@@ -259,6 +260,7 @@ class Engine:
         if tokens is None:
             return None
         self.last_logits = None
+        self.decode_runs += 1
         rows = tokens.tolist()            # waits for the run
         dt = time.perf_counter() - t0
         m = self.metrics

@@ -109,6 +109,30 @@ def test_greedy_bfloat16_follows_the_plain_logits(model_dirs):
             assert row[tok] >= row.max() - 0.03 * np.abs(row).max(), (j, tok, int(row.argmax()))
 
 
+def test_greedy_bfloat16_in_queued_decode_runs_follows_the_plain_logits(model_dirs):
+    """Three requests decoded 40 tokens each, mostly in runs of eight queued graph replays whose
+    tokens stay on the GPU between steps (with dummy rows: three requests run in the graph for
+    four): every token chosen is the best, or as good as the best within twice the error bound
+    of a bfloat16 logit, under the plain logits of the engine's own prefix."""
+    from replay_common import BF16_MAX_FACTOR, bf16_bounds
+    from kappai_amd.engine import Engine
+    from kappai_amd.sampling import SamplingParams
+    prompts = prompts_for("B", [19, 6, 33], seed=8)
+    eng = Engine(str(model_dirs["B"]), dtype="bfloat16", num_pages=64, max_batch=4, decode_run=8)
+    got = eng.generate(prompts, SamplingParams.greedy(n_predict=40))
+    assert eng.decode_runs >= 3 and eng.runner.graph_replays >= 24
+    cfg, w = P.read_model_dir(model_dirs["B"])
+    for i, (p, g) in enumerate(zip(prompts, got)):
+        assert len(g) == 40
+        seq = {f"s{i}": p + g}
+        logits = P.forward(cfg, w, p + g)
+        keys = [(f"s{i}", len(p) - 1 + j) for j in range(len(g))]
+        bound = BF16_MAX_FACTOR * bf16_bounds(model_dirs["B"], seq, keys)[0] * np.abs(logits).max()
+        for j, tok in enumerate(g):
+            row = logits[len(p) - 1 + j]
+            assert row[tok] >= row.max() - 2 * bound, (i, j, tok, int(row.argmax()), bound)
+
+
 def test_preemption_gives_the_same_tokens(model_dirs):
     """With so few pages that requests are preempted and computed again, greedy output is what
     it is with plenty of pages."""

@@ -174,6 +174,34 @@ def test_conv_mixer_order_of_the_three_parts():
     assert np.allclose(P.short_conv_mixer(xb, lw, cfg), p[:, D:2 * D] * p[:, :D] * p[:, 2 * D:])
 
 
+def test_conv_mixer_biases_are_those_of_the_library_layers():
+    """With ``conv_bias`` the checkpoint holds a bias for each of the three linear maps of the
+    mixer: ``in_proj.bias``, ``conv.bias`` (the depthwise convolution's own, so it is added to the
+    filter's output, before the C gate) and ``out_proj.bias``.  kappai's LFM2 has no biases, so
+    this is pinned by the library routines that such tensors belong to: a linear layer with bias,
+    a grouped 1-d convolution with bias and left padding, a linear layer with bias.  A bias added
+    after the gate, or to the gated input, fails."""
+    import torch
+    import torch.nn.functional as F
+    D, L, T = 6, 4, 9
+    cfg = {"hidden_size": D}
+    lw = {"in_proj": RNG.normal(size=(3 * D, D)), "in_proj_bias": RNG.normal(size=3 * D),
+          "conv": RNG.normal(size=(D, L)), "conv_bias": RNG.normal(size=D),
+          "out_proj": RNG.normal(size=(D, D)), "out_proj_bias": RNG.normal(size=D)}
+    xb = RNG.normal(size=(T, D))
+    t = {k: torch.from_numpy(np.asarray(v)) for k, v in lw.items()}
+    p = F.linear(torch.from_numpy(xb), t["in_proj"], t["in_proj_bias"])
+    Bg, Cg, xg = p[:, :D], p[:, D:2 * D], p[:, 2 * D:]
+    bx = (Bg * xg).T[None]                                   # [1, channels, time]
+    s = F.conv1d(bx, t["conv"][:, None, :], t["conv_bias"], padding=L - 1, groups=D)[0, :, :T].T
+    want = F.linear(Cg * s, t["out_proj"], t["out_proj_bias"]).numpy()
+    got = P.short_conv_mixer(xb, lw, cfg)
+    assert np.abs(got - want).max() < 1e-12
+    # the plausible mistakes give something else
+    late = F.linear(Cg * (s - t["conv_bias"]) + t["conv_bias"], t["out_proj"], t["out_proj_bias"]).numpy()
+    assert np.abs(got - late).max() > 1e-3
+
+
 # -- feed-forward, head --------------------------------------------------------------------------
 def test_swiglu():
     xb = RNG.normal(size=(4, 8))
