@@ -150,10 +150,10 @@ class DecodeBench:
         self.cache.allocate_storage(model.dtype, device)
         gen = torch.Generator(device=device).manual_seed(seed)
         for g in self.cache.paged_groups:
-            for pools in (g.k_pools, g.v_pools):
-                for cid in pools:
-                    pools[cid].copy_(torch.randn(pools[cid].shape, generator=gen, device=device,
-                                                 dtype=torch.float32) * 0.5)
+            for pools in g.pools.values():
+                for t in pools.values():
+                    t.copy_(torch.randn(t.shape, generator=gen, device=device,
+                                        dtype=torch.float32) * 0.5)
         self.runner = StepRunner(model, self.cache, device, decode_graphs=graphs)
         self.requests = [self.cache.open(i) for i in range(batch)]
         for rc in self.requests:

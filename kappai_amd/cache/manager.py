@@ -19,7 +19,7 @@ from typing import Dict, Hashable, List, Optional, Sequence, Union
 
 import torch
 
-from .specs import FixedState, PagedKV
+from .specs import FixedState, PagedSpec
 
 
 class CacheError(RuntimeError):
@@ -90,11 +90,11 @@ class PageAllocator:
 
 @dataclass
 class PagedGroup:
-    spec: PagedKV
+    spec: PagedSpec
     cache_ids: List[int]
     allocator: PageAllocator
-    k_pools: Dict[int, torch.Tensor] = field(default_factory=dict)   # cache id -> pool
-    v_pools: Dict[int, torch.Tensor] = field(default_factory=dict)
+    # cache id -> {pool name: tensor [pages + 1, *page_shape]}, as the spec's pools() names them
+    pools: Dict[int, Dict[str, torch.Tensor]] = field(default_factory=dict)
 
 
 @dataclass
@@ -106,12 +106,15 @@ class StateGroup:
 
 @dataclass
 class PagedLayerView:
-    """What a paged layer sees: its pools and the index of its group's block tables."""
-    k_pool: Optional[torch.Tensor]
-    v_pool: Optional[torch.Tensor]
+    """What a paged layer sees: its pools by the names its spec gave them (empty before
+    ``allocate_storage``) and the index of its group's block tables."""
+    pools: Dict[str, torch.Tensor]
     group: int
-    spec: PagedKV
+    spec: PagedSpec
     page_size: int
+
+    def pool(self, name: str) -> Optional[torch.Tensor]:
+        return self.pools.get(name)
 
 
 @dataclass
@@ -137,7 +140,7 @@ class RequestCache:
         return f"RequestCache({self.request_id!r}, slot={self.slot}, length={self.length})"
 
 
-Spec = Union[PagedKV, FixedState, None]
+Spec = Union[PagedSpec, FixedState, None]
 
 
 class CacheManager:
@@ -158,7 +161,7 @@ class CacheManager:
         for cid, spec in enumerate(self.cache_specs):
             if spec is None:
                 continue
-            if isinstance(spec, PagedKV):
+            if isinstance(spec, PagedSpec):
                 groups, kind = self.paged_groups, "paged"
             elif isinstance(spec, FixedState):
                 groups, kind = self.state_groups, "state"
@@ -185,19 +188,23 @@ class CacheManager:
 
     # -- device storage -------------------------------------------------------------------
     def allocate_storage(self, dtype: torch.dtype, device, poison: bool = False) -> None:
-        """Create the key pools [pages, kv_heads, page_size, head_dim], the value pools (stored
-        transposed: [pages, kv_heads, head_dim, page_size]) and the slot arrays.  ``poison``
-        fills the pools with NaN so that a read of a key nobody wrote shows."""
+        """Create, for every layer of a paged group, the tensors its spec names
+        (``[pages + 1, *page_shape]`` each), and the slot arrays.  ``poison`` fills them with NaN
+        so that a read of something nobody wrote shows."""
         self.device, self.dtype = device, dtype
         for g in self.paged_groups:
             n = g.allocator.num_pages + 1          # the last page is scratch (see scratch_page)
-            kshape = (n, g.spec.num_kv_heads, self.page_size, g.spec.head_dim)
-            vshape = (n, g.spec.num_kv_heads, g.spec.head_dim, self.page_size)
             for cid in g.cache_ids:
-                for pools, shape in ((g.k_pools, kshape), (g.v_pools, vshape)):
-                    t = torch.empty(shape, dtype=dtype, device=device)
-                    t.fill_(float("nan")) if poison else t.zero_()
-                    pools[cid] = t
+                made = {}
+                for pool in g.spec.pools(self.page_size):
+                    pdt = dtype if pool.dtype is None else getattr(torch, pool.dtype)
+                    t = torch.empty((n, *pool.page_shape), dtype=pdt, device=device)
+                    if poison and pdt.is_floating_point:
+                        t.fill_(float("nan"))
+                    else:
+                        t.zero_()
+                    made[pool.name] = t
+                g.pools[cid] = made
         for g in self.state_groups:
             sdt = getattr(torch, g.spec.dtype)
             for cid in g.cache_ids:
@@ -217,9 +224,9 @@ class CacheManager:
         return self.num_slots
 
     def bytes_per_token(self, dtype_bytes: int) -> int:
-        """Bytes of keys and values that one token takes over all paged layers (kappai:
+        """Bytes that one token takes over all paged layers (kappai:
         model_kv_cache_bytes_quant, src/memory.c:292)."""
-        return sum(2 * g.spec.num_kv_heads * g.spec.head_dim * dtype_bytes * len(g.cache_ids)
+        return sum(g.spec.bytes_per_token(dtype_bytes) * len(g.cache_ids)
                    for g in self.paged_groups)
 
     def view(self, cache_id: int):
@@ -228,10 +235,72 @@ class CacheManager:
         kind, gi = self._where[cache_id]
         if kind == "paged":
             g = self.paged_groups[gi]
-            return PagedLayerView(g.k_pools.get(cache_id), g.v_pools.get(cache_id), gi, g.spec,
-                                  self.page_size)
+            return PagedLayerView(g.pools.get(cache_id, {}), gi, g.spec, self.page_size)
         g = self.state_groups[gi]
         return StateLayerView(g.states.get(cache_id), gi, g.spec)
+
+    # -- looking into a request's cache ------------------------------------------------------
+    def export_range(self, rc: RequestCache, cache_id: int, pos_start: int = 0,
+                     n_rows: Optional[int] = None) -> Dict[str, torch.Tensor]:
+        """What the paged cache ``cache_id`` holds for positions ``pos_start .. pos_start +
+        n_rows - 1`` of the request, gathered out of its pages: ``{pool name: [n_rows, *rest]}``
+        with the token first and the other axes of a page in their order (keys
+        ``[n, kv_heads, head_dim]``, values the same, whatever the page's layout).  For looking
+        at a request when a page goes wrong (kappai: kvcache_export_range, src/kvcache.c:887-901).
+        A position whose page a window has given back is an error."""
+        self._check_live(rc)
+        kind, gi = self._where.get(cache_id, (None, None))
+        if kind != "paged":
+            raise CacheError(f"cache {cache_id} is not a paged cache")
+        g = self.paged_groups[gi]
+        if cache_id not in g.pools:
+            raise CacheError("allocate_storage has not been called")
+        n_rows = rc.length - pos_start if n_rows is None else n_rows
+        if pos_start < 0 or n_rows < 0 or pos_start + n_rows > rc.length:
+            raise CacheError(f"{rc}: positions {pos_start}..{pos_start + n_rows - 1} are not all "
+                             "stored")
+        pos = torch.arange(pos_start, pos_start + n_rows)
+        blocks = torch.tensor(rc.blocks[gi] or [0], dtype=torch.long)
+        pages = blocks[pos // self.page_size] if n_rows else pos
+        if n_rows and int(pages.min()) < 0:
+            gone = int(pos[pages < 0][0])
+            raise CacheError(f"{rc}: position {gone} of cache {cache_id} lies in a page that its "
+                             f"window ({g.spec.window}) has given back")
+        slots = pos % self.page_size
+        out = {}
+        for pool in g.spec.pools(self.page_size):
+            t = g.pools[cache_id][pool.name]
+            moved = t.movedim(1 + pool.slot_axis, 1)            # [pages, slot, *rest]
+            out[pool.name] = moved[pages.to(t.device), slots.to(t.device)].clone()
+        return out
+
+    def export_state(self, rc: RequestCache, cache_id: int) -> torch.Tensor:
+        """A copy of the request's slot of the fixed-size state ``cache_id`` (kappai:
+        kvcache_export_state, src/kvcache.c:924-945)."""
+        self._check_live(rc)
+        kind, gi = self._where.get(cache_id, (None, None))
+        if kind != "state":
+            raise CacheError(f"cache {cache_id} is not a fixed-size state")
+        g = self.state_groups[gi]
+        if cache_id not in g.states:
+            raise CacheError("allocate_storage has not been called")
+        return g.states[cache_id][rc.slot].clone()
+
+    def dump(self, rc: RequestCache) -> dict:
+        """Everything the request holds, for debugging: its length, slot and block tables, and
+        per cache id what ``export_range`` (the positions still kept) or ``export_state`` gives."""
+        self._check_live(rc)
+        out = {"request": rc.request_id, "length": rc.length, "slot": rc.slot,
+               "blocks": [list(b) for b in rc.blocks], "caches": {}}
+        for cid, (kind, gi) in sorted(self._where.items()):
+            if kind == "state":
+                out["caches"][cid] = {"kind": "state", "state": self.export_state(rc, cid)}
+                continue
+            first = next((i for i, b in enumerate(rc.blocks[gi]) if b >= 0), 0) * self.page_size
+            first = min(first, rc.length)
+            out["caches"][cid] = {"kind": "paged", "first_position": first,
+                                  **self.export_range(rc, cid, first, rc.length - first)}
+        return out
 
     # -- requests -------------------------------------------------------------------------
     @property

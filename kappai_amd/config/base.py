@@ -11,7 +11,7 @@ from __future__ import annotations
 import json
 from dataclasses import dataclass, fields
 from pathlib import Path
-from typing import Any, Callable, Dict, Optional
+from typing import Any, Callable, Dict, List, Optional, Union
 
 
 class ConfigError(ValueError):
@@ -82,6 +82,10 @@ class ModelConfig:
     """What every architecture's configuration offers to the rest of the engine."""
 
     architecture: str
+    # What the engine reads beside ``vocab_size``.  An architecture whose config.json gives them
+    # fills them in from its own keys; the defaults mean "the file says nothing".
+    max_position_embeddings: int = 0                       # longest sequence; 0: none named
+    eos_token_id: Optional[Union[int, List[int]]] = None   # token(s) that end a generation
 
     # -- to be provided by the architecture -------------------------------------------
     @classmethod

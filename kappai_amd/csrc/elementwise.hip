@@ -179,6 +179,27 @@ extern "C" int kappai_add_residual(float* resid, const void* delta, long n, int 
   KAPPAI_RETURN_LAUNCH_STATUS();
 }
 
+// out[i] = parts[0][i] + parts[1][i] + ... in this order, in float: the partial sums of a
+// product split over K, for a consumer that does not add them itself
+__global__ void sum_partials_kernel(const float* __restrict__ parts, int n_parts, size_t n,
+                                    float* __restrict__ out) {
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  float acc = parts[i];
+  for (int s = 1; s < n_parts; ++s) acc += parts[(size_t)s * n + i];
+  out[i] = acc;
+}
+
+extern "C" int kappai_sum_partials(const float* parts, int n_parts, long n, float* out,
+                                   hipStream_t stream) {
+  if (n <= 0 || n_parts < 1) return n_parts < 1 ? (int)hipErrorInvalidValue : 0;
+  const int threads = 256;
+  const unsigned blocks = (unsigned)((n + threads - 1) / threads);
+  hipLaunchKernelGGL(sum_partials_kernel, dim3(blocks), dim3(threads), 0, stream, parts, n_parts,
+                     (size_t)n, out);
+  KAPPAI_RETURN_LAUNCH_STATUS();
+}
+
 // ---------------------------------------------------------------------------------------
 // act[t, f] = silu(gu[t, f]) * gu[t, F + f],  silu(z) = z / (1 + exp(-z))
 //                                                      (src/backend/cpu/quants.h:369-371)

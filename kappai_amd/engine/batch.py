@@ -33,7 +33,8 @@ class RowBatch:
     seg_start[S+1] (first row of each segment), seg_pos0[S] (position of that row),
     seg_slot[S] (the request's state slot), block_tables[g] [S, max_blocks] for every paged
     group g, logit_rows[n] (rows whose logits are wanted, in the order asked), q_tiles: the
-    segments cut into runs of at most ATTENTION_TILE_ROWS rows for the attention kernel."""
+    segments cut into runs of at most ``Model.q_tile_rows`` rows, laid out only when a part of
+    the model asks for it (the tiled attention kernel does)."""
     n_rows: int
     n_segments: int
     n_logit_rows: int
@@ -51,9 +52,6 @@ class RowBatch:
     host: Dict[str, np.ndarray] = field(default_factory=dict)
 
 
-ATTENTION_TILE_ROWS = 32
-
-
 def tile_place(index: int, tiles_in_segment: int) -> int:
     """The fourth number of a q tile; 0 (place unknown) when the segment has more tiles than
     the 16 bits of either half hold."""
@@ -62,9 +60,11 @@ def tile_place(index: int, tiles_in_segment: int) -> int:
     return index | (tiles_in_segment << 16)
 
 
-def layout_rows(entries: Sequence[StepEntry], cache: CacheManager, vocab_size: int):
+def layout_rows(entries: Sequence[StepEntry], cache: CacheManager, vocab_size: int,
+                tile_rows: Optional[int] = None):
     """Host side of ``RowBatch``: checks the entries and lays the tables out as int32
-    arrays.  Returns (dict of arrays, sizes)."""
+    arrays.  Returns (dict of arrays, sizes).  ``tile_rows``: cut the segments into tiles of at
+    most that many rows (``q_tiles``); None: no such table."""
     if not entries:
         raise ValueError("a step needs at least one entry")
     seen = set()
@@ -94,12 +94,12 @@ def layout_rows(entries: Sequence[StepEntry], cache: CacheManager, vocab_size: i
         row_seg.append(np.full(n, si, dtype=np.int32))
         max_position = max(max_position, p0 + n - 1)
         seg_start.append(base + n)
-        n_seg_tiles = (n + ATTENTION_TILE_ROWS - 1) // ATTENTION_TILE_ROWS
-        for j, r in enumerate(range(0, n, ATTENTION_TILE_ROWS)):
-            # the fourth number tells a kernel where the tile stands in its segment
-            # (index | tiles of the segment << 16), so that it can pair tiles of one segment
-            q_tiles.append((si, base + r, min(ATTENTION_TILE_ROWS, n - r),
-                            tile_place(j, n_seg_tiles)))
+        if tile_rows:
+            n_seg_tiles = (n + tile_rows - 1) // tile_rows
+            for j, r in enumerate(range(0, n, tile_rows)):
+                # the fourth number tells a kernel where the tile stands in its segment
+                # (index | tiles of the segment << 16), so that it can pair tiles of one segment
+                q_tiles.append((si, base + r, min(tile_rows, n - r), tile_place(j, n_seg_tiles)))
         seg_pos0.append(p0)
         seg_slot.append(e.cache.slot)
         logit_rows.extend(base + int(w) for w in e.want)
@@ -120,8 +120,9 @@ def layout_rows(entries: Sequence[StepEntry], cache: CacheManager, vocab_size: i
         "seg_pos0": np.asarray(seg_pos0, dtype=np.int32),
         "seg_slot": np.asarray(seg_slot, dtype=np.int32),
         "logit_rows": np.asarray(logit_rows, dtype=np.int32),
-        "q_tiles": np.asarray(q_tiles, dtype=np.int32).reshape(-1, 4),
     }
+    if tile_rows:
+        arrays["q_tiles"] = np.asarray(q_tiles, dtype=np.int32).reshape(-1, 4)
     for gi, bt in enumerate(tables):
         arrays[f"block_table_{gi}"] = bt
     sizes = {

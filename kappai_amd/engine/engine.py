@@ -102,7 +102,7 @@ class Engine:
             model = load_model(config.model, config.dtype, self.device)
         self.model = model
         mc = model.config
-        model_ctx = getattr(mc, "max_position_embeddings", 0) or 0
+        model_ctx = mc.max_position_embeddings or 0
         self.ctx_size = min(config.ctx_size, model_ctx) if config.ctx_size and model_ctx else (
             config.ctx_size or model_ctx)
         specs = model.cache_specs()
@@ -121,7 +121,7 @@ class Engine:
         self.cache = CacheManager(specs, config.page_size, num_pages, config.max_batch)
         self.cache.allocate_storage(model.dtype, self.device)
         self.runner = StepRunner(model, self.cache, self.device)
-        eos = getattr(mc, "eos_token_id", None)
+        eos = mc.eos_token_id
         self.scheduler = Scheduler(
             self.cache,
             SchedulerConfig(config.token_budget, config.chunk, config.max_batch, self.ctx_size),

@@ -57,8 +57,10 @@ class _DecodeGraph:
         n_groups = len(cache.paged_groups)
         self.B, self.n_logit, self.width = B, n_logit, ctx_cap // cache.page_size + 1
         shapes = [("tokens", (B,)), ("row_pos", (B,)), ("row_seg", (B,)), ("seg_start", (B + 1,)),
-                  ("seg_pos0", (B,)), ("seg_slot", (B,)), ("logit_rows", (n_logit,)),
-                  ("q_tiles", (B, 4))]
+                  ("seg_pos0", (B,)), ("seg_slot", (B,)), ("logit_rows", (n_logit,))]
+        tiled = bool(runner.model.q_tile_rows)
+        if tiled:
+            shapes.append(("q_tiles", (B, 4)))
         shapes += [(f"block_table_{g}", (B, self.width)) for g in range(n_groups)]
         self.offsets, total = {}, 0
         for k, shp in shapes:
@@ -76,15 +78,16 @@ class _DecodeGraph:
             n_rows=B, n_segments=B, n_logit_rows=n_logit, max_position=ctx_cap - 1,
             max_segment_rows=1, tokens=views["tokens"], row_pos=views["row_pos"],
             row_seg=views["row_seg"], seg_start=views["seg_start"], seg_pos0=views["seg_pos0"],
-            seg_slot=views["seg_slot"], logit_rows=views["logit_rows"], q_tiles=views["q_tiles"],
+            seg_slot=views["seg_slot"], logit_rows=views["logit_rows"], q_tiles=views.get("q_tiles"),
             block_tables=[views[f"block_table_{g}"] for g in range(n_groups)], host={})
         # what never changes
         self.h["row_seg"][:] = np.arange(B)
         self.h["seg_start"][:] = np.arange(B + 1)
-        self.h["q_tiles"][:, 0] = np.arange(B)
-        self.h["q_tiles"][:, 1] = np.arange(B)
-        self.h["q_tiles"][:, 2] = 1
-        self.h["q_tiles"][:, 3] = 1 << 16         # tile 0 of 1 in its segment
+        if tiled:
+            self.h["q_tiles"][:, 0] = np.arange(B)
+            self.h["q_tiles"][:, 1] = np.arange(B)
+            self.h["q_tiles"][:, 2] = 1
+            self.h["q_tiles"][:, 3] = 1 << 16         # tile 0 of 1 in its segment
         # a warm-up run on the scratch page and the scratch slot: every kernel of this shape is
         # loaded and has run once before the capture, and no request's cache is touched
         self.h["seg_slot"][:] = cache.scratch_slot
@@ -210,7 +213,8 @@ class StepRunner:
         self._staged.record()
 
     def make_batch(self, entries: Sequence[StepEntry]) -> RowBatch:
-        arrays, sizes = layout_rows(entries, self.cache, self.model.vocab_size)
+        arrays, sizes = layout_rows(entries, self.cache, self.model.vocab_size,
+                                    getattr(self.model, "q_tile_rows", None))
         dev = self._upload(arrays)
         return RowBatch(
             n_rows=sizes["n_rows"], n_segments=sizes["n_segments"],
@@ -218,7 +222,7 @@ class StepRunner:
             max_segment_rows=sizes["max_segment_rows"],
             tokens=dev["tokens"], row_pos=dev["row_pos"], row_seg=dev["row_seg"],
             seg_start=dev["seg_start"], seg_pos0=dev["seg_pos0"], seg_slot=dev["seg_slot"],
-            logit_rows=dev["logit_rows"], q_tiles=dev["q_tiles"],
+            logit_rows=dev["logit_rows"], q_tiles=dev.get("q_tiles"),
             block_tables=[dev[f"block_table_{g}"] for g in range(sizes["n_groups"])],
             host=arrays)
 

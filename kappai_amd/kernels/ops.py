@@ -204,6 +204,18 @@ def add_residual(resid: torch.Tensor, delta: torch.Tensor) -> None:
         _stream()), "add_residual")
 
 
+def sum_partial_sums(parts: torch.Tensor) -> torch.Tensor:
+    """float32 [T, D] from the partial sums [S, T, D] of a product split over K, added in order:
+    for a consumer (a norm, a block) that takes a plain update only."""
+    _gpu("parts", parts, F32)
+    _need(parts.dim() == 3, "sum_partial_sums: [S, T, D] is needed")
+    out = torch.empty(parts.shape[1:], dtype=F32, device=parts.device)
+    check(library("elementwise").kappai_sum_partials(
+        _ptr(parts), _c_int(parts.shape[0]), _c_long(out.numel()), _ptr(out), _stream()),
+        "sum_partials")
+    return out
+
+
 def stream_read(buf: torch.Tensor) -> int:
     """Launches one plain read of ``buf`` (a kernel that only loads) and returns the bytes it
     reads: the yardstick for the kernels that stream weights and cache."""

@@ -14,7 +14,7 @@ from typing import Dict, List, Optional, Sequence
 import torch
 
 from ..config.base import ModelConfig
-from ..parts.base import Block, Hidden, Norm, PositionEncoding
+from ..parts.base import Block, Hidden, Norm, PositionEncoding, summed_delta
 from ..parts.embedding import OutputHead, TokenEmbedding
 from ..weights.spec import TensorSpec
 
@@ -100,6 +100,15 @@ class Model:
         return all(getattr(p, "capturable", True) for p in self._parts())
 
     @property
+    def q_tile_rows(self) -> Optional[int]:
+        """Rows of the tiles that the step function cuts segments into for the parts that ask for
+        such a table (None: nobody does)."""
+        asked = {r for r in (getattr(b, "q_tile_rows", None) for b in self.layers) if r}
+        if len(asked) > 1:
+            raise ValueError(f"the layers ask for tiles of different sizes: {sorted(asked)}")
+        return asked.pop() if asked else None
+
+    @property
     def vocab_size(self) -> int:
         return self.config.vocab_size
 
@@ -122,9 +131,10 @@ class Model:
             h = block.forward(h, batch, view, shared_cache=call.reads_cache_of is not None)
         if batch.n_logit_rows == 0:
             return torch.empty((0, self.vocab_size), dtype=torch.float32, device=x.device)
+        delta = summed_delta(self.final_norm, h.delta)
         if (getattr(self.final_norm, "can_defer", False)
                 and getattr(self.head, "takes_pending_norm", False)):
-            xb = self.final_norm.add_norm(h.resid, h.delta, rows=batch.logit_rows, defer=True)
+            xb = self.final_norm.add_norm(h.resid, delta, rows=batch.logit_rows, defer=True)
         else:
-            xb = self.final_norm.add_norm(h.resid, h.delta, rows=batch.logit_rows)
+            xb = self.final_norm.add_norm(h.resid, delta, rows=batch.logit_rows)
         return self.head.forward(xb)

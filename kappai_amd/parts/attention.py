@@ -24,6 +24,7 @@ from .linear import PARTIAL_SUMS_MIN_ROWS, Linear
 
 class GroupedQueryAttention(Mixer):
     takes_pending_norm = True      # its first product may make the normalised rows itself
+    q_tile_rows = ops.ATTENTION_TILE_ROWS     # the tiled attention kernel's rows a tile
 
     def __init__(self, prefix: str, width: int, num_heads: int, num_kv_heads: int, head_dim: int,
                  dtype: torch.dtype, position: Optional[PositionEncoding] = None,
@@ -80,12 +81,13 @@ class GroupedQueryAttention(Mixer):
             x, partial_sums=batch.max_segment_rows == 1 and x.shape[0] > PARTIAL_SUMS_MIN_ROWS)
         rot = self.position.rotation(x.device, batch.max_position) if self.position else None
         tables = batch.block_tables[cache.group]
+        k_pool, v_pool = cache.pool("k"), cache.pool("v")
         q = ops.qk_norm_rope_store(
             proj, H, G, d, self.q_norm_w, self.k_norm_w, self.qk_norm_eps or 0.0,
             rot.cos if rot else None, rot.sin if rot else None, rot.rot_dim if rot else 0,
-            rot.mode if rot else ops.ROT_NONE, cache.k_pool, cache.v_pool, batch.row_pos,
+            rot.mode if rot else ops.ROT_NONE, k_pool, v_pool, batch.row_pos,
             batch.row_seg, tables, cache.page_size, store_kv=not shared_cache)
-        ctx = ops.paged_attention(q, H, G, d, cache.k_pool, cache.v_pool, batch.row_pos,
+        ctx = ops.paged_attention(q, H, G, d, k_pool, v_pool, batch.row_pos,
                                   batch.row_seg, tables, cache.page_size, self.scale,
                                   window=self.window or 0, q_tiles=batch.q_tiles,
                                   single_rows=batch.max_segment_rows == 1,

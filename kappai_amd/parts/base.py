@@ -28,6 +28,10 @@ class Part:
     # part that reads the batch's tables on the host sets this to False.
     capturable = True
 
+    # Rows of a tile if the part's kernels want the step's segments cut into tiles of at most
+    # that many rows (``RowBatch.q_tiles``); None: the table is not laid out for this part.
+    q_tile_rows: Optional[int] = None
+
     def tensor_specs(self) -> List[TensorSpec]:
         """Full names, shapes and roles of the tensors this part reads from the file."""
         return []
@@ -43,11 +47,29 @@ class Part:
 class Norm(Part):
     """``add_norm`` adds ``delta`` (may be None) into the float32 residual in place and
     returns the normalised rows in the compute dtype.  With ``rows`` only those rows are
-    normalised and the residual is left as it is."""
+    normalised and the residual is left as it is.
+
+    ``delta`` is [T, width] in the compute dtype or in float32.  The parts before a norm may
+    also hand on float32 partial sums [S, T, width] of a product split over its input
+    dimension; a norm that adds them itself (in order, in float32) says so with
+    ``takes_partial_sums = True``, any other norm gets them summed by ``summed_delta`` (what
+    blocks and the model call before ``add_norm``) and never sees three dimensions."""
+
+    takes_partial_sums = False
 
     def add_norm(self, resid: torch.Tensor, delta: Optional[torch.Tensor],
                  rows: Optional[torch.Tensor] = None) -> torch.Tensor:
         raise NotImplementedError
+
+
+def summed_delta(norm: Norm, delta):
+    """``delta`` as ``norm`` takes it: partial sums [S, T, width] are added up first unless the
+    norm adds them itself."""
+    if (delta is not None and getattr(delta, "dim", lambda: 2)() == 3
+            and not getattr(norm, "takes_partial_sums", False)):
+        from ..kernels import ops
+        return ops.sum_partial_sums(delta)
+    return delta
 
 
 class PositionEncoding(Part):

@@ -6,7 +6,7 @@ from typing import Dict, List
 import torch
 
 from ..weights.spec import TensorSpec
-from .base import Block, FeedForward, Hidden, Mixer, Norm, register_part
+from .base import Block, FeedForward, Hidden, Mixer, Norm, register_part, summed_delta
 
 
 def _takes_defer(norm) -> bool:
@@ -29,6 +29,10 @@ class PreNormBlock(Block):
     def capturable(self) -> bool:
         return all(p.capturable for p in self._parts())
 
+    @property
+    def q_tile_rows(self):
+        return self.mixer.q_tile_rows
+
     def tensor_specs(self) -> List[TensorSpec]:
         return [s for p in self._parts() for s in p.tensor_specs()]
 
@@ -48,6 +52,7 @@ class PreNormBlock(Block):
 
     @staticmethod
     def _normed(norm, resid, delta, consumer):
+        delta = summed_delta(norm, delta)
         if getattr(consumer, "takes_pending_norm", False) and _takes_defer(norm):
             return norm.add_norm(resid, delta, defer=True)
         return norm.add_norm(resid, delta)

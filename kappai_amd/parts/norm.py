@@ -20,6 +20,7 @@ FRAGMENT_ROWS_MIN = 8
 
 
 class RMSNorm(Norm):
+    takes_partial_sums = True      # the kernel adds [S, T, width] partial sums itself, in order
     can_defer = True      # add_norm(..., defer=True) may hand out an ops.PendingNorm or
                           # ops.FragmentRows in place of a tensor
 

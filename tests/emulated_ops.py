@@ -32,6 +32,13 @@ def add_rmsnorm(resid, delta, weight, eps, out_dtype, rows=None, write_resid=Tru
     return y.to(out_dtype)
 
 
+def sum_partial_sums(parts):
+    out = parts[0].to(F32).clone()
+    for p in parts[1:]:
+        out += p
+    return out
+
+
 def add_residual(resid, delta):
     resid.add_(delta.to(F32))
 
@@ -208,7 +215,7 @@ def repeat_penalty(logits, row_start, tokens, penalty):
                 logits[r, tok] = logits[r, tok] / pen if logits[r, tok] > 0 else logits[r, tok] * pen
 
 
-ALL = ["embed_rows", "add_rmsnorm", "add_residual", "swiglu", "cast", "linear", "linear_swiglu",
+ALL = ["embed_rows", "add_rmsnorm", "add_residual", "sum_partial_sums", "swiglu", "cast", "linear", "linear_swiglu",
        "interleave_gate_up", "shortconv", "linear_shortconv_step",
        "qk_norm_rope_store", "paged_attention", "sample_rows", "sample_filtered",
        "repeat_penalty"]

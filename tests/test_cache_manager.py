@@ -186,3 +186,71 @@ def test_one_token_shortcuts_equal_the_general_calls():
             versions.append(rb.version)
         assert versions[-1] > versions[0]           # page changes are counted
         assert len(set(versions)) < len(versions)   # and only they
+
+
+def test_a_need_describes_its_own_pools():
+    """The manager serves a kind of growing state it has never heard of: one pool of latent
+    vectors in float32 and one of int32 marks, two layers in a group."""
+    from dataclasses import dataclass
+    from typing import Optional
+
+    import torch
+
+    from kappai_amd.cache import PagedSpec, PoolSpec
+
+    @dataclass(frozen=True)
+    class Latent(PagedSpec):
+        rank: int = 0
+        window: Optional[int] = None
+
+        def pools(self, page_size):
+            return (PoolSpec("latent", (page_size, self.rank), slot_axis=0, dtype="float32"),
+                    PoolSpec("mark", (2, page_size), slot_axis=1, dtype="int32"))
+
+        def bytes_per_token(self, elem_bytes):
+            return self.rank * 4 + 2 * 4
+
+    cm = CacheManager([Latent(rank=5), PagedKV(2, 16), Latent(rank=5), FixedState((3,))], 4, 6, 2)
+    assert [g.cache_ids for g in cm.paged_groups] == [[0, 2], [1]]
+    assert cm.bytes_per_token(2) == 2 * (5 * 4 + 8) + 2 * 2 * 16 * 2
+    cm.allocate_storage(torch.bfloat16, "cpu", poison=True)
+    v = cm.view(2)
+    assert v.pool("latent").shape == (7, 4, 5) and v.pool("latent").dtype == torch.float32
+    assert v.pool("mark").shape == (7, 2, 4) and v.pool("mark").dtype == torch.int32
+    assert torch.isnan(v.pool("latent")).all() and not v.pool("mark").any()
+    kv = cm.view(1)
+    assert kv.pool("k").shape == (7, 2, 4, 16) and kv.pool("v").shape == (7, 2, 16, 4)
+    assert kv.pool("k").dtype == torch.bfloat16
+
+
+def test_dump_gathers_a_request_out_of_its_pages():
+    import torch
+    cm = CacheManager([PagedKV(2, 8), FixedState((3, 2)), PagedKV(2, 8, window=5)], 4, 8, 2)
+    cm.allocate_storage(torch.float32, "cpu")
+    other = cm.open("other")
+    cm.extend(other, 3)
+    cm.commit(other, 3)
+    rc = cm.open("r")
+    n = 11
+    cm.extend(rc, n)
+    k = torch.arange(n * 2 * 8, dtype=torch.float32).reshape(n, 2, 8)
+    for cid in (0, 2):
+        gi = cm.view(cid).group
+        for p in range(n):
+            page = rc.blocks[gi][p // 4]
+            cm.view(cid).pool("k")[page, :, p % 4, :] = k[p] + cid
+            cm.view(cid).pool("v")[page, :, :, p % 4] = -k[p] - cid
+    cm.view(1).state[rc.slot] = 7.0
+    cm.commit(rc, n)                      # the window of cache 2 gives its first page back
+    got = cm.export_range(rc, 0, 2, 7)
+    assert torch.equal(got["k"], k[2:9]) and torch.equal(got["v"], -k[2:9])
+    with pytest.raises(CacheError, match="given back"):
+        cm.export_range(rc, 2, 0, 4)
+    with pytest.raises(CacheError, match="not all stored"):
+        cm.export_range(rc, 0, 5, 9)
+    d = cm.dump(rc)
+    assert d["length"] == n and d["caches"][1]["kind"] == "state"
+    assert torch.equal(d["caches"][1]["state"], torch.full((3, 2), 7.0))
+    assert d["caches"][0]["first_position"] == 0 and torch.equal(d["caches"][0]["k"], k)
+    first = d["caches"][2]["first_position"]
+    assert first == 4 and torch.equal(d["caches"][2]["v"], -k[first:] - 2)

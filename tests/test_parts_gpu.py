@@ -28,7 +28,8 @@ def one_segment_batch(cm, n, rid="r", first=True, rc=None):
     rc = rc or cm.open(rid)
     cm.extend(rc, n)
     runner = StepRunner.__new__(StepRunner)
-    runner.model = type("M", (), {"vocab_size": 10 ** 9})()
+    from kappai_amd.kernels import ops
+    runner.model = type("M", (), {"vocab_size": 10 ** 9, "q_tile_rows": ops.ATTENTION_TILE_ROWS})()
     runner.cache, runner.device, runner._staging, runner._staged = cm, torch.device(DEV), None, None
     batch = runner.make_batch([StepEntry(rc, [0] * n, [])])
     return rc, batch
@@ -441,3 +442,122 @@ def test_toy_feed_forward_with_routing_and_an_absolute_position_encoding():
         diff = (cut - whole).abs().amax(dim=1) / float(whole.abs().max())
         assert float(diff.median()) < tol and float((diff > tol).float().mean()) < (
             0.0 if dtype == "float32" else 0.1) + 1e-9
+
+
+def test_toy_norm_that_knows_nothing_of_partial_sums(monkeypatch):
+    """A LayerNorm written to the Norm interface as documented (``add_norm(resid, delta, rows)``
+    with a plain update), registered from the test and built into blocks around the engine's
+    own conv mixer, attention and SwiGLU.  In bfloat16 decode steps those parts hand on float32
+    partial sums of products split over their input dimension; the block sums them for a norm
+    that does not say it takes them.  Decoding token by token equals the whole prompt, and
+    bfloat16 stays near float32."""
+    import tempfile
+
+    from kappai_amd.config import ModelConfig, config_from_dict, register_architecture
+    from kappai_amd.engine import StepEntry, StepRunner
+    from kappai_amd.engine.replay import make_replay_cache
+    from kappai_amd.kernels import ops
+    from kappai_amd.models import Model, load_model
+    from kappai_amd.parts import Norm, OutputHead, TokenEmbedding, make_part, register_part
+    from kappai_amd.weights import write_random_model
+    from kappai_amd.weights.spec import INIT_ONES, INIT_SMALL, VECTOR, TensorSpec
+
+    class ToyLayerNorm(Norm):
+        def __init__(self, name, width, eps, dtype):
+            self.name, self.width, self.eps, self.dtype = name, width, eps, dtype
+
+        def tensor_specs(self):
+            return [TensorSpec(self.name + ".weight", (self.width,), VECTOR, INIT_ONES),
+                    TensorSpec(self.name + ".bias", (self.width,), VECTOR, INIT_SMALL)]
+
+        def bind(self, tensors):
+            self.w = tensors[self.name + ".weight"].float()
+            self.b = tensors[self.name + ".bias"].float()
+
+        def add_norm(self, resid, delta, rows=None):
+            assert delta is None or delta.dim() == 2, "a plain update is what the interface promises"
+            x = resid
+            if delta is not None:
+                if rows is None:
+                    resid += delta.float()
+                else:
+                    x = resid + delta.float()
+            if rows is not None:
+                x = x[rows.long()]
+            return torch.nn.functional.layer_norm(x, (self.width,), self.w, self.b, self.eps).to(
+                self.dtype)
+
+    register_part("norm", "toy_layernorm", ToyLayerNorm)
+
+    @dataclass
+    class Toy3Config(ModelConfig):
+        width: int = 0
+        vocab_size: int = 0
+
+        @classmethod
+        def from_dict(cls, raw):
+            return cls(architecture="Toy3ForCausalLM", width=raw["width"],
+                       vocab_size=raw["vocab_size"], max_position_embeddings=512)
+
+        def to_dict(self):
+            return {"architectures": ["Toy3ForCausalLM"], "width": self.width,
+                    "vocab_size": self.vocab_size}
+
+    def build(cfg, dtype):
+        def norm(name):
+            return make_part("norm", "toy_layernorm", name=name, width=cfg.width, eps=1e-5,
+                             dtype=dtype)
+
+        def block(i, mixer):
+            p = f"l.{i}."
+            return make_part("block", "pre_norm", mixer_norm=norm(p + "n1"), mixer=mixer,
+                             ffn_norm=norm(p + "n2"),
+                             feed_forward=make_part("feed_forward", "swiglu", prefix=p + "ff.",
+                                                    width=cfg.width, hidden=1024, dtype=dtype))
+        emb = TokenEmbedding("emb", cfg.vocab_size, cfg.width)
+        layers = [block(0, make_part("mixer", "conv", prefix="l.0.conv.", width=cfg.width,
+                                     kernel_size=3, dtype=dtype)),
+                  block(1, make_part("mixer", "attention", prefix="l.1.att.", width=cfg.width,
+                                     num_heads=4, num_kv_heads=2, head_dim=32, dtype=dtype,
+                                     position=None, qk_norm_eps=None))]
+        return Model(cfg, dtype, emb, layers, norm("final"),
+                     OutputHead("head", cfg.vocab_size, cfg.width, tied_to=emb))
+
+    register_architecture("Toy3ForCausalLM", Toy3Config, build)
+    cfg = config_from_dict({"architectures": ["Toy3ForCausalLM"], "width": 128, "vocab_size": 90})
+    assert cfg.eos_token_id is None and cfg.max_position_embeddings == 512
+    summed = []
+    real_sum = ops.sum_partial_sums
+    monkeypatch.setattr(ops, "sum_partial_sums", lambda p: (summed.append(tuple(p.shape)),
+                                                            real_sum(p))[1])
+    toks = [int(t) for t in np.random.default_rng(3).integers(0, 90, size=40)]
+    results = {}
+    for dtype in ("float32", "bfloat16"):
+        with tempfile.TemporaryDirectory() as tmp:
+            write_random_model(tmp, cfg, seed=5, std=0.08)
+            model = load_model(tmp, dtype, DEV)
+
+        def run(portions):
+            cache = make_replay_cache(model, 64)
+            cache.allocate_storage(model.dtype, DEV, poison=True)
+            runner = StepRunner(model, cache, DEV)
+            rc, done, rows = cache.open("t"), 0, []
+            for n in portions:
+                rows.append(runner.step([StepEntry(rc, toks[done:done + n], list(range(n)))]).cpu())
+                done += n
+            return torch.cat(rows)
+
+        summed.clear()
+        whole = run([40])
+        cut = run([17] + [1] * 23)
+        scale = float(whole.abs().max())
+        assert torch.isfinite(whole).all() and scale > 0.1
+        if dtype == "float32":
+            assert not summed          # true 32-bit products are never split
+            assert float((cut - whole).abs().max()) < 2e-5 * scale
+        else:
+            assert any(s[0] > 1 and s[1] == 1 for s in summed), "no decode step handed on partial sums"
+            assert float((cut - whole).abs().max()) < 3e-2 * scale
+        results[dtype] = whole
+    err = float((results["bfloat16"] - results["float32"]).abs().max())
+    assert err < 3e-2 * float(results["float32"].abs().max())
