@@ -751,31 +751,37 @@ struct ConvStep {
   int L;
 };
 
-// PRO (at most NORM_ROWS rows, K <= NORM_MAX_K): the rows are not read from A but made here, by
-// every block for itself, as the RMSNorm of resid + delta (kappai: src/backend/cpu/scalar/
-// quants.c:1507-1512; delta absent, bfloat16, or n_parts float partial sums), with the thread
-// layout and the order of sums of add_rmsnorm_row_kernel, so that the kernel between two
-// products of a decode step is saved.  The first block also writes the updated residual to
-// resid_out, which must not be resid itself (the other blocks still read it).
-#define NORM_ROWS 4
-#define NORM_MAX_K 4096
-struct NormIn {
-  const float* resid;      // [M, K]
-  const void* delta;       // null, bf16 [M, K] or float [n_parts][M][K]
+// Two ways of saving the RMSNorm kernel between two products of a decode step (one row tile,
+// at most 16 rows).  RMSNorm(x) W^T = (x * w) W^T / rms(x) row by row (kappai:
+// src/backend/cpu/scalar/quants.c:1507-1512 for the norm), so the product can run on x * w and
+// be scaled afterwards:
+//   ResidOut (a product whose result is added to the residual stream, plain epilogue, float, K
+//     not split over blocks): resid[m][n] += sum (+ bias) in place, in float; and when `rows` is
+//     set the block also writes what the next product reads, rows[m][n] = bf16(resid[m][n] *
+//     norm_w[n]) (row order, or the fragment order of add_rmsnorm when rows_frag), and
+//     ss[blockIdx.x][m] = the sum of resid[m][n]^2 over its 16 columns;
+//   RowScale (the product that follows): its rows are such x * w, and every result is
+//     multiplied by 1 / sqrt(sum_p ss[p][m] / K + eps) before bias and epilogue.
+struct RowScale {
+  const float* ss;   // [n_parts][M], or null: rows are used as they are
   int n_parts;
-  int delta_f32;
-  const float* w;          // [K]
   float eps;
-  float* resid_out;        // [M, K], or null when there is no delta
+};
+struct ResidOut {
+  float* resid;          // [M, ldr], or null: the result goes to C
+  int ldr;
+  const float* norm_w;   // [N]; null: no rows for a next product
+  bf16_t* rows;          // [M, N] or 16 rows in fragment order
+  int rows_frag;
+  float* ss;             // [gridDim.x][M]
 };
 
-template <typename TO, int MT, int NW, int EPI, int NT, bool PRO = false>
+template <typename TO, int MT, int NW, int EPI, int NT>
 __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny_kernel(
     const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, const float* __restrict__ bias,
-    TO* __restrict__ C, int M, int N, int K, int lda, int ldc, ConvStep cs, NormIn nin,
-    int w_frag, int a_frag) {
+    TO* __restrict__ C, int M, int N, int K, int lda, int ldc, ConvStep cs, RowScale rsc,
+    ResidOut ro, int w_frag, int a_frag) {
   static_assert(NT == 1 || EPI == 0, "several column tiles a wave: plain products only");
-  static_assert(!PRO || (MT == 1 && NT == 1), "normalised rows: one row tile");
   // row groups of W a block streams: gate/up, the three conv gates, or NT column tiles
   constexpr int NG = EPI == 1 ? 2 : (EPI == 2 ? 3 : (EPI == 3 ? 2 : NT));
   __shared__ float red[NW][NG * MT][WAVE][4];
@@ -817,52 +823,6 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny_kernel(
     arow[t] = a_frag ? A + ((size_t)(kg / 8) * 16 + (gm < M ? gm : 0)) * 8
                      : A + (size_t)(gm < M ? gm : 0) * lda + kg;
   }
-  __shared__ __attribute__((aligned(16))) bf16_t xs[PRO ? NORM_ROWS : 1][PRO ? NORM_MAX_K : 8];
-  __shared__ float red16[PRO ? 16 : 1];
-  auto make_rows = [&]() {
-    const bool writer = blockIdx.x == 0 && blockIdx.y == 0 && nin.resid_out != nullptr;
-    for (int m = 0; m < M; ++m) {
-      const float* x = nin.resid + (size_t)m * K;
-      // one pass when the block has a thread for every 8 values (the usual case), else the
-      // values are made again after the sum of squares is known
-      float v[8], w8[8];
-      auto make = [&](int j) {
-        load8(x + j, v);
-        if (nin.delta && nin.delta_f32) {
-          const float* d = reinterpret_cast<const float*>(nin.delta) + (size_t)m * K + j;
-          for (int p = 0; p < nin.n_parts; ++p) {
-            float d8[8];
-            load8(d + (size_t)p * M * K, d8);
-#pragma unroll
-            for (int e = 0; e < 8; ++e) v[e] += d8[e];
-          }
-        } else if (nin.delta) {
-          float d8[8];
-          load8(reinterpret_cast<const bf16_t*>(nin.delta) + (size_t)m * K + j, d8);
-#pragma unroll
-          for (int e = 0; e < 8; ++e) v[e] += d8[e];
-        }
-      };
-      float ss = 0.f;
-      const int first = tid * 8;
-      for (int j = first; j < K; j += NW * WAVE * 8) {
-        make(j);
-        if (writer) store8(nin.resid_out + (size_t)m * K + j, v);
-#pragma unroll
-        for (int e = 0; e < 8; ++e) ss += v[e] * v[e];
-      }
-      ss = block_sum(ss, red16);
-      const float scale = 1.0f / sqrtf(ss / (float)K + nin.eps);
-      for (int j = first; j < K; j += NW * WAVE * 8) {
-        if (K > NW * WAVE * 8) make(j);          // else v still holds the thread's only 8
-        load8(nin.w + j, w8);
-#pragma unroll
-        for (int e = 0; e < 8; ++e) w8[e] = v[e] * scale * w8[e];
-        store8(&xs[m][j], w8);
-      }
-    }
-    __syncthreads();
-  };
   const int kblk = ((K + 32 * (int)gridDim.y - 1) / (32 * (int)gridDim.y)) * 32;   // K a block
   const int kb0 = blockIdx.y * kblk, kb1 = min(K, kb0 + kblk);
   const int kper = ((kb1 - kb0 + 32 * NW - 1) / (32 * NW)) * 32;
@@ -871,33 +831,6 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny_kernel(
   C += (size_t)blockIdx.y * M * ldc;
   // loads in flight a lane: U * (NG + MT)
   constexpr int U = (NG + MT) <= 3 ? SK_UNROLL : ((NG + MT) <= 6 ? 4 : 2);
-  auto load_w = [&](int k, u32x4_t (&wv)[U][NG]) {
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const int gk = k + 32 * u;
-      const bool kin = gk + kg < k1;
-#pragma unroll
-      for (int r = 0; r < NG; ++r)
-        wv[u][r] = (kin && gn + (EPI == 0 ? r * 16 : 0) < N && group_ok(r))
-                       ? load16(wrow + r * group_rows * K + (size_t)gk * kmul)
-                       : zero;
-    }
-  };
-  auto load_a = [&](int k, u32x4_t (&av)[U][MT]) {
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const int gk = k + 32 * u;
-      const bool kin = gk + kg < k1;
-#pragma unroll
-      for (int t = 0; t < MT; ++t) {
-        if constexpr (PRO)
-          av[u][t] = (kin && col < M) ? *reinterpret_cast<const u32x4_t*>(&xs[col % NORM_ROWS][gk + kg])
-                                      : zero;
-        else
-          av[u][t] = (kin && t * 16 + col < M) ? load16(arow[t] + (size_t)gk * (a_frag ? 16 : 1)) : zero;
-      }
-    }
-  };
   auto products = [&](const u32x4_t (&wv)[U][NG], const u32x4_t (&av)[U][MT]) {
 #pragma unroll
     for (int u = 0; u < U; ++u)
@@ -908,17 +841,7 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny_kernel(
           acc[r * MT + t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
               as_bf16x8(av[u][t]), as_bf16x8(wv[u][r]), acc[r * MT + t], 0, 0, 0);
   };
-  if constexpr (PRO) {
-    // the first loads of W are under way while the rows are made
-    u32x4_t wv[U][NG], av[U][MT];
-    load_w(k0, wv);
-    make_rows();
-    for (int k = k0; k < k1; k += 32 * U) {
-      if (k != k0) load_w(k, wv);
-      load_a(k, av);
-      products(wv, av);
-    }
-  } else {
+  {
     for (int k = k0; k < k1; k += 32 * U) {
       // the loads of W and of A alternate, in the order of K
       u32x4_t wv[U][NG], av[U][MT];
@@ -942,7 +865,18 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny_kernel(
   for (int t = 0; t < NG * MT; ++t)
 #pragma unroll
     for (int v = 0; v < 4; ++v) red[wave][t][lane][v] = acc[t][v];
+  // 1 / rms of the rows (RowScale): wave w makes it for rows w, w + NW, ...
+  __shared__ float row_scale[16 * MT];
+  if (rsc.ss != nullptr) {
+    for (int m = wave; m < M; m += NW) {
+      float part = 0.f;
+      for (int p = lane; p < rsc.n_parts; p += WAVE) part += rsc.ss[(size_t)p * M + m];
+      part = wave_sum(part);
+      if (lane == 0) row_scale[m] = 1.0f / sqrtf(part / (float)K + rsc.eps);
+    }
+  }
   __syncthreads();
+  auto scale_of = [&](int gm) { return rsc.ss != nullptr ? row_scale[gm] : 1.0f; };
   // the first MT waves each sum one row tile over the NW partial results, in a fixed order
   if (EPI == 0 && NT > 1) {
     // waves take the NT * MT tiles in turn
@@ -958,7 +892,7 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny_kernel(
         float sum = red[0][tile][lane][v];
 #pragma unroll
         for (int w = 1; w < NW; ++w) sum += red[w][tile][lane][v];
-        store_out(C + (size_t)gm * ldc + gnr, sum + bv);
+        store_out(C + (size_t)gm * ldc + gnr, sum * scale_of(gm) + bv);
       }
     }
   } else if (wave < MT && gn < N && (EPI != 3 || col < 8)) {
@@ -968,14 +902,16 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny_kernel(
     for (int v = 0; v < 4; ++v) {
       const int gm = t * 16 + 4 * (lane / 16) + v;
       if (gm < M) {
+        const float rs = scale_of(gm);
         float sum = red[0][t][lane][v];
 #pragma unroll
         for (int w = 1; w < NW; ++w) sum += red[w][t][lane][v];
+        sum *= rs;
         if (EPI == 1) {
           float up = red[0][MT + t][lane][v];
 #pragma unroll
           for (int w = 1; w < NW; ++w) up += red[w][MT + t][lane][v];
-          store_out(C + (size_t)gm * ldc + gn, silu_f(sum) * up);
+          store_out(C + (size_t)gm * ldc + gn, silu_f(sum) * (up * rs));
         } else if (EPI == 2 || EPI == 3) {
           // where the other two gates of this channel lie: EPI 2 in row groups 1 and 2 of this
           // lane, EPI 3 the C gate 8 columns further in group 0 and the x gate in group 1
@@ -987,6 +923,8 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny_kernel(
             cg += red[w][cg_t][cg_lane][v];
             xg += red[w][xg_t][lane][v];
           }
+          cg *= rs;
+          xg *= rs;
           float bg = sum;
           if (bias) {
             bg += bias[gn];
@@ -1009,47 +947,70 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny_kernel(
           }
           s += wc[H] * bx;
           store_out(C + (size_t)gm * ldc + gn, to_f32(f32_to_bf16(cg)) * s);
+        } else if (EPI == 0 && ro.resid != nullptr) {
+          // the result joins the residual stream here (ResidOut)
+          float* rp = ro.resid + (size_t)gm * ro.ldr + gn;
+          const float x = *rp + (sum + bv);
+          *rp = x;
+          if (ro.rows != nullptr) {
+            const size_t at = ro.rows_frag ? ((size_t)(gn / 8) * 16 + gm) * 8 + gn % 8
+                                           : (size_t)gm * N + gn;
+            ro.rows[at] = f32_to_bf16(x * ro.norm_w[gn]);
+          }
         } else {
           store_out(C + (size_t)gm * ldc + gn, sum + bv);
         }
       }
     }
   }
+  if (EPI == 0 && NT == 1 && MT == 1 && ro.rows != nullptr && wave == 0) {
+    // sums of squares of the new residual over this block's 16 columns, row by row: a lane
+    // holds column lane % 16 of rows 4 (lane / 16) + v and reads back what it has just written
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+      const int gm = 4 * (lane / 16) + v;
+      float x = 0.f;
+      if (gm < M && gn < N) x = ro.resid[(size_t)gm * ro.ldr + gn];
+      float q = x * x;
+      q += __shfl_xor(q, 1, WAVE);
+      q += __shfl_xor(q, 2, WAVE);
+      q += __shfl_xor(q, 4, WAVE);
+      q += __shfl_xor(q, 8, WAVE);
+      if (lane % 16 == 0 && gm < M) ro.ss[(size_t)blockIdx.x * M + gm] = q;
+    }
+  }
 }
+
+struct Fuse {
+  RowScale rsc;
+  ResidOut ro;
+};
 
 template <typename TO, int MT, int NW, int EPI, int NT = 1>
 static void launch_skinny(const bf16_t* A, const bf16_t* W, const float* bias, TO* C, int M, int N,
                           int K, int lda, int ldc, int ksplit, ConvStep cs, hipStream_t stream,
-                          const NormIn* nin = nullptr, const bf16_t* Wf = nullptr,
-                          int a_frag = 0) {
+                          const Fuse& fuse = Fuse{}, const bf16_t* Wf = nullptr, int a_frag = 0) {
   // Wf: the copy of W in fragment order (see the kernel), or null
   const int w_frag = Wf != nullptr;
   if (Wf) W = Wf;
   const dim3 grid(EPI == 3 ? (N + 7) / 8 : (N + 16 * NT - 1) / (16 * NT), ksplit);
-  if constexpr (MT == 1 && NT == 1 && EPI != 2) {
-    if (nin) {
-      hipLaunchKernelGGL((gemm_bf16_skinny_kernel<TO, MT, NW, EPI, NT, true>), grid,
-                         dim3(NW * WAVE), 0, stream, A, W, bias, C, M, N, K, lda, ldc, cs, *nin,
-                         w_frag, 0);
-      return;
-    }
-  }
   hipLaunchKernelGGL((gemm_bf16_skinny_kernel<TO, MT, NW, EPI, NT>), grid, dim3(NW * WAVE), 0,
-                     stream, A, W, bias, C, M, N, K, lda, ldc, cs, NormIn{}, w_frag, a_frag);
+                     stream, A, W, bias, C, M, N, K, lda, ldc, cs, fuse.rsc, fuse.ro, w_frag,
+                     a_frag);
 }
 
 // more waves a block when there are few blocks, so that about 2048 waves or more stream W
 template <typename TO, int MT, int EPI>
 static void launch_skinny_mt(const bf16_t* A, const bf16_t* W, const float* bias, TO* C, int M,
                              int N, int K, int lda, int ldc, int ksplit, ConvStep cs,
-                             hipStream_t stream, const NormIn* nin = nullptr,
+                             hipStream_t stream, const Fuse& fuse = Fuse{},
                              const bf16_t* Wf = nullptr, int a_frag = 0) {
   // several row tiles and a plain product: a wave takes two column tiles for every fragment
   // of A it loads, which halves the reads of A (every block reads all of it)
   if constexpr (EPI == 0 && MT >= 2) {
     if (N >= 64) {
       launch_skinny<TO, MT, 4, EPI, 2>(A, W, bias, C, M, N, K, lda, ldc, ksplit, cs, stream,
-                                       nullptr, Wf, a_frag);
+                                       Fuse{}, Wf, a_frag);
       return;
     }
   }
@@ -1058,9 +1019,9 @@ static void launch_skinny_mt(const bf16_t* A, const bf16_t* W, const float* bias
   // With W in fragment order one tile a wave is the faster up to 11 rows (50 against 56 us at 8
   // rows, 56 either way at 12, 62 against 56 at 16).
   if constexpr (EPI == 0 && MT == 1) {
-    if (!nin && M >= (Wf ? 12 : 8) && (long)(N / 64) * ksplit >= 512) {
+    if (!fuse.ro.resid && M >= (Wf ? 12 : 8) && (long)(N / 64) * ksplit >= 512) {
       launch_skinny<TO, MT, 4, EPI, 4>(A, W, bias, C, M, N, K, lda, ldc, ksplit, cs, stream,
-                                       nullptr, Wf, a_frag);
+                                       fuse, Wf, a_frag);
       return;
     }
   }
@@ -1069,13 +1030,13 @@ static void launch_skinny_mt(const bf16_t* A, const bf16_t* W, const float* bias
   constexpr int NG = EPI == 1 ? 2 : (EPI == 2 ? 3 : (EPI == 3 ? 2 : 1));
   constexpr int MAXW = 48 / (MT * NG);                    // 1 KB of LDS a wave, group and row tile
   if (blocks * 4 >= 2048 || kb <= 512 || MAXW < 8)
-    launch_skinny<TO, MT, 4, EPI>(A, W, bias, C, M, N, K, lda, ldc, ksplit, cs, stream, nin, Wf, a_frag);
+    launch_skinny<TO, MT, 4, EPI>(A, W, bias, C, M, N, K, lda, ldc, ksplit, cs, stream, fuse, Wf, a_frag);
   else if (blocks * 8 >= 2048 || kb <= 1024 || MAXW < 16)
     launch_skinny<TO, MT, (MAXW >= 8 ? 8 : 4), EPI>(A, W, bias, C, M, N, K, lda, ldc, ksplit, cs,
-                                                    stream, nin, Wf, a_frag);
+                                                    stream, fuse, Wf, a_frag);
   else
     launch_skinny<TO, MT, (MAXW >= 16 ? 16 : 4), EPI>(A, W, bias, C, M, N, K, lda, ldc, ksplit, cs,
-                                                      stream, nin, Wf, a_frag);
+                                                      stream, fuse, Wf, a_frag);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -1309,9 +1270,15 @@ static bool launch_shared_rows(const bf16_t* A, const bf16_t* W, const float* bi
 template <typename TO, int EPI>
 static int launch_bf16(const bf16_t* A, const bf16_t* W, const float* bias, TO* C, int M, int N,
                        int K, int lda, int ldc, int force_kernel, int ksplit, hipStream_t stream,
-                       ConvStep cs = ConvStep{}, const bf16_t* Wf = nullptr, int a_frag = 0) {
+                       ConvStep cs = ConvStep{}, const bf16_t* Wf = nullptr, int a_frag = 0,
+                       const Fuse& fuse = Fuse{}) {
   // a_frag: the rows of A lie in fragment order, which only the kernel for 1 to 16 rows reads
   if (a_frag && (M > 16 || force_kernel == 1 || force_kernel >= 3)) return (int)hipErrorInvalidValue;
+  // so are the row scale and the residual epilogue (and the latter only with K in one piece)
+  const bool fused = fuse.rsc.ss != nullptr || fuse.ro.resid != nullptr;
+  if (fused && (M > 16 || force_kernel == 1 || force_kernel >= 3)) return (int)hipErrorInvalidValue;
+  if (fuse.ro.resid != nullptr && (EPI != 0 || ksplit != 1)) return (int)hipErrorInvalidValue;
+  if (fuse.rsc.ss != nullptr && ksplit != 1) return (int)hipErrorInvalidValue;
   // Wf: W once more in fragment order, for the kernels of 1 to 64 rows (see the first of them);
   // the others read W
   // N counts output columns; with the SwiGLU epilogue W has 2N rows
@@ -1338,19 +1305,19 @@ static int launch_bf16(const bf16_t* A, const bf16_t* W, const float* bias, TO* 
     const int mt = (M + 15) / 16;
     switch (mt) {
       case 1:
-        launch_skinny_mt<TO, 1, EPI>(A, W, bias, C, M, N, K, lda, ldc, ksplit, cs, stream, nullptr,
+        launch_skinny_mt<TO, 1, EPI>(A, W, bias, C, M, N, K, lda, ldc, ksplit, cs, stream, fuse,
                                      Wf, a_frag);
         break;
       case 2:
-        launch_skinny_mt<TO, 2, EPI>(A, W, bias, C, M, N, K, lda, ldc, ksplit, cs, stream, nullptr,
+        launch_skinny_mt<TO, 2, EPI>(A, W, bias, C, M, N, K, lda, ldc, ksplit, cs, stream, Fuse{},
                                      Wf);
         break;
       case 3:
-        launch_skinny_mt<TO, 3, EPI>(A, W, bias, C, M, N, K, lda, ldc, ksplit, cs, stream, nullptr,
+        launch_skinny_mt<TO, 3, EPI>(A, W, bias, C, M, N, K, lda, ldc, ksplit, cs, stream, Fuse{},
                                      Wf);
         break;
       default:
-        launch_skinny_mt<TO, 4, EPI>(A, W, bias, C, M, N, K, lda, ldc, ksplit, cs, stream, nullptr,
+        launch_skinny_mt<TO, 4, EPI>(A, W, bias, C, M, N, K, lda, ldc, ksplit, cs, stream, Fuse{},
                                      Wf);
         break;
     }
@@ -1373,35 +1340,62 @@ static bool frag_ok(const void* W_frag, int rows, int K) {
   return W_frag == nullptr || (K % 32 == 0 && rows % 16 == 0 && ((uintptr_t)W_frag % 16) == 0);
 }
 
+// The fused forms (at most 16 rows, see RowScale and ResidOut in the kernel for 1 to 16 rows):
+// scale_ss [scale_parts][M] (or null) scales every result row by 1 / sqrt(sum of its parts / K +
+// scale_eps); resid [M, ldr] (or null; float output, ksplit 1) receives the result added in place
+// instead of C, and with norm_w also rows_out (bf16(resid * norm_w), [M, N] or fragment order)
+// and ss_out [(N + 15) / 16][M].
+static bool fuse_ok(const Fuse& f, int M, int N, int K, int out_is_f32, int ksplit) {
+  if (f.rsc.ss != nullptr && (M > 16 || f.rsc.n_parts < 1 || ksplit != 1)) return false;
+  if (f.ro.resid != nullptr) {
+    if (M > 16 || !out_is_f32 || ksplit != 1 || f.ro.ldr < N) return false;
+    if (f.ro.norm_w != nullptr && (f.ro.rows == nullptr || f.ro.ss == nullptr)) return false;
+    if (f.ro.rows_frag && (N % 32)) return false;
+  } else if (f.ro.norm_w != nullptr || f.ro.rows != nullptr) {
+    return false;
+  }
+  return true;
+}
+
 extern "C" int kappai_gemm_bf16(const void* A, const void* W, const void* W_frag, const float* bias,
                                 void* C, int M, int N, int K, int lda, int ldc, int out_is_f32,
-                                int force_kernel, int ksplit, int a_frag, hipStream_t stream) {
+                                int force_kernel, int ksplit, int a_frag, const float* scale_ss,
+                                int scale_parts, float scale_eps, float* resid, int ldr,
+                                const float* norm_w, void* rows_out, int rows_frag, float* ss_out,
+                                hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
   if ((K % 8) || (lda % 8) || ksplit < 1 || ksplit > 64) return (int)hipErrorInvalidValue;
   if (!frag_ok(W_frag, N, K) || (a_frag && (K % 32))) return (int)hipErrorInvalidValue;
   if (force_kernel == 2 && M > 64) return (int)hipErrorInvalidValue;
   if (ksplit > 1 && !out_is_f32) return (int)hipErrorInvalidValue;
+  Fuse fuse{RowScale{scale_ss, scale_parts, scale_eps},
+            ResidOut{resid, ldr, resid && rows_out ? norm_w : nullptr,
+                     resid ? (bf16_t*)rows_out : nullptr, rows_frag, ss_out}};
+  if (!fuse_ok(fuse, M, N, K, out_is_f32, ksplit)) return (int)hipErrorInvalidValue;
   if (out_is_f32)
     return launch_bf16<float, 0>((const bf16_t*)A, (const bf16_t*)W, bias, (float*)C, M, N, K, lda,
                                  ldc, force_kernel, ksplit, stream, ConvStep{},
-                                 (const bf16_t*)W_frag, a_frag);
+                                 (const bf16_t*)W_frag, a_frag, fuse);
   return launch_bf16<bf16_t, 0>((const bf16_t*)A, (const bf16_t*)W, bias, (bf16_t*)C, M, N, K, lda,
                                 ldc, force_kernel, 1, stream, ConvStep{}, (const bf16_t*)W_frag,
-                                a_frag);
+                                a_frag, fuse);
 }
 
 // C[M, F] = silu(A Wg^T) * (A Wu^T) with W = gate and up rows interleaved in groups of 16,
 // [2F, K]; F must be a multiple of 16.
 extern "C" int kappai_gemm_bf16_swiglu(const void* A, const void* W, const void* W_frag, void* C,
                                        int M, int F, int K, int lda, int ldc, int force_kernel,
-                                       int a_frag, hipStream_t stream) {
+                                       int a_frag, const float* scale_ss, int scale_parts,
+                                       float scale_eps, hipStream_t stream) {
   if (M <= 0 || F <= 0) return 0;
   if ((K % 8) || (lda % 8) || (F % 16)) return (int)hipErrorInvalidValue;
   if (force_kernel == 2 && M > 64) return (int)hipErrorInvalidValue;
   if (!frag_ok(W_frag, 2 * F, K) || (a_frag && (K % 32))) return (int)hipErrorInvalidValue;
+  Fuse fuse{RowScale{scale_ss, scale_parts, scale_eps}, ResidOut{}};
+  if (!fuse_ok(fuse, M, F, K, 0, 1)) return (int)hipErrorInvalidValue;
   return launch_bf16<bf16_t, 1>((const bf16_t*)A, (const bf16_t*)W, nullptr, (bf16_t*)C, M, F, K,
                                 lda, ldc, force_kernel, 1, stream, ConvStep{},
-                                (const bf16_t*)W_frag, a_frag);
+                                (const bf16_t*)W_frag, a_frag, fuse);
 }
 
 // Conv layer decode step in one kernel: C[M, D] = Cgate * conv(Bgate * x | state) from A [M, K]
@@ -1412,11 +1406,14 @@ extern "C" int kappai_gemm_bf16_shortconv_step(const void* A, const void* W, con
                                                const float* taps, const float* conv_bias,
                                                float* state, const int* seg_pos0,
                                                const int* seg_slot, int L, int a_frag,
-                                               hipStream_t stream) {
+                                               const float* scale_ss, int scale_parts,
+                                               float scale_eps, hipStream_t stream) {
   if (M <= 0 || D <= 0) return 0;
   if ((K % 8) || (lda % 8) || (D % 16) || M > 64 || L < 2) return (int)hipErrorInvalidValue;
   if (!frag_ok(W_frag, 3 * D, K) || (a_frag && ((K % 32) || M > 16)))
     return (int)hipErrorInvalidValue;
+  Fuse fuse{RowScale{scale_ss, scale_parts, scale_eps}, ResidOut{}};
+  if (!fuse_ok(fuse, M, D, K, 0, 1)) return (int)hipErrorInvalidValue;
   const bf16_t* wf = (const bf16_t*)W_frag;
   ConvStep cs{taps, conv_bias, state, seg_pos0, seg_slot, L};
   if (D / 16 < 256) {
@@ -1426,86 +1423,23 @@ extern "C" int kappai_gemm_bf16_shortconv_step(const void* A, const void* W, con
     bf16_t* c = (bf16_t*)C;
     switch ((M + 15) / 16) {
       case 1:
-        launch_skinny_mt<bf16_t, 1, 3>(a, w, bias, c, M, D, K, lda, D, 1, cs, stream, nullptr, wf,
+        launch_skinny_mt<bf16_t, 1, 3>(a, w, bias, c, M, D, K, lda, D, 1, cs, stream, fuse, wf,
                                        a_frag);
         break;
       case 2:
-        launch_skinny_mt<bf16_t, 2, 3>(a, w, bias, c, M, D, K, lda, D, 1, cs, stream, nullptr, wf);
+        launch_skinny_mt<bf16_t, 2, 3>(a, w, bias, c, M, D, K, lda, D, 1, cs, stream, Fuse{}, wf);
         break;
       case 3:
-        launch_skinny_mt<bf16_t, 3, 3>(a, w, bias, c, M, D, K, lda, D, 1, cs, stream, nullptr, wf);
+        launch_skinny_mt<bf16_t, 3, 3>(a, w, bias, c, M, D, K, lda, D, 1, cs, stream, Fuse{}, wf);
         break;
       default:
-        launch_skinny_mt<bf16_t, 4, 3>(a, w, bias, c, M, D, K, lda, D, 1, cs, stream, nullptr, wf);
+        launch_skinny_mt<bf16_t, 4, 3>(a, w, bias, c, M, D, K, lda, D, 1, cs, stream, Fuse{}, wf);
         break;
     }
     KAPPAI_RETURN_LAUNCH_STATUS();
   }
   return launch_bf16<bf16_t, 2>((const bf16_t*)A, (const bf16_t*)W, bias, (bf16_t*)C, M, D, K, lda,
-                                D, 2, 1, stream, cs, wf, a_frag);
-}
-
-// The same products for at most NORM_ROWS rows that are still to be made: A = RMSNorm(resid +
-// delta) * norm_w, computed inside the product kernel (see NormIn).  delta: null, bfloat16 [M, K]
-// (delta_f32 = 0, n_parts = 1) or float [n_parts][M][K]; resid_out [M, K] receives resid + delta
-// when there is a delta (it must not be resid).  K a multiple of 8, at most NORM_MAX_K.
-static bool norm_in_ok(int M, int K, const NormIn& n) {
-  if (M < 1 || M > NORM_ROWS || (K % 8) || K > NORM_MAX_K || !n.resid || !n.w) return false;
-  if (n.delta && (n.n_parts < 1 || (!n.delta_f32 && n.n_parts != 1) || !n.resid_out ||
-                  n.resid_out == n.resid))
-    return false;
-  return true;
-}
-
-extern "C" int kappai_gemm_bf16_normed(const float* resid, const void* delta, int delta_f32,
-                                       int n_parts, const float* norm_w, float eps,
-                                       float* resid_out, const void* W, const void* W_frag,
-                                       const float* bias, void* C, int M, int N, int K, int ldc,
-                                       int out_is_f32, int ksplit, hipStream_t stream) {
-  if (N <= 0) return 0;
-  if (!frag_ok(W_frag, N, K)) return (int)hipErrorInvalidValue;
-  NormIn nin{resid, delta, delta ? n_parts : 0, delta_f32, norm_w, eps, delta ? resid_out : nullptr};
-  if (!norm_in_ok(M, K, nin) || ksplit < 1 || ksplit > 64 || (ksplit > 1 && !out_is_f32))
-    return (int)hipErrorInvalidValue;
-  if (out_is_f32)
-    launch_skinny_mt<float, 1, 0>(nullptr, (const bf16_t*)W, bias, (float*)C, M, N, K, K, ldc,
-                                  ksplit, ConvStep{}, stream, &nin, (const bf16_t*)W_frag);
-  else
-    launch_skinny_mt<bf16_t, 1, 0>(nullptr, (const bf16_t*)W, bias, (bf16_t*)C, M, N, K, K, ldc, 1,
-                                   ConvStep{}, stream, &nin, (const bf16_t*)W_frag);
-  KAPPAI_RETURN_LAUNCH_STATUS();
-}
-
-// The conv layer's decode step (8 channels a block) on rows that are still to be made (see
-// NormIn): RMSNorm, in_proj, gates, FIR and state shift of a single decoded row in one kernel.
-// D below 4096 (the 16-channel form takes no pending norm), K at most NORM_MAX_K.
-extern "C" int kappai_gemm_bf16_shortconv_step_normed(
-    const float* resid, const void* delta, int delta_f32, int n_parts, const float* norm_w, float eps,
-    float* resid_out, const void* W, const void* W_frag, const float* bias, void* C, int M, int D,
-    int K, const float* taps, const float* conv_bias, float* state, const int* seg_pos0,
-    const int* seg_slot, int L, hipStream_t stream) {
-  if (D <= 0) return 0;
-  NormIn nin{resid, delta, delta ? n_parts : 0, delta_f32, norm_w, eps, delta ? resid_out : nullptr};
-  if (!norm_in_ok(M, K, nin) || (D % 16) || D / 16 >= 256 || L < 2 || !frag_ok(W_frag, 3 * D, K))
-    return (int)hipErrorInvalidValue;
-  ConvStep cs{taps, conv_bias, state, seg_pos0, seg_slot, L};
-  launch_skinny_mt<bf16_t, 1, 3>(nullptr, (const bf16_t*)W, bias, (bf16_t*)C, M, D, K, K, D, 1, cs,
-                                 stream, &nin, (const bf16_t*)W_frag);
-  KAPPAI_RETURN_LAUNCH_STATUS();
-}
-
-extern "C" int kappai_gemm_bf16_swiglu_normed(const float* resid, const void* delta, int delta_f32,
-                                              int n_parts, const float* norm_w, float eps,
-                                              float* resid_out, const void* W,
-                                              const void* W_frag, void* C, int M, int F, int K,
-                                              int ldc, hipStream_t stream) {
-  if (F <= 0) return 0;
-  if (!frag_ok(W_frag, 2 * F, K)) return (int)hipErrorInvalidValue;
-  NormIn nin{resid, delta, delta ? n_parts : 0, delta_f32, norm_w, eps, delta ? resid_out : nullptr};
-  if (!norm_in_ok(M, K, nin) || (F % 16)) return (int)hipErrorInvalidValue;
-  launch_skinny_mt<bf16_t, 1, 1>(nullptr, (const bf16_t*)W, nullptr, (bf16_t*)C, M, F, K, K, ldc, 1,
-                                 ConvStep{}, stream, &nin, (const bf16_t*)W_frag);
-  KAPPAI_RETURN_LAUNCH_STATUS();
+                                D, 2, 1, stream, cs, wf, a_frag, fuse);
 }
 
 // ---------------------------------------------------------------------------------------

@@ -121,6 +121,9 @@ def add_rmsnorm(resid: torch.Tensor, delta: Optional[torch.Tensor], weight: torc
     return FragmentRows(out, n, resid) if fragment else out
 
 
+FRAGMENT_ROWS_FROM = 8     # from this many rows on, rows for the next product go in fragment order
+
+
 class FragmentRows:
     """At most 16 normalised rows [n, D] of a decode step, stored in the order in which the
     product kernel for 1 to 16 rows loads its activations ([D / 32][(k % 32) / 8][16 rows][8
@@ -128,7 +131,7 @@ class FragmentRows:
     touches whole cache lines of neighbouring rows instead of half a line of every row.
     ``linear``, ``linear_swiglu`` and ``linear_shortconv_step`` take it in place of the rows;
     ``materialize`` gives the rows as an ordinary tensor.  ``resid_after`` is the residual the
-    norm has updated (the interface of ``PendingNorm``, so that a part takes either)."""
+    norm has updated (the interface of ``ScaledRows``, so that a part takes either)."""
 
     def __init__(self, data: torch.Tensor, n_rows: int, resid: torch.Tensor):
         self.data, self.resid_after = data, resid
@@ -145,54 +148,57 @@ class FragmentRows:
                 .contiguous())
 
 
-NORM_FUSE_MAX_ROWS = 1        # rows a product kernel normalises by itself
-NORM_FUSE_MAX_WIDTH = 4096
+FUSED_MAX_ROWS = 16        # rows of a decode step whose products fold norm and residual sum in
 
 
-class PendingNorm:
-    """Rows that are still to be made: ``RMSNorm(resid + delta) * weight``.  ``linear`` and
-    ``linear_swiglu`` take it in place of their input and make the rows inside the product
-    kernel (every block for itself), which saves the kernel between two products of a decode
-    step with very few rows.  ``resid`` is not changed; after the product ``resid_after`` holds
-    resid + delta (a new tensor, or ``resid`` itself without a delta).  ``materialize`` runs the
-    ordinary kernel instead."""
+class Added:
+    """What a product hands back when it has added its result into the residual stream itself
+    (``AddInto``): there is no update left to add.  ``resid`` is the stream it added to."""
 
-    def __init__(self, resid: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Tensor,
-                 eps: float, out_dtype):
-        self.resid, self.delta, self.weight, self.eps, self.dtype = resid, delta, weight, eps, out_dtype
-        self.shape, self.device = resid.shape, resid.device
-        self.resid_after: Optional[torch.Tensor] = None
+    def __init__(self, resid: torch.Tensor):
+        self.resid = resid
 
-    @staticmethod
-    def fits(resid: torch.Tensor, delta: Optional[torch.Tensor], out_dtype) -> bool:
-        if not (resid.is_cuda and out_dtype == BF16 and resid.dtype == F32 and resid.dim() == 2
-                and resid.is_contiguous()):
-            return False
-        M, D = resid.shape
-        if not (1 <= M <= NORM_FUSE_MAX_ROWS and D % 8 == 0 and D <= NORM_FUSE_MAX_WIDTH):
-            return False
-        if delta is None:
-            return True
-        if not delta.is_contiguous():
-            return False
-        if delta.dim() == 3:
-            return delta.dtype == F32 and delta.shape[1:] == resid.shape and delta.shape[0] <= 8
-        return delta.shape == resid.shape and delta.dtype in (F32, BF16)
+
+class ScaledRows(Added):
+    """At most 16 rows of a decode step, on their way from a product that added its result into
+    the residual stream (``AddInto`` with a norm weight) to the product after the RMSNorm that
+    follows: ``data`` holds bf16(resid * weight), not yet divided by the rows' root mean square
+    ([n, D], or 16 rows in fragment order), and ``ss`` [parts, n] the sums of resid^2 over ranges
+    of columns.  ``linear``, ``linear_swiglu`` and ``linear_shortconv_step`` take it in place of
+    the normalised rows and scale their results by 1 / sqrt(sum of the parts / D + eps), which is
+    the same product (RMSNorm(x) W^T = (x * w) W^T / rms(x)) without a kernel in between.
+    ``materialize`` runs the ordinary norm kernel on the residual instead.  ``resid_after`` is
+    the residual to go on with (the interface of ``FragmentRows``)."""
+
+    def __init__(self, data: torch.Tensor, n_rows: int, fragment: bool, ss: torch.Tensor,
+                 weight: torch.Tensor, eps: float, resid: torch.Tensor):
+        super().__init__(resid)
+        self.data, self.fragment, self.ss, self.weight, self.eps = data, fragment, ss, weight, eps
+        self.resid_after = resid
+        self.shape = torch.Size((n_rows, resid.shape[1]))
+        self.device, self.dtype = data.device, data.dtype
 
     def materialize(self) -> torch.Tensor:
-        x = add_rmsnorm(self.resid, self.delta, self.weight, self.eps, self.dtype)
-        self.resid_after = self.resid
-        return x
+        return add_rmsnorm(self.resid, None, self.weight, self.eps, self.dtype)
 
-    def _kernel_args(self):
-        """(resid, delta, delta_f32, n_parts, weight, eps, resid_out) for the product kernels."""
-        if self.resid_after is None:
-            self.resid_after = self.resid if self.delta is None else torch.empty_like(self.resid)
-        d = self.delta
-        n_parts = d.shape[0] if d is not None and d.dim() == 3 else 1
-        return (_ptr(self.resid), _ptr(d), _c_int(1 if d is not None and d.dtype == F32 else 0),
-                _c_int(n_parts), _ptr(self.weight), _c_float(self.eps),
-                _ptr(self.resid_after if d is not None else None))
+    def _scale_args(self):
+        return (_ptr(self.ss), _c_int(self.ss.shape[0]), _c_float(self.eps))
+
+
+_NO_SCALE = (_vp(0), _c_int(0), _c_float(0.0))
+
+
+class AddInto:
+    """Asks a product to add its result into ``resid`` (float32 [M, N], in place, in float32)
+    instead of returning it (kappai fuses the residual sum into the product the same way,
+    src/recipe/graph_passes.c:455).  With ``norm_weight`` (and ``eps``) the RMSNorm that follows
+    is folded in as well: the product hands back ``ScaledRows`` for the product after that norm.
+    A product that cannot do it (more than 16 rows, float32 weights, ...) returns its result as
+    always, and the caller goes on as without this."""
+
+    def __init__(self, resid: torch.Tensor, norm_weight: Optional[torch.Tensor] = None,
+                 eps: float = 0.0):
+        self.resid, self.norm_weight, self.eps = resid, norm_weight, float(eps)
 
 
 def add_residual(resid: torch.Tensor, delta: torch.Tensor) -> None:
@@ -328,21 +334,29 @@ def split_k_for(M: int, N: int, K: int) -> int:
 def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
            out_dtype=None, force_kernel: int = 0, partial_sums: bool = False,
            split_k: Optional[int] = None,
-           weight_frag: Optional[torch.Tensor] = None) -> torch.Tensor:
+           weight_frag: Optional[torch.Tensor] = None,
+           add_into: Optional[AddInto] = None):
     """``x [M, K] @ weight[N, K]^T (+ bias)``.  A bfloat16 matrix runs on the matrix cores
     with float accumulation; a float32 matrix runs in true 32-bit arithmetic, whatever the
     activations' dtype.  ``x`` may be a view with a row stride.  With ``partial_sums`` the
     result may come back as float32 [S, M, N], the sums over S ranges of K, for a consumer
     that adds them (a matrix with few columns is then streamed by enough blocks).  ``x`` may
-    be a ``PendingNorm``: the rows are then made inside the product kernel.  ``weight_frag``
-    (``fragment_order(weight)``) is read in place of ``weight`` by the kernel for 1 to 16 rows."""
-    if isinstance(x, PendingNorm):
-        if (weight.dtype != BF16 or force_kernel or weight.dim() != 2
-                or weight.shape[1] != x.shape[1] or weight.data_ptr() % 16):
-            x = x.materialize()
-        else:
-            return _linear_normed(x, weight, bias, out_dtype, partial_sums, split_k, weight_frag)
+    be ``ScaledRows`` or ``FragmentRows``.  ``weight_frag`` (``fragment_order(weight)``) is read
+    in place of ``weight`` by the kernel for 1 to 16 rows.  ``add_into``: see ``AddInto``; the
+    result is then ``Added`` or ``ScaledRows`` when the product could add its result itself."""
     a_frag = 0
+    scale = None
+    if isinstance(x, ScaledRows):
+        if (weight.dtype != BF16 or force_kernel not in (0, 2) or weight.dim() != 2
+                or weight.shape[1] != x.shape[1] or weight.data_ptr() % 16
+                or weight.shape[1] % 8):
+            x = x.materialize()          # only the kernel for 1 to 16 rows scales its results
+        else:
+            scale, partial_sums = x, False          # its kernel keeps K in one piece
+            if x.fragment:
+                a_frag, n_frag, x = 1, x.shape[0], x.data
+            else:
+                x = x.data
     if isinstance(x, FragmentRows):
         if (weight.dtype != BF16 or force_kernel not in (0, 2) or weight.dim() != 2
                 or weight.shape[1] != x.shape[1] or weight.data_ptr() % 16):
@@ -374,6 +388,7 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] =
     if not (K % 8 == 0 and lda % 8 == 0 and xb.data_ptr() % 16 == 0
             and weight.data_ptr() % 16 == 0):
         # the matrix-core kernels read 16 bytes at a time; anything else goes the plain way
+        _need(scale is None, "linear: scaled rows reached the plain kernel")
         _need(not force_kernel,
               lambda: f"linear: K ({K}) and the row stride ({lda}) must be multiples of 8 and "
                       "the tensors 16-byte aligned for the kernel that was asked for")
@@ -384,6 +399,30 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] =
             _c_int(lda), _c_int(N), _c_int(0 if out_dtype == BF16 else 1), _stream()),
             "gemm_bf16_any")
         return out
+    scale_args = scale._scale_args() if scale is not None else _NO_SCALE
+    if (add_into is not None and M <= FUSED_MAX_ROWS and force_kernel in (0, 2)
+            and add_into.resid.dtype == F32 and add_into.resid.is_contiguous()
+            and tuple(add_into.resid.shape) == (M, N)):
+        # the result joins the residual stream inside the kernel
+        resid, nw = add_into.resid, add_into.norm_weight
+        _gpu("resid", resid, F32)
+        rows = ss = None
+        fragment = False
+        if nw is not None:
+            _gpu("norm_weight", nw, F32)
+            _need(nw.shape == (N,), lambda: f"linear: norm weight {tuple(nw.shape)} for N={N}")
+            fragment = FRAGMENT_ROWS_FROM <= M and FragmentRows.fits(M, N, BF16)
+            rows = torch.empty((16 if fragment else M, N), dtype=BF16, device=x.device)
+            ss = torch.empty(((N + 15) // 16, M), dtype=F32, device=x.device)
+        check(library("gemm").kappai_gemm_bf16(
+            _ptr(xb), _ptr(weight), _frag(weight, weight_frag), _ptr(bias), _vp(0), _c_int(M),
+            _c_int(N), _c_int(K), _c_int(lda), _c_int(N), _c_int(1), _c_int(force_kernel),
+            _c_int(1), _c_int(a_frag), *scale_args, _ptr(resid), _c_int(resid.stride(0)),
+            _ptr(nw), _ptr(rows), _c_int(1 if fragment else 0), _ptr(ss), _stream()),
+            "gemm_bf16 (into the residual)")
+        if nw is None:
+            return Added(resid)
+        return ScaledRows(rows, M, fragment, ss, nw, add_into.eps, resid)
     ksplit = (split_k or split_k_for(M, N, K)) if partial_sums else 1
     if ksplit > 1:
         out = torch.empty((ksplit, M, N), dtype=F32, device=x.device)
@@ -395,30 +434,8 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] =
         _ptr(xb), _ptr(weight), _frag(weight, weight_frag), _ptr(bias), _ptr(out), _c_int(M),
         _c_int(N), _c_int(K),
         _c_int(lda), _c_int(N), _c_int(out_is_f32), _c_int(force_kernel), _c_int(ksplit),
-        _c_int(a_frag), _stream()), "gemm_bf16")
-    return out
-
-
-def _linear_normed(x: PendingNorm, weight, bias, out_dtype, partial_sums, split_k,
-                   weight_frag=None) -> torch.Tensor:
-    _gpu("weight", weight, BF16)
-    M, K = x.shape
-    N = weight.shape[0]
-    out_dtype = out_dtype or x.dtype
-    if bias is not None:
-        _gpu("bias", bias, F32)
-        _need(bias.shape == (N,), lambda: f"linear: bias {tuple(bias.shape)} for N={N}")
-    ksplit = (split_k or split_k_for(M, N, K)) if partial_sums else 1
-    if ksplit > 1:
-        out = torch.empty((ksplit, M, N), dtype=F32, device=x.device)
-        out_is_f32 = 1
-    else:
-        out = torch.empty((M, N), dtype=out_dtype, device=x.device)
-        out_is_f32 = 0 if out_dtype == BF16 else 1
-    check(library("gemm").kappai_gemm_bf16_normed(
-        *x._kernel_args(), _ptr(weight), _frag(weight, weight_frag), _ptr(bias), _ptr(out),
-        _c_int(M), _c_int(N), _c_int(K),
-        _c_int(N), _c_int(out_is_f32), _c_int(ksplit), _stream()), "gemm_bf16_normed")
+        _c_int(a_frag), *scale_args, _vp(0), _c_int(0), _vp(0), _vp(0), _c_int(0), _vp(0),
+        _stream()), "gemm_bf16")
     return out
 
 
@@ -441,22 +458,16 @@ def linear_swiglu(x: torch.Tensor, weight: torch.Tensor, force_kernel: int = 0,
                   weight_frag: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``silu(x Wg^T) * (x Wu^T)`` in one kernel: ``weight`` [2F, K] holds the gate and up
     matrices interleaved by ``interleave_gate_up``; bfloat16 only.  Returns [M, F].  ``x`` may
-    be a ``PendingNorm``."""
-    if isinstance(x, PendingNorm):
-        if (force_kernel or weight.dtype != BF16 or weight.dim() != 2
+    be ``ScaledRows`` or ``FragmentRows``."""
+    scale = None
+    if isinstance(x, ScaledRows):
+        if (force_kernel not in (0, 2) or weight.dtype != BF16 or weight.dim() != 2
                 or weight.shape[1] != x.shape[1] or weight.shape[0] % (2 * SWIGLU_GROUP)
-                or weight.data_ptr() % 16):
+                or weight.data_ptr() % 16 or weight.shape[1] % 8):
             x = x.materialize()
         else:
-            _gpu("weight", weight, BF16)
-            M, K = x.shape
-            F = weight.shape[0] // 2
-            out = torch.empty((M, F), dtype=BF16, device=x.device)
-            check(library("gemm").kappai_gemm_bf16_swiglu_normed(
-                *x._kernel_args(), _ptr(weight), _frag(weight, weight_frag), _ptr(out), _c_int(M),
-                _c_int(F), _c_int(K),
-                _c_int(F), _stream()), "gemm_bf16_swiglu_normed")
-            return out
+            scale = x
+            x = FragmentRows(x.data, x.shape[0], x.resid) if x.fragment else x.data
     a_frag, n_frag = 0, 0
     if isinstance(x, FragmentRows):
         if force_kernel not in (0, 2) or weight.dim() != 2 or weight.shape[1] != x.shape[1]:
@@ -481,7 +492,8 @@ def linear_swiglu(x: torch.Tensor, weight: torch.Tensor, force_kernel: int = 0,
     check(library("gemm").kappai_gemm_bf16_swiglu(
         _ptr(x), _ptr(weight), _frag(weight, weight_frag), _ptr(out), _c_int(M), _c_int(F), _c_int(K),
         _c_int(lda), _c_int(F),
-        _c_int(force_kernel), _c_int(a_frag), _stream()), "gemm_bf16_swiglu")
+        _c_int(force_kernel), _c_int(a_frag),
+        *(scale._scale_args() if scale is not None else _NO_SCALE), _stream()), "gemm_bf16_swiglu")
     return out
 
 
@@ -493,23 +505,23 @@ def linear_shortconv_step(x: torch.Tensor, in_proj: torch.Tensor, in_bias: Optio
     """A conv layer's decode step in one kernel, for a batch in which every row is its own
     segment: ``proj = x in_proj^T (+ bias)`` cut into (B | C | x), ``C * conv(B * x)`` with the
     rows' state slots read and shifted.  bfloat16, at most 64 rows, width a multiple of 16.
-    Equals ``shortconv(linear(x, in_proj, in_bias), ...)``.  ``x`` may be a ``PendingNorm``
-    (widths below 4096): the kernel then makes the normalised row itself as well; or
+    Equals ``shortconv(linear(x, in_proj, in_bias), ...)``.  ``x`` may be ``ScaledRows`` or
     ``FragmentRows``."""
-    pending = x if isinstance(x, PendingNorm) else None
-    if pending is not None and not (in_proj.dtype == BF16 and in_proj.dim() == 2
-                                    and taps.dim() == 2 and taps.shape[0] // 16 < 256
-                                    and in_proj.shape[1] == x.shape[1]
-                                    and in_proj.data_ptr() % 16 == 0):
-        x, pending = x.materialize(), None
+    scale = None
+    if isinstance(x, ScaledRows):
+        if (in_proj.dtype != BF16 or in_proj.dim() != 2 or in_proj.shape[1] != x.shape[1]
+                or in_proj.data_ptr() % 16 or in_proj.shape[1] % 8):
+            x = x.materialize()
+        else:
+            scale = x
+            x = FragmentRows(x.data, x.shape[0], x.resid) if x.fragment else x.data
     a_frag, n_frag = 0, 0
     if isinstance(x, FragmentRows):
         if in_proj.dim() != 2 or in_proj.shape[1] != x.shape[1]:
             x = x.materialize()
         else:
             a_frag, n_frag, x = 1, x.shape[0], x.data
-    if pending is None:
-        _gpu("x", x, BF16, contiguous=False)
+    _gpu("x", x, BF16, contiguous=False)
     _gpu("in_proj", in_proj, BF16)
     _gpu("taps", taps, F32)
     _gpu("state", state, F32)
@@ -524,28 +536,21 @@ def linear_shortconv_step(x: torch.Tensor, in_proj: torch.Tensor, in_bias: Optio
     _need(seg_pos0.shape == (M,) and seg_slot.shape == (M,), "one segment a row")
     _need(L >= 2 and state.dim() == 3 and state.shape[1:] == (D, L - 1),
           lambda: f"state {tuple(state.shape)} for D={D}, L={L}")
-    if pending is None:
-        lda = x.stride(0) if M > 1 else K
-        _need((x.stride(1) == 1 or K == 1) and K % 8 == 0 and lda % 8 == 0
-              and x.data_ptr() % 16 == 0 and in_proj.data_ptr() % 16 == 0,
-              "linear_shortconv_step: K and the row stride must be multiples of 8, tensors aligned")
+    lda = x.stride(0) if M > 1 else K
+    _need((x.stride(1) == 1 or K == 1) and K % 8 == 0 and lda % 8 == 0
+          and x.data_ptr() % 16 == 0 and in_proj.data_ptr() % 16 == 0,
+          "linear_shortconv_step: K and the row stride must be multiples of 8, tensors aligned")
     for n, t, shp in (("in_bias", in_bias, (3 * D,)), ("conv_bias", conv_bias, (D,))):
         if t is not None:
             _gpu(n, t, F32)
             _need(t.shape == shp, lambda: f"{n} must be {shp}")
     out = torch.empty((M, D), dtype=BF16, device=x.device)
-    if pending is not None:
-        check(library("gemm").kappai_gemm_bf16_shortconv_step_normed(
-            *pending._kernel_args(), _ptr(in_proj), _frag(in_proj, weight_frag), _ptr(in_bias),
-            _ptr(out), _c_int(M), _c_int(D), _c_int(K), _ptr(taps), _ptr(conv_bias), _ptr(state),
-            _ptr(seg_pos0), _ptr(seg_slot), _c_int(L), _stream()),
-            "gemm_bf16_shortconv_step_normed")
-        return out
     check(library("gemm").kappai_gemm_bf16_shortconv_step(
         _ptr(x), _ptr(in_proj), _frag(in_proj, weight_frag), _ptr(in_bias), _ptr(out), _c_int(M),
         _c_int(D), _c_int(K),
         _c_int(lda), _ptr(taps), _ptr(conv_bias), _ptr(state), _ptr(seg_pos0), _ptr(seg_slot),
-        _c_int(L), _c_int(a_frag), _stream()), "gemm_bf16_shortconv_step")
+        _c_int(L), _c_int(a_frag), *(scale._scale_args() if scale is not None else _NO_SCALE),
+        _stream()), "gemm_bf16_shortconv_step")
     return out
 
 

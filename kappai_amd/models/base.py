@@ -128,12 +128,18 @@ class Model:
             view = None
             if block.cache_spec() is not None:
                 view = cache.view(self.cache_id(ci))
-            h = block.forward(h, batch, view, shared_cache=call.reads_cache_of is not None)
+            shared = call.reads_cache_of is not None
+            if getattr(block, "takes_next_block", False):
+                nxt = (self.layers[self.schedule[ci + 1].layer] if ci + 1 < len(self.schedule)
+                       else None)
+                h = block.forward(h, batch, view, shared_cache=shared, next_block=nxt)
+            else:
+                h = block.forward(h, batch, view, shared_cache=shared)
         if batch.n_logit_rows == 0:
             return torch.empty((0, self.vocab_size), dtype=torch.float32, device=x.device)
         delta = summed_delta(self.final_norm, h.delta)
         if (getattr(self.final_norm, "can_defer", False)
-                and getattr(self.head, "takes_pending_norm", False)):
+                and getattr(self.head, "takes_deferred_rows", False)):
             xb = self.final_norm.add_norm(h.resid, delta, rows=batch.logit_rows, defer=True)
         else:
             xb = self.final_norm.add_norm(h.resid, delta, rows=batch.logit_rows)

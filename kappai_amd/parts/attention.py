@@ -23,7 +23,8 @@ from .linear import PARTIAL_SUMS_MIN_ROWS, Linear
 
 
 class GroupedQueryAttention(Mixer):
-    takes_pending_norm = True      # its first product may make the normalised rows itself
+    takes_deferred_rows = True     # its first product takes what ops.linear takes
+    adds_residual = True           # its last product can add into the residual stream
     q_tile_rows = ops.ATTENTION_TILE_ROWS     # the tiled attention kernel's rows a tile
 
     def __init__(self, prefix: str, width: int, num_heads: int, num_kv_heads: int, head_dim: int,
@@ -73,7 +74,7 @@ class GroupedQueryAttention(Mixer):
             self.q_norm_w = tensors[self._qn + ".weight"].to(torch.float32).contiguous()
             self.k_norm_w = tensors[self._kn + ".weight"].to(torch.float32).contiguous()
 
-    def forward(self, x, batch, cache, shared_cache: bool = False):
+    def forward(self, x, batch, cache, shared_cache: bool = False, into=None):
         H, G, d = self.H, self.G, self.d
         # decode with more than 16 rows: the projection may come as sums over ranges of its input
         # dimension (more blocks stream the matrix), which the next kernel adds up
@@ -92,7 +93,7 @@ class GroupedQueryAttention(Mixer):
                                   window=self.window or 0, q_tiles=batch.q_tiles,
                                   single_rows=batch.max_segment_rows == 1,
                                   max_position=batch.max_position)
-        return self.out.forward(ctx, partial_sums=True)
+        return self.out.forward(ctx, partial_sums=True, add_into=into)
 
     def weight_bytes(self) -> int:
         return self.qkv.weight_bytes() + self.out.weight_bytes() + 2 * self.d * 4

@@ -64,10 +64,13 @@ class Norm(Part):
 
 def summed_delta(norm: Norm, delta):
     """``delta`` as ``norm`` takes it: partial sums [S, T, width] are added up first unless the
-    norm adds them itself."""
-    if (delta is not None and getattr(delta, "dim", lambda: 2)() == 3
+    norm adds them itself, and what a product returns that has added its result into the
+    residual itself (``ops.Added``) becomes None unless the norm knows of such things."""
+    from ..kernels import ops
+    if isinstance(delta, ops.Added) and not getattr(norm, "can_defer", False):
+        return None                  # a product has added its result into the residual itself
+    if (isinstance(delta, torch.Tensor) and delta.dim() == 3
             and not getattr(norm, "takes_partial_sums", False)):
-        from ..kernels import ops
         return ops.sum_partial_sums(delta)
     return delta
 
@@ -85,10 +88,21 @@ class PositionEncoding(Part):
 
 
 class Mixer(Part):
-    """A token mixer.  ``cache_spec`` says what it needs from the cache manager (PagedKV,
+    """A token mixer.  ``cache_spec`` says what it needs from the cache manager (a PagedSpec,
     FixedState or None); ``forward`` gets the normalised rows [T, width] in the compute
     dtype, the step's ``RowBatch`` and its cache view, and returns [T, width] in the compute
-    dtype, or float32 partial sums [S, T, width] that the next norm adds up."""
+    dtype, or float32 partial sums [S, T, width] that the next norm adds up.
+
+    Two optional abilities, for decode steps with few rows, each announced by a flag:
+    ``takes_deferred_rows = True``: ``x`` may arrive as ``ops.ScaledRows`` or
+    ``ops.FragmentRows`` (what ``ops.linear`` and its relatives take in place of rows) when the
+    norm before the part can hand them out.
+    ``adds_residual = True``: ``forward`` takes ``into=ops.AddInto(...)`` (or None) and passes it
+    to its last product, which then adds the result into the residual stream itself and folds
+    the following norm in; the part returns what that product returned."""
+
+    takes_deferred_rows = False
+    adds_residual = False
 
     def cache_spec(self):
         return None
@@ -98,6 +112,13 @@ class Mixer(Part):
 
 
 class FeedForward(Part):
+    """``forward(x, batch)`` returns [T, width] or float32 partial sums [S, T, width].  The two
+    optional abilities of ``Mixer`` (``takes_deferred_rows``, ``adds_residual`` with an ``into``
+    argument) hold here as well."""
+
+    takes_deferred_rows = False
+    adds_residual = False
+
     def forward(self, x: torch.Tensor, batch) -> torch.Tensor:
         raise NotImplementedError
 
@@ -109,13 +130,17 @@ class Hidden:
     [S, T, width]).  The next norm adds it while it normalises, so the sum is made in float32
     and costs no pass of its own."""
     resid: torch.Tensor
-    delta: Optional[torch.Tensor] = None
+    delta: Optional[object] = None      # a tensor, or ops.Added / ops.ScaledRows: nothing to add
 
 
 class Block(Part):
     """An arrangement of parts around the residual stream."""
 
     mixer: Mixer
+
+    # True if ``forward`` takes ``next_block``: the block that runs after this one (None after
+    # the last), so that this block's last product can fold that block's first norm in.
+    takes_next_block = False
 
     def cache_spec(self):
         return self.mixer.cache_spec()

@@ -5,6 +5,7 @@ from typing import Dict, List
 
 import torch
 
+from ..kernels import ops
 from ..weights.spec import TensorSpec
 from .base import Block, FeedForward, Hidden, Mixer, Norm, register_part, summed_delta
 
@@ -40,20 +41,47 @@ class PreNormBlock(Block):
         for p in self._parts():
             p.bind(tensors)
 
-    def forward(self, h: Hidden, batch, cache, shared_cache: bool = False) -> Hidden:
-        # a part that says so may get its rows as a pending norm, which its first product makes
+    takes_next_block = True
+
+    def first_norm(self):
+        """The norm a block before this one may fold into its last product, and the part that
+        takes its rows."""
+        return self.mixer_norm, self.mixer
+
+    def forward(self, h: Hidden, batch, cache, shared_cache: bool = False,
+                next_block=None) -> Hidden:
+        # decode steps with few rows: a product may add its result into the residual stream
+        # itself and hand the next product its rows without a norm kernel in between
         resid = h.resid
         x = self._normed(self.mixer_norm, resid, h.delta, self.mixer)
-        mixed = self.mixer.forward(x, batch, cache, shared_cache=shared_cache)
+        into = self._into(self.mixer, resid, self.ffn_norm, self.feed_forward)
+        if into is not None:
+            mixed = self.mixer.forward(x, batch, cache, shared_cache=shared_cache, into=into)
+        else:
+            mixed = self.mixer.forward(x, batch, cache, shared_cache=shared_cache)
         resid = self._resid_after(x, resid)
         x = self._normed(self.ffn_norm, resid, mixed, self.feed_forward)
-        out = self.feed_forward.forward(x, batch)
+        nxt = getattr(next_block, "first_norm", None)
+        norm, consumer = nxt() if nxt is not None else (None, None)
+        into = self._into(self.feed_forward, resid, norm, consumer)
+        out = (self.feed_forward.forward(x, batch, into=into) if into is not None
+               else self.feed_forward.forward(x, batch))
         return Hidden(self._resid_after(x, resid), out)
+
+    @staticmethod
+    def _into(producer, resid, norm, consumer):
+        """What ``producer`` may add its result into, or None when it does not do such things."""
+        if not getattr(producer, "adds_residual", False):
+            return None
+        fold = getattr(norm, "fold", None)
+        if fold is not None and getattr(consumer, "takes_deferred_rows", False):
+            return ops.AddInto(resid, *fold())
+        return ops.AddInto(resid)
 
     @staticmethod
     def _normed(norm, resid, delta, consumer):
         delta = summed_delta(norm, delta)
-        if getattr(consumer, "takes_pending_norm", False) and _takes_defer(norm):
+        if getattr(consumer, "takes_deferred_rows", False) and _takes_defer(norm):
             return norm.add_norm(resid, delta, defer=True)
         return norm.add_norm(resid, delta)
 
@@ -61,7 +89,7 @@ class PreNormBlock(Block):
     def _resid_after(x, resid):
         after = getattr(x, "resid_after", resid) if not isinstance(x, torch.Tensor) else resid
         if after is None:
-            raise RuntimeError("a part that takes a pending norm did not use it")
+            raise RuntimeError("a part that takes deferred rows did not use them")
         return after
 
     def weight_bytes(self) -> int:

@@ -49,7 +49,7 @@ class OutputHead(Part):
         else:
             self.linear.bind(tensors)
 
-    takes_pending_norm = True      # a plain product: it takes what ops.linear takes
+    takes_deferred_rows = True     # a plain product: it takes what ops.linear takes
 
     def forward(self, x) -> torch.Tensor:
         return self.linear.forward(x, out_dtype=torch.float32)

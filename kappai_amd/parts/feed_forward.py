@@ -15,7 +15,8 @@ from .linear import Linear
 
 
 class SwiGLU(FeedForward):
-    takes_pending_norm = True      # its first product may make the normalised rows itself
+    takes_deferred_rows = True     # its first product takes what ops.linear takes
+    adds_residual = True           # its last product can add into the residual stream
 
     def __init__(self, prefix: str, width: int, hidden: int, dtype: torch.dtype, names=None):
         n = {"gate": "w1", "up": "w3", "down": "w2"}
@@ -37,12 +38,13 @@ class SwiGLU(FeedForward):
         if self.fused:
             self.gate_up.set_weight(ops.interleave_gate_up(w[:self.hidden], w[self.hidden:]))
 
-    def forward(self, x, batch):
+    def forward(self, x, batch, into=None):
         if self.fused and x.dtype == torch.bfloat16:
             return self.down.forward(
                 ops.linear_swiglu(x, self.gate_up.weight, weight_frag=self.gate_up.weight_frag),
-                partial_sums=True)
-        return self.down.forward(ops.swiglu(self.gate_up.forward(x)), partial_sums=True)
+                partial_sums=True, add_into=into)
+        return self.down.forward(ops.swiglu(self.gate_up.forward(x)), partial_sums=True,
+                                 add_into=into)
 
     def weight_bytes(self) -> int:
         return self.gate_up.weight_bytes() + self.down.weight_bytes()

@@ -68,11 +68,14 @@ class Linear(Part):
         """Use a tensor that another part owns (a tied output head)."""
         self.set_weight(weight)
 
-    def forward(self, x: torch.Tensor, out_dtype=None, partial_sums: bool = False) -> torch.Tensor:
+    def forward(self, x: torch.Tensor, out_dtype=None, partial_sums: bool = False, add_into=None):
         """``partial_sums``: the caller hands the result to a norm as the pending residual
-        update, which may then arrive as float32 sums over ranges of the input dimension."""
+        update, which may then arrive as float32 sums over ranges of the input dimension.
+        ``add_into`` (``ops.AddInto``): the product may add its result into the residual stream
+        itself; what it returns then says so (``ops.Added``, ``ops.ScaledRows``)."""
         return ops.linear(x, self.weight, self.bias, out_dtype=out_dtype,
-                          partial_sums=partial_sums, weight_frag=self.weight_frag)
+                          partial_sums=partial_sums, weight_frag=self.weight_frag,
+                          add_into=add_into)
 
     def weight_bytes(self) -> int:
         n = self.weight.numel() * self.weight.element_size()

@@ -21,7 +21,7 @@ FRAGMENT_ROWS_MIN = 8
 
 class RMSNorm(Norm):
     takes_partial_sums = True      # the kernel adds [S, T, width] partial sums itself, in order
-    can_defer = True      # add_norm(..., defer=True) may hand out an ops.PendingNorm or
+    can_defer = True      # add_norm(..., defer=True) may hand out ops.ScaledRows or
                           # ops.FragmentRows in place of a tensor
 
     def __init__(self, name: str, width: int, eps: float, dtype: torch.dtype):
@@ -34,12 +34,24 @@ class RMSNorm(Norm):
     def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
         self.weight = tensors[self.name + ".weight"].to(torch.float32).contiguous()
 
+    def fold(self):
+        """(weight, eps) for a product that folds this norm in (``ops.AddInto``): the norm is
+        ``x * weight / rms(x)``, so the product before it can hand on ``x * weight`` and the sums
+        of squares, and the product after it divides."""
+        return self.weight, self.eps
+
     def add_norm(self, resid, delta, rows=None, defer: bool = False):
-        """``defer``: the caller's next part takes what the product kernels take in place of
-        the rows: an ``ops.PendingNorm`` (one row: the product kernel makes it itself) or
-        ``ops.FragmentRows`` (8 to 16 rows, made here in the order the product loads them)."""
-        if defer and rows is None and ops.PendingNorm.fits(resid, delta, self.dtype):
-            return ops.PendingNorm(resid, delta, self.weight, self.eps, self.dtype)
+        """``delta`` may also be what a product hands back that has added its result into
+        ``resid`` itself: ``ops.Added``, or ``ops.ScaledRows`` made for this norm.  ``defer``: the
+        caller's next part takes what the product kernels take in place of the rows: such
+        ``ops.ScaledRows`` as they are, or ``ops.FragmentRows`` (8 to 16 rows, made here in the
+        order the product loads them)."""
+        if isinstance(delta, ops.Added):
+            if (defer and rows is None and isinstance(delta, ops.ScaledRows)
+                    and delta.weight is self.weight and delta.eps == self.eps
+                    and delta.resid is resid):
+                return delta
+            delta = None             # the sum is in ``resid`` already
         n = resid.shape[0] if rows is None else rows.shape[0]
         fragment = (defer and FRAGMENT_ROWS and resid.is_cuda and n >= FRAGMENT_ROWS_MIN
                     and ops.FragmentRows.fits(n, self.width, self.dtype)

@@ -23,7 +23,7 @@ from .linear import PARTIAL_SUMS_MIN_ROWS, Linear
 # leave CUs without a block).  From this width on it beats the separate product (which may split
 # K) plus the small step kernel for any number of rows up to 64; between FUSED_STEP_NARROW_WIDTH
 # and it only up to 16 rows (at a width of 2048, W in fragment order: 8.3 against 9.9 us for one
-# row, which it also normalises itself when the norm before it is pending; 11.0 against 11.1 at
+# row; 11.0 against 11.1 at
 # 8 rows, 11.5 against 12.8 at 16; at a width of 1024 the separate kernels win).
 FUSED_STEP_MIN_WIDTH = 4096
 FUSED_STEP_NARROW_WIDTH = 2048
@@ -31,7 +31,8 @@ FUSED_STEP_NARROW_ROWS = 16
 
 
 class GatedShortConv(Mixer):
-    takes_pending_norm = True      # its first product may make the normalised rows itself
+    takes_deferred_rows = True     # its first product takes what ops.linear takes
+    adds_residual = True           # its last product can add into the residual stream
 
     def __init__(self, prefix: str, width: int, kernel_size: int, dtype: torch.dtype,
                  bias: bool = False, names=None):
@@ -67,23 +68,21 @@ class GatedShortConv(Mixer):
         if self.has_bias:
             self.conv_bias = tensors[self._conv + ".bias"].to(torch.float32).contiguous()
 
-    def forward(self, x, batch, cache, shared_cache: bool = False):
+    def forward(self, x, batch, cache, shared_cache: bool = False, into=None):
         if shared_cache:
             raise ValueError("a short convolution's state cannot be read by another layer")
         w = self.in_proj.weight
-        if isinstance(x, ops.PendingNorm) and self.width >= FUSED_STEP_MIN_WIDTH:
-            x = x.materialize()            # the 16-channel form of the fused step reads rows
         rows = x.shape[0]
         wide_enough = self.width >= FUSED_STEP_MIN_WIDTH or (
             self.width >= FUSED_STEP_NARROW_WIDTH and rows <= FUSED_STEP_NARROW_ROWS)
         if (batch.max_segment_rows == 1 and rows <= 64
-                and (isinstance(x, ops.PendingNorm) or x.dtype == torch.bfloat16)
+                and x.dtype == torch.bfloat16
                 and w.dtype == torch.bfloat16 and self.width % 16 == 0 and wide_enough):
             # decode: projection, convolution and state shift in one kernel
             y = ops.linear_shortconv_step(x, w, self.in_proj.bias, self.taps, self.conv_bias,
                                           cache.state, batch.seg_pos0, batch.seg_slot,
                                           weight_frag=self.in_proj.weight_frag)
-            return self.out_proj.forward(y, partial_sums=True)
+            return self.out_proj.forward(y, partial_sums=True, add_into=into)
         # decode with more than 16 rows: the projection may come as sums over ranges of its input
         # dimension (more blocks stream the matrix), which the step kernel adds up; with fewer
         # rows the unsplit product and the plain step are as fast or faster
@@ -91,7 +90,7 @@ class GatedShortConv(Mixer):
             x, partial_sums=batch.max_segment_rows == 1 and x.shape[0] > PARTIAL_SUMS_MIN_ROWS)
         y = ops.shortconv(proj, self.taps, self.conv_bias, cache.state, batch.row_seg,
                           batch.seg_start, batch.seg_pos0, batch.seg_slot)
-        return self.out_proj.forward(y, partial_sums=True)
+        return self.out_proj.forward(y, partial_sums=True, add_into=into)
 
     def weight_bytes(self) -> int:
         return self.in_proj.weight_bytes() + self.out_proj.weight_bytes() + self.width * self.L * 4

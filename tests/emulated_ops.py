@@ -54,7 +54,8 @@ def cast(x, dtype):
 
 
 def linear(x, weight, bias=None, out_dtype=None, force_kernel=0, partial_sums=False,
-           split_k=None, weight_frag=None):
+           split_k=None, weight_frag=None, add_into=None):
+    # ``add_into`` is an offer the stand-in does not take up: the result comes back as always
     out_dtype = out_dtype or x.dtype
     y = x.to(F32) @ weight.to(F32).T
     if bias is not None:

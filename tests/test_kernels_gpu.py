@@ -252,7 +252,7 @@ def test_linear_block256_split_k(ops):
 def test_products_read_the_fragment_order_copy(ops, M, N, K):
     """With the copy of the matrix in fragment order beside it every product gives bit for bit
     what it gives without: plain, with bias, as partial sums over K ranges, with the SwiGLU
-    epilogue, with a pending RMSNorm as its input, and as the fused conv step (the kernel for 1 to
+    epilogue, adding into the residual stream, on scaled rows, and as the fused conv step (the kernel for 1 to
     16 rows reads the copy; with more rows it is passed and not read)."""
     x = rand((M, K), BF16, 60).to(DEV)
     w, b = rand((N, K), BF16, 61, 0.1).to(DEV), rand((N,), F32, 62).to(DEV)
@@ -280,14 +280,22 @@ def test_products_read_the_fragment_order_copy(ops, M, N, K):
         if N % 32 == 0:
             assert torch.equal(ops.linear_swiglu(x, w, force_kernel=SHARED_ROWS, weight_frag=wf),
                                ops.linear_swiglu(x, w, force_kernel=SHARED_ROWS))
-    if M <= ops.NORM_FUSE_MAX_ROWS and K <= ops.NORM_FUSE_MAX_WIDTH:
-        resid, wn = rand((M, K), F32, 63, 2.0).to(DEV), (1 + rand((K,), F32, 64, 0.1)).to(DEV)
-        delta = rand((M, K), BF16, 65).to(DEV)
+    if M <= ops.FUSED_MAX_ROWS:
+        # the product that adds into the residual stream, and the one that scales its rows
+        wn = (1 + rand((N,), F32, 64, 0.1)).to(DEV)
         outs = []
         for frag in (wf, None):
-            pend = ops.PendingNorm(resid, delta, wn, 1e-5, BF16)
-            outs.append(ops.linear(pend, w, b, out_dtype=F32, weight_frag=frag))
-        assert torch.equal(outs[0], outs[1])
+            resid = rand((M, N), F32, 63, 2.0).to(DEV)
+            rows = ops.linear(x, w, b, weight_frag=frag, add_into=ops.AddInto(resid, wn, 1e-5))
+            data = (ops.FragmentRows(rows.data, M, resid).materialize() if rows.fragment
+                    else rows.data)             # (the row slots beyond M hold nothing)
+            outs.append((resid, data, rows.ss))
+        assert all(torch.equal(a, c) for a, c in zip(*outs))
+        if N == K:
+            rows = ops.linear(x, w, b, add_into=ops.AddInto(rand((M, N), F32, 63, 2.0).to(DEV), wn,
+                                                            1e-5))
+            assert torch.equal(ops.linear(rows, w, b, out_dtype=F32, weight_frag=wf),
+                               ops.linear(rows, w, b, out_dtype=F32))
     if N % 48 == 0 and M <= 64:
         D, L = N // 3, 3
         taps = rand((D, L), F32, 66, 0.5).to(DEV)
@@ -427,72 +435,96 @@ def test_linear_partial_sums(ops, M, N, K):
                                        write_resid=False), BF16_ULP, "selected rows")
 
 
-@pytest.mark.parametrize("M", [1, 2, 4])
-@pytest.mark.parametrize("N,K", [(48, 64), (6144, 2048), (200, 520), (1000, 4096), (64, 2048)])
-@pytest.mark.parametrize("delta_kind", ["none", "bf16", "f32", "parts"])
-def test_linear_makes_the_normalised_rows_itself(ops, M, N, K, delta_kind):
-    """A product whose input is a pending RMSNorm: the same result as the norm kernel followed by
-    the product, the residual untouched and resid + delta in a tensor of its own."""
-    resid = rand((M, K), F32, 80, 2.0)
-    wn = 1 + rand((K,), F32, 81, 0.1)
-    w, b = rand((N, K), BF16, 82, 0.1), rand((N,), F32, 83)
-    delta = {"none": None, "bf16": rand((M, K), BF16, 84), "f32": rand((M, K), F32, 84),
-             "parts": rand((3, M, K), F32, 84)}[delta_kind]
-    d_dev = None if delta is None else delta.to(DEV)
-    r_dev = resid.to(DEV)
-    x = ops.add_rmsnorm(r_dev.clone(), d_dev, wn.to(DEV), 1e-5, BF16)
-    for bias in (None, b.to(DEV)):
-        pend = ops.PendingNorm(r_dev, d_dev, wn.to(DEV), 1e-5, BF16)
-        got = ops.linear(pend, w.to(DEV), bias, out_dtype=F32)
-        want = ops.linear(x, w.to(DEV), bias, out_dtype=F32)
-        close(got, want.cpu().double(), 2 * BF16_ULP, "product of the pending norm")
-        assert torch.equal(r_dev.cpu(), resid), "the residual was changed"
-        total = resid.clone()
-        if delta is not None:
-            for part in (delta if delta.dim() == 3 else [delta]):
-                total += part.float()
-            assert pend.resid_after.data_ptr() != r_dev.data_ptr()
-        else:
-            assert pend.resid_after is r_dev
-        close(pend.resid_after, total.double(), 1e-6, "resid + delta")
-    # partial sums out of it, as the consumers of a split product take them
-    pend = ops.PendingNorm(r_dev, d_dev, wn.to(DEV), 1e-5, BF16)
-    parts = ops.linear(pend, w.to(DEV), partial_sums=True, split_k=2)
-    assert parts.shape == (2, M, N) and parts.dtype == F32
-    close(parts.sum(0), ops.linear(x, w.to(DEV), out_dtype=F32).cpu().double(), 2 * BF16_ULP,
-          "partial sums")
+def folded_reference(resid, delta, wn, eps, w2, b2):
+    """float64: the residual after the sum, and RMSNorm(resid + delta) W2^T + b2."""
+    total = resid.double() + delta.double()
+    xn = total / torch.sqrt((total * total).mean(dim=1, keepdim=True) + eps) * wn.double()
+    y = xn @ w2.double().T
+    return total, (y if b2 is None else y + b2.double())
 
 
-@pytest.mark.parametrize("M,F,K", [(1, 8192, 2048), (3, 48, 136), (4, 320, 1024), (1, 64, 2048),
-                                   (2, 32, 4096)])
-def test_linear_swiglu_makes_the_normalised_rows_itself(ops, M, F, K):
-    resid, wn = rand((M, K), F32, 85, 2.0), 1 + rand((K,), F32, 86, 0.1)
-    delta = rand((4, M, K), F32, 87)
-    wg, wu = rand((F, K), BF16, 88, 0.1), rand((F, K), BF16, 89, 0.1)
+@pytest.mark.parametrize("M", [1, 2, 5, 8, 16])
+@pytest.mark.parametrize("N,K,N2", [(48, 64, 80), (2048, 2048, 6144), (200, 520, 304),
+                                    (1024, 4096, 64), (2048, 8192, 1000)])
+def test_products_fold_the_residual_sum_and_the_norm(ops, M, N, K, N2):
+    """Two products of a decode step without a norm kernel between them: the first adds its
+    result into the residual stream in place and hands on bf16(resid * norm weight) and the sums
+    of squares, the second scales its results by the rows' 1 / rms.  Against float64, with the
+    error of one bfloat16 rounding of the rows; and against the two products with the norm
+    kernel between them."""
+    x = rand((M, K), BF16, 80)
+    w1, b1 = rand((N, K), BF16, 81, 0.1), rand((N,), F32, 82)
+    wn = 1 + rand((N,), F32, 83, 0.1)
+    w2, b2 = rand((N2, N), BF16, 84, 0.1), rand((N2,), F32, 85)
+    resid0 = rand((M, N), F32, 86, 2.0)
+    delta = x.double() @ w1.double().T + b1.double()
+    total, want = folded_reference(resid0, delta, wn, 1e-5, w2, b2)
+    for frag in (False, True):
+        f1 = ops.fragment_order(w1.to(DEV)) if frag else None
+        f2 = ops.fragment_order(w2.to(DEV)) if frag else None
+        resid = resid0.to(DEV)
+        rows = ops.linear(x.to(DEV), w1.to(DEV), b1.to(DEV), weight_frag=f1,
+                          add_into=ops.AddInto(resid, wn.to(DEV), 1e-5))
+        assert isinstance(rows, ops.ScaledRows) and rows.resid is resid
+        assert rows.fragment == (M >= 8 and N % 32 == 0)
+        close(resid, total, 1e-5, "residual after the sum")
+        close(rows.ss.sum(0), (total * total).sum(1), 1e-5, "sums of squares")
+        got = ops.linear(rows, w2.to(DEV), b2.to(DEV), out_dtype=F32, weight_frag=f2)
+        close(got, want, 2 * BF16_ULP, "product on scaled rows")
+        # what the ordinary norm kernel would have fed the second product with
+        xn = ops.add_rmsnorm(resid, None, wn.to(DEV), 1e-5, BF16)
+        close(got, ops.linear(xn, w2.to(DEV), b2.to(DEV), out_dtype=F32).cpu().double(),
+              2 * BF16_ULP, "against norm kernel + product")
+        assert torch.equal(rows.materialize(), xn)
+    # without a norm weight the product only adds
+    resid = resid0.to(DEV)
+    added = ops.linear(x.to(DEV), w1.to(DEV), None, add_into=ops.AddInto(resid))
+    assert type(added) is ops.Added
+    close(resid, resid0.double() + x.double() @ w1.double().T, 1e-5, "residual after the sum")
+
+
+@pytest.mark.parametrize("M,F,K", [(1, 8192, 2048), (3, 48, 136), (8, 320, 1024), (16, 64, 2048)])
+def test_linear_swiglu_on_scaled_rows(ops, M, F, K):
+    x = rand((M, 96), BF16, 87)
+    w1, wn = rand((K, 96), BF16, 88, 0.1), 1 + rand((K,), F32, 89, 0.1)
+    wg, wu = rand((F, K), BF16, 90, 0.1), rand((F, K), BF16, 91, 0.1)
     w = ops.interleave_gate_up(wg.to(DEV), wu.to(DEV))
-    x = ops.add_rmsnorm(resid.to(DEV), delta.to(DEV), wn.to(DEV), 1e-5, BF16)
-    pend = ops.PendingNorm(resid.to(DEV), delta.to(DEV), wn.to(DEV), 1e-5, BF16)
-    got = ops.linear_swiglu(pend, w)
-    close(got.float(), ops.linear_swiglu(x, w).float().cpu().double(), 2 * BF16_ULP, "swiglu")
-    close(pend.resid_after, (resid + delta.sum(0)).double(), 1e-5, "resid + delta")
+    resid = rand((M, K), F32, 92, 2.0).to(DEV)
+    rows = ops.linear(x.to(DEV), w1.to(DEV), add_into=ops.AddInto(resid, wn.to(DEV), 1e-5))
+    got = ops.linear_swiglu(rows, w, weight_frag=ops.fragment_order(w))
+    xn = resid.cpu().double()
+    xn = xn / torch.sqrt((xn * xn).mean(dim=1, keepdim=True) + 1e-5) * wn.double()
+    g, u = xn @ wg.double().T, xn @ wu.double().T
+    close(got.float(), g / (1 + torch.exp(-g)) * u, 3 * BF16_ULP, "swiglu on scaled rows")
 
 
-def test_pending_norm_falls_back_to_the_norm_kernel(ops):
-    """A float32 matrix (or anything else the fused kernel does not take) makes the rows with
-    the ordinary kernel, which updates the residual in place."""
-    resid, wn = rand((1, 64), F32, 90, 2.0), 1 + rand((64,), F32, 91, 0.1)
-    delta, w = rand((1, 64), BF16, 92), rand((24, 64), F32, 93)
-    r_dev = resid.to(DEV)
-    pend = ops.PendingNorm(r_dev, delta.to(DEV), wn.to(DEV), 1e-5, BF16)
-    got = ops.linear(pend, w.to(DEV))
-    assert pend.resid_after is r_dev
-    close(r_dev, (resid + delta.float()).double(), 1e-6, "residual updated in place")
-    x = ref.add_rmsnorm(resid.clone(), delta, wn, 1e-5, BF16)
-    close(got.float(), x.double() @ w.double().T, BF16_ULP, "product")
-    assert not ops.PendingNorm.fits(rand((9, 64), F32, 1).to(DEV), None, BF16)
-    assert not ops.PendingNorm.fits(rand((1, 64), F32, 1).to(DEV), None, F32)
-    assert not ops.PendingNorm.fits(rand((1, 8192), F32, 1).to(DEV), None, BF16)
-    assert ops.PendingNorm.fits(rand((1, 64), F32, 1).to(DEV), rand((2, 1, 64), F32, 2).to(DEV), BF16)
+def test_products_that_cannot_fold_go_the_ordinary_way(ops):
+    """More than 16 rows, or a float32 matrix: ``add_into`` is not taken up and the product
+    comes back as always; scaled rows that meet a float32 matrix are made by the norm kernel."""
+    x, w = rand((20, 64), BF16, 93).to(DEV), rand((32, 64), BF16, 94, 0.1).to(DEV)
+    resid = rand((20, 32), F32, 95).to(DEV)
+    before = resid.clone()
+    out = ops.linear(x, w, add_into=ops.AddInto(resid))
+    assert isinstance(out, torch.Tensor) and torch.equal(resid, before)
+    out = ops.linear(x[:4].float(), w.float(), add_into=ops.AddInto(resid[:4].contiguous()))
+    assert isinstance(out, torch.Tensor) and out.dtype == F32
+    wn = (1 + rand((32,), F32, 96, 0.1)).to(DEV)
+    r4 = resid[:4].contiguous()
+    rows = ops.linear(x[:4], w, add_into=ops.AddInto(r4, wn, 1e-5))
+    w32 = rand((24, 32), F32, 97).to(DEV)
+    got = ops.linear(rows, w32)
+    xn = ref.add_rmsnorm(r4.cpu().clone(), None, wn.cpu(), 1e-5, BF16)
+    close(got.float(), xn.double() @ w32.cpu().double().T, BF16_ULP, "product")
+    # a width that is no multiple of 8: the product after the folded norm runs in the plain
+    # kernel, which scales nothing, so the rows are made by the norm kernel first
+    x, w = rand((3, 80), BF16, 98).to(DEV), rand((100, 80), BF16, 99, 0.1).to(DEV)
+    wn, r3 = (1 + rand((100,), F32, 100, 0.1)).to(DEV), rand((3, 100), F32, 101, 2.0).to(DEV)
+    rows = ops.linear(x, w, add_into=ops.AddInto(r3, wn, 1e-5))
+    assert isinstance(rows, ops.ScaledRows)
+    w2 = rand((24, 100), BF16, 102, 0.1).to(DEV)
+    xn = ref.add_rmsnorm(r3.cpu().clone(), None, wn.cpu(), 1e-5, BF16)
+    close(ops.linear(rows, w2, out_dtype=F32), xn.double() @ w2.cpu().double().T, BF16_ULP,
+          "product in the plain kernel")
 
 
 @pytest.mark.parametrize("M,N,K", [(1, 7, 20), (5, 301, 100), (70, 33, 84), (3, 64, 1001)])
@@ -601,37 +633,32 @@ def test_linear_shortconv_step(ops, M, D, K, L, bias):
 
 
 @pytest.mark.parametrize("D,K,L,bias,frag", [(2048, 2048, 3, False, True), (96, 96, 4, True, True),
-                                             (48, 120, 2, True, False), (3072, 1024, 3, False, True)])
-@pytest.mark.parametrize("delta_kind", ["none", "bf16", "parts"])
-def test_linear_shortconv_step_on_a_pending_norm(ops, D, K, L, bias, frag, delta_kind):
-    """A single decoded row whose RMSNorm is still pending: norm, in_proj, gates, FIR and state
-    shift in one kernel give what the norm kernel followed by the fused step gives, and the
-    residual comes back in a tensor of its own."""
-    M = 1
+                                             (48, 120, 2, True, False), (3072, 1024, 3, False, True),
+                                             (4096, 512, 3, False, True)])
+@pytest.mark.parametrize("M", [1, 8, 13])
+def test_linear_shortconv_step_on_scaled_rows(ops, D, K, L, bias, frag, M):
+    """The fused conv step of decoded rows whose RMSNorm is folded into the products around it
+    gives what the norm kernel followed by the fused step gives."""
+    x0 = rand((M, 64), BF16, 89).to(DEV)
+    w0 = rand((K, 64), BF16, 90, 0.2).to(DEV)
     resid = rand((M, K), F32, 90, 2.0).to(DEV)
     wn = (1 + rand((K,), F32, 91, 0.1)).to(DEV)
-    delta = {"none": None, "bf16": rand((M, K), BF16, 92), "parts": rand((3, M, K), F32, 92)}[delta_kind]
-    d_dev = None if delta is None else delta.to(DEV)
     w = rand((3 * D, K), BF16, 93, 0.2).to(DEV)
     wf = ops.fragment_order(w) if frag else None
     assert (wf is not None) == (frag and K % 32 == 0)
     b_in = rand((3 * D,), F32, 94, 0.2).to(DEV) if bias else None
     b_cv = rand((D,), F32, 95, 0.2).to(DEV) if bias else None
     taps = rand((D, L), F32, 96, 0.5).to(DEV)
-    state0 = rand((3, D, L - 1), F32, 97).to(DEV)
-    pos0 = torch.tensor([5], dtype=torch.int32, device=DEV)
-    slot = torch.tensor([1], dtype=torch.int32, device=DEV)
+    state0 = rand((M + 2, D, L - 1), F32, 97).to(DEV)
+    pos0 = torch.full((M,), 5, dtype=torch.int32, device=DEV)
+    slot = torch.arange(1, M + 1, dtype=torch.int32, device=DEV)
     st_a, st_b = state0.clone(), state0.clone()
-    pend = ops.PendingNorm(resid, d_dev, wn, 1e-5, BF16)
-    got = ops.linear_shortconv_step(pend, w, b_in, taps, b_cv, st_a, pos0, slot, weight_frag=wf)
-    r2 = resid.clone()
-    x = ops.add_rmsnorm(r2, d_dev, wn, 1e-5, BF16)
+    rows = ops.linear(x0, w0, add_into=ops.AddInto(resid, wn, 1e-5))
+    got = ops.linear_shortconv_step(rows, w, b_in, taps, b_cv, st_a, pos0, slot, weight_frag=wf)
+    x = ops.add_rmsnorm(resid, None, wn, 1e-5, BF16)
     want = ops.linear_shortconv_step(x, w, b_in, taps, b_cv, st_b, pos0, slot, weight_frag=wf)
-    close(got.float(), want.float().cpu().double(), 2 * BF16_ULP, "fused step of the pending norm")
-    close(st_a, st_b.cpu().double(), 2 * BF16_ULP, "state")
-    close(pend.resid_after, r2.cpu().double(), 1e-6, "resid + delta")
-    if delta is not None:
-        assert pend.resid_after.data_ptr() != resid.data_ptr()
+    close(got.float(), want.float().cpu().double(), 3 * BF16_ULP, "fused step on scaled rows")
+    close(st_a, st_b.cpu().double(), 3 * BF16_ULP, "state")
 
 
 # ---------------------------------------------------------------------------------------

@@ -154,9 +154,16 @@ def test_feed_forward_norm_and_block(dtype, tol):
     lwc = {"in_proj": wb["b.c.in_proj.weight"], "out_proj": wb["b.c.out_proj.weight"],
            "conv": wb["b.c.conv.weight"].reshape(W, 3)}
     xr = xr + P.short_conv_mixer(P.rmsnorm(xr, wb["b.n1.weight"], 1e-5), lwc, {"hidden_size": W})
-    assert rel_err(h.resid, xr) < tol                      # the first sum is in; the second pending
     lwf = {n: wb[f"b.f.{n}.weight"] for n in ("w1", "w2", "w3")}
-    assert rel_err(h.delta, P.swiglu_feed_forward(P.rmsnorm(xr, wb["b.n2.weight"], 1e-5), lwf)) < tol
+    ffn = P.swiglu_feed_forward(P.rmsnorm(xr, wb["b.n2.weight"], 1e-5), lwf)
+    from kappai_amd.kernels import ops
+    if isinstance(h.delta, ops.Added):
+        # few rows in bfloat16: both products added their results into the stream themselves
+        assert dtype == BF16 and T <= ops.FUSED_MAX_ROWS
+        assert rel_err(h.resid, xr + ffn) < tol
+    else:
+        assert rel_err(h.resid, xr) < tol                  # the first sum is in; the second pending
+        assert rel_err(h.delta, ffn) < tol
 
 
 def test_rotary_tables():
@@ -447,9 +454,10 @@ def test_toy_feed_forward_with_routing_and_an_absolute_position_encoding():
 def test_toy_norm_that_knows_nothing_of_partial_sums(monkeypatch):
     """A LayerNorm written to the Norm interface as documented (``add_norm(resid, delta, rows)``
     with a plain update), registered from the test and built into blocks around the engine's
-    own conv mixer, attention and SwiGLU.  In bfloat16 decode steps those parts hand on float32
-    partial sums of products split over their input dimension; the block sums them for a norm
-    that does not say it takes them.  Decoding token by token equals the whole prompt, and
+    own conv mixer, attention and SwiGLU.  In bfloat16 those parts hand on float32 partial sums
+    of products split over their input dimension (steps of more than 16 rows) or add their
+    results into the residual stream themselves (fewer rows); the block sums the former for a
+    norm that does not say it takes them and passes the latter on as no update.  Decoding token by token equals the whole prompt, and
     bfloat16 stays near float32."""
     import tempfile
 
@@ -556,7 +564,9 @@ def test_toy_norm_that_knows_nothing_of_partial_sums(monkeypatch):
             assert not summed          # true 32-bit products are never split
             assert float((cut - whole).abs().max()) < 2e-5 * scale
         else:
-            assert any(s[0] > 1 and s[1] == 1 for s in summed), "no decode step handed on partial sums"
+            # (the portion of 17 rows does; the single rows are added into the stream by the
+            # products themselves, which the toy norm sees as no update at all)
+            assert any(s[0] > 1 for s in summed), "no step handed on partial sums"
             assert float((cut - whole).abs().max()) < 3e-2 * scale
         results[dtype] = whole
     err = float((results["bfloat16"] - results["float32"]).abs().max())
