@@ -759,7 +759,7 @@ struct ConvStep {
 //     not split over blocks): resid[m][n] += sum (+ bias) in place, in float; and when `rows` is
 //     set the block also writes what the next product reads, rows[m][n] = bf16(resid[m][n] *
 //     norm_w[n]) (row order, or the fragment order of add_rmsnorm when rows_frag), and
-//     ss[blockIdx.x][m] = the sum of resid[m][n]^2 over its 16 columns;
+//     ss[blockIdx.x][m] = the sum of resid[m][n]^2 over its 8 columns (gemm_bf16_into_resid);
 //   RowScale (the product that follows): its rows are such x * w, and every result is
 //     multiplied by 1 / sqrt(sum_p ss[p][m] / K + eps) before bias and epilogue.
 struct RowScale {
@@ -780,8 +780,13 @@ template <typename TO, int MT, int NW, int EPI, int NT>
 __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny_kernel(
     const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, const float* __restrict__ bias,
     TO* __restrict__ C, int M, int N, int K, int lda, int ldc, ConvStep cs, RowScale rsc,
-    ResidOut ro, int w_frag, int a_frag) {
+    int w_frag, int a_frag, int c_frag) {
   static_assert(NT == 1 || EPI == 0, "several column tiles a wave: plain products only");
+  // c_frag (one row tile, the SwiGLU and conv epilogues): the result is written as 16 rows in
+  // fragment order, which is how the product that follows likes to read it (see a_frag)
+  auto out_at = [&](int gm, int gn_) {
+    return c_frag ? ((size_t)(gn_ / 8) * 16 + gm) * 8 + gn_ % 8 : (size_t)gm * ldc + gn_;
+  };
   // row groups of W a block streams: gate/up, the three conv gates, or NT column tiles
   constexpr int NG = EPI == 1 ? 2 : (EPI == 2 ? 3 : (EPI == 3 ? 2 : NT));
   __shared__ float red[NW][NG * MT][WAVE][4];
@@ -823,6 +828,21 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny_kernel(
     arow[t] = a_frag ? A + ((size_t)(kg / 8) * 16 + (gm < M ? gm : 0)) * 8
                      : A + (size_t)(gm < M ? gm : 0) * lda + kg;
   }
+  // What the epilogue needs from memory is asked for early, so that it has arrived when the
+  // stream of W has gone through: the residual values and norm weight of this block's columns
+  // (ResidOut) now, and 1 / rms of the rows (RowScale; wave w makes it for rows w, w + NW, ...)
+  // behind the first loads of W, whose wait it then shares.
+  __shared__ float row_scale[16 * MT];
+  bool scale_made = rsc.ss == nullptr;
+  auto make_row_scale = [&]() {
+    for (int m = wave; m < M; m += NW) {
+      float part = 0.f;
+      for (int p = lane; p < rsc.n_parts; p += WAVE) part += rsc.ss[(size_t)p * M + m];
+      part = wave_sum(part);
+      if (lane == 0) row_scale[m] = 1.0f / sqrtf(part / (float)K + rsc.eps);
+    }
+    scale_made = true;
+  };
   const int kblk = ((K + 32 * (int)gridDim.y - 1) / (32 * (int)gridDim.y)) * 32;   // K a block
   const int kb0 = blockIdx.y * kblk, kb1 = min(K, kb0 + kblk);
   const int kper = ((kb1 - kb0 + 32 * NW - 1) / (32 * NW)) * 32;
@@ -858,23 +878,15 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny_kernel(
         for (int t = 0; t < MT; ++t)
           av[u][t] = (kin && t * 16 + col < M) ? load16(arow[t] + (size_t)gk * (a_frag ? 16 : 1)) : zero;
       }
+      if (!scale_made) make_row_scale();
       products(wv, av);
     }
   }
+  if (!scale_made) make_row_scale();       // (a wave without a K range of its own)
 #pragma unroll
   for (int t = 0; t < NG * MT; ++t)
 #pragma unroll
     for (int v = 0; v < 4; ++v) red[wave][t][lane][v] = acc[t][v];
-  // 1 / rms of the rows (RowScale): wave w makes it for rows w, w + NW, ...
-  __shared__ float row_scale[16 * MT];
-  if (rsc.ss != nullptr) {
-    for (int m = wave; m < M; m += NW) {
-      float part = 0.f;
-      for (int p = lane; p < rsc.n_parts; p += WAVE) part += rsc.ss[(size_t)p * M + m];
-      part = wave_sum(part);
-      if (lane == 0) row_scale[m] = 1.0f / sqrtf(part / (float)K + rsc.eps);
-    }
-  }
   __syncthreads();
   auto scale_of = [&](int gm) { return rsc.ss != nullptr ? row_scale[gm] : 1.0f; };
   // the first MT waves each sum one row tile over the NW partial results, in a fixed order
@@ -911,7 +923,7 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny_kernel(
           float up = red[0][MT + t][lane][v];
 #pragma unroll
           for (int w = 1; w < NW; ++w) up += red[w][MT + t][lane][v];
-          store_out(C + (size_t)gm * ldc + gn, silu_f(sum) * (up * rs));
+          store_out(C + out_at(gm, gn), silu_f(sum) * (up * rs));
         } else if (EPI == 2 || EPI == 3) {
           // where the other two gates of this channel lie: EPI 2 in row groups 1 and 2 of this
           // lane, EPI 3 the C gate 8 columns further in group 0 and the x gate in group 1
@@ -946,44 +958,135 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny_kernel(
             prev = next;
           }
           s += wc[H] * bx;
-          store_out(C + (size_t)gm * ldc + gn, to_f32(f32_to_bf16(cg)) * s);
-        } else if (EPI == 0 && ro.resid != nullptr) {
-          // the result joins the residual stream here (ResidOut)
-          float* rp = ro.resid + (size_t)gm * ro.ldr + gn;
-          const float x = *rp + (sum + bv);
-          *rp = x;
-          if (ro.rows != nullptr) {
-            const size_t at = ro.rows_frag ? ((size_t)(gn / 8) * 16 + gm) * 8 + gn % 8
-                                           : (size_t)gm * N + gn;
-            ro.rows[at] = f32_to_bf16(x * ro.norm_w[gn]);
-          }
+          store_out(C + out_at(gm, gn), to_f32(f32_to_bf16(cg)) * s);
         } else {
           store_out(C + (size_t)gm * ldc + gn, sum + bv);
         }
       }
     }
   }
-  if (EPI == 0 && NT == 1 && MT == 1 && ro.rows != nullptr && wave == 0) {
-    // sums of squares of the new residual over this block's 16 columns, row by row: a lane
-    // holds column lane % 16 of rows 4 (lane / 16) + v and reads back what it has just written
+}
+
+// A product whose result joins the residual stream (ResidOut; at most 16 rows, K in one piece).
+// Such products have few columns (the model's width), so a block owns 8 of them, and the two
+// halves of the matrix tile's 16 columns take the two halves of K: column j < 8 is row n0 + j of
+// W over K's first half, column j + 8 the same row over the second half.  The rows of A of the
+// two halves meet the one fragment of W in two matrix instructions, whose valid halves are added
+// at the end.  Twice as many blocks stream W as with 16 columns a block, and K needs no split
+// over blocks, so the residual sum can be made here, in a fixed order.
+template <int NW>
+__global__ __launch_bounds__(NW * WAVE) void gemm_bf16_into_resid_kernel(
+    const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, const float* __restrict__ bias,
+    int M, int N, int K, int lda, ResidOut ro, int w_frag, int a_frag) {
+  __shared__ float red[NW][2][WAVE][4];
+  const int tid = threadIdx.x;
+  const int lane = tid % WAVE, wave = tid / WAVE;
+  const int col = lane % 16, kg = (lane / 16) * 8;
+  const int half = col / 8;
+  const int gn = blockIdx.x * 8 + col % 8;               // the lane's row of W
+  const int khalf = ((K / 2 + 31) / 32) * 32;            // the second half starts here
+  const u32x4_t zero = {0u, 0u, 0u, 0u};
+  // what the epilogue needs, asked for before the stream of W
+  float resid_in[4] = {0.f, 0.f, 0.f, 0.f};
+  float norm_w_in = 0.f;
+  if (wave == 0 && half == 0 && gn < N) {
 #pragma unroll
     for (int v = 0; v < 4; ++v) {
       const int gm = 4 * (lane / 16) + v;
-      float x = 0.f;
-      if (gm < M && gn < N) x = ro.resid[(size_t)gm * ro.ldr + gn];
-      float q = x * x;
+      if (gm < M) resid_in[v] = ro.resid[(size_t)gm * ro.ldr + gn];
+    }
+    if (ro.rows != nullptr) norm_w_in = ro.norm_w[gn];
+  }
+  const size_t wr = gn < N ? gn : 0;
+  const int kmul = w_frag ? 16 : 1;                      // see the kernel above for the two orders
+  const bf16_t* wrow = (w_frag ? W + (wr / 16) * 16 * K + ((size_t)(kg / 8) * 16 + wr % 16) * 8
+                               : W + wr * K + kg) + (size_t)half * khalf * kmul;
+  const int am = col < M ? col : 0;                      // the lane's row of A
+  const int amul = a_frag ? 16 : 1;
+  const bf16_t* arow = a_frag ? A + ((size_t)(kg / 8) * 16 + am) * 8 : A + (size_t)am * lda + kg;
+  const int kper = ((khalf + 32 * NW - 1) / (32 * NW)) * 32;
+  const int k0 = wave * kper, k1 = min(khalf, k0 + kper);
+  f32x4_t acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
+  constexpr int U = SK_UNROLL;
+  for (int k = k0; k < k1; k += 32 * U) {
+    u32x4_t wv[U], a0[U], a1[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int gk = k + 32 * u;
+      const bool in0 = gk + kg < k1 && gk + kg < K;       // within the wave's range of a half
+      const bool in1 = in0 && khalf + gk + kg < K;        // and, for the second half, within K
+      wv[u] = ((half ? in1 : in0) && gn < N) ? load16(wrow + (size_t)gk * kmul) : zero;
+      a0[u] = (in0 && col < M) ? load16(arow + (size_t)gk * amul) : zero;
+      a1[u] = (in1 && col < M) ? load16(arow + (size_t)(khalf + gk) * amul) : zero;
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      acc0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(a0[u]), as_bf16x8(wv[u]), acc0, 0, 0, 0);
+      acc1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(a1[u]), as_bf16x8(wv[u]), acc1, 0, 0, 0);
+    }
+  }
+#pragma unroll
+  for (int v = 0; v < 4; ++v) {
+    red[wave][0][lane][v] = acc0[v];
+    red[wave][1][lane][v] = acc1[v];
+  }
+  __syncthreads();
+  if (wave != 0) return;
+  // columns 0-7: the first half's sums of this lane and the second half's of the lane 8 further
+  const bool mine = half == 0 && gn < N;
+  const float bv = (bias && mine) ? bias[gn] : 0.f;
+#pragma unroll
+  for (int v = 0; v < 4; ++v) {
+    const int gm = 4 * (lane / 16) + v;
+    float q = 0.f;
+    if (mine && gm < M) {
+      float lo = red[0][0][lane][v], hi = red[0][1][lane + 8][v];
+#pragma unroll
+      for (int w = 1; w < NW; ++w) {
+        lo += red[w][0][lane][v];
+        hi += red[w][1][lane + 8][v];
+      }
+      const float x = resid_in[v] + ((lo + hi) + bv);
+      ro.resid[(size_t)gm * ro.ldr + gn] = x;
+      if (ro.rows != nullptr) {
+        const size_t at = ro.rows_frag ? ((size_t)(gn / 8) * 16 + gm) * 8 + gn % 8
+                                       : (size_t)gm * N + gn;
+        ro.rows[at] = f32_to_bf16(x * norm_w_in);
+      }
+      q = x * x;
+    }
+    if (ro.rows != nullptr) {
+      // the sum of squares over the block's 8 columns, row by row
       q += __shfl_xor(q, 1, WAVE);
       q += __shfl_xor(q, 2, WAVE);
       q += __shfl_xor(q, 4, WAVE);
-      q += __shfl_xor(q, 8, WAVE);
-      if (lane % 16 == 0 && gm < M) ro.ss[(size_t)blockIdx.x * M + gm] = q;
+      if (col == 0 && gm < M) ro.ss[(size_t)blockIdx.x * M + gm] = q;
     }
   }
+}
+
+static void launch_into_resid(const bf16_t* A, const bf16_t* W, const float* bias, int M, int N,
+                              int K, int lda, const ResidOut& ro, hipStream_t stream,
+                              const bf16_t* Wf, int a_frag) {
+  const int w_frag = Wf != nullptr;
+  if (Wf) W = Wf;
+  const dim3 grid((N + 7) / 8);
+  // K a wave: 128 or more where K allows it
+  if (K >= 4096)
+    hipLaunchKernelGGL((gemm_bf16_into_resid_kernel<16>), grid, dim3(16 * WAVE), 0, stream, A, W,
+                       bias, M, N, K, lda, ro, w_frag, a_frag);
+  else if (K >= 1024)
+    hipLaunchKernelGGL((gemm_bf16_into_resid_kernel<8>), grid, dim3(8 * WAVE), 0, stream, A, W,
+                       bias, M, N, K, lda, ro, w_frag, a_frag);
+  else
+    hipLaunchKernelGGL((gemm_bf16_into_resid_kernel<4>), grid, dim3(4 * WAVE), 0, stream, A, W,
+                       bias, M, N, K, lda, ro, w_frag, a_frag);
 }
 
 struct Fuse {
   RowScale rsc;
   ResidOut ro;
+  int c_frag = 0;
 };
 
 template <typename TO, int MT, int NW, int EPI, int NT = 1>
@@ -995,8 +1098,8 @@ static void launch_skinny(const bf16_t* A, const bf16_t* W, const float* bias, T
   if (Wf) W = Wf;
   const dim3 grid(EPI == 3 ? (N + 7) / 8 : (N + 16 * NT - 1) / (16 * NT), ksplit);
   hipLaunchKernelGGL((gemm_bf16_skinny_kernel<TO, MT, NW, EPI, NT>), grid, dim3(NW * WAVE), 0,
-                     stream, A, W, bias, C, M, N, K, lda, ldc, cs, fuse.rsc, fuse.ro, w_frag,
-                     a_frag);
+                     stream, A, W, bias, C, M, N, K, lda, ldc, cs, fuse.rsc, w_frag, a_frag,
+                     (MT == 1 && EPI != 0) ? fuse.c_frag : 0);
 }
 
 // more waves a block when there are few blocks, so that about 2048 waves or more stream W
@@ -1019,7 +1122,7 @@ static void launch_skinny_mt(const bf16_t* A, const bf16_t* W, const float* bias
   // With W in fragment order one tile a wave is the faster up to 11 rows (50 against 56 us at 8
   // rows, 56 either way at 12, 62 against 56 at 16).
   if constexpr (EPI == 0 && MT == 1) {
-    if (!fuse.ro.resid && M >= (Wf ? 12 : 8) && (long)(N / 64) * ksplit >= 512) {
+    if (M >= (Wf ? 12 : 8) && (long)(N / 64) * ksplit >= 512) {
       launch_skinny<TO, MT, 4, EPI, 4>(A, W, bias, C, M, N, K, lda, ldc, ksplit, cs, stream,
                                        fuse, Wf, a_frag);
       return;
@@ -1275,9 +1378,14 @@ static int launch_bf16(const bf16_t* A, const bf16_t* W, const float* bias, TO* 
   // a_frag: the rows of A lie in fragment order, which only the kernel for 1 to 16 rows reads
   if (a_frag && (M > 16 || force_kernel == 1 || force_kernel >= 3)) return (int)hipErrorInvalidValue;
   // so are the row scale and the residual epilogue (and the latter only with K in one piece)
-  const bool fused = fuse.rsc.ss != nullptr || fuse.ro.resid != nullptr;
+  const bool fused = fuse.rsc.ss != nullptr || fuse.ro.resid != nullptr || fuse.c_frag;
+  if (fuse.c_frag && (EPI == 0 || (N % 32))) return (int)hipErrorInvalidValue;
   if (fused && (M > 16 || force_kernel == 1 || force_kernel >= 3)) return (int)hipErrorInvalidValue;
-  if (fuse.ro.resid != nullptr && (EPI != 0 || ksplit != 1)) return (int)hipErrorInvalidValue;
+  if (fuse.ro.resid != nullptr) {
+    if (EPI != 0 || ksplit != 1 || fuse.rsc.ss != nullptr) return (int)hipErrorInvalidValue;
+    launch_into_resid(A, W, bias, M, N, K, lda, fuse.ro, stream, Wf, a_frag);
+    KAPPAI_RETURN_LAUNCH_STATUS();
+  }
   if (fuse.rsc.ss != nullptr && ksplit != 1) return (int)hipErrorInvalidValue;
   // Wf: W once more in fragment order, for the kernels of 1 to 64 rows (see the first of them);
   // the others read W
@@ -1344,9 +1452,10 @@ static bool frag_ok(const void* W_frag, int rows, int K) {
 // scale_ss [scale_parts][M] (or null) scales every result row by 1 / sqrt(sum of its parts / K +
 // scale_eps); resid [M, ldr] (or null; float output, ksplit 1) receives the result added in place
 // instead of C, and with norm_w also rows_out (bf16(resid * norm_w), [M, N] or fragment order)
-// and ss_out [(N + 15) / 16][M].
+// and ss_out [(N + 7) / 8][M].
 static bool fuse_ok(const Fuse& f, int M, int N, int K, int out_is_f32, int ksplit) {
   if (f.rsc.ss != nullptr && (M > 16 || f.rsc.n_parts < 1 || ksplit != 1)) return false;
+  if (f.c_frag && M > 16) return false;
   if (f.ro.resid != nullptr) {
     if (M > 16 || !out_is_f32 || ksplit != 1 || f.ro.ldr < N) return false;
     if (f.ro.norm_w != nullptr && (f.ro.rows == nullptr || f.ro.ss == nullptr)) return false;
@@ -1386,12 +1495,12 @@ extern "C" int kappai_gemm_bf16(const void* A, const void* W, const void* W_frag
 extern "C" int kappai_gemm_bf16_swiglu(const void* A, const void* W, const void* W_frag, void* C,
                                        int M, int F, int K, int lda, int ldc, int force_kernel,
                                        int a_frag, const float* scale_ss, int scale_parts,
-                                       float scale_eps, hipStream_t stream) {
+                                       float scale_eps, int c_frag, hipStream_t stream) {
   if (M <= 0 || F <= 0) return 0;
   if ((K % 8) || (lda % 8) || (F % 16)) return (int)hipErrorInvalidValue;
   if (force_kernel == 2 && M > 64) return (int)hipErrorInvalidValue;
   if (!frag_ok(W_frag, 2 * F, K) || (a_frag && (K % 32))) return (int)hipErrorInvalidValue;
-  Fuse fuse{RowScale{scale_ss, scale_parts, scale_eps}, ResidOut{}};
+  Fuse fuse{RowScale{scale_ss, scale_parts, scale_eps}, ResidOut{}, c_frag};
   if (!fuse_ok(fuse, M, F, K, 0, 1)) return (int)hipErrorInvalidValue;
   return launch_bf16<bf16_t, 1>((const bf16_t*)A, (const bf16_t*)W, nullptr, (bf16_t*)C, M, F, K,
                                 lda, ldc, force_kernel, 1, stream, ConvStep{},
@@ -1407,13 +1516,13 @@ extern "C" int kappai_gemm_bf16_shortconv_step(const void* A, const void* W, con
                                                float* state, const int* seg_pos0,
                                                const int* seg_slot, int L, int a_frag,
                                                const float* scale_ss, int scale_parts,
-                                               float scale_eps, hipStream_t stream) {
+                                               float scale_eps, int c_frag, hipStream_t stream) {
   if (M <= 0 || D <= 0) return 0;
   if ((K % 8) || (lda % 8) || (D % 16) || M > 64 || L < 2) return (int)hipErrorInvalidValue;
   if (!frag_ok(W_frag, 3 * D, K) || (a_frag && ((K % 32) || M > 16)))
     return (int)hipErrorInvalidValue;
-  Fuse fuse{RowScale{scale_ss, scale_parts, scale_eps}, ResidOut{}};
-  if (!fuse_ok(fuse, M, D, K, 0, 1)) return (int)hipErrorInvalidValue;
+  Fuse fuse{RowScale{scale_ss, scale_parts, scale_eps}, ResidOut{}, c_frag};
+  if (!fuse_ok(fuse, M, D, K, 0, 1) || (c_frag && (D % 32))) return (int)hipErrorInvalidValue;
   const bf16_t* wf = (const bf16_t*)W_frag;
   ConvStep cs{taps, conv_bias, state, seg_pos0, seg_slot, L};
   if (D / 16 < 256) {

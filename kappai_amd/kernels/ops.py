@@ -413,7 +413,7 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] =
             _need(nw.shape == (N,), lambda: f"linear: norm weight {tuple(nw.shape)} for N={N}")
             fragment = FRAGMENT_ROWS_FROM <= M and FragmentRows.fits(M, N, BF16)
             rows = torch.empty((16 if fragment else M, N), dtype=BF16, device=x.device)
-            ss = torch.empty(((N + 15) // 16, M), dtype=F32, device=x.device)
+            ss = torch.empty(((N + 7) // 8, M), dtype=F32, device=x.device)
         check(library("gemm").kappai_gemm_bf16(
             _ptr(xb), _ptr(weight), _frag(weight, weight_frag), _ptr(bias), _vp(0), _c_int(M),
             _c_int(N), _c_int(K), _c_int(lda), _c_int(N), _c_int(1), _c_int(force_kernel),
@@ -454,11 +454,17 @@ def interleave_gate_up(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
     return torch.cat([g, u], dim=1).reshape(2 * F, K).contiguous()
 
 
+def _out_in_fragment_order(wanted: bool, M: int, N: int, force_kernel: int) -> bool:
+    return (wanted and FRAGMENT_ROWS_FROM <= M <= FUSED_MAX_ROWS and N % 32 == 0
+            and force_kernel in (0, 2))
+
+
 def linear_swiglu(x: torch.Tensor, weight: torch.Tensor, force_kernel: int = 0,
-                  weight_frag: Optional[torch.Tensor] = None) -> torch.Tensor:
+                  weight_frag: Optional[torch.Tensor] = None, out_fragment: bool = False):
     """``silu(x Wg^T) * (x Wu^T)`` in one kernel: ``weight`` [2F, K] holds the gate and up
     matrices interleaved by ``interleave_gate_up``; bfloat16 only.  Returns [M, F].  ``x`` may
-    be ``ScaledRows`` or ``FragmentRows``."""
+    be ``ScaledRows`` or ``FragmentRows``.  ``out_fragment``: with 8 to 16 rows the result may
+    come back as ``FragmentRows`` for the product that follows."""
     scale = None
     if isinstance(x, ScaledRows):
         if (force_kernel not in (0, 2) or weight.dtype != BF16 or weight.dim() != 2
@@ -488,20 +494,23 @@ def linear_swiglu(x: torch.Tensor, weight: torch.Tensor, force_kernel: int = 0,
     _need(K % 8 == 0 and lda % 8 == 0 and x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0,
           lambda: f"linear_swiglu: K ({K}) and the row stride ({lda}) must be multiples of 8 "
                   "and the tensors 16-byte aligned")
-    out = torch.empty((M, F), dtype=BF16, device=x.device)
+    c_frag = _out_in_fragment_order(out_fragment, M, F, force_kernel)
+    out = torch.empty((16 if c_frag else M, F), dtype=BF16, device=x.device)
     check(library("gemm").kappai_gemm_bf16_swiglu(
         _ptr(x), _ptr(weight), _frag(weight, weight_frag), _ptr(out), _c_int(M), _c_int(F), _c_int(K),
         _c_int(lda), _c_int(F),
         _c_int(force_kernel), _c_int(a_frag),
-        *(scale._scale_args() if scale is not None else _NO_SCALE), _stream()), "gemm_bf16_swiglu")
-    return out
+        *(scale._scale_args() if scale is not None else _NO_SCALE), _c_int(1 if c_frag else 0),
+        _stream()), "gemm_bf16_swiglu")
+    return FragmentRows(out, M, None) if c_frag else out
 
 
 def linear_shortconv_step(x: torch.Tensor, in_proj: torch.Tensor, in_bias: Optional[torch.Tensor],
                           taps: torch.Tensor, conv_bias: Optional[torch.Tensor],
                           state: torch.Tensor, seg_pos0: torch.Tensor,
                           seg_slot: torch.Tensor,
-                          weight_frag: Optional[torch.Tensor] = None) -> torch.Tensor:
+                          weight_frag: Optional[torch.Tensor] = None,
+                          out_fragment: bool = False):
     """A conv layer's decode step in one kernel, for a batch in which every row is its own
     segment: ``proj = x in_proj^T (+ bias)`` cut into (B | C | x), ``C * conv(B * x)`` with the
     rows' state slots read and shifted.  bfloat16, at most 64 rows, width a multiple of 16.
@@ -544,14 +553,15 @@ def linear_shortconv_step(x: torch.Tensor, in_proj: torch.Tensor, in_bias: Optio
         if t is not None:
             _gpu(n, t, F32)
             _need(t.shape == shp, lambda: f"{n} must be {shp}")
-    out = torch.empty((M, D), dtype=BF16, device=x.device)
+    c_frag = _out_in_fragment_order(out_fragment, M, D, 0)
+    out = torch.empty((16 if c_frag else M, D), dtype=BF16, device=x.device)
     check(library("gemm").kappai_gemm_bf16_shortconv_step(
         _ptr(x), _ptr(in_proj), _frag(in_proj, weight_frag), _ptr(in_bias), _ptr(out), _c_int(M),
         _c_int(D), _c_int(K),
         _c_int(lda), _ptr(taps), _ptr(conv_bias), _ptr(state), _ptr(seg_pos0), _ptr(seg_slot),
         _c_int(L), _c_int(a_frag), *(scale._scale_args() if scale is not None else _NO_SCALE),
-        _stream()), "gemm_bf16_shortconv_step")
-    return out
+        _c_int(1 if c_frag else 0), _stream()), "gemm_bf16_shortconv_step")
+    return FragmentRows(out, M, None) if c_frag else out
 
 
 # ---------------------------------------------------------------------------------------

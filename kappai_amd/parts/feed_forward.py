@@ -41,7 +41,8 @@ class SwiGLU(FeedForward):
     def forward(self, x, batch, into=None):
         if self.fused and x.dtype == torch.bfloat16:
             return self.down.forward(
-                ops.linear_swiglu(x, self.gate_up.weight, weight_frag=self.gate_up.weight_frag),
+                ops.linear_swiglu(x, self.gate_up.weight, weight_frag=self.gate_up.weight_frag,
+                                  out_fragment=True),
                 partial_sums=True, add_into=into)
         return self.down.forward(ops.swiglu(self.gate_up.forward(x)), partial_sums=True,
                                  add_into=into)

@@ -73,7 +73,7 @@ def interleave_gate_up(gate, up):
     return torch.cat([g, u], dim=1).reshape(2 * F, K).contiguous()
 
 
-def linear_swiglu(x, weight, force_kernel=0, weight_frag=None):
+def linear_swiglu(x, weight, force_kernel=0, weight_frag=None, out_fragment=False):
     F = weight.shape[0] // 2
     y = (x.to(F32) @ weight.to(F32).T).reshape(x.shape[0], F // SWIGLU_GROUP, 2, SWIGLU_GROUP)
     g, u = y[:, :, 0, :].reshape(-1, F), y[:, :, 1, :].reshape(-1, F)
@@ -103,7 +103,7 @@ def shortconv(proj, taps, bias, state, row_seg, seg_start, seg_pos0, seg_slot):
 
 
 def linear_shortconv_step(x, in_proj, in_bias, taps, conv_bias, state, seg_pos0, seg_slot,
-                          weight_frag=None):
+                          weight_frag=None, out_fragment=False):
     M = x.shape[0]
     proj = linear(x, in_proj, in_bias)
     row_seg = torch.arange(M, dtype=torch.int32)

@@ -498,6 +498,37 @@ def test_linear_swiglu_on_scaled_rows(ops, M, F, K):
     close(got.float(), g / (1 + torch.exp(-g)) * u, 3 * BF16_ULP, "swiglu on scaled rows")
 
 
+@pytest.mark.parametrize("M", [1, 8, 11, 16])
+def test_epilogues_write_rows_in_fragment_order(ops, M):
+    """With 8 to 16 rows the SwiGLU product and the fused conv step can hand their result to the
+    next product in the order in which it loads rows: the same numbers, bit for bit, and the
+    next product gives the same result from either."""
+    K, F, D, L = 256, 320, 96, 3
+    x = rand((M, K), BF16, 110).to(DEV)
+    w = ops.interleave_gate_up(rand((F, K), BF16, 111, 0.1).to(DEV), rand((F, K), BF16, 112, 0.1).to(DEV))
+    plain, frag = ops.linear_swiglu(x, w), ops.linear_swiglu(x, w, out_fragment=True)
+    w2 = rand((48, F), BF16, 113, 0.1).to(DEV)
+    if M >= 8:
+        assert isinstance(frag, ops.FragmentRows) and frag.shape == (M, F)
+        assert torch.equal(frag.materialize(), plain)
+        assert torch.equal(ops.linear(frag, w2, out_dtype=F32), ops.linear(plain, w2, out_dtype=F32))
+    else:
+        assert torch.equal(frag, plain)
+    wi = rand((3 * D, K), BF16, 114, 0.2).to(DEV)
+    taps = rand((D, L), F32, 115, 0.5).to(DEV)
+    state = rand((M + 1, D, L - 1), F32, 116).to(DEV)
+    pos0 = torch.full((M,), 3, dtype=torch.int32, device=DEV)
+    slot = torch.arange(M, dtype=torch.int32, device=DEV)
+    st_a, st_b = state.clone(), state.clone()
+    plain = ops.linear_shortconv_step(x, wi, None, taps, None, st_a, pos0, slot)
+    frag = ops.linear_shortconv_step(x, wi, None, taps, None, st_b, pos0, slot, out_fragment=True)
+    assert torch.equal(st_a, st_b)
+    if M >= 8:
+        assert torch.equal(frag.materialize(), plain)
+    else:
+        assert torch.equal(frag, plain)
+
+
 def test_products_that_cannot_fold_go_the_ordinary_way(ops):
     """More than 16 rows, or a float32 matrix: ``add_into`` is not taken up and the product
     comes back as always; scaled rows that meet a float32 matrix are made by the norm kernel."""
