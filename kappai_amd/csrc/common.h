@@ -60,15 +60,44 @@ __device__ __forceinline__ void store8(bf16_t* p, const float* v) {
   *reinterpret_cast<uint4*>(p) = o;
 }
 
+// Exchanges inside a wave without a trip through LDS: the partner lane ^ 1 or ^ 2 (inside a quad)
+// and the lanes 4 and 8 further in a row of 16 come by data-parallel moves, the partners lane ^ 16
+// and lane ^ 32 by the row and half swaps of gfx950.
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float v) {
+  return __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(v), CTRL, 0xf, 0xf, false));
+}
+__device__ __forceinline__ float lane_xor16(float x) {
+  const uint32_t u = __float_as_uint(x);
+  const auto r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+  // r[0] = the even rows' values in both rows of a pair, r[1] = the odd rows'
+  return __uint_as_float((threadIdx.x & 16) ? r[0] : r[1]);
+}
+__device__ __forceinline__ float lane_xor32(float x) {
+  const uint32_t u = __float_as_uint(x);
+  const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  return __uint_as_float((threadIdx.x & 32) ? r[0] : r[1]);
+}
+
+// Sum and maximum over the 64 lanes, the same value in every lane, in a fixed order: quads, the
+// row of 16 (two rotations), the pair of rows, the two halves.
 __device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int m = WAVE / 2; m > 0; m >>= 1) v += __shfl_xor(v, m, WAVE);
+  v += dpp_move<0xB1>(v);     // quad_perm [1, 0, 3, 2]
+  v += dpp_move<0x4E>(v);     // quad_perm [2, 3, 0, 1]
+  v += dpp_move<0x124>(v);    // row_ror 4
+  v += dpp_move<0x128>(v);    // row_ror 8
+  v += lane_xor16(v);
+  v += lane_xor32(v);
   return v;
 }
 
 __device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-  for (int m = WAVE / 2; m > 0; m >>= 1) v = fmaxf(v, __shfl_xor(v, m, WAVE));
+  v = fmaxf(v, dpp_move<0xB1>(v));
+  v = fmaxf(v, dpp_move<0x4E>(v));
+  v = fmaxf(v, dpp_move<0x124>(v));
+  v = fmaxf(v, dpp_move<0x128>(v));
+  v = fmaxf(v, lane_xor16(v));
+  v = fmaxf(v, lane_xor32(v));
   return v;
 }
 

@@ -763,7 +763,7 @@ struct ConvStep {
 //   RowScale (the product that follows): its rows are such x * w, and every result is
 //     multiplied by 1 / sqrt(sum_p ss[p][m] / K + eps) before bias and epilogue.
 struct RowScale {
-  const float* ss;   // [n_parts][M], or null: rows are used as they are
+  const float* ss;   // [n_parts][16] (a row's value at [p][m]), or null: rows are used as they are
   int n_parts;
   float eps;
 };
@@ -773,11 +773,11 @@ struct ResidOut {
   const float* norm_w;   // [N]; null: no rows for a next product
   bf16_t* rows;          // [M, N] or 16 rows in fragment order
   int rows_frag;
-  float* ss;             // [gridDim.x][M]
+  float* ss;             // [gridDim.x][16]: a part holds one value a row, rows beyond M unwritten
 };
 
 template <typename TO, int MT, int NW, int EPI, int NT>
-__global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny_kernel(
+__global__ __launch_bounds__((NW < 16 ? NW + 1 : NW) * WAVE) void gemm_bf16_skinny_kernel(
     const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, const float* __restrict__ bias,
     TO* __restrict__ C, int M, int N, int K, int lda, int ldc, ConvStep cs, RowScale rsc,
     int w_frag, int a_frag, int c_frag) {
@@ -828,21 +828,42 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny_kernel(
     arow[t] = a_frag ? A + ((size_t)(kg / 8) * 16 + (gm < M ? gm : 0)) * 8
                      : A + (size_t)(gm < M ? gm : 0) * lda + kg;
   }
-  // What the epilogue needs from memory is asked for early, so that it has arrived when the
-  // stream of W has gone through: the residual values and norm weight of this block's columns
-  // (ResidOut) now, and 1 / rms of the rows (RowScale; wave w makes it for rows w, w + NW, ...)
-  // behind the first loads of W, whose wait it then shares.
-  __shared__ float row_scale[16 * MT];
-  bool scale_made = rsc.ss == nullptr;
-  auto make_row_scale = [&]() {
-    for (int m = wave; m < M; m += NW) {
-      float part = 0.f;
-      for (int p = lane; p < rsc.n_parts; p += WAVE) part += rsc.ss[(size_t)p * M + m];
-      part = wave_sum(part);
-      if (lane == 0) row_scale[m] = 1.0f / sqrtf(part / (float)K + rsc.eps);
+  __shared__ float row_ss[16];
+  if (wave == NW) {
+    // The block's extra wave (launched only with a RowScale) adds up the rows' sums of squares
+    // while the others stream W: a lane takes parts lane, lane + 64, ... of all rows at once (a
+    // part is 16 floats, one a row), four parts' loads in flight, then the lanes are summed.
+    float q[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) q[i] = 0.f;
+    for (int p0 = 0; p0 < rsc.n_parts; p0 += 4 * WAVE) {
+      float4 v[4][4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int p = p0 + u * WAVE + lane;
+        const float4* src = reinterpret_cast<const float4*>(rsc.ss + (size_t)p * 16);
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          v[u][j] = (p < rsc.n_parts && 4 * j < M) ? src[j] : make_float4(0.f, 0.f, 0.f, 0.f);
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          q[4 * j] += v[u][j].x; q[4 * j + 1] += v[u][j].y;
+          q[4 * j + 2] += v[u][j].z; q[4 * j + 3] += v[u][j].w;
+        }
     }
-    scale_made = true;
-  };
+    // (all 16 without a branch between them, so that the sixteen chains of exchanges overlap)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) q[i] = wave_sum(q[i]);
+    if (lane < 16) {
+      float t = q[0];
+#pragma unroll
+      for (int i = 1; i < 16; ++i) t = lane == i ? q[i] : t;
+      row_ss[lane] = t;
+    }
+  }
   const int kblk = ((K + 32 * (int)gridDim.y - 1) / (32 * (int)gridDim.y)) * 32;   // K a block
   const int kb0 = blockIdx.y * kblk, kb1 = min(K, kb0 + kblk);
   const int kper = ((kb1 - kb0 + 32 * NW - 1) / (32 * NW)) * 32;
@@ -878,17 +899,20 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny_kernel(
         for (int t = 0; t < MT; ++t)
           av[u][t] = (kin && t * 16 + col < M) ? load16(arow[t] + (size_t)gk * (a_frag ? 16 : 1)) : zero;
       }
-      if (!scale_made) make_row_scale();
       products(wv, av);
     }
   }
-  if (!scale_made) make_row_scale();       // (a wave without a K range of its own)
+  if (wave < NW) {
 #pragma unroll
-  for (int t = 0; t < NG * MT; ++t)
+    for (int t = 0; t < NG * MT; ++t)
 #pragma unroll
-    for (int v = 0; v < 4; ++v) red[wave][t][lane][v] = acc[t][v];
+      for (int v = 0; v < 4; ++v) red[wave][t][lane][v] = acc[t][v];
+  }
   __syncthreads();
-  auto scale_of = [&](int gm) { return rsc.ss != nullptr ? row_scale[gm] : 1.0f; };
+  if (wave >= NW) return;
+  auto scale_of = [&](int gm) {
+    return rsc.ss != nullptr ? 1.0f / sqrtf(row_ss[gm] / (float)K + rsc.eps) : 1.0f;
+  };
   // the first MT waves each sum one row tile over the NW partial results, in a fixed order
   if (EPI == 0 && NT > 1) {
     // waves take the NT * MT tiles in turn
@@ -1060,7 +1084,7 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_into_resid_kernel(
       q += __shfl_xor(q, 1, WAVE);
       q += __shfl_xor(q, 2, WAVE);
       q += __shfl_xor(q, 4, WAVE);
-      if (col == 0 && gm < M) ro.ss[(size_t)blockIdx.x * M + gm] = q;
+      if (col == 0 && gm < M) ro.ss[(size_t)blockIdx.x * 16 + gm] = q;
     }
   }
 }
@@ -1097,7 +1121,10 @@ static void launch_skinny(const bf16_t* A, const bf16_t* W, const float* bias, T
   const int w_frag = Wf != nullptr;
   if (Wf) W = Wf;
   const dim3 grid(EPI == 3 ? (N + 7) / 8 : (N + 16 * NT - 1) / (16 * NT), ksplit);
-  hipLaunchKernelGGL((gemm_bf16_skinny_kernel<TO, MT, NW, EPI, NT>), grid, dim3(NW * WAVE), 0,
+  // one wave more when there are row scales to make (launch_skinny_mt keeps NW below 16 then)
+  const int waves = fuse.rsc.ss != nullptr ? NW + 1 : NW;
+  if (waves * WAVE > 1024) return;
+  hipLaunchKernelGGL((gemm_bf16_skinny_kernel<TO, MT, NW, EPI, NT>), grid, dim3(waves * WAVE), 0,
                      stream, A, W, bias, C, M, N, K, lda, ldc, cs, fuse.rsc, w_frag, a_frag,
                      (MT == 1 && EPI != 0) ? fuse.c_frag : 0);
 }
@@ -1135,6 +1162,9 @@ static void launch_skinny_mt(const bf16_t* A, const bf16_t* W, const float* bias
   if (blocks * 4 >= 2048 || kb <= 512 || MAXW < 8)
     launch_skinny<TO, MT, 4, EPI>(A, W, bias, C, M, N, K, lda, ldc, ksplit, cs, stream, fuse, Wf, a_frag);
   else if (blocks * 8 >= 2048 || kb <= 1024 || MAXW < 16)
+    launch_skinny<TO, MT, (MAXW >= 8 ? 8 : 4), EPI>(A, W, bias, C, M, N, K, lda, ldc, ksplit, cs,
+                                                    stream, fuse, Wf, a_frag);
+  else if (fuse.rsc.ss != nullptr)      // (the block needs room for the wave that makes the scales)
     launch_skinny<TO, MT, (MAXW >= 8 ? 8 : 4), EPI>(A, W, bias, C, M, N, K, lda, ldc, ksplit, cs,
                                                     stream, fuse, Wf, a_frag);
   else
@@ -1449,10 +1479,10 @@ static bool frag_ok(const void* W_frag, int rows, int K) {
 }
 
 // The fused forms (at most 16 rows, see RowScale and ResidOut in the kernel for 1 to 16 rows):
-// scale_ss [scale_parts][M] (or null) scales every result row by 1 / sqrt(sum of its parts / K +
+// scale_ss [scale_parts][16] (or null) scales every result row by 1 / sqrt(sum of its parts / K +
 // scale_eps); resid [M, ldr] (or null; float output, ksplit 1) receives the result added in place
 // instead of C, and with norm_w also rows_out (bf16(resid * norm_w), [M, N] or fragment order)
-// and ss_out [(N + 7) / 8][M].
+// and ss_out [(N + 7) / 8][16].
 static bool fuse_ok(const Fuse& f, int M, int N, int K, int out_is_f32, int ksplit) {
   if (f.rsc.ss != nullptr && (M > 16 || f.rsc.n_parts < 1 || ksplit != 1)) return false;
   if (f.c_frag && M > 16) return false;

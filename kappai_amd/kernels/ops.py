@@ -163,8 +163,8 @@ class ScaledRows(Added):
     """At most 16 rows of a decode step, on their way from a product that added its result into
     the residual stream (``AddInto`` with a norm weight) to the product after the RMSNorm that
     follows: ``data`` holds bf16(resid * weight), not yet divided by the rows' root mean square
-    ([n, D], or 16 rows in fragment order), and ``ss`` [parts, n] the sums of resid^2 over ranges
-    of columns.  ``linear``, ``linear_swiglu`` and ``linear_shortconv_step`` take it in place of
+    ([n, D], or 16 rows in fragment order), and ``ss`` [parts, 16] the sums of resid^2 over ranges
+    of columns (row m at [:, m]; the columns beyond n hold nothing).  ``linear``, ``linear_swiglu`` and ``linear_shortconv_step`` take it in place of
     the normalised rows and scale their results by 1 / sqrt(sum of the parts / D + eps), which is
     the same product (RMSNorm(x) W^T = (x * w) W^T / rms(x)) without a kernel in between.
     ``materialize`` runs the ordinary norm kernel on the residual instead.  ``resid_after`` is
@@ -413,7 +413,7 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] =
             _need(nw.shape == (N,), lambda: f"linear: norm weight {tuple(nw.shape)} for N={N}")
             fragment = FRAGMENT_ROWS_FROM <= M and FragmentRows.fits(M, N, BF16)
             rows = torch.empty((16 if fragment else M, N), dtype=BF16, device=x.device)
-            ss = torch.empty(((N + 7) // 8, M), dtype=F32, device=x.device)
+            ss = torch.empty(((N + 7) // 8, 16), dtype=F32, device=x.device)
         check(library("gemm").kappai_gemm_bf16(
             _ptr(xb), _ptr(weight), _frag(weight, weight_frag), _ptr(bias), _vp(0), _c_int(M),
             _c_int(N), _c_int(K), _c_int(lda), _c_int(N), _c_int(1), _c_int(force_kernel),
