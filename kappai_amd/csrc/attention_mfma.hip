@@ -780,25 +780,20 @@ __global__ __launch_bounds__(8 * WAVE) void attn_prefill_shared_kernel(
 // keys whose loads a wave has in flight at once (their registers: keys * HEAD_DIM / 64)
 #define D_KPW (HEAD_DIM <= 64 ? 128 : (HEAD_DIM <= 128 ? 64 : 32))
 
-__global__ __launch_bounds__(64) void attn_decode_kernel(
+// One wave's share of a row's attention: the query heads of kv head g (columns) against the keys
+// of the chunks c0 = first, first + stride, ... below k_end (D_KPW keys each), with a running
+// maximum and sum per column.  Leaves the unnormalised output in o (lane: column lane % 16, d
+// rows 16 mt + 4 (lane / 16) + v), the maximum (in units of log 2) in m_run, the sum in l_run.
+__device__ __forceinline__ void attn_decode_wave(
     const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ k_pool,
-    const bf16_t* __restrict__ vt_pool, float* __restrict__ part_o, float* __restrict__ part_ml,
-    const int* __restrict__ row_pos, const int* __restrict__ row_seg,
-    const int* __restrict__ block_tables, int max_blocks, int H, int G, int ps, int window,
-    float scale, int keys_per_split, int n_splits) {
-  const int t = blockIdx.x, g = blockIdx.y, split = blockIdx.z, lane = threadIdx.x;
+    const bf16_t* __restrict__ vt_pool, const int* __restrict__ bt, int max_blocks, int t, int g,
+    int H, int G, int ps, float scale, int lo, int hi, int first, int stride, int k_end,
+    f32x4_t (&o)[D_MT], float& m_run, float& l_run) {
+  const int lane = threadIdx.x % WAVE;
   const int rep = H / G;
   const int col = lane % 16, kg = lane / 16;
-  const int pos = row_pos[t];
-  const int* bt = block_tables + (size_t)row_seg[t] * max_blocks;
-  const int lo = (window > 0 && pos + 1 > window) ? pos + 1 - window : 0;
-  const int k_begin = (lo / 32) * 32 + split * keys_per_split;
-  const int k_end = min(k_begin + keys_per_split, pos + 1);     // exclusive
-  const int hi = k_end - 1;
   const bool head_ok = col < rep;
   const int h = g * rep + (head_ok ? col : 0);
-  const size_t pbase = ((size_t)t * H + h) * n_splits + split;
-
   bf16x8_t qf[D_KS];
   {
     const bf16_t* qr = q + (size_t)t * q_stride + (size_t)h * HEAD_DIM;
@@ -810,10 +805,10 @@ __global__ __launch_bounds__(64) void attn_decode_kernel(
       qf[ks] = as_frag(v);
     }
   }
-  f32x4_t o[D_MT];
 #pragma unroll
   for (int mt = 0; mt < D_MT; ++mt) o[mt] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
-  float m_run = -INFINITY, l_run = 0.f;
+  m_run = -INFINITY;
+  l_run = 0.f;
   const float sc = scale * LOG2E;
 
   // A wave takes its keys in chunks of D_KPW: first the chunk's page ids (one load, handed
@@ -821,7 +816,7 @@ __global__ __launch_bounds__(64) void attn_decode_kernel(
   // each), then the matrix products and the softmax: two memory round trips a chunk, whatever
   // its length.
   constexpr int NCH = D_KPW / 32;
-  for (int c0 = k_begin; c0 < k_end; c0 += D_KPW) {
+  for (int c0 = first; c0 < k_end; c0 += stride) {
     const int first_page = c0 / ps;
     int my_page = -1;
     if (first_page + lane < max_blocks && (first_page + lane) * ps <= hi)
@@ -898,6 +893,31 @@ __global__ __launch_bounds__(64) void attn_decode_kernel(
       }
     }
   }
+}
+
+// The keys of a row split over blocks: block (t, g, split) is one wave that takes the keys
+// k_begin + split * keys_per_split .. and writes its partial result; attn_merge adds them up.
+__global__ __launch_bounds__(64) void attn_decode_kernel(
+    const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ k_pool,
+    const bf16_t* __restrict__ vt_pool, float* __restrict__ part_o, float* __restrict__ part_ml,
+    const int* __restrict__ row_pos, const int* __restrict__ row_seg,
+    const int* __restrict__ block_tables, int max_blocks, int H, int G, int ps, int window,
+    float scale, int keys_per_split, int n_splits) {
+  const int t = blockIdx.x, g = blockIdx.y, split = blockIdx.z, lane = threadIdx.x;
+  const int rep = H / G;
+  const int col = lane % 16, kg = lane / 16;
+  const int pos = row_pos[t];
+  const int* bt = block_tables + (size_t)row_seg[t] * max_blocks;
+  const int lo = (window > 0 && pos + 1 > window) ? pos + 1 - window : 0;
+  const int k_begin = (lo / 32) * 32 + split * keys_per_split;
+  const int k_end = min(k_begin + keys_per_split, pos + 1);     // exclusive
+  const bool head_ok = col < rep;
+  const int h = g * rep + (head_ok ? col : 0);
+  const size_t pbase = ((size_t)t * H + h) * n_splits + split;
+  f32x4_t o[D_MT];
+  float m_run, l_run;
+  attn_decode_wave(q, q_stride, k_pool, vt_pool, bt, max_blocks, t, g, H, G, ps, scale, lo,
+                   k_end - 1, k_begin, D_KPW, k_end, o, m_run, l_run);
   if (!head_ok) return;
   if (kg == 0) {
     part_ml[2 * pbase] = m_run;
@@ -907,6 +927,66 @@ __global__ __launch_bounds__(64) void attn_decode_kernel(
 #pragma unroll
   for (int mt = 0; mt < D_MT; ++mt)
     *reinterpret_cast<f32x4_t*>(po + 16 * mt + 4 * kg) = o[mt];
+}
+
+// (eight waves at most: a wave keeps a whole chunk's loads in registers, which 16 waves a block
+// would not leave room for)
+#define D_BLOCK_MAX_WAVES 8
+// The keys of a row split over the waves of one block (t, g): wave w takes the chunks w, w + NW,
+// ... of D_KPW keys, the waves' results meet in LDS and are added up there in the order of the
+// waves, so that nothing goes through memory and no second kernel is needed.  The split of a row's
+// keys depends on the row's own position and on the number of waves only.  For batches with
+// (rows x kv heads) enough to fill the chip, or contexts short enough for one block.
+// LDS: sh_o [NW][rep][HEAD_DIM], then sh_m [NW][16], sh_l [NW][16] (floats).
+__global__ __launch_bounds__(D_BLOCK_MAX_WAVES * WAVE) void attn_decode_block_kernel(
+    const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ k_pool,
+    const bf16_t* __restrict__ vt_pool, bf16_t* __restrict__ out, int out_stride,
+    const int* __restrict__ row_pos, const int* __restrict__ row_seg,
+    const int* __restrict__ block_tables, int max_blocks, int H, int G, int ps, int window,
+    float scale) {
+  extern __shared__ float sh_dec[];
+  const int t = blockIdx.x, g = blockIdx.y;
+  const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE, NW = blockDim.x / WAVE;
+  const int rep = H / G;
+  const int col = lane % 16, kg = lane / 16;
+  const int pos = row_pos[t];
+  const int* bt = block_tables + (size_t)row_seg[t] * max_blocks;
+  const int lo = (window > 0 && pos + 1 > window) ? pos + 1 - window : 0;
+  const int k_begin = (lo / 32) * 32;
+  const int k_end = pos + 1;
+  f32x4_t o[D_MT];
+  float m_run, l_run;
+  attn_decode_wave(q, q_stride, k_pool, vt_pool, bt, max_blocks, t, g, H, G, ps, scale, lo, pos,
+                   k_begin + wave * D_KPW, NW * D_KPW, k_end, o, m_run, l_run);
+  float* sh_o = sh_dec;
+  float* sh_m = sh_dec + (size_t)NW * rep * HEAD_DIM;
+  float* sh_l = sh_m + NW * 16;
+  if (col < rep) {
+    float* po = sh_o + ((size_t)wave * rep + col) * HEAD_DIM;
+#pragma unroll
+    for (int mt = 0; mt < D_MT; ++mt)
+      *reinterpret_cast<f32x4_t*>(po + 16 * mt + 4 * kg) = o[mt];
+    if (kg == 0) {
+      sh_m[wave * 16 + col] = m_run;
+      sh_l[wave * 16 + col] = l_run;
+    }
+  }
+  __syncthreads();
+  // out[t, g rep + c, e] for (c, e) in turn over the block's threads
+  for (int i = threadIdx.x; i < rep * HEAD_DIM; i += blockDim.x) {
+    const int c = i / HEAD_DIM, e = i % HEAD_DIM;
+    float M = -INFINITY;
+    for (int w = 0; w < NW; ++w) M = fmaxf(M, sh_m[w * 16 + c]);
+    float L = 0.f, acc = 0.f;
+    for (int w = 0; w < NW; ++w) {
+      const float m = sh_m[w * 16 + c];
+      const float wgt = m == -INFINITY ? 0.f : fast_exp2(m - M);
+      L += sh_l[w * 16 + c] * wgt;
+      acc = fmaf(sh_o[((size_t)w * rep + c) * HEAD_DIM + e], wgt, acc);
+    }
+    const float inv = L > 0.f ? 1.0f / L : 0.f;
+    out[(size_t)t * out_stride + (size_t)(g * rep + c) * HEAD_DIM + e] = f32_to_bf16(acc * inv);
+  }
 }
 
 // out[t, h, :] = sum_s o_s 2^(m_s - M) / sum_s l_s 2^(m_s - M).  Four waves share the splits
@@ -967,6 +1047,37 @@ __global__ __launch_bounds__(MERGE_WAVES * WAVE) void attn_merge_kernel(
 }
 
 extern "C" int kappai_attn_keys_per_wave(void) { return D_KPW; }
+
+// Waves of a block of the decode kernel that merges in LDS, for `rep` query heads a kv head:
+// as many as 64 KB of LDS hold partial results for (D_BLOCK_MAX_WAVES at most), 0 if not even two.
+extern "C" int kappai_attn_decode_block_waves(int rep) {
+  if (rep < 1 || rep > 16) return 0;
+  const int per_wave = (rep * HEAD_DIM + 32) * (int)sizeof(float);
+  int nw = (64 * 1024) / per_wave;
+  nw = nw > D_BLOCK_MAX_WAVES ? D_BLOCK_MAX_WAVES : nw;
+  return nw >= 2 ? nw : 0;
+}
+
+// Decode attention with the keys of a row split over the `n_waves` waves of one block per (row, kv
+// head); no workspace, no second kernel.
+extern "C" int kappai_attn_decode_block(const void* q, int q_stride, const void* k_pool,
+                                        const void* vt_pool, void* out, int out_stride,
+                                        const int* row_pos, const int* row_seg,
+                                        const int* block_tables, int max_blocks, int T, int H,
+                                        int G, int ps, int window, float scale, int n_waves,
+                                        hipStream_t stream) {
+  if (T <= 0) return 0;
+  if (ps % 16 || G < 1 || H % G || H / G > 16 || G > 65535 || (q_stride % 8) || n_waves < 1 ||
+      n_waves > kappai_attn_decode_block_waves(H / G))
+    return (int)hipErrorInvalidValue;
+  const int rep = H / G;
+  const size_t lds = (size_t)n_waves * (rep * HEAD_DIM + 32) * sizeof(float);
+  hipLaunchKernelGGL(attn_decode_block_kernel, dim3(T, G), dim3(n_waves * WAVE), lds, stream,
+                     (const bf16_t*)q, q_stride, (const bf16_t*)k_pool, (const bf16_t*)vt_pool,
+                     (bf16_t*)out, out_stride, row_pos, row_seg, block_tables, max_blocks, H, G, ps,
+                     window, scale);
+  KAPPAI_RETURN_LAUNCH_STATUS();
+}
 
 extern "C" int kappai_attn_head_dim(void) { return HEAD_DIM; }
 

@@ -18,6 +18,11 @@ MAX_HEAD_DIM = 512
 MAX_GRID_Y = 65535
 DECODE_WAVES = 2048       # waves the split-key decode attention aims to have at work
 DECODE_MAX_SPLITS = 128   # partial results of a row's head that the merge kernel adds up at most
+# Keys up to which one block a (row, kv head) takes them all, its waves merging in LDS (8 requests
+# at 200 keys: 7.4 us against 9.4 for the split kernel and its merge; even at 1024 keys, and from
+# there on the split kernel wins: 22 against 35 us at 4096 keys, a wave taking its chunks one
+# after the other where the split kernel has a wave for each)
+DECODE_BLOCK_MAX_KEYS = 512
 
 _c_int, _c_float, _c_long, _vp = ctypes.c_int, ctypes.c_float, ctypes.c_long, ctypes.c_void_p
 
@@ -716,7 +721,8 @@ def paged_attention(q: torch.Tensor, n_heads: int, n_kv_heads: int, head_dim: in
     ``max_position`` sizes the splits), else the tiled kernel over ``q_tiles`` [tiles, 4] =
     (segment, first row, rows <= 32, place of the tile in its segment: index | tiles << 16, or 0).
     Everything else, float32 included, runs the plain
-    kernel.  ``kernel`` = "rows" | "prefill" | "decode" forces one (for tests);
+    kernel.  ``kernel`` = "rows" | "prefill" | "decode" | "decode-block" | "decode-split" forces
+    one (for tests);
     ``prefill_variant`` 1 / 2 forces the tiled kernel's form (2: key tiles shared by four query
     heads of a kv head through LDS; head sizes 64 and 128 only)."""
     H, G, d = n_heads, n_kv_heads, head_dim
@@ -768,10 +774,25 @@ def paged_attention(q: torch.Tensor, n_heads: int, n_kv_heads: int, head_dim: in
             _c_int(window or 0), _c_float(scale), _c_int(prefill_variant), _stream()),
             "attn_prefill")
         return out
-    _need(kernel == "decode", lambda: f"unknown attention kernel {kernel!r}")
+    _need(kernel in ("decode", "decode-block", "decode-split"),
+          lambda: f"unknown attention kernel {kernel!r}")
     _need(H // G <= 16, "the decode kernel takes at most 16 query heads per kv head")
     _need(max_position is not None, "the decode kernel needs the batch's largest position")
     n_keys = min(max_position + 1, window) + 32 if window else max_position + 1
+    # With few keys a block per (row, kv head) splits them over its waves and merges in LDS;
+    # else the keys are split over blocks, whose partial results a second kernel merges.
+    block_waves = lib.kappai_attn_decode_block_waves(H // G)
+    if kernel == "decode":
+        kernel = ("decode-block" if block_waves and n_keys <= DECODE_BLOCK_MAX_KEYS
+                  else "decode-split")
+    if kernel == "decode-block":
+        _need(block_waves > 0, "too many query heads a kv head for the block form")
+        check(lib.kappai_attn_decode_block(
+            _ptr(q), _c_int(q.stride(0)), _ptr(k_pool), _ptr(v_pool), _ptr(out), _c_int(H * d),
+            _ptr(row_pos), _ptr(row_seg), _ptr(block_tables), _c_int(block_tables.shape[1]),
+            _c_int(T), _c_int(H), _c_int(G), _c_int(page_size), _c_int(window or 0),
+            _c_float(scale), _c_int(block_waves), _stream()), "attn_decode_block")
+        return out
     # one wave keeps the loads of `kpw` keys in flight; splits are whole numbers of that, and
     # at most DECODE_MAX_SPLITS of them are merged
     kpw = lib.kappai_attn_keys_per_wave()

@@ -758,6 +758,8 @@ ATT_CASES = [
     (4, 1, 64, 48, [120, 0, 66], [80, 33, 2], 64, 1, True, 50),                 # window, page 48
     (4, 2, 64, 16, [20000, 9000], [1, 1], 64, 1, True, 0),       # decode over more than 64 key splits
     (8, 2, 64, 16, [12000], [70], 64, 1, True, 0),               # a portion after a long history
+    (16, 1, 256, 16, [300, 40], [1, 1], 256, 1, False, 0),      # decode: four waves' results fit LDS
+    (8, 4, 128, 32, [5000, 0, 129, 1023, 1024, 77], [1] * 6, 128, 1, True, 0),    # decode, head 128
 ]
 
 
@@ -792,14 +794,16 @@ def test_store_and_attention(ops, dtype, case):
                                ps, scale, window=window)
     kernels = ["rows"]
     if dtype == BF16 and ps % 16 == 0 and d % 16 == 0 and d <= 256:
-        kernels += ["prefill"] + (["decode"] if c["single"] and H // G <= 16 else [])
+        kernels += ["prefill"] + (["decode-split", "decode-block"]
+                                  if c["single"] and H // G <= 16 else [])
         if d in (64, 128) and (H // G) % 4 == 0:
             kernels += ["prefill-shared"]
     for kernel in kernels:
         got = ops.paged_attention(dev["qkv"], H, G, d, dev["k_pool"], dev["v_pool"],
                                   dev["row_pos"], dev["row_seg"], dev["bt"], ps, scale,
                                   window=window, q_tiles=dev["q_tiles"], single_rows=c["single"],
-                                  max_position=c["max_pos"], kernel=kernel.split("-")[0],
+                                  max_position=c["max_pos"],
+                                  kernel=kernel if kernel.startswith("decode") else kernel.split("-")[0],
                                   prefill_variant=2 if kernel == "prefill-shared" else 1)
         close(got.float(), want, tol * 2, f"attention kernel {kernel}")
 
@@ -890,7 +894,8 @@ def test_attention_finds_one_far_key(ops, dtype):
         # the query's own key (position n) must exist too: store zeros for it
         dev["k_pool"][bt[0, n // ps], :, n % ps, :] = 0
         want = marker.float().repeat_interleave(H // G, dim=0).reshape(1, H * d)
-        for kernel in (["rows", "prefill", "decode"] if dtype == BF16 else ["rows"]):
+        for kernel in (["rows", "prefill", "decode-split", "decode-block"] if dtype == BF16
+                       else ["rows"]):
             got = ops.paged_attention(dev["qkv"], H, G, d, dev["k_pool"], dev["v_pool"],
                                       dev["row_pos"], dev["row_seg"], dev["bt"], ps,
                                       1.0 / math.sqrt(d), q_tiles=dev["q_tiles"], single_rows=True,
