@@ -7,10 +7,14 @@ The default run has the layer sizes of the LFM2-1.2B shape with random bfloat16 
 W untimed and K timed decode steps at batch 8 with every request holding a context of 4,096
 tokens at the last step (one step = one token for every request: row tables, model,
 sampling on the GPU, token ids back on the host), a prefill of 2,048 tokens, and decode at
-batch 1 and 64.  It prints ONE JSON line.  Token ids are uniform random with a fixed seed
-and the cache contents that stand for the earlier context are random numbers: no dataset
-is involved ("data": "synthetic").  kappai publishes no numbers for this architecture, so
-"vs_baseline" is null; the roofline fractions are against MI355X's published peaks.
+batch 1 and 64.  It prints ONE JSON line.  The model is a folder that the framework's own
+random-weights mode writes (config.json, model.safetensors) and its own loader reads; token ids
+are uniform random with a fixed seed, and every request's context is computed by real prompt
+steps before its decoding is timed: no dataset is involved ("data": "synthetic").  kappai
+publishes no numbers for this architecture, so "vs_baseline" is null; the roofline fractions are
+against MI355X's published peaks, and beside them against what a kernel that only reads and a
+kernel that only multiplies reach on the same box ("kernels": the engine's own products and
+attention kernels at the shapes of the run, timed one by one outside the timed step).
 """
 from __future__ import annotations
 
@@ -108,26 +112,29 @@ def run_workload(key, dtype, device):
 
 
 def random_model(raw, dtype, device, seed=0, std=0.02):
-    """The model of ``raw`` with N(0, std) weights made on the GPU (norm weights 1)."""
-    import torch
+    """The model of ``raw`` with N(0, std) weights (norm weights 1), through the framework's own
+    random-weights mode and loader: the folder is written once (under the temp folder, named by
+    the configuration and the seed) and loaded like any checkpoint."""
+    import hashlib
+    import tempfile
 
     from kappai_amd.config import config_from_dict
-    from kappai_amd.models import build_model
-    from kappai_amd.weights import parse_dtype
+    from kappai_amd.models import load_model
+    from kappai_amd.weights import write_random_model
 
     cfg = config_from_dict(raw)
-    tdt = parse_dtype(dtype)
-    model = build_model(cfg, tdt)
-    gen = torch.Generator(device=device).manual_seed(seed)
-    tensors = {}
-    for spec in model.tensor_specs():
-        if spec.init == "ones":
-            t = torch.ones(spec.shape, dtype=torch.float32, device=device)
-        else:
-            t = torch.randn(spec.shape, generator=gen, dtype=torch.float32, device=device) * std
-        tensors[spec.name] = t.to(tdt)
-    model.bind(tensors)
-    return model
+    tag = hashlib.sha256(json.dumps([cfg.to_dict(), seed, std], sort_keys=True).encode())
+    folder = os.path.join(tempfile.gettempdir(),
+                          f"kappai_amd_bench_{os.getuid()}_{tag.hexdigest()[:16]}")
+    done = os.path.join(folder, ".complete")
+    if not os.path.exists(done):
+        t0 = time.perf_counter()
+        os.makedirs(folder, mode=0o700, exist_ok=True)
+        write_random_model(folder, cfg, seed=seed, std=std)
+        open(done, "w").close()
+        print(f"bench.py: wrote {folder} in {time.perf_counter() - t0:.1f} s", file=sys.stderr,
+              flush=True)
+    return load_model(folder, dtype, device)
 
 
 def sync():
@@ -136,8 +143,9 @@ def sync():
 
 
 class DecodeBench:
-    """``batch`` requests whose caches hold ``start`` tokens of random keys and values, then
-    decoded greedily one token a step."""
+    """``batch`` requests whose contexts of ``start`` random tokens are computed by prompt steps
+    (portions of at most 2,048 tokens, one request a step), then decoded greedily one token a
+    step."""
 
     def __init__(self, model, batch, start, total, page_size, device, seed=1, graphs=True):
         import torch
@@ -148,18 +156,15 @@ class DecodeBench:
         pages = batch * ((total + page_size - 1) // page_size)
         self.cache = CacheManager(model.cache_specs(), page_size, pages, batch)
         self.cache.allocate_storage(model.dtype, device)
-        gen = torch.Generator(device=device).manual_seed(seed)
-        for g in self.cache.paged_groups:
-            for pools in g.pools.values():
-                for t in pools.values():
-                    t.copy_(torch.randn(t.shape, generator=gen, device=device,
-                                        dtype=torch.float32) * 0.5)
         self.runner = StepRunner(model, self.cache, device, decode_graphs=graphs)
         self.requests = [self.cache.open(i) for i in range(batch)]
+        gen = torch.Generator().manual_seed(seed)
         for rc in self.requests:
-            self.cache.extend(rc, start)
-            self.cache.commit(rc, start)
-        self.tokens = [int(t) for t in torch.randint(0, model.vocab_size, (batch,), generator=torch.Generator().manual_seed(seed))]
+            prompt = torch.randint(0, model.vocab_size, (start,), generator=gen).tolist()
+            for at in range(0, start, 2048):
+                self.runner.step([StepEntry(rc, prompt[at:at + 2048], [])])
+        sync()
+        self.tokens = [int(t) for t in torch.randint(0, model.vocab_size, (batch,), generator=gen)]
         self.temp = torch.zeros(batch, dtype=torch.float32, device=device)
         self.uni = torch.zeros(batch, dtype=torch.float32, device=device)
         self.model = model
@@ -221,6 +226,142 @@ def measured_read_bandwidth(device, mb=256, buffers=5, reps=20):
     return total / (time.perf_counter() - t0) / 1e9
 
 
+def measured_mfma_tflops(device, iters=20000):
+    """TFLOP/s of a kernel that only issues bfloat16 matrix instructions from registers."""
+    from kappai_amd.kernels import ops
+    ops.mfma_probe(200, device)
+    sync()
+    t0 = time.perf_counter()
+    flops = ops.mfma_probe(iters, device)
+    sync()
+    return flops / (time.perf_counter() - t0) / 1e12
+
+
+def graph_time(fn, reps):
+    """Seconds per call of ``fn(i)``, from a captured graph of ``reps`` calls replayed twice
+    (kernels one after the other as in a step, no host in between)."""
+    import torch
+    fn(0)
+    sync()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        for i in range(reps):
+            fn(i)
+    g.replay()
+    sync()
+    t0 = time.perf_counter()
+    g.replay()
+    g.replay()
+    sync()
+    return (time.perf_counter() - t0) / (2 * reps)
+
+
+def kernel_rates(model, cfg, batch, context, prefill_tokens, page_size, device, read_gbs,
+                 mfma_tflops, dtype):
+    """The engine's own kernels by class, one by one at the shapes of this run, each over the
+    layers of the model in turn (cold weights, as in a step): the products of a decode step (K3),
+    decode attention over the cache (K10) and the output head (K11) in GB/s of what they have to
+    read, the products of a prompt step (K4) and its attention (K9) in TFLOP/s.  Every figure
+    also as a fraction of the published peak and of what the read-only / multiply-only kernels
+    reach on this box."""
+    import math
+
+    import torch
+
+    from kappai_amd.kernels import ops
+    if dtype != "bfloat16":
+        return {}
+    BF = torch.bfloat16
+    D, F = cfg.hidden_size, cfg.ff_dim
+    H, G, d = cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim
+    ffs = [blk.feed_forward for blk in model.layers]
+    convs = [blk.mixer for blk in model.layers if hasattr(blk.mixer, "in_proj")]
+    out = {}
+
+    def rate_gbs(name, seconds, nbytes):
+        gbs = nbytes / seconds / 1e9
+        out[name] = {"us": round(seconds * 1e6, 2), "gbs": round(gbs, 1),
+                     "frac": round(gbs / HBM_PEAK_GBS, 4), "frac_measured": round(gbs / read_gbs, 4)}
+
+    def rate_tflops(name, seconds, flops):
+        tf = flops / seconds / 1e12
+        out[name] = {"us": round(seconds * 1e6, 2), "tflops": round(tf, 1),
+                     "frac": round(tf / MFMA_PEAK_TFLOPS["bfloat16"], 4),
+                     "frac_measured": round(tf / mfma_tflops, 4)}
+
+    g = torch.Generator(device=device).manual_seed(5)
+    x = torch.randn(batch, D, generator=g, device=device).to(BF)
+    act = torch.randn(batch, F, generator=g, device=device).to(BF)
+    resid = torch.randn(batch, D, generator=g, device=device)
+    n = len(ffs)
+    # K3: products of a decode step
+    gu = [f.gate_up for f in ffs]
+    if all(f.fused for f in ffs):
+        t = graph_time(lambda i: ops.linear_swiglu(x, gu[i % n].weight,
+                                                   weight_frag=gu[i % n].weight_frag), 2 * n)
+        rate_gbs("k3_decode_gate_up", t, gu[0].weight_bytes())
+    dn = [f.down for f in ffs]
+    t = graph_time(lambda i: dn[i % n].forward(act, add_into=ops.AddInto(resid)), 2 * n)
+    rate_gbs("k3_decode_down", t, dn[0].weight_bytes())
+    if convs:
+        ip = [c.in_proj for c in convs]
+        t = graph_time(lambda i: ops.linear(x, ip[i % len(ip)].weight,
+                                            weight_frag=ip[i % len(ip)].weight_frag), 2 * len(ip))
+        rate_gbs("k3_decode_in_proj", t, ip[0].weight_bytes())
+    # K11: the output head on `batch` rows
+    head = model.head.linear
+    t = graph_time(lambda i: head.forward(x, out_dtype=torch.float32), 4)
+    rate_gbs("k11_head", t, head.weight_bytes())
+    # K10: decode attention of `batch` requests over `context` keys
+    if cfg.attention_layers and d % 16 == 0:
+        per = (context + page_size - 1) // page_size
+        n_pool = 3
+        kp = [torch.randn(batch * per + 1, G, page_size, d, generator=g, device=device).to(BF)
+              for _ in range(n_pool)]
+        vp = [torch.randn(batch * per + 1, G, d, page_size, generator=g, device=device).to(BF)
+              for _ in range(n_pool)]
+        q = torch.randn(batch, (H + 2 * G) * d, generator=g, device=device).to(BF)
+        bt = torch.arange(batch * per, dtype=torch.int32, device=device).view(batch, per)
+        pos = torch.full((batch,), context - 1, dtype=torch.int32, device=device)
+        seg = torch.arange(batch, dtype=torch.int32, device=device)
+        t = graph_time(lambda i: ops.paged_attention(
+            q, H, G, d, kp[i % n_pool], vp[i % n_pool], pos, seg, bt, page_size,
+            1.0 / math.sqrt(d), single_rows=True, max_position=context - 1), 2 * n_pool)
+        rate_gbs("k10_decode_attention", t, batch * context * G * d * 2 * 2)
+        del kp, vp
+    # K4: products of a prompt step of `prefill_tokens` rows
+    T = prefill_tokens
+    xp = torch.randn(T, D, generator=g, device=device).to(BF)
+    actp = torch.randn(T, F, generator=g, device=device).to(BF)
+    if all(f.fused for f in ffs):
+        t = graph_time(lambda i: ops.linear_swiglu(xp, gu[i % n].weight), n)
+        rate_tflops("k4_prefill_gate_up", t, 2.0 * T * D * 2 * F)
+    t = graph_time(lambda i: dn[i % n].forward(actp, partial_sums=True), n)
+    rate_tflops("k4_prefill_down", t, 2.0 * T * F * D)
+    if convs:
+        t = graph_time(lambda i: ops.linear(xp, ip[i % len(ip)].weight), len(ip))
+        rate_tflops("k4_prefill_in_proj", t, 2.0 * T * D * 3 * D)
+    # K9: attention of one prompt of `prefill_tokens` tokens over itself
+    if cfg.attention_layers and d % 16 == 0:
+        per = (T + page_size - 1) // page_size
+        kp = torch.randn(per + 1, G, page_size, d, generator=g, device=device).to(BF)
+        vp = torch.randn(per + 1, G, d, page_size, generator=g, device=device).to(BF)
+        qp = torch.randn(T, (H + 2 * G) * d, generator=g, device=device).to(BF)
+        bt = torch.arange(per, dtype=torch.int32, device=device).view(1, per)
+        pos = torch.arange(T, dtype=torch.int32, device=device)
+        seg = torch.zeros(T, dtype=torch.int32, device=device)
+        R = ops.ATTENTION_TILE_ROWS
+        nt = (T + R - 1) // R
+        tiles = torch.tensor([(0, r, min(R, T - r), j | (nt << 16) if nt <= 0x7fff else 0)
+                              for j, r in enumerate(range(0, T, R))], dtype=torch.int32,
+                             device=device)
+        t = graph_time(lambda i: ops.paged_attention(
+            qp, H, G, d, kp, vp, pos, seg, bt, page_size, 1.0 / math.sqrt(d), q_tiles=tiles,
+            max_position=T - 1), 4)
+        rate_tflops("k9_prefill_attention", t, 4.0 * d * H * (T * (T + 1) // 2))
+    return out
+
+
 def prefill_flops(cfg, n_tokens, n_layers_run):
     """Multiply-adds x 2 of a whole prompt of ``n_tokens``: every projection, attention over
     the causal half, and the head for the last row."""
@@ -250,6 +391,8 @@ def main() -> int:
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--page-size", type=int, default=16)
     ap.add_argument("--skip-points", action="store_true", help="only the headline batch")
+    ap.add_argument("--skip-kernels", action="store_true",
+                    help="leave out the kernel-by-kernel rates")
     ap.add_argument("--no-graphs", action="store_true",
                     help="launch decode steps kernel by kernel (for counter collection)")
     ap.add_argument("--workload", default="decode", choices=["decode"] + sorted(WORKLOADS),
@@ -310,6 +453,8 @@ def main() -> int:
             points[f"decode_b{b}"] = round(b * K / dtb, 1)
 
     read_gbs = measured_read_bandwidth(device)
+    # (the probe multiplies bfloat16; a float32 run has no matrix-core yardstick)
+    mfma_tflops = measured_mfma_tflops(device) if args.dtype == "bfloat16" else None
 
     # prefill of one prompt, whole, logits at its last token
     T = args.prefill_tokens
@@ -329,6 +474,11 @@ def main() -> int:
     pre_s = min(times[1:])
     flops = prefill_flops(cfg, T, n_layers)
     peak = MFMA_PEAK_TFLOPS[args.dtype] * 1e12
+    del runner, cm
+    torch.cuda.empty_cache()
+    kernels = {} if args.skip_kernels else kernel_rates(
+        model, cfg, args.batch, args.context, T, args.page_size, device, read_gbs, mfma_tflops,
+        args.dtype)
 
     out = {
         "metric": f"decode tok/s at batch {args.batch} (LFM2-1.2B shape, context {args.context})",
@@ -347,13 +497,18 @@ def main() -> int:
             "parallelism": "single GPU",
         },
         "prefill": {"value": round(T / pre_s, 1), "tokens": T, "ms": round(pre_s * 1e3, 3),
-                    "frac": round(flops / pre_s / peak, 5)},
+                    "frac": round(flops / pre_s / peak, 5),
+                    # what a kernel that only multiplies gets on this box, and the step against it
+                    "measured_mfma_tflops": mfma_tflops and round(mfma_tflops, 1),
+                    "frac_of_measured_mfma": mfma_tflops and round(
+                        flops / pre_s / (mfma_tflops * 1e12), 5)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 5),
                      # what a kernel that only reads gets on this box, and the step against that
                      "measured_read": round(read_gbs, 1),
                      "frac_of_measured_read": round(achieved / read_gbs, 5)},
         "points": points,
+        "kernels": kernels,
     }
     print(json.dumps(out))
     return 0

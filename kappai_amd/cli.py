@@ -78,7 +78,9 @@ def build_parser() -> argparse.ArgumentParser:
                    help="last-n tokens considered by repeat penalty (default 64)")
     g.add_argument("-s", "--seed", type=int, default=0, help="RNG seed (0 = random)")
     d = ap.add_argument_group("Tools / debug")
-    d.add_argument("--time", action="store_true", help="print per-step timing")
+    d.add_argument("--time", action="store_true",
+                   help="print the time of every step, and after the run the time by stage of "
+                        "the forward pass for steps with prompt portions and for decode steps")
     d.add_argument("--debug-forward", action="store_true",
                    help="print the top logits of every sampled row")
     d.add_argument("--debug", action="store_true", help="print the engine's decisions")
@@ -122,8 +124,14 @@ def main(argv=None) -> int:
         model=model_dir, dtype=args.dtype, ctx_size=args.ctx_size, page_size=args.page_size,
         num_pages=args.num_pages, max_batch=args.max_batch, token_budget=args.token_budget,
         chunk=args.chunk,
-        # per-step output (logits, timing) needs every step waited for
-        decode_run=1 if (args.debug_forward or args.dump_logits or args.time) else 8))
+        # per-step output (logits, timing) needs every step waited for, and the times by stage
+        # need steps that are launched kernel by kernel
+        decode_run=1 if (args.debug_forward or args.dump_logits or args.time) else 8,
+        decode_graphs=not args.time))
+    stage_records = {"prefill": [], "decode": []}
+    if args.time:
+        from .kernels import profile
+        profile.STAGE_TIMES.start()
     params = SamplingParams(
         temperature=args.temperature, top_k=args.top_k, top_p=args.top_p, min_p=args.min_p,
         repeat_penalty=args.repeat_penalty, repeat_last_n=args.repeat_last_n, seed=args.seed,
@@ -135,10 +143,13 @@ def main(argv=None) -> int:
     try:
         while engine.has_unfinished():
             t0 = time.perf_counter()
+            prefilled = engine.metrics.prefill_tokens
             outs = engine.step()
             if args.time:
                 print(f"step {engine.metrics.steps}: {(time.perf_counter() - t0) * 1e3:.3f} ms, "
                       f"{len(outs)} tokens", file=sys.stderr)
+                kind = "prefill" if engine.metrics.prefill_tokens > prefilled else "decode"
+                stage_records[kind] += profile.STAGE_TIMES.take()
             if (args.debug_forward or dump) and engine.last_logits is not None and outs:
                 lg = engine.last_logits.float().cpu()
                 if dump:
@@ -167,6 +178,17 @@ def main(argv=None) -> int:
         line = engine.metrics.line(args.metrics)
         if line:
             print(line, file=sys.stderr)
+        if args.time:
+            # kappai prints its table after prefill and after decoding (src/context.c:1597-1625)
+            m = engine.metrics
+            # (a step with prompt portions beside decoded tokens is booked under prefill whole;
+            # the engine's clock shares such a step's time out by tokens)
+            walls = {"prefill": m.prefill_seconds * 1e6, "decode": m.decode_seconds * 1e6}
+            for kind in ("prefill", "decode"):
+                if stage_records[kind]:
+                    print(profile.STAGE_TIMES.report(kind, walls[kind], stage_records[kind]),
+                          file=sys.stderr)
+            profile.STAGE_TIMES.stop()
     except KeyboardInterrupt:
         print("\ninterrupted", file=sys.stderr)
         status = 130

@@ -290,3 +290,44 @@ extern "C" int kappai_stream_read(const void* p, long bytes, uint32_t* sink, lon
                      (const stream_u32x4_t*)p, n_per_block, sink);
   KAPPAI_RETURN_LAUNCH_STATUS();
 }
+
+// ---------------------------------------------------------------------------------------
+// The other yardstick: what the matrix cores do when nothing feeds them but registers.  Every
+// wave issues `iters` rounds of eight independent v_mfma_f32_32x32x16_bf16 (32 x 32 x 16
+// multiply-adds each); 1024 blocks of four waves keep every SIMD of the chip busy.
+// ---------------------------------------------------------------------------------------
+typedef __attribute__((ext_vector_type(8))) __bf16 probe_bf16x8_t;
+typedef __attribute__((ext_vector_type(16))) float probe_f32x16_t;
+__global__ __launch_bounds__(256) void mfma_probe_kernel(float* __restrict__ out, int iters) {
+  probe_bf16x8_t a, b;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    a[i] = (__bf16)(threadIdx.x * 0.001f + i);
+    b[i] = (__bf16)(1.0f + i * 0.01f);
+  }
+  probe_f32x16_t acc[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc[j][v] = 0.f;
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc[j], 0, 0, 0);
+  }
+  float sum = 0.f;
+#pragma unroll
+  for (int j = 0; j < 8; ++j)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) sum += acc[j][v];
+  out[(size_t)blockIdx.x * 256 + threadIdx.x] = sum;
+}
+
+// Launches the probe; `out` holds 1024 * 256 floats.  *flops receives the multiply-adds x 2.
+extern "C" int kappai_mfma_probe(float* out, int iters, double* flops, hipStream_t stream) {
+  const int blocks = 1024;
+  if (iters < 1 || out == nullptr) return (int)hipErrorInvalidValue;
+  if (flops) *flops = (double)blocks * 4 * (double)iters * 8 * (2.0 * 32 * 32 * 16);
+  hipLaunchKernelGGL(mfma_probe_kernel, dim3(blocks), dim3(256), 0, stream, out, iters);
+  KAPPAI_RETURN_LAUNCH_STATUS();
+}

@@ -36,6 +36,7 @@ class EngineConfig:
     max_batch: int = 64                  # requests live at the same time (state slots)
     token_budget: int = 2048
     chunk: int = 2048
+    decode_graphs: bool = True           # replay decode steps from captured HIP graphs
     decode_run: int = 8                  # decode steps queued back to back when nothing but
                                          # decoding is going on (1: every step is waited for)
     warm_kernels: bool = True            # run one prompt portion of zeros at start-up, so that
@@ -120,7 +121,8 @@ class Engine:
             raise RuntimeError("not enough free GPU memory for a single cache page")
         self.cache = CacheManager(specs, config.page_size, num_pages, config.max_batch)
         self.cache.allocate_storage(model.dtype, self.device)
-        self.runner = StepRunner(model, self.cache, self.device)
+        self.runner = StepRunner(model, self.cache, self.device,
+                                 decode_graphs=config.decode_graphs)
         eos = mc.eos_token_id
         self.scheduler = Scheduler(
             self.cache,

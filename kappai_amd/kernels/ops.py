@@ -238,6 +238,16 @@ def stream_read(buf: torch.Tensor) -> int:
     return n.value
 
 
+def mfma_probe(iters: int = 20000, device="cuda:0") -> float:
+    """Launches a kernel that only issues bfloat16 matrix instructions from registers and returns
+    the floating-point operations it performs: the yardstick for the products of prompt steps."""
+    out = torch.empty(1024 * 256, dtype=F32, device=device)
+    flops = ctypes.c_double(0.0)
+    check(library("elementwise").kappai_mfma_probe(
+        _ptr(out), _c_int(iters), ctypes.byref(flops), _stream()), "mfma_probe")
+    return flops.value
+
+
 def swiglu(gate_up: torch.Tensor) -> torch.Tensor:
     """``silu(gate_up[:, :F]) * gate_up[:, F:]`` for a fused [T, 2F] projection."""
     _gpu("gate_up", gate_up, (F32, BF16))

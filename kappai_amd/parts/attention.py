@@ -16,7 +16,7 @@ from typing import Dict, List, Optional
 import torch
 
 from ..cache.specs import PagedKV
-from ..kernels import ops
+from ..kernels import ops, profile
 from ..weights.spec import INIT_ONES, VECTOR, TensorSpec
 from .base import Mixer, PositionEncoding, register_part
 from .linear import PARTIAL_SUMS_MIN_ROWS, Linear
@@ -44,9 +44,11 @@ class GroupedQueryAttention(Mixer):
         self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(head_dim)
         self.qkv = Linear([prefix + n["q"], prefix + n["k"], prefix + n["v"]], width,
                           [num_heads * head_dim, num_kv_heads * head_dim, num_kv_heads * head_dim],
-                          bias=bias)
-        self.q_only = Linear([prefix + n["q"]], width, [num_heads * head_dim], bias=bias)
-        self.out = Linear([prefix + n["o"]], num_heads * head_dim, [width], bias=bias)
+                          bias=bias, stage="matmul_qkv")
+        self.q_only = Linear([prefix + n["q"]], width, [num_heads * head_dim], bias=bias,
+                             stage="matmul_qkv")
+        self.out = Linear([prefix + n["o"]], num_heads * head_dim, [width], bias=bias,
+                          stage="matmul_attn_out")
         self._qn, self._kn = prefix + n["q_norm"], prefix + n["k_norm"]
         self.q_norm_w: Optional[torch.Tensor] = None
         self.k_norm_w: Optional[torch.Tensor] = None
@@ -83,16 +85,18 @@ class GroupedQueryAttention(Mixer):
         rot = self.position.rotation(x.device, batch.max_position) if self.position else None
         tables = batch.block_tables[cache.group]
         k_pool, v_pool = cache.pool("k"), cache.pool("v")
-        q = ops.qk_norm_rope_store(
-            proj, H, G, d, self.q_norm_w, self.k_norm_w, self.qk_norm_eps or 0.0,
-            rot.cos if rot else None, rot.sin if rot else None, rot.rot_dim if rot else 0,
-            rot.mode if rot else ops.ROT_NONE, k_pool, v_pool, batch.row_pos,
-            batch.row_seg, tables, cache.page_size, store_kv=not shared_cache)
-        ctx = ops.paged_attention(q, H, G, d, k_pool, v_pool, batch.row_pos,
-                                  batch.row_seg, tables, cache.page_size, self.scale,
-                                  window=self.window or 0, q_tiles=batch.q_tiles,
-                                  single_rows=batch.max_segment_rows == 1,
-                                  max_position=batch.max_position)
+        with profile.scope("rope_kvput"):
+            q = ops.qk_norm_rope_store(
+                proj, H, G, d, self.q_norm_w, self.k_norm_w, self.qk_norm_eps or 0.0,
+                rot.cos if rot else None, rot.sin if rot else None, rot.rot_dim if rot else 0,
+                rot.mode if rot else ops.ROT_NONE, k_pool, v_pool, batch.row_pos,
+                batch.row_seg, tables, cache.page_size, store_kv=not shared_cache)
+        with profile.scope("attn"):
+            ctx = ops.paged_attention(q, H, G, d, k_pool, v_pool, batch.row_pos,
+                                      batch.row_seg, tables, cache.page_size, self.scale,
+                                      window=self.window or 0, q_tiles=batch.q_tiles,
+                                      single_rows=batch.max_segment_rows == 1,
+                                      max_position=batch.max_position)
         return self.out.forward(ctx, partial_sums=True, add_into=into)
 
     def weight_bytes(self) -> int:

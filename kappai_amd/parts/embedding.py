@@ -5,7 +5,7 @@ from typing import Dict, List, Optional
 
 import torch
 
-from ..kernels import ops
+from ..kernels import ops, profile
 from ..weights.spec import INIT_NORMAL, TABLE, TensorSpec
 from .base import Part
 from .linear import Linear
@@ -26,7 +26,8 @@ class TokenEmbedding(Part):
         self.table = tensors[self.name + ".weight"]
 
     def forward(self, tokens: torch.Tensor) -> torch.Tensor:
-        return ops.embed_rows(tokens, self.table)
+        with profile.scope("embd"):
+            return ops.embed_rows(tokens, self.table)
 
     def weight_bytes(self) -> int:
         return 0   # a step reads one row per token, not the table
@@ -37,7 +38,7 @@ class OutputHead(Part):
     table itself (kappai: src/model.c:2562-2571)."""
 
     def __init__(self, name: str, vocab: int, width: int, tied_to: Optional[TokenEmbedding]):
-        self.linear = Linear([name], width, [vocab])
+        self.linear = Linear([name], width, [vocab], stage="logits_matmul")
         self.tied_to = tied_to
 
     def tensor_specs(self) -> List[TensorSpec]:

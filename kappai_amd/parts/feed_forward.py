@@ -8,7 +8,7 @@ from typing import Dict, List
 
 import torch
 
-from ..kernels import ops
+from ..kernels import ops, profile
 from ..weights.spec import TensorSpec
 from .base import FeedForward, register_part
 from .linear import Linear
@@ -23,8 +23,9 @@ class SwiGLU(FeedForward):
         n.update(names or {})
         self.width, self.hidden, self.dtype = width, hidden, dtype
         self.fused = False
-        self.gate_up = Linear([prefix + n["gate"], prefix + n["up"]], width, [hidden, hidden])
-        self.down = Linear([prefix + n["down"]], hidden, [width])
+        self.gate_up = Linear([prefix + n["gate"], prefix + n["up"]], width, [hidden, hidden],
+                              stage="matmul_ffn_gate_up")
+        self.down = Linear([prefix + n["down"]], hidden, [width], stage="matmul_ffn_down")
 
     def tensor_specs(self) -> List[TensorSpec]:
         return self.gate_up.tensor_specs() + self.down.tensor_specs()
@@ -40,12 +41,14 @@ class SwiGLU(FeedForward):
 
     def forward(self, x, batch, into=None):
         if self.fused and x.dtype == torch.bfloat16:
-            return self.down.forward(
-                ops.linear_swiglu(x, self.gate_up.weight, weight_frag=self.gate_up.weight_frag,
-                                  out_fragment=True),
-                partial_sums=True, add_into=into)
-        return self.down.forward(ops.swiglu(self.gate_up.forward(x)), partial_sums=True,
-                                 add_into=into)
+            with profile.scope("matmul_ffn_gate_up", self.gate_up.weight_bytes()):
+                act = ops.linear_swiglu(x, self.gate_up.weight,
+                                        weight_frag=self.gate_up.weight_frag, out_fragment=True)
+            return self.down.forward(act, partial_sums=True, add_into=into)
+        gate_up = self.gate_up.forward(x)
+        with profile.scope("ffn_act"):
+            act = ops.swiglu(gate_up)
+        return self.down.forward(act, partial_sums=True, add_into=into)
 
     def weight_bytes(self) -> int:
         return self.gate_up.weight_bytes() + self.down.weight_bytes()

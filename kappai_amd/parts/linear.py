@@ -6,7 +6,7 @@ from typing import Dict, List, Optional, Sequence
 
 import torch
 
-from ..kernels import ops
+from ..kernels import ops, profile
 from ..weights.spec import INIT_NORMAL, INIT_SMALL, MATRIX, VECTOR, TensorSpec
 from .base import Part
 
@@ -29,8 +29,9 @@ class Linear(Part):
     (kappai's optional load-time fusion of q,k,v and gate,up, src/model.c:930-948)."""
 
     def __init__(self, names: Sequence[str], in_features: int, out_features: Sequence[int],
-                 bias: bool = False):
+                 bias: bool = False, stage: str = "matmul"):
         self.names = list(names)
+        self.stage = stage              # the row of the --time table this product is booked under
         self.in_features = in_features
         self.out_features = list(out_features)
         self.has_bias = bias
@@ -73,9 +74,10 @@ class Linear(Part):
         update, which may then arrive as float32 sums over ranges of the input dimension.
         ``add_into`` (``ops.AddInto``): the product may add its result into the residual stream
         itself; what it returns then says so (``ops.Added``, ``ops.ScaledRows``)."""
-        return ops.linear(x, self.weight, self.bias, out_dtype=out_dtype,
-                          partial_sums=partial_sums, weight_frag=self.weight_frag,
-                          add_into=add_into)
+        with profile.scope(self.stage, self.weight_bytes()):
+            return ops.linear(x, self.weight, self.bias, out_dtype=out_dtype,
+                              partial_sums=partial_sums, weight_frag=self.weight_frag,
+                              add_into=add_into)
 
     def weight_bytes(self) -> int:
         n = self.weight.numel() * self.weight.element_size()

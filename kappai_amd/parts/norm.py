@@ -7,7 +7,7 @@ from typing import Dict, List, Optional
 
 import torch
 
-from ..kernels import ops
+from ..kernels import ops, profile
 from ..weights.spec import INIT_ONES, VECTOR, TensorSpec
 from .base import Norm, register_part
 
@@ -56,8 +56,9 @@ class RMSNorm(Norm):
         fragment = (defer and FRAGMENT_ROWS and resid.is_cuda and n >= FRAGMENT_ROWS_MIN
                     and ops.FragmentRows.fits(n, self.width, self.dtype)
                     and (delta is None or delta.dim() == 2 or delta.shape[0] <= 8))
-        return ops.add_rmsnorm(resid, delta, self.weight, self.eps, self.dtype, rows=rows,
-                               write_resid=rows is None, fragment=fragment)
+        with profile.scope("rmsnorm" if rows is None else "logits_norm"):
+            return ops.add_rmsnorm(resid, delta, self.weight, self.eps, self.dtype, rows=rows,
+                                   write_resid=rows is None, fragment=fragment)
 
     def weight_bytes(self) -> int:
         return self.width * 4

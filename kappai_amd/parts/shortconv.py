@@ -13,7 +13,7 @@ from typing import Dict, List, Optional
 import torch
 
 from ..cache.specs import FixedState
-from ..kernels import ops
+from ..kernels import ops, profile
 from ..weights.spec import INIT_NORMAL, INIT_SMALL, VECTOR, TensorSpec
 from .base import Mixer, register_part
 from .linear import PARTIAL_SUMS_MIN_ROWS, Linear
@@ -42,8 +42,10 @@ class GatedShortConv(Mixer):
             raise ValueError(f"a short convolution needs at least 2 taps, got {kernel_size}")
         self.prefix, self.width, self.L, self.dtype, self.has_bias = (
             prefix, width, kernel_size, dtype, bias)
-        self.in_proj = Linear([prefix + n["in"]], width, [3 * width], bias=bias)
-        self.out_proj = Linear([prefix + n["out"]], width, [width], bias=bias)
+        self.in_proj = Linear([prefix + n["in"]], width, [3 * width], bias=bias,
+                              stage="matmul_in_proj")
+        self.out_proj = Linear([prefix + n["out"]], width, [width], bias=bias,
+                               stage="matmul_out_proj")
         self._conv = prefix + n["conv"]
         self.taps: Optional[torch.Tensor] = None
         self.conv_bias: Optional[torch.Tensor] = None
@@ -79,17 +81,20 @@ class GatedShortConv(Mixer):
                 and x.dtype == torch.bfloat16
                 and w.dtype == torch.bfloat16 and self.width % 16 == 0 and wide_enough):
             # decode: projection, convolution and state shift in one kernel
-            y = ops.linear_shortconv_step(x, w, self.in_proj.bias, self.taps, self.conv_bias,
-                                          cache.state, batch.seg_pos0, batch.seg_slot,
-                                          weight_frag=self.in_proj.weight_frag, out_fragment=True)
+            with profile.scope("matmul_in_proj", self.in_proj.weight_bytes()):
+                y = ops.linear_shortconv_step(x, w, self.in_proj.bias, self.taps, self.conv_bias,
+                                              cache.state, batch.seg_pos0, batch.seg_slot,
+                                              weight_frag=self.in_proj.weight_frag,
+                                              out_fragment=True)
             return self.out_proj.forward(y, partial_sums=True, add_into=into)
         # decode with more than 16 rows: the projection may come as sums over ranges of its input
         # dimension (more blocks stream the matrix), which the step kernel adds up; with fewer
         # rows the unsplit product and the plain step are as fast or faster
         proj = self.in_proj.forward(
             x, partial_sums=batch.max_segment_rows == 1 and x.shape[0] > PARTIAL_SUMS_MIN_ROWS)
-        y = ops.shortconv(proj, self.taps, self.conv_bias, cache.state, batch.row_seg,
-                          batch.seg_start, batch.seg_pos0, batch.seg_slot)
+        with profile.scope("short_conv"):
+            y = ops.shortconv(proj, self.taps, self.conv_bias, cache.state, batch.row_seg,
+                              batch.seg_start, batch.seg_pos0, batch.seg_slot)
         return self.out_proj.forward(y, partial_sums=True, add_into=into)
 
     def weight_bytes(self) -> int:

@@ -14,7 +14,7 @@ from typing import List, Optional, Sequence
 import numpy as np
 import torch
 
-from ..kernels import ops
+from ..kernels import ops, profile
 from .params import SamplingParams
 from .rng import RandomStream
 
@@ -128,6 +128,10 @@ class Sampler:
                out: Optional[torch.Tensor] = None):
         """Queue the kernels that choose a token for every row; returns (int32 tokens on the GPU,
         rows that the host still has to draw).  Nothing here waits for the GPU."""
+        with profile.scope("sample"):
+            return self._launch(logits, samplers, out)
+
+    def _launch(self, logits, samplers, out):
         n, vocab = logits.shape
         dev = logits.device
         temps, unis, host_rows, filt = [], [], [], []

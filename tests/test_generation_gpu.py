@@ -281,6 +281,28 @@ def test_command_line(model_dirs, tmp_path):
     assert len(out.stdout.split()) == 4
 
 
+def test_command_line_times_by_stage(model_dirs):
+    """--time: the tokens are those of a run without it, and after the run there is a table of
+    the time by stage for the steps with prompt portions and one for the decode steps."""
+    prompt = prompts_for("B", [21], seed=9)[0]
+    base = [sys.executable, "-m", "kappai_amd", "-m", str(model_dirs["B"]), "--dtype", "bfloat16",
+            "-p", ",".join(map(str, prompt)), "-n", "5", "-t", "0", "--num-pages", "16"]
+    plain_run = subprocess.run(base, cwd=str(ROOT), capture_output=True, text=True, timeout=300)
+    timed = subprocess.run(base + ["--time"], cwd=str(ROOT), capture_output=True, text=True,
+                           timeout=300)
+    assert timed.returncode == 0, timed.stderr
+    assert timed.stdout.split() == plain_run.stdout.split()
+    err = timed.stderr
+    assert "[profile] prefill  accounted=" in err and "[profile] decode  accounted=" in err
+    decode = err[err.index("[profile] decode"):]
+    for stage in ("embd", "matmul_qkv", "matmul_attn_out", "matmul_in_proj", "matmul_ffn_gate_up",
+                  "matmul_ffn_down", "rope_kvput", "attn", "logits_matmul", "sample"):
+        assert f"  {stage} " in decode, (stage, decode)
+    # 4 decode steps x 3 attention layers
+    row = next(line for line in decode.splitlines() if line.startswith("  attn "))
+    assert int(row.split()[2]) == 12, row
+
+
 def test_smoke_entry():
     sys.path.insert(0, str(ROOT))
     import __graft_entry__
