@@ -37,6 +37,8 @@ class EngineConfig:
     token_budget: int = 2048
     chunk: int = 2048
     decode_graphs: bool = True           # replay decode steps from captured HIP graphs
+    c_forward: bool = True               # steps through the C side (kappai_forward) when the model
+                                         # is made of parts it knows
     decode_run: int = 8                  # decode steps queued back to back when nothing but
                                          # decoding is going on (1: every step is waited for)
     warm_kernels: bool = True            # run one prompt portion of zeros at start-up, so that
@@ -122,7 +124,8 @@ class Engine:
         self.cache = CacheManager(specs, config.page_size, num_pages, config.max_batch)
         self.cache.allocate_storage(model.dtype, self.device)
         self.runner = StepRunner(model, self.cache, self.device,
-                                 decode_graphs=config.decode_graphs)
+                                 decode_graphs=config.decode_graphs,
+                                 c_forward=config.c_forward)
         eos = mc.eos_token_id
         self.scheduler = Scheduler(
             self.cache,

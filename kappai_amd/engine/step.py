@@ -16,8 +16,10 @@ import numpy as np
 import torch
 
 from ..cache.manager import CacheManager, OutOfPages, RequestCache
+from ..kernels import profile
 from ..models.base import Model
 from .batch import RowBatch, StepEntry, layout_rows
+from .cforward import CForward, Workspace
 
 
 CONTEXT_BUCKET_MIN = 1024     # decode graphs are captured for contexts up to a power of two
@@ -100,11 +102,13 @@ class _DecodeGraph:
         self._ring_done: List[Optional[torch.cuda.Event]] = [None] * DECODE_RING
         self._ring_at = 0
         self._upload(runner)
-        runner.model.forward(self.batch, cache)
+        # (a workspace of the graph's own: its kernels keep addresses inside it)
+        self.workspace = Workspace()
+        runner.forward(self.batch, self.workspace)
         torch.cuda.synchronize(dev)
         self.graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(self.graph):
-            self.logits = runner.model.forward(self.batch, cache)
+            self.logits = runner.forward(self.batch, self.workspace)
 
     def _upload(self, runner: "StepRunner") -> None:
         """The mirror to the device through the next pinned buffer of the graph's ring, so that
@@ -162,9 +166,14 @@ class _DecodeGraph:
 
 class StepRunner:
     def __init__(self, model: Model, cache: CacheManager, device="cuda:0",
-                 decode_graphs: bool = True):
+                 decode_graphs: bool = True, c_forward: bool = True):
+        """``c_forward``: run steps through the C side (``kappai_forward``) when the model is made
+        of parts it knows; False runs every step from the parts' own ``forward`` methods."""
         self.model, self.cache = model, cache
         self.device = torch.device(device)
+        self.c_forward = c_forward and self.device.type == "cuda"
+        self._cplan: Optional[CForward] = None
+        self._cplan_tried = False
         self._staging: Optional[torch.Tensor] = None     # pinned host buffer for the tables
         self._staged = None                               # event: last copy out of it is done
         self.steps_run = 0
@@ -174,6 +183,19 @@ class StepRunner:
         self._graphs = {}
         self._graph_seen = {}
         self.graph_replays = 0
+
+    # -- the forward pass of a step ----------------------------------------------------------
+    def forward(self, batch: RowBatch, workspace: Optional[Workspace] = None) -> torch.Tensor:
+        """The model over the rows of ``batch``: one call into C when there is a plan for the
+        model (made at the first step, when the cache's storage exists) and nobody is timing the
+        stages, else part by part from the host."""
+        if self.c_forward and not self._cplan_tried:
+            self._cplan_tried = True
+            if CForward.plannable(self.model):
+                self._cplan = CForward(self.model, self.cache, self.device)
+        if self._cplan is not None and not profile.STAGE_TIMES.enabled:
+            return self._cplan.forward(batch, workspace)
+        return self.model.forward(batch, self.cache)
 
     # -- tables to the device ----------------------------------------------------------------
     def _upload(self, arrays) -> dict:
@@ -333,7 +355,7 @@ class StepRunner:
                 logits = self._decode_step(entries)
             if logits is None:
                 batch = self.make_batch(entries)
-                logits = self.model.forward(batch, self.cache)
+                logits = self.forward(batch)
         except Exception:
             for e in entries:
                 self.cache.trim_uncommitted(e.cache)

@@ -26,7 +26,7 @@ GPU_ARCH = "gfx950"
 HIPCC_FLAGS = ["-O3", "-std=c++17", f"--offload-arch={GPU_ARCH}", "-shared", "-fPIC",
                "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
                "-Wno-unused-command-line-argument", "-Wno-pass-failed"]
-LIBRARIES = ["elementwise", "gemm", "shortconv", "attention", "sampling"]
+LIBRARIES = ["elementwise", "gemm", "shortconv", "attention", "sampling", "engine"]
 # libraries compiled once per value of a constant: name -> (constant, values built ahead)
 VARIANT_LIBRARIES = {"attention_mfma": ("HEAD_DIM", [16, 32, 48, 64, 80, 128, 256])}
 

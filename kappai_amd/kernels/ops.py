@@ -272,35 +272,6 @@ def cast(x: torch.Tensor, dtype) -> torch.Tensor:
 
 
 # ---------------------------------------------------------------------------------------
-def _split_k_large(M: int, N: int, K: int) -> int:
-    """K ranges for a product with more than 64 rows whose consumer adds partial sums: the
-    number that a model of the block kernel's time likes best (within 12 % of the best of a
-    sweep over 40 shapes, 1 % on average).  A 128 x 128 block that has a CU to itself takes
-    about 0.62 us per 64 of K whatever else goes on, so a product with few blocks is bound by
-    the length of K and gains almost linearly from being cut, until the chip is full (two
-    blocks a CU, each then a quarter slower; with 140 blocks of 256 x 256 or more the kernel
-    takes its 256 x 256 form, about 1 us per 64 of K) or the float partial sums ([S, M, N],
-    written here and read again by the consumer) cost more than the cut saves.  Every range is
-    a multiple of 128 long, as the kernel asks."""
-    best, best_t = 1, None
-    for split in range(1, 9):
-        if K % (128 * split) or (split > 1 and K // split < 256):
-            continue
-        steps = K / split / 64
-        blocks256 = ((M + 255) // 256) * ((N + 255) // 256) * split
-        rem = blocks256 % 256       # the kernel's own rule for its 256 x 256 form (gemm.hip)
-        if (140 <= blocks256 <= 256) or (blocks256 > 256 and (
-                rem == 0 or (256 - rem) * 10 < 3 * blocks256)):
-            t = -(-blocks256 // 256) * (steps * 1.0 + 4.5)
-        else:
-            blocks = ((M + 127) // 128) * ((N + 127) // 128) * split
-            t = -(-blocks // 512) * (steps * 0.62 * (1.25 if blocks > 256 else 1.0) + 2.5)
-        t += (split * M * N * 8 if split > 1 else M * N * 4) / 5e6     # written and read again
-        if best_t is None or t < best_t - 1e-9:
-            best, best_t = split, t
-    return best
-
-
 def fragment_order(weight: torch.Tensor) -> Optional[torch.Tensor]:
     """A copy of a bfloat16 matrix [N, K] in the order in which the product kernel for 1 to 16
     rows loads it: pieces of 16 rows x 32 of K, each laid out lane by lane ([N / 16][K / 32]
@@ -331,19 +302,11 @@ def _frag(weight: torch.Tensor, weight_frag: Optional[torch.Tensor]) -> _vp:
 def split_k_for(M: int, N: int, K: int) -> int:
     """How many K ranges a product is cut into when its consumer takes partial sums (1: not
     split).  Decode (M <= 64): so that about 512 blocks stream the matrix (17 rows and more: what
-    suits the kernel that takes them).  Larger M: see ``_split_k_large``."""
-    if M > 64:
-        return _split_k_large(M, N, K)
-    if M > 16:
-        # the kernel that shares the rows through LDS: blocks of 64 columns, K ranges that are
-        # multiples of 512 and at least 1024 long, 128 blocks or more
-        split = min(8, K // 1024)
-        while split > 1 and K % (512 * split):
-            split -= 1
-        if split >= 1 and K % (512 * split) == 0 and ((N + 63) // 64) * split >= 128:
-            return split
-    col_groups = (N + 15) // 16
-    return max(1, min(8, 512 // col_groups, K // 512))
+    suits the kernel that takes them).  Larger M: the number that a model of the block kernel's
+    time likes best (a product with few blocks is bound by the length of K and gains from being
+    cut until the chip is full or the float partial sums cost more than the cut saves).  The rule
+    itself lives beside the C side's step (``csrc/engine.hip``), which asks it as well."""
+    return int(library("engine").kappai_split_k_for(_c_int(M), _c_int(N), _c_int(K)))
 
 
 def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,

@@ -190,6 +190,36 @@ def test_decode_graphs_replay_what_eager_steps_compute(tmp_path, model_dirs, dty
             assert np.array_equal(a, b)
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D", "E", "F", "G", "H"])
+def test_steps_from_c_equal_steps_from_the_host(tmp_path, model_dirs, name, dtype):
+    """A step is launched by one call into C (kappai_forward) when the model is made of the
+    framework's own parts, and part by part from the host otherwise.  Both run the same kernels
+    on the same choices: the mixed schedule gives bit for bit the same logits either way, with
+    and without decode graphs."""
+    from kappai_amd.engine.replay import TraceReplayer, make_replay_cache
+    from kappai_amd.engine.step import StepRunner
+    cfg = TINY[name][0]
+    requests = make_requests(cfg["vocab_size"], MIXED_LENGTHS[name][:7], seed=22)
+    steps, index, peak = schedules.mixed(requests)
+    results = {}
+    for c_forward in (True, False):
+        for graphs in (False, True):
+            model = gpu_model(model_dirs[name], dtype)
+            cache = make_replay_cache(model, peak)
+            cache.allocate_storage(model.dtype, "cuda:0", poison=True)
+            runner = StepRunner(model, cache, "cuda:0", decode_graphs=graphs, c_forward=c_forward)
+            rep = TraceReplayer(runner, tmp_path / f"c{c_forward}g{graphs}")
+            results[(c_forward, graphs)] = [rep.run_step(obj) for obj in steps]
+            assert (runner._cplan is not None) == c_forward
+    base = results[(False, False)]
+    for key, res in results.items():
+        for a, b in zip(base, res):
+            assert (a is None) == (b is None)
+            if a is not None:
+                assert np.array_equal(a, b), key
+
+
 # A wider configuration with a long prompt, so that the kernels for large steps run inside the
 # engine: the 128 x 128 / 256 x 256 block products (K a multiple of 128, more than 64 rows) and
 # the prefill attention that shares key tiles between four heads of a kv head (head size 64,
