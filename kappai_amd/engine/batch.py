@@ -7,6 +7,7 @@ request; a decoded token is a segment of length one.
 """
 from __future__ import annotations
 
+import itertools
 from dataclasses import dataclass, field
 from typing import Dict, List, Optional, Sequence
 
@@ -64,13 +65,14 @@ def layout_rows(entries: Sequence[StepEntry], cache: CacheManager, vocab_size: i
                 tile_rows: Optional[int] = None):
     """Host side of ``RowBatch``: checks the entries and lays the tables out as int32
     arrays.  Returns (dict of arrays, sizes).  ``tile_rows``: cut the segments into tiles of at
-    most that many rows (``q_tiles``); None: no such table."""
+    most that many rows (``q_tiles``); None: no such table.  The tables are made for all entries
+    at once (a step of many single decoded tokens costs a few numpy calls, not a few per entry)."""
     if not entries:
         raise ValueError("a step needs at least one entry")
+    S = len(entries)
     seen = set()
-    tokens, row_pos, row_seg, seg_start, seg_pos0, seg_slot, logit_rows = [], [], [], [0], [], [], []
-    q_tiles = []
-    max_position = 0
+    counts, pos0, slots, logit_rows = [], [], [], []
+    base = 0
     for si, e in enumerate(entries):
         n = len(e.tokens)
         if n < 1:
@@ -78,57 +80,67 @@ def layout_rows(entries: Sequence[StepEntry], cache: CacheManager, vocab_size: i
         if id(e.cache) in seen:
             raise ValueError(f"request {e.cache.request_id!r} appears twice in one step")
         seen.add(id(e.cache))
-        toks = np.asarray(e.tokens, dtype=np.int64)
-        if toks.ndim != 1 or int(toks.min()) < 0 or int(toks.max()) >= vocab_size:
-            bad = next(int(t) for t in toks.reshape(-1) if not 0 <= int(t) < vocab_size)
-            raise ValueError(f"entry {si} ({e.cache.request_id!r}): token id {bad} is outside "
-                             f"the vocabulary of {vocab_size}")
         for w in e.want:
             if not 0 <= int(w) < n:
                 raise ValueError(f"entry {si} ({e.cache.request_id!r}): wanted place {w} is "
                                  f"outside its {n} tokens")
-        base = seg_start[-1]
-        p0 = e.cache.length
-        tokens.append(toks.astype(np.int32))
-        row_pos.append(np.arange(p0, p0 + n, dtype=np.int32))
-        row_seg.append(np.full(n, si, dtype=np.int32))
-        max_position = max(max_position, p0 + n - 1)
-        seg_start.append(base + n)
-        if tile_rows:
-            n_seg_tiles = (n + tile_rows - 1) // tile_rows
-            for j, r in enumerate(range(0, n, tile_rows)):
-                # the fourth number tells a kernel where the tile stands in its segment
-                # (index | tiles of the segment << 16), so that it can pair tiles of one segment
-                q_tiles.append((si, base + r, min(tile_rows, n - r), tile_place(j, n_seg_tiles)))
-        seg_pos0.append(p0)
-        seg_slot.append(e.cache.slot)
-        logit_rows.extend(base + int(w) for w in e.want)
-    S = len(entries)
-    tables = []
-    for gi in range(len(cache.paged_groups)):
+            logit_rows.append(base + int(w))
+        counts.append(n)
+        pos0.append(e.cache.length)
+        slots.append(e.cache.slot)
+        base += n
+    T = base
+    try:
+        tokens = np.fromiter(itertools.chain.from_iterable(e.tokens for e in entries),
+                             dtype=np.int64, count=T)
+    except (TypeError, ValueError):
+        tokens = np.concatenate([np.asarray(e.tokens, dtype=np.int64).reshape(-1)
+                                 for e in entries])
+    if int(tokens.min()) < 0 or int(tokens.max()) >= vocab_size:
+        at = int(np.flatnonzero((tokens < 0) | (tokens >= vocab_size))[0])
+        si = int(np.searchsorted(np.cumsum(counts), at, side="right"))
+        raise ValueError(f"entry {si} ({entries[si].cache.request_id!r}): token id "
+                         f"{int(tokens[at])} is outside the vocabulary of {vocab_size}")
+    n_arr = np.asarray(counts, dtype=np.int64)
+    p0_arr = np.asarray(pos0, dtype=np.int64)
+    seg_start = np.zeros(S + 1, dtype=np.int64)
+    np.cumsum(n_arr, out=seg_start[1:])
+    row_seg = np.repeat(np.arange(S, dtype=np.int64), n_arr)
+    row_pos = np.arange(T, dtype=np.int64) - np.repeat(seg_start[:-1] - p0_arr, n_arr)
+    max_position = int((p0_arr + n_arr).max()) - 1
+    arrays = {
+        "tokens": tokens.astype(np.int32),
+        "row_pos": row_pos.astype(np.int32),
+        "row_seg": row_seg.astype(np.int32),
+        "seg_start": seg_start.astype(np.int32),
+        "seg_pos0": p0_arr.astype(np.int32),
+        "seg_slot": np.asarray(slots, dtype=np.int32),
+        "logit_rows": np.asarray(logit_rows, dtype=np.int32),
+    }
+    if tile_rows:
+        # tile j of a segment: (segment, first row, rows, place); the fourth number tells a kernel
+        # where the tile stands in its segment (index | tiles of the segment << 16, or 0 when the
+        # segment has more tiles than 15 bits hold), so that it can pair tiles of one segment
+        nt = (n_arr + tile_rows - 1) // tile_rows
+        tile_seg = np.repeat(np.arange(S, dtype=np.int64), nt)
+        first_tile = np.cumsum(nt) - nt
+        idx = np.arange(int(nt.sum()), dtype=np.int64) - np.repeat(first_tile, nt)
+        rows = np.minimum(tile_rows, n_arr[tile_seg] - idx * tile_rows)
+        nts = nt[tile_seg]
+        place = np.where(nts > 0x7fff, 0, idx | (nts << 16))
+        arrays["q_tiles"] = np.stack(
+            [tile_seg, seg_start[tile_seg] + idx * tile_rows, rows, place], axis=1).astype(np.int32)
+    n_groups = len(cache.paged_groups)
+    for gi in range(n_groups):
         width = max(1, max(len(e.cache.blocks[gi]) for e in entries))
         bt = np.full((S, width), -1, dtype=np.int32)
         for si, e in enumerate(entries):
             b = e.cache.blocks[gi]
             bt[si, :len(b)] = b
-        tables.append(bt)
-    arrays = {
-        "tokens": np.concatenate(tokens),
-        "row_pos": np.concatenate(row_pos),
-        "row_seg": np.concatenate(row_seg),
-        "seg_start": np.asarray(seg_start, dtype=np.int32),
-        "seg_pos0": np.asarray(seg_pos0, dtype=np.int32),
-        "seg_slot": np.asarray(seg_slot, dtype=np.int32),
-        "logit_rows": np.asarray(logit_rows, dtype=np.int32),
-    }
-    if tile_rows:
-        arrays["q_tiles"] = np.asarray(q_tiles, dtype=np.int32).reshape(-1, 4)
-    for gi, bt in enumerate(tables):
         arrays[f"block_table_{gi}"] = bt
     sizes = {
-        "n_rows": seg_start[-1], "n_segments": S, "n_logit_rows": len(logit_rows),
-        "max_position": max_position,
-        "max_segment_rows": max(len(e.tokens) for e in entries),
-        "n_groups": len(tables),
+        "n_rows": T, "n_segments": S, "n_logit_rows": len(logit_rows),
+        "max_position": max_position, "max_segment_rows": int(n_arr.max()),
+        "n_groups": n_groups,
     }
     return arrays, sizes
