@@ -864,6 +864,39 @@ __global__ __launch_bounds__((NW < 16 ? NW + 1 : NW) * WAVE) void gemm_bf16_skin
       row_ss[lane] = t;
     }
   }
+  // The conv step's epilogue (EPI 2, 3) needs the rows' state, the channel's taps and the biases:
+  // asked for now by the lanes that will use them (two round trips, the slot first), so that they
+  // have arrived when the stream of W has gone through.  Up to CONV_PRE taps are held this way;
+  // a longer filter reads the rest when it gets there.
+  constexpr int CONV_PRE = 4;
+  float st_pre[4][CONV_PRE], tap_pre[CONV_PRE + 1], conv_bias_pre = 0.f;
+  float gate_bias_pre[3] = {0.f, 0.f, 0.f};
+  bool fresh_pre[4] = {true, true, true, true};
+  float* st_ptr[4] = {nullptr, nullptr, nullptr, nullptr};
+  if ((EPI == 2 || EPI == 3) && wave < MT && gn < N && (EPI != 3 || col < 8)) {
+    const int H = cs.L - 1;
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+      const int gm = wave * 16 + 4 * (lane / 16) + v;
+      if (gm < M) {
+        fresh_pre[v] = cs.seg_pos0[gm] == 0;
+        st_ptr[v] = cs.state + ((size_t)cs.seg_slot[gm] * N + gn) * H;
+      }
+    }
+#pragma unroll
+    for (int v = 0; v < 4; ++v)
+#pragma unroll
+      for (int k = 0; k < CONV_PRE; ++k)
+        st_pre[v][k] = (st_ptr[v] != nullptr && !fresh_pre[v] && k < H) ? st_ptr[v][k] : 0.f;
+#pragma unroll
+    for (int k = 0; k <= CONV_PRE; ++k) tap_pre[k] = k <= H ? cs.taps[(size_t)gn * cs.L + k] : 0.f;
+    if (cs.conv_bias) conv_bias_pre = cs.conv_bias[gn];
+    if (bias) {
+      gate_bias_pre[0] = bias[gn];
+      gate_bias_pre[1] = bias[N + gn];
+      gate_bias_pre[2] = bias[2 * N + gn];
+    }
+  }
   const int kblk = ((K + 32 * (int)gridDim.y - 1) / (32 * (int)gridDim.y)) * 32;   // K a block
   const int kb0 = blockIdx.y * kblk, kb1 = min(K, kb0 + kblk);
   const int kper = ((kb1 - kb0 + 32 * NW - 1) / (32 * NW)) * 32;
@@ -961,27 +994,42 @@ __global__ __launch_bounds__((NW < 16 ? NW + 1 : NW) * WAVE) void gemm_bf16_skin
           }
           cg *= rs;
           xg *= rs;
-          float bg = sum;
-          if (bias) {
-            bg += bias[gn];
-            cg += bias[N + gn];
-            xg += bias[2 * N + gn];
-          }
+          const float bg = sum + gate_bias_pre[0];
+          cg += gate_bias_pre[1];
+          xg += gate_bias_pre[2];
           // the three gates are rounded as the unfused path stores them
           const float bx = to_f32(f32_to_bf16(bg)) * to_f32(f32_to_bf16(xg));
           const int H = cs.L - 1;
-          const bool fresh = cs.seg_pos0[gm] == 0;
-          float* st = cs.state + ((size_t)cs.seg_slot[gm] * N + gn) * H;
+          const bool fresh = fresh_pre[v];
+          float* st = st_ptr[v];
           const float* wc = cs.taps + (size_t)gn * cs.L;
-          float s = cs.conv_bias ? cs.conv_bias[gn] : 0.f;
-          float prev = fresh ? 0.f : st[0];
-          for (int k = 0; k < H; ++k) {
-            s += wc[k] * prev;
-            const float next = (k + 1 < H) ? (fresh ? 0.f : st[k + 1]) : bx;
-            st[k] = next;
-            prev = next;
+          float s = conv_bias_pre;
+          if (H <= CONV_PRE) {
+            // everything is in registers already
+            float prev = st_pre[v][0];
+#pragma unroll
+            for (int k = 0; k < CONV_PRE; ++k) {
+              if (k < H) {
+                s += tap_pre[k] * prev;
+                const float next = (k + 1 < H) ? st_pre[v][k + 1 < CONV_PRE ? k + 1 : 0] : bx;
+                st[k] = next;
+                prev = next;
+              }
+            }
+            float last = tap_pre[0];
+#pragma unroll
+            for (int k = 1; k <= CONV_PRE; ++k) last = k == H ? tap_pre[k] : last;
+            s += last * bx;
+          } else {
+            float prev = fresh ? 0.f : st[0];
+            for (int k = 0; k < H; ++k) {
+              s += wc[k] * prev;
+              const float next = (k + 1 < H) ? (fresh ? 0.f : st[k + 1]) : bx;
+              st[k] = next;
+              prev = next;
+            }
+            s += wc[H] * bx;
           }
-          s += wc[H] * bx;
           store_out(C + out_at(gm, gn), to_f32(f32_to_bf16(cg)) * s);
         } else {
           store_out(C + (size_t)gm * ldc + gn, sum + bv);

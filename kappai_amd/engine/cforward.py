@@ -19,10 +19,9 @@ from typing import List, Optional
 import torch
 
 from ..cache.specs import PagedKV
-from ..kernels import ops, profile
+from ..kernels import ops, profile, tuning
 from ..kernels.lib import KernelLaunchError, library
 from ..parts import attention as attention_part
-from ..parts import linear as linear_part
 from ..parts import norm as norm_part
 from ..parts import shortconv as shortconv_part
 from ..parts.block import PreNormBlock
@@ -239,11 +238,11 @@ class CForward:
         m.final_norm = NormDesc(model.final_norm.weight.data_ptr(), model.final_norm.eps)
         m.head = _linear(model.head.linear)
         m.kernels = ctypes.pointer(self.kernels)
-        m.fused_step_min_width = shortconv_part.FUSED_STEP_MIN_WIDTH
-        m.fused_step_narrow_width = shortconv_part.FUSED_STEP_NARROW_WIDTH
-        m.fused_step_narrow_rows = shortconv_part.FUSED_STEP_NARROW_ROWS
-        m.partial_sums_min_rows = linear_part.PARTIAL_SUMS_MIN_ROWS
-        m.fragment_rows_min = norm_part.FRAGMENT_ROWS_MIN if norm_part.FRAGMENT_ROWS else 1 << 30
+        m.fused_step_min_width = tuning.FUSED_STEP_MIN_WIDTH
+        m.fused_step_narrow_width = tuning.FUSED_STEP_NARROW_WIDTH
+        m.fused_step_narrow_rows = tuning.FUSED_STEP_NARROW_ROWS
+        m.partial_sums_min_rows = tuning.PARTIAL_SUMS_MIN_ROWS
+        m.fragment_rows_min = tuning.FRAGMENT_ROWS_MIN if tuning.FRAGMENT_ROWS else 1 << 30
         m.fragment_rows_from = ops.FRAGMENT_ROWS_FROM
         m.fused_max_rows = ops.FUSED_MAX_ROWS
         m.decode_waves, m.decode_max_splits = ops.DECODE_WAVES, ops.DECODE_MAX_SPLITS

@@ -1,0 +1,35 @@
+"""The numbers by which the parts and the kernels' faces choose between forms of a kernel.
+
+They were measured on LFM2-sized layers (widths of 1024 to 4096) on one MI355X and decide speed
+only: every form gives the same result for the shapes it takes.  They live here, not in the
+parts, so that a part holds no size of any particular model; the C side of a step gets the same
+numbers in its model description.
+"""
+
+# A projection whose consumer can add partial sums asks for them only above this many rows:
+# 6144 x 2048 plus the conv step takes 13.0 us unsplit and 13.3 us in two K ranges at 8 rows, 18 us
+# and 12 us at 64 rows.
+PARTIAL_SUMS_MIN_ROWS = 16
+
+# Every bfloat16 matrix is kept a second time in the order in which the product kernel for 1 to
+# 16 rows loads it (``ops.fragment_order``): decode steps stream that copy 10-20 % faster (a step
+# at batch 8: about a tenth), steps with more rows read the matrix as the checkpoint has it.  The
+# price is the matrices' memory once more; False keeps one copy.
+FRAGMENT_COPIES = True
+
+# The norm kernel hands its rows on in fragment order from this many rows on (up to 16): a step of
+# the 1.2B shape takes 1.06 against 1.08 ms at 16 rows, 0.994 against 1.000 at 12, even at 8; with
+# fewer rows the ordinary order is as fast or faster.
+FRAGMENT_ROWS = True
+FRAGMENT_ROWS_MIN = 8
+
+# The conv layer's fused decode kernel (in_proj, gates, FIR, state shift in one) gives one block 16
+# channels (8 below a width of 4096, where 16 would leave CUs without a block).  From
+# FUSED_STEP_MIN_WIDTH on it beats the separate product (which may split K) plus the small step
+# kernel for any number of rows up to 64; between FUSED_STEP_NARROW_WIDTH and it only up to
+# FUSED_STEP_NARROW_ROWS rows (at a width of 2048, W in fragment order: 8.3 against 9.9 us for one
+# row; 11.0 against 11.1 at 8 rows, 11.5 against 12.8 at 16; at a width of 1024 the separate
+# kernels win).
+FUSED_STEP_MIN_WIDTH = 4096
+FUSED_STEP_NARROW_WIDTH = 2048
+FUSED_STEP_NARROW_ROWS = 16

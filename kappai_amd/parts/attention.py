@@ -16,10 +16,10 @@ from typing import Dict, List, Optional
 import torch
 
 from ..cache.specs import PagedKV
-from ..kernels import ops, profile
+from ..kernels import ops, profile, tuning
 from ..weights.spec import INIT_ONES, VECTOR, TensorSpec
 from .base import Mixer, PositionEncoding, register_part
-from .linear import PARTIAL_SUMS_MIN_ROWS, Linear
+from .linear import Linear
 
 
 class GroupedQueryAttention(Mixer):
@@ -81,7 +81,7 @@ class GroupedQueryAttention(Mixer):
         # decode with more than 16 rows: the projection may come as sums over ranges of its input
         # dimension (more blocks stream the matrix), which the next kernel adds up
         proj = (self.q_only if shared_cache else self.qkv).forward(
-            x, partial_sums=batch.max_segment_rows == 1 and x.shape[0] > PARTIAL_SUMS_MIN_ROWS)
+            x, partial_sums=batch.max_segment_rows == 1 and x.shape[0] > tuning.PARTIAL_SUMS_MIN_ROWS)
         rot = self.position.rotation(x.device, batch.max_position) if self.position else None
         tables = batch.block_tables[cache.group]
         k_pool, v_pool = cache.pool("k"), cache.pool("v")

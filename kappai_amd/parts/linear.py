@@ -6,21 +6,12 @@ from typing import Dict, List, Optional, Sequence
 
 import torch
 
-from ..kernels import ops, profile
+from ..kernels import ops, profile, tuning
 from ..weights.spec import INIT_NORMAL, INIT_SMALL, MATRIX, VECTOR, TensorSpec
 from .base import Part
 
 
-# A projection whose consumer can add partial sums asks for them only above this many rows:
-# measured on the 1.2B shape, 6144 x 2048 plus the conv step takes 13.0 us unsplit and 13.3 us
-# in two K ranges at 8 rows, 18 us and 12 us at 64 rows.
-PARTIAL_SUMS_MIN_ROWS = 16
-
-# Every bfloat16 matrix is kept a second time in the order in which the product kernel for 1 to
-# 16 rows loads it (``ops.fragment_order``): decode steps stream that copy 10-20 % faster (a step
-# at batch 8: about a tenth), steps with more rows read the matrix as the checkpoint has it.  The
-# price is the matrices' memory once more; False keeps one copy.
-FRAGMENT_COPIES = True
+# (how many rows, whether a second copy: kernels/tuning.py)
 
 
 class Linear(Part):
@@ -63,7 +54,7 @@ class Linear(Part):
     def set_weight(self, weight: torch.Tensor) -> None:
         """The matrix of the product, and its copy in fragment order when it is to have one."""
         self.weight = weight
-        self.weight_frag = ops.fragment_order(weight) if FRAGMENT_COPIES else None
+        self.weight_frag = ops.fragment_order(weight) if tuning.FRAGMENT_COPIES else None
 
     def bind_shared(self, weight: torch.Tensor) -> None:
         """Use a tensor that another part owns (a tied output head)."""

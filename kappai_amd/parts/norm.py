@@ -7,16 +7,9 @@ from typing import Dict, List, Optional
 
 import torch
 
-from ..kernels import ops, profile
+from ..kernels import ops, profile, tuning
 from ..weights.spec import INIT_ONES, VECTOR, TensorSpec
 from .base import Norm, register_part
-
-
-# Decode steps of 8 to 16 rows hand their normalised rows on in fragment order (a step of the
-# 1.2B shape: 1.06 against 1.08 ms at 16 rows, 0.994 against 1.000 at 12, even at 8; with
-# fewer rows the ordinary order is as fast or faster).
-FRAGMENT_ROWS = True
-FRAGMENT_ROWS_MIN = 8
 
 
 class RMSNorm(Norm):
@@ -53,7 +46,8 @@ class RMSNorm(Norm):
                 return delta
             delta = None             # the sum is in ``resid`` already
         n = resid.shape[0] if rows is None else rows.shape[0]
-        fragment = (defer and FRAGMENT_ROWS and resid.is_cuda and n >= FRAGMENT_ROWS_MIN
+        fragment = (defer and tuning.FRAGMENT_ROWS and resid.is_cuda
+                    and n >= tuning.FRAGMENT_ROWS_MIN
                     and ops.FragmentRows.fits(n, self.width, self.dtype)
                     and (delta is None or delta.dim() == 2 or delta.shape[0] <= 8))
         with profile.scope("rmsnorm" if rows is None else "logits_norm"):

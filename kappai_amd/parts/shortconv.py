@@ -13,21 +13,10 @@ from typing import Dict, List, Optional
 import torch
 
 from ..cache.specs import FixedState
-from ..kernels import ops, profile
+from ..kernels import ops, profile, tuning
 from ..weights.spec import INIT_NORMAL, INIT_SMALL, VECTOR, TensorSpec
 from .base import Mixer, register_part
-from .linear import PARTIAL_SUMS_MIN_ROWS, Linear
-
-
-# The fused decode kernel gives one block 16 channels (8 below a width of 4096, where 16 would
-# leave CUs without a block).  From this width on it beats the separate product (which may split
-# K) plus the small step kernel for any number of rows up to 64; between FUSED_STEP_NARROW_WIDTH
-# and it only up to 16 rows (at a width of 2048, W in fragment order: 8.3 against 9.9 us for one
-# row; 11.0 against 11.1 at
-# 8 rows, 11.5 against 12.8 at 16; at a width of 1024 the separate kernels win).
-FUSED_STEP_MIN_WIDTH = 4096
-FUSED_STEP_NARROW_WIDTH = 2048
-FUSED_STEP_NARROW_ROWS = 16
+from .linear import Linear
 
 
 class GatedShortConv(Mixer):
@@ -75,8 +64,9 @@ class GatedShortConv(Mixer):
             raise ValueError("a short convolution's state cannot be read by another layer")
         w = self.in_proj.weight
         rows = x.shape[0]
-        wide_enough = self.width >= FUSED_STEP_MIN_WIDTH or (
-            self.width >= FUSED_STEP_NARROW_WIDTH and rows <= FUSED_STEP_NARROW_ROWS)
+        wide_enough = self.width >= tuning.FUSED_STEP_MIN_WIDTH or (
+            self.width >= tuning.FUSED_STEP_NARROW_WIDTH
+            and rows <= tuning.FUSED_STEP_NARROW_ROWS)
         if (batch.max_segment_rows == 1 and rows <= 64
                 and x.dtype == torch.bfloat16
                 and w.dtype == torch.bfloat16 and self.width % 16 == 0 and wide_enough):
@@ -91,7 +81,7 @@ class GatedShortConv(Mixer):
         # dimension (more blocks stream the matrix), which the step kernel adds up; with fewer
         # rows the unsplit product and the plain step are as fast or faster
         proj = self.in_proj.forward(
-            x, partial_sums=batch.max_segment_rows == 1 and x.shape[0] > PARTIAL_SUMS_MIN_ROWS)
+            x, partial_sums=batch.max_segment_rows == 1 and x.shape[0] > tuning.PARTIAL_SUMS_MIN_ROWS)
         with profile.scope("short_conv"):
             y = ops.shortconv(proj, self.taps, self.conv_bias, cache.state, batch.row_seg,
                               batch.seg_start, batch.seg_pos0, batch.seg_slot)

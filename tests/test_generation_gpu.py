@@ -224,7 +224,7 @@ def test_fragment_copies_change_no_token(tmp_path):
     import copy
     from kappai_amd.config import config_from_dict
     from kappai_amd.engine import Engine
-    from kappai_amd.parts import linear, norm
+    from kappai_amd.kernels import tuning
     from kappai_amd.sampling import SamplingParams
     from kappai_amd.weights import write_random_model
     raw = {"architectures": ["Lfm2ForCausalLM"], "model_type": "lfm2", "hidden_size": 256,
@@ -242,19 +242,19 @@ def test_fragment_copies_change_no_token(tmp_path):
     params = [SamplingParams.greedy(n_predict=24), SamplingParams(seed=3, n_predict=24),
               SamplingParams.greedy(n_predict=10), SamplingParams(seed=4, top_k=0, n_predict=24),
               SamplingParams.greedy(n_predict=24)] * 2
-    assert len(prompts) >= norm.FRAGMENT_ROWS_MIN      # decode steps with rows enough for the order
+    assert len(prompts) >= tuning.FRAGMENT_ROWS_MIN      # decode steps with rows enough for the order
     outs = []
-    assert linear.FRAGMENT_COPIES and norm.FRAGMENT_ROWS
+    assert tuning.FRAGMENT_COPIES and tuning.FRAGMENT_ROWS
     try:
         for copies, rows in ((True, True), (False, True), (True, False), (False, False)):
-            linear.FRAGMENT_COPIES, norm.FRAGMENT_ROWS = copies, rows
+            tuning.FRAGMENT_COPIES, tuning.FRAGMENT_ROWS = copies, rows
             eng = Engine(str(folder), dtype="bfloat16", num_pages=128, max_batch=10, chunk=32,
                          token_budget=48)
             frag = [blk.feed_forward.down.weight_frag for blk in eng.model.layers]
             assert all((f is not None) == copies for f in frag)
             outs.append(eng.generate(prompts, params))
     finally:
-        linear.FRAGMENT_COPIES, norm.FRAGMENT_ROWS = True, True
+        tuning.FRAGMENT_COPIES, tuning.FRAGMENT_ROWS = True, True
     assert outs[0] == outs[1] == outs[2] == outs[3]
 
 
