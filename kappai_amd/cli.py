@@ -127,6 +127,7 @@ def main(argv=None) -> int:
         # per-step output (logits, timing) needs every step waited for, and the times by stage
         # need steps that are launched kernel by kernel
         decode_run=1 if (args.debug_forward or args.dump_logits or args.time) else 8,
+        pipeline=not (args.debug_forward or args.dump_logits or args.time),
         decode_graphs=not args.time))
     stage_records = {"prefill": [], "decode": []}
     if args.time:

@@ -30,6 +30,25 @@ extern "C" int kappai_embed_rows(const int* ids, const void* table, int table_is
 }
 
 // ---------------------------------------------------------------------------------------
+// tokens[dst_rows[i]] = chosen[src_idx[i]]: token ids that the last step's sampling kernels
+// left on the GPU go to their rows of this step's token table without a trip through the host.
+// ---------------------------------------------------------------------------------------
+__global__ void place_tokens_kernel(int* __restrict__ tokens, const int* __restrict__ dst_rows,
+                                    const int* __restrict__ chosen,
+                                    const int* __restrict__ src_idx, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) tokens[dst_rows[i]] = chosen[src_idx[i]];
+}
+
+extern "C" int kappai_place_tokens(int* tokens, const int* dst_rows, const int* chosen,
+                                   const int* src_idx, int n, hipStream_t stream) {
+  if (n <= 0) return 0;
+  hipLaunchKernelGGL(place_tokens_kernel, dim3((n + 255) / 256), dim3(256), 0, stream, tokens,
+                     dst_rows, chosen, src_idx, n);
+  KAPPAI_RETURN_LAUNCH_STATUS();
+}
+
+// ---------------------------------------------------------------------------------------
 // RMSNorm with the residual sum folded in:
 //   x = resid[r] (+ delta[r]);  if write_resid: resid[r] = x;
 //   out[i] = x * rsqrt(mean(x^2) + eps) * w           (src/backend/cpu/scalar/quants.c:1507-1512)

@@ -18,7 +18,7 @@ from ..cache.manager import CacheManager
 from ..models import Model, load_model
 from ..sampling import RequestSampler, Sampler, SamplingParams
 from .batch import StepEntry
-from .scheduler import FAILED, RUNNING, Request, Scheduler, SchedulerConfig
+from .scheduler import FAILED, RUNNING, Request, Scheduler, SchedulerConfig, TokensUnread
 from .step import StepRunner
 
 
@@ -41,6 +41,9 @@ class EngineConfig:
                                          # is made of parts it knows
     decode_run: int = 8                  # decode steps queued back to back when nothing but
                                          # decoding is going on (1: every step is waited for)
+    pipeline: bool = True                # a step with prompt portions in it is decided and
+                                         # queued before the tokens of the step before it have
+                                         # been read (they go to their rows on the GPU)
     warm_kernels: bool = True            # run one prompt portion of zeros at start-up, so that
                                          # the first request does not pay for loading the kernels
 
@@ -75,6 +78,17 @@ class Metrics:
                 parts.append(f"TTFT: {self.first_token_ms:.2f} ms" if self.first_token_ms >= 0
                              else "TTFT: --")
         return "[ " + " | ".join(parts) + " ]" if parts else ""
+
+
+@dataclass
+class _TokensOnTheWay:
+    """What a step's sampling kernels chose, not read yet: on the GPU (for the next step's rows)
+    and on its way into pinned host memory; ``copied`` is recorded behind that copy."""
+    requests: List[Request]
+    place: Dict[int, int]                # id(request) -> its place in ``tokens``
+    tokens: torch.Tensor                 # int32 [n] on the GPU
+    host: torch.Tensor                   # pinned, filled when ``copied`` has happened
+    copied: "torch.cuda.Event"
 
 
 @dataclass
@@ -138,6 +152,10 @@ class Engine:
         self._t_first_add: Optional[float] = None
         self.last_logits: Optional[torch.Tensor] = None
         self.decode_runs = 0              # runs of queued decode steps taken so far
+        self.pipelined_steps = 0          # steps queued before their predecessor's tokens were read
+        self._on_the_way: List[_TokensOnTheWay] = []
+        self._host_ring: List[torch.Tensor] = []
+        self._host_at = 0
         if config.warm_kernels:
             self._warm_kernels()
 
@@ -191,18 +209,74 @@ class Engine:
         return req is not None and self.scheduler.abort(req)
 
     def has_unfinished(self) -> bool:
-        return self.scheduler.has_unfinished()
+        return self.scheduler.has_unfinished() or bool(self._on_the_way)
 
     # -- one engine step -----------------------------------------------------------------------
+    def _read_tokens(self, records: List[_TokensOnTheWay]) -> List[StepOutput]:
+        """Wait for these steps' tokens and hand them to their requests."""
+        outputs: List[StepOutput] = []
+        for rec in records:
+            rec.copied.synchronize()
+            tokens = rec.host[:len(rec.requests)].tolist()
+            if tokens and self.metrics.first_token_ms < 0 and self._t_first_add is not None:
+                self.metrics.first_token_ms = (time.perf_counter() - self._t_first_add) * 1e3
+            for req, tok in zip(rec.requests, tokens):
+                done = self.scheduler.resolve_token(req, tok)
+                if done is None:
+                    continue              # the request had ended before this token
+                req.sampler.observe([tok])
+                outputs.append(StepOutput(req.request_id, tok, done, req.finish_reason))
+        return outputs
+
+    def _read_all(self) -> List[StepOutput]:
+        records, self._on_the_way = self._on_the_way, []
+        return self._read_tokens(records)
+
+    def _pinned(self, n: int) -> torch.Tensor:
+        """The next of a few pinned buffers for token ids on their way to the host."""
+        if len(self._host_ring) < 4:
+            self._host_ring.append(torch.empty(max(n, self.config.max_batch), dtype=torch.int32,
+                                               pin_memory=True))
+            return self._host_ring[-1]
+        self._host_at = (self._host_at + 1) % len(self._host_ring)
+        if self._host_ring[self._host_at].numel() < n:
+            self._host_ring[self._host_at] = torch.empty(n, dtype=torch.int32, pin_memory=True)
+        return self._host_ring[self._host_at]
+
+    def _can_go_ahead(self, entries) -> bool:
+        """Whether this step may be queued before the last step's tokens have been read: it
+        holds a prompt portion (steps of decoded tokens alone are queued in runs instead), and
+        every token it asks for can be chosen on the GPU."""
+        if not self.config.pipeline or not any(e.n_tokens > 1 for e in entries):
+            return False
+        return Sampler.runs_on_device([e.request.sampler for e in entries if e.samples],
+                                      self.model.vocab_size)
+
     def step(self) -> List[StepOutput]:
         """Schedule, run one step of the model, sample, and report every request that got a
-        token or ended."""
+        token or ended.  A step that goes ahead of its predecessor's tokens reports those of the
+        step before it instead; its own come with the next call."""
         outputs: List[StepOutput] = []
-        entries, failed = self.scheduler.schedule()
-        for req in failed:
+        failed_all: List[Request] = []
+        while True:
+            try:
+                entries, failed = self.scheduler.schedule()
+            except TokensUnread:
+                if not self._on_the_way:
+                    raise
+                outputs += self._read_all()
+                continue
+            failed_all += failed
+            ahead = bool(entries) and self._can_go_ahead(entries)
+            if ahead or not self._on_the_way:
+                break
+            outputs += self._read_all()   # the step needs them: read, and decide again
+        for req in failed_all:
             outputs.append(StepOutput(req.request_id, None, True, req.finish_reason))
         if not entries:
             return outputs
+        if ahead:
+            return outputs + self._step_ahead(entries)
         run = self._decode_run(entries)
         if run is not None:
             return outputs + run
@@ -221,9 +295,24 @@ class Engine:
         else:
             tokens = []
             torch.cuda.synchronize(self.device)
-        dt = time.perf_counter() - t0
+        self._count(self._tally(entries), time.perf_counter() - t0)
+        m = self.metrics
+        if tokens and m.first_token_ms < 0 and self._t_first_add is not None:
+            m.first_token_ms = (time.perf_counter() - self._t_first_add) * 1e3
+        for req, tok in zip(sampling, tokens):
+            req.sampler.observe([tok])
+            done = self.scheduler.append_token(req, tok)
+            outputs.append(StepOutput(req.request_id, tok, done, req.finish_reason))
+        return outputs
+
+    @staticmethod
+    def _tally(entries):
+        """(prompt tokens, decoded tokens) of a step, before its own tokens are recorded."""
         n_prefill = sum(e.n_tokens for e in entries if e.n_tokens > 1 or not e.request.output)
-        n_decode = sum(e.n_tokens for e in entries) - n_prefill
+        return n_prefill, sum(e.n_tokens for e in entries) - n_prefill
+
+    def _count(self, tally, dt: float) -> None:
+        n_prefill, n_decode = tally
         m = self.metrics
         m.steps += 1
         total = n_prefill + n_decode
@@ -231,12 +320,46 @@ class Engine:
         m.decode_tokens += n_decode
         m.prefill_seconds += dt * n_prefill / total
         m.decode_seconds += dt * n_decode / total
-        if tokens and m.first_token_ms < 0 and self._t_first_add is not None:
-            m.first_token_ms = (time.perf_counter() - self._t_first_add) * 1e3
-        for req, tok in zip(sampling, tokens):
-            req.sampler.observe([tok])
-            done = self.scheduler.append_token(req, tok)
-            outputs.append(StepOutput(req.request_id, tok, done, req.finish_reason))
+
+    def _step_ahead(self, entries) -> List[StepOutput]:
+        """Queue the step without having read what the step before it chose: the rows of the
+        requests that decode take their tokens from the GPU.  Then wait for the tokens of the
+        step before (the GPU is busy with this one meanwhile) and report them."""
+        t0 = time.perf_counter()
+        newest = self._on_the_way[-1] if self._on_the_way else None
+        step_entries, pairs = [], []
+        for i, e in enumerate(entries):
+            req = e.request
+            toks = req.tokens_from(req.computed, e.n_tokens)
+            if req.unread:                # its one pending token is the one on the way
+                if e.n_tokens != 1 or req.unread != 1 or newest is None or \
+                        id(req) not in newest.place:
+                    raise RuntimeError(f"request {req.request_id!r}: unread tokens out of step")
+                toks = [0]
+                pairs.append((i, newest.place[id(req)]))
+            step_entries.append(StepEntry(req.cache, toks, [e.n_tokens - 1] if e.samples else []))
+        logits = self.runner.step(step_entries,
+                                  placed=(newest.tokens, pairs) if pairs else None)
+        self.scheduler.advance(entries)
+        tally = self._tally(entries)
+        self.last_logits = logits
+        self.pipelined_steps += 1
+        older, self._on_the_way = self._on_the_way, []
+        sampling = [e.request for e in entries if e.samples]
+        if sampling:
+            n = len(sampling)
+            chosen = torch.empty(n, dtype=torch.int32, device=self.device)
+            self.sampler.launch(logits, [r.sampler for r in sampling], out=chosen)
+            host = self._pinned(n)
+            host[:n].copy_(chosen, non_blocking=True)
+            copied = torch.cuda.Event()
+            copied.record()
+            self._on_the_way.append(_TokensOnTheWay(
+                sampling, {id(r): i for i, r in enumerate(sampling)}, chosen, host, copied))
+            for r in sampling:
+                self.scheduler.expect_token(r)
+        outputs = self._read_tokens(older)
+        self._count(tally, time.perf_counter() - t0)
         return outputs
 
     def _decode_run(self, entries) -> Optional[List[StepOutput]]:
@@ -305,6 +428,7 @@ class Engine:
         return result
 
     def shutdown(self) -> None:
+        self._on_the_way.clear()
         for req in list(self.scheduler.running):
             self.scheduler.finish(req, "shutdown")
         self.scheduler.waiting.clear()

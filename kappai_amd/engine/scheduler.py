@@ -15,6 +15,16 @@ prompt and the tokens it has generated (state of fixed size cannot be rewound: k
 poisons an interrupted hybrid session for the same reason, src/context.c:1438-1441).  A
 request that cannot fit although it is alone fails with "context exceeds cache".
 
+A step's tokens need not be read back before the next step is decided: ``expect_token`` notes
+that a request has a token on the way (its place in ``output`` holds ``UNREAD``), the request
+goes on as if that token were no end-of-sequence token, and ``resolve_token`` puts the token
+in once it has been read.  What can be known without the token is known at once: a request
+that reaches ``n_predict`` or the end of the context with it takes no further step
+(``DRAINING``) and ends when the token arrives.  A request whose unread token turns out to be
+an end-of-sequence token has run one step too many; that step's token is dropped.  Nothing
+that holds unread tokens is preempted or failed: ``schedule`` raises ``TokensUnread`` first,
+and the caller reads the tokens and asks again.
+
 The scheduler decides; it runs nothing.  It needs a cache manager's bookkeeping only.
 """
 from __future__ import annotations
@@ -27,6 +37,13 @@ from ..cache.manager import CacheManager, RequestCache
 from ..sampling.params import SamplingParams
 
 WAITING, RUNNING, FINISHED, FAILED = "waiting", "running", "finished", "failed"
+DRAINING = "draining"      # holds its cache, takes no further step, ends when its token is read
+UNREAD = -1                # stands in ``Request.output`` for a token that is still on the GPU
+
+
+class TokensUnread(Exception):
+    """A decision needs tokens that have not been read back yet (a request that holds some
+    would be preempted or failed).  Nothing has been taken from any request."""
 
 
 @dataclass
@@ -42,6 +59,9 @@ class Request:
     admitted_at: int = -1                    # admission counter, for choosing whom to preempt
     preemptions: int = 0
     sampler: object = None                   # per-request sampling state, owned by the engine
+    unread: int = 0                          # tokens at the end of ``output`` that are UNREAD
+    dropped: int = 0                         # tokens on the way that are to be thrown away
+    draining_reason: Optional[str] = None
 
     @property
     def tokens(self) -> List[int]:
@@ -103,7 +123,15 @@ class Scheduler:
         return bool(self.waiting or self.running)
 
     # -- decisions -----------------------------------------------------------------------
+    def _tokens_first(self) -> None:
+        """Before room is made at somebody's cost: tokens on the way may end requests and give
+        their pages back, and a request that holds some cannot be computed again."""
+        for r in self.running:
+            if r.unread:
+                raise TokensUnread(r.request_id)
+
     def _preempt(self, victim: Request) -> None:
+        self._tokens_first()
         self.cache.close(victim.cache)
         victim.cache = None
         victim.computed = 0
@@ -113,7 +141,10 @@ class Scheduler:
         self.running.remove(victim)
         self.waiting.appendleft(victim)
 
-    def _fail(self, request: Request, reason: str, finished: List[Request]) -> None:
+    def _fail(self, request: Request, reason: str, finished: List[Request],
+              waiting: bool = False) -> None:
+        if not waiting:
+            self._tokens_first()
         if request.cache is not None:
             self.cache.close(request.cache)
             request.cache = None
@@ -132,6 +163,7 @@ class Scheduler:
             entries = self._schedule_once(failed)
             if entries or not self.running:
                 return entries, failed
+            self._tokens_first()
             victim = max(self.running, key=lambda r: r.admitted_at)
             if len(self.running) == 1:
                 self._fail(victim, "context exceeds cache", failed)
@@ -157,6 +189,7 @@ class Scheduler:
             if req.state != RUNNING or req.pending != 1 or req.computed == 0 or budget < 1:
                 continue
             while not take(req, 1):
+                self._tokens_first()
                 victim = max(self.running, key=lambda r: r.admitted_at)
                 if victim is req and len(self.running) == 1:
                     self._fail(req, "context exceeds cache", failed)
@@ -178,7 +211,7 @@ class Scheduler:
         for req in sorted(self.running, key=lambda r: r.admitted_at):
             if budget < 1:
                 break
-            if any(e.request is req for e in entries) or req.pending < 1:
+            if any(e.request is req for e in entries) or req.pending < 1 or req.state != RUNNING:
                 continue
             n = min(req.pending, cfg.chunk, budget)
             if take(req, n):
@@ -190,7 +223,7 @@ class Scheduler:
             total = len(req.prompt) + len(req.output)
             if total > self.max_context:
                 self.waiting.popleft()
-                self._fail(req, "context exceeds cache", failed)
+                self._fail(req, "context exceeds cache", failed, waiting=True)
                 continue
             if self.cache.num_free_slots < 1:
                 break
@@ -199,7 +232,7 @@ class Scheduler:
             if not self.cache.can_extend(probe, n, reserve):
                 if not self.running and not entries:
                     self.waiting.popleft()
-                    self._fail(req, "context exceeds cache", failed)
+                    self._fail(req, "context exceeds cache", failed, waiting=True)
                     continue
                 break
             self.waiting.popleft()
@@ -218,24 +251,60 @@ class Scheduler:
         for e in entries:
             e.request.computed += e.n_tokens
 
+    def _end_by_count(self, request: Request) -> Optional[str]:
+        if 0 <= request.params.n_predict <= len(request.output):
+            return "length"
+        if len(request.prompt) + len(request.output) >= self.max_context:
+            return "context"
+        return None
+
     def append_token(self, request: Request, token: int) -> bool:
         """Record a sampled token.  Returns True when the request has finished (its cache is
         given back): end-of-sequence token, ``n_predict`` reached, or the context is full
         (kappai: src/context.c:1332-1334, 1399, 1444-1448)."""
         request.output.append(int(token))
-        reason = None
-        if int(token) in self.eos:
-            reason = "eos"
-        elif 0 <= request.params.n_predict <= len(request.output):
-            reason = "length"
-        elif len(request.prompt) + len(request.output) >= self.max_context:
-            reason = "context"
+        reason = "eos" if int(token) in self.eos else self._end_by_count(request)
         if reason is None:
             return False
         self.finish(request, reason)
         return True
 
+    def expect_token(self, request: Request) -> None:
+        """A token has been chosen for the request on the GPU and not been read yet."""
+        request.output.append(UNREAD)
+        request.unread += 1
+        reason = self._end_by_count(request)
+        if reason is not None:
+            request.state, request.draining_reason = DRAINING, reason
+
+    def resolve_token(self, request: Request, token: int) -> Optional[bool]:
+        """The oldest unread token of the request has arrived.  Returns None when the token is
+        one to be thrown away (the request had ended before it), else whether the request has
+        finished with it."""
+        if request.dropped:
+            request.dropped -= 1
+            return None
+        if request.unread < 1:
+            raise ValueError(f"request {request.request_id!r} expects no token")
+        at = len(request.output) - request.unread
+        request.output[at] = int(token)
+        request.unread -= 1
+        if int(token) in self.eos:
+            request.dropped = request.unread      # steps taken past the end
+            del request.output[at + 1:]
+            request.unread = 0
+            self.finish(request, "eos")
+            return True
+        if request.state == DRAINING and request.unread == 0:
+            self.finish(request, request.draining_reason)
+            return True
+        return False
+
     def finish(self, request: Request, reason: str) -> None:
+        if request.unread:                        # ended from outside with tokens on the way
+            del request.output[len(request.output) - request.unread:]
+            request.dropped += request.unread
+            request.unread = 0
         if request.cache is not None:
             self.cache.close(request.cache)
             request.cache = None

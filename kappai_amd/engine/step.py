@@ -16,7 +16,7 @@ import numpy as np
 import torch
 
 from ..cache.manager import CacheManager, OutOfPages, RequestCache
-from ..kernels import profile
+from ..kernels import ops, profile
 from ..models.base import Model
 from .batch import RowBatch, StepEntry, layout_rows
 from .cforward import CForward, Workspace
@@ -234,10 +234,20 @@ class StepRunner:
         self._staged = torch.cuda.Event()
         self._staged.record()
 
-    def make_batch(self, entries: Sequence[StepEntry]) -> RowBatch:
+    def make_batch(self, entries: Sequence[StepEntry], placed=None) -> RowBatch:
+        """``placed``: see ``step``."""
         arrays, sizes = layout_rows(entries, self.cache, self.model.vocab_size,
                                     getattr(self.model, "q_tile_rows", None))
+        if placed is not None and placed[1]:
+            chosen, pairs = placed
+            for ei, at in pairs:
+                if not (0 <= ei < len(entries) and 0 <= at < chosen.numel()):
+                    raise ValueError(f"placed token: entry {ei} or place {at} does not exist")
+            arrays["place_dst"] = arrays["seg_start"][[ei for ei, _ in pairs]]
+            arrays["place_src"] = np.asarray([at for _, at in pairs], dtype=np.int32)
         dev = self._upload(arrays)
+        if "place_dst" in arrays:
+            ops.place_tokens(dev["tokens"], dev["place_dst"], placed[0], dev["place_src"])
         return RowBatch(
             n_rows=sizes["n_rows"], n_segments=sizes["n_segments"],
             n_logit_rows=sizes["n_logit_rows"], max_position=sizes["max_position"],
@@ -328,15 +338,20 @@ class StepRunner:
         return out
 
     # -- one step ----------------------------------------------------------------------------
-    def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+    def step(self, entries: Sequence[StepEntry], placed=None) -> torch.Tensor:
         """Run the entries' tokens as one batch from the cache that earlier steps left and
         return float32 logits [wanted, vocab] on the GPU, in the order of the entries and of
         their ``want``.  If the pages do not suffice, ``OutOfPages`` is raised and neither
-        the cache nor any request has changed."""
+        the cache nor any request has changed.
+
+        ``placed`` = (int32 tensor on the GPU, [(entry, place), ...]): the first token of each
+        of these entries is not the one in its ``tokens`` but the one at that place of the
+        tensor, which the GPU has or will have when the step runs (what sampling kernels wrote
+        for the step before, not read back yet)."""
         entries = list(entries)
         if not entries:
             raise ValueError("a step needs at least one entry")
-        single = all(len(e.tokens) == 1 for e in entries)
+        single = all(len(e.tokens) == 1 for e in entries) and placed is None
         extended: List[StepEntry] = []
         try:
             for e in entries:
@@ -354,7 +369,7 @@ class StepRunner:
             if self.decode_graphs and single:
                 logits = self._decode_step(entries)
             if logits is None:
-                batch = self.make_batch(entries)
+                batch = self.make_batch(entries, placed)
                 logits = self.forward(batch)
         except Exception:
             for e in entries:

@@ -81,6 +81,21 @@ def embed_rows(ids: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
     return out
 
 
+def place_tokens(tokens: torch.Tensor, dst_rows: torch.Tensor, chosen: torch.Tensor,
+                 src_idx: torch.Tensor) -> None:
+    """``tokens[dst_rows[i]] = chosen[src_idx[i]]`` (all int32, on the GPU): token ids that
+    sampling kernels left on the GPU go into a step's token table.  The host vouches for the
+    indices (rows of this step, places in ``chosen``)."""
+    for name, t in (("tokens", tokens), ("dst_rows", dst_rows), ("chosen", chosen),
+                    ("src_idx", src_idx)):
+        _gpu(name, t, I32)
+        _need(t.dim() == 1, lambda: f"place_tokens: {name} must have one dimension")
+    _need(dst_rows.shape == src_idx.shape, "place_tokens: as many rows as places")
+    check(library("elementwise").kappai_place_tokens(
+        _ptr(tokens), _ptr(dst_rows), _ptr(chosen), _ptr(src_idx), _c_int(dst_rows.shape[0]),
+        _stream()), "place_tokens")
+
+
 def add_rmsnorm(resid: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Tensor,
                 eps: float, out_dtype, rows: Optional[torch.Tensor] = None,
                 write_resid: bool = True, fragment: bool = False):

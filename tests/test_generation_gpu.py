@@ -205,9 +205,9 @@ def test_random_engine_options_give_the_same_tokens(model_dirs):
                        max_batch=rng.choice([1, 2, 3, 8]),
                        token_budget=rng.choice([1, 3, 17, 64, 2048]),
                        chunk=rng.choice([1, 2, 5, 33, 2048]), decode_run=rng.choice([1, 2, 8]),
-                       warm_kernels=rng.random() < 0.5)
+                       warm_kernels=rng.random() < 0.5, pipeline=rng.random() < 0.7)
         roomy = Engine(str(model_dirs[name]), dtype="float32", num_pages=256, page_size=16,
-                       max_batch=8, decode_run=1, warm_kernels=False)
+                       max_batch=8, decode_run=1, warm_kernels=False, pipeline=False)
         want = roomy.generate(prompts, params)
         eng = Engine(str(model_dirs[name]), dtype="float32", **options)
         got = eng.generate(prompts, params)
@@ -378,6 +378,57 @@ def test_end_of_sequence_inside_a_decode_run(model_dirs, tmp_path):
         assert eng.cache.num_free_pages() == 256 and eng.cache.num_free_slots == 8
 
 
+def test_steps_ahead_of_their_tokens_give_the_same_tokens(model_dirs, tmp_path):
+    """Steps with prompt portions in them are queued before the tokens of the step before have
+    been read: the requests that decode beside the prompts take their tokens on the GPU.  The
+    tokens must be those of steps that are waited for one by one: greedy and sampled requests,
+    one that draws its end-of-sequence token while prompts are under way (it has taken a step
+    too many by the time that is known), a roomy pool and one so tight that the scheduler has
+    to ask for the tokens before it preempts."""
+    import random
+    from kappai_amd.engine import Engine, EngineConfig
+    from kappai_amd.sampling import SamplingParams
+    rng = random.Random(5)
+    vocab = TINY["B"][0]["vocab_size"]
+    n = 14
+    prompts = [[rng.randrange(vocab) for _ in range(rng.randint(3, 150))] for _ in range(n)]
+    params = [SamplingParams.greedy(n_predict=rng.randint(2, 40)) if i % 2 else
+              SamplingParams(temperature=0.9, top_k=rng.choice([0, 20]), top_p=1.0, min_p=0.0,
+                             seed=70 + i, n_predict=rng.randint(2, 40)) for i in range(n)]
+
+    def run(folder, pipeline, pages):
+        eng = Engine(EngineConfig(model=str(folder), dtype="float32", num_pages=pages,
+                                  max_batch=6, token_budget=48, chunk=40, pipeline=pipeline))
+        out = eng.generate(prompts, params)
+        eng.cache.check()
+        assert eng.cache.num_free_pages() == pages and eng.cache.num_free_slots == 6
+        assert not eng._on_the_way
+        return out, eng
+
+    free, _ = run(model_dirs["B"], False, 400)
+    # an end-of-sequence token: one that a request draws while others' prompts are under way
+    counts = {}
+    for o in free:
+        for t in o[1:6]:
+            counts[t] = counts.get(t, 0) + 1
+    eos = max(counts, key=counts.get)
+    cfg = json.loads((model_dirs["B"] / "config.json").read_text())
+    cfg["eos_token_id"] = eos
+    folder = tmp_path / "with_eos"
+    folder.mkdir()
+    (folder / "config.json").write_text(json.dumps(cfg))
+    (folder / "model.safetensors").write_bytes((model_dirs["B"] / "model.safetensors").read_bytes())
+    want, _ = run(folder, False, 400)
+    assert any(o[-1] == eos and len(o) < p.n_predict for o, p in zip(want, params))
+    got, eng = run(folder, True, 400)
+    assert got == want
+    assert eng.pipelined_steps > 20
+    assert sum(r.dropped for r in eng.requests.values()) == 0     # all thrown away by now
+    tight, eng = run(folder, True, 26)
+    assert tight == want
+    assert eng.scheduler.preempted_total > 0 and eng.pipelined_steps > 20
+
+
 def test_random_workload_with_and_without_graphs(model_dirs):
     """Forty requests of random lengths and options through the scheduler, prompts in portions
     beside decoded tokens: captured graphs, runs of queued decode steps, batches filled up with
@@ -403,7 +454,7 @@ def test_random_workload_with_and_without_graphs(model_dirs):
     for graphs, pages in ((False, 2000), (True, 2000), (True, 90)):
         eng = Engine(EngineConfig(model=str(model_dirs["B"]), dtype="float32", num_pages=pages,
                                   max_batch=16, token_budget=128, chunk=96,
-                                  decode_run=8 if graphs else 1))
+                                  decode_run=8 if graphs else 1, pipeline=graphs))
         eng.runner.decode_graphs = graphs
         results[(graphs, pages)] = eng.generate(prompts, params)
         eng.cache.check()

@@ -5,8 +5,8 @@ import random
 import pytest
 
 from kappai_amd.cache import CacheManager, FixedState, PagedKV
-from kappai_amd.engine.scheduler import (FAILED, FINISHED, RUNNING, WAITING, Request, Scheduler,
-                                         SchedulerConfig)
+from kappai_amd.engine.scheduler import (DRAINING, FAILED, FINISHED, RUNNING, UNREAD, WAITING,
+                                         Request, Scheduler, SchedulerConfig, TokensUnread)
 from kappai_amd.sampling import SamplingParams
 
 SPECS = [FixedState((8, 2)), PagedKV(2, 16), FixedState((8, 2)), PagedKV(2, 16)]
@@ -209,3 +209,164 @@ def test_random_load_always_ends(seed):
             assert r.finish_reason == "context exceeds cache"
     assert cm.num_free_pages() == cm.paged_groups[0].allocator.num_pages
     assert cm.num_free_slots == cm.num_slots
+
+
+# ---- tokens that are read a step late ------------------------------------------------------
+class Lagged:
+    """Drives the scheduler the way an engine does that queues a step before it has read the
+    tokens of the step before: ``expect_token`` after each step, ``resolve_token`` a step later
+    (or at once, when the scheduler asks for the tokens)."""
+
+    def __init__(self, cm, sch, token_of):
+        self.cm, self.sch, self.token_of = cm, sch, token_of
+        self.on_the_way = []             # requests whose tokens have not been read, by step
+        self.asked = 0                   # times the scheduler wanted the tokens first
+        self.dropped = 0
+
+    def read(self, steps):
+        finished = []
+        for requests in steps:
+            for r in requests:
+                if r.dropped:
+                    done = self.sch.resolve_token(r, 12345)
+                    assert done is None
+                    self.dropped += 1
+                    continue
+                at = len(r.output) - r.unread
+                if self.sch.resolve_token(r, self.token_of(r, at)):
+                    finished.append(r)
+        return finished
+
+    def step(self):
+        finished = []
+        while True:
+            try:
+                entries, failed = self.sch.schedule()
+                break
+            except TokensUnread:
+                assert self.on_the_way
+                self.asked += 1
+                steps, self.on_the_way = self.on_the_way, []
+                finished += self.read(steps)
+        for e in entries:
+            self.cm.extend(e.request.cache, e.n_tokens)
+        for e in entries:
+            self.cm.commit(e.request.cache, e.n_tokens)
+        self.sch.advance(entries)
+        older, self.on_the_way = self.on_the_way, []
+        sampling = [e.request for e in entries if e.samples]
+        if sampling:
+            self.on_the_way.append(sampling)
+            for r in sampling:
+                self.sch.expect_token(r)
+        finished += self.read(older)
+        self.cm.check()
+        return entries, failed, finished
+
+    def unfinished(self):
+        return self.sch.has_unfinished() or bool(self.on_the_way)
+
+
+def test_tokens_read_a_step_late():
+    """a's third token is the end-of-sequence token.  Read a step late, it is known only after
+    a has taken one step more; that step's token is thrown away.  b ends by its count, which is
+    known without its token: it takes no step too many."""
+    cm, sch = make(token_budget=64)
+    lag = Lagged(cm, sch, lambda r, at: 99 if (r.request_id, at) == ("a", 2) else 10 + at)
+    a, b = req("a", 4), req("b", 6, n_predict=2)
+    sch.add(a)
+    sch.add(b)
+    e, _, fin = lag.step()               # prompts; nothing read yet
+    assert [(x.request.request_id, x.n_tokens) for x in e] == [("a", 4), ("b", 6)] and not fin
+    assert a.output == [UNREAD] and a.unread == 1 and a.pending == 1
+    e, _, fin = lag.step()               # both decode from tokens they have not seen
+    assert [(x.request.request_id, x.n_tokens, x.samples) for x in e] == [
+        ("a", 1, True), ("b", 1, True)]
+    assert a.output == [10, UNREAD] and b.output == [10, UNREAD]
+    assert b.state == DRAINING and not fin       # b's second token is its last, whatever it is
+    e, _, fin = lag.step()
+    assert [x.request.request_id for x in e] == ["a"]
+    assert [(r.request_id, r.finish_reason) for r in fin] == [("b", "length")]
+    assert b.output == [10, 11] and b.cache is None
+    e, _, fin = lag.step()               # a runs once more while its end token is on the way
+    assert [x.request.request_id for x in e] == ["a"]
+    assert [(r.request_id, r.finish_reason) for r in fin] == [("a", "eos")]
+    assert a.output == [10, 11, 99] and a.dropped == 1 and a.cache is None
+    assert lag.unfinished()              # the token of the step too many is still on the way
+    e, _, fin = lag.step()
+    assert not e and not fin and lag.dropped == 1 and not lag.unfinished()
+    assert cm.num_free_pages() == 64 and cm.num_free_slots == 8
+
+
+def test_nobody_with_unread_tokens_is_preempted():
+    """Three pages of 4 tokens; a and b hold one each and both need a second.  With their
+    tokens on the way the scheduler asks for the tokens instead of preempting b; once they are
+    in, b is preempted with an output that holds no placeholder."""
+    cm, sch = make(pages=3, token_budget=64)
+    lag = Lagged(cm, sch, lambda r, at: 10 + at)
+    a, b = req("a", 4, n_predict=6), req("b", 4, n_predict=6)
+    sch.add(a)
+    sch.add(b)
+    lag.step()
+    assert a.unread == 1 and b.unread == 1 and lag.asked == 0
+    with pytest.raises(TokensUnread):
+        sch.schedule()
+    assert a.state == RUNNING and b.state == RUNNING and b.cache is not None   # nothing taken
+    e, _, _ = lag.step()
+    assert lag.asked == 1 and [x.request.request_id for x in e] == ["a"]
+    assert b.state == WAITING and b.output == [10] and b.unread == 0 and b.preemptions == 1
+    while lag.unfinished():
+        lag.step()
+    assert a.output == [10 + i for i in range(6)] and b.output == a.output
+    assert cm.num_free_pages() == 3
+
+
+def test_abort_with_a_token_on_the_way():
+    cm, sch = make(token_budget=64)
+    lag = Lagged(cm, sch, lambda r, at: 10 + at)
+    a = req("a", 4)
+    sch.add(a)
+    lag.step()
+    lag.step()
+    assert a.output == [10, UNREAD]
+    assert sch.abort(a)
+    assert a.output == [10] and a.dropped == 1 and a.unread == 0 and a.cache is None
+    _, _, fin = lag.step()
+    assert not fin and lag.dropped == 1 and not lag.unfinished()
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_random_load_read_late_gives_the_same_tokens(seed):
+    """The same load with tokens read at once and read a step late: every request ends the same
+    way with the same output, whatever was preempted on the way."""
+    def token_of(r, at):
+        h = hash((r.request_id, at)) % 97
+        return 99 if h < 4 else h        # now and then an end-of-sequence token
+
+    def load(lagged):
+        rng = random.Random(seed)
+        cm, sch = make(pages=rng.randint(6, 30), slots=rng.randint(1, 6),
+                       page_size=rng.choice([1, 4, 16]), token_budget=rng.choice([4, 16, 64]),
+                       chunk=rng.choice([3, 8, 64]))
+        reqs = [req(f"r{i}", rng.randint(1, 30), n_predict=rng.randint(1, 12)) for i in range(25)]
+        pending = list(reqs)
+        lag = Lagged(cm, sch, token_of)
+        steps = 0
+        while pending or (lag.unfinished() if lagged else sch.has_unfinished()):
+            if pending and rng.random() < 0.5:
+                sch.add(pending.pop(0))
+            if lagged:
+                entries, _, _ = lag.step()
+            else:
+                entries, _, _ = run_step(cm, sch, next_token=lambda r: token_of(r, len(r.output)))
+            assert sum(e.n_tokens for e in entries) <= sch.config.token_budget
+            steps += 1
+            assert steps < 5000
+        assert cm.num_free_pages() == cm.paged_groups[0].allocator.num_pages
+        assert cm.num_free_slots == cm.num_slots
+        return [(r.state, r.finish_reason, list(r.output)) for r in reqs], lag
+
+    at_once, _ = load(False)
+    late, lag = load(True)
+    assert late == at_once
+    assert all(UNREAD not in out for _, _, out in late)
