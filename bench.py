@@ -179,26 +179,71 @@ class DecodeBench:
         from kappai_amd.kernels import ops
         ops.sample_rows(logits, self.temp, self.uni, out=out_row)
 
-    def run(self, warmup, steps, run_len=8):
+    def run(self, warmup, steps, run_len=8, ahead=True):
         """``steps`` decode steps, taken the way the engine takes them when nothing but decoding
         is going on: up to ``run_len`` steps queued back to back, each step's token handed to the
-        next on the GPU, the host reading the tokens at the end of the run."""
-        for _ in range(warmup):
+        next on the GPU, and a run queued before the host has read the tokens of the run before
+        it (they travel to pinned memory behind the run's last kernel)."""
+        from kappai_amd.kernels import ops
+        torch = self.torch
+        B = len(self.requests)
+        hosts = [torch.empty((run_len, B), dtype=torch.int32, pin_memory=True) for _ in range(2)]
+        state = {"before": None, "runs": 0}   # before: (tokens of the last run on the GPU, host
+                                               # copy, event behind the copy)
+
+        def read(rec):
+            rec[2].synchronize()
+            self.tokens = rec[1][rec[0].shape[0] - 1].tolist()
+
+        def take(steps):
+            left = steps
+            while left > 0:
+                n = min(run_len, left)
+                before = state["before"]
+                out = None
+                if n > 1:
+                    placed = None
+                    if before is not None:
+                        last = (before[0].shape[0] - 1) * B
+                        placed = (before[0].view(-1), [(i, last + i) for i in range(B)])
+                    out = self.runner.decode_run(self.requests, self.tokens, n, self._choose,
+                                                 placed=placed)
+                if out is None:
+                    if before is not None:
+                        read(before)
+                        state["before"] = None
+                    self.step()
+                    left -= 1
+                    continue
+                host = hosts[state["runs"] % 2]
+                ops.tokens_to_host(out, host)
+                done = torch.cuda.Event()
+                done.record()
+                if before is not None:
+                    read(before)
+                state["before"] = (out, host, done)
+                if not ahead:            # every run read before the next is queued
+                    read(state["before"])
+                    state["before"] = None
+                state["runs"] += 1
+                left -= n
+            if state["before"] is not None:
+                read(state["before"])
+                state["before"] = None
+
+        # warm-up: single steps first (the second of a shape captures its graph), then, when
+        # there are steps enough, two short runs, so that everything a run needs has run once
+        singles = warmup - 4 if warmup >= 6 else warmup
+        for _ in range(singles):
             self.step()
+        if warmup > singles:
+            full = run_len
+            run_len = 2
+            take(warmup - singles)
+            run_len = full
         sync()
         t0 = time.perf_counter()
-        left = steps
-        while left > 0:
-            n = min(run_len, left)
-            out = None
-            if n > 1:
-                out = self.runner.decode_run(self.requests, self.tokens, n, self._choose)
-            if out is None:
-                self.step()
-                left -= 1
-            else:
-                self.tokens = out[-1].tolist()
-                left -= n
+        take(steps)
         sync()
         return time.perf_counter() - t0
 

@@ -49,6 +49,22 @@ extern "C" int kappai_place_tokens(int* tokens, const int* dst_rows, const int* 
 }
 
 // ---------------------------------------------------------------------------------------
+// dst[i] = src[i]: token ids to pinned host memory by a kernel.  (A copy command from device to
+// host that is still pending makes the host wait when the next copy from host to device is
+// queued behind it; a kernel that writes to host memory does not.)
+// ---------------------------------------------------------------------------------------
+__global__ void copy_ints_kernel(int* __restrict__ dst, const int* __restrict__ src, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) dst[i] = src[i];
+}
+
+extern "C" int kappai_copy_ints(int* dst, const int* src, int n, hipStream_t stream) {
+  if (n <= 0) return 0;
+  hipLaunchKernelGGL(copy_ints_kernel, dim3((n + 255) / 256), dim3(256), 0, stream, dst, src, n);
+  KAPPAI_RETURN_LAUNCH_STATUS();
+}
+
+// ---------------------------------------------------------------------------------------
 // RMSNorm with the residual sum folded in:
 //   x = resid[r] (+ delta[r]);  if write_resid: resid[r] = x;
 //   out[i] = x * rsqrt(mean(x^2) + eps) * w           (src/backend/cpu/scalar/quants.c:1507-1512)

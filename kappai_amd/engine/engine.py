@@ -15,6 +15,7 @@ from typing import Dict, List, Optional, Sequence, Union
 import torch
 
 from ..cache.manager import CacheManager
+from ..kernels import ops
 from ..models import Model, load_model
 from ..sampling import RequestSampler, Sampler, SamplingParams
 from .batch import StepEntry
@@ -82,13 +83,19 @@ class Metrics:
 
 @dataclass
 class _TokensOnTheWay:
-    """What a step's sampling kernels chose, not read yet: on the GPU (for the next step's rows)
-    and on its way into pinned host memory; ``copied`` is recorded behind that copy."""
+    """What the sampling kernels of a step (or of a run of decode steps) chose, not read yet: on
+    the GPU (for the rows of the step after) and on its way into pinned host memory; ``copied``
+    is recorded behind that copy."""
     requests: List[Request]
-    place: Dict[int, int]                # id(request) -> its place in ``tokens``
-    tokens: torch.Tensor                 # int32 [n] on the GPU
+    place: Dict[int, int]                # id(request) -> its column
+    tokens: torch.Tensor                 # int32 [steps * len(requests)] on the GPU, step by step
     host: torch.Tensor                   # pinned, filled when ``copied`` has happened
     copied: "torch.cuda.Event"
+    steps: int = 1
+
+    def last(self, request: Request) -> int:
+        """Where in ``tokens`` the request's newest token stands."""
+        return (self.steps - 1) * len(self.requests) + self.place[id(request)]
 
 
 @dataclass
@@ -175,6 +182,15 @@ class Engine:
             warm = RequestSampler(SamplingParams.greedy())
             self.sampler.sample(logits, [warm])
             self.sampler.sample(self.runner.step([StepEntry(rc, [0], [0])]), [warm])
+            if self.config.pipeline and n + 3 <= (self.ctx_size or 1 << 30) and \
+                    self.cache.can_extend(rc, 2):
+                # what a step ahead of its tokens uses beside that: a token placed on the GPU,
+                # and the chosen tokens' own way into pinned memory
+                chosen = torch.zeros(1, dtype=torch.int32, device=self.device)
+                logits = self.runner.step([StepEntry(rc, [0, 0], [1])], placed=(chosen, [(0, 0)]))
+                self.sampler.launch(logits, [warm], out=chosen)
+                ops.tokens_to_host(chosen, self._pinned(1))
+                torch.cuda.synchronize(self.device)
         finally:
             self.cache.close(rc)
         self.runner.steps_run = 0
@@ -217,16 +233,33 @@ class Engine:
         outputs: List[StepOutput] = []
         for rec in records:
             rec.copied.synchronize()
-            tokens = rec.host[:len(rec.requests)].tolist()
+            width = len(rec.requests)
+            tokens = rec.host[:rec.steps * width].tolist()
             if tokens and self.metrics.first_token_ms < 0 and self._t_first_add is not None:
                 self.metrics.first_token_ms = (time.perf_counter() - self._t_first_add) * 1e3
-            for req, tok in zip(rec.requests, tokens):
-                done = self.scheduler.resolve_token(req, tok)
-                if done is None:
-                    continue              # the request had ended before this token
-                req.sampler.observe([tok])
-                outputs.append(StepOutput(req.request_id, tok, done, req.finish_reason))
+            for s in range(rec.steps):
+                for req, tok in zip(rec.requests, tokens[s * width:(s + 1) * width]):
+                    done = self.scheduler.resolve_token(req, tok)
+                    if done is None:
+                        continue          # the request had ended before this token
+                    req.sampler.observe([tok])
+                    outputs.append(StepOutput(req.request_id, tok, done, req.finish_reason))
         return outputs
+
+    def _send_home(self, requests: List[Request], chosen: torch.Tensor, steps: int) -> None:
+        """The tokens that kernels already queued will write into ``chosen`` start their way to
+        the host, and every request notes how many it has coming."""
+        n = chosen.numel()
+        host = self._pinned(n)
+        ops.tokens_to_host(chosen, host)
+        copied = torch.cuda.Event()
+        copied.record()
+        self._on_the_way.append(_TokensOnTheWay(
+            requests, {id(r): i for i, r in enumerate(requests)}, chosen, host, copied, steps))
+        for _ in range(steps):
+            for r in requests:
+                if r.state == RUNNING:    # (it may have reached its count inside the run)
+                    self.scheduler.expect_token(r)
 
     def _read_all(self) -> List[StepOutput]:
         records, self._on_the_way = self._on_the_way, []
@@ -243,19 +276,35 @@ class Engine:
             self._host_ring[self._host_at] = torch.empty(n, dtype=torch.int32, pin_memory=True)
         return self._host_ring[self._host_at]
 
-    def _can_go_ahead(self, entries) -> bool:
-        """Whether this step may be queued before the last step's tokens have been read: it
-        holds a prompt portion (steps of decoded tokens alone are queued in runs instead), and
-        every token it asks for can be chosen on the GPU."""
-        if not self.config.pipeline or not any(e.n_tokens > 1 for e in entries):
+    def _can_go_ahead(self, entries, allowed: bool = True) -> bool:
+        """Whether this step may be queued before the last step's tokens have been read: every
+        token it asks for can be chosen on the GPU, and it holds a prompt portion or is the
+        first of a run of decode steps."""
+        if not allowed or not self.config.pipeline or not Sampler.runs_on_device(
+                [e.request.sampler for e in entries if e.samples], self.model.vocab_size):
             return False
-        return Sampler.runs_on_device([e.request.sampler for e in entries if e.samples],
-                                      self.model.vocab_size)
+        if any(e.n_tokens > 1 for e in entries):
+            return True
+        return self._run_length(entries) >= 2
 
-    def step(self) -> List[StepOutput]:
+    def _run_length(self, entries) -> int:
+        """How many decode steps these entries can take back to back (0: they are not all single
+        decoded tokens): nobody may pass its own limits inside the run."""
+        n = self.config.decode_run
+        if n < 2 or any(e.n_tokens != 1 or not e.samples for e in entries):
+            return 0
+        for e in entries:
+            r = e.request
+            if r.params.n_predict >= 0:
+                n = min(n, r.params.n_predict - len(r.output))
+            n = min(n, self.scheduler.max_context - (len(r.prompt) + len(r.output)))
+        return n
+
+    def step(self, go_ahead: bool = True) -> List[StepOutput]:
         """Schedule, run one step of the model, sample, and report every request that got a
         token or ended.  A step that goes ahead of its predecessor's tokens reports those of the
-        step before it instead; its own come with the next call."""
+        step before it instead; its own come with the next call.  ``go_ahead=False``: this step
+        is waited for."""
         outputs: List[StepOutput] = []
         failed_all: List[Request] = []
         while True:
@@ -267,7 +316,7 @@ class Engine:
                 outputs += self._read_all()
                 continue
             failed_all += failed
-            ahead = bool(entries) and self._can_go_ahead(entries)
+            ahead = bool(entries) and self._can_go_ahead(entries, go_ahead)
             if ahead or not self._on_the_way:
                 break
             outputs += self._read_all()   # the step needs them: read, and decide again
@@ -276,7 +325,11 @@ class Engine:
         if not entries:
             return outputs
         if ahead:
-            return outputs + self._step_ahead(entries)
+            took = self._step_ahead(entries)
+            if took is not None:
+                return outputs + took
+            outputs += self._read_all()   # (no graph for the run yet, or too few pages)
+            return outputs + self.step(go_ahead=False)
         run = self._decode_run(entries)
         if run is not None:
             return outputs + run
@@ -331,13 +384,15 @@ class Engine:
         for i, e in enumerate(entries):
             req = e.request
             toks = req.tokens_from(req.computed, e.n_tokens)
-            if req.unread:                # its one pending token is the one on the way
-                if e.n_tokens != 1 or req.unread != 1 or newest is None or \
-                        id(req) not in newest.place:
+            if req.unread:                # the token it goes on from is the newest on the way
+                if e.n_tokens != 1 or newest is None or id(req) not in newest.place:
                     raise RuntimeError(f"request {req.request_id!r}: unread tokens out of step")
                 toks = [0]
-                pairs.append((i, newest.place[id(req)]))
+                pairs.append((i, newest.last(req)))
             step_entries.append(StepEntry(req.cache, toks, [e.n_tokens - 1] if e.samples else []))
+        run = self._run_length(entries)
+        if run >= 2:
+            return self._run_ahead(entries, run, newest, pairs, t0)
         logits = self.runner.step(step_entries,
                                   placed=(newest.tokens, pairs) if pairs else None)
         self.scheduler.advance(entries)
@@ -347,19 +402,41 @@ class Engine:
         older, self._on_the_way = self._on_the_way, []
         sampling = [e.request for e in entries if e.samples]
         if sampling:
-            n = len(sampling)
-            chosen = torch.empty(n, dtype=torch.int32, device=self.device)
+            chosen = torch.empty(len(sampling), dtype=torch.int32, device=self.device)
             self.sampler.launch(logits, [r.sampler for r in sampling], out=chosen)
-            host = self._pinned(n)
-            host[:n].copy_(chosen, non_blocking=True)
-            copied = torch.cuda.Event()
-            copied.record()
-            self._on_the_way.append(_TokensOnTheWay(
-                sampling, {id(r): i for i, r in enumerate(sampling)}, chosen, host, copied))
-            for r in sampling:
-                self.scheduler.expect_token(r)
+            self._send_home(sampling, chosen, 1)
         outputs = self._read_tokens(older)
         self._count(tally, time.perf_counter() - t0)
+        return outputs
+
+    def _run_ahead(self, entries, n: int, newest, pairs, t0) -> Optional[List[StepOutput]]:
+        """A run of ``n`` decode steps queued before the tokens on the way have been read: the
+        first step takes them on the GPU (``pairs``: (entry, place in ``newest.tokens``)).
+        Returns None, with nothing changed, when the run cannot be queued."""
+        reqs = [e.request for e in entries]
+        samplers = [r.sampler for r in reqs]
+
+        def choose(logits, step, out_row):
+            self.sampler.launch(logits, samplers, out=out_row)
+
+        first = [0 if r.unread else r.tokens_from(r.computed, 1)[0] for r in reqs]
+        tokens = self.runner.decode_run(
+            [r.cache for r in reqs], first, n, choose,
+            placed=(newest.tokens, pairs) if pairs else None)
+        if tokens is None:
+            return None
+        self.last_logits = None
+        self.decode_runs += 1
+        self.pipelined_steps += n
+        for r in reqs:
+            r.computed += n
+        older, self._on_the_way = self._on_the_way, []
+        self._send_home(reqs, tokens.view(-1), n)
+        outputs = self._read_tokens(older)
+        m = self.metrics
+        m.steps += n
+        m.decode_tokens += n * len(reqs)
+        m.decode_seconds += time.perf_counter() - t0
         return outputs
 
     def _decode_run(self, entries) -> Optional[List[StepOutput]]:
@@ -367,14 +444,8 @@ class Engine:
         token goes to the next on the GPU and the host reads them all at the end.  A request
         that meets its end-of-sequence token inside the run has run a few steps too many; they
         are dropped with its cache.  Returns None when the steps have to be taken one by one."""
-        n = self.config.decode_run
-        if n < 2 or any(e.n_tokens != 1 or not e.samples for e in entries):
-            return None
+        n = self._run_length(entries)
         reqs = [e.request for e in entries]
-        for r in reqs:       # nobody may pass its own limits inside the run
-            if r.params.n_predict >= 0:
-                n = min(n, r.params.n_predict - len(r.output))
-            n = min(n, self.scheduler.max_context - (len(r.prompt) + len(r.output)))
         samplers = [r.sampler for r in reqs]
         if n < 2 or not Sampler.runs_on_device(samplers, self.model.vocab_size):
             return None

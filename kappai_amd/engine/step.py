@@ -63,6 +63,7 @@ class _DecodeGraph:
         tiled = bool(runner.model.q_tile_rows)
         if tiled:
             shapes.append(("q_tiles", (B, 4)))
+        shapes += [("place_dst", (B,)), ("place_src", (B,))]
         shapes += [(f"block_table_{g}", (B, self.width)) for g in range(n_groups)]
         self.offsets, total = {}, 0
         for k, shp in shapes:
@@ -76,6 +77,7 @@ class _DecodeGraph:
         self.static = torch.zeros(self.total, dtype=torch.int32, device=dev)
         views = {k: self.static[self.offsets[k]:self.offsets[k] + int(np.prod(shp))].view(shp)
                  for k, shp in shapes}
+        self.views = views
         self.batch = RowBatch(
             n_rows=B, n_segments=B, n_logit_rows=n_logit, max_position=ctx_cap - 1,
             max_segment_rows=1, tokens=views["tokens"], row_pos=views["row_pos"],
@@ -120,15 +122,20 @@ class _DecodeGraph:
         if self._ring[i] is None:
             self._ring[i] = torch.empty(self.total, dtype=torch.int32, pin_memory=True)
         self._ring[i].numpy()[:] = self.mirror
-        self.static.copy_(self._ring[i], non_blocking=True)
+        ops.ints_from_host(self._ring[i], self.static)
         ev = self._ring_done[i] = torch.cuda.Event()
         ev.record()
 
     def run(self, runner: "StepRunner", caches, tokens, pos, slots, logit_rows,
-            device_tokens: Optional[torch.Tensor] = None) -> torch.Tensor:
+            device_tokens: Optional[torch.Tensor] = None, placed=None) -> torch.Tensor:
         """``tokens`` from the host, or ``device_tokens`` (int32 [B] on the GPU, e.g. what the last
-        step's sampling kernel wrote) copied into place on the GPU."""
+        step's sampling kernel wrote) copied into place on the GPU, or the host's with some of
+        them replaced on the GPU (``placed``, as in ``StepRunner.step``)."""
         h = self.h
+        if placed is not None:
+            for k, (row, at) in enumerate(placed[1]):
+                h["place_dst"][k] = row
+                h["place_src"][k] = at
         n = len(caches)                  # rows n .. B-1 are dummies: token 0 at position 0 of
         if device_tokens is None:        # the scratch slot and page, logits nobody reads
             h["tokens"][:n] = tokens
@@ -160,6 +167,10 @@ class _DecodeGraph:
         self._upload(runner)
         if device_tokens is not None:
             self.batch.tokens[:n].copy_(device_tokens)
+        elif placed is not None and placed[1]:
+            m = len(placed[1])
+            ops.place_tokens(self.batch.tokens, self.views["place_dst"][:m], placed[0],
+                             self.views["place_src"][:m])
         self.graph.replay()
         return self.logits if n == self.B else self.logits[:n]
 
@@ -211,7 +222,7 @@ class StepRunner:
             a = arrays[k].reshape(-1)
             host[offsets[k]:offsets[k] + a.size] = a
         dev = torch.empty(total, dtype=torch.int32, device=self.device)
-        dev.copy_(self._staging[:total], non_blocking=True)
+        ops.ints_from_host(self._staging[:total], dev)
         self._mark_staged()
         return {k: dev[offsets[k]:offsets[k] + arrays[k].size].view(arrays[k].shape)
                 for k in order}
@@ -299,15 +310,22 @@ class StepRunner:
         return graph.run(self, caches, tokens, pos, slots, logit_rows)
 
     def decode_run(self, caches: Sequence[RequestCache], first_tokens: Sequence[int], n_steps: int,
-                   choose, out: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+                   choose, out: Optional[torch.Tensor] = None,
+                   placed=None) -> Optional[torch.Tensor]:
         """``n_steps`` decode steps of the same requests, queued back to back: the token a step
         chooses goes to the next step on the GPU, and the host does not wait in between.
         ``choose(logits, step, out_row)`` queues the kernels that write one token per request
         (int32) into ``out_row``.  Returns the tokens [n_steps, B] on the GPU (not yet waited
         for), or None when the run cannot be made this way (no captured graph for the shape
         yet, not enough pages for all the steps): then nothing has changed.  After the run
-        every cache holds ``n_steps`` more tokens."""
+        every cache holds ``n_steps`` more tokens.  ``placed`` = (int32 tensor on the GPU, [(request,
+        place), ...]): the first token of these requests is the one at that place of the tensor
+        (chosen by kernels that are queued already), not the one in ``first_tokens``."""
         B = len(caches)
+        if placed is not None:
+            for row, at in placed[1]:
+                if not (0 <= row < B and 0 <= at < placed[0].numel()):
+                    raise ValueError(f"placed token: request {row} or place {at} does not exist")
         if not self.decode_graphs or B == 0 or n_steps < 1 or n_steps > DECODE_RING:
             return None
         if len({id(c) for c in caches}) != B:
@@ -329,7 +347,8 @@ class StepRunner:
                 self.cache.extend_one(c)
             pos = np.fromiter((c.length for c in caches), dtype=np.int32, count=B)
             logits = graph.run(self, caches, tokens, pos, slots, rows,
-                               device_tokens=None if s == 0 else out[s - 1])
+                               device_tokens=None if s == 0 else out[s - 1],
+                               placed=placed if s == 0 else None)
             for c in caches:
                 self.cache.commit_one(c)
             choose(logits, s, out[s])

@@ -96,6 +96,36 @@ def place_tokens(tokens: torch.Tensor, dst_rows: torch.Tensor, chosen: torch.Ten
         _stream()), "place_tokens")
 
 
+def tokens_to_host(src: torch.Tensor, dst: torch.Tensor) -> None:
+    """The int32 values of ``src`` (on the GPU) into ``dst``, pinned host memory of at least as
+    many, written by a kernel: they are there once an event recorded behind this call has
+    happened.  Unlike a copy command towards the host, this does not make the host wait when it
+    queues the next copy towards the GPU."""
+    _gpu("src", src, I32)
+    _need(isinstance(dst, torch.Tensor) and not dst.is_cuda and dst.is_pinned()
+          and dst.dtype is I32 and dst.is_contiguous(),
+          "tokens_to_host: dst must be contiguous pinned host memory of int32")
+    n = src.numel()
+    _need(dst.numel() >= n, lambda: f"tokens_to_host: {n} values for {dst.numel()} places")
+    check(library("elementwise").kappai_copy_ints(
+        ctypes.c_void_p(dst.data_ptr()), _ptr(src), _c_int(n), _stream()), "tokens_to_host")
+
+
+def ints_from_host(src: torch.Tensor, dst: torch.Tensor) -> None:
+    """The int32 values of ``src`` (pinned host memory, written by the host before this call)
+    into ``dst`` on the GPU, read by a kernel: the tables of a step go this way, so that a step
+    is kernels only and the host never waits inside a copy command while steps are queued
+    ahead."""
+    _gpu("dst", dst, I32)
+    _need(isinstance(src, torch.Tensor) and not src.is_cuda and src.is_pinned()
+          and src.dtype is I32 and src.is_contiguous(),
+          "ints_from_host: src must be contiguous pinned host memory of int32")
+    n = src.numel()
+    _need(dst.numel() >= n, lambda: f"ints_from_host: {n} values for {dst.numel()} places")
+    check(library("elementwise").kappai_copy_ints(
+        _ptr(dst), ctypes.c_void_p(src.data_ptr()), _c_int(n), _stream()), "ints_from_host")
+
+
 def add_rmsnorm(resid: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Tensor,
                 eps: float, out_dtype, rows: Optional[torch.Tensor] = None,
                 write_resid: bool = True, fragment: bool = False):

@@ -105,7 +105,7 @@ class Sampler:
                                                 pin_memory=True)
         buf.numpy()[:packed.size] = packed
         d = torch.empty(packed.size, dtype=torch.float32, device=dev)
-        d.copy_(buf[:packed.size], non_blocking=True)
+        ops.ints_from_host(buf[:packed.size].view(torch.int32), d.view(torch.int32))
         ev = self._pinned_done[i] = torch.cuda.Event()
         ev.record()
         return d
