@@ -345,17 +345,23 @@ static void launch_tile_cfg(const bf16_t* A, const bf16_t* W, const float* bias,
 
 template <int N> struct IntC { static constexpr int value = N; };
 
-template <typename TO, int EPI, int WT, bool DEEP = false>
+template <typename TO, int EPI, int WT, bool DEEP = false, int WN_ = 0>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4 / WT, 4 / WT)))
 void gemm_bf16_block256_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W,
                                const float* __restrict__ bias, TO* __restrict__ C, int M, int N,
                                int K, int lda, int ldc, int tiles_n) {
-  // WT x WT accumulator tiles of 32 x 32 a wave: 4 -> 256 x 256 blocks, 2 -> 128 x 128
-  static_assert(!DEEP || WT == 2, "four LDS buffers: the 128 x 128 form only");
-  constexpr int BM = WT * 64, BN = WT * 64, BK = 64;
-  constexpr int WROWS = WT * 32;                               // rows (columns) of a wave's tile
-  constexpr int NPROD = WT * WT, NREAD = 2 * WT;               // per 16 of K
-  constexpr int NLOAD = 4 * WT, HALF = NLOAD / 2;              // load instructions a wave and tile
+  // WTM x WTN accumulator tiles of 32 x 32 a wave (WTN = WT unless WN_ is given): 4 x 4 ->
+  // 256 x 256 blocks, 2 x 2 -> 128 x 128, 4 x 3 -> 256 rows x 192 columns (for a product whose
+  // 256 x 256 blocks would leave a quarter of the chip without one)
+  constexpr int WTM = WT, WTN = WN_ ? WN_ : WT;
+  static_assert(!DEEP || (WTM == 2 && WTN == 2), "four LDS buffers: the 128 x 128 form only");
+  static_assert(WTN <= WTM && 2 * WTN >= WTM, "the load slots are laid out for the rows' side");
+  constexpr int BM = WTM * 64, BN = WTN * 64, BK = 64;
+  constexpr int WROWS_M = WTM * 32, WROWS_N = WTN * 32;        // rows, columns of a wave's tile
+  constexpr int NPROD = WTM * WTN, NREAD = WTM + WTN;          // per 16 of K
+  // load instructions a wave and tile: the waves that bring A issue NLOAD, those that bring W
+  // the first NLOAD_W of the same slots
+  constexpr int NLOAD = 4 * WTM, NLOAD_W = 4 * WTN, HALF = NLOAD / 2;
   constexpr int A_TILE = BM * BK, BUF = (BM + BN) * BK;        // in bf16
   extern __shared__ __attribute__((aligned(1024))) bf16_t lds[];
   const int tid = threadIdx.x, lane = tid % WAVE;
@@ -367,11 +373,11 @@ void gemm_bf16_block256_kernel(const bf16_t* __restrict__ A, const bf16_t* __res
   const int nk = kblk / BK;
   C += (size_t)blockIdx.y * M * ldc;
 
-  f32x16_t acc[WT][WT];
+  f32x16_t acc[WTM][WTN];
 #pragma unroll
-  for (int i = 0; i < WT; ++i)
+  for (int i = 0; i < WTM; ++i)
 #pragma unroll
-    for (int j = 0; j < WT; ++j)
+    for (int j = 0; j < WTN; ++j)
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
@@ -384,7 +390,9 @@ void gemm_bf16_block256_kernel(const bf16_t* __restrict__ A, const bf16_t* __res
                    (size_t)blockIdx.y * kblk * sizeof(bf16_t);
   const int ld = brings_a ? lda : K;
   const int last_row = (brings_a ? M : N) - 1;
-  const int row0 = brings_a ? m0 + wave * WROWS : n0 + (wave - 2) * WROWS;
+  const int row0 = brings_a ? m0 + wave * WROWS_M : n0 + (wave - 2) * WROWS_N;
+  const int lds_row0 = brings_a ? wave * WROWS_M : BM + (wave - 2) * WROWS_N;   // in the buffer
+  const int my_loads = brings_a ? NLOAD : NLOAD_W;
   const int lrow = lane / 8;
   uint32_t roff[NLOAD];
 #pragma unroll
@@ -403,8 +411,9 @@ void gemm_bf16_block256_kernel(const bf16_t* __restrict__ A, const bf16_t* __res
     return reinterpret_cast<const char*>(((uint64_t)hi << 32) | lo);
   };
   auto load_one = [&](int buf, const char* base, int i) {
+    if (NLOAD_W < NLOAD && i >= my_loads) return;       // (uniform over the wave)
     __builtin_amdgcn_global_load_lds(KAPPAI_GPTR(base + roff[i]),
-                                     KAPPAI_LPTR(lds + buf * BUF + (wave * NLOAD + i) * 8 * BK), 16,
+                                     KAPPAI_LPTR(lds + buf * BUF + (lds_row0 + i * 8) * BK), 16,
                                      0, 0);
   };
   // fragments of the 16 of K number s: chunks 2s and 2s+1; lane -> (row lane%32, chunk 2s+lane/32)
@@ -412,14 +421,14 @@ void gemm_bf16_block256_kernel(const bf16_t* __restrict__ A, const bf16_t* __res
   int aoff[4], woff[4];
 #pragma unroll
   for (int s = 0; s < 4; ++s) {
-    aoff[s] = (wm * WROWS + r_in) * BK + (((s * 2 + hh) ^ ((r_in >> 1) & 7)) * 8);
-    woff[s] = A_TILE + (wn * WROWS + r_in) * BK + (((s * 2 + hh) ^ ((r_in >> 1) & 7)) * 8);
+    aoff[s] = (wm * WROWS_M + r_in) * BK + (((s * 2 + hh) ^ ((r_in >> 1) & 7)) * 8);
+    woff[s] = A_TILE + (wn * WROWS_N + r_in) * BK + (((s * 2 + hh) ^ ((r_in >> 1) & 7)) * 8);
   }
-  bf16x8_t fa[2][WT], fw[2][WT];
+  bf16x8_t fa[2][WTM], fw[2][WTN];
   // in the order the products ask for them: w0 a0, the other w, the other a
   auto read_one = [&](int fb, int buf, int s, int idx) {
-    const bool is_w = idx == 0 || (idx >= 2 && idx <= WT);
-    const int n = idx <= 1 ? 0 : idx <= WT ? idx - 1 : idx - WT;
+    const bool is_w = idx == 0 || (idx >= 2 && idx <= WTN);
+    const int n = idx <= 1 ? 0 : idx <= WTN ? idx - 1 : idx - WTN;
     if (is_w)
       fw[fb][n] = as_bf16x8(
           *reinterpret_cast<const u32x4_t*>(lds + buf * BUF + woff[s] + n * 32 * BK));
@@ -428,7 +437,7 @@ void gemm_bf16_block256_kernel(const bf16_t* __restrict__ A, const bf16_t* __res
           *reinterpret_cast<const u32x4_t*>(lds + buf * BUF + aoff[s] + n * 32 * BK));
   };
   auto product = [&](int fb, int t) {
-    const int i = t / WT, j = t % WT;
+    const int i = t / WTN, j = t % WTN;
     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fw[fb][j], fa[fb][i], acc[i][j], 0, 0, 0);
   };
   // One tile of K out of buffer U.  next: there is a tile kt+1 (its second half is loaded
@@ -450,7 +459,7 @@ void gemm_bf16_block256_kernel(const bf16_t* __restrict__ A, const bf16_t* __res
     }
     // the last 16 of K: a few products first, so that the matrix cores have work while the
     // wave waits at the barrier
-    constexpr int PRE = WT == 4 ? 4 : 1;
+    constexpr int PRE = WTM == 4 ? 4 : 1;
     constexpr int REST = NPROD - PRE;
     constexpr int SPREAD = REST < 8 ? REST : 8;         // slots that also read and load
     constexpr int READS_PER = (NREAD + SPREAD - 1) / SPREAD;
@@ -489,11 +498,11 @@ void gemm_bf16_block256_kernel(const bf16_t* __restrict__ A, const bf16_t* __res
     auto load_deep = [&](int kt, const char* base, int i) {
       __builtin_amdgcn_global_load_lds(
           KAPPAI_GPTR(base + roff[i]),
-          KAPPAI_LPTR(lds + (kt & 3) * BUF + (wave * NLOAD + i) * 8 * BK), 16, 0, 0);
+          KAPPAI_LPTR(lds + (kt & 3) * BUF + (lds_row0 + i * 8) * BK), 16, 0, 0);
     };
     auto read_deep = [&](int fb, const bf16_t* buf, int s, int idx) {
-      const bool is_w = idx == 0 || (idx >= 2 && idx <= WT);
-      const int n = idx <= 1 ? 0 : idx <= WT ? idx - 1 : idx - WT;
+      const bool is_w = idx == 0 || (idx >= 2 && idx <= WTN);
+      const int n = idx <= 1 ? 0 : idx <= WTN ? idx - 1 : idx - WTN;
       if (is_w)
         fw[fb][n] = as_bf16x8(*reinterpret_cast<const u32x4_t*>(buf + woff[s] + n * 32 * BK));
       else
@@ -583,16 +592,16 @@ void gemm_bf16_block256_kernel(const bf16_t* __restrict__ A, const bf16_t* __res
   // Epilogue: a wave turns 32 rows of its tile at a time through its own piece of LDS.
   // acc[i][j][4g + e] is C[row (wm*WT+i)*32 + lane%32][column (wn*WT+j)*32 + 8g + 4*(lane/32) + e].
   __syncthreads();                               // everybody is done with the last tile
-  constexpr int OUT_COLS = EPI == 1 ? WROWS / 2 : WROWS;   // columns a wave writes
+  constexpr int OUT_COLS = EPI == 1 ? WROWS_N / 2 : WROWS_N;   // columns a wave writes
   constexpr int ROW_BYTES = OUT_COLS * (int)sizeof(TO) + 16;
   char* mine = reinterpret_cast<char*>(lds) + wave * 32 * ROW_BYTES;
   const int out_n = EPI == 1 ? N / 2 : N;
-  const int col0 = EPI == 1 ? (n0 + wn * WROWS) / 2 : n0 + wn * WROWS;
+  const int col0 = EPI == 1 ? (n0 + wn * WROWS_N) / 2 : n0 + wn * WROWS_N;
 #pragma unroll
-  for (int i = 0; i < WT; ++i) {
+  for (int i = 0; i < WTM; ++i) {
     char* wrow = mine + r_in * ROW_BYTES;
 #pragma unroll
-    for (int j = 0; j < WT; ++j) {
+    for (int j = 0; j < WTN; ++j) {
 #pragma unroll
       for (int g = 0; g < (EPI == 1 ? 2 : 4); ++g) {
         float v4[4];
@@ -623,13 +632,15 @@ void gemm_bf16_block256_kernel(const bf16_t* __restrict__ A, const bf16_t* __res
     }
     // rows back out, 16 bytes a lane
     constexpr int CHUNKS = OUT_COLS * (int)sizeof(TO) / 16;   // per row
-    constexpr int ROWS_PER = WAVE / CHUNKS;
+    constexpr int ROWS_PER = WAVE / CHUNKS;                   // (lanes left over sit out)
     constexpr int PER = 16 / (int)sizeof(TO);                 // columns a chunk
+    constexpr bool EVEN = WAVE % CHUNKS == 0 && 32 % ROWS_PER == 0;
 #pragma unroll
-    for (int it = 0; it < 32 / ROWS_PER; ++it) {
+    for (int it = 0; it < (32 + ROWS_PER - 1) / ROWS_PER; ++it) {
       const int rr = it * ROWS_PER + lane / CHUNKS, ch = lane % CHUNKS;
+      if (!EVEN && (lane >= ROWS_PER * CHUNKS || rr >= 32)) continue;
       const u32x4_t v = *reinterpret_cast<const u32x4_t*>(mine + rr * ROW_BYTES + ch * 16);
-      const int gm = m0 + (wm * WT + i) * 32 + rr, gn = col0 + ch * PER;
+      const int gm = m0 + (wm * WTM + i) * 32 + rr, gn = col0 + ch * PER;
       if (gm < M && gn < out_n) *reinterpret_cast<u32x4_t*>(C + (size_t)gm * ldc + gn) = v;
     }
   }
@@ -644,20 +655,20 @@ static bool block256_fits(const bf16_t* A, const bf16_t* W, TO* C, int M, int n_
          (long long)M * lda < limit && (long long)n_rows_w * K < limit;
 }
 
-template <typename TO, int EPI, int WT, bool DEEP = false>
+template <typename TO, int EPI, int WT, bool DEEP = false, int WN_ = 0>
 static void launch_block256(const bf16_t* A, const bf16_t* W, const float* bias, TO* C, int M,
                             int n_rows_w, int K, int lda, int ldc, int ksplit,
                             hipStream_t stream) {
-  constexpr int B = WT * 64;                     // block edge
-  constexpr size_t lds_bytes = (DEEP ? 4 : 2) * (B + B) * 64 * sizeof(bf16_t);
-  auto kern = gemm_bf16_block256_kernel<TO, EPI, WT, DEEP>;
+  constexpr int B = WT * 64, BN = (WN_ ? WN_ : WT) * 64;       // block: B rows x BN columns
+  constexpr size_t lds_bytes = (DEEP ? 4 : 2) * (B + BN) * 64 * sizeof(bf16_t);
+  auto kern = gemm_bf16_block256_kernel<TO, EPI, WT, DEEP, WN_>;
   static bool attr_set = false;
   if (!attr_set) {
     (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
                               (int)lds_bytes);
     attr_set = true;
   }
-  const int tn = (n_rows_w + B - 1) / B, tm = (M + B - 1) / B;
+  const int tn = (n_rows_w + BN - 1) / BN, tm = (M + B - 1) / B;
   hipLaunchKernelGGL(kern, dim3(tm * tn, ksplit), dim3(256), lds_bytes, stream, A, W, bias, C, M,
                      n_rows_w, K, lda, ldc, tn);
 }
@@ -676,7 +687,7 @@ static bool use_256_form(long blocks256) {
 // of K, two LDS buffers), 3 = 256x128 blocks (tiles of 64 of K, one LDS buffer), 4 = 256x256
 // blocks of the same kernel (tiles of 64 of K), 5 = the 256x256 kernel with one wave a SIMD, 6 = its
 // 128x128 form (when the sizes fit them, else 3), 8 = the 128x128 form with four LDS buffers, one
-// block a CU
+// block a CU, 9 = the one-wave-a-SIMD kernel with blocks of 256 rows x 192 columns
 template <typename TO, int EPI>
 static void launch_tile(const bf16_t* A, const bf16_t* W, const float* bias, TO* C, int M,
                         int n_rows_w, int K, int lda, int ldc, int ksplit, int shape,
@@ -692,8 +703,19 @@ static void launch_tile(const bf16_t* A, const bf16_t* W, const float* bias, TO*
     const long blocks128 = (long)((M + 127) / 128) * ((n_rows_w + 127) / 128) * ksplit;
     const bool deep = blocks128 <= 256 && K / ksplit >= 2048;
     shape = !fits ? (big >= 128 ? 3 : 1) : use_256_form(blocks256) ? 5 : deep ? 8 : 6;
+    if (fits && EPI == 0) {
+      // blocks of 256 rows x 192 columns when they fill their rounds and come to fewer rounds'
+      // worth of work than 256 x 256 (in_proj of 2048 rows: 192 blocks of 256 x 256 leave 64 CUs
+      // idle, 256 blocks of 256 x 192 none: 49 against 55 us), or where 256 x 256 blocks would
+      // not fill theirs (6144 columns at 4096 rows: 94 against 106 us in 128 x 128 blocks)
+      const long blocks192 = (long)((M + 255) / 256) * ((n_rows_w + 191) / 192) * ksplit;
+      const long r256 = (blocks256 + 255) / 256, r192 = (blocks192 + 255) / 256;
+      if (use_256_form(blocks192) && (shape != 5 || r192 * (192 + 16) < r256 * (256 + 16)))
+        shape = 9;
+    }
   }
-  if ((shape == 5 || shape == 6 || shape == 8) && !fits) shape = 3;
+  if ((shape == 5 || shape == 6 || shape == 8 || shape == 9) && !fits) shape = 3;
+  if (shape == 9 && EPI != 0) shape = 5;
   switch (shape) {
     case 5:
       if constexpr (EPI != 2)
@@ -706,6 +728,11 @@ static void launch_tile(const bf16_t* A, const bf16_t* W, const float* bias, TO*
     case 8:
       if constexpr (EPI != 2)
         launch_block256<TO, EPI, 2, true>(A, W, bias, C, M, n_rows_w, K, lda, ldc, ksplit, stream);
+      break;
+    case 9:
+      if constexpr (EPI == 0)
+        launch_block256<TO, EPI, 4, false, 3>(A, W, bias, C, M, n_rows_w, K, lda, ldc, ksplit,
+                                              stream);
       break;
     case 1:
       launch_tile_cfg<TO, EPI, 1, 2, 4, 2, 32, 2, 2>(A, W, bias, C, M, n_rows_w, K, lda, ldc, ksplit,
@@ -1519,7 +1546,7 @@ static int launch_bf16(const bf16_t* A, const bf16_t* W, const float* bias, TO* 
 // K, lda must be multiples of 8 and A, W 16-byte aligned (checked by the caller).
 // force_kernel: 0 = by M, 1 = tile kernel, 2 = skinny kernel (M <= 64 only), 3..8 = tile kernel
 // with block shape 1..6 (see launch_tile), 9 = shared-rows kernel (17 to 64 rows, K / ksplit a
-// multiple of 512), 10 = block shape 8; for tests and tuning.
+// multiple of 512), 10 = block shape 8, 11 = block shape 9; for tests and tuning.
 // ksplit > 1 (float output only): C is [ksplit][M][ldc] partial sums over K ranges.
 // W_frag: null, or W again in fragment order (K a multiple of 32, rows a multiple of 16).
 static bool frag_ok(const void* W_frag, int rows, int K) {

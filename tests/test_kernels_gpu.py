@@ -156,12 +156,13 @@ def test_linear_swiglu(ops, M, F, K):
 BLOCK256 = 7          # force_kernel: 256 x 256 blocks, one wave a SIMD
 BLOCK128 = 8          # the same kernel with 128 x 128 blocks
 BLOCK128_DEEP = 10    # 128 x 128 blocks with four LDS buffers (tiles 0-2 loaded ahead)
+BLOCK192 = 11         # blocks of 256 rows x 192 columns
 
 
 @pytest.mark.parametrize("M,N,K", [(256, 256, 128), (300, 520, 256), (129, 8, 128), (1000, 1096, 384),
                                    (2048, 2048, 2048), (513, 264, 1280)])
 @pytest.mark.parametrize("out_dtype", [F32, BF16])
-@pytest.mark.parametrize("block", [BLOCK256, BLOCK128, BLOCK128_DEEP])
+@pytest.mark.parametrize("block", [BLOCK256, BLOCK128, BLOCK128_DEEP, BLOCK192])
 def test_linear_block256(ops, M, N, K, out_dtype, block):
     """The large-product kernel at sizes that end inside its 256 x 256 blocks, with a row stride
     on the input, with bias, and against the other tiled kernel on the same data."""
