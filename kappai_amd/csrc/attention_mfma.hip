@@ -780,6 +780,99 @@ __global__ __launch_bounds__(8 * WAVE) void attn_prefill_shared_kernel(
 // keys whose loads a wave has in flight at once (their registers: keys * HEAD_DIM / 64)
 #define D_KPW (HEAD_DIM <= 64 ? 128 : (HEAD_DIM <= 128 ? 64 : 32))
 
+// The per-head RMSNorm, the rotation and the storing of a decoded row's own key and value, done in
+// the attention kernel's prologue instead of a kernel of their own (kappai: QK-norm, then RoPE,
+// then the cache write, src/models/lfm.c:36-44).  For head sizes that are multiples of 64, where
+// the rotation's partner d / 2 further lies in the same lane; rotate-half over the whole head.
+struct QkFuse {
+  int on;                   // 0: q is ready and the row's key and value are in the pools
+  int kv;                   // the row's own key and value come from the projection beside q (k of
+                            // kv head g at column (H + g) d, v at (H + G + g) d) and go to the pools
+  const float* q_norm_w;    // [d] or null
+  const float* k_norm_w;
+  float eps;
+  const float* cos_tab;     // [positions][d / 2], or null: no rotation
+  const float* sin_tab;
+  bf16_t* k_pool_w;         // the pools once more, to be written
+  bf16_t* vt_pool_w;
+};
+
+// What the prologue reads beside the projection, asked for before the first keys so that it has
+// arrived when they have: the lane's norm weights at d = 32 ks + 8 kg and, for the first half of
+// the head, the cosines and sines of its position.
+struct QkTables {
+  float wq[(HEAD_DIM + 31) / 32][8], wk[(HEAD_DIM + 31) / 32][8];
+  float cs[(HEAD_DIM + 63) / 64][8], sn[(HEAD_DIM + 63) / 64][8];
+};
+
+__device__ __forceinline__ void load8f(const float* __restrict__ p, float (&v)[8]) {
+  const float4 a = *reinterpret_cast<const float4*>(p), b = *reinterpret_cast<const float4*>(p + 4);
+  v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+}
+
+__device__ __forceinline__ void qk_load_tables(const QkFuse& qk, int pos, int kg, QkTables& tb) {
+  constexpr int KS = (HEAD_DIM + 31) / 32, HALF = HEAD_DIM / 2;
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) {
+    if (qk.q_norm_w != nullptr) load8f(qk.q_norm_w + 32 * ks + 8 * kg, tb.wq[ks]);
+    if (qk.k_norm_w != nullptr && qk.kv) load8f(qk.k_norm_w + 32 * ks + 8 * kg, tb.wk[ks]);
+  }
+  if (qk.cos_tab != nullptr) {
+#pragma unroll
+    for (int ks = 0; ks < KS / 2; ++ks) {
+      load8f(qk.cos_tab + (size_t)pos * HALF + 32 * ks + 8 * kg, tb.cs[ks]);
+      load8f(qk.sin_tab + (size_t)pos * HALF + 32 * ks + 8 * kg, tb.sn[ks]);
+    }
+  }
+}
+
+// raw[ks] = the lane's eight values at d = 32 ks + 8 kg of one head; returns them normalised over
+// the head (the four lanes kg = 0..3 with the same lane % 16 hold a head together), weighted
+// (w: the lane's weights, when has_w) and rotated (cs, sn, when rotate), rounded to bfloat16
+__device__ __forceinline__ void qk_norm_rotate(u32x4_t (&raw)[(HEAD_DIM + 31) / 32], bool has_w,
+                                               const float (&w)[(HEAD_DIM + 31) / 32][8], float eps,
+                                               bool rotate,
+                                               const float (&cs)[(HEAD_DIM + 63) / 64][8],
+                                               const float (&sn)[(HEAD_DIM + 63) / 64][8]) {
+  constexpr int KS = (HEAD_DIM + 31) / 32;
+  float x[KS][8];
+  float ss = 0.f;
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) {
+    const uint32_t r[4] = {raw[ks].x, raw[ks].y, raw[ks].z, raw[ks].w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      x[ks][2 * i] = __uint_as_float(r[i] << 16);
+      x[ks][2 * i + 1] = __uint_as_float(r[i] & 0xffff0000u);
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) ss = fmaf(x[ks][i], x[ks][i], ss);
+  }
+  ss += __shfl_xor(ss, 16, WAVE);
+  ss += other_half(ss);
+  if (has_w) {
+    const float sc = 1.0f / sqrtf(ss / (float)HEAD_DIM + eps);
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+      for (int i = 0; i < 8; ++i) x[ks][i] = x[ks][i] * sc * w[ks][i];
+  }
+  if (rotate) {
+#pragma unroll
+    for (int ks = 0; ks < KS / 2; ++ks)
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const float lo = x[ks][i], hi = x[ks + KS / 2][i];
+        x[ks][i] = lo * cs[ks][i] - hi * sn[ks][i];
+        x[ks + KS / 2][i] = lo * sn[ks][i] + hi * cs[ks][i];
+      }
+  }
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks)
+    raw[ks] = (u32x4_t){pack_bf16(x[ks][0], x[ks][1]), pack_bf16(x[ks][2], x[ks][3]),
+                        pack_bf16(x[ks][4], x[ks][5]), pack_bf16(x[ks][6], x[ks][7])};
+}
+
 // One wave's share of a row's attention: the query heads of kv head g (columns) against the keys
 // of the chunks c0 = first, first + stride, ... below k_end (D_KPW keys each), with a running
 // maximum and sum per column.  Leaves the unnormalised output in o (lane: column lane % 16, d
@@ -788,23 +881,54 @@ __device__ __forceinline__ void attn_decode_wave(
     const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ k_pool,
     const bf16_t* __restrict__ vt_pool, const int* __restrict__ bt, int max_blocks, int t, int g,
     int H, int G, int ps, float scale, int lo, int hi, int first, int stride, int k_end,
-    f32x4_t (&o)[D_MT], float& m_run, float& l_run) {
+    f32x4_t (&o)[D_MT], float& m_run, float& l_run, const QkFuse& qk, int pos) {
   const int lane = threadIdx.x % WAVE;
   const int rep = H / G;
   const int col = lane % 16, kg = lane / 16;
   const bool head_ok = col < rep;
   const int h = g * rep + (head_ok ? col : 0);
   bf16x8_t qf[D_KS];
+  u32x4_t qraw[D_KS];
+  u32x4_t k_new[D_KS];                 // the row's own key, in the K fragment's order of d
+  uint32_t v_new[D_MT];                // its value at d = 16 mt + col
+  QkTables tb;
+  const bool fused = HEAD_DIM % 64 == 0 && qk.on;
+  const bool own_kv = fused && qk.kv;
   {
-    const bf16_t* qr = q + (size_t)t * q_stride + (size_t)h * HEAD_DIM;
+    const bf16_t* row = q + (size_t)t * q_stride;
+    const bf16_t* qr = row + (size_t)h * HEAD_DIM;
 #pragma unroll
     for (int ks = 0; ks < D_KS; ++ks) {
       u32x4_t v = {0u, 0u, 0u, 0u};
       const int d0 = 32 * ks + 8 * kg;
       if (head_ok && d0 < HEAD_DIM) v = *reinterpret_cast<const u32x4_t*>(qr + d0);
-      qf[ks] = as_frag(v);
+      qraw[ks] = v;
+    }
+    if constexpr (HEAD_DIM % 64 == 0) {
+      if (fused) {
+        // everything the prologue needs is asked for here; it is worked on when the first keys
+        // have been asked for as well
+        if (own_kv) {
+          const bf16_t* kr = row + (size_t)(H + g) * HEAD_DIM;
+          const bf16_t* vr = row + (size_t)(H + G + g) * HEAD_DIM;
+#pragma unroll
+          for (int ks = 0; ks < D_KS; ++ks)
+            k_new[ks] = *reinterpret_cast<const u32x4_t*>(kr + 32 * ks + 8 * kg);
+#pragma unroll
+          for (int mt = 0; mt < D_MT; ++mt) v_new[mt] = vr[16 * mt + col];
+        }
+        qk_load_tables(qk, pos, kg, tb);
+      }
+    }
+    if (!fused) {
+#pragma unroll
+      for (int ks = 0; ks < D_KS; ++ks) qf[ks] = as_frag(qraw[ks]);
     }
   }
+  bool prologue_due = fused;
+  // the wave whose chunks hold the row's own position puts its key and value into the pools
+  const bool owner = own_kv && pos >= first && pos < k_end &&
+                     ((pos - first) / D_KPW) % (stride / D_KPW) == 0;
 #pragma unroll
   for (int mt = 0; mt < D_MT; ++mt) o[mt] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
   m_run = -INFINITY;
@@ -841,6 +965,60 @@ __device__ __forceinline__ void attn_decode_wave(
 #pragma unroll
       for (int mt = 0; mt < D_MT; ++mt)
         vv[c][mt] = load_vt8_pg(vt_pool, pv, G, g, ps, 16 * mt + col, kb + 8 * kg, lo, hi);
+    }
+    if constexpr (HEAD_DIM % 64 == 0) {
+      if (prologue_due) {
+        prologue_due = false;
+        if (own_kv) qk_norm_rotate(k_new, qk.k_norm_w != nullptr, tb.wk, qk.eps,
+                                   qk.cos_tab != nullptr, tb.cs, tb.sn);
+        qk_norm_rotate(qraw, qk.q_norm_w != nullptr, tb.wq, qk.eps, qk.cos_tab != nullptr, tb.cs,
+                       tb.sn);
+#pragma unroll
+        for (int ks = 0; ks < D_KS; ++ks)
+          qf[ks] = as_frag(head_ok ? qraw[ks] : (u32x4_t){0u, 0u, 0u, 0u});
+        if (owner) {
+          const size_t pg = (size_t)bt[pos / ps] * G + g;
+          if (col == 0) {
+#pragma unroll
+            for (int ks = 0; ks < D_KS; ++ks)
+              *reinterpret_cast<u32x4_t*>(qk.k_pool_w + (pg * ps + pos % ps) * HEAD_DIM + 32 * ks +
+                                          8 * kg) = k_new[ks];
+          }
+          if (kg == 0) {
+#pragma unroll
+            for (int mt = 0; mt < D_MT; ++mt)
+              qk.vt_pool_w[(pg * HEAD_DIM + 16 * mt + col) * ps + pos % ps] = (bf16_t)v_new[mt];
+          }
+        }
+      }
+    }
+    if (own_kv && pos >= c0 && pos < c0 + D_KPW) {
+      // the pools do not hold the row's own key and value yet (or only just): they are taken
+      // from the registers
+#pragma unroll
+      for (int c = 0; c < NCH; ++c) {
+        const int kb = c0 + 32 * c;
+#pragma unroll
+        for (int tt = 0; tt < 2; ++tt) {
+          if (kb + 8 * (col / 4) + 4 * tt + col % 4 == pos) {
+#pragma unroll
+            for (int ks = 0; ks < D_KS; ++ks) kf[c][tt][ks] = k_new[ks];
+          }
+        }
+        const int e = pos - (kb + 8 * kg);
+        if (e >= 0 && e < 8) {
+          const uint32_t keep = (e & 1) ? 0x0000ffffu : 0xffff0000u;
+#pragma unroll
+          for (int mt = 0; mt < D_MT; ++mt) {
+            const uint32_t put = (v_new[mt] & 0xffffu) << ((e & 1) * 16);
+            uint32_t w[4] = {vv[c][mt].x, vv[c][mt].y, vv[c][mt].z, vv[c][mt].w};
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+              if (i == e / 2) w[i] = (w[i] & keep) | put;
+            vv[c][mt] = (u32x4_t){w[0], w[1], w[2], w[3]};
+          }
+        }
+      }
     }
 #pragma unroll
     for (int c = 0; c < NCH; ++c) {
@@ -902,7 +1080,7 @@ __global__ __launch_bounds__(64) void attn_decode_kernel(
     const bf16_t* __restrict__ vt_pool, float* __restrict__ part_o, float* __restrict__ part_ml,
     const int* __restrict__ row_pos, const int* __restrict__ row_seg,
     const int* __restrict__ block_tables, int max_blocks, int H, int G, int ps, int window,
-    float scale, int keys_per_split, int n_splits) {
+    float scale, int keys_per_split, int n_splits, QkFuse qk) {
   const int t = blockIdx.x, g = blockIdx.y, split = blockIdx.z, lane = threadIdx.x;
   const int rep = H / G;
   const int col = lane % 16, kg = lane / 16;
@@ -917,7 +1095,7 @@ __global__ __launch_bounds__(64) void attn_decode_kernel(
   f32x4_t o[D_MT];
   float m_run, l_run;
   attn_decode_wave(q, q_stride, k_pool, vt_pool, bt, max_blocks, t, g, H, G, ps, scale, lo,
-                   k_end - 1, k_begin, D_KPW, k_end, o, m_run, l_run);
+                   k_end - 1, k_begin, D_KPW, k_end, o, m_run, l_run, qk, pos);
   if (!head_ok) return;
   if (kg == 0) {
     part_ml[2 * pbase] = m_run;
@@ -943,7 +1121,7 @@ __global__ __launch_bounds__(D_BLOCK_MAX_WAVES * WAVE) void attn_decode_block_ke
     const bf16_t* __restrict__ vt_pool, bf16_t* __restrict__ out, int out_stride,
     const int* __restrict__ row_pos, const int* __restrict__ row_seg,
     const int* __restrict__ block_tables, int max_blocks, int H, int G, int ps, int window,
-    float scale) {
+    float scale, QkFuse qk) {
   extern __shared__ float sh_dec[];
   const int t = blockIdx.x, g = blockIdx.y;
   const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE, NW = blockDim.x / WAVE;
@@ -957,7 +1135,7 @@ __global__ __launch_bounds__(D_BLOCK_MAX_WAVES * WAVE) void attn_decode_block_ke
   f32x4_t o[D_MT];
   float m_run, l_run;
   attn_decode_wave(q, q_stride, k_pool, vt_pool, bt, max_blocks, t, g, H, G, ps, scale, lo, pos,
-                   k_begin + wave * D_KPW, NW * D_KPW, k_end, o, m_run, l_run);
+                   k_begin + wave * D_KPW, NW * D_KPW, k_end, o, m_run, l_run, qk, pos);
   float* sh_o = sh_dec;
   float* sh_m = sh_dec + (size_t)NW * rep * HEAD_DIM;
   float* sh_l = sh_m + NW * 16;
@@ -1058,14 +1236,11 @@ extern "C" int kappai_attn_decode_block_waves(int rep) {
   return nw >= 2 ? nw : 0;
 }
 
-// Decode attention with the keys of a row split over the `n_waves` waves of one block per (row, kv
-// head); no workspace, no second kernel.
-extern "C" int kappai_attn_decode_block(const void* q, int q_stride, const void* k_pool,
-                                        const void* vt_pool, void* out, int out_stride,
-                                        const int* row_pos, const int* row_seg,
-                                        const int* block_tables, int max_blocks, int T, int H,
-                                        int G, int ps, int window, float scale, int n_waves,
-                                        hipStream_t stream) {
+static int launch_decode_block(const void* q, int q_stride, const void* k_pool,
+                               const void* vt_pool, void* out, int out_stride, const int* row_pos,
+                               const int* row_seg, const int* block_tables, int max_blocks, int T,
+                               int H, int G, int ps, int window, float scale, int n_waves,
+                               const QkFuse& qk, hipStream_t stream) {
   if (T <= 0) return 0;
   if (ps % 16 || G < 1 || H % G || H / G > 16 || G > 65535 || (q_stride % 8) || n_waves < 1 ||
       n_waves > kappai_attn_decode_block_waves(H / G))
@@ -1075,8 +1250,56 @@ extern "C" int kappai_attn_decode_block(const void* q, int q_stride, const void*
   hipLaunchKernelGGL(attn_decode_block_kernel, dim3(T, G), dim3(n_waves * WAVE), lds, stream,
                      (const bf16_t*)q, q_stride, (const bf16_t*)k_pool, (const bf16_t*)vt_pool,
                      (bf16_t*)out, out_stride, row_pos, row_seg, block_tables, max_blocks, H, G, ps,
-                     window, scale);
+                     window, scale, qk);
   KAPPAI_RETURN_LAUNCH_STATUS();
+}
+
+// Decode attention with the keys of a row split over the `n_waves` waves of one block per (row, kv
+// head); no workspace, no second kernel.
+extern "C" int kappai_attn_decode_block(const void* q, int q_stride, const void* k_pool,
+                                        const void* vt_pool, void* out, int out_stride,
+                                        const int* row_pos, const int* row_seg,
+                                        const int* block_tables, int max_blocks, int T, int H,
+                                        int G, int ps, int window, float scale, int n_waves,
+                                        hipStream_t stream) {
+  return launch_decode_block(q, q_stride, k_pool, vt_pool, out, out_stride, row_pos, row_seg,
+                             block_tables, max_blocks, T, H, G, ps, window, scale, n_waves,
+                             QkFuse{}, stream);
+}
+
+// 1 when the decode kernels of this head size can do the per-head norm, the rotation and the
+// storing of the rows' own keys and values themselves (kappai_attn_decode_qk, _block_qk)
+extern "C" int kappai_attn_decode_takes_qk(void) { return HEAD_DIM % 64 == 0 ? 1 : 0; }
+
+// The arguments that the _qk entry points add: qkv [T, row_stride] is the projection as it comes
+// out of its product (q heads, then with store_kv the k heads and the v heads); q_norm_w /
+// k_norm_w [d] float or null; cos_tab / sin_tab [positions, d / 2] float (rotate-half over the
+// whole head) or both null; the pools are written at each row's own position when store_kv.
+static bool qk_args_ok(const void* qkv, int row_stride, const float* q_norm_w,
+                       const float* k_norm_w, const float* cos_tab, const float* sin_tab,
+                       const void* k_pool, const void* vt_pool) {
+  return HEAD_DIM % 64 == 0 && row_stride % 8 == 0 && ((uintptr_t)qkv % 16) == 0 &&
+         ((uintptr_t)q_norm_w % 16) == 0 && ((uintptr_t)k_norm_w % 16) == 0 &&
+         ((uintptr_t)cos_tab % 16) == 0 && ((uintptr_t)sin_tab % 16) == 0 &&
+         (cos_tab == nullptr) == (sin_tab == nullptr) && ((uintptr_t)k_pool % 16) == 0 &&
+         vt_pool != nullptr;
+}
+
+extern "C" int kappai_attn_decode_block_qk(const void* qkv, int row_stride, void* k_pool,
+                                           void* vt_pool, void* out, int out_stride,
+                                           const int* row_pos, const int* row_seg,
+                                           const int* block_tables, int max_blocks, int T, int H,
+                                           int G, int ps, int window, float scale, int n_waves,
+                                           const float* q_norm_w, const float* k_norm_w, float eps,
+                                           const float* cos_tab, const float* sin_tab,
+                                           int store_kv, hipStream_t stream) {
+  if (!qk_args_ok(qkv, row_stride, q_norm_w, k_norm_w, cos_tab, sin_tab, k_pool, vt_pool))
+    return (int)hipErrorInvalidValue;
+  const QkFuse qk{1, store_kv ? 1 : 0, q_norm_w, k_norm_w, eps, cos_tab, sin_tab, (bf16_t*)k_pool,
+                  (bf16_t*)vt_pool};
+  return launch_decode_block(qkv, row_stride, k_pool, vt_pool, out, out_stride, row_pos, row_seg,
+                             block_tables, max_blocks, T, H, G, ps, window, scale, n_waves, qk,
+                             stream);
 }
 
 extern "C" int kappai_attn_head_dim(void) { return HEAD_DIM; }
@@ -1113,12 +1336,11 @@ extern "C" int kappai_attn_prefill(const void* q, int q_stride, const void* k_po
   KAPPAI_RETURN_LAUNCH_STATUS();
 }
 
-extern "C" int kappai_attn_decode(const void* q, int q_stride, const void* k_pool,
-                                  const void* vt_pool, void* out, int out_stride, float* part_o,
-                                  float* part_ml, const int* row_pos, const int* row_seg,
-                                  const int* block_tables, int max_blocks, int T, int H, int G,
-                                  int ps, int window, float scale, int keys_per_split,
-                                  int n_splits, hipStream_t stream) {
+static int launch_decode(const void* q, int q_stride, const void* k_pool, const void* vt_pool,
+                         void* out, int out_stride, float* part_o, float* part_ml,
+                         const int* row_pos, const int* row_seg, const int* block_tables,
+                         int max_blocks, int T, int H, int G, int ps, int window, float scale,
+                         int keys_per_split, int n_splits, const QkFuse& qk, hipStream_t stream) {
   if (T <= 0) return 0;
   if (ps % 16 || G < 1 || H % G || H / G > 16 || G > 65535 || n_splits < 1 || n_splits > 65535 ||
       keys_per_split < D_KPW || keys_per_split % D_KPW || (q_stride % 8))
@@ -1126,11 +1348,43 @@ extern "C" int kappai_attn_decode(const void* q, int q_stride, const void* k_poo
   hipLaunchKernelGGL(attn_decode_kernel, dim3(T, G, n_splits), dim3(WAVE), 0, stream,
                      (const bf16_t*)q, q_stride, (const bf16_t*)k_pool, (const bf16_t*)vt_pool,
                      part_o, part_ml, row_pos, row_seg, block_tables, max_blocks, H, G, ps, window,
-                     scale, keys_per_split, n_splits);
+                     scale, keys_per_split, n_splits, qk);
   hipLaunchKernelGGL(attn_merge_kernel, dim3(T, H), dim3(MERGE_WAVES * WAVE), 0, stream,
                      (const float*)part_o, (const float*)part_ml, (bf16_t*)out, out_stride, H,
                      n_splits);
   KAPPAI_RETURN_LAUNCH_STATUS();
+}
+
+extern "C" int kappai_attn_decode(const void* q, int q_stride, const void* k_pool,
+                                  const void* vt_pool, void* out, int out_stride, float* part_o,
+                                  float* part_ml, const int* row_pos, const int* row_seg,
+                                  const int* block_tables, int max_blocks, int T, int H, int G,
+                                  int ps, int window, float scale, int keys_per_split,
+                                  int n_splits, hipStream_t stream) {
+  return launch_decode(q, q_stride, k_pool, vt_pool, out, out_stride, part_o, part_ml, row_pos,
+                       row_seg, block_tables, max_blocks, T, H, G, ps, window, scale,
+                       keys_per_split, n_splits, QkFuse{}, stream);
+}
+
+// kappai_attn_decode with the norm, the rotation and the store of the rows' own keys and values in
+// the kernel's prologue (see kappai_attn_decode_block_qk for the added arguments).  Every split of
+// a row must find the row's position inside the keys the splits cover: the caller's n_splits *
+// keys_per_split reach beyond the longest context, as for kappai_attn_decode.
+extern "C" int kappai_attn_decode_qk(const void* qkv, int row_stride, void* k_pool, void* vt_pool,
+                                     void* out, int out_stride, float* part_o, float* part_ml,
+                                     const int* row_pos, const int* row_seg,
+                                     const int* block_tables, int max_blocks, int T, int H, int G,
+                                     int ps, int window, float scale, int keys_per_split,
+                                     int n_splits, const float* q_norm_w, const float* k_norm_w,
+                                     float eps, const float* cos_tab, const float* sin_tab,
+                                     int store_kv, hipStream_t stream) {
+  if (!qk_args_ok(qkv, row_stride, q_norm_w, k_norm_w, cos_tab, sin_tab, k_pool, vt_pool))
+    return (int)hipErrorInvalidValue;
+  const QkFuse qk{1, store_kv ? 1 : 0, q_norm_w, k_norm_w, eps, cos_tab, sin_tab, (bf16_t*)k_pool,
+                  (bf16_t*)vt_pool};
+  return launch_decode(qkv, row_stride, k_pool, vt_pool, out, out_stride, part_o, part_ml, row_pos,
+                       row_seg, block_tables, max_blocks, T, H, G, ps, window, scale,
+                       keys_per_split, n_splits, qk, stream);
 }
 
 // ---------------------------------------------------------------------------------------

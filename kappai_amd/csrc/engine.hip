@@ -393,6 +393,16 @@ Carry conv_mixer(Ctx& c, const kappai_layer_call& L, Rows x, float* resid, const
                 &into, region);
 }
 
+// ops.decode_form: few keys go to the kernel that splits them over the waves of a block
+int decode_keys(const Ctx& c, const kappai_layer_call& L) {
+  int n_keys = c.b->max_position + 1;
+  if (L.window) n_keys = (n_keys < L.window ? n_keys : L.window) + 32;
+  return n_keys;
+}
+bool decode_block_form(const Ctx& c, const kappai_layer_call& L, int rep) {
+  return L.mfma->decode_block_waves(rep) > 0 && decode_keys(c, L) <= c.m->decode_block_max_keys;
+}
+
 // parts/attention.py with ops.qk_norm_rope_store and ops.paged_attention
 Carry attention_mixer(Ctx& c, const kappai_layer_call& L, Rows x, float* resid, const Into& into) {
   const kappai_kernels& k = *c.m->kernels;
@@ -424,10 +434,23 @@ Carry attention_mixer(Ctx& c, const kappai_layer_call& L, Rows x, float* resid, 
   const int* tables = b.block_tables[L.group];
   const int max_blocks = b.max_blocks[L.group];
   const int store = L.shared_cache ? 0 : 1;
+  const bool single = b.max_segment_rows == 1;
+  // decode: the attention kernels take the projection as it is and do norm, rotation and store
+  // themselves (parts/attention.py: _prologue_in_kernel)
+  const bool qk_in_kernel =
+      c.m->fused_qk && single && proj.kind == C_DELTA && !proj.is_f32 && L.mfma != nullptr &&
+      H / G <= 16 && qkv.n % 8 == 0 && aligned16(proj.data) && ps % 16 == 0 && d % 16 == 0 &&
+      d <= 256 && (L.rot_mode == 0 || (L.rot_mode == 1 && L.rot_dim == d)) &&
+      L.mfma->decode_takes_qk != nullptr && L.mfma->decode_takes_qk() &&
+      !decode_block_form(c, L, H / G);
   // q in place in the projection, or (from partial sums) a new bfloat16 [M, H d]
   void* q;
   int q_stride, q_bf16;
-  if (proj.kind == C_PARTS) {
+  if (qk_in_kernel) {
+    q_bf16 = 1;
+    q_stride = qkv.n;
+    q = proj.data;
+  } else if (proj.kind == C_PARTS) {
     q_bf16 = 1;
     q_stride = H * d;
     q = c.a->take(R_BLOCK, (size_t)M * H * d * 2);
@@ -447,17 +470,24 @@ Carry attention_mixer(Ctx& c, const kappai_layer_call& L, Rows x, float* resid, 
                                    0, nullptr, H * d, c.stream));
   }
   void* ctx = c.a->take(R_BLOCK, (size_t)M * H * d * elem(q_bf16));
-  const bool single = b.max_segment_rows == 1;
+  const float* cos_t = L.rot_mode ? L.cos_table : nullptr;
+  const float* sin_t = L.rot_mode ? L.sin_table : nullptr;
   const bool mfma_ok = q_bf16 && L.mfma != nullptr && ps % 16 == 0 && d % 16 == 0 && d <= 256 &&
                        q_stride % 8 == 0 && aligned16(q);
   if (mfma_ok && single && H / G <= 16) {
-    int n_keys = b.max_position + 1;
-    if (L.window) n_keys = (n_keys < L.window ? n_keys : L.window) + 32;
+    const int n_keys = decode_keys(c, L);
     const int block_waves = L.mfma->decode_block_waves(H / G);
-    if (block_waves > 0 && n_keys <= c.m->decode_block_max_keys) {
-      LAUNCH(c, L.mfma->attn_decode_block(q, q_stride, L.k_pool, L.v_pool, ctx, H * d, b.row_pos,
-                                          b.row_seg, tables, max_blocks, M, H, G, ps, L.window,
-                                          L.scale, block_waves, c.stream));
+    if (decode_block_form(c, L, H / G)) {
+      if (qk_in_kernel)
+        LAUNCH(c, L.mfma->attn_decode_block_qk(q, q_stride, L.k_pool, L.v_pool, ctx, H * d,
+                                               b.row_pos, b.row_seg, tables, max_blocks, M, H, G,
+                                               ps, L.window, L.scale, block_waves, L.q_norm_w,
+                                               L.k_norm_w, L.qk_eps, cos_t, sin_t, store,
+                                               c.stream));
+      else
+        LAUNCH(c, L.mfma->attn_decode_block(q, q_stride, L.k_pool, L.v_pool, ctx, H * d, b.row_pos,
+                                            b.row_seg, tables, max_blocks, M, H, G, ps, L.window,
+                                            L.scale, block_waves, c.stream));
     } else {
       const int kpw = L.mfma->keys_per_wave();
       int n_splits = c.m->decode_max_splits;
@@ -470,9 +500,16 @@ Carry attention_mixer(Ctx& c, const kappai_layer_call& L, Rows x, float* resid, 
       n_splits = (n_keys + keys_per_split - 1) / keys_per_split;
       float* part_o = (float*)c.a->take(R_BLOCK, (size_t)M * H * n_splits * d * 4);
       float* part_ml = (float*)c.a->take(R_BLOCK, (size_t)M * H * n_splits * 2 * 4);
-      LAUNCH(c, L.mfma->attn_decode(q, q_stride, L.k_pool, L.v_pool, ctx, H * d, part_o, part_ml,
-                                    b.row_pos, b.row_seg, tables, max_blocks, M, H, G, ps,
-                                    L.window, L.scale, keys_per_split, n_splits, c.stream));
+      if (qk_in_kernel)
+        LAUNCH(c, L.mfma->attn_decode_qk(q, q_stride, L.k_pool, L.v_pool, ctx, H * d, part_o,
+                                         part_ml, b.row_pos, b.row_seg, tables, max_blocks, M, H,
+                                         G, ps, L.window, L.scale, keys_per_split, n_splits,
+                                         L.q_norm_w, L.k_norm_w, L.qk_eps, cos_t, sin_t, store,
+                                         c.stream));
+      else
+        LAUNCH(c, L.mfma->attn_decode(q, q_stride, L.k_pool, L.v_pool, ctx, H * d, part_o, part_ml,
+                                      b.row_pos, b.row_seg, tables, max_blocks, M, H, G, ps,
+                                      L.window, L.scale, keys_per_split, n_splits, c.stream));
     }
   } else if (mfma_ok && b.q_tiles != nullptr) {
     LAUNCH(c, L.mfma->attn_prefill(q, q_stride, L.k_pool, L.v_pool, ctx, H * d, b.q_tiles,

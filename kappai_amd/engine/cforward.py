@@ -29,7 +29,7 @@ from ..parts.embedding import OutputHead, TokenEmbedding
 from ..parts.feed_forward import SwiGLU
 from ..parts.rotary import RotaryEncoding
 
-ENGINE_ABI = 3
+ENGINE_ABI = 4
 MAX_GROUPS = 8
 
 
@@ -45,7 +45,8 @@ class Kernels(Structure):
 
 class AttentionKernels(Structure):
     _fields_ = _ptrs(["keys_per_wave", "decode_block_waves", "attn_prefill", "attn_decode",
-                      "attn_decode_block"])
+                      "attn_decode_block", "decode_takes_qk", "attn_decode_qk",
+                      "attn_decode_block_qk"])
 
 
 class LinearDesc(Structure):
@@ -81,7 +82,7 @@ class ModelDesc(Structure):
         ("fused_step_narrow_rows", c_int), ("partial_sums_min_rows", c_int),
         ("fragment_rows_min", c_int), ("fragment_rows_from", c_int), ("fused_max_rows", c_int),
         ("decode_waves", c_int), ("decode_max_splits", c_int), ("decode_block_max_keys", c_int),
-        ("attention_tile_rows", c_int)]
+        ("attention_tile_rows", c_int), ("fused_qk", c_int)]
 
 
 class BatchDesc(Structure):
@@ -248,6 +249,7 @@ class CForward:
         m.decode_waves, m.decode_max_splits = ops.DECODE_WAVES, ops.DECODE_MAX_SPLITS
         m.decode_block_max_keys = ops.DECODE_BLOCK_MAX_KEYS
         m.attention_tile_rows = ops.ATTENTION_TILE_ROWS
+        m.fused_qk = 1 if tuning.FUSED_QK else 0
         self.desc = m
         self.workspace = Workspace()
 
@@ -260,6 +262,9 @@ class CForward:
             a.attn_prefill = _address(lib.kappai_attn_prefill)
             a.attn_decode = _address(lib.kappai_attn_decode)
             a.attn_decode_block = _address(lib.kappai_attn_decode_block)
+            a.decode_takes_qk = _address(lib.kappai_attn_decode_takes_qk)
+            a.attn_decode_qk = _address(lib.kappai_attn_decode_qk)
+            a.attn_decode_block_qk = _address(lib.kappai_attn_decode_block_qk)
             self._mfma[head_dim] = a
         return self._mfma[head_dim]
 

@@ -7,6 +7,7 @@ live on the GPU; nothing here computes on the CPU.
 from __future__ import annotations
 
 import ctypes
+from dataclasses import dataclass
 from typing import Optional
 
 import torch
@@ -724,12 +725,47 @@ def qk_norm_rope_store(qkv: torch.Tensor, n_heads: int, n_kv_heads: int, head_di
     return qkv if parts is None else q_out
 
 
+@dataclass
+class QkPrologue:
+    """What the decode attention kernels do themselves when they are given the projection as it
+    comes out of its product: per-head RMSNorm of q and k (weights [d] float32, or None), the
+    rotate-half rotation over the whole head (``cos`` / ``sin`` [positions, d / 2] float32, or
+    None for no rotation), and with ``store_kv`` the storing of each row's own key and value
+    (which then stand beside q in the projection: q heads, k heads, v heads)."""
+    q_norm_w: Optional[torch.Tensor]
+    k_norm_w: Optional[torch.Tensor]
+    eps: float
+    cos: Optional[torch.Tensor]
+    sin: Optional[torch.Tensor]
+    store_kv: bool = True
+
+
+def decode_form(n_heads: int, n_kv_heads: int, head_dim: int, max_position: int,
+                window: int = 0) -> str:
+    """Which of the two decode kernels a step takes: with few keys ("decode-block") a block per
+    (row, kv head) splits them over its waves and merges in LDS; else ("decode-split") the keys
+    are split over blocks, whose partial results a second kernel merges."""
+    n_keys = min(max_position + 1, window) + 32 if window else max_position + 1
+    lib = library("attention_mfma", HEAD_DIM=head_dim)
+    block_waves = lib.kappai_attn_decode_block_waves(n_heads // n_kv_heads)
+    return "decode-block" if block_waves and n_keys <= DECODE_BLOCK_MAX_KEYS else "decode-split"
+
+
+def decode_takes_qk(head_dim: int, page_size: int) -> bool:
+    """Whether the decode attention kernels of this head size take a ``QkPrologue`` (head sizes
+    that are multiples of 64, where a lane holds both halves of a rotation pair)."""
+    if head_dim % 16 or head_dim > 256 or page_size % 16:
+        return False
+    return bool(library("attention_mfma", HEAD_DIM=head_dim).kappai_attn_decode_takes_qk())
+
+
 def paged_attention(q: torch.Tensor, n_heads: int, n_kv_heads: int, head_dim: int,
                     k_pool: torch.Tensor, v_pool: torch.Tensor, row_pos: torch.Tensor,
                     row_seg: torch.Tensor, block_tables: torch.Tensor, page_size: int,
                     scale: float, window: int = 0, q_tiles: Optional[torch.Tensor] = None,
                     single_rows: bool = False, max_position: Optional[int] = None,
-                    kernel: str = "auto", prefill_variant: int = 0) -> torch.Tensor:
+                    kernel: str = "auto", prefill_variant: int = 0,
+                    qk: Optional[QkPrologue] = None) -> torch.Tensor:
     """Causal attention of every row over the keys of its request that are in the cache
     (its own included; the last ``window`` of them when a window is set).  ``q`` is
     [T, >= H d] with a row stride (the q columns of the fused projection).  Returns [T, H d].
@@ -742,7 +778,10 @@ def paged_attention(q: torch.Tensor, n_heads: int, n_kv_heads: int, head_dim: in
     kernel.  ``kernel`` = "rows" | "prefill" | "decode" | "decode-block" | "decode-split" forces
     one (for tests);
     ``prefill_variant`` 1 / 2 forces the tiled kernel's form (2: key tiles shared by four query
-    heads of a kv head through LDS; head sizes 64 and 128 only)."""
+    heads of a kv head through LDS; head sizes 64 and 128 only).
+
+    ``qk`` (decode kernels only, see ``decode_takes_qk``): ``q`` is the raw projection and the
+    kernel normalises and rotates q and the rows' own keys itself and stores keys and values."""
     H, G, d = n_heads, n_kv_heads, head_dim
     _gpu("q", q, (F32, BF16), contiguous=False)
     T = q.shape[0]
@@ -796,20 +835,37 @@ def paged_attention(q: torch.Tensor, n_heads: int, n_kv_heads: int, head_dim: in
           lambda: f"unknown attention kernel {kernel!r}")
     _need(H // G <= 16, "the decode kernel takes at most 16 query heads per kv head")
     _need(max_position is not None, "the decode kernel needs the batch's largest position")
+    qk_args = ()
+    if qk is not None:
+        _need(bool(lib.kappai_attn_decode_takes_qk()),
+              lambda: f"the decode kernels of head size {d} do not take the norm and the rotation")
+        _need(q.shape[1] >= (H + 2 * G) * d if qk.store_kv else True,
+              "paged_attention: keys and values to store must stand beside q in the projection")
+        for name, w in (("q_norm_w", qk.q_norm_w), ("k_norm_w", qk.k_norm_w)):
+            if w is not None:
+                _gpu(name, w, F32)
+                _need(w.shape == (d,), lambda: f"{name}: one weight for each of the {d} of a head")
+        _need((qk.cos is None) == (qk.sin is None), "cos and sin tables come together")
+        if qk.cos is not None:
+            _gpu("cos", qk.cos, F32)
+            _gpu("sin", qk.sin, F32)
+            _need(qk.cos.shape == qk.sin.shape and qk.cos.dim() == 2
+                  and qk.cos.shape[1] == d // 2 and qk.cos.shape[0] > max_position,
+                  lambda: f"rotation tables {tuple(qk.cos.shape)} for positions up to "
+                          f"{max_position} of heads of {d}")
+        qk_args = (_ptr(qk.q_norm_w), _ptr(qk.k_norm_w), _c_float(qk.eps), _ptr(qk.cos),
+                   _ptr(qk.sin), _c_int(1 if qk.store_kv else 0))
     n_keys = min(max_position + 1, window) + 32 if window else max_position + 1
-    # With few keys a block per (row, kv head) splits them over its waves and merges in LDS;
-    # else the keys are split over blocks, whose partial results a second kernel merges.
     block_waves = lib.kappai_attn_decode_block_waves(H // G)
     if kernel == "decode":
-        kernel = ("decode-block" if block_waves and n_keys <= DECODE_BLOCK_MAX_KEYS
-                  else "decode-split")
+        kernel = decode_form(H, G, d, max_position, window)
     if kernel == "decode-block":
         _need(block_waves > 0, "too many query heads a kv head for the block form")
-        check(lib.kappai_attn_decode_block(
+        check((lib.kappai_attn_decode_block_qk if qk is not None else lib.kappai_attn_decode_block)(
             _ptr(q), _c_int(q.stride(0)), _ptr(k_pool), _ptr(v_pool), _ptr(out), _c_int(H * d),
             _ptr(row_pos), _ptr(row_seg), _ptr(block_tables), _c_int(block_tables.shape[1]),
             _c_int(T), _c_int(H), _c_int(G), _c_int(page_size), _c_int(window or 0),
-            _c_float(scale), _c_int(block_waves), _stream()), "attn_decode_block")
+            _c_float(scale), _c_int(block_waves), *qk_args, _stream()), "attn_decode_block")
         return out
     # one wave keeps the loads of `kpw` keys in flight; splits are whole numbers of that, and
     # at most DECODE_MAX_SPLITS of them are merged
@@ -822,12 +878,12 @@ def paged_attention(q: torch.Tensor, n_heads: int, n_kv_heads: int, head_dim: in
     n_splits = (n_keys + keys_per_split - 1) // keys_per_split
     part_o = torch.empty((T, H, n_splits, d), dtype=F32, device=q.device)
     part_ml = torch.empty((T, H, n_splits, 2), dtype=F32, device=q.device)
-    check(lib.kappai_attn_decode(
+    check((lib.kappai_attn_decode_qk if qk is not None else lib.kappai_attn_decode)(
         _ptr(q), _c_int(q.stride(0)), _ptr(k_pool), _ptr(v_pool), _ptr(out), _c_int(H * d),
         _ptr(part_o), _ptr(part_ml), _ptr(row_pos), _ptr(row_seg), _ptr(block_tables),
         _c_int(block_tables.shape[1]), _c_int(T), _c_int(H), _c_int(G), _c_int(page_size),
         _c_int(window or 0), _c_float(scale), _c_int(keys_per_split), _c_int(n_splits),
-        _stream()), "attn_decode")
+        *qk_args, _stream()), "attn_decode")
     return out
 
 

@@ -85,6 +85,18 @@ class GroupedQueryAttention(Mixer):
         rot = self.position.rotation(x.device, batch.max_position) if self.position else None
         tables = batch.block_tables[cache.group]
         k_pool, v_pool = cache.pool("k"), cache.pool("v")
+        single = batch.max_segment_rows == 1
+        if self._prologue_in_kernel(proj, rot, single, cache.page_size, batch.max_position):
+            # decode: norm, rotation and store inside the attention kernel
+            with profile.scope("attn"):
+                ctx = ops.paged_attention(
+                    proj, H, G, d, k_pool, v_pool, batch.row_pos, batch.row_seg, tables,
+                    cache.page_size, self.scale, window=self.window or 0, single_rows=True,
+                    max_position=batch.max_position, kernel="decode",
+                    qk=ops.QkPrologue(self.q_norm_w, self.k_norm_w, self.qk_norm_eps or 0.0,
+                                      rot.cos if rot else None, rot.sin if rot else None,
+                                      store_kv=not shared_cache))
+            return self.out.forward(ctx, partial_sums=True, add_into=into)
         with profile.scope("rope_kvput"):
             q = ops.qk_norm_rope_store(
                 proj, H, G, d, self.q_norm_w, self.k_norm_w, self.qk_norm_eps or 0.0,
@@ -95,9 +107,28 @@ class GroupedQueryAttention(Mixer):
             ctx = ops.paged_attention(q, H, G, d, k_pool, v_pool, batch.row_pos,
                                       batch.row_seg, tables, cache.page_size, self.scale,
                                       window=self.window or 0, q_tiles=batch.q_tiles,
-                                      single_rows=batch.max_segment_rows == 1,
+                                      single_rows=single,
                                       max_position=batch.max_position)
         return self.out.forward(ctx, partial_sums=True, add_into=into)
+
+    def _prologue_in_kernel(self, proj, rot, single_rows: bool, page_size: int,
+                            max_position: int) -> bool:
+        """Whether the decode attention kernels take the projection as it is (see
+        ``ops.QkPrologue``): a step of single rows whose projection came as bfloat16 rows, few
+        enough query heads a kv head for the decode kernels, a head size they do it for, no
+        rotation or rotate-half over the whole head, and keys enough for the kernel that splits
+        them over blocks (where a block is one wave; in the other every wave of a block would do
+        the prologue again, which costs what the kernel saved)."""
+        if not (tuning.FUSED_QK and single_rows and isinstance(proj, torch.Tensor)
+                and proj.dim() == 2 and proj.dtype == torch.bfloat16 and proj.is_cuda
+                and self.H // self.G <= 16 and proj.stride(0) % 8 == 0
+                and proj.data_ptr() % 16 == 0):
+            return False
+        if rot is not None and not (rot.mode == ops.ROT_HALF and rot.rot_dim == self.d):
+            return False
+        return (ops.decode_takes_qk(self.d, page_size)
+                and ops.decode_form(self.H, self.G, self.d, max_position,
+                                    self.window or 0) == "decode-split")
 
     def weight_bytes(self) -> int:
         return self.qkv.weight_bytes() + self.out.weight_bytes() + 2 * self.d * 4

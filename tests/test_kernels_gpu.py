@@ -809,6 +809,75 @@ def test_store_and_attention(ops, dtype, case):
         close(got.float(), want, tol * 2, f"attention kernel {kernel}")
 
 
+QK_CASES = [
+    # H, G, d, page, tokens held, rotation, norm, window, store
+    (8, 2, 64, 16, [0, 1, 31, 32, 33, 500, 63, 64, 127, 128, 4095], True, True, 0, True),
+    (32, 8, 64, 16, [300, 4000], True, True, 0, True),
+    (8, 4, 128, 32, [5000, 0, 129, 1023, 1024, 77, 63, 64], True, True, 0, True),
+    (4, 4, 64, 64, [63, 64, 200], False, True, 0, True),           # no rotation
+    (6, 3, 64, 16, [15, 16, 700], True, False, 0, True),           # no norm
+    (4, 2, 64, 16, [90, 5, 450], True, True, 24, True),            # window
+    (16, 1, 256, 16, [300, 40, 0], True, True, 0, True),
+    (8, 2, 64, 16, [0, 40, 127, 128, 2000], True, True, 0, False),  # q only: keys are stored already
+]
+
+
+@pytest.mark.parametrize("case", QK_CASES)
+@pytest.mark.parametrize("kernel", ["decode-split", "decode-block"])
+def test_decode_attention_with_norm_rotation_and_store_inside(ops, case, kernel):
+    """The decode kernels given the raw projection (``ops.QkPrologue``) against the kernel that
+    normalises, rotates and stores followed by the same decode kernel: the same keys and values
+    in the same slots of the pools (nothing else touched), and the same attention, at positions
+    at the start of a page, at its end, at the edges of a wave's chunk of keys and far out."""
+    H, G, d, ps, before, rotate, norm, window, store = case
+    n = len(before)
+    c = paged_case(11, BF16, H, G, d, ps, before, [1] * n)
+    if not store:        # the layer whose keys are read has stored this step's already
+        for s, p in enumerate(before):
+            page = c["bt"][s, p // ps]
+            c["k_pool"][page, :, p % ps, :] = rand((G, d), BF16, 900 + s)
+            c["v_pool"][page, :, :, p % ps] = rand((G, d), BF16, 950 + s)
+    qn = (1 + rand((d,), F32, 30, 0.2)).to(DEV) if norm else None
+    kn = (1 + rand((d,), F32, 31, 0.2)).to(DEV) if norm else None
+    cos, sin = rope_tables(max(before) + 1, d)
+    cos, sin = (cos.to(DEV), sin.to(DEV)) if rotate else (None, None)
+    dev = {k: (v.to(DEV) if torch.is_tensor(v) else v) for k, v in c.items()}
+    scale = 1.0 / math.sqrt(d)
+    assert ops.decode_takes_qk(d, ps)
+    # the two kernels
+    k1, v1 = dev["k_pool"].clone(), dev["v_pool"].clone()
+    q = ops.qk_norm_rope_store(dev["qkv"].clone(), H, G, d, qn, kn, 1e-5, cos, sin,
+                               d if rotate else 0, 1 if rotate else 0, k1, v1, dev["row_pos"],
+                               dev["row_seg"], dev["bt"], ps, store_kv=store)
+    want = ops.paged_attention(q, H, G, d, k1, v1, dev["row_pos"], dev["row_seg"], dev["bt"], ps,
+                               scale, window=window, single_rows=True, max_position=c["max_pos"],
+                               kernel=kernel)
+    # the one
+    k2, v2 = dev["k_pool"].clone(), dev["v_pool"].clone()
+    got = ops.paged_attention(dev["qkv"], H, G, d, k2, v2, dev["row_pos"], dev["row_seg"],
+                              dev["bt"], ps, scale, window=window, single_rows=True,
+                              max_position=c["max_pos"], kernel=kernel,
+                              qk=ops.QkPrologue(qn, kn, 1e-5, cos, sin, store_kv=store))
+    nan = lambda t: torch.nan_to_num(t.float().cpu(), nan=-7.0)
+    assert torch.equal(torch.isnan(k1.float()).cpu(), torch.isnan(k2.float()).cpu()), "slots"
+    assert torch.equal(nan(v1), nan(v2)), "v pages"
+    # (the sums of squares are added in another order: a key may differ in its last bit)
+    close(nan(k2), nan(k1).double(), BF16_ULP, "k pages")
+    close(got.float(), want.float().cpu().double(), 2 * BF16_ULP, "attention")
+    if not store:
+        assert torch.equal(nan(k2), nan(dev["k_pool"])) and torch.equal(nan(v2), nan(dev["v_pool"]))
+
+
+def test_decode_attention_refuses_a_prologue_it_cannot_do(ops):
+    c = paged_case(12, BF16, 4, 2, 48, 16, [5], [1])
+    dev = {k: (v.to(DEV) if torch.is_tensor(v) else v) for k, v in c.items()}
+    assert not ops.decode_takes_qk(48, 16)
+    with pytest.raises(ValueError, match="do not take the norm"):
+        ops.paged_attention(dev["qkv"], 4, 2, 48, dev["k_pool"], dev["v_pool"], dev["row_pos"],
+                            dev["row_seg"], dev["bt"], 16, 0.1, single_rows=True, max_position=5,
+                            kernel="decode", qk=ops.QkPrologue(None, None, 1e-5, None, None))
+
+
 @pytest.mark.parametrize("case", ATT_CASES)
 @pytest.mark.parametrize("n_parts", [1, 3])
 def test_store_from_partial_sums(ops, case, n_parts):

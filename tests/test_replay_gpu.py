@@ -263,6 +263,61 @@ def test_long_prompt_on_a_wide_model(tmp_path, dtype, shape):
     assert_matches_plain(got, folder, requests, dtype)
 
 
+def test_decode_attention_with_its_prologue_inside_from_c_and_from_the_host(tmp_path):
+    """With more than 512 keys and a head size of 64 a decode step's attention kernel does the
+    per-head norm, the rotation and the store of the new key and value itself.  The C side of a
+    step and the host's parts must make that choice alike (bit-equal logits), the host's parts
+    must have made it (no call of the separate kernel in those steps), and both ways the logits
+    stay within the bound of the plain implementation's rounding."""
+    import copy
+    from kappai_amd.config import config_from_dict
+    from kappai_amd.engine.replay import TraceReplayer, make_replay_cache
+    from kappai_amd.engine.step import StepRunner
+    from kappai_amd.kernels import ops, tuning
+    from kappai_amd.weights import write_random_model
+    separate = []                    # rows of every call of the kernel that is to be left out
+    plain_kernel = ops.qk_norm_rope_store
+
+    def spy(qkv, *args, **kwargs):
+        separate.append(qkv.shape[-2])
+        return plain_kernel(qkv, *args, **kwargs)
+
+    folder = write_random_model(tmp_path / "wide", config_from_dict(copy.deepcopy(WIDE)), seed=8,
+                                std=0.02, norm_jitter=0.05)
+    requests = make_requests(WIDE["vocab_size"], [640, 530], seed=17)
+    plans = {"r0": (0, [632] + [1] * 8), "r1": (0, [522] + [1] * 8)}
+    steps, index, peak = schedules.build(requests, plans, want="last")
+    results = {}
+    for fused in (True, False):
+        for c_forward in (True, False):
+            tuning.FUSED_QK = fused
+            ops.qk_norm_rope_store = spy
+            del separate[:]
+            try:
+                model = gpu_model(folder, "bfloat16")
+                cache = make_replay_cache(model, peak)
+                cache.allocate_storage(model.dtype, "cuda:0", poison=True)
+                runner = StepRunner(model, cache, "cuda:0", decode_graphs=False,
+                                    c_forward=c_forward)
+                rep = TraceReplayer(runner, tmp_path / f"f{fused}c{c_forward}")
+                outputs = {}
+                for obj in steps:
+                    res = rep.run_step(obj)
+                    if res is not None:
+                        outputs[obj["step"]] = res
+            finally:
+                tuning.FUSED_QK = True
+                ops.qk_norm_rope_store = plain_kernel
+            if not c_forward:        # two attention layers; one prompt step, eight decode steps
+                assert separate == ([1154] * 2 if fused else [1154] * 2 + [2] * 16), separate
+            results[(fused, c_forward)] = collect(index, outputs, model.vocab_size)
+    for fused in (True, False):
+        a, b = results[(fused, True)], results[(fused, False)]
+        assert a.keys() == b.keys()
+        assert all(np.array_equal(a[k], b[k]) for k in a), fused
+        assert_matches_plain(a, folder, requests, "bfloat16")
+
+
 # Products with 17 to 64 rows and many rows of W run in a kernel of their own (activation rows
 # shared through LDS): hidden size and feed-forward width are multiples of 512 here, and gate/up
 # and the output head have 8192 rows, so a decode step of 40 requests takes it where a step of 8
