@@ -780,10 +780,14 @@ __global__ __launch_bounds__(8 * WAVE) void attn_prefill_shared_kernel(
 // keys whose loads a wave has in flight at once (their registers: keys * HEAD_DIM / 64)
 #define D_KPW (HEAD_DIM <= 64 ? 128 : (HEAD_DIM <= 128 ? 64 : 32))
 
+// head sizes whose decode kernel can take the prologue below: the rotation's partner d / 2 further
+// must lie in the same lane, and the registers must hold it beside a chunk of keys
+#define D_QK_FUSABLE (HEAD_DIM % 64 == 0 && HEAD_DIM <= 128)
+
 // The per-head RMSNorm, the rotation and the storing of a decoded row's own key and value, done in
 // the attention kernel's prologue instead of a kernel of their own (kappai: QK-norm, then RoPE,
-// then the cache write, src/models/lfm.c:36-44).  For head sizes that are multiples of 64, where
-// the rotation's partner d / 2 further lies in the same lane; rotate-half over the whole head.
+// then the cache write, src/models/lfm.c:36-44).  For head sizes of 64 and 128; rotate-half over
+// the whole head.
 struct QkFuse {
   int on;                   // 0: q is ready and the row's key and value are in the pools
   int kv;                   // the row's own key and value come from the projection beside q (k of
@@ -877,6 +881,7 @@ __device__ __forceinline__ void qk_norm_rotate(u32x4_t (&raw)[(HEAD_DIM + 31) / 
 // of the chunks c0 = first, first + stride, ... below k_end (D_KPW keys each), with a running
 // maximum and sum per column.  Leaves the unnormalised output in o (lane: column lane % 16, d
 // rows 16 mt + 4 (lane / 16) + v), the maximum (in units of log 2) in m_run, the sum in l_run.
+template <bool FUSABLE>
 __device__ __forceinline__ void attn_decode_wave(
     const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ k_pool,
     const bf16_t* __restrict__ vt_pool, const int* __restrict__ bt, int max_blocks, int t, int g,
@@ -892,7 +897,7 @@ __device__ __forceinline__ void attn_decode_wave(
   u32x4_t k_new[D_KS];                 // the row's own key, in the K fragment's order of d
   uint32_t v_new[D_MT];                // its value at d = 16 mt + col
   QkTables tb;
-  const bool fused = HEAD_DIM % 64 == 0 && qk.on;
+  const bool fused = FUSABLE && D_QK_FUSABLE && qk.on;
   const bool own_kv = fused && qk.kv;
   {
     const bf16_t* row = q + (size_t)t * q_stride;
@@ -904,7 +909,7 @@ __device__ __forceinline__ void attn_decode_wave(
       if (head_ok && d0 < HEAD_DIM) v = *reinterpret_cast<const u32x4_t*>(qr + d0);
       qraw[ks] = v;
     }
-    if constexpr (HEAD_DIM % 64 == 0) {
+    if constexpr (FUSABLE && D_QK_FUSABLE) {
       if (fused) {
         // everything the prologue needs is asked for here; it is worked on when the first keys
         // have been asked for as well
@@ -966,7 +971,7 @@ __device__ __forceinline__ void attn_decode_wave(
       for (int mt = 0; mt < D_MT; ++mt)
         vv[c][mt] = load_vt8_pg(vt_pool, pv, G, g, ps, 16 * mt + col, kb + 8 * kg, lo, hi);
     }
-    if constexpr (HEAD_DIM % 64 == 0) {
+    if constexpr (FUSABLE && D_QK_FUSABLE) {
       if (prologue_due) {
         prologue_due = false;
         if (own_kv) qk_norm_rotate(k_new, qk.k_norm_w != nullptr, tb.wk, qk.eps,
@@ -1094,8 +1099,8 @@ __global__ __launch_bounds__(64) void attn_decode_kernel(
   const size_t pbase = ((size_t)t * H + h) * n_splits + split;
   f32x4_t o[D_MT];
   float m_run, l_run;
-  attn_decode_wave(q, q_stride, k_pool, vt_pool, bt, max_blocks, t, g, H, G, ps, scale, lo,
-                   k_end - 1, k_begin, D_KPW, k_end, o, m_run, l_run, qk, pos);
+  attn_decode_wave<true>(q, q_stride, k_pool, vt_pool, bt, max_blocks, t, g, H, G, ps, scale, lo,
+                         k_end - 1, k_begin, D_KPW, k_end, o, m_run, l_run, qk, pos);
   if (!head_ok) return;
   if (kg == 0) {
     part_ml[2 * pbase] = m_run;
@@ -1121,7 +1126,7 @@ __global__ __launch_bounds__(D_BLOCK_MAX_WAVES * WAVE) void attn_decode_block_ke
     const bf16_t* __restrict__ vt_pool, bf16_t* __restrict__ out, int out_stride,
     const int* __restrict__ row_pos, const int* __restrict__ row_seg,
     const int* __restrict__ block_tables, int max_blocks, int H, int G, int ps, int window,
-    float scale, QkFuse qk) {
+    float scale) {
   extern __shared__ float sh_dec[];
   const int t = blockIdx.x, g = blockIdx.y;
   const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE, NW = blockDim.x / WAVE;
@@ -1134,8 +1139,11 @@ __global__ __launch_bounds__(D_BLOCK_MAX_WAVES * WAVE) void attn_decode_block_ke
   const int k_end = pos + 1;
   f32x4_t o[D_MT];
   float m_run, l_run;
-  attn_decode_wave(q, q_stride, k_pool, vt_pool, bt, max_blocks, t, g, H, G, ps, scale, lo, pos,
-                   k_begin + wave * D_KPW, NW * D_KPW, k_end, o, m_run, l_run, qk, pos);
+  // (without the prologue: eight waves a block leave no registers for it, and every wave would
+  // do it again)
+  attn_decode_wave<false>(q, q_stride, k_pool, vt_pool, bt, max_blocks, t, g, H, G, ps, scale, lo,
+                          pos, k_begin + wave * D_KPW, NW * D_KPW, k_end, o, m_run, l_run,
+                          QkFuse{}, pos);
   float* sh_o = sh_dec;
   float* sh_m = sh_dec + (size_t)NW * rep * HEAD_DIM;
   float* sh_l = sh_m + NW * 16;
@@ -1236,11 +1244,14 @@ extern "C" int kappai_attn_decode_block_waves(int rep) {
   return nw >= 2 ? nw : 0;
 }
 
-static int launch_decode_block(const void* q, int q_stride, const void* k_pool,
-                               const void* vt_pool, void* out, int out_stride, const int* row_pos,
-                               const int* row_seg, const int* block_tables, int max_blocks, int T,
-                               int H, int G, int ps, int window, float scale, int n_waves,
-                               const QkFuse& qk, hipStream_t stream) {
+// Decode attention with the keys of a row split over the `n_waves` waves of one block per (row, kv
+// head); no workspace, no second kernel.
+extern "C" int kappai_attn_decode_block(const void* q, int q_stride, const void* k_pool,
+                                        const void* vt_pool, void* out, int out_stride,
+                                        const int* row_pos, const int* row_seg,
+                                        const int* block_tables, int max_blocks, int T, int H,
+                                        int G, int ps, int window, float scale, int n_waves,
+                                        hipStream_t stream) {
   if (T <= 0) return 0;
   if (ps % 16 || G < 1 || H % G || H / G > 16 || G > 65535 || (q_stride % 8) || n_waves < 1 ||
       n_waves > kappai_attn_decode_block_waves(H / G))
@@ -1250,56 +1261,27 @@ static int launch_decode_block(const void* q, int q_stride, const void* k_pool,
   hipLaunchKernelGGL(attn_decode_block_kernel, dim3(T, G), dim3(n_waves * WAVE), lds, stream,
                      (const bf16_t*)q, q_stride, (const bf16_t*)k_pool, (const bf16_t*)vt_pool,
                      (bf16_t*)out, out_stride, row_pos, row_seg, block_tables, max_blocks, H, G, ps,
-                     window, scale, qk);
+                     window, scale);
   KAPPAI_RETURN_LAUNCH_STATUS();
 }
 
-// Decode attention with the keys of a row split over the `n_waves` waves of one block per (row, kv
-// head); no workspace, no second kernel.
-extern "C" int kappai_attn_decode_block(const void* q, int q_stride, const void* k_pool,
-                                        const void* vt_pool, void* out, int out_stride,
-                                        const int* row_pos, const int* row_seg,
-                                        const int* block_tables, int max_blocks, int T, int H,
-                                        int G, int ps, int window, float scale, int n_waves,
-                                        hipStream_t stream) {
-  return launch_decode_block(q, q_stride, k_pool, vt_pool, out, out_stride, row_pos, row_seg,
-                             block_tables, max_blocks, T, H, G, ps, window, scale, n_waves,
-                             QkFuse{}, stream);
-}
+// 1 when the decode kernel of this head size that splits the keys over blocks can do the per-head
+// norm, the rotation and the storing of the rows' own keys and values itself
+// (kappai_attn_decode_qk)
+extern "C" int kappai_attn_decode_takes_qk(void) { return D_QK_FUSABLE ? 1 : 0; }
 
-// 1 when the decode kernels of this head size can do the per-head norm, the rotation and the
-// storing of the rows' own keys and values themselves (kappai_attn_decode_qk, _block_qk)
-extern "C" int kappai_attn_decode_takes_qk(void) { return HEAD_DIM % 64 == 0 ? 1 : 0; }
-
-// The arguments that the _qk entry points add: qkv [T, row_stride] is the projection as it comes
-// out of its product (q heads, then with store_kv the k heads and the v heads); q_norm_w /
+// The arguments that kappai_attn_decode_qk adds: qkv [T, row_stride] is the projection as it
+// comes out of its product (q heads, then with store_kv the k heads and the v heads); q_norm_w /
 // k_norm_w [d] float or null; cos_tab / sin_tab [positions, d / 2] float (rotate-half over the
 // whole head) or both null; the pools are written at each row's own position when store_kv.
 static bool qk_args_ok(const void* qkv, int row_stride, const float* q_norm_w,
                        const float* k_norm_w, const float* cos_tab, const float* sin_tab,
                        const void* k_pool, const void* vt_pool) {
-  return HEAD_DIM % 64 == 0 && row_stride % 8 == 0 && ((uintptr_t)qkv % 16) == 0 &&
+  return D_QK_FUSABLE && row_stride % 8 == 0 && ((uintptr_t)qkv % 16) == 0 &&
          ((uintptr_t)q_norm_w % 16) == 0 && ((uintptr_t)k_norm_w % 16) == 0 &&
          ((uintptr_t)cos_tab % 16) == 0 && ((uintptr_t)sin_tab % 16) == 0 &&
          (cos_tab == nullptr) == (sin_tab == nullptr) && ((uintptr_t)k_pool % 16) == 0 &&
          vt_pool != nullptr;
-}
-
-extern "C" int kappai_attn_decode_block_qk(const void* qkv, int row_stride, void* k_pool,
-                                           void* vt_pool, void* out, int out_stride,
-                                           const int* row_pos, const int* row_seg,
-                                           const int* block_tables, int max_blocks, int T, int H,
-                                           int G, int ps, int window, float scale, int n_waves,
-                                           const float* q_norm_w, const float* k_norm_w, float eps,
-                                           const float* cos_tab, const float* sin_tab,
-                                           int store_kv, hipStream_t stream) {
-  if (!qk_args_ok(qkv, row_stride, q_norm_w, k_norm_w, cos_tab, sin_tab, k_pool, vt_pool))
-    return (int)hipErrorInvalidValue;
-  const QkFuse qk{1, store_kv ? 1 : 0, q_norm_w, k_norm_w, eps, cos_tab, sin_tab, (bf16_t*)k_pool,
-                  (bf16_t*)vt_pool};
-  return launch_decode_block(qkv, row_stride, k_pool, vt_pool, out, out_stride, row_pos, row_seg,
-                             block_tables, max_blocks, T, H, G, ps, window, scale, n_waves, qk,
-                             stream);
 }
 
 extern "C" int kappai_attn_head_dim(void) { return HEAD_DIM; }
@@ -1367,7 +1349,7 @@ extern "C" int kappai_attn_decode(const void* q, int q_stride, const void* k_poo
 }
 
 // kappai_attn_decode with the norm, the rotation and the store of the rows' own keys and values in
-// the kernel's prologue (see kappai_attn_decode_block_qk for the added arguments).  Every split of
+// the kernel's prologue (see qk_args_ok for the added arguments).  Every split of
 // a row must find the row's position inside the keys the splits cover: the caller's n_splits *
 // keys_per_split reach beyond the longest context, as for kappai_attn_decode.
 extern "C" int kappai_attn_decode_qk(const void* qkv, int row_stride, void* k_pool, void* vt_pool,

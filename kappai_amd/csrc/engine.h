@@ -20,7 +20,7 @@
 extern "C" {
 #endif
 
-#define KAPPAI_ENGINE_ABI 4          // bumped with every change of the structs below
+#define KAPPAI_ENGINE_ABI 5          // bumped with every change of the structs below
 #define KAPPAI_MAX_GROUPS 8          // paged groups a batch can carry block tables for
 
 // ---- the kernels' launchers, by address (they live in libraries of their own) ---------------
@@ -67,16 +67,14 @@ typedef struct kappai_attention_kernels {
   int (*attn_decode_block)(const void*, int, const void*, const void*, void*, int, const int*,
                            const int*, const int*, int, int, int, int, int, int, float, int,
                            hipStream_t);
-  // the decode kernels with the per-head norm, the rotation and the store of the rows' own keys
-  // and values in their prologue (decode_takes_qk() says whether this head size has them)
+  // the decode kernel that splits the keys over blocks, with the per-head norm, the rotation and
+  // the store of the rows' own keys and values in its prologue (decode_takes_qk() says whether
+  // this head size has it)
   int (*decode_takes_qk)(void);
   int (*attn_decode_qk)(const void*, int, void*, void*, void*, int, float*, float*, const int*,
                         const int*, const int*, int, int, int, int, int, int, float, int, int,
                         const float*, const float*, float, const float*, const float*, int,
                         hipStream_t);
-  int (*attn_decode_block_qk)(const void*, int, void*, void*, void*, int, const int*, const int*,
-                              const int*, int, int, int, int, int, int, float, int, const float*,
-                              const float*, float, const float*, const float*, int, hipStream_t);
 } kappai_attention_kernels;
 
 // ---- the model --------------------------------------------------------------------------------

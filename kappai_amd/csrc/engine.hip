@@ -478,16 +478,9 @@ Carry attention_mixer(Ctx& c, const kappai_layer_call& L, Rows x, float* resid, 
     const int n_keys = decode_keys(c, L);
     const int block_waves = L.mfma->decode_block_waves(H / G);
     if (decode_block_form(c, L, H / G)) {
-      if (qk_in_kernel)
-        LAUNCH(c, L.mfma->attn_decode_block_qk(q, q_stride, L.k_pool, L.v_pool, ctx, H * d,
-                                               b.row_pos, b.row_seg, tables, max_blocks, M, H, G,
-                                               ps, L.window, L.scale, block_waves, L.q_norm_w,
-                                               L.k_norm_w, L.qk_eps, cos_t, sin_t, store,
-                                               c.stream));
-      else
-        LAUNCH(c, L.mfma->attn_decode_block(q, q_stride, L.k_pool, L.v_pool, ctx, H * d, b.row_pos,
-                                            b.row_seg, tables, max_blocks, M, H, G, ps, L.window,
-                                            L.scale, block_waves, c.stream));
+      LAUNCH(c, L.mfma->attn_decode_block(q, q_stride, L.k_pool, L.v_pool, ctx, H * d, b.row_pos,
+                                          b.row_seg, tables, max_blocks, M, H, G, ps, L.window,
+                                          L.scale, block_waves, c.stream));
     } else {
       const int kpw = L.mfma->keys_per_wave();
       int n_splits = c.m->decode_max_splits;

@@ -29,7 +29,7 @@ from ..parts.embedding import OutputHead, TokenEmbedding
 from ..parts.feed_forward import SwiGLU
 from ..parts.rotary import RotaryEncoding
 
-ENGINE_ABI = 4
+ENGINE_ABI = 5
 MAX_GROUPS = 8
 
 
@@ -45,8 +45,7 @@ class Kernels(Structure):
 
 class AttentionKernels(Structure):
     _fields_ = _ptrs(["keys_per_wave", "decode_block_waves", "attn_prefill", "attn_decode",
-                      "attn_decode_block", "decode_takes_qk", "attn_decode_qk",
-                      "attn_decode_block_qk"])
+                      "attn_decode_block", "decode_takes_qk", "attn_decode_qk"])
 
 
 class LinearDesc(Structure):
@@ -264,7 +263,6 @@ class CForward:
             a.attn_decode_block = _address(lib.kappai_attn_decode_block)
             a.decode_takes_qk = _address(lib.kappai_attn_decode_takes_qk)
             a.attn_decode_qk = _address(lib.kappai_attn_decode_qk)
-            a.attn_decode_block_qk = _address(lib.kappai_attn_decode_block_qk)
             self._mfma[head_dim] = a
         return self._mfma[head_dim]
 

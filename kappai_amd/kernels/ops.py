@@ -753,7 +753,7 @@ def decode_form(n_heads: int, n_kv_heads: int, head_dim: int, max_position: int,
 
 def decode_takes_qk(head_dim: int, page_size: int) -> bool:
     """Whether the decode attention kernels of this head size take a ``QkPrologue`` (head sizes
-    that are multiples of 64, where a lane holds both halves of a rotation pair)."""
+    64 and 128: a lane holds both halves of a rotation pair, and the registers the prologue)."""
     if head_dim % 16 or head_dim > 256 or page_size % 16:
         return False
     return bool(library("attention_mfma", HEAD_DIM=head_dim).kappai_attn_decode_takes_qk())
@@ -858,14 +858,16 @@ def paged_attention(q: torch.Tensor, n_heads: int, n_kv_heads: int, head_dim: in
     n_keys = min(max_position + 1, window) + 32 if window else max_position + 1
     block_waves = lib.kappai_attn_decode_block_waves(H // G)
     if kernel == "decode":
-        kernel = decode_form(H, G, d, max_position, window)
+        kernel = "decode-split" if qk is not None else decode_form(H, G, d, max_position, window)
     if kernel == "decode-block":
         _need(block_waves > 0, "too many query heads a kv head for the block form")
-        check((lib.kappai_attn_decode_block_qk if qk is not None else lib.kappai_attn_decode_block)(
+        _need(qk is None, "the decode kernel that keeps a row's keys in one block takes q ready "
+                          "made and the keys stored")
+        check(lib.kappai_attn_decode_block(
             _ptr(q), _c_int(q.stride(0)), _ptr(k_pool), _ptr(v_pool), _ptr(out), _c_int(H * d),
             _ptr(row_pos), _ptr(row_seg), _ptr(block_tables), _c_int(block_tables.shape[1]),
             _c_int(T), _c_int(H), _c_int(G), _c_int(page_size), _c_int(window or 0),
-            _c_float(scale), _c_int(block_waves), *qk_args, _stream()), "attn_decode_block")
+            _c_float(scale), _c_int(block_waves), _stream()), "attn_decode_block")
         return out
     # one wave keeps the loads of `kpw` keys in flight; splits are whole numbers of that, and
     # at most DECODE_MAX_SPLITS of them are merged

@@ -35,6 +35,6 @@ FUSED_STEP_NARROW_WIDTH = 2048
 FUSED_STEP_NARROW_ROWS = 16
 
 # A decode step's attention kernels normalise and rotate q and the row's own key themselves and
-# store key and value (head sizes that are multiples of 64, rotate-half over the whole head, a
+# store key and value (head sizes 64 and 128, rotate-half over the whole head, a
 # projection that comes as bfloat16 rows): one kernel a layer less, 4.9 us each at batch 8.
 FUSED_QK = True
