@@ -892,6 +892,16 @@ __device__ __forceinline__ void attn_decode_wave(
   const int col = lane % 16, kg = lane / 16;
   const bool head_ok = col < rep;
   const int h = g * rep + (head_ok ? col : 0);
+  // the page ids of the first chunk of keys: asked for before anything else, so that the keys
+  // can be asked for as soon as they are there, whatever else is still on its way
+  auto ask_pages = [&](int c0) {
+    const int first_page = c0 / ps;
+    int my_page = -1;
+    if (first_page + lane < max_blocks && (first_page + lane) * ps <= hi)
+      my_page = bt[first_page + lane];
+    return my_page;
+  };
+  int pages_first = first < k_end ? ask_pages(first) : -1;
   bf16x8_t qf[D_KS];
   u32x4_t qraw[D_KS];
   u32x4_t k_new[D_KS];                 // the row's own key, in the K fragment's order of d
@@ -943,18 +953,18 @@ __device__ __forceinline__ void attn_decode_wave(
   // A wave takes its keys in chunks of D_KPW: first the chunk's page ids (one load, handed
   // round by shuffles), then every key and value load of the chunk at once (16 bytes a lane
   // each), then the matrix products and the softmax: two memory round trips a chunk, whatever
-  // its length.
+  // its length.  (Two chunks' loads in flight at once were measured: the registers they take
+  // halve the waves a SIMD holds, and 64 requests at 4096 keys took 140 us instead of 100.)
   constexpr int NCH = D_KPW / 32;
-  for (int c0 = first; c0 < k_end; c0 += stride) {
+  struct Chunk {
+    u32x4_t kf[NCH][2][D_KS];
+    u32x4_t vv[NCH][D_MT];
+  };
+  auto ask = [&](int c0, int my_page, Chunk& ch) {
     const int first_page = c0 / ps;
-    int my_page = -1;
-    if (first_page + lane < max_blocks && (first_page + lane) * ps <= hi)
-      my_page = bt[first_page + lane];
     // Row r of the key tile tt (of the 32 keys from kb) is key kb + 8 (r / 4) + 4 tt + r % 4:
     // the lane that holds rows 4 kg .. 4 kg + 3 of both tiles' scores then holds the keys
     // kb + 8 kg .. + 7 in order, and their values are ONE 16-byte piece of a V^T row.
-    u32x4_t kf[NCH][2][D_KS];
-    u32x4_t vv[NCH][D_MT];
 #pragma unroll
     for (int c = 0; c < NCH; ++c) {
       const int kb = c0 + 32 * c;
@@ -964,67 +974,44 @@ __device__ __forceinline__ void attn_decode_wave(
         const int page = __shfl(my_page, min(key / ps - first_page, WAVE - 1), WAVE);
 #pragma unroll
         for (int ks = 0; ks < D_KS; ++ks)
-          kf[c][tt][ks] = load_k8_pg(k_pool, page, G, g, ps, key, 32 * ks + 8 * kg, lo, hi);
+          ch.kf[c][tt][ks] = load_k8_pg(k_pool, page, G, g, ps, key, 32 * ks + 8 * kg, lo, hi);
       }
       const int pv = __shfl(my_page, min((kb + 8 * kg) / ps - first_page, WAVE - 1), WAVE);
 #pragma unroll
       for (int mt = 0; mt < D_MT; ++mt)
-        vv[c][mt] = load_vt8_pg(vt_pool, pv, G, g, ps, 16 * mt + col, kb + 8 * kg, lo, hi);
+        ch.vv[c][mt] = load_vt8_pg(vt_pool, pv, G, g, ps, 16 * mt + col, kb + 8 * kg, lo, hi);
     }
-    if constexpr (FUSABLE && D_QK_FUSABLE) {
-      if (prologue_due) {
-        prologue_due = false;
-        if (own_kv) qk_norm_rotate(k_new, qk.k_norm_w != nullptr, tb.wk, qk.eps,
-                                   qk.cos_tab != nullptr, tb.cs, tb.sn);
-        qk_norm_rotate(qraw, qk.q_norm_w != nullptr, tb.wq, qk.eps, qk.cos_tab != nullptr, tb.cs,
-                       tb.sn);
+  };
+  // the pools do not hold the row's own key and value yet (or only just): the chunk that holds
+  // the row's position takes them from the registers
+  auto own = [&](int c0, Chunk& ch) {
+    if (!(own_kv && pos >= c0 && pos < c0 + D_KPW)) return;
 #pragma unroll
-        for (int ks = 0; ks < D_KS; ++ks)
-          qf[ks] = as_frag(head_ok ? qraw[ks] : (u32x4_t){0u, 0u, 0u, 0u});
-        if (owner) {
-          const size_t pg = (size_t)bt[pos / ps] * G + g;
-          if (col == 0) {
+    for (int c = 0; c < NCH; ++c) {
+      const int kb = c0 + 32 * c;
 #pragma unroll
-            for (int ks = 0; ks < D_KS; ++ks)
-              *reinterpret_cast<u32x4_t*>(qk.k_pool_w + (pg * ps + pos % ps) * HEAD_DIM + 32 * ks +
-                                          8 * kg) = k_new[ks];
-          }
-          if (kg == 0) {
+      for (int tt = 0; tt < 2; ++tt) {
+        if (kb + 8 * (col / 4) + 4 * tt + col % 4 == pos) {
 #pragma unroll
-            for (int mt = 0; mt < D_MT; ++mt)
-              qk.vt_pool_w[(pg * HEAD_DIM + 16 * mt + col) * ps + pos % ps] = (bf16_t)v_new[mt];
-          }
+          for (int ks = 0; ks < D_KS; ++ks) ch.kf[c][tt][ks] = k_new[ks];
+        }
+      }
+      const int e = pos - (kb + 8 * kg);
+      if (e >= 0 && e < 8) {
+        const uint32_t keep = (e & 1) ? 0x0000ffffu : 0xffff0000u;
+#pragma unroll
+        for (int mt = 0; mt < D_MT; ++mt) {
+          const uint32_t put = (v_new[mt] & 0xffffu) << ((e & 1) * 16);
+          uint32_t w[4] = {ch.vv[c][mt].x, ch.vv[c][mt].y, ch.vv[c][mt].z, ch.vv[c][mt].w};
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            if (i == e / 2) w[i] = (w[i] & keep) | put;
+          ch.vv[c][mt] = (u32x4_t){w[0], w[1], w[2], w[3]};
         }
       }
     }
-    if (own_kv && pos >= c0 && pos < c0 + D_KPW) {
-      // the pools do not hold the row's own key and value yet (or only just): they are taken
-      // from the registers
-#pragma unroll
-      for (int c = 0; c < NCH; ++c) {
-        const int kb = c0 + 32 * c;
-#pragma unroll
-        for (int tt = 0; tt < 2; ++tt) {
-          if (kb + 8 * (col / 4) + 4 * tt + col % 4 == pos) {
-#pragma unroll
-            for (int ks = 0; ks < D_KS; ++ks) kf[c][tt][ks] = k_new[ks];
-          }
-        }
-        const int e = pos - (kb + 8 * kg);
-        if (e >= 0 && e < 8) {
-          const uint32_t keep = (e & 1) ? 0x0000ffffu : 0xffff0000u;
-#pragma unroll
-          for (int mt = 0; mt < D_MT; ++mt) {
-            const uint32_t put = (v_new[mt] & 0xffffu) << ((e & 1) * 16);
-            uint32_t w[4] = {vv[c][mt].x, vv[c][mt].y, vv[c][mt].z, vv[c][mt].w};
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-              if (i == e / 2) w[i] = (w[i] & keep) | put;
-            vv[c][mt] = (u32x4_t){w[0], w[1], w[2], w[3]};
-          }
-        }
-      }
-    }
+  };
+  auto work = [&](int c0, const Chunk& ch) {
 #pragma unroll
     for (int c = 0; c < NCH; ++c) {
       const int kb = c0 + 32 * c;
@@ -1035,8 +1022,8 @@ __device__ __forceinline__ void attn_decode_wave(
         s[tt] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int ks = 0; ks < D_KS; ++ks)
-          s[tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_frag(kf[c][tt][ks]), qf[ks], s[tt], 0,
-                                                          0, 0);
+          s[tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_frag(ch.kf[c][tt][ks]), qf[ks], s[tt],
+                                                          0, 0, 0);
       }
       // lane holds, for head `col`, keys kb + 8*kg + 4*tt + v
       float mloc = -INFINITY;
@@ -1072,14 +1059,49 @@ __device__ __forceinline__ void attn_decode_wave(
 #pragma unroll
       for (int mt = 0; mt < D_MT; ++mt) {
         o[mt] = o[mt] * corr;
-        o[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_frag(vv[c][mt]), pf, o[mt], 0, 0, 0);
+        o[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_frag(ch.vv[c][mt]), pf, o[mt], 0, 0, 0);
       }
     }
+  };
+  for (int c0 = first; c0 < k_end; c0 += stride) {
+    Chunk ca;
+    ask(c0, c0 == first ? pages_first : ask_pages(c0), ca);
+    if constexpr (FUSABLE && D_QK_FUSABLE) {
+      if (prologue_due) {
+        prologue_due = false;
+        if (own_kv) qk_norm_rotate(k_new, qk.k_norm_w != nullptr, tb.wk, qk.eps,
+                                   qk.cos_tab != nullptr, tb.cs, tb.sn);
+        qk_norm_rotate(qraw, qk.q_norm_w != nullptr, tb.wq, qk.eps, qk.cos_tab != nullptr, tb.cs,
+                       tb.sn);
+#pragma unroll
+        for (int ks = 0; ks < D_KS; ++ks)
+          qf[ks] = as_frag(head_ok ? qraw[ks] : (u32x4_t){0u, 0u, 0u, 0u});
+        if (owner) {
+          const size_t pg = (size_t)bt[pos / ps] * G + g;
+          if (col == 0) {
+#pragma unroll
+            for (int ks = 0; ks < D_KS; ++ks)
+              *reinterpret_cast<u32x4_t*>(qk.k_pool_w + (pg * ps + pos % ps) * HEAD_DIM + 32 * ks +
+                                          8 * kg) = k_new[ks];
+          }
+          if (kg == 0) {
+#pragma unroll
+            for (int mt = 0; mt < D_MT; ++mt)
+              qk.vt_pool_w[(pg * HEAD_DIM + 16 * mt + col) * ps + pos % ps] = (bf16_t)v_new[mt];
+          }
+        }
+      }
+    }
+    own(c0, ca);
+    work(c0, ca);
   }
 }
 
 // The keys of a row split over blocks: block (t, g, split) is one wave that takes the keys
 // k_begin + split * keys_per_split .. and writes its partial result; attn_merge adds them up.
+// (FUSED: with the prologue of QkFuse; a kernel of its own, because the prologue's registers would
+// halve the waves a SIMD holds for the steps that do not use it)
+template <bool FUSED>
 __global__ __launch_bounds__(64) void attn_decode_kernel(
     const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ k_pool,
     const bf16_t* __restrict__ vt_pool, float* __restrict__ part_o, float* __restrict__ part_ml,
@@ -1099,8 +1121,8 @@ __global__ __launch_bounds__(64) void attn_decode_kernel(
   const size_t pbase = ((size_t)t * H + h) * n_splits + split;
   f32x4_t o[D_MT];
   float m_run, l_run;
-  attn_decode_wave<true>(q, q_stride, k_pool, vt_pool, bt, max_blocks, t, g, H, G, ps, scale, lo,
-                         k_end - 1, k_begin, D_KPW, k_end, o, m_run, l_run, qk, pos);
+  attn_decode_wave<FUSED>(q, q_stride, k_pool, vt_pool, bt, max_blocks, t, g, H, G, ps, scale, lo,
+                          k_end - 1, k_begin, D_KPW, k_end, o, m_run, l_run, qk, pos);
   if (!head_ok) return;
   if (kg == 0) {
     part_ml[2 * pbase] = m_run;
@@ -1327,10 +1349,16 @@ static int launch_decode(const void* q, int q_stride, const void* k_pool, const 
   if (ps % 16 || G < 1 || H % G || H / G > 16 || G > 65535 || n_splits < 1 || n_splits > 65535 ||
       keys_per_split < D_KPW || keys_per_split % D_KPW || (q_stride % 8))
     return (int)hipErrorInvalidValue;
-  hipLaunchKernelGGL(attn_decode_kernel, dim3(T, G, n_splits), dim3(WAVE), 0, stream,
-                     (const bf16_t*)q, q_stride, (const bf16_t*)k_pool, (const bf16_t*)vt_pool,
-                     part_o, part_ml, row_pos, row_seg, block_tables, max_blocks, H, G, ps, window,
-                     scale, keys_per_split, n_splits, qk);
+  if (qk.on)
+    hipLaunchKernelGGL(attn_decode_kernel<true>, dim3(T, G, n_splits), dim3(WAVE), 0, stream,
+                       (const bf16_t*)q, q_stride, (const bf16_t*)k_pool, (const bf16_t*)vt_pool,
+                       part_o, part_ml, row_pos, row_seg, block_tables, max_blocks, H, G, ps,
+                       window, scale, keys_per_split, n_splits, qk);
+  else
+    hipLaunchKernelGGL(attn_decode_kernel<false>, dim3(T, G, n_splits), dim3(WAVE), 0, stream,
+                       (const bf16_t*)q, q_stride, (const bf16_t*)k_pool, (const bf16_t*)vt_pool,
+                       part_o, part_ml, row_pos, row_seg, block_tables, max_blocks, H, G, ps,
+                       window, scale, keys_per_split, n_splits, qk);
   hipLaunchKernelGGL(attn_merge_kernel, dim3(T, H), dim3(MERGE_WAVES * WAVE), 0, stream,
                      (const float*)part_o, (const float*)part_ml, (bf16_t*)out, out_stride, H,
                      n_splits);

@@ -145,7 +145,8 @@ typedef struct kappai_model {
   int fused_max_rows;               // rows up to which products fold residual sum and norm in
   int decode_waves, decode_max_splits, decode_block_max_keys;
   int attention_tile_rows;
-  int fused_qk;                     // decode attention does norm, rotation and store itself
+  int fused_qk;                     // rows up to which decode attention does norm, rotation and
+                                    // store itself (0: never)
 } kappai_model;
 
 // ---- the rows of a step -------------------------------------------------------------------------

@@ -438,7 +438,7 @@ Carry attention_mixer(Ctx& c, const kappai_layer_call& L, Rows x, float* resid, 
   // decode: the attention kernels take the projection as it is and do norm, rotation and store
   // themselves (parts/attention.py: _prologue_in_kernel)
   const bool qk_in_kernel =
-      c.m->fused_qk && single && proj.kind == C_DELTA && !proj.is_f32 && L.mfma != nullptr &&
+      M <= c.m->fused_qk && single && proj.kind == C_DELTA && !proj.is_f32 && L.mfma != nullptr &&
       H / G <= 16 && qkv.n % 8 == 0 && aligned16(proj.data) && ps % 16 == 0 && d % 16 == 0 &&
       d <= 256 && (L.rot_mode == 0 || (L.rot_mode == 1 && L.rot_dim == d)) &&
       L.mfma->decode_takes_qk != nullptr && L.mfma->decode_takes_qk() &&

@@ -248,7 +248,7 @@ class CForward:
         m.decode_waves, m.decode_max_splits = ops.DECODE_WAVES, ops.DECODE_MAX_SPLITS
         m.decode_block_max_keys = ops.DECODE_BLOCK_MAX_KEYS
         m.attention_tile_rows = ops.ATTENTION_TILE_ROWS
-        m.fused_qk = 1 if tuning.FUSED_QK else 0
+        m.fused_qk = tuning.FUSED_QK_MAX_ROWS if tuning.FUSED_QK else 0
         self.desc = m
         self.workspace = Workspace()
 

@@ -34,7 +34,11 @@ FUSED_STEP_MIN_WIDTH = 4096
 FUSED_STEP_NARROW_WIDTH = 2048
 FUSED_STEP_NARROW_ROWS = 16
 
-# A decode step's attention kernels normalise and rotate q and the row's own key themselves and
-# store key and value (head sizes 64 and 128, rotate-half over the whole head, a
-# projection that comes as bfloat16 rows): one kernel a layer less, 4.9 us each at batch 8.
+# A decode step's attention kernel normalises and rotates q and the row's own key itself and
+# stores key and value (head sizes 64 and 128, rotate-half over the whole head, a projection that
+# comes as bfloat16 rows, more than 512 keys) for steps of up to FUSED_QK_MAX_ROWS rows: every
+# wave of the kernel does that work again, which a few hundred waves do faster than a kernel of
+# its own would (a step of the 1.2B shape: 10 us less at 1 to 4 rows) and a thousand or more do
+# not (7 us more at 6 rows, 12 at 8, 40 at 12).  0 switches it off.
 FUSED_QK = True
+FUSED_QK_MAX_ROWS = 4

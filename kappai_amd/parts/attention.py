@@ -114,13 +114,14 @@ class GroupedQueryAttention(Mixer):
     def _prologue_in_kernel(self, proj, rot, single_rows: bool, page_size: int,
                             max_position: int) -> bool:
         """Whether the decode attention kernels take the projection as it is (see
-        ``ops.QkPrologue``): a step of single rows whose projection came as bfloat16 rows, few
+        ``ops.QkPrologue``): a step of a few single rows whose projection came as bfloat16 rows, few
         enough query heads a kv head for the decode kernels, a head size they do it for, no
         rotation or rotate-half over the whole head, and keys enough for the kernel that splits
         them over blocks (where a block is one wave; in the other every wave of a block would do
         the prologue again, which costs what the kernel saved)."""
         if not (tuning.FUSED_QK and single_rows and isinstance(proj, torch.Tensor)
-                and proj.dim() == 2 and proj.dtype == torch.bfloat16 and proj.is_cuda
+                and proj.dim() == 2 and proj.shape[0] <= tuning.FUSED_QK_MAX_ROWS
+                and proj.dtype == torch.bfloat16 and proj.is_cuda
                 and self.H // self.G <= 16 and proj.stride(0) % 8 == 0
                 and proj.data_ptr() % 16 == 0):
             return False
