@@ -118,7 +118,13 @@ __device__ __forceinline__ bf16x8_t as_bf16x8(u32x4_t v) {
 __device__ __forceinline__ void store_out(float* p, float v) { *p = v; }
 __device__ __forceinline__ void store_out(bf16_t* p, float v) { *p = f32_to_bf16(v); }
 
-__device__ __forceinline__ float silu_f(float g) { return g / (1.0f + expf(-g)); }
+// silu(g) = g / (1 + e^-g) for the epilogues that store bfloat16: the hardware's 2^x and reciprocal
+// (each good to about an ulp of float, far below a bfloat16's rounding) instead of expf and a
+// division, which were 9 of the 132 us of gate/up at 2048 rows.  e^-g overflows to infinity for
+// g < -88: the reciprocal is then 0 and the result -0, as it should be.
+__device__ __forceinline__ float silu_f(float g) {
+  return g * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * g));
+}
 
 // Block = WAVES_M x WAVES_N waves, each owning (WM*32) x (WN*32) of the result as WM*WN
 // accumulator tiles of 32x32: per 16 of K a wave reads WM+WN fragments from LDS for WM*WN
