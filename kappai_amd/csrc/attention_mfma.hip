@@ -1107,8 +1107,11 @@ __global__ __launch_bounds__(64) void attn_decode_kernel(
     const bf16_t* __restrict__ vt_pool, float* __restrict__ part_o, float* __restrict__ part_ml,
     const int* __restrict__ row_pos, const int* __restrict__ row_seg,
     const int* __restrict__ block_tables, int max_blocks, int H, int G, int ps, int window,
-    float scale, int keys_per_split, int n_splits, QkFuse qk) {
-  const int t = blockIdx.x, g = blockIdx.y, split = blockIdx.z, lane = threadIdx.x;
+    float scale, int keys_per_split, int n_splits, QkFuse qk, const int* __restrict__ row_ids) {
+  // (row_ids: the kernel's rows are these rows of the step, partial results are kept by their
+  // place in the list)
+  const int t = row_ids ? row_ids[blockIdx.x] : blockIdx.x;
+  const int g = blockIdx.y, split = blockIdx.z, lane = threadIdx.x;
   const int rep = H / G;
   const int col = lane % 16, kg = lane / 16;
   const int pos = row_pos[t];
@@ -1118,7 +1121,7 @@ __global__ __launch_bounds__(64) void attn_decode_kernel(
   const int k_end = min(k_begin + keys_per_split, pos + 1);     // exclusive
   const bool head_ok = col < rep;
   const int h = g * rep + (head_ok ? col : 0);
-  const size_t pbase = ((size_t)t * H + h) * n_splits + split;
+  const size_t pbase = ((size_t)blockIdx.x * H + h) * n_splits + split;
   f32x4_t o[D_MT];
   float m_run, l_run;
   attn_decode_wave<FUSED>(q, q_stride, k_pool, vt_pool, bt, max_blocks, t, g, H, G, ps, scale, lo,
@@ -1202,13 +1205,14 @@ __global__ __launch_bounds__(D_BLOCK_MAX_WAVES * WAVE) void attn_decode_block_ke
 #define MERGE_WAVES 4
 __global__ __launch_bounds__(MERGE_WAVES * WAVE) void attn_merge_kernel(
     const float* __restrict__ part_o, const float* __restrict__ part_ml,
-    bf16_t* __restrict__ out, int out_stride, int H, int n_splits) {
+    bf16_t* __restrict__ out, int out_stride, int H, int n_splits,
+    const int* __restrict__ row_ids) {
   constexpr int NPL = (HEAD_DIM + WAVE - 1) / WAVE;
   __shared__ float sh_acc[MERGE_WAVES][NPL * WAVE];
   __shared__ float sh_l[MERGE_WAVES];
-  const int t = blockIdx.x, h = blockIdx.y;
+  const int t = row_ids ? row_ids[blockIdx.x] : blockIdx.x, h = blockIdx.y;
   const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE;
-  const size_t base = ((size_t)t * H + h) * n_splits;
+  const size_t base = ((size_t)blockIdx.x * H + h) * n_splits;
   float M = -INFINITY;
   for (int s = lane; s < n_splits; s += WAVE) M = fmaxf(M, part_ml[2 * (base + s)]);
   M = wave_max(M);
@@ -1344,7 +1348,8 @@ static int launch_decode(const void* q, int q_stride, const void* k_pool, const 
                          void* out, int out_stride, float* part_o, float* part_ml,
                          const int* row_pos, const int* row_seg, const int* block_tables,
                          int max_blocks, int T, int H, int G, int ps, int window, float scale,
-                         int keys_per_split, int n_splits, const QkFuse& qk, hipStream_t stream) {
+                         int keys_per_split, int n_splits, const QkFuse& qk, const int* row_ids,
+                         hipStream_t stream) {
   if (T <= 0) return 0;
   if (ps % 16 || G < 1 || H % G || H / G > 16 || G > 65535 || n_splits < 1 || n_splits > 65535 ||
       keys_per_split < D_KPW || keys_per_split % D_KPW || (q_stride % 8))
@@ -1353,15 +1358,15 @@ static int launch_decode(const void* q, int q_stride, const void* k_pool, const 
     hipLaunchKernelGGL(attn_decode_kernel<true>, dim3(T, G, n_splits), dim3(WAVE), 0, stream,
                        (const bf16_t*)q, q_stride, (const bf16_t*)k_pool, (const bf16_t*)vt_pool,
                        part_o, part_ml, row_pos, row_seg, block_tables, max_blocks, H, G, ps,
-                       window, scale, keys_per_split, n_splits, qk);
+                       window, scale, keys_per_split, n_splits, qk, row_ids);
   else
     hipLaunchKernelGGL(attn_decode_kernel<false>, dim3(T, G, n_splits), dim3(WAVE), 0, stream,
                        (const bf16_t*)q, q_stride, (const bf16_t*)k_pool, (const bf16_t*)vt_pool,
                        part_o, part_ml, row_pos, row_seg, block_tables, max_blocks, H, G, ps,
-                       window, scale, keys_per_split, n_splits, qk);
+                       window, scale, keys_per_split, n_splits, qk, row_ids);
   hipLaunchKernelGGL(attn_merge_kernel, dim3(T, H), dim3(MERGE_WAVES * WAVE), 0, stream,
                      (const float*)part_o, (const float*)part_ml, (bf16_t*)out, out_stride, H,
-                     n_splits);
+                     n_splits, row_ids);
   KAPPAI_RETURN_LAUNCH_STATUS();
 }
 
@@ -1373,7 +1378,24 @@ extern "C" int kappai_attn_decode(const void* q, int q_stride, const void* k_poo
                                   int n_splits, hipStream_t stream) {
   return launch_decode(q, q_stride, k_pool, vt_pool, out, out_stride, part_o, part_ml, row_pos,
                        row_seg, block_tables, max_blocks, T, H, G, ps, window, scale,
-                       keys_per_split, n_splits, QkFuse{}, stream);
+                       keys_per_split, n_splits, QkFuse{}, nullptr, stream);
+}
+
+// kappai_attn_decode for some rows of a step: row_ids [T] names them (rows of q, row_pos, row_seg
+// and out), part_o / part_ml hold T rows.  For the single decoded tokens of a step that also
+// holds prompt portions: a row that stands alone over a long context is one tile for the tiled
+// kernel, whose block then walks all its keys by itself.
+extern "C" int kappai_attn_decode_rows(const void* q, int q_stride, const void* k_pool,
+                                       const void* vt_pool, void* out, int out_stride,
+                                       float* part_o, float* part_ml, const int* row_ids,
+                                       const int* row_pos, const int* row_seg,
+                                       const int* block_tables, int max_blocks, int T, int H,
+                                       int G, int ps, int window, float scale, int keys_per_split,
+                                       int n_splits, hipStream_t stream) {
+  if (row_ids == nullptr) return (int)hipErrorInvalidValue;
+  return launch_decode(q, q_stride, k_pool, vt_pool, out, out_stride, part_o, part_ml, row_pos,
+                       row_seg, block_tables, max_blocks, T, H, G, ps, window, scale,
+                       keys_per_split, n_splits, QkFuse{}, row_ids, stream);
 }
 
 // kappai_attn_decode with the norm, the rotation and the store of the rows' own keys and values in
@@ -1394,7 +1416,7 @@ extern "C" int kappai_attn_decode_qk(const void* qkv, int row_stride, void* k_po
                   (bf16_t*)vt_pool};
   return launch_decode(qkv, row_stride, k_pool, vt_pool, out, out_stride, part_o, part_ml, row_pos,
                        row_seg, block_tables, max_blocks, T, H, G, ps, window, scale,
-                       keys_per_split, n_splits, qk, stream);
+                       keys_per_split, n_splits, qk, nullptr, stream);
 }
 
 // ---------------------------------------------------------------------------------------

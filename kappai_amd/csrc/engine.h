@@ -20,7 +20,7 @@
 extern "C" {
 #endif
 
-#define KAPPAI_ENGINE_ABI 5          // bumped with every change of the structs below
+#define KAPPAI_ENGINE_ABI 6          // bumped with every change of the structs below
 #define KAPPAI_MAX_GROUPS 8          // paged groups a batch can carry block tables for
 
 // ---- the kernels' launchers, by address (they live in libraries of their own) ---------------
@@ -70,6 +70,10 @@ typedef struct kappai_attention_kernels {
   // the decode kernel that splits the keys over blocks, with the per-head norm, the rotation and
   // the store of the rows' own keys and values in its prologue (decode_takes_qk() says whether
   // this head size has it)
+  // kappai_attn_decode for the rows that a list names
+  int (*attn_decode_rows)(const void*, int, const void*, const void*, void*, int, float*, float*,
+                          const int*, const int*, const int*, const int*, int, int, int, int, int,
+                          int, float, int, int, hipStream_t);
   int (*decode_takes_qk)(void);
   int (*attn_decode_qk)(const void*, int, void*, void*, void*, int, float*, float*, const int*,
                         const int*, const int*, int, int, int, int, int, int, float, int, int,
@@ -161,6 +165,9 @@ typedef struct kappai_batch {
   const int* logit_rows;            // [n_logit_rows]
   const int* q_tiles;               // [n_tiles, 4] or null
   int n_tiles;
+  const int* lone_rows;             // [n_lone_rows] or null: single decoded tokens beside prompt
+  int n_lone_rows;                  // portions that q_tiles leaves out
+  int max_lone_position;
   int n_groups;
   const int* block_tables[KAPPAI_MAX_GROUPS];   // [n_segments, max_blocks[g]]
   int max_blocks[KAPPAI_MAX_GROUPS];

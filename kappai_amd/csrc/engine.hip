@@ -403,6 +403,20 @@ bool decode_block_form(const Ctx& c, const kappai_layer_call& L, int rep) {
   return L.mfma->decode_block_waves(rep) > 0 && decode_keys(c, L) <= c.m->decode_block_max_keys;
 }
 
+// how the split decode kernel cuts n_keys keys of `rows` rows (ops._decode_split)
+void decode_splits(const Ctx& c, const kappai_layer_call& L, int rows, int G, int n_keys,
+                   int* keys_per_split, int* n_splits) {
+  const int kpw = L.mfma->keys_per_wave();
+  int s = c.m->decode_max_splits;
+  if ((n_keys + kpw - 1) / kpw < s) s = (n_keys + kpw - 1) / kpw;
+  int by_waves = c.m->decode_waves / (rows * G);
+  if (by_waves < 1) by_waves = 1;
+  if (by_waves < s) s = by_waves;
+  if (s < 1) s = 1;
+  *keys_per_split = ((n_keys + s - 1) / s + kpw - 1) / kpw * kpw;
+  *n_splits = (n_keys + *keys_per_split - 1) / *keys_per_split;
+}
+
 // parts/attention.py with ops.qk_norm_rope_store and ops.paged_attention
 Carry attention_mixer(Ctx& c, const kappai_layer_call& L, Rows x, float* resid, const Into& into) {
   const kappai_kernels& k = *c.m->kernels;
@@ -482,15 +496,8 @@ Carry attention_mixer(Ctx& c, const kappai_layer_call& L, Rows x, float* resid, 
                                           b.row_seg, tables, max_blocks, M, H, G, ps, L.window,
                                           L.scale, block_waves, c.stream));
     } else {
-      const int kpw = L.mfma->keys_per_wave();
-      int n_splits = c.m->decode_max_splits;
-      if ((n_keys + kpw - 1) / kpw < n_splits) n_splits = (n_keys + kpw - 1) / kpw;
-      int by_waves = c.m->decode_waves / (M * G);
-      if (by_waves < 1) by_waves = 1;
-      if (by_waves < n_splits) n_splits = by_waves;
-      if (n_splits < 1) n_splits = 1;
-      const int keys_per_split = ((n_keys + n_splits - 1) / n_splits + kpw - 1) / kpw * kpw;
-      n_splits = (n_keys + keys_per_split - 1) / keys_per_split;
+      int keys_per_split, n_splits;
+      decode_splits(c, L, M, G, n_keys, &keys_per_split, &n_splits);
       float* part_o = (float*)c.a->take(R_BLOCK, (size_t)M * H * n_splits * d * 4);
       float* part_ml = (float*)c.a->take(R_BLOCK, (size_t)M * H * n_splits * 2 * 4);
       if (qk_in_kernel)
@@ -508,6 +515,26 @@ Carry attention_mixer(Ctx& c, const kappai_layer_call& L, Rows x, float* resid, 
     LAUNCH(c, L.mfma->attn_prefill(q, q_stride, L.k_pool, L.v_pool, ctx, H * d, b.q_tiles,
                                    b.n_tiles, b.row_pos, tables, max_blocks, H, G, ps, L.window,
                                    L.scale, 0, c.stream));
+    if (b.lone_rows != nullptr && b.n_lone_rows > 0) {
+      // the single decoded tokens beside the portions: keys split over blocks (ops._decode_split)
+      if (H / G > 16 || b.max_lone_position < 0) {
+        snprintf(g_error, sizeof g_error, "kappai_forward: rows left out of the tiles need the "
+                                          "decode kernel and their largest position");
+        c.status = (int)hipErrorInvalidValue;
+        return none;
+      }
+      const int R = b.n_lone_rows;
+      int n_keys = b.max_lone_position + 1;
+      if (L.window) n_keys = (n_keys < L.window ? n_keys : L.window) + 32;
+      int keys_per_split, n_splits;
+      decode_splits(c, L, R, G, n_keys, &keys_per_split, &n_splits);
+      float* part_o = (float*)c.a->take(R_BLOCK, (size_t)R * H * n_splits * d * 4);
+      float* part_ml = (float*)c.a->take(R_BLOCK, (size_t)R * H * n_splits * 2 * 4);
+      LAUNCH(c, L.mfma->attn_decode_rows(q, q_stride, L.k_pool, L.v_pool, ctx, H * d, part_o,
+                                         part_ml, b.lone_rows, b.row_pos, b.row_seg, tables,
+                                         max_blocks, R, H, G, ps, L.window, L.scale,
+                                         keys_per_split, n_splits, c.stream));
+    }
   } else {
     LAUNCH(c, k.paged_attention_rows(q, q_stride, L.k_pool, L.v_pool, ctx, H * d, b.row_pos,
                                      b.row_seg, tables, max_blocks, M, H, G, d, ps, L.window,

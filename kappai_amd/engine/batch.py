@@ -49,6 +49,10 @@ class RowBatch:
     seg_slot: torch.Tensor
     logit_rows: torch.Tensor
     q_tiles: Optional[torch.Tensor] = None      # [tiles, 4]: (segment, first row, rows, place)
+    # the single decoded tokens of a step that also holds prompt portions, when they are left out
+    # of q_tiles (``Part.lone_rows_from``): their rows, and the largest of their positions
+    lone_rows: Optional[torch.Tensor] = None
+    max_lone_position: int = -1
     block_tables: List[torch.Tensor] = field(default_factory=list)
     host: Dict[str, np.ndarray] = field(default_factory=dict)
 
@@ -62,11 +66,14 @@ def tile_place(index: int, tiles_in_segment: int) -> int:
 
 
 def layout_rows(entries: Sequence[StepEntry], cache: CacheManager, vocab_size: int,
-                tile_rows: Optional[int] = None):
+                tile_rows: Optional[int] = None, lone_rows_from: Optional[int] = None):
     """Host side of ``RowBatch``: checks the entries and lays the tables out as int32
     arrays.  Returns (dict of arrays, sizes).  ``tile_rows``: cut the segments into tiles of at
-    most that many rows (``q_tiles``); None: no such table.  The tables are made for all entries
-    at once (a step of many single decoded tokens costs a few numpy calls, not a few per entry)."""
+    most that many rows (``q_tiles``); None: no such table.  ``lone_rows_from``: in a step with
+    segments of several rows, the segments of a single row go into ``lone_rows`` instead of
+    ``q_tiles`` when the longest of their contexts has at least that many keys.  The tables are
+    made for all entries at once (a step of many single decoded tokens costs a few numpy calls,
+    not a few per entry)."""
     if not entries:
         raise ValueError("a step needs at least one entry")
     S = len(entries)
@@ -117,11 +124,18 @@ def layout_rows(entries: Sequence[StepEntry], cache: CacheManager, vocab_size: i
         "seg_slot": np.asarray(slots, dtype=np.int32),
         "logit_rows": np.asarray(logit_rows, dtype=np.int32),
     }
+    max_lone_position = -1
     if tile_rows:
         # tile j of a segment: (segment, first row, rows, place); the fourth number tells a kernel
         # where the tile stands in its segment (index | tiles of the segment << 16, or 0 when the
         # segment has more tiles than 15 bits hold), so that it can pair tiles of one segment
         nt = (n_arr + tile_rows - 1) // tile_rows
+        lone = n_arr == 1
+        if (lone_rows_from and lone.any() and not lone.all() and cache.page_size % 16 == 0
+                and int(p0_arr[lone].max()) + 1 >= lone_rows_from):
+            arrays["lone_rows"] = seg_start[:-1][lone].astype(np.int32)
+            max_lone_position = int(p0_arr[lone].max())
+            nt = np.where(lone, 0, nt)
         tile_seg = np.repeat(np.arange(S, dtype=np.int64), nt)
         first_tile = np.cumsum(nt) - nt
         idx = np.arange(int(nt.sum()), dtype=np.int64) - np.repeat(first_tile, nt)
@@ -141,6 +155,6 @@ def layout_rows(entries: Sequence[StepEntry], cache: CacheManager, vocab_size: i
     sizes = {
         "n_rows": T, "n_segments": S, "n_logit_rows": len(logit_rows),
         "max_position": max_position, "max_segment_rows": int(n_arr.max()),
-        "n_groups": n_groups,
+        "n_groups": n_groups, "max_lone_position": max_lone_position,
     }
     return arrays, sizes

@@ -29,7 +29,7 @@ from ..parts.embedding import OutputHead, TokenEmbedding
 from ..parts.feed_forward import SwiGLU
 from ..parts.rotary import RotaryEncoding
 
-ENGINE_ABI = 5
+ENGINE_ABI = 6
 MAX_GROUPS = 8
 
 
@@ -45,7 +45,8 @@ class Kernels(Structure):
 
 class AttentionKernels(Structure):
     _fields_ = _ptrs(["keys_per_wave", "decode_block_waves", "attn_prefill", "attn_decode",
-                      "attn_decode_block", "decode_takes_qk", "attn_decode_qk"])
+                      "attn_decode_block", "attn_decode_rows", "decode_takes_qk",
+                      "attn_decode_qk"])
 
 
 class LinearDesc(Structure):
@@ -90,7 +91,9 @@ class BatchDesc(Structure):
         ("max_segment_rows", c_int), ("tokens", c_void_p), ("row_pos", c_void_p),
         ("row_seg", c_void_p), ("seg_start", c_void_p), ("seg_pos0", c_void_p),
         ("seg_slot", c_void_p), ("logit_rows", c_void_p), ("q_tiles", c_void_p),
-        ("n_tiles", c_int), ("n_groups", c_int), ("block_tables", c_void_p * MAX_GROUPS),
+        ("n_tiles", c_int), ("lone_rows", c_void_p), ("n_lone_rows", c_int),
+        ("max_lone_position", c_int), ("n_groups", c_int),
+        ("block_tables", c_void_p * MAX_GROUPS),
         ("max_blocks", c_int * MAX_GROUPS)]
 
 
@@ -261,6 +264,7 @@ class CForward:
             a.attn_prefill = _address(lib.kappai_attn_prefill)
             a.attn_decode = _address(lib.kappai_attn_decode)
             a.attn_decode_block = _address(lib.kappai_attn_decode_block)
+            a.attn_decode_rows = _address(lib.kappai_attn_decode_rows)
             a.decode_takes_qk = _address(lib.kappai_attn_decode_takes_qk)
             a.attn_decode_qk = _address(lib.kappai_attn_decode_qk)
             self._mfma[head_dim] = a
@@ -277,6 +281,9 @@ class CForward:
         b.logit_rows = batch.logit_rows.data_ptr()
         if batch.q_tiles is not None:
             b.q_tiles, b.n_tiles = batch.q_tiles.data_ptr(), batch.q_tiles.shape[0]
+        if batch.lone_rows is not None:
+            b.lone_rows, b.n_lone_rows = batch.lone_rows.data_ptr(), batch.lone_rows.shape[0]
+            b.max_lone_position = batch.max_lone_position
         if len(batch.block_tables) > MAX_GROUPS:
             raise ValueError(f"a step carries block tables for at most {MAX_GROUPS} groups")
         b.n_groups = len(batch.block_tables)

@@ -248,7 +248,8 @@ class StepRunner:
     def make_batch(self, entries: Sequence[StepEntry], placed=None) -> RowBatch:
         """``placed``: see ``step``."""
         arrays, sizes = layout_rows(entries, self.cache, self.model.vocab_size,
-                                    getattr(self.model, "q_tile_rows", None))
+                                    getattr(self.model, "q_tile_rows", None),
+                                    getattr(self.model, "lone_rows_from", None))
         if placed is not None and placed[1]:
             chosen, pairs = placed
             for ei, at in pairs:
@@ -266,6 +267,7 @@ class StepRunner:
             tokens=dev["tokens"], row_pos=dev["row_pos"], row_seg=dev["row_seg"],
             seg_start=dev["seg_start"], seg_pos0=dev["seg_pos0"], seg_slot=dev["seg_slot"],
             logit_rows=dev["logit_rows"], q_tiles=dev.get("q_tiles"),
+            lone_rows=dev.get("lone_rows"), max_lone_position=sizes["max_lone_position"],
             block_tables=[dev[f"block_table_{g}"] for g in range(sizes["n_groups"])],
             host=arrays)
 

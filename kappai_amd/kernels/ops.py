@@ -765,7 +765,8 @@ def paged_attention(q: torch.Tensor, n_heads: int, n_kv_heads: int, head_dim: in
                     scale: float, window: int = 0, q_tiles: Optional[torch.Tensor] = None,
                     single_rows: bool = False, max_position: Optional[int] = None,
                     kernel: str = "auto", prefill_variant: int = 0,
-                    qk: Optional[QkPrologue] = None) -> torch.Tensor:
+                    qk: Optional[QkPrologue] = None, lone_rows: Optional[torch.Tensor] = None,
+                    max_lone_position: int = -1) -> torch.Tensor:
     """Causal attention of every row over the keys of its request that are in the cache
     (its own included; the last ``window`` of them when a window is set).  ``q`` is
     [T, >= H d] with a row stride (the q columns of the fused projection).  Returns [T, H d].
@@ -781,7 +782,11 @@ def paged_attention(q: torch.Tensor, n_heads: int, n_kv_heads: int, head_dim: in
     heads of a kv head through LDS; head sizes 64 and 128 only).
 
     ``qk`` (decode kernels only, see ``decode_takes_qk``): ``q`` is the raw projection and the
-    kernel normalises and rotates q and the rows' own keys itself and stores keys and values."""
+    kernel normalises and rotates q and the rows' own keys itself and stores keys and values.
+
+    ``lone_rows`` (int32, with ``max_lone_position``; tiled kernel only): rows that ``q_tiles``
+    leaves out, the single decoded tokens of a step that also holds prompt portions.  They go
+    through the decode kernel that splits keys over blocks."""
     H, G, d = n_heads, n_kv_heads, head_dim
     _gpu("q", q, (F32, BF16), contiguous=False)
     T = q.shape[0]
@@ -830,6 +835,13 @@ def paged_attention(q: torch.Tensor, n_heads: int, n_kv_heads: int, head_dim: in
             _c_int(block_tables.shape[1]), _c_int(H), _c_int(G), _c_int(page_size),
             _c_int(window or 0), _c_float(scale), _c_int(prefill_variant), _stream()),
             "attn_prefill")
+        if lone_rows is not None:
+            _gpu("lone_rows", lone_rows, I32)
+            _need(H // G <= 16 and lone_rows.dim() == 1 and max_lone_position >= 0,
+                  "paged_attention: rows left out of the tiles need the decode kernel (at most 16 "
+                  "query heads a kv head) and their largest position")
+            _decode_split(lib, q, H, G, d, k_pool, v_pool, row_pos, row_seg, block_tables,
+                          page_size, scale, window, max_lone_position, out, lone_rows)
         return out
     _need(kernel in ("decode", "decode-block", "decode-split"),
           lambda: f"unknown attention kernel {kernel!r}")
@@ -869,6 +881,17 @@ def paged_attention(q: torch.Tensor, n_heads: int, n_kv_heads: int, head_dim: in
             _c_int(T), _c_int(H), _c_int(G), _c_int(page_size), _c_int(window or 0),
             _c_float(scale), _c_int(block_waves), _stream()), "attn_decode_block")
         return out
+    _decode_split(lib, q, H, G, d, k_pool, v_pool, row_pos, row_seg, block_tables, page_size, scale,
+                  window, max_position, out, None, qk_args)
+    return out
+
+
+def _decode_split(lib, q, H, G, d, k_pool, v_pool, row_pos, row_seg, block_tables, page_size, scale,
+                  window, max_position, out, row_ids, qk_args=()):
+    """The decode kernel that splits a row's keys over blocks, and its merge, for all rows or
+    (``row_ids``) some of them."""
+    T = q.shape[0] if row_ids is None else row_ids.shape[0]
+    n_keys = min(max_position + 1, window) + 32 if window else max_position + 1
     # one wave keeps the loads of `kpw` keys in flight; splits are whole numbers of that, and
     # at most DECODE_MAX_SPLITS of them are merged
     kpw = lib.kappai_attn_keys_per_wave()
@@ -880,13 +903,18 @@ def paged_attention(q: torch.Tensor, n_heads: int, n_kv_heads: int, head_dim: in
     n_splits = (n_keys + keys_per_split - 1) // keys_per_split
     part_o = torch.empty((T, H, n_splits, d), dtype=F32, device=q.device)
     part_ml = torch.empty((T, H, n_splits, 2), dtype=F32, device=q.device)
-    check((lib.kappai_attn_decode_qk if qk is not None else lib.kappai_attn_decode)(
-        _ptr(q), _c_int(q.stride(0)), _ptr(k_pool), _ptr(v_pool), _ptr(out), _c_int(H * d),
-        _ptr(part_o), _ptr(part_ml), _ptr(row_pos), _ptr(row_seg), _ptr(block_tables),
-        _c_int(block_tables.shape[1]), _c_int(T), _c_int(H), _c_int(G), _c_int(page_size),
-        _c_int(window or 0), _c_float(scale), _c_int(keys_per_split), _c_int(n_splits),
-        *qk_args, _stream()), "attn_decode")
-    return out
+    head = (_ptr(q), _c_int(q.stride(0)), _ptr(k_pool), _ptr(v_pool), _ptr(out), _c_int(H * d),
+            _ptr(part_o), _ptr(part_ml))
+    tail = (_ptr(row_pos), _ptr(row_seg), _ptr(block_tables), _c_int(block_tables.shape[1]),
+            _c_int(T), _c_int(H), _c_int(G), _c_int(page_size), _c_int(window or 0),
+            _c_float(scale), _c_int(keys_per_split), _c_int(n_splits))
+    if row_ids is not None:
+        check(lib.kappai_attn_decode_rows(*head, _ptr(row_ids), *tail, _stream()),
+              "attn_decode_rows")
+    elif qk_args:
+        check(lib.kappai_attn_decode_qk(*head, *tail, *qk_args, _stream()), "attn_decode_qk")
+    else:
+        check(lib.kappai_attn_decode(*head, *tail, _stream()), "attn_decode")
 
 
 # ---------------------------------------------------------------------------------------

@@ -42,3 +42,10 @@ FUSED_STEP_NARROW_ROWS = 16
 # not (7 us more at 6 rows, 12 at 8, 40 at 12).  0 switches it off.
 FUSED_QK = True
 FUSED_QK_MAX_ROWS = 4
+
+# In a step that holds prompt portions, a single decoded token is one tile for the tiled attention
+# kernel, and the block that gets it walks all its keys alone: 58 us at 2048 keys, 0.9 ms at 32 k,
+# however short the portions beside it are.  From this many keys on such rows go to the decode
+# kernel (keys split over blocks) instead: a second kernel and its merge (10-25 us a layer) against
+# that walk.  16 requests with 32 k-token prompts: prompt steps 19 -> 14 ms.
+LONE_ROWS_FROM = 1024

@@ -109,6 +109,15 @@ class Model:
         return asked.pop() if asked else None
 
     @property
+    def lone_rows_from(self) -> Optional[int]:
+        """The context length from which the single decoded tokens of a mixed step are listed
+        apart from the tiles (None: never): only when every part that asks for tiles says the
+        same."""
+        tiled = [b for b in self.layers if getattr(b, "q_tile_rows", None)]
+        asked = {getattr(b, "lone_rows_from", None) for b in tiled}
+        return asked.pop() if len(asked) == 1 else None
+
+    @property
     def vocab_size(self) -> int:
         return self.config.vocab_size
 

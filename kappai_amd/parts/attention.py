@@ -53,6 +53,13 @@ class GroupedQueryAttention(Mixer):
         self.q_norm_w: Optional[torch.Tensor] = None
         self.k_norm_w: Optional[torch.Tensor] = None
 
+    @property
+    def lone_rows_from(self) -> Optional[int]:
+        # (what the decode kernel needs; the page size is checked where the table is laid out)
+        ok = (self.dtype == torch.bfloat16 and self.H // self.G <= 16 and self.d % 16 == 0
+              and self.d <= 256)
+        return tuning.LONE_ROWS_FROM if ok and tuning.LONE_ROWS_FROM else None
+
     def cache_spec(self):
         return PagedKV(self.G, self.d, self.window)
 
@@ -108,7 +115,9 @@ class GroupedQueryAttention(Mixer):
                                       batch.row_seg, tables, cache.page_size, self.scale,
                                       window=self.window or 0, q_tiles=batch.q_tiles,
                                       single_rows=single,
-                                      max_position=batch.max_position)
+                                      max_position=batch.max_position,
+                                      lone_rows=getattr(batch, "lone_rows", None),
+                                      max_lone_position=getattr(batch, "max_lone_position", -1))
         return self.out.forward(ctx, partial_sums=True, add_into=into)
 
     def _prologue_in_kernel(self, proj, rot, single_rows: bool, page_size: int,

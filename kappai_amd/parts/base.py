@@ -32,6 +32,12 @@ class Part:
     # that many rows (``RowBatch.q_tiles``); None: the table is not laid out for this part.
     q_tile_rows: Optional[int] = None
 
+    # A part that asks for tiles may run the single decoded tokens of a step that also holds
+    # prompt portions through another kernel when their context is long: from this many keys on
+    # (the step's longest such context decides for all of them) they are left out of the tile
+    # table and listed in ``RowBatch.lone_rows`` instead.  None: every row is in a tile.
+    lone_rows_from: Optional[int] = None
+
     def tensor_specs(self) -> List[TensorSpec]:
         """Full names, shapes and roles of the tensors this part reads from the file."""
         return []

@@ -34,6 +34,10 @@ class PreNormBlock(Block):
     def q_tile_rows(self):
         return self.mixer.q_tile_rows
 
+    @property
+    def lone_rows_from(self):
+        return self.mixer.lone_rows_from
+
     def tensor_specs(self) -> List[TensorSpec]:
         return [s for p in self._parts() for s in p.tensor_specs()]
 

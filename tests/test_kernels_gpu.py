@@ -866,6 +866,38 @@ def test_decode_attention_with_norm_rotation_and_store_inside(ops, case, kernel=
         assert torch.equal(nan(k2), nan(dev["k_pool"])) and torch.equal(nan(v2), nan(dev["v_pool"]))
 
 
+@pytest.mark.parametrize("H,G,d,window", [(8, 2, 64, 0), (4, 4, 128, 0), (6, 3, 48, 700)])
+def test_lone_rows_beside_portions(ops, H, G, d, window):
+    """A step of two prompt portions and three single decoded tokens, two of them over long
+    contexts: with the single rows left out of the tile table and run through the decode kernel
+    (``lone_rows``) the result is that of the tiled kernel over all rows, and of the plain
+    kernel."""
+    ps = 16
+    before, new = [0, 2100, 40, 1300, 7], [70, 1, 33, 1, 1]
+    c = paged_case(13, BF16, H, G, d, ps, before, new)
+    qn, kn = (1 + rand((d,), F32, 30, 0.2)).to(DEV), (1 + rand((d,), F32, 31, 0.2)).to(DEV)
+    cos, sin = rope_tables(max(a + b for a, b in zip(before, new)) + 1, d)
+    dev = {k: (v.to(DEV) if torch.is_tensor(v) else v) for k, v in c.items()}
+    q = ops.qk_norm_rope_store(dev["qkv"], H, G, d, qn, kn, 1e-5, cos.to(DEV), sin.to(DEV), d, 1,
+                               dev["k_pool"], dev["v_pool"], dev["row_pos"], dev["row_seg"],
+                               dev["bt"], ps)
+    scale = 1.0 / math.sqrt(d)
+    args = (q, H, G, d, dev["k_pool"], dev["v_pool"], dev["row_pos"], dev["row_seg"], dev["bt"], ps,
+            scale)
+    plain = ops.paged_attention(*args, window=window, kernel="rows")
+    tiled = ops.paged_attention(*args, window=window, q_tiles=dev["q_tiles"], kernel="prefill",
+                                max_position=c["max_pos"])
+    close(tiled.float(), plain.float().cpu().double(), 2 * BF16_ULP, "all rows in tiles")
+    lone = torch.tensor([70, 104, 105], dtype=torch.int32)
+    tiles = torch.tensor([t for t in c["q_tiles"].tolist() if t[0] in (0, 2)], dtype=torch.int32)
+    got = ops.paged_attention(*args, window=window, q_tiles=tiles.to(DEV), kernel="prefill",
+                              max_position=c["max_pos"], lone_rows=lone.to(DEV),
+                              max_lone_position=2100)
+    close(got.float(), plain.float().cpu().double(), 2 * BF16_ULP, "lone rows apart")
+    rest = [i for i in range(c["T"]) if i not in (70, 104, 105)]
+    assert torch.equal(got[rest].cpu(), tiled[rest].cpu()), "the rows in tiles are not touched"
+
+
 def test_decode_attention_refuses_a_prologue_it_cannot_do(ops):
     c = paged_case(12, BF16, 4, 2, 48, 16, [5], [1])
     dev = {k: (v.to(DEV) if torch.is_tensor(v) else v) for k, v in c.items()}

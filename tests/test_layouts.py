@@ -37,3 +37,51 @@ def test_rows_in_fragment_order_come_back_as_rows():
     assert not ops.FragmentRows.fits(17, 2048, torch.bfloat16)       # one tile of 16 rows
     assert not ops.FragmentRows.fits(8, 2040, torch.bfloat16)        # whole pieces of 32 of K
     assert not ops.FragmentRows.fits(8, 2048, torch.float32)
+
+
+def test_row_tables_of_a_step():
+    """The int32 tables that ``layout_rows`` makes for a step of two prompt portions and three
+    single decoded tokens: rows, positions, segments, tiles of at most 32 rows; and with a limit
+    for lone rows, the single tokens leave the tile table once the longest of their contexts
+    reaches it (never in a step of single tokens only, where no tiles are used)."""
+    import numpy as np
+    from kappai_amd.cache import CacheManager, PagedKV
+    from kappai_amd.engine.batch import StepEntry, layout_rows
+    cm = CacheManager([PagedKV(2, 16)], 16, 400, 8)
+    held = {"a": 0, "b": 1500, "c": 40, "d": 70, "e": 2999}
+    caches = {}
+    for name, n in held.items():
+        caches[name] = cm.open(name)
+        if n:
+            cm.extend(caches[name], n)
+            cm.commit(caches[name], n)
+    new = {"a": 70, "b": 1, "c": 33, "d": 1, "e": 1}
+    entries = []
+    for name, n in new.items():
+        cm.extend(caches[name], n)
+        entries.append(StepEntry(caches[name], list(range(n)), [n - 1]))
+    arrays, sizes = layout_rows(entries, cm, 100, tile_rows=32)
+    assert sizes["n_rows"] == 106 and sizes["max_segment_rows"] == 70
+    assert sizes["max_position"] == 2999 and sizes["max_lone_position"] == -1
+    assert "lone_rows" not in arrays
+    assert arrays["seg_start"].tolist() == [0, 70, 71, 104, 105, 106]
+    assert arrays["logit_rows"].tolist() == [69, 70, 103, 104, 105]
+    assert arrays["row_pos"][[0, 69, 70, 71, 103, 104, 105]].tolist() == [0, 69, 1500, 40, 72, 70,
+                                                                         2999]
+    tiles = arrays["q_tiles"].tolist()
+    assert [t[:3] for t in tiles] == [[0, 0, 32], [0, 32, 32], [0, 64, 6], [1, 70, 1], [2, 71, 32],
+                                      [2, 103, 1], [3, 104, 1], [4, 105, 1]]
+    assert [t[3] for t in tiles[:3]] == [0 | 3 << 16, 1 | 3 << 16, 2 | 3 << 16]
+    # the longest lone context (3000 keys) reaches the limit: all three single tokens leave
+    arrays, sizes = layout_rows(entries, cm, 100, tile_rows=32, lone_rows_from=3000)
+    assert arrays["lone_rows"].tolist() == [70, 104, 105] and sizes["max_lone_position"] == 2999
+    assert [t[:3] for t in arrays["q_tiles"].tolist()] == [[0, 0, 32], [0, 32, 32], [0, 64, 6],
+                                                           [2, 71, 32], [2, 103, 1]]
+    assert arrays["q_tiles"].dtype == np.int32 and arrays["lone_rows"].dtype == np.int32
+    # it does not: nothing changes
+    arrays, sizes = layout_rows(entries, cm, 100, tile_rows=32, lone_rows_from=3001)
+    assert "lone_rows" not in arrays and len(arrays["q_tiles"]) == 8
+    # single tokens only: a decode step, which has no use for the list
+    singles = [e for e in entries if len(e.tokens) == 1]
+    arrays, sizes = layout_rows(singles, cm, 100, tile_rows=32, lone_rows_from=100)
+    assert "lone_rows" not in arrays and sizes["max_lone_position"] == -1

@@ -318,6 +318,55 @@ def test_decode_attention_with_its_prologue_inside_from_c_and_from_the_host(tmp_
         assert_matches_plain(a, folder, requests, "bfloat16")
 
 
+@pytest.mark.parametrize("dtype", ["bfloat16", "float32"])
+def test_decoded_tokens_over_long_contexts_beside_prompt_portions(tmp_path, dtype):
+    """Two requests decode at more than a thousand tokens of context while a third one's prompt
+    runs in portions beside them: in such steps the single rows are listed apart from the tiles
+    of the portions and take the decode kernel (bfloat16; float32 runs the plain kernel over
+    all rows).  Every logit against the plain implementation, from C and from the host's parts
+    bit for bit alike."""
+    import copy
+    from kappai_amd.config import config_from_dict
+    from kappai_amd.engine.replay import TraceReplayer, make_replay_cache
+    from kappai_amd.engine.step import StepRunner
+    from kappai_amd.weights import write_random_model
+    folder = write_random_model(tmp_path / "wide", config_from_dict(copy.deepcopy(WIDE)), seed=9,
+                                std=0.02, norm_jitter=0.05)
+    requests = make_requests(WIDE["vocab_size"], [1100, 1040, 150], seed=18)
+    # r0 and r1 whole, then one token a step; r2 arrives later, in portions beside them
+    plans = {"r0": (0, [1092] + [1] * 8), "r1": (0, [1032] + [1] * 8), "r2": (2, [70, 2, 45, 33])}
+    steps, index, peak = schedules.build(requests, plans, want="last")
+    results = {}
+    for c_forward in (True, False):
+        model = gpu_model(folder, dtype)
+        assert model.lone_rows_from == (1024 if dtype == "bfloat16" else None)
+        cache = make_replay_cache(model, peak)
+        cache.allocate_storage(model.dtype, "cuda:0", poison=True)
+        runner = StepRunner(model, cache, "cuda:0", c_forward=c_forward)
+        seen = []
+        make = runner.make_batch
+
+        def spy(entries, placed=None):
+            batch = make(entries, placed)
+            seen.append(None if batch.lone_rows is None else batch.lone_rows.tolist())
+            return batch
+
+        runner.make_batch = spy
+        rep = TraceReplayer(runner, tmp_path / f"c{c_forward}")
+        outputs = {}
+        for obj in steps:
+            res = rep.run_step(obj)
+            if res is not None:
+                outputs[obj["step"]] = res
+        if dtype == "bfloat16":
+            assert [rows for rows in seen if rows is not None] == [[0, 1]] * 4, seen
+        else:
+            assert all(rows is None for rows in seen)
+        results[c_forward] = collect(index, outputs, model.vocab_size)
+    assert all(np.array_equal(results[True][k], results[False][k]) for k in results[True])
+    assert_matches_plain(results[True], folder, requests, dtype)
+
+
 # Products with 17 to 64 rows and many rows of W run in a kernel of their own (activation rows
 # shared through LDS): hidden size and feed-forward width are multiples of 512 here, and gate/up
 # and the output head have 8192 rows, so a decode step of 40 requests takes it where a step of 8
