@@ -709,15 +709,15 @@ static void launch_tile(const bf16_t* A, const bf16_t* W, const float* bias, TO*
     const long blocks128 = (long)((M + 127) / 128) * ((n_rows_w + 127) / 128) * ksplit;
     const bool deep = blocks128 <= 256 && K / ksplit >= 2048;
     shape = !fits ? (big >= 128 ? 3 : 1) : use_256_form(blocks256) ? 5 : deep ? 8 : 6;
-    if (fits && EPI == 0) {
+    if (shape == 5 && EPI == 0) {
       // blocks of 256 rows x 192 columns when they fill their rounds and come to fewer rounds'
       // worth of work than 256 x 256 (in_proj of 2048 rows: 192 blocks of 256 x 256 leave 64 CUs
-      // idle, 256 blocks of 256 x 192 none: 49 against 55 us), or where 256 x 256 blocks would
-      // not fill theirs (6144 columns at 4096 rows: 94 against 106 us in 128 x 128 blocks)
+      // idle, 256 blocks of 256 x 192 none: 49 against 55 us).  Only against the 256 x 256 form:
+      // where the 128 x 128 form was chosen (rows or columns that fill their last tiles badly, K
+      // split into ranges) the 192 form was measured slower (2063 x 2048 x 7168: 88 against 74 us).
       const long blocks192 = (long)((M + 255) / 256) * ((n_rows_w + 191) / 192) * ksplit;
       const long r256 = (blocks256 + 255) / 256, r192 = (blocks192 + 255) / 256;
-      if (use_256_form(blocks192) && (shape != 5 || r192 * (192 + 16) < r256 * (256 + 16)))
-        shape = 9;
+      if (use_256_form(blocks192) && r192 * (192 + 16) < r256 * (256 + 16)) shape = 9;
     }
   }
   if ((shape == 5 || shape == 6 || shape == 8 || shape == 9) && !fits) shape = 3;
