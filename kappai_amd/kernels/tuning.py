@@ -44,8 +44,10 @@ FUSED_QK = True
 FUSED_QK_MAX_ROWS = 4
 
 # In a step that holds prompt portions, a single decoded token is one tile for the tiled attention
-# kernel, and the block that gets it walks all its keys alone: 58 us at 2048 keys, 0.9 ms at 32 k,
-# however short the portions beside it are.  From this many keys on such rows go to the decode
-# kernel (keys split over blocks) instead: a second kernel and its merge (10-25 us a layer) against
-# that walk.  16 requests with 32 k-token prompts: prompt steps 19 -> 14 ms.
-LONE_ROWS_FROM = 1024
+# kernel, and the block that gets it walks all its keys alone: 0.9 ms at 32 k keys, however short
+# the portions beside it are.  From this many keys on such rows go to the decode kernel (keys
+# split over blocks) instead: a second kernel and its merge (25-30 us a layer for up to 63 rows)
+# against that walk.  16 requests with 32 k-token prompts: prompt steps 19 -> 14 ms.  With up to
+# 63 rows of at most 2300 keys beside portions of 512 rows the two kernels took 49 us a layer where
+# the tiled kernel alone took 43, hence not from 1024 on.
+LONE_ROWS_FROM = 4096

@@ -319,7 +319,7 @@ def test_decode_attention_with_its_prologue_inside_from_c_and_from_the_host(tmp_
 
 
 @pytest.mark.parametrize("dtype", ["bfloat16", "float32"])
-def test_decoded_tokens_over_long_contexts_beside_prompt_portions(tmp_path, dtype):
+def test_decoded_tokens_over_long_contexts_beside_prompt_portions(tmp_path, dtype, monkeypatch):
     """Two requests decode at more than a thousand tokens of context while a third one's prompt
     runs in portions beside them: in such steps the single rows are listed apart from the tiles
     of the portions and take the decode kernel (bfloat16; float32 runs the plain kernel over
@@ -332,9 +332,11 @@ def test_decoded_tokens_over_long_contexts_beside_prompt_portions(tmp_path, dtyp
     from kappai_amd.weights import write_random_model
     folder = write_random_model(tmp_path / "wide", config_from_dict(copy.deepcopy(WIDE)), seed=9,
                                 std=0.02, norm_jitter=0.05)
+    from kappai_amd.kernels import tuning
     requests = make_requests(WIDE["vocab_size"], [1100, 1040, 150], seed=18)
     # r0 and r1 whole, then one token a step; r2 arrives later, in portions beside them
     plans = {"r0": (0, [1092] + [1] * 8), "r1": (0, [1032] + [1] * 8), "r2": (2, [70, 2, 45, 33])}
+    monkeypatch.setattr(tuning, "LONE_ROWS_FROM", 1024)     # (a thousand tokens get there)
     steps, index, peak = schedules.build(requests, plans, want="last")
     results = {}
     for c_forward in (True, False):
