@@ -54,6 +54,18 @@ class KeyReader:
             raise ConfigError(f"{self.where}: key '{self._name(key)}' must be an integer, got {v!r}")
         return int(v)
 
+    def int_or_ints(self, key, default=_MISSING):
+        """One integer or a list of them (checkpoints write ``eos_token_id`` either way)."""
+        v = self._get(key, default)
+        if v is None:
+            return None
+        items = v if isinstance(v, (list, tuple)) else [v]
+        for x in items:
+            if isinstance(x, bool) or not isinstance(x, (int, float)) or int(x) != x:
+                raise ConfigError(f"{self.where}: key '{self._name(key)}' must be an integer or a "
+                                  f"list of integers, got {v!r}")
+        return [int(x) for x in items] if isinstance(v, (list, tuple)) else int(v)
+
     def float(self, key, default=_MISSING) -> Optional[float]:
         v = self._get(key, default)
         if v is None:

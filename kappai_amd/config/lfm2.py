@@ -7,7 +7,7 @@ names of the architecture's own config.json keys.
 from __future__ import annotations
 
 from dataclasses import dataclass
-from typing import Any, Dict, List, Optional
+from typing import Any, Dict, List, Optional, Union
 
 from .base import ConfigError, KeyReader, ModelConfig
 
@@ -63,7 +63,7 @@ class Lfm2Config(ModelConfig):
     conv_bias: bool = False
     tie_embedding: bool = True
     max_position_embeddings: int = 0         # 0: config.json names no longest sequence
-    eos_token_id: Optional[int] = None
+    eos_token_id: Optional[Union[int, List[int]]] = None    # one id or several
     bos_token_id: Optional[int] = None
     pad_token_id: Optional[int] = None
 
@@ -124,7 +124,7 @@ class Lfm2Config(ModelConfig):
             conv_bias=r.bool("conv_bias", False),
             tie_embedding=r.bool(("tie_embedding", "tie_word_embeddings"), True),
             max_position_embeddings=r.int("max_position_embeddings", 0),
-            eos_token_id=r.int("eos_token_id", None),
+            eos_token_id=r.int_or_ints("eos_token_id", None),
             bos_token_id=r.int("bos_token_id", None),
             pad_token_id=r.int("pad_token_id", None),
         )

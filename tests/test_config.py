@@ -109,6 +109,23 @@ def test_rejected(change, match):
         config_from_dict(raw)
 
 
+def test_end_of_sequence_ids_one_or_several():
+    """Checkpoints write ``eos_token_id`` as one id or as a list; both are kept as written, and
+    anything else is refused."""
+    raw = copy.deepcopy(LFM2_1_2B)
+    assert config_from_dict(raw).eos_token_id is None
+    raw["eos_token_id"] = 7
+    cfg = config_from_dict(raw)
+    assert cfg.eos_token_id == 7 and cfg.to_dict()["eos_token_id"] == 7
+    raw["eos_token_id"] = [7, 2]
+    cfg = config_from_dict(raw)
+    assert cfg.eos_token_id == [7, 2] and cfg.to_dict()["eos_token_id"] == [7, 2]
+    for bad in ("7", [7, "2"], 7.5, [True]):
+        raw["eos_token_id"] = bad
+        with pytest.raises(ConfigError, match="eos_token_id"):
+            config_from_dict(raw)
+
+
 def test_head_dim_defaults_to_width_over_heads():
     raw = copy.deepcopy(TINY_A)
     del raw["head_dim"]
