@@ -64,6 +64,27 @@ extern "C" int kappai_copy_ints(int* dst, const int* src, int n, hipStream_t str
   KAPPAI_RETURN_LAUNCH_STATUS();
 }
 
+// Rows that lie in the order of the matrix cores' fragments ([D / 32][4 groups of 8 of K][16
+// rows][8 values], what the norm writes for the product kernel of 1 to 16 rows) as ordinary rows
+// [n_rows, D], for a consumer that reads rows: 16-byte chunk c of row m lies at chunk c * 16 + m.
+__global__ void rows_from_fragments_kernel(const uint4* __restrict__ frag, uint4* __restrict__ out,
+                                           int n_rows, int chunks) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n_rows * chunks) return;
+  const int m = i / chunks, c = i % chunks;
+  out[i] = frag[(size_t)c * 16 + m];
+}
+extern "C" int kappai_rows_from_fragments(const void* frag, void* out, int n_rows, int D,
+                                          hipStream_t stream) {
+  if (n_rows <= 0) return 0;
+  if (n_rows > 16 || D % 32 || ((uintptr_t)frag % 16) || ((uintptr_t)out % 16))
+    return (int)hipErrorInvalidValue;
+  const int chunks = D / 8;                               // 8 bfloat16 values a chunk
+  hipLaunchKernelGGL(rows_from_fragments_kernel, dim3((n_rows * chunks + 255) / 256), dim3(256), 0,
+                     stream, (const uint4*)frag, (uint4*)out, n_rows, chunks);
+  KAPPAI_RETURN_LAUNCH_STATUS();
+}
+
 // ---------------------------------------------------------------------------------------
 // RMSNorm with the residual sum folded in:
 //   x = resid[r] (+ delta[r]);  if write_resid: resid[r] = x;

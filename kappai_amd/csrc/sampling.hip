@@ -598,6 +598,171 @@ __global__ __launch_bounds__(FILT_THREADS) void sample_filtered_kernel(
                                         keep, top_p[i], min_p[i], uniform[i])];
 }
 
+// ---------------------------------------------------------------------------------------
+// The same draw for a top-k above 1024 (kappai keeps any top-k below the vocabulary,
+// src/sampler.c:218-223): the candidates no longer fit LDS.  One block per entry sorts the
+// whole row with its indices in a workspace in global memory (bitonic, descending value,
+// ascending index on ties: the passes that stay inside 4096 neighbours run in LDS, the others
+// in place), takes the first `keep`, and walks them in the reference's order of operations:
+// exponentials by all threads, every running sum by one thread, chunk by chunk through LDS.
+// A setting for experiments, not for serving: 2 to 3 ms for a vocabulary of 65,536.
+// ---------------------------------------------------------------------------------------
+#define WIDE_CHUNK 4096
+__global__ __launch_bounds__(FILT_THREADS) void sample_filtered_wide_kernel(
+    const float* __restrict__ logits, const int* __restrict__ rows, const int* __restrict__ keep_n,
+    const float* __restrict__ temperature, const float* __restrict__ top_p,
+    const float* __restrict__ min_p, const float* __restrict__ uniform, int* __restrict__ out,
+    int V, int n2, float* __restrict__ ws_val, int* __restrict__ ws_idx) {
+  __shared__ float s_val[WIDE_CHUNK];
+  __shared__ int s_idx[WIDE_CHUNK];
+  __shared__ int sh_stop, sh_int;
+  const int i = blockIdx.x, tid = threadIdx.x;
+  const float* lg = logits + (size_t)rows[i] * V;
+  float* val = ws_val + (size_t)i * n2;
+  int* idx = ws_idx + (size_t)i * n2;
+  const int keep = max(1, min(keep_n[i], V));
+  for (int e = tid; e < n2; e += FILT_THREADS) {
+    val[e] = e < V ? lg[e] : -INFINITY;
+    idx[e] = e < V ? e : 0x7fffffff;
+  }
+  __syncthreads();
+  // ---- the sort ---------------------------------------------------------------------------
+  const int len = min(WIDE_CHUNK, n2);           // both powers of two
+  // stages k_from..k_to, of each the passes with j < len, chunk by chunk in LDS
+  auto local_passes = [&](int k_from, int k_to) {
+    for (int c0 = 0; c0 < n2; c0 += len) {
+      for (int e = tid; e < len; e += FILT_THREADS) {
+        s_val[e] = val[c0 + e];
+        s_idx[e] = idx[c0 + e];
+      }
+      __syncthreads();
+      for (int k = k_from; k <= k_to; k <<= 1)
+        for (int j = min(k >> 1, len >> 1); j > 0; j >>= 1) {
+          for (int a = tid; a < len; a += FILT_THREADS) {
+            const int b = a ^ j;
+            if (b > a) {
+              const bool desc = ((c0 + a) & k) == 0;
+              const float va = s_val[a], vb = s_val[b];
+              const int ia = s_idx[a], ib = s_idx[b];
+              const bool a_first = va > vb || (va == vb && ia < ib);
+              if (a_first != desc) { s_val[a] = vb; s_val[b] = va; s_idx[a] = ib; s_idx[b] = ia; }
+            }
+          }
+          __syncthreads();
+        }
+      for (int e = tid; e < len; e += FILT_THREADS) {
+        val[c0 + e] = s_val[e];
+        idx[c0 + e] = s_idx[e];
+      }
+      __syncthreads();
+    }
+  };
+  local_passes(2, len);
+  for (int k = 2 * len; k <= n2; k <<= 1) {
+    for (int j = k >> 1; j >= len; j >>= 1) {
+      for (int a = tid; a < n2; a += FILT_THREADS) {
+        const int b = a ^ j;
+        if (b > a) {
+          const bool desc = (a & k) == 0;
+          const float va = val[a], vb = val[b];
+          const int ia = idx[a], ib = idx[b];
+          const bool a_first = va > vb || (va == vb && ia < ib);
+          if (a_first != desc) { val[a] = vb; val[b] = va; idx[a] = ib; idx[b] = ia; }
+        }
+      }
+      __syncthreads();
+    }
+    local_passes(k, k);
+  }
+  // ---- temperature: val[e] becomes p(e) -----------------------------------------------------
+  const float inv_t = 1.0f / temperature[i];
+  const float mx = val[0] * inv_t;
+  __syncthreads();
+  for (int e = tid; e < keep; e += FILT_THREADS) val[e] = expf(val[e] * inv_t - mx);
+  __syncthreads();
+  // thread 0 walks p(0..n) in order, a chunk at a time out of LDS; body(e, p) returns true to stop
+  auto walk = [&](int n, auto&& body) {
+    for (int c0 = 0; c0 < n; c0 += WIDE_CHUNK) {
+      const int m = min(WIDE_CHUNK, n - c0);
+      for (int e = tid; e < m; e += FILT_THREADS) s_val[e] = val[c0 + e];
+      if (tid == 0) sh_stop = 0;
+      __syncthreads();
+      if (tid == 0)
+        for (int e = 0; e < m; ++e)
+          if (body(c0 + e, s_val[e])) { sh_stop = 1; break; }
+      __syncthreads();
+      if (sh_stop) break;
+    }
+  };
+  auto share = [&](int v) {                      // thread 0's value, for everybody
+    __syncthreads();
+    if (tid == 0) sh_int = v;
+    __syncthreads();
+    return sh_int;
+  };
+  // (src/sampler.c:271-332, as narrow_and_draw above; only thread 0's numbers mean anything)
+  float sum = 0.f;
+  walk(keep, [&](int, float p) { sum += p; return false; });
+  const float tp = top_p[i], mp = min_p[i];
+  int kept = keep;
+  if (tp < 1.0f) {
+    float cum = 0.f;
+    int k1 = keep;
+    walk(keep, [&](int e, float p) {
+      cum += p / sum;
+      if (cum > tp) { k1 = e + 1; return true; }
+      return false;
+    });
+    kept = share(k1);
+  }
+  if (mp > 0.f) {
+    float floor_p = 0.f;
+    int n = 0;
+    walk(kept, [&](int e, float p) {
+      const float q = p / sum;
+      if (e == 0) floor_p = mp * q;
+      if (q >= floor_p) { n = e + 1; return false; }
+      return true;
+    });
+    kept = share(n > 0 ? n : 1);
+  }
+  float psum = 0.f;
+  walk(kept, [&](int, float p) { psum += p; return false; });
+  const float target = uniform[i] * psum;
+  float acc = 0.f;
+  int pick = kept - 1;
+  walk(kept, [&](int e, float p) {
+    acc += p;
+    if (target < acc) { pick = e; return true; }
+    return false;
+  });
+  if (tid == 0) out[rows[i]] = idx[pick];
+}
+
+// The workspace of the kernel above: floats and ints for `n_entries` rows of `n2` values each,
+// n2 the power of two that holds the vocabulary.
+extern "C" int kappai_sample_filtered_wide_n2(int V) {
+  int n2 = 1;
+  while (n2 < V) n2 <<= 1;
+  return n2;
+}
+
+// As kappai_sample_filtered, for any keep_n[i] up to the vocabulary; ws_val and ws_idx hold
+// n_entries * kappai_sample_filtered_wide_n2(V) values each.
+extern "C" int kappai_sample_filtered_wide(const float* logits, const int* rows, const int* keep_n,
+                                           const float* temperature, const float* top_p,
+                                           const float* min_p, const float* uniform, int* out,
+                                           int n_entries, int V, float* ws_val, int* ws_idx,
+                                           hipStream_t stream) {
+  if (n_entries <= 0) return 0;
+  if (V < 1 || V > (1 << 30) || ws_val == nullptr || ws_idx == nullptr)
+    return (int)hipErrorInvalidValue;
+  hipLaunchKernelGGL(sample_filtered_wide_kernel, dim3(n_entries), dim3(FILT_THREADS), 0, stream,
+                     logits, rows, keep_n, temperature, top_p, min_p, uniform, out, V,
+                     kappai_sample_filtered_wide_n2(V), ws_val, ws_idx);
+  KAPPAI_RETURN_LAUNCH_STATUS();
+}
+
 // rows[i] names the row of `logits` (and of `out`) that entry i samples for; keep_n[i] <= 1024.
 extern "C" int kappai_sample_filtered(const float* logits, const int* rows, const int* keep_n,
                                       const float* temperature, const float* top_p,

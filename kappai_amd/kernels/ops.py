@@ -195,8 +195,10 @@ class FragmentRows:
 
     def materialize(self) -> torch.Tensor:
         n, D = self.shape
-        return (self.data.view(D // 32, 4, 16, 8).permute(2, 0, 1, 3).reshape(16, D)[:n]
-                .contiguous())
+        out = torch.empty((n, D), dtype=self.dtype, device=self.device)
+        check(library("elementwise").kappai_rows_from_fragments(
+            _ptr(self.data), _ptr(out), _c_int(n), _c_int(D), _stream()), "rows_from_fragments")
+        return out
 
 
 FUSED_MAX_ROWS = 16        # rows of a decode step whose products fold norm and residual sum in
@@ -242,7 +244,7 @@ _NO_SCALE = (_vp(0), _c_int(0), _c_float(0.0))
 class AddInto:
     """Asks a product to add its result into ``resid`` (float32 [M, N], in place, in float32)
     instead of returning it (kappai fuses the residual sum into the product the same way,
-    src/recipe/graph_passes.c:455).  With ``norm_weight`` (and ``eps``) the RMSNorm that follows
+    src/recipe/graph_passes.c:135-163).  With ``norm_weight`` (and ``eps``) the RMSNorm that follows
     is folded in as well: the product hands back ``ScaledRows`` for the product after that norm.
     A product that cannot do it (more than 16 rows, float32 weights, ...) returns its result as
     always, and the caller goes on as without this."""
@@ -944,10 +946,11 @@ FILTER_MAX_KEEP = 1024     # candidates the filtered-sampling kernel can hold
 
 def sample_filtered(logits: torch.Tensor, rows: torch.Tensor, keep: torch.Tensor,
                     temperature: torch.Tensor, top_p: torch.Tensor, min_p: torch.Tensor,
-                    uniform: torch.Tensor, out: torch.Tensor) -> None:
+                    uniform: torch.Tensor, out: torch.Tensor, wide: bool = False) -> None:
     """For every entry i: draw a token for row ``rows[i]`` of ``logits`` from its ``keep[i]``
-    (at most 1024) largest logits after temperature, top-p and min-p, at ``uniform[i]``, and
-    write it to ``out[rows[i]]`` (int32)."""
+    largest logits after temperature, top-p and min-p, at ``uniform[i]``, and write it to
+    ``out[rows[i]]`` (int32).  ``keep[i]`` is at most ``FILTER_MAX_KEEP``, or, with ``wide``, any
+    number up to the vocabulary (a slower kernel that sorts whole rows in a workspace)."""
     _gpu("logits", logits, F32)
     _gpu("rows", rows, I32)
     _gpu("keep", keep, I32)
@@ -958,6 +961,16 @@ def sample_filtered(logits: torch.Tensor, rows: torch.Tensor, keep: torch.Tensor
         _gpu(name, t, F32)
         _need(t.shape == (n,), lambda: f"{name}: one value per entry")
     _need(keep.shape == (n,) and out.shape == (logits.shape[0],), "sample_filtered: table sizes")
+    if wide:
+        lib = library("sampling")
+        n2 = int(lib.kappai_sample_filtered_wide_n2(_c_int(logits.shape[1])))
+        ws_val = torch.empty((n, n2), dtype=F32, device=logits.device)
+        ws_idx = torch.empty((n, n2), dtype=I32, device=logits.device)
+        check(lib.kappai_sample_filtered_wide(
+            _ptr(logits), _ptr(rows), _ptr(keep), _ptr(temperature), _ptr(top_p), _ptr(min_p),
+            _ptr(uniform), _ptr(out), _c_int(n), _c_int(logits.shape[1]), _ptr(ws_val),
+            _ptr(ws_idx), _stream()), "sample_filtered_wide")
+        return
     check(library("sampling").kappai_sample_filtered(
         _ptr(logits), _ptr(rows), _ptr(keep), _ptr(temperature), _ptr(top_p), _ptr(min_p),
         _ptr(uniform), _ptr(out), _c_int(n), _c_int(logits.shape[1]), _stream()), "sample_filtered")

@@ -5,7 +5,8 @@ choice, the whole-vocabulary temperature draw, the repeat penalty and the draw f
 narrowed candidates (top-k, top-p, min-p; kappai's order of operations,
 src/sampler.c:218-332) run in HIP kernels on the logits where they lie; the draw's uniform
 number comes from the request's own random stream on the host, so that a request's tokens
-do not depend on what else is in the batch.  Only a top-k above 1024 is drawn on the host.
+do not depend on what else is in the batch.  A top-k above 1024 takes a slower kernel that
+sorts the whole row in a workspace of its own.
 """
 from __future__ import annotations
 
@@ -43,44 +44,6 @@ class RequestSampler:
         return self.recent[len(self.recent) - n:] if n else []
 
 
-def filtered_draw(logits: np.ndarray, p: SamplingParams, u: float) -> int:
-    """Host draw with top-k / top-p / min-p (src/sampler.c:218-332): candidates by
-    descending logit, softmax of logit/T in float32, top-p keeps the token that crosses the
-    mass, min-p is relative to the best, then an inverse-CDF draw over what is left."""
-    lg = np.asarray(logits, dtype=np.float32)
-    vocab = lg.shape[0]
-    if 0 < p.top_k < vocab:
-        keep = p.top_k
-    elif p.top_p < 1.0 or p.min_p > 0.0:
-        keep = min(vocab, FILTER_CAP)
-    else:
-        keep = vocab
-    if keep < vocab:
-        part = np.argpartition(-lg, keep - 1)[:keep]
-        order = part[np.argsort(-lg[part], kind="stable")]
-    else:
-        order = np.argsort(-lg, kind="stable")
-    vals = lg[order]
-    inv = np.float32(1.0) / np.float32(p.temperature)
-    e = np.exp(vals * inv - vals[0] * inv, dtype=np.float32)
-    cum = np.cumsum(e, dtype=np.float32)
-    total = cum[-1]
-    kept = len(e)
-    if p.top_p < 1.0:
-        over = np.nonzero(cum / total > np.float32(p.top_p))[0]
-        if over.size:
-            kept = int(over[0]) + 1
-    if p.min_p > 0.0:
-        floor = np.float32(p.min_p) * (e[0] / total)
-        ok = (e[:kept] / total) >= floor
-        n = int(np.argmin(ok)) if not ok.all() else kept
-        kept = n if n > 0 else 1
-    cum = np.cumsum(e[:kept], dtype=np.float32)
-    target = np.float32(u) * cum[-1]
-    i = int(np.searchsorted(cum, target, side="right"))
-    return int(order[min(i, kept - 1)])
-
-
 class Sampler:
     """Samples one token for each row of ``logits`` [n, vocab] (float32, on the GPU; changed
     in place where a repeat penalty applies)."""
@@ -112,29 +75,21 @@ class Sampler:
 
     @staticmethod
     def runs_on_device(samplers: Sequence[RequestSampler], vocab: int) -> bool:
-        """True when every row's token can be chosen without the host seeing the logits or the
-        row's earlier tokens: no repeat penalty, no narrowing beyond what the kernel holds."""
-        for s in samplers:
-            p = s.params
-            if p.repeat_penalty != 1.0:
-                return False
-            if not p.is_greedy() and p.is_filtered(vocab):
-                keep = p.top_k if 0 < p.top_k < vocab else min(vocab, FILTER_CAP)
-                if keep > ops.FILTER_MAX_KEEP:
-                    return False
-        return True
+        """True when every row's token can be chosen without the host seeing the row's earlier
+        tokens: no repeat penalty."""
+        return all(s.params.repeat_penalty == 1.0 for s in samplers)
 
     def launch(self, logits: torch.Tensor, samplers: Sequence[RequestSampler],
                out: Optional[torch.Tensor] = None):
-        """Queue the kernels that choose a token for every row; returns (int32 tokens on the GPU,
-        rows that the host still has to draw).  Nothing here waits for the GPU."""
+        """Queue the kernels that choose a token for every row; returns the int32 tokens on the
+        GPU.  Nothing here waits for the GPU."""
         with profile.scope("sample"):
             return self._launch(logits, samplers, out)
 
     def _launch(self, logits, samplers, out):
         n, vocab = logits.shape
         dev = logits.device
-        temps, unis, host_rows, filt = [], [], [], []
+        temps, unis, filt, wide = [], [], [], []
         for i, s in enumerate(samplers):
             p = s.params
             if p.is_greedy():
@@ -144,16 +99,17 @@ class Sampler:
                 temps.append(0.0)            # the kernel's choice for this row is replaced
                 unis.append(0.0)
                 keep = p.top_k if 0 < p.top_k < vocab else min(vocab, FILTER_CAP)
-                if keep <= ops.FILTER_MAX_KEEP:
-                    filt.append((i, keep, float(p.temperature), float(p.top_p), float(p.min_p),
-                                 s.rng.uniform()))
-                else:
-                    host_rows.append(i)
+                (filt if keep <= ops.FILTER_MAX_KEEP else wide).append(
+                    (i, keep, float(p.temperature), float(p.top_p), float(p.min_p),
+                     s.rng.uniform()))
             else:
                 temps.append(float(p.temperature))
                 unis.append(s.rng.uniform())
         # every per-row number goes to the GPU in ONE copy: [temperature | uniform] for all
         # rows, then [row | keep | temperature | top_p | min_p | uniform] for the narrowed ones
+        # (those that keep more than the kernel for narrowed rows holds come last)
+        mf = len(filt)
+        filt = filt + wide
         m = len(filt)
         if not any(temps) and not m and (n, str(dev)) in self._zeros:
             out_dev = ops.sample_rows(logits, *self._zeros[(n, str(dev))], out=out)
@@ -175,9 +131,12 @@ class Sampler:
             if m:
                 di = d[2 * n:2 * n + 2 * m].view(torch.int32)
                 f = d[2 * n + 2 * m:]
-                ops.sample_filtered(logits, di[:m], di[m:], f[:m], f[m:2 * m], f[2 * m:3 * m],
-                                    f[3 * m:4 * m], out_dev)
-        return out_dev, host_rows
+                cols = (di[:m], di[m:], f[:m], f[m:2 * m], f[2 * m:3 * m], f[3 * m:4 * m])
+                if mf:
+                    ops.sample_filtered(logits, *(c[:mf] for c in cols), out_dev)
+                if m > mf:
+                    ops.sample_filtered(logits, *(c[mf:] for c in cols), out_dev, wide=True)
+        return out_dev
 
     def sample(self, logits: torch.Tensor, samplers: Sequence[RequestSampler]) -> List[int]:
         n, vocab = logits.shape
@@ -198,10 +157,4 @@ class Sampler:
                 logits, torch.tensor(starts, dtype=torch.int32, device=dev),
                 torch.tensor(toks or [0], dtype=torch.int32, device=dev),
                 torch.tensor(pens, dtype=torch.float32, device=dev))
-        out_dev, host_rows = self.launch(logits, samplers)
-        out = out_dev.tolist()
-        if host_rows:
-            rows = logits[torch.tensor(host_rows, device=dev)].cpu().numpy()
-            for row, i in zip(rows, host_rows):
-                out[i] = filtered_draw(row, samplers[i].params, samplers[i].rng.uniform())
-        return [int(t) for t in out]
+        return [int(t) for t in self.launch(logits, samplers).tolist()]

@@ -78,6 +78,35 @@ def test_sampled_float32_tiny_b_in_portions(model_dirs):
         assert g == want, (i, g, want)
 
 
+def test_every_way_of_drawing_in_one_batch():
+    """One batch of rows that each draw differently (greedy, the whole vocabulary, narrowed to a
+    few, a top-k above what the kernel for narrowed rows holds, a repeat penalty) over several
+    steps, every row against a plain sampler of its own with the same seed: a row's tokens do not
+    depend on what its neighbours ask for."""
+    import torch
+    from kappai_amd.sampling import RequestSampler, Sampler, SamplingParams
+    V = 3001
+    opts = [dict(temperature=0.0), dict(temperature=0.9, top_k=0, top_p=1.0, min_p=0.0),
+            dict(temperature=0.8, top_k=40, top_p=0.9, min_p=0.1),
+            dict(temperature=1.5, top_k=2000, top_p=0.98, min_p=0.0),
+            dict(temperature=1.1, top_k=1500, top_p=1.0, min_p=0.001),
+            dict(temperature=0.7, top_k=12, top_p=1.0, min_p=0.0, repeat_penalty=1.3, repeat_last_n=4),
+            dict(temperature=2.0, top_k=3000, top_p=1.0, min_p=0.0)]
+    ours = [RequestSampler(SamplingParams(seed=11 + i, **o)) for i, o in enumerate(opts)]
+    plain = [S.PlainSampler(11 + i, **{"top_k": 40, "top_p": 0.9, "min_p": 0.1, **o})
+             for i, o in enumerate(opts)]
+    sampler = Sampler()
+    rng = np.random.default_rng(8)
+    for step in range(6):
+        logits = (rng.normal(size=(len(opts), V)) * 2.5).astype(np.float32)
+        got = sampler.sample(torch.from_numpy(logits).to("cuda:0"), ours)
+        for i, tok in enumerate(got):
+            want = plain[i].sample(logits[i].copy())
+            assert tok == want, (step, i, opts[i], tok, want)
+            ours[i].observe([tok])
+            plain[i].observe(tok)
+
+
 def test_default_options_and_repeat_penalty(model_dirs):
     """kappai's default options (top-k 40, top-p 0.9, min-p 0.1) and a repeat penalty."""
     from kappai_amd.engine import Engine

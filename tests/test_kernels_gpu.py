@@ -1097,6 +1097,49 @@ def test_sample_filtered(ops):
                 assert logits[r, got[r]] == logits[r, want[r]], (V, r, got[r], want[r])
 
 
+def test_sample_filtered_with_a_top_k_above_what_lds_holds(ops):
+    """A top-k above 1024 (the kernel that sorts the whole row in a workspace) against the plain
+    sampler: vocabularies below and above a power of two and above the 4096 values that one pass
+    of its sort holds in LDS, top-k just above the other kernel's limit and just below the
+    vocabulary, with and without top-p and min-p, ties at the edge of the top-k."""
+    from plain import sampler as plain_sampler
+    rng = np.random.default_rng(6)
+    for V in (1500, 4096, 5000, 65536, 70001):
+        opts = [(0.8, 1025, 0.9, 0.1), (1.3, V - 1, 1.0, 0.0), (0.5, 1400, 0.6, 0.0),
+                (1.0, V - 3, 1.0, 0.3), (2.0, 1200, 0.999, 0.0), (5.0, V - 1, 0.9999, 0.0)]
+        n = len(opts)
+        logits = (rng.normal(size=(n, V)) * 3).astype(np.float32)
+        logits[0, 1000:1100] = logits[0].max() + 1.0       # equal values across the top-k edge
+        logits[2] = np.round(logits[2] * 4) / 4            # ties everywhere
+        rows, keep, temp, tp, mp, uni, want = [], [], [], [], [], [], {}
+        for r, (t, k, p, m) in enumerate(opts):
+            u = float(np.float32(rng.random()))
+            rows.append(r); keep.append(k); temp.append(t); tp.append(p); mp.append(m); uni.append(u)
+            want[r] = plain_sampler.sample_filtered(logits[r], t, k, p, m, u)
+        out = torch.full((n,), -1, dtype=torch.int32, device=DEV)
+        f32 = lambda v: torch.tensor(v, dtype=torch.float32, device=DEV)
+        i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=DEV)
+        ops.sample_filtered(torch.from_numpy(logits).to(DEV), i32(rows), i32(keep), f32(temp),
+                            f32(tp), f32(mp), f32(uni), out, wide=True)
+        got = out.cpu().tolist()
+        for r in range(n):
+            if got[r] != want[r]:
+                # equal logits may be ordered differently: the pick must then have the same value
+                assert logits[r, got[r]] == logits[r, want[r]], (V, r, got[r], want[r])
+    # the two kernels agree where both can run
+    V = 3000
+    logits = torch.from_numpy((rng.normal(size=(8, V)) * 2).astype(np.float32)).to(DEV)
+    args = (torch.arange(8, dtype=torch.int32, device=DEV),
+            torch.tensor([1, 2, 40, 64, 65, 500, 1024, 1000], dtype=torch.int32, device=DEV),
+            torch.full((8,), 0.9, device=DEV), torch.full((8,), 0.95, device=DEV),
+            torch.full((8,), 0.02, device=DEV), torch.rand(8, generator=torch.Generator().manual_seed(2)).to(DEV))
+    a = torch.full((8,), -1, dtype=torch.int32, device=DEV)
+    b = torch.full((8,), -1, dtype=torch.int32, device=DEV)
+    ops.sample_filtered(logits, *args, a)
+    ops.sample_filtered(logits, *args, b, wide=True)
+    assert a.tolist() == b.tolist()
+
+
 def test_repeat_penalty(ops):
     logits = torch.tensor([[1.0, 0.9, 0.0, -1.0], [2.0, -2.0, 0.5, 0.0]])
     row_start = torch.tensor([0, 3, 4], dtype=torch.int32)
