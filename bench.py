@@ -342,16 +342,14 @@ def kernel_rates(model, cfg, batch, context, prefill_tokens, page_size, device, 
     # K3: products of a decode step
     gu = [f.gate_up for f in ffs]
     if all(f.fused for f in ffs):
-        t = graph_time(lambda i: ops.linear_swiglu(x, gu[i % n].weight,
-                                                   weight_frag=gu[i % n].weight_frag), 2 * n)
+        t = graph_time(lambda i: ops.linear_swiglu(x, gu[i % n].weight), 2 * n)
         rate_gbs("k3_decode_gate_up", t, gu[0].weight_bytes())
     dn = [f.down for f in ffs]
     t = graph_time(lambda i: dn[i % n].forward(act, add_into=ops.AddInto(resid)), 2 * n)
     rate_gbs("k3_decode_down", t, dn[0].weight_bytes())
     if convs:
         ip = [c.in_proj for c in convs]
-        t = graph_time(lambda i: ops.linear(x, ip[i % len(ip)].weight,
-                                            weight_frag=ip[i % len(ip)].weight_frag), 2 * len(ip))
+        t = graph_time(lambda i: ops.linear(x, ip[i % len(ip)].weight), 2 * len(ip))
         rate_gbs("k3_decode_in_proj", t, ip[0].weight_bytes())
     # K11: the output head on `batch` rows
     head = model.head.linear

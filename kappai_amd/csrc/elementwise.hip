@@ -16,11 +16,40 @@ __global__ void embed_rows_kernel(const int* __restrict__ ids, const TW* __restr
   for (int i = threadIdx.x; i < D; i += blockDim.x) dst[i] = to_f32(src[i]);
 }
 
+// The same from a bfloat16 table that is kept in the order of the matrix cores' fragments (a
+// tied output head's matrix, see gemm.hip: pieces of 16 rows x 32 columns, a lane's 8 values at
+// lane = (column % 32) / 8 * 16 + row % 16); D a multiple of 32.
+__global__ void embed_rows_fragments_kernel(const int* __restrict__ ids,
+                                            const bf16_t* __restrict__ table,
+                                            float* __restrict__ out, int D) {
+  const int t = blockIdx.x;
+  const size_t r = (size_t)ids[t];
+  const bf16_t* src = table + (r / 16) * 16 * D + (r % 16) * 8;
+  float* dst = out + (size_t)t * D;
+  // a thread takes 8 neighbouring columns: 16 bytes of the piece, 32 bytes of the row
+  for (int c = threadIdx.x; c < D / 8; c += blockDim.x) {
+    const uint4 v = *reinterpret_cast<const uint4*>(src + (size_t)(c / 4) * 512 + (c % 4) * 128);
+    const uint32_t u[4] = {v.x, v.y, v.z, v.w};
+    float4 lo, hi;
+    lo.x = __uint_as_float(u[0] << 16), lo.y = __uint_as_float(u[0] & 0xffff0000u);
+    lo.z = __uint_as_float(u[1] << 16), lo.w = __uint_as_float(u[1] & 0xffff0000u);
+    hi.x = __uint_as_float(u[2] << 16), hi.y = __uint_as_float(u[2] & 0xffff0000u);
+    hi.z = __uint_as_float(u[3] << 16), hi.w = __uint_as_float(u[3] & 0xffff0000u);
+    *reinterpret_cast<float4*>(dst + 8 * c) = lo;
+    *reinterpret_cast<float4*>(dst + 8 * c + 4) = hi;
+  }
+}
+
+// table_is_bf16: 0 = float32 rows, 1 = bfloat16 rows, 2 = bfloat16 in fragment order
 extern "C" int kappai_embed_rows(const int* ids, const void* table, int table_is_bf16, float* out,
                                  int T, int D, hipStream_t stream) {
   if (T <= 0) return 0;
   const int threads = D >= 1024 ? 256 : (D >= 256 ? 128 : 64);
-  if (table_is_bf16)
+  if (table_is_bf16 == 2) {
+    if (D % 32 || ((uintptr_t)table % 16) || ((uintptr_t)out % 16)) return (int)hipErrorInvalidValue;
+    hipLaunchKernelGGL(embed_rows_fragments_kernel, dim3(T), dim3(threads), 0, stream, ids,
+                       (const bf16_t*)table, out, D);
+  } else if (table_is_bf16)
     hipLaunchKernelGGL(embed_rows_kernel<bf16_t>, dim3(T), dim3(threads), 0, stream, ids,
                        (const bf16_t*)table, out, D);
   else

@@ -83,8 +83,8 @@ typedef struct kappai_attention_kernels {
 
 // ---- the model --------------------------------------------------------------------------------
 typedef struct kappai_linear {
-  const void* w;        // [n, k], bfloat16 or float32
-  const void* w_frag;   // the bfloat16 matrix once more in fragment order, or null
+  const void* w;        // [n, k], bfloat16 or float32; null when the matrix is kept in w_frag only
+  const void* w_frag;   // the bfloat16 matrix in fragment order, or null
   const float* bias;    // [n] or null
   int n, k;
   int w_is_f32;
@@ -135,7 +135,7 @@ typedef struct kappai_model {
   int compute_bf16;                 // activations and cache in bfloat16 (else float32)
   int width, vocab, page_size;
   const void* embed_table;          // [vocab, width]
-  int embed_is_bf16;
+  int embed_is_bf16;                // 0: float32 rows, 1: bfloat16 rows, 2: bfloat16 in fragment order
   int n_calls;
   const kappai_layer_call* calls;
   kappai_norm final_norm;

@@ -266,6 +266,13 @@ Carry linear(Ctx& c, Rows x, const kappai_linear& lin, int out_bf16, bool partia
   const bool scaled = x.ss != nullptr;
   if (!(K % 8 == 0 && lda % 8 == 0 && aligned16(xb) && aligned16(lin.w))) {
     // the matrix-core kernels read 16 bytes at a time; anything else goes the plain way
+    if (lin.w == nullptr) {
+      snprintf(g_error, sizeof g_error, "kappai_forward: a matrix kept in fragment order met "
+                                        "rows that are not 16-byte aligned (K = %d, row stride %d)",
+               K, lda);
+      c.status = (int)hipErrorInvalidValue;
+      return out;
+    }
     if (scaled || x.frag) {
       snprintf(g_error, sizeof g_error, "kappai_forward: rows in kernel order reached the plain "
                                         "product kernel (K = %d)", K);
@@ -627,9 +634,11 @@ int run(const kappai_model* m, const kappai_batch* b, Arena& arena, float* logit
         LAUNCH(c, k.gemm_bf16(xh, head.w, head.w_frag, head.bias, logits, n, head.n, D, D, head.n,
                               1, 0, 1, xb.frag, nullptr, 0, 0.f, nullptr, 0, nullptr, nullptr, 0,
                               nullptr, stream));
-      else
+      else if (head.w != nullptr)
         LAUNCH(c, k.gemm_bf16_any(xh, head.w, head.bias, logits, n, head.n, D, D, head.n, 1,
                                   stream));
+      else
+        c.status = (int)hipErrorInvalidValue;    // (a matrix in fragment order has D % 32 == 0)
     }
   }
   if (arena.overflow) {

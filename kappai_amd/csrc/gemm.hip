@@ -163,7 +163,7 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * WAVE)
     __attribute__((amdgpu_waves_per_eu(OCC, OCC))) void gemm_bf16_tile_kernel(
         const bf16_t* __restrict__ A, const bf16_t* __restrict__ W,
         const float* __restrict__ bias, TO* __restrict__ C, int M, int N, int K, int lda, int ldc,
-        int tiles_n) {
+        int tiles_n, int w_frag) {
   constexpr int BM = WAVES_M * WM * 32, BN = WAVES_N * WN * 32;
   constexpr int LDS_STRIDE = BK + 8;   // in bf16: rows stay 16-byte aligned, banks are spread
   constexpr int THREADS = WAVES_M * WAVES_N * WAVE;
@@ -209,7 +209,12 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * WAVE)
     for (int c = 0; c < W_CHUNKS; ++c) {
       const int idx = tid + c * THREADS;
       const int r = chunk_row(idx), gk = k0 + chunk_col(idx);
-      rw[c] = (n0 + r < N && gk < kend) ? load16(W + (size_t)(n0 + r) * K + gk) : zero;
+      // (w_frag: W in fragment order, see gemm_bf16_skinny_kernel: the chunk of row n0 + r at gk)
+      const size_t wr = (size_t)(n0 + r);
+      const bf16_t* wp = w_frag ? W + (wr / 16) * 16 * K + (size_t)(gk / 32) * 512 +
+                                      (((gk % 32) / 8) * 16 + wr % 16) * 8
+                                : W + wr * K + gk;
+      rw[c] = (n0 + r < N && gk < kend) ? load16(wp) : zero;
     }
   };
   auto stage = [&](int buf) {
@@ -310,7 +315,7 @@ template <typename TO, int EPI, int WAVES_M, int WAVES_N, int WM, int WN, int BK
           int OCC>
 static void launch_tile_cfg(const bf16_t* A, const bf16_t* W, const float* bias, TO* C, int M,
                             int n_rows_w, int K, int lda, int ldc, int ksplit,
-                            hipStream_t stream) {
+                            hipStream_t stream, int w_frag = 0) {
   constexpr int BM = WAVES_M * WM * 32, BN = WAVES_N * WN * 32;
   constexpr size_t lds_bytes = (size_t)NBUF * (BM + BN) * (BK + 8) * sizeof(bf16_t);
   auto kern = gemm_bf16_tile_kernel<TO, EPI, WAVES_M, WAVES_N, WM, WN, BK, NBUF, OCC>;
@@ -322,7 +327,7 @@ static void launch_tile_cfg(const bf16_t* A, const bf16_t* W, const float* bias,
   }
   const int tn = (n_rows_w + BN - 1) / BN, tm = (M + BM - 1) / BM;
   hipLaunchKernelGGL(kern, dim3(tm * tn, ksplit), dim3(WAVES_M * WAVES_N * WAVE), lds_bytes,
-                     stream, A, W, bias, C, M, n_rows_w, K, lda, ldc, tn);
+                     stream, A, W, bias, C, M, n_rows_w, K, lda, ldc, tn, w_frag);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -355,7 +360,7 @@ template <typename TO, int EPI, int WT, bool DEEP = false, int WN_ = 0>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4 / WT, 4 / WT)))
 void gemm_bf16_block256_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W,
                                const float* __restrict__ bias, TO* __restrict__ C, int M, int N,
-                               int K, int lda, int ldc, int tiles_n) {
+                               int K, int lda, int ldc, int tiles_n, int w_frag) {
   // WTM x WTN accumulator tiles of 32 x 32 a wave (WTN = WT unless WN_ is given): 4 x 4 ->
   // 256 x 256 blocks, 2 x 2 -> 128 x 128, 4 x 3 -> 256 rows x 192 columns (for a product whose
   // 256 x 256 blocks would leave a quarter of the chip without one)
@@ -391,9 +396,17 @@ void gemm_bf16_block256_kernel(const bf16_t* __restrict__ A, const bf16_t* __res
   // receives the row's chunk (lane%8) ^ ((row/2)%8).  Waves 0, 1 bring the A tile, waves 2, 3 the W
   // tile, NLOAD instructions each; rows past the end of the matrix repeat its last row (their
   // products are never stored).
+  //
+  // w_frag: W lies in fragment order ([rows / 16][K / 32] pieces of 16 rows x 32 of K, 1 KB each,
+  // the lane's 16 bytes at lane = (k % 32) / 8 * 16 + row % 16; see gemm_bf16_skinny_kernel).  A
+  // load instruction of the W waves then brings one piece, instruction i the piece (16 rows
+  // number i / 2 of the wave's rows, 32 of K number i % 2 of the tile), which lands in LDS as it
+  // lies in memory: a fragment read (16 lanes = 16 rows of one group of 8 of K = 256 contiguous
+  // bytes) is free of bank conflicts without a permutation.
   const bool brings_a = wave < 2;
+  const bool frag_w = !brings_a && w_frag;
   const char* gk = reinterpret_cast<const char*>(brings_a ? A : W) +
-                   (size_t)blockIdx.y * kblk * sizeof(bf16_t);
+                   (size_t)blockIdx.y * kblk * (frag_w ? 16 : 1) * sizeof(bf16_t);
   const int ld = brings_a ? lda : K;
   const int last_row = (brings_a ? M : N) - 1;
   const int row0 = brings_a ? m0 + wave * WROWS_M : n0 + (wave - 2) * WROWS_N;
@@ -406,12 +419,17 @@ void gemm_bf16_block256_kernel(const bf16_t* __restrict__ A, const bf16_t* __res
     const int lchunk = (lane % 8) ^ (((i * 8 + lrow) >> 1) & 7);
     roff[i] = (uint32_t)(min(row0 + i * 8 + lrow, last_row) * ld + lchunk * 8) *
               (uint32_t)sizeof(bf16_t);
+    if (frag_w)
+      roff[i] = (uint32_t)(min(row0 / 16 + i / 2, last_row / 16) * 16 * K + (i % 2) * 512 +
+                           lane * 8) * (uint32_t)sizeof(bf16_t);
   }
+  // bytes from one tile of 64 of K to the next: a row's 128 bytes, or two pieces
+  const uint32_t kstep = frag_w ? 2048u : (uint32_t)(BK * sizeof(bf16_t));
   // the address of a load is a wave-uniform 64-bit base (the tile's first column) plus the
   // lane's 32-bit row offset; pinning the base into scalar registers keeps the compiler from
   // folding the two into sixteen 64-bit per-lane pointers
   auto tile_base = [&](int kt) {
-    const uint64_t p = reinterpret_cast<uint64_t>(gk) + (uint64_t)kt * (BK * sizeof(bf16_t));
+    const uint64_t p = reinterpret_cast<uint64_t>(gk) + (uint64_t)kt * kstep;
     const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)p);
     const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(p >> 32));
     return reinterpret_cast<const char*>(((uint64_t)hi << 32) | lo);
@@ -429,6 +447,9 @@ void gemm_bf16_block256_kernel(const bf16_t* __restrict__ A, const bf16_t* __res
   for (int s = 0; s < 4; ++s) {
     aoff[s] = (wm * WROWS_M + r_in) * BK + (((s * 2 + hh) ^ ((r_in >> 1) & 7)) * 8);
     woff[s] = A_TILE + (wn * WROWS_N + r_in) * BK + (((s * 2 + hh) ^ ((r_in >> 1) & 7)) * 8);
+    if (w_frag)     // piece (r_in / 16, s / 2) of the wave's rows, group (s % 2) * 2 + hh of its K
+      woff[s] = A_TILE + wn * WROWS_N * BK + ((r_in / 16) * 2 + s / 2) * 512 +
+                (((s % 2) * 2 + hh) * 16 + r_in % 16) * 8;
   }
   bf16x8_t fa[2][WTM], fw[2][WTN];
   // in the order the products ask for them: w0 a0, the other w, the other a
@@ -664,7 +685,7 @@ static bool block256_fits(const bf16_t* A, const bf16_t* W, TO* C, int M, int n_
 template <typename TO, int EPI, int WT, bool DEEP = false, int WN_ = 0>
 static void launch_block256(const bf16_t* A, const bf16_t* W, const float* bias, TO* C, int M,
                             int n_rows_w, int K, int lda, int ldc, int ksplit,
-                            hipStream_t stream) {
+                            hipStream_t stream, int w_frag = 0) {
   constexpr int B = WT * 64, BN = (WN_ ? WN_ : WT) * 64;       // block: B rows x BN columns
   constexpr size_t lds_bytes = (DEEP ? 4 : 2) * (B + BN) * 64 * sizeof(bf16_t);
   auto kern = gemm_bf16_block256_kernel<TO, EPI, WT, DEEP, WN_>;
@@ -676,7 +697,7 @@ static void launch_block256(const bf16_t* A, const bf16_t* W, const float* bias,
   }
   const int tn = (n_rows_w + BN - 1) / BN, tm = (M + B - 1) / B;
   hipLaunchKernelGGL(kern, dim3(tm * tn, ksplit), dim3(256), lds_bytes, stream, A, W, bias, C, M,
-                     n_rows_w, K, lda, ldc, tn);
+                     n_rows_w, K, lda, ldc, tn, w_frag);
 }
 
 // The 256 x 256 form (one block a CU, 40-55 us per round of up to 256 blocks at K = 2048) against
@@ -697,7 +718,7 @@ static bool use_256_form(long blocks256) {
 template <typename TO, int EPI>
 static void launch_tile(const bf16_t* A, const bf16_t* W, const float* bias, TO* C, int M,
                         int n_rows_w, int K, int lda, int ldc, int ksplit, int shape,
-                        hipStream_t stream) {
+                        hipStream_t stream, const bf16_t* Wf = nullptr) {
   const bool fits = EPI != 2 && block256_fits<TO, EPI>(A, W, C, M, n_rows_w, K, lda, ldc, ksplit);
   if (shape == 0) {
     const int big = ((M + 255) / 256) * ((n_rows_w + 127) / 128) * ksplit;
@@ -722,39 +743,46 @@ static void launch_tile(const bf16_t* A, const bf16_t* W, const float* bias, TO*
   }
   if ((shape == 5 || shape == 6 || shape == 8 || shape == 9) && !fits) shape = 3;
   if (shape == 9 && EPI != 0) shape = 5;
+  // Wf: W in fragment order (W may then be null).  The one-wave-a-SIMD kernel reads it faster
+  // than rows (gate/up of 2048 rows 122 against 135 us, in_proj 50 against 56: a tile's loads
+  // are pieces of 1 KB), the older tile kernel a little slower (47 against 43 us), so that one
+  // takes the rows when there are any.
+  const bool block_form = shape == 5 || shape == 6 || shape == 8 || shape == 9;
+  const int w_frag = Wf != nullptr && (W == nullptr || block_form);
+  if (w_frag) W = Wf;
   switch (shape) {
     case 5:
       if constexpr (EPI != 2)
-        launch_block256<TO, EPI, 4>(A, W, bias, C, M, n_rows_w, K, lda, ldc, ksplit, stream);
+        launch_block256<TO, EPI, 4>(A, W, bias, C, M, n_rows_w, K, lda, ldc, ksplit, stream, w_frag);
       break;
     case 6:
       if constexpr (EPI != 2)
-        launch_block256<TO, EPI, 2>(A, W, bias, C, M, n_rows_w, K, lda, ldc, ksplit, stream);
+        launch_block256<TO, EPI, 2>(A, W, bias, C, M, n_rows_w, K, lda, ldc, ksplit, stream, w_frag);
       break;
     case 8:
       if constexpr (EPI != 2)
-        launch_block256<TO, EPI, 2, true>(A, W, bias, C, M, n_rows_w, K, lda, ldc, ksplit, stream);
+        launch_block256<TO, EPI, 2, true>(A, W, bias, C, M, n_rows_w, K, lda, ldc, ksplit, stream, w_frag);
       break;
     case 9:
       if constexpr (EPI == 0)
         launch_block256<TO, EPI, 4, false, 3>(A, W, bias, C, M, n_rows_w, K, lda, ldc, ksplit,
-                                              stream);
+                                              stream, w_frag);
       break;
     case 1:
       launch_tile_cfg<TO, EPI, 1, 2, 4, 2, 32, 2, 2>(A, W, bias, C, M, n_rows_w, K, lda, ldc, ksplit,
-                                                  stream);
+                                                  stream, w_frag);
       break;
     case 2:
       launch_tile_cfg<TO, EPI, 2, 2, 4, 2, 32, 2, 2>(A, W, bias, C, M, n_rows_w, K, lda, ldc, ksplit,
-                                                  stream);
+                                                  stream, w_frag);
       break;
     case 3:
       launch_tile_cfg<TO, EPI, 2, 2, 4, 2, 64, 1, 2>(A, W, bias, C, M, n_rows_w, K, lda, ldc, ksplit,
-                                                  stream);
+                                                  stream, w_frag);
       break;
     default:
       launch_tile_cfg<TO, EPI, 2, 2, 4, 4, 64, 2, 1>(A, W, bias, C, M, n_rows_w, K, lda, ldc, ksplit,
-                                                  stream);
+                                                  stream, w_frag);
       break;
   }
 }
@@ -1498,8 +1526,7 @@ static int launch_bf16(const bf16_t* A, const bf16_t* W, const float* bias, TO* 
     KAPPAI_RETURN_LAUNCH_STATUS();
   }
   if (fuse.rsc.ss != nullptr && ksplit != 1) return (int)hipErrorInvalidValue;
-  // Wf: W once more in fragment order, for the kernels of 1 to 64 rows (see the first of them);
-  // the others read W
+  // Wf: W in fragment order (see the kernel for 1 to 16 rows); W may be null when Wf is there
   // N counts output columns; with the SwiGLU epilogue W has 2N rows
   // a very wide plain product (the output head) with more than 32 rows streams faster through
   // the 128 x 128 blocks than through the decode kernel, which reads the rows once per 32 columns
@@ -1544,7 +1571,7 @@ static int launch_bf16(const bf16_t* A, const bf16_t* W, const float* bias, TO* 
     // rows of W = columns the tiles run over
     launch_tile<TO, EPI>(A, W, bias, C, M, EPI == 1 ? 2 * N : N, K, lda, ldc, ksplit,
                          force_kernel >= 3 ? force_kernel - 2 : (wide_head && M <= 64 ? 6 : 0),
-                         stream);
+                         stream, Wf);
   }
   KAPPAI_RETURN_LAUNCH_STATUS();
 }
@@ -1554,7 +1581,8 @@ static int launch_bf16(const bf16_t* A, const bf16_t* W, const float* bias, TO* 
 // with block shape 1..6 (see launch_tile), 9 = shared-rows kernel (17 to 64 rows, K / ksplit a
 // multiple of 512), 10 = block shape 8, 11 = block shape 9; for tests and tuning.
 // ksplit > 1 (float output only): C is [ksplit][M][ldc] partial sums over K ranges.
-// W_frag: null, or W again in fragment order (K a multiple of 32, rows a multiple of 16).
+// W_frag: null, or W in fragment order (K a multiple of 32, rows a multiple of 16); W may then
+// be null: every kernel reads the fragment order (only kappai_gemm_bf16_any needs rows).
 static bool frag_ok(const void* W_frag, int rows, int K) {
   return W_frag == nullptr || (K % 32 == 0 && rows % 16 == 0 && ((uintptr_t)W_frag % 16) == 0);
 }

@@ -127,9 +127,10 @@ def _tensor_ptr(t: Optional[torch.Tensor]):
 
 def _linear(lin) -> LinearDesc:
     w = lin.weight
-    frag = lin.weight_frag
-    return LinearDesc(w.data_ptr(), _tensor_ptr(frag), _tensor_ptr(lin.bias), w.shape[0],
-                      w.shape[1], 1 if w.dtype == torch.float32 else 0)
+    in_fragments = isinstance(w, ops.InFragments)
+    return LinearDesc(None if in_fragments else w.data_ptr(), w.data_ptr() if in_fragments else None,
+                      _tensor_ptr(lin.bias), w.shape[0], w.shape[1],
+                      1 if w.dtype == torch.float32 else 0)
 
 
 class Workspace:
@@ -235,8 +236,10 @@ class CForward:
         m = ModelDesc()
         m.abi, m.compute_bf16 = ENGINE_ABI, 1 if bf16 else 0
         m.width, m.vocab, m.page_size = model.embedding.width, model.vocab_size, cache.page_size
-        m.embed_table = model.embedding.table.data_ptr()
-        m.embed_is_bf16 = 1 if model.embedding.table.dtype == torch.bfloat16 else 0
+        table = model.embedding.table
+        m.embed_table = table.data_ptr()
+        m.embed_is_bf16 = (2 if isinstance(table, ops.InFragments)
+                           else 1 if table.dtype == torch.bfloat16 else 0)
         m.n_calls, m.calls = len(model.schedule), calls
         m.final_norm = NormDesc(model.final_norm.weight.data_ptr(), model.final_norm.eps)
         m.head = _linear(model.head.linear)

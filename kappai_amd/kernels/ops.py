@@ -70,14 +70,18 @@ def _is_bf16(dtype) -> int:
 
 # ---------------------------------------------------------------------------------------
 def embed_rows(ids: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
-    """float32 [T, D] rows of ``table`` ([V, D], float32 or bfloat16) at ``ids`` (int32)."""
+    """float32 [T, D] rows of ``table`` ([V, D], float32 or bfloat16, or ``InFragments``: a tied
+    output head's matrix) at ``ids`` (int32)."""
     _gpu("ids", ids, I32)
-    _gpu("table", table, (F32, BF16))
+    kind = 2 if isinstance(table, InFragments) else None
+    if kind is None:
+        _gpu("table", table, (F32, BF16))
+        kind = _is_bf16(table.dtype)
     _need(ids.dim() == 1 and table.dim() == 2, "embed_rows: ids [T], table [V, D]")
     T, D = ids.shape[0], table.shape[1]
     out = torch.empty((T, D), dtype=F32, device=table.device)
     check(library("elementwise").kappai_embed_rows(
-        _ptr(ids), _ptr(table), _c_int(_is_bf16(table.dtype)), _ptr(out), _c_int(T), _c_int(D),
+        _ptr(ids), _ptr(table), _c_int(kind), _ptr(out), _c_int(T), _c_int(D),
         _stream()), "embed_rows")
     return out
 
@@ -324,9 +328,11 @@ def fragment_order(weight: torch.Tensor) -> Optional[torch.Tensor]:
     """A copy of a bfloat16 matrix [N, K] in the order in which the product kernel for 1 to 16
     rows loads it: pieces of 16 rows x 32 of K, each laid out lane by lane ([N / 16][K / 32]
     [(k % 32) / 8][row % 16][8 values]), so that one load instruction of a wave reads 1 KB in
-    one piece.  None when the shape does not allow it (N a multiple of 16, K of 32).  The
-    products take it beside the matrix itself (``weight_frag``); the kernels for more rows read
-    the matrix as it is."""
+    one piece.  None when the shape does not allow it (N a multiple of 16, K of 32).  Every
+    product kernel for bfloat16 reads a matrix in this order (the kernels for few rows 10-20 %
+    faster than rows, the block kernels for prompts up to 10 %: a tile's 64 of K of 16 rows are
+    2 KB in two pieces instead of 16 pieces of 128 bytes), so a matrix is kept in this order
+    only: ``InFragments``."""
     if weight.dtype != BF16 or weight.dim() != 2:
         return None
     N, K = weight.shape
@@ -336,15 +342,68 @@ def fragment_order(weight: torch.Tensor) -> Optional[torch.Tensor]:
             .contiguous().view(N, K))
 
 
-def _frag(weight: torch.Tensor, weight_frag: Optional[torch.Tensor]) -> _vp:
+class InFragments:
+    """A bfloat16 matrix [N, K] of which only ``fragment_order(matrix)`` is kept.  ``linear``,
+    ``linear_swiglu``, ``linear_shortconv_step`` and ``embed_rows`` take it in place of the
+    matrix; it has the matrix's ``shape`` and ``dtype``.  ``rows(n)``: its first ``n`` rows (a
+    multiple of 16), sharing the memory."""
+
+    def __init__(self, data: torch.Tensor):
+        _gpu("fragments", data, BF16)
+        _need(data.dim() == 2 and data.shape[0] % 16 == 0 and data.shape[1] % 32 == 0
+              and data.data_ptr() % 16 == 0,
+              lambda: f"fragments: [N, K] with N a multiple of 16 and K of 32, got {tuple(data.shape)}")
+        self.data = data
+        self.shape, self.dtype, self.device = data.shape, data.dtype, data.device
+
+    @classmethod
+    def of(cls, weight: torch.Tensor) -> Optional["InFragments"]:
+        """``weight`` in fragment order, or None when its shape or dtype does not allow it."""
+        frag = fragment_order(weight) if weight.is_cuda else None
+        return None if frag is None else cls(frag)
+
+    def dim(self) -> int:
+        return 2
+
+    def data_ptr(self) -> int:
+        return self.data.data_ptr()
+
+    def numel(self) -> int:
+        return self.data.numel()
+
+    def element_size(self) -> int:
+        return self.data.element_size()
+
+    def rows(self, n: int) -> "InFragments":
+        _need(0 < n <= self.shape[0] and n % 16 == 0, lambda: f"fragments: the first {n} rows")
+        return InFragments(self.data[:n])
+
+    def materialize(self) -> torch.Tensor:
+        """The matrix as rows again (for tests and tools; a copy made by torch)."""
+        N, K = self.shape
+        return (self.data.view(N // 16, K // 32, 4, 16, 8).permute(0, 3, 1, 2, 4)
+                .reshape(N, K).contiguous())
+
+
+def _matrix(weight, weight_frag: Optional[torch.Tensor]):
+    """The two addresses the product kernels take: (the matrix as rows or null, the matrix in
+    fragment order or null)."""
+    if isinstance(weight, InFragments):
+        _need(weight_frag is None, "a matrix kept in fragment order has no second copy")
+        return _vp(0), _vp(weight.data.data_ptr())
     if weight_frag is None:
-        return _vp(0)
+        return _vp(weight.data_ptr()), _vp(0)
     _gpu("weight_frag", weight_frag, BF16)
     _need(weight_frag.shape == weight.shape and weight.shape[0] % 16 == 0
           and weight.shape[1] % 32 == 0 and weight_frag.data_ptr() % 16 == 0,
           "weight_frag: the fragment-order copy must have the matrix's shape [N, K] with N a "
           "multiple of 16 and K of 32")
-    return _vp(weight_frag.data_ptr())
+    return _vp(weight.data_ptr()), _vp(weight_frag.data_ptr())
+
+
+def _gpu_matrix(name: str, weight, dtype) -> None:
+    if not isinstance(weight, InFragments):
+        _gpu(name, weight, dtype)
 
 
 def split_k_for(M: int, N: int, K: int) -> int:
@@ -367,8 +426,9 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] =
     activations' dtype.  ``x`` may be a view with a row stride.  With ``partial_sums`` the
     result may come back as float32 [S, M, N], the sums over S ranges of K, for a consumer
     that adds them (a matrix with few columns is then streamed by enough blocks).  ``x`` may
-    be ``ScaledRows`` or ``FragmentRows``.  ``weight_frag`` (``fragment_order(weight)``) is read
-    in place of ``weight`` by the kernel for 1 to 16 rows.  ``add_into``: see ``AddInto``; the
+    be ``ScaledRows`` or ``FragmentRows``.  ``weight`` may be ``InFragments`` (a bfloat16 matrix
+    kept in fragment order only); or ``weight_frag`` (``fragment_order(weight)``) may come beside
+    the rows, which the kernels that are faster with it read.  ``add_into``: see ``AddInto``; the
     result is then ``Added`` or ``ScaledRows`` when the product could add its result itself."""
     a_frag = 0
     scale = None
@@ -390,7 +450,7 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] =
         else:
             a_frag, n_frag, x = 1, x.shape[0], x.data     # 16 row slots, n_frag of them filled
     _gpu("x", x, (F32, BF16), contiguous=False)
-    _gpu("weight", weight, (F32, BF16))
+    _gpu_matrix("weight", weight, (F32, BF16))
     _need(x.dim() == 2 and weight.dim() == 2 and x.shape[1] == weight.shape[1],
           lambda: f"linear: x {tuple(x.shape)} does not meet weight {tuple(weight.shape)}")
     _need(x.stride(1) == 1 or x.shape[1] == 1, "linear: x must have unit stride along K")
@@ -419,6 +479,8 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] =
               lambda: f"linear: K ({K}) and the row stride ({lda}) must be multiples of 8 and "
                       "the tensors 16-byte aligned for the kernel that was asked for")
         _need(M <= MAX_GRID_Y, lambda: f"linear: {M} rows with a width that is no multiple of 8")
+        _need(not isinstance(weight, InFragments),
+              "linear: a matrix kept in fragment order needs 16-byte aligned rows of x")
         out = torch.empty((M, N), dtype=out_dtype, device=x.device)
         check(library("gemm").kappai_gemm_bf16_any(
             _ptr(xb), _ptr(weight), _ptr(bias), _ptr(out), _c_int(M), _c_int(N), _c_int(K),
@@ -441,7 +503,7 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] =
             rows = torch.empty((16 if fragment else M, N), dtype=BF16, device=x.device)
             ss = torch.empty(((N + 7) // 8, 16), dtype=F32, device=x.device)
         check(library("gemm").kappai_gemm_bf16(
-            _ptr(xb), _ptr(weight), _frag(weight, weight_frag), _ptr(bias), _vp(0), _c_int(M),
+            _ptr(xb), *_matrix(weight, weight_frag), _ptr(bias), _vp(0), _c_int(M),
             _c_int(N), _c_int(K), _c_int(lda), _c_int(N), _c_int(1), _c_int(force_kernel),
             _c_int(1), _c_int(a_frag), *scale_args, _ptr(resid), _c_int(resid.stride(0)),
             _ptr(nw), _ptr(rows), _c_int(1 if fragment else 0), _ptr(ss), _stream()),
@@ -457,7 +519,7 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] =
         out = torch.empty((M, N), dtype=out_dtype, device=x.device)
         out_is_f32 = 0 if out_dtype == BF16 else 1
     check(library("gemm").kappai_gemm_bf16(
-        _ptr(xb), _ptr(weight), _frag(weight, weight_frag), _ptr(bias), _ptr(out), _c_int(M),
+        _ptr(xb), *_matrix(weight, weight_frag), _ptr(bias), _ptr(out), _c_int(M),
         _c_int(N), _c_int(K),
         _c_int(lda), _c_int(N), _c_int(out_is_f32), _c_int(force_kernel), _c_int(ksplit),
         _c_int(a_frag), *scale_args, _vp(0), _c_int(0), _vp(0), _vp(0), _c_int(0), _vp(0),
@@ -507,7 +569,7 @@ def linear_swiglu(x: torch.Tensor, weight: torch.Tensor, force_kernel: int = 0,
         else:
             a_frag, n_frag, x = 1, x.shape[0], x.data
     _gpu("x", x, BF16, contiguous=False)
-    _gpu("weight", weight, BF16)
+    _gpu_matrix("weight", weight, BF16)
     _need(x.dim() == 2 and weight.dim() == 2 and x.shape[1] == weight.shape[1]
           and weight.shape[0] % (2 * SWIGLU_GROUP) == 0,
           lambda: f"linear_swiglu: x {tuple(x.shape)}, weight {tuple(weight.shape)}")
@@ -523,7 +585,7 @@ def linear_swiglu(x: torch.Tensor, weight: torch.Tensor, force_kernel: int = 0,
     c_frag = _out_in_fragment_order(out_fragment, M, F, force_kernel)
     out = torch.empty((16 if c_frag else M, F), dtype=BF16, device=x.device)
     check(library("gemm").kappai_gemm_bf16_swiglu(
-        _ptr(x), _ptr(weight), _frag(weight, weight_frag), _ptr(out), _c_int(M), _c_int(F), _c_int(K),
+        _ptr(x), *_matrix(weight, weight_frag), _ptr(out), _c_int(M), _c_int(F), _c_int(K),
         _c_int(lda), _c_int(F),
         _c_int(force_kernel), _c_int(a_frag),
         *(scale._scale_args() if scale is not None else _NO_SCALE), _c_int(1 if c_frag else 0),
@@ -557,7 +619,7 @@ def linear_shortconv_step(x: torch.Tensor, in_proj: torch.Tensor, in_bias: Optio
         else:
             a_frag, n_frag, x = 1, x.shape[0], x.data
     _gpu("x", x, BF16, contiguous=False)
-    _gpu("in_proj", in_proj, BF16)
+    _gpu_matrix("in_proj", in_proj, BF16)
     _gpu("taps", taps, F32)
     _gpu("state", state, F32)
     _gpu("seg_pos0", seg_pos0, I32)
@@ -582,7 +644,7 @@ def linear_shortconv_step(x: torch.Tensor, in_proj: torch.Tensor, in_bias: Optio
     c_frag = _out_in_fragment_order(out_fragment, M, D, 0)
     out = torch.empty((16 if c_frag else M, D), dtype=BF16, device=x.device)
     check(library("gemm").kappai_gemm_bf16_shortconv_step(
-        _ptr(x), _ptr(in_proj), _frag(in_proj, weight_frag), _ptr(in_bias), _ptr(out), _c_int(M),
+        _ptr(x), *_matrix(in_proj, weight_frag), _ptr(in_bias), _ptr(out), _c_int(M),
         _c_int(D), _c_int(K),
         _c_int(lda), _ptr(taps), _ptr(conv_bias), _ptr(state), _ptr(seg_pos0), _ptr(seg_slot),
         _c_int(L), _c_int(a_frag), *(scale._scale_args() if scale is not None else _NO_SCALE),

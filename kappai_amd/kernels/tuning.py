@@ -11,11 +11,11 @@ numbers in its model description.
 # and 12 us at 64 rows.
 PARTIAL_SUMS_MIN_ROWS = 16
 
-# Every bfloat16 matrix is kept a second time in the order in which the product kernel for 1 to
-# 16 rows loads it (``ops.fragment_order``): decode steps stream that copy 10-20 % faster (a step
-# at batch 8: about a tenth), steps with more rows read the matrix as the checkpoint has it.  The
-# price is the matrices' memory once more; False keeps one copy.
-FRAGMENT_COPIES = True
+# Every bfloat16 matrix whose shape allows it (rows a multiple of 16, columns of 32) is kept in
+# the order in which the product kernels load it (``ops.fragment_order``), and only so: decode
+# steps stream it 10-20 % faster than rows (a step at batch 8: about a tenth), the block kernels
+# of prompt steps up to 10 %.  False keeps the matrices as the checkpoint has them.
+FRAGMENT_ORDER = True
 
 # The norm kernel hands its rows on in fragment order from this many rows on (up to 16): a step of
 # the 1.2B shape takes 1.06 against 1.08 ms at 16 rows, 0.994 against 1.000 at 12, even at 8; with

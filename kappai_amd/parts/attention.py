@@ -44,9 +44,8 @@ class GroupedQueryAttention(Mixer):
         self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(head_dim)
         self.qkv = Linear([prefix + n["q"], prefix + n["k"], prefix + n["v"]], width,
                           [num_heads * head_dim, num_kv_heads * head_dim, num_kv_heads * head_dim],
-                          bias=bias, stage="matmul_qkv")
-        self.q_only = Linear([prefix + n["q"]], width, [num_heads * head_dim], bias=bias,
-                             stage="matmul_qkv")
+                          bias=bias, stage="matmul_qkv", cut_rows_at=[num_heads * head_dim])
+        self.q_only: Optional[Linear] = None      # the q rows alone (bind)
         self.out = Linear([prefix + n["o"]], num_heads * head_dim, [width], bias=bias,
                           stage="matmul_attn_out")
         self._qn, self._kn = prefix + n["q_norm"], prefix + n["k_norm"]
@@ -74,11 +73,7 @@ class GroupedQueryAttention(Mixer):
         self.qkv.bind(tensors)
         self.out.bind(tensors)
         # the q rows of the stacked matrix, for a layer that reads another layer's keys
-        self.q_only.weight = self.qkv.weight[: self.H * self.d]
-        frag = self.qkv.weight_frag          # whole pieces of 16 rows: the q rows come first
-        self.q_only.weight_frag = (None if frag is None or (self.H * self.d) % 16
-                                   else frag[: self.H * self.d])
-        self.q_only.bias = None if self.qkv.bias is None else self.qkv.bias[: self.H * self.d]
+        self.q_only = self.qkv.first_rows(self.H * self.d)
         if self.qk_norm_eps is not None:
             self.q_norm_w = tensors[self._qn + ".weight"].to(torch.float32).contiguous()
             self.k_norm_w = tensors[self._kn + ".weight"].to(torch.float32).contiguous()

@@ -47,6 +47,9 @@ class OutputHead(Part):
     def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
         if self.tied_to is not None:
             self.linear.bind_shared(self.tied_to.table)
+            if isinstance(self.linear.weight, ops.InFragments):
+                # one matrix, in the order the products read it: the embedding reads that too
+                self.tied_to.table = self.linear.weight
         else:
             self.linear.bind(tensors)
 

@@ -31,19 +31,19 @@ class SwiGLU(FeedForward):
         return self.gate_up.tensor_specs() + self.down.tensor_specs()
 
     def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
-        self.gate_up.bind(tensors)
+        def interleaved(w):
+            # the fused product wants gate and up rows in turns of 16
+            self.fused = (w.dtype == torch.bfloat16 and self.hidden % ops.SWIGLU_GROUP == 0
+                          and self.width % 8 == 0)
+            return ops.interleave_gate_up(w[:self.hidden], w[self.hidden:]) if self.fused else None
+
+        self.gate_up.bind(tensors, arrange=interleaved)
         self.down.bind(tensors)
-        w = self.gate_up.weight
-        self.fused = (w.dtype == torch.bfloat16 and self.hidden % ops.SWIGLU_GROUP == 0
-                      and self.width % 8 == 0)
-        if self.fused:
-            self.gate_up.set_weight(ops.interleave_gate_up(w[:self.hidden], w[self.hidden:]))
 
     def forward(self, x, batch, into=None):
         if self.fused and x.dtype == torch.bfloat16:
             with profile.scope("matmul_ffn_gate_up", self.gate_up.weight_bytes()):
-                act = ops.linear_swiglu(x, self.gate_up.weight,
-                                        weight_frag=self.gate_up.weight_frag, out_fragment=True)
+                act = ops.linear_swiglu(x, self.gate_up.weight, out_fragment=True)
             return self.down.forward(act, partial_sums=True, add_into=into)
         gate_up = self.gate_up.forward(x)
         with profile.scope("ffn_act"):

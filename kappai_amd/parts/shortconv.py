@@ -74,7 +74,6 @@ class GatedShortConv(Mixer):
             with profile.scope("matmul_in_proj", self.in_proj.weight_bytes()):
                 y = ops.linear_shortconv_step(x, w, self.in_proj.bias, self.taps, self.conv_bias,
                                               cache.state, batch.seg_pos0, batch.seg_slot,
-                                              weight_frag=self.in_proj.weight_frag,
                                               out_fragment=True)
             return self.out_proj.forward(y, partial_sums=True, add_into=into)
         # decode with more than 16 rows: the projection may come as sums over ranges of its input

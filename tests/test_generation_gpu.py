@@ -245,11 +245,12 @@ def test_random_engine_options_give_the_same_tokens(model_dirs):
         assert eng.cache.num_free_pages() == options["num_pages"]
 
 
-def test_fragment_copies_change_no_token(tmp_path):
-    """The copies of the matrices in fragment order, and the normalised rows of a decode step in
-    that order, are layouts only: a model with and without them generates the same tokens in
+def test_fragment_order_changes_no_token(tmp_path):
+    """The matrices kept in fragment order, and the normalised rows of a decode step in that
+    order, are layouts only: a model with and without them generates the same tokens in
     bfloat16, greedy and sampled, through prompt portions, decode graphs and queued decode steps
-    (sizes at which every matrix has a copy)."""
+    (sizes at which every matrix can be kept so; the tied head's matrix is then the embedding's
+    table as well)."""
     import copy
     from kappai_amd.config import config_from_dict
     from kappai_amd.engine import Engine
@@ -273,17 +274,21 @@ def test_fragment_copies_change_no_token(tmp_path):
               SamplingParams.greedy(n_predict=24)] * 2
     assert len(prompts) >= tuning.FRAGMENT_ROWS_MIN      # decode steps with rows enough for the order
     outs = []
-    assert tuning.FRAGMENT_COPIES and tuning.FRAGMENT_ROWS
+    from kappai_amd.kernels import ops
+    assert tuning.FRAGMENT_ORDER and tuning.FRAGMENT_ROWS
     try:
-        for copies, rows in ((True, True), (False, True), (True, False), (False, False)):
-            tuning.FRAGMENT_COPIES, tuning.FRAGMENT_ROWS = copies, rows
+        for order, rows in ((True, True), (False, True), (True, False), (False, False)):
+            tuning.FRAGMENT_ORDER, tuning.FRAGMENT_ROWS = order, rows
             eng = Engine(str(folder), dtype="bfloat16", num_pages=128, max_batch=10, chunk=32,
                          token_budget=48)
-            frag = [blk.feed_forward.down.weight_frag for blk in eng.model.layers]
-            assert all((f is not None) == copies for f in frag)
+            kept = [blk.feed_forward.down.weight for blk in eng.model.layers]
+            kept += [blk.mixer.out.weight if hasattr(blk.mixer, "out") else blk.mixer.in_proj.weight
+                     for blk in eng.model.layers]
+            kept += [eng.model.head.linear.weight, eng.model.embedding.table]
+            assert all(isinstance(w, ops.InFragments) == order for w in kept)
             outs.append(eng.generate(prompts, params))
     finally:
-        tuning.FRAGMENT_COPIES, tuning.FRAGMENT_ROWS = True, True
+        tuning.FRAGMENT_ORDER, tuning.FRAGMENT_ROWS = True, True
     assert outs[0] == outs[1] == outs[2] == outs[3]
 
 

@@ -312,6 +312,60 @@ def test_products_read_the_fragment_order_copy(ops, M, N, K):
         assert torch.equal(outs[0], outs[1]) and torch.equal(states[0], states[1])
 
 
+@pytest.mark.parametrize("M", [1, 8, 16, 24, 40, 64, 65, 200, 300, 1000, 2048])
+@pytest.mark.parametrize("N,K", [(16, 32), (48, 96), (2048, 2048), (1008, 4128), (6144, 1024),
+                                 (1536, 512), (8192, 256)])
+def test_products_read_a_matrix_kept_in_fragment_order_only(ops, M, N, K):
+    """A matrix of which only the fragment order is kept (``ops.InFragments``) gives bit for bit
+    what its rows give, whatever kernel the row count picks: the kernels for 1 to 16 and 17 to 64
+    rows, the block kernel in each of its forms (its loads of W are then pieces of 1 KB), the
+    older tile kernel where K is no multiple of 128; plain, with bias, as partial sums, with the
+    SwiGLU epilogue."""
+    x = rand((M, K), BF16, 160).to(DEV)
+    w, b = rand((N, K), BF16, 161, 0.1).to(DEV), rand((N,), F32, 162).to(DEV)
+    kept = ops.InFragments.of(w)
+    assert kept is not None and kept.shape == w.shape and kept.dtype == BF16
+    assert torch.equal(kept.materialize(), w)
+    forces = [0]
+    if M > 64:
+        forces += [3, 4, 5, 6] + ([BLOCK256, BLOCK128, BLOCK128_DEEP, BLOCK192] if K % 128 == 0 else [])
+    elif M > 16 and K % 512 == 0:
+        forces += [SHARED_ROWS]
+    for force in forces:
+        for bias in (None, b):
+            for out_dtype in (BF16, F32):
+                assert torch.equal(
+                    ops.linear(x, kept, bias, out_dtype=out_dtype, force_kernel=force),
+                    ops.linear(x, w, bias, out_dtype=out_dtype, force_kernel=force)), (force, out_dtype)
+        if K % 256 == 0 and (force != SHARED_ROWS or K % 1024 == 0):
+            assert torch.equal(ops.linear(x, kept, partial_sums=True, split_k=2, force_kernel=force),
+                               ops.linear(x, w, partial_sums=True, split_k=2, force_kernel=force)), force
+        if N % 32 == 0 and force != BLOCK192:
+            assert torch.equal(ops.linear_swiglu(x, kept, force_kernel=force),
+                               ops.linear_swiglu(x, w, force_kernel=force)), force
+    # the first rows of the matrix by themselves (the q rows of a stacked q, k, v)
+    if N >= 32:
+        first = (N // 32) * 16
+        assert torch.equal(ops.linear(x, kept.rows(first)), ops.linear(x, w[:first].contiguous()))
+    # rows of it as an embedding table
+    ids = torch.tensor([0, N - 1, N // 2, 17 % N, 16 % N], dtype=torch.int32, device=DEV)
+    assert torch.equal(ops.embed_rows(ids, kept), ops.embed_rows(ids, w))
+
+
+def test_a_matrix_kept_in_fragment_order_refuses_what_needs_its_rows(ops):
+    w = rand((64, 64), BF16, 163).to(DEV)
+    kept = ops.InFragments.of(w)
+    assert ops.InFragments.of(w[:40].contiguous()) is None and ops.InFragments.of(w.float()) is None
+    with pytest.raises(ValueError, match="second copy"):
+        ops.linear(rand((4, 64), BF16, 164).to(DEV), kept, weight_frag=kept.data)
+    with pytest.raises(ValueError, match="rows"):
+        kept.rows(24)
+    # rows of x that are not 16-byte aligned would need the plain kernel, which reads rows of W
+    x = rand((4, 72), BF16, 165).to(DEV)[:, 4:68]
+    with pytest.raises(ValueError, match="aligned"):
+        ops.linear(x, kept)
+
+
 @pytest.mark.parametrize("M", [1, 2, 5, 8, 13, 16])
 @pytest.mark.parametrize("N,K", [(16, 32), (48, 96), (2048, 2048), (1008, 4128), (6144, 1024),
                                  (12288, 4096)])

@@ -2,6 +2,7 @@
 that the decode products read, and the normalised rows of a decode step in the same order.
 Both put element (row, k) of a piece of 16 rows x 32 of K at lane (k % 32) / 8 * 16 + row % 16,
 value k % 8 of that lane: the order in which a 16x16x32 matrix instruction takes its operands."""
+import pytest
 import torch
 
 from kappai_amd.kernels import ops
@@ -23,6 +24,7 @@ def test_matrix_copy_in_fragment_order():
     assert ops.fragment_order(w.float()) is None
 
 
+@pytest.mark.gpu
 def test_rows_in_fragment_order_come_back_as_rows():
     n, D = 11, 96
     rows = torch.arange(n * D, dtype=torch.float32).remainder(241).to(torch.bfloat16).reshape(n, D)
@@ -30,9 +32,9 @@ def test_rows_in_fragment_order_come_back_as_rows():
     for i in range(n):
         for k in range(D):
             data[(k // 32) * 512 + place_in_piece(i, k)] = rows[i, k]
-    frag = ops.FragmentRows(data.reshape(16, D), n, resid=torch.zeros(n, D))
+    frag = ops.FragmentRows(data.reshape(16, D).to("cuda:0"), n, resid=torch.zeros(n, D))
     assert frag.shape == (n, D) and frag.dtype == torch.bfloat16
-    assert torch.equal(frag.materialize(), rows)
+    assert torch.equal(frag.materialize().cpu(), rows)
     assert ops.FragmentRows.fits(16, 2048, torch.bfloat16)
     assert not ops.FragmentRows.fits(17, 2048, torch.bfloat16)       # one tile of 16 rows
     assert not ops.FragmentRows.fits(8, 2040, torch.bfloat16)        # whole pieces of 32 of K
