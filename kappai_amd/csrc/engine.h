@@ -20,7 +20,7 @@
 extern "C" {
 #endif
 
-#define KAPPAI_ENGINE_ABI 6          // bumped with every change of the structs below
+#define KAPPAI_ENGINE_ABI 7          // bumped with every change of the structs below
 #define KAPPAI_MAX_GROUPS 8          // paged groups a batch can carry block tables for
 
 // ---- the kernels' launchers, by address (they live in libraries of their own) ---------------
@@ -44,8 +44,8 @@ typedef struct kappai_kernels {
                                   const int*, int, int, const float*, int, float, int, hipStream_t);
   int (*shortconv)(const void*, const float*, const float*, float*, void*, const int*, const int*,
                    const int*, const int*, int, int, int, int, int, hipStream_t);
-  int (*shortconv_step_parts)(const float*, int, const float*, const float*, float*, void*,
-                              const int*, const int*, int, int, int, hipStream_t);
+  int (*shortconv_parts)(const float*, int, const float*, const float*, float*, void*, const int*,
+                         const int*, const int*, const int*, int, int, int, int, hipStream_t);
   int (*qk_norm_rope_store)(void*, int, const float*, const float*, float, const float*,
                             const float*, int, int, void*, void*, const int*, const int*,
                             const int*, int, int, int, int, int, int, int, int, const float*, int,
@@ -144,6 +144,7 @@ typedef struct kappai_model {
   // the choices that the parts make by size (the same numbers the host's parts use)
   int fused_step_min_width, fused_step_narrow_width, fused_step_narrow_rows;
   int partial_sums_min_rows;        // projections hand on partial sums above this many rows
+  int partial_sums_max_rows;        // and up to this many (more, when every segment is one row)
   int fragment_rows_min;            // the norm writes fragment order from this many rows on
   int fragment_rows_from;           // products write fragment order from this many rows on
   int fused_max_rows;               // rows up to which products fold residual sum and norm in

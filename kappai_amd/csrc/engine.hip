@@ -354,6 +354,12 @@ Rows as_rows(const Carry& y, int M, int D, int is_bf16) {
 // ---------------------------------------------------------------------------------------------
 // the parts
 // ---------------------------------------------------------------------------------------------
+// When in_proj and qkv hand their consumer partial sums over K ranges (tuning.takes_partial_sums)
+bool takes_partial_sums(const Ctx& c, int M) {
+  return M > c.m->partial_sums_min_rows &&
+         (M <= c.m->partial_sums_max_rows || c.b->max_segment_rows == 1);
+}
+
 // parts/shortconv.py
 Carry conv_mixer(Ctx& c, const kappai_layer_call& L, Rows x, float* resid, const Into& into) {
   const kappai_kernels& k = *c.m->kernels;
@@ -378,9 +384,9 @@ Carry conv_mixer(Ctx& c, const kappai_layer_call& L, Rows x, float* resid, const
     yr.frag = c_frag;
     return linear(c, yr, L.out_proj, c.m->compute_bf16, true, &into, region);
   }
-  // decode with more than 16 rows: the projection may come as sums over ranges of its input
-  // dimension, which the step kernel adds up
-  const bool parts = b.max_segment_rows == 1 && M > c.m->partial_sums_min_rows;
+  // more than 16 rows (decode at any batch size, short prompt portions): the projection may come
+  // as sums over ranges of its input dimension, which the conv kernel adds up
+  const bool parts = takes_partial_sums(c, M);
   Carry proj = linear(c, x, L.in_proj, c.m->compute_bf16, parts, nullptr, R_BLOCK);
   if (!c.ok() && !c.dry) return none;
   void* y;
@@ -388,8 +394,9 @@ Carry conv_mixer(Ctx& c, const kappai_layer_call& L, Rows x, float* resid, const
   if (proj.kind == C_PARTS) {
     y_bf16 = 1;
     y = c.a->take(R_BLOCK, (size_t)M * D * 2);
-    LAUNCH(c, k.shortconv_step_parts((const float*)proj.data, proj.parts, L.taps, L.conv_bias,
-                                     L.state, y, b.seg_pos0, b.seg_slot, M, D, taps, c.stream));
+    LAUNCH(c, k.shortconv_parts((const float*)proj.data, proj.parts, L.taps, L.conv_bias, L.state,
+                                y, b.row_seg, b.seg_start, b.seg_pos0, b.seg_slot, M, b.n_segments,
+                                D, taps, c.stream));
   } else {
     y_bf16 = proj.is_f32 ? 0 : 1;
     y = c.a->take(R_BLOCK, (size_t)M * D * elem(y_bf16));
@@ -437,7 +444,7 @@ Carry attention_mixer(Ctx& c, const kappai_layer_call& L, Rows x, float* resid, 
     if (qkv.w_frag != nullptr && (H * d) % 16) qkv.w_frag = nullptr;
   }
   if (!takes_kernel_order(qkv, x.D)) x = plain_rows(c, x, resid);
-  const bool parts = b.max_segment_rows == 1 && M > c.m->partial_sums_min_rows;
+  const bool parts = takes_partial_sums(c, M);
   Carry proj = linear(c, x, qkv, c.m->compute_bf16, parts, nullptr, R_BLOCK);
   if (!c.ok() && !c.dry) return none;
   if (L.rot_mode != 0 && b.max_position >= L.rot_positions) {

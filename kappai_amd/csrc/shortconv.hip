@@ -8,8 +8,27 @@
 // into the state; segments shorter than L-1 shift the old state through.
 #include "common.h"
 
+// The projection as the kernels below read it: a tensor [T, 3D], or (PartsIn) the float sums
+// over n_parts ranges of its input dimension, [n_parts][T][3D] (a product split over K): they are
+// added in order and rounded to bfloat16, which is what the unsplit product would have stored.
 template <typename T>
-__global__ void shortconv_out_kernel(const T* __restrict__ proj, const float* __restrict__ w,
+struct RowsIn {
+  const T* proj;
+  __device__ float at(size_t i) const { return to_f32(proj[i]); }
+};
+struct PartsIn {
+  const float* parts;
+  int n_parts;
+  size_t plane;      // T * 3D
+  __device__ float at(size_t i) const {
+    float sum = parts[i];
+    for (int s = 1; s < n_parts; ++s) sum += parts[s * plane + i];
+    return to_f32(f32_to_bf16(sum));
+  }
+};
+
+template <typename T, typename IN>
+__global__ void shortconv_out_kernel(IN in, const float* __restrict__ w,
                                      const float* __restrict__ bias,
                                      const float* __restrict__ state, T* __restrict__ out,
                                      const int* __restrict__ row_seg,
@@ -30,14 +49,14 @@ __global__ void shortconv_out_kernel(const T* __restrict__ proj, const float* __
     const int src = r - H + k;               // segment-relative row of the tap's input
     float bx;
     if (src >= 0) {
-      const T* p = proj + (size_t)(t - r + src) * 3 * D;
-      bx = to_f32(p[c]) * to_f32(p[2 * D + c]);
+      const size_t p = (size_t)(t - r + src) * 3 * D;
+      bx = in.at(p + c) * in.at(p + 2 * D + c);
     } else {
       bx = fresh ? 0.f : st[H + src];
     }
     sum += wc[k] * bx;
   }
-  const float cg = to_f32(proj[(size_t)t * 3 * D + D + c]);
+  const float cg = in.at((size_t)t * 3 * D + D + c);
   from_f32(out + (size_t)t * D + c, cg * sum);
 }
 
@@ -57,28 +76,51 @@ __device__ __forceinline__ void sc_unpack8(sc_u32x4_t v, float* f) {
   }
 }
 
-template <int L>
+// PARTS: the projection comes as float sums over n_parts ranges of its input dimension (see
+// PartsIn); 8 channels of a gate are then two loads of 16 bytes a range, and a thread takes one
+// row only (RUN 1): the steps that come this way have few rows, and the sums are the work.
+template <int L, bool PARTS, int RUN>
 __global__ __launch_bounds__(256) void shortconv_out_vec_kernel(
-    const bf16_t* __restrict__ proj, const float* __restrict__ w, const float* __restrict__ bias,
+    const bf16_t* __restrict__ proj, const float* __restrict__ parts, int n_parts,
+    const float* __restrict__ w, const float* __restrict__ bias,
     const float* __restrict__ state, bf16_t* __restrict__ out, const int* __restrict__ row_seg,
     const int* __restrict__ seg_start, const int* __restrict__ seg_pos0,
     const int* __restrict__ seg_slot, int T, int D) {
   constexpr int H = L - 1;
   const int c0 = (blockIdx.y * blockDim.x + threadIdx.x) * 8;
-  const int t0 = blockIdx.x * SC_RUN;
+  const int t0 = blockIdx.x * RUN;
   if (c0 >= D) return;
   const size_t ld = (size_t)3 * D;
-  // rows t0-H .. t0+SC_RUN-1: the gates of the run and of the rows just before it
-  sc_u32x4_t vb[SC_RUN + H], vx[SC_RUN + H], vc[SC_RUN];
+  // 8 channels of a gate of one row (at: the row's offset plus the gate's), as bfloat16
+  auto gate8 = [&](size_t at) -> sc_u32x4_t {
+    if (!PARTS) return *reinterpret_cast<const sc_u32x4_t*>(proj + at);
+    const size_t plane = (size_t)T * ld;
+    float4 lo = *reinterpret_cast<const float4*>(parts + at);
+    float4 hi = *reinterpret_cast<const float4*>(parts + at + 4);
+    for (int s = 1; s < n_parts; ++s) {
+      const float4 a = *reinterpret_cast<const float4*>(parts + s * plane + at);
+      const float4 b = *reinterpret_cast<const float4*>(parts + s * plane + at + 4);
+      lo.x += a.x; lo.y += a.y; lo.z += a.z; lo.w += a.w;
+      hi.x += b.x; hi.y += b.y; hi.z += b.z; hi.w += b.w;
+    }
+    sc_u32x4_t r;
+    r[0] = pack_bf16x2(lo.x, lo.y);
+    r[1] = pack_bf16x2(lo.z, lo.w);
+    r[2] = pack_bf16x2(hi.x, hi.y);
+    r[3] = pack_bf16x2(hi.z, hi.w);
+    return r;
+  };
+  // rows t0-H .. t0+RUN-1: the gates of the run and of the rows just before it
+  sc_u32x4_t vb[RUN + H], vx[RUN + H], vc[RUN];
   const sc_u32x4_t zero = {0u, 0u, 0u, 0u};
 #pragma unroll
-  for (int i = 0; i < SC_RUN + H; ++i) {
+  for (int i = 0; i < RUN + H; ++i) {
     const int t = t0 - H + i;
     const bool in = t >= 0 && t < T;
-    const bf16_t* p = proj + (size_t)(in ? t : 0) * ld + c0;
-    vb[i] = in ? *reinterpret_cast<const sc_u32x4_t*>(p) : zero;
-    vx[i] = in ? *reinterpret_cast<const sc_u32x4_t*>(p + 2 * D) : zero;
-    if (i >= H) vc[i - H] = in ? *reinterpret_cast<const sc_u32x4_t*>(p + D) : zero;
+    const size_t p = (size_t)(in ? t : 0) * ld + c0;
+    vb[i] = in ? gate8(p) : zero;
+    vx[i] = in ? gate8(p + 2 * D) : zero;
+    if (i >= H) vc[i - H] = in ? gate8(p + D) : zero;
   }
   // the 8 channels' taps lie together: 8 L floats from a 16-byte aligned address
   float wt[8 * L], bs[8];
@@ -98,9 +140,9 @@ __global__ __launch_bounds__(256) void shortconv_out_vec_kernel(
       bs[4] = b1.x, bs[5] = b1.y, bs[6] = b1.z, bs[7] = b1.w;
     }
   }
-  float bx[SC_RUN + H][8];
+  float bx[RUN + H][8];
 #pragma unroll
-  for (int i = 0; i < SC_RUN + H; ++i) {
+  for (int i = 0; i < RUN + H; ++i) {
     float b[8], x[8];
     sc_unpack8(vb[i], b);
     sc_unpack8(vx[i], x);
@@ -108,7 +150,7 @@ __global__ __launch_bounds__(256) void shortconv_out_vec_kernel(
     for (int j = 0; j < 8; ++j) bx[i][j] = b[j] * x[j];
   }
 #pragma unroll
-  for (int r = 0; r < SC_RUN; ++r) {
+  for (int r = 0; r < RUN; ++r) {
     const int t = t0 + r;
     if (t >= T) break;
     const int seg = row_seg[t];
@@ -139,8 +181,8 @@ __global__ __launch_bounds__(256) void shortconv_out_vec_kernel(
   }
 }
 
-template <typename T>
-__global__ void shortconv_state_kernel(const T* __restrict__ proj, float* __restrict__ state,
+template <typename IN>
+__global__ void shortconv_state_kernel(IN in, float* __restrict__ state,
                                        const int* __restrict__ seg_start,
                                        const int* __restrict__ seg_pos0,
                                        const int* __restrict__ seg_slot, int D, int L) {
@@ -158,8 +200,8 @@ __global__ void shortconv_state_kernel(const T* __restrict__ proj, float* __rest
     const int src = n - H + j;
     float v;
     if (src >= 0) {
-      const T* p = proj + (size_t)(t0 + src) * 3 * D;
-      v = to_f32(p[c]) * to_f32(p[2 * D + c]);
+      const size_t p = (size_t)(t0 + src) * 3 * D;
+      v = in.at(p + c) * in.at(p + 2 * D + c);
     } else {
       v = fresh ? 0.f : st[n + j];
     }
@@ -228,29 +270,22 @@ __global__ void shortconv_step_parts_kernel(const float* __restrict__ parts, int
                               seg_pos0[t] == 0, L));
 }
 
-extern "C" int kappai_shortconv_step_parts(const float* parts, int n_parts, const float* w,
-                                           const float* bias, float* state, void* out,
-                                           const int* seg_pos0, const int* seg_slot, int T, int D,
-                                           int L, hipStream_t stream) {
-  if (T <= 0) return 0;
-  if (L < 2 || n_parts < 1 || D < 1) return (int)hipErrorInvalidValue;
-  const int threads = D >= 256 ? 256 : 64;
-  hipLaunchKernelGGL(shortconv_step_parts_kernel, dim3(T, (D + threads - 1) / threads),
-                     dim3(threads), 0, stream, parts, n_parts, w, bias, state, (bf16_t*)out,
-                     seg_pos0, seg_slot, T, D, L);
-  KAPPAI_RETURN_LAUNCH_STATUS();
-}
-
-extern "C" int kappai_shortconv(const void* proj, const float* w, const float* bias, float* state,
-                                void* out, const int* row_seg, const int* seg_start,
-                                const int* seg_pos0, const int* seg_slot, int T, int S, int D,
-                                int L, int is_bf16, hipStream_t stream) {
+// proj [T, 3D] (float32 or bfloat16), or null with `parts` [n_parts][T][3D]: float sums over
+// ranges of the projection's input dimension (the result is then bfloat16).
+static int shortconv_launch(const void* proj, const float* parts, int n_parts, const float* w,
+                            const float* bias, float* state, void* out, const int* row_seg,
+                            const int* seg_start, const int* seg_pos0, const int* seg_slot, int T,
+                            int S, int D, int L, int is_bf16, hipStream_t stream) {
   if (T <= 0 || S <= 0) return 0;
   if (L < 2) return (int)hipErrorInvalidValue;
   const int threads = D >= 256 ? 256 : 64;
   dim3 g1(T, (D + threads - 1) / threads), g2(S, (D + threads - 1) / threads);
+  const PartsIn pin{parts, n_parts, (size_t)T * 3 * D};
   if (T == S) {   // one row a segment: row t is segment t
-    if (is_bf16)
+    if (parts)
+      hipLaunchKernelGGL(shortconv_step_parts_kernel, g1, dim3(threads), 0, stream, parts, n_parts,
+                         w, bias, state, (bf16_t*)out, seg_pos0, seg_slot, T, D, L);
+    else if (is_bf16)
       hipLaunchKernelGGL(shortconv_step_kernel<bf16_t>, g1, dim3(threads), 0, stream,
                          (const bf16_t*)proj, w, bias, state, (bf16_t*)out, seg_pos0, seg_slot, D,
                          L);
@@ -259,33 +294,68 @@ extern "C" int kappai_shortconv(const void* proj, const float* w, const float* b
                          (const float*)proj, w, bias, state, (float*)out, seg_pos0, seg_slot, D, L);
     KAPPAI_RETURN_LAUNCH_STATUS();
   }
-  if (is_bf16 && D % 8 == 0 && L <= SC_HMAX + 1 && ((uintptr_t)proj % 16) == 0 &&
+  const void* in_ptr = parts ? (const void*)parts : proj;
+  if (is_bf16 && D % 8 == 0 && L <= SC_HMAX + 1 && ((uintptr_t)in_ptr % 16) == 0 &&
       ((uintptr_t)out % 16) == 0 && ((uintptr_t)w % 16) == 0 && (!bias || ((uintptr_t)bias % 16) == 0)) {
     const int groups = D / 8;
     const int th = groups >= 256 ? 256 : 64;
-    const dim3 gv((T + SC_RUN - 1) / SC_RUN, (groups + th - 1) / th);
-#define SC_LAUNCH(LL)                                                                           \
-  hipLaunchKernelGGL(shortconv_out_vec_kernel<LL>, gv, dim3(th), 0, stream, (const bf16_t*)proj, \
-                     w, bias, (const float*)state, (bf16_t*)out, row_seg, seg_start, seg_pos0,  \
-                     seg_slot, T, D)
-    if (L == 2) SC_LAUNCH(2);
-    else if (L == 3) SC_LAUNCH(3);
-    else SC_LAUNCH(4);
+    const int run = parts ? 1 : SC_RUN;
+    const dim3 gv((T + run - 1) / run, (groups + th - 1) / th);
+#define SC_LAUNCH_AS(LL, PP)                                                                     \
+  hipLaunchKernelGGL((shortconv_out_vec_kernel<LL, PP, (PP ? 1 : SC_RUN)>), gv, dim3(th), 0, stream, \
+                     (const bf16_t*)proj, parts, n_parts, w, bias, (const float*)state,          \
+                     (bf16_t*)out, row_seg, seg_start, seg_pos0, seg_slot, T, D)
+#define SC_LAUNCH(LL)                                                                            \
+  if (parts) SC_LAUNCH_AS(LL, true);                                                             \
+  else SC_LAUNCH_AS(LL, false)
+    if (L == 2) { SC_LAUNCH(2); }
+    else if (L == 3) { SC_LAUNCH(3); }
+    else { SC_LAUNCH(4); }
 #undef SC_LAUNCH
-    hipLaunchKernelGGL(shortconv_state_kernel<bf16_t>, g2, dim3(threads), 0, stream,
-                       (const bf16_t*)proj, state, seg_start, seg_pos0, seg_slot, D, L);
+#undef SC_LAUNCH_AS
+  } else if (parts) {
+    hipLaunchKernelGGL((shortconv_out_kernel<bf16_t, PartsIn>), g1, dim3(threads), 0, stream, pin, w,
+                       bias, (const float*)state, (bf16_t*)out, row_seg, seg_start, seg_pos0,
+                       seg_slot, D, L);
   } else if (is_bf16) {
-    hipLaunchKernelGGL(shortconv_out_kernel<bf16_t>, g1, dim3(threads), 0, stream,
-                       (const bf16_t*)proj, w, bias, (const float*)state, (bf16_t*)out, row_seg,
-                       seg_start, seg_pos0, seg_slot, D, L);
-    hipLaunchKernelGGL(shortconv_state_kernel<bf16_t>, g2, dim3(threads), 0, stream,
-                       (const bf16_t*)proj, state, seg_start, seg_pos0, seg_slot, D, L);
+    hipLaunchKernelGGL((shortconv_out_kernel<bf16_t, RowsIn<bf16_t>>), g1, dim3(threads), 0, stream,
+                       RowsIn<bf16_t>{(const bf16_t*)proj}, w, bias, (const float*)state,
+                       (bf16_t*)out, row_seg, seg_start, seg_pos0, seg_slot, D, L);
   } else {
-    hipLaunchKernelGGL(shortconv_out_kernel<float>, g1, dim3(threads), 0, stream,
-                       (const float*)proj, w, bias, (const float*)state, (float*)out, row_seg,
-                       seg_start, seg_pos0, seg_slot, D, L);
-    hipLaunchKernelGGL(shortconv_state_kernel<float>, g2, dim3(threads), 0, stream,
-                       (const float*)proj, state, seg_start, seg_pos0, seg_slot, D, L);
+    hipLaunchKernelGGL((shortconv_out_kernel<float, RowsIn<float>>), g1, dim3(threads), 0, stream,
+                       RowsIn<float>{(const float*)proj}, w, bias, (const float*)state, (float*)out,
+                       row_seg, seg_start, seg_pos0, seg_slot, D, L);
   }
+  // then the state: the last L - 1 values of B * x of every segment
+  if (parts)
+    hipLaunchKernelGGL(shortconv_state_kernel<PartsIn>, g2, dim3(threads), 0, stream, pin, state,
+                       seg_start, seg_pos0, seg_slot, D, L);
+  else if (is_bf16)
+    hipLaunchKernelGGL(shortconv_state_kernel<RowsIn<bf16_t>>, g2, dim3(threads), 0, stream,
+                       RowsIn<bf16_t>{(const bf16_t*)proj}, state, seg_start, seg_pos0, seg_slot, D,
+                       L);
+  else
+    hipLaunchKernelGGL(shortconv_state_kernel<RowsIn<float>>, g2, dim3(threads), 0, stream,
+                       RowsIn<float>{(const float*)proj}, state, seg_start, seg_pos0, seg_slot, D, L);
   KAPPAI_RETURN_LAUNCH_STATUS();
+}
+
+extern "C" int kappai_shortconv(const void* proj, const float* w, const float* bias, float* state,
+                                void* out, const int* row_seg, const int* seg_start,
+                                const int* seg_pos0, const int* seg_slot, int T, int S, int D,
+                                int L, int is_bf16, hipStream_t stream) {
+  return shortconv_launch(proj, nullptr, 0, w, bias, state, out, row_seg, seg_start, seg_pos0,
+                          seg_slot, T, S, D, L, is_bf16, stream);
+}
+
+// The same from the float partial sums of the projection, [n_parts][T][3D], for segments of any
+// length; the result is bfloat16.
+extern "C" int kappai_shortconv_parts(const float* parts, int n_parts, const float* w,
+                                      const float* bias, float* state, void* out,
+                                      const int* row_seg, const int* seg_start,
+                                      const int* seg_pos0, const int* seg_slot, int T, int S, int D,
+                                      int L, hipStream_t stream) {
+  if (parts == nullptr || n_parts < 1 || D < 1) return (int)hipErrorInvalidValue;
+  return shortconv_launch(nullptr, parts, n_parts, w, bias, state, out, row_seg, seg_start,
+                          seg_pos0, seg_slot, T, S, D, L, 1, stream);
 }

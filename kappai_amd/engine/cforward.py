@@ -29,7 +29,7 @@ from ..parts.embedding import OutputHead, TokenEmbedding
 from ..parts.feed_forward import SwiGLU
 from ..parts.rotary import RotaryEncoding
 
-ENGINE_ABI = 6
+ENGINE_ABI = 7
 MAX_GROUPS = 8
 
 
@@ -40,7 +40,7 @@ def _ptrs(names):
 class Kernels(Structure):
     _fields_ = _ptrs(["embed_rows", "add_rmsnorm", "swiglu", "cast", "gemm_f32", "gemm_bf16",
                       "gemm_bf16_any", "gemm_bf16_swiglu", "gemm_bf16_shortconv_step", "shortconv",
-                      "shortconv_step_parts", "qk_norm_rope_store", "paged_attention_rows"])
+                      "shortconv_parts", "qk_norm_rope_store", "paged_attention_rows"])
 
 
 class AttentionKernels(Structure):
@@ -80,6 +80,7 @@ class ModelDesc(Structure):
         ("head", LinearDesc), ("kernels", POINTER(Kernels)),
         ("fused_step_min_width", c_int), ("fused_step_narrow_width", c_int),
         ("fused_step_narrow_rows", c_int), ("partial_sums_min_rows", c_int),
+        ("partial_sums_max_rows", c_int),
         ("fragment_rows_min", c_int), ("fragment_rows_from", c_int), ("fused_max_rows", c_int),
         ("decode_waves", c_int), ("decode_max_splits", c_int), ("decode_block_max_keys", c_int),
         ("attention_tile_rows", c_int), ("fused_qk", c_int)]
@@ -192,7 +193,7 @@ class CForward:
                          ("gemm_bf16_swiglu", gm.kappai_gemm_bf16_swiglu),
                          ("gemm_bf16_shortconv_step", gm.kappai_gemm_bf16_shortconv_step),
                          ("shortconv", sc.kappai_shortconv),
-                         ("shortconv_step_parts", sc.kappai_shortconv_step_parts),
+                         ("shortconv_parts", sc.kappai_shortconv_parts),
                          ("qk_norm_rope_store", at.kappai_qk_norm_rope_store),
                          ("paged_attention_rows", at.kappai_paged_attention_rows)):
             setattr(k, name, _address(fn))
@@ -248,6 +249,7 @@ class CForward:
         m.fused_step_narrow_width = tuning.FUSED_STEP_NARROW_WIDTH
         m.fused_step_narrow_rows = tuning.FUSED_STEP_NARROW_ROWS
         m.partial_sums_min_rows = tuning.PARTIAL_SUMS_MIN_ROWS
+        m.partial_sums_max_rows = tuning.PARTIAL_SUMS_MAX_ROWS
         m.fragment_rows_min = tuning.FRAGMENT_ROWS_MIN if tuning.FRAGMENT_ROWS else 1 << 30
         m.fragment_rows_from = ops.FRAGMENT_ROWS_FROM
         m.fused_max_rows = ops.FUSED_MAX_ROWS

@@ -658,13 +658,14 @@ def shortconv(proj: torch.Tensor, taps: torch.Tensor, bias: Optional[torch.Tenso
               seg_pos0: torch.Tensor, seg_slot: torch.Tensor) -> torch.Tensor:
     """Gated causal depthwise convolution of ``proj`` [T, 3D] = (B | C | x) per segment with
     taps [D, L]; reads and then updates ``state`` [slots, D, L-1] (float32) of every
-    segment's slot.  Returns C * conv(B * x) as [T, D].  When every segment is a single row,
-    ``proj`` may be the float32 partial sums [S, T, 3D] of a projection split over its input
-    dimension: they are added in order and rounded to bfloat16 first, and the result is
-    bfloat16."""
+    segment's slot.  Returns C * conv(B * x) as [T, D].  ``proj`` may be the float32 partial
+    sums [S, T, 3D] of a projection split over its input dimension: they are added in order and
+    rounded to bfloat16 first, and the result is bfloat16."""
     _gpu("proj", proj, (F32, BF16))
+    parts = None
     if proj.dim() == 3:
-        return _shortconv_step_parts(proj, taps, bias, state, seg_pos0, seg_slot)
+        _need(proj.dtype == F32, "shortconv: partial sums are float32")
+        parts, proj = proj, proj[0]
     _gpu("taps", taps, F32)
     _gpu("state", state, F32)
     for n, t in (("row_seg", row_seg), ("seg_start", seg_start), ("seg_pos0", seg_pos0),
@@ -682,34 +683,18 @@ def shortconv(proj: torch.Tensor, taps: torch.Tensor, bias: Optional[torch.Tenso
     if bias is not None:
         _gpu("bias", bias, F32)
         _need(bias.shape == (D,), "shortconv: bias must be [D]")
+    if parts is not None:
+        out = torch.empty((T, D), dtype=BF16, device=proj.device)
+        check(library("shortconv").kappai_shortconv_parts(
+            _ptr(parts), _c_int(parts.shape[0]), _ptr(taps), _ptr(bias), _ptr(state), _ptr(out),
+            _ptr(row_seg), _ptr(seg_start), _ptr(seg_pos0), _ptr(seg_slot), _c_int(T), _c_int(S),
+            _c_int(D), _c_int(L), _stream()), "shortconv_parts")
+        return out
     out = torch.empty((T, D), dtype=proj.dtype, device=proj.device)
     check(library("shortconv").kappai_shortconv(
         _ptr(proj), _ptr(taps), _ptr(bias), _ptr(state), _ptr(out), _ptr(row_seg), _ptr(seg_start),
         _ptr(seg_pos0), _ptr(seg_slot), _c_int(T), _c_int(S), _c_int(D), _c_int(L),
         _c_int(_is_bf16(proj.dtype)), _stream()), "shortconv")
-    return out
-
-
-def _shortconv_step_parts(parts, taps, bias, state, seg_pos0, seg_slot) -> torch.Tensor:
-    _gpu("taps", taps, F32)
-    _gpu("state", state, F32)
-    _gpu("seg_pos0", seg_pos0, I32)
-    _gpu("seg_slot", seg_slot, I32)
-    S, T, W = parts.shape
-    D, L = taps.shape
-    _need(parts.dtype == F32 and W == 3 * D and parts.is_contiguous(),
-          lambda: f"shortconv: partial sums {tuple(parts.shape)} for D={D}")
-    _need(seg_pos0.shape[0] == T and seg_slot.shape[0] == T,
-          "shortconv: partial sums are taken only when every segment is a single row")
-    _need(L >= 2 and state.dim() == 3 and state.shape[1:] == (D, L - 1),
-          lambda: f"shortconv: state {tuple(state.shape)} for D={D}, L={L}")
-    if bias is not None:
-        _gpu("bias", bias, F32)
-        _need(bias.shape == (D,), "shortconv: bias must be [D]")
-    out = torch.empty((T, D), dtype=BF16, device=parts.device)
-    check(library("shortconv").kappai_shortconv_step_parts(
-        _ptr(parts), _c_int(S), _ptr(taps), _ptr(bias), _ptr(state), _ptr(out), _ptr(seg_pos0),
-        _ptr(seg_slot), _c_int(T), _c_int(D), _c_int(L), _stream()), "shortconv_step_parts")
     return out
 
 

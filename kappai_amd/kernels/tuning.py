@@ -10,6 +10,17 @@ numbers in its model description.
 # 6144 x 2048 plus the conv step takes 13.0 us unsplit and 13.3 us in two K ranges at 8 rows, 18 us
 # and 12 us at 64 rows.
 PARTIAL_SUMS_MIN_ROWS = 16
+# ... and in steps of up to this many rows whatever their segments (short prompt portions): with
+# few rows the products of in_proj and qkv have too few blocks to fill the chip unless K is cut
+# (in_proj of 128 rows: 9-12 us in four ranges against 22 us whole; the float partial sums of
+# 512 rows would already cost more than the cut saves).  Above it only steps of single rows
+# (decode at large batches) hand on partial sums.
+PARTIAL_SUMS_MAX_ROWS = 256
+
+
+def takes_partial_sums(rows: int, single_rows: bool) -> bool:
+    """Whether in_proj / qkv of a step of ``rows`` rows hand their consumer partial sums."""
+    return rows > PARTIAL_SUMS_MIN_ROWS and (rows <= PARTIAL_SUMS_MAX_ROWS or single_rows)
 
 # Every bfloat16 matrix whose shape allows it (rows a multiple of 16, columns of 32) is kept in
 # the order in which the product kernels load it (``ops.fragment_order``), and only so: decode

@@ -80,10 +80,10 @@ class GroupedQueryAttention(Mixer):
 
     def forward(self, x, batch, cache, shared_cache: bool = False, into=None):
         H, G, d = self.H, self.G, self.d
-        # decode with more than 16 rows: the projection may come as sums over ranges of its input
-        # dimension (more blocks stream the matrix), which the next kernel adds up
+        # more than 16 rows (decode, short prompt portions): the projection may come as sums over
+        # ranges of its input dimension (more blocks stream the matrix), which the next kernel adds up
         proj = (self.q_only if shared_cache else self.qkv).forward(
-            x, partial_sums=batch.max_segment_rows == 1 and x.shape[0] > tuning.PARTIAL_SUMS_MIN_ROWS)
+            x, partial_sums=tuning.takes_partial_sums(x.shape[0], batch.max_segment_rows == 1))
         rot = self.position.rotation(x.device, batch.max_position) if self.position else None
         tables = batch.block_tables[cache.group]
         k_pool, v_pool = cache.pool("k"), cache.pool("v")

@@ -76,11 +76,11 @@ class GatedShortConv(Mixer):
                                               cache.state, batch.seg_pos0, batch.seg_slot,
                                               out_fragment=True)
             return self.out_proj.forward(y, partial_sums=True, add_into=into)
-        # decode with more than 16 rows: the projection may come as sums over ranges of its input
-        # dimension (more blocks stream the matrix), which the step kernel adds up; with fewer
-        # rows the unsplit product and the plain step are as fast or faster
+        # more than 16 rows (decode, short prompt portions): the projection may come as sums over
+        # ranges of its input dimension (more blocks stream the matrix), which the conv kernel
+        # adds up; with fewer rows the unsplit product and the plain step are as fast or faster
         proj = self.in_proj.forward(
-            x, partial_sums=batch.max_segment_rows == 1 and x.shape[0] > tuning.PARTIAL_SUMS_MIN_ROWS)
+            x, partial_sums=tuning.takes_partial_sums(x.shape[0], batch.max_segment_rows == 1))
         with profile.scope("short_conv"):
             y = ops.shortconv(proj, self.taps, self.conv_bias, cache.state, batch.row_seg,
                               batch.seg_start, batch.seg_pos0, batch.seg_slot)

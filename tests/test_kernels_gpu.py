@@ -1022,9 +1022,34 @@ def test_shortconv_step_from_partial_sums(ops, D, L, bias, n_parts):
                              pos0, slot.to(DEV))
         assert got.dtype == BF16 and torch.equal(got.cpu(), want.cpu()), f"step {step}"
         assert torch.equal(st_p.cpu(), st_w.cpu()), f"state after step {step}"
-    with pytest.raises(ValueError, match="single row"):
-        ops.shortconv(parts.to(DEV), taps.to(DEV), dev(cb), st_p, seg, seg_start[:5], pos0[:4],
-                      slot[:4].to(DEV))
+
+
+@pytest.mark.parametrize("D,L,bias,n_parts", [(64, 3, False, 2), (2048, 3, False, 4), (100, 4, True, 3),
+                                              (48, 2, True, 2), (320, 5, False, 8)])
+def test_shortconv_of_prompt_portions_from_partial_sums(ops, D, L, bias, n_parts):
+    """Segments of several rows (prompt portions beside single decoded tokens) from float partial
+    sums of the projection: the same output and state, bit for bit, as from their bfloat16 sum,
+    over two steps, whichever of the conv kernels the sizes pick."""
+    slots = 6
+    taps, cb = rand((D, L), F32, 170, 0.5), (rand((D,), F32, 171, 0.3) if bias else None)
+    state0 = rand((slots, D, L - 1), F32, 172)
+    st_p, st_w = state0.to(DEV).clone(), state0.to(DEV).clone()
+    dev = lambda t: None if t is None else t.to(DEV)
+    for step, (lens, pos0, slot) in enumerate([([1, 2, 9, 70], [0, 5, 0, 17], [3, 0, 5, 1]),
+                                               ([2, 1, 1, 3], [1, 7, 9, 87], [3, 0, 5, 1])]):
+        T = sum(lens)
+        parts = rand((n_parts, T, 3 * D), F32, 173 + step)
+        total = parts[0].clone()
+        for i in range(1, n_parts):
+            total += parts[i]
+        seg_start = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+        row_seg = np.repeat(np.arange(len(lens)), lens).astype(np.int32)
+        meta = [torch.from_numpy(a).to(DEV) for a in (row_seg, seg_start, np.asarray(pos0, np.int32),
+                                                      np.asarray(slot, np.int32))]
+        got = ops.shortconv(parts.to(DEV), taps.to(DEV), dev(cb), st_p, *meta)
+        want = ops.shortconv(total.to(BF16).to(DEV), taps.to(DEV), dev(cb), st_w, *meta)
+        assert got.dtype == BF16 and torch.equal(got.cpu(), want.cpu()), f"step {step}"
+        assert torch.equal(st_p.cpu(), st_w.cpu()), f"state after step {step}"
 
 
 @pytest.mark.parametrize("dtype", [F32, BF16])
