@@ -743,10 +743,10 @@ static void launch_tile(const bf16_t* A, const bf16_t* W, const float* bias, TO*
   }
   if ((shape == 5 || shape == 6 || shape == 8 || shape == 9) && !fits) shape = 3;
   if (shape == 9 && EPI != 0) shape = 5;
-  // Wf: W in fragment order (W may then be null).  The one-wave-a-SIMD kernel reads it faster
-  // than rows (gate/up of 2048 rows 122 against 135 us, in_proj 50 against 56: a tile's loads
-  // are pieces of 1 KB), the older tile kernel a little slower (47 against 43 us), so that one
-  // takes the rows when there are any.
+  // Wf: W in fragment order (W may then be null).  The one-wave-a-SIMD kernel reads it as fast as
+  // rows or a little faster (gate/up of 2048 rows 119.5 against 122-124 us in turns on one box, the
+  // other products equal: a tile's loads are pieces of 1 KB), the older tile kernel a little
+  // slower (47 against 43 us), so that one takes the rows when there are any.
   const bool block_form = shape == 5 || shape == 6 || shape == 8 || shape == 9;
   const int w_frag = Wf != nullptr && (W == nullptr || block_form);
   if (w_frag) W = Wf;

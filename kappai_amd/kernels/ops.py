@@ -330,7 +330,7 @@ def fragment_order(weight: torch.Tensor) -> Optional[torch.Tensor]:
     [(k % 32) / 8][row % 16][8 values]), so that one load instruction of a wave reads 1 KB in
     one piece.  None when the shape does not allow it (N a multiple of 16, K of 32).  Every
     product kernel for bfloat16 reads a matrix in this order (the kernels for few rows 10-20 %
-    faster than rows, the block kernels for prompts up to 10 %: a tile's 64 of K of 16 rows are
+    faster than rows, the block kernels for prompts as fast: a tile's 64 of K of 16 rows are
     2 KB in two pieces instead of 16 pieces of 128 bytes), so a matrix is kept in this order
     only: ``InFragments``."""
     if weight.dtype != BF16 or weight.dim() != 2:

@@ -25,7 +25,8 @@ def takes_partial_sums(rows: int, single_rows: bool) -> bool:
 # Every bfloat16 matrix whose shape allows it (rows a multiple of 16, columns of 32) is kept in
 # the order in which the product kernels load it (``ops.fragment_order``), and only so: decode
 # steps stream it 10-20 % faster than rows (a step at batch 8: about a tenth), the block kernels
-# of prompt steps up to 10 %.  False keeps the matrices as the checkpoint has them.
+# of prompt steps as fast as rows, and the matrices' memory is needed once.  False keeps the
+# matrices as the checkpoint has them.
 FRAGMENT_ORDER = True
 
 # The norm kernel hands its rows on in fragment order from this many rows on (up to 16): a step of
