@@ -5,6 +5,7 @@ fails it."""
 import math
 
 import numpy as np
+import pytest
 import scipy.signal
 import scipy.special
 
@@ -237,6 +238,25 @@ def test_whole_model_invariants(tmp_path):
     w1 = dict(w)
     w1["model.layers.1.self_attn.out_proj.weight"] = np.zeros_like(w["model.layers.1.self_attn.out_proj.weight"])
     assert np.abs(P.forward(cfg, w1, toks) - full).max() > 1e-3
+
+
+@pytest.mark.parametrize("name", ["A", "B", "C", "E", "F"])
+def test_two_statements_of_the_whole_model_agree(tmp_path, name):
+    """The whole-sequence statement (``plain/lfm2.py``: no state, masks and sums over the whole
+    sequence) and the token-by-token statement (``plain/lfm2_steps.py``: a shift register per conv
+    layer, keys and values appended per token, rotation as complex numbers), written apart from
+    each other, give the same logits for every position.  A wrong tap order, a state that is
+    shifted the wrong way, a rotation with the wrong sign or pairing, a norm on the wrong side of
+    the rotation, or a head read from the wrong kv group would have to be wrong in both forms."""
+    from plain import lfm2_steps
+    d = write_tiny(name, tmp_path / name.lower())
+    cfg, w = P.read_model_dir(d)
+    rng = np.random.default_rng(31)
+    toks = [int(t) for t in rng.integers(0, cfg["vocab_size"], size=14)]
+    whole = P.forward(cfg, w, toks)
+    steps = lfm2_steps.forward_by_steps(cfg, w, toks)
+    assert steps.shape == whole.shape
+    assert np.abs(steps - whole).max() < 1e-10 * max(1.0, np.abs(whole).max())
 
 
 def test_conv_bias_and_untied_head_are_used(tmp_path):
