@@ -573,3 +573,56 @@ def test_trace_semantics(tmp_path, model_dirs):
                 assert res is None and not (out_dir / f"{obj['step']}.f32").exists()
         cache.check()
         assert not cache.live_requests()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_the_order_of_the_entries_only_orders_the_logits(tmp_path, model_dirs, name, dtype):
+    """A mixed step (two prompt portions, two single decoded tokens) in two different orders of
+    its entries: the logits of every (request, place) are the same, only their order in the
+    output follows the entries; so are the logits of the steps that come after, from the cache
+    that the step left (kappai: a batch's segments are independent of each other,
+    src/recipe/exec.c:704-758)."""
+    from kappai_amd.engine.replay import TraceReplayer, make_replay_cache
+    from kappai_amd.engine.step import StepRunner
+    vocab = TINY[name][0]["vocab_size"]
+    requests = make_requests(vocab, [40, 23, 31, 12], seed=19)
+    a, b, c, d = (requests[f"r{i}"] for i in range(4))
+    ids = {"a": "r0", "b": "r1", "c": "r2", "d": "r3"}
+    before = [{"step": 0, "entries": [{"id": "a", "tokens": a[:17], "want": []},
+                                      {"id": "b", "tokens": b[:22], "want": []}], "end": []},
+              {"step": 1, "entries": [{"id": "c", "tokens": c[:9], "want": []}], "end": []}]
+    mixed = [{"id": "a", "tokens": a[17:38], "want": [0, 20]}, {"id": "b", "tokens": b[22:23], "want": [0]},
+             {"id": "c", "tokens": c[9:10], "want": [0]}, {"id": "d", "tokens": d, "want": [3, 11]}]
+    first_place = {"a": 17, "b": 22, "c": 9, "d": 0}
+    after = [{"step": 3, "entries": [{"id": "a", "tokens": a[38:], "want": [0, 1]},
+                                     {"id": "c", "tokens": c[10:], "want": [20]}],
+              "end": ["a", "b", "c", "d"]}]
+    model = gpu_model(model_dirs[name], dtype)
+    results = []
+    for order in ([0, 1, 2, 3], [3, 2, 0, 1], [1, 3, 2, 0]):
+        cache = make_replay_cache(model, 4 * 64)
+        cache.allocate_storage(model.dtype, "cuda:0", poison=True)
+        rep = TraceReplayer(StepRunner(model, cache, "cuda:0"), tmp_path / f"{dtype}{order[0]}")
+        for obj in before:
+            assert rep.run_step(obj) is None
+        entries = [mixed[i] for i in order]
+        rows = rep.run_step({"step": 2, "entries": entries, "end": []})
+        got = {}
+        at = 0
+        for e in entries:
+            for wnt in e["want"]:
+                got[(ids[e["id"]], first_place[e["id"]] + wnt)] = rows[at]
+                at += 1
+        assert at == rows.shape[0] == 6
+        later = rep.run_step(after[0])
+        got[("r0", 38)], got[("r0", 39)], got[("r2", 30)] = later[0], later[1], later[2]
+        cache.check()
+        assert not cache.live_requests()
+        results.append(got)
+    # every order against the plain implementation, and the orders against each other
+    assert_matches_plain(results[0], model_dirs[name], requests, dtype)
+    for other in results[1:]:
+        assert other.keys() == results[0].keys()
+        for key in other:
+            assert np.array_equal(other[key], results[0][key]), (key, "depends on the entries' order")
