@@ -263,6 +263,48 @@ def test_long_prompt_on_a_wide_model(tmp_path, dtype, shape):
     assert_matches_plain(got, folder, requests, dtype)
 
 
+@pytest.mark.parametrize("shape", ["wide", "wide_heads"])
+def test_short_portions_on_a_wide_model_from_c_and_from_the_host(tmp_path, shape):
+    """Steps of 17 to 256 rows on models wide enough for their in_proj and qkv products to be cut
+    into K ranges (portions of 150 and 70 rows beside single decoded tokens, a portion of 40, a
+    step of 20 single rows' worth of two requests): the conv and qk-norm kernels add the float
+    partial sums up.  Launched from C and part by part from the host the logits are bit for bit
+    the same, and both follow the plain implementation."""
+    import copy
+    from kappai_amd.config import config_from_dict
+    from kappai_amd.engine.replay import TraceReplayer, make_replay_cache
+    from kappai_amd.engine.step import StepRunner
+    from kappai_amd.kernels import ops, tuning
+    from kappai_amd.weights import write_random_model
+    raw = globals()["WIDE" if shape == "wide" else "WIDE_HEADS"]
+    folder = write_random_model(tmp_path / "wide", config_from_dict(copy.deepcopy(raw)), seed=6,
+                                std=0.02, norm_jitter=0.05)
+    assert ops.split_k_for(150, 3 * raw["hidden_size"], raw["hidden_size"]) > 1      # in_proj is cut
+    assert tuning.takes_partial_sums(150, False) and not tuning.takes_partial_sums(300, False)
+    requests = make_requests(raw["vocab_size"], [230, 75, 60], seed=16)
+    plans = {"r0": (0, [150, 70] + [1] * 10), "r1": (1, [70] + [1] * 5), "r2": (2, [40, 20])}
+    steps, index, peak = schedules.build(requests, plans)
+    model = gpu_model(folder, "bfloat16")
+    results = {}
+    for c_forward in (True, False):
+        cache = make_replay_cache(model, peak)
+        cache.allocate_storage(model.dtype, "cuda:0", poison=True)
+        runner = StepRunner(model, cache, "cuda:0", decode_graphs=False, c_forward=c_forward)
+        rep = TraceReplayer(runner, tmp_path / f"c{c_forward}")
+        outputs = {}
+        for obj in steps:
+            res = rep.run_step(obj)
+            if res is not None:
+                outputs[obj["step"]] = res
+        cache.check()
+        results[c_forward] = outputs
+    assert results[True].keys() == results[False].keys()
+    for step in results[True]:
+        assert np.array_equal(results[True][step], results[False][step]), step
+    got = collect(index, results[True], model.vocab_size)
+    assert_matches_plain(got, folder, requests, "bfloat16")
+
+
 def test_decode_attention_with_its_prologue_inside_from_c_and_from_the_host(tmp_path):
     """With more than 512 keys and a head size of 64 a decode step's attention kernel does the
     per-head norm, the rotation and the store of the new key and value itself.  The C side of a
