@@ -176,9 +176,9 @@ class DecodeBench:
         logits = self.runner.step(entries)
         self.tokens = ops.sample_rows(logits, self.temp, self.uni).tolist()
 
-    def _choose(self, logits, step, out_row):
+    def _choose(self, logits, step, out_row, also):
         from kappai_amd.kernels import ops
-        ops.sample_rows(logits, self.temp, self.uni, out=out_row)
+        ops.sample_rows(logits, self.temp, self.uni, out=out_row, also=also)
 
     def run(self, warmup, steps, run_len=8, ahead=True):
         """``steps`` decode steps, taken the way the engine takes them when nothing but decoding

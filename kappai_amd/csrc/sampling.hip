@@ -7,9 +7,16 @@
 
 #define SAMPLE_THREADS 1024
 
+// The chosen token goes to `out` and, when given, to `out2` as well (the token table of the
+// step that comes next, so that no copy runs between two decode steps queued back to back).
+__device__ __forceinline__ void put(int* __restrict__ out, int* __restrict__ out2, int at, int token) {
+  out[at] = token;
+  if (out2 != nullptr) out2[at] = token;
+}
+
 __global__ __launch_bounds__(SAMPLE_THREADS) void sample_rows_kernel(
     const float* __restrict__ logits, const float* __restrict__ temperature,
-    const float* __restrict__ uniform, int* __restrict__ out, int V) {
+    const float* __restrict__ uniform, int* __restrict__ out, int* __restrict__ out2, int V) {
   __shared__ float redf[SAMPLE_THREADS / WAVE];
   __shared__ int redi[SAMPLE_THREADS / WAVE];
   __shared__ double part[SAMPLE_THREADS];
@@ -50,7 +57,7 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_rows_kernel(
   for (int w = 1; w < nw; ++w)
     if (redf[w] > bv || (redf[w] == bv && redi[w] < bi)) { bv = redf[w]; bi = redi[w]; }
   if (!(temp > 0.f)) {
-    if (tid == 0) out[r] = bi == 0x7fffffff ? 0 : bi;
+    if (tid == 0) put(out, out2, r, bi == 0x7fffffff ? 0 : bi);
     return;
   }
 
@@ -84,7 +91,7 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_rows_kernel(
     found = pick;
   }
   __syncthreads();
-  if (tid == 0) out[r] = found;
+  if (tid == 0) put(out, out2, r, found);
 }
 
 // The same for rows of at most SAMPLE_THREADS * 4 * SR_STEPS values, which a block keeps in
@@ -103,7 +110,7 @@ __device__ __forceinline__ double wave_sum_f64(double v) {
 
 __global__ __launch_bounds__(SAMPLE_THREADS) void sample_rows_held_kernel(
     const float* __restrict__ logits, const float* __restrict__ temperature,
-    const float* __restrict__ uniform, int* __restrict__ out, int V) {
+    const float* __restrict__ uniform, int* __restrict__ out, int* __restrict__ out2, int V) {
   __shared__ float redf[SR_WAVES];
   __shared__ int redi[SR_WAVES];
   __shared__ double part[SR_WAVES * SR_STEPS];
@@ -152,7 +159,7 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_rows_held_kernel(
   for (int w = 1; w < SR_WAVES; ++w)
     if (redf[w] > bv || (redf[w] == bv && redi[w] < bi)) { bv = redf[w]; bi = redi[w]; }
   if (!(temp > 0.f)) {
-    if (tid == 0) out[r] = bi == 0x7fffffff ? 0 : bi;
+    if (tid == 0) put(out, out2, r, bi == 0x7fffffff ? 0 : bi);
     return;
   }
   // ---- e = exp(l/T - max/T); sums per (wave, step) in double ---------------------------------
@@ -210,7 +217,7 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_rows_held_kernel(
   __syncthreads();
   const int p = sh_part;
   if (p < 0 || wave != p / SR_STEPS) {
-    if (p < 0 && tid == 0) out[r] = found;                // the draw fell on the very end
+    if (p < 0 && tid == 0) put(out, out2, r, found);                // the draw fell on the very end
     return;
   }
   // ---- the wave that owns the part finds the lane, the lane its value --------------------------
@@ -237,7 +244,7 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_rows_held_kernel(
   // rounding may leave the point just past the last lane's sum: the last lane with values takes it
   const unsigned long long any = __ballot(here);
   if (any == 0ull) {
-    if (lane == 0) out[r] = min(w0 + 256 * st_p + 255, w1 - 1);
+    if (lane == 0) put(out, out2, r, min(w0 + 256 * st_p + 255, w1 - 1));
     return;
   }
   if (here) {
@@ -249,21 +256,21 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_rows_held_kernel(
       acc += (double)e[c];
       if (target < acc) { pick = c; break; }
     }
-    out[r] = min(w0 + 256 * st_p + 4 * lane + pick, w1 - 1);
+    put(out, out2, r, min(w0 + 256 * st_p + 4 * lane + pick, w1 - 1));
   }
 }
 
 extern "C" int kappai_sample_rows(const float* logits, const float* temperature,
-                                  const float* uniform, int* out, int n_rows, int V,
+                                  const float* uniform, int* out, int* out2, int n_rows, int V,
                                   hipStream_t stream) {
   if (n_rows <= 0) return 0;
   if (V < 1) return (int)hipErrorInvalidValue;
   if (V <= SAMPLE_THREADS * 4 * SR_STEPS)
     hipLaunchKernelGGL(sample_rows_held_kernel, dim3(n_rows), dim3(SAMPLE_THREADS), 0, stream,
-                       logits, temperature, uniform, out, V);
+                       logits, temperature, uniform, out, out2, V);
   else
     hipLaunchKernelGGL(sample_rows_kernel, dim3(n_rows), dim3(SAMPLE_THREADS), 0, stream, logits,
-                       temperature, uniform, out, V);
+                       temperature, uniform, out, out2, V);
   KAPPAI_RETURN_LAUNCH_STATUS();
 }
 
@@ -362,7 +369,7 @@ __global__ __launch_bounds__(FILT_THREADS) void sample_filtered_kernel(
     const float* __restrict__ logits, const int* __restrict__ rows, const int* __restrict__ keep_n,
     const float* __restrict__ temperature, const float* __restrict__ top_p,
     const float* __restrict__ min_p, const float* __restrict__ uniform, int* __restrict__ out,
-    int V) {
+    int* __restrict__ out2, int V) {
   __shared__ uint32_t hist_p[FILT_BINS][FILT_SUBS];
   __shared__ uint32_t hist[FILT_BINS];
   __shared__ uint32_t sh_prefix, sh_remaining, sh_count;
@@ -561,7 +568,7 @@ __global__ __launch_bounds__(FILT_THREADS) void sample_filtered_kernel(
     const float q = p / sum;
     auto q_of = [&](int e) { return __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(q), e)); };
     const int pick = narrow_and_draw(p_of, q_of, keep, top_p[i], min_p[i], uniform[i]);
-    if (lane == 0) out[rows[i]] = __builtin_amdgcn_readlane(id, pick);
+    if (lane == 0) put(out, out2, rows[i], __builtin_amdgcn_readlane(id, pick));
     return;
   }
   for (int e = keep + tid; e < n2; e += FILT_THREADS) { cval[e] = -INFINITY; cidx[e] = 0x7fffffff; }
@@ -594,8 +601,9 @@ __global__ __launch_bounds__(FILT_THREADS) void sample_filtered_kernel(
   if (tid < keep) cq[tid] = cval[tid] / sh_sum;
   __syncthreads();
   if (tid == 0)
-    out[rows[i]] = cidx[narrow_and_draw([&](int e) { return cval[e]; }, [&](int e) { return cq[e]; },
-                                        keep, top_p[i], min_p[i], uniform[i])];
+    put(out, out2, rows[i],
+        cidx[narrow_and_draw([&](int e) { return cval[e]; }, [&](int e) { return cq[e]; }, keep,
+                             top_p[i], min_p[i], uniform[i])]);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -612,7 +620,7 @@ __global__ __launch_bounds__(FILT_THREADS) void sample_filtered_wide_kernel(
     const float* __restrict__ logits, const int* __restrict__ rows, const int* __restrict__ keep_n,
     const float* __restrict__ temperature, const float* __restrict__ top_p,
     const float* __restrict__ min_p, const float* __restrict__ uniform, int* __restrict__ out,
-    int V, int n2, float* __restrict__ ws_val, int* __restrict__ ws_idx) {
+    int* __restrict__ out2, int V, int n2, float* __restrict__ ws_val, int* __restrict__ ws_idx) {
   __shared__ float s_val[WIDE_CHUNK];
   __shared__ int s_idx[WIDE_CHUNK];
   __shared__ int sh_stop, sh_int;
@@ -736,7 +744,7 @@ __global__ __launch_bounds__(FILT_THREADS) void sample_filtered_wide_kernel(
     if (target < acc) { pick = e; return true; }
     return false;
   });
-  if (tid == 0) out[rows[i]] = idx[pick];
+  if (tid == 0) put(out, out2, rows[i], idx[pick]);
 }
 
 // The workspace of the kernel above: floats and ints for `n_entries` rows of `n2` values each,
@@ -752,13 +760,13 @@ extern "C" int kappai_sample_filtered_wide_n2(int V) {
 extern "C" int kappai_sample_filtered_wide(const float* logits, const int* rows, const int* keep_n,
                                            const float* temperature, const float* top_p,
                                            const float* min_p, const float* uniform, int* out,
-                                           int n_entries, int V, float* ws_val, int* ws_idx,
-                                           hipStream_t stream) {
+                                           int* out2, int n_entries, int V, float* ws_val,
+                                           int* ws_idx, hipStream_t stream) {
   if (n_entries <= 0) return 0;
   if (V < 1 || V > (1 << 30) || ws_val == nullptr || ws_idx == nullptr)
     return (int)hipErrorInvalidValue;
   hipLaunchKernelGGL(sample_filtered_wide_kernel, dim3(n_entries), dim3(FILT_THREADS), 0, stream,
-                     logits, rows, keep_n, temperature, top_p, min_p, uniform, out, V,
+                     logits, rows, keep_n, temperature, top_p, min_p, uniform, out, out2, V,
                      kappai_sample_filtered_wide_n2(V), ws_val, ws_idx);
   KAPPAI_RETURN_LAUNCH_STATUS();
 }
@@ -767,14 +775,14 @@ extern "C" int kappai_sample_filtered_wide(const float* logits, const int* rows,
 extern "C" int kappai_sample_filtered(const float* logits, const int* rows, const int* keep_n,
                                       const float* temperature, const float* top_p,
                                       const float* min_p, const float* uniform, int* out,
-                                      int n_entries, int V, hipStream_t stream) {
+                                      int* out2, int n_entries, int V, hipStream_t stream) {
   if (n_entries <= 0) return 0;
   if (V < 1) return (int)hipErrorInvalidValue;
   if (V <= FILT_THREADS * 4 * FILT_STEPS)
     hipLaunchKernelGGL(sample_filtered_kernel<true>, dim3(n_entries), dim3(FILT_THREADS), 0, stream,
-                       logits, rows, keep_n, temperature, top_p, min_p, uniform, out, V);
+                       logits, rows, keep_n, temperature, top_p, min_p, uniform, out, out2, V);
   else
     hipLaunchKernelGGL(sample_filtered_kernel<false>, dim3(n_entries), dim3(FILT_THREADS), 0,
-                       stream, logits, rows, keep_n, temperature, top_p, min_p, uniform, out, V);
+                       stream, logits, rows, keep_n, temperature, top_p, min_p, uniform, out, out2, V);
   KAPPAI_RETURN_LAUNCH_STATUS();
 }

@@ -416,8 +416,8 @@ class Engine:
         reqs = [e.request for e in entries]
         samplers = [r.sampler for r in reqs]
 
-        def choose(logits, step, out_row):
-            self.sampler.launch(logits, samplers, out=out_row)
+        def choose(logits, step, out_row, also):
+            self.sampler.launch(logits, samplers, out=out_row, also=also)
 
         first = [0 if r.unread else r.tokens_from(r.computed, 1)[0] for r in reqs]
         tokens = self.runner.decode_run(
@@ -451,8 +451,8 @@ class Engine:
             return None
         first = [r.tokens_from(r.computed, 1)[0] for r in reqs]
 
-        def choose(logits, step, out_row):
-            self.sampler.launch(logits, samplers, out=out_row)
+        def choose(logits, step, out_row, also):
+            self.sampler.launch(logits, samplers, out=out_row, also=also)
 
         t0 = time.perf_counter()
         tokens = self.runner.decode_run([r.cache for r in reqs], first, n, choose)

@@ -112,9 +112,10 @@ class _DecodeGraph:
         with torch.cuda.graph(self.graph):
             self.logits = runner.forward(self.batch, self.workspace)
 
-    def _upload(self, runner: "StepRunner") -> None:
+    def _upload(self, runner: "StepRunner", keep_tokens: bool = False) -> None:
         """The mirror to the device through the next pinned buffer of the graph's ring, so that
-        several steps can be queued before the first of them has run."""
+        several steps can be queued before the first of them has run.  ``keep_tokens``: all of it
+        but the token table, which kernels queued before have filled on the GPU."""
         i = self._ring_at
         self._ring_at = (i + 1) % len(self._ring)
         if self._ring_done[i] is not None:
@@ -122,23 +123,31 @@ class _DecodeGraph:
         if self._ring[i] is None:
             self._ring[i] = torch.empty(self.total, dtype=torch.int32, pin_memory=True)
         self._ring[i].numpy()[:] = self.mirror
-        ops.ints_from_host(self._ring[i], self.static)
+        first = self.offsets["row_pos"] if keep_tokens else 0      # (the token table comes first)
+        ops.ints_from_host(self._ring[i][first:], self.static[first:])
         ev = self._ring_done[i] = torch.cuda.Event()
         ev.record()
 
+    def token_table(self, n: int) -> torch.Tensor:
+        """Where the next replay reads the tokens of its first ``n`` rows."""
+        return self.views["tokens"][:n]
+
     def run(self, runner: "StepRunner", caches, tokens, pos, slots, logit_rows,
-            device_tokens: Optional[torch.Tensor] = None, placed=None) -> torch.Tensor:
+            device_tokens: Optional[torch.Tensor] = None, placed=None,
+            tokens_in_place: bool = False) -> torch.Tensor:
         """``tokens`` from the host, or ``device_tokens`` (int32 [B] on the GPU, e.g. what the last
         step's sampling kernel wrote) copied into place on the GPU, or the host's with some of
-        them replaced on the GPU (``placed``, as in ``StepRunner.step``)."""
+        them replaced on the GPU (``placed``, as in ``StepRunner.step``), or none of these:
+        ``tokens_in_place`` says that kernels queued before this call write the tokens into
+        ``token_table`` themselves."""
         h = self.h
         if placed is not None:
             for k, (row, at) in enumerate(placed[1]):
                 h["place_dst"][k] = row
                 h["place_src"][k] = at
         n = len(caches)                  # rows n .. B-1 are dummies: token 0 at position 0 of
-        if device_tokens is None:        # the scratch slot and page, logits nobody reads
-            h["tokens"][:n] = tokens
+        if device_tokens is None and not tokens_in_place:     # the scratch slot and page, logits
+            h["tokens"][:n] = tokens                           # nobody reads
         h["tokens"][n:] = 0
         h["row_pos"][:n] = pos
         h["row_pos"][n:] = 0
@@ -164,8 +173,10 @@ class _DecodeGraph:
                 for g, page in enumerate(self.scratch[1]):
                     h[f"block_table_{g}"][si] = page
                 self.rows_of[si] = None
-        self._upload(runner)
-        if device_tokens is not None:
+        self._upload(runner, keep_tokens=tokens_in_place)
+        if tokens_in_place:
+            pass
+        elif device_tokens is not None:
             self.batch.tokens[:n].copy_(device_tokens)
         elif placed is not None and placed[1]:
             m = len(placed[1])
@@ -316,8 +327,9 @@ class StepRunner:
                    placed=None) -> Optional[torch.Tensor]:
         """``n_steps`` decode steps of the same requests, queued back to back: the token a step
         chooses goes to the next step on the GPU, and the host does not wait in between.
-        ``choose(logits, step, out_row)`` queues the kernels that write one token per request
-        (int32) into ``out_row``.  Returns the tokens [n_steps, B] on the GPU (not yet waited
+        ``choose(logits, step, out_row, also)`` queues the kernels that write one token per request
+        (int32) into ``out_row`` and, when ``also`` is a tensor, into it as well (the token table
+        of the next step: no copy runs between two steps).  Returns the tokens [n_steps, B] on the GPU (not yet waited
         for), or None when the run cannot be made this way (no captured graph for the shape
         yet, not enough pages for all the steps): then nothing has changed.  After the run
         every cache holds ``n_steps`` more tokens.  ``placed`` = (int32 tensor on the GPU, [(request,
@@ -349,11 +361,10 @@ class StepRunner:
                 self.cache.extend_one(c)
             pos = np.fromiter((c.length for c in caches), dtype=np.int32, count=B)
             logits = graph.run(self, caches, tokens, pos, slots, rows,
-                               device_tokens=None if s == 0 else out[s - 1],
-                               placed=placed if s == 0 else None)
+                               placed=placed if s == 0 else None, tokens_in_place=s > 0)
             for c in caches:
                 self.cache.commit_one(c)
-            choose(logits, s, out[s])
+            choose(logits, s, out[s], graph.token_table(B) if s + 1 < n_steps else None)
             self.graph_replays += 1
             self.steps_run += 1
         return out

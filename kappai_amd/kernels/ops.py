@@ -967,11 +967,21 @@ def _decode_split(lib, q, H, G, d, k_pool, v_pool, row_pos, row_seg, block_table
 
 
 # ---------------------------------------------------------------------------------------
+def _also(also: Optional[torch.Tensor], n: int) -> _vp:
+    if also is None:
+        return _vp(0)
+    _gpu("also", also, I32)
+    _need(also.shape == (n,), "also: a second place for one token a row")
+    return _vp(also.data_ptr())
+
+
 def sample_rows(logits: torch.Tensor, temperature: torch.Tensor, uniform: torch.Tensor,
-                out: Optional[torch.Tensor] = None) -> torch.Tensor:
+                out: Optional[torch.Tensor] = None,
+                also: Optional[torch.Tensor] = None) -> torch.Tensor:
     """One token per row of ``logits`` [n, V] (float32): argmax (lowest id on ties) where the
     row's temperature is <= 0, else an inverse-CDF draw of softmax(logits / T) at the row's
-    uniform number.  ``out`` (int32 [n]) receives the tokens when given."""
+    uniform number.  ``out`` (int32 [n]) receives the tokens when given, ``also`` (int32 [n])
+    receives them as well (the token table of the step that comes next)."""
     _gpu("logits", logits, F32)
     _gpu("temperature", temperature, F32)
     _gpu("uniform", uniform, F32)
@@ -983,8 +993,8 @@ def sample_rows(logits: torch.Tensor, temperature: torch.Tensor, uniform: torch.
         _gpu("out", out, I32)
         _need(out.shape == (n,), "sample_rows: out must hold one token a row")
     check(library("sampling").kappai_sample_rows(
-        _ptr(logits), _ptr(temperature), _ptr(uniform), _ptr(out), _c_int(n), _c_int(V),
-        _stream()), "sample_rows")
+        _ptr(logits), _ptr(temperature), _ptr(uniform), _ptr(out), _also(also, n), _c_int(n),
+        _c_int(V), _stream()), "sample_rows")
     return out
 
 
@@ -993,11 +1003,13 @@ FILTER_MAX_KEEP = 1024     # candidates the filtered-sampling kernel can hold
 
 def sample_filtered(logits: torch.Tensor, rows: torch.Tensor, keep: torch.Tensor,
                     temperature: torch.Tensor, top_p: torch.Tensor, min_p: torch.Tensor,
-                    uniform: torch.Tensor, out: torch.Tensor, wide: bool = False) -> None:
+                    uniform: torch.Tensor, out: torch.Tensor, wide: bool = False,
+                    also: Optional[torch.Tensor] = None) -> None:
     """For every entry i: draw a token for row ``rows[i]`` of ``logits`` from its ``keep[i]``
     largest logits after temperature, top-p and min-p, at ``uniform[i]``, and write it to
     ``out[rows[i]]`` (int32).  ``keep[i]`` is at most ``FILTER_MAX_KEEP``, or, with ``wide``, any
-    number up to the vocabulary (a slower kernel that sorts whole rows in a workspace)."""
+    number up to the vocabulary (a slower kernel that sorts whole rows in a workspace).  ``also``:
+    a second tensor like ``out`` that receives the same tokens."""
     _gpu("logits", logits, F32)
     _gpu("rows", rows, I32)
     _gpu("keep", keep, I32)
@@ -1015,12 +1027,13 @@ def sample_filtered(logits: torch.Tensor, rows: torch.Tensor, keep: torch.Tensor
         ws_idx = torch.empty((n, n2), dtype=I32, device=logits.device)
         check(lib.kappai_sample_filtered_wide(
             _ptr(logits), _ptr(rows), _ptr(keep), _ptr(temperature), _ptr(top_p), _ptr(min_p),
-            _ptr(uniform), _ptr(out), _c_int(n), _c_int(logits.shape[1]), _ptr(ws_val),
-            _ptr(ws_idx), _stream()), "sample_filtered_wide")
+            _ptr(uniform), _ptr(out), _also(also, logits.shape[0]), _c_int(n),
+            _c_int(logits.shape[1]), _ptr(ws_val), _ptr(ws_idx), _stream()), "sample_filtered_wide")
         return
     check(library("sampling").kappai_sample_filtered(
         _ptr(logits), _ptr(rows), _ptr(keep), _ptr(temperature), _ptr(top_p), _ptr(min_p),
-        _ptr(uniform), _ptr(out), _c_int(n), _c_int(logits.shape[1]), _stream()), "sample_filtered")
+        _ptr(uniform), _ptr(out), _also(also, logits.shape[0]), _c_int(n), _c_int(logits.shape[1]),
+        _stream()), "sample_filtered")
 
 
 def repeat_penalty(logits: torch.Tensor, row_start: torch.Tensor, tokens: torch.Tensor,

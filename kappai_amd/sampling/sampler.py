@@ -80,13 +80,14 @@ class Sampler:
         return all(s.params.repeat_penalty == 1.0 for s in samplers)
 
     def launch(self, logits: torch.Tensor, samplers: Sequence[RequestSampler],
-               out: Optional[torch.Tensor] = None):
+               out: Optional[torch.Tensor] = None, also: Optional[torch.Tensor] = None):
         """Queue the kernels that choose a token for every row; returns the int32 tokens on the
-        GPU.  Nothing here waits for the GPU."""
+        GPU.  ``also``: a second int32 tensor [rows] that receives them too.  Nothing here waits
+        for the GPU."""
         with profile.scope("sample"):
-            return self._launch(logits, samplers, out)
+            return self._launch(logits, samplers, out, also)
 
-    def _launch(self, logits, samplers, out):
+    def _launch(self, logits, samplers, out, also=None):
         n, vocab = logits.shape
         dev = logits.device
         temps, unis, filt, wide = [], [], [], []
@@ -112,7 +113,7 @@ class Sampler:
         filt = filt + wide
         m = len(filt)
         if not any(temps) and not m and (n, str(dev)) in self._zeros:
-            out_dev = ops.sample_rows(logits, *self._zeros[(n, str(dev))], out=out)
+            out_dev = ops.sample_rows(logits, *self._zeros[(n, str(dev))], out=out, also=also)
         else:
             packed = np.zeros(2 * n + 6 * m, dtype=np.float32)
             packed[:n] = temps
@@ -127,15 +128,15 @@ class Sampler:
             d = self._to_device(packed, dev)
             if not any(temps) and not m:
                 self._zeros[(n, str(dev))] = (d[:n], d[n:2 * n])
-            out_dev = ops.sample_rows(logits, d[:n], d[n:2 * n], out=out)
+            out_dev = ops.sample_rows(logits, d[:n], d[n:2 * n], out=out, also=also)
             if m:
                 di = d[2 * n:2 * n + 2 * m].view(torch.int32)
                 f = d[2 * n + 2 * m:]
                 cols = (di[:m], di[m:], f[:m], f[m:2 * m], f[2 * m:3 * m], f[3 * m:4 * m])
                 if mf:
-                    ops.sample_filtered(logits, *(c[:mf] for c in cols), out_dev)
+                    ops.sample_filtered(logits, *(c[:mf] for c in cols), out_dev, also=also)
                 if m > mf:
-                    ops.sample_filtered(logits, *(c[mf:] for c in cols), out_dev, wide=True)
+                    ops.sample_filtered(logits, *(c[mf:] for c in cols), out_dev, wide=True, also=also)
         return out_dev
 
     def sample(self, logits: torch.Tensor, samplers: Sequence[RequestSampler]) -> List[int]:

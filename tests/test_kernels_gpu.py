@@ -1176,6 +1176,33 @@ def test_sample_filtered(ops):
                 assert logits[r, got[r]] == logits[r, want[r]], (V, r, got[r], want[r])
 
 
+def test_sampling_kernels_write_a_second_place(ops):
+    """Every sampling kernel writes its tokens to ``also`` as well when given (the token table of
+    the decode step that is queued next): the same tokens in both places, nothing else of
+    ``also`` touched."""
+    rng = np.random.default_rng(9)
+    for V in (3000, 70001):
+        n = 6
+        logits = torch.from_numpy((rng.normal(size=(n, V)) * 3).astype(np.float32)).to(DEV)
+        temp = torch.tensor([0.0, 0.9, 0.0, 1.2, 0.0, 0.7], device=DEV)
+        uni = torch.rand(n, generator=torch.Generator().manual_seed(3)).to(DEV)
+        out = torch.full((n,), -1, dtype=torch.int32, device=DEV)
+        also = torch.full((n,), -7, dtype=torch.int32, device=DEV)
+        ops.sample_rows(logits, temp, uni, out=out, also=also)
+        assert torch.equal(out, also) and torch.equal(out, ops.sample_rows(logits, temp, uni))
+        rows = torch.tensor([1, 3], dtype=torch.int32, device=DEV)
+        args = (rows, torch.tensor([40, 900], dtype=torch.int32, device=DEV), temp[rows.long()],
+                torch.tensor([0.9, 0.95], device=DEV), torch.tensor([0.05, 0.0], device=DEV),
+                uni[rows.long()])
+        before = out.clone()
+        ops.sample_filtered(logits, *args, out, also=also)
+        assert torch.equal(out, also)
+        assert torch.equal(out[[0, 2, 4, 5]], before[[0, 2, 4, 5]])
+        wide = (rows, torch.tensor([1500, 2000], dtype=torch.int32, device=DEV)) + args[2:]
+        ops.sample_filtered(logits, *wide, out, wide=True, also=also)
+        assert torch.equal(out, also) and torch.equal(out[[0, 2, 4, 5]], before[[0, 2, 4, 5]])
+
+
 def test_sample_filtered_with_a_top_k_above_what_lds_holds(ops):
     """A top-k above 1024 (the kernel that sorts the whole row in a workspace) against the plain
     sampler: vocabularies below and above a power of two and above the 4096 values that one pass
