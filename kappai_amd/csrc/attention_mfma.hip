@@ -1201,8 +1201,11 @@ __global__ __launch_bounds__(D_BLOCK_MAX_WAVES * WAVE) void attn_decode_block_ke
 }
 
 // out[t, h, :] = sum_s o_s 2^(m_s - M) / sum_s l_s 2^(m_s - M).  Four waves share the splits
-// (wave w takes s = w, w+4, ...); each computes its splits' weights one per lane.
+// (wave w takes s = w, w+4, ...); each computes its splits' weights one per lane.  The partial
+// outputs of MERGE_AHEAD splits are asked for before the maxima, so that with up to 32 splits
+// the kernel waits for memory once.
 #define MERGE_WAVES 4
+#define MERGE_AHEAD 8
 __global__ __launch_bounds__(MERGE_WAVES * WAVE) void attn_merge_kernel(
     const float* __restrict__ part_o, const float* __restrict__ part_ml,
     bf16_t* __restrict__ out, int out_stride, int H, int n_splits,
@@ -1213,6 +1216,20 @@ __global__ __launch_bounds__(MERGE_WAVES * WAVE) void attn_merge_kernel(
   const int t = row_ids ? row_ids[blockIdx.x] : blockIdx.x, h = blockIdx.y;
   const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE;
   const size_t base = ((size_t)blockIdx.x * H + h) * n_splits;
+  // the partial outputs of this wave's splits number j .. j + MERGE_AHEAD - 1
+  float o[MERGE_AHEAD][NPL];
+  auto ask = [&](int j) {
+#pragma unroll
+    for (int k = 0; k < MERGE_AHEAD; ++k) {
+      const int sk = wave + MERGE_WAVES * (j + k);
+#pragma unroll
+      for (int i = 0; i < NPL; ++i) {
+        const int e = lane + i * WAVE;
+        o[k][i] = (sk < n_splits && e < HEAD_DIM) ? part_o[(base + sk) * HEAD_DIM + e] : 0.f;
+      }
+    }
+  };
+  ask(0);
   float M = -INFINITY;
   for (int s = lane; s < n_splits; s += WAVE) M = fmaxf(M, part_ml[2 * (base + s)]);
   M = wave_max(M);
@@ -1230,14 +1247,15 @@ __global__ __launch_bounds__(MERGE_WAVES * WAVE) void attn_merge_kernel(
       l = part_ml[2 * (base + s) + 1] * wgt;
     }
     L += wave_sum(l);
-    for (int k = 0; k < WAVE; ++k) {
-      const int sk = wave + MERGE_WAVES * (j0 + k);
-      if (sk >= n_splits) break;
-      const float wk = __shfl(wgt, k, WAVE);
+    for (int k0 = 0; k0 < WAVE; k0 += MERGE_AHEAD) {
+      if (wave + MERGE_WAVES * (j0 + k0) >= n_splits) break;
+      if (j0 + k0 > 0) ask(j0 + k0);
 #pragma unroll
-      for (int i = 0; i < NPL; ++i) {
-        const int e = lane + i * WAVE;
-        if (e < HEAD_DIM) acc[i] = fmaf(part_o[(base + sk) * HEAD_DIM + e], wk, acc[i]);
+      for (int k = 0; k < MERGE_AHEAD; ++k) {
+        // a split past the end has the weight 0 and the partial output 0
+        const float wk = __shfl(wgt, k0 + k, WAVE);
+#pragma unroll
+        for (int i = 0; i < NPL; ++i) acc[i] = fmaf(o[k][i], wk, acc[i]);
       }
     }
   }
@@ -1248,13 +1266,13 @@ __global__ __launch_bounds__(MERGE_WAVES * WAVE) void attn_merge_kernel(
   if (wave != 0) return;
   L = (sh_l[0] + sh_l[1]) + (sh_l[2] + sh_l[3]);
   const float inv = L > 0.f ? 1.0f / L : 0.f;
-  bf16_t* o = out + (size_t)t * out_stride + (size_t)h * HEAD_DIM;
+  bf16_t* dst = out + (size_t)t * out_stride + (size_t)h * HEAD_DIM;
 #pragma unroll
   for (int i = 0; i < NPL; ++i) {
     const int e = lane + i * WAVE;
     const float v = (sh_acc[0][i * WAVE + lane] + sh_acc[1][i * WAVE + lane]) +
                     (sh_acc[2][i * WAVE + lane] + sh_acc[3][i * WAVE + lane]);
-    if (e < HEAD_DIM) o[e] = f32_to_bf16(v * inv);
+    if (e < HEAD_DIM) dst[e] = f32_to_bf16(v * inv);
   }
 }
 
