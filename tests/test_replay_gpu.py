@@ -519,7 +519,7 @@ def test_the_whole_1_2b_model(tmp_path, sizes_1_2b_dir, dtype):
         got = replay_in_process(folder, dtype, steps, index, peak, tmp_path / family)
         assert len(got) == total
         assert_matches_plain(got, folder, requests, dtype, what=family)
-    _models.pop((str(folder), dtype), None)        # 2.3 to 4.7 GB on the GPU (twice in bfloat16)
+    _models.pop((str(folder), dtype), None)        # 2.3 GB on the GPU in bfloat16, 4.7 GB in float32
 
 
 # A pool of more than 2^31 elements (8.7 GB of bfloat16 keys and as much of values in the one
