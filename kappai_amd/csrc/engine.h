@@ -20,7 +20,7 @@
 extern "C" {
 #endif
 
-#define KAPPAI_ENGINE_ABI 7          // bumped with every change of the structs below
+#define KAPPAI_ENGINE_ABI 8          // bumped with every change of the structs below
 #define KAPPAI_MAX_GROUPS 8          // paged groups a batch can carry block tables for
 
 // ---- the kernels' launchers, by address (they live in libraries of their own) ---------------
@@ -157,6 +157,7 @@ typedef struct kappai_model {
 // ---- the rows of a step -------------------------------------------------------------------------
 typedef struct kappai_batch {
   int n_rows, n_segments, n_logit_rows, max_position, max_segment_rows;
+  int logits_of_every_row;          // logit_rows is 0, 1, ..., n_rows - 1
   const int* tokens;                // [n_rows]
   const int* row_pos;               // [n_rows]
   const int* row_seg;               // [n_rows]

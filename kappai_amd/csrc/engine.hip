@@ -615,18 +615,28 @@ int run(const kappai_model* m, const kappai_batch* b, Arena& arena, float* logit
                              : attention_mixer(c, L, x, resid, into_ffn);
     if (!c.ok()) break;
     Rows x2 = normed(c, L.ffn_norm, resid, mixed, T, L.gate_up);
-    const Into into_next{resid, next ? &next->mixer_norm : nullptr};
+    // the norm after the last call is the final one; the head can take rows made for it when
+    // every row of the step wants its logits, in the rows' order
+    const kappai_norm* after = next ? &next->mixer_norm
+                               : (b->logits_of_every_row && b->n_logit_rows == T &&
+                                  takes_kernel_order(m->head, D)) ? &m->final_norm : nullptr;
+    const Into into_next{resid, after};
     carry = swiglu_ffn(c, L, x2, resid, into_next);
   }
   if (c.ok() && b->n_logit_rows > 0) {
     arena.reset(R_BLOCK);
     const int n = b->n_logit_rows;
-    Carry for_norm = carry;
-    if (carry.kind == C_SCALED) for_norm = Carry();      // made for no norm that runs here
-    const bool fragment = n >= m->fragment_rows_min && fragment_fits(c, n, D) &&
-                          (for_norm.kind != C_PARTS || for_norm.parts <= 8) &&
-                          takes_kernel_order(m->head, D);
-    Rows xb = norm_kernel(c, m->final_norm, resid, for_norm, T, b->logit_rows, n, fragment);
+    Rows xb;
+    if (carry.kind == C_SCALED && carry.scaled.norm == &m->final_norm) {
+      xb = carry.scaled;               // the last product made the rows, the head divides by rms
+    } else {
+      Carry for_norm = carry;
+      if (carry.kind == C_SCALED) for_norm = Carry();      // made for no norm that runs here
+      const bool fragment = n >= m->fragment_rows_min && fragment_fits(c, n, D) &&
+                            (for_norm.kind != C_PARTS || for_norm.parts <= 8) &&
+                            takes_kernel_order(m->head, D);
+      xb = norm_kernel(c, m->final_norm, resid, for_norm, T, b->logit_rows, n, fragment);
+    }
     // the head: a plain product with float results, straight into the caller's tensor
     const kappai_linear& head = m->head;
     if (head.w_is_f32) {
@@ -639,8 +649,9 @@ int run(const kappai_model* m, const kappai_batch* b, Arena& arena, float* logit
       if (!xb.is_bf16) xh = cast_to(c, xb.data, (size_t)n * D, 0, 1);
       if (D % 8 == 0 && aligned16(xh) && aligned16(head.w))
         LAUNCH(c, k.gemm_bf16(xh, head.w, head.w_frag, head.bias, logits, n, head.n, D, D, head.n,
-                              1, 0, 1, xb.frag, nullptr, 0, 0.f, nullptr, 0, nullptr, nullptr, 0,
-                              nullptr, stream));
+                              1, 0, 1, xb.frag, xb.ss, xb.ss ? xb.ss_parts : 0,
+                              xb.ss ? xb.eps : 0.f, nullptr, 0, nullptr, nullptr, 0, nullptr,
+                              stream));
       else if (head.w != nullptr)
         LAUNCH(c, k.gemm_bf16_any(xh, head.w, head.bias, logits, n, head.n, D, D, head.n, 1,
                                   stream));

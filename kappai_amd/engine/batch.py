@@ -33,7 +33,9 @@ class RowBatch:
     tokens[T], row_pos[T] (absolute position), row_seg[T] (segment of the row),
     seg_start[S+1] (first row of each segment), seg_pos0[S] (position of that row),
     seg_slot[S] (the request's state slot), block_tables[g] [S, max_blocks] for every paged
-    group g, logit_rows[n] (rows whose logits are wanted, in the order asked), q_tiles: the
+    group g, logit_rows[n] (rows whose logits are wanted, in the order asked;
+    ``logits_of_every_row``: these are the rows 0 .. T-1 in order, which the host knows and a
+    part that could fold the last norm into a product cannot read from the GPU), q_tiles: the
     segments cut into runs of at most ``Model.q_tile_rows`` rows, laid out only when a part of
     the model asks for it (the tiled attention kernel does)."""
     n_rows: int
@@ -53,6 +55,7 @@ class RowBatch:
     # of q_tiles (``Part.lone_rows_from``): their rows, and the largest of their positions
     lone_rows: Optional[torch.Tensor] = None
     max_lone_position: int = -1
+    logits_of_every_row: bool = False
     block_tables: List[torch.Tensor] = field(default_factory=list)
     host: Dict[str, np.ndarray] = field(default_factory=dict)
 
@@ -156,5 +159,6 @@ def layout_rows(entries: Sequence[StepEntry], cache: CacheManager, vocab_size: i
         "n_rows": T, "n_segments": S, "n_logit_rows": len(logit_rows),
         "max_position": max_position, "max_segment_rows": int(n_arr.max()),
         "n_groups": n_groups, "max_lone_position": max_lone_position,
+        "logits_of_every_row": logit_rows == list(range(T)),
     }
     return arrays, sizes

@@ -29,7 +29,7 @@ from ..parts.embedding import OutputHead, TokenEmbedding
 from ..parts.feed_forward import SwiGLU
 from ..parts.rotary import RotaryEncoding
 
-ENGINE_ABI = 7
+ENGINE_ABI = 8
 MAX_GROUPS = 8
 
 
@@ -89,7 +89,8 @@ class ModelDesc(Structure):
 class BatchDesc(Structure):
     _fields_ = [
         ("n_rows", c_int), ("n_segments", c_int), ("n_logit_rows", c_int), ("max_position", c_int),
-        ("max_segment_rows", c_int), ("tokens", c_void_p), ("row_pos", c_void_p),
+        ("max_segment_rows", c_int), ("logits_of_every_row", c_int),
+        ("tokens", c_void_p), ("row_pos", c_void_p),
         ("row_seg", c_void_p), ("seg_start", c_void_p), ("seg_pos0", c_void_p),
         ("seg_slot", c_void_p), ("logit_rows", c_void_p), ("q_tiles", c_void_p),
         ("n_tiles", c_int), ("lone_rows", c_void_p), ("n_lone_rows", c_int),
@@ -279,6 +280,7 @@ class CForward:
         b = BatchDesc()
         b.n_rows, b.n_segments, b.n_logit_rows = batch.n_rows, batch.n_segments, batch.n_logit_rows
         b.max_position, b.max_segment_rows = batch.max_position, batch.max_segment_rows
+        b.logits_of_every_row = 1 if batch.logits_of_every_row else 0
         b.tokens, b.row_pos, b.row_seg = (batch.tokens.data_ptr(), batch.row_pos.data_ptr(),
                                           batch.row_seg.data_ptr())
         b.seg_start, b.seg_pos0, b.seg_slot = (batch.seg_start.data_ptr(), batch.seg_pos0.data_ptr(),

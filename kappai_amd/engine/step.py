@@ -83,7 +83,8 @@ class _DecodeGraph:
             max_segment_rows=1, tokens=views["tokens"], row_pos=views["row_pos"],
             row_seg=views["row_seg"], seg_start=views["seg_start"], seg_pos0=views["seg_pos0"],
             seg_slot=views["seg_slot"], logit_rows=views["logit_rows"], q_tiles=views.get("q_tiles"),
-            block_tables=[views[f"block_table_{g}"] for g in range(n_groups)], host={})
+            block_tables=[views[f"block_table_{g}"] for g in range(n_groups)], host={},
+            logits_of_every_row=n_logit == B)
         # what never changes
         self.h["row_seg"][:] = np.arange(B)
         self.h["seg_start"][:] = np.arange(B + 1)
@@ -279,6 +280,7 @@ class StepRunner:
             seg_start=dev["seg_start"], seg_pos0=dev["seg_pos0"], seg_slot=dev["seg_slot"],
             logit_rows=dev["logit_rows"], q_tiles=dev.get("q_tiles"),
             lone_rows=dev.get("lone_rows"), max_lone_position=sizes["max_lone_position"],
+            logits_of_every_row=sizes["logits_of_every_row"],
             block_tables=[dev[f"block_table_{g}"] for g in range(sizes["n_groups"])],
             host=arrays)
 

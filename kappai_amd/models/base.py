@@ -14,6 +14,7 @@ from typing import Dict, List, Optional, Sequence
 import torch
 
 from ..config.base import ModelConfig
+from ..kernels import ops
 from ..parts.base import Block, Hidden, Norm, PositionEncoding, summed_delta
 from ..parts.embedding import OutputHead, TokenEmbedding
 from ..weights.spec import TensorSpec
@@ -121,6 +122,11 @@ class Model:
     def vocab_size(self) -> int:
         return self.config.vocab_size
 
+    def first_norm(self):
+        """What the last block of the schedule sees in place of a next block: the final norm and
+        the head that takes its rows."""
+        return self.final_norm, self.head
+
     # -- the forward pass of one step ------------------------------------------------------
     def forward(self, batch, cache) -> torch.Tensor:
         """Run the rows of ``batch`` through every call of the schedule and return float32
@@ -139,8 +145,12 @@ class Model:
                 view = cache.view(self.cache_id(ci))
             shared = call.reads_cache_of is not None
             if getattr(block, "takes_next_block", False):
-                nxt = (self.layers[self.schedule[ci + 1].layer] if ci + 1 < len(self.schedule)
-                       else None)
+                if ci + 1 < len(self.schedule):
+                    nxt = self.layers[self.schedule[ci + 1].layer]
+                else:
+                    # after the last call comes the final norm, whose rows the head takes; a
+                    # block can make them only when every row wants its logits
+                    nxt = self if getattr(batch, "logits_of_every_row", False) else None
                 h = block.forward(h, batch, view, shared_cache=shared, next_block=nxt)
             else:
                 h = block.forward(h, batch, view, shared_cache=shared)
@@ -149,7 +159,10 @@ class Model:
         delta = summed_delta(self.final_norm, h.delta)
         if (getattr(self.final_norm, "can_defer", False)
                 and getattr(self.head, "takes_deferred_rows", False)):
-            xb = self.final_norm.add_norm(h.resid, delta, rows=batch.logit_rows, defer=True)
+            made = (isinstance(delta, ops.ScaledRows)
+                    and getattr(batch, "logits_of_every_row", False))
+            xb = self.final_norm.add_norm(h.resid, delta, rows=None if made else batch.logit_rows,
+                                          defer=True)
         else:
             xb = self.final_norm.add_norm(h.resid, delta, rows=batch.logit_rows)
         return self.head.forward(xb)
