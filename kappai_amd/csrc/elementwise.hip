@@ -241,6 +241,74 @@ extern "C" int kappai_add_rmsnorm(float* resid, const void* delta, int delta_is_
   KAPPAI_RETURN_LAUNCH_STATUS();
 }
 
+// The embedding and the first norm in one kernel: resid[i] = table[ids[i]] (float32) and
+// out[i] = resid[i] * rsqrt(mean(resid[i]^2) + eps) * w, the arithmetic of embed_rows followed by
+// add_rmsnorm_row, bit for bit.  KIND: the table's layout as in kappai_embed_rows.
+template <typename T, int KIND>
+__global__ __launch_bounds__(1024) void embed_rmsnorm_row_kernel(
+    const int* __restrict__ ids, const void* __restrict__ table, float* __restrict__ resid,
+    const float* __restrict__ w, T* __restrict__ out, int D, float eps, int out_frag) {
+  __shared__ float red[16];
+  const int i = blockIdx.x;
+  const size_t r = (size_t)ids[i];
+  const int j = threadIdx.x * 8;
+  const bool in = j < D;
+  float v[8], w8[8];
+  float ss = 0.f;
+  if (in) {
+    load8(w + j, w8);
+    if (KIND == 0) {
+      load8((const float*)table + r * D + j, v);
+    } else if (KIND == 1) {
+      load8((const bf16_t*)table + r * D + j, v);
+    } else {
+      const int c = j / 8;                      // the row's 16-byte chunk: piece c / 4, group c % 4
+      load8((const bf16_t*)table + (r / 16) * 16 * D + (r % 16) * 8 + (size_t)(c / 4) * 512 +
+                (c % 4) * 128, v);
+    }
+    store8(resid + (size_t)i * D + j, v);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) ss += v[e] * v[e];
+  }
+  ss = block_sum(ss, red);
+  const float scale = 1.0f / sqrtf(ss / (float)D + eps);
+  if (in) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) w8[e] = v[e] * scale * w8[e];
+    const size_t at = out_frag ? (size_t)(j / 32) * 512 + ((size_t)((j % 32) / 8) * 16 + i) * 8
+                               : (size_t)i * D + j;
+    store8(out + at, w8);
+  }
+}
+
+// Refuses (hipErrorInvalidValue) what the row kernel does not take: the caller then runs
+// kappai_embed_rows and kappai_add_rmsnorm.
+extern "C" int kappai_embed_rmsnorm(const int* ids, const void* table, int table_is_bf16,
+                                    float* resid, const float* w, void* out, int T, int D,
+                                    float eps, int is_bf16, int out_frag, hipStream_t stream) {
+  if (T <= 0) return 0;
+  if (D % 8 || D > 8192 || (table_is_bf16 == 2 && D % 32) || ((uintptr_t)table % 16) ||
+      ((uintptr_t)resid % 16) || ((uintptr_t)out % 16) || ((uintptr_t)w % 16) ||
+      table_is_bf16 < 0 || table_is_bf16 > 2)
+    return (int)hipErrorInvalidValue;
+  if (out_frag && (!is_bf16 || T > 16 || D % 32)) return (int)hipErrorInvalidValue;
+  const int threads = ((D / 8 + WAVE - 1) / WAVE) * WAVE;
+#define KAPPAI_EMBED_NORM(TT, KIND)                                                              \
+  hipLaunchKernelGGL((embed_rmsnorm_row_kernel<TT, KIND>), dim3(T), dim3(threads), 0, stream,    \
+                     ids, table, resid, w, (TT*)out, D, eps, out_frag)
+  if (is_bf16) {
+    if (table_is_bf16 == 0) KAPPAI_EMBED_NORM(bf16_t, 0);
+    else if (table_is_bf16 == 1) KAPPAI_EMBED_NORM(bf16_t, 1);
+    else KAPPAI_EMBED_NORM(bf16_t, 2);
+  } else {
+    if (table_is_bf16 == 0) KAPPAI_EMBED_NORM(float, 0);
+    else if (table_is_bf16 == 1) KAPPAI_EMBED_NORM(float, 1);
+    else KAPPAI_EMBED_NORM(float, 2);
+  }
+#undef KAPPAI_EMBED_NORM
+  KAPPAI_RETURN_LAUNCH_STATUS();
+}
+
 // resid[r] += delta[r] without a norm (the last residual sum of a model whose output is
 // the hidden state itself)
 template <typename T>

@@ -26,6 +26,8 @@ extern "C" {
 // ---- the kernels' launchers, by address (they live in libraries of their own) ---------------
 typedef struct kappai_kernels {
   int (*embed_rows)(const int*, const void*, int, float*, int, int, hipStream_t);
+  int (*embed_rmsnorm)(const int*, const void*, int, float*, const float*, void*, int, int, float,
+                       int, int, hipStream_t);
   int (*add_rmsnorm)(float*, const void*, int, int, long, const float*, void*, const int*, int, int,
                      float, int, int, int, hipStream_t);
   int (*swiglu)(const void*, void*, int, int, int, hipStream_t);

@@ -217,6 +217,26 @@ Rows normed(Ctx& c, const kappai_norm& norm, float* resid, const Carry& carry, i
   return norm_kernel(c, norm, resid, carry, M, nullptr, 0, fragment);
 }
 
+// The first norm of a step together with the embedding that fills the residual stream.
+Rows embedded_and_normed(Ctx& c, const kappai_norm& norm, float* resid, int M,
+                         const kappai_linear& consumer) {
+  const int D = c.m->width;
+  const bool fragment = M >= c.m->fragment_rows_min && fragment_fits(c, M, D) &&
+                        takes_kernel_order(consumer, D);
+  Rows out;
+  out.is_bf16 = c.m->compute_bf16;
+  out.M = M;
+  out.D = D;
+  out.ld = D;
+  out.frag = fragment ? 1 : 0;
+  out.norm = &norm;
+  out.data = c.a->take(R_BLOCK, (size_t)(fragment ? 16 : M) * D * elem(out.is_bf16));
+  LAUNCH(c, c.m->kernels->embed_rmsnorm(c.b->tokens, c.m->embed_table, c.m->embed_is_bf16, resid,
+                                        norm.w, out.data, M, D, norm.eps, out.is_bf16,
+                                        fragment ? 1 : 0, c.stream));
+  return out;
+}
+
 void* cast_to(Ctx& c, const void* x, size_t n, int from_bf16, int to_bf16) {
   void* out = c.a->take(R_BLOCK, n * elem(to_bf16));
   LAUNCH(c, c.m->kernels->cast(x, out, (long)n, from_bf16, to_bf16, c.stream));
@@ -601,7 +621,13 @@ int run(const kappai_model* m, const kappai_batch* b, Arena& arena, float* logit
   const kappai_kernels& k = *m->kernels;
   const int T = b->n_rows, D = m->width;
   float* resid = (float*)arena.take(R_STEP, (size_t)T * D * 4);
-  LAUNCH(c, k.embed_rows(b->tokens, m->embed_table, m->embed_is_bf16, resid, T, D, stream));
+  // the embedding and the first call's norm are one kernel where the norm's row kernel takes
+  // the width (the same arithmetic as the two kernels, bit for bit)
+  const bool embed_with_norm = m->n_calls > 0 && D % 8 == 0 && D <= 8192 &&
+                               (m->embed_is_bf16 != 2 || D % 32 == 0) &&
+                               aligned16(m->embed_table) && aligned16(m->calls[0].mixer_norm.w);
+  if (!embed_with_norm)
+    LAUNCH(c, k.embed_rows(b->tokens, m->embed_table, m->embed_is_bf16, resid, T, D, stream));
   Carry carry;
   for (int ci = 0; ci < m->n_calls && c.ok(); ++ci) {
     const kappai_layer_call& L = m->calls[ci];
@@ -609,7 +635,8 @@ int run(const kappai_model* m, const kappai_batch* b, Arena& arena, float* logit
     arena.reset(R_BLOCK);
     const bool conv = L.mixer == KAPPAI_MIXER_CONV;
     const kappai_linear& first = conv ? L.in_proj : L.qkv;
-    Rows x = normed(c, L.mixer_norm, resid, carry, T, first);
+    Rows x = (ci == 0 && embed_with_norm) ? embedded_and_normed(c, L.mixer_norm, resid, T, first)
+                                          : normed(c, L.mixer_norm, resid, carry, T, first);
     const Into into_ffn{resid, &L.ffn_norm};
     const Carry mixed = conv ? conv_mixer(c, L, x, resid, into_ffn)
                              : attention_mixer(c, L, x, resid, into_ffn);

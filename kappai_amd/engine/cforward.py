@@ -38,7 +38,7 @@ def _ptrs(names):
 
 
 class Kernels(Structure):
-    _fields_ = _ptrs(["embed_rows", "add_rmsnorm", "swiglu", "cast", "gemm_f32", "gemm_bf16",
+    _fields_ = _ptrs(["embed_rows", "embed_rmsnorm", "add_rmsnorm", "swiglu", "cast", "gemm_f32", "gemm_bf16",
                       "gemm_bf16_any", "gemm_bf16_swiglu", "gemm_bf16_shortconv_step", "shortconv",
                       "shortconv_parts", "qk_norm_rope_store", "paged_attention_rows"])
 
@@ -187,7 +187,9 @@ class CForward:
         k = Kernels()
         el, gm, sc, at = (library("elementwise"), library("gemm"), library("shortconv"),
                           library("attention"))
-        for name, fn in (("embed_rows", el.kappai_embed_rows), ("add_rmsnorm", el.kappai_add_rmsnorm),
+        for name, fn in (("embed_rows", el.kappai_embed_rows),
+                         ("embed_rmsnorm", el.kappai_embed_rmsnorm),
+                         ("add_rmsnorm", el.kappai_add_rmsnorm),
                          ("swiglu", el.kappai_swiglu), ("cast", el.kappai_cast),
                          ("gemm_f32", gm.kappai_gemm_f32), ("gemm_bf16", gm.kappai_gemm_bf16),
                          ("gemm_bf16_any", gm.kappai_gemm_bf16_any),

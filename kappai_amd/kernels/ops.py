@@ -86,6 +86,35 @@ def embed_rows(ids: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
     return out
 
 
+def embed_rmsnorm(ids: torch.Tensor, table: torch.Tensor, weight: torch.Tensor, eps: float,
+                  out_dtype, fragment: bool = False):
+    """``embed_rows`` and the RMSNorm of its rows in one kernel: (float32 rows [T, D], the
+    normalised rows as ``add_rmsnorm`` would return them), the same bits as the two kernels.  For
+    widths that are multiples of 8 up to 8192 (of 32 for a table in fragment order)."""
+    _gpu("ids", ids, I32)
+    _gpu("weight", weight, F32)
+    kind = 2 if isinstance(table, InFragments) else None
+    if kind is None:
+        _gpu("table", table, (F32, BF16))
+        kind = _is_bf16(table.dtype)
+    _need(ids.dim() == 1 and table.dim() == 2, "embed_rmsnorm: ids [T], table [V, D]")
+    T, D = ids.shape[0], table.shape[1]
+    _need(weight.shape == (D,), lambda: f"embed_rmsnorm: weight {tuple(weight.shape)} for D={D}")
+    _need(D % 8 == 0 and D <= 8192 and (kind != 2 or D % 32 == 0),
+          lambda: f"embed_rmsnorm: a width of {D} takes embed_rows and add_rmsnorm")
+    if fragment:
+        _need(FragmentRows.fits(T, D, out_dtype),
+              "embed_rmsnorm: rows in fragment order need bfloat16, at most 16 rows and a width "
+              "that is a multiple of 32 (up to 8192)")
+    resid = torch.empty((T, D), dtype=F32, device=weight.device)
+    out = torch.empty((16 if fragment else T, D), dtype=out_dtype, device=weight.device)
+    check(library("elementwise").kappai_embed_rmsnorm(
+        _ptr(ids), _ptr(table), _c_int(kind), _ptr(resid), _ptr(weight), _ptr(out), _c_int(T),
+        _c_int(D), _c_float(eps), _c_int(_is_bf16(out_dtype)), _c_int(1 if fragment else 0),
+        _stream()), "embed_rmsnorm")
+    return resid, (FragmentRows(out, T, resid) if fragment else out)
+
+
 def place_tokens(tokens: torch.Tensor, dst_rows: torch.Tensor, chosen: torch.Tensor,
                  src_idx: torch.Tensor) -> None:
     """``tokens[dst_rows[i]] = chosen[src_idx[i]]`` (all int32, on the GPU): token ids that

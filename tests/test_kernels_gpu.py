@@ -47,6 +47,34 @@ def test_embed_rows(ops, dtype):
     assert torch.equal(got.cpu(), table[ids.long()].float())
 
 
+@pytest.mark.parametrize("dtype", [F32, BF16])
+@pytest.mark.parametrize("D", [96, 1000, 2048, 4104])
+def test_embedding_and_first_norm_in_one_kernel(ops, dtype, D):
+    """The kernel that embeds and normalises gives the bits of the two kernels it stands for: from
+    float rows, bfloat16 rows and a bfloat16 table kept in fragment order, as plain rows and as
+    rows in fragment order."""
+    V = 208
+    w = (1 + rand((D,), F32, 4, 0.2)).to(DEV)
+    tables = [rand((V, D), F32, 1).to(DEV), rand((V, D), BF16, 2).to(DEV)]
+    if D % 32 == 0:
+        tables.append(ops.InFragments.of(tables[1]))
+    for T in (1, 7, 13, 40):
+        ids = torch.randint(0, V, (T,), generator=torch.Generator().manual_seed(T)).int().to(DEV)
+        for table in tables:
+            for fragment in (False, True):
+                if fragment and not ops.FragmentRows.fits(T, D, dtype):
+                    continue
+                want_resid = ops.embed_rows(ids, table)
+                want = ops.add_rmsnorm(want_resid.clone(), None, w, 1e-5, dtype, fragment=fragment)
+                resid, got = ops.embed_rmsnorm(ids, table, w, 1e-5, dtype, fragment=fragment)
+                assert torch.equal(resid, want_resid)
+                if fragment:
+                    got, want = got.materialize(), want.materialize()
+                assert torch.equal(got, want), (T, D, fragment, type(table).__name__)
+    with pytest.raises(ValueError):
+        ops.embed_rmsnorm(ids, rand((V, 100), BF16, 3).to(DEV), w[:100].contiguous(), 1e-5, dtype)
+
+
 def test_stream_read_stays_inside_the_buffer(ops):
     """The read-only yardstick kernel reads whole pieces of 32 KB for each of its 512 blocks and
     never more than the buffer holds; a buffer too small for one piece a block is refused."""
