@@ -1097,8 +1097,40 @@ __device__ __forceinline__ void attn_decode_wave(
   }
 }
 
+// How many keys a split takes in this step.  The host sizes the grid for up to n_splits splits of
+// at least kps_min keys from the step's longest context; what the rows really hold decides here:
+// as many keys a split that the rows' keys together give D_TARGET_WAVES waves work (requests of
+// mixed lengths then get shorter splits than their longest context alone would give them, and
+// no wave walks a long row's keys by itself while the rest of the chip has nothing to do), and
+// no fewer than the longest row needs to fit into n_splits.  Every wave of the step computes the
+// same number from the same table; splits past a row's keys do nothing and are not merged.
+#define D_TARGET_WAVES 2048
+__device__ __forceinline__ int keys_of_row(int pos, int window) {
+  const int lo = (window > 0 && pos + 1 > window) ? pos + 1 - window : 0;
+  return pos + 1 - (lo / 32) * 32;
+}
+__device__ __forceinline__ int step_keys_per_split(const int* __restrict__ row_pos,
+                                                   const int* __restrict__ row_ids, int n_rows,
+                                                   int window, int G, int kps_min, int n_splits) {
+  const int lane = threadIdx.x % WAVE;
+  int total32 = 0, longest = 0;                  // the sum in units of 32 keys, rounded up by row
+  for (int i = lane; i < n_rows; i += WAVE) {
+    const int n = keys_of_row(row_pos[row_ids ? row_ids[i] : i], window);
+    total32 += (n + 31) / 32;
+    longest = max(longest, n);
+  }
+  total32 = wave_sum(total32);
+  longest = wave_max(longest);
+  const long long want = ((long long)total32 * G * 32 + D_TARGET_WAVES - 1) / D_TARGET_WAVES;
+  int kps = want > (1 << 30) ? (1 << 30) : (int)want;
+  kps = max(kps, (longest + n_splits - 1) / n_splits);
+  kps = max(kps, kps_min);
+  return (kps + D_KPW - 1) / D_KPW * D_KPW;
+}
+
 // The keys of a row split over blocks: block (t, g, split) is one wave that takes the keys
-// k_begin + split * keys_per_split .. and writes its partial result; attn_merge adds them up.
+// k_begin + split * kps .. (kps: step_keys_per_split, at least the caller's keys_per_split) and
+// writes its partial result; attn_merge adds up those of the splits that had keys.
 // (FUSED: with the prologue of QkFuse; a kernel of its own, because the prologue's registers would
 // halve the waves a SIMD holds for the steps that do not use it)
 template <bool FUSED>
@@ -1110,18 +1142,27 @@ __global__ __launch_bounds__(64) void attn_decode_kernel(
     float scale, int keys_per_split, int n_splits, QkFuse qk, const int* __restrict__ row_ids) {
   // (row_ids: the kernel's rows are these rows of the step, partial results are kept by their
   // place in the list)
-  const int t = row_ids ? row_ids[blockIdx.x] : blockIdx.x;
+  // Blocks go to the CUs in the order of their numbers, the row's number fastest: with a number
+  // of rows that divides the number of CUs, a CU would get the same row in every (kv head,
+  // split), and rows of different lengths would load the CUs unevenly.  Hence the rows are
+  // taken in an order that turns with the kv head and the split.
   const int g = blockIdx.y, split = blockIdx.z, lane = threadIdx.x;
+  const int ti = (int)((blockIdx.x + 7u * (blockIdx.y + gridDim.y * blockIdx.z)) % gridDim.x);
+  const int t = row_ids ? row_ids[ti] : ti;
   const int rep = H / G;
   const int col = lane % 16, kg = lane / 16;
   const int pos = row_pos[t];
-  const int* bt = block_tables + (size_t)row_seg[t] * max_blocks;
+  const int seg = row_seg[t];
+  const int kps = step_keys_per_split(row_pos, row_ids, (int)gridDim.x, window, G, keys_per_split,
+                                      n_splits);
+  const int* bt = block_tables + (size_t)seg * max_blocks;
   const int lo = (window > 0 && pos + 1 > window) ? pos + 1 - window : 0;
-  const int k_begin = (lo / 32) * 32 + split * keys_per_split;
-  const int k_end = min(k_begin + keys_per_split, pos + 1);     // exclusive
+  const int k_begin = (lo / 32) * 32 + split * kps;
+  if (k_begin > pos) return;                                   // a split past the row's keys
+  const int k_end = min(k_begin + kps, pos + 1);                // exclusive
   const bool head_ok = col < rep;
   const int h = g * rep + (head_ok ? col : 0);
-  const size_t pbase = ((size_t)blockIdx.x * H + h) * n_splits + split;
+  const size_t pbase = ((size_t)ti * H + h) * n_splits + split;
   f32x4_t o[D_MT];
   float m_run, l_run;
   attn_decode_wave<FUSED>(q, q_stride, k_pool, vt_pool, bt, max_blocks, t, g, H, G, ps, scale, lo,
@@ -1208,14 +1249,19 @@ __global__ __launch_bounds__(D_BLOCK_MAX_WAVES * WAVE) void attn_decode_block_ke
 #define MERGE_AHEAD 8
 __global__ __launch_bounds__(MERGE_WAVES * WAVE) void attn_merge_kernel(
     const float* __restrict__ part_o, const float* __restrict__ part_ml,
-    bf16_t* __restrict__ out, int out_stride, int H, int n_splits,
-    const int* __restrict__ row_ids) {
+    bf16_t* __restrict__ out, int out_stride, int H, int splits_stride,
+    const int* __restrict__ row_ids, const int* __restrict__ row_pos, int window, int G,
+    int kps_min) {
   constexpr int NPL = (HEAD_DIM + WAVE - 1) / WAVE;
   __shared__ float sh_acc[MERGE_WAVES][NPL * WAVE];
   __shared__ float sh_l[MERGE_WAVES];
   const int t = row_ids ? row_ids[blockIdx.x] : blockIdx.x, h = blockIdx.y;
   const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE;
-  const size_t base = ((size_t)blockIdx.x * H + h) * n_splits;
+  const size_t base = ((size_t)blockIdx.x * H + h) * splits_stride;
+  // the splits of this row that had keys (the decode kernel's own rule)
+  const int kps = step_keys_per_split(row_pos, row_ids, (int)gridDim.x, window, G, kps_min,
+                                      splits_stride);
+  const int n_splits = (keys_of_row(row_pos[t], window) + kps - 1) / kps;
   // the partial outputs of this wave's splits number j .. j + MERGE_AHEAD - 1
   float o[MERGE_AHEAD][NPL];
   auto ask = [&](int j) {
@@ -1384,7 +1430,7 @@ static int launch_decode(const void* q, int q_stride, const void* k_pool, const 
                        window, scale, keys_per_split, n_splits, qk, row_ids);
   hipLaunchKernelGGL(attn_merge_kernel, dim3(T, H), dim3(MERGE_WAVES * WAVE), 0, stream,
                      (const float*)part_o, (const float*)part_ml, (bf16_t*)out, out_stride, H,
-                     n_splits, row_ids);
+                     n_splits, row_ids, row_pos, window, G, keys_per_split);
   KAPPAI_RETURN_LAUNCH_STATUS();
 }
 

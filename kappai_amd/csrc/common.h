@@ -101,6 +101,29 @@ __device__ __forceinline__ float wave_max(float v) {
   return v;
 }
 
+// The same for integers (the moves carry bits, whatever they mean).
+__device__ __forceinline__ int wave_sum(int v) {
+  const auto mv = [](auto f, int x) { return __float_as_int(f(__int_as_float(x))); };
+  v += mv(dpp_move<0xB1>, v);
+  v += mv(dpp_move<0x4E>, v);
+  v += mv(dpp_move<0x124>, v);
+  v += mv(dpp_move<0x128>, v);
+  v += mv(lane_xor16, v);
+  v += mv(lane_xor32, v);
+  return v;
+}
+
+__device__ __forceinline__ int wave_max(int v) {
+  const auto mv = [](auto f, int x) { return __float_as_int(f(__int_as_float(x))); };
+  v = max(v, mv(dpp_move<0xB1>, v));
+  v = max(v, mv(dpp_move<0x4E>, v));
+  v = max(v, mv(dpp_move<0x124>, v));
+  v = max(v, mv(dpp_move<0x128>, v));
+  v = max(v, mv(lane_xor16, v));
+  v = max(v, mv(lane_xor32, v));
+  return v;
+}
+
 // Sum over a block of up to 1024 threads; `red` is LDS for 16 floats.  All threads get
 // the result.  Ends with a barrier so that `red` may be used again at once.
 __device__ __forceinline__ float block_sum(float v, float* red) {

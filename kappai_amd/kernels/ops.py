@@ -17,7 +17,9 @@ from .lib import check, library
 F32, BF16, I32 = torch.float32, torch.bfloat16, torch.int32
 MAX_HEAD_DIM = 512
 MAX_GRID_Y = 65535
-DECODE_WAVES = 2048       # waves the split-key decode attention aims to have at work
+DECODE_WAVES = 4096       # blocks the grid of the split-key decode attention provides for: the
+                          # kernel itself aims at half as many at work, counting the keys the
+                          # rows really hold (requests of mixed lengths get shorter splits)
 DECODE_MAX_SPLITS = 128   # partial results of a row's head that the merge kernel adds up at most
 # Keys up to which one block a (row, kv head) takes them all, its waves merging in LDS (8 requests
 # at 200 keys: 7.4 us against 9.4 for the split kernel and its merge; even at 1024 keys, and from
@@ -973,8 +975,11 @@ def _decode_split(lib, q, H, G, d, k_pool, v_pool, row_pos, row_seg, block_table
     # one wave keeps the loads of `kpw` keys in flight; splits are whole numbers of that, and
     # at most DECODE_MAX_SPLITS of them are merged
     kpw = lib.kappai_attn_keys_per_wave()
-    # and no more splits than it takes to have DECODE_WAVES waves at work: with many rows a
-    # wave rather takes several chunks in turn than writes a partial result for each
+    # and no more splits than DECODE_WAVES blocks: with many rows a wave rather takes several
+    # chunks in turn than writes a partial result for each.  These are the most splits and the
+    # fewest keys a split of this step; the kernels settle on a number of keys a split from the
+    # rows' own lengths (step_keys_per_split in csrc/attention_mfma.hip) and leave the rest of
+    # the splits empty.
     n_splits = max(1, min(DECODE_MAX_SPLITS, (n_keys + kpw - 1) // kpw,
                           max(1, DECODE_WAVES // (T * G))))
     keys_per_split = ((n_keys + n_splits - 1) // n_splits + kpw - 1) // kpw * kpw
