@@ -30,6 +30,9 @@ int kappai_attn_decode_static_init(void);
 // splits) without the two workspace arguments: the partial results
 //     part_o  [T, H, n_splits, HEAD_DIM] float   and   part_ml [T, H, n_splits, 2] float
 // live in the library's own device array.  Same inputs, same output, same kernels, bit for bit.
+// (n_splits is the most splits a row may have and keys_per_split the fewest keys of a split, as
+// for kappai_attn_decode: the kernels settle on the keys per split from the rows' lengths, and
+// the splits past a row's keys are neither written nor read.)
 // Returns hipErrorInvalidValue, with a message that kappai_attn_decode_static_error() returns,
 // when T * H * n_splits * (HEAD_DIM + 2) exceeds KAPPAI_ATTN_STATIC_SCRATCH_FLOATS or an
 // argument is one that kappai_attn_decode refuses.
