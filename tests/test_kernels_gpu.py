@@ -1111,6 +1111,54 @@ def test_attention_finds_one_far_key(ops, dtype):
                   f"far key at {far}, kernel {kernel}")
 
 
+@pytest.mark.parametrize("lengths", ["many long rows", "a few long rows", "a window"])
+def test_decode_attention_over_many_rows_of_mixed_lengths(ops, lengths):
+    """The decode kernel settles the keys per split from the lengths of all the step's rows: more
+    rows than a wave has lanes, where the rows' keys together decide (many long rows) and where
+    the longest row does (a few long ones among short ones), and with a window.  Every row against
+    the plain attention over its own keys; one far key of the longest row is made to stand out."""
+    H, G, d, ps = 4, 2, 64, 16
+    window = 0
+    gen = np.random.default_rng(5)
+    if lengths == "many long rows":
+        lens = [int(x) for x in gen.integers(2500, 3001, 100)] + [int(x) for x in gen.integers(1, 200, 50)]
+    elif lengths == "a few long rows":
+        lens = [6000, 5999, 4097] + [int(x) for x in gen.integers(1, 100, 67)]
+    else:
+        lens, window = [int(x) for x in gen.integers(1, 1500, 90)], 300
+    gen.shuffle(lens)
+    T = len(lens)
+    blocks = [(n + ps - 1) // ps for n in lens]
+    n_pages = sum(blocks) + 1
+    perm = gen.permutation(n_pages - 1) + 1
+    bt = np.zeros((T, max(blocks)), dtype=np.int32)
+    k = 0
+    for t in range(T):
+        bt[t, :blocks[t]] = perm[k:k + blocks[t]]
+        k += blocks[t]
+    k_pool = rand((n_pages, G, ps, d), BF16, 21)
+    v_pool = rand((n_pages, G, d, ps), BF16, 22)
+    qkv = rand((T, (H + 2 * G) * d), BF16, 23)
+    # the longest row: its key number 70 matches the query of head 1 and nothing else does
+    far_row, far = int(np.argmax(lens)), 70 if not window else max(lens) - window + 5
+    qkv[far_row, d:2 * d] = 0
+    qkv[far_row, d + 3] = 60.0
+    k_pool[torch.from_numpy(bt[far_row, :blocks[far_row]]).long(), 0, :, 3] = 0
+    k_pool[bt[far_row, far // ps], 0, far % ps, 3] = 8.0
+    row_pos = torch.tensor([n - 1 for n in lens], dtype=torch.int32)
+    row_seg = torch.arange(T, dtype=torch.int32)
+    scale = 1.0 / math.sqrt(d)
+    want = ref.paged_attention(qkv.float(), H, G, d, k_pool.float(), v_pool.float(), row_pos,
+                               row_seg, torch.from_numpy(bt), ps, scale, window=window)
+    got = ops.paged_attention(qkv.to(DEV), H, G, d, k_pool.to(DEV), v_pool.to(DEV),
+                              row_pos.to(DEV), row_seg.to(DEV), torch.from_numpy(bt).to(DEV), ps,
+                              scale, window=window, single_rows=True, max_position=max(lens) - 1,
+                              kernel="decode-split")
+    close(got.float().cpu(), want, 2 * BF16_ULP, f"decode attention, {lengths}")
+    marker = v_pool[bt[far_row, far // ps], 0, :, far % ps].float()
+    close(got[far_row, d:2 * d].float().cpu(), marker, 2 * BF16_ULP, "the far key's value")
+
+
 def test_attention_shared_tiles_find_one_far_key(ops):
     """The same for the kernel that shares key tiles between four heads of a kv head: a prompt
     portion of 40 rows after 700 cached keys; every row's query matches one far key only."""
