@@ -1112,6 +1112,9 @@ __device__ __forceinline__ int keys_of_row(int pos, int window) {
 __device__ __forceinline__ int step_keys_per_split(const int* __restrict__ row_pos,
                                                    const int* __restrict__ row_ids, int n_rows,
                                                    int window, int G, int kps_min, int n_splits) {
+  // a grid of no more blocks than the waves aimed at: the rows' keys cannot ask for longer
+  // splits than the grid's own (small batches; nothing is read)
+  if ((long long)n_rows * G * n_splits <= D_TARGET_WAVES) return kps_min;
   const int lane = threadIdx.x % WAVE;
   int total32 = 0, longest = 0;                  // the sum in units of 32 keys, rounded up by row
   for (int i = lane; i < n_rows; i += WAVE) {
