@@ -1156,8 +1156,11 @@ __global__ __launch_bounds__(64) void attn_decode_kernel(
   const int col = lane % 16, kg = lane / 16;
   const int pos = row_pos[t];
   const int seg = row_seg[t];
-  const int kps = step_keys_per_split(row_pos, row_ids, (int)gridDim.x, window, G, keys_per_split,
-                                      n_splits);
+  // (the form with the prologue runs for a few rows, where the rows' lengths cannot matter, and
+  // has no registers to spare: its splits are the caller's)
+  const int kps = FUSED ? keys_per_split
+                        : step_keys_per_split(row_pos, row_ids, (int)gridDim.x, window, G,
+                                              keys_per_split, n_splits);
   const int* bt = block_tables + (size_t)seg * max_blocks;
   const int lo = (window > 0 && pos + 1 > window) ? pos + 1 - window : 0;
   const int k_begin = (lo / 32) * 32 + split * kps;
@@ -1254,7 +1257,7 @@ __global__ __launch_bounds__(MERGE_WAVES * WAVE) void attn_merge_kernel(
     const float* __restrict__ part_o, const float* __restrict__ part_ml,
     bf16_t* __restrict__ out, int out_stride, int H, int splits_stride,
     const int* __restrict__ row_ids, const int* __restrict__ row_pos, int window, int G,
-    int kps_min) {
+    int kps_min, int planned) {
   constexpr int NPL = (HEAD_DIM + WAVE - 1) / WAVE;
   __shared__ float sh_acc[MERGE_WAVES][NPL * WAVE];
   __shared__ float sh_l[MERGE_WAVES];
@@ -1262,8 +1265,9 @@ __global__ __launch_bounds__(MERGE_WAVES * WAVE) void attn_merge_kernel(
   const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE;
   const size_t base = ((size_t)blockIdx.x * H + h) * splits_stride;
   // the splits of this row that had keys (the decode kernel's own rule)
-  const int kps = step_keys_per_split(row_pos, row_ids, (int)gridDim.x, window, G, kps_min,
-                                      splits_stride);
+  const int kps = planned ? step_keys_per_split(row_pos, row_ids, (int)gridDim.x, window, G,
+                                                kps_min, splits_stride)
+                          : kps_min;
   const int n_splits = (keys_of_row(row_pos[t], window) + kps - 1) / kps;
   // the partial outputs of this wave's splits number j .. j + MERGE_AHEAD - 1
   float o[MERGE_AHEAD][NPL];
@@ -1433,7 +1437,7 @@ static int launch_decode(const void* q, int q_stride, const void* k_pool, const 
                        window, scale, keys_per_split, n_splits, qk, row_ids);
   hipLaunchKernelGGL(attn_merge_kernel, dim3(T, H), dim3(MERGE_WAVES * WAVE), 0, stream,
                      (const float*)part_o, (const float*)part_ml, (bf16_t*)out, out_stride, H,
-                     n_splits, row_ids, row_pos, window, G, keys_per_split);
+                     n_splits, row_ids, row_pos, window, G, keys_per_split, qk.on ? 0 : 1);
   KAPPAI_RETURN_LAUNCH_STATUS();
 }
 
