@@ -1112,9 +1112,6 @@ __device__ __forceinline__ int keys_of_row(int pos, int window) {
 __device__ __forceinline__ int step_keys_per_split(const int* __restrict__ row_pos,
                                                    const int* __restrict__ row_ids, int n_rows,
                                                    int window, int G, int kps_min, int n_splits) {
-  // a grid of no more blocks than the waves aimed at: the rows' keys cannot ask for longer
-  // splits than the grid's own (small batches; nothing is read)
-  if ((long long)n_rows * G * n_splits <= D_TARGET_WAVES) return kps_min;
   const int lane = threadIdx.x % WAVE;
   int total32 = 0, longest = 0;                  // the sum in units of 32 keys, rounded up by row
   for (int i = lane; i < n_rows; i += WAVE) {
@@ -1136,7 +1133,9 @@ __device__ __forceinline__ int step_keys_per_split(const int* __restrict__ row_p
 // writes its partial result; attn_merge adds up those of the splits that had keys.
 // (FUSED: with the prologue of QkFuse; a kernel of its own, because the prologue's registers would
 // halve the waves a SIMD holds for the steps that do not use it)
-template <bool FUSED>
+// (PLAN: the keys per split come from step_keys_per_split, else they are the caller's: a kernel of
+// its own, because the rule's code costs half a microsecond even where it is skipped)
+template <bool FUSED, bool PLAN>
 __global__ __launch_bounds__(64) void attn_decode_kernel(
     const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ k_pool,
     const bf16_t* __restrict__ vt_pool, float* __restrict__ part_o, float* __restrict__ part_ml,
@@ -1156,11 +1155,9 @@ __global__ __launch_bounds__(64) void attn_decode_kernel(
   const int col = lane % 16, kg = lane / 16;
   const int pos = row_pos[t];
   const int seg = row_seg[t];
-  // (the form with the prologue runs for a few rows, where the rows' lengths cannot matter, and
-  // has no registers to spare: its splits are the caller's)
-  const int kps = FUSED ? keys_per_split
-                        : step_keys_per_split(row_pos, row_ids, (int)gridDim.x, window, G,
-                                              keys_per_split, n_splits);
+  const int kps = PLAN ? step_keys_per_split(row_pos, row_ids, (int)gridDim.x, window, G,
+                                             keys_per_split, n_splits)
+                       : keys_per_split;
   const int* bt = block_tables + (size_t)seg * max_blocks;
   const int lo = (window > 0 && pos + 1 > window) ? pos + 1 - window : 0;
   const int k_begin = (lo / 32) * 32 + split * kps;
@@ -1264,27 +1261,40 @@ __global__ __launch_bounds__(MERGE_WAVES * WAVE) void attn_merge_kernel(
   const int t = row_ids ? row_ids[blockIdx.x] : blockIdx.x, h = blockIdx.y;
   const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE;
   const size_t base = ((size_t)blockIdx.x * H + h) * splits_stride;
-  // the splits of this row that had keys (the decode kernel's own rule)
-  const int kps = planned ? step_keys_per_split(row_pos, row_ids, (int)gridDim.x, window, G,
-                                                kps_min, splits_stride)
-                          : kps_min;
-  const int n_splits = (keys_of_row(row_pos[t], window) + kps - 1) / kps;
-  // the partial outputs of this wave's splits number j .. j + MERGE_AHEAD - 1
+  // the partial outputs of this wave's splits number j .. j + MERGE_AHEAD - 1, of the first
+  // `bound` splits
   float o[MERGE_AHEAD][NPL];
-  auto ask = [&](int j) {
+  auto ask = [&](int j, int bound) {
 #pragma unroll
     for (int k = 0; k < MERGE_AHEAD; ++k) {
       const int sk = wave + MERGE_WAVES * (j + k);
 #pragma unroll
       for (int i = 0; i < NPL; ++i) {
         const int e = lane + i * WAVE;
-        o[k][i] = (sk < n_splits && e < HEAD_DIM) ? part_o[(base + sk) * HEAD_DIM + e] : 0.f;
+        o[k][i] = (sk < bound && e < HEAD_DIM) ? part_o[(base + sk) * HEAD_DIM + e] : 0.f;
       }
     }
   };
-  ask(0);
-  float M = -INFINITY;
-  for (int s = lane; s < n_splits; s += WAVE) M = fmaxf(M, part_ml[2 * (base + s)]);
+  // The first partial outputs and maxima are asked for before the number of splits that had keys
+  // is known (it takes the row's position): whatever the grid has room for is loaded, and what
+  // lies past the row's splits (never written, or by an earlier step) is dropped afterwards.
+  ask(0, splits_stride);
+  const float m_first = lane < splits_stride ? part_ml[2 * (base + lane)] : -INFINITY;
+  float2 ml_first = make_float2(-INFINITY, 0.f);        // of the split wave + MERGE_WAVES * lane
+  if (wave + MERGE_WAVES * lane < splits_stride)
+    ml_first = *reinterpret_cast<const float2*>(part_ml + 2 * (base + wave + MERGE_WAVES * lane));
+  // the splits of this row that had keys (the decode kernel's own rule)
+  const int kps = planned ? step_keys_per_split(row_pos, row_ids, (int)gridDim.x, window, G,
+                                                kps_min, splits_stride)
+                          : kps_min;
+  const int n_splits = (keys_of_row(row_pos[t], window) + kps - 1) / kps;
+#pragma unroll
+  for (int k = 0; k < MERGE_AHEAD; ++k)
+#pragma unroll
+    for (int i = 0; i < NPL; ++i)
+      if (wave + MERGE_WAVES * k >= n_splits) o[k][i] = 0.f;
+  float M = lane < n_splits ? m_first : -INFINITY;
+  for (int s = lane + WAVE; s < n_splits; s += WAVE) M = fmaxf(M, part_ml[2 * (base + s)]);
   M = wave_max(M);
   float L = 0.f;
   float acc[NPL];
@@ -1295,14 +1305,15 @@ __global__ __launch_bounds__(MERGE_WAVES * WAVE) void attn_merge_kernel(
     const int s = wave + MERGE_WAVES * (j0 + lane);
     float wgt = 0.f, l = 0.f;
     if (s < n_splits) {
-      const float m = part_ml[2 * (base + s)];
-      wgt = m == -INFINITY ? 0.f : fast_exp2(m - M);
-      l = part_ml[2 * (base + s) + 1] * wgt;
+      const float2 ml = j0 == 0 ? ml_first
+                                : *reinterpret_cast<const float2*>(part_ml + 2 * (base + s));
+      wgt = ml.x == -INFINITY ? 0.f : fast_exp2(ml.x - M);
+      l = ml.y * wgt;
     }
     L += wave_sum(l);
     for (int k0 = 0; k0 < WAVE; k0 += MERGE_AHEAD) {
       if (wave + MERGE_WAVES * (j0 + k0) >= n_splits) break;
-      if (j0 + k0 > 0) ask(j0 + k0);
+      if (j0 + k0 > 0) ask(j0 + k0, n_splits);
 #pragma unroll
       for (int k = 0; k < MERGE_AHEAD; ++k) {
         // a split past the end has the weight 0 and the partial output 0
@@ -1425,19 +1436,22 @@ static int launch_decode(const void* q, int q_stride, const void* k_pool, const 
   if (ps % 16 || G < 1 || H % G || H / G > 16 || G > 65535 || n_splits < 1 || n_splits > 65535 ||
       keys_per_split < D_KPW || keys_per_split % D_KPW || (q_stride % 8))
     return (int)hipErrorInvalidValue;
-  if (qk.on)
-    hipLaunchKernelGGL(attn_decode_kernel<true>, dim3(T, G, n_splits), dim3(WAVE), 0, stream,
-                       (const bf16_t*)q, q_stride, (const bf16_t*)k_pool, (const bf16_t*)vt_pool,
-                       part_o, part_ml, row_pos, row_seg, block_tables, max_blocks, H, G, ps,
-                       window, scale, keys_per_split, n_splits, qk, row_ids);
-  else
-    hipLaunchKernelGGL(attn_decode_kernel<false>, dim3(T, G, n_splits), dim3(WAVE), 0, stream,
-                       (const bf16_t*)q, q_stride, (const bf16_t*)k_pool, (const bf16_t*)vt_pool,
-                       part_o, part_ml, row_pos, row_seg, block_tables, max_blocks, H, G, ps,
-                       window, scale, keys_per_split, n_splits, qk, row_ids);
+  // The rows' own lengths decide the keys per split when the grid has more blocks than the waves
+  // aimed at (else they could not ask for longer splits than the grid's own), and not in the form
+  // with the prologue, which runs for a few rows and has no registers to spare.
+  const bool plan = !qk.on && (long long)T * G * n_splits > D_TARGET_WAVES;
+#define KAPPAI_DECODE(FUSED, PLAN)                                                               \
+  hipLaunchKernelGGL((attn_decode_kernel<FUSED, PLAN>), dim3(T, G, n_splits), dim3(WAVE), 0,     \
+                     stream, (const bf16_t*)q, q_stride, (const bf16_t*)k_pool,                  \
+                     (const bf16_t*)vt_pool, part_o, part_ml, row_pos, row_seg, block_tables,    \
+                     max_blocks, H, G, ps, window, scale, keys_per_split, n_splits, qk, row_ids)
+  if (qk.on) KAPPAI_DECODE(true, false);
+  else if (plan) KAPPAI_DECODE(false, true);
+  else KAPPAI_DECODE(false, false);
+#undef KAPPAI_DECODE
   hipLaunchKernelGGL(attn_merge_kernel, dim3(T, H), dim3(MERGE_WAVES * WAVE), 0, stream,
                      (const float*)part_o, (const float*)part_ml, (bf16_t*)out, out_stride, H,
-                     n_splits, row_ids, row_pos, window, G, keys_per_split, qk.on ? 0 : 1);
+                     n_splits, row_ids, row_pos, window, G, keys_per_split, plan ? 1 : 0);
   KAPPAI_RETURN_LAUNCH_STATUS();
 }
 
