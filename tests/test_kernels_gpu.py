@@ -980,6 +980,39 @@ def test_lone_rows_beside_portions(ops, H, G, d, window):
     assert torch.equal(got[rest].cpu(), tiled[rest].cpu()), "the rows in tiles are not touched"
 
 
+def test_many_lone_rows_of_mixed_lengths_beside_a_portion(ops):
+    """Single decoded tokens over 3,000 to 13,000 keys beside a prompt portion, enough of them for
+    the decode kernel to settle the keys per split from the listed rows' own lengths (the rows
+    reach it through a list): every row against the plain kernel."""
+    H, G, d, ps = 4, 2, 64, 16
+    gen = np.random.default_rng(9)
+    lens = [32] + [int(x) for x in gen.integers(3000, 13001, 24)]       # tokens held after the step
+    new = [32] + [1] * 24
+    S = len(lens)
+    blocks = [(n + ps - 1) // ps for n in lens]
+    n_pages = sum(blocks) + 1
+    perm = gen.permutation(n_pages - 1) + 1
+    bt = np.zeros((S, max(blocks)), dtype=np.int32)
+    k = 0
+    for s_ in range(S):
+        bt[s_, :blocks[s_]] = perm[k:k + blocks[s_]]
+        k += blocks[s_]
+    k_pool = rand((n_pages, G, ps, d), BF16, 21).to(DEV)
+    v_pool = rand((n_pages, G, d, ps), BF16, 22).to(DEV)
+    T = sum(new)
+    q = rand((T, H * d), BF16, 23).to(DEV)
+    row_seg = torch.tensor(np.repeat(np.arange(S), new), dtype=torch.int32).to(DEV)
+    row_pos = torch.tensor(list(range(32)) + [n - 1 for n in lens[1:]], dtype=torch.int32).to(DEV)
+    tiles = torch.tensor([[0, 0, 32, 0 | (1 << 16)]], dtype=torch.int32).to(DEV)
+    lone = torch.arange(32, T, dtype=torch.int32).to(DEV)
+    args = (q, H, G, d, k_pool, v_pool, row_pos, row_seg, torch.from_numpy(bt).to(DEV), ps,
+            1.0 / math.sqrt(d))
+    plain = ops.paged_attention(*args, kernel="rows")
+    got = ops.paged_attention(*args, q_tiles=tiles, kernel="prefill", max_position=max(lens) - 1,
+                              lone_rows=lone, max_lone_position=max(lens) - 1)
+    close(got.float(), plain.float().cpu().double(), 2 * BF16_ULP, "lone rows of mixed lengths")
+
+
 def test_decode_attention_refuses_a_prologue_it_cannot_do(ops):
     c = paged_case(12, BF16, 4, 2, 48, 16, [5], [1])
     dev = {k: (v.to(DEV) if torch.is_tensor(v) else v) for k, v in c.items()}
