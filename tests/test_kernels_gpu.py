@@ -1158,7 +1158,7 @@ def test_decode_attention_over_many_rows_of_mixed_lengths(ops, lengths):
     elif lengths == "a few long rows":
         lens = [6000, 5999, 4097] + [int(x) for x in gen.integers(1, 100, 67)]
     else:
-        lens, window = [int(x) for x in gen.integers(1, 1500, 90)], 300
+        lens, window = [int(x) for x in gen.integers(1, 6000, 150)], 3000
     gen.shuffle(lens)
     T = len(lens)
     blocks = [(n + ps - 1) // ps for n in lens]
