@@ -474,6 +474,62 @@ def test_decode_steps_of_forty_requests(tmp_path, dtype):
         assert_matches_plain(got, folder, requests, dtype, what=f"{group} side by side")
 
 
+MIXED_LENGTHS_MODEL = {
+    "architectures": ["Lfm2ForCausalLM"], "model_type": "lfm2",
+    "hidden_size": 512, "num_hidden_layers": 3,
+    "layer_types": ["full_attention", "conv", "full_attention"],
+    "num_attention_heads": 16, "num_key_value_heads": 8, "head_dim": 64,
+    "intermediate_size": 1024, "block_auto_adjust_ff_dim": False,
+    "vocab_size": 777, "norm_eps": 1e-5, "rope_theta": 10000.0,
+    "conv_L_cache": 3, "conv_bias": False, "tie_embedding": True,
+    "max_position_embeddings": 4096,
+}
+
+
+def test_requests_of_mixed_lengths_decoded_side_by_side(tmp_path):
+    """Twelve requests of 150 to 2,300 tokens decoded side by side from captured graphs, in
+    bfloat16: with eight kv heads the decode attention has more blocks than waves to aim at and
+    settles the keys per split from the rows' own lengths, which change from request to request.
+    Every decoded position against the plain implementation, and the graph's steps against the
+    same steps run eagerly (bit for bit)."""
+    import copy
+    from kappai_amd.cache import CacheManager
+    from kappai_amd.config import config_from_dict
+    from kappai_amd.engine import StepEntry, StepRunner
+    from kappai_amd.weights import write_random_model
+    cfg = copy.deepcopy(MIXED_LENGTHS_MODEL)
+    folder = write_random_model(tmp_path / "mixed", config_from_dict(cfg), seed=4, std=0.04,
+                                norm_jitter=0.05)
+    n_decode = 5
+    lengths = [2300, 150, 1900, 640, 333, 2047, 1025, 512, 1500, 200, 897, 1211]
+    requests = make_requests(cfg["vocab_size"], lengths, seed=31)
+    model = gpu_model(folder, "bfloat16")
+    ids = list(requests)
+    results = {}
+    for graphs in (True, False):
+        cache = CacheManager(model.cache_specs(), 16, sum((n + 15) // 16 + 1 for n in lengths),
+                             len(ids))
+        cache.allocate_storage(model.dtype, "cuda:0", poison=True)
+        runner = StepRunner(model, cache, "cuda:0", decode_graphs=graphs)
+        caches = {rid: cache.open(rid) for rid in ids}
+        got = {}
+        for rid in ids:              # the prompts one by one, then the decode steps of all
+            runner.step([StepEntry(caches[rid], requests[rid][:-n_decode], [])])
+        for s in range(n_decode):
+            entries = [StepEntry(caches[rid], [requests[rid][s - n_decode]], [0]) for rid in ids]
+            rows = runner.step(entries).cpu().numpy()
+            for rid, row in zip(ids, rows):
+                got[(rid, len(requests[rid]) - n_decode + s)] = row
+        for rid in ids:
+            cache.close(caches[rid])
+        cache.check()
+        if graphs:
+            assert runner.graph_replays >= n_decode - 2
+        results[graphs] = got
+    assert all(np.array_equal(results[True][k], results[False][k]) for k in results[True])
+    assert_matches_plain(results[True], folder, requests, "bfloat16", what="mixed lengths")
+
+
 # LFM2-1.2B as the benchmark runs it, all sixteen layers (attention at 2, 5, 8, 10, 12, 14): width
 # 2048, 32 query heads over 8 kv heads of size 64, feed-forward 8192 from intermediate_size 12288,
 # 65,536 tokens, tied head.  The plain implementation in float64 takes some ten seconds for the
