@@ -23,14 +23,17 @@ _LAYER_TYPE_NAMES = {"conv": "conv", "full_attention": "attention", "attention":
 def adjusted_ff_dim(intermediate_size: int, auto_adjust: bool, multiple_of: int,
                     multiplier: Optional[float]) -> int:
     """Width of the SwiGLU hidden layer.  With ``block_auto_adjust_ff_dim`` the width is
-    two thirds of ``intermediate_size``, times ``block_ffn_dim_multiplier`` when given,
-    rounded up to a multiple of ``block_multiple_of``; otherwise ``intermediate_size``
-    itself.  (kappai reads the finished number, src/model.c:2329-2350.)"""
+    two thirds of ``intermediate_size``; when ``block_ffn_dim_multiplier`` is a number the
+    width is multiplied by it and then rounded up to a multiple of ``block_multiple_of``
+    (a multiplier of null leaves the two thirds as they are, unrounded); without
+    ``block_auto_adjust_ff_dim`` it is ``intermediate_size`` itself.  (kappai reads the
+    finished number, src/model.c:2329-2350.)"""
     if not auto_adjust:
         return intermediate_size
     f = (2 * intermediate_size) // 3
-    if multiplier is not None:
-        f = int(multiplier * f)
+    if multiplier is None:
+        return f
+    f = int(multiplier * f)
     return multiple_of * ((f + multiple_of - 1) // multiple_of)
 
 
@@ -53,9 +56,9 @@ class Lfm2Config(ModelConfig):
     num_key_value_heads: int = 0
     head_dim: int = 0
     intermediate_size: int = 0
-    block_auto_adjust_ff_dim: bool = False
+    block_auto_adjust_ff_dim: bool = True
     block_multiple_of: int = 256
-    block_ffn_dim_multiplier: Optional[float] = None
+    block_ffn_dim_multiplier: Optional[float] = 1.0      # None: config.json says null
     vocab_size: int = 0
     norm_eps: float = 0.0
     rope_theta: float = 0.0
@@ -113,10 +116,16 @@ class Lfm2Config(ModelConfig):
             num_attention_heads=heads,
             num_key_value_heads=r.int("num_key_value_heads"),
             head_dim=head_dim,
-            intermediate_size=r.int(("intermediate_size", "block_ff_dim")),
-            block_auto_adjust_ff_dim=r.bool("block_auto_adjust_ff_dim", False),
+            # the keys of the feed-forward width as the architecture's configuration files
+            # define them: block_ff_dim, where present, is the number the rule starts from
+            # (intermediate_size is its newer spelling); a file without the switch adjusts; a
+            # file without the multiplier has 1.0, one that says null has none
+            intermediate_size=r.int(("block_ff_dim", "intermediate_size")),
+            block_auto_adjust_ff_dim=r.bool("block_auto_adjust_ff_dim", True),
             block_multiple_of=r.int("block_multiple_of", 256),
-            block_ffn_dim_multiplier=r.float("block_ffn_dim_multiplier", None),
+            block_ffn_dim_multiplier=(None if "block_ffn_dim_multiplier" in raw
+                                      and raw["block_ffn_dim_multiplier"] is None
+                                      else r.float("block_ffn_dim_multiplier", 1.0)),
             vocab_size=r.int("vocab_size"),
             norm_eps=r.float(("norm_eps", "block_norm_eps")),
             rope_theta=_rope_theta(r),
@@ -185,8 +194,7 @@ class Lfm2Config(ModelConfig):
             "tie_embedding": self.tie_embedding,
             "max_position_embeddings": self.max_position_embeddings,
         }
-        if self.block_ffn_dim_multiplier is not None:
-            d["block_ffn_dim_multiplier"] = self.block_ffn_dim_multiplier
+        d["block_ffn_dim_multiplier"] = self.block_ffn_dim_multiplier     # null when None
         for k in ("eos_token_id", "bos_token_id", "pad_token_id"):
             if getattr(self, k) is not None:
                 d[k] = getattr(self, k)

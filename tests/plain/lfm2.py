@@ -58,19 +58,22 @@ def read_model_dir(model_dir):
 # --------------------------------------------------------------------------------------
 def feed_forward_width(cfg: dict) -> int:
     """Width of the SwiGLU hidden layer.  kappai reads it ready-made from
-    ``feed_forward_length`` (src/model.c:2329-2350); a config.json gives
-    ``intermediate_size`` and, with ``block_auto_adjust_ff_dim``, asks for
-    F = floor(2I/3), times ``block_ffn_dim_multiplier`` when set, rounded up to a
-    multiple of ``block_multiple_of``."""
-    inter = int(cfg["intermediate_size"])
-    if not cfg.get("block_auto_adjust_ff_dim", False):
+    ``feed_forward_length`` (src/model.c:2329-2350); a config.json gives ``block_ff_dim``
+    (or, in its place, ``intermediate_size``) = I and, unless ``block_auto_adjust_ff_dim`` is
+    false, asks for F = floor(2I/3); a ``block_ffn_dim_multiplier`` (1.0 when the key is
+    absent) multiplies F, which is then rounded up to a multiple of ``block_multiple_of``; a
+    multiplier of null does neither."""
+    inter = cfg.get("block_ff_dim")
+    inter = int(cfg["intermediate_size"] if inter is None else inter)
+    if not cfg.get("block_auto_adjust_ff_dim", True):
         return inter
     f = (2 * inter) // 3
-    mult = cfg.get("block_ffn_dim_multiplier")
-    if mult is not None:
-        f = int(mult * f)
+    mult = cfg.get("block_ffn_dim_multiplier", 1.0)
+    if mult is None:
+        return f
+    f = int(mult * f)
     m = int(cfg.get("block_multiple_of", 256))
-    return m * ((f + m - 1) // m)
+    return -(-f // m) * m
 
 
 def rmsnorm(x, w, eps):

@@ -29,8 +29,34 @@ def test_feed_forward_width_examples():
     assert adjusted_ff_dim(480, True, 64, 1.0) == 320
     assert adjusted_ff_dim(192, False, 256, None) == 192
     assert adjusted_ff_dim(480, True, 64, None) == 320
+    assert adjusted_ff_dim(500, True, 64, None) == 333      # no multiplier: not rounded either
+    assert adjusted_ff_dim(500, True, 64, 1.0) == 384
+    assert adjusted_ff_dim(500, True, 64, 1.5) == 512       # int(1.5 * 333) = 499
     for cfg in (TINY_A, TINY_B, TINY_C, LFM2_1_2B):
         assert config_from_dict(copy.deepcopy(cfg)).ff_dim == plain.feed_forward_width(cfg)
+
+
+def test_feed_forward_width_when_keys_are_absent():
+    """A config.json without the switch adjusts (two thirds), without the multiplier has 1.0
+    (so the width is rounded), with a multiplier of null is not rounded, and ``block_ff_dim``
+    is the number the rule starts from when both spellings are there.  Product and plain
+    implementation are held to the same four cases."""
+    base = copy.deepcopy(TINY_A)
+    for k in ("block_auto_adjust_ff_dim", "block_multiple_of", "block_ffn_dim_multiplier"):
+        base.pop(k, None)
+    base["intermediate_size"] = 500
+    cases = [({}, 512),                                              # 333 -> next 256
+             ({"block_multiple_of": 64}, 384),
+             ({"block_multiple_of": 64, "block_ffn_dim_multiplier": None}, 333),
+             ({"block_auto_adjust_ff_dim": False}, 500),
+             ({"block_ff_dim": 300, "block_multiple_of": 8}, 200),
+             ({"block_ff_dim": 300, "block_auto_adjust_ff_dim": False}, 300)]
+    for extra, want in cases:
+        raw = dict(copy.deepcopy(base), **extra)
+        cfg = config_from_dict(copy.deepcopy(raw))
+        assert cfg.ff_dim == want == plain.feed_forward_width(raw), (extra, cfg.ff_dim)
+        again = config_from_dict(cfg.to_dict())
+        assert again.ff_dim == want and again == cfg
 
 
 def test_lfm2_1_2b_shape():
@@ -71,7 +97,7 @@ def test_required_keys(key):
 def test_other_spellings_of_the_same_keys():
     """Exports of the architecture's own tools have named some keys differently over time
     (block_ff_dim, block_norm_eps, num_heads, tie_word_embeddings, rope_parameters.rope_theta);
-    the key of today wins where both are there.  A config without max_position_embeddings
+    the key of today wins where both are there (but ``block_ff_dim``, which the width rule starts from).  A config without max_position_embeddings
     names no longest sequence."""
     raw = copy.deepcopy(TINY_A)
     want = config_from_dict(copy.deepcopy(raw))
