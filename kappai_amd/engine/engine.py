@@ -136,6 +136,11 @@ class Engine:
         num_pages = config.num_pages
         if not num_pages:
             free, _ = torch.cuda.mem_get_info(self.device)
+            if config.decode_graphs:
+                # the captured decode graphs keep logits and workspaces of their own; at most a
+                # tenth of the free memory is set aside for them
+                free -= min(StepRunner.graph_bytes_bound(mc.vocab_size, config.max_batch),
+                            free // 10)
             num_pages = int(free * config.memory_fraction) // page_bytes
             if self.ctx_size:      # no more than every live request at full context
                 cap = config.max_batch * ((self.ctx_size + config.page_size - 1) // config.page_size)

@@ -312,17 +312,35 @@ class StepRunner:
         rows_b = _batch_bucket(B) if len(logit_rows) == B else B
         n_logit = rows_b if len(logit_rows) == B else len(logit_rows)
         key = (rows_b, n_logit, ctx_cap)
-        graph = self._graphs.get(key)
+        graph = self._used_graph(key)
         if graph is None:
             self._graph_seen[key] = self._graph_seen.get(key, 0) + 1
             if self._graph_seen[key] < 2:
                 return None
             if len(self._graphs) >= MAX_DECODE_GRAPHS:
-                self._graphs.pop(next(iter(self._graphs)))
+                self._graphs.pop(next(iter(self._graphs)))     # the one used longest ago
             graph = self._graphs[key] = _DecodeGraph(self, rows_b, n_logit, ctx_cap)
         slots = np.fromiter((c.slot for c in caches), dtype=np.int32, count=B)
         self.graph_replays += 1
         return graph.run(self, caches, tokens, pos, slots, logit_rows)
+
+    def _used_graph(self, key) -> Optional[_DecodeGraph]:
+        """The captured graph of this shape, moved to the end of the dictionary: its order is
+        the order of last use, so the graph that is dropped when a new shape arrives is the one
+        used longest ago, not a hot one."""
+        graph = self._graphs.pop(key, None)
+        if graph is not None:
+            self._graphs[key] = graph
+        return graph
+
+    @staticmethod
+    def graph_bytes_bound(vocab_size: int, max_batch: int) -> int:
+        """An upper bound on the device memory that captured decode graphs hold beside the cache:
+        each keeps its own logits [rows, vocab] in float32 and a workspace for its activations
+        (taken as a quarter of that again); the rows are the batch bucket of ``max_batch`` at
+        most, and ``MAX_DECODE_GRAPHS`` are kept."""
+        rows = _batch_bucket(max(1, max_batch))
+        return int(MAX_DECODE_GRAPHS * rows * vocab_size * 4 * 1.25)
 
     def decode_run(self, caches: Sequence[RequestCache], first_tokens: Sequence[int], n_steps: int,
                    choose, out: Optional[torch.Tensor] = None,
@@ -348,7 +366,7 @@ class StepRunner:
             return None
         ctx_cap = _context_bucket(max(c.length for c in caches) + n_steps)
         rows_b = _batch_bucket(B)
-        graph = self._graphs.get((rows_b, rows_b, ctx_cap))
+        graph = self._used_graph((rows_b, rows_b, ctx_cap))
         if graph is None or not self.cache.can_extend_all(caches, n_steps):
             return None
         tokens = np.asarray(first_tokens, dtype=np.int64)

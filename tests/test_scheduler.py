@@ -370,3 +370,18 @@ def test_random_load_read_late_gives_the_same_tokens(seed):
     late, lag = load(True)
     assert late == at_once
     assert all(UNREAD not in out for _, _, out in late)
+
+
+def test_decode_graphs_are_dropped_in_order_of_last_use():
+    """The step function keeps a bounded number of captured decode graphs; the one it drops for a
+    new shape is the one used longest ago, and the memory set aside for them is bounded."""
+    from kappai_amd.engine.step import MAX_DECODE_GRAPHS, StepRunner
+
+    runner = StepRunner.__new__(StepRunner)
+    runner._graphs = {("a",): 1, ("b",): 2, ("c",): 3}
+    assert runner._used_graph(("a",)) == 1
+    assert list(runner._graphs) == [("b",), ("c",), ("a",)]
+    assert runner._used_graph(("nobody",)) is None and len(runner._graphs) == 3
+    assert next(iter(runner._graphs)) == ("b",)          # what the next capture would drop
+    bound = StepRunner.graph_bytes_bound(65536, 60)      # 60 rows run in the graph of 64
+    assert bound == int(MAX_DECODE_GRAPHS * 64 * 65536 * 4 * 1.25)

@@ -2,7 +2,9 @@
 ``csrc/no_alloc.h``), called through ctypes: it keeps the splits' partial results in a device
 array of the library's own and must give, bit for bit, what ``kappai_attn_decode`` gives with a
 workspace from the caller, also on a second call with a smaller input, which finds the first
-call's partial results still in the array."""
+call's partial results still in the array.  That it allocates nothing is checked twice: the
+driver's count of free device memory does not move across the call, and the call can be recorded
+into a HIP graph, where an allocation is an error."""
 import ctypes
 import math
 
@@ -54,12 +56,43 @@ def run_both(lib, case, T, H, G, d, ps, keys_per_split, n_splits):
     assert rc == 0, rc
     got = torch.full((T, H * d), float("nan"), dtype=torch.bfloat16, device=DEV)
     torch.cuda.synchronize()
-    before = torch.cuda.memory_allocated(DEV)
+    # the driver's own count of free bytes (torch's allocator counter would not see a hipMalloc
+    # inside the library); the array's address was looked up before (init), so nothing is left
+    # that the call may take
+    free_before = torch.cuda.mem_get_info(DEV)[0]
     rc = lib.kappai_attn_decode_static(*common(got), *tables)
     assert rc == 0, (rc, lib.kappai_attn_decode_static_error().decode())
     torch.cuda.synchronize()
-    assert torch.cuda.memory_allocated(DEV) == before
+    assert torch.cuda.mem_get_info(DEV)[0] == free_before
     return got.cpu(), want.cpu()
+
+
+def capture_static(lib, case, T, H, G, d, ps, keys_per_split, n_splits, replays=3):
+    """The same call recorded into a HIP graph: while a stream is being captured (torch captures
+    in the mode that forbids it on every thread) a hipMalloc or hipFree fails and ends the
+    capture with an error, so a call that allocates and frees again is caught here where the
+    count of free bytes would not show it.  Returns the output of every replay."""
+    scale = c_float(1.0 / math.sqrt(d))
+    out = torch.full((T, H * d), float("nan"), dtype=torch.bfloat16, device=DEV)
+    graph = torch.cuda.CUDAGraph()
+    torch.cuda.synchronize()
+    with torch.cuda.graph(graph):
+        rc = lib.kappai_attn_decode_static(
+            vp(case["q"].data_ptr()), c_int(case["q"].stride(0)), vp(case["k_pool"].data_ptr()),
+            vp(case["v_pool"].data_ptr()), vp(out.data_ptr()), c_int(H * d),
+            vp(case["row_pos"].data_ptr()), vp(case["row_seg"].data_ptr()),
+            vp(case["bt"].data_ptr()), c_int(case["bt"].shape[1]), c_int(T), c_int(H), c_int(G),
+            c_int(ps), c_int(0), scale, c_int(keys_per_split), c_int(n_splits),
+            vp(torch.cuda.current_stream().cuda_stream))
+    assert rc == 0, (rc, lib.kappai_attn_decode_static_error().decode())
+    outs = []
+    for _ in range(replays):
+        out.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        outs.append(out.cpu().clone())
+    return outs
 
 
 @pytest.mark.parametrize("d", [64, 128])
@@ -82,6 +115,8 @@ def test_static_decode_matches_the_workspace_form_twice(d):
         got, want = run_both(lib, case, T, H, G, d, ps, keys_per_split, n_splits)
         assert not torch.isnan(want.float()).any()
         assert torch.equal(got.view(torch.int16), want.view(torch.int16)), (d, lengths)
+        for replayed in capture_static(lib, case, T, H, G, d, ps, keys_per_split, n_splits):
+            assert torch.equal(replayed.view(torch.int16), want.view(torch.int16)), (d, lengths)
 
 
 def test_static_decode_refuses_what_its_array_cannot_hold():
