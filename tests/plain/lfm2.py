@@ -117,30 +117,33 @@ def softmax_rows(scores):
     return e / np.sum(e, axis=-1, keepdims=True)
 
 
-def causal_attention(q, k, v, window=None):
+def causal_attention(q, k, v, window=None, rows=None):
     """q: [T, H, d], k/v: [T, G, d].  Row p sees keys 0..p; head h reads kv head
     h // (H/G) (src/backend/cpu/scalar/core.c:647); scores scaled by 1/sqrt(d)
     (src/recipe/builders.c:244-248); softmax then sum of values
     (src/backend/cpu/scalar/core.c:415-433).  With a window W a row sees only its last W
-    keys, itself included (src/backend/cpu/scalar/core.c:636-640)."""
+    keys, itself included (src/backend/cpu/scalar/core.c:636-640).  ``rows``: only these rows
+    are worked out (the others stay zero), for sequences too long to afford them all."""
     T, H, d = q.shape
     G = k.shape[1]
     rep = H // G
     scale = 1.0 / math.sqrt(d)
     out = np.zeros((T, H, d), dtype=np.float64)
-    for h in range(H):
-        g = h // rep
-        for p in range(T):
-            lo = 0
-            if window is not None and window > 0 and p + 1 > window:
-                lo = p + 1 - window
-            sc = (k[lo:p + 1, g, :] @ q[p, h, :]) * scale
-            a = softmax_rows(sc[None, :])[0]
-            out[p, h, :] = a @ v[lo:p + 1, g, :]
+    which = range(T) if rows is None else sorted(int(r) for r in rows)
+    for g in range(G):
+        kg, vg = np.ascontiguousarray(k[:, g, :]), np.ascontiguousarray(v[:, g, :])
+        for h in range(g * rep, (g + 1) * rep):
+            for p in which:
+                lo = 0
+                if window is not None and window > 0 and p + 1 > window:
+                    lo = p + 1 - window
+                sc = (kg[lo:p + 1] @ q[p, h, :]) * scale
+                a = softmax_rows(sc[None, :])[0]
+                out[p, h, :] = a @ vg[lo:p + 1]
     return out
 
 
-def gqa_attention_mixer(xb, lw, cfg, positions, rnd=lambda a: a, window=None):
+def gqa_attention_mixer(xb, lw, cfg, positions, rnd=lambda a: a, window=None, rows=None):
     """The attention layer's mixer in the reference's order (src/models/lfm.c:32-51):
     q,k,v projections; per-head RMSNorm of q and k with the layers' eps; NEOX RoPE on q
     and k; attention over the stored keys; output projection.  ``rnd`` marks the places
@@ -158,7 +161,7 @@ def gqa_attention_mixer(xb, lw, cfg, positions, rnd=lambda a: a, window=None):
     k = per_head_rmsnorm(k, lw["k_layernorm"], eps)
     q = rnd(rope_neox(q, positions, theta))
     k = rnd(rope_neox(k, positions, theta))
-    o = rnd(causal_attention(q, k, v, window=window)).reshape(T, H * d)
+    o = rnd(causal_attention(q, k, v, window=window, rows=rows)).reshape(T, H * d)
     return rnd(o @ lw["out_proj"].T)
 
 
@@ -261,8 +264,29 @@ def layer_weights(w, i, kind, cfg):
 # --------------------------------------------------------------------------------------
 # the whole model
 # --------------------------------------------------------------------------------------
-def forward(cfg: dict, w: dict, tokens, rnd=lambda a: a, return_hidden=False):
+def rows_needed(kinds, taps: int, rows):
+    """For each layer the rows of its output that the logits at ``rows`` depend on without
+    going through a later attention layer's keys and values: a conv layer needs the ``taps - 1``
+    rows before each row it is asked for, an attention layer the keys and values of all rows,
+    hence everything before it whole (None)."""
+    need, cur = [None] * len(kinds), set(int(r) for r in rows)
+    for i in reversed(range(len(kinds))):
+        need[i] = cur
+        if cur is None or kinds[i] == "attention":
+            cur = None
+        else:
+            cur = {r - j for r in cur for j in range(taps) if r - j >= 0}
+    return need
+
+
+def forward(cfg: dict, w: dict, tokens, rnd=lambda a: a, return_hidden=False, rows=None):
     """Logits [T, V] of one whole sequence.
+
+    ``rows``: only the logits at these rows are wanted (the others come back as NaN): an
+    attention layer then works out only the rows that these depend on (``rows_needed``), which
+    makes a sequence of tens of thousands of tokens affordable when only the last attention
+    layer has many keys to walk for few rows.  Everything that costs time in proportion to the
+    length (norms, projections, the FIR, the feed-forward) still runs over all rows.
 
     Order as src/recipe/exec.c:704-758: embedding rows without scale
     (src/recipe/scratch.c:195-235); per layer (src/models/lfm.c:7-62 with the tail of
@@ -276,20 +300,28 @@ def forward(cfg: dict, w: dict, tokens, rnd=lambda a: a, return_hidden=False):
     positions = np.arange(T)
     E = w["model.embed_tokens.weight"]
     x = E[tokens].astype(np.float64)
-    for i, kind in enumerate(layer_kinds(cfg)):
+    kinds = layer_kinds(cfg)
+    need = [None] * len(kinds) if rows is None else rows_needed(kinds, int(cfg["conv_L_cache"]),
+                                                                rows)
+    for i, kind in enumerate(kinds):
         lw = layer_weights(w, i, kind, cfg)
         xb = rnd(rmsnorm(x, lw["operator_norm"], eps))
         if kind == "conv":
             x = x + short_conv_mixer(xb, lw, cfg, rnd)
         else:
-            x = x + gqa_attention_mixer(xb, lw, cfg, positions, rnd)
+            x = x + gqa_attention_mixer(xb, lw, cfg, positions, rnd, rows=need[i])
         xb = rnd(rmsnorm(x, lw["ffn_norm"], eps))
         x = x + swiglu_feed_forward(xb, lw, rnd)
     if return_hidden:
         return x
     xb = rnd(rmsnorm(x, w["model.embedding_norm.weight"], eps))
     head = E if cfg.get("tie_embedding", True) else w["lm_head.weight"]
-    return xb @ head.T
+    if rows is None:
+        return xb @ head.T
+    logits = np.full((T, head.shape[0]), np.nan)
+    wanted = sorted(int(r) for r in rows)
+    logits[wanted] = xb[wanted] @ head.T
+    return logits
 
 
 def round_bf16(a):

@@ -259,6 +259,30 @@ def test_two_statements_of_the_whole_model_agree(tmp_path, name):
     assert np.abs(steps - whole).max() < 1e-10 * max(1.0, np.abs(whole).max())
 
 
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_logits_of_some_rows_only(tmp_path, name):
+    """``forward(..., rows=...)`` works out, in the attention layers, only the rows that the
+    wanted logits depend on (what long sequences need to stay affordable): the wanted rows equal
+    those of the whole computation, the others are marked as not computed; the rows a
+    layer must deliver follow the FIR's reach backwards and stop at an attention layer, which
+    needs every row before it."""
+    assert P.rows_needed(["conv", "attention", "conv"], 3, [9]) == [None, {7, 8, 9}, {9}]
+    assert P.rows_needed(["attention", "conv", "conv"], 4, [1, 20]) == [
+        {0, 1, 14, 15, 16, 17, 18, 19, 20}, {0, 1, 17, 18, 19, 20}, {1, 20}]
+    assert P.rows_needed(["attention", "attention"], 3, [5]) == [None, {5}]
+    d = write_tiny(name, tmp_path / name.lower())
+    cfg, w = P.read_model_dir(d)
+    rng = np.random.default_rng(32)
+    toks = [int(t) for t in rng.integers(0, cfg["vocab_size"], size=23)]
+    whole = P.forward(cfg, w, toks)
+    for rows in ([22], [0, 7, 21, 22], list(range(23))):
+        some = P.forward(cfg, w, toks, rows=rows)
+        # (not bit for bit: the head's product over fewer rows adds in another order)
+        assert np.abs(some[rows] - whole[rows]).max() < 1e-12 * np.abs(whole).max()
+        others = [r for r in range(23) if r not in rows]
+        assert np.isnan(some[others]).all()
+
+
 def test_conv_bias_and_untied_head_are_used(tmp_path):
     d = write_tiny("B", tmp_path / "b")
     cfg, w = P.read_model_dir(d)
