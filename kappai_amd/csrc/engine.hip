@@ -1,18 +1,22 @@
 // kappai_forward: a whole step launched from C (see engine.h).
 //
-// This file holds no kernel.  It is the host side of the framework's own parts, written once more
-// in C: the order of kernels of a pre-norm block, the choices that depend on the number of rows
-// (which product kernel, partial sums over K, rows in fragment order, the residual sum and the
-// norm folded into products), and a workspace that the activations of a step are cut from.  The
-// same step run from the host's parts, kernel by kernel, gives bit for bit the same logits; the
-// host keeps that path for models with parts this file does not know and for timing by stage.
+// This file holds no kernel and knows no part by name.  It owns what every part needs: the
+// workspace that the activations of a step are cut from, the products with their choices by
+// number of rows (which kernel, partial sums over K, rows in fragment order, the residual sum and
+// a norm folded in), the registry of runners, and the walk itself: embedding, every call of the
+// schedule through the function its description names, final norm and head.  The framework's own
+// parts are registered from engine_parts.hip like anybody else's.
 //
-// Order of a block as kappai's (src/models/lfm.c:7-62, src/recipe/builders.c:378-388):
-// x += mixer(norm(x)); x += ffn(norm(x)).
+// kappai: an operation list run through a table of handlers that each operation registered
+// (src/recipe.h:577-580, src/recipe/exec.c:467-517); order of a step src/recipe/exec.c:704-758.
 #include "engine.h"
 
 #include <stdio.h>
 #include <string.h>
+
+#include <mutex>
+#include <string>
+#include <vector>
 
 namespace {
 
@@ -21,7 +25,8 @@ thread_local char g_error[320];
 // ---------------------------------------------------------------------------------------------
 // workspace: four regions, each a stack that a dry run measures first
 // ---------------------------------------------------------------------------------------------
-enum Region { R_STEP = 0, R_CARRY_A = 1, R_CARRY_B = 2, R_BLOCK = 3, N_REGIONS = 4 };
+enum Region { R_STEP = KAPPAI_REGION_STEP, R_CARRY_A = 1, R_CARRY_B = 2,
+              R_BLOCK = KAPPAI_REGION_BLOCK, N_REGIONS = 4 };
 
 struct Arena {
   char* base = nullptr;              // null: dry run, only the sizes are followed
@@ -31,7 +36,7 @@ struct Arena {
   size_t limit[N_REGIONS] = {0, 0, 0, 0};
   bool overflow = false;
 
-  void* take(Region r, size_t bytes) {
+  void* take(int r, size_t bytes) {
     bytes = (bytes + 255) / 256 * 256;
     const size_t at = used[r];
     used[r] += bytes;
@@ -43,41 +48,11 @@ struct Arena {
     }
     return base + offset[r] + at;
   }
-  void reset(Region r) { used[r] = 0; }
+  void reset(int r) { used[r] = 0; }
 };
 
-// ---------------------------------------------------------------------------------------------
-// what travels between kernels
-// ---------------------------------------------------------------------------------------------
-// Rows on their way into a product: plain [M, D] with a row stride, 16 row slots in fragment
-// order, or either of the two still to be divided by the rows' root mean square (scaled).
-struct Rows {
-  void* data = nullptr;
-  int is_bf16 = 0;
-  int M = 0, D = 0, ld = 0;
-  int frag = 0;
-  const float* ss = nullptr;       // scaled rows: [ss_parts][16]
-  int ss_parts = 0;
-  float eps = 0.f;
-  const kappai_norm* norm = nullptr;   // the norm the scaled rows were made for
-};
-
-// What a part hands to the norm after it.
-enum CarryKind { C_NOTHING = 0, C_DELTA = 1, C_PARTS = 2, C_SCALED = 3 };
-struct Carry {
-  CarryKind kind = C_NOTHING;      // nothing: the sum is in the residual stream already
-  void* data = nullptr;            // delta [M, D] / partial sums [parts][M][D] float
-  int is_f32 = 0;
-  int parts = 1;
-  Rows scaled;                     // C_SCALED
-};
-
-struct Into {                      // ops.AddInto
-  float* resid = nullptr;
-  const kappai_norm* norm = nullptr;
-};
-
-struct Ctx {
+// The step as the walk sees it; runners see its first member only.
+struct Step : kappai_step {
   const kappai_model* m;
   const kappai_batch* b;
   Arena* a;
@@ -85,16 +60,10 @@ struct Ctx {
   bool dry;
   int status = 0;
   int carry_turn = 0;
-
-  // The region for what a part hands to the norm after it.  What the region held is two parts
-  // old by now and has been consumed (the part's own input lies in the other region).
-  Region next_carry_region() {
-    const Region r = (carry_turn++ & 1) ? R_CARRY_B : R_CARRY_A;
-    a->reset(r);
-    return r;
-  }
   bool ok() const { return status == 0 && !a->overflow; }
 };
+
+Step& of(kappai_step* s) { return *static_cast<Step*>(s); }
 
 #define LAUNCH(ctx, call)                         \
   do {                                            \
@@ -105,6 +74,11 @@ struct Ctx {
   } while (0)
 
 inline size_t elem(int is_bf16) { return is_bf16 ? 2 : 4; }
+
+void refuse(Step& c, const char* message) {
+  snprintf(g_error, sizeof g_error, "kappai_forward: %s", message);
+  c.status = (int)hipErrorInvalidValue;
+}
 
 // ---------------------------------------------------------------------------------------------
 // how many K ranges (the rule the host's parts use as well)
@@ -155,102 +129,122 @@ int split_k_for(int M, int N, int K) {
   return s < 1 ? 1 : s;
 }
 
+// how the split decode kernel cuts n_keys keys of `rows` rows
+void decode_splits(int kpw, int max_splits, int waves, int rows, int G, int n_keys,
+                   int* keys_per_split, int* n_splits) {
+  int s = max_splits;
+  if ((n_keys + kpw - 1) / kpw < s) s = (n_keys + kpw - 1) / kpw;
+  int by_waves = waves / (rows * G);
+  if (by_waves < 1) by_waves = 1;
+  if (by_waves < s) s = by_waves;
+  if (s < 1) s = 1;
+  *keys_per_split = ((n_keys + s - 1) / s + kpw - 1) / kpw * kpw;
+  *n_splits = (n_keys + *keys_per_split - 1) / *keys_per_split;
+}
+
 // ---------------------------------------------------------------------------------------------
-// the products
+// what every part may ask of the step
 // ---------------------------------------------------------------------------------------------
 bool aligned16(const void* p) { return ((uintptr_t)p % 16) == 0; }
 
 // Can the kernel for 1 to 16 rows of this matrix read rows in fragment order / scale its results?
-bool takes_kernel_order(const kappai_linear& lin, int D) {
-  return !lin.w_is_f32 && lin.k == D && aligned16(lin.w) && lin.k % 8 == 0;
+int takes_kernel_order(const kappai_linear* lin, int D) {
+  return lin != nullptr && !lin->w_is_f32 && lin->k == D && aligned16(lin->w) && lin->k % 8 == 0;
 }
 
-bool fragment_fits(const Ctx& c, int M, int D) {         // ops.FragmentRows.fits for bfloat16
-  return c.m->compute_bf16 && M >= 1 && M <= 16 && D % 32 == 0 && D <= 8192;
-}
-
-// RMSNorm by its own kernel.  rows: only these (the residual is then left alone).
-Rows norm_kernel(Ctx& c, const kappai_norm& norm, float* resid, const Carry& carry, int M,
-                 const int* rows, int n_rows, bool fragment) {
-  const int D = c.m->width;
-  const int n = rows ? n_rows : M;
-  Rows out;
-  out.is_bf16 = c.m->compute_bf16;
-  out.M = n;
-  out.D = D;
-  out.ld = D;
-  out.frag = fragment ? 1 : 0;
-  out.norm = &norm;
-  out.data = c.a->take(R_BLOCK, (size_t)(fragment ? 16 : n) * D * elem(out.is_bf16));
-  const void* delta = nullptr;
-  int delta_f32 = 0, n_part = 1;
-  long pstride = 0;
-  if (carry.kind == C_DELTA) {
-    delta = carry.data;
-    delta_f32 = carry.is_f32;
-  } else if (carry.kind == C_PARTS) {
-    delta = carry.data;
-    delta_f32 = 1;
-    n_part = carry.parts;
-    pstride = (long)M * D;
-  }
-  LAUNCH(c, c.m->kernels->add_rmsnorm(resid, delta, delta_f32, n_part, pstride, norm.w, out.data,
-                                      rows, n, D, norm.eps, rows ? 0 : 1, out.is_bf16,
-                                      fragment ? 1 : 0, c.stream));
-  return out;
-}
-
-// The rows that the product `consumer` reads after `norm` (RMSNorm.add_norm with defer): scaled
-// rows made for this norm go through as they are, else the norm's kernel runs, writing fragment
-// order when that suits the number of rows and the consumer.
-Rows normed(Ctx& c, const kappai_norm& norm, float* resid, const Carry& carry, int M,
-            const kappai_linear& consumer) {
-  const int D = c.m->width;
-  if (carry.kind == C_SCALED) {
-    if (carry.scaled.norm == &norm && takes_kernel_order(consumer, D)) return carry.scaled;
-    Carry none;                                  // the sum is in the residual already
-    return norm_kernel(c, norm, resid, none, M, nullptr, 0, false);
-  }
-  const bool fragment = M >= c.m->fragment_rows_min && fragment_fits(c, M, D) &&
-                        (carry.kind != C_PARTS || carry.parts <= 8) &&
-                        takes_kernel_order(consumer, D);
-  return norm_kernel(c, norm, resid, carry, M, nullptr, 0, fragment);
-}
-
-// The first norm of a step together with the embedding that fills the residual stream.
-Rows embedded_and_normed(Ctx& c, const kappai_norm& norm, float* resid, int M,
-                         const kappai_linear& consumer) {
-  const int D = c.m->width;
-  const bool fragment = M >= c.m->fragment_rows_min && fragment_fits(c, M, D) &&
-                        takes_kernel_order(consumer, D);
-  Rows out;
-  out.is_bf16 = c.m->compute_bf16;
-  out.M = M;
-  out.D = D;
-  out.ld = D;
-  out.frag = fragment ? 1 : 0;
-  out.norm = &norm;
-  out.data = c.a->take(R_BLOCK, (size_t)(fragment ? 16 : M) * D * elem(out.is_bf16));
-  LAUNCH(c, c.m->kernels->embed_rmsnorm(c.b->tokens, c.m->embed_table, c.m->embed_is_bf16, resid,
-                                        norm.w, out.data, M, D, norm.eps, out.is_bf16,
-                                        fragment ? 1 : 0, c.stream));
-  return out;
-}
-
-void* cast_to(Ctx& c, const void* x, size_t n, int from_bf16, int to_bf16) {
+void* cast_to(Step& c, const void* x, size_t n, int from_bf16, int to_bf16) {
   void* out = c.a->take(R_BLOCK, n * elem(to_bf16));
   LAUNCH(c, c.m->kernels->cast(x, out, (long)n, from_bf16, to_bf16, c.stream));
   return out;
 }
 
-// ops.linear.  out_bf16: the dtype of a plain result.  partial_sums: the result may come as float
-// planes over K ranges.  into: the product may add its result into the residual stream.
+// RMSNorm by its own kernel.  rows: only these (the residual is then left alone).
+kappai_rows rms_norm(Step& c, const kappai_fold* norm, float* resid, const kappai_carry& carry,
+                     int M, const int* rows, int n_rows, int fragment) {
+  const int D = c.m->width;
+  const int n = rows ? n_rows : M;
+  kappai_rows out = {};
+  out.is_bf16 = c.m->compute_bf16;
+  out.M = n;
+  out.D = D;
+  out.ld = D;
+  out.frag = fragment ? 1 : 0;
+  out.norm = norm;
+  out.data = c.a->take(R_BLOCK, (size_t)(fragment ? 16 : n) * D * elem(out.is_bf16));
+  const void* delta = nullptr;
+  int delta_f32 = 0, n_part = 1;
+  long pstride = 0;
+  if (carry.kind == KAPPAI_CARRY_DELTA) {
+    delta = carry.data;
+    delta_f32 = carry.is_f32;
+  } else if (carry.kind == KAPPAI_CARRY_PARTS) {
+    delta = carry.data;
+    delta_f32 = 1;
+    n_part = carry.parts;
+    pstride = (long)M * D;
+  } else if (carry.kind == KAPPAI_CARRY_EMBEDDING) {
+    refuse(c, "a norm kernel was asked for rows of a residual stream that is not filled yet");
+    return out;
+  }
+  LAUNCH(c, c.m->kernels->add_rmsnorm(resid, delta, delta_f32, n_part, pstride, norm->w, out.data,
+                                      rows, n, D, norm->eps, rows ? 0 : 1, out.is_bf16,
+                                      fragment ? 1 : 0, c.stream));
+  return out;
+}
+
+// Scaled rows or rows in fragment order that a kernel cannot take are made by the norm's own
+// kernel from the residual stream instead.
+kappai_rows plain_rows(Step& c, const kappai_rows& x, float* resid) {
+  if (x.ss == nullptr && !x.frag) return x;
+  if (x.norm == nullptr) {
+    refuse(c, "rows in kernel order that name no norm cannot be made anew");
+    return x;
+  }
+  kappai_carry none = {};
+  return rms_norm(c, x.norm, resid, none, x.M, nullptr, 0, 0);
+}
+
+kappai_carry plain_carry(Step& c, kappai_carry carry, float* resid, int M) {
+  const int D = c.m->width;
+  kappai_carry out = {};
+  switch (carry.kind) {
+    case KAPPAI_CARRY_EMBEDDING:
+      LAUNCH(c, c.m->kernels->embed_rows(c.b->tokens, c.m->embed_table, c.m->embed_is_bf16, resid,
+                                         M, D, c.stream));
+      return out;
+    case KAPPAI_CARRY_SCALED:
+      return out;                          // the sum is in the stream already
+    case KAPPAI_CARRY_PARTS:
+      out.kind = KAPPAI_CARRY_DELTA;
+      out.is_f32 = 1;
+      out.parts = 1;
+      out.data = c.a->take(R_BLOCK, (size_t)M * D * 4);
+      LAUNCH(c, c.m->kernels->sum_partials((const float*)carry.data, carry.parts, (long)M * D,
+                                           (float*)out.data, c.stream));
+      return out;
+    default:
+      return carry;
+  }
+}
+
+bool fragment_fits(const Step& c, int M, int D) {         // 8 to 16 bfloat16 rows of whole pieces
+  return c.m->compute_bf16 && M >= 1 && M <= 16 && D % 32 == 0 && D <= 8192;
+}
+
+// The products.  out_bf16: the dtype of a plain result.  partial_sums: the result may come as
+// float planes over K ranges.  into: the product may add its result into the residual stream.
 // region: where a result that outlives the block goes (the carry to the next norm).
-Carry linear(Ctx& c, Rows x, const kappai_linear& lin, int out_bf16, bool partial_sums,
-             const Into* into, Region region) {
+kappai_carry linear(Step& c, kappai_rows x, const kappai_linear& lin, int out_bf16,
+                    bool partial_sums, const kappai_into* into, int region) {
   const kappai_kernels& k = *c.m->kernels;
-  Carry out;
+  const kappai_tuning& tune = c.m->tuning;
+  kappai_carry out = {};
+  out.parts = 1;
   const int M = x.M, K = x.D, N = lin.n;
+  if (region < 0 || region >= N_REGIONS) {
+    refuse(c, "a product was given a region of the workspace that does not exist");
+    return out;
+  }
   if (lin.k != K) {
     snprintf(g_error, sizeof g_error, "kappai_forward: rows of width %d meet a matrix [%d, %d]", K,
              lin.n, lin.k);
@@ -259,13 +253,17 @@ Carry linear(Ctx& c, Rows x, const kappai_linear& lin, int out_bf16, bool partia
   }
   if (lin.w_is_f32) {
     // a matrix stored in 32 bits: true 32-bit arithmetic whatever the activations are
+    if (x.ss != nullptr || x.frag) {
+      refuse(c, "rows in kernel order reached a matrix stored in 32 bits");
+      return out;
+    }
     const float* xf = x.is_bf16 ? (const float*)cast_to(c, x.data, (size_t)M * K, 1, 0)
                                 : (const float*)x.data;
     const int lda = x.is_bf16 ? K : x.ld;
     float* o = (float*)c.a->take(out_bf16 ? R_BLOCK : region, (size_t)M * N * 4);
     LAUNCH(c, k.gemm_f32(xf, (const float*)lin.w, lin.bias, o, M, N, K, M > 1 ? lda : K, N,
                          c.stream));
-    out.kind = C_DELTA;
+    out.kind = KAPPAI_CARRY_DELTA;
     if (out_bf16) {
       out.data = c.a->take(region, (size_t)M * N * 2);
       LAUNCH(c, k.cast(o, out.data, (long)M * N, 0, 1, c.stream));
@@ -299,21 +297,21 @@ Carry linear(Ctx& c, Rows x, const kappai_linear& lin, int out_bf16, bool partia
       c.status = (int)hipErrorInvalidValue;
       return out;
     }
-    out.kind = C_DELTA;
+    out.kind = KAPPAI_CARRY_DELTA;
     out.is_f32 = out_bf16 ? 0 : 1;
     out.data = c.a->take(region, (size_t)M * N * elem(out_bf16));
     LAUNCH(c, k.gemm_bf16_any(xb, lin.w, lin.bias, out.data, M, N, K, lda, N, out_bf16 ? 0 : 1,
                               c.stream));
     return out;
   }
-  if (into != nullptr && M <= c.m->fused_max_rows) {
+  if (into != nullptr && M <= tune.fused_max_rows) {
     // the result joins the residual stream inside the kernel
-    const kappai_norm* norm = into->norm;
+    const kappai_fold* norm = into->norm;
     void* rows = nullptr;
     float* ss = nullptr;
     int fragment = 0;
     if (norm != nullptr) {
-      fragment = (M >= c.m->fragment_rows_from && fragment_fits(c, M, N)) ? 1 : 0;
+      fragment = (M >= tune.fragment_rows_from && fragment_fits(c, M, N)) ? 1 : 0;
       rows = c.a->take(region, (size_t)(fragment ? 16 : M) * N * 2);
       ss = (float*)c.a->take(region, (size_t)((N + 7) / 8) * 16 * 4);
     }
@@ -321,8 +319,8 @@ Carry linear(Ctx& c, Rows x, const kappai_linear& lin, int out_bf16, bool partia
                           x.frag, scaled ? x.ss : nullptr, scaled ? x.ss_parts : 0,
                           scaled ? x.eps : 0.f, into->resid, N, norm ? norm->w : nullptr, rows,
                           fragment, ss, c.stream));
-    if (norm == nullptr) return out;             // C_NOTHING
-    out.kind = C_SCALED;
+    if (norm == nullptr) return out;             // nothing left to add
+    out.kind = KAPPAI_CARRY_SCALED;
     out.scaled.data = rows;
     out.scaled.is_bf16 = 1;
     out.scaled.M = M;
@@ -337,12 +335,12 @@ Carry linear(Ctx& c, Rows x, const kappai_linear& lin, int out_bf16, bool partia
   }
   const int ksplit = (partial_sums && !scaled) ? split_k_for(M, N, K) : 1;
   if (ksplit > 1) {
-    out.kind = C_PARTS;
+    out.kind = KAPPAI_CARRY_PARTS;
     out.is_f32 = 1;
     out.parts = ksplit;
     out.data = c.a->take(region, (size_t)ksplit * M * N * 4);
   } else {
-    out.kind = C_DELTA;
+    out.kind = KAPPAI_CARRY_DELTA;
     out.is_f32 = out_bf16 ? 0 : 1;
     out.data = c.a->take(region, (size_t)M * N * elem(out_bf16));
   }
@@ -353,320 +351,138 @@ Carry linear(Ctx& c, Rows x, const kappai_linear& lin, int out_bf16, bool partia
   return out;
 }
 
-// Scaled rows or rows in fragment order that a kernel cannot take are made by the norm's own
-// kernel from the residual stream instead (ops.ScaledRows.materialize).
-Rows plain_rows(Ctx& c, const Rows& x, float* resid) {
-  if (x.ss == nullptr && !x.frag) return x;
-  Carry none;
-  return norm_kernel(c, *x.norm, resid, none, x.M, nullptr, 0, false);
+// ---- the same, as runners call it -------------------------------------------------------------
+const kappai_model* api_model(kappai_step* s) { return of(s).m; }
+const kappai_batch* api_batch(kappai_step* s) { return of(s).b; }
+hipStream_t api_stream(kappai_step* s) { return of(s).stream; }
+int api_dry(kappai_step* s) { return of(s).dry ? 1 : 0; }
+int api_ok(kappai_step* s) { return of(s).ok() ? 1 : 0; }
+void* api_take(kappai_step* s, int region, size_t bytes) {
+  if (region < 0 || region >= N_REGIONS) {
+    refuse(of(s), "a part asked for memory from a region of the workspace that does not exist");
+    return nullptr;
+  }
+  return of(s).a->take(region, bytes);
+}
+// The region for what a part hands to the norm after it.  What the region held is two parts old
+// by now and has been consumed (the part's own input lies in the other region).
+int api_carry_region(kappai_step* s) {
+  Step& c = of(s);
+  const int r = (c.carry_turn++ & 1) ? R_CARRY_B : R_CARRY_A;
+  c.a->reset(r);
+  return r;
+}
+void api_launched(kappai_step* s, int status) {
+  if (status != 0 && of(s).status == 0) of(s).status = status;
+}
+void api_fail(kappai_step* s, const char* message) { refuse(of(s), message); }
+kappai_carry api_linear(kappai_step* s, kappai_rows x, const kappai_linear* lin, int out_bf16,
+                        int partial_sums, const kappai_into* into, int region) {
+  return linear(of(s), x, *lin, out_bf16, partial_sums != 0, into, region);
+}
+kappai_rows api_plain_rows(kappai_step* s, kappai_rows x, float* resid) {
+  return plain_rows(of(s), x, resid);
+}
+kappai_carry api_plain_carry(kappai_step* s, kappai_carry carry, float* resid, int M) {
+  return plain_carry(of(s), carry, resid, M);
+}
+void* api_cast(kappai_step* s, const void* x, size_t n, int from_bf16, int to_bf16) {
+  return cast_to(of(s), x, n, from_bf16, to_bf16);
+}
+kappai_rows api_rms_norm(kappai_step* s, const kappai_fold* norm, float* resid, kappai_carry carry,
+                         int M, const int* rows, int n_rows, int fragment) {
+  return rms_norm(of(s), norm, resid, carry, M, rows, n_rows, fragment);
 }
 
-Rows as_rows(const Carry& y, int M, int D, int is_bf16) {
-  Rows r;
-  r.data = y.data;
-  r.is_bf16 = is_bf16;
-  r.M = M;
-  r.D = D;
-  r.ld = D;
+const kappai_step_api g_api = {api_model,      api_batch,       api_stream,    api_dry,
+                               api_ok,         api_take,        api_carry_region, api_launched,
+                               api_fail,       api_linear,      api_plain_rows, api_plain_carry,
+                               api_cast,       takes_kernel_order, api_rms_norm};
+
+// ---------------------------------------------------------------------------------------------
+// the registry of runners
+// ---------------------------------------------------------------------------------------------
+struct Runner {
+  std::string name;
+  int kind;
+  void* fn;
+  int desc_bytes;
+};
+std::mutex& registry_lock() {
+  static std::mutex m;
+  return m;
+}
+std::vector<Runner>& registry() {
+  static std::vector<Runner> r;
   return r;
 }
 
 // ---------------------------------------------------------------------------------------------
-// the parts
+// the walk
 // ---------------------------------------------------------------------------------------------
-// When in_proj and qkv hand their consumer partial sums over K ranges (tuning.takes_partial_sums)
-bool takes_partial_sums(const Ctx& c, int M) {
-  return M > c.m->partial_sums_min_rows &&
-         (M <= c.m->partial_sums_max_rows || c.b->max_segment_rows == 1);
-}
-
-// parts/shortconv.py
-Carry conv_mixer(Ctx& c, const kappai_layer_call& L, Rows x, float* resid, const Into& into) {
-  const kappai_kernels& k = *c.m->kernels;
-  const kappai_batch& b = *c.b;
-  const int M = x.M, D = c.m->width, taps = L.taps_per_channel;
-  const Region region = c.next_carry_region();
-  const bool wide_enough = D >= c.m->fused_step_min_width ||
-                           (D >= c.m->fused_step_narrow_width && M <= c.m->fused_step_narrow_rows);
-  Carry none;
-  if (b.max_segment_rows == 1 && M <= 64 && x.is_bf16 && !L.in_proj.w_is_f32 && D % 16 == 0 &&
-      wide_enough) {
-    // decode: projection, convolution and state shift in one kernel
-    if (!(takes_kernel_order(L.in_proj, D))) x = plain_rows(c, x, resid);
-    const int c_frag = (M >= c.m->fragment_rows_from && M <= c.m->fused_max_rows && D % 32 == 0 &&
-                        takes_kernel_order(L.out_proj, D));
-    void* y = c.a->take(R_BLOCK, (size_t)(c_frag ? 16 : M) * D * 2);
-    LAUNCH(c, k.gemm_bf16_shortconv_step(x.data, L.in_proj.w, L.in_proj.w_frag, L.in_proj.bias, y,
-                                         M, D, D, M > 1 ? x.ld : D, L.taps, L.conv_bias, L.state,
-                                         b.seg_pos0, b.seg_slot, taps, x.frag, x.ss, x.ss_parts,
-                                         x.eps, c_frag, c.stream));
-    Rows yr = as_rows(Carry{C_DELTA, y}, M, D, 1);
-    yr.frag = c_frag;
-    return linear(c, yr, L.out_proj, c.m->compute_bf16, true, &into, region);
-  }
-  // more than 16 rows (decode at any batch size, short prompt portions): the projection may come
-  // as sums over ranges of its input dimension, which the conv kernel adds up
-  const bool parts = takes_partial_sums(c, M);
-  Carry proj = linear(c, x, L.in_proj, c.m->compute_bf16, parts, nullptr, R_BLOCK);
-  if (!c.ok() && !c.dry) return none;
-  void* y;
-  int y_bf16;
-  if (proj.kind == C_PARTS) {
-    y_bf16 = 1;
-    y = c.a->take(R_BLOCK, (size_t)M * D * 2);
-    LAUNCH(c, k.shortconv_parts((const float*)proj.data, proj.parts, L.taps, L.conv_bias, L.state,
-                                y, b.row_seg, b.seg_start, b.seg_pos0, b.seg_slot, M, b.n_segments,
-                                D, taps, c.stream));
-  } else {
-    y_bf16 = proj.is_f32 ? 0 : 1;
-    y = c.a->take(R_BLOCK, (size_t)M * D * elem(y_bf16));
-    LAUNCH(c, k.shortconv(proj.data, L.taps, L.conv_bias, L.state, y, b.row_seg, b.seg_start,
-                          b.seg_pos0, b.seg_slot, M, b.n_segments, D, taps, y_bf16, c.stream));
-  }
-  return linear(c, as_rows(Carry{C_DELTA, y}, M, D, y_bf16), L.out_proj, c.m->compute_bf16, true,
-                &into, region);
-}
-
-// ops.decode_form: few keys go to the kernel that splits them over the waves of a block
-int decode_keys(const Ctx& c, const kappai_layer_call& L) {
-  int n_keys = c.b->max_position + 1;
-  if (L.window) n_keys = (n_keys < L.window ? n_keys : L.window) + 32;
-  return n_keys;
-}
-bool decode_block_form(const Ctx& c, const kappai_layer_call& L, int rep) {
-  return L.mfma->decode_block_waves(rep) > 0 && decode_keys(c, L) <= c.m->decode_block_max_keys;
-}
-
-// how the split decode kernel cuts n_keys keys of `rows` rows (ops._decode_split)
-void decode_splits(const Ctx& c, const kappai_layer_call& L, int rows, int G, int n_keys,
-                   int* keys_per_split, int* n_splits) {
-  const int kpw = L.mfma->keys_per_wave();
-  int s = c.m->decode_max_splits;
-  if ((n_keys + kpw - 1) / kpw < s) s = (n_keys + kpw - 1) / kpw;
-  int by_waves = c.m->decode_waves / (rows * G);
-  if (by_waves < 1) by_waves = 1;
-  if (by_waves < s) s = by_waves;
-  if (s < 1) s = 1;
-  *keys_per_split = ((n_keys + s - 1) / s + kpw - 1) / kpw * kpw;
-  *n_splits = (n_keys + *keys_per_split - 1) / *keys_per_split;
-}
-
-// parts/attention.py with ops.qk_norm_rope_store and ops.paged_attention
-Carry attention_mixer(Ctx& c, const kappai_layer_call& L, Rows x, float* resid, const Into& into) {
-  const kappai_kernels& k = *c.m->kernels;
-  const kappai_batch& b = *c.b;
-  const int M = x.M, H = L.heads, G = L.kv_heads, d = L.head_dim, ps = c.m->page_size;
-  const Region region = c.next_carry_region();
-  Carry none;
-  kappai_linear qkv = L.qkv;
-  if (L.shared_cache) {          // the q rows of the stacked matrix, whole pieces of 16 rows
-    qkv.n = H * d;
-    if (qkv.w_frag != nullptr && (H * d) % 16) qkv.w_frag = nullptr;
-  }
-  if (!takes_kernel_order(qkv, x.D)) x = plain_rows(c, x, resid);
-  const bool parts = takes_partial_sums(c, M);
-  Carry proj = linear(c, x, qkv, c.m->compute_bf16, parts, nullptr, R_BLOCK);
-  if (!c.ok() && !c.dry) return none;
-  if (L.rot_mode != 0 && b.max_position >= L.rot_positions) {
-    snprintf(g_error, sizeof g_error, "kappai_forward: position %d is beyond the rotation table of "
-                                      "%d positions", b.max_position, L.rot_positions);
-    c.status = (int)hipErrorInvalidValue;
-    return none;
-  }
-  if (L.group < 0 || L.group >= b.n_groups) {
-    c.status = (int)hipErrorInvalidValue;
-    snprintf(g_error, sizeof g_error, "kappai_forward: the batch has no block tables of group %d",
-             L.group);
-    return none;
-  }
-  const int* tables = b.block_tables[L.group];
-  const int max_blocks = b.max_blocks[L.group];
-  const int store = L.shared_cache ? 0 : 1;
-  const bool single = b.max_segment_rows == 1;
-  // decode: the attention kernels take the projection as it is and do norm, rotation and store
-  // themselves (parts/attention.py: _prologue_in_kernel)
-  const bool qk_in_kernel =
-      M <= c.m->fused_qk && single && proj.kind == C_DELTA && !proj.is_f32 && L.mfma != nullptr &&
-      H / G <= 16 && qkv.n % 8 == 0 && aligned16(proj.data) && ps % 16 == 0 && d % 16 == 0 &&
-      d <= 256 && (L.rot_mode == 0 || (L.rot_mode == 1 && L.rot_dim == d)) &&
-      L.mfma->decode_takes_qk != nullptr && L.mfma->decode_takes_qk() &&
-      !decode_block_form(c, L, H / G);
-  // q in place in the projection, or (from partial sums) a new bfloat16 [M, H d]
-  void* q;
-  int q_stride, q_bf16;
-  if (qk_in_kernel) {
-    q_bf16 = 1;
-    q_stride = qkv.n;
-    q = proj.data;
-  } else if (proj.kind == C_PARTS) {
-    q_bf16 = 1;
-    q_stride = H * d;
-    q = c.a->take(R_BLOCK, (size_t)M * H * d * 2);
-    LAUNCH(c, k.qk_norm_rope_store(nullptr, qkv.n, L.q_norm_w, L.k_norm_w, L.qk_eps, L.cos_table,
-                                   L.sin_table, L.rot_mode ? L.rot_dim : 0, L.rot_mode, L.k_pool,
-                                   L.v_pool, b.row_pos, b.row_seg, store ? tables : nullptr,
-                                   store ? max_blocks : 0, M, H, G, d, ps, store, 1,
-                                   (const float*)proj.data, proj.parts, q, H * d, c.stream));
-  } else {
-    q_bf16 = proj.is_f32 ? 0 : 1;
-    q_stride = qkv.n;
-    q = proj.data;
-    LAUNCH(c, k.qk_norm_rope_store(q, q_stride, L.q_norm_w, L.k_norm_w, L.qk_eps, L.cos_table,
-                                   L.sin_table, L.rot_mode ? L.rot_dim : 0, L.rot_mode, L.k_pool,
-                                   L.v_pool, b.row_pos, b.row_seg, store ? tables : nullptr,
-                                   store ? max_blocks : 0, M, H, G, d, ps, store, q_bf16, nullptr,
-                                   0, nullptr, H * d, c.stream));
-  }
-  void* ctx = c.a->take(R_BLOCK, (size_t)M * H * d * elem(q_bf16));
-  const float* cos_t = L.rot_mode ? L.cos_table : nullptr;
-  const float* sin_t = L.rot_mode ? L.sin_table : nullptr;
-  const bool mfma_ok = q_bf16 && L.mfma != nullptr && ps % 16 == 0 && d % 16 == 0 && d <= 256 &&
-                       q_stride % 8 == 0 && aligned16(q);
-  if (mfma_ok && single && H / G <= 16) {
-    const int n_keys = decode_keys(c, L);
-    const int block_waves = L.mfma->decode_block_waves(H / G);
-    if (decode_block_form(c, L, H / G)) {
-      LAUNCH(c, L.mfma->attn_decode_block(q, q_stride, L.k_pool, L.v_pool, ctx, H * d, b.row_pos,
-                                          b.row_seg, tables, max_blocks, M, H, G, ps, L.window,
-                                          L.scale, block_waves, c.stream));
-    } else {
-      int keys_per_split, n_splits;
-      decode_splits(c, L, M, G, n_keys, &keys_per_split, &n_splits);
-      float* part_o = (float*)c.a->take(R_BLOCK, (size_t)M * H * n_splits * d * 4);
-      float* part_ml = (float*)c.a->take(R_BLOCK, (size_t)M * H * n_splits * 2 * 4);
-      if (qk_in_kernel)
-        LAUNCH(c, L.mfma->attn_decode_qk(q, q_stride, L.k_pool, L.v_pool, ctx, H * d, part_o,
-                                         part_ml, b.row_pos, b.row_seg, tables, max_blocks, M, H,
-                                         G, ps, L.window, L.scale, keys_per_split, n_splits,
-                                         L.q_norm_w, L.k_norm_w, L.qk_eps, cos_t, sin_t, store,
-                                         c.stream));
-      else
-        LAUNCH(c, L.mfma->attn_decode(q, q_stride, L.k_pool, L.v_pool, ctx, H * d, part_o, part_ml,
-                                      b.row_pos, b.row_seg, tables, max_blocks, M, H, G, ps,
-                                      L.window, L.scale, keys_per_split, n_splits, c.stream));
-    }
-  } else if (mfma_ok && b.q_tiles != nullptr) {
-    LAUNCH(c, L.mfma->attn_prefill(q, q_stride, L.k_pool, L.v_pool, ctx, H * d, b.q_tiles,
-                                   b.n_tiles, b.row_pos, tables, max_blocks, H, G, ps, L.window,
-                                   L.scale, 0, c.stream));
-    if (b.lone_rows != nullptr && b.n_lone_rows > 0) {
-      // the single decoded tokens beside the portions: keys split over blocks (ops._decode_split)
-      if (H / G > 16 || b.max_lone_position < 0) {
-        snprintf(g_error, sizeof g_error, "kappai_forward: rows left out of the tiles need the "
-                                          "decode kernel and their largest position");
-        c.status = (int)hipErrorInvalidValue;
-        return none;
-      }
-      const int R = b.n_lone_rows;
-      int n_keys = b.max_lone_position + 1;
-      if (L.window) n_keys = (n_keys < L.window ? n_keys : L.window) + 32;
-      int keys_per_split, n_splits;
-      decode_splits(c, L, R, G, n_keys, &keys_per_split, &n_splits);
-      float* part_o = (float*)c.a->take(R_BLOCK, (size_t)R * H * n_splits * d * 4);
-      float* part_ml = (float*)c.a->take(R_BLOCK, (size_t)R * H * n_splits * 2 * 4);
-      LAUNCH(c, L.mfma->attn_decode_rows(q, q_stride, L.k_pool, L.v_pool, ctx, H * d, part_o,
-                                         part_ml, b.lone_rows, b.row_pos, b.row_seg, tables,
-                                         max_blocks, R, H, G, ps, L.window, L.scale,
-                                         keys_per_split, n_splits, c.stream));
-    }
-  } else {
-    LAUNCH(c, k.paged_attention_rows(q, q_stride, L.k_pool, L.v_pool, ctx, H * d, b.row_pos,
-                                     b.row_seg, tables, max_blocks, M, H, G, d, ps, L.window,
-                                     L.scale, q_bf16, c.stream));
-  }
-  return linear(c, as_rows(Carry{C_DELTA, ctx}, M, H * d, q_bf16), L.attn_out, c.m->compute_bf16,
-                true, &into, region);
-}
-
-// parts/feed_forward.py
-Carry swiglu_ffn(Ctx& c, const kappai_layer_call& L, Rows x, float* resid, const Into& into) {
-  const kappai_kernels& k = *c.m->kernels;
-  const int M = x.M, D = c.m->width, F = L.hidden;
-  const Region region = c.next_carry_region();
-  Carry none;
-  if (L.ffn_fused && x.is_bf16) {
-    if (!takes_kernel_order(L.gate_up, D)) x = plain_rows(c, x, resid);
-    const int c_frag = (M >= c.m->fragment_rows_from && M <= c.m->fused_max_rows && F % 32 == 0 &&
-                        takes_kernel_order(L.down, F));
-    void* act = c.a->take(R_BLOCK, (size_t)(c_frag ? 16 : M) * F * 2);
-    LAUNCH(c, k.gemm_bf16_swiglu(x.data, L.gate_up.w, L.gate_up.w_frag, act, M, F, D,
-                                 M > 1 ? x.ld : D, F, 0, x.frag, x.ss, x.ss_parts, x.eps, c_frag,
-                                 c.stream));
-    Rows ar = as_rows(Carry{C_DELTA, act}, M, F, 1);
-    ar.frag = c_frag;
-    return linear(c, ar, L.down, c.m->compute_bf16, true, &into, region);
-  }
-  Carry gu = linear(c, x, L.gate_up, c.m->compute_bf16, false, nullptr, R_BLOCK);
-  if (!c.ok() && !c.dry) return none;
-  const int act_bf16 = gu.is_f32 ? 0 : 1;
-  void* act = c.a->take(R_BLOCK, (size_t)M * F * elem(act_bf16));
-  LAUNCH(c, k.swiglu(gu.data, act, M, F, act_bf16, c.stream));
-  return linear(c, as_rows(Carry{C_DELTA, act}, M, F, act_bf16), L.down, c.m->compute_bf16, true,
-                &into, region);
-}
-
 bool model_ok(const kappai_model* m) {
   if (m == nullptr || m->abi != KAPPAI_ENGINE_ABI || m->kernels == nullptr || m->n_calls < 0 ||
-      m->width < 1 || m->vocab < 1 || (m->n_calls > 0 && m->calls == nullptr)) {
+      m->width < 1 || m->vocab < 1 || (m->n_calls > 0 && m->calls == nullptr) ||
+      m->final_norm.run == nullptr) {
     snprintf(g_error, sizeof g_error, "kappai_forward: the model description is incomplete or was "
                                       "filled in for another version of this library");
     return false;
   }
+  for (int ci = 0; ci < m->n_calls; ++ci)
+    if (m->calls[ci].run == nullptr) {
+      snprintf(g_error, sizeof g_error, "kappai_forward: call %d of the schedule names no runner",
+               ci);
+      return false;
+    }
   return true;
 }
 
 int run(const kappai_model* m, const kappai_batch* b, Arena& arena, float* logits,
         hipStream_t stream, bool dry) {
-  Ctx c{m, b, &arena, stream, dry};
+  Step c;
+  c.api = &g_api;
+  c.m = m;
+  c.b = b;
+  c.a = &arena;
+  c.stream = stream;
+  c.dry = dry;
   const kappai_kernels& k = *m->kernels;
   const int T = b->n_rows, D = m->width;
   float* resid = (float*)arena.take(R_STEP, (size_t)T * D * 4);
-  // the embedding and the first call's norm are one kernel where the norm's row kernel takes
-  // the width (the same arithmetic as the two kernels, bit for bit)
-  const bool embed_with_norm = m->n_calls > 0 && D % 8 == 0 && D <= 8192 &&
-                               (m->embed_is_bf16 != 2 || D % 32 == 0) &&
-                               aligned16(m->embed_table) && aligned16(m->calls[0].mixer_norm.w);
-  if (!embed_with_norm)
-    LAUNCH(c, k.embed_rows(b->tokens, m->embed_table, m->embed_is_bf16, resid, T, D, stream));
-  Carry carry;
+  // The head as the part that takes the final norm's rows.
+  kappai_part head_part = {};
+  head_part.flags = KAPPAI_TAKES_DEFERRED_ROWS;
+  head_part.first = &m->head;
+  // After the last call comes the final norm, whose rows the head takes; a block can make them
+  // only when every row wants its logits, in the rows' order, and the head reads such rows.
+  const bool every_row = b->logits_of_every_row && b->n_logit_rows == T &&
+                         takes_kernel_order(&m->head, D);
+  // the embedding is looked up by the first norm that runs (which may do both in one kernel)
+  kappai_carry carry = {};
+  carry.kind = KAPPAI_CARRY_EMBEDDING;
   for (int ci = 0; ci < m->n_calls && c.ok(); ++ci) {
-    const kappai_layer_call& L = m->calls[ci];
-    const kappai_layer_call* next = ci + 1 < m->n_calls ? &m->calls[ci + 1] : nullptr;
+    const kappai_call& call = m->calls[ci];
+    const kappai_call* next = ci + 1 < m->n_calls ? &m->calls[ci + 1] : nullptr;
     arena.reset(R_BLOCK);
-    const bool conv = L.mixer == KAPPAI_MIXER_CONV;
-    const kappai_linear& first = conv ? L.in_proj : L.qkv;
-    Rows x = (ci == 0 && embed_with_norm) ? embedded_and_normed(c, L.mixer_norm, resid, T, first)
-                                          : normed(c, L.mixer_norm, resid, carry, T, first);
-    const Into into_ffn{resid, &L.ffn_norm};
-    const Carry mixed = conv ? conv_mixer(c, L, x, resid, into_ffn)
-                             : attention_mixer(c, L, x, resid, into_ffn);
-    if (!c.ok()) break;
-    Rows x2 = normed(c, L.ffn_norm, resid, mixed, T, L.gate_up);
-    // the norm after the last call is the final one; the head can take rows made for it when
-    // every row of the step wants its logits, in the rows' order
-    const kappai_norm* after = next ? &next->mixer_norm
-                               : (b->logits_of_every_row && b->n_logit_rows == T &&
-                                  takes_kernel_order(m->head, D)) ? &m->final_norm : nullptr;
-    const Into into_next{resid, after};
-    carry = swiglu_ffn(c, L, x2, resid, into_next);
+    const kappai_norm_part* after_norm = next ? next->first_norm
+                                              : (every_row ? &m->final_norm : nullptr);
+    const kappai_part* after_consumer = next ? next->first_consumer
+                                             : (every_row ? &head_part : nullptr);
+    carry = call.run(&c, call.desc, resid, carry, after_norm, after_consumer);
   }
   if (c.ok() && b->n_logit_rows > 0) {
     arena.reset(R_BLOCK);
     const int n = b->n_logit_rows;
-    Rows xb;
-    if (carry.kind == C_SCALED && carry.scaled.norm == &m->final_norm) {
-      xb = carry.scaled;               // the last product made the rows, the head divides by rms
-    } else {
-      Carry for_norm = carry;
-      if (carry.kind == C_SCALED) for_norm = Carry();      // made for no norm that runs here
-      const bool fragment = n >= m->fragment_rows_min && fragment_fits(c, n, D) &&
-                            (for_norm.kind != C_PARTS || for_norm.parts <= 8) &&
-                            takes_kernel_order(m->head, D);
-      xb = norm_kernel(c, m->final_norm, resid, for_norm, T, b->logit_rows, n, fragment);
-    }
+    // rows made for the final norm by the last product stand for all rows in order
+    const bool made = carry.kind == KAPPAI_CARRY_SCALED && every_row;
+    kappai_rows xb = m->final_norm.run(&c, m->final_norm.desc, resid, carry, T,
+                                       made ? nullptr : b->logit_rows, made ? 0 : n, &head_part);
+    if (c.ok() && (xb.M != n || xb.D != D)) refuse(c, "the final norm returned rows of another shape");
     // the head: a plain product with float results, straight into the caller's tensor
     const kappai_linear& head = m->head;
-    if (head.w_is_f32) {
+    if (!c.ok()) {
+    } else if (head.w_is_f32) {
+      xb = plain_rows(c, xb, resid);
       const float* xf = xb.is_bf16 ? (const float*)cast_to(c, xb.data, (size_t)n * D, 1, 0)
                                    : (const float*)xb.data;
       LAUNCH(c, k.gemm_f32(xf, (const float*)head.w, head.bias, logits, n, head.n, D, D, head.n,
@@ -679,7 +495,7 @@ int run(const kappai_model* m, const kappai_batch* b, Arena& arena, float* logit
                               1, 0, 1, xb.frag, xb.ss, xb.ss ? xb.ss_parts : 0,
                               xb.ss ? xb.eps : 0.f, nullptr, 0, nullptr, nullptr, 0, nullptr,
                               stream));
-      else if (head.w != nullptr)
+      else if (head.w != nullptr && !xb.frag && xb.ss == nullptr)
         LAUNCH(c, k.gemm_bf16_any(xh, head.w, head.bias, logits, n, head.n, D, D, head.n, 1,
                                   stream));
       else
@@ -694,39 +510,79 @@ int run(const kappai_model* m, const kappai_batch* b, Arena& arena, float* logit
   return c.status;
 }
 
-bool batch_ok(const kappai_model* m, const kappai_batch* b) {
+bool batch_ok(const kappai_batch* b) {
   if (b == nullptr || b->n_rows < 1 || b->n_segments < 1 || b->n_logit_rows < 0 ||
       b->n_groups < 0 || b->n_groups > KAPPAI_MAX_GROUPS) {
     snprintf(g_error, sizeof g_error, "kappai_forward: a step needs rows and segments");
     return false;
   }
-  (void)m;
   return true;
 }
 
 }  // namespace
 
+extern "C" int kappai_register_runner(const char* name, int kind, void* fn, int desc_bytes) {
+  if (name == nullptr || fn == nullptr || kind < KAPPAI_RUNNER_PART || kind > KAPPAI_RUNNER_BLOCK ||
+      desc_bytes < 0) {
+    snprintf(g_error, sizeof g_error, "kappai_register_runner: a runner needs a name, a kind and "
+                                      "a function");
+    return (int)hipErrorInvalidValue;
+  }
+  std::lock_guard<std::mutex> hold(registry_lock());
+  for (const Runner& r : registry())
+    if (r.name == name && r.kind == kind) {
+      if (r.fn == fn && r.desc_bytes == desc_bytes) return 0;
+      snprintf(g_error, sizeof g_error, "kappai_register_runner: '%s' is registered already, with "
+                                        "another function or description", name);
+      return (int)hipErrorInvalidValue;
+    }
+  registry().push_back(Runner{name, kind, fn, desc_bytes});
+  return 0;
+}
+
+extern "C" void* kappai_runner(const char* name, int kind, int* desc_bytes) {
+  if (name == nullptr) return nullptr;
+  std::lock_guard<std::mutex> hold(registry_lock());
+  for (const Runner& r : registry())
+    if (r.name == name && r.kind == kind) {
+      if (desc_bytes != nullptr) *desc_bytes = r.desc_bytes;
+      return r.fn;
+    }
+  return nullptr;
+}
+
 extern "C" int kappai_engine_layout(int* sizes, int n) {
-  const int mine[8] = {KAPPAI_ENGINE_ABI,
-                       (int)sizeof(kappai_kernels),
-                       (int)sizeof(kappai_attention_kernels),
-                       (int)sizeof(kappai_linear),
-                       (int)sizeof(kappai_norm),
-                       (int)sizeof(kappai_layer_call),
-                       (int)sizeof(kappai_model),
-                       (int)sizeof(kappai_batch)};
-  for (int i = 0; i < n && i < 8; ++i) sizes[i] = mine[i];
-  return 8;
+  const int mine[] = {KAPPAI_ENGINE_ABI,
+                      (int)sizeof(kappai_kernels),
+                      (int)sizeof(kappai_attention_kernels),
+                      (int)sizeof(kappai_linear),
+                      (int)sizeof(kappai_fold),
+                      (int)sizeof(kappai_rows),
+                      (int)sizeof(kappai_carry),
+                      (int)sizeof(kappai_part),
+                      (int)sizeof(kappai_norm_part),
+                      (int)sizeof(kappai_call),
+                      (int)sizeof(kappai_tuning),
+                      (int)sizeof(kappai_model),
+                      (int)sizeof(kappai_batch)};
+  const int count = (int)(sizeof mine / sizeof mine[0]);
+  for (int i = 0; i < n && i < count; ++i) sizes[i] = mine[i];
+  return count;
 }
 
 extern "C" const char* kappai_forward_error(void) { return g_error; }
 
 extern "C" int kappai_split_k_for(int M, int N, int K) { return split_k_for(M, N, K); }
 
+extern "C" void kappai_decode_splits(int keys_per_wave, int max_splits, int waves, int rows, int G,
+                                     int n_keys, int* keys_per_split, int* n_splits) {
+  decode_splits(keys_per_wave, max_splits, waves, rows, G, n_keys, keys_per_split, n_splits);
+}
+
 extern "C" size_t kappai_forward_workspace_bytes(const kappai_model* model,
                                                  const kappai_batch* batch) {
   g_error[0] = 0;
-  if (!model_ok(model) || !batch_ok(model, batch)) return 0;
+  if (!model_ok(model) || !batch_ok(batch)) return 0;
   Arena arena;
   if (run(model, batch, arena, nullptr, nullptr, true) != 0) return 0;
   size_t total = 0;
@@ -738,7 +594,7 @@ extern "C" int kappai_forward(const kappai_model* model, const kappai_batch* bat
                               void* workspace, size_t workspace_bytes, float* logits,
                               hipStream_t stream) {
   g_error[0] = 0;
-  if (!model_ok(model) || !batch_ok(model, batch)) return (int)hipErrorInvalidValue;
+  if (!model_ok(model) || !batch_ok(batch)) return (int)hipErrorInvalidValue;
   if (workspace == nullptr || (batch->n_logit_rows > 0 && logits == nullptr)) {
     snprintf(g_error, sizeof g_error, "kappai_forward: no workspace or no place for the logits");
     return (int)hipErrorInvalidValue;

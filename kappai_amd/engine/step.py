@@ -19,7 +19,7 @@ from ..cache.manager import CacheManager, OutOfPages, RequestCache
 from ..kernels import ops, profile
 from ..models.base import Model
 from .batch import RowBatch, StepEntry, layout_rows
-from .cforward import CForward, Workspace
+from .cforward import CForward, NotDescribed, Workspace
 
 
 CONTEXT_BUCKET_MIN = 1024     # decode graphs are captured for contexts up to a power of two
@@ -190,8 +190,9 @@ class _DecodeGraph:
 class StepRunner:
     def __init__(self, model: Model, cache: CacheManager, device="cuda:0",
                  decode_graphs: bool = True, c_forward: bool = True):
-        """``c_forward``: run steps through the C side (``kappai_forward``) when the model is made
-        of parts it knows; False runs every step from the parts' own ``forward`` methods."""
+        """``c_forward``: run steps through the C side (``kappai_forward``) when every part of the
+        model describes itself for it; False runs every step from the parts' own ``forward``
+        methods."""
         self.model, self.cache = model, cache
         self.device = torch.device(device)
         self.c_forward = c_forward and self.device.type == "cuda"
@@ -215,7 +216,10 @@ class StepRunner:
         if self.c_forward and not self._cplan_tried:
             self._cplan_tried = True
             if CForward.plannable(self.model):
-                self._cplan = CForward(self.model, self.cache, self.device)
+                try:
+                    self._cplan = CForward(self.model, self.cache, self.device)
+                except NotDescribed:       # a part without a description for the C side
+                    self._cplan = None
         if self._cplan is not None and not profile.STAGE_TIMES.enabled:
             return self._cplan.forward(batch, workspace)
         return self.model.forward(batch, self.cache)

@@ -18,7 +18,7 @@ import tempfile
 import threading
 import time
 from pathlib import Path
-from typing import Dict, List
+from typing import Dict, List, Optional
 
 CSRC = Path(__file__).resolve().parent.parent / "csrc"
 GPU_ARCH = "gfx950"
@@ -27,6 +27,8 @@ HIPCC_FLAGS = ["-O3", "-std=c++17", f"--offload-arch={GPU_ARCH}", "-shared", "-f
                "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
                "-Wno-unused-command-line-argument", "-Wno-pass-failed"]
 LIBRARIES = ["elementwise", "gemm", "shortconv", "attention", "sampling", "engine"]
+# libraries made of more sources than the one of their own name
+EXTRA_SOURCES = {"engine": ["engine_parts"]}
 # libraries compiled once per value of a constant: name -> (constant, values built ahead)
 VARIANT_LIBRARIES = {"attention_mfma": ("HEAD_DIM", [16, 32, 48, 64, 80, 128, 256])}
 
@@ -59,9 +61,13 @@ def _built_name(name: str, defines) -> str:
     return name + "".join(f"__{k}{v}" for k, v in sorted((defines or {}).items()))
 
 
-def _source_hash(name: str, defines=None) -> str:
+def _sources(name: str) -> List[Path]:
+    return [CSRC / f"{n}.hip" for n in [name] + EXTRA_SOURCES.get(name, [])]
+
+
+def _source_hash(name: str, defines=None, sources=None) -> str:
     h = hashlib.sha256()
-    for p in [CSRC / f"{name}.hip"] + sorted(CSRC.glob("*.h")):
+    for p in list(sources or _sources(name)) + sorted(CSRC.glob("*.h")):
         h.update(p.name.encode())
         h.update(p.read_bytes())
     h.update(" ".join(HIPCC_FLAGS + _defines_flags(defines)).encode())
@@ -136,18 +142,23 @@ def _find_built(built: str, want_hash: str):
     return None
 
 
-def compile_library(name: str, verbose: bool = True, defines=None) -> Path:
-    """Compile ``csrc/<name>.hip`` now, whether or not a built library is there."""
-    src = CSRC / f"{name}.hip"
-    if not src.is_file():
-        raise KernelBuildError(f"{src}: no such kernel source")
-    out_dir = _writable_build_dir()
+def compile_library(name: str, verbose: bool = True, defines=None, sources=None,
+                    out_dir: Optional[Path] = None) -> Path:
+    """Compile ``csrc/<name>.hip`` (with the other sources of its library) now, whether or not a
+    built library is there.  ``sources`` / ``out_dir``: a library of somebody else's
+    (``library_at``)."""
+    srcs = list(sources or _sources(name))
+    for src in srcs:
+        if not src.is_file():
+            raise KernelBuildError(f"{src}: no such kernel source")
+    out_dir = out_dir or _writable_build_dir()
     built = _built_name(name, defines)
     so, tag = out_dir / f"{built}.so", out_dir / f"{built}.hash"
     tmp = out_dir / f".{built}.{os.getpid()}.{threading.get_ident()}.so"
-    cmd = [_hipcc(), *HIPCC_FLAGS, *_defines_flags(defines), f"-I{CSRC}", str(src), "-o", str(tmp)]
-    what = src.name + (" (" + ", ".join(f"{k}={v}" for k, v in sorted(defines.items())) + ")"
-                       if defines else "")
+    cmd = [_hipcc(), *HIPCC_FLAGS, *_defines_flags(defines), f"-I{CSRC}", *map(str, srcs), "-o",
+           str(tmp)]
+    what = " + ".join(src.name for src in srcs) + (
+        " (" + ", ".join(f"{k}={v}" for k, v in sorted(defines.items())) + ")" if defines else "")
     if verbose:
         print(f"[kappai_amd] compiling {what} for {GPU_ARCH} ...", file=sys.stderr, flush=True)
     t0 = time.time()
@@ -164,7 +175,7 @@ def compile_library(name: str, verbose: bool = True, defines=None) -> Path:
         tmp.unlink(missing_ok=True)
         raise KernelBuildError(f"hipcc failed on {what}:\n{out}")
     os.replace(tmp, so)
-    tag.write_text(_source_hash(name, defines))
+    tag.write_text(_source_hash(name, defines, srcs))
     if verbose:
         print(f"[kappai_amd] built {so.name} in {time.time() - t0:.1f} s", file=sys.stderr,
               flush=True)
@@ -217,6 +228,33 @@ def library(name: str, **defines) -> ctypes.CDLL:
         except OSError as exc:
             raise KernelBuildError(f"cannot load {so}: {exc}") from exc
         _loaded[built] = lib
+        return lib
+
+
+def library_at(source, build: bool = True, force: bool = False) -> ctypes.CDLL:
+    """The library of one ``.hip`` file that lives outside this package (a part of somebody
+    else's, with its kernel and the function that runs it from C): compiled like the package's
+    own, with ``csrc`` on the include path, into ``_build`` beside the source, and loaded."""
+    src = Path(source).resolve()
+    key = f"@{src}"
+    lib = _loaded.get(key)
+    if lib is not None and not force:
+        return lib
+    with _lock:
+        out_dir = src.parent / "_build"
+        want = _source_hash(src.stem, None, [src])
+        so, tag = out_dir / f"{src.stem}.so", out_dir / f"{src.stem}.hash"
+        fresh = so.is_file() and tag.is_file() and tag.read_text().strip() == want
+        if force or not fresh:
+            if not build:
+                raise KernelBuildError(f"{so} is missing or older than its source")
+            out_dir.mkdir(parents=True, exist_ok=True)
+            compile_library(src.stem, sources=[src], out_dir=out_dir)
+        try:
+            lib = ctypes.CDLL(str(so))
+        except OSError as exc:
+            raise KernelBuildError(f"cannot load {so}: {exc}") from exc
+        _loaded[key] = lib
         return lib
 
 

@@ -966,6 +966,16 @@ def paged_attention(q: torch.Tensor, n_heads: int, n_kv_heads: int, head_dim: in
     return out
 
 
+def decode_splits(keys_per_wave: int, rows: int, n_kv_heads: int, n_keys: int):
+    """(fewest keys a split, most splits a row) of the decode kernel that splits keys over blocks:
+    the rule lives in C (``kappai_decode_splits``), where a step launched from C uses it too."""
+    kps, n = _c_int(0), _c_int(0)
+    library("engine").kappai_decode_splits(
+        _c_int(keys_per_wave), _c_int(DECODE_MAX_SPLITS), _c_int(DECODE_WAVES), _c_int(rows),
+        _c_int(n_kv_heads), _c_int(n_keys), ctypes.byref(kps), ctypes.byref(n))
+    return kps.value, n.value
+
+
 def _decode_split(lib, q, H, G, d, k_pool, v_pool, row_pos, row_seg, block_tables, page_size, scale,
                   window, max_position, out, row_ids, qk_args=()):
     """The decode kernel that splits a row's keys over blocks, and its merge, for all rows or
@@ -980,10 +990,7 @@ def _decode_split(lib, q, H, G, d, k_pool, v_pool, row_pos, row_seg, block_table
     # fewest keys a split of this step; the kernels settle on a number of keys a split from the
     # rows' own lengths (step_keys_per_split in csrc/attention_mfma.hip) and leave the rest of
     # the splits empty.
-    n_splits = max(1, min(DECODE_MAX_SPLITS, (n_keys + kpw - 1) // kpw,
-                          max(1, DECODE_WAVES // (T * G))))
-    keys_per_split = ((n_keys + n_splits - 1) // n_splits + kpw - 1) // kpw * kpw
-    n_splits = (n_keys + keys_per_split - 1) // keys_per_split
+    keys_per_split, n_splits = decode_splits(kpw, T, G, n_keys)
     part_o = torch.empty((T, H, n_splits, d), dtype=F32, device=q.device)
     part_ml = torch.empty((T, H, n_splits, 2), dtype=F32, device=q.device)
     head = (_ptr(q), _c_int(q.stride(0)), _ptr(k_pool), _ptr(v_pool), _ptr(out), _c_int(H * d),

@@ -127,6 +127,24 @@ class Model:
         the head that takes its rows."""
         return self.final_norm, self.head
 
+    def c_calls(self, plan):
+        """The schedule as the C side of a step runs it: every call's block described by itself
+        (``Block.c_call``), or None when a block has no description.  The C walk does what
+        ``forward`` below does, which is why the two are defined side by side: a subclass that
+        changes ``forward`` gets no walk from C unless it describes one."""
+        from ..parts.cdesc import defined_together
+        calls = []
+        for ci, call in enumerate(self.schedule):
+            block = self.layers[call.layer]
+            if not defined_together(block, "forward", "c_call"):
+                return None
+            view = plan.cache.view(self.cache_id(ci)) if block.cache_spec() is not None else None
+            described = block.c_call(plan, view, call.reads_cache_of is not None)
+            if described is None:
+                return None
+            calls.append(described)
+        return calls
+
     # -- the forward pass of one step ------------------------------------------------------
     def forward(self, batch, cache) -> torch.Tensor:
         """Run the rows of ``batch`` through every call of the schedule and return float32

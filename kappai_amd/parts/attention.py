@@ -18,8 +18,23 @@ import torch
 from ..cache.specs import PagedKV
 from ..kernels import ops, profile, tuning
 from ..weights.spec import INIT_ONES, VECTOR, TensorSpec
+import ctypes
+from ctypes import POINTER, Structure, c_float, c_int, c_void_p
+
 from .base import Mixer, PositionEncoding, register_part
+from .cdesc import AttentionKernels, LinearDesc, tensor_ptr
 from .linear import Linear
+
+
+class AttentionMixerDesc(Structure):
+    """``kappai_attention_mixer`` of csrc/engine_parts.h."""
+    _fields_ = [
+        ("qkv", LinearDesc), ("out", LinearDesc), ("q_norm_w", c_void_p), ("k_norm_w", c_void_p),
+        ("qk_eps", c_float), ("heads", c_int), ("kv_heads", c_int), ("head_dim", c_int),
+        ("window", c_int), ("scale", c_float), ("cos_table", c_void_p), ("sin_table", c_void_p),
+        ("rot_dim", c_int), ("rot_mode", c_int), ("rot_positions", c_int), ("k_pool", c_void_p),
+        ("v_pool", c_void_p), ("group", c_int), ("shared_cache", c_int),
+        ("mfma", POINTER(AttentionKernels))]
 
 
 class GroupedQueryAttention(Mixer):
@@ -114,6 +129,35 @@ class GroupedQueryAttention(Mixer):
                                       lone_rows=getattr(batch, "lone_rows", None),
                                       max_lone_position=getattr(batch, "max_lone_position", -1))
         return self.out.forward(ctx, partial_sums=True, add_into=into)
+
+    def c_part(self, plan, view, shared_cache: bool = False):
+        """The runner "mixer.attention" (csrc/engine_parts.hip) makes the same choices as
+        ``forward``.  The rotation tables grow with the context, so the description is brought
+        up to date before every step."""
+        first = plan.linear(self.qkv)
+        d = AttentionMixerDesc()
+        d.qkv, d.out = first, plan.linear(self.out)
+        d.q_norm_w, d.k_norm_w = tensor_ptr(self.q_norm_w), tensor_ptr(self.k_norm_w)
+        d.qk_eps = self.qk_norm_eps or 0.0
+        d.heads, d.kv_heads, d.head_dim = self.H, self.G, self.d
+        d.window, d.scale = self.window or 0, self.scale
+        d.k_pool, d.v_pool = view.pool("k").data_ptr(), view.pool("v").data_ptr()
+        d.group = view.group
+        d.shared_cache = 1 if shared_cache else 0
+        d.rot_mode = ops.ROT_NONE
+        if plan.bf16 and self.d % 16 == 0 and self.d <= 256:
+            d.mfma = ctypes.pointer(plan.attention_kernels(self.d))
+        if self.position is not None:
+            def rotation_tables(batch, d=d, position=self.position, device=plan.device):
+                rot = position.rotation(device, batch.max_position)
+                if rot is None:
+                    d.rot_mode = ops.ROT_NONE
+                    return
+                d.cos_table, d.sin_table = rot.cos.data_ptr(), rot.sin.data_ptr()
+                d.rot_dim, d.rot_mode, d.rot_positions = rot.rot_dim, rot.mode, rot.cos.shape[0]
+            plan.on_step(rotation_tables)
+        return plan.part("mixer.attention", d, takes_deferred_rows=True, adds_residual=True,
+                         first=first)
 
     def _prologue_in_kernel(self, proj, rot, single_rows: bool, page_size: int,
                             max_position: int) -> bool:

@@ -7,7 +7,16 @@ import torch
 
 from ..kernels import ops
 from ..weights.spec import TensorSpec
+from ctypes import Structure
+
 from .base import Block, FeedForward, Hidden, Mixer, Norm, register_part, summed_delta
+from .cdesc import NormPartDesc, PartDesc, defined_together
+
+
+class PreNormBlockDesc(Structure):
+    """``kappai_pre_norm_block`` of csrc/engine_parts.h."""
+    _fields_ = [("mixer_norm", NormPartDesc), ("mixer", PartDesc), ("ffn_norm", NormPartDesc),
+                ("feed_forward", PartDesc)]
 
 
 def _takes_defer(norm) -> bool:
@@ -95,6 +104,25 @@ class PreNormBlock(Block):
         if after is None:
             raise RuntimeError("a part that takes deferred rows did not use them")
         return after
+
+    def c_call(self, plan, view, shared_cache: bool = False):
+        """The block as the C side of a step runs it (runner "block.pre_norm"): the four parts'
+        own descriptions side by side, or None when one of them has none.  A part whose class
+        changed ``forward`` (or a norm's ``add_norm``) without giving a description of its own
+        counts as having none."""
+        for part, method, c_method in ((self.mixer_norm, "add_norm", "c_norm"),
+                                       (self.mixer, "forward", "c_part"),
+                                       (self.ffn_norm, "add_norm", "c_norm"),
+                                       (self.feed_forward, "forward", "c_part")):
+            if not defined_together(part, method, c_method):
+                return None
+        n1, n2 = self.mixer_norm.c_norm(plan), self.ffn_norm.c_norm(plan)
+        mixer = self.mixer.c_part(plan, view, shared_cache)
+        feed_forward = self.feed_forward.c_part(plan, None, False)
+        if n1 is None or n2 is None or mixer is None or feed_forward is None:
+            return None
+        return plan.call("block.pre_norm", PreNormBlockDesc(n1, mixer, n2, feed_forward),
+                         first_norm=n1, first_consumer=mixer)
 
     def weight_bytes(self) -> int:
         return sum(p.weight_bytes() for p in self._parts())

@@ -29,6 +29,10 @@ class TokenEmbedding(Part):
         with profile.scope("embd"):
             return ops.embed_rows(tokens, self.table)
 
+    def c_table(self):
+        """The table as the C side of a step looks rows up in it."""
+        return self.table
+
     def weight_bytes(self) -> int:
         return 0   # a step reads one row per token, not the table
 
@@ -57,6 +61,10 @@ class OutputHead(Part):
 
     def forward(self, x) -> torch.Tensor:
         return self.linear.forward(x, out_dtype=torch.float32)
+
+    def c_linear(self):
+        """The head's product as the C side of a step runs it (float32 logits)."""
+        return self.linear
 
     def weight_bytes(self) -> int:
         return self.linear.weight_bytes()

@@ -10,8 +10,17 @@ import torch
 
 from ..kernels import ops, profile
 from ..weights.spec import TensorSpec
+from ctypes import Structure, c_int
+
 from .base import FeedForward, register_part
+from .cdesc import LinearDesc
 from .linear import Linear
+
+
+class SwiGLUDesc(Structure):
+    """``kappai_swiglu`` of csrc/engine_parts.h."""
+    _fields_ = [("gate_up", LinearDesc), ("down", LinearDesc), ("hidden", c_int),
+                ("fused", c_int)]
 
 
 class SwiGLU(FeedForward):
@@ -49,6 +58,14 @@ class SwiGLU(FeedForward):
         with profile.scope("ffn_act"):
             act = ops.swiglu(gate_up)
         return self.down.forward(act, partial_sums=True, add_into=into)
+
+    def c_part(self, plan, view=None, shared_cache: bool = False):
+        """The runner "feed_forward.swiglu" (csrc/engine_parts.hip) makes the same choices as
+        ``forward``."""
+        first = plan.linear(self.gate_up)
+        desc = SwiGLUDesc(first, plan.linear(self.down), self.hidden, 1 if self.fused else 0)
+        return plan.part("feed_forward.swiglu", desc, takes_deferred_rows=True,
+                         adds_residual=True, first=first)
 
     def weight_bytes(self) -> int:
         return self.gate_up.weight_bytes() + self.down.weight_bytes()

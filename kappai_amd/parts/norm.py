@@ -10,6 +10,7 @@ import torch
 from ..kernels import ops, profile, tuning
 from ..weights.spec import INIT_ONES, VECTOR, TensorSpec
 from .base import Norm, register_part
+from .cdesc import FoldDesc
 
 
 class RMSNorm(Norm):
@@ -53,6 +54,12 @@ class RMSNorm(Norm):
         with profile.scope("rmsnorm" if rows is None else "logits_norm"):
             return ops.add_rmsnorm(resid, delta, self.weight, self.eps, self.dtype, rows=rows,
                                    write_resid=rows is None, fragment=fragment)
+
+    def c_norm(self, plan):
+        """The norm as the C side of a step runs it: the runner "norm.rms" reads weight and eps,
+        which is also all a product needs to fold the norm in."""
+        fold = plan.keep(FoldDesc(self.weight.data_ptr(), self.eps))
+        return plan.norm("norm.rms", fold, fold=fold)
 
     def weight_bytes(self) -> int:
         return self.width * 4

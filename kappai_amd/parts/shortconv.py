@@ -15,8 +15,17 @@ import torch
 from ..cache.specs import FixedState
 from ..kernels import ops, profile, tuning
 from ..weights.spec import INIT_NORMAL, INIT_SMALL, VECTOR, TensorSpec
+from ctypes import Structure, c_int, c_void_p
+
 from .base import Mixer, register_part
+from .cdesc import LinearDesc, tensor_ptr
 from .linear import Linear
+
+
+class ConvMixerDesc(Structure):
+    """``kappai_conv_mixer`` of csrc/engine_parts.h."""
+    _fields_ = [("in_proj", LinearDesc), ("out_proj", LinearDesc), ("taps", c_void_p),
+                ("conv_bias", c_void_p), ("taps_per_channel", c_int), ("state", c_void_p)]
 
 
 class GatedShortConv(Mixer):
@@ -85,6 +94,16 @@ class GatedShortConv(Mixer):
             y = ops.shortconv(proj, self.taps, self.conv_bias, cache.state, batch.row_seg,
                               batch.seg_start, batch.seg_pos0, batch.seg_slot)
         return self.out_proj.forward(y, partial_sums=True, add_into=into)
+
+    def c_part(self, plan, view, shared_cache: bool = False):
+        """The runner "mixer.conv" (csrc/engine_parts.hip) makes the same choices as ``forward``."""
+        if shared_cache:
+            return None
+        first = plan.linear(self.in_proj)
+        desc = ConvMixerDesc(first, plan.linear(self.out_proj), self.taps.data_ptr(),
+                             tensor_ptr(self.conv_bias), self.L, view.state.data_ptr())
+        return plan.part("mixer.conv", desc, takes_deferred_rows=True, adds_residual=True,
+                         first=first)
 
     def weight_bytes(self) -> int:
         return self.in_proj.weight_bytes() + self.out_proj.weight_bytes() + self.width * self.L * 4

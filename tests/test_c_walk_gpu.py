@@ -1,0 +1,300 @@
+"""The C side of a step takes parts by registry: a mixer that the framework has never heard of,
+defined here with a HIP kernel and a runner of its own (``tests/toy_parts/running_mean.hip``),
+is registered, built into a toy architecture and stepped through ``kappai_forward`` without a
+change to the framework's files, bit for bit equal to the same steps run part by part from the
+host; and what has no description for the C side runs from the host as before."""
+import ctypes
+from ctypes import Structure, c_int, c_void_p
+from dataclasses import dataclass
+from pathlib import Path
+
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+TOY_SOURCE = Path(__file__).resolve().parent / "toy_parts" / "running_mean.hip"
+
+
+def toy_library():
+    from kappai_amd.kernels.lib import library_at
+    lib = library_at(TOY_SOURCE)
+    lib.toy_running_mean_run.restype = None       # only its address is used
+    return lib
+
+
+def define_toy():
+    """Registers the toy mixer and the toy architecture (once) and returns the mixer's class."""
+    from kappai_amd.cache import FixedState
+    from kappai_amd.config import ModelConfig, register_architecture
+    from kappai_amd.kernels import ops
+    from kappai_amd.models import LayerCall, Model
+    from kappai_amd.parts import Linear, Mixer, OutputHead, TokenEmbedding, make_part, register_part
+    from kappai_amd.parts.cdesc import RUNNER_PART, LinearDesc
+
+    from kappai_amd.parts import MIXERS
+    if "toy_running_mean_hip" in MIXERS:
+        return MIXERS["toy_running_mean_hip"]
+
+    class ToyDesc(Structure):
+        """``toy_running_mean`` of tests/toy_parts/running_mean.hip."""
+        _fields_ = [("proj", LinearDesc), ("state", c_void_p)]
+
+    class RunningMeanHip(Mixer):
+        """out_t = W * mean(x_0 .. x_t); state [width] float32: the running sum."""
+
+        def __init__(self, prefix, width, dtype):
+            self.width, self.dtype = width, dtype
+            self.proj = Linear([prefix + "proj"], width, [width])
+
+        def cache_spec(self):
+            return FixedState((self.width,), "float32")
+
+        def tensor_specs(self):
+            return self.proj.tensor_specs()
+
+        def bind(self, tensors):
+            self.proj.bind(tensors)
+
+        def forward(self, x, batch, cache, shared_cache=False):
+            lib = toy_library()
+            mean = torch.empty((x.shape[0], self.width), dtype=x.dtype, device=x.device)
+            rc = lib.toy_running_mean_launch(
+                c_void_p(x.data_ptr()), c_int(x.stride(0)), c_void_p(mean.data_ptr()),
+                c_void_p(cache.state.data_ptr()), c_void_p(batch.seg_start.data_ptr()),
+                c_void_p(batch.seg_pos0.data_ptr()), c_void_p(batch.seg_slot.data_ptr()),
+                c_int(batch.n_segments), c_int(self.width),
+                c_int(1 if x.dtype == torch.bfloat16 else 0), ops._stream())
+            assert rc == 0, rc
+            return self.proj.forward(mean)
+
+        def c_part(self, plan, view, shared_cache=False):
+            lib = toy_library()
+            assert lib.toy_running_mean_desc_bytes() == ctypes.sizeof(ToyDesc)
+            plan.register_runner("mixer.toy_running_mean", RUNNER_PART, lib.toy_running_mean_run,
+                                 ToyDesc)
+            first = plan.linear(self.proj)
+            return plan.part("mixer.toy_running_mean", ToyDesc(first, view.state.data_ptr()))
+
+    register_part("mixer", "toy_running_mean_hip", RunningMeanHip)
+
+    class ChangedForward(RunningMeanHip):
+        """A subclass that changes ``forward`` and says nothing about C: twice the mean."""
+
+        def forward(self, x, batch, cache, shared_cache=False):
+            return 2 * super().forward(x, batch, cache, shared_cache)
+
+    register_part("mixer", "toy_running_mean_changed", ChangedForward)
+
+    @dataclass
+    class ToyConfig(ModelConfig):
+        width: int = 0
+        vocab_size: int = 0
+        heads: int = 0
+        head_dim: int = 0
+        ff: int = 0
+        eps: float = 1e-5
+        mixer: str = "toy_running_mean_hip"
+        max_position_embeddings: int = 512
+
+        @classmethod
+        def from_dict(cls, raw):
+            return cls(architecture="ToyHipForCausalLM", **{k: raw[k] for k in
+                       ("width", "vocab_size", "heads", "head_dim", "ff", "eps", "mixer")})
+
+        def to_dict(self):
+            return {"architectures": ["ToyHipForCausalLM"], "width": self.width,
+                    "vocab_size": self.vocab_size, "heads": self.heads, "head_dim": self.head_dim,
+                    "ff": self.ff, "eps": self.eps, "mixer": self.mixer}
+
+    def build_toy(cfg, dtype):
+        def norm(name):
+            return make_part("norm", "rmsnorm", name=name, width=cfg.width, eps=cfg.eps,
+                             dtype=dtype)
+
+        def block(i, mixer):
+            p = f"blocks.{i}."
+            return make_part("block", "pre_norm", mixer_norm=norm(p + "n1"), mixer=mixer,
+                             ffn_norm=norm(p + "n2"),
+                             feed_forward=make_part("feed_forward", "swiglu", prefix=p + "ff.",
+                                                    width=cfg.width, hidden=cfg.ff, dtype=dtype))
+        rot = make_part("position_encoding", "rotary", head_dim=cfg.head_dim, theta=100.0)
+
+        def attn(i):
+            return make_part("mixer", "attention", prefix=f"blocks.{i}.att.", width=cfg.width,
+                             num_heads=cfg.heads, num_kv_heads=cfg.heads // 2,
+                             head_dim=cfg.head_dim, dtype=dtype, position=rot, qk_norm_eps=1e-5)
+        layers = [block(0, make_part("mixer", cfg.mixer, prefix="blocks.0.mix.", width=cfg.width,
+                                     dtype=dtype)),
+                  block(1, attn(1)), block(2, attn(2))]
+        emb = TokenEmbedding("emb", cfg.vocab_size, cfg.width)
+        # block 0 runs twice (two states), block 2 reads the keys that block 1 stored
+        schedule = [LayerCall(0), LayerCall(1), LayerCall(0), LayerCall(2, reads_cache_of=1)]
+        return Model(cfg, dtype, emb, layers, norm("final"),
+                     OutputHead("head", cfg.vocab_size, cfg.width, tied_to=emb), schedule=schedule)
+
+    register_architecture("ToyHipForCausalLM", ToyConfig, build_toy)
+    return RunningMeanHip
+
+
+TOY = {"architectures": ["ToyHipForCausalLM"], "width": 64, "vocab_size": 211, "heads": 4,
+       "head_dim": 32, "ff": 96, "eps": 1e-5, "mixer": "toy_running_mean_hip"}
+
+
+def toy_model(tmp_path, dtype, mixer="toy_running_mean_hip"):
+    from kappai_amd.config import config_from_dict
+    from kappai_amd.models import load_model
+    from kappai_amd.weights import write_random_model
+    define_toy()
+    folder = tmp_path / f"toy_{mixer}"
+    if not folder.exists():
+        write_random_model(folder, config_from_dict(dict(TOY, mixer=mixer)), seed=5, std=0.2,
+                           norm_jitter=0.1)
+    return load_model(folder, dtype, DEV)
+
+
+def replay(model, steps, peak, out_dir, c_forward, graphs):
+    from kappai_amd.engine.replay import TraceReplayer, make_replay_cache
+    from kappai_amd.engine.step import StepRunner
+    cache = make_replay_cache(model, peak)
+    cache.allocate_storage(model.dtype, DEV, poison=True)
+    runner = StepRunner(model, cache, DEV, decode_graphs=graphs, c_forward=c_forward)
+    rep = TraceReplayer(runner, out_dir)
+    results = [rep.run_step(obj) for obj in steps]
+    cache.check()
+    return results, runner
+
+
+def test_the_toy_kernel_is_a_running_mean():
+    """The toy's kernel against torch: a portion after a history (the sum so far in the state),
+    a fresh request beside it (whatever the slot held before is not read)."""
+    lib = toy_library()
+    D = 70
+    x = torch.randn(9, D, generator=torch.Generator().manual_seed(1))
+    state = torch.full((3, D), float("nan"))
+    history = torch.randn(4, D, generator=torch.Generator().manual_seed(2))
+    state[2] = history.sum(0)
+    seg_start = torch.tensor([0, 5, 9], dtype=torch.int32, device=DEV)
+    seg_pos0 = torch.tensor([4, 0], dtype=torch.int32, device=DEV)
+    seg_slot = torch.tensor([2, 0], dtype=torch.int32, device=DEV)
+    xd, sd = x.to(DEV), state.to(DEV)
+    out = torch.empty_like(xd)
+    rc = lib.toy_running_mean_launch(
+        c_void_p(xd.data_ptr()), c_int(D), c_void_p(out.data_ptr()), c_void_p(sd.data_ptr()),
+        c_void_p(seg_start.data_ptr()), c_void_p(seg_pos0.data_ptr()),
+        c_void_p(seg_slot.data_ptr()), c_int(2), c_int(D), c_int(0),
+        c_void_p(torch.cuda.current_stream().cuda_stream))
+    assert rc == 0
+    want = torch.cat([(history.sum(0) + torch.cumsum(x[:5], 0)) / torch.arange(5, 10)[:, None],
+                      torch.cumsum(x[5:], 0) / torch.arange(1, 5)[:, None]])
+    assert float((out.cpu() - want).abs().max()) < 1e-5
+    assert float((sd[2].cpu() - (history.sum(0) + x[:5].sum(0))).abs().max()) < 1e-5
+    assert float((sd[0].cpu() - x[5:].sum(0)).abs().max()) < 1e-5
+    assert torch.isnan(sd[1]).all()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_mixer_from_outside_runs_from_c(tmp_path, dtype):
+    """The toy architecture (the toy mixer run twice with two states, attention, an attention
+    call that reads another call's keys) under the mixed schedule: launched from C it gives bit
+    for bit what the host's part-by-part walk gives, with and without decode graphs, and the
+    portions give what whole prompts give."""
+    import schedules
+    from replay_common import collect, make_requests
+    model = toy_model(tmp_path, dtype)
+    requests = make_requests(TOY["vocab_size"], [70, 45, 100, 37, 83, 64, 29], seed=22)
+    steps, index, peak = schedules.mixed(requests)
+    results = {}
+    for c_forward in (True, False):
+        for graphs in (False, True):
+            res, runner = replay(model, steps, peak, tmp_path / f"c{c_forward}g{graphs}",
+                                 c_forward, graphs)
+            assert (runner._cplan is not None) == c_forward, "the toy model has a description"
+            if graphs:
+                assert runner.graph_replays > 0
+            results[(c_forward, graphs)] = res
+    base = results[(False, False)]
+    for key, res in results.items():
+        for a, b in zip(base, res):
+            assert (a is None) == (b is None)
+            if a is not None:
+                assert np.array_equal(a, b), key
+    # and cut into portions it is the model that whole prompts give
+    whole_steps, whole_index, whole_peak = schedules.whole(requests)
+    whole, _ = replay(model, whole_steps, whole_peak, tmp_path / "whole", True, False)
+    got = collect(index, {s["step"]: r for s, r in zip(steps, base) if r is not None},
+                  TOY["vocab_size"])
+    ref = collect(whole_index, {s["step"]: r for s, r in zip(whole_steps, whole) if r is not None},
+                  TOY["vocab_size"])
+    scale = max(float(np.abs(v).max()) for v in ref.values())
+    tol = 2e-5 if dtype == "float32" else 4e-2
+    worst = max(float(np.abs(got[k] - ref[k]).max()) for k in ref) / scale
+    assert worst < tol, worst
+
+
+def test_the_toy_mixer_does_what_it_says_inside_the_model(tmp_path):
+    """With every other part's contribution removed (out projections and down projections zero),
+    the logits are head(norm(embedding + W mean(norm(embedding)) twice over)): worked out in
+    float64 from the weights, against the C walk."""
+    model = toy_model(tmp_path, "float32")
+    for blk in model.layers:
+        blk.feed_forward.down.weight.zero_()
+        if hasattr(blk.mixer, "out"):
+            blk.mixer.out.weight.zero_()
+    toks = [int(t) for t in np.random.default_rng(3).integers(0, TOY["vocab_size"], size=19)]
+    steps = [{"step": 0, "entries": [{"id": "a", "tokens": toks, "want": list(range(19))}],
+              "end": ["a"]}]
+    (got,), runner = replay(model, steps, 64, tmp_path / "zeroed", True, False)
+    assert runner._cplan is not None
+    E = model.embedding.table.double().cpu().numpy()
+    blk = model.layers[0]
+    W = blk.mixer.proj.weight.double().cpu().numpy()
+    n1 = blk.mixer_norm.weight.double().cpu().numpy()
+    fin = model.final_norm.weight.double().cpu().numpy()
+
+    def rms(x, w):
+        return x / np.sqrt((x * x).mean(-1, keepdims=True) + TOY["eps"]) * w
+    x = E[toks]
+    for _ in range(2):                       # block 0 runs twice
+        xb = rms(x, n1)
+        x = x + (np.cumsum(xb, 0) / np.arange(1, 20)[:, None]) @ W.T
+    want = rms(x, fin) @ E.T
+    assert float(np.abs(got - want).max()) < 2e-5 * float(np.abs(want).max())
+
+
+def test_a_part_that_changed_forward_without_a_description_runs_from_the_host(tmp_path):
+    """A subclass of the toy mixer changes ``forward`` and gives no description of its own: it
+    must not inherit its parent's runner.  Its model runs part by part from the host, and its
+    logits differ from the parent's."""
+    steps = [{"step": 0, "entries": [{"id": "a", "tokens": [5, 9, 200, 17, 3], "want": [4]}],
+              "end": ["a"]}]
+    changed = toy_model(tmp_path, "float32", mixer="toy_running_mean_changed")
+    (got,), runner = replay(changed, steps, 64, tmp_path / "changed", True, False)
+    assert runner._cplan is None
+    parent = toy_model(tmp_path, "float32")
+    (base,), runner = replay(parent, steps, 64, tmp_path / "parent", True, False)
+    assert runner._cplan is not None
+    assert float(np.abs(got - base).max()) > 1e-3
+
+
+def test_runners_are_looked_up_by_name_and_checked():
+    """The registry: the framework's own parts are there under their names; an unknown name and
+    a description of another size are refused with a message."""
+    from kappai_amd.engine.cforward import engine_library
+    from kappai_amd.kernels.lib import KernelLaunchError
+    from kappai_amd.parts.cdesc import RUNNER_NORM, RUNNER_PART, CPlan, FoldDesc, LinearDesc
+
+    plan = CPlan(engine_library(), type("M", (), {"dtype": torch.float32})(), None, DEV)
+    assert plan.runner("norm.rms", RUNNER_NORM, FoldDesc)
+    with pytest.raises(KernelLaunchError, match="no runner is registered"):
+        plan.runner("mixer.nobody", RUNNER_PART, FoldDesc)
+    with pytest.raises(KernelLaunchError, match="no runner is registered"):
+        plan.runner("norm.rms", RUNNER_PART, FoldDesc)            # another kind
+    with pytest.raises(KernelLaunchError, match="reads a description of"):
+        plan.runner("mixer.conv", RUNNER_PART, LinearDesc)
+    lib = toy_library()
+    plan.register_runner("mixer.toy_again", RUNNER_PART, lib.toy_running_mean_run, FoldDesc)
+    plan.register_runner("mixer.toy_again", RUNNER_PART, lib.toy_running_mean_run, FoldDesc)
+    with pytest.raises(KernelLaunchError, match="registered already"):
+        plan.register_runner("mixer.toy_again", RUNNER_PART, lib.toy_running_mean_launch, FoldDesc)

@@ -97,10 +97,7 @@ def decode_split_plan(ops, T, G, d, n_keys):
     """(most splits, planned) as ``ops._decode_split`` and the kernel's launcher settle them."""
     from kappai_amd.kernels.lib import library
     kpw = library("attention_mfma", HEAD_DIM=d).kappai_attn_keys_per_wave()
-    n_splits = max(1, min(ops.DECODE_MAX_SPLITS, (n_keys + kpw - 1) // kpw,
-                          max(1, ops.DECODE_WAVES // (T * G))))
-    kps = ((n_keys + n_splits - 1) // n_splits + kpw - 1) // kpw * kpw
-    n_splits = (n_keys + kps - 1) // kps
+    _, n_splits = ops.decode_splits(kpw, T, G, n_keys)
     return n_splits, T * G * n_splits > ops.DECODE_WAVES // 2
 
 
