@@ -8,7 +8,10 @@ W untimed and K timed decode steps at batch 8 with every request holding a conte
 tokens at the last step (one step = one token for every request: row tables, model,
 sampling on the GPU, token ids back on the host), a prefill of 2,048 tokens (a step among eight
 such prompts queued one behind the other, as the decode steps are queued; "alone_ms" is one such
-step with the GPU idle before it), and decode at batch 1 and 64.  It prints ONE JSON line.  The model is a folder that the framework's own
+step with the GPU idle before it), and further points: decode at batch 1 and 64, decode at the
+headline batch with contexts of 32,768 tokens, prompt steps of 128 and 512 tokens ("points":
+tokens a second; "points_frac": each point's share of the peak that bounds it, HBM for decode
+steps and the matrix cores for prompt steps).  It prints ONE JSON line.  The model is a folder that the framework's own
 random-weights mode writes (config.json, model.safetensors) and its own loader reads; token ids
 are uniform random with a fixed seed, and every request's context is computed by real prompt
 steps before its decoding is timed: no dataset is involved ("data": "synthetic").  kappai
@@ -253,23 +256,28 @@ class DecodeBench:
             self.cache.close(rc)
 
 
-def measured_read_bandwidth(device, mb=256, buffers=5, reps=20):
-    """GB/s of a kernel that only reads: buffers of ``mb`` MB taken in turn (more than the
-    memory-side cache holds), ``reps`` reads between two synchronisations."""
+def measured_read_bandwidth(device, mb=256, buffers=8, reps=24):
+    """GB/s of a kernel that only reads: buffers of ``mb`` MB taken in turn (2 GB together, eight
+    times what the memory-side cache holds), ``reps`` reads between two synchronisations; the best
+    of several numbers of blocks sharing a read, so that the figure is what reading reaches on
+    this box and not what one launch shape reaches."""
     import torch
 
     from kappai_amd.kernels import ops
     bufs = [torch.empty(mb * 1000 * 1000 // 4, dtype=torch.int32, device=device).random_()
             for _ in range(buffers)]
-    for b in bufs:
-        ops.stream_read(b)
-    sync()
-    t0 = time.perf_counter()
-    total = 0
-    for i in range(reps):
-        total += ops.stream_read(bufs[i % buffers])
-    sync()
-    return total / (time.perf_counter() - t0) / 1e9
+    best = 0.0
+    for blocks in (512, 1024, 2048, 4096):
+        for b in bufs:
+            ops.stream_read(b, blocks)
+        sync()
+        t0 = time.perf_counter()
+        total = 0
+        for i in range(reps):
+            total += ops.stream_read(bufs[i % buffers], blocks)
+        sync()
+        best = max(best, total / (time.perf_counter() - t0) / 1e9)
+    return best
 
 
 def measured_mfma_tflops(device, iters=20000):
@@ -304,8 +312,11 @@ def graph_time(fn, reps):
 
 def kernel_rates(model, cfg, batch, context, prefill_tokens, page_size, device, read_gbs,
                  mfma_tflops, dtype):
-    """The engine's own kernels by class, one by one at the shapes of this run, each over the
-    layers of the model in turn (cold weights, as in a step): the products of a decode step (K3),
+    """The engine's own kernels by class, one by one at the shapes of this run, each over
+    distinct matrices in turn that together exceed the memory-side cache several times (the
+    model's own layers, and copies where those are too few: 2 GB for the head and for the cache
+    of the decode attention), so that every call reads from memory as in a step: the products of
+    a decode step (K3),
     decode attention over the cache (K10) and the output head (K11) in GB/s of what they have to
     read, the products of a prompt step (K4) and its attention (K9) in TFLOP/s.  Every figure
     also as a fraction of the published peak and of what the read-only / multiply-only kernels
@@ -348,18 +359,31 @@ def kernel_rates(model, cfg, batch, context, prefill_tokens, page_size, device, 
     dn = [f.down for f in ffs]
     t = graph_time(lambda i: dn[i % n].forward(act, add_into=ops.AddInto(resid)), 2 * n)
     rate_gbs("k3_decode_down", t, dn[0].weight_bytes())
+    def copies(weight, total_bytes):
+        """The matrix and copies of it, ``total_bytes`` together."""
+        nbytes = weight.numel() * weight.element_size()
+        k = max(1, -(-total_bytes // nbytes) - 1)
+        clone = (lambda w: ops.InFragments(w.data.clone())) if isinstance(
+            weight, ops.InFragments) else (lambda w: w.clone())
+        return [weight] + [clone(weight) for _ in range(k)]
+
     if convs:
-        ip = [c.in_proj for c in convs]
-        t = graph_time(lambda i: ops.linear(x, ip[i % len(ip)].weight), 2 * len(ip))
-        rate_gbs("k3_decode_in_proj", t, ip[0].weight_bytes())
+        ip = [c.in_proj.weight for c in convs]
+        while sum(w.numel() * 2 for w in ip) < 1 << 30:
+            ip = ip + copies(ip[0], 0)[1:]
+        t = graph_time(lambda i: ops.linear(x, ip[i % len(ip)]), len(ip))
+        rate_gbs("k3_decode_in_proj", t, convs[0].in_proj.weight_bytes())
     # K11: the output head on `batch` rows
     head = model.head.linear
-    t = graph_time(lambda i: head.forward(x, out_dtype=torch.float32), 4)
+    heads = copies(head.weight, 2 << 30)
+    t = graph_time(lambda i: ops.linear(x, heads[i % len(heads)], head.bias,
+                                        out_dtype=torch.float32), len(heads))
     rate_gbs("k11_head", t, head.weight_bytes())
+    del heads
     # K10: decode attention of `batch` requests over `context` keys
     if cfg.attention_layers and d % 16 == 0:
         per = (context + page_size - 1) // page_size
-        n_pool = 3
+        n_pool = max(3, -(-(2 << 30) // (batch * per * G * page_size * d * 2 * 2)))
         kp = [torch.randn(batch * per + 1, G, page_size, d, generator=g, device=device).to(BF)
               for _ in range(n_pool)]
         vp = [torch.randn(batch * per + 1, G, d, page_size, generator=g, device=device).to(BF)
@@ -370,7 +394,7 @@ def kernel_rates(model, cfg, batch, context, prefill_tokens, page_size, device, 
         seg = torch.arange(batch, dtype=torch.int32, device=device)
         t = graph_time(lambda i: ops.paged_attention(
             q, H, G, d, kp[i % n_pool], vp[i % n_pool], pos, seg, bt, page_size,
-            1.0 / math.sqrt(d), single_rows=True, max_position=context - 1), 2 * n_pool)
+            1.0 / math.sqrt(d), single_rows=True, max_position=context - 1), n_pool)
         rate_gbs("k10_decode_attention", t, batch * context * G * d * 2 * 2)
         del kp, vp
     # K4: products of a prompt step of `prefill_tokens` rows
@@ -383,7 +407,7 @@ def kernel_rates(model, cfg, batch, context, prefill_tokens, page_size, device, 
     t = graph_time(lambda i: dn[i % n].forward(actp, partial_sums=True), n)
     rate_tflops("k4_prefill_down", t, 2.0 * T * F * D)
     if convs:
-        t = graph_time(lambda i: ops.linear(xp, ip[i % len(ip)].weight), len(ip))
+        t = graph_time(lambda i: ops.linear(xp, ip[i % len(ip)]), len(convs))
         rate_tflops("k4_prefill_in_proj", t, 2.0 * T * D * 3 * D)
     # K9: attention of one prompt of `prefill_tokens` tokens over itself
     if cfg.attention_layers and d % 16 == 0:
@@ -438,6 +462,12 @@ def main() -> int:
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--page-size", type=int, default=16)
     ap.add_argument("--skip-points", action="store_true", help="only the headline batch")
+    ap.add_argument("--long-context", type=int, default=32768,
+                    help="a further decode point at the headline batch with contexts of this many "
+                         "tokens (0: none)")
+    ap.add_argument("--short-prompts", type=lambda v: [int(x) for x in v.split(",") if x],
+                    default=[128, 512],
+                    help="further prompt-step points: tokens a prompt, comma separated")
     ap.add_argument("--skip-kernels", action="store_true",
                     help="leave out the kernel-by-kernel rates")
     ap.add_argument("--no-graphs", action="store_true",
@@ -467,68 +497,93 @@ def main() -> int:
     cfg = model.config
     elem = 2 if args.dtype == "bfloat16" else 4
     K, W = args.steps, args.warmup
-    start = args.context - (K + W)
-    if start < 1:
+    if args.context - (K + W) < 1:
         print("bench.py: --context must exceed --steps + --warmup")
         return 2
 
-    def decode(batch):
-        b = DecodeBench(model, batch, start, args.context, args.page_size, device,
+    def decode(batch, context=None):
+        """(seconds of the K timed steps, tok/s, share of the HBM peak) of decoding at ``batch``
+        with contexts of ``context`` tokens at the last step.  The bytes a decode step has to
+        read: every weight once, and the cache of the live requests at their mean length."""
+        context = context or args.context
+        first = context - (K + W)
+        b = DecodeBench(model, batch, first, context, args.page_size, device,
                         graphs=not args.no_graphs)
         dt = b.run(W, K)
         kv_bytes = b.cache.bytes_per_token(elem)
         b.close()
         del b
         torch.cuda.empty_cache()
-        return dt, kv_bytes
+        mean_ctx = first + W + (K - 1) / 2.0
+        step_bytes = model.weight_bytes_per_step() + batch * mean_ctx * kv_bytes
+        return dt, batch * K / dt, step_bytes / (dt / K) / 1e9
 
-    dt, kv_bytes_per_token = decode(args.batch)
+    dt, value, achieved = decode(args.batch)
     ms_per_step = dt / K * 1e3
-    value = args.batch * K / dt
-    # bytes a decode step has to read: every weight once, the cache of the live requests
-    mean_ctx = start + W + (K - 1) / 2.0
-    step_bytes = model.weight_bytes_per_step() + args.batch * mean_ctx * kv_bytes_per_token
-    achieved = step_bytes / (dt / K) / 1e9
 
-    points = {}
+    # further points: tokens a second, and beside each its share of the peak that bounds it (HBM
+    # for decode steps, the matrix cores for prompt steps) in points_frac
+    points, points_frac = {}, {}
     if not args.skip_points:
         for b in (1, 64):
             if b == args.batch:
                 points[f"decode_b{b}"] = round(value, 1)
+                points_frac[f"decode_b{b}"] = round(achieved / HBM_PEAK_GBS, 4)
                 continue
-            dtb, _ = decode(b)
-            points[f"decode_b{b}"] = round(b * K / dtb, 1)
+            _, rate, gbs = decode(b)
+            points[f"decode_b{b}"] = round(rate, 1)
+            points_frac[f"decode_b{b}"] = round(gbs / HBM_PEAK_GBS, 4)
+        if args.long_context > K + W and args.long_context != args.context:
+            _, rate, gbs = decode(args.batch, args.long_context)
+            points[f"decode_b{args.batch}_ctx{args.long_context}"] = round(rate, 1)
+            points_frac[f"decode_b{args.batch}_ctx{args.long_context}"] = round(
+                gbs / HBM_PEAK_GBS, 4)
 
     read_gbs = measured_read_bandwidth(device)
     # (the probe multiplies bfloat16; a float32 run has no matrix-core yardstick)
     mfma_tflops = measured_mfma_tflops(device) if args.dtype == "bfloat16" else None
 
     # prefill of one prompt, whole, logits at its last token
-    T = args.prefill_tokens
-    cm = CacheManager(model.cache_specs(), args.page_size, (T + args.page_size - 1) // args.page_size + 1, 1)
-    cm.allocate_storage(model.dtype, device)
-    runner = StepRunner(model, cm, device)
-    toks = [int(t) for t in torch.randint(0, cfg.vocab_size, (T,), generator=torch.Generator().manual_seed(2))]
-    def prompt_steps(n):
-        """n prompts of T tokens, one step each, queued one behind the other; seconds a step."""
-        sync()
-        t0 = time.perf_counter()
-        for i in range(n):
-            rc = cm.open(f"p{i}")
-            runner.step([StepEntry(rc, toks, [T - 1])])
-            cm.close(rc)                     # (its pages go to the next prompt: one stream, in order)
-        sync()
-        return (time.perf_counter() - t0) / n
-
-    # one step by itself (the GPU idle before and after it), and PREFILL_STEPS of them back to
-    # back, which is how an engine with work waiting runs them and how the decode steps above are
-    # timed: the host's launches then run ahead of the kernels and the chip keeps its clocks
-    alone_s = min(prompt_steps(1) for _ in range(3))
-    pre_s = min(prompt_steps(PREFILL_STEPS) for _ in range(2))
-    flops = prefill_flops(cfg, T, n_layers)
     peak = MFMA_PEAK_TFLOPS[args.dtype] * 1e12
-    del runner, cm
-    torch.cuda.empty_cache()
+
+    def prefill(T):
+        """(seconds of a step alone, seconds of a step among PREFILL_STEPS queued one behind the
+        other, flops of a step) for prompts of ``T`` tokens."""
+        cm = CacheManager(model.cache_specs(), args.page_size,
+                          (T + args.page_size - 1) // args.page_size + 1, 1)
+        cm.allocate_storage(model.dtype, device)
+        runner = StepRunner(model, cm, device)
+        toks = [int(t) for t in torch.randint(0, cfg.vocab_size, (T,),
+                                              generator=torch.Generator().manual_seed(2))]
+
+        def prompt_steps(n):
+            """n prompts of T tokens, one step each, queued one behind the other; seconds a step."""
+            sync()
+            t0 = time.perf_counter()
+            for i in range(n):
+                rc = cm.open(f"p{i}")
+                runner.step([StepEntry(rc, toks, [T - 1])])
+                cm.close(rc)                 # (its pages go to the next prompt: one stream, in order)
+            sync()
+            return (time.perf_counter() - t0) / n
+
+        # one step by itself (the GPU idle before and after it), and PREFILL_STEPS of them back to
+        # back, which is how an engine with work waiting runs them and how the decode steps above
+        # are timed: the host's launches then run ahead of the kernels and the chip keeps its clocks
+        alone = min(prompt_steps(1) for _ in range(3))
+        queued = min(prompt_steps(PREFILL_STEPS) for _ in range(2))
+        del runner, cm
+        torch.cuda.empty_cache()
+        return alone, queued, prefill_flops(cfg, T, n_layers)
+
+    T = args.prefill_tokens
+    alone_s, pre_s, flops = prefill(T)
+    if not args.skip_points:
+        for t_short in args.short_prompts:
+            if t_short != T:
+                _, queued, fl = prefill(t_short)
+                points[f"prefill_t{t_short}"] = round(t_short / queued, 1)
+                points_frac[f"prefill_t{t_short}"] = round(fl / queued / peak, 4)
     kernels = {} if args.skip_kernels else kernel_rates(
         model, cfg, args.batch, args.context, T, args.page_size, device, read_gbs, mfma_tflops,
         args.dtype)
@@ -564,6 +619,7 @@ def main() -> int:
                      "measured_read": round(read_gbs, 1),
                      "frac_of_measured_read": round(achieved / read_gbs, 5)},
         "points": points,
+        "points_frac": points_frac,
         "kernels": kernels,
     }
     print(json.dumps(out))

@@ -430,11 +430,13 @@ __global__ __launch_bounds__(256) void stream_read_kernel(const stream_u32x4_t* 
   if ((acc.x ^ acc.y ^ acc.z ^ acc.w) == 0x9e3779b9u && sink != nullptr) sink[0] = acc.x;
 }
 
-// Reads the first `bytes` of `p` (rounded down to what 512 blocks share evenly in pieces of
-// 32 KB) once.  Returns the bytes read through *bytes_read.
+// Reads the first `bytes` of `p` (rounded down to what `blocks` blocks share evenly in pieces of
+// 32 KB) once.  Returns the bytes read through *bytes_read.  blocks: 0 for 512, else how many
+// blocks share the read (the bench takes the best of several).
 extern "C" int kappai_stream_read(const void* p, long bytes, uint32_t* sink, long* bytes_read,
-                                  hipStream_t stream) {
-  const int blocks = 512;
+                                  int blocks, hipStream_t stream) {
+  if (blocks == 0) blocks = 512;
+  if (blocks < 1 || blocks > 65535) return (int)hipErrorInvalidValue;
   const size_t piece = 8 * 256;                                  // 16-byte elements a block and turn
   const size_t n_per_block = ((size_t)bytes / 16 / blocks / piece) * piece;
   if (bytes_read) *bytes_read = (long)(n_per_block * blocks * 16);

@@ -310,14 +310,15 @@ def sum_partial_sums(parts: torch.Tensor) -> torch.Tensor:
     return out
 
 
-def stream_read(buf: torch.Tensor) -> int:
+def stream_read(buf: torch.Tensor, blocks: int = 0) -> int:
     """Launches one plain read of ``buf`` (a kernel that only loads) and returns the bytes it
-    reads: the yardstick for the kernels that stream weights and cache."""
+    reads: the yardstick for the kernels that stream weights and cache.  ``blocks``: how many
+    blocks of four waves share the read (0: 512)."""
     _gpu("buf", buf)
     n = ctypes.c_long(0)
     check(library("elementwise").kappai_stream_read(
         _ptr(buf), _c_long(buf.numel() * buf.element_size()), _vp(0), ctypes.byref(n),
-        _stream()), "stream_read")
+        _c_int(blocks), _stream()), "stream_read")
     return n.value
 
 

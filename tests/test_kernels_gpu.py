@@ -82,6 +82,10 @@ def test_stream_read_stays_inside_the_buffer(ops):
         buf = torch.zeros(n_bytes // 4, dtype=torch.int32, device=DEV)
         got = ops.stream_read(buf)
         assert 0 < got <= n_bytes and got % (512 * 32768) == 0 and n_bytes - got < 512 * 32768
+        for blocks in (256, 2048):
+            got = ops.stream_read(buf, blocks=blocks)
+            assert 0 < got <= n_bytes and got % (blocks * 32768) == 0
+            assert n_bytes - got < blocks * 32768
     torch.cuda.synchronize()
     with pytest.raises(RuntimeError):
         ops.stream_read(torch.zeros(1000, dtype=torch.int32, device=DEV))
