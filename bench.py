@@ -35,31 +35,12 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, GB/s
 MFMA_PEAK_TFLOPS = {"bfloat16": 2500.0, "float32": 157.3}      # dense
 
-LFM2_1_2B = {
-    "architectures": ["Lfm2ForCausalLM"], "model_type": "lfm2", "hidden_size": 2048,
-    "num_hidden_layers": 16,
-    "layer_types": ["conv", "conv", "full_attention", "conv", "conv", "full_attention", "conv",
-                    "conv", "full_attention", "conv", "full_attention", "conv", "full_attention",
-                    "conv", "full_attention", "conv"],
-    "num_attention_heads": 32, "num_key_value_heads": 8, "head_dim": 64,
-    "intermediate_size": 12288, "block_auto_adjust_ff_dim": True, "block_multiple_of": 256,
-    "block_ffn_dim_multiplier": 1.0, "vocab_size": 65536, "norm_eps": 1e-5,
-    "rope_theta": 1000000.0, "conv_L_cache": 3, "conv_bias": False, "tie_embedding": True,
-    "max_position_embeddings": 128000,
-}
+def _shape(name):
+    from kappai_amd.config import named_shape
+    return named_shape(name)
 
 
-def lfm2_shape(hidden, layers, attention_at, heads, kv_heads, intermediate):
-    raw = dict(LFM2_1_2B)
-    raw.update(hidden_size=hidden, num_hidden_layers=layers, num_attention_heads=heads,
-               num_key_value_heads=kv_heads, intermediate_size=intermediate,
-               layer_types=["full_attention" if i in attention_at else "conv"
-                            for i in range(layers)])
-    return raw
-
-
-LFM2_350M = lfm2_shape(1024, 16, (2, 5, 8, 10, 12, 14), 16, 8, 6656)
-LFM2_2_6B = lfm2_shape(2048, 30, (2, 6, 10, 14, 18, 21, 24, 27), 32, 8, 10752)
+LFM2_1_2B, LFM2_350M, LFM2_2_6B = _shape("lfm2-1.2b"), _shape("lfm2-350m"), _shape("lfm2-2.6b")
 
 # Serving workloads (through Engine: scheduler, prompt portions beside decoded tokens, sampling)
 WORKLOADS = {

@@ -54,9 +54,15 @@ def build_parser() -> argparse.ArgumentParser:
     e.add_argument("--max-batch", type=int, default=64, help="requests live at the same time")
     e.add_argument("--token-budget", type=int, default=2048, help="tokens per step at most")
     e.add_argument("--chunk", type=int, default=2048, help="longest prompt portion in a step")
-    e.add_argument("--random-weights", metavar="CONFIG.json", help="make a model folder with "
-                   "random weights from this config.json and run it")
+    e.add_argument("--random-weights", metavar="SHAPE|CONFIG.json", help="make a model folder "
+                   "with random weights and run it: the name of a shape (tiny-a, tiny-b, "
+                   "lfm2-350m, lfm2-1.2b, lfm2-2.6b) or a config.json; with --model the folder is "
+                   "written there")
     e.add_argument("--weight-seed", type=int, default=0, help="seed of --random-weights")
+    e.add_argument("--weight-std", type=float, default=0.02,
+                   help="--random-weights: matrices and tables are N(0, std) (default 0.02)")
+    e.add_argument("--norm-jitter", type=float, default=0.0,
+                   help="--random-weights: norm weights are 1 + N(0, jitter) (default 0: all 1)")
     g = ap.add_argument_group("LLM behavior")
     g.add_argument("-p", "--prompt", action="append", type=parse_ids, default=[],
                    help="prompt as token ids, comma or space separated; may be given several "
@@ -111,14 +117,24 @@ def main(argv=None) -> int:
     model_dir = args.model
     tmp = None
     if args.random_weights:
-        from .config import config_from_dict
+        from .config import SHAPES, config_from_dict, named_shape
         from .weights import write_random_model
-        cfg = config_from_dict(json.loads(Path(args.random_weights).read_text()))
+        spec = args.random_weights
+        if spec.strip().lower() in SHAPES:
+            raw = named_shape(spec)
+        elif Path(spec).is_file():
+            raw = json.loads(Path(spec).read_text())
+        else:
+            ap.error(f"--random-weights: {spec!r} is neither a file nor one of the shapes "
+                     f"{', '.join(sorted(SHAPES))}")
+        cfg = config_from_dict(raw)
         if not model_dir:
             tmp = tempfile.TemporaryDirectory(prefix="kappai_amd_model_")
             model_dir = tmp.name
-        write_random_model(model_dir, cfg, args.weight_seed)
-        print(f"wrote random weights (seed {args.weight_seed}) to {model_dir}", file=sys.stderr)
+        write_random_model(model_dir, cfg, args.weight_seed, std=args.weight_std,
+                           norm_jitter=args.norm_jitter)
+        print(f"wrote random weights (seed {args.weight_seed}, std {args.weight_std}, norm jitter "
+              f"{args.norm_jitter}) to {model_dir}", file=sys.stderr)
 
     engine = Engine(EngineConfig(
         model=model_dir, dtype=args.dtype, ctx_size=args.ctx_size, page_size=args.page_size,

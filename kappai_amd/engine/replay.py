@@ -8,7 +8,9 @@ src/test/test_hybrid.c:164-386).
 Input, one JSON object a line:
     {"step": 0, "entries": [{"id": "a", "tokens": [5, 17, 3], "want": [0, 2]}], "end": []}
 For a step in which something is wanted, ``<out>/<step>.f32`` holds the logits at the wanted
-places as little-endian float32 [wanted, vocab].  After every step a line ``done <step>``.
+places as little-endian float32 [wanted, vocab], and ``<out>/index.jsonl`` gets a line that says
+which rows these are: ``{"step": 0, "file": "0.f32", "vocab": V, "rows": [[id, position], ...]}``
+(the position of the token in its request).  After every step a line ``done <step>``.
 """
 from __future__ import annotations
 
@@ -45,21 +47,28 @@ class TraceReplayer:
         self.out_dir.mkdir(parents=True, exist_ok=True)
         self.live: Dict[str, RequestCache] = {}
         self.log = log or (lambda s: None)
+        self.index_path = self.out_dir / "index.jsonl"
+        self.index_path.write_text("")
 
     def run_step(self, obj: dict) -> Optional[np.ndarray]:
         step = obj["step"]
-        entries = []
+        entries, rows = [], []
         for e in obj.get("entries", []):
             rid = e["id"]
             if rid not in self.live:
                 self.live[rid] = self.cache.open(rid)
-            entries.append(StepEntry(self.live[rid], list(e["tokens"]), list(e.get("want", []))))
+            want = list(e.get("want", []))
+            rows += [[rid, self.live[rid].length + int(w)] for w in want]
+            entries.append(StepEntry(self.live[rid], list(e["tokens"]), want))
         result = None
         if entries:
             logits = self.runner.step(entries)
             if logits.shape[0] > 0:
                 result = logits.detach().to("cpu").numpy().astype("<f4", copy=False)
                 result.tofile(self.out_dir / f"{step}.f32")
+                with open(self.index_path, "a") as f:
+                    f.write(json.dumps({"step": step, "file": f"{step}.f32",
+                                        "vocab": int(result.shape[1]), "rows": rows}) + "\n")
         for rid in obj.get("end", []):
             if rid in self.live:
                 self.cache.close(self.live.pop(rid))

@@ -26,9 +26,24 @@ GPU_ARCH = "gfx950"
 HIPCC_FLAGS = ["-O3", "-std=c++17", f"--offload-arch={GPU_ARCH}", "-shared", "-fPIC",
                "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
                "-Wno-unused-command-line-argument", "-Wno-pass-failed"]
-LIBRARIES = ["elementwise", "gemm", "shortconv", "attention", "sampling", "engine"]
+LIBRARIES = ["elementwise", "gemm", "shortconv", "attention", "sampling", "engine", "engine_api"]
 # libraries made of more sources than the one of their own name
 EXTRA_SOURCES = {"engine": ["engine_parts"]}
+
+
+def _python_flags() -> List[str]:
+    """What a library that talks to the interpreter is compiled and linked with."""
+    import sysconfig
+    flags = [f"-I{sysconfig.get_paths()['include']}"]
+    libdir = sysconfig.get_config_var("LIBDIR")
+    if libdir:
+        flags.append(f"-L{libdir}")
+    version = sysconfig.get_config_var("LDVERSION") or sysconfig.get_python_version()
+    return flags + [f"-lpython{version}", "-ldl"]
+
+
+# flags of single libraries beside HIPCC_FLAGS: name -> function that returns them
+EXTRA_FLAGS = {"engine_api": _python_flags}
 # libraries compiled once per value of a constant: name -> (constant, values built ahead)
 VARIANT_LIBRARIES = {"attention_mfma": ("HEAD_DIM", [16, 32, 48, 64, 80, 128, 256])}
 
@@ -70,8 +85,12 @@ def _source_hash(name: str, defines=None, sources=None) -> str:
     for p in list(sources or _sources(name)) + sorted(CSRC.glob("*.h")):
         h.update(p.name.encode())
         h.update(p.read_bytes())
-    h.update(" ".join(HIPCC_FLAGS + _defines_flags(defines)).encode())
+    h.update(" ".join(HIPCC_FLAGS + _defines_flags(defines) + _extra_flags(name)).encode())
     return h.hexdigest()
+
+
+def _extra_flags(name: str) -> List[str]:
+    return EXTRA_FLAGS[name]() if name in EXTRA_FLAGS else []
 
 
 def _tree_build_dir() -> Path:
@@ -156,7 +175,7 @@ def compile_library(name: str, verbose: bool = True, defines=None, sources=None,
     so, tag = out_dir / f"{built}.so", out_dir / f"{built}.hash"
     tmp = out_dir / f".{built}.{os.getpid()}.{threading.get_ident()}.so"
     cmd = [_hipcc(), *HIPCC_FLAGS, *_defines_flags(defines), f"-I{CSRC}", *map(str, srcs), "-o",
-           str(tmp)]
+           str(tmp), *_extra_flags(name)]
     what = " + ".join(src.name for src in srcs) + (
         " (" + ", ".join(f"{k}={v}" for k, v in sorted(defines.items())) + ")" if defines else "")
     if verbose:

@@ -59,6 +59,24 @@ def test_feed_forward_width_when_keys_are_absent():
         assert again.ff_dim == want and again == cfg
 
 
+def test_named_shapes():
+    """The shapes that --random-weights and the benchmark know by name: the sizes of the
+    architecture's three published models and the two tiny configurations of the tests."""
+    from kappai_amd.config import SHAPES, named_shape
+    for name, ff, layers, attention in (
+            ("lfm2-1.2b", 8192, 16, [2, 5, 8, 10, 12, 14]),
+            ("lfm2-350m", 4608, 16, [2, 5, 8, 10, 12, 14]),
+            ("LFM2-2.6B", 7168, 30, [2, 6, 10, 14, 18, 21, 24, 27]),
+            ("tiny-a", 192, 4, [1, 3]), ("tiny-b", 320, 6, [0, 3, 4])):
+        cfg = config_from_dict(named_shape(name))
+        assert (cfg.ff_dim, cfg.num_hidden_layers, cfg.attention_layers) == (ff, layers, attention)
+    assert named_shape("tiny-a") == TINY_A and named_shape("tiny-b") == TINY_B
+    named_shape("tiny-a")["hidden_size"] = 1          # a copy: the table is not changed
+    assert SHAPES["tiny-a"]["hidden_size"] == 64
+    with pytest.raises(KeyError, match="known: lfm2-1.2b"):
+        named_shape("lfm2-7b")
+
+
 def test_lfm2_1_2b_shape():
     c = config_from_dict(copy.deepcopy(LFM2_1_2B))
     assert isinstance(c, Lfm2Config)

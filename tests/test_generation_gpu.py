@@ -313,6 +313,23 @@ def test_command_line(model_dirs, tmp_path):
         cwd=str(tmp_path), capture_output=True, text=True, timeout=300)
     assert out.returncode == 0, out.stderr
     assert len(out.stdout.split()) == 4
+    # random-weights mode from the name of a shape, with the weights' spread given: the folder is
+    # the one that the same call of the library writes (Tiny B: norm weights 1 + N(0, 0.1))
+    made = tmp_path / "made"
+    out = subprocess.run(
+        [sys.executable, str(ROOT / "bin" / "kappai-cli"), "--random-weights", "tiny-b",
+         "--model", str(made), "--weight-seed", "1", "--weight-std", "0.05", "--norm-jitter",
+         "0.1", "--dtype", "float32", "-n", "5", "-t", "0", "--num-pages", "16", "7 8 9 10"],
+        cwd=str(tmp_path), capture_output=True, text=True, timeout=300)
+    assert out.returncode == 0, out.stderr
+    same = write_tiny("B", tmp_path / "same")
+    assert (made / "model.safetensors").read_bytes() == (same / "model.safetensors").read_bytes()
+    want, _ = plain_generate(same, [7, 8, 9, 10], 5, lambda: S.PlainSampler(1, temperature=0.0))
+    assert [int(t) for t in out.stdout.split()] == want
+    out = subprocess.run(
+        [sys.executable, str(ROOT / "bin" / "kappai-cli"), "--random-weights", "lfm2-9b", "1 2"],
+        cwd=str(tmp_path), capture_output=True, text=True, timeout=300)
+    assert out.returncode == 2 and "neither a file nor one of the shapes" in out.stderr
 
 
 def test_command_line_times_by_stage(model_dirs):

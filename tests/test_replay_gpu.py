@@ -161,6 +161,12 @@ def test_trace_run_program(tmp_path, model_dirs, dtype):
     assert proc.wait(timeout=120) == 0
     got = collect(index, read_outputs(out, index, cfg["vocab_size"]), cfg["vocab_size"])
     assert_matches_plain(got, model_dirs["A"], requests, dtype)
+    # the index beside the files names the same rows: (request, position) in output order
+    lines = [json.loads(line) for line in (out / "index.jsonl").read_text().splitlines()]
+    assert [ln["step"] for ln in lines] == [s for s, idx in enumerate(index) if idx]
+    for ln in lines:
+        assert ln["file"] == f"{ln['step']}.f32" and ln["vocab"] == cfg["vocab_size"]
+        assert [tuple(r) for r in ln["rows"]] == index[ln["step"]]
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
