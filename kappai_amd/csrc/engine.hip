@@ -113,7 +113,18 @@ int split_k_large(int M, int N, int K) {
   return best;
 }
 
+// 65 to 128 rows: the kernel with 32 x 32 tiles gives a block 64 columns and takes K ranges that
+// are multiples of 256; as many ranges (a power of two, at most 8) that about 256 blocks stream
+// the matrix (in_proj of the 1.2B shape two, qkv four, out_proj and down eight: from a sweep)
+int split_k_rows32(int N, int K) {
+  const long col_blocks = (N + 63) / 64;
+  int split = 1;
+  while (split < 8 && K % (512 * split) == 0 && col_blocks * split * 2 <= 256) split *= 2;
+  return split;
+}
+
 int split_k_for(int M, int N, int K) {
+  if (M > 64 && M <= 128 && K % 256 == 0 && N % 16 == 0) return split_k_rows32(N, K);
   if (M > 64) return split_k_large(M, N, K);
   if (M > 16) {
     // the kernel that shares the rows through LDS: blocks of 64 columns, K ranges that are

@@ -13,6 +13,8 @@
 //                    waves split K and meet in LDS (v_mfma_f32_16x16x32_bf16).
 //   gemm_bf16_shared_rows  17 <= M <= 64 and a W with many rows: as above, but two waves that
 //                    stream different rows of W share the rows of A through LDS.
+//   gemm_bf16_rows32 65 <= M <= 128: the same idea with 32 x 32 tiles (v_mfma_f32_32x32x16_bf16),
+//                    W from its fragment-order copy.
 //   gemm_bf16_any    K or a row stride that is no multiple of 8: a plain kernel, so that no
 //                    width is refused.
 #include "common.h"
@@ -1509,6 +1511,234 @@ static bool launch_shared_rows(const bf16_t* A, const bf16_t* W, const float* bi
   return true;
 }
 
+// ---------------------------------------------------------------------------------------
+// 65 to 128 rows (short prompt portions, decode at large batches): 32 x 32 tiles, rows via LDS
+// ---------------------------------------------------------------------------------------
+// The block kernels above need hundreds of rows to fill their tiles, and the kernel for 17 to 64
+// rows reads every fragment of A once per 16 x 16 tile.  Here a block is 2 x 4 waves: wave
+// (wn, wk) owns 32 rows of W (one 32 x 32 tile of the result for each 32 rows of A,
+// v_mfma_f32_32x32x16_bf16: half the LDS reads per product of the 16 x 16 form) and, of every
+// run of 256 of the block's K range, the 64 number wk.  The block's rows of A go through LDS run
+// by run (global_load_lds, two buffers of rows x 256, rows of 128 bytes per 64 of K permuted as
+// in the block kernel: a fragment read is free of bank conflicts), W comes from its
+// fragment-order copy straight into registers, one run ahead: a load instruction takes the two
+// pieces of the wave's 32 rows, 256 bytes of each of two groups of 8 of K.  The waves meet in LDS
+// at the end to add their K parts in a fixed order.  K can be cut over blocks as well (float
+// partial sums), which is what fills the chip for the products with few rows of W.
+// Measured at the LFM2-1.2B shapes, W cold, 128 rows: gate/up 23.2 against 26.7 us (the 128 x 128
+// block form), in_proj 13.0 against 14.1, qkv 9.1 against 12.4, out_proj 7.4 against 8.0, down
+// 15.5 against 20.6.  A wave that owns 64 rows of W (half the reads of A from L2 and LDS) was
+// slower (29 us for gate/up), and so were 4 x 2 waves.
+//
+// Host side guarantees: W in fragment order, K / gridDim.y a multiple of 256, lda a multiple of
+// 8, M * lda < 2^31.  Rows of A past M repeat the last row, pieces of W past the end the last
+// piece (their products are not stored).
+#define R32_NWN 2
+#define R32_NWK 4
+template <typename TO, int MT, int EPI>
+__global__ __launch_bounds__(R32_NWN * R32_NWK * WAVE) void gemm_bf16_rows32_kernel(
+    const bf16_t* __restrict__ A, const bf16_t* __restrict__ Wf, const float* __restrict__ bias,
+    TO* __restrict__ C, int M, int n_rows_w, int K, int lda, int ldc) {
+  constexpr int NWN = R32_NWN, NWK = R32_NWK, NW = NWN * NWK, ROWS = 32 * MT, RUN = NWK * 64;
+  constexpr int BUF = ROWS * RUN;                       // bf16 elements a buffer
+  constexpr int INSTR = ROWS * NWK / 8;                 // load instructions a run (8 rows x 128 B)
+  constexpr int PER_WAVE = INSTR / NW;
+  static_assert(INSTR % NW == 0, "the loads of a run are dealt round the waves evenly");
+  extern __shared__ __attribute__((aligned(1024))) bf16_t lds[];
+  const int tid = threadIdx.x, lane = tid % WAVE;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / WAVE);
+  const int wn = wave / NWK, wk = wave % NWK;
+  const int r_in = lane % 32, hh = lane / 32;
+  const int kblk = K / (int)gridDim.y;
+  const int nruns = kblk / RUN;
+  const int kb0 = blockIdx.y * kblk;
+  C += (size_t)blockIdx.y * M * ldc;
+
+  // W: lane -> row wrow0 + r_in, the 8 of K number hh (+ 2 for the second 16) of a piece of 16
+  // rows x 32 of K; step s of a run (16 of K) lies in piece s / 2, half s % 2
+  const int wrow0 = (blockIdx.x * NWN + wn) * 32;
+  const int piece_row = min((wrow0 + r_in) / 16, n_rows_w / 16 - 1);
+  const bf16_t* wbase = Wf + ((size_t)piece_row * (K / 32) + (kb0 + wk * 64) / 32) * 512 +
+                        (hh * 16 + r_in % 16) * 8;
+  auto load_w = [&](u32x4_t (&wv)[4], int run) {
+    const bf16_t* p = wbase + (size_t)run * (RUN / 32) * 512;
+#pragma unroll
+    for (int s = 0; s < 4; ++s) wv[s] = load16(p + (s / 2) * 512 + (s % 2) * 256);
+  };
+
+  // A: instruction j of a run brings rows (j % (ROWS / 8)) * 8 + lane / 8 of the 64 number
+  // j / (ROWS / 8) of the run; in LDS: the four 64s one after the other, rows of 128 bytes
+  uint32_t aoff[PER_WAVE];
+#pragma unroll
+  for (int i = 0; i < PER_WAVE; ++i) {
+    const int j = i * NW + wave;
+    const int slice = j / (ROWS / 8), row = (j % (ROWS / 8)) * 8 + lane / 8;
+    const int chunk = (lane % 8) ^ ((row >> 1) & 7);
+    aoff[i] = (uint32_t)(min(row, M - 1) * lda + kb0 + slice * 64 + chunk * 8) *
+              (uint32_t)sizeof(bf16_t);
+  }
+  auto stage = [&](int buf, int run) {
+    const uint64_t p = reinterpret_cast<uint64_t>(A) + (uint64_t)run * (RUN * sizeof(bf16_t));
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)p);
+    const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(p >> 32));
+    const char* base = reinterpret_cast<const char*>(((uint64_t)hi << 32) | lo);
+#pragma unroll
+    for (int i = 0; i < PER_WAVE; ++i) {
+      const int j = i * NW + wave;
+      const int slice = j / (ROWS / 8), rowblk = j % (ROWS / 8);
+      __builtin_amdgcn_global_load_lds(
+          KAPPAI_GPTR(base + aoff[i]),
+          KAPPAI_LPTR(lds + buf * BUF + (slice * ROWS + rowblk * 8) * 64), 16, 0, 0);
+    }
+  };
+
+  f32x16_t acc[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc[t][v] = 0.f;
+  // fragment of A: lane -> row 32 t + r_in, chunk 2 s + hh of the wave's 64
+  int roff[4];
+#pragma unroll
+  for (int s = 0; s < 4; ++s)
+    roff[s] = (wk * ROWS + r_in) * 64 + (((2 * s + hh) ^ ((r_in >> 1) & 7)) * 8);
+  auto products = [&](const u32x4_t (&wv)[4], int buf) {
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      u32x4_t av[MT];
+#pragma unroll
+      for (int t = 0; t < MT; ++t)
+        av[t] = *reinterpret_cast<const u32x4_t*>(lds + buf * BUF + roff[s] + t * 32 * 64);
+#pragma unroll
+      for (int t = 0; t < MT; ++t)
+        acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(wv[s]), as_bf16x8(av[t]), acc[t],
+                                                         0, 0, 0);
+    }
+  };
+
+  // W one run ahead in two register sets used in turn, A one run ahead in the other LDS buffer.
+  // In every round the loads of A are issued before those of W, and loads come back in the order
+  // they were issued: waiting until only the last round's four loads of W are out means that the
+  // run of A issued before them has landed (and the run of W before that).
+  u32x4_t wv[2][4];
+  stage(0, 0);
+  load_w(wv[0], 0);
+  for (int c = 0; c < nruns; c += 2) {
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+      const int cc = c + s;
+      if (cc >= nruns) break;
+      // run cc of A was issued before the four loads of run cc of W, which may stay out
+      __builtin_amdgcn_s_waitcnt(0x0F70 | 4);       // vmcnt(4)
+      // everybody's part of run cc is there and nobody reads the other buffer any more (a bare
+      // barrier: a fence would wait for the loads of W that are meant to stay in flight)
+      __builtin_amdgcn_s_barrier();
+      SCHED_FENCE();
+      if (cc + 1 < nruns) {
+        stage((s + 1) & 1, cc + 1);
+        load_w(wv[(s + 1) & 1], cc + 1);
+      }
+      products(wv[s], s & 1);
+    }
+  }
+  // the K parts meet: wave (wn, wk) adds up and stores row tiles wk, wk + 4, ...
+  // acc[t][v] is C[row 32 t + r_in][column wrow0 + 8 (v / 4) + 4 hh + v % 4]
+  __syncthreads();
+  float* red = reinterpret_cast<float*>(lds);
+  constexpr int RSTRIDE = MT * 16 * WAVE;               // floats a wave
+#pragma unroll
+  for (int t = 0; t < MT; ++t)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) red[wave * RSTRIDE + (t * 16 + v) * WAVE + lane] = acc[t][v];
+  __syncthreads();
+  for (int t = wk; t < MT; t += NWK) {
+    float sum[16];
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      sum[v] = red[(wn * NWK) * RSTRIDE + (t * 16 + v) * WAVE + lane];
+#pragma unroll
+      for (int w = 1; w < NWK; ++w)
+        sum[v] += red[(wn * NWK + w) * RSTRIDE + (t * 16 + v) * WAVE + lane];
+    }
+    const int gm = 32 * t + r_in;
+    if (gm >= M) continue;
+    if (EPI == 1) {
+      // rows 0..15 of the wave's W are gate rows, 16..31 the up rows of the same 16 columns:
+      // registers v and v + 8 of a lane
+      if (wrow0 + 16 < n_rows_w) {
+#pragma unroll
+        for (int g = 0; g < 2; ++g) {
+          uint2 pk;
+          pk.x = pack_bf16x2(silu_f(sum[4 * g]) * sum[4 * g + 8],
+                             silu_f(sum[4 * g + 1]) * sum[4 * g + 9]);
+          pk.y = pack_bf16x2(silu_f(sum[4 * g + 2]) * sum[4 * g + 10],
+                             silu_f(sum[4 * g + 3]) * sum[4 * g + 11]);
+          if constexpr (sizeof(TO) == 2)
+            *reinterpret_cast<uint2*>(C + (size_t)gm * ldc + wrow0 / 2 + 8 * g + 4 * hh) = pk;
+        }
+      }
+    } else {
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int gn = wrow0 + 8 * g + 4 * hh;
+        if (gn >= n_rows_w) continue;
+        float o[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          o[e] = sum[4 * g + e] + ((bias && blockIdx.y == 0) ? bias[gn + e] : 0.f);
+        TO* dst = C + (size_t)gm * ldc + gn;
+        if constexpr (sizeof(TO) == 2) {
+          uint2 pk;
+          pk.x = pack_bf16x2(o[0], o[1]);
+          pk.y = pack_bf16x2(o[2], o[3]);
+          *reinterpret_cast<uint2*>(dst) = pk;
+        } else {
+          *reinterpret_cast<float4*>(dst) = make_float4(o[0], o[1], o[2], o[3]);
+        }
+      }
+    }
+  }
+}
+
+template <typename TO, int MT, int EPI>
+static void launch_rows32_cfg(const bf16_t* A, const bf16_t* Wf, const float* bias, TO* C, int M,
+                              int n_rows_w, int K, int lda, int ldc, int ksplit,
+                              hipStream_t stream) {
+  constexpr int NW = R32_NWN * R32_NWK, ROWS = 32 * MT, RUN = R32_NWK * 64;
+  constexpr size_t stage_bytes = 2 * (size_t)ROWS * RUN * sizeof(bf16_t);
+  constexpr size_t red_bytes = (size_t)NW * MT * 16 * WAVE * sizeof(float);
+  constexpr size_t lds_bytes = stage_bytes > red_bytes ? stage_bytes : red_bytes;
+  static_assert(lds_bytes <= 160 * 1024, "a block's LDS");
+  auto kern = gemm_bf16_rows32_kernel<TO, MT, EPI>;
+  static bool attr_set = false;       // more than 64 KB of LDS has to be asked for once
+  if (!attr_set) {
+    (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
+                              (int)lds_bytes);
+    attr_set = true;
+  }
+  hipLaunchKernelGGL(kern, dim3((n_rows_w + 32 * R32_NWN - 1) / (32 * R32_NWN), ksplit),
+                     dim3(NW * WAVE), lds_bytes, stream, A, Wf, bias, C, M, n_rows_w, K, lda, ldc);
+}
+
+// Returns false when the shape does not fit (the caller then takes a block kernel).  The output
+// must allow the kernel's stores of four values (8 or 16 bytes).
+template <typename TO, int EPI>
+static bool launch_rows32(const bf16_t* A, const bf16_t* Wf, const float* bias, TO* C, int M,
+                          int n_rows_w, int K, int lda, int ldc, int ksplit, hipStream_t stream) {
+  const int out_cols = EPI == 1 ? n_rows_w / 2 : n_rows_w;
+  if (Wf == nullptr || M < 1 || M > 128 || ksplit < 1 || K % (ksplit * R32_NWK * 64) ||
+      n_rows_w % (EPI == 1 ? 32 : 16) || (lda % 8) || (long)M * lda >= (1L << 31) - 2048 ||
+      (out_cols % 4) || (ldc % 4) || ((uintptr_t)C % 16) || (EPI == 1 && sizeof(TO) != 2))
+    return false;
+  switch ((M + 31) / 32) {
+    case 1: launch_rows32_cfg<TO, 1, EPI>(A, Wf, bias, C, M, n_rows_w, K, lda, ldc, ksplit, stream); break;
+    case 2: launch_rows32_cfg<TO, 2, EPI>(A, Wf, bias, C, M, n_rows_w, K, lda, ldc, ksplit, stream); break;
+    case 3: launch_rows32_cfg<TO, 3, EPI>(A, Wf, bias, C, M, n_rows_w, K, lda, ldc, ksplit, stream); break;
+    default: launch_rows32_cfg<TO, 4, EPI>(A, Wf, bias, C, M, n_rows_w, K, lda, ldc, ksplit, stream); break;
+  }
+  return true;
+}
+
 template <typename TO, int EPI>
 static int launch_bf16(const bf16_t* A, const bf16_t* W, const float* bias, TO* C, int M, int N,
                        int K, int lda, int ldc, int force_kernel, int ksplit, hipStream_t stream,
@@ -1547,6 +1777,18 @@ static int launch_bf16(const bf16_t* A, const bf16_t* W, const float* bias, TO* 
   } else if (force_kernel == 9) {
     return (int)hipErrorInvalidValue;
   }
+  // 65 to 128 rows: 32 x 32 tiles with the rows through LDS, when W is there in fragment order
+  if constexpr (EPI != 2) {
+    if (force_kernel == 12 || (force_kernel == 0 && M > 64 && M <= 128 && Wf != nullptr &&
+                               !wide_head)) {
+      if (launch_rows32<TO, EPI>(A, Wf, bias, C, M, EPI == 1 ? 2 * N : N, K, lda, ldc, ksplit,
+                                 stream))
+        KAPPAI_RETURN_LAUNCH_STATUS();
+      if (force_kernel == 12) return (int)hipErrorInvalidValue;
+    }
+  } else if (force_kernel == 12) {
+    return (int)hipErrorInvalidValue;
+  }
   if (M <= 64 && force_kernel != 1 && force_kernel < 3 && !wide_head) {
     const int mt = (M + 15) / 16;
     switch (mt) {
@@ -1579,7 +1821,8 @@ static int launch_bf16(const bf16_t* A, const bf16_t* W, const float* bias, TO* 
 // K, lda must be multiples of 8 and A, W 16-byte aligned (checked by the caller).
 // force_kernel: 0 = by M, 1 = tile kernel, 2 = skinny kernel (M <= 64 only), 3..8 = tile kernel
 // with block shape 1..6 (see launch_tile), 9 = shared-rows kernel (17 to 64 rows, K / ksplit a
-// multiple of 512), 10 = block shape 8, 11 = block shape 9; for tests and tuning.
+// multiple of 512), 10 = block shape 8, 11 = block shape 9, 12 = the kernel for 65 to 128 rows
+// (1 to 128 rows, W in fragment order, K / ksplit a multiple of 256); for tests and tuning.
 // ksplit > 1 (float output only): C is [ksplit][M][ldc] partial sums over K ranges.
 // W_frag: null, or W in fragment order (K a multiple of 32, rows a multiple of 16); W may then
 // be null: every kernel reads the fragment order (only kappai_gemm_bf16_any needs rows).

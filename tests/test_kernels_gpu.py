@@ -263,6 +263,79 @@ def test_linear_shared_rows_split_k(ops, M, N, K, S):
     close(parts.sum(0), x.double() @ w.double().T + b.double(), 2e-5, "sum of the partial sums")
 
 
+ROWS32 = 12           # force_kernel: 65 to 128 rows (it takes 1 to 128), 32 x 32 tiles, rows via LDS
+
+
+@pytest.mark.parametrize("M", [1, 31, 65, 96, 97, 128])
+@pytest.mark.parametrize("N,K", [(64, 256), (208, 1024), (2048, 2048), (8208, 1536)])
+@pytest.mark.parametrize("out_dtype", [F32, BF16])
+def test_linear_rows32(ops, M, N, K, out_dtype):
+    """The kernel for 65 to 128 rows: every row-tile count, matrices that end inside a block's 64
+    columns or inside a wave's 32 (208 = 6 tiles and a half), one and several runs of K, a row
+    stride, bias; the matrix in fragment order only, and beside its rows."""
+    wide = rand((M, K + 8), BF16, 151)
+    x, w, b = wide[:, :K], rand((N, K), BF16, 152), rand((N,), F32, 153)
+    want = x.double() @ w.double().T
+    tol = 2e-5 if out_dtype == F32 else BF16_ULP
+    xd, wd = wide.to(DEV)[:, :K], w.to(DEV)
+    kept = ops.InFragments.of(wd)
+    got = ops.linear(xd, kept, out_dtype=out_dtype, force_kernel=ROWS32)
+    close(got.float(), want, tol, "rows32")
+    got = ops.linear(xd, wd, b.to(DEV), out_dtype=out_dtype, force_kernel=ROWS32,
+                     weight_frag=ops.fragment_order(wd))
+    close(got.float(), want + b.double(), tol, "rows32 with bias")
+
+
+@pytest.mark.parametrize("M,F,K", [(65, 48, 256), (100, 1008, 1024), (128, 8192, 2048)])
+def test_linear_swiglu_rows32(ops, M, F, K):
+    x, wg, wu = rand((M, K), BF16, 154), rand((F, K), BF16, 155, 0.2), rand((F, K), BF16, 156, 0.2)
+    w = ops.InFragments.of(ops.interleave_gate_up(wg.to(DEV), wu.to(DEV)))
+    g, u = x.double() @ wg.double().T, x.double() @ wu.double().T
+    want = g / (1 + torch.exp(-g)) * u
+    got = ops.linear_swiglu(x.to(DEV), w, force_kernel=ROWS32)
+    close(got.float(), want, BF16_ULP, "rows32")
+    if M > 64:          # and it is what such a step takes by itself: the same bits
+        assert torch.equal(ops.linear_swiglu(x.to(DEV), w), got)
+
+
+@pytest.mark.parametrize("M,N,K,S", [(128, 2048, 8192, 8), (70, 112, 3072, 3), (99, 2048, 2048, 2),
+                                     (128, 6144, 2048, 1)])
+def test_linear_rows32_split_k(ops, M, N, K, S):
+    x, w, b = rand((M, K), BF16, 157), rand((N, K), BF16, 158, 0.05), rand((N,), F32, 159)
+    kept = ops.InFragments.of(w.to(DEV))
+    parts = ops.linear(x.to(DEV), kept, b.to(DEV), partial_sums=True, split_k=S,
+                       force_kernel=ROWS32)
+    want = x.double() @ w.double().T + b.double()
+    if S == 1:
+        assert parts.shape == (M, N)
+        close(parts.float(), want, BF16_ULP, "one range")
+        return
+    assert parts.shape == (S, M, N) and parts.dtype == F32
+    close(parts.sum(0), want, 2e-5, "sum of the partial sums")
+
+
+def test_linear_rows32_is_what_steps_of_65_to_128_rows_take(ops):
+    """Without a kernel asked for, a product of 65 to 128 rows over a matrix in fragment order is
+    this kernel's (bit for bit), with the K ranges that the rule gives it; a matrix kept as rows
+    only, or a K that is no multiple of 256, goes to the block kernels as before."""
+    x, w = rand((100, 2048), BF16, 160).to(DEV), rand((3072, 2048), BF16, 161, 0.05).to(DEV)
+    kept = ops.InFragments.of(w)
+    assert torch.equal(ops.linear(x, kept), ops.linear(x, kept, force_kernel=ROWS32))
+    assert ops.split_k_for(100, 3072, 2048) == 4 and ops.split_k_for(100, 6144, 2048) == 2
+    assert ops.split_k_for(128, 2048, 8192) == 8 and ops.split_k_for(65, 16384, 2048) == 1
+    parts = ops.linear(x, kept, partial_sums=True)
+    assert parts.shape == (4, 100, 3072)
+    assert torch.equal(parts, ops.linear(x, kept, partial_sums=True, force_kernel=ROWS32))
+    close(ops.linear(x, w).float(), x.double().cpu() @ w.double().cpu().T, BF16_ULP, "rows only")
+    with pytest.raises(RuntimeError):
+        ops.linear(x, w, force_kernel=ROWS32)                 # no fragment order
+    x3, w3 = x[:, :1920].contiguous(), ops.InFragments.of(w[:, :1920].contiguous())
+    with pytest.raises(RuntimeError):
+        ops.linear(x3, w3, force_kernel=ROWS32)               # 1920 is no multiple of 256
+    close(ops.linear(x3, w3).float(), x3.double().cpu() @ w[:, :1920].double().cpu().T, BF16_ULP,
+          "K = 1920")
+
+
 def test_linear_shared_rows_refuses_what_does_not_fit(ops):
     x, w = rand((32, 520), BF16, 60).to(DEV), rand((64, 520), BF16, 61).to(DEV)
     with pytest.raises(RuntimeError):
@@ -365,6 +438,14 @@ def test_products_read_a_matrix_kept_in_fragment_order_only(ops, M, N, K):
         forces += [3, 4, 5, 6] + ([BLOCK256, BLOCK128, BLOCK128_DEEP, BLOCK192] if K % 128 == 0 else [])
     elif M > 16 and K % 512 == 0:
         forces += [SHARED_ROWS]
+    if 64 < M <= 128 and K % 256 == 0:
+        # the kernel for 65 to 128 rows exists for the fragment order only: left to itself the
+        # product over the kept matrix is that kernel's, over the rows a block kernel's; the two
+        # add in another order, so they agree to rounding, not bit for bit
+        forces.remove(0)
+        close(ops.linear(x, kept, b, out_dtype=F32).float(),
+              ops.linear(x, w, b, out_dtype=F32).double(), 2e-5, "another kernel for the kept matrix")
+        assert torch.equal(ops.linear(x, kept, b), ops.linear(x, kept, b, force_kernel=ROWS32))
     for force in forces:
         for bias in (None, b):
             for out_dtype in (BF16, F32):
@@ -380,7 +461,11 @@ def test_products_read_a_matrix_kept_in_fragment_order_only(ops, M, N, K):
     # the first rows of the matrix by themselves (the q rows of a stacked q, k, v)
     if N >= 32:
         first = (N // 32) * 16
-        assert torch.equal(ops.linear(x, kept.rows(first)), ops.linear(x, w[:first].contiguous()))
+        got, want = ops.linear(x, kept.rows(first)), ops.linear(x, w[:first].contiguous())
+        if 64 < M <= 128 and K % 256 == 0:     # (two kernels, as above)
+            close(got.float(), want.double(), BF16_ULP, "the first rows")
+        else:
+            assert torch.equal(got, want)
     # rows of it as an embedding table
     ids = torch.tensor([0, N - 1, N // 2, 17 % N, 16 % N], dtype=torch.int32, device=DEV)
     assert torch.equal(ops.embed_rows(ids, kept), ops.embed_rows(ids, w))
