@@ -10,6 +10,7 @@
 // kappai: an operation list run through a table of handlers that each operation registered
 // (src/recipe.h:577-580, src/recipe/exec.c:467-517); order of a step src/recipe/exec.c:704-758.
 #include "engine.h"
+#include "gemm_rules.h"
 
 #include <stdio.h>
 #include <string.h>
@@ -113,18 +114,24 @@ int split_k_large(int M, int N, int K) {
   return best;
 }
 
-// 65 to 128 rows: the kernel with 32 x 32 tiles gives a block 64 columns and takes K ranges that
-// are multiples of 256; as many ranges (a power of two, at most 8) that about 256 blocks stream
-// the matrix (in_proj of the 1.2B shape two, qkv four, out_proj and down eight: from a sweep)
+// 25 to 128 rows: the kernel with 32 x 32 tiles gives a block 64 columns and takes K ranges that
+// are multiples of 256; as many equal ranges (at most 8: the norm's row kernel adds up to eight
+// planes, more take its slower form, 13 against 5 us) that up to 256 blocks stream the matrix
+// (from sweeps at the 1.2B and 350M shapes: in_proj two and four, qkv four, out_proj eight and
+// four, down eight and six; twice as many blocks were 5 to 40 % slower)
 int split_k_rows32(int N, int K) {
   const long col_blocks = (N + 63) / 64;
+  const int runs = K / KAPPAI_ROWS32_RUN;
   int split = 1;
-  while (split < 8 && K % (512 * split) == 0 && col_blocks * split * 2 <= 256) split *= 2;
+  for (int d = 2; d <= 8 && d <= runs; ++d)
+    if (runs % d == 0 && col_blocks * d <= 256) split = d;
   return split;
 }
 
 int split_k_for(int M, int N, int K) {
-  if (M > 64 && M <= 128 && K % 256 == 0 && N % 16 == 0) return split_k_rows32(N, K);
+  if (M > KAPPAI_ROWS32_MIN_ROWS && M <= KAPPAI_ROWS32_MAX_ROWS && K % KAPPAI_ROWS32_RUN == 0 &&
+      N % 16 == 0)
+    return split_k_rows32(N, K);
   if (M > 64) return split_k_large(M, N, K);
   if (M > 16) {
     // the kernel that shares the rows through LDS: blocks of 64 columns, K ranges that are

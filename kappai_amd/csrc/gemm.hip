@@ -13,11 +13,12 @@
 //                    waves split K and meet in LDS (v_mfma_f32_16x16x32_bf16).
 //   gemm_bf16_shared_rows  17 <= M <= 64 and a W with many rows: as above, but two waves that
 //                    stream different rows of W share the rows of A through LDS.
-//   gemm_bf16_rows32 65 <= M <= 128: the same idea with 32 x 32 tiles (v_mfma_f32_32x32x16_bf16),
+//   gemm_bf16_rows32 25 <= M <= 128: the same idea with 32 x 32 tiles (v_mfma_f32_32x32x16_bf16),
 //                    W from its fragment-order copy.
 //   gemm_bf16_any    K or a row stride that is no multiple of 8: a plain kernel, so that no
 //                    width is refused.
 #include "common.h"
+#include "gemm_rules.h"
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
 typedef __attribute__((ext_vector_type(4))) float f32x4_t;
@@ -731,7 +732,8 @@ static void launch_tile(const bf16_t* A, const bf16_t* W, const float* bias, TO*
     // with four LDS buffers (0.46 against 0.62-0.87 us per 64 of K; its start costs 2 us more)
     const long blocks128 = (long)((M + 127) / 128) * ((n_rows_w + 127) / 128) * ksplit;
     const bool deep = blocks128 <= 256 && K / ksplit >= 2048;
-    shape = !fits ? (big >= 128 ? 3 : 1) : use_256_form(blocks256) ? 5 : deep ? 8 : 6;
+    // (up to 128 rows a block of 256 rows would be half empty)
+    shape = !fits ? (big >= 128 ? 3 : 1) : (M > 128 && use_256_form(blocks256)) ? 5 : deep ? 8 : 6;
     if (shape == 5 && EPI == 0) {
       // blocks of 256 rows x 192 columns when they fill their rounds and come to fewer rounds'
       // worth of work than 256 x 256 (in_proj of 2048 rows: 192 blocks of 256 x 256 leave 64 CUs
@@ -1512,10 +1514,12 @@ static bool launch_shared_rows(const bf16_t* A, const bf16_t* W, const float* bi
 }
 
 // ---------------------------------------------------------------------------------------
-// 65 to 128 rows (short prompt portions, decode at large batches): 32 x 32 tiles, rows via LDS
+// 25 to 128 rows (decode at batches of that size, short prompt portions): 32 x 32 tiles, rows
+// via LDS
 // ---------------------------------------------------------------------------------------
 // The block kernels above need hundreds of rows to fill their tiles, and the kernel for 17 to 64
-// rows reads every fragment of A once per 16 x 16 tile.  Here a block is 2 x 4 waves: wave
+// rows reads every fragment of A once per 16 x 16 tile (it still runs where this one does not
+// fit: a matrix kept as rows, a K range that is no multiple of 256).  Here a block is 2 x 4 waves: wave
 // (wn, wk) owns 32 rows of W (one 32 x 32 tile of the result for each 32 rows of A,
 // v_mfma_f32_32x32x16_bf16: half the LDS reads per product of the 16 x 16 form) and, of every
 // run of 256 of the block's K range, the 64 number wk.  The block's rows of A go through LDS run
@@ -1527,14 +1531,16 @@ static bool launch_shared_rows(const bf16_t* A, const bf16_t* W, const float* bi
 // partial sums), which is what fills the chip for the products with few rows of W.
 // Measured at the LFM2-1.2B shapes, W cold, 128 rows: gate/up 23.2 against 26.7 us (the 128 x 128
 // block form), in_proj 13.0 against 14.1, qkv 9.1 against 12.4, out_proj 7.4 against 8.0, down
-// 15.5 against 20.6.  A wave that owns 64 rows of W (half the reads of A from L2 and LDS) was
-// slower (29 us for gate/up), and so were 4 x 2 waves.
+// 15.5 against 20.6; 64 rows against the kernel for 17 to 64 rows: gate/up 18.4 against 20.5, qkv
+// 7.0 against 10.7, in_proj 10.0 against 11.0.  A wave that owns 64 rows of W (half the reads of A
+// from L2 and LDS) was slower (29 us for gate/up at 128 rows), and so were 4 x 2 waves.
 //
 // Host side guarantees: W in fragment order, K / gridDim.y a multiple of 256, lda a multiple of
 // 8, M * lda < 2^31.  Rows of A past M repeat the last row, pieces of W past the end the last
 // piece (their products are not stored).
 #define R32_NWN 2
 #define R32_NWK 4
+static_assert(R32_NWK * 64 == KAPPAI_ROWS32_RUN, "the rule for K ranges counts in runs");
 template <typename TO, int MT, int EPI>
 __global__ __launch_bounds__(R32_NWN * R32_NWK * WAVE) void gemm_bf16_rows32_kernel(
     const bf16_t* __restrict__ A, const bf16_t* __restrict__ Wf, const float* __restrict__ bias,
@@ -1726,7 +1732,7 @@ template <typename TO, int EPI>
 static bool launch_rows32(const bf16_t* A, const bf16_t* Wf, const float* bias, TO* C, int M,
                           int n_rows_w, int K, int lda, int ldc, int ksplit, hipStream_t stream) {
   const int out_cols = EPI == 1 ? n_rows_w / 2 : n_rows_w;
-  if (Wf == nullptr || M < 1 || M > 128 || ksplit < 1 || K % (ksplit * R32_NWK * 64) ||
+  if (Wf == nullptr || M < 1 || M > KAPPAI_ROWS32_MAX_ROWS || ksplit < 1 || K % (ksplit * R32_NWK * 64) ||
       n_rows_w % (EPI == 1 ? 32 : 16) || (lda % 8) || (long)M * lda >= (1L << 31) - 2048 ||
       (out_cols % 4) || (ldc % 4) || ((uintptr_t)C % 16) || (EPI == 1 && sizeof(TO) != 2))
     return false;
@@ -1762,6 +1768,20 @@ static int launch_bf16(const bf16_t* A, const bf16_t* W, const float* bias, TO* 
   // the 128 x 128 blocks than through the decode kernel, which reads the rows once per 32 columns
   const bool wide_head = EPI == 0 && M > 32 && N >= 16384 && force_kernel == 0 && ksplit == 1 &&
                          block256_fits<TO, EPI>(A, W, C, M, N, K, lda, ldc, ksplit);
+  // 25 to 128 rows: 32 x 32 tiles with the rows through LDS, when W is there in fragment order
+  // and the shape fits (else the kernels below)
+  if constexpr (EPI != 2) {
+    if (force_kernel == 12 || (force_kernel == 0 && M > KAPPAI_ROWS32_MIN_ROWS &&
+                               M <= KAPPAI_ROWS32_MAX_ROWS &&
+                               Wf != nullptr && !wide_head)) {
+      if (launch_rows32<TO, EPI>(A, Wf, bias, C, M, EPI == 1 ? 2 * N : N, K, lda, ldc, ksplit,
+                                 stream))
+        KAPPAI_RETURN_LAUNCH_STATUS();
+      if (force_kernel == 12) return (int)hipErrorInvalidValue;
+    }
+  } else if (force_kernel == 12) {
+    return (int)hipErrorInvalidValue;
+  }
   // 17 to 64 rows and blocks enough to fill half the chip: the rows go through LDS
   if constexpr (EPI != 2) {
     const int n_rows_w = EPI == 1 ? 2 * N : N;
@@ -1769,24 +1789,12 @@ static int launch_bf16(const bf16_t* A, const bf16_t* W, const float* bias, TO* 
     // (with W in fragment order the kernel for few rows keeps up to 24 rows: gate/up 16.6
     // against 17.5 us at 24 rows, 15.7 against 17.6 at 17)
     if (force_kernel == 9 ||
-        (force_kernel == 0 && M > (Wf ? 24 : 16) && M <= 64 && sr_blocks >= 128)) {
+        (force_kernel == 0 && M > (Wf ? 24 : 16) && M <= 64 && sr_blocks >= 128 && !wide_head)) {
       if (launch_shared_rows<TO, EPI>(A, W, bias, C, M, n_rows_w, K, lda, ldc, ksplit, stream, Wf))
         KAPPAI_RETURN_LAUNCH_STATUS();
       if (force_kernel == 9) return (int)hipErrorInvalidValue;
     }
   } else if (force_kernel == 9) {
-    return (int)hipErrorInvalidValue;
-  }
-  // 65 to 128 rows: 32 x 32 tiles with the rows through LDS, when W is there in fragment order
-  if constexpr (EPI != 2) {
-    if (force_kernel == 12 || (force_kernel == 0 && M > 64 && M <= 128 && Wf != nullptr &&
-                               !wide_head)) {
-      if (launch_rows32<TO, EPI>(A, Wf, bias, C, M, EPI == 1 ? 2 * N : N, K, lda, ldc, ksplit,
-                                 stream))
-        KAPPAI_RETURN_LAUNCH_STATUS();
-      if (force_kernel == 12) return (int)hipErrorInvalidValue;
-    }
-  } else if (force_kernel == 12) {
     return (int)hipErrorInvalidValue;
   }
   if (M <= 64 && force_kernel != 1 && force_kernel < 3 && !wide_head) {
@@ -1821,7 +1829,7 @@ static int launch_bf16(const bf16_t* A, const bf16_t* W, const float* bias, TO* 
 // K, lda must be multiples of 8 and A, W 16-byte aligned (checked by the caller).
 // force_kernel: 0 = by M, 1 = tile kernel, 2 = skinny kernel (M <= 64 only), 3..8 = tile kernel
 // with block shape 1..6 (see launch_tile), 9 = shared-rows kernel (17 to 64 rows, K / ksplit a
-// multiple of 512), 10 = block shape 8, 11 = block shape 9, 12 = the kernel for 65 to 128 rows
+// multiple of 512), 10 = block shape 8, 11 = block shape 9, 12 = the kernel for 25 to 128 rows
 // (1 to 128 rows, W in fragment order, K / ksplit a multiple of 256); for tests and tuning.
 // ksplit > 1 (float output only): C is [ksplit][M][ldc] partial sums over K ranges.
 // W_frag: null, or W in fragment order (K a multiple of 32, rows a multiple of 16); W may then
