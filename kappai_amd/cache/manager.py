@@ -17,6 +17,7 @@ from __future__ import annotations
 from dataclasses import dataclass, field
 from typing import Dict, Hashable, List, Optional, Sequence, Union
 
+import numpy as np
 import torch
 
 from .specs import FixedState, PagedSpec
@@ -135,6 +136,17 @@ class RequestCache:
         self.blocks: List[List[int]] = [[] for _ in range(n_paged_groups)]  # -1 = given back
         self.closed = False
         self.version = 0        # counts changes of `blocks`, for callers that mirror them
+        self._arrays = [(-1, None)] * n_paged_groups      # (version, blocks[g] as int32 array)
+
+    def block_array(self, group: int):
+        """``blocks[group]`` as an int32 array, made anew only when the list has changed (a page
+        is taken every ``page_size`` tokens, so the step function copies the same array into its
+        tables for many steps in a row)."""
+        version, array = self._arrays[group]
+        if version != self.version:
+            array = np.asarray(self.blocks[group], dtype=np.int32)
+            self._arrays[group] = (self.version, array)
+        return array
 
     def __repr__(self):
         return f"RequestCache({self.request_id!r}, slot={self.slot}, length={self.length})"
@@ -421,6 +433,7 @@ class CacheManager:
                 if page >= 0:
                     g.allocator.give_back(page, rc.request_id)
             rc.blocks[gi] = []
+        rc.version += 1
         self._free_slots.append(rc.slot)
         del self._live[rc.request_id]
         rc.closed = True
@@ -436,6 +449,9 @@ class CacheManager:
             g.allocator.check()
             seen = {}
             for rc in self._live.values():
+                if rc.block_array(gi).tolist() != rc.blocks[gi]:
+                    raise CacheError(f"{rc.request_id!r}: the array form of its block table of "
+                                     f"group {gi} is out of date")
                 for page in rc.blocks[gi]:
                     if page < 0:
                         continue

@@ -152,8 +152,8 @@ def layout_rows(entries: Sequence[StepEntry], cache: CacheManager, vocab_size: i
         width = max(1, max(len(e.cache.blocks[gi]) for e in entries))
         bt = np.full((S, width), -1, dtype=np.int32)
         for si, e in enumerate(entries):
-            b = e.cache.blocks[gi]
-            bt[si, :len(b)] = b
+            b = e.cache.block_array(gi)      # (kept by the request until its pages change)
+            bt[si, :b.size] = b
         arrays[f"block_table_{gi}"] = bt
     sizes = {
         "n_rows": T, "n_segments": S, "n_logit_rows": len(logit_rows),

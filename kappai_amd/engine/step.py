@@ -165,9 +165,9 @@ class _DecodeGraph:
             if seen is None or seen[0] is not rc or seen[1] != rc.version:
                 for g in range(len(rc.blocks)):
                     row = h[f"block_table_{g}"][si]
-                    b = rc.blocks[g]
-                    row[:len(b)] = b
-                    row[len(b):] = -1
+                    b = rc.block_array(g)
+                    row[:b.size] = b
+                    row[b.size:] = -1
                 self.rows_of[si] = (rc, rc.version)
         for si in range(n, self.B):
             if self.rows_of[si] is not None:
