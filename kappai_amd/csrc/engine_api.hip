@@ -15,6 +15,7 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include <mutex>
 #include <string>
 #include <vector>
 
@@ -82,6 +83,8 @@ std::string package_root() {
 // Starts an interpreter if the process has none.  After this, every entry takes the lock with
 // PyGILState_Ensure whoever owns the interpreter.
 bool interpreter_ready() {
+  static std::mutex starting;        // two first calls at once start one interpreter
+  std::lock_guard<std::mutex> guard(starting);
   if (Py_IsInitialized()) return true;
   Py_InitializeEx(0);
   if (!Py_IsInitialized()) {
@@ -140,6 +143,16 @@ long call_long(kappai_engine* engine, const char* method, const char* format, ..
     return -1;
   }
   return value;
+}
+
+// An engine that kappai_engine_create returned, in a process whose interpreter still runs (the
+// lock must not be asked for without one).
+bool engine_ok(const kappai_engine* engine) {
+  if (engine == nullptr || engine->session == nullptr || !Py_IsInitialized()) {
+    set_error("kappai_engine: no engine");
+    return false;
+  }
+  return true;
 }
 
 bool sampling_ok(const kappai_sampling* s) {
@@ -238,6 +251,7 @@ extern "C" int kappai_engine_add_request(kappai_engine* engine, const int* ids, 
     set_error("kappai_engine_add_request: a prompt needs at least one token");
     return -1;
   }
+  if (!engine_ok(engine)) return -1;
   Locked lock;
   return (int)call_long(engine, "add_request", "(KififffiKi)", (unsigned long long)(uintptr_t)ids,
                         n, (double)s->temperature, s->top_k, (double)s->top_p, (double)s->min_p,
@@ -247,12 +261,14 @@ extern "C" int kappai_engine_add_request(kappai_engine* engine, const int* ids, 
 
 extern "C" int kappai_engine_abort(kappai_engine* engine, int request_id) {
   g_error[0] = 0;
+  if (!engine_ok(engine)) return -1;
   Locked lock;
   return (int)call_long(engine, "abort", "(i)", request_id);
 }
 
 extern "C" int kappai_engine_has_work(kappai_engine* engine) {
   g_error[0] = 0;
+  if (!engine_ok(engine)) return -1;
   Locked lock;
   return (int)call_long(engine, "has_work", "()");
 }
@@ -264,6 +280,7 @@ extern "C" int kappai_engine_step(kappai_engine* engine, kappai_step_output* out
     set_error("kappai_engine_step: no place for the outputs");
     return -1;
   }
+  if (!engine_ok(engine)) return -1;
   Locked lock;
   return (int)call_long(engine, "step", "(Ki)", (unsigned long long)(uintptr_t)outputs, capacity);
 }
@@ -271,6 +288,7 @@ extern "C" int kappai_engine_step(kappai_engine* engine, kappai_step_output* out
 extern "C" int kappai_engine_output(kappai_engine* engine, int request_id, int* tokens,
                                     int capacity) {
   g_error[0] = 0;
+  if (!engine_ok(engine)) return -1;
   Locked lock;
   return (int)call_long(engine, "output", "(iKi)", request_id,
                         (unsigned long long)(uintptr_t)tokens, tokens ? capacity : 0);
@@ -278,6 +296,7 @@ extern "C" int kappai_engine_output(kappai_engine* engine, int request_id, int* 
 
 extern "C" int kappai_engine_release(kappai_engine* engine, int request_id) {
   g_error[0] = 0;
+  if (!engine_ok(engine)) return -1;
   Locked lock;
   return (int)call_long(engine, "release", "(i)", request_id);
 }
@@ -290,6 +309,7 @@ extern "C" int kappai_engine_generate(kappai_engine* engine, const int* ids, int
     set_error("kappai_engine_generate: a prompt needs at least one token");
     return -1;
   }
+  if (!engine_ok(engine)) return -1;
   Locked lock;
   return (int)call_long(engine, "generate", "(KififffiKiKi)", (unsigned long long)(uintptr_t)ids,
                         n, (double)s->temperature, s->top_k, (double)s->top_p, (double)s->min_p,
@@ -320,6 +340,7 @@ extern "C" int kappai_engine_forward(kappai_engine* engine, const kappai_forward
     want.insert(want.end(), e.want, e.want + e.n_want);
   }
   if (want.empty()) want.push_back(0);            // (an address to hand over; its count is 0)
+  if (!engine_ok(engine)) return -1;
   Locked lock;
   return (int)call_long(engine, "forward", "(iKKKKKKK)", n_entries,
                         (unsigned long long)(uintptr_t)ids.data(),
@@ -333,6 +354,7 @@ extern "C" int kappai_engine_forward(kappai_engine* engine, const kappai_forward
 
 extern "C" int kappai_engine_end(kappai_engine* engine, int request_id) {
   g_error[0] = 0;
+  if (!engine_ok(engine)) return -1;
   Locked lock;
   return (int)call_long(engine, "end", "(i)", request_id);
 }
@@ -343,6 +365,7 @@ extern "C" int kappai_engine_get_stats(kappai_engine* engine, kappai_engine_stat
     set_error("kappai_engine_get_stats: no place for the numbers");
     return -1;
   }
+  if (!engine_ok(engine)) return -1;
   Locked lock;
   const long n = call_long(engine, "stats", "(Ki)", (unsigned long long)(uintptr_t)stats,
                            (int)(sizeof *stats / sizeof(double)));

@@ -44,6 +44,12 @@ int main(int argc, char** argv) {
   LOAD(kappai_engine_error)
   const int n_predict = atoi(argv[4]);
 
+  /* before any engine exists (and before this process has an interpreter) a call is refused */
+  if (p_kappai_engine_has_work(NULL) != -1 || strstr(p_kappai_engine_error(), "no engine") == NULL) {
+    fprintf(stderr, "a call without an engine was not refused\n");
+    return 1;
+  }
+
   kappai_engine_config config;
   p_kappai_engine_config_default(&config);
   config.model = argv[2];
