@@ -276,20 +276,31 @@ extern "C" int kappai_sample_rows(const float* logits, const float* temperature,
 
 // logits[row[i], tok[i]] is divided by penalty[i] when positive, multiplied otherwise.  The
 // caller lists every token of a row's window once per occurrence, as the reference applies
-// the penalty once per occurrence; entries of one (row, token) must therefore be serialised:
-// one thread walks the whole list of a row.
-__global__ void repeat_penalty_kernel(float* __restrict__ logits, const int* __restrict__ row_start,
-                                      const int* __restrict__ toks,
-                                      const float* __restrict__ penalty, int V) {
-  const int r = blockIdx.x;
-  if (threadIdx.x != 0) return;
+// the penalty once per occurrence (src/sampler.c:205-216).  One wave per row: a lane takes the
+// entries lane, lane + 64, ...; the lane that holds a token's first entry counts the token's
+// entries and applies the penalty to that one logit as many times, one after the other in a
+// register, which gives the bits of the reference's walk over the list (entries of different
+// tokens do not touch each other, and a logit keeps its sign under the penalty, so the order
+// among them does not matter).
+__global__ __launch_bounds__(WAVE) void repeat_penalty_kernel(
+    float* __restrict__ logits, const int* __restrict__ row_start, const int* __restrict__ toks,
+    const float* __restrict__ penalty, int V) {
+  const int r = blockIdx.x, lane = threadIdx.x;
   const float pen = penalty[r];
   if (pen == 1.0f) return;
   float* lg = logits + (size_t)r * V;
-  for (int i = row_start[r]; i < row_start[r + 1]; ++i) {
+  const int lo = row_start[r], hi = row_start[r + 1];
+  for (int i = lo + lane; i < hi; i += WAVE) {
     const int tok = toks[i];
     if (tok < 0 || tok >= V) continue;
-    lg[tok] = lg[tok] > 0.f ? lg[tok] / pen : lg[tok] * pen;
+    bool first = true;
+    for (int j = lo; j < i && first; ++j) first = toks[j] != tok;
+    if (!first) continue;
+    int times = 1;
+    for (int j = i + 1; j < hi; ++j) times += toks[j] == tok ? 1 : 0;
+    float v = lg[tok];
+    for (int t = 0; t < times; ++t) v = v > 0.f ? v / pen : v * pen;
+    lg[tok] = v;
   }
 }
 

@@ -1467,3 +1467,29 @@ def test_repeat_penalty(ops):
     ref.repeat_penalty(want, row_start, toks, pen)
     assert torch.allclose(dev.cpu(), want)
     assert want[0].tolist() == pytest.approx([0.25, 0.9, 0.0, -2.0])
+
+
+def test_repeat_penalty_of_long_windows_is_the_walk_over_the_list_bit_for_bit(ops):
+    """Windows longer than a wave with tokens that come up many times, tokens out of range and
+    rows without a penalty: the kernel's lanes share the list, the result is that of one walk
+    over it in order (what the reference does, src/sampler.c:205-216), to the last bit."""
+    g = torch.Generator().manual_seed(3)
+    V, rows = 1000, 5
+    logits = torch.randn(rows, V, generator=g) * 3
+    logits[0, 7] = 0.0
+    lens = [300, 0, 64, 65, 1]
+    toks = torch.cat([torch.randint(0, 40, (n,), generator=g) for n in lens]).to(torch.int32)
+    toks[5], toks[17] = -1, V + 3
+    row_start = torch.tensor([0] + list(np.cumsum(lens)), dtype=torch.int32)
+    pen = torch.tensor([1.3, 2.0, 1.0, 0.7, 1.1])
+    dev = logits.to(DEV).clone()
+    ops.repeat_penalty(dev, row_start.to(DEV), toks.to(DEV), pen.to(DEV))
+    want = logits.clone()
+    for r in range(rows):
+        if float(pen[r]) == 1.0:
+            continue
+        for t in toks[int(row_start[r]):int(row_start[r + 1])].tolist():
+            if 0 <= t < V:
+                v = want[r, t]
+                want[r, t] = v / pen[r] if v > 0 else v * pen[r]
+    assert torch.equal(dev.cpu(), want)
