@@ -2,7 +2,10 @@
 defined here with a HIP kernel and a runner of its own (``tests/toy_parts/running_mean.hip``),
 is registered, built into a toy architecture and stepped through ``kappai_forward`` without a
 change to the framework's files, bit for bit equal to the same steps run part by part from the
-host; and what has no description for the C side runs from the host as before."""
+host; and what has no description for the C side runs from the host as before.  The same for a
+norm and an arrangement of parts from outside (``tests/toy_parts/layer_norm_block.hip``:
+LayerNorm, and a block whose mixer and feed-forward read the same normalised rows) around the
+framework's own mixers and feed-forward."""
 import ctypes
 from ctypes import Structure, c_int, c_void_p
 from dataclasses import dataclass
@@ -15,6 +18,7 @@ import torch
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 TOY_SOURCE = Path(__file__).resolve().parent / "toy_parts" / "running_mean.hip"
+TOY_BLOCK_SOURCE = Path(__file__).resolve().parent / "toy_parts" / "layer_norm_block.hip"
 
 
 def toy_library():
@@ -298,3 +302,317 @@ def test_runners_are_looked_up_by_name_and_checked():
     plan.register_runner("mixer.toy_again", RUNNER_PART, lib.toy_running_mean_run, FoldDesc)
     with pytest.raises(KernelLaunchError, match="registered already"):
         plan.register_runner("mixer.toy_again", RUNNER_PART, lib.toy_running_mean_launch, FoldDesc)
+
+
+# ---------------------------------------------------------------------------------------------
+# a norm and a block from outside
+# ---------------------------------------------------------------------------------------------
+def toy_block_library():
+    from kappai_amd.kernels.lib import library_at
+    lib = library_at(TOY_BLOCK_SOURCE)
+    lib.toy_layer_norm_run.restype = None         # only their addresses are used
+    lib.toy_parallel_block_run.restype = None
+    return lib
+
+
+def define_toy_block():
+    """Registers the toy norm, the toy block and an architecture made of them (once)."""
+    from kappai_amd.config import ModelConfig, register_architecture
+    from kappai_amd.kernels import ops
+    from kappai_amd.models import Model
+    from kappai_amd.parts import (NORMS, Block, Hidden, Norm, OutputHead, TokenEmbedding,
+                                  make_part, register_part)
+    from kappai_amd.parts.base import summed_delta
+    from kappai_amd.parts.cdesc import (RUNNER_BLOCK, RUNNER_NORM, NormPartDesc, PartDesc,
+                                        defined_together)
+    from kappai_amd.weights.spec import INIT_ONES, INIT_SMALL, VECTOR, TensorSpec
+    if "toy_layer_norm" in NORMS:
+        return
+
+    class LayerNormDesc(Structure):
+        """``toy_layer_norm`` of tests/toy_parts/layer_norm_block.hip."""
+        _fields_ = [("w", c_void_p), ("b", c_void_p), ("eps", ctypes.c_float)]
+
+    class ParallelBlockDesc(Structure):
+        """``toy_parallel_block`` of tests/toy_parts/layer_norm_block.hip."""
+        _fields_ = [("norm", NormPartDesc), ("mixer", PartDesc), ("feed_forward", PartDesc)]
+
+    class ToyLayerNorm(Norm):
+        """``(x - mean) / sqrt(var + eps) * w + b``; adds the update into the stream first."""
+
+        def __init__(self, name, width, eps, dtype):
+            self.name, self.width, self.eps, self.dtype = name, width, float(eps), dtype
+
+        def tensor_specs(self):
+            return [TensorSpec(self.name + ".weight", (self.width,), VECTOR, INIT_ONES),
+                    TensorSpec(self.name + ".bias", (self.width,), VECTOR, INIT_SMALL)]
+
+        def bind(self, tensors):
+            self.weight = tensors[self.name + ".weight"].to(torch.float32).contiguous()
+            self.bias = tensors[self.name + ".bias"].to(torch.float32).contiguous()
+
+        def add_norm(self, resid, delta, rows=None):
+            n = resid.shape[0] if rows is None else rows.shape[0]
+            out = torch.empty((n, self.width), dtype=self.dtype, device=resid.device)
+            kind = 0 if delta is None else 2 if delta.dtype == torch.float32 else 1
+            rc = toy_block_library().toy_layer_norm_launch(
+                c_void_p(resid.data_ptr()), c_void_p(delta.data_ptr() if delta is not None else 0),
+                c_int(kind), c_void_p(self.weight.data_ptr()), c_void_p(self.bias.data_ptr()),
+                c_void_p(out.data_ptr()), c_int(1 if self.dtype == torch.bfloat16 else 0),
+                c_void_p(rows.data_ptr() if rows is not None else 0), c_int(n), c_int(self.width),
+                ctypes.c_float(self.eps), ops._stream())
+            assert rc == 0, rc
+            return out
+
+        def c_norm(self, plan):
+            lib = toy_block_library()
+            assert lib.toy_layer_norm_desc_bytes() == ctypes.sizeof(LayerNormDesc)
+            plan.register_runner("norm.toy_layer", RUNNER_NORM, lib.toy_layer_norm_run,
+                                 LayerNormDesc)
+            return plan.norm("norm.toy_layer", LayerNormDesc(self.weight.data_ptr(),
+                                                             self.bias.data_ptr(), self.eps))
+
+    register_part("norm", "toy_layer_norm", ToyLayerNorm)
+
+    class ParallelBlock(Block):
+        """``h = norm(x); x += mixer(h); x += feed_forward(h)``."""
+
+        def __init__(self, norm, mixer, feed_forward):
+            self.norm, self.mixer, self.feed_forward = norm, mixer, feed_forward
+
+        def _parts(self):
+            return (self.norm, self.mixer, self.feed_forward)
+
+        capturable = True
+
+        @property
+        def q_tile_rows(self):
+            return self.mixer.q_tile_rows
+
+        @property
+        def lone_rows_from(self):
+            return self.mixer.lone_rows_from
+
+        def tensor_specs(self):
+            return [t for p in self._parts() for t in p.tensor_specs()]
+
+        def bind(self, tensors):
+            for p in self._parts():
+                p.bind(tensors)
+
+        def weight_bytes(self):
+            return sum(p.weight_bytes() for p in self._parts())
+
+        def forward(self, h, batch, cache, shared_cache=False):
+            resid = h.resid
+            x = self.norm.add_norm(resid, summed_delta(self.norm, h.delta))
+            mixed = summed_delta(self.norm, self.mixer.forward(x, batch, cache,
+                                                               shared_cache=shared_cache))
+            if mixed is not None:
+                rc = toy_block_library().toy_add_launch(
+                    c_void_p(resid.data_ptr()), c_void_p(mixed.data_ptr()),
+                    c_int(1 if mixed.dtype == torch.float32 else 0),
+                    ctypes.c_long(mixed.numel()), ops._stream())
+                assert rc == 0, rc
+            return Hidden(resid, self.feed_forward.forward(x, batch))
+
+        def c_call(self, plan, view, shared_cache=False):
+            for part, method, c_method in ((self.norm, "add_norm", "c_norm"),
+                                           (self.mixer, "forward", "c_part"),
+                                           (self.feed_forward, "forward", "c_part")):
+                if not defined_together(part, method, c_method):
+                    return None
+            lib = toy_block_library()
+            assert lib.toy_parallel_block_desc_bytes() == ctypes.sizeof(ParallelBlockDesc)
+            plan.register_runner("block.toy_parallel", RUNNER_BLOCK, lib.toy_parallel_block_run,
+                                 ParallelBlockDesc)
+            norm = self.norm.c_norm(plan)
+            mixer = self.mixer.c_part(plan, view, shared_cache)
+            feed_forward = self.feed_forward.c_part(plan, None, False)
+            if norm is None or mixer is None or feed_forward is None:
+                return None
+            return plan.call("block.toy_parallel", ParallelBlockDesc(norm, mixer, feed_forward))
+
+    register_part("block", "toy_parallel", ParallelBlock)
+
+    @dataclass
+    class ToyBlockConfig(ModelConfig):
+        width: int = 0
+        vocab_size: int = 0
+        heads: int = 0
+        head_dim: int = 0
+        ff: int = 0
+        taps: int = 3
+        eps: float = 1e-5
+        max_position_embeddings: int = 512
+
+        KEYS = ("width", "vocab_size", "heads", "head_dim", "ff", "taps", "eps")
+
+        @classmethod
+        def from_dict(cls, raw):
+            return cls(architecture="ToyParallelForCausalLM", **{k: raw[k] for k in cls.KEYS})
+
+        def to_dict(self):
+            return {"architectures": ["ToyParallelForCausalLM"],
+                    **{k: getattr(self, k) for k in self.KEYS}}
+
+    def build(cfg, dtype):
+        def layer_norm(name):
+            return make_part("norm", "toy_layer_norm", name=name, width=cfg.width, eps=cfg.eps,
+                             dtype=dtype)
+
+        def rms(name):
+            return make_part("norm", "rmsnorm", name=name, width=cfg.width, eps=cfg.eps,
+                             dtype=dtype)
+
+        def ffn(p):
+            return make_part("feed_forward", "swiglu", prefix=p + "ff.", width=cfg.width,
+                             hidden=cfg.ff, dtype=dtype)
+        rot = make_part("position_encoding", "rotary", head_dim=cfg.head_dim, theta=100.0)
+
+        def attn(p):
+            return make_part("mixer", "attention", prefix=p + "att.", width=cfg.width,
+                             num_heads=cfg.heads, num_kv_heads=cfg.heads // 2,
+                             head_dim=cfg.head_dim, dtype=dtype, position=rot, qk_norm_eps=1e-5)
+
+        def conv(p):
+            return make_part("mixer", "conv", prefix=p + "conv.", width=cfg.width,
+                             kernel_size=cfg.taps, dtype=dtype, bias=True)
+        layers = [
+            make_part("block", "toy_parallel", norm=layer_norm("blocks.0.n"), mixer=conv("blocks.0."),
+                      feed_forward=ffn("blocks.0.")),
+            make_part("block", "pre_norm", mixer_norm=rms("blocks.1.n1"), mixer=attn("blocks.1."),
+                      ffn_norm=layer_norm("blocks.1.n2"), feed_forward=ffn("blocks.1.")),
+            make_part("block", "toy_parallel", norm=layer_norm("blocks.2.n"), mixer=attn("blocks.2."),
+                      feed_forward=ffn("blocks.2.")),
+            make_part("block", "pre_norm", mixer_norm=rms("blocks.3.n1"), mixer=conv("blocks.3."),
+                      ffn_norm=rms("blocks.3.n2"), feed_forward=ffn("blocks.3.")),
+        ]
+        emb = TokenEmbedding("emb", cfg.vocab_size, cfg.width)
+        return Model(cfg, dtype, emb, layers, layer_norm("final"),
+                     OutputHead("head", cfg.vocab_size, cfg.width, tied_to=emb))
+
+    register_architecture("ToyParallelForCausalLM", ToyBlockConfig, build)
+
+
+TOY_BLOCK = {"architectures": ["ToyParallelForCausalLM"], "width": 96, "vocab_size": 173,
+             "heads": 4, "head_dim": 16, "ff": 160, "taps": 3, "eps": 1e-5}
+
+
+def toy_block_model(tmp_path, dtype):
+    from kappai_amd.config import config_from_dict
+    from kappai_amd.models import load_model
+    from kappai_amd.weights import write_random_model
+    define_toy_block()
+    folder = tmp_path / "toy_block"
+    if not folder.exists():
+        write_random_model(folder, config_from_dict(dict(TOY_BLOCK)), seed=9, std=0.2,
+                           norm_jitter=0.1)
+    return load_model(folder, dtype, DEV)
+
+
+def test_the_toy_norm_is_a_layer_norm():
+    """The toy's kernel against torch: all rows with an update that joins the stream, and some
+    rows only, which leaves the stream as it was."""
+    lib = toy_block_library()
+    g = torch.Generator().manual_seed(4)
+    T, D, eps = 7, 70, 1e-3
+    resid, delta = torch.randn(T, D, generator=g), torch.randn(T, D, generator=g)
+    w, b = torch.randn(D, generator=g), torch.randn(D, generator=g)
+    want = torch.nn.functional.layer_norm((resid + delta).double(), (D,), w.double(), b.double(), eps)
+
+    def launch(r, d, out, rows):
+        rc = lib.toy_layer_norm_launch(
+            c_void_p(r.data_ptr()), c_void_p(d.data_ptr()), c_int(2), c_void_p(wd.data_ptr()),
+            c_void_p(bd.data_ptr()), c_void_p(out.data_ptr()), c_int(0),
+            c_void_p(rows.data_ptr() if rows is not None else 0), c_int(out.shape[0]), c_int(D),
+            ctypes.c_float(eps), c_void_p(torch.cuda.current_stream().cuda_stream))
+        assert rc == 0
+    wd, bd = w.to(DEV), b.to(DEV)
+    r, d = resid.to(DEV), delta.to(DEV)
+    out = torch.empty(T, D, device=DEV)
+    launch(r, d, out, None)
+    assert float((out.cpu().double() - want).abs().max()) < 1e-5
+    assert torch.equal(r.cpu(), resid + delta)
+    r = resid.to(DEV)
+    rows = torch.tensor([5, 0, 3], dtype=torch.int32, device=DEV)
+    some = torch.empty(3, D, device=DEV)
+    launch(r, d, some, rows)
+    assert float((some.cpu().double() - want[[5, 0, 3]]).abs().max()) < 1e-5
+    assert torch.equal(r.cpu(), resid)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_norm_and_a_block_from_outside_run_from_c(tmp_path, dtype):
+    """An architecture whose blocks are the toy arrangement (around the framework's conv and
+    attention mixers) and the framework's own (with the toy norm as its second norm), toy norm
+    before the head: launched from C it gives bit for bit what the host's part-by-part walk
+    gives under the mixed schedule, with and without decode graphs, and the portions give what
+    whole prompts give."""
+    import schedules
+    from replay_common import collect, make_requests
+    model = toy_block_model(tmp_path, dtype)
+    requests = make_requests(TOY_BLOCK["vocab_size"], [70, 45, 100, 37, 83, 64, 29], seed=23)
+    steps, index, peak = schedules.mixed(requests)
+    results = {}
+    for c_forward in (True, False):
+        for graphs in (False, True):
+            res, runner = replay(model, steps, peak, tmp_path / f"b{c_forward}g{graphs}",
+                                 c_forward, graphs)
+            assert (runner._cplan is not None) == c_forward, "the toy blocks have descriptions"
+            if graphs:
+                assert runner.graph_replays > 0
+            results[(c_forward, graphs)] = res
+    base = results[(False, False)]
+    for key, res in results.items():
+        for a, b in zip(base, res):
+            assert (a is None) == (b is None)
+            if a is not None:
+                assert np.array_equal(a, b), key
+    whole_steps, whole_index, whole_peak = schedules.whole(requests)
+    whole, _ = replay(model, whole_steps, whole_peak, tmp_path / "bwhole", True, False)
+    vocab = TOY_BLOCK["vocab_size"]
+    got = collect(index, {s["step"]: r for s, r in zip(steps, base) if r is not None}, vocab)
+    ref = collect(whole_index, {s["step"]: r for s, r in zip(whole_steps, whole) if r is not None},
+                  vocab)
+    scale = max(float(np.abs(v).max()) for v in ref.values())
+    tol = 2e-5 if dtype == "float32" else 4e-2
+    worst = max(float(np.abs(got[k] - ref[k]).max()) for k in ref) / scale
+    assert worst < tol, worst
+
+
+def test_the_toy_block_does_what_it_says_inside_the_model(tmp_path):
+    """A sequence through the model with the mixers and feed-forwards of all blocks but the first
+    switched off (their last products zero): the logits are head(LN(x + conv(h) + ffn(h))) with
+    h = LN(embedding), worked out in float64 from the file's tensors with the plain
+    implementation's conv mixer and feed-forward, against the C walk."""
+    from plain import lfm2 as P
+    model = toy_block_model(tmp_path, "float32")
+    for blk in model.layers[1:]:
+        blk.feed_forward.down.weight.zero_()
+        mixer_out = blk.mixer.out if hasattr(blk.mixer, "out") else blk.mixer.out_proj
+        mixer_out.weight.zero_()
+        if mixer_out.bias is not None:
+            mixer_out.bias.zero_()
+    toks = [int(t) for t in np.random.default_rng(5).integers(0, TOY_BLOCK["vocab_size"], size=11)]
+    steps = [{"step": 0, "entries": [{"id": "a", "tokens": toks, "want": list(range(11))}],
+              "end": ["a"]}]
+    (got,), runner = replay(model, steps, 64, tmp_path / "bzero", True, False)
+    assert runner._cplan is not None
+    w = {k: np.asarray(v, dtype=np.float64) for k, v in
+         P.read_safetensors(tmp_path / "toy_block" / "model.safetensors").items()}
+
+    def ln(x, name):
+        mu = x.mean(-1, keepdims=True)
+        var = ((x - mu) ** 2).mean(-1, keepdims=True)
+        return (x - mu) / np.sqrt(var + TOY_BLOCK["eps"]) * w[name + ".weight"] + w[name + ".bias"]
+    x = w["emb.weight"][toks]
+    h = ln(x, "blocks.0.n")
+    conv = {"in_proj": w["blocks.0.conv.in_proj.weight"], "in_proj_bias": w["blocks.0.conv.in_proj.bias"],
+            "conv": w["blocks.0.conv.conv.weight"].reshape(TOY_BLOCK["width"], TOY_BLOCK["taps"]),
+            "conv_bias": w["blocks.0.conv.conv.bias"], "out_proj": w["blocks.0.conv.out_proj.weight"],
+            "out_proj_bias": w["blocks.0.conv.out_proj.bias"]}
+    ff = {k: w[f"blocks.0.ff.{k}.weight"] for k in ("w1", "w2", "w3")}
+    x = x + P.short_conv_mixer(h, conv, {"hidden_size": TOY_BLOCK["width"]}) + P.swiglu_feed_forward(h, ff)
+    want = ln(x, "final") @ w["emb.weight"].T
+    assert float(np.abs(got - want).max()) < 2e-5 * float(np.abs(want).max())
