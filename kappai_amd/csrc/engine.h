@@ -28,7 +28,7 @@
 extern "C" {
 #endif
 
-#define KAPPAI_ENGINE_ABI 9          // bumped with every change of the structs below
+#define KAPPAI_ENGINE_ABI 10         // bumped with every change of the structs below
 #define KAPPAI_MAX_GROUPS 8          // paged groups a batch can carry block tables for
 
 // ---- the kernels' launchers, by address (they live in libraries of their own) ---------------
@@ -251,6 +251,14 @@ typedef struct kappai_tuning {
                                     // store itself (0: never)
 } kappai_tuning;
 
+// What may change the embedded rows before the first call of the schedule (an encoding of
+// positions that is added to them): resid holds the step's M rows, looked up already.
+typedef void (*kappai_embedded_fn)(kappai_step*, const void* desc, float* resid, int M);
+typedef struct kappai_embedded_part {
+  kappai_embedded_fn run;          // null: nothing does
+  const void* desc;
+} kappai_embedded_part;
+
 typedef struct kappai_model {
   int abi;                          // KAPPAI_ENGINE_ABI of the side that filled this in
   int compute_bf16;                 // activations and cache in bfloat16 (else float32)
@@ -263,6 +271,7 @@ typedef struct kappai_model {
   kappai_linear head;
   const kappai_kernels* kernels;
   kappai_tuning tuning;
+  kappai_embedded_part on_embedding;
 } kappai_model;
 
 // ---- the rows of a step -------------------------------------------------------------------------
@@ -287,9 +296,11 @@ typedef struct kappai_batch {
 } kappai_batch;
 
 // ---- the registry of runners ----------------------------------------------------------------
-enum { KAPPAI_RUNNER_PART = 0, KAPPAI_RUNNER_NORM = 1, KAPPAI_RUNNER_BLOCK = 2 };
+enum { KAPPAI_RUNNER_PART = 0, KAPPAI_RUNNER_NORM = 1, KAPPAI_RUNNER_BLOCK = 2,
+       KAPPAI_RUNNER_EMBEDDED = 3 };
 
-// Registers `fn` (a kappai_part_fn, kappai_norm_fn or kappai_block_fn, as `kind` says) under
+// Registers `fn` (a kappai_part_fn, kappai_norm_fn, kappai_block_fn or kappai_embedded_fn, as
+// `kind` says) under
 // `name`; desc_bytes is the size of the description it reads, which the host checks its own
 // layout against.  A name can be registered again with the same function only.  Returns 0, or
 // hipErrorInvalidValue (the message through kappai_forward_error).

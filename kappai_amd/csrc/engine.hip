@@ -478,6 +478,11 @@ int run(const kappai_model* m, const kappai_batch* b, Arena& arena, float* logit
   // the embedding is looked up by the first norm that runs (which may do both in one kernel)
   kappai_carry carry = {};
   carry.kind = KAPPAI_CARRY_EMBEDDING;
+  if (m->on_embedding.run != nullptr) {
+    // something changes the embedded rows: they are looked up now
+    carry = plain_carry(c, carry, resid, T);
+    m->on_embedding.run(&c, m->on_embedding.desc, resid, T);
+  }
   for (int ci = 0; ci < m->n_calls && c.ok(); ++ci) {
     const kappai_call& call = m->calls[ci];
     const kappai_call* next = ci + 1 < m->n_calls ? &m->calls[ci + 1] : nullptr;
@@ -540,7 +545,7 @@ bool batch_ok(const kappai_batch* b) {
 }  // namespace
 
 extern "C" int kappai_register_runner(const char* name, int kind, void* fn, int desc_bytes) {
-  if (name == nullptr || fn == nullptr || kind < KAPPAI_RUNNER_PART || kind > KAPPAI_RUNNER_BLOCK ||
+  if (name == nullptr || fn == nullptr || kind < KAPPAI_RUNNER_PART || kind > KAPPAI_RUNNER_EMBEDDED ||
       desc_bytes < 0) {
     snprintf(g_error, sizeof g_error, "kappai_register_runner: a runner needs a name, a kind and "
                                       "a function");

@@ -20,10 +20,11 @@ import torch
 
 from ..kernels import ops, tuning
 from ..kernels.lib import KernelLaunchError, library
-from ..parts.cdesc import (AttentionKernels, CallDesc, CarryDesc, CPlan, FoldDesc, LinearDesc,
-                           NormPartDesc, PartDesc, RowsDesc, address_of, defined_together)
+from ..parts.cdesc import (AttentionKernels, CallDesc, CarryDesc, CPlan, EmbeddedPartDesc,
+                           FoldDesc, LinearDesc, NormPartDesc, PartDesc, RowsDesc, address_of,
+                           defined_together)
 
-ENGINE_ABI = 9
+ENGINE_ABI = 10
 MAX_GROUPS = 8
 
 
@@ -51,7 +52,8 @@ class ModelDesc(Structure):
         ("abi", c_int), ("compute_bf16", c_int), ("width", c_int), ("vocab", c_int),
         ("page_size", c_int), ("embed_table", c_void_p), ("embed_is_bf16", c_int),
         ("n_calls", c_int), ("calls", POINTER(CallDesc)), ("final_norm", NormPartDesc),
-        ("head", LinearDesc), ("kernels", POINTER(Kernels)), ("tuning", TuningDesc)]
+        ("head", LinearDesc), ("kernels", POINTER(Kernels)), ("tuning", TuningDesc),
+        ("on_embedding", EmbeddedPartDesc)]
 
 
 class BatchDesc(Structure):
@@ -110,10 +112,13 @@ class CForward:
     @staticmethod
     def plannable(model) -> bool:
         """Whether the model as a whole can be walked from C: it is bound, its embedding, final
-        norm and head describe themselves, nothing is added to the embedded rows, and its
-        ``forward`` is the one the C walk repeats.  Whether every block describes itself shows
-        when the plan is built (``NotDescribed``)."""
-        if model.embedding_position is not None or not model.bound:
+        norm and head describe themselves, so does what changes the embedded rows (if anything
+        does), and its ``forward`` is the one the C walk repeats.  Whether every block describes
+        itself shows when the plan is built (``NotDescribed``)."""
+        if not model.bound:
+            return False
+        if model.embedding_position is not None and not defined_together(
+                model.embedding_position, "on_embedding", "c_embedded"):
             return False
         if model.dtype not in (torch.bfloat16, torch.float32):
             return False
@@ -146,7 +151,11 @@ class CForward:
         self.kernels = k
         described = model.c_calls(plan)
         final_norm = model.final_norm.c_norm(plan)
-        if described is None or final_norm is None:
+        on_embedding = None
+        if model.embedding_position is not None:
+            on_embedding = model.embedding_position.c_embedded(plan)
+        if described is None or final_norm is None or (
+                model.embedding_position is not None and on_embedding is None):
             raise NotDescribed()
         calls = (CallDesc * max(len(described), 1))()
         for ci, call in enumerate(described):
@@ -161,6 +170,8 @@ class CForward:
                            else 1 if table.dtype == torch.bfloat16 else 0)
         m.n_calls, m.calls = len(described), calls
         m.final_norm = final_norm
+        if on_embedding is not None:
+            m.on_embedding = on_embedding
         m.head = plan.linear(model.head.c_linear())
         m.kernels = ctypes.pointer(self.kernels)
         t = m.tuning

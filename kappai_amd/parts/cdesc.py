@@ -6,7 +6,9 @@ from C gives itself one more method, which builds its description and names its 
 
 * a mixer or a feed-forward: ``c_part(plan, view, shared_cache) -> PartDesc or None``,
 * a norm: ``c_norm(plan) -> NormPartDesc or None``,
-* a block: ``c_call(plan, view, shared_cache) -> CallDesc or None``
+* a block: ``c_call(plan, view, shared_cache) -> CallDesc or None``,
+* a position encoding that changes the embedded rows: ``c_embedded(plan) -> EmbeddedPartDesc or
+  None``
 
 (``None``: not from C in this configuration; the model then runs from the parts' ``forward``
 methods).  ``plan`` is a ``CPlan``: it looks runners up by name, checks that the description has
@@ -25,7 +27,7 @@ from typing import Callable, List, Optional
 
 import torch
 
-RUNNER_PART, RUNNER_NORM, RUNNER_BLOCK = 0, 1, 2
+RUNNER_PART, RUNNER_NORM, RUNNER_BLOCK, RUNNER_EMBEDDED = 0, 1, 2, 3
 TAKES_DEFERRED_ROWS, ADDS_RESIDUAL = 1, 2
 
 
@@ -61,6 +63,10 @@ class NormPartDesc(Structure):
 class CallDesc(Structure):
     _fields_ = [("run", c_void_p), ("desc", c_void_p), ("first_norm", POINTER(NormPartDesc)),
                 ("first_consumer", POINTER(PartDesc))]
+
+
+class EmbeddedPartDesc(Structure):
+    _fields_ = [("run", c_void_p), ("desc", c_void_p)]
 
 
 class AttentionKernels(Structure):
@@ -169,6 +175,12 @@ class CPlan:
             self.runner(runner, RUNNER_BLOCK, type(desc)), ctypes.addressof(desc),
             ctypes.pointer(first_norm) if first_norm is not None else None,
             ctypes.pointer(first_consumer) if first_consumer is not None else None))
+
+    def embedded(self, runner: str, desc) -> EmbeddedPartDesc:
+        """What changes the embedded rows before the first call (an encoding of positions)."""
+        self.keep(desc)
+        return self.keep(EmbeddedPartDesc(self.runner(runner, RUNNER_EMBEDDED, type(desc)),
+                                          ctypes.addressof(desc)))
 
     def attention_kernels(self, head_dim: int) -> AttentionKernels:
         """The launchers of the matrix-core attention library of one head size."""

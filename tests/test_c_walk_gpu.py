@@ -5,7 +5,8 @@ change to the framework's files, bit for bit equal to the same steps run part by
 host; and what has no description for the C side runs from the host as before.  The same for a
 norm and an arrangement of parts from outside (``tests/toy_parts/layer_norm_block.hip``:
 LayerNorm, and a block whose mixer and feed-forward read the same normalised rows) around the
-framework's own mixers and feed-forward."""
+framework's own mixers and feed-forward, and for an encoding of positions that is added to the
+embedded rows (``tests/toy_parts/learned_positions.hip``)."""
 import ctypes
 from ctypes import Structure, c_int, c_void_p
 from dataclasses import dataclass
@@ -19,6 +20,7 @@ pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 TOY_SOURCE = Path(__file__).resolve().parent / "toy_parts" / "running_mean.hip"
 TOY_BLOCK_SOURCE = Path(__file__).resolve().parent / "toy_parts" / "layer_norm_block.hip"
+TOY_POSITIONS_SOURCE = Path(__file__).resolve().parent / "toy_parts" / "learned_positions.hip"
 
 
 def toy_library():
@@ -616,3 +618,147 @@ def test_the_toy_block_does_what_it_says_inside_the_model(tmp_path):
     x = x + P.short_conv_mixer(h, conv, {"hidden_size": TOY_BLOCK["width"]}) + P.swiglu_feed_forward(h, ff)
     want = ln(x, "final") @ w["emb.weight"].T
     assert float(np.abs(got - want).max()) < 2e-5 * float(np.abs(want).max())
+
+
+# ---------------------------------------------------------------------------------------------
+# an encoding of positions from outside, added to the embedded rows
+# ---------------------------------------------------------------------------------------------
+def toy_positions_library():
+    from kappai_amd.kernels.lib import library_at
+    lib = library_at(TOY_POSITIONS_SOURCE)
+    lib.toy_learned_positions_run.restype = None
+    return lib
+
+
+def define_toy_positions():
+    from kappai_amd.config import ModelConfig, register_architecture
+    from kappai_amd.kernels import ops
+    from kappai_amd.models import Model
+    from kappai_amd.parts import (POSITION_ENCODINGS, OutputHead, PositionEncoding,
+                                  TokenEmbedding, make_part, register_part)
+    from kappai_amd.parts.cdesc import RUNNER_EMBEDDED
+    from kappai_amd.weights.spec import INIT_NORMAL, TABLE, TensorSpec
+    if "toy_learned_hip" in POSITION_ENCODINGS:
+        return
+
+    class PositionsDesc(Structure):
+        """``toy_learned_positions`` of tests/toy_parts/learned_positions.hip."""
+        _fields_ = [("table", c_void_p), ("table_is_bf16", c_int), ("positions", c_int)]
+
+    class LearnedPositionsHip(PositionEncoding):
+        """x_t += table[position of t]."""
+
+        def __init__(self, name, n_positions, width):
+            self.name, self.n, self.width = name, n_positions, width
+
+        def tensor_specs(self):
+            return [TensorSpec(self.name + ".weight", (self.n, self.width), TABLE, INIT_NORMAL)]
+
+        def bind(self, tensors):
+            self.table = tensors[self.name + ".weight"].contiguous()
+
+        def on_embedding(self, x, batch):
+            rc = toy_positions_library().toy_add_positions_launch(
+                c_void_p(x.data_ptr()), c_void_p(self.table.data_ptr()),
+                c_int(1 if self.table.dtype == torch.bfloat16 else 0),
+                c_void_p(batch.row_pos.data_ptr()), c_int(x.shape[0]), c_int(self.width),
+                c_int(self.n), ops._stream())
+            assert rc == 0, rc
+
+        def c_embedded(self, plan):
+            lib = toy_positions_library()
+            assert lib.toy_learned_positions_desc_bytes() == ctypes.sizeof(PositionsDesc)
+            plan.register_runner("embedded.toy_learned", RUNNER_EMBEDDED,
+                                 lib.toy_learned_positions_run, PositionsDesc)
+            return plan.embedded("embedded.toy_learned", PositionsDesc(
+                self.table.data_ptr(), 1 if self.table.dtype == torch.bfloat16 else 0, self.n))
+
+    register_part("position_encoding", "toy_learned_hip", LearnedPositionsHip)
+
+    @dataclass
+    class ToyPositionsConfig(ModelConfig):
+        width: int = 0
+        vocab_size: int = 0
+        heads: int = 0
+        head_dim: int = 0
+        ff: int = 0
+        eps: float = 1e-5
+        max_position_embeddings: int = 256
+
+        KEYS = ("width", "vocab_size", "heads", "head_dim", "ff", "eps")
+
+        @classmethod
+        def from_dict(cls, raw):
+            return cls(architecture="ToyPositionsForCausalLM", **{k: raw[k] for k in cls.KEYS})
+
+        def to_dict(self):
+            return {"architectures": ["ToyPositionsForCausalLM"],
+                    **{k: getattr(self, k) for k in self.KEYS}}
+
+    def build(cfg, dtype):
+        def rms(name):
+            return make_part("norm", "rmsnorm", name=name, width=cfg.width, eps=cfg.eps,
+                             dtype=dtype)
+
+        def block(i, mixer):
+            p = f"blocks.{i}."
+            return make_part("block", "pre_norm", mixer_norm=rms(p + "n1"), mixer=mixer,
+                             ffn_norm=rms(p + "n2"),
+                             feed_forward=make_part("feed_forward", "swiglu", prefix=p + "ff.",
+                                                    width=cfg.width, hidden=cfg.ff, dtype=dtype))
+        # attention without rotation: the positions come from the table alone
+        layers = [block(i, make_part("mixer", "attention", prefix=f"blocks.{i}.att.",
+                                     width=cfg.width, num_heads=cfg.heads,
+                                     num_kv_heads=cfg.heads // 2, head_dim=cfg.head_dim,
+                                     dtype=dtype, position=None, qk_norm_eps=None))
+                  for i in range(2)]
+        emb = TokenEmbedding("emb", cfg.vocab_size, cfg.width)
+        positions = make_part("position_encoding", "toy_learned_hip", name="pos",
+                              n_positions=cfg.max_position_embeddings, width=cfg.width)
+        return Model(cfg, dtype, emb, layers, rms("final"),
+                     OutputHead("head", cfg.vocab_size, cfg.width, tied_to=emb),
+                     embedding_position=positions)
+
+    register_architecture("ToyPositionsForCausalLM", ToyPositionsConfig, build)
+
+
+TOY_POSITIONS = {"architectures": ["ToyPositionsForCausalLM"], "width": 64, "vocab_size": 131,
+                 "heads": 4, "head_dim": 16, "ff": 96, "eps": 1e-5}
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_positions_added_to_the_embedded_rows_run_from_c(tmp_path, dtype):
+    """A learned row per position added to the embedded rows by a kernel from outside, attention
+    without rotation: from C bit for bit what the host's walk gives under the mixed schedule,
+    with and without graphs; and the model does depend on the positions (a request whose table
+    rows are moved gives other logits)."""
+    import schedules
+    from kappai_amd.config import config_from_dict
+    from kappai_amd.models import load_model
+    from kappai_amd.weights import write_random_model
+    from replay_common import make_requests
+    define_toy_positions()
+    folder = tmp_path / "toy_positions"
+    write_random_model(folder, config_from_dict(dict(TOY_POSITIONS)), seed=11, std=0.2,
+                       norm_jitter=0.1)
+    model = load_model(folder, dtype, DEV)
+    requests = make_requests(TOY_POSITIONS["vocab_size"], [70, 45, 100, 37, 83], seed=24)
+    steps, index, peak = schedules.mixed(requests)
+    results = {}
+    for c_forward in (True, False):
+        for graphs in (False, True):
+            res, runner = replay(model, steps, peak, tmp_path / f"p{c_forward}g{graphs}",
+                                 c_forward, graphs)
+            assert (runner._cplan is not None) == c_forward
+            results[(c_forward, graphs)] = res
+    base = results[(False, False)]
+    for key, res in results.items():
+        for a, b in zip(base, res):
+            assert (a is None) == (b is None)
+            if a is not None:
+                assert np.array_equal(a, b), key
+    # the positions matter: with the table's rows rolled by one the logits move
+    model.embedding_position.table.copy_(torch.roll(model.embedding_position.table, 1, 0))
+    moved, _ = replay(model, steps, peak, tmp_path / "pmoved", True, False)
+    first = next(i for i, a in enumerate(base) if a is not None)
+    assert float(np.abs(moved[first] - base[first]).max()) > 1e-3
