@@ -1399,9 +1399,9 @@ __global__ __launch_bounds__(NWN * NWK * WAVE) void gemm_bf16_shared_rows_kernel
   };
 
   // W is loaded NSETS - 1 chunks ahead into register sets used in turn; A one chunk ahead.  In
-  // every round the loads of A are issued before those of W, and loads come back in the order
-  // they were issued: waiting until only the last round's loads of W are out means that the
-  // chunk of A issued before them has landed.  NSETS is even, so that the LDS buffer of a round
+  // every pass of the loop the loads of A are issued before those of W, and loads come back in
+  // the order they were issued: waiting until only the latest pass's loads of W are out means that
+  // the chunk of A issued before them has landed.  NSETS is even, so that the LDS buffer of a pass
   // is known at compile time (else the compiler waits for every load before it reads LDS).
   u32x4_t wv[NSETS][UK][2];
   stage(0, 0);
@@ -1623,9 +1623,9 @@ __global__ __launch_bounds__(R32_NWN * R32_NWK * WAVE) void gemm_bf16_rows32_ker
   };
 
   // W one run ahead in two register sets used in turn, A one run ahead in the other LDS buffer.
-  // In every round the loads of A are issued before those of W, and loads come back in the order
-  // they were issued: waiting until only the last round's four loads of W are out means that the
-  // run of A issued before them has landed (and the run of W before that).
+  // In every pass of the loop the loads of A are issued before those of W, and loads come back in
+  // the order they were issued: waiting until only the latest pass's four loads of W are out means
+  // that the run of A issued before them has landed (and the run of W before that).
   u32x4_t wv[2][4];
   stage(0, 0);
   load_w(wv[0], 0);
