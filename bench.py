@@ -53,9 +53,10 @@ WORKLOADS = {
 }
 
 
-def run_workload(key, dtype, device):
-    """One serving workload from start to end through ``Engine.generate`` with greedy sampling:
-    all requests arrive together.  Prints one JSON line: generated tokens a second over the
+def run_workload(key, dtype, device, repeat_penalty=1.0):
+    """One serving workload from start to end through ``Engine.generate`` with greedy sampling
+    (after a repeat penalty over the last 64 tokens, if one is asked for): all requests arrive
+    together.  Prints one JSON line: generated tokens a second over the
     whole run (prompts included in the time), and the engine's own prefill / decode rates."""
     import torch
 
@@ -75,7 +76,10 @@ def run_workload(key, dtype, device):
                for L in lengths]
     sync()
     t0 = time.perf_counter()
-    out = eng.generate(prompts, SamplingParams.greedy(n_predict=w["n_predict"]))
+    import dataclasses
+    params = dataclasses.replace(SamplingParams.greedy(n_predict=w["n_predict"]),
+                                 repeat_penalty=float(repeat_penalty))
+    out = eng.generate(prompts, params)
     sync()
     dt = time.perf_counter() - t0
     m = eng.metrics
@@ -88,7 +92,8 @@ def run_workload(key, dtype, device):
                    "num_layers": cfg.num_hidden_layers, "attention_layers": len(cfg.attention_layers),
                    "ff_dim": cfg.ff_dim, "requests": n, "prompt_tokens": sum(lengths),
                    "generated_tokens": generated, "chunk": w["chunk"],
-                   "token_budget": w["token_budget"], "ctx_size": w["ctx"]},
+                   "token_budget": w["token_budget"], "ctx_size": w["ctx"],
+                   "repeat_penalty": float(repeat_penalty)},
         "engine": {"steps": m.steps, "prefill_tok_s": round(m.pp, 1), "decode_tok_s": round(m.tg, 1),
                    "ttft_ms": round(m.first_token_ms, 2), "graph_replays": eng.runner.graph_replays,
                    "preemptions": eng.scheduler.preempted_total},
@@ -456,12 +461,15 @@ def main() -> int:
     ap.add_argument("--workload", default="decode", choices=["decode"] + sorted(WORKLOADS),
                     help="decode: the headline run; the others are serving workloads through "
                          "the engine's scheduler")
+    ap.add_argument("--repeat-penalty", type=float, default=1.0,
+                    help="serving workloads: a repeat penalty over the last 64 tokens before "
+                         "the greedy choice (1: none)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this engine runs on one GPU; --gpus must be 1 (nothing was measured)")
         return 2
     if args.workload != "decode":
-        return run_workload(args.workload, args.dtype, "cuda:0")
+        return run_workload(args.workload, args.dtype, "cuda:0", args.repeat_penalty)
 
     import torch
 

@@ -314,6 +314,94 @@ extern "C" int kappai_repeat_penalty(float* logits, const int* row_start, const 
 }
 
 // ---------------------------------------------------------------------------------------
+// The tokens a request has seen, kept on the GPU: history[slot] is a ring of `cap` token ids and
+// seen[slot] counts what went into it.  With it the repeat penalty needs nothing from the host
+// at the time of a step, so a step can be queued before the tokens of the one before it have
+// been read.  (kappai keeps the same ring on the host: src/sampler.c recent / recent_head.)
+// ---------------------------------------------------------------------------------------
+// history[slots[i]] := toks[starts[i] .. starts[i + 1]) (at most cap tokens, the oldest first)
+__global__ __launch_bounds__(WAVE) void history_set_kernel(
+    int* __restrict__ history, int* __restrict__ seen, const int* __restrict__ slots,
+    const int* __restrict__ starts, const int* __restrict__ toks, int cap) {
+  const int i = blockIdx.x, lane = threadIdx.x;
+  const int slot = slots[i], lo = starts[i], n = min(starts[i + 1] - lo, cap);
+  for (int j = lane; j < n; j += WAVE) history[(size_t)slot * cap + j] = toks[lo + j];
+  if (lane == 0) seen[slot] = n;
+}
+
+// entry i: the penalty of row rows[i] over the last last_n[i] tokens of history[slots[i]], as
+// repeat_penalty_kernel applies it to a list
+__global__ __launch_bounds__(WAVE) void repeat_penalty_history_kernel(
+    float* __restrict__ logits, const int* __restrict__ rows, const int* __restrict__ slots,
+    const float* __restrict__ penalty, const int* __restrict__ last_n,
+    const int* __restrict__ history, const int* __restrict__ seen, int V, int cap) {
+  const int i = blockIdx.x, lane = threadIdx.x;
+  const float pen = penalty[i];
+  if (pen == 1.0f) return;
+  float* lg = logits + (size_t)rows[i] * V;
+  const int slot = slots[i];
+  const int* ring = history + (size_t)slot * cap;
+  const int total = seen[slot];
+  const int n = min(min(last_n[i], total), cap);
+  const int first = total - n;                          // the window: tokens first .. total - 1
+  auto at = [&](int j) { return ring[(first + j) % cap]; };
+  for (int j = lane; j < n; j += WAVE) {
+    const int tok = at(j);
+    if (tok < 0 || tok >= V) continue;
+    bool is_first = true;
+    for (int e = 0; e < j && is_first; ++e) is_first = at(e) != tok;
+    if (!is_first) continue;
+    int times = 1;
+    for (int e = j + 1; e < n; ++e) times += at(e) == tok ? 1 : 0;
+    float v = lg[tok];
+    for (int t = 0; t < times; ++t) v = v > 0.f ? v / pen : v * pen;
+    lg[tok] = v;
+  }
+}
+
+// entry i: the token chosen for row rows[i] joins history[slots[i]]
+__global__ void history_append_kernel(const int* __restrict__ chosen, const int* __restrict__ rows,
+                                      const int* __restrict__ slots, int* __restrict__ history,
+                                      int* __restrict__ seen, int n, int cap) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const int slot = slots[i];
+  const int total = seen[slot];
+  history[(size_t)slot * cap + total % cap] = chosen[rows[i]];
+  seen[slot] = total + 1;         // (a request's tokens are far fewer than an int counts)
+}
+
+extern "C" int kappai_history_set(int* history, int* seen, const int* slots, const int* starts,
+                                  const int* toks, int n, int cap, hipStream_t stream) {
+  if (n <= 0) return 0;
+  if (cap < 1) return (int)hipErrorInvalidValue;
+  hipLaunchKernelGGL(history_set_kernel, dim3(n), dim3(WAVE), 0, stream, history, seen, slots,
+                     starts, toks, cap);
+  KAPPAI_RETURN_LAUNCH_STATUS();
+}
+
+extern "C" int kappai_repeat_penalty_history(float* logits, const int* rows, const int* slots,
+                                             const float* penalty, const int* last_n,
+                                             const int* history, const int* seen, int n, int V,
+                                             int cap, hipStream_t stream) {
+  if (n <= 0) return 0;
+  if (cap < 1 || V < 1) return (int)hipErrorInvalidValue;
+  hipLaunchKernelGGL(repeat_penalty_history_kernel, dim3(n), dim3(WAVE), 0, stream, logits, rows,
+                     slots, penalty, last_n, history, seen, V, cap);
+  KAPPAI_RETURN_LAUNCH_STATUS();
+}
+
+extern "C" int kappai_history_append(const int* chosen, const int* rows, const int* slots,
+                                     int* history, int* seen, int n, int cap,
+                                     hipStream_t stream) {
+  if (n <= 0) return 0;
+  if (cap < 1) return (int)hipErrorInvalidValue;
+  hipLaunchKernelGGL(history_append_kernel, dim3((n + 63) / 64), dim3(64), 0, stream, chosen, rows,
+                     slots, history, seen, n, cap);
+  KAPPAI_RETURN_LAUNCH_STATUS();
+}
+
+// ---------------------------------------------------------------------------------------
 // Draw with narrowed candidates (kappai: src/sampler.c:218-332): the `keep` largest logits
 // (top-k, or the best 1024 when only top-p / min-p narrow), sorted by descending logit;
 // softmax of logit/T in float; top-p keeps the token that crosses the mass; min-p is relative

@@ -349,7 +349,8 @@ class Engine:
         sampling = [e.request for e in entries if e.samples]
         self.last_logits = logits
         if sampling:                      # reading the tokens back waits for the step
-            tokens = self.sampler.sample(logits, [r.sampler for r in sampling])
+            tokens = self.sampler.sample(logits, [r.sampler for r in sampling],
+                                         slots=[r.cache.slot for r in sampling])
         else:
             tokens = []
             torch.cuda.synchronize(self.device)
@@ -408,7 +409,8 @@ class Engine:
         sampling = [e.request for e in entries if e.samples]
         if sampling:
             chosen = torch.empty(len(sampling), dtype=torch.int32, device=self.device)
-            self.sampler.launch(logits, [r.sampler for r in sampling], out=chosen)
+            self.sampler.launch(logits, [r.sampler for r in sampling], out=chosen,
+                                slots=[r.cache.slot for r in sampling])
             self._send_home(sampling, chosen, 1)
         outputs = self._read_tokens(older)
         self._count(tally, time.perf_counter() - t0)
@@ -420,9 +422,10 @@ class Engine:
         Returns None, with nothing changed, when the run cannot be queued."""
         reqs = [e.request for e in entries]
         samplers = [r.sampler for r in reqs]
+        slots = [r.cache.slot for r in reqs]
 
         def choose(logits, step, out_row, also):
-            self.sampler.launch(logits, samplers, out=out_row, also=also)
+            self.sampler.launch(logits, samplers, out=out_row, also=also, slots=slots)
 
         first = [0 if r.unread else r.tokens_from(r.computed, 1)[0] for r in reqs]
         tokens = self.runner.decode_run(
@@ -455,9 +458,10 @@ class Engine:
         if n < 2 or not Sampler.runs_on_device(samplers, self.model.vocab_size):
             return None
         first = [r.tokens_from(r.computed, 1)[0] for r in reqs]
+        slots = [r.cache.slot for r in reqs]
 
         def choose(logits, step, out_row, also):
-            self.sampler.launch(logits, samplers, out=out_row, also=also)
+            self.sampler.launch(logits, samplers, out=out_row, also=also, slots=slots)
 
         t0 = time.perf_counter()
         tokens = self.runner.decode_run([r.cache for r in reqs], first, n, choose)

@@ -1091,3 +1091,54 @@ def repeat_penalty(logits: torch.Tensor, row_start: torch.Tensor, tokens: torch.
     check(library("sampling").kappai_repeat_penalty(
         _ptr(logits), _ptr(row_start), _ptr(tokens), _ptr(penalty), _c_int(n), _c_int(V),
         _stream()), "repeat_penalty")
+
+
+def history_set(history: torch.Tensor, seen: torch.Tensor, slots: torch.Tensor,
+                starts: torch.Tensor, tokens: torch.Tensor) -> None:
+    """``history[slots[i]]`` (a ring of token ids, int32 [slots, cap]) becomes
+    ``tokens[starts[i]:starts[i+1]]`` (at most cap, the oldest first) and ``seen[slots[i]]`` their
+    number: what a request has seen before its first token is chosen on the GPU."""
+    for name, t in (("history", history), ("seen", seen), ("slots", slots), ("starts", starts),
+                    ("tokens", tokens)):
+        _gpu(name, t, I32)
+    n = slots.shape[0]
+    _need(history.dim() == 2 and seen.shape == (history.shape[0],) and starts.shape == (n + 1,),
+          "history_set: a ring and a count per slot, starts per entry")
+    check(library("sampling").kappai_history_set(
+        _ptr(history), _ptr(seen), _ptr(slots), _ptr(starts), _ptr(tokens), _c_int(n),
+        _c_int(history.shape[1]), _stream()), "history_set")
+
+
+def repeat_penalty_history(logits: torch.Tensor, rows: torch.Tensor, slots: torch.Tensor,
+                           penalty: torch.Tensor, last_n: torch.Tensor, history: torch.Tensor,
+                           seen: torch.Tensor) -> None:
+    """In place: for entry i the repeat penalty ``penalty[i]`` of row ``rows[i]`` over the last
+    ``last_n[i]`` tokens of ``history[slots[i]]``, once per occurrence as ``repeat_penalty``
+    applies it to a list."""
+    _gpu("logits", logits, F32)
+    _gpu("penalty", penalty, F32)
+    for name, t in (("rows", rows), ("slots", slots), ("last_n", last_n), ("history", history),
+                    ("seen", seen)):
+        _gpu(name, t, I32)
+    n = rows.shape[0]
+    _need(slots.shape == (n,) and penalty.shape == (n,) and last_n.shape == (n,)
+          and history.dim() == 2 and seen.shape == (history.shape[0],),
+          "repeat_penalty_history: tables per entry, a ring and a count per slot")
+    check(library("sampling").kappai_repeat_penalty_history(
+        _ptr(logits), _ptr(rows), _ptr(slots), _ptr(penalty), _ptr(last_n), _ptr(history),
+        _ptr(seen), _c_int(n), _c_int(logits.shape[1]), _c_int(history.shape[1]), _stream()),
+        "repeat_penalty_history")
+
+
+def history_append(chosen: torch.Tensor, rows: torch.Tensor, slots: torch.Tensor,
+                   history: torch.Tensor, seen: torch.Tensor) -> None:
+    """The token ``chosen[rows[i]]`` joins ``history[slots[i]]`` for every entry i."""
+    for name, t in (("chosen", chosen), ("rows", rows), ("slots", slots), ("history", history),
+                    ("seen", seen)):
+        _gpu(name, t, I32)
+    n = rows.shape[0]
+    _need(slots.shape == (n,) and history.dim() == 2 and seen.shape == (history.shape[0],),
+          "history_append: tables per entry, a ring and a count per slot")
+    check(library("sampling").kappai_history_append(
+        _ptr(chosen), _ptr(rows), _ptr(slots), _ptr(history), _ptr(seen), _c_int(n),
+        _c_int(history.shape[1]), _stream()), "history_append")

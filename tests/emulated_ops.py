@@ -216,10 +216,42 @@ def repeat_penalty(logits, row_start, tokens, penalty):
                 logits[r, tok] = logits[r, tok] / pen if logits[r, tok] > 0 else logits[r, tok] * pen
 
 
+def history_set(history, seen, slots, starts, tokens):
+    cap = history.shape[1]
+    for i in range(slots.shape[0]):
+        lo, hi = int(starts[i]), int(starts[i + 1])
+        n = min(hi - lo, cap)
+        history[int(slots[i]), :n] = tokens[lo:lo + n]
+        seen[int(slots[i])] = n
+
+
+def repeat_penalty_history(logits, rows, slots, penalty, last_n, history, seen):
+    cap = history.shape[1]
+    for i in range(rows.shape[0]):
+        pen = float(penalty[i])
+        if pen == 1.0:
+            continue
+        slot, total = int(slots[i]), int(seen[int(slots[i])])
+        n = min(int(last_n[i]), total, cap)
+        r = int(rows[i])
+        for j in range(total - n, total):
+            tok = int(history[slot, j % cap])
+            if 0 <= tok < logits.shape[1]:
+                logits[r, tok] = logits[r, tok] / pen if logits[r, tok] > 0 else logits[r, tok] * pen
+
+
+def history_append(chosen, rows, slots, history, seen):
+    cap = history.shape[1]
+    for i in range(rows.shape[0]):
+        slot = int(slots[i])
+        history[slot, int(seen[slot]) % cap] = chosen[int(rows[i])]
+        seen[slot] += 1
+
+
 ALL = ["embed_rows", "add_rmsnorm", "add_residual", "sum_partial_sums", "swiglu", "cast", "linear", "linear_swiglu",
        "interleave_gate_up", "shortconv", "linear_shortconv_step",
        "qk_norm_rope_store", "paged_attention", "sample_rows", "sample_filtered",
-       "repeat_penalty"]
+       "repeat_penalty", "history_set", "repeat_penalty_history", "history_append"]
 
 
 def install(monkeypatch):

@@ -121,6 +121,36 @@ def test_default_options_and_repeat_penalty(model_dirs):
         assert g == want, (i, g, want)
 
 
+def test_repeat_penalty_goes_ahead_of_its_tokens(model_dirs):
+    """Requests with a repeat penalty (windows of 8 and 64 tokens, one over the prompt's end)
+    beside requests without: the steps are queued before the tokens of the steps before them
+    have been read (the recent tokens are kept on the GPU), with so few pages that requests are
+    preempted and computed again, and every request's tokens are those of the plain
+    implementation with a plain sampler of the same seed, and those of a run in which every step
+    is waited for."""
+    from kappai_amd.engine import Engine, EngineConfig
+    from kappai_amd.sampling import SamplingParams
+    prompts = prompts_for("C", [9, 21, 14, 30, 5], seed=4)
+    opts = [dict(repeat_penalty=1.3, repeat_last_n=8), dict(repeat_penalty=1.6, repeat_last_n=64),
+            dict(), dict(repeat_penalty=1.15, repeat_last_n=3, temperature=0.0), dict()]
+    params = [SamplingParams(seed=50, n_predict=20, **o) for o in opts]
+    results = {}
+    for pipeline in (True, False):
+        eng = Engine(EngineConfig(model=str(model_dirs["C"]), dtype="float32", num_pages=14,
+                                  page_size=8, max_batch=4, chunk=6, token_budget=12,
+                                  pipeline=pipeline))
+        results[pipeline] = eng.generate(prompts, params)
+        if pipeline:
+            assert eng.pipelined_steps > 0, "nothing was queued ahead"
+            assert eng.scheduler.preempted_total > 0, "the pool was meant to be too small"
+        eng.shutdown()
+    assert results[True] == results[False]
+    for i, (p, g) in enumerate(zip(prompts, results[True])):
+        want, _ = plain_generate(model_dirs["C"], p, 20, lambda: S.PlainSampler(
+            50 + i, **{"top_k": 40, "top_p": 0.9, "min_p": 0.1, **opts[i]}))
+        assert g == want, (i, g, want)
+
+
 def test_greedy_bfloat16_follows_the_plain_logits(model_dirs):
     """In bfloat16 the chain may leave the plain one at a near tie; every token the engine
     picks must be (nearly) the best under the plain logits for the engine's own prefix."""

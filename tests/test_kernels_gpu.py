@@ -1493,3 +1493,38 @@ def test_repeat_penalty_of_long_windows_is_the_walk_over_the_list_bit_for_bit(op
                 v = want[r, t]
                 want[r, t] = v / pen[r] if v > 0 else v * pen[r]
     assert torch.equal(dev.cpu(), want)
+
+
+def test_token_history_on_the_gpu(ops):
+    """The rings of recent tokens: written anew for some slots, appended to token by token past
+    their capacity, and the repeat penalty over their last n tokens, against the same walk on the
+    host (bit for bit): windows shorter and longer than what a ring has seen, a window that
+    wraps round the ring's end, a token that comes up many times, a row without a penalty."""
+    g = torch.Generator().manual_seed(7)
+    cap, slots, V = 32, 5, 200
+    hist = torch.full((slots, cap), -7, dtype=torch.int32)
+    seen = torch.zeros(slots, dtype=torch.int32)
+    dh, ds = hist.to(DEV), seen.to(DEV)
+    first = {3: [5, 9, 5, 5, 1], 0: list(range(40, 40 + cap)), 4: [17]}
+    sl = torch.tensor(list(first), dtype=torch.int32)
+    starts = torch.tensor(np.cumsum([0] + [len(v) for v in first.values()]), dtype=torch.int32)
+    toks = torch.tensor([t for v in first.values() for t in v], dtype=torch.int32)
+    ops.history_set(dh, ds, sl.to(DEV), starts.to(DEV), toks.to(DEV))
+    ref.history_set(hist, seen, sl, starts, toks)
+    # 50 steps of three requests (rows 2, 0, 1 of the logits; slots 3, 0, 4)
+    rows = torch.tensor([2, 0, 1], dtype=torch.int32)
+    use = torch.tensor([3, 0, 4], dtype=torch.int32)
+    pen = torch.tensor([1.7, 1.2, 1.0])
+    last_n = torch.tensor([6, 64, 3], dtype=torch.int32)
+    for step in range(50):
+        logits = torch.randn(3, V, generator=g) * 2
+        dl = logits.to(DEV).clone()
+        ops.repeat_penalty_history(dl, rows.to(DEV), use.to(DEV), pen.to(DEV), last_n.to(DEV), dh, ds)
+        ref.repeat_penalty_history(logits, rows, use, pen, last_n, hist, seen)
+        assert torch.equal(dl.cpu(), logits), step
+        chosen = torch.randint(0, 12, (3,), generator=g, dtype=torch.int32)
+        ops.history_append(chosen.to(DEV), rows.to(DEV), use.to(DEV), dh, ds)
+        ref.history_append(chosen, rows, use, hist, seen)
+    assert torch.equal(dh.cpu(), hist) and torch.equal(ds.cpu(), seen)
+    assert seen.tolist() == [cap + 50, 0, 0, 55, 51]
+    assert (hist[1] == -7).all() and (hist[2] == -7).all()

@@ -27,8 +27,16 @@ def test_params():
 
 def test_what_the_host_has_to_see():
     """Steps may be queued ahead of their tokens for every way of drawing that needs no earlier
-    token of the row: only the repeat penalty does."""
+    token of the row from the host: the repeat penalty looks at earlier tokens, which are kept on
+    the GPU up to a window of ``HISTORY_CAP``; only a longer window needs the host's list."""
+    from kappai_amd.sampling.sampler import HISTORY_CAP
     plain = [RequestSampler(SamplingParams(top_k=k, top_p=0.9)) for k in (0, 40, 5000)]
     assert Sampler.runs_on_device(plain, 65536)
-    assert not Sampler.runs_on_device(plain + [RequestSampler(SamplingParams(repeat_penalty=1.1))],
-                                      65536)
+    assert Sampler.runs_on_device(plain + [RequestSampler(SamplingParams(repeat_penalty=1.1))],
+                                  65536)
+    assert Sampler.runs_on_device(
+        [RequestSampler(SamplingParams(repeat_penalty=1.1, repeat_last_n=HISTORY_CAP))], 65536)
+    assert not Sampler.runs_on_device(plain + [RequestSampler(SamplingParams(
+        repeat_penalty=1.1, repeat_last_n=HISTORY_CAP + 1))], 65536)
+    assert Sampler.runs_on_device([RequestSampler(SamplingParams(
+        repeat_penalty=1.0, repeat_last_n=HISTORY_CAP + 1))], 65536)
