@@ -28,8 +28,9 @@
 extern "C" {
 #endif
 
-#define KAPPAI_ENGINE_ABI 10         // bumped with every change of the structs below
+#define KAPPAI_ENGINE_ABI 11         // bumped with every change of the structs below
 #define KAPPAI_MAX_GROUPS 8          // paged groups a batch can carry block tables for
+#define KAPPAI_MAX_TABLES 8         // tables and numbers of the parts' own in a step
 
 // ---- the kernels' launchers, by address (they live in libraries of their own) ---------------
 typedef struct kappai_kernels {
@@ -285,11 +286,12 @@ typedef struct kappai_batch {
   const int* seg_pos0;              // [n_segments]
   const int* seg_slot;              // [n_segments]
   const int* logit_rows;            // [n_logit_rows]
-  const int* q_tiles;               // [n_tiles, 4] or null
-  int n_tiles;
-  const int* lone_rows;             // [n_lone_rows] or null: single decoded tokens beside prompt
-  int n_lone_rows;                  // portions that q_tiles leaves out
-  int max_lone_position;
+  // What the parts' own layouts made for this step (parts.base.StepTables): tables on the GPU
+  // and numbers, by the places the plan gave their names (CPlan.table / CPlan.number).  A table
+  // that was not laid out in this step is null with 0 rows, such a number is -1.
+  const int* tables[KAPPAI_MAX_TABLES];
+  int table_rows[KAPPAI_MAX_TABLES];        // the table's first dimension
+  int numbers[KAPPAI_MAX_TABLES];
   int n_groups;
   const int* block_tables[KAPPAI_MAX_GROUPS];   // [n_segments, max_blocks[g]]
   int max_blocks[KAPPAI_MAX_GROUPS];

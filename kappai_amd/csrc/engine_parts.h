@@ -36,6 +36,10 @@ typedef struct kappai_attention_mixer {
   int group;                        // which block tables of the batch
   int shared_cache;                 // reads the keys another call stored: q only, nothing stored
   const kappai_attention_kernels* mfma;
+  // places in kappai_batch::tables / numbers: the tiles of the step's segments ([tiles, 4]), the
+  // single rows left out of them, and the largest position among those (see AttentionTiles in
+  // parts/attention.py)
+  int tiles_table, lone_table, lone_number;
 } kappai_attention_mixer;
 
 // "feed_forward.swiglu" (parts/feed_forward.py)

@@ -234,6 +234,14 @@ kappai_carry attention_mixer(kappai_step* s, const void* desc, kappai_rows x, fl
   const float* sin_t = L.rot_mode ? L.sin_table : nullptr;
   const bool mfma_ok = q_bf16 && L.mfma != nullptr && ps % 16 == 0 && d % 16 == 0 && d <= 256 &&
                        q_stride % 8 == 0 && aligned16(q);
+  // the tables that the host's part asked the step for (AttentionTiles): the segments' tiles, the
+  // single rows left out of them and the largest of their positions
+  auto table_ok = [](int at) { return at >= 0 && at < KAPPAI_MAX_TABLES; };
+  const int* q_tiles = table_ok(L.tiles_table) ? b.tables[L.tiles_table] : nullptr;
+  const int n_tiles = table_ok(L.tiles_table) ? b.table_rows[L.tiles_table] : 0;
+  const int* lone_rows = table_ok(L.lone_table) ? b.tables[L.lone_table] : nullptr;
+  const int n_lone_rows = table_ok(L.lone_table) ? b.table_rows[L.lone_table] : 0;
+  const int max_lone_position = table_ok(L.lone_number) ? b.numbers[L.lone_number] : -1;
   if (mfma_ok && single && H / G <= 16) {
     const int n_keys = decode_keys(b, L);
     const int block_waves = L.mfma->decode_block_waves(H / G);
@@ -258,18 +266,18 @@ kappai_carry attention_mixer(kappai_step* s, const void* desc, kappai_rows x, fl
                                       b.row_pos, b.row_seg, tables, max_blocks, M, H, G, ps,
                                       L.window, L.scale, keys_per_split, n_splits, stream));
     }
-  } else if (mfma_ok && b.q_tiles != nullptr) {
-    LAUNCH(s, L.mfma->attn_prefill(q, q_stride, L.k_pool, L.v_pool, ctx, H * d, b.q_tiles,
-                                   b.n_tiles, b.row_pos, tables, max_blocks, H, G, ps, L.window,
+  } else if (mfma_ok && q_tiles != nullptr) {
+    LAUNCH(s, L.mfma->attn_prefill(q, q_stride, L.k_pool, L.v_pool, ctx, H * d, q_tiles,
+                                   n_tiles, b.row_pos, tables, max_blocks, H, G, ps, L.window,
                                    L.scale, 0, stream));
-    if (b.lone_rows != nullptr && b.n_lone_rows > 0) {
+    if (lone_rows != nullptr && n_lone_rows > 0) {
       // the single decoded tokens beside the portions: keys split over blocks
-      if (H / G > 16 || b.max_lone_position < 0) {
+      if (H / G > 16 || max_lone_position < 0) {
         api.fail(s, "rows left out of the tiles need the decode kernel and their largest position");
         return none;
       }
-      const int R = b.n_lone_rows;
-      int n_keys = b.max_lone_position + 1;
+      const int R = n_lone_rows;
+      int n_keys = max_lone_position + 1;
       if (L.window) n_keys = (n_keys < L.window ? n_keys : L.window) + 32;
       int keys_per_split, n_splits;
       kappai_decode_splits(L.mfma->keys_per_wave(), tune.decode_max_splits, tune.decode_waves, R,
@@ -277,7 +285,7 @@ kappai_carry attention_mixer(kappai_step* s, const void* desc, kappai_rows x, fl
       float* part_o = (float*)api.take(s, KAPPAI_REGION_BLOCK, (size_t)R * H * n_splits * d * 4);
       float* part_ml = (float*)api.take(s, KAPPAI_REGION_BLOCK, (size_t)R * H * n_splits * 2 * 4);
       LAUNCH(s, L.mfma->attn_decode_rows(q, q_stride, L.k_pool, L.v_pool, ctx, H * d, part_o,
-                                         part_ml, b.lone_rows, b.row_pos, b.row_seg, tables,
+                                         part_ml, lone_rows, b.row_pos, b.row_seg, tables,
                                          max_blocks, R, H, G, ps, L.window, L.scale,
                                          keys_per_split, n_splits, stream));
     }

@@ -35,9 +35,9 @@ class RowBatch:
     seg_slot[S] (the request's state slot), block_tables[g] [S, max_blocks] for every paged
     group g, logit_rows[n] (rows whose logits are wanted, in the order asked;
     ``logits_of_every_row``: these are the rows 0 .. T-1 in order, which the host knows and a
-    part that could fold the last norm into a product cannot read from the GPU), q_tiles: the
-    segments cut into runs of at most ``Model.q_tile_rows`` rows, laid out only when a part of
-    the model asks for it (the tiled attention kernel does)."""
+    part that could fold the last norm into a product cannot read from the GPU).  ``extra`` and
+    ``numbers``: what the parts' own ``StepTables`` laid out for this step, tables on the GPU and
+    ints on the host, by name."""
     n_rows: int
     n_segments: int
     n_logit_rows: int
@@ -50,14 +50,38 @@ class RowBatch:
     seg_pos0: torch.Tensor
     seg_slot: torch.Tensor
     logit_rows: torch.Tensor
-    q_tiles: Optional[torch.Tensor] = None      # [tiles, 4]: (segment, first row, rows, place)
-    # the single decoded tokens of a step that also holds prompt portions, when they are left out
-    # of q_tiles (``Part.lone_rows_from``): their rows, and the largest of their positions
-    lone_rows: Optional[torch.Tensor] = None
-    max_lone_position: int = -1
+    extra: Dict[str, torch.Tensor] = field(default_factory=dict)
+    numbers: Dict[str, int] = field(default_factory=dict)
     logits_of_every_row: bool = False
     block_tables: List[torch.Tensor] = field(default_factory=list)
     host: Dict[str, np.ndarray] = field(default_factory=dict)
+
+
+@dataclass
+class HostStep:
+    """What a ``StepTables`` builds from: the step's own tables on the host."""
+    arrays: Dict[str, np.ndarray]
+    sizes: Dict[str, object]
+    page_size: int
+
+
+def build_step_tables(tables, step: HostStep):
+    """Every family's arrays and numbers for this step: ({name: int32 array}, {name: int})."""
+    arrays: Dict[str, np.ndarray] = {}
+    numbers: Dict[str, int] = {}
+    for t in tables:
+        made, nums = t.build(step)
+        for name, a in made.items():
+            if name in arrays or name in step.arrays:
+                raise ValueError(f"two tables of a step are called {name!r}")
+            if a.dtype != np.int32:
+                raise ValueError(f"the table {name!r} of {t.family!r} is not int32")
+            arrays[name] = a
+        for name, v in nums.items():
+            if name in numbers:
+                raise ValueError(f"two numbers of a step are called {name!r}")
+            numbers[name] = int(v)
+    return arrays, numbers
 
 
 def tile_place(index: int, tiles_in_segment: int) -> int:
@@ -68,15 +92,12 @@ def tile_place(index: int, tiles_in_segment: int) -> int:
     return index | (tiles_in_segment << 16)
 
 
-def layout_rows(entries: Sequence[StepEntry], cache: CacheManager, vocab_size: int,
-                tile_rows: Optional[int] = None, lone_rows_from: Optional[int] = None):
+def layout_rows(entries: Sequence[StepEntry], cache: CacheManager, vocab_size: int, tables=()):
     """Host side of ``RowBatch``: checks the entries and lays the tables out as int32
-    arrays.  Returns (dict of arrays, sizes).  ``tile_rows``: cut the segments into tiles of at
-    most that many rows (``q_tiles``); None: no such table.  ``lone_rows_from``: in a step with
-    segments of several rows, the segments of a single row go into ``lone_rows`` instead of
-    ``q_tiles`` when the longest of their contexts has at least that many keys.  The tables are
-    made for all entries at once (a step of many single decoded tokens costs a few numpy calls,
-    not a few per entry)."""
+    arrays.  Returns (dict of arrays, sizes).  ``tables``: the ``StepTables`` of the model's
+    parts, whose arrays join the dict (their names in ``sizes["extra"]``, their numbers in
+    ``sizes["numbers"]``).  The tables are made for all entries at once (a step of many single
+    decoded tokens costs a few numpy calls, not a few per entry)."""
     if not entries:
         raise ValueError("a step needs at least one entry")
     S = len(entries)
@@ -127,26 +148,6 @@ def layout_rows(entries: Sequence[StepEntry], cache: CacheManager, vocab_size: i
         "seg_slot": np.asarray(slots, dtype=np.int32),
         "logit_rows": np.asarray(logit_rows, dtype=np.int32),
     }
-    max_lone_position = -1
-    if tile_rows:
-        # tile j of a segment: (segment, first row, rows, place); the fourth number tells a kernel
-        # where the tile stands in its segment (index | tiles of the segment << 16, or 0 when the
-        # segment has more tiles than 15 bits hold), so that it can pair tiles of one segment
-        nt = (n_arr + tile_rows - 1) // tile_rows
-        lone = n_arr == 1
-        if (lone_rows_from and lone.any() and not lone.all() and cache.page_size % 16 == 0
-                and int(p0_arr[lone].max()) + 1 >= lone_rows_from):
-            arrays["lone_rows"] = seg_start[:-1][lone].astype(np.int32)
-            max_lone_position = int(p0_arr[lone].max())
-            nt = np.where(lone, 0, nt)
-        tile_seg = np.repeat(np.arange(S, dtype=np.int64), nt)
-        first_tile = np.cumsum(nt) - nt
-        idx = np.arange(int(nt.sum()), dtype=np.int64) - np.repeat(first_tile, nt)
-        rows = np.minimum(tile_rows, n_arr[tile_seg] - idx * tile_rows)
-        nts = nt[tile_seg]
-        place = np.where(nts > 0x7fff, 0, idx | (nts << 16))
-        arrays["q_tiles"] = np.stack(
-            [tile_seg, seg_start[tile_seg] + idx * tile_rows, rows, place], axis=1).astype(np.int32)
     n_groups = len(cache.paged_groups)
     for gi in range(n_groups):
         width = max(1, max(len(e.cache.blocks[gi]) for e in entries))
@@ -158,7 +159,11 @@ def layout_rows(entries: Sequence[StepEntry], cache: CacheManager, vocab_size: i
     sizes = {
         "n_rows": T, "n_segments": S, "n_logit_rows": len(logit_rows),
         "max_position": max_position, "max_segment_rows": int(n_arr.max()),
-        "n_groups": n_groups, "max_lone_position": max_lone_position,
+        "n_groups": n_groups,
         "logits_of_every_row": logit_rows == list(range(T)),
     }
+    extra, numbers = build_step_tables(tables, HostStep(arrays, sizes, cache.page_size))
+    arrays.update(extra)
+    sizes["extra"] = list(extra)
+    sizes["numbers"] = numbers
     return arrays, sizes

@@ -24,8 +24,9 @@ from ..parts.cdesc import (AttentionKernels, CallDesc, CarryDesc, CPlan, Embedde
                            FoldDesc, LinearDesc, NormPartDesc, PartDesc, RowsDesc, address_of,
                            defined_together)
 
-ENGINE_ABI = 10
+ENGINE_ABI = 11
 MAX_GROUPS = 8
+MAX_TABLES = 8         # KAPPAI_MAX_TABLES
 
 
 def _ptrs(names):
@@ -62,9 +63,9 @@ class BatchDesc(Structure):
         ("max_segment_rows", c_int), ("logits_of_every_row", c_int),
         ("tokens", c_void_p), ("row_pos", c_void_p),
         ("row_seg", c_void_p), ("seg_start", c_void_p), ("seg_pos0", c_void_p),
-        ("seg_slot", c_void_p), ("logit_rows", c_void_p), ("q_tiles", c_void_p),
-        ("n_tiles", c_int), ("lone_rows", c_void_p), ("n_lone_rows", c_int),
-        ("max_lone_position", c_int), ("n_groups", c_int),
+        ("seg_slot", c_void_p), ("logit_rows", c_void_p),
+        ("tables", c_void_p * MAX_TABLES), ("table_rows", c_int * MAX_TABLES),
+        ("numbers", c_int * MAX_TABLES), ("n_groups", c_int),
         ("block_tables", c_void_p * MAX_GROUPS),
         ("max_blocks", c_int * MAX_GROUPS)]
 
@@ -200,11 +201,14 @@ class CForward:
         b.seg_start, b.seg_pos0, b.seg_slot = (batch.seg_start.data_ptr(), batch.seg_pos0.data_ptr(),
                                                batch.seg_slot.data_ptr())
         b.logit_rows = batch.logit_rows.data_ptr()
-        if batch.q_tiles is not None:
-            b.q_tiles, b.n_tiles = batch.q_tiles.data_ptr(), batch.q_tiles.shape[0]
-        if batch.lone_rows is not None:
-            b.lone_rows, b.n_lone_rows = batch.lone_rows.data_ptr(), batch.lone_rows.shape[0]
-            b.max_lone_position = batch.max_lone_position
+        for at, name in enumerate(self.plan.tables):
+            t = batch.extra.get(name)
+            if t is not None:
+                b.tables[at], b.table_rows[at] = t.data_ptr(), t.shape[0]
+        for at in range(MAX_TABLES):
+            b.numbers[at] = -1
+        for at, name in enumerate(self.plan.numbers):
+            b.numbers[at] = batch.numbers.get(name, -1)
         if len(batch.block_tables) > MAX_GROUPS:
             raise ValueError(f"a step carries block tables for at most {MAX_GROUPS} groups")
         b.n_groups = len(batch.block_tables)

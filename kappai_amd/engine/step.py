@@ -18,7 +18,7 @@ import torch
 from ..cache.manager import CacheManager, OutOfPages, RequestCache
 from ..kernels import ops, profile
 from ..models.base import Model
-from .batch import RowBatch, StepEntry, layout_rows
+from .batch import HostStep, RowBatch, StepEntry, build_step_tables, layout_rows
 from .cforward import CForward, NotDescribed, Workspace
 
 
@@ -60,9 +60,19 @@ class _DecodeGraph:
         self.B, self.n_logit, self.width = B, n_logit, ctx_cap // cache.page_size + 1
         shapes = [("tokens", (B,)), ("row_pos", (B,)), ("row_seg", (B,)), ("seg_start", (B + 1,)),
                   ("seg_pos0", (B,)), ("seg_slot", (B,)), ("logit_rows", (n_logit,))]
-        tiled = bool(runner.model.q_tile_rows)
-        if tiled:
-            shapes.append(("q_tiles", (B, 4)))
+        # the parts' own tables, as they come out for B single rows
+        self.tables = list(runner.step_tables)
+        self.sizes = {"n_rows": B, "n_segments": B, "n_logit_rows": n_logit,
+                      "max_position": ctx_cap - 1, "max_segment_rows": 1, "n_groups": n_groups,
+                      "logits_of_every_row": n_logit == B}
+        z = np.zeros(B, dtype=np.int32)
+        extra, numbers = build_step_tables(self.tables, HostStep(
+            {"tokens": z, "row_pos": z, "row_seg": np.arange(B, dtype=np.int32),
+             "seg_start": np.arange(B + 1, dtype=np.int32), "seg_pos0": z, "seg_slot": z,
+             "logit_rows": (np.arange(n_logit) % B).astype(np.int32)}, self.sizes,
+            cache.page_size))
+        self.numbers = numbers
+        shapes += [(name, a.shape) for name, a in extra.items()]
         shapes += [("place_dst", (B,)), ("place_src", (B,))]
         shapes += [(f"block_table_{g}", (B, self.width)) for g in range(n_groups)]
         self.offsets, total = {}, 0
@@ -82,17 +92,17 @@ class _DecodeGraph:
             n_rows=B, n_segments=B, n_logit_rows=n_logit, max_position=ctx_cap - 1,
             max_segment_rows=1, tokens=views["tokens"], row_pos=views["row_pos"],
             row_seg=views["row_seg"], seg_start=views["seg_start"], seg_pos0=views["seg_pos0"],
-            seg_slot=views["seg_slot"], logit_rows=views["logit_rows"], q_tiles=views.get("q_tiles"),
+            seg_slot=views["seg_slot"], logit_rows=views["logit_rows"],
+            extra={name: views[name] for name in extra}, numbers=dict(numbers),
             block_tables=[views[f"block_table_{g}"] for g in range(n_groups)], host={},
             logits_of_every_row=n_logit == B)
         # what never changes
         self.h["row_seg"][:] = np.arange(B)
         self.h["seg_start"][:] = np.arange(B + 1)
-        if tiled:
-            self.h["q_tiles"][:, 0] = np.arange(B)
-            self.h["q_tiles"][:, 1] = np.arange(B)
-            self.h["q_tiles"][:, 2] = 1
-            self.h["q_tiles"][:, 3] = 1 << 16         # tile 0 of 1 in its segment
+        for name, a in extra.items():
+            self.h[name][...] = a
+        # tables that depend on more than the number of rows are built again for every replay
+        self.rebuilt = [t for t in self.tables if not t.decode_constant]
         # a warm-up run on the scratch page and the scratch slot: every kernel of this shape is
         # loaded and has run once before the capture, and no request's cache is touched
         self.h["seg_slot"][:] = cache.scratch_slot
@@ -174,6 +184,19 @@ class _DecodeGraph:
                 for g, page in enumerate(self.scratch[1]):
                     h[f"block_table_{g}"][si] = page
                 self.rows_of[si] = None
+        if self.rebuilt:
+            made, nums = build_step_tables(self.rebuilt, HostStep(
+                {k: h[k] for k in ("tokens", "row_pos", "row_seg", "seg_start", "seg_pos0",
+                                   "seg_slot", "logit_rows")}, self.sizes,
+                runner.cache.page_size))
+            for name, a in made.items():
+                if name not in h or a.shape != h[name].shape:
+                    raise RuntimeError(f"the table {name!r} changed its shape between the steps of "
+                                       f"a captured graph; its part must not be capturable")
+                h[name][...] = a
+            if any(self.numbers.get(k) != v for k, v in nums.items()):
+                raise RuntimeError("a number that a launch is sized by changed between the steps "
+                                   "of a captured graph; its part must not be capturable")
         self._upload(runner, keep_tokens=tokens_in_place)
         if tokens_in_place:
             pass
@@ -207,6 +230,9 @@ class StepRunner:
         self._graphs = {}
         self._graph_seen = {}
         self.graph_replays = 0
+        # what the model's parts want laid out beside the step's own tables
+        tables = getattr(model, "step_tables", None)
+        self.step_tables = list(tables()) if callable(tables) else []
 
     # -- the forward pass of a step ----------------------------------------------------------
     def forward(self, batch: RowBatch, workspace: Optional[Workspace] = None) -> torch.Tensor:
@@ -263,9 +289,7 @@ class StepRunner:
 
     def make_batch(self, entries: Sequence[StepEntry], placed=None) -> RowBatch:
         """``placed``: see ``step``."""
-        arrays, sizes = layout_rows(entries, self.cache, self.model.vocab_size,
-                                    getattr(self.model, "q_tile_rows", None),
-                                    getattr(self.model, "lone_rows_from", None))
+        arrays, sizes = layout_rows(entries, self.cache, self.model.vocab_size, self.step_tables)
         if placed is not None and placed[1]:
             chosen, pairs = placed
             for ei, at in pairs:
@@ -282,9 +306,8 @@ class StepRunner:
             max_segment_rows=sizes["max_segment_rows"],
             tokens=dev["tokens"], row_pos=dev["row_pos"], row_seg=dev["row_seg"],
             seg_start=dev["seg_start"], seg_pos0=dev["seg_pos0"], seg_slot=dev["seg_slot"],
-            logit_rows=dev["logit_rows"], q_tiles=dev.get("q_tiles"),
-            lone_rows=dev.get("lone_rows"), max_lone_position=sizes["max_lone_position"],
-            logits_of_every_row=sizes["logits_of_every_row"],
+            logit_rows=dev["logit_rows"], extra={name: dev[name] for name in sizes["extra"]},
+            numbers=sizes["numbers"], logits_of_every_row=sizes["logits_of_every_row"],
             block_tables=[dev[f"block_table_{g}"] for g in range(sizes["n_groups"])],
             host=arrays)
 

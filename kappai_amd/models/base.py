@@ -100,23 +100,17 @@ class Model:
         """True if every part allows decode steps to be captured in HIP graphs."""
         return all(getattr(p, "capturable", True) for p in self._parts())
 
-    @property
-    def q_tile_rows(self) -> Optional[int]:
-        """Rows of the tiles that the step function cuts segments into for the parts that ask for
-        such a table (None: nobody does)."""
-        asked = {r for r in (getattr(b, "q_tile_rows", None) for b in self.layers) if r}
-        if len(asked) > 1:
-            raise ValueError(f"the layers ask for tiles of different sizes: {sorted(asked)}")
-        return asked.pop() if asked else None
-
-    @property
-    def lone_rows_from(self) -> Optional[int]:
-        """The context length from which the single decoded tokens of a mixed step are listed
-        apart from the tiles (None: never): only when every part that asks for tiles says the
-        same."""
-        tiled = [b for b in self.layers if getattr(b, "q_tile_rows", None)]
-        asked = {getattr(b, "lone_rows_from", None) for b in tiled}
-        return asked.pop() if len(asked) == 1 else None
+    def step_tables(self) -> list:
+        """The tables that the parts ask of a step beside the framework's own
+        (``parts.base.StepTables``), one set per family."""
+        families = {}
+        for part in [*self.layers, self.embedding_position]:
+            asked = getattr(part, "step_tables", None)
+            if asked is None:
+                continue
+            for t in (asked if isinstance(asked, (list, tuple)) else [asked]):
+                families.setdefault(t.family, []).append(t)
+        return [ts[0].combine(ts[1:]) for ts in families.values()]
 
     @property
     def vocab_size(self) -> int:

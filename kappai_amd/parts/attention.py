@@ -11,8 +11,10 @@ projection.
 from __future__ import annotations
 
 import math
+from dataclasses import dataclass
 from typing import Dict, List, Optional
 
+import numpy as np
 import torch
 
 from ..cache.specs import PagedKV
@@ -21,7 +23,7 @@ from ..weights.spec import INIT_ONES, VECTOR, TensorSpec
 import ctypes
 from ctypes import POINTER, Structure, c_float, c_int, c_void_p
 
-from .base import Mixer, PositionEncoding, register_part
+from .base import Mixer, PositionEncoding, StepTables, register_part
 from .cdesc import AttentionKernels, LinearDesc, tensor_ptr
 from .linear import Linear
 
@@ -34,13 +36,62 @@ class AttentionMixerDesc(Structure):
         ("window", c_int), ("scale", c_float), ("cos_table", c_void_p), ("sin_table", c_void_p),
         ("rot_dim", c_int), ("rot_mode", c_int), ("rot_positions", c_int), ("k_pool", c_void_p),
         ("v_pool", c_void_p), ("group", c_int), ("shared_cache", c_int),
-        ("mfma", POINTER(AttentionKernels))]
+        ("mfma", POINTER(AttentionKernels)), ("tiles_table", c_int), ("lone_table", c_int),
+        ("lone_number", c_int)]
+
+
+@dataclass(frozen=True)
+class AttentionTiles(StepTables):
+    """What the tiled attention kernel walks: ``q_tiles`` [tiles, 4], the segments cut into runs
+    of at most ``rows`` rows, tile j of a segment as (segment, first row, rows, place); the
+    fourth number tells a kernel where the tile stands in its segment (index | tiles of the
+    segment << 16, or 0 when the segment has more tiles than 15 bits hold), so that it can pair
+    tiles of one segment.  ``lone_from``: in a step that holds segments of several rows, the
+    segments of a single row are left out of the tiles and listed in ``lone_rows`` (with the
+    number ``max_lone_position``) when the longest of their contexts has at least that many
+    keys: the block that got such a row as a tile would walk all its keys alone, so these rows
+    go to the decode kernel."""
+    rows: int
+    lone_from: Optional[int] = None
+
+    family = "attention_tiles"
+    decode_constant = True
+
+    def combine(self, others):
+        rows = {self.rows} | {o.rows for o in others}
+        if len(rows) > 1:
+            raise ValueError(f"the layers ask for tiles of different sizes: {sorted(rows)}")
+        lone = {self.lone_from} | {o.lone_from for o in others}
+        return AttentionTiles(self.rows, lone.pop() if len(lone) == 1 else None)
+
+    def build(self, step):
+        seg_start = step.arrays["seg_start"].astype(np.int64)
+        p0 = step.arrays["seg_pos0"].astype(np.int64)
+        n = seg_start[1:] - seg_start[:-1]
+        S = n.shape[0]
+        arrays, numbers = {}, {"max_lone_position": -1}
+        nt = (n + self.rows - 1) // self.rows
+        lone = n == 1
+        if (self.lone_from and lone.any() and not lone.all() and step.page_size % 16 == 0
+                and int(p0[lone].max()) + 1 >= self.lone_from):
+            arrays["lone_rows"] = seg_start[:-1][lone].astype(np.int32)
+            numbers["max_lone_position"] = int(p0[lone].max())
+            nt = np.where(lone, 0, nt)
+        tile_seg = np.repeat(np.arange(S, dtype=np.int64), nt)
+        first_tile = np.cumsum(nt) - nt
+        idx = np.arange(int(nt.sum()), dtype=np.int64) - np.repeat(first_tile, nt)
+        rows = np.minimum(self.rows, n[tile_seg] - idx * self.rows)
+        nts = nt[tile_seg]
+        place = np.where(nts > 0x7fff, 0, idx | (nts << 16))
+        arrays["q_tiles"] = np.stack(
+            [tile_seg, seg_start[tile_seg] + idx * self.rows, rows, place],
+            axis=1).astype(np.int32)
+        return arrays, numbers
 
 
 class GroupedQueryAttention(Mixer):
     takes_deferred_rows = True     # its first product takes what ops.linear takes
     adds_residual = True           # its last product can add into the residual stream
-    q_tile_rows = ops.ATTENTION_TILE_ROWS     # the tiled attention kernel's rows a tile
 
     def __init__(self, prefix: str, width: int, num_heads: int, num_kv_heads: int, head_dim: int,
                  dtype: torch.dtype, position: Optional[PositionEncoding] = None,
@@ -68,11 +119,13 @@ class GroupedQueryAttention(Mixer):
         self.k_norm_w: Optional[torch.Tensor] = None
 
     @property
-    def lone_rows_from(self) -> Optional[int]:
-        # (what the decode kernel needs; the page size is checked where the table is laid out)
+    def step_tables(self) -> AttentionTiles:
+        # single rows beside portions: what the decode kernel needs (the page size is checked
+        # where the table is laid out)
         ok = (self.dtype == torch.bfloat16 and self.H // self.G <= 16 and self.d % 16 == 0
               and self.d <= 256)
-        return tuning.LONE_ROWS_FROM if ok and tuning.LONE_ROWS_FROM else None
+        return AttentionTiles(ops.ATTENTION_TILE_ROWS,
+                              tuning.LONE_ROWS_FROM if ok and tuning.LONE_ROWS_FROM else None)
 
     def cache_spec(self):
         return PagedKV(self.G, self.d, self.window)
@@ -123,11 +176,12 @@ class GroupedQueryAttention(Mixer):
         with profile.scope("attn"):
             ctx = ops.paged_attention(q, H, G, d, k_pool, v_pool, batch.row_pos,
                                       batch.row_seg, tables, cache.page_size, self.scale,
-                                      window=self.window or 0, q_tiles=batch.q_tiles,
-                                      single_rows=single,
+                                      window=self.window or 0,
+                                      q_tiles=batch.extra.get("q_tiles"), single_rows=single,
                                       max_position=batch.max_position,
-                                      lone_rows=getattr(batch, "lone_rows", None),
-                                      max_lone_position=getattr(batch, "max_lone_position", -1))
+                                      lone_rows=batch.extra.get("lone_rows"),
+                                      max_lone_position=batch.numbers.get("max_lone_position",
+                                                                          -1))
         return self.out.forward(ctx, partial_sums=True, add_into=into)
 
     def c_part(self, plan, view, shared_cache: bool = False):
@@ -145,6 +199,8 @@ class GroupedQueryAttention(Mixer):
         d.group = view.group
         d.shared_cache = 1 if shared_cache else 0
         d.rot_mode = ops.ROT_NONE
+        d.tiles_table, d.lone_table = plan.table("q_tiles"), plan.table("lone_rows")
+        d.lone_number = plan.number("max_lone_position")
         if plan.bf16 and self.d % 16 == 0 and self.d <= 256:
             d.mfma = ctypes.pointer(plan.attention_kernels(self.d))
         if self.position is not None:

@@ -20,6 +20,36 @@ import torch
 from ..weights.spec import TensorSpec
 
 
+class StepTables:
+    """More int32 tables of a step, laid out on the host for a part whose kernels want them (the
+    segments cut into tiles, some rows listed apart, the chunks of a scan, ...).
+
+    ``family``: tables of one family are built once a step, however many layers ask for them;
+    ``combine`` says what is built when the layers ask differently.  ``build(step)`` gets the
+    step's own tables on the host (``step.arrays``: tokens, row_pos, row_seg, seg_start,
+    seg_pos0, seg_slot, logit_rows as numpy int32 arrays; ``step.sizes``: n_rows, n_segments,
+    max_position, max_segment_rows; ``step.page_size``) and returns ``(arrays, numbers)``: more
+    int32 arrays by name, and ints by name that stay on the host (what a launch is sized by).
+    Names are the family's own; an array that is not needed in a step is left out.
+    ``decode_constant``: in a step of nothing but single rows the arrays depend on the number of
+    rows only, so that a captured decode graph fills them in once; else they are built again for
+    every replay and must keep their shapes."""
+
+    family: str = ""
+    decode_constant: bool = False
+
+    def build(self, step):
+        raise NotImplementedError
+
+    def combine(self, others: List["StepTables"]) -> "StepTables":
+        """The one set of tables for ``self`` and ``others`` of the same family."""
+        for o in others:
+            if o != self:
+                raise ValueError(f"layers ask for different tables of the family {self.family!r}: "
+                                 f"{self!r} and {o!r}")
+        return self
+
+
 class Part:
     """Anything that owns tensors of the checkpoint."""
 
@@ -28,15 +58,10 @@ class Part:
     # part that reads the batch's tables on the host sets this to False.
     capturable = True
 
-    # Rows of a tile if the part's kernels want the step's segments cut into tiles of at most
-    # that many rows (``RowBatch.q_tiles``); None: the table is not laid out for this part.
-    q_tile_rows: Optional[int] = None
-
-    # A part that asks for tiles may run the single decoded tokens of a step that also holds
-    # prompt portions through another kernel when their context is long: from this many keys on
-    # (the step's longest such context decides for all of them) they are left out of the tile
-    # table and listed in ``RowBatch.lone_rows`` instead.  None: every row is in a tile.
-    lone_rows_from: Optional[int] = None
+    # More tables of the step that the part's kernels want beside the framework's own (a
+    # ``StepTables``), or None.  The step function builds them on the host with its own tables and
+    # brings them to the GPU in the same copy: ``RowBatch.extra[name]``, ``RowBatch.numbers[name]``.
+    step_tables: Optional["StepTables"] = None
 
     def tensor_specs(self) -> List[TensorSpec]:
         """Full names, shapes and roles of the tensors this part reads from the file."""
@@ -150,6 +175,12 @@ class Block(Part):
 
     def cache_spec(self):
         return self.mixer.cache_spec()
+
+    @property
+    def step_tables(self):
+        """The tables its parts ask of a step (a list)."""
+        asked = getattr(self.mixer, "step_tables", None)
+        return [] if asked is None else [asked]
 
     def forward(self, h: Hidden, batch, cache, shared_cache: bool = False) -> Hidden:
         raise NotImplementedError

@@ -40,12 +40,8 @@ class PreNormBlock(Block):
         return all(p.capturable for p in self._parts())
 
     @property
-    def q_tile_rows(self):
-        return self.mixer.q_tile_rows
-
-    @property
-    def lone_rows_from(self):
-        return self.mixer.lone_rows_from
+    def step_tables(self):
+        return [t for t in (p.step_tables for p in self._parts()) if t is not None]
 
     def tensor_specs(self) -> List[TensorSpec]:
         return [s for p in self._parts() for s in p.tensor_specs()]

@@ -104,6 +104,8 @@ class CPlan:
         self._keep: List[object] = []
         self._before_step: List[Callable] = []
         self._mfma = {}
+        self.tables: List[str] = []       # names of the parts' own step tables, by their place
+        self.numbers: List[str] = []      # in kappai_batch::tables / numbers
         engine_lib.kappai_runner.restype = c_void_p
         engine_lib.kappai_runner.argtypes = [ctypes.c_char_p, c_int, POINTER(c_int)]
         engine_lib.kappai_register_runner.argtypes = [ctypes.c_char_p, c_int, c_void_p, c_int]
@@ -121,6 +123,27 @@ class CPlan:
     def before_step(self, batch) -> None:
         for fn in self._before_step:
             fn(batch)
+
+    # -- the parts' own tables of a step -----------------------------------------------------------
+    MAX_TABLES = 8
+
+    def table(self, name: str) -> int:
+        """The place in ``kappai_batch::tables`` where the runner finds ``RowBatch.extra[name]``
+        (what the part's ``StepTables`` lays out under that name)."""
+        return self._place(self.tables, name)
+
+    def number(self, name: str) -> int:
+        """The place in ``kappai_batch::numbers`` of ``RowBatch.numbers[name]``."""
+        return self._place(self.numbers, name)
+
+    def _place(self, names: List[str], name: str) -> int:
+        if name not in names:
+            if len(names) >= self.MAX_TABLES:
+                from ..kernels.lib import KernelLaunchError
+                raise KernelLaunchError(f"a step carries at most {self.MAX_TABLES} tables and "
+                                        f"numbers of the parts' own")
+            names.append(name)
+        return names.index(name)
 
     # -- runners ---------------------------------------------------------------------------------
     def register_runner(self, name: str, kind: int, fn, desc_type) -> None:

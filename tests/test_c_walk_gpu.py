@@ -387,14 +387,6 @@ def define_toy_block():
 
         capturable = True
 
-        @property
-        def q_tile_rows(self):
-            return self.mixer.q_tile_rows
-
-        @property
-        def lone_rows_from(self):
-            return self.mixer.lone_rows_from
-
         def tensor_specs(self):
             return [t for p in self._parts() for t in p.tensor_specs()]
 
@@ -636,6 +628,7 @@ def define_toy_positions():
     from kappai_amd.models import Model
     from kappai_amd.parts import (POSITION_ENCODINGS, OutputHead, PositionEncoding,
                                   TokenEmbedding, make_part, register_part)
+    from kappai_amd.parts.base import StepTables
     from kappai_amd.parts.cdesc import RUNNER_EMBEDDED
     from kappai_amd.weights.spec import INIT_NORMAL, TABLE, TensorSpec
     if "toy_learned_hip" in POSITION_ENCODINGS:
@@ -643,13 +636,34 @@ def define_toy_positions():
 
     class PositionsDesc(Structure):
         """``toy_learned_positions`` of tests/toy_parts/learned_positions.hip."""
-        _fields_ = [("table", c_void_p), ("table_is_bf16", c_int), ("positions", c_int)]
+        _fields_ = [("table", c_void_p), ("table_is_bf16", c_int), ("positions", c_int),
+                    ("rows_table", c_int)]
+
+    class TableRows(StepTables):
+        """A table of the step that the part lays out itself, on the host: the table's row for
+        every row of the step (its position, the last row for anything beyond).  It depends on the
+        positions, so a captured decode graph has it built again for every replay."""
+        family = "toy_table_rows"
+        decode_constant = False
+
+        def __init__(self, n):
+            self.n = n
+
+        def __eq__(self, other):
+            return isinstance(other, TableRows) and other.n == self.n
+
+        def build(self, step):
+            TableRows.built += 1
+            return {"toy_table_rows": np.minimum(step.arrays["row_pos"], self.n - 1).astype(np.int32)}, {}
+
+    TableRows.built = 0
 
     class LearnedPositionsHip(PositionEncoding):
         """x_t += table[position of t]."""
 
         def __init__(self, name, n_positions, width):
             self.name, self.n, self.width = name, n_positions, width
+            self.step_tables = TableRows(n_positions)
 
         def tensor_specs(self):
             return [TensorSpec(self.name + ".weight", (self.n, self.width), TABLE, INIT_NORMAL)]
@@ -661,8 +675,8 @@ def define_toy_positions():
             rc = toy_positions_library().toy_add_positions_launch(
                 c_void_p(x.data_ptr()), c_void_p(self.table.data_ptr()),
                 c_int(1 if self.table.dtype == torch.bfloat16 else 0),
-                c_void_p(batch.row_pos.data_ptr()), c_int(x.shape[0]), c_int(self.width),
-                c_int(self.n), ops._stream())
+                c_void_p(batch.extra["toy_table_rows"].data_ptr()), c_int(x.shape[0]),
+                c_int(self.width), c_int(self.n), ops._stream())
             assert rc == 0, rc
 
         def c_embedded(self, plan):
@@ -671,7 +685,8 @@ def define_toy_positions():
             plan.register_runner("embedded.toy_learned", RUNNER_EMBEDDED,
                                  lib.toy_learned_positions_run, PositionsDesc)
             return plan.embedded("embedded.toy_learned", PositionsDesc(
-                self.table.data_ptr(), 1 if self.table.dtype == torch.bfloat16 else 0, self.n))
+                self.table.data_ptr(), 1 if self.table.dtype == torch.bfloat16 else 0, self.n,
+                plan.table("toy_table_rows")))
 
     register_part("position_encoding", "toy_learned_hip", LearnedPositionsHip)
 
@@ -729,9 +744,11 @@ TOY_POSITIONS = {"architectures": ["ToyPositionsForCausalLM"], "width": 64, "voc
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_positions_added_to_the_embedded_rows_run_from_c(tmp_path, dtype):
     """A learned row per position added to the embedded rows by a kernel from outside, attention
-    without rotation: from C bit for bit what the host's walk gives under the mixed schedule,
-    with and without graphs; and the model does depend on the positions (a request whose table
-    rows are moved gives other logits)."""
+    without rotation, the kernel reading a table of the step that the part lays out itself
+    (``StepTables``, beside the attention's tiles; built again for every replay of a decode
+    graph): from C bit for bit what the host's walk gives under the mixed schedule, with and
+    without graphs; and the model does depend on the positions (a request whose table rows are
+    moved gives other logits)."""
     import schedules
     from kappai_amd.config import config_from_dict
     from kappai_amd.models import load_model
@@ -750,6 +767,10 @@ def test_positions_added_to_the_embedded_rows_run_from_c(tmp_path, dtype):
             res, runner = replay(model, steps, peak, tmp_path / f"p{c_forward}g{graphs}",
                                  c_forward, graphs)
             assert (runner._cplan is not None) == c_forward
+            assert sorted(t.family for t in runner.step_tables) == ["attention_tiles",
+                                                                    "toy_table_rows"]
+            if graphs:
+                assert runner.graph_replays > 0
             results[(c_forward, graphs)] = res
     base = results[(False, False)]
     for key, res in results.items():

@@ -29,7 +29,9 @@ def one_segment_batch(cm, n, rid="r", first=True, rc=None):
     cm.extend(rc, n)
     runner = StepRunner.__new__(StepRunner)
     from kappai_amd.kernels import ops
-    runner.model = type("M", (), {"vocab_size": 10 ** 9, "q_tile_rows": ops.ATTENTION_TILE_ROWS})()
+    from kappai_amd.parts.attention import AttentionTiles
+    runner.model = type("M", (), {"vocab_size": 10 ** 9})()
+    runner.step_tables = [AttentionTiles(ops.ATTENTION_TILE_ROWS)]
     runner.cache, runner.device, runner._staging, runner._staged = cm, torch.device(DEV), None, None
     batch = runner.make_batch([StepEntry(rc, [0] * n, [])])
     return rc, batch

@@ -389,7 +389,8 @@ def test_decoded_tokens_over_long_contexts_beside_prompt_portions(tmp_path, dtyp
     results = {}
     for c_forward in (True, False):
         model = gpu_model(folder, dtype)
-        assert model.lone_rows_from == (1024 if dtype == "bfloat16" else None)
+        (tiles,) = model.step_tables()
+        assert tiles.lone_from == (1024 if dtype == "bfloat16" else None)
         cache = make_replay_cache(model, peak)
         cache.allocate_storage(model.dtype, "cuda:0", poison=True)
         runner = StepRunner(model, cache, "cuda:0", c_forward=c_forward)
@@ -398,7 +399,8 @@ def test_decoded_tokens_over_long_contexts_beside_prompt_portions(tmp_path, dtyp
 
         def spy(entries, placed=None):
             batch = make(entries, placed)
-            seen.append(None if batch.lone_rows is None else batch.lone_rows.tolist())
+            lone = batch.extra.get("lone_rows")
+            seen.append(None if lone is None else lone.tolist())
             return batch
 
         runner.make_batch = spy
