@@ -151,6 +151,28 @@ def test_repeat_penalty_goes_ahead_of_its_tokens(model_dirs):
         assert g == want, (i, g, want)
 
 
+def test_repeat_penalty_over_a_window_longer_than_the_ring(model_dirs):
+    """A repeat penalty over the last 300 tokens (more than the 256 kept on the GPU) beside one
+    over 8: such steps take the host's lists and are waited for, and when the long window's
+    request has ended the other goes on from its ring, which is written anew; every request's
+    tokens are the plain implementation's."""
+    from kappai_amd.engine import Engine
+    from kappai_amd.sampling import SamplingParams
+    prompts = prompts_for("C", [310, 12], seed=6)
+    opts = [dict(repeat_penalty=1.4, repeat_last_n=300, n_predict=6),
+            dict(repeat_penalty=1.3, repeat_last_n=8, n_predict=24)]
+    params = [SamplingParams(seed=60, **o) for o in opts]
+    eng = Engine(str(model_dirs["C"]), dtype="float32", num_pages=64, max_batch=2)
+    got = eng.generate(prompts, params)
+    assert eng.pipelined_steps > 0, "the steps after the long window's end were meant to go ahead"
+    for i, (p, g) in enumerate(zip(prompts, got)):
+        o = dict(opts[i])
+        n = o.pop("n_predict")
+        want, _ = plain_generate(model_dirs["C"], p, n, lambda: S.PlainSampler(
+            60 + i, **{"top_k": 40, "top_p": 0.9, "min_p": 0.1, **o}))
+        assert g == want, (i, g, want)
+
+
 def test_greedy_bfloat16_follows_the_plain_logits(model_dirs):
     """In bfloat16 the chain may leave the plain one at a near tie; every token the engine
     picks must be (nearly) the best under the plain logits for the engine's own prefix."""
